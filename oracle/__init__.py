@@ -1,0 +1,153 @@
+"""CPU oracle for the GGUF quantized-matmul path -- TEST INFRASTRUCTURE ONLY.
+
+ctypes binding of ``oracle/ggml_ref.c`` (a scalar C restatement of the ggml CPU semantics).
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import this package; the shipped library never does.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libggml_ref.so")
+
+F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (a second or two)."""
+    src = os.path.join(_HERE, "ggml_ref.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-B", "-C", _HERE, "libggml_ref.so"])
+    return _SO
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = ctypes.CDLL(_SO)
+        i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+        L.ref_block_size.restype = i64; L.ref_block_size.argtypes = [ci]
+        L.ref_type_size.restype = i64; L.ref_type_size.argtypes = [ci]
+        L.ref_row_size.restype = i64; L.ref_row_size.argtypes = [ci, i64]
+        L.ref_fp32_to_fp16.restype = ctypes.c_uint16; L.ref_fp32_to_fp16.argtypes = [ctypes.c_float]
+        L.ref_fp16_to_fp32.restype = ctypes.c_float; L.ref_fp16_to_fp32.argtypes = [ctypes.c_uint16]
+        L.ref_quantize.restype = ci; L.ref_quantize.argtypes = [ci, vp, vp, i64, i64, ci]
+        L.ref_dequantize_row.restype = ci; L.ref_dequantize_row.argtypes = [ci, vp, vp, i64]
+        L.ref_get_scale_min_k4.restype = None; L.ref_get_scale_min_k4.argtypes = [ci, vp, vp, vp]
+        L.ref_unpack_scales_kmask.restype = None; L.ref_unpack_scales_kmask.argtypes = [vp, vp, vp]
+        for name in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K"):
+            f = getattr(L, "ref_vec_dot_" + name)
+            f.restype = ctypes.c_float; f.argtypes = [i64, vp, vp]
+        L.ref_vec_dot_type.restype = ci; L.ref_vec_dot_type.argtypes = [ci]
+        L.ref_mul_mat.restype = ci
+        L.ref_mul_mat.argtypes = [ci, vp, i64, i64, vp, i64, vp, vp, ci]
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray) -> ctypes.c_void_p:
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def block_size(t: int) -> int:
+    return int(lib().ref_block_size(t))
+
+
+def type_size(t: int) -> int:
+    return int(lib().ref_type_size(t))
+
+
+def row_size(t: int, k: int) -> int:
+    return int(lib().ref_row_size(t, k))
+
+
+def vec_dot_type(t: int) -> int:
+    return int(lib().ref_vec_dot_type(t))
+
+
+def fp32_to_fp16(f: float) -> int:
+    return int(lib().ref_fp32_to_fp16(f))
+
+
+def fp16_to_fp32(h: int) -> float:
+    return float(lib().ref_fp16_to_fp32(h))
+
+
+def quantize(t: int, x: np.ndarray, nthreads: int = 1) -> np.ndarray:
+    """x: f32 [rows, k] -> uint8 [rows, row_size(t, k)] of GGUF-layout blocks."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if x.ndim == 1:
+        x = x[None, :]
+    rows, k = x.shape
+    rb = row_size(t, k)
+    if rb < 0:
+        raise ValueError(f"k={k} is not a multiple of the block size of type {t}")
+    out = np.zeros((rows, rb), dtype=np.uint8)
+    if lib().ref_quantize(t, _p(x), _p(out), k, rows, nthreads) != 0:
+        raise ValueError("ref_quantize failed")
+    return out
+
+
+def dequantize(t: int, blocks: np.ndarray, k: int) -> np.ndarray:
+    """blocks: uint8 [rows, row_size] -> f32 [rows, k]."""
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    if blocks.ndim == 1:
+        blocks = blocks[None, :]
+    rows = blocks.shape[0]
+    assert blocks.shape[1] == row_size(t, k)
+    out = np.empty((rows, k), dtype=np.float32)
+    for r in range(rows):
+        if lib().ref_dequantize_row(t, _p(blocks[r]), _p(out[r]), k) != 0:
+            raise ValueError("ref_dequantize_row failed")
+    return out
+
+
+_DOTS = {Q4_0: "q4_0_q8_0", Q8_0: "q8_0_q8_0", Q4_K: "q4_K_q8_K", Q6_K: "q6_K_q8_K"}
+
+
+def vec_dot(wtype: int, k: int, wrow: np.ndarray, xqrow: np.ndarray) -> float:
+    f = getattr(lib(), "ref_vec_dot_" + _DOTS[wtype])
+    wrow = np.ascontiguousarray(wrow, dtype=np.uint8)
+    xqrow = np.ascontiguousarray(xqrow, dtype=np.uint8)
+    assert wrow.size == row_size(wtype, k) and xqrow.size == row_size(vec_dot_type(wtype), k)
+    return float(f(k, _p(wrow), _p(xqrow)))
+
+
+def mul_mat(wtype: int, w: np.ndarray, k: int, m: int, x: np.ndarray, nthreads: int = 1,
+            return_xq: bool = False):
+    """w: uint8 GGUF blocks of m rows; x: f32 [n, k] -> y f32 [n, m] (y[n, m] = dot(W_m, Q(x_n)))."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if x.ndim == 1:
+        x = x[None, :]
+    n = x.shape[0]
+    assert x.shape[1] == k and w.size == m * row_size(wtype, k)
+    y = np.empty((n, m), dtype=np.float32)
+    xq = np.zeros((n, row_size(vec_dot_type(wtype), k)), dtype=np.uint8)
+    if lib().ref_mul_mat(wtype, _p(w), k, m, _p(x), n, _p(y), _p(xq), nthreads) != 0:
+        raise ValueError("ref_mul_mat failed")
+    return (y, xq) if return_xq else y
+
+
+def scale_min_k4(j: int, s12: np.ndarray):
+    s12 = np.ascontiguousarray(s12, dtype=np.uint8)
+    sc = np.zeros(1, np.uint8); m = np.zeros(1, np.uint8)
+    lib().ref_get_scale_min_k4(j, _p(s12), _p(sc), _p(m))
+    return int(sc[0]), int(m[0])
+
+
+def unpack_scales_kmask(s12: np.ndarray):
+    s12 = np.ascontiguousarray(s12, dtype=np.uint8)
+    sc = np.zeros(8, np.uint8); m = np.zeros(8, np.uint8)
+    lib().ref_unpack_scales_kmask(_p(s12), _p(sc), _p(m))
+    return sc, m

@@ -1,0 +1,85 @@
+/*
+ * CPU oracle for the GGUF block-quantized matmul path  --  TEST INFRASTRUCTURE ONLY.
+ *
+ * A scalar C restatement of the ggml CPU backend's semantics for
+ *   mul_mat(W quantized {Q4_0,Q8_0,Q4_K,Q6_K}, X f32) -> Y f32
+ * i.e. activation quantization to Q8_0 / Q8_K followed by the per-type integer dot products.
+ * Nothing in the shipped library links or calls this file: it is the checker the GPU path is
+ * compared against, and the timed "port" CPU baseline.
+ *
+ * The arithmetic lives in llama.cpp (ggml) at the tag the reference pins in
+ * /root/reference/LLAMA_CPP_VERSION:1 (b10488); that source is fetched at configure time
+ * (/root/reference/llama/server/CMakeLists.txt:112-188) and is not present offline, so this
+ * file restates the published algorithms (ggml-quants.c *_ref quantizers, ggml-cpu/quants.c
+ * generic vec_dot loops, ggml-cpu.c mul_mat driver).  What the reference itself pins:
+ *   block/type sizes      /root/reference/fs/ggml/ggml.go:407-513, ggml_test.go:163-213
+ *   ggml_type ids         /root/reference/fs/ggml/type.go:250-293
+ *   call shape            /root/reference/ml/backend.go:151 (Tensor.Mulmat)
+ *
+ * Parity status per function (what pins it is in tests/test_oracle_*.py):
+ *   fp16<->fp32, q8_0/q8_K quantizers, 6-bit scale unpack, four vec_dots, dequantizers,
+ *   mul_mat driver:  pinned (numpy float16, closed forms, fp64 brute force, KATs).
+ *   weight encoders q4_K / q6_K (make_qkx2_quants / make_qx_quants searches):
+ *   PARITY UNPINNED bit-for-bit against llama-quantize (only self-consistency and error
+ *   bounds are checked); q4_0 / q8_0 encoders are closed forms and pinned.
+ */
+#ifndef GGML_REF_H
+#define GGML_REF_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml_type ids, /root/reference/fs/ggml/type.go:250-268 */
+enum { REF_TYPE_F32 = 0, REF_TYPE_Q4_0 = 2, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12,
+       REF_TYPE_Q6_K = 14, REF_TYPE_Q8_K = 15 };
+
+int64_t ref_block_size(int type);               /* elements per block, 0 if unknown */
+int64_t ref_type_size(int type);                /* bytes per block                 */
+int64_t ref_row_size(int type, int64_t k);      /* bytes of a row of k elements, -1 if k % block */
+
+uint16_t ref_fp32_to_fp16(float f);
+float    ref_fp16_to_fp32(uint16_t h);
+
+/* activation quantizers (canonical scalar *_ref semantics) */
+void ref_quantize_row_q8_0(const float *x, void *y, int64_t k);
+void ref_quantize_row_q8_K(const float *x, void *y, int64_t k);
+
+/* weight encoders */
+void ref_quantize_row_q4_0(const float *x, void *y, int64_t k);
+void ref_quantize_row_q4_K(const float *x, void *y, int64_t k);
+void ref_quantize_row_q6_K(const float *x, void *y, int64_t k);
+/* dispatch on type (2, 8, 12, 14, 15); rows are independent. returns 0 or -1 */
+int  ref_quantize(int type, const float *x, void *y, int64_t k, int64_t rows, int nthreads);
+
+/* dequantizers */
+int  ref_dequantize_row(int type, const void *x, float *y, int64_t k);
+
+/* 6-bit scale/min unpack of a Q4_K block header (both published formulations) */
+void ref_get_scale_min_k4(int j, const uint8_t *s12, uint8_t *sc, uint8_t *m);
+void ref_unpack_scales_kmask(const uint8_t *s12, uint8_t sc[8], uint8_t m[8]);
+
+/* dot products: n elements, x = weight row blocks, y = activation row blocks */
+float ref_vec_dot_q4_0_q8_0(int64_t n, const void *x, const void *y);
+float ref_vec_dot_q8_0_q8_0(int64_t n, const void *x, const void *y);
+float ref_vec_dot_q4_K_q8_K(int64_t n, const void *x, const void *y);
+float ref_vec_dot_q6_K_q8_K(int64_t n, const void *x, const void *y);
+
+/* the activation type the CPU path quantizes to for a given weight type (8 or 15), -1 unknown */
+int  ref_vec_dot_type(int wtype);
+
+/*
+ * mul_mat driver: W is M rows of K elements in GGUF block layout, X is N rows of K floats,
+ * Y[n*M + m] = vec_dot(W row m, Q(X row n)).  xq_out (optional) receives the quantized
+ * activation rows (N * row_size(vec_dot_type, K) bytes).  returns 0 or -1 on bad arguments.
+ */
+int  ref_mul_mat(int wtype, const void *w, int64_t k, int64_t m,
+                 const float *x, int64_t n, float *y, void *xq_out, int nthreads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
