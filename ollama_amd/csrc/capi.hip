@@ -1,0 +1,556 @@
+// C ABI of the library (include/mi_qmm.h): argument checking, device memory, kernel dispatch.
+// Everything that computes runs on the GPU; there is no CPU fallback in this file.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "../../include/mi_qmm.h"
+#include "internal.h"
+
+using namespace miqmm;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                       \
+    do {                                                                                    \
+        hipError_t e_ = (expr);                                                             \
+        if (e_ != hipSuccess)                                                               \
+            return fail(e_ == hipErrorOutOfMemory ? MI_QMM_ERR_NOMEM : MI_QMM_ERR_HIP,      \
+                        "%s: %s", #expr, hipGetErrorString(e_));                            \
+    } while (0)
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+struct mi_qmm_ctx {
+    int device = 0;
+    int num_cus = 0;
+    int clock_mhz = 0;
+    char name[128] = {0};
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    // growable scratch: quantized activation planes and host<->device staging
+    void *act_buf = nullptr;  size_t act_cap = 0;
+    void *io_buf = nullptr;   size_t io_cap = 0;
+};
+
+struct mi_qmm_weight {
+    int device = 0;
+    void *base = nullptr;
+    size_t bytes = 0;
+    DevWeight dev{};
+};
+
+struct mi_qmm_act {
+    int device = 0;
+    int type = 0;
+    int64_t k = 0, n_max = 0, n = 0;
+    void *base = nullptr;
+};
+
+namespace {
+
+int reserve(void **buf, size_t *cap, size_t need, hipStream_t s) {
+    if (need <= *cap) return MI_QMM_OK;
+    if (*buf) {
+        HIP_TRY(hipStreamSynchronize(s));  // queued kernels may still read the old buffer
+        HIP_TRY(hipFree(*buf));
+        *buf = nullptr;
+        *cap = 0;
+    }
+    need = align_up(need + need / 4, 1 << 20);
+    HIP_TRY(hipMalloc(buf, need));
+    *cap = need;
+    return MI_QMM_OK;
+}
+
+struct ActPlanes { int8_t *qs; float *d; int16_t *bsums; size_t total; };
+
+// carve the activation scratch into planes for N rows of K elements
+ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N) {
+    const int64_t blk = q8_type == T_Q8_0 ? QK : QKK;
+    const int64_t sums = q8_type == T_Q8_0 ? QK : 16;
+    ActPlanes p;
+    size_t off = 0;
+    p.qs = (int8_t *)((char *)base + off);     off = align_up(off + (size_t)(N * K), 256);
+    p.d = (float *)((char *)base + off);       off = align_up(off + (size_t)(N * (K / blk)) * 4, 256);
+    p.bsums = (int16_t *)((char *)base + off); off = align_up(off + (size_t)(N * (K / sums)) * 2, 256);
+    p.total = off;
+    return p;
+}
+
+int check_ctx(mi_qmm_ctx *ctx) {
+    if (!ctx) return fail(MI_QMM_ERR_INVALID, "ctx is NULL");
+    HIP_TRY(hipSetDevice(ctx->device));  // calls may arrive on any OS thread
+    return MI_QMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *mi_qmm_last_error(void) { return g_err; }
+const char *mi_qmm_version(void) { return "mi_qmm 0.1 (gfx950)"; }
+
+// ---- size tables, every id of /root/reference/fs/ggml/ggml.go:407-513 ------------------------
+int64_t mi_qmm_block_size(int t) {
+    switch (t) {
+    case 0: case 1: case 24: case 25: case 26: case 27: case 28: case 30: return 1;  // F32 F16 I8..F64 BF16
+    case 2: case 3: case 6: case 7: case 8: case 9: case 20: case 39: return 32;     // Q4_0..Q8_1 IQ4_NL MXFP4
+    case 40: return 64;                                                              // NVFP4
+    case 41: return 128;                                                             // Q1_0
+    case 10: case 11: case 12: case 13: case 14: case 15: case 16: case 17: case 18: case 19: case 21:
+    case 22: case 23: case 29: case 34: case 35: return 256;                         // K-quants, IQ*, TQ*
+    default: return 0;
+    }
+}
+
+int64_t mi_qmm_type_size(int t) {
+    const int64_t b = mi_qmm_block_size(t);
+    switch (t) {
+    case 0: return 4;
+    case 1: return 2;
+    case 2: return 2 + b / 2;
+    case 3: return 2 + 2 + b / 2;
+    case 6: return 2 + 4 + b / 2;
+    case 7: return 2 + 2 + 4 + b / 2;
+    case 8: return 2 + b;
+    case 9: return 2 + 2 + b;
+    case 10: return b / 16 + b / 4 + 2 + 2;
+    case 11: return b / 8 + b / 4 + 12 + 2;
+    case 12: return 2 + 2 + 12 + b / 2;
+    case 13: return 2 + 2 + 12 + b / 8 + b / 2;
+    case 14: return b / 2 + b / 4 + b / 16 + 2;
+    case 15: return 4 + b + 2 * b / 16;
+    case 16: return 2 + 2 * b / 8;
+    case 17: return 2 + 2 * b / 8 + b / 32;
+    case 18: return 2 + b / 4 + b / 8;
+    case 19: return 2 + b / 8 + b / 16;
+    case 20: return 2 + b / 2;
+    case 21: return 2 + b / 4 + b / 8 + b / 32 + 4;
+    case 22: return 2 + b / 4 + b / 16;
+    case 23: return 2 + 2 + b / 2 + b / 64;
+    case 24: return 1;
+    case 25: return 2;
+    case 26: return 4;
+    case 27: return 8;
+    case 28: return 8;
+    case 29: return b / 8 + b / 16 + b / 32;
+    case 30: return 2;
+    case 39: return 1 + b / 2;
+    case 40: return 4 + b / 2;
+    case 41: return 2 + b / 8;
+    default: return 0;  // includes TQ1_0/TQ2_0 (34, 35), which the reference's TypeSize leaves at 0
+    }
+}
+
+int64_t mi_qmm_row_size(int t, int64_t k) {
+    const int64_t b = mi_qmm_block_size(t), s = mi_qmm_type_size(t);
+    if (b == 0 || s == 0 || k < 0 || k % b != 0) return -1;
+    return k / b * s;
+}
+
+int mi_qmm_vec_dot_type(int wt) {
+    switch (wt) {
+    case T_Q4_0: case T_Q8_0: return T_Q8_0;
+    case T_Q4_K: case T_Q6_K: return T_Q8_K;
+    default: return -1;
+    }
+}
+
+// ---- lifetime -----------------------------------------------------------------------------------
+int mi_qmm_init(int device_ordinal, mi_qmm_ctx **out) {
+    if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(MI_QMM_ERR_NODEVICE, "no HIP device visible (%s); this library has no CPU path",
+                    e == hipSuccess ? "device count 0" : hipGetErrorString(e));
+    if (device_ordinal < 0 || device_ordinal >= count)
+        return fail(MI_QMM_ERR_NODEVICE, "device ordinal %d out of range (0..%d)", device_ordinal, count - 1);
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device_ordinal));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(MI_QMM_ERR_NODEVICE, "device %d is %s; the kernels are built for gfx950 only",
+                    device_ordinal, prop.gcnArchName);
+    HIP_TRY(hipSetDevice(device_ordinal));
+    mi_qmm_ctx *c = new (std::nothrow) mi_qmm_ctx();
+    if (!c) return fail(MI_QMM_ERR_NOMEM, "host allocation failed");
+    c->device = device_ordinal;
+    c->num_cus = prop.multiProcessorCount;
+    c->clock_mhz = prop.clockRate / 1000;
+    snprintf(c->name, sizeof(c->name), "%s (%s)", prop.name, prop.gcnArchName);
+    e = hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete c;
+        return fail(MI_QMM_ERR_HIP, "hipStreamCreate: %s", hipGetErrorString(e));
+    }
+    c->stream = c->own_stream;
+    *out = c;
+    return MI_QMM_OK;
+}
+
+void mi_qmm_destroy(mi_qmm_ctx *ctx) {
+    if (!ctx) return;
+    if (hipSetDevice(ctx->device) == hipSuccess) {
+        (void)hipStreamSynchronize(ctx->stream);
+        if (ctx->act_buf) (void)hipFree(ctx->act_buf);
+        if (ctx->io_buf) (void)hipFree(ctx->io_buf);
+        if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
+    }
+    delete ctx;
+}
+
+int mi_qmm_set_stream(mi_qmm_ctx *ctx, void *hip_stream) {
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    return MI_QMM_OK;
+}
+
+int mi_qmm_sync(mi_qmm_ctx *ctx) {
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return MI_QMM_OK;
+}
+
+int mi_qmm_device_info(mi_qmm_ctx *ctx, int *compute_units, int *clock_mhz, char *name, int name_len) {
+    if (!ctx) return fail(MI_QMM_ERR_INVALID, "ctx is NULL");
+    if (compute_units) *compute_units = ctx->num_cus;
+    if (clock_mhz) *clock_mhz = ctx->clock_mhz;
+    if (name && name_len > 0) snprintf(name, (size_t)name_len, "%s", ctx->name);
+    return MI_QMM_OK;
+}
+
+// ---- weights --------------------------------------------------------------------------------------
+int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k, int64_t m, int src_location,
+                         mi_qmm_weight **out) {
+    if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (mi_qmm_vec_dot_type(type) < 0)
+        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (2, 8, 12, 14)", type);
+    if (k <= 0 || m <= 0) return fail(MI_QMM_ERR_INVALID, "k=%lld m=%lld must be positive", (long long)k, (long long)m);
+    const int64_t row = mi_qmm_row_size(type, k);
+    if (row < 0)
+        return fail(MI_QMM_ERR_INVALID, "k=%lld is not a multiple of the block size %lld of type %d",
+                    (long long)k, (long long)mi_qmm_block_size(type), type);
+    if (type == T_Q4_0 || type == T_Q8_0) {
+        // the activation quantizer pairs these with Q8_0 planes read as 16-byte pieces
+        if (k % QK != 0) return fail(MI_QMM_ERR_INVALID, "k not a multiple of 32");
+    }
+    if (!bytes) return fail(MI_QMM_ERR_INVALID, "gguf_bytes is NULL");
+    if (src_location != MI_QMM_HOST && src_location != MI_QMM_DEVICE)
+        return fail(MI_QMM_ERR_INVALID, "src_location must be MI_QMM_HOST or MI_QMM_DEVICE");
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+
+    const size_t total = (size_t)(row * m);
+    // plane sizes (bytes), each plane 256-byte aligned inside one allocation
+    size_t s0 = 0, s1 = 0, s2 = 0, sd = 0;
+    switch (type) {
+    case T_Q4_K: s0 = total; break;
+    case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
+    case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
+    case T_Q6_K: s0 = (size_t)(m * (k / 2)); s1 = (size_t)(m * (k / 4)); s2 = (size_t)(m * (k / 16));
+                 sd = (size_t)(m * (k / QKK)) * 2; break;
+    }
+    const size_t o0 = 0, o1 = align_up(o0 + s0, 256), o2 = align_up(o1 + s1, 256), od = align_up(o2 + s2, 256);
+    const size_t dev_bytes = align_up(od + sd, 256) + 256;  // tail slack: 16-byte loads never leave the allocation
+
+    mi_qmm_weight *w = new (std::nothrow) mi_qmm_weight();
+    if (!w) return fail(MI_QMM_ERR_NOMEM, "host allocation failed");
+    w->device = ctx->device;
+    hipError_t e = hipMalloc(&w->base, dev_bytes);
+    if (e != hipSuccess) {
+        delete w;
+        return fail(MI_QMM_ERR_NOMEM, "hipMalloc(%zu) for weight: %s", dev_bytes, hipGetErrorString(e));
+    }
+    w->bytes = dev_bytes;
+    uint8_t *b = (uint8_t *)w->base;
+    w->dev.p0 = b + o0;
+    w->dev.p1 = s1 ? b + o1 : nullptr;
+    w->dev.p2 = s2 ? b + o2 : nullptr;
+    w->dev.d = sd ? (const uint16_t *)(b + od) : nullptr;
+    w->dev.K = k; w->dev.M = m; w->dev.type = type;
+
+    void *staging = nullptr;
+    const uint8_t *src = (const uint8_t *)bytes;
+    auto cleanup = [&](int code, const char *what, hipError_t err) {
+        if (staging) (void)hipFree(staging);
+        (void)hipFree(w->base);
+        delete w;
+        return fail(code, "%s: %s", what, hipGetErrorString(err));
+    };
+    if (type == T_Q4_K) {
+        e = hipMemcpyAsync(b + o0, bytes, total,
+                           src_location == MI_QMM_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice, ctx->stream);
+        if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(weight)", e);
+    } else {
+        if (src_location == MI_QMM_HOST) {
+            e = hipMalloc(&staging, total);
+            if (e != hipSuccess) return cleanup(MI_QMM_ERR_NOMEM, "hipMalloc(staging)", e);
+            e = hipMemcpyAsync(staging, bytes, total, hipMemcpyHostToDevice, ctx->stream);
+            if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(staging)", e);
+            src = (const uint8_t *)staging;
+        }
+        e = launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
+        if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
+    }
+    e = hipStreamSynchronize(ctx->stream);  // the caller's bytes must not be needed after return
+    if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipStreamSynchronize(upload)", e);
+    if (staging) (void)hipFree(staging);
+    *out = w;
+    return MI_QMM_OK;
+}
+
+void mi_qmm_weight_free(mi_qmm_weight *w) {
+    if (!w) return;
+    if (hipSetDevice(w->device) == hipSuccess && w->base) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(w->base);
+    }
+    delete w;
+}
+
+int mi_qmm_weight_info(const mi_qmm_weight *w, int *type, int64_t *k, int64_t *m, int64_t *device_bytes) {
+    if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
+    if (type) *type = w->dev.type;
+    if (k) *k = w->dev.K;
+    if (m) *m = w->dev.M;
+    if (device_bytes) *device_bytes = (int64_t)w->bytes;
+    return MI_QMM_OK;
+}
+
+// ---- activation quantization ---------------------------------------------------------------------
+int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k, int64_t n, void *out_blocks,
+                        int location) {
+    if (q8_type != T_Q8_0 && q8_type != T_Q8_K)
+        return fail(MI_QMM_ERR_UNSUPPORTED, "activation type %d is not Q8_0 (8) or Q8_K (15)", q8_type);
+    if (k < 0 || n < 0) return fail(MI_QMM_ERR_INVALID, "k=%lld n=%lld must be non-negative", (long long)k, (long long)n);
+    const int64_t row = mi_qmm_row_size(q8_type, k);
+    if (row < 0)
+        return fail(MI_QMM_ERR_INVALID, "k=%lld is not a multiple of the block size %lld of type %d",
+                    (long long)k, (long long)mi_qmm_block_size(q8_type), q8_type);
+    if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
+        return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    if (k * n == 0) return MI_QMM_OK;
+    if (!x || !out_blocks) return fail(MI_QMM_ERR_INVALID, "x or out_blocks is NULL");
+
+    const ActPlanes probe = plan_act(nullptr, q8_type, k, n);
+    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+    const ActPlanes p = plan_act(ctx->act_buf, q8_type, k, n);
+    const size_t xbytes = (size_t)(n * k) * 4, obytes = (size_t)(n * row);
+    const float *dx = x;
+    uint8_t *dout = (uint8_t *)out_blocks;
+    if (location == MI_QMM_HOST) {
+        const size_t xoff = align_up(obytes, 256);
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, xoff + xbytes, ctx->stream))) return rc;
+        dout = (uint8_t *)ctx->io_buf;
+        dx = (const float *)((char *)ctx->io_buf + xoff);
+        HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    HIP_TRY(launch_quantize_act(q8_type, dx, k, n, p.qs, p.d, p.bsums, ctx->stream));
+    HIP_TRY(launch_pack_act_gguf(q8_type, p.qs, p.d, p.bsums, k, n, dout, ctx->stream));
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(out_blocks, dout, obytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+}  // extern "C"
+
+// ---- the product ------------------------------------------------------------------------------------
+namespace {
+
+// dy: device output [n][M].  Picks the kernel and queues it on the ctx's stream.
+int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path) {
+    const int64_t K = w->dev.K, M = w->dev.M, n = a.N;
+    bool use_gemm;
+    if (path == MI_QMM_PATH_GEMM) use_gemm = true;
+    else if (path == MI_QMM_PATH_GEMV) use_gemm = false;
+    else use_gemm = n >= 32 && gemm_supports(w->dev.type, K, M);
+    if (use_gemm && !gemm_supports(w->dev.type, K, M))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "the MFMA GEMM does not cover type %d with K=%lld M=%lld", w->dev.type,
+                    (long long)K, (long long)M);
+    if (!use_gemm && K > gemv_max_k(w->dev.type))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "K=%lld exceeds the GEMV limit %lld for type %d", (long long)K,
+                    (long long)gemv_max_k(w->dev.type), w->dev.type);
+    if (use_gemm) {
+        HIP_TRY(launch_gemm(w->dev, a, dy, M, ctx->num_cus, ctx->stream));
+    } else {
+        for (int64_t c0 = 0; c0 < n; c0 += 8) {
+            const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
+            HIP_TRY(launch_gemv(w->dev, a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
+        }
+    }
+    return MI_QMM_OK;
+}
+
+int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, int path) {
+    if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
+    if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
+        return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
+    if (path != MI_QMM_PATH_AUTO && path != MI_QMM_PATH_GEMV && path != MI_QMM_PATH_GEMM)
+        return fail(MI_QMM_ERR_INVALID, "unknown path %d", path);
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    if (w->device != ctx->device)
+        return fail(MI_QMM_ERR_INVALID, "weight lives on device %d, ctx on device %d", w->device, ctx->device);
+    return MI_QMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location,
+                       int path) {
+    if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
+    int rc = check_product_args(ctx, w, location, path);
+    if (rc) return rc;
+    if (n == 0) return MI_QMM_OK;
+    if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
+    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+
+    const int64_t K = w->dev.K, M = w->dev.M;
+    const int q8 = mi_qmm_vec_dot_type(w->dev.type);
+    const ActPlanes probe = plan_act(nullptr, q8, K, n);
+    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+    const ActPlanes p = plan_act(ctx->act_buf, q8, K, n);
+
+    const size_t xbytes = (size_t)(n * K) * 4, ybytes = (size_t)(n * M) * 4;
+    const float *dx = x;
+    float *dy = y;
+    if (location == MI_QMM_HOST) {
+        const size_t yoff = align_up(xbytes, 256);
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, yoff + ybytes, ctx->stream))) return rc;
+        dx = (const float *)ctx->io_buf;
+        dy = (float *)((char *)ctx->io_buf + yoff);
+        HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, ctx->stream));
+    DevAct a;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.K = K; a.N = (int)n; a.type = q8;
+    if ((rc = run_product(ctx, w, a, dy, path))) return rc;
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location) {
+    return mi_qmm_mulmat_path(ctx, w, x, n, y, location, MI_QMM_PATH_AUTO);
+}
+
+// ---- two-phase form ----------------------------------------------------------------------------------
+int mi_qmm_act_create(mi_qmm_ctx *ctx, int q8_type, int64_t k, int64_t n_max, mi_qmm_act **out) {
+    if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (q8_type != T_Q8_0 && q8_type != T_Q8_K)
+        return fail(MI_QMM_ERR_UNSUPPORTED, "activation type %d is not Q8_0 (8) or Q8_K (15)", q8_type);
+    if (k <= 0 || n_max <= 0 || n_max > INT32_MAX)
+        return fail(MI_QMM_ERR_INVALID, "k=%lld n_max=%lld must be positive", (long long)k, (long long)n_max);
+    if (mi_qmm_row_size(q8_type, k) < 0)
+        return fail(MI_QMM_ERR_INVALID, "k=%lld is not a multiple of the block size %lld of type %d",
+                    (long long)k, (long long)mi_qmm_block_size(q8_type), q8_type);
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    mi_qmm_act *a = new (std::nothrow) mi_qmm_act();
+    if (!a) return fail(MI_QMM_ERR_NOMEM, "host allocation failed");
+    a->device = ctx->device; a->type = q8_type; a->k = k; a->n_max = n_max;
+    const ActPlanes probe = plan_act(nullptr, q8_type, k, n_max);
+    hipError_t e = hipMalloc(&a->base, probe.total + 256);
+    if (e != hipSuccess) {
+        delete a;
+        return fail(MI_QMM_ERR_NOMEM, "hipMalloc(%zu) for activations: %s", probe.total, hipGetErrorString(e));
+    }
+    *out = a;
+    return MI_QMM_OK;
+}
+
+void mi_qmm_act_free(mi_qmm_act *act) {
+    if (!act) return;
+    if (hipSetDevice(act->device) == hipSuccess && act->base) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(act->base);
+    }
+    delete act;
+}
+
+int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_t n, int location) {
+    if (!act) return fail(MI_QMM_ERR_INVALID, "act is NULL");
+    if (n < 0 || n > act->n_max)
+        return fail(MI_QMM_ERR_INVALID, "n=%lld outside 0..n_max=%lld", (long long)n, (long long)act->n_max);
+    if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
+        return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    if (act->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "act and ctx are on different devices");
+    act->n = n;
+    if (n == 0) return MI_QMM_OK;
+    if (!x) return fail(MI_QMM_ERR_INVALID, "x is NULL");
+    // planes are carved for n_max so their addresses do not move between calls
+    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
+    const float *dx = x;
+    if (location == MI_QMM_HOST) {
+        const size_t xbytes = (size_t)(n * act->k) * 4;
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, xbytes, ctx->stream))) return rc;
+        dx = (const float *)ctx->io_buf;
+        HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    HIP_TRY(launch_quantize_act(act->type, dx, act->k, n, p.qs, p.d, p.bsums, ctx->stream));
+    if (location == MI_QMM_HOST) HIP_TRY(hipStreamSynchronize(ctx->stream));  // x may be reused by the caller
+    return MI_QMM_OK;
+}
+
+int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *act, float *y, int location,
+                     int path) {
+    if (!act) return fail(MI_QMM_ERR_INVALID, "act is NULL");
+    int rc = check_product_args(ctx, w, location, path);
+    if (rc) return rc;
+    if (act->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "act and ctx are on different devices");
+    if (act->type != mi_qmm_vec_dot_type(w->dev.type) || act->k != w->dev.K)
+        return fail(MI_QMM_ERR_INVALID, "act (type %d, k=%lld) does not match weight (type %d needs %d, k=%lld)",
+                    act->type, (long long)act->k, w->dev.type, mi_qmm_vec_dot_type(w->dev.type), (long long)w->dev.K);
+    const int64_t n = act->n, M = w->dev.M;
+    if (n == 0) return MI_QMM_OK;
+    if (!y) return fail(MI_QMM_ERR_INVALID, "y is NULL");
+    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
+    DevAct a;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.K = act->k; a.N = (int)n; a.type = act->type;
+    float *dy = y;
+    const size_t ybytes = (size_t)(n * M) * 4;
+    if (location == MI_QMM_HOST) {
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, ybytes, ctx->stream))) return rc;
+        dy = (float *)ctx->io_buf;
+    }
+    if ((rc = run_product(ctx, w, a, dy, path))) return rc;
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,52 @@
+// GGUF block formats on the quantized-matmul path, and the device-private layouts the kernels read.
+//
+// Block byte layouts follow the size formulas in /root/reference/fs/ggml/ggml.go:450-473:
+//   Q4_0  2 + 32/2             = 18   fp16 d; u8 qs[16]  (low nibbles = elements 0..15, high = 16..31; value q-8)
+//   Q8_0  2 + 32               = 34   fp16 d; i8 qs[32]
+//   Q4_K  2 + 2 + 12 + 256/2   = 144  fp16 d, dmin; u8 scales[12] (8 x 6-bit scale + 8 x 6-bit min); u8 qs[128]
+//   Q6_K  256/2 + 256/4 + 16+2 = 210  u8 ql[128]; u8 qh[64]; i8 scales[16]; fp16 d   (value q-32)
+//   Q8_K  4 + 256 + 2*16       = 292  f32 d; i8 qs[256]; i16 bsums[16]
+#pragma once
+
+#include <stdint.h>
+
+namespace miqmm {
+
+enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15 };
+
+constexpr int QK = 32;    // elements per Q4_0 / Q8_0 block
+constexpr int QKK = 256;  // elements per K-quant super-block
+constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q6_K_BYTES = 210, Q8_K_BYTES = 292;
+
+// Weight tensor as the kernels see it.  Device-private "plane" layout chosen so that every
+// wavefront load is a run of aligned 16-byte pieces:
+//   Q4_K : p0 = the GGUF blocks unchanged (144 B is already 16-B aligned: header 16 B + qs 128 B)
+//   Q4_0 : p0 = qs plane, 16 B per block, [M][K/32][16];           d = fp16 plane [M][K/32]
+//   Q8_0 : p0 = qs plane, 32 B per block, [M][K];                  d = fp16 plane [M][K/32]
+//   Q6_K : p0 = ql plane [M][K/2]; p1 = qh plane [M][K/4]; p2 = scales plane [M][K/16] (i8);
+//          d = fp16 plane [M][K/256]
+// Byte order inside each plane is the GGUF order; only the interleaving of fields is undone.
+struct DevWeight {
+    const uint8_t *p0;
+    const uint8_t *p1;
+    const uint8_t *p2;
+    const uint16_t *d;
+    int64_t K, M;
+    int type;
+};
+
+// Quantized activations as the kernels see them (structure of arrays, one row per activation row):
+//   qs    [N][K]      int8 quants
+//   d     [N][K/B]    fp32 block scale (B = 32 for Q8_0 where the value is the fp16-rounded scale
+//                     widened exactly; B = 256 for Q8_K)
+//   bsums [N][K/S]    int16 partial sums of quants (S = 32 for Q8_0: one per block; S = 16 for Q8_K)
+struct DevAct {
+    const int8_t *qs;
+    const float *d;
+    const int16_t *bsums;
+    int64_t K;
+    int N;
+    int type;  // T_Q8_0 or T_Q8_K
+};
+
+}  // namespace miqmm

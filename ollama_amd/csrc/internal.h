@@ -1,0 +1,34 @@
+// Launchers shared between the C ABI (capi.hip) and the kernel translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "formats.h"
+
+namespace miqmm {
+
+// kernel 1: f32 rows -> Q8_0 / Q8_K planes (bit-exact with the scalar CPU quantizers)
+hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs,
+                               float *d, int16_t *bsums, hipStream_t s);
+// planes -> GGUF block bytes (34 B / 292 B blocks), for callers that want the bytes
+hipError_t launch_pack_act_gguf(int q8_type, const int8_t *qs, const float *d, const int16_t *bsums,
+                                int64_t K, int64_t N, uint8_t *out, hipStream_t s);
+
+// upload-time re-layout GGUF blocks -> planes (Q4_0, Q8_0, Q6_K); Q4_K is copied unchanged
+hipError_t launch_relayout(int type, const uint8_t *gguf, int64_t K, int64_t M, uint8_t *p0,
+                           uint8_t *p1, uint8_t *p2, uint16_t *d, hipStream_t s);
+
+// kernels 2 and 4: streaming GEMV / skinny GEMM, ncols in 1..8.  y[n*ldy + m].
+// returns hipErrorInvalidValue if the shape is outside the kernel's limits (caller reports it).
+hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y,
+                       int64_t ldy, int num_cus, hipStream_t s);
+// largest K the GEMV handles for a weight type
+int64_t gemv_max_k(int type);
+
+// kernel 3: int8-MFMA GEMM, any N >= 1.  y[n*ldy + m]
+hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, int num_cus,
+                       hipStream_t s);
+bool gemm_supports(int type, int64_t K, int64_t M);
+
+}  // namespace miqmm

@@ -1,0 +1,266 @@
+"""ctypes binding of libmi_qmm.so (the C ABI declared in include/mi_qmm.h).
+
+Fails loudly when the library has not been built: nothing here computes on the CPU.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi_qmm.so")
+
+F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
+HOST, DEVICE = 0, 1
+PATH_AUTO, PATH_GEMV, PATH_GEMM = 0, 1, 2
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, -3, -4, -5
+
+EXPORTS = [
+    "mi_qmm_block_size", "mi_qmm_type_size", "mi_qmm_row_size", "mi_qmm_vec_dot_type",
+    "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync",
+    "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
+    "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
+    "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8",
+    "mi_qmm_last_error", "mi_qmm_version", "mi_qmm_device_info",
+]
+
+
+class QmmError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"mi_qmm error {code}: {msg}")
+        self.code = code
+
+
+def build(verbose: bool = False) -> str:
+    """Compile the HIP library in-tree with hipcc for gfx950 (cross-compiles without a GPU)."""
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j8", "-B"]
+    subprocess.run(cmd, check=True, stdout=None if verbose else subprocess.DEVNULL,
+                   stderr=None if verbose else subprocess.DEVNULL)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                           "(there is no CPU fallback)")
+    L = ctypes.CDLL(LIB_PATH)
+    i64, vp, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+    L.mi_qmm_block_size.restype = i64; L.mi_qmm_block_size.argtypes = [ci]
+    L.mi_qmm_type_size.restype = i64; L.mi_qmm_type_size.argtypes = [ci]
+    L.mi_qmm_row_size.restype = i64; L.mi_qmm_row_size.argtypes = [ci, i64]
+    L.mi_qmm_vec_dot_type.restype = ci; L.mi_qmm_vec_dot_type.argtypes = [ci]
+    L.mi_qmm_init.restype = ci; L.mi_qmm_init.argtypes = [ci, ctypes.POINTER(vp)]
+    L.mi_qmm_destroy.restype = None; L.mi_qmm_destroy.argtypes = [vp]
+    L.mi_qmm_set_stream.restype = ci; L.mi_qmm_set_stream.argtypes = [vp, vp]
+    L.mi_qmm_sync.restype = ci; L.mi_qmm_sync.argtypes = [vp]
+    L.mi_qmm_weight_upload.restype = ci
+    L.mi_qmm_weight_upload.argtypes = [vp, ci, vp, i64, i64, ci, ctypes.POINTER(vp)]
+    L.mi_qmm_weight_free.restype = None; L.mi_qmm_weight_free.argtypes = [vp]
+    L.mi_qmm_weight_info.restype = ci
+    L.mi_qmm_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
+                                     ctypes.POINTER(i64)]
+    L.mi_qmm_quantize_act.restype = ci; L.mi_qmm_quantize_act.argtypes = [vp, ci, vp, i64, i64, vp, ci]
+    L.mi_qmm_mulmat.restype = ci; L.mi_qmm_mulmat.argtypes = [vp, vp, vp, i64, vp, ci]
+    L.mi_qmm_mulmat_path.restype = ci; L.mi_qmm_mulmat_path.argtypes = [vp, vp, vp, i64, vp, ci, ci]
+    L.mi_qmm_act_create.restype = ci; L.mi_qmm_act_create.argtypes = [vp, ci, i64, i64, ctypes.POINTER(vp)]
+    L.mi_qmm_act_free.restype = None; L.mi_qmm_act_free.argtypes = [vp]
+    L.mi_qmm_act_quantize.restype = ci; L.mi_qmm_act_quantize.argtypes = [vp, vp, vp, i64, ci]
+    L.mi_qmm_mulmat_q8.restype = ci; L.mi_qmm_mulmat_q8.argtypes = [vp, vp, vp, vp, ci, ci]
+    L.mi_qmm_last_error.restype = ctypes.c_char_p; L.mi_qmm_last_error.argtypes = []
+    L.mi_qmm_version.restype = ctypes.c_char_p; L.mi_qmm_version.argtypes = []
+    L.mi_qmm_device_info.restype = ci
+    L.mi_qmm_device_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.c_char_p, ci]
+    _lib = L
+    return L
+
+
+def last_error() -> str:
+    return lib().mi_qmm_last_error().decode()
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise QmmError(rc, last_error())
+
+
+def block_size(t: int) -> int:
+    return int(lib().mi_qmm_block_size(t))
+
+
+def type_size(t: int) -> int:
+    return int(lib().mi_qmm_type_size(t))
+
+
+def row_size(t: int, k: int) -> int:
+    return int(lib().mi_qmm_row_size(t, k))
+
+
+def vec_dot_type(t: int) -> int:
+    return int(lib().mi_qmm_vec_dot_type(t))
+
+
+def _ptr(a) -> ctypes.c_void_p:
+    if a is None:
+        return ctypes.c_void_p(None)
+    if isinstance(a, np.ndarray):
+        return ctypes.c_void_p(a.ctypes.data)
+    return ctypes.c_void_p(int(a))  # raw device / host address
+
+
+class Weight:
+    """A weight tensor resident in HBM (mi_qmm_weight)."""
+
+    def __init__(self, handle, ggml_type: int, k: int, m: int):
+        self._h = handle
+        self.type, self.k, self.m = ggml_type, k, m
+
+    @property
+    def device_bytes(self) -> int:
+        nb = ctypes.c_int64()
+        _check(lib().mi_qmm_weight_info(self._h, None, None, None, ctypes.byref(nb)))
+        return nb.value
+
+    @property
+    def gguf_bytes(self) -> int:
+        return row_size(self.type, self.k) * self.m
+
+    def free(self):
+        if self._h:
+            lib().mi_qmm_weight_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Act:
+    """Quantized activations resident on the device (mi_qmm_act), reusable across calls."""
+
+    def __init__(self, handle, q8_type: int, k: int, n_max: int):
+        self._h = handle
+        self.type, self.k, self.n_max, self.n = q8_type, k, n_max, 0
+
+    def free(self):
+        if self._h:
+            lib().mi_qmm_act_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context:
+    """One device + stream + scratch (mi_qmm_ctx)."""
+
+    def __init__(self, device: int = 0):
+        h = ctypes.c_void_p()
+        _check(lib().mi_qmm_init(device, ctypes.byref(h)))
+        self._h = h
+
+    def close(self):
+        if self._h:
+            lib().mi_qmm_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def device_info(self):
+        cus, mhz = ctypes.c_int(), ctypes.c_int()
+        name = ctypes.create_string_buffer(128)
+        _check(lib().mi_qmm_device_info(self._h, ctypes.byref(cus), ctypes.byref(mhz), name, 128))
+        return {"compute_units": cus.value, "clock_mhz": mhz.value, "name": name.value.decode()}
+
+    def set_stream(self, stream_ptr: int | None):
+        _check(lib().mi_qmm_set_stream(self._h, ctypes.c_void_p(stream_ptr or None)))
+
+    def sync(self):
+        _check(lib().mi_qmm_sync(self._h))
+
+    def upload(self, ggml_type: int, gguf_bytes, k: int, m: int, location: int = HOST) -> Weight:
+        if isinstance(gguf_bytes, np.ndarray):
+            gguf_bytes = np.ascontiguousarray(gguf_bytes, dtype=np.uint8)
+            rs = row_size(ggml_type, k)
+            if rs >= 0 and gguf_bytes.size != rs * m:
+                raise ValueError(f"weight bytes {gguf_bytes.size} != m*row_size = {rs * m}")
+        h = ctypes.c_void_p()
+        _check(lib().mi_qmm_weight_upload(self._h, ggml_type, _ptr(gguf_bytes), k, m, location, ctypes.byref(h)))
+        return Weight(h, ggml_type, k, m)
+
+    def quantize_act(self, q8_type: int, x: np.ndarray) -> np.ndarray:
+        """x f32 [n, k] -> uint8 [n, row_size] GGUF-layout Q8_0 / Q8_K blocks computed on the GPU."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        n, k = x.shape
+        rs = row_size(q8_type, k)
+        out = np.zeros((n, max(rs, 0)), dtype=np.uint8)
+        _check(lib().mi_qmm_quantize_act(self._h, q8_type, _ptr(x), k, n, _ptr(out), HOST))
+        return out
+
+    def mulmat(self, w: Weight, x: np.ndarray, path: int = PATH_AUTO) -> np.ndarray:
+        """x f32 [n, k] -> y f32 [n, m]; host arrays in and out."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        n, k = x.shape
+        if k != w.k:
+            raise ValueError(f"x has k={k}, weight has k={w.k}")
+        y = np.empty((n, w.m), dtype=np.float32)
+        _check(lib().mi_qmm_mulmat_path(self._h, w._h, _ptr(x), n, _ptr(y), HOST, path))
+        return y
+
+    def mulmat_device(self, w: Weight, x_ptr: int, n: int, y_ptr: int, path: int = PATH_AUTO):
+        """device pointers in and out; queued on the ctx stream, returns without waiting."""
+        _check(lib().mi_qmm_mulmat_path(self._h, w._h, ctypes.c_void_p(x_ptr), n, ctypes.c_void_p(y_ptr),
+                                        DEVICE, path))
+
+    # ---- two-phase form -------------------------------------------------------------------------
+    def act_create(self, q8_type: int, k: int, n_max: int) -> Act:
+        h = ctypes.c_void_p()
+        _check(lib().mi_qmm_act_create(self._h, q8_type, k, n_max, ctypes.byref(h)))
+        return Act(h, q8_type, k, n_max)
+
+    def act_quantize(self, act: Act, x, n: int | None = None, location: int = HOST):
+        """x: numpy f32 [n, k] (HOST) or a device address with n given (DEVICE)."""
+        if isinstance(x, np.ndarray):
+            x = np.ascontiguousarray(x, dtype=np.float32)
+            if x.ndim == 1:
+                x = x[None, :]
+            if x.shape[1] != act.k:
+                raise ValueError(f"x has k={x.shape[1]}, act has k={act.k}")
+            n = x.shape[0]
+        _check(lib().mi_qmm_act_quantize(self._h, act._h, _ptr(x), n, location))
+        act.n = n
+
+    def mulmat_q8(self, w: Weight, act: Act, path: int = PATH_AUTO) -> np.ndarray:
+        y = np.empty((act.n, w.m), dtype=np.float32)
+        _check(lib().mi_qmm_mulmat_q8(self._h, w._h, act._h, _ptr(y), HOST, path))
+        return y
+
+    def mulmat_q8_device(self, w: Weight, act: Act, y_ptr: int, path: int = PATH_AUTO):
+        _check(lib().mi_qmm_mulmat_q8(self._h, w._h, act._h, ctypes.c_void_p(y_ptr), DEVICE, path))

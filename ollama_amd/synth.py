@@ -1,0 +1,112 @@
+"""Synthetic GGUF weight blocks for benchmarks and smoke runs (numpy, host side, no GPU work).
+
+These are simple *valid* encoders -- round-to-nearest on a per-sub-block min/max grid -- not the
+iterative searches llama-quantize runs (make_qkx2_quants / make_qx_quants; reached in the product
+through /root/reference/server/quantization.go:125-181).  Any valid block exercises the matmul path
+identically: its cost and its arithmetic do not depend on how the scales were chosen.  Block layouts
+are the ones in csrc/formats.h.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
+
+
+def _f16_bytes(v: np.ndarray) -> np.ndarray:
+    return np.ascontiguousarray(v.astype("<f2")).view(np.uint8).reshape(v.shape + (2,))
+
+
+def encode_q8_0(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 32, 32)
+    d = np.abs(b).max(axis=2) / np.float32(127)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(d[..., None] > 0, np.rint(b / d[..., None]), 0).clip(-127, 127).astype(np.int8)
+    out = np.empty((m, k // 32, 34), np.uint8)
+    out[..., 0:2] = _f16_bytes(d)
+    out[..., 2:] = q.view(np.uint8)
+    return out.reshape(m, -1)
+
+
+def encode_q4_0(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 32, 32)
+    idx = np.abs(b).argmax(axis=2)
+    mx = np.take_along_axis(b, idx[..., None], axis=2)[..., 0]
+    d = mx / np.float32(-8)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(d[..., None] != 0, np.rint(b / d[..., None]) + 8, 8).clip(0, 15).astype(np.uint8)
+    out = np.empty((m, k // 32, 18), np.uint8)
+    out[..., 0:2] = _f16_bytes(d)
+    out[..., 2:] = q[..., :16] | (q[..., 16:] << 4)
+    return out.reshape(m, -1)
+
+
+def encode_q4_K(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 256, 8, 32)
+    lo = np.minimum(b.min(axis=3), 0)
+    scale = (b.max(axis=3) - lo) / np.float32(15)
+    mins = -lo
+    d = (scale.max(axis=2) / np.float32(63)).astype(np.float16)
+    dmin = (mins.max(axis=2) / np.float32(63)).astype(np.float16)
+    df, dmf = d.astype(np.float32), dmin.astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(df[..., None] > 0, np.rint(scale / df[..., None]), 0).clip(0, 63).astype(np.uint8)
+        mn = np.where(dmf[..., None] > 0, np.rint(mins / dmf[..., None]), 0).clip(0, 63).astype(np.uint8)
+        eff = df[..., None] * sc
+        q = np.where(eff[..., None] > 0, np.rint((b + (dmf[..., None] * mn)[..., None]) / eff[..., None]), 0)
+    q = q.clip(0, 15).astype(np.uint8)
+    out = np.zeros((m, k // 256, 144), np.uint8)
+    out[..., 0:2] = _f16_bytes(d)
+    out[..., 2:4] = _f16_bytes(dmin)
+    s = out[..., 4:16]
+    for j in range(4):
+        s[..., j] = (sc[..., j] & 63) | ((sc[..., j + 4] >> 4) << 6)
+        s[..., j + 4] = (mn[..., j] & 63) | ((mn[..., j + 4] >> 4) << 6)
+        s[..., j + 8] = (sc[..., j + 4] & 15) | ((mn[..., j + 4] & 15) << 4)
+    qq = q.reshape(m, k // 256, 4, 2, 32)
+    out[..., 16:] = (qq[..., 0, :] | (qq[..., 1, :] << 4)).reshape(m, k // 256, 128)
+    return out.reshape(m, -1)
+
+
+def encode_q6_K(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 256, 16, 16)
+    scale = np.abs(b).max(axis=3) / np.float32(31)
+    d = (scale.max(axis=2) / np.float32(127)).astype(np.float16)
+    df = d.astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(df[..., None] > 0, np.rint(scale / df[..., None]), 0).clip(0, 127).astype(np.int8)
+        eff = df[..., None] * sc
+        q = np.where(eff[..., None] > 0, np.rint(b / eff[..., None]), 0).clip(-32, 31)
+    e = (q + 32).astype(np.uint8).reshape(m, k // 256, 2, 4, 32)  # halves of 128, four runs of 32
+    out = np.empty((m, k // 256, 210), np.uint8)
+    ql = np.empty((m, k // 256, 2, 64), np.uint8)
+    ql[..., 0:32] = (e[..., 0, :] & 15) | ((e[..., 2, :] & 15) << 4)
+    ql[..., 32:64] = (e[..., 1, :] & 15) | ((e[..., 3, :] & 15) << 4)
+    qh = (e[..., 0, :] >> 4) | ((e[..., 1, :] >> 4) << 2) | ((e[..., 2, :] >> 4) << 4) | ((e[..., 3, :] >> 4) << 6)
+    out[..., 0:128] = ql.reshape(m, k // 256, 128)
+    out[..., 128:192] = qh.reshape(m, k // 256, 64)
+    out[..., 192:208] = sc.view(np.uint8)
+    out[..., 208:210] = _f16_bytes(d)
+    return out.reshape(m, -1)
+
+
+ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q6_K: encode_q6_K}
+
+
+def weights(ggml_type: int, m: int, k: int, seed: int, std: float = 0.02, chunk_rows: int = 2048) -> np.ndarray:
+    """N(0, std) weights drawn from ``seed`` and encoded to ``ggml_type``: uint8 [m, row_size]."""
+    rng = np.random.default_rng(seed)
+    enc = ENCODERS[ggml_type]
+    parts = []
+    for r0 in range(0, m, chunk_rows):
+        r = min(chunk_rows, m - r0)
+        parts.append(enc(rng.standard_normal((r, k), dtype=np.float32) * np.float32(std)))
+    return np.concatenate(parts, axis=0)

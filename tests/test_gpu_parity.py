@@ -1,0 +1,229 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same inputs.
+
+Bars: quantized activation bytes bit-exact; fp32 outputs within 1e-3 on
+|y-ref| / max(|ref|, 1e-2*rms(ref))  (see npref.rel_err for why the floor is 1% of the RMS).
+"""
+import numpy as np
+import pytest
+
+import npref
+import oracle
+from npref import Q4_0, Q4_K, Q6_K, Q8_0, Q8_K
+from ollama_amd import qmm
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+WTYPES = [Q4_0, Q8_0, Q4_K, Q6_K]
+NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = qmm.Context(0)
+    yield c
+    c.close()
+
+
+def _weights(t, m, k, seed, nthreads=16):
+    rng = np.random.default_rng(seed)
+    return oracle.quantize(t, (rng.standard_normal((m, k), dtype=np.float32) * np.float32(0.02)), nthreads=nthreads)
+
+
+# ---- kernel 1: activation quantization, bit-exact ---------------------------------------------
+@pytest.mark.parametrize("qt", [Q8_0, Q8_K])
+@pytest.mark.parametrize("n,k", [(1, 256), (1, 4096), (3, 1024), (8, 4096), (1, 14336), (512, 4096), (5, 14336)])
+def test_quantize_act_bit_exact(ctx, qt, n, k):
+    rng = np.random.default_rng(n * 100003 + k + qt)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.quantize_act(qt, x)
+    want = oracle.quantize(qt, x, nthreads=8)
+    assert got.shape == want.shape
+    assert np.array_equal(got, want), f"{np.count_nonzero(got != want)} bytes differ"
+
+
+@pytest.mark.parametrize("qt", [Q8_0, Q8_K])
+def test_quantize_act_edge_cases_bit_exact(ctx, qt):
+    rng = np.random.default_rng(99)
+    k = 1024
+    rows = []
+    rows.append(np.zeros(k, np.float32))                                   # all-zero blocks
+    r = np.zeros(k, np.float32); r[3] = 5.0; r[9] = -5.0; r[300] = -7.0; r[301] = 7.0   # ties, first wins
+    rows.append(r)
+    rows.append(np.full(k, -0.3, np.float32))                              # constant
+    rows.append((np.arange(k, dtype=np.float32) - 512))                    # ramp with exact halves
+    r = np.zeros(k, np.float32); r[::32] = 127; r[1::32] = 2.5; r[2::32] = -2.5; r[3::32] = 0.5
+    rows.append(r)                                                         # x*id = k+0.5: roundf vs rint
+    rows.append(rng.standard_normal(k).astype(np.float32) * np.float32(1e-30))   # tiny
+    rows.append(rng.standard_normal(k).astype(np.float32) * np.float32(1e20))    # huge
+    rows.append(rng.standard_normal(k).astype(np.float32) * np.float32(3e4))
+    r = rng.standard_normal(k).astype(np.float32); r[:256] = 0; r[512:544] = 0    # zero blocks among live ones
+    rows.append(r)
+    rows.append(np.round(rng.standard_normal(k) * 40).astype(np.float32) / 2)    # many exact .5 products
+    x = np.stack(rows)
+    got = ctx.quantize_act(qt, x)
+    want = oracle.quantize(qt, x)
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, f"first differing (row, byte): {bad[:5].tolist()}"
+
+
+def test_quantize_act_empty_and_errors(ctx):
+    assert ctx.quantize_act(Q8_K, np.zeros((0, 256), np.float32)).shape == (0, 292)
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.quantize_act(Q8_K, np.zeros((1, 100), np.float32))
+    assert e.value.code == qmm.ERR_INVALID
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.quantize_act(9, np.zeros((1, 32), np.float32))
+    assert e.value.code == qmm.ERR_UNSUPPORTED
+
+
+# ---- kernels 2/4: GEMV, small and ragged shapes ---------------------------------------------------
+SMALL = [(256, 1), (256, 7), (512, 33), (1024, 100), (2048, 64), (2304, 5), (4096, 257), (6144, 31), (14336, 19)]
+
+
+@pytest.mark.parametrize("t", WTYPES)
+@pytest.mark.parametrize("k,m", SMALL)
+def test_gemv_small_shapes(ctx, t, k, m):
+    w_raw = _weights(t, m, k, seed=k * 31 + m + t)
+    W = ctx.upload(t, w_raw, k, m)
+    rng = np.random.default_rng(k + m)
+    for n in (1, 2, 3, 8):
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        got = ctx.mulmat(W, x, path=qmm.PATH_GEMV)
+        want = oracle.mul_mat(t, w_raw, k, m, x, nthreads=8)
+        assert got.shape == (n, m)
+        err = npref.rel_err(got, want)
+        assert err <= TOL, f"{NAMES[t]} k={k} m={m} n={n}: rel err {err}"
+    W.free()
+
+
+@pytest.mark.parametrize("t", WTYPES)
+def test_gemv_every_column_count_and_groups(ctx, t):
+    k, m = 1024, 96
+    w_raw = _weights(t, m, k, seed=7 + t)
+    W = ctx.upload(t, w_raw, k, m)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((19, k), dtype=np.float32)
+    want = oracle.mul_mat(t, w_raw, k, m, x, nthreads=8)
+    for n in list(range(1, 10)) + [16, 17, 19]:   # > 8 runs in column groups of 8
+        got = ctx.mulmat(W, x[:n], path=qmm.PATH_GEMV)
+        assert npref.rel_err(got, want[:n]) <= TOL, n
+    W.free()
+
+
+@pytest.mark.parametrize("t", WTYPES)
+def test_gemv_random_block_bytes(ctx, t):
+    """weights made of random bytes reach every bit pattern of nibbles, 6-bit scales and high bits"""
+    rng = np.random.default_rng(1234 + t)
+    k, m = 2048, 40
+    nb = m * k // npref.BLOCK[t]
+    raw = rng.integers(0, 256, (nb, npref.BYTES[t]), dtype=np.uint8)
+    h = np.abs(rng.standard_normal(nb * 2) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 4)
+    if t in (Q4_0, Q8_0):
+        raw[:, 0:2] = h[:, 0:2]
+    elif t == Q4_K:
+        raw[:, 0:4] = h
+    else:
+        raw[:, 208:210] = h[:, 0:2]
+    W = ctx.upload(t, raw.reshape(-1), k, m)
+    x = rng.standard_normal((4, k), dtype=np.float32)
+    got = ctx.mulmat(W, x, path=qmm.PATH_GEMV)
+    want = oracle.mul_mat(t, raw.reshape(-1), k, m, x, nthreads=8)
+    assert npref.rel_err(got, want) <= TOL
+    # and against exact arithmetic: no worse than the oracle's own rounding noise by much
+    xq = oracle.quantize(oracle.vec_dot_type(t), x)
+    exact = npref.matmul_f64(t, raw.reshape(-1), k, m, oracle.vec_dot_type(t), xq, 4)
+    assert npref.rel_err(got, exact) <= TOL
+    W.free()
+
+
+def test_mulmat_linearity_in_weights_rows(ctx):
+    """size-independent property: rows are independent -- a row-permuted weight gives permuted outputs"""
+    t, k, m = Q4_K, 4096, 512
+    w_raw = _weights(t, m, k, seed=21)
+    perm = np.random.default_rng(3).permutation(m)
+    x = np.random.default_rng(4).standard_normal((2, k), dtype=np.float32)
+    W1 = ctx.upload(t, w_raw, k, m)
+    W2 = ctx.upload(t, w_raw[perm], k, m)
+    y1, y2 = ctx.mulmat(W1, x), ctx.mulmat(W2, x)
+    assert np.array_equal(y1[:, perm], y2)  # bit-identical: same lanes, same order per row
+    W1.free(); W2.free()
+
+
+# ---- the benchmark configurations at full size -----------------------------------------------------
+def _config_case(ctx, t, m, k, ns, seed_w, seed_x):
+    w_raw = _weights(t, m, k, seed=seed_w)
+    W = ctx.upload(t, w_raw, k, m)
+    assert W.gguf_bytes == w_raw.size
+    rng = np.random.default_rng(seed_x)
+    for n in ns:
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        got = ctx.mulmat(W, x)
+        want = oracle.mul_mat(t, w_raw, k, m, x, nthreads=16)
+        err = npref.rel_err(got, want)
+        nrm = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
+        assert err <= TOL, f"{NAMES[t]} {m}x{k} n={n}: rel err {err}, normwise {nrm}"
+        assert nrm <= 1e-5
+    W.free()
+
+
+def test_config1_q4_0_gemv(ctx):
+    _config_case(ctx, Q4_0, 4096, 4096, [1], 1001, 2001)
+
+
+def test_config2_q8_0_skinny(ctx):
+    _config_case(ctx, Q8_0, 4096, 4096, [1, 2, 4, 8], 1002, 2002)
+
+
+def test_config3_q4_K_ffn_gate_up(ctx):
+    _config_case(ctx, Q4_K, 14336, 4096, [1], 1003, 2003)
+
+
+def test_config3_q4_K_ffn_down(ctx):
+    _config_case(ctx, Q4_K, 4096, 14336, [1], 1003, 2013)
+
+
+def test_config4_q6_K_output_head(ctx):
+    _config_case(ctx, Q6_K, 128256, 4096, [1, 8], 1004, 2004)
+
+
+# ---- error behaviour -------------------------------------------------------------------------------------
+def test_upload_and_mulmat_errors(ctx):
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.upload(13, np.zeros(176, np.uint8), 256, 1)      # Q5_K is not on this path
+    assert e.value.code == qmm.ERR_UNSUPPORTED
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.upload(Q4_0, np.zeros(18, np.uint8), 31, 1)      # row not a multiple of the block
+    assert e.value.code == qmm.ERR_INVALID
+    W = ctx.upload(Q4_K, np.zeros(144, np.uint8), 256, 1)
+    with pytest.raises(ValueError):
+        ctx.mulmat(W, np.zeros((1, 512), np.float32))
+    assert ctx.mulmat(W, np.zeros((0, 256), np.float32)).shape == (0, 1)
+    assert not ctx.mulmat(W, np.ones((2, 256), np.float32)).any()   # zero weights -> zero outputs
+    W.free()
+
+
+# ---- two-phase form: quantize once, multiply by several weights --------------------------------------
+def test_two_phase_matches_fused(ctx):
+    k = 4096
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((3, k), dtype=np.float32)
+    act = ctx.act_create(Q8_K, k, 8)
+    ctx.act_quantize(act, x)
+    for t, m in ((Q4_K, 300), (Q6_K, 129)):
+        w_raw = _weights(t, m, k, seed=m)
+        W = ctx.upload(t, w_raw, k, m)
+        assert np.array_equal(ctx.mulmat_q8(W, act), ctx.mulmat(W, x))
+        W.free()
+    # a smaller batch afterwards reuses the same storage
+    ctx.act_quantize(act, x[:1])
+    w_raw = _weights(Q4_K, 64, k, seed=9)
+    W = ctx.upload(Q4_K, w_raw, k, 64)
+    assert np.array_equal(ctx.mulmat_q8(W, act), ctx.mulmat(W, x[:1]))
+    # type / shape mismatches are rejected
+    W8 = ctx.upload(Q8_0, _weights(Q8_0, 8, k, seed=1), k, 8)
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_q8(W8, act)
+    assert e.value.code == qmm.ERR_INVALID
+    with pytest.raises(qmm.QmmError):
+        ctx.act_quantize(act, np.zeros((9, k), np.float32))   # more rows than n_max
+    W.free(); W8.free(); act.free()
