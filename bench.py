@@ -63,7 +63,10 @@ def main() -> int:
     torch.cuda.set_device(dev)
     ctx = qmm.Context(0)
     info = ctx.device_info()
-    stream = torch.cuda.current_stream()
+    # a real (non-null) stream: the library launches on it and the HIP events below are recorded on it
+    stream = torch.cuda.Stream(device=dev)
+    torch.cuda.set_stream(stream)
+    assert stream.cuda_stream != 0
     ctx.set_stream(stream.cuda_stream)
 
     # ---- synthetic weights: one encoded FFN, the other pool entries are row-rotated copies
@@ -176,7 +179,7 @@ def main() -> int:
         xh = x.cpu().numpy()
         reps, t_cpu = 0, 0.0
         t_begin = time.time()
-        while t_cpu < args.cpu_seconds and reps < 1000:
+        while t_cpu < args.cpu_seconds:
             t1 = time.time()
             oracle.mul_mat(Q4_K, base["gate"], FFN_K, FFN_M, xh, nthreads=threads)
             t_cpu += time.time() - t1

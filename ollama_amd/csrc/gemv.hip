@@ -6,16 +6,20 @@
 // /root/reference/ml/backend.go:151, for batch <= 8.
 //
 // Shape of the computation (HBM-bound: every weight byte is read exactly once):
-//   * A wavefront owns a fixed slice of K ("segment": 2048 elements, 1024 for Q8_0) and walks down
-//     the rows.  Each lane's piece of every row is one aligned 16-byte load, consecutive lanes read
-//     consecutive 16-byte pieces, so a wave reads 1 KiB runs of the row.
+//   * A wavefront owns a fixed slice of K (a "segment": 4096 elements for the K-quants, 2048 for
+//     Q4_0, 1024 for Q8_0) and walks down the rows.  A lane's piece of a row is one or two aligned
+//     16-byte loads and the wave as a whole reads a contiguous run of the row.
 //   * Because the lane's K positions never change, its Q8 activation quants (and the block scale and
 //     partial sums that go with them) are loaded ONCE into registers and reused for every row: the
-//     inner loop reads nothing but weights.
+//     inner loop reads nothing but weights.  Those loads are issued before the first weight loads:
+//     the memory counter retires in order, so anything issued after the weights could only be waited
+//     for by draining every weight load as well.
 //   * Nibbles / 6-bit values are unpacked in registers, multiplied with v_dot4_i32_i8, the sub-block
-//     scales applied in-lane, and the lane partials reduced across the wave; waves that own different
-//     K segments of the same rows combine through LDS at the end of the workgroup.
-//   * U rows are in flight per wave (all loads issued before the first use) to cover HBM latency.
+//     scales applied in-lane.  The U rows of a pass are reduced across the wave together (the
+//     lane-index bits that are summed over select which row a lane keeps), and waves that own
+//     different K segments of the same rows combine through LDS at the end of the workgroup.
+//   * Rows are processed in passes of U with two register buffers, so up to 2U rows per wave are in
+//     flight; for the FFN shapes that is every row the wave owns, i.e. one exposed HBM latency.
 #include <hip/hip_fp16.h>
 
 #include "internal.h"
@@ -32,13 +36,42 @@ __device__ __forceinline__ float h2f(unsigned int bits16) {
     return __half2float(__ushort_as_half((unsigned short)bits16));
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+__device__ __forceinline__ uint4 ld16(const uint8_t *p) { return *reinterpret_cast<const uint4 *>(p); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
 
-__device__ __forceinline__ uint4 ld16(const uint8_t *p) { return *reinterpret_cast<const uint4 *>(p); }
+// Reduce U per-lane values over the 64 lanes at once.  On return every lane whose (lane & (U-1))
+// equals u holds the total of v[u].  The xor-1 / xor-2 exchange steps double as the transposition:
+// a lane keeps the value of "its" row and hands the other one to its partner.
+template <int U>
+__device__ __forceinline__ float reduce_rows(const float (&v)[U], int lane) {
+    float w;
+    if (U == 4) {
+        const bool b0 = lane & 1, b1 = lane & 2;
+        const float k01 = b0 ? v[1] : v[0], g01 = b0 ? v[0] : v[1];
+        const float k23 = b0 ? v[3] : v[2], g23 = b0 ? v[2] : v[3];
+        const float s01 = k01 + dpp_mov<0xB1>(g01);  // quad_perm [1,0,3,2]: lane ^ 1
+        const float s23 = k23 + dpp_mov<0xB1>(g23);
+        const float k = b1 ? s23 : s01, g = b1 ? s01 : s23;
+        w = k + dpp_mov<0x4E>(g);                    // quad_perm [2,3,0,1]: lane ^ 2
+    } else if (U == 2) {
+        const bool b0 = lane & 1;
+        const float k = b0 ? v[1] : v[0], g = b0 ? v[0] : v[1];
+        w = k + dpp_mov<0xB1>(g);
+        w += dpp_mov<0x4E>(w);
+    } else {
+        w = v[0] + dpp_mov<0xB1>(v[0]);
+        w += dpp_mov<0x4E>(w);
+    }
+    w += dpp_mov<0x124>(w);  // row_ror:4  -- the other quads of the row of 16; keeps lane & 3
+    w += dpp_mov<0x128>(w);  // row_ror:8
+    w += __shfl_xor(w, 16);
+    w += __shfl_xor(w, 32);
+    return w;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Per-type policies.  Each provides
@@ -47,78 +80,82 @@ __device__ __forceinline__ uint4 ld16(const uint8_t *p) { return *reinterpret_ca
 //   Act                      per-lane, per-column activation registers
 //   Raw                      the lane's loaded weight bytes for one row
 //   geo(), load_act(), load(), dot()
-// A lane whose K slice lies beyond K (ragged last segment) is "dead": its activation registers are
-// zero and its weight loads are redirected to the start of the row, so it contributes exactly 0.
+// A lane whose K slice lies beyond K (ragged last segment) is "dead": it loads nothing, its weight
+// and activation registers are zero, and it contributes exactly 0.
 // ---------------------------------------------------------------------------------------------
 
 struct PolQ4K {
-    static constexpr int SEG = 2048;  // 8 super-blocks, 8 lanes each
+    static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
+    static constexpr bool HEAVY = true;
+    // lane c (0..3) of a super-block owns qs bytes [32c, 32c+32): low nibbles are sub-block 2c,
+    // high nibbles sub-block 2c+1 (32 elements each), and with them scales/mins 2c and 2c+1.
     struct Geo {
         int64_t row_bytes;
-        int off;      // byte offset of the lane's super-block in the row
-        int l8;       // lane within the super-block: chunk c = l8>>1 (32 qs bytes), half = l8&1
-        int sh16;     // 16*(c&1): position of the (sc[2c], sc[2c+1]) pair inside a scales word
-        int sh8;      // 8*(l8&3): position of m[l8] inside a scales word
+        int off;    // byte offset of the lane's super-block in the row
+        int qoff;   // byte offset of the lane's 32 qs bytes in the row
+        int sh;     // 16*(c&1): where the (2c, 2c+1) byte pair sits inside a scales word
+        bool hi;    // c >= 2: sub-blocks 4..7 use the split 4+2 bit packing
         bool live;
     };
-    struct Act { int q[8]; float d; int s; };
-    struct Raw { uint4 hdr, qv; };
+    struct Act { int lo[8], hi[8]; float d; int s_lo, s_hi; };
+    struct Raw { uint4 hdr, q0, q1; };
 
     static __device__ __forceinline__ Geo geo(const DevWeight &w, int seg, int lane) {
         Geo g;
-        const int sb = seg * 8 + (lane >> 3);
+        const int sb = seg * 16 + (lane >> 2), c = lane & 3;
         g.row_bytes = w.K / QKK * Q4_K_BYTES;
         g.live = (int64_t)sb * QKK < w.K;
-        g.off = g.live ? sb * Q4_K_BYTES : 0;
-        g.l8 = lane & 7;
-        g.sh16 = 16 * ((g.l8 >> 1) & 1);
-        g.sh8 = 8 * (g.l8 & 3);
+        g.off = sb * Q4_K_BYTES;
+        g.qoff = g.off + 16 + 32 * c;
+        g.sh = 16 * (c & 1);
+        g.hi = c >= 2;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        const int sb = seg * 8 + (lane >> 3);
-        const int c = g.l8 >> 1, half = g.l8 & 1;
-        if (!g.live) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) r.q[i] = 0;
-            r.d = 0.f; r.s = 0;
-            return;
+        const int sb = seg * 16 + (lane >> 2), c = lane & 3;
+        int4 v[4] = {};
+        float dd = 0.f;
+        int b0 = 0, b1 = 0, b2 = 0, b3 = 0;
+        if (g.live) {
+            const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)sb * QKK + 64 * c);
+            v[0] = q[0]; v[1] = q[1]; v[2] = q[2]; v[3] = q[3];
+            dd = a.d[(int64_t)n * (a.K / QKK) + sb];
+            const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)sb * 16 + 4 * c;
+            b0 = bs[0]; b1 = bs[1]; b2 = bs[2]; b3 = bs[3];
         }
-        // low nibbles of the lane's 16 qs bytes are elements 64c+16*half.. of sub-block 2c,
-        // high nibbles the same offsets of sub-block 2c+1 (32 elements further)
-        const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)sb * QKK + 64 * c + 16 * half;
-        const int4 lo = *reinterpret_cast<const int4 *>(q), hi = *reinterpret_cast<const int4 *>(q + 32);
-        r.q[0] = lo.x; r.q[1] = lo.y; r.q[2] = lo.z; r.q[3] = lo.w;
-        r.q[4] = hi.x; r.q[5] = hi.y; r.q[6] = hi.z; r.q[7] = hi.w;
-        r.d = a.d[(int64_t)n * (a.K / QKK) + sb];
-        const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)sb * 16 + 2 * g.l8;
-        r.s = (int)bs[0] + (int)bs[1];  // sum of q8 over sub-block l8 (the lane owns min l8)
+        r.lo[0] = v[0].x; r.lo[1] = v[0].y; r.lo[2] = v[0].z; r.lo[3] = v[0].w;
+        r.lo[4] = v[1].x; r.lo[5] = v[1].y; r.lo[6] = v[1].z; r.lo[7] = v[1].w;
+        r.hi[0] = v[2].x; r.hi[1] = v[2].y; r.hi[2] = v[2].z; r.hi[3] = v[2].w;
+        r.hi[4] = v[3].x; r.hi[5] = v[3].y; r.hi[6] = v[3].z; r.hi[7] = v[3].w;
+        r.d = dd;
+        r.s_lo = b0 + b1;  // sum of q8 over sub-block 2c
+        r.s_hi = b2 + b3;  // ... and 2c+1
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        const uint8_t *p = w.p0 + row * g.row_bytes + g.off;
-        Raw r;
-        r.hdr = ld16(p);
-        r.qv = ld16(p + 16 + 16 * g.l8);
+        Raw r = {};
+        if (g.live) {
+            const uint8_t *p = w.p0 + row * g.row_bytes;
+            r.hdr = ld16(p + g.off);
+            r.q0 = ld16(p + g.qoff);
+            r.q1 = ld16(p + g.qoff + 16);
+        }
         return r;
     }
     template <int NC>
     static __device__ __forceinline__ void dot(const Raw &r, const Geo &g, const Act (&a)[NC], float (&acc)[NC]) {
         // hdr.x = d | dmin<<16 ; hdr.y = scales[0..3] ; hdr.z = scales[4..7] ; hdr.w = scales[8..11]
         const float dw = h2f(r.hdr.x & 0xffff), dminw = h2f(r.hdr.x >> 16);
-        // (sc[2c], sc[2c+1]) as two bytes
-        const unsigned t0 = r.hdr.y >> g.sh16, t2 = r.hdr.w >> g.sh16;
-        const unsigned pairA = t0 & 0x3f3fu;
-        const unsigned pairB = (t2 & 0x0f0fu) | ((t0 >> 2) & 0x3030u);
-        const unsigned pair = (g.l8 < 4) ? pairA : pairB;
-        const int sc_lo = pair & 0xff, sc_hi = pair >> 8;
-        // m[l8]
-        const unsigned ma = r.hdr.z >> g.sh8, mb = r.hdr.w >> g.sh8;
-        const int mA = ma & 63, mB = ((mb >> 4) & 0xf) | ((ma >> 2) & 0x30);
-        const int mn = (g.l8 < 4) ? mA : mB;
-        const unsigned v[4] = {r.qv.x, r.qv.y, r.qv.z, r.qv.w};
-        int lo[4], hi[4];
+        const unsigned ty = r.hdr.y >> g.sh, tz = r.hdr.z >> g.sh, tw = r.hdr.w >> g.sh;
+        // byte pairs (sc[2c], sc[2c+1]) and (m[2c], m[2c+1])
+        const unsigned scA = ty & 0x3f3fu, mA = tz & 0x3f3fu;
+        const unsigned scB = (tw & 0x0f0fu) | ((ty >> 2) & 0x3030u);
+        const unsigned mB = ((tw >> 4) & 0x0f0fu) | ((tz >> 2) & 0x3030u);
+        const unsigned scp = g.hi ? scB : scA, mp = g.hi ? mB : mA;
+        const int sc_lo = scp & 0xff, sc_hi = scp >> 8, m_lo = mp & 0xff, m_hi = mp >> 8;
+        const unsigned v[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        int lo[8], hi[8];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < 8; i++) {
             lo[i] = (int)(v[i] & 0x0f0f0f0fu);
             hi[i] = (int)((v[i] >> 4) & 0x0f0f0f0fu);
         }
@@ -126,49 +163,54 @@ struct PolQ4K {
         for (int n = 0; n < NC; n++) {
             int dl = 0, dh = 0;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                dl = dot4(lo[i], a[n].q[i], dl);
-                dh = dot4(hi[i], a[n].q[4 + i], dh);
+            for (int i = 0; i < 8; i++) {
+                dl = dot4(lo[i], a[n].lo[i], dl);
+                dh = dot4(hi[i], a[n].hi[i], dh);
             }
             const int isum = __mul24(sc_lo, dl) + __mul24(sc_hi, dh);
-            acc[n] += (dw * a[n].d) * (float)isum - (dminw * a[n].d) * (float)__mul24(mn, a[n].s);
+            const int msum = __mul24(m_lo, a[n].s_lo) + __mul24(m_hi, a[n].s_hi);
+            acc[n] = __builtin_fmaf(dw * a[n].d, (float)isum, acc[n]);
+            acc[n] = __builtin_fmaf(-(dminw * a[n].d), (float)msum, acc[n]);
         }
     }
 };
 
 struct PolQ4_0 {
     static constexpr int SEG = 2048;  // 64 blocks, one per lane
+    static constexpr bool HEAVY = false;
     struct Geo { int64_t qrow, drow; int blk; bool live; };
     struct Act { int q[8]; float d; int s8; };
-    struct Raw { uint4 qv; unsigned short dh; };
+    struct Raw { uint4 qv; unsigned dh; };
 
     static __device__ __forceinline__ Geo geo(const DevWeight &w, int seg, int lane) {
         Geo g;
-        const int blk = seg * 64 + lane;
-        g.live = (int64_t)blk * QK < w.K;
-        g.blk = g.live ? blk : 0;
+        g.blk = seg * 64 + lane;
+        g.live = (int64_t)g.blk * QK < w.K;
         g.qrow = w.K / 2;
         g.drow = w.K / QK;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        if (!g.live) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) r.q[i] = 0;
-            r.d = 0.f; r.s8 = 0;
-            return;
+        int4 lo = {}, hi = {};
+        float dd = 0.f;
+        int s = 0;
+        if (g.live) {
+            const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.blk * QK);
+            lo = q[0]; hi = q[1];
+            dd = a.d[(int64_t)n * (a.K / QK) + g.blk];
+            s = a.bsums[(int64_t)n * (a.K / QK) + g.blk];
         }
-        const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)g.blk * QK;
-        const int4 lo = *reinterpret_cast<const int4 *>(q), hi = *reinterpret_cast<const int4 *>(q + 16);
         r.q[0] = lo.x; r.q[1] = lo.y; r.q[2] = lo.z; r.q[3] = lo.w;
         r.q[4] = hi.x; r.q[5] = hi.y; r.q[6] = hi.z; r.q[7] = hi.w;
-        r.d = a.d[(int64_t)n * (a.K / QK) + g.blk];
-        r.s8 = 8 * (int)a.bsums[(int64_t)n * (a.K / QK) + g.blk];
+        r.d = dd;
+        r.s8 = 8 * s;
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r;
-        r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.blk * 16);
-        r.dh = w.d[row * g.drow + g.blk];
+        Raw r = {};
+        if (g.live) {
+            r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.blk * 16);
+            r.dh = w.d[row * g.drow + g.blk];
+        }
         return r;
     }
     template <int NC>
@@ -196,32 +238,35 @@ struct PolQ4_0 {
 
 struct PolQ8_0 {
     static constexpr int SEG = 1024;  // 32 blocks, two lanes (16 quants each) per block
+    static constexpr bool HEAVY = false;
     struct Geo { int64_t qrow, drow; int hb; bool live; };
     struct Act { int q[4]; float d; };
-    struct Raw { uint4 qv; unsigned short dh; };
+    struct Raw { uint4 qv; unsigned dh; };
 
     static __device__ __forceinline__ Geo geo(const DevWeight &w, int seg, int lane) {
         Geo g;
-        const int hb = seg * 64 + lane;  // half-block index along the row
-        g.live = (int64_t)hb * 16 < w.K;
-        g.hb = g.live ? hb : 0;
+        g.hb = seg * 64 + lane;  // half-block index along the row
+        g.live = (int64_t)g.hb * 16 < w.K;
         g.qrow = w.K;
         g.drow = w.K / QK;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        if (!g.live) {
-            r.q[0] = r.q[1] = r.q[2] = r.q[3] = 0; r.d = 0.f;
-            return;
+        int4 v = {};
+        float dd = 0.f;
+        if (g.live) {
+            v = *reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.hb * 16);
+            dd = a.d[(int64_t)n * (a.K / QK) + (g.hb >> 1)];
         }
-        const int4 v = *reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.hb * 16);
         r.q[0] = v.x; r.q[1] = v.y; r.q[2] = v.z; r.q[3] = v.w;
-        r.d = a.d[(int64_t)n * (a.K / QK) + (g.hb >> 1)];
+        r.d = dd;
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r;
-        r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.hb * 16);
-        r.dh = w.d[row * g.drow + (g.hb >> 1)];
+        Raw r = {};
+        if (g.live) {
+            r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.hb * 16);
+            r.dh = w.d[row * g.drow + (g.hb >> 1)];
+        }
         return r;
     }
     template <int NC>
@@ -239,80 +284,92 @@ struct PolQ8_0 {
 };
 
 struct PolQ6K {
-    static constexpr int SEG = 2048;  // 8 super-blocks, 8 lanes each
-    // lane (h = l8>>2, t = l8&3) of a super-block reads ql bytes [64h+16t, +16): their low nibbles are
-    // elements 128h + eo + i, their high nibbles elements 128h + eo + 64 + i, eo = 16(t&1) + 32(t>>1);
-    // the two high bits come from qh bytes [32h + 16(t&1), +16) at bit 2(t>>1) (low) and +4 (high).
-    struct Geo {
-        int64_t lrow, hrow, srow, drow;
-        int sb, loff, hoff, soff;
-        int shl;  // 4 - 2(t>>1): left shift that brings the low element's 2 bits to bit 4
-        int shr;  // 2(t>>1):     right shift that brings the high element's 2 bits to bit 4
-        bool live;
-    };
-    struct Act { int q[8]; float d; int s_lo, s_hi; };
-    struct Raw { uint4 ql, qh; int sc_lo, sc_hi; unsigned short dh; };
+    static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
+    static constexpr bool HEAVY = true;
+    // lane (h = l4>>1, t = l4&1) of a super-block owns, in half h (128 elements):
+    //   ql bytes [64h+16t, +16) and [64h+32+16t, +16), qh bytes [32h+16t, +16)
+    // which hold four runs of 16 elements e = 128h + 16t + 32r + i (r = 0..3):
+    //   r=0: low nibbles of the first ql piece,  high bits qh>>0
+    //   r=1: low nibbles of the second ql piece, high bits qh>>2
+    //   r=2: high nibbles of the first piece,    high bits qh>>4
+    //   r=3: high nibbles of the second piece,   high bits qh>>6
+    // each run is one 16-element scale group: scales[8h + t + 2r].
+    struct Geo { int64_t lrow, hrow, srow, drow; int sb, loff, hoff, soff, e0, sh; bool live; };
+    struct Act { int q[4][4]; float d; int s32[4]; };
+    struct Raw { uint4 l0, l1, qh; uint2 sc8; unsigned dh; };
 
     static __device__ __forceinline__ Geo geo(const DevWeight &w, int seg, int lane) {
         Geo g;
-        const int sb = seg * 8 + (lane >> 3), l8 = lane & 7, h = l8 >> 2, t = l8 & 3;
-        g.live = (int64_t)sb * QKK < w.K;
-        g.sb = g.live ? sb : 0;
+        const int l4 = lane & 3, h = l4 >> 1, t = l4 & 1;
+        g.sb = seg * 16 + (lane >> 2);
+        g.live = (int64_t)g.sb * QKK < w.K;
         g.lrow = w.K / 2; g.hrow = w.K / 4; g.srow = w.K / 16; g.drow = w.K / QKK;
         g.loff = g.sb * 128 + 64 * h + 16 * t;
-        g.hoff = g.sb * 64 + 32 * h + 16 * (t & 1);
-        g.soff = g.sb * 16 + 8 * h + t;
-        g.shl = 4 - 2 * (t >> 1);
-        g.shr = 2 * (t >> 1);
+        g.hoff = g.sb * 64 + 32 * h + 16 * t;
+        g.soff = g.sb * 16 + 8 * h;  // the half's 8 scale bytes; the lane uses bytes t, t+2, t+4, t+6
+        g.sh = 8 * t;
+        g.e0 = 128 * h + 16 * t;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        // dead lanes read super-block 0 (always present) and zero what they read
-        const int l8 = lane & 7, h = l8 >> 2, t = l8 & 3;
-        const int e0 = 128 * h + 16 * (t & 1) + 32 * (t >> 1);
-        const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)g.sb * QKK + e0;
-        const int4 lo = *reinterpret_cast<const int4 *>(q), hi = *reinterpret_cast<const int4 *>(q + 64);
-        const int keep = g.live ? -1 : 0;
-        r.q[0] = lo.x & keep; r.q[1] = lo.y & keep; r.q[2] = lo.z & keep; r.q[3] = lo.w & keep;
-        r.q[4] = hi.x & keep; r.q[5] = hi.y & keep; r.q[6] = hi.z & keep; r.q[7] = hi.w & keep;
-        const float dd = a.d[(int64_t)n * (a.K / QKK) + g.sb];
-        r.d = g.live ? dd : 0.f;
-        const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)g.sb * 16 + (e0 >> 4);
-        const int b0 = bs[0], b4 = bs[4];
-        r.s_lo = (32 * b0) & keep;
-        r.s_hi = (32 * b4) & keep;
+        int4 v[4] = {};
+        float dd = 0.f;
+        int b[4] = {0, 0, 0, 0};
+        if (g.live) {
+            const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)g.sb * QKK + g.e0;
+            const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)g.sb * 16 + (g.e0 >> 4);
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                v[rr] = *reinterpret_cast<const int4 *>(q + 32 * rr);
+                b[rr] = bs[2 * rr];
+            }
+            dd = a.d[(int64_t)n * (a.K / QKK) + g.sb];
+        }
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            r.q[rr][0] = v[rr].x; r.q[rr][1] = v[rr].y; r.q[rr][2] = v[rr].z; r.q[rr][3] = v[rr].w;
+            r.s32[rr] = 32 * b[rr];
+        }
+        r.d = dd;
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r;
-        r.ql = ld16(w.p0 + row * g.lrow + g.loff);
-        r.qh = ld16(w.p1 + row * g.hrow + g.hoff);
-        const int8_t *sc = reinterpret_cast<const int8_t *>(w.p2) + row * g.srow + g.soff;
-        r.sc_lo = sc[0];
-        r.sc_hi = sc[4];
-        r.dh = w.d[row * g.drow + g.sb];
+        Raw r = {};
+        if (g.live) {
+            const uint8_t *pl = w.p0 + row * g.lrow + g.loff;
+            r.l0 = ld16(pl);
+            r.l1 = ld16(pl + 32);
+            r.qh = ld16(w.p1 + row * g.hrow + g.hoff);
+            r.sc8 = *reinterpret_cast<const uint2 *>(w.p2 + row * g.srow + g.soff);
+            r.dh = w.d[row * g.drow + g.sb];
+        }
         return r;
     }
     template <int NC>
     static __device__ __forceinline__ void dot(const Raw &r, const Geo &g, const Act (&a)[NC], float (&acc)[NC]) {
         const float dw = h2f(r.dh);
-        const unsigned l[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w};
+        const int sc[4] = {(int)(int8_t)(r.sc8.x >> g.sh), (int)(int8_t)(r.sc8.x >> (g.sh + 16)),
+                           (int)(int8_t)(r.sc8.y >> g.sh), (int)(int8_t)(r.sc8.y >> (g.sh + 16))};
+        const unsigned l0[4] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w}, l1[4] = {r.l1.x, r.l1.y, r.l1.z, r.l1.w};
         const unsigned hq[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
-        int lo[4], hi[4];
+        int e[4][4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            lo[i] = (int)((l[i] & 0x0f0f0f0fu) | ((hq[i] << g.shl) & 0x30303030u));
-            hi[i] = (int)(((l[i] >> 4) & 0x0f0f0f0fu) | ((hq[i] >> g.shr) & 0x30303030u));
+            e[0][i] = (int)((l0[i] & 0x0f0f0f0fu) | ((hq[i] << 4) & 0x30303030u));
+            e[1][i] = (int)((l1[i] & 0x0f0f0f0fu) | ((hq[i] << 2) & 0x30303030u));
+            e[2][i] = (int)(((l0[i] >> 4) & 0x0f0f0f0fu) | (hq[i] & 0x30303030u));
+            e[3][i] = (int)(((l1[i] >> 4) & 0x0f0f0f0fu) | ((hq[i] >> 2) & 0x30303030u));
         }
 #pragma unroll
         for (int n = 0; n < NC; n++) {
-            int dl = -a[n].s_lo, dh = -a[n].s_hi;  // sum (q-32)*y = sum q*y - 32*sum y
+            int isum = 0;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                dl = dot4(lo[i], a[n].q[i], dl);
-                dh = dot4(hi[i], a[n].q[4 + i], dh);
+            for (int rr = 0; rr < 4; rr++) {
+                int s = -a[n].s32[rr];  // sum (q-32)*y = sum q*y - 32*sum y
+#pragma unroll
+                for (int i = 0; i < 4; i++) s = dot4(e[rr][i], a[n].q[rr][i], s);
+                isum += __mul24(sc[rr], s);
             }
-            const int isum = __mul24(r.sc_lo, dl) + __mul24(r.sc_hi, dh);
-            acc[n] += (dw * a[n].d) * (float)isum;
+            acc[n] = __builtin_fmaf(dw * a[n].d, (float)isum, acc[n]);
         }
     }
 };
@@ -320,143 +377,167 @@ struct PolQ6K {
 // ---------------------------------------------------------------------------------------------
 // The kernel.  Workgroup = KW x RW waves: wave (kseg, rg) owns K segments kseg, kseg+KW, ...
 // (SPW of them, held in registers) and rows r0+rg, r0+rg+RW, r0+rg+2RW, ... of the workgroup's row
-// range, U of them in flight at a time.  part[] (LDS) receives one partial per (row, column, kseg);
-// after a barrier the workgroup sums over kseg and stores y.
+// range.  With KW == 1 a wave's totals are final and go straight to y; otherwise part[] (LDS)
+// receives one partial per (row, column, kseg) and after a barrier the workgroup sums over kseg.
 // ---------------------------------------------------------------------------------------------
-template <class P, int NC, int SPW, int U>
-__device__ __forceinline__ void rows_step(const DevWeight &w, const typename P::Geo (&g)[SPW],
-                                          const typename P::Act (&act)[SPW][NC], int64_t r, int rw,
-                                          int64_t r0, int lane, int kseg, int kw, float *part) {
-    typename P::Raw raw[U][SPW];
-#pragma unroll
-    for (int u = 0; u < U; u++)
-#pragma unroll
-        for (int s = 0; s < SPW; s++) raw[u][s] = P::load(w, g[s], r + (int64_t)u * rw);
+template <class P, int SPW, int U>
+__device__ __forceinline__ void load_pass(const DevWeight &w, const typename P::Geo (&g)[SPW],
+                                          typename P::Raw (&raw)[U][SPW], int64_t rbase, int rw, int i0,
+                                          int nrw) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
-        float acc[NC];
+        const int i = min(i0 + u, nrw - 1);  // past the wave's last row: re-read it (dropped later)
 #pragma unroll
-        for (int n = 0; n < NC; n++) acc[n] = 0.f;
+        for (int s = 0; s < SPW; s++) raw[u][s] = P::load(w, g[s], rbase + (int64_t)i * rw);
+    }
+}
+
+template <class P, int NC, int SPW, int U, bool DIRECT>
+__device__ __forceinline__ void compute_pass(const typename P::Geo (&g)[SPW],
+                                             const typename P::Act (&act)[SPW][NC],
+                                             const typename P::Raw (&raw)[U][SPW], int rl0, int rw, int i0,
+                                             int nrw, int lane, int kseg, int kw, float *part, float *yrow0,
+                                             int64_t ldy) {
+    float acc[NC][U];
 #pragma unroll
-        for (int s = 0; s < SPW; s++) P::template dot<NC>(raw[u][s], g[s], act[s], acc);
+    for (int u = 0; u < U; u++) {
+        float a1[NC];
 #pragma unroll
-        for (int n = 0; n < NC; n++) acc[n] = wave_sum(acc[n]);
-        if (lane == 0) {
-            const int rl = (int)(r + (int64_t)u * rw - r0);
+        for (int n = 0; n < NC; n++) a1[n] = 0.f;
 #pragma unroll
-            for (int n = 0; n < NC; n++) part[(rl * NC + n) * kw + kseg] = acc[n];
+        for (int s = 0; s < SPW; s++) P::template dot<NC>(raw[u][s], g[s], act[s], a1);
+#pragma unroll
+        for (int n = 0; n < NC; n++) acc[n][u] = a1[n];
+    }
+    const int u = lane & (U - 1);  // the row of the pass this lane ends up holding
+    const bool writer = lane < U && i0 + u < nrw;
+    const int rl = rl0 + (i0 + u) * rw;  // row index inside the workgroup's range
+#pragma unroll
+    for (int n = 0; n < NC; n++) {
+        const float tot = reduce_rows<U>(acc[n], lane);
+        if (writer) {
+            if (DIRECT) yrow0[(int64_t)n * ldy + rl] = tot;
+            else part[(rl * NC + n) * kw + kseg] = tot;
         }
     }
 }
 
-template <class P, int NC, int SPW, int U>
+template <class P, int NC, int SPW, int U, bool DIRECT>
 __global__ __launch_bounds__(512) void gemv_kernel(DevWeight w, DevAct a, int col0, float *__restrict__ y,
-                                                    int64_t ldy, int rows_per_wg, int kw, int rw) {
-    extern __shared__ float part[];  // [rows_per_wg][NC][kw]
+                                                   int64_t ldy, int rows_per_wg, int kw, int rw) {
+    extern __shared__ float part[];  // [rows_per_wg][NC][kw], unused when DIRECT
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int kseg = wave % kw, rg = wave / kw;
+    const int kseg = DIRECT ? 0 : wave % kw, rg = DIRECT ? wave : wave / kw;
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
     const int64_t r1 = min(w.M, r0 + (int64_t)rows_per_wg);
+    const int nrows = (int)(r1 - r0);
+    const int nrw = (nrows - rg + rw - 1) / rw;  // rows of this wave: r0 + rg + i*rw, i < nrw
+    float *yrow0 = y + (int64_t)col0 * ldy + r0;
 
-    typename P::Geo g[SPW];
-    typename P::Act act[SPW][NC];
+    if (nrw > 0) {
+        typename P::Geo g[SPW];
+        typename P::Act act[SPW][NC];
 #pragma unroll
-    for (int s = 0; s < SPW; s++) {
-        g[s] = P::geo(w, kseg + s * kw, lane);
+        for (int s = 0; s < SPW; s++) {
+            g[s] = P::geo(w, kseg + s * kw, lane);
 #pragma unroll
-        for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg + s * kw, lane, g[s], act[s][n]);
+            for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg + s * kw, lane, g[s], act[s][n]);
+        }
+        typename P::Raw bufA[U][SPW], bufB[U][SPW];
+        const int64_t rbase = r0 + rg;
+        load_pass<P, SPW, U>(w, g, bufA, rbase, rw, 0, nrw);
+        if (U < nrw) load_pass<P, SPW, U>(w, g, bufB, rbase, rw, U, nrw);
+        for (int i0 = 0; i0 < nrw; i0 += 2 * U) {
+            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0, nrw, lane, kseg, kw, part, yrow0, ldy);
+            if (i0 + 2 * U < nrw) load_pass<P, SPW, U>(w, g, bufA, rbase, rw, i0 + 2 * U, nrw);
+            if (i0 + U < nrw) {
+                compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + U, nrw, lane, kseg, kw, part, yrow0,
+                                                    ldy);
+                if (i0 + 3 * U < nrw) load_pass<P, SPW, U>(w, g, bufB, rbase, rw, i0 + 3 * U, nrw);
+            }
+        }
     }
-
-    int64_t r = r0 + rg;
-    for (; r + (int64_t)(U - 1) * rw < r1; r += (int64_t)U * rw)
-        rows_step<P, NC, SPW, U>(w, g, act, r, rw, r0, lane, kseg, kw, part);
-    for (; r < r1; r += rw)  // fewer than U rows left for this wave
-        rows_step<P, NC, SPW, 1>(w, g, act, r, rw, r0, lane, kseg, kw, part);
+    if (DIRECT) return;
 
     __syncthreads();
-    const int nrows = (int)(r1 - r0);
     for (int i = threadIdx.x; i < nrows * NC; i += blockDim.x) {
         const int n = i / nrows, rl = i - n * nrows;  // consecutive threads -> consecutive rows
         float s = 0.f;
         for (int k = 0; k < kw; k++) s += part[(rl * NC + n) * kw + k];
-        y[(int64_t)(col0 + n) * ldy + r0 + rl] = s;
+        yrow0[(int64_t)n * ldy + rl] = s;
     }
 }
 
 struct Plan { int kw, rw, spw, rows_per_wg; unsigned grid; size_t lds; };
 
-// At most 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs).
+// 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), two workgroups per CU.
 template <class P>
 bool make_plan(const DevWeight &w, int nc, int num_cus, Plan &p) {
     const int nseg = (int)((w.K + P::SEG - 1) / P::SEG);
     if (nseg < 1) return false;
-    p.spw = nseg <= 8 ? 1 : nseg <= 16 ? 2 : nseg <= 32 ? 4 : nseg <= 64 ? 8 : 0;
+    p.spw = nseg <= 8 ? 1 : nseg <= 16 ? 2 : nseg <= 32 ? 4 : 0;
     if (!p.spw) return false;
     p.kw = (nseg + p.spw - 1) / p.spw;
     p.rw = 8 / p.kw;
-    const int wg_per_cu = 2;  // 16 waves per CU when the kernel fits 128 VGPRs, else 8
-    const int64_t target_wgs = (int64_t)num_cus * wg_per_cu;
+    const int64_t target_wgs = (int64_t)num_cus * 2;
     int64_t rows = (w.M + target_wgs - 1) / target_wgs;
     const int64_t lds_cap_rows = 8192 / (nc * p.kw);  // <= 32 KiB of partials
     if (rows > lds_cap_rows) rows = lds_cap_rows;
     if (rows < 1) rows = 1;
     p.rows_per_wg = (int)rows;
     p.grid = (unsigned)((w.M + rows - 1) / rows);
-    p.lds = (size_t)rows * nc * p.kw * sizeof(float);
+    p.lds = p.kw == 1 ? 0 : (size_t)rows * nc * p.kw * sizeof(float);
     return true;
 }
 
-template <class P, int NC, int U>
-hipError_t launch_nc(const DevWeight &w, const DevAct &a, int col0, float *y, int64_t ldy, int num_cus,
-                     hipStream_t s) {
-    Plan p;
-    if (!make_plan<P>(w, NC, num_cus, p) || p.spw != 1) return hipErrorInvalidValue;
+template <class P, int NC, int SPW, int U>
+void launch_one(const Plan &p, const DevWeight &w, const DevAct &a, int col0, float *y, int64_t ldy, hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
-    gemv_kernel<P, NC, 1, U><<<p.grid, block, p.lds, s>>>(w, a, col0, y, ldy, p.rows_per_wg, p.kw, p.rw);
-    return hipGetLastError();
-}
-
-// long rows (more than 8 segments): several segments per wave, one column per launch
-template <class P>
-hipError_t launch_long(const DevWeight &w, const DevAct &a, int col0, int nc, float *y, int64_t ldy,
-                       int num_cus, hipStream_t s) {
-    Plan p;
-    if (!make_plan<P>(w, 1, num_cus, p)) return hipErrorInvalidValue;
-    const dim3 block(64 * p.kw * p.rw);
-    for (int c = col0; c < col0 + nc; c++) {
-        if (p.spw == 2)
-            gemv_kernel<P, 1, 2, 2><<<p.grid, block, p.lds, s>>>(w, a, c, y, ldy, p.rows_per_wg, p.kw, p.rw);
-        else if (p.spw == 4)
-            gemv_kernel<P, 1, 4, 2><<<p.grid, block, p.lds, s>>>(w, a, c, y, ldy, p.rows_per_wg, p.kw, p.rw);
-        else
-            gemv_kernel<P, 1, 8, 1><<<p.grid, block, p.lds, s>>>(w, a, c, y, ldy, p.rows_per_wg, p.kw, p.rw);
-    }
-    return hipGetLastError();
+    if (p.kw == 1)
+        gemv_kernel<P, NC, SPW, U, true><<<p.grid, block, 0, s>>>(w, a, col0, y, ldy, p.rows_per_wg, p.kw, p.rw);
+    else
+        gemv_kernel<P, NC, SPW, U, false><<<p.grid, block, p.lds, s>>>(w, a, col0, y, ldy, p.rows_per_wg, p.kw, p.rw);
 }
 
 template <class P>
 hipError_t launch_type(const DevWeight &w, const DevAct &a, int col0, int nc, float *y, int64_t ldy,
                        int num_cus, hipStream_t s) {
-    if (w.K > 8 * (int64_t)P::SEG) return launch_long<P>(w, a, col0, nc, y, ldy, num_cus, s);
+    Plan p;
+    if (!make_plan<P>(w, nc, num_cus, p)) return hipErrorInvalidValue;
+    if (p.spw > 1) {
+        // long rows: several segments per wave, one column per launch
+        if (!make_plan<P>(w, 1, num_cus, p)) return hipErrorInvalidValue;
+        for (int c = col0; c < col0 + nc; c++) {
+            if (p.spw == 2) launch_one<P, 1, 2, (P::HEAVY ? 1 : 2)>(p, w, a, c, y, ldy, s);
+            else launch_one<P, 1, 4, 1>(p, w, a, c, y, ldy, s);
+        }
+        return hipGetLastError();
+    }
+    // rows in flight per wave = 2*U; the heavier K-quant policies use smaller passes to stay within
+    // 128 VGPRs (four waves per SIMD) for one column and 256 for eight
+    constexpr int UA = P::HEAVY ? 2 : 4, UB = P::HEAVY ? 1 : 2;
     switch (nc) {
-    case 1: return launch_nc<P, 1, 4>(w, a, col0, y, ldy, num_cus, s);
-    case 2: return launch_nc<P, 2, 4>(w, a, col0, y, ldy, num_cus, s);
-    case 3: return launch_nc<P, 3, 2>(w, a, col0, y, ldy, num_cus, s);
-    case 4: return launch_nc<P, 4, 2>(w, a, col0, y, ldy, num_cus, s);
-    case 5: return launch_nc<P, 5, 2>(w, a, col0, y, ldy, num_cus, s);
-    case 6: return launch_nc<P, 6, 2>(w, a, col0, y, ldy, num_cus, s);
-    case 7: return launch_nc<P, 7, 2>(w, a, col0, y, ldy, num_cus, s);
-    case 8: return launch_nc<P, 8, 2>(w, a, col0, y, ldy, num_cus, s);
+    case 1: launch_one<P, 1, 1, UA>(p, w, a, col0, y, ldy, s); break;
+    case 2: launch_one<P, 2, 1, UA>(p, w, a, col0, y, ldy, s); break;
+    case 3: launch_one<P, 3, 1, UB>(p, w, a, col0, y, ldy, s); break;
+    case 4: launch_one<P, 4, 1, UB>(p, w, a, col0, y, ldy, s); break;
+    case 5: launch_one<P, 5, 1, UB>(p, w, a, col0, y, ldy, s); break;
+    case 6: launch_one<P, 6, 1, UB>(p, w, a, col0, y, ldy, s); break;
+    case 7: launch_one<P, 7, 1, UB>(p, w, a, col0, y, ldy, s); break;
+    case 8: launch_one<P, 8, 1, UB>(p, w, a, col0, y, ldy, s); break;
     default: return hipErrorInvalidValue;
     }
+    return hipGetLastError();
 }
 
 }  // namespace
 
 int64_t gemv_max_k(int type) {
     switch (type) {
-    case T_Q8_0: return 64 * (int64_t)PolQ8_0::SEG;
-    case T_Q4_0: case T_Q4_K: case T_Q6_K: return 64 * (int64_t)2048;
+    case T_Q8_0: return 32 * (int64_t)PolQ8_0::SEG;
+    case T_Q4_0: return 32 * (int64_t)PolQ4_0::SEG;
+    case T_Q4_K: return 32 * (int64_t)PolQ4K::SEG;
+    case T_Q6_K: return 32 * (int64_t)PolQ6K::SEG;
     default: return 0;
     }
 }
