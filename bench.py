@@ -99,8 +99,7 @@ def main() -> int:
     def step():
         for ent in pool:
             ctx.act_quantize(act_x, x.data_ptr(), 1, qmm.DEVICE)
-            ctx.mulmat_q8_device(ent["gate"], act_x, y_gate.data_ptr())
-            ctx.mulmat_q8_device(ent["up"], act_x, y_up.data_ptr())
+            ctx.mulmat_q8_multi_device([ent["gate"], ent["up"]], act_x, [y_gate.data_ptr(), y_up.data_ptr()])
             ctx.act_quantize(act_h, h.data_ptr(), 1, qmm.DEVICE)
             ctx.mulmat_q8_device(ent["down"], act_h, y_down.data_ptr())
 

@@ -128,6 +128,12 @@ int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_
 int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *act, float *y,
                      int location, int path);
 
+/* several weights of one type and k against the same activations: ys[i] receives f32 [n][m_i].
+ * For n <= 8 and count <= 4 this is ONE kernel launch over the concatenated rows (decode: gate+up,
+ * q+k+v); otherwise it is the same as calling mi_qmm_mulmat_q8 per weight. */
+int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count,
+                           const mi_qmm_act *act, float *const *ys, int location);
+
 /* ---- diagnostics */
 const char *mi_qmm_last_error(void); /* thread-local, never NULL */
 const char *mi_qmm_version(void);

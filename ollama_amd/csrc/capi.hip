@@ -553,4 +553,54 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
     return MI_QMM_OK;
 }
 
+int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const mi_qmm_act *act,
+                           float *const *ys, int location) {
+    if (!ws || !ys || count < 1) return fail(MI_QMM_ERR_INVALID, "ws/ys is NULL or count < 1");
+    if (!act) return fail(MI_QMM_ERR_INVALID, "act is NULL");
+    for (int i = 0; i < count; i++)
+        if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
+    bool same = true;
+    for (int i = 1; i < count; i++)
+        same = same && ws[i]->dev.type == ws[0]->dev.type && ws[i]->dev.K == ws[0]->dev.K;
+    if (!same || count > gemv_max_multi() || act->n > 8 || ws[0]->dev.K > gemv_max_k(ws[0]->dev.type)) {
+        for (int i = 0; i < count; i++) {
+            int rc = mi_qmm_mulmat_q8(ctx, ws[i], act, ys[i], location, MI_QMM_PATH_AUTO);
+            if (rc) return rc;
+        }
+        return MI_QMM_OK;
+    }
+    int rc = check_product_args(ctx, ws[0], location, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    if (act->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "act and ctx are on different devices");
+    if (act->type != mi_qmm_vec_dot_type(ws[0]->dev.type) || act->k != ws[0]->dev.K)
+        return fail(MI_QMM_ERR_INVALID, "act (type %d, k=%lld) does not match the weights (type %d, k=%lld)",
+                    act->type, (long long)act->k, ws[0]->dev.type, (long long)ws[0]->dev.K);
+    if (act->n == 0) return MI_QMM_OK;
+    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
+    DevAct a;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.K = act->k; a.N = (int)act->n; a.type = act->type;
+    DevWeight dw[8];
+    for (int i = 0; i < count; i++) {
+        if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
+        dw[i] = ws[i]->dev;
+    }
+    float *dys[8];
+    size_t offs[9] = {0};
+    for (int i = 0; i < count; i++) {
+        dys[i] = ys[i];
+        offs[i + 1] = offs[i] + align_up((size_t)(act->n * dw[i].M) * 4, 256);
+    }
+    if (location == MI_QMM_HOST) {
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
+        for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
+    }
+    HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));
+    if (location == MI_QMM_HOST) {
+        for (int i = 0; i < count; i++)
+            HIP_TRY(hipMemcpyAsync(ys[i], dys[i], (size_t)(act->n * dw[i].M) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
 }  // extern "C"

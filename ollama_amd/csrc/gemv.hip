@@ -28,7 +28,8 @@ namespace miqmm {
 
 namespace {
 
-constexpr int MAXC = 8;  // activation columns per launch
+constexpr int MAXC = 8;       // activation columns per launch
+constexpr int MAX_MULTI = 4;  // weight tensors per launch
 
 __device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
 
@@ -80,13 +81,17 @@ __device__ __forceinline__ float reduce_rows(const float (&v)[U], int lane) {
 //   Act                      per-lane, per-column activation registers
 //   Raw                      the lane's loaded weight bytes for one row
 //   geo(), load_act(), load(), dot()
-// A lane whose K slice lies beyond K (ragged last segment) is "dead": it loads nothing, its weight
-// and activation registers are zero, and it contributes exactly 0.
+// A lane whose K slice lies beyond K (ragged last segment) is "dead": its loads are redirected to the
+// start of the row / activation row (branch-free, so all loads of a pass stay in one basic block and
+// the compiler can wait for exactly the loads it needs) and its activation registers are forced to
+// zero, so it contributes exactly 0.
 // ---------------------------------------------------------------------------------------------
 
 struct PolQ4K {
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
     static constexpr bool HEAVY = true;
+    static constexpr int WGS_PER_CU = 1;  // few fat waves: up to 256 VGPRs, 8 rows in flight each
+    static constexpr int U1 = 4, U2 = 2;  // rows per pass for one / two activation columns
     // lane c (0..3) of a super-block owns qs bytes [32c, 32c+32): low nibbles are sub-block 2c,
     // high nibbles sub-block 2c+1 (32 elements each), and with them scales/mins 2c and 2c+1.
     struct Geo {
@@ -105,44 +110,41 @@ struct PolQ4K {
         const int sb = seg * 16 + (lane >> 2), c = lane & 3;
         g.row_bytes = w.K / QKK * Q4_K_BYTES;
         g.live = (int64_t)sb * QKK < w.K;
-        g.off = sb * Q4_K_BYTES;
+        g.off = g.live ? sb * Q4_K_BYTES : 0;
         g.qoff = g.off + 16 + 32 * c;
         g.sh = 16 * (c & 1);
         g.hi = c >= 2;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        const int sb = seg * 16 + (lane >> 2), c = lane & 3;
-        int4 v[4] = {};
-        float dd = 0.f;
-        int b0 = 0, b1 = 0, b2 = 0, b3 = 0;
-        if (g.live) {
-            const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)sb * QKK + 64 * c);
-            v[0] = q[0]; v[1] = q[1]; v[2] = q[2]; v[3] = q[3];
-            dd = a.d[(int64_t)n * (a.K / QKK) + sb];
-            const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)sb * 16 + 4 * c;
-            b0 = bs[0]; b1 = bs[1]; b2 = bs[2]; b3 = bs[3];
-        }
-        r.lo[0] = v[0].x; r.lo[1] = v[0].y; r.lo[2] = v[0].z; r.lo[3] = v[0].w;
-        r.lo[4] = v[1].x; r.lo[5] = v[1].y; r.lo[6] = v[1].z; r.lo[7] = v[1].w;
-        r.hi[0] = v[2].x; r.hi[1] = v[2].y; r.hi[2] = v[2].z; r.hi[3] = v[2].w;
-        r.hi[4] = v[3].x; r.hi[5] = v[3].y; r.hi[6] = v[3].z; r.hi[7] = v[3].w;
-        r.d = dd;
-        r.s_lo = b0 + b1;  // sum of q8 over sub-block 2c
-        r.s_hi = b2 + b3;  // ... and 2c+1
+        const int sb = g.live ? seg * 16 + (lane >> 2) : 0, c = lane & 3;
+        const int keep = g.live ? -1 : 0;
+        const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)sb * QKK + 64 * c);
+        const int4 v0 = q[0], v1 = q[1], v2 = q[2], v3 = q[3];
+        const float dd = a.d[(int64_t)n * (a.K / QKK) + sb];
+        const int2 bs = *reinterpret_cast<const int2 *>(a.bsums + (int64_t)n * (a.K / 16) + (int64_t)sb * 16 + 4 * c);
+        r.lo[0] = v0.x & keep; r.lo[1] = v0.y & keep; r.lo[2] = v0.z & keep; r.lo[3] = v0.w & keep;
+        r.lo[4] = v1.x & keep; r.lo[5] = v1.y & keep; r.lo[6] = v1.z & keep; r.lo[7] = v1.w & keep;
+        r.hi[0] = v2.x & keep; r.hi[1] = v2.y & keep; r.hi[2] = v2.z & keep; r.hi[3] = v2.w & keep;
+        r.hi[4] = v3.x & keep; r.hi[5] = v3.y & keep; r.hi[6] = v3.z & keep; r.hi[7] = v3.w & keep;
+        r.d = g.live ? dd : 0.f;
+        r.s_lo = (((short)bs.x) + (bs.x >> 16)) & keep;  // sum of q8 over sub-block 2c
+        r.s_hi = (((short)bs.y) + (bs.y >> 16)) & keep;  // ... and 2c+1
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r = {};
-        if (g.live) {
-            const uint8_t *p = w.p0 + row * g.row_bytes;
-            r.hdr = ld16(p + g.off);
-            r.q0 = ld16(p + g.qoff);
-            r.q1 = ld16(p + g.qoff + 16);
-        }
+        Raw r;
+        const uint8_t *p = w.p0 + row * g.row_bytes;
+        r.hdr = ld16(p + g.off);
+        r.q0 = ld16(p + g.qoff);
+        r.q1 = ld16(p + g.qoff + 16);
         return r;
     }
     template <int NC>
     static __device__ __forceinline__ void dot(const Raw &r, const Geo &g, const Act (&a)[NC], float (&acc)[NC]) {
+#if defined(GEMV_VARIANT) && GEMV_VARIANT == 1
+        acc[0] += __int_as_float((r.hdr.x ^ r.hdr.y ^ r.hdr.z ^ r.hdr.w ^ r.q0.x ^ r.q0.y ^ r.q0.z ^ r.q0.w ^ r.q1.x ^ r.q1.y ^ r.q1.z ^ r.q1.w) & 0x3fffffff) + a[0].d;
+        return;
+#endif
         // hdr.x = d | dmin<<16 ; hdr.y = scales[0..3] ; hdr.z = scales[4..7] ; hdr.w = scales[8..11]
         const float dw = h2f(r.hdr.x & 0xffff), dminw = h2f(r.hdr.x >> 16);
         const unsigned ty = r.hdr.y >> g.sh, tz = r.hdr.z >> g.sh, tw = r.hdr.w >> g.sh;
@@ -178,6 +180,8 @@ struct PolQ4K {
 struct PolQ4_0 {
     static constexpr int SEG = 2048;  // 64 blocks, one per lane
     static constexpr bool HEAVY = false;
+    static constexpr int WGS_PER_CU = 2;
+    static constexpr int U1 = 4, U2 = 4;
     struct Geo { int64_t qrow, drow; int blk; bool live; };
     struct Act { int q[8]; float d; int s8; };
     struct Raw { uint4 qv; unsigned dh; };
@@ -186,31 +190,26 @@ struct PolQ4_0 {
         Geo g;
         g.blk = seg * 64 + lane;
         g.live = (int64_t)g.blk * QK < w.K;
+        if (!g.live) g.blk = 0;
         g.qrow = w.K / 2;
         g.drow = w.K / QK;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        int4 lo = {}, hi = {};
-        float dd = 0.f;
-        int s = 0;
-        if (g.live) {
-            const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.blk * QK);
-            lo = q[0]; hi = q[1];
-            dd = a.d[(int64_t)n * (a.K / QK) + g.blk];
-            s = a.bsums[(int64_t)n * (a.K / QK) + g.blk];
-        }
-        r.q[0] = lo.x; r.q[1] = lo.y; r.q[2] = lo.z; r.q[3] = lo.w;
-        r.q[4] = hi.x; r.q[5] = hi.y; r.q[6] = hi.z; r.q[7] = hi.w;
-        r.d = dd;
-        r.s8 = 8 * s;
+        const int keep = g.live ? -1 : 0;
+        const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.blk * QK);
+        const int4 lo = q[0], hi = q[1];
+        const float dd = a.d[(int64_t)n * (a.K / QK) + g.blk];
+        const int s = a.bsums[(int64_t)n * (a.K / QK) + g.blk];
+        r.q[0] = lo.x & keep; r.q[1] = lo.y & keep; r.q[2] = lo.z & keep; r.q[3] = lo.w & keep;
+        r.q[4] = hi.x & keep; r.q[5] = hi.y & keep; r.q[6] = hi.z & keep; r.q[7] = hi.w & keep;
+        r.d = g.live ? dd : 0.f;
+        r.s8 = (8 * s) & keep;
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r = {};
-        if (g.live) {
-            r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.blk * 16);
-            r.dh = w.d[row * g.drow + g.blk];
-        }
+        Raw r;
+        r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.blk * 16);
+        r.dh = w.d[row * g.drow + g.blk];
         return r;
     }
     template <int NC>
@@ -239,6 +238,8 @@ struct PolQ4_0 {
 struct PolQ8_0 {
     static constexpr int SEG = 1024;  // 32 blocks, two lanes (16 quants each) per block
     static constexpr bool HEAVY = false;
+    static constexpr int WGS_PER_CU = 2;
+    static constexpr int U1 = 4, U2 = 4;
     struct Geo { int64_t qrow, drow; int hb; bool live; };
     struct Act { int q[4]; float d; };
     struct Raw { uint4 qv; unsigned dh; };
@@ -247,26 +248,22 @@ struct PolQ8_0 {
         Geo g;
         g.hb = seg * 64 + lane;  // half-block index along the row
         g.live = (int64_t)g.hb * 16 < w.K;
+        if (!g.live) g.hb = 0;
         g.qrow = w.K;
         g.drow = w.K / QK;
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        int4 v = {};
-        float dd = 0.f;
-        if (g.live) {
-            v = *reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.hb * 16);
-            dd = a.d[(int64_t)n * (a.K / QK) + (g.hb >> 1)];
-        }
-        r.q[0] = v.x; r.q[1] = v.y; r.q[2] = v.z; r.q[3] = v.w;
-        r.d = dd;
+        const int keep = g.live ? -1 : 0;
+        const int4 v = *reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.hb * 16);
+        const float dd = a.d[(int64_t)n * (a.K / QK) + (g.hb >> 1)];
+        r.q[0] = v.x & keep; r.q[1] = v.y & keep; r.q[2] = v.z & keep; r.q[3] = v.w & keep;
+        r.d = g.live ? dd : 0.f;
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r = {};
-        if (g.live) {
-            r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.hb * 16);
-            r.dh = w.d[row * g.drow + (g.hb >> 1)];
-        }
+        Raw r;
+        r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.hb * 16);
+        r.dh = w.d[row * g.drow + (g.hb >> 1)];
         return r;
     }
     template <int NC>
@@ -286,6 +283,8 @@ struct PolQ8_0 {
 struct PolQ6K {
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
     static constexpr bool HEAVY = true;
+    static constexpr int WGS_PER_CU = 1;  // few fat waves: up to 256 VGPRs, 8 rows in flight each
+    static constexpr int U1 = 2, U2 = 1;
     // lane (h = l4>>1, t = l4&1) of a super-block owns, in half h (128 elements):
     //   ql bytes [64h+16t, +16) and [64h+32+16t, +16), qh bytes [32h+16t, +16)
     // which hold four runs of 16 elements e = 128h + 16t + 32r + i (r = 0..3):
@@ -303,6 +302,7 @@ struct PolQ6K {
         const int l4 = lane & 3, h = l4 >> 1, t = l4 & 1;
         g.sb = seg * 16 + (lane >> 2);
         g.live = (int64_t)g.sb * QKK < w.K;
+        if (!g.live) g.sb = 0;
         g.lrow = w.K / 2; g.hrow = w.K / 4; g.srow = w.K / 16; g.drow = w.K / QKK;
         g.loff = g.sb * 128 + 64 * h + 16 * t;
         g.hoff = g.sb * 64 + 32 * h + 16 * t;
@@ -312,36 +312,33 @@ struct PolQ6K {
         return g;
     }
     static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
-        int4 v[4] = {};
-        float dd = 0.f;
-        int b[4] = {0, 0, 0, 0};
-        if (g.live) {
-            const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)g.sb * QKK + g.e0;
-            const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)g.sb * 16 + (g.e0 >> 4);
-#pragma unroll
-            for (int rr = 0; rr < 4; rr++) {
-                v[rr] = *reinterpret_cast<const int4 *>(q + 32 * rr);
-                b[rr] = bs[2 * rr];
-            }
-            dd = a.d[(int64_t)n * (a.K / QKK) + g.sb];
-        }
+        const int keep = g.live ? -1 : 0;
+        const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)g.sb * QKK + g.e0;
+        const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)g.sb * 16 + (g.e0 >> 4);
+        int4 v[4];
+        int b[4];
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
-            r.q[rr][0] = v[rr].x; r.q[rr][1] = v[rr].y; r.q[rr][2] = v[rr].z; r.q[rr][3] = v[rr].w;
-            r.s32[rr] = 32 * b[rr];
+            v[rr] = *reinterpret_cast<const int4 *>(q + 32 * rr);
+            b[rr] = bs[2 * rr];
         }
-        r.d = dd;
+        const float dd = a.d[(int64_t)n * (a.K / QKK) + g.sb];
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            r.q[rr][0] = v[rr].x & keep; r.q[rr][1] = v[rr].y & keep;
+            r.q[rr][2] = v[rr].z & keep; r.q[rr][3] = v[rr].w & keep;
+            r.s32[rr] = (32 * b[rr]) & keep;
+        }
+        r.d = g.live ? dd : 0.f;
     }
     static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
-        Raw r = {};
-        if (g.live) {
-            const uint8_t *pl = w.p0 + row * g.lrow + g.loff;
-            r.l0 = ld16(pl);
-            r.l1 = ld16(pl + 32);
-            r.qh = ld16(w.p1 + row * g.hrow + g.hoff);
-            r.sc8 = *reinterpret_cast<const uint2 *>(w.p2 + row * g.srow + g.soff);
-            r.dh = w.d[row * g.drow + g.sb];
-        }
+        Raw r;
+        const uint8_t *pl = w.p0 + row * g.lrow + g.loff;
+        r.l0 = ld16(pl);
+        r.l1 = ld16(pl + 32);
+        r.qh = ld16(w.p1 + row * g.hrow + g.hoff);
+        r.sc8 = *reinterpret_cast<const uint2 *>(w.p2 + row * g.srow + g.soff);
+        r.dh = w.d[row * g.drow + g.sb];
         return r;
     }
     template <int NC>
@@ -414,7 +411,12 @@ __device__ __forceinline__ void compute_pass(const typename P::Geo (&g)[SPW],
     const int rl = rl0 + (i0 + u) * rw;  // row index inside the workgroup's range
 #pragma unroll
     for (int n = 0; n < NC; n++) {
+#if defined(GEMV_VARIANT) && GEMV_VARIANT == 2
+        float tot = 0.f;
+        for (int uu = 0; uu < U; uu++) tot += acc[n][uu];
+#else
         const float tot = reduce_rows<U>(acc[n], lane);
+#endif
         if (writer) {
             if (DIRECT) yrow0[(int64_t)n * ldy + rl] = tot;
             else part[(rl * NC + n) * kw + kseg] = tot;
@@ -422,40 +424,78 @@ __device__ __forceinline__ void compute_pass(const typename P::Geo (&g)[SPW],
     }
 }
 
+// Up to MAX_MULTI weight tensors that share K, type and the activations (gate and up, or q/k/v) go
+// through one launch: the grid is the concatenation of the tensors' workgroup ranges.
+struct MultiArgs {
+    DevWeight w[MAX_MULTI];
+    float *y[MAX_MULTI];
+    int64_t ldy[MAX_MULTI];
+    int wg_end[MAX_MULTI];  // exclusive prefix end of each tensor's workgroup range
+    int count;
+};
+
 template <class P, int NC, int SPW, int U, bool DIRECT>
-__global__ __launch_bounds__(512) void gemv_kernel(DevWeight w, DevAct a, int col0, float *__restrict__ y,
-                                                   int64_t ldy, int rows_per_wg, int kw, int rw) {
+__global__ __launch_bounds__(512, 2) void gemv_kernel(MultiArgs ma, DevAct a, int col0, int rows_per_wg, int kw,
+                                                   int rw_log2) {
     extern __shared__ float part[];  // [rows_per_wg][NC][kw], unused when DIRECT
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int kseg = DIRECT ? 0 : wave % kw, rg = DIRECT ? wave : wave / kw;
-    const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
+    int t = 0, wg = blockIdx.x;
+#pragma unroll
+    for (int i = 0; i < MAX_MULTI - 1; i++)
+        if (i + 1 < ma.count && (int)blockIdx.x >= ma.wg_end[i]) { t = i + 1; wg = blockIdx.x - ma.wg_end[i]; }
+    const DevWeight &w = ma.w[t];
+    float *__restrict__ y = ma.y[t];
+    const int64_t ldy = ma.ldy[t];
+    // the wave index is uniform across the wave: keep it (and all row arithmetic that follows from it)
+    // in scalar registers
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = 1 << rw_log2;
+    const int rg = wave & (rw - 1), kseg = wave >> rw_log2;  // rw is a power of two: no divisions here
+    const int64_t r0 = (int64_t)wg * rows_per_wg;
     const int64_t r1 = min(w.M, r0 + (int64_t)rows_per_wg);
     const int nrows = (int)(r1 - r0);
-    const int nrw = (nrows - rg + rw - 1) / rw;  // rows of this wave: r0 + rg + i*rw, i < nrw
+    const int nrw = (nrows - rg + rw - 1) >> rw_log2;  // rows of this wave: r0 + rg + i*rw, i < nrw
     float *yrow0 = y + (int64_t)col0 * ldy + r0;
 
     if (nrw > 0) {
+        // The first pass of weight loads goes out before anything else: every instruction ahead of it
+        // delays the moment the wave starts pulling on HBM.  The activation loads follow, then the
+        // second pass; the memory counter retires in order, so the first compute pass waits for
+        // weights(A) + activations only, while weights(B) stay in flight.
         typename P::Geo g[SPW];
-        typename P::Act act[SPW][NC];
 #pragma unroll
-        for (int s = 0; s < SPW; s++) {
-            g[s] = P::geo(w, kseg + s * kw, lane);
-#pragma unroll
-            for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg + s * kw, lane, g[s], act[s][n]);
-        }
+        for (int s = 0; s < SPW; s++) g[s] = P::geo(w, kseg + s * kw, lane);
         typename P::Raw bufA[U][SPW], bufB[U][SPW];
         const int64_t rbase = r0 + rg;
         load_pass<P, SPW, U>(w, g, bufA, rbase, rw, 0, nrw);
-        if (U < nrw) load_pass<P, SPW, U>(w, g, bufB, rbase, rw, U, nrw);
-        for (int i0 = 0; i0 < nrw; i0 += 2 * U) {
+        typename P::Act act[SPW][NC];
+#if defined(GEMV_VARIANT) && GEMV_VARIANT == 3
+        __builtin_memset(act, 1, sizeof(act));
+#else
+#pragma unroll
+        for (int s = 0; s < SPW; s++)
+#pragma unroll
+            for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg + s * kw, lane, g[s], act[s][n]);
+#endif
+        load_pass<P, SPW, U>(w, g, bufB, rbase, rw, U, nrw);  // clamped to the last row if nrw <= U
+        // steady state: no branches around the loads, so each compute waits for its own pass only
+        int i0 = 0;
+        for (; i0 + 4 * U <= nrw; i0 += 2 * U) {
             compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0, nrw, lane, kseg, kw, part, yrow0, ldy);
-            if (i0 + 2 * U < nrw) load_pass<P, SPW, U>(w, g, bufA, rbase, rw, i0 + 2 * U, nrw);
-            if (i0 + U < nrw) {
-                compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + U, nrw, lane, kseg, kw, part, yrow0,
-                                                    ldy);
-                if (i0 + 3 * U < nrw) load_pass<P, SPW, U>(w, g, bufB, rbase, rw, i0 + 3 * U, nrw);
-            }
+            load_pass<P, SPW, U>(w, g, bufA, rbase, rw, i0 + 2 * U, nrw);
+            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + U, nrw, lane, kseg, kw, part, yrow0, ldy);
+            load_pass<P, SPW, U>(w, g, bufB, rbase, rw, i0 + 3 * U, nrw);
         }
+        // tail: fewer than 4U rows left, of which up to 2U are already loaded
+        compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0, nrw, lane, kseg, kw, part, yrow0, ldy);
+        const bool more_a = i0 + 2 * U < nrw, more_b = i0 + 3 * U < nrw;
+        if (more_a) load_pass<P, SPW, U>(w, g, bufA, rbase, rw, i0 + 2 * U, nrw);
+        if (i0 + U < nrw)
+            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + U, nrw, lane, kseg, kw, part, yrow0, ldy);
+        if (more_b) load_pass<P, SPW, U>(w, g, bufB, rbase, rw, i0 + 3 * U, nrw);
+        if (more_a)
+            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0 + 2 * U, nrw, lane, kseg, kw, part, yrow0, ldy);
+        if (more_b)
+            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + 3 * U, nrw, lane, kseg, kw, part, yrow0, ldy);
     }
     if (DIRECT) return;
 
@@ -468,63 +508,75 @@ __global__ __launch_bounds__(512) void gemv_kernel(DevWeight w, DevAct a, int co
     }
 }
 
-struct Plan { int kw, rw, spw, rows_per_wg; unsigned grid; size_t lds; };
+struct Plan { int kw, rw, rw_log2, spw, rows_per_wg; unsigned grid; size_t lds; };
 
-// 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), two workgroups per CU.
+// 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), one or two workgroups per CU.
+// total_m is the number of rows over all tensors of the launch.
 template <class P>
-bool make_plan(const DevWeight &w, int nc, int num_cus, Plan &p) {
-    const int nseg = (int)((w.K + P::SEG - 1) / P::SEG);
+bool make_plan(int64_t K, int64_t total_m, int nc, int num_cus, Plan &p) {
+    const int nseg = (int)((K + P::SEG - 1) / P::SEG);
     if (nseg < 1) return false;
     p.spw = nseg <= 8 ? 1 : nseg <= 16 ? 2 : nseg <= 32 ? 4 : 0;
     if (!p.spw) return false;
     p.kw = (nseg + p.spw - 1) / p.spw;
-    p.rw = 8 / p.kw;
-    const int64_t target_wgs = (int64_t)num_cus * 2;
-    int64_t rows = (w.M + target_wgs - 1) / target_wgs;
+    p.rw_log2 = p.kw >= 5 ? 0 : p.kw >= 3 ? 1 : p.kw == 2 ? 2 : 3;  // largest power of two with kw*rw <= 8
+    p.rw = 1 << p.rw_log2;
+    const int64_t target_wgs = (int64_t)num_cus * P::WGS_PER_CU;
+    int64_t rows = (total_m + target_wgs - 1) / target_wgs;
     const int64_t lds_cap_rows = 8192 / (nc * p.kw);  // <= 32 KiB of partials
     if (rows > lds_cap_rows) rows = lds_cap_rows;
     if (rows < 1) rows = 1;
     p.rows_per_wg = (int)rows;
-    p.grid = (unsigned)((w.M + rows - 1) / rows);
     p.lds = p.kw == 1 ? 0 : (size_t)rows * nc * p.kw * sizeof(float);
     return true;
 }
 
 template <class P, int NC, int SPW, int U>
-void launch_one(const Plan &p, const DevWeight &w, const DevAct &a, int col0, float *y, int64_t ldy, hipStream_t s) {
+void launch_one(const Plan &p, const MultiArgs &ma, const DevAct &a, int col0, hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
     if (p.kw == 1)
-        gemv_kernel<P, NC, SPW, U, true><<<p.grid, block, 0, s>>>(w, a, col0, y, ldy, p.rows_per_wg, p.kw, p.rw);
+        gemv_kernel<P, NC, SPW, U, true><<<p.grid, block, 0, s>>>(ma, a, col0, p.rows_per_wg, p.kw, p.rw_log2);
     else
-        gemv_kernel<P, NC, SPW, U, false><<<p.grid, block, p.lds, s>>>(w, a, col0, y, ldy, p.rows_per_wg, p.kw, p.rw);
+        gemv_kernel<P, NC, SPW, U, false><<<p.grid, block, p.lds, s>>>(ma, a, col0, p.rows_per_wg, p.kw, p.rw_log2);
 }
 
 template <class P>
-hipError_t launch_type(const DevWeight &w, const DevAct &a, int col0, int nc, float *y, int64_t ldy,
+hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int nc,
                        int num_cus, hipStream_t s) {
+    int64_t total_m = 0;
+    for (int i = 0; i < count; i++) total_m += ws[i].M;
     Plan p;
-    if (!make_plan<P>(w, nc, num_cus, p)) return hipErrorInvalidValue;
+    if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
+    if (p.spw > 1 && !make_plan<P>(ws[0].K, total_m, 1, num_cus, p)) return hipErrorInvalidValue;
+    MultiArgs ma;
+    ma.count = count;
+    int64_t wgs = 0;
+    for (int i = 0; i < MAX_MULTI; i++) {
+        const int j = i < count ? i : count - 1;
+        ma.w[i] = ws[j]; ma.y[i] = ys[j]; ma.ldy[i] = ws[j].M;
+        if (i < count) wgs += (ws[i].M + p.rows_per_wg - 1) / p.rows_per_wg;
+        ma.wg_end[i] = (int)wgs;
+    }
+    if (wgs > 0x7fffffff) return hipErrorInvalidValue;
+    p.grid = (unsigned)wgs;
     if (p.spw > 1) {
         // long rows: several segments per wave, one column per launch
-        if (!make_plan<P>(w, 1, num_cus, p)) return hipErrorInvalidValue;
         for (int c = col0; c < col0 + nc; c++) {
-            if (p.spw == 2) launch_one<P, 1, 2, (P::HEAVY ? 1 : 2)>(p, w, a, c, y, ldy, s);
-            else launch_one<P, 1, 4, 1>(p, w, a, c, y, ldy, s);
+            if (p.spw == 2) launch_one<P, 1, 2, (P::HEAVY ? 1 : 2)>(p, ma, a, c, s);
+            else launch_one<P, 1, 4, 1>(p, ma, a, c, s);
         }
         return hipGetLastError();
     }
-    // rows in flight per wave = 2*U; the heavier K-quant policies use smaller passes to stay within
-    // 128 VGPRs (four waves per SIMD) for one column and 256 for eight
-    constexpr int UA = P::HEAVY ? 2 : 4, UB = P::HEAVY ? 1 : 2;
+    constexpr int UB = P::HEAVY ? 1 : 2;
     switch (nc) {
-    case 1: launch_one<P, 1, 1, UA>(p, w, a, col0, y, ldy, s); break;
-    case 2: launch_one<P, 2, 1, UA>(p, w, a, col0, y, ldy, s); break;
-    case 3: launch_one<P, 3, 1, UB>(p, w, a, col0, y, ldy, s); break;
-    case 4: launch_one<P, 4, 1, UB>(p, w, a, col0, y, ldy, s); break;
-    case 5: launch_one<P, 5, 1, UB>(p, w, a, col0, y, ldy, s); break;
-    case 6: launch_one<P, 6, 1, UB>(p, w, a, col0, y, ldy, s); break;
-    case 7: launch_one<P, 7, 1, UB>(p, w, a, col0, y, ldy, s); break;
-    case 8: launch_one<P, 8, 1, UB>(p, w, a, col0, y, ldy, s); break;
+    case 1: launch_one<P, 1, 1, P::U1>(p, ma, a, col0, s); break;
+    case 2: launch_one<P, 2, 1, P::U2>(p, ma, a, col0, s); break;
+    case 3: launch_one<P, 3, 1, UB>(p, ma, a, col0, s); break;
+    case 4: launch_one<P, 4, 1, UB>(p, ma, a, col0, s); break;
+    case 5: launch_one<P, 5, 1, UB>(p, ma, a, col0, s); break;
+    case 6: launch_one<P, 6, 1, UB>(p, ma, a, col0, s); break;
+    case 7: launch_one<P, 7, 1, UB>(p, ma, a, col0, s); break;
+    case 8: launch_one<P, 8, 1, UB>(p, ma, a, col0, s); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -542,18 +594,29 @@ int64_t gemv_max_k(int type) {
     }
 }
 
-hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int64_t ldy,
-                       int num_cus, hipStream_t s) {
-    if (ncols < 1 || ncols > MAXC || w.M < 1 || w.K < 1 || w.K > gemv_max_k(w.type) || a.K != w.K ||
-        col0 < 0 || col0 + ncols > a.N)
+int gemv_max_multi() { return MAX_MULTI; }
+
+hipError_t launch_gemv_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols,
+                             int num_cus, hipStream_t s) {
+    if (count < 1 || count > MAX_MULTI || ncols < 1 || ncols > MAXC || col0 < 0 || col0 + ncols > a.N)
         return hipErrorInvalidValue;
-    switch (w.type) {
-    case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(w, a, col0, ncols, y, ldy, num_cus, s) : hipErrorInvalidValue;
-    case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(w, a, col0, ncols, y, ldy, num_cus, s) : hipErrorInvalidValue;
-    case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(w, a, col0, ncols, y, ldy, num_cus, s) : hipErrorInvalidValue;
-    case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(w, a, col0, ncols, y, ldy, num_cus, s) : hipErrorInvalidValue;
+    for (int i = 0; i < count; i++)
+        if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || ws[i].M < 1 || !ys[i]) return hipErrorInvalidValue;
+    if (ws[0].K < 1 || ws[0].K > gemv_max_k(ws[0].type) || a.K != ws[0].K) return hipErrorInvalidValue;
+    switch (ws[0].type) {
+    case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int64_t ldy,
+                       int num_cus, hipStream_t s) {
+    if (ldy != w.M) return hipErrorInvalidValue;
+    float *ys[1] = {y};
+    return launch_gemv_multi(&w, ys, 1, a, col0, ncols, num_cus, s);
 }
 
 }  // namespace miqmm

@@ -23,6 +23,10 @@ hipError_t launch_relayout(int type, const uint8_t *gguf, int64_t K, int64_t M, 
 // returns hipErrorInvalidValue if the shape is outside the kernel's limits (caller reports it).
 hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y,
                        int64_t ldy, int num_cus, hipStream_t s);
+// several weight tensors of one type and K against the same activations in one launch
+hipError_t launch_gemv_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols,
+                             int num_cus, hipStream_t s);
+int gemv_max_multi();
 // largest K the GEMV handles for a weight type
 int64_t gemv_max_k(int type);
 

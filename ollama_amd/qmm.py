@@ -11,7 +11,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmi_qmm.so")
+# MI_QMM_LIB points at an alternative build of the library (e.g. an experimental variant)
+LIB_PATH = os.environ.get("MI_QMM_LIB") or os.path.join(_HERE, "libmi_qmm.so")
 
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 HOST, DEVICE = 0, 1
@@ -23,7 +24,7 @@ EXPORTS = [
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
-    "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8",
+    "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_last_error", "mi_qmm_version", "mi_qmm_device_info",
 ]
 
@@ -75,6 +76,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_act_free.restype = None; L.mi_qmm_act_free.argtypes = [vp]
     L.mi_qmm_act_quantize.restype = ci; L.mi_qmm_act_quantize.argtypes = [vp, vp, vp, i64, ci]
     L.mi_qmm_mulmat_q8.restype = ci; L.mi_qmm_mulmat_q8.argtypes = [vp, vp, vp, vp, ci, ci]
+    L.mi_qmm_mulmat_q8_multi.restype = ci
+    L.mi_qmm_mulmat_q8_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, ctypes.POINTER(vp), ci]
     L.mi_qmm_last_error.restype = ctypes.c_char_p; L.mi_qmm_last_error.argtypes = []
     L.mi_qmm_version.restype = ctypes.c_char_p; L.mi_qmm_version.argtypes = []
     L.mi_qmm_device_info.restype = ci
@@ -264,3 +267,17 @@ class Context:
 
     def mulmat_q8_device(self, w: Weight, act: Act, y_ptr: int, path: int = PATH_AUTO):
         _check(lib().mi_qmm_mulmat_q8(self._h, w._h, act._h, ctypes.c_void_p(y_ptr), DEVICE, path))
+
+    def mulmat_q8_multi(self, ws, act: Act):
+        """several weights against the same activations; host arrays out"""
+        ys = [np.empty((act.n, w.m), dtype=np.float32) for w in ws]
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[y.ctypes.data for y in ys])
+        _check(lib().mi_qmm_mulmat_q8_multi(self._h, wh, len(ws), act._h, yp, HOST))
+        return ys
+
+    def mulmat_q8_multi_device(self, ws, act: Act, y_ptrs):
+        """device outputs; one launch for up to 4 weights of one type and k when n <= 8"""
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[ctypes.c_void_p(int(p)) for p in y_ptrs])
+        _check(lib().mi_qmm_mulmat_q8_multi(self._h, wh, len(ws), act._h, yp, DEVICE))

@@ -227,3 +227,25 @@ def test_two_phase_matches_fused(ctx):
     with pytest.raises(qmm.QmmError):
         ctx.act_quantize(act, np.zeros((9, k), np.float32))   # more rows than n_max
     W.free(); W8.free(); act.free()
+
+
+def test_multi_weight_launch_matches_single(ctx):
+    """gate+up (and q/k/v with different row counts) through one launch give the same bits as one
+    launch per weight"""
+    k = 4096
+    rng = np.random.default_rng(31)
+    for t in (Q4_K, Q8_0, Q6_K):
+        ms = [1024, 300, 4096]
+        raws = [_weights(t, m, k, seed=100 + m) for m in ms]
+        Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+        act = ctx.act_create(qmm.vec_dot_type(t), k, 16)
+        for n in (1, 3, 9):                                # 9 > 8 columns falls back to per-weight calls
+            x = rng.standard_normal((n, k), dtype=np.float32)
+            ctx.act_quantize(act, x)
+            want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV) for W in Ws]
+            got = ctx.mulmat_q8_multi(Ws, act)
+            for y, wnt in zip(got, want):
+                assert np.array_equal(y, wnt)
+        act.free()
+        for W in Ws:
+            W.free()
