@@ -141,7 +141,7 @@ struct PolQ4K {
     }
     template <int NC>
     static __device__ __forceinline__ void dot(const Raw &r, const Geo &g, const Act (&a)[NC], float (&acc)[NC]) {
-#if defined(GEMV_VARIANT) && GEMV_VARIANT == 1
+#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 1 || GEMV_VARIANT == 5)
         acc[0] += __int_as_float((r.hdr.x ^ r.hdr.y ^ r.hdr.z ^ r.hdr.w ^ r.q0.x ^ r.q0.y ^ r.q0.z ^ r.q0.w ^ r.q1.x ^ r.q1.y ^ r.q1.z ^ r.q1.w) & 0x3fffffff) + a[0].d;
         return;
 #endif
@@ -418,7 +418,11 @@ __device__ __forceinline__ void compute_pass(const typename P::Geo (&g)[SPW],
         const float tot = reduce_rows<U>(acc[n], lane);
 #endif
         if (writer) {
+#if defined(GEMV_VARIANT) && GEMV_VARIANT == 4
+            if (DIRECT && tot == 1234.5f) yrow0[(int64_t)n * ldy + rl] = tot;
+#else
             if (DIRECT) yrow0[(int64_t)n * ldy + rl] = tot;
+#endif
             else part[(rl * NC + n) * kw + kseg] = tot;
         }
     }
@@ -468,7 +472,7 @@ __global__ __launch_bounds__(512, 2) void gemv_kernel(MultiArgs ma, DevAct a, in
         const int64_t rbase = r0 + rg;
         load_pass<P, SPW, U>(w, g, bufA, rbase, rw, 0, nrw);
         typename P::Act act[SPW][NC];
-#if defined(GEMV_VARIANT) && GEMV_VARIANT == 3
+#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 3 || GEMV_VARIANT == 5)
         __builtin_memset(act, 1, sizeof(act));
 #else
 #pragma unroll

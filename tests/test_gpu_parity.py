@@ -249,3 +249,70 @@ def test_multi_weight_launch_matches_single(ctx):
         act.free()
         for W in Ws:
             W.free()
+
+
+# ---- kernel 3: int8-MFMA GEMM ---------------------------------------------------------------------
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("k,m,n", [(256, 1, 1), (256, 32, 32), (512, 31, 33), (1024, 128, 128), (1024, 257, 200),
+                                   (4096, 160, 65), (2304, 100, 7), (14336, 64, 40)])
+def test_gemm_small_and_ragged_shapes(ctx, t, k, m, n):
+    w_raw = _weights(t, m, k, seed=k + 7 * m + t)
+    W = ctx.upload(t, w_raw, k, m)
+    x = np.random.default_rng(k + n).standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(W, x, path=qmm.PATH_GEMM)
+    want = oracle.mul_mat(t, w_raw, k, m, x, nthreads=16)
+    err = npref.rel_err(got, want)
+    assert err <= TOL, f"{NAMES[t]} k={k} m={m} n={n}: rel err {err}"
+    # the GEMV computes the same integers; only fp32 summation order differs
+    assert npref.rel_err(got, ctx.mulmat(W, x, path=qmm.PATH_GEMV)) <= TOL
+    W.free()
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+def test_gemm_random_block_bytes(ctx, t):
+    """every nibble / 6-bit scale / high-bit / int8-scale pattern, incl. negative Q6_K scales"""
+    rng = np.random.default_rng(4321 + t)
+    k, m, n = 1024, 96, 48
+    nb = m * k // 256
+    raw = rng.integers(0, 256, (nb, npref.BYTES[t]), dtype=np.uint8)
+    hbytes = np.abs(rng.standard_normal(nb * 2) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 4)
+    if t == Q4_K:
+        raw[:, 0:4] = hbytes
+    else:
+        raw[:, 208:210] = hbytes[:, 0:2]
+    W = ctx.upload(t, raw.reshape(-1), k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(W, x, path=qmm.PATH_GEMM)
+    want = oracle.mul_mat(t, raw.reshape(-1), k, m, x, nthreads=16)
+    assert npref.rel_err(got, want) <= TOL
+    W.free()
+
+
+def test_gemm_unsupported_types_use_gemv_groups(ctx):
+    """Q4_0 / Q8_0 have no MFMA kernel: AUTO keeps large batches on the GEMV, forcing GEMM is an error"""
+    k, m, n = 1024, 64, 40
+    for t in (Q4_0, Q8_0):
+        w_raw = _weights(t, m, k, seed=t)
+        W = ctx.upload(t, w_raw, k, m)
+        x = np.random.default_rng(t).standard_normal((n, k), dtype=np.float32)
+        assert npref.rel_err(ctx.mulmat(W, x), oracle.mul_mat(t, w_raw, k, m, x, nthreads=8)) <= TOL
+        with pytest.raises(qmm.QmmError) as e:
+            ctx.mulmat(W, x, path=qmm.PATH_GEMM)
+        assert e.value.code == qmm.ERR_UNSUPPORTED
+        W.free()
+
+
+@pytest.mark.parametrize("name,t,m,k", [("q_proj", Q4_K, 4096, 4096), ("k_proj", Q4_K, 1024, 4096),
+                                        ("ffn_gate", Q4_K, 14336, 4096), ("ffn_down", Q6_K, 4096, 14336)])
+def test_config5_prefill_layer_batch512(ctx, name, t, m, k):
+    """the Llama-3-8B-shaped layer of the prefill configuration at batch 512 (o = q shape, v = k shape,
+    up = gate shape)"""
+    w_raw = _weights(t, m, k, seed=1005 + m % 97)
+    W = ctx.upload(t, w_raw, k, m)
+    x = np.random.default_rng(2005).standard_normal((512, k), dtype=np.float32)
+    got = ctx.mulmat(W, x)  # AUTO -> GEMM at n = 512
+    want = oracle.mul_mat(t, w_raw, k, m, x, nthreads=16)
+    err = npref.rel_err(got, want)
+    nrm = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
+    assert err <= TOL and nrm <= 1e-5, f"{name}: rel err {err}, normwise {nrm}"
+    W.free()
