@@ -78,10 +78,13 @@ int reserve(void **buf, size_t *cap, size_t need, hipStream_t s) {
     return MI_QMM_OK;
 }
 
-struct ActPlanes { int8_t *qs; float *d; int16_t *bsums; size_t total; };
+struct ActPlanes { int8_t *qs; float *d; int16_t *bsums; uint8_t *sd8; uint8_t *sd16; size_t total; };
 
 // carve the activation scratch into planes for N rows of K elements
 ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N) {
+    // the GEMM reads Q8_K activation rows in tiles of 128 without bounds checks (results of rows past
+    // N are dropped), so the planes are sized in whole tiles
+    if (q8_type == T_Q8_K) N = (N + 127) / 128 * 128;
     const int64_t blk = q8_type == T_Q8_0 ? QK : QKK;
     const int64_t sums = q8_type == T_Q8_0 ? QK : 16;
     ActPlanes p;
@@ -89,6 +92,11 @@ ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N) {
     p.qs = (int8_t *)((char *)base + off);     off = align_up(off + (size_t)(N * K), 256);
     p.d = (float *)((char *)base + off);       off = align_up(off + (size_t)(N * (K / blk)) * 4, 256);
     p.bsums = (int16_t *)((char *)base + off); off = align_up(off + (size_t)(N * (K / sums)) * 2, 256);
+    p.sd8 = p.sd16 = nullptr;
+    if (q8_type == T_Q8_K) {  // block-sum digit planes read by the MFMA GEMM
+        p.sd8 = (uint8_t *)base + off;  off = align_up(off + (size_t)(N * (K / QKK)) * 16, 256);
+        p.sd16 = (uint8_t *)base + off; off = align_up(off + (size_t)(N * (K / QKK)) * 32, 256);
+    }
     p.total = off;
     return p;
 }
@@ -368,7 +376,7 @@ int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k,
         dx = (const float *)((char *)ctx->io_buf + xoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    HIP_TRY(launch_quantize_act(q8_type, dx, k, n, p.qs, p.d, p.bsums, ctx->stream));
+    HIP_TRY(launch_quantize_act(q8_type, dx, k, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
     HIP_TRY(launch_pack_act_gguf(q8_type, p.qs, p.d, p.bsums, k, n, dout, ctx->stream));
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(out_blocks, dout, obytes, hipMemcpyDeviceToHost, ctx->stream));
@@ -448,9 +456,9 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         dy = (float *)((char *)ctx->io_buf + yoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, ctx->stream));
+    HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
     DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.K = K; a.N = (int)n; a.type = q8;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
     if ((rc = run_product(ctx, w, a, dy, path))) return rc;
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
@@ -519,7 +527,7 @@ int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_
         dx = (const float *)ctx->io_buf;
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    HIP_TRY(launch_quantize_act(act->type, dx, act->k, n, p.qs, p.d, p.bsums, ctx->stream));
+    HIP_TRY(launch_quantize_act(act->type, dx, act->k, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
     if (location == MI_QMM_HOST) HIP_TRY(hipStreamSynchronize(ctx->stream));  // x may be reused by the caller
     return MI_QMM_OK;
 }
@@ -538,7 +546,7 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
     if (!y) return fail(MI_QMM_ERR_INVALID, "y is NULL");
     const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
     DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.K = act->k; a.N = (int)n; a.type = act->type;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = act->k; a.N = (int)n; a.type = act->type;
     float *dy = y;
     const size_t ybytes = (size_t)(n * M) * 4;
     if (location == MI_QMM_HOST) {
@@ -578,7 +586,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     if (act->n == 0) return MI_QMM_OK;
     const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
     DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.K = act->k; a.N = (int)act->n; a.type = act->type;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = act->k; a.N = (int)act->n; a.type = act->type;
     DevWeight dw[8];
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);

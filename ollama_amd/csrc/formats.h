@@ -40,10 +40,15 @@ struct DevWeight {
 //   d     [N][K/B]    fp32 block scale (B = 32 for Q8_0 where the value is the fp16-rounded scale
 //                     widened exactly; B = 256 for Q8_K)
 //   bsums [N][K/S]    int16 partial sums of quants (S = 32 for Q8_0: one per block; S = 16 for Q8_K)
+// Q8_K only, for the MFMA GEMM (block sums as two int8 digits, S = 64*S_h + S_l, S_l in 0..63):
+//   sd8   [N][K/256][16]   S_j = bsums[2j] + bsums[2j+1], j = 0..7:  bytes [S_l(0..7) | S_h(0..7)]
+//   sd16  [N][K/256][32]   S_g = bsums[g], g = 0..15:                bytes [S_l(0..15) | S_h(0..15)]
 struct DevAct {
     const int8_t *qs;
     const float *d;
     const int16_t *bsums;
+    const uint8_t *sd8;
+    const uint8_t *sd16;
     int64_t K;
     int N;
     int type;  // T_Q8_0 or T_Q8_K

@@ -9,8 +9,9 @@
 namespace miqmm {
 
 // kernel 1: f32 rows -> Q8_0 / Q8_K planes (bit-exact with the scalar CPU quantizers)
+// sd8 / sd16: block-sum digit planes for the GEMM (Q8_K only; may be null)
 hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs,
-                               float *d, int16_t *bsums, hipStream_t s);
+                               float *d, int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s);
 // planes -> GGUF block bytes (34 B / 292 B blocks), for callers that want the bytes
 hipError_t launch_pack_act_gguf(int q8_type, const int8_t *qs, const float *d, const int16_t *bsums,
                                 int64_t K, int64_t N, uint8_t *out, hipStream_t s);

@@ -56,7 +56,8 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float4 *__rest
 // one wave per super-block of 256; 4 waves per workgroup.  nblk = N*K/256.
 __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__restrict__ x,
                                                             int *__restrict__ qs, float *__restrict__ d,
-                                                            int16_t *__restrict__ bsums, int64_t nblk) {
+                                                            int16_t *__restrict__ bsums, uint8_t *__restrict__ sd8,
+                                                            uint8_t *__restrict__ sd16, int64_t nblk) {
     const int lane = threadIdx.x & 63;
     const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (blk >= nblk) return;  // whole wave leaves together
@@ -90,9 +91,19 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__rest
     int sum = q[0] + q[1] + q[2] + q[3];
     sum += __shfl_xor(sum, 1);
     sum += __shfl_xor(sum, 2);
+    const int pair = sum + __shfl_xor(sum, 4);  // bsums[2j] + bsums[2j+1] in lanes 8j .. 8j+7
     qs[blk * 64 + lane] = pack4(q[0], q[1], q[2], q[3]);
     if ((lane & 3) == 0) bsums[blk * 16 + (lane >> 2)] = (int16_t)sum;
     if (lane == 0) d[blk] = dd;
+    // block sums as two int8 digits (s = 64*(s >> 6) + (s & 63)) for the int8-MFMA GEMM
+    if (sd16 && (lane & 3) == 0) {
+        sd16[blk * 32 + (lane >> 2)] = (uint8_t)(sum & 63);
+        sd16[blk * 32 + 16 + (lane >> 2)] = (uint8_t)(sum >> 6);
+    }
+    if (sd8 && (lane & 7) == 0) {
+        sd8[blk * 16 + (lane >> 3)] = (uint8_t)(pair & 63);
+        sd8[blk * 16 + 8 + (lane >> 3)] = (uint8_t)(pair >> 6);
+    }
 }
 
 // planes -> GGUF bytes; one thread per output byte (a convenience path, not on the hot path)
@@ -131,7 +142,7 @@ __global__ void pack_q8_K_kernel(const int8_t *__restrict__ qs, const float *__r
 }  // namespace
 
 hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs, float *d,
-                               int16_t *bsums, hipStream_t s) {
+                               int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s) {
     if (N * K == 0) return hipSuccess;
     if (q8_type == T_Q8_0) {
         const int64_t nblk = N * K / QK;
@@ -141,7 +152,7 @@ hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N
     } else if (q8_type == T_Q8_K) {
         const int64_t nblk = N * K / QKK;
         const unsigned grid = (unsigned)((nblk + 3) / 4);
-        quantize_q8_K_kernel<<<grid, 256, 0, s>>>((const float4 *)x, (int *)qs, d, bsums, nblk);
+        quantize_q8_K_kernel<<<grid, 256, 0, s>>>((const float4 *)x, (int *)qs, d, bsums, sd8, sd16, nblk);
     } else {
         return hipErrorInvalidValue;
     }
