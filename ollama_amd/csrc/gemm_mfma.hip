@@ -264,44 +264,73 @@ __global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(DevWeight w, DevAct
         // memory instructions in flight
         const int64_t sbn = min(sb + 2, nsb - 1);
         BOperand b;
+#if defined(GEMV_VARIANT) && GEMV_VARIANT == 15
+        __builtin_memset(&b, 1, sizeof(b)); b.d = __int_as_float(raw.hdr.x);
+#else
         G::expand(raw, h, b);
+#endif
+#if !(defined(GEMV_VARIANT) && (GEMV_VARIANT == 16 || GEMV_VARIANT == 18))
         stage_copy(lds[(sb + 2) % 3], sbn);  // that stage was last read in iteration sb-1: every wave has passed its barrier
+#endif
+#if !(defined(GEMV_VARIANT) && (GEMV_VARIANT == 17 || GEMV_VARIANT == 18))
         G::load_raw(w, row, sbn, h, raw);
+#endif
+        // The matrix cores and the vector ALU are fed from one in-order instruction stream per wave, and
+        // there is one wave per SIMD: to keep both busy the fp32 epilogue of sub-tile t-1 is interleaved
+        // by hand with the MFMAs of sub-tile t -- per k-step two MFMAs (64 matrix-core cycles), then
+        // the epilogue of two outputs -- with scheduling barriers pinning that order.
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        v16i ah[2], al[2], xl[2], xh[2];
 #pragma unroll
-        for (int t = 0; t < TNT; t++) {
-            __builtin_amdgcn_sched_barrier(0);  // keep the sub-tiles apart: hoisting all A loads costs 128 VGPRs
-            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            const uint8_t *arow = cur.q + (32 * t + r) * 256;
-            float fm[16];
-            {
-                const v4i sv = *reinterpret_cast<const v4i *>(cur.s + (32 * t + r) * G::SD + (G::SD == 32 ? 16 * h : 0));
-                const v16i xl = mfma(sv, b.min_lo, zero), xh = mfma(sv, b.min_hi, zero);
-#pragma unroll
-                for (int i = 0; i < 16; i++) fm[i] = G::fold_min(b.dmin, xh[i], xl[i]);
-            }
-            v16i ah = zero, al = zero;
-            // A operand pieces are fetched two k-steps ahead of the MFMAs that consume them
+        for (int t = 0; t <= TNT; t++) {
+            const int p = t & 1, q = p ^ 1;  // accumulator set being produced / consumed
+            const uint8_t *arow = cur.q + (32 * (t < TNT ? t : 0) + r) * 256;
             v4i abuf[3];
-            abuf[0] = *reinterpret_cast<const v4i *>(arow + (0 ^ swz));
-            abuf[1] = *reinterpret_cast<const v4i *>(arow + (32 ^ swz));
+            if (t < TNT) {
+                const v4i sv = *reinterpret_cast<const v4i *>(cur.s + (32 * t + r) * G::SD + (G::SD == 32 ? 16 * h : 0));
+                abuf[0] = *reinterpret_cast<const v4i *>(arow + (0 ^ swz));
+                abuf[1] = *reinterpret_cast<const v4i *>(arow + (32 ^ swz));
+                xl[p] = mfma(sv, b.min_lo, zero);
+                xh[p] = mfma(sv, b.min_hi, zero);
+                ah[p] = zero;
+                al[p] = zero;
+            }
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                if (s + 2 < 8) abuf[(s + 2) % 3] = *reinterpret_cast<const v4i *>(arow + ((32 * (s + 2)) ^ swz));
-                const v4i av = abuf[s % 3];
-                ah = mfma(av, b.hi[s], ah);
-                al = mfma(av, b.lo[s], al);
-            }
-            // ---- fp32 epilogue of the super-block: accumulator i is activation row 8(i/4) + 4h + i%4
+                if (t < TNT) {
+                    if (s + 2 < 8) abuf[(s + 2) % 3] = *reinterpret_cast<const v4i *>(arow + ((32 * (s + 2)) ^ swz));
+                    const v4i av = abuf[s % 3];
+#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 12 || GEMV_VARIANT == 14)
+                    ah[p][s] ^= av[0] ^ b.hi[s][1]; al[p][s] ^= av[2] ^ b.lo[s][3];   // MFMAs removed
+#else
+                    ah[p] = mfma(av, b.hi[s], ah[p]);
+                    al[p] = mfma(av, b.lo[s], al[p]);
+#endif
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (t > 0) {  // outputs 2s and 2s+1 of sub-tile t-1; accumulator i is activation row 8(i/4) + 4h + i%4
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float yd = cur.yd[32 * t + 8 * (i >> 2) + 4 * h + (i & 3)];
-                acc[t][i] = __builtin_fmaf(yd, G::combine(b.d, ah[i], al[i], fm[i]), acc[t][i]);
+                    for (int i = 2 * s; i < 2 * s + 2; i++) {
+                        const float yd = cur.yd[32 * (t - 1) + 8 * (i >> 2) + 4 * h + (i & 3)];
+                        const float fm = G::fold_min(b.dmin, xh[q][i], xl[q][i]);
+#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 11 || GEMV_VARIANT == 14)
+                        acc[t - 1][i] += __int_as_float(ah[q][i] ^ al[q][i]) + yd + fm * 0.f;
+#else
+                        acc[t - 1][i] = __builtin_fmaf(yd, G::combine(b.d, ah[q][i], al[q][i], fm), acc[t - 1][i]);
+#endif
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         // the youngest QI + RAW_LOADS memory instructions are the quant copies and packed-weight loads
         // for super-block sb+2; everything older (stage sb+1, weights sb+1) must have landed
         constexpr int KEEP = QI + G::RAW_LOADS;
+#if defined(GEMV_VARIANT) && GEMV_VARIANT >= 16 && GEMV_VARIANT <= 18
+        __builtin_amdgcn_s_waitcnt(0);
+#else
         __builtin_amdgcn_s_waitcnt((KEEP & 15) | (7 << 4) | (15 << 8) | ((KEEP >> 4) << 14));
+#endif
         // a bare barrier: __syncthreads() carries a fence that drains every outstanding load, i.e. it
         // would wait for the copies issued a moment ago.  What must be ordered here is LDS only: the
         // copies of the next stage are complete (the wait above, in every wave) and this wave's reads
