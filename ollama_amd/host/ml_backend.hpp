@@ -1,0 +1,161 @@
+// C++ host-side mirror of the reference's tensor-backend interface for the Mulmat path, over the
+// C ABI in include/mi_qmm.h.  The reference declares it in Go:
+//   ml.Backend  /root/reference/ml/backend.go:16-33    Load / Get(name) / NewContext / Close
+//   ml.Context  /root/reference/ml/backend.go:94-128   FromFloats / Compute / Close
+//   ml.Tensor   /root/reference/ml/backend.go:130-153  Dim / Shape / Floats / Mulmat / MulmatFullPrec
+// Same names, same argument meaning (ggml shapes: dimension 0 contiguous, W = [K, M], x = [K, N],
+// W.Mulmat(ctx, x) = [M, N]) and the same error behaviour: tensor ops have no error return, so a
+// failure throws (the Go interface panics).  Mulmat is lazy; Compute runs the pending nodes, sharing
+// one activation quantization between all nodes that read the same x.
+#pragma once
+
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/mi_qmm.h"
+
+namespace ollama_amd {
+
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const std::string &what) : std::runtime_error(what), code(c) {}
+};
+
+inline void check(int rc) {
+    if (rc != MI_QMM_OK) throw Error(rc, mi_qmm_last_error());
+}
+
+class Context;
+
+class Tensor {
+public:
+    int Dim(int n) const { return n < (int)shape_.size() ? (int)shape_[n] : 1; }
+    const std::vector<int64_t> &Shape() const { return shape_; }
+    int GGMLType() const { return type_; }
+    // values in ggml order (dimension 0 contiguous); throws until Compute has produced them
+    const std::vector<float> &Floats() const {
+        if (!ready_) throw Error(MI_QMM_ERR_INVALID, "tensor has no data yet: call Context::Compute first");
+        return data_;
+    }
+    // self = quantized weight [K, M], t2 = f32 activations [K, N] -> lazy [M, N]
+    std::shared_ptr<Tensor> Mulmat(Context &ctx, const std::shared_ptr<Tensor> &t2);
+    std::shared_ptr<Tensor> MulmatFullPrec(Context &ctx, const std::shared_ptr<Tensor> &t2) { return Mulmat(ctx, t2); }
+
+    ~Tensor() { mi_qmm_weight_free(weight_); }
+
+private:
+    friend class Backend;
+    friend class Context;
+    std::vector<int64_t> shape_;
+    int type_ = MI_QMM_TYPE_F32;
+    mi_qmm_weight *weight_ = nullptr;
+    std::vector<float> data_;
+    bool ready_ = false;
+    Tensor *op_w_ = nullptr;             // pending Mulmat: weight
+    std::shared_ptr<Tensor> op_x_;       // pending Mulmat: activations
+    std::shared_ptr<Tensor> self_keep_;  // keeps the weight alive while a node refers to it
+};
+
+class Backend {
+public:
+    explicit Backend(int device = 0) { check(mi_qmm_init(device, &ctx_)); }
+    ~Backend() { Close(); }
+    Backend(const Backend &) = delete;
+    Backend &operator=(const Backend &) = delete;
+
+    // One GGUF tensor: type id, shape [K, M], M rows of K elements in GGUF block layout (what fs/ggml
+    // hands out, /root/reference/fs/ggml/gguf.go:281-308).  The bytes are copied to the device.
+    void Load(const std::string &name, int ggml_type, int64_t k, int64_t m, const void *gguf_bytes) {
+        auto t = std::make_shared<Tensor>();
+        t->shape_ = {k, m};
+        t->type_ = ggml_type;
+        check(mi_qmm_weight_upload(ctx_, ggml_type, gguf_bytes, k, m, MI_QMM_HOST, &t->weight_));
+        tensors_[name] = t;
+    }
+    std::shared_ptr<Tensor> Get(const std::string &name) const {
+        auto it = tensors_.find(name);
+        return it == tensors_.end() ? nullptr : it->second;  // nil for an unknown name, like the reference
+    }
+    std::unique_ptr<Context> NewContext();
+    void Close() {
+        tensors_.clear();
+        if (ctx_) mi_qmm_destroy(ctx_);
+        ctx_ = nullptr;
+    }
+    mi_qmm_ctx *handle() const { return ctx_; }
+
+private:
+    mi_qmm_ctx *ctx_ = nullptr;
+    std::map<std::string, std::shared_ptr<Tensor>> tensors_;
+};
+
+class Context {
+public:
+    explicit Context(Backend &b) : b_(b) {}
+    std::shared_ptr<Tensor> FromFloats(const std::vector<float> &s, std::vector<int64_t> shape) {
+        int64_t n = 1;
+        for (auto d : shape) n *= d;
+        if (n != (int64_t)s.size()) throw Error(MI_QMM_ERR_INVALID, "FromFloats: value count does not match the shape");
+        auto t = std::make_shared<Tensor>();
+        t->shape_ = std::move(shape);
+        t->data_ = s;
+        t->ready_ = true;
+        return t;
+    }
+    // run every pending Mulmat node; nodes that read the same x share one quantization
+    void Compute() {
+        std::map<std::pair<Tensor *, int>, std::vector<Tensor *>> by_x;
+        for (auto &n : nodes_)
+            if (!n->ready_) by_x[{n->op_x_.get(), mi_qmm_vec_dot_type(n->op_w_->type_)}].push_back(n.get());
+        for (auto &kv : by_x) {
+            Tensor *x = kv.first.first;
+            const int64_t k = x->Dim(0), n = (int64_t)x->data_.size() / k;
+            mi_qmm_act *act = nullptr;
+            check(mi_qmm_act_create(b_.handle(), kv.first.second, k, n, &act));
+            int rc = mi_qmm_act_quantize(b_.handle(), act, x->data_.data(), n, MI_QMM_HOST);
+            for (size_t i = 0; rc == MI_QMM_OK && i < kv.second.size(); i += 4) {
+                const mi_qmm_weight *ws[4];
+                float *ys[4];
+                int cnt = 0;
+                for (size_t j = i; j < kv.second.size() && j < i + 4; j++, cnt++) {
+                    Tensor *t = kv.second[j];
+                    t->data_.assign((size_t)(n * t->Dim(0)), 0.f);
+                    ws[cnt] = t->op_w_->weight_;
+                    ys[cnt] = t->data_.data();
+                }
+                rc = mi_qmm_mulmat_q8_multi(b_.handle(), ws, cnt, act, ys, MI_QMM_HOST);
+            }
+            mi_qmm_act_free(act);
+            check(rc);
+            for (Tensor *t : kv.second) t->ready_ = true;
+        }
+    }
+    void Close() { nodes_.clear(); }
+
+private:
+    friend class Tensor;
+    Backend &b_;
+    std::vector<std::shared_ptr<Tensor>> nodes_;
+};
+
+inline std::unique_ptr<Context> Backend::NewContext() { return std::unique_ptr<Context>(new Context(*this)); }
+
+inline std::shared_ptr<Tensor> Tensor::Mulmat(Context &ctx, const std::shared_ptr<Tensor> &t2) {
+    if (!weight_) throw Error(MI_QMM_ERR_INVALID, "Mulmat: the receiver must be a quantized weight from Backend::Get");
+    if (!t2 || t2->type_ != MI_QMM_TYPE_F32) throw Error(MI_QMM_ERR_INVALID, "Mulmat: activations must be f32");
+    if (t2->Dim(0) != Dim(0)) throw Error(MI_QMM_ERR_INVALID, "Mulmat: inner dimensions differ");
+    auto out = std::make_shared<Tensor>();
+    out->shape_ = {shape_[1]};
+    for (size_t i = 1; i < t2->shape_.size(); i++) out->shape_.push_back(t2->shape_[i]);
+    out->op_w_ = this;
+    out->op_x_ = t2;
+    ctx.nodes_.push_back(out);
+    return out;
+}
+
+}  // namespace ollama_amd

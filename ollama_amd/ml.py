@@ -1,0 +1,192 @@
+"""Host-side mirror of the reference's tensor-backend interface for the Mulmat path.
+
+Names, argument meaning and error behaviour follow /root/reference/ml/backend.go:
+  Backend   :16-33   Load / Get(name) / NewContext / Close        (weights live here until Close)
+  Context   :94-128  FromFloats / Compute / Close                 (tensors die with the context)
+  Tensor    :130-153 Dim / Stride / Shape / DType / Bytes / Floats / Mulmat / MulmatFullPrec
+  DType     :404-412
+The reference's tensor ops build a lazy graph and have no error returns: Mulmat records a node,
+Compute runs it, and a failure is a panic -- here a raised exception.  Shapes are ggml's: dimension 0
+is the contiguous one, a weight is [K, M], activations are [K, N], ``W.Mulmat(ctx, x)`` is [M, N].
+
+Everything that computes goes through the C ABI (``ollama_amd.qmm``).  Compute hoists the activation
+quantization: all Mulmat nodes of a graph that read the same ``x`` share one quantization, and the
+decode-sized ones (N <= 8) of the same weight type run as one multi-tensor launch.
+"""
+from __future__ import annotations
+
+import enum
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import qmm
+
+
+class DType(enum.IntEnum):  # /root/reference/ml/backend.go:404-412
+    Other = 0
+    F32 = 1
+    F16 = 2
+    Q80 = 3
+    Q40 = 4
+    I32 = 5
+    MXFP4 = 6
+
+
+_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40}
+
+
+class Tensor:
+    """A node of the graph: a weight, an input, or a pending Mulmat result."""
+
+    def __init__(self, shape: Sequence[int], ggml_type: int = qmm.F32):
+        self._shape = [int(d) for d in shape]
+        self._type = ggml_type
+        self._weight: Optional[qmm.Weight] = None      # resident quantized weight
+        self._raw: Optional[np.ndarray] = None          # GGUF bytes of a weight (kept for Bytes())
+        self._data: Optional[np.ndarray] = None          # f32 values, flat in ggml order
+        self._op: Optional[Tuple["Tensor", "Tensor"]] = None  # (W, x) of a pending Mulmat
+
+    # -- shape queries, /root/reference/ml/backend.go:131-135
+    def Dim(self, n: int) -> int:
+        return self._shape[n] if n < len(self._shape) else 1
+
+    def Stride(self, n: int) -> int:
+        """bytes between consecutive elements along dimension n (ggml nb[n])"""
+        if self._type != qmm.F32:
+            row = qmm.row_size(self._type, self._shape[0])
+            return qmm.type_size(self._type) if n == 0 else row * int(np.prod(self._shape[1:n], dtype=np.int64))
+        return 4 * int(np.prod(self._shape[:n], dtype=np.int64))
+
+    def Shape(self) -> List[int]:
+        return list(self._shape)
+
+    def DType(self) -> DType:
+        return _GGML_TO_DTYPE.get(self._type, DType.Other)
+
+    # -- data access, :138-140
+    def Bytes(self) -> bytes:
+        if self._raw is not None:
+            return self._raw.tobytes()
+        return self.Floats().tobytes()
+
+    def Floats(self) -> np.ndarray:
+        if self._data is None:
+            raise RuntimeError("tensor has no data yet: call Context.Compute on it first")
+        return self._data
+
+    # -- the op, :151-152
+    def Mulmat(self, ctx: "Context", t2: "Tensor") -> "Tensor":
+        """self = W [K, M] (quantized weight), t2 = x [K, N] f32  ->  [M, N] f32, lazily."""
+        if self._weight is None:
+            raise TypeError("Mulmat: the receiver must be a quantized weight obtained from Backend.Get")
+        if t2._type != qmm.F32:
+            raise TypeError("Mulmat: activations must be f32")
+        if t2.Dim(0) != self.Dim(0):
+            raise ValueError(f"Mulmat: inner dimensions differ: {self.Shape()} x {t2.Shape()}")
+        out = Tensor([self.Dim(1)] + t2._shape[1:])
+        out._op = (self, t2)
+        ctx._nodes.append(out)
+        return out
+
+    def MulmatFullPrec(self, ctx: "Context", t2: "Tensor") -> "Tensor":
+        """The quantized path already accumulates block sums in exact integers and scales in fp32."""
+        return self.Mulmat(ctx, t2)
+
+
+class Context:
+    """Holds the tensors of one graph; Compute runs the pending Mulmat nodes."""
+
+    def __init__(self, backend: "Backend"):
+        self._b = backend
+        self._nodes: List[Tensor] = []
+        self._closed = False
+
+    def FromFloats(self, s: Sequence[float], *shape: int) -> Tensor:
+        arr = np.ascontiguousarray(s, dtype=np.float32).reshape(-1)
+        if int(np.prod(shape, dtype=np.int64)) != arr.size:
+            raise ValueError(f"FromFloats: {arr.size} values for shape {list(shape)}")
+        t = Tensor(shape)
+        t._data = arr
+        return t
+
+    def Forward(self, *tensors: Tensor) -> "Context":
+        return self
+
+    def Compute(self, *tensors: Tensor) -> None:
+        """Run every pending node the given tensors depend on (here: all pending Mulmat nodes)."""
+        if self._closed:
+            raise RuntimeError("Compute on a closed context")
+        pending = [t for t in self._nodes if t._data is None and t._op is not None]
+        c = self._b._ctx
+        # group by activation tensor: one quantization per (x, q8 type)
+        by_x: Dict[Tuple[int, int], List[Tensor]] = {}
+        for t in pending:
+            W, x = t._op
+            by_x.setdefault((id(x), qmm.vec_dot_type(W._type)), []).append(t)
+        for (_, q8), nodes in by_x.items():
+            x = nodes[0]._op[1]
+            k = x.Dim(0)
+            n = x.Floats().size // k
+            act = c.act_create(q8, k, max(n, 1))
+            try:
+                c.act_quantize(act, x.Floats().reshape(n, k))
+                # decode-sized products of one weight type go out as multi-tensor launches
+                by_type: Dict[int, List[Tensor]] = {}
+                for t in nodes:
+                    by_type.setdefault(t._op[0]._type, []).append(t)
+                for group in by_type.values():
+                    for i in range(0, len(group), 4):
+                        part = group[i:i + 4]
+                        ys = c.mulmat_q8_multi([t._op[0]._weight for t in part], act)
+                        for t, y in zip(part, ys):
+                            t._data = y.reshape(-1)  # [n][m] row-major == ggml [M, N] with dim 0 contiguous
+            finally:
+                act.free()
+
+    def Close(self) -> None:
+        self._nodes.clear()
+        self._closed = True
+
+
+class Backend:
+    """Weights resident on one MI355X.  ``tensors`` maps a GGUF tensor name to
+    (ggml_type, shape [K, M], block bytes) -- what fs/ggml hands out for a tensor
+    (/root/reference/fs/ggml/gguf.go:281-308)."""
+
+    def __init__(self, tensors: Dict[str, Tuple[int, Sequence[int], np.ndarray]], device: int = 0):
+        self._ctx = qmm.Context(device)
+        self._tensors: Dict[str, Tensor] = {}
+        self._spec = tensors
+        self._loaded = False
+
+    def Load(self, progress=None) -> None:
+        total = max(len(self._spec), 1)
+        for i, (name, (ggml_type, shape, raw)) in enumerate(self._spec.items()):
+            if len(shape) != 2:
+                raise ValueError(f"{name}: only 2-D weights take part in Mulmat, got shape {list(shape)}")
+            k, m = int(shape[0]), int(shape[1])
+            raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1)
+            t = Tensor([k, m], ggml_type)
+            t._weight = self._ctx.upload(ggml_type, raw, k, m)
+            t._raw = raw
+            self._tensors[name] = t
+            if progress:
+                progress((i + 1) / total)
+        self._loaded = True
+
+    def Get(self, name: str) -> Optional[Tensor]:
+        return self._tensors.get(name)  # nil for an unknown name, like the reference
+
+    def NewContext(self) -> Context:
+        return Context(self)
+
+    def BackendDevices(self):
+        return [self._ctx.device_info()]
+
+    def Close(self) -> None:
+        for t in self._tensors.values():
+            if t._weight is not None:
+                t._weight.free()
+        self._tensors.clear()
+        self._ctx.close()

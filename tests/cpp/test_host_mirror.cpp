@@ -1,0 +1,83 @@
+// GPU test program (run by tests/test_gpu_host_mirror.py): drives the C++ mirror of the reference's
+// ml.Backend / Context / Tensor interface and checks every Mulmat against the CPU oracle.
+// Links libmi_qmm.so (the product) and oracle/libggml_ref.so (the checker; test infrastructure).
+#include <cmath>
+#include <cstdio>
+#include <random>
+#include <vector>
+
+#include "../../ollama_amd/host/ml_backend.hpp"
+#include "../../oracle/ggml_ref.h"
+
+using namespace ollama_amd;
+
+static std::vector<float> randn(size_t n, float std, unsigned seed) {
+    std::mt19937 g(seed);
+    std::normal_distribution<float> d(0.f, std);
+    std::vector<float> v(n);
+    for (auto &x : v) x = d(g);
+    return v;
+}
+
+static double rel_err(const std::vector<float> &y, const std::vector<float> &ref) {
+    double ss = 0;
+    for (float r : ref) ss += (double)r * r;
+    const double floor_ = 1e-2 * std::sqrt(ss / ref.size());
+    double worst = 0;
+    for (size_t i = 0; i < ref.size(); i++) {
+        const double den = std::fmax(std::fabs((double)ref[i]), floor_);
+        worst = std::fmax(worst, std::fabs((double)y[i] - ref[i]) / (den > 0 ? den : 1));
+    }
+    return worst;
+}
+
+int main() {
+    try {
+        Backend backend(0);
+        struct Spec { const char *name; int type; int64_t k, m; };
+        const Spec specs[] = {{"blk.0.attn_q.weight", MI_QMM_TYPE_Q4_K, 1024, 512}, {"blk.0.attn_k.weight", MI_QMM_TYPE_Q4_K, 1024, 128},
+                              {"blk.0.ffn_down.weight", MI_QMM_TYPE_Q6_K, 1024, 256}, {"output.weight", MI_QMM_TYPE_Q8_0, 1024, 300},
+                              {"legacy.weight", MI_QMM_TYPE_Q4_0, 1024, 64}};
+        std::vector<std::vector<uint8_t>> raws;
+        for (const Spec &s : specs) {
+            auto wf = randn((size_t)(s.k * s.m), 0.02f, 17 + (unsigned)s.m);
+            std::vector<uint8_t> raw((size_t)(ref_row_size(s.type, s.k) * s.m));
+            if (ref_quantize(s.type, wf.data(), raw.data(), s.k, s.m, 4) != 0) { printf("FAIL: encode %s\n", s.name); return 1; }
+            backend.Load(s.name, s.type, s.k, s.m, raw.data());
+            raws.push_back(std::move(raw));
+        }
+        if (backend.Get("missing.weight") != nullptr) { printf("FAIL: Get of an unknown name\n"); return 1; }
+        int failures = 0;
+        for (int64_t n : {1, 3, 40}) {  // decode, skinny, prefill-sized batch
+            auto ctx = backend.NewContext();
+            auto xv = randn((size_t)(1024 * n), 1.0f, 99 + (unsigned)n);
+            auto x = ctx->FromFloats(xv, {1024, n});
+            std::vector<std::shared_ptr<Tensor>> outs;
+            for (const Spec &s : specs) outs.push_back(backend.Get(s.name)->Mulmat(*ctx, x));
+            ctx->Compute();
+            for (size_t i = 0; i < outs.size(); i++) {
+                const Spec &s = specs[i];
+                std::vector<float> ref((size_t)(s.m * n));
+                if (ref_mul_mat(s.type, raws[i].data(), s.k, s.m, xv.data(), n, ref.data(), nullptr, 4) != 0) return 1;
+                const double e = rel_err(outs[i]->Floats(), ref);
+                const bool shape_ok = outs[i]->Dim(0) == s.m && outs[i]->Dim(1) == n;
+                printf("%-24s n=%-3lld rel err %.2e %s\n", s.name, (long long)n, e, (e <= 1e-3 && shape_ok) ? "ok" : "FAIL");
+                if (!(e <= 1e-3) || !shape_ok) failures++;
+            }
+            ctx->Close();
+        }
+        // error behaviour: mismatched inner dimension throws, like the Go interface panics
+        bool threw = false;
+        try {
+            auto ctx = backend.NewContext();
+            backend.Get("output.weight")->Mulmat(*ctx, ctx->FromFloats(std::vector<float>(512), {512, 1}));
+        } catch (const Error &) { threw = true; }
+        if (!threw) { printf("FAIL: dimension mismatch did not throw\n"); failures++; }
+        backend.Close();
+        printf(failures ? "host mirror: %d FAILURES\n" : "host mirror: all ok\n", failures);
+        return failures ? 1 : 0;
+    } catch (const Error &e) {
+        printf("FAIL: mi_qmm error %d: %s\n", e.code, e.what());
+        return 2;
+    }
+}

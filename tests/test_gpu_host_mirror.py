@@ -1,0 +1,73 @@
+"""The host-side mirrors of the reference's ml.Backend / ml.Context / ml.Tensor interface
+(/root/reference/ml/backend.go:16-33, 94-128, 130-153) driven the way a model's forward pass drives
+them -- Get the weights, FromFloats the activations, Mulmat, Compute, Floats -- and checked against
+the CPU oracle."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import npref
+import oracle
+from ollama_amd import qmm
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_python_mirror_layer_graph():
+    from ollama_amd import ml
+
+    k = 2048
+    rng = np.random.default_rng(8)
+    spec = {}
+    raws = {}
+    for name, t, m in [("blk.0.attn_q.weight", qmm.Q4_K, 2048), ("blk.0.attn_k.weight", qmm.Q4_K, 512),
+                       ("blk.0.attn_v.weight", qmm.Q4_K, 512), ("blk.0.ffn_gate.weight", qmm.Q4_K, 1536),
+                       ("blk.0.ffn_up.weight", qmm.Q4_K, 1536), ("blk.0.ffn_down.weight", qmm.Q6_K, 640),
+                       ("output.weight", qmm.Q8_0, 1000), ("token_embd.weight", qmm.Q4_0, 96)]:
+        raw = oracle.quantize(t, (rng.standard_normal((m, k), dtype=np.float32) * np.float32(0.02)), nthreads=8)
+        spec[name] = (t, [k, m], raw)
+        raws[name] = (t, m, raw)
+    seen = []
+    b = ml.Backend(spec)
+    b.Load(progress=seen.append)
+    assert seen and seen[-1] == 1.0
+    assert b.Get("nope.weight") is None
+    w = b.Get("output.weight")
+    assert w.Shape() == [k, 1000] and w.DType() == ml.DType.Q80 and w.Dim(1) == 1000
+    assert w.Stride(0) == 34 and w.Stride(1) == qmm.row_size(qmm.Q8_0, k)
+    assert w.Bytes() == raws["output.weight"][2].tobytes()
+    for n in (1, 5, 48):   # decode, skinny, prefill-sized (GEMM for the K-quants)
+        ctx = b.NewContext()
+        xv = rng.standard_normal((n, k), dtype=np.float32)
+        x = ctx.FromFloats(xv.reshape(-1), k, n)
+        outs = {name: b.Get(name).Mulmat(ctx, x) for name in spec}
+        full = b.Get("blk.0.attn_q.weight").MulmatFullPrec(ctx, x)
+        with pytest.raises(RuntimeError):
+            outs["output.weight"].Floats()      # lazy until Compute
+        ctx.Compute(*outs.values())
+        for name, out in outs.items():
+            t, m, raw = raws[name]
+            assert out.Shape() == [m, n] and out.DType() == ml.DType.F32
+            want = oracle.mul_mat(t, raw, k, m, xv, nthreads=8)
+            assert npref.rel_err(out.Floats().reshape(n, m), want) <= 1e-3, (name, n)
+        assert np.array_equal(full.Floats(), outs["blk.0.attn_q.weight"].Floats())
+        ctx.Close()
+    ctx = b.NewContext()
+    with pytest.raises(ValueError):
+        b.Get("output.weight").Mulmat(ctx, ctx.FromFloats(np.zeros(512, np.float32), 512, 1))
+    with pytest.raises(TypeError):
+        ctx.FromFloats(np.zeros(k, np.float32), k, 1).Mulmat(ctx, ctx.FromFloats(np.zeros(k, np.float32), k, 1))
+    b.Close()
+
+
+def test_cpp_mirror_program():
+    exe = os.path.join(ROOT, "tests", "cpp", "test_host_mirror")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} is not built; run __graft_entry__.build()")
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(p.stdout, p.stderr)
+    assert p.returncode == 0, p.stdout[-2000:] + p.stderr[-2000:]
+    assert "host mirror: all ok" in p.stdout
