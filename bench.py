@@ -44,7 +44,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=32, help="distinct FFN weight sets in the rotating pool")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget (0 = skip)")
-    ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the batch-512 prefill GEMM section")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic, for scaling rocprofv3 HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path has no multi-GPU part); use --gpus 1",
@@ -169,6 +171,71 @@ def main() -> int:
             "bytes_per_launch": int(bytes_per_launch),
         },
     }
+
+    # ---- prefill GEMM: one Llama-3-8B-shaped layer at batch 512 (secondary metric of BASELINE.json)
+    if not args.no_gemm:
+        NB = 512
+        layer = [("attn_q", Q4_K, 4096, 4096), ("attn_k", Q4_K, 1024, 4096), ("attn_v", Q4_K, 1024, 4096),
+                 ("attn_o", Q4_K, 4096, 4096), ("ffn_gate", Q4_K, 14336, 4096), ("ffn_up", Q4_K, 14336, 4096),
+                 ("ffn_down", Q6_K, 4096, 14336)]
+        small = {}
+        for name, t, m, k in layer:
+            if (t, m, k) not in small:
+                rows = min(m, 2048)
+                raw = synth.weights(t, rows, k, seed=1005 + m % 89)
+                small[(t, m, k)] = np.tile(raw, ((m + rows - 1) // rows, 1))[:m]
+        copies = 3  # rotate three copies of the layer (414 MB) so weights are not cache-resident
+        gw = [[ctx.upload(t, np.roll(small[(t, m, k)], 11 * c, axis=0), k, m) for name, t, m, k in layer]
+              for c in range(copies)]
+        xb = torch.randn(NB, 4096, generator=g, dtype=torch.float32).to(dev)
+        hb = torch.randn(NB, 14336, generator=g, dtype=torch.float32).to(dev)
+        ys = [torch.empty(NB, m, dtype=torch.float32, device=dev) for name, t, m, k in layer]
+        actb_x = ctx.act_create(Q8_K, 4096, NB)
+        actb_h = ctx.act_create(Q8_K, 14336, NB)
+
+        def layer_pass():
+            for c in range(copies):
+                ctx.act_quantize(actb_x, xb.data_ptr(), NB, qmm.DEVICE)
+                for i in range(6):
+                    ctx.mulmat_q8_device(gw[c][i], actb_x, ys[i].data_ptr())
+                ctx.act_quantize(actb_h, hb.data_ptr(), NB, qmm.DEVICE)
+                ctx.mulmat_q8_device(gw[c][6], actb_h, ys[6].data_ptr())
+
+        layer_pass()
+        gsteps = max(2, args.steps // 4)
+        t_g = timed(layer_pass, gsteps) / (gsteps * copies)
+        ops = sum(2.0 * NB * m * k for name, t, m, k in layer)
+        per = {}
+        for i, (name, t, m, k) in enumerate(layer):
+            if name in ("attn_v", "ffn_up", "attn_o"):
+                continue
+            act = actb_h if k == 14336 else actb_x
+            fn = lambda i=i, act=act: [ctx.mulmat_q8_device(gw[c][i], act, ys[i].data_ptr()) for c in range(copies)]
+            fn()
+            tm = timed(fn, gsteps) / (gsteps * copies)
+            per[name] = {"us": round(tm * 1e6, 1), "tops": round(2.0 * NB * m * k / tm / 1e12, 1)}
+        out["gemm"] = {
+            "metric": "prefill GEMM TOPS (int8 MFMA)",
+            "workload": "one Llama-3-8B-shaped layer, batch 512: q/o 4096x4096, k/v 1024x4096, gate/up 14336x4096 Q4_K; "
+                        "down 4096x14336 Q6_K; activations quantized to Q8_K on GPU inside the timed region",
+            "value": round(ops / t_g / 1e12, 1),
+            "unit": "TOPS",
+            "us_per_layer": round(t_g * 1e6, 1),
+            "gop_per_layer": round(ops / 1e9, 2),
+            "roofline": {"bound": "mfma", "achieved": round(ops / t_g / 1e12, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": round(ops / t_g / 1e12 / INT8_PEAK_TOPS, 4)},
+            "per_matrix": per,
+        }
+        for row in gw:
+            for wt in row:
+                wt.free()
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     # ---- CPU baseline: the oracle (scalar port of the ggml CPU path) on this host's cores -------
     if args.cpu_seconds > 0:
