@@ -481,25 +481,20 @@ __global__ __launch_bounds__(512, 2) void gemv_kernel(MultiArgs ma, DevAct a, in
             for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg + s * kw, lane, g[s], act[s][n]);
 #endif
         load_pass<P, SPW, U>(w, g, bufB, rbase, rw, U, nrw);  // clamped to the last row if nrw <= U
-        // steady state: no branches around the loads, so each compute waits for its own pass only
+        // Steady state: no branches around the loads, so the compiler can make each compute pass wait
+        // for exactly its own loads while the next pass stays in flight.  The loop runs as long as rows
+        // remain beyond the two loaded passes; loads that reach past the wave's last row re-read that
+        // row (at most 2U-1 redundant row loads per wave, served by the caches).
         int i0 = 0;
-        for (; i0 + 4 * U <= nrw; i0 += 2 * U) {
+        for (; i0 + 2 * U < nrw; i0 += 2 * U) {
             compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0, nrw, lane, kseg, kw, part, yrow0, ldy);
             load_pass<P, SPW, U>(w, g, bufA, rbase, rw, i0 + 2 * U, nrw);
             compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + U, nrw, lane, kseg, kw, part, yrow0, ldy);
             load_pass<P, SPW, U>(w, g, bufB, rbase, rw, i0 + 3 * U, nrw);
         }
-        // tail: fewer than 4U rows left, of which up to 2U are already loaded
         compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0, nrw, lane, kseg, kw, part, yrow0, ldy);
-        const bool more_a = i0 + 2 * U < nrw, more_b = i0 + 3 * U < nrw;
-        if (more_a) load_pass<P, SPW, U>(w, g, bufA, rbase, rw, i0 + 2 * U, nrw);
         if (i0 + U < nrw)
             compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + U, nrw, lane, kseg, kw, part, yrow0, ldy);
-        if (more_b) load_pass<P, SPW, U>(w, g, bufB, rbase, rw, i0 + 3 * U, nrw);
-        if (more_a)
-            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufA, rg, rw, i0 + 2 * U, nrw, lane, kseg, kw, part, yrow0, ldy);
-        if (more_b)
-            compute_pass<P, NC, SPW, U, DIRECT>(g, act, bufB, rg, rw, i0 + 3 * U, nrw, lane, kseg, kw, part, yrow0, ldy);
     }
     if (DIRECT) return;
 
