@@ -22,6 +22,8 @@
 //     flight; for the FFN shapes that is every row the wave owns, i.e. one exposed HBM latency.
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
+
 #include "internal.h"
 
 namespace miqmm {
@@ -89,9 +91,9 @@ __device__ __forceinline__ float reduce_rows(const float (&v)[U], int lane) {
 
 struct PolQ4K {
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
+    static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;  // Q8_K: one scale per 256, one sum per 16
+    static constexpr bool USES_BSUMS = true;
     static constexpr bool HEAVY = true;
-    static constexpr int WGS_PER_CU = 1;  // few fat waves: up to 256 VGPRs, 8 rows in flight each
-    static constexpr int U1 = 4, U2 = 2;  // rows per pass for one / two activation columns
     // lane c (0..3) of a super-block owns qs bytes [32c, 32c+32): low nibbles are sub-block 2c,
     // high nibbles sub-block 2c+1 (32 elements each), and with them scales/mins 2c and 2c+1.
     struct Geo {
@@ -116,7 +118,8 @@ struct PolQ4K {
         g.hi = c >= 2;
         return g;
     }
-    static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
+    template <class AV>
+    static __device__ __forceinline__ void load_act(const AV &a, int n, int seg, int lane, const Geo &g, Act &r) {
         const int sb = g.live ? seg * 16 + (lane >> 2) : 0, c = lane & 3;
         const int keep = g.live ? -1 : 0;
         const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)sb * QKK + 64 * c);
@@ -141,10 +144,6 @@ struct PolQ4K {
     }
     template <int NC>
     static __device__ __forceinline__ void dot(const Raw &r, const Geo &g, const Act (&a)[NC], float (&acc)[NC]) {
-#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 1 || GEMV_VARIANT == 5)
-        acc[0] += __int_as_float((r.hdr.x ^ r.hdr.y ^ r.hdr.z ^ r.hdr.w ^ r.q0.x ^ r.q0.y ^ r.q0.z ^ r.q0.w ^ r.q1.x ^ r.q1.y ^ r.q1.z ^ r.q1.w) & 0x3fffffff) + a[0].d;
-        return;
-#endif
         // hdr.x = d | dmin<<16 ; hdr.y = scales[0..3] ; hdr.z = scales[4..7] ; hdr.w = scales[8..11]
         const float dw = h2f(r.hdr.x & 0xffff), dminw = h2f(r.hdr.x >> 16);
         const unsigned ty = r.hdr.y >> g.sh, tz = r.hdr.z >> g.sh, tw = r.hdr.w >> g.sh;
@@ -179,9 +178,9 @@ struct PolQ4K {
 
 struct PolQ4_0 {
     static constexpr int SEG = 2048;  // 64 blocks, one per lane
+    static constexpr int ACT_BLK = QK, ACT_BSUM = QK;  // Q8_0: one scale and one sum per 32
+    static constexpr bool USES_BSUMS = true;
     static constexpr bool HEAVY = false;
-    static constexpr int WGS_PER_CU = 2;
-    static constexpr int U1 = 4, U2 = 4;
     struct Geo { int64_t qrow, drow; int blk; bool live; };
     struct Act { int q[8]; float d; int s8; };
     struct Raw { uint4 qv; unsigned dh; };
@@ -195,7 +194,8 @@ struct PolQ4_0 {
         g.drow = w.K / QK;
         return g;
     }
-    static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
+    template <class AV>
+    static __device__ __forceinline__ void load_act(const AV &a, int n, int seg, int lane, const Geo &g, Act &r) {
         const int keep = g.live ? -1 : 0;
         const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.blk * QK);
         const int4 lo = q[0], hi = q[1];
@@ -237,9 +237,9 @@ struct PolQ4_0 {
 
 struct PolQ8_0 {
     static constexpr int SEG = 1024;  // 32 blocks, two lanes (16 quants each) per block
+    static constexpr int ACT_BLK = QK, ACT_BSUM = QK;
+    static constexpr bool USES_BSUMS = false;
     static constexpr bool HEAVY = false;
-    static constexpr int WGS_PER_CU = 2;
-    static constexpr int U1 = 4, U2 = 4;
     struct Geo { int64_t qrow, drow; int hb; bool live; };
     struct Act { int q[4]; float d; };
     struct Raw { uint4 qv; unsigned dh; };
@@ -253,7 +253,8 @@ struct PolQ8_0 {
         g.drow = w.K / QK;
         return g;
     }
-    static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
+    template <class AV>
+    static __device__ __forceinline__ void load_act(const AV &a, int n, int seg, int lane, const Geo &g, Act &r) {
         const int keep = g.live ? -1 : 0;
         const int4 v = *reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.hb * 16);
         const float dd = a.d[(int64_t)n * (a.K / QK) + (g.hb >> 1)];
@@ -282,9 +283,9 @@ struct PolQ8_0 {
 
 struct PolQ6K {
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
+    static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;  // Q8_K: one scale per 256, one sum per 16
+    static constexpr bool USES_BSUMS = true;
     static constexpr bool HEAVY = true;
-    static constexpr int WGS_PER_CU = 1;  // few fat waves: up to 256 VGPRs, 8 rows in flight each
-    static constexpr int U1 = 2, U2 = 1;
     // lane (h = l4>>1, t = l4&1) of a super-block owns, in half h (128 elements):
     //   ql bytes [64h+16t, +16) and [64h+32+16t, +16), qh bytes [32h+16t, +16)
     // which hold four runs of 16 elements e = 128h + 16t + 32r + i (r = 0..3):
@@ -311,7 +312,8 @@ struct PolQ6K {
         g.e0 = 128 * h + 16 * t;
         return g;
     }
-    static __device__ __forceinline__ void load_act(const DevAct &a, int n, int seg, int lane, const Geo &g, Act &r) {
+    template <class AV>
+    static __device__ __forceinline__ void load_act(const AV &a, int n, int seg, int lane, const Geo &g, Act &r) {
         const int keep = g.live ? -1 : 0;
         const int8_t *q = a.qs + (int64_t)n * a.K + (int64_t)g.sb * QKK + g.e0;
         const int16_t *bs = a.bsums + (int64_t)n * (a.K / 16) + (int64_t)g.sb * 16 + (g.e0 >> 4);
@@ -411,18 +413,9 @@ __device__ __forceinline__ void compute_pass(const typename P::Geo (&g)[SPW],
     const int rl = rl0 + (i0 + u) * rw;  // row index inside the workgroup's range
 #pragma unroll
     for (int n = 0; n < NC; n++) {
-#if defined(GEMV_VARIANT) && GEMV_VARIANT == 2
-        float tot = 0.f;
-        for (int uu = 0; uu < U; uu++) tot += acc[n][uu];
-#else
         const float tot = reduce_rows<U>(acc[n], lane);
-#endif
         if (writer) {
-#if defined(GEMV_VARIANT) && GEMV_VARIANT == 4
-            if (DIRECT && tot == 1234.5f) yrow0[(int64_t)n * ldy + rl] = tot;
-#else
             if (DIRECT) yrow0[(int64_t)n * ldy + rl] = tot;
-#endif
             else part[(rl * NC + n) * kw + kseg] = tot;
         }
     }
@@ -472,14 +465,10 @@ __global__ __launch_bounds__(512, 2) void gemv_kernel(MultiArgs ma, DevAct a, in
         const int64_t rbase = r0 + rg;
         load_pass<P, SPW, U>(w, g, bufA, rbase, rw, 0, nrw);
         typename P::Act act[SPW][NC];
-#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 3 || GEMV_VARIANT == 5)
-        __builtin_memset(act, 1, sizeof(act));
-#else
 #pragma unroll
         for (int s = 0; s < SPW; s++)
 #pragma unroll
             for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg + s * kw, lane, g[s], act[s][n]);
-#endif
         load_pass<P, SPW, U>(w, g, bufB, rbase, rw, U, nrw);  // clamped to the last row if nrw <= U
         // Steady state: no branches around the loads, so the compiler can make each compute pass wait
         // for exactly its own loads while the next pass stays in flight.  The loop runs as long as rows
@@ -507,6 +496,147 @@ __global__ __launch_bounds__(512, 2) void gemv_kernel(MultiArgs ma, DevAct a, in
     }
 }
 
+// Sum over the 64 lanes; the total is valid in lanes 48..63.  Cross-lane moves only (quad swaps,
+// rotations inside rows of 16, then the row broadcasts), no LDS round trip.
+template <int CTRL, int ROWS>
+__device__ __forceinline__ float dpp_row(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROWS, 0xf, false));
+}
+__device__ __forceinline__ float wave_total(float w) {
+    w += dpp_mov<0xB1>(w);
+    w += dpp_mov<0x4E>(w);
+    w += dpp_mov<0x124>(w);
+    w += dpp_mov<0x128>(w);
+    w += dpp_row<0x142, 0xa>(w);  // row_bcast:15 -- lane 15 of rows 0 and 2 into rows 1 and 3
+    w += dpp_row<0x143, 0xc>(w);  // row_bcast:31 -- lane 31 into rows 2 and 3
+    return w;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The thin-wave kernel: many small waves instead of a few unrolled ones.
+//
+// A dispatch starts with a cold instruction cache, and straight-line code is fetched at roughly
+// 0.2 us per KiB -- an unrolled, double-buffered 8 KiB kernel spends a fifth of a 33 MB launch
+// fetching itself.  Here a wave runs a rolled loop over a handful of rows (one row of weights in
+// registers, the next one in flight), the body is about 1 KiB, and the memory-level parallelism
+// comes from occupancy: 6-8 waves per SIMD, each with a row in flight.
+// ---------------------------------------------------------------------------------------------
+// The activations as the kernel sees them once staged in LDS: same layout as DevAct, columns
+// col0 .. col0+NC-1 only.
+struct LdsAct {
+    const int8_t *qs;
+    const float *d;
+    const int16_t *bsums;
+    int64_t K;
+};
+
+// Kernel arguments of the thin kernel, arranged so that the tensor a workgroup belongs to is picked
+// with compares and selects on values that are all fetched by one batch of scalar loads: a select
+// chain that indexes the argument block with a computed index makes each pointer load wait for the
+// previous one, a microsecond of latency before the first HBM request.
+struct ThinArgs {
+    const uint8_t *p0[MAX_MULTI], *p1[MAX_MULTI], *p2[MAX_MULTI];
+    const uint16_t *d[MAX_MULTI];
+    float *y[MAX_MULTI];
+    int64_t M[MAX_MULTI];
+    int wg_end[MAX_MULTI];  // exclusive end of each tensor's workgroup range; INT_MAX past the last tensor
+    int64_t K;
+    int type;
+};
+
+template <class P, int NC, bool DIRECT, bool STAGE>
+__global__ __launch_bounds__(512, 2) void gemv_thin_kernel(ThinArgs ta, DevAct a, int col0, int rows_per_wave,
+                                                        int kw, int rw_log2) {
+    // LDS: the NC activation columns (quants, block scales, block sums), then, unless DIRECT, the
+    // partial sums [rows_per_wg][NC][kw].
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int bid = blockIdx.x;
+    const int e0 = ta.wg_end[0], e1 = ta.wg_end[1], e2 = ta.wg_end[2];
+    const int t = (bid >= e0) + (bid >= e1) + (bid >= e2);
+    const int wg = bid - (t == 0 ? 0 : t == 1 ? e0 : t == 2 ? e1 : e2);
+#define THIN_SEL(f) (t == 0 ? ta.f[0] : t == 1 ? ta.f[1] : t == 2 ? ta.f[2] : ta.f[3])
+    const DevWeight w{THIN_SEL(p0), THIN_SEL(p1), THIN_SEL(p2), THIN_SEL(d), ta.K, THIN_SEL(M), ta.type};
+    float *__restrict__ y = THIN_SEL(y);
+#undef THIN_SEL
+    const int64_t ldy = w.M;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = 1 << rw_log2;
+    const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
+    const int rows_per_wg = rows_per_wave << rw_log2;
+    const int64_t r0 = (int64_t)wg * rows_per_wg;
+    const int nrows = (int)min((int64_t)rows_per_wg, w.M - r0);
+    const int rl0 = rg * rows_per_wave;                    // the wave's rows: r0 + rl0 + i, i < nrw
+    const int nrw = max(0, min(rows_per_wave, nrows - rl0));
+    float *yrow0 = y + (int64_t)col0 * ldy + r0;
+
+    const typename P::Geo g = P::geo(w, kseg, lane);
+    typename P::Raw cur;
+    if (nrw > 0) cur = P::load(w, g, r0 + rl0);  // weights first: nothing ahead of the HBM request
+
+    // Optionally stage the activations in LDS once per workgroup instead of loading them per wave.
+    const int64_t K = a.K;
+    const int nblk = (int)(K / P::ACT_BLK);
+    const int nbs = P::USES_BSUMS ? (int)(K / P::ACT_BSUM) : 0;
+    const size_t act_bytes = STAGE ? (((size_t)NC * (K + nblk * 4 + nbs * 2)) + 15) / 16 * 16 : 0;
+    int8_t *lqs = reinterpret_cast<int8_t *>(smem);
+    float *ld_ = reinterpret_cast<float *>(smem + (size_t)NC * K);
+    int16_t *lbs = reinterpret_cast<int16_t *>(smem + (size_t)NC * K + (size_t)NC * nblk * 4);
+    if (STAGE) {
+        const int4 *src = reinterpret_cast<const int4 *>(a.qs + (int64_t)col0 * K);
+        for (int i = threadIdx.x; i < NC * (int)(K / 16); i += blockDim.x) reinterpret_cast<int4 *>(lqs)[i] = src[i];
+        const float *sd = a.d + (int64_t)col0 * nblk;
+        for (int i = threadIdx.x; i < NC * nblk; i += blockDim.x) ld_[i] = sd[i];
+        if (P::USES_BSUMS) {
+            const int16_t *sb = a.bsums + (int64_t)col0 * nbs;
+            for (int i = threadIdx.x; i < NC * nbs; i += blockDim.x) lbs[i] = sb[i];
+        }
+        __syncthreads();
+    }
+    float *part = reinterpret_cast<float *>(smem + act_bytes);
+
+    if (nrw > 0) {
+        typename P::Act act[NC];
+        if (STAGE) {
+            const LdsAct la{lqs, ld_, lbs, K};
+#pragma unroll
+            for (int n = 0; n < NC; n++) P::load_act(la, n, kseg, lane, g, act[n]);
+        } else {
+#pragma unroll
+            for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg, lane, g, act[n]);
+        }
+        float keep[NC];  // lane 63-i ends up holding the total of the wave's row i
+#pragma unroll
+        for (int n = 0; n < NC; n++) keep[n] = 0.f;
+#pragma unroll 1
+        for (int i = 0; i < nrw; i++) {
+            float acc[NC];
+#pragma unroll
+            for (int n = 0; n < NC; n++) acc[n] = 0.f;
+            P::template dot<NC>(cur, g, act, acc);
+            if (i + 1 < nrw) cur = P::load(w, g, r0 + rl0 + i + 1);  // wave-uniform branch
+#pragma unroll
+            for (int n = 0; n < NC; n++) {
+                const float tot = wave_total(acc[n]);  // valid in lanes 48..63
+                if (DIRECT) keep[n] = lane == 63 - i ? tot : keep[n];
+                else if (lane == 63) part[((rl0 + i) * NC + n) * kw + kseg] = tot;
+            }
+        }
+        if (DIRECT && lane > 63 - nrw) {
+#pragma unroll
+            for (int n = 0; n < NC; n++) yrow0[(int64_t)n * ldy + rl0 + (63 - lane)] = keep[n];
+        }
+    }
+    if (DIRECT) return;
+
+    __syncthreads();
+    for (int i = threadIdx.x; i < nrows * NC; i += blockDim.x) {
+        const int n = i / nrows, rl = i - n * nrows;
+        float sum = 0.f;
+        for (int k = 0; k < kw; k++) sum += part[(rl * NC + n) * kw + k];
+        yrow0[(int64_t)n * ldy + rl] = sum;
+    }
+}
+
 struct Plan { int kw, rw, rw_log2, spw, rows_per_wg; unsigned grid; size_t lds; };
 
 // 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), one or two workgroups per CU.
@@ -520,7 +650,7 @@ bool make_plan(int64_t K, int64_t total_m, int nc, int num_cus, Plan &p) {
     p.kw = (nseg + p.spw - 1) / p.spw;
     p.rw_log2 = p.kw >= 5 ? 0 : p.kw >= 3 ? 1 : p.kw == 2 ? 2 : 3;  // largest power of two with kw*rw <= 8
     p.rw = 1 << p.rw_log2;
-    const int64_t target_wgs = (int64_t)num_cus * P::WGS_PER_CU;
+    const int64_t target_wgs = (int64_t)num_cus * (P::HEAVY ? 1 : 2);
     int64_t rows = (total_m + target_wgs - 1) / target_wgs;
     const int64_t lds_cap_rows = 8192 / (nc * p.kw);  // <= 32 KiB of partials
     if (rows > lds_cap_rows) rows = lds_cap_rows;
@@ -528,6 +658,35 @@ bool make_plan(int64_t K, int64_t total_m, int nc, int num_cus, Plan &p) {
     p.rows_per_wg = (int)rows;
     p.lds = p.kw == 1 ? 0 : (size_t)rows * nc * p.kw * sizeof(float);
     return true;
+}
+
+// Thin plan: kw waves side by side along K (one segment each) times rw row groups, four waves per
+// workgroup (kw of them when K has more than four segments), a few consecutive rows per wave.
+constexpr size_t THIN_LDS_MAX = 64 * 1024;
+
+template <class P>
+bool make_thin_plan(int64_t K, int64_t total_m, int nc, int rows_per_wave, Plan &p) {
+    const int nseg = (int)((K + P::SEG - 1) / P::SEG);
+    if (nseg < 1 || nseg > 8) return false;
+    p.spw = 1;
+    p.kw = nseg;
+    p.rw_log2 = p.kw >= 3 ? 0 : p.kw == 2 ? 1 : 2;
+    p.rw = 1 << p.rw_log2;
+    if (rows_per_wave <= 0) rows_per_wave = (nc >= 4 || total_m > 65536) ? 4 : 2;
+    if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
+    p.rows_per_wg = p.rw * rows_per_wave;
+    p.lds = p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float);
+    return p.lds <= THIN_LDS_MAX;
+}
+
+template <class P, int NC>
+void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, int col0, hipStream_t s) {
+    const dim3 block(64 * p.kw * p.rw);
+    const int rpw = p.rows_per_wg >> p.rw_log2;
+    if (p.kw == 1)
+        gemv_thin_kernel<P, NC, true, false><<<p.grid, block, p.lds, s>>>(ma, a, col0, rpw, p.kw, p.rw_log2);
+    else
+        gemv_thin_kernel<P, NC, false, false><<<p.grid, block, p.lds, s>>>(ma, a, col0, rpw, p.kw, p.rw_log2);
 }
 
 template <class P, int NC, int SPW, int U>
@@ -545,8 +704,14 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i].M;
     Plan p;
-    if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
-    if (p.spw > 1 && !make_plan<P>(ws[0].K, total_m, 1, num_cus, p)) return hipErrorInvalidValue;
+    static const char *mode_env = getenv("MI_QMM_GEMV_DEBUG");  // "fat" | "thin[:rows_per_wave]"
+    const bool force_fat = mode_env && mode_env[0] == 'f';
+    const int rpw_env = mode_env && mode_env[0] == 't' && mode_env[4] == ':' ? atoi(mode_env + 5) : 0;
+    const bool thin = !force_fat && make_thin_plan<P>(ws[0].K, total_m, nc, rpw_env, p);
+    if (!thin) {
+        if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
+        if (p.spw > 1 && !make_plan<P>(ws[0].K, total_m, 1, num_cus, p)) return hipErrorInvalidValue;
+    }
     MultiArgs ma;
     ma.count = count;
     int64_t wgs = 0;
@@ -558,6 +723,28 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
     }
     if (wgs > 0x7fffffff) return hipErrorInvalidValue;
     p.grid = (unsigned)wgs;
+    if (thin) {
+        ThinArgs ta;
+        for (int i = 0; i < MAX_MULTI; i++) {
+            const int j = i < count ? i : count - 1;
+            ta.p0[i] = ws[j].p0; ta.p1[i] = ws[j].p1; ta.p2[i] = ws[j].p2; ta.d[i] = ws[j].d;
+            ta.y[i] = ys[j]; ta.M[i] = ws[j].M;
+            ta.wg_end[i] = i < count ? ma.wg_end[i] : 0x7fffffff;
+        }
+        ta.K = ws[0].K; ta.type = ws[0].type;
+        switch (nc) {
+        case 1: launch_thin<P, 1>(p, ta, a, col0, s); break;
+        case 2: launch_thin<P, 2>(p, ta, a, col0, s); break;
+        case 3: launch_thin<P, 3>(p, ta, a, col0, s); break;
+        case 4: launch_thin<P, 4>(p, ta, a, col0, s); break;
+        case 5: launch_thin<P, 5>(p, ta, a, col0, s); break;
+        case 6: launch_thin<P, 6>(p, ta, a, col0, s); break;
+        case 7: launch_thin<P, 7>(p, ta, a, col0, s); break;
+        case 8: launch_thin<P, 8>(p, ta, a, col0, s); break;
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     if (p.spw > 1) {
         // long rows: several segments per wave, one column per launch
         for (int c = col0; c < col0 + nc; c++) {
@@ -566,19 +753,7 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
         }
         return hipGetLastError();
     }
-    constexpr int UB = P::HEAVY ? 1 : 2;
-    switch (nc) {
-    case 1: launch_one<P, 1, 1, P::U1>(p, ma, a, col0, s); break;
-    case 2: launch_one<P, 2, 1, P::U2>(p, ma, a, col0, s); break;
-    case 3: launch_one<P, 3, 1, UB>(p, ma, a, col0, s); break;
-    case 4: launch_one<P, 4, 1, UB>(p, ma, a, col0, s); break;
-    case 5: launch_one<P, 5, 1, UB>(p, ma, a, col0, s); break;
-    case 6: launch_one<P, 6, 1, UB>(p, ma, a, col0, s); break;
-    case 7: launch_one<P, 7, 1, UB>(p, ma, a, col0, s); break;
-    case 8: launch_one<P, 8, 1, UB>(p, ma, a, col0, s); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
+    return hipErrorInvalidValue;  // not reached: K within eight segments always takes the thin plan
 }
 
 }  // namespace

@@ -77,7 +77,8 @@ def test_quantize_act_empty_and_errors(ctx):
 
 
 # ---- kernels 2/4: GEMV, small and ragged shapes ---------------------------------------------------
-SMALL = [(256, 1), (256, 7), (512, 33), (1024, 100), (2048, 64), (2304, 5), (4096, 257), (6144, 31), (14336, 19)]
+SMALL = [(256, 1), (256, 7), (512, 33), (1024, 100), (2048, 64), (2304, 5), (4096, 257), (6144, 31), (14336, 19),
+         (28672, 3)]
 
 
 @pytest.mark.parametrize("t", WTYPES)
