@@ -112,6 +112,14 @@ int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64
                   int location);
 int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n,
                        float *y, int location, int path);
+/* several weights of the same k against the same f32 activations x [n][k]: ys[i] receives
+ * f32 [n][m_i].  These are the mul_mat nodes of one graph that share src1 (gate and up, or q/k/v),
+ * which Context.Compute (/root/reference/ml/backend.go:110) sees together.  For weights of one
+ * type, n <= 8 and count <= 4 this is ONE kernel launch: the decode GEMV quantizes x in its
+ * prologue and walks the concatenated rows of all weights.  Otherwise it is the same as calling
+ * mi_qmm_mulmat per weight. */
+int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x,
+                        int64_t n, float *const *ys, int location);
 
 /* ---- two-phase form: quantize once, multiply by several weights (gate and up, or q/k/v, share
  *      one x).  In ggml's graph the from_float step belongs to each mul_mat node; a backend that

@@ -456,10 +456,16 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         dy = (float *)((char *)ctx->io_buf + yoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
-    DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
-    if ((rc = run_product(ctx, w, a, dy, path))) return rc;
+    if (path != MI_QMM_PATH_GEMM && n <= 8 && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
+        // decode: one launch, the GEMV quantizes x in its prologue
+        float *ys[1] = {dy};
+        HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
+    } else {
+        HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+        DevAct a;
+        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
+        if ((rc = run_product(ctx, w, a, dy, path))) return rc;
+    }
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -469,6 +475,62 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
 
 int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location) {
     return mi_qmm_mulmat_path(ctx, w, x, n, y, location, MI_QMM_PATH_AUTO);
+}
+
+int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x, int64_t n,
+                        float *const *ys, int location) {
+    if (!ws || !ys || count < 1) return fail(MI_QMM_ERR_INVALID, "ws/ys is NULL or count < 1");
+    for (int i = 0; i < count; i++)
+        if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
+    if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
+    bool same_type = true;
+    for (int i = 1; i < count; i++) {
+        if (ws[i]->dev.K != ws[0]->dev.K)
+            return fail(MI_QMM_ERR_INVALID, "ws[%d] has k=%lld, ws[0] has k=%lld: one x cannot serve both", i,
+                        (long long)ws[i]->dev.K, (long long)ws[0]->dev.K);
+        same_type = same_type && ws[i]->dev.type == ws[0]->dev.type;
+    }
+    const int64_t K = ws[0]->dev.K;
+    int64_t total_m = 0;
+    for (int i = 0; i < count; i++) total_m += ws[i]->dev.M;
+    if (!same_type || count > gemv_max_multi() || n > 8 || n == 0 ||
+        !gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)) {
+        for (int i = 0; i < count; i++) {
+            int rc = mi_qmm_mulmat_path(ctx, ws[i], x, n, ys[i], location, MI_QMM_PATH_AUTO);
+            if (rc) return rc;
+        }
+        return MI_QMM_OK;
+    }
+    int rc = check_product_args(ctx, ws[0], location, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    if (!x) return fail(MI_QMM_ERR_INVALID, "x is NULL");
+    DevWeight dw[8];
+    for (int i = 0; i < count; i++) {
+        if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
+        dw[i] = ws[i]->dev;
+    }
+    const size_t xbytes = (size_t)(n * K) * 4;
+    const float *dx = x;
+    float *dys[8];
+    size_t offs[9];
+    offs[0] = align_up(xbytes, 256);
+    for (int i = 0; i < count; i++) {
+        dys[i] = ys[i];
+        offs[i + 1] = offs[i] + align_up((size_t)(n * dw[i].M) * 4, 256);
+    }
+    if (location == MI_QMM_HOST) {
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
+        dx = (const float *)ctx->io_buf;
+        for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
+        HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    HIP_TRY(launch_gemv_f32_multi(dw, dys, count, dx, (int)n, ctx->num_cus, ctx->stream));
+    if (location == MI_QMM_HOST) {
+        for (int i = 0; i < count; i++)
+            HIP_TRY(hipMemcpyAsync(ys[i], dys[i], (size_t)(n * dw[i].M) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
 }
 
 // ---- two-phase form ----------------------------------------------------------------------------------

@@ -25,6 +25,7 @@
 #include <cstdlib>
 
 #include "internal.h"
+#include "quant_dev.h"
 
 namespace miqmm {
 
@@ -544,9 +545,12 @@ struct ThinArgs {
     int type;
 };
 
-template <class P, int NC, bool DIRECT, bool STAGE>
-__global__ __launch_bounds__(512, 2) void gemv_thin_kernel(ThinArgs ta, DevAct a, int col0, int rows_per_wave,
-                                                        int kw, int rw_log2) {
+// workgroup size limit: 16 waves leave a wave 128 VGPRs, enough for up to three activation columns
+constexpr int thin_max_waves(int nc, bool f32) { return f32 ? (nc <= 3 ? 16 : 8) : 4; }
+
+template <class P, int NC, bool DIRECT, bool F32>
+__global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(ThinArgs ta, DevAct a, const float *__restrict__ xf,
+                                                         int col0, int rows_per_wave, int kw, int rw_log2) {
     // LDS: the NC activation columns (quants, block scales, block sums), then, unless DIRECT, the
     // partial sums [rows_per_wg][NC][kw].
     extern __shared__ __align__(16) uint8_t smem[];
@@ -570,33 +574,72 @@ __global__ __launch_bounds__(512, 2) void gemv_thin_kernel(ThinArgs ta, DevAct a
     float *yrow0 = y + (int64_t)col0 * ldy + r0;
 
     const typename P::Geo g = P::geo(w, kseg, lane);
-    typename P::Raw cur;
-    if (nrw > 0) cur = P::load(w, g, r0 + rl0);  // weights first: nothing ahead of the HBM request
 
-    // Optionally stage the activations in LDS once per workgroup instead of loading them per wave.
-    const int64_t K = a.K;
+    // With f32 activations the workgroup quantizes them itself, into LDS, in the layout of DevAct
+    // (columns col0 .. col0+NC-1 only): a wave takes 256 consecutive elements at a time, the same
+    // lane-to-element mapping as the stand-alone quantization kernel, so the values are the same bits.
+    const int64_t K = ta.K;
     const int nblk = (int)(K / P::ACT_BLK);
     const int nbs = P::USES_BSUMS ? (int)(K / P::ACT_BSUM) : 0;
-    const size_t act_bytes = STAGE ? (((size_t)NC * (K + nblk * 4 + nbs * 2)) + 15) / 16 * 16 : 0;
+    const size_t act_bytes = F32 ? (((size_t)NC * (K + nblk * 4 + nbs * 2)) + 15) / 16 * 16 : 0;
     int8_t *lqs = reinterpret_cast<int8_t *>(smem);
     float *ld_ = reinterpret_cast<float *>(smem + (size_t)NC * K);
     int16_t *lbs = reinterpret_cast<int16_t *>(smem + (size_t)NC * K + (size_t)NC * nblk * 4);
-    if (STAGE) {
-        const int4 *src = reinterpret_cast<const int4 *>(a.qs + (int64_t)col0 * K);
-        for (int i = threadIdx.x; i < NC * (int)(K / 16); i += blockDim.x) reinterpret_cast<int4 *>(lqs)[i] = src[i];
-        const float *sd = a.d + (int64_t)col0 * nblk;
-        for (int i = threadIdx.x; i < NC * nblk; i += blockDim.x) ld_[i] = sd[i];
-        if (P::USES_BSUMS) {
-            const int16_t *sb = a.bsums + (int64_t)col0 * nbs;
-            for (int i = threadIdx.x; i < NC * nbs; i += blockDim.x) lbs[i] = sb[i];
+    // Order of the memory requests: the wave's pieces of x (L2 hits, they come back first), then its
+    // first row of weights (HBM).  The memory counter retires in order, so the quantization can start
+    // as soon as x is there while the weights are still in flight.
+    constexpr int XPRE = 4;  // pieces of x a wave requests ahead of its weights
+    const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col0 * K);
+    const int total4 = (int)((int64_t)NC * K / 4);  // float4 pieces over all NC columns
+    const int nwaves = blockDim.x >> 6;
+    float4 xpre[XPRE];
+    if (F32) {
+#pragma unroll
+        for (int j = 0; j < XPRE; j++) {
+            const int i4 = (wave + j * nwaves) * 64 + lane;
+            xpre[j] = x4[min(i4, total4 - 1)];  // clamped: the loads stay unconditional
         }
+    }
+    typename P::Raw cur;
+    if (nrw > 0) cur = P::load(w, g, r0 + rl0);
+    if (F32) {
+        auto quantize_piece = [&](int c, float4 v) {
+            const int i4 = c * 64 + lane;
+            const bool live = i4 < total4;  // Q8_0 only: K*NC need not be a multiple of 256
+            if (!live) v = make_float4(0.f, 0.f, 0.f, 0.f);
+            float dd;
+            if (P::ACT_BLK == QKK) {
+                int sum16, pair;
+                const int packed = q8_K_quantize_lane(v, lane, dd, sum16, pair);
+                reinterpret_cast<int *>(lqs)[i4] = packed;
+                if (lane == 0) ld_[c] = dd;
+                if (P::USES_BSUMS && (lane & 3) == 0) lbs[c * 16 + (lane >> 2)] = (int16_t)sum16;
+            } else {
+                int sum;
+                const int packed = q8_0_quantize_lane(v, dd, sum);
+                if (live) {
+                    reinterpret_cast<int *>(lqs)[i4] = packed;
+                    if ((lane & 7) == 0) {
+                        ld_[i4 >> 3] = dd;
+                        if (P::USES_BSUMS) lbs[i4 >> 3] = (int16_t)sum;
+                    }
+                }
+            }
+        };
+#pragma unroll
+        for (int j = 0; j < XPRE; j++) {
+            const int c = wave + j * nwaves;
+            if (c * 64 < total4) quantize_piece(c, xpre[j]);  // wave-uniform
+        }
+        for (int c = wave + XPRE * nwaves; c * 64 < total4; c += nwaves)
+            quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
         __syncthreads();
     }
     float *part = reinterpret_cast<float *>(smem + act_bytes);
 
     if (nrw > 0) {
         typename P::Act act[NC];
-        if (STAGE) {
+        if (F32) {
             const LdsAct la{lqs, ld_, lbs, K};
 #pragma unroll
             for (int n = 0; n < NC; n++) P::load_act(la, n, kseg, lane, g, act[n]);
@@ -660,33 +703,62 @@ bool make_plan(int64_t K, int64_t total_m, int nc, int num_cus, Plan &p) {
     return true;
 }
 
-// Thin plan: kw waves side by side along K (one segment each) times rw row groups, four waves per
-// workgroup (kw of them when K has more than four segments), a few consecutive rows per wave.
+// Thin plan: kw waves side by side along K (one segment each) times rw row groups, a few consecutive
+// rows per wave.  Four waves per workgroup (kw of them when K has more than four segments); with f32
+// activations the workgroup also quantizes all of x into LDS first, so it is made larger (up to 16
+// waves) to spread that work and to keep the number of times x is read from L2 down.
 constexpr size_t THIN_LDS_MAX = 64 * 1024;
 
 template <class P>
-bool make_thin_plan(int64_t K, int64_t total_m, int nc, int rows_per_wave, Plan &p) {
+size_t thin_act_lds(int64_t K, int nc) {
+    const size_t b = (size_t)nc * (K + K / P::ACT_BLK * 4 + (P::USES_BSUMS ? K / P::ACT_BSUM * 2 : 0));
+    return (b + 15) / 16 * 16;
+}
+
+template <class P>
+bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, int rows_per_wave, Plan &p) {
     const int nseg = (int)((K + P::SEG - 1) / P::SEG);
     if (nseg < 1 || nseg > 8) return false;
     p.spw = 1;
     p.kw = nseg;
-    p.rw_log2 = p.kw >= 3 ? 0 : p.kw == 2 ? 1 : 2;
+    const int max_waves = p.kw > thin_max_waves(nc, f32) ? p.kw : thin_max_waves(nc, f32);
+    p.rw_log2 = 0;
+    while (p.kw << (p.rw_log2 + 1) <= max_waves) p.rw_log2++;
+    static const char *rw_env = getenv("MI_QMM_GEMV_RW");
+    if (rw_env && f32) { p.rw_log2 = atoi(rw_env); while (p.kw << p.rw_log2 > thin_max_waves(nc, f32) && p.rw_log2 > 0) p.rw_log2--; }
     p.rw = 1 << p.rw_log2;
-    if (rows_per_wave <= 0) rows_per_wave = (nc >= 4 || total_m > 65536) ? 4 : 2;
+    if (rows_per_wave <= 0) {
+        if (f32) {
+            // every workgroup re-quantizes x: keep them to one resident round (at most 1.75 per CU),
+            // an even number of rows per wave
+            const int64_t rows_per_rw = (total_m + (int64_t)448 * p.rw - 1) / ((int64_t)448 * p.rw);
+            rows_per_wave = (int)((rows_per_rw + 1) / 2 * 2);
+            if (rows_per_wave < 2) rows_per_wave = 2;
+        } else {
+            rows_per_wave = (nc >= 4 || total_m > 65536) ? 4 : 2;
+        }
+    }
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
-    p.lds = p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float);
+    p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float));
     return p.lds <= THIN_LDS_MAX;
 }
 
 template <class P, int NC>
-void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, int col0, hipStream_t s) {
+void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, const float *xf, int col0, hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
     const int rpw = p.rows_per_wg >> p.rw_log2;
-    if (p.kw == 1)
-        gemv_thin_kernel<P, NC, true, false><<<p.grid, block, p.lds, s>>>(ma, a, col0, rpw, p.kw, p.rw_log2);
-    else
-        gemv_thin_kernel<P, NC, false, false><<<p.grid, block, p.lds, s>>>(ma, a, col0, rpw, p.kw, p.rw_log2);
+    if (xf) {
+        if (p.kw == 1)
+            gemv_thin_kernel<P, NC, true, true><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
+        else
+            gemv_thin_kernel<P, NC, false, true><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
+    } else {
+        if (p.kw == 1)
+            gemv_thin_kernel<P, NC, true, false><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
+        else
+            gemv_thin_kernel<P, NC, false, false><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
+    }
 }
 
 template <class P, int NC, int SPW, int U>
@@ -699,15 +771,16 @@ void launch_one(const Plan &p, const MultiArgs &ma, const DevAct &a, int col0, h
 }
 
 template <class P>
-hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int nc,
-                       int num_cus, hipStream_t s) {
+hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const DevAct &a, const float *xf, int col0,
+                       int nc, int num_cus, hipStream_t s) {
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i].M;
     Plan p;
     static const char *mode_env = getenv("MI_QMM_GEMV_DEBUG");  // "fat" | "thin[:rows_per_wave]"
     const bool force_fat = mode_env && mode_env[0] == 'f';
     const int rpw_env = mode_env && mode_env[0] == 't' && mode_env[4] == ':' ? atoi(mode_env + 5) : 0;
-    const bool thin = !force_fat && make_thin_plan<P>(ws[0].K, total_m, nc, rpw_env, p);
+    const bool thin = !force_fat && make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, rpw_env, p);
+    if (xf && !thin) return hipErrorInvalidValue;  // callers ask gemv_f32_supported() first
     if (!thin) {
         if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
         if (p.spw > 1 && !make_plan<P>(ws[0].K, total_m, 1, num_cus, p)) return hipErrorInvalidValue;
@@ -733,14 +806,14 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
         }
         ta.K = ws[0].K; ta.type = ws[0].type;
         switch (nc) {
-        case 1: launch_thin<P, 1>(p, ta, a, col0, s); break;
-        case 2: launch_thin<P, 2>(p, ta, a, col0, s); break;
-        case 3: launch_thin<P, 3>(p, ta, a, col0, s); break;
-        case 4: launch_thin<P, 4>(p, ta, a, col0, s); break;
-        case 5: launch_thin<P, 5>(p, ta, a, col0, s); break;
-        case 6: launch_thin<P, 6>(p, ta, a, col0, s); break;
-        case 7: launch_thin<P, 7>(p, ta, a, col0, s); break;
-        case 8: launch_thin<P, 8>(p, ta, a, col0, s); break;
+        case 1: launch_thin<P, 1>(p, ta, a, xf, col0, s); break;
+        case 2: launch_thin<P, 2>(p, ta, a, xf, col0, s); break;
+        case 3: launch_thin<P, 3>(p, ta, a, xf, col0, s); break;
+        case 4: launch_thin<P, 4>(p, ta, a, xf, col0, s); break;
+        case 5: launch_thin<P, 5>(p, ta, a, xf, col0, s); break;
+        case 6: launch_thin<P, 6>(p, ta, a, xf, col0, s); break;
+        case 7: launch_thin<P, 7>(p, ta, a, xf, col0, s); break;
+        case 8: launch_thin<P, 8>(p, ta, a, xf, col0, s); break;
         default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
@@ -770,20 +843,29 @@ int64_t gemv_max_k(int type) {
 
 int gemv_max_multi() { return MAX_MULTI; }
 
-hipError_t launch_gemv_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols,
-                             int num_cus, hipStream_t s) {
+namespace {
+
+hipError_t dispatch(const DevWeight *ws, float *const *ys, int count, const DevAct &a, const float *xf, int col0,
+                    int ncols, int num_cus, hipStream_t s) {
     if (count < 1 || count > MAX_MULTI || ncols < 1 || ncols > MAXC || col0 < 0 || col0 + ncols > a.N)
         return hipErrorInvalidValue;
     for (int i = 0; i < count; i++)
         if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || ws[i].M < 1 || !ys[i]) return hipErrorInvalidValue;
     if (ws[0].K < 1 || ws[0].K > gemv_max_k(ws[0].type) || a.K != ws[0].K) return hipErrorInvalidValue;
     switch (ws[0].type) {
-    case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
-    case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
-    case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
-    case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(ws, ys, count, a, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
+}
+
+}  // namespace
+
+hipError_t launch_gemv_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols,
+                             int num_cus, hipStream_t s) {
+    return dispatch(ws, ys, count, a, nullptr, col0, ncols, num_cus, s);
 }
 
 hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int64_t ldy,
@@ -791,6 +873,30 @@ hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols,
     if (ldy != w.M) return hipErrorInvalidValue;
     float *ys[1] = {y};
     return launch_gemv_multi(&w, ys, 1, a, col0, ncols, num_cus, s);
+}
+
+bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
+    // Beyond 64 Ki rows (an output head) the redundant per-workgroup quantization costs more than the
+    // launch it saves.
+    if (ncols < 1 || ncols > MAXC || K < 1 || total_m < 1 || total_m > 65536) return false;
+    Plan p;
+    switch (type) {
+    case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, ncols, true, 0, p);
+    case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, ncols, true, 0, p);
+    case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, ncols, true, 0, p);
+    case T_Q8_0: return make_thin_plan<PolQ8_0>(K, total_m, ncols, true, 0, p);
+    default: return false;
+    }
+}
+
+hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols,
+                                 int num_cus, hipStream_t s) {
+    if (!x || count < 1) return hipErrorInvalidValue;
+    DevAct a{};  // only the geometry is read: the kernel quantizes x itself
+    a.K = ws[0].K;
+    a.N = ncols;
+    a.type = (ws[0].type == T_Q4_K || ws[0].type == T_Q6_K) ? T_Q8_K : T_Q8_0;
+    return dispatch(ws, ys, count, a, x, 0, ncols, num_cus, s);
 }
 
 }  // namespace miqmm

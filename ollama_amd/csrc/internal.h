@@ -28,6 +28,11 @@ hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols,
 hipError_t launch_gemv_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols,
                              int num_cus, hipStream_t s);
 int gemv_max_multi();
+// The same products from f32 activations x [ncols][K] (device): the kernel quantizes x in its own
+// prologue, saving the separate quantization launch.  Ask gemv_f32_supported() first.
+bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols);
+hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols,
+                                 int num_cus, hipStream_t s);
 // largest K the GEMV handles for a weight type
 int64_t gemv_max_k(int type);
 

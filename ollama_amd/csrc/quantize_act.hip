@@ -1,28 +1,17 @@
 // Kernel 1: on-GPU activation quantization to ggml's Q8_0 / Q8_K block formats.
 //
-// Semantics are the scalar CPU quantizers' (quantize_row_q8_0_ref / quantize_row_q8_K_ref of ggml,
-// the from_float step of the CPU mul_mat that Tensor.Mulmat -- /root/reference/ml/backend.go:151 --
-// ends in); the bytes produced are identical to the CPU's:
-//   Q8_0: amax over 32; d = amax/127 (IEEE fp32 divide); id = d ? 1/d : 0; q = roundf(x*id)
-//         (half away from zero); stored scale = fp16_rne(d).
-//   Q8_K: first element of largest |x| over 256, with its sign: max; iscale = -127/max;
-//         q = min(127, rne(iscale*x)) on the fp32-rounded product; bsums = sums of 16; d = 1/iscale.
-//         An all-zero block is all zero bytes.
-// This file is compiled with -ffp-contract=off: none of the expressions above may be fused.
+// The block quantizers themselves (and the CPU semantics they reproduce bit for bit) are in
+// quant_dev.h; this file holds the stand-alone kernels that write the structure-of-arrays planes the
+// GEMV / GEMM kernels read, and the repacking of those planes into GGUF block bytes.
 //
 // HBM-bound and tiny next to the weight stream (N*K*4 bytes in, ~N*K*1.14 out); one float4 per lane,
 // cross-lane max / sums over the 8 (Q8_0) or 64 (Q8_K) lanes that share a block.
-#include <hip/hip_fp16.h>
-
 #include "internal.h"
+#include "quant_dev.h"
 
 namespace miqmm {
 
 namespace {
-
-__device__ __forceinline__ int pack4(int a, int b, int c, int d) {
-    return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
-}
 
 // 8 lanes per block of 32; 8 blocks per wave.  nblk = N*K/32 blocks in total.
 __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float4 *__restrict__ x,
@@ -31,23 +20,14 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float4 *__rest
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t blk = t >> 3;
     const bool live = blk < nblk;
-    float4 v = live ? x[t] : make_float4(0.f, 0.f, 0.f, 0.f);
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
-    const float dd = amax / 127.0f;
-    const float id = dd != 0.0f ? 1.0f / dd : 0.0f;
-    const int q0 = (int)roundf(v.x * id), q1 = (int)roundf(v.y * id);
-    const int q2 = (int)roundf(v.z * id), q3 = (int)roundf(v.w * id);
-    int sum = q0 + q1 + q2 + q3;
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
-    sum += __shfl_xor(sum, 4);
+    const float4 v = live ? x[t] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float dd;
+    int sum;
+    const int packed = q8_0_quantize_lane(v, dd, sum);
     if (live) {
-        qs[t] = pack4(q0, q1, q2, q3);
+        qs[t] = packed;
         if ((t & 7) == 0) {
-            d[blk] = __half2float(__float2half_rn(dd));  // the scale the CPU stores and later reads
+            d[blk] = dd;
             bsums[blk] = (int16_t)sum;
         }
     }
@@ -61,38 +41,10 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__rest
     const int lane = threadIdx.x & 63;
     const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (blk >= nblk) return;  // whole wave leaves together
-    const float4 v = x[blk * 64 + lane];
-    // first strictly-greater scan, ascending index
-    float amax = 0.0f, mx = 0.0f;
-    int idx = 0;
-    const float e[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float ax = fabsf(e[i]);
-        if (ax > amax) { amax = ax; mx = e[i]; idx = lane * 4 + i; }
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float oa = __shfl_xor(amax, off), om = __shfl_xor(mx, off);
-        const int oi = __shfl_xor(idx, off);
-        if (oa > amax || (oa == amax && oi < idx)) { amax = oa; mx = om; idx = oi; }
-    }
-    int q[4] = {0, 0, 0, 0};
-    float dd = 0.0f;
-    if (amax != 0.0f) {
-        const float iscale = -127.0f / mx;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float p = iscale * e[i];
-            q[i] = min(127, (int)rintf(p));
-        }
-        dd = 1.0f / iscale;
-    }
-    int sum = q[0] + q[1] + q[2] + q[3];
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
-    const int pair = sum + __shfl_xor(sum, 4);  // bsums[2j] + bsums[2j+1] in lanes 8j .. 8j+7
-    qs[blk * 64 + lane] = pack4(q[0], q[1], q[2], q[3]);
+    float dd;
+    int sum, pair;
+    const int packed = q8_K_quantize_lane(x[blk * 64 + lane], lane, dd, sum, pair);
+    qs[blk * 64 + lane] = packed;
     if ((lane & 3) == 0) bsums[blk * 16 + (lane >> 2)] = (int16_t)sum;
     if (lane == 0) d[blk] = dd;
     // block sums as two int8 digits (s = 64*(s >> 6) + (s & 63)) for the int8-MFMA GEMM

@@ -107,31 +107,38 @@ public:
         t->ready_ = true;
         return t;
     }
-    // run every pending Mulmat node; nodes that read the same x share one quantization
+    // Run every pending Mulmat node.  Nodes that read the same x are handled together: decode-sized
+    // ones (n <= 8) go out four weights at a time through the entry point that quantizes x inside the
+    // GEMV launch; larger ones share one quantization of x.
     void Compute() {
         std::map<std::pair<Tensor *, int>, std::vector<Tensor *>> by_x;
         for (auto &n : nodes_)
-            if (!n->ready_) by_x[{n->op_x_.get(), mi_qmm_vec_dot_type(n->op_w_->type_)}].push_back(n.get());
+            if (!n->ready_) by_x[{n->op_x_.get(), n->op_w_->type_}].push_back(n.get());
         for (auto &kv : by_x) {
             Tensor *x = kv.first.first;
             const int64_t k = x->Dim(0), n = (int64_t)x->data_.size() / k;
-            mi_qmm_act *act = nullptr;
-            check(mi_qmm_act_create(b_.handle(), kv.first.second, k, n, &act));
-            int rc = mi_qmm_act_quantize(b_.handle(), act, x->data_.data(), n, MI_QMM_HOST);
-            for (size_t i = 0; rc == MI_QMM_OK && i < kv.second.size(); i += 4) {
-                const mi_qmm_weight *ws[4];
-                float *ys[4];
-                int cnt = 0;
-                for (size_t j = i; j < kv.second.size() && j < i + 4; j++, cnt++) {
-                    Tensor *t = kv.second[j];
-                    t->data_.assign((size_t)(n * t->Dim(0)), 0.f);
-                    ws[cnt] = t->op_w_->weight_;
-                    ys[cnt] = t->data_.data();
+            for (Tensor *t : kv.second) t->data_.assign((size_t)(n * t->Dim(0)), 0.f);
+            if (n <= 8) {
+                for (size_t i = 0; i < kv.second.size(); i += 4) {
+                    const mi_qmm_weight *ws[4];
+                    float *ys[4];
+                    int cnt = 0;
+                    for (size_t j = i; j < kv.second.size() && j < i + 4; j++, cnt++) {
+                        ws[cnt] = kv.second[j]->op_w_->weight_;
+                        ys[cnt] = kv.second[j]->data_.data();
+                    }
+                    check(mi_qmm_mulmat_multi(b_.handle(), ws, cnt, x->data_.data(), n, ys, MI_QMM_HOST));
                 }
-                rc = mi_qmm_mulmat_q8_multi(b_.handle(), ws, cnt, act, ys, MI_QMM_HOST);
+            } else {
+                mi_qmm_act *act = nullptr;
+                check(mi_qmm_act_create(b_.handle(), mi_qmm_vec_dot_type(kv.first.second), k, n, &act));
+                int rc = mi_qmm_act_quantize(b_.handle(), act, x->data_.data(), n, MI_QMM_HOST);
+                for (size_t i = 0; rc == MI_QMM_OK && i < kv.second.size(); i++)
+                    rc = mi_qmm_mulmat_q8(b_.handle(), kv.second[i]->op_w_->weight_, act, kv.second[i]->data_.data(),
+                                          MI_QMM_HOST, MI_QMM_PATH_AUTO);
+                mi_qmm_act_free(act);
+                check(rc);
             }
-            mi_qmm_act_free(act);
-            check(rc);
             for (Tensor *t : kv.second) t->ready_ = true;
         }
     }

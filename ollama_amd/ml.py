@@ -9,9 +9,9 @@ The reference's tensor ops build a lazy graph and have no error returns: Mulmat 
 Compute runs it, and a failure is a panic -- here a raised exception.  Shapes are ggml's: dimension 0
 is the contiguous one, a weight is [K, M], activations are [K, N], ``W.Mulmat(ctx, x)`` is [M, N].
 
-Everything that computes goes through the C ABI (``ollama_amd.qmm``).  Compute hoists the activation
-quantization: all Mulmat nodes of a graph that read the same ``x`` share one quantization, and the
-decode-sized ones (N <= 8) of the same weight type run as one multi-tensor launch.
+Everything that computes goes through the C ABI (``ollama_amd.qmm``).  Compute groups the Mulmat
+nodes of a graph by the ``x`` they read: decode-sized ones (N <= 8) of the same weight type run as one
+multi-tensor launch that quantizes ``x`` in its prologue; larger ones share one quantization of ``x``.
 """
 from __future__ import annotations
 
@@ -119,30 +119,39 @@ class Context:
             raise RuntimeError("Compute on a closed context")
         pending = [t for t in self._nodes if t._data is None and t._op is not None]
         c = self._b._ctx
-        # group by activation tensor: one quantization per (x, q8 type)
-        by_x: Dict[Tuple[int, int], List[Tensor]] = {}
+        # group by activation tensor
+        by_x: Dict[int, List[Tensor]] = {}
         for t in pending:
-            W, x = t._op
-            by_x.setdefault((id(x), qmm.vec_dot_type(W._type)), []).append(t)
-        for (_, q8), nodes in by_x.items():
+            by_x.setdefault(id(t._op[1]), []).append(t)
+        for nodes in by_x.values():
             x = nodes[0]._op[1]
             k = x.Dim(0)
             n = x.Floats().size // k
-            act = c.act_create(q8, k, max(n, 1))
-            try:
-                c.act_quantize(act, x.Floats().reshape(n, k))
-                # decode-sized products of one weight type go out as multi-tensor launches
-                by_type: Dict[int, List[Tensor]] = {}
-                for t in nodes:
-                    by_type.setdefault(t._op[0]._type, []).append(t)
+            xs = x.Floats().reshape(n, k)
+            by_type: Dict[int, List[Tensor]] = {}
+            for t in nodes:
+                by_type.setdefault(t._op[0]._type, []).append(t)
+            if n <= 8:
+                # decode: the GEMV quantizes x itself; weights of one type share a launch, four at a time
                 for group in by_type.values():
                     for i in range(0, len(group), 4):
                         part = group[i:i + 4]
-                        ys = c.mulmat_q8_multi([t._op[0]._weight for t in part], act)
+                        ys = c.mulmat_multi([t._op[0]._weight for t in part], xs)
                         for t, y in zip(part, ys):
                             t._data = y.reshape(-1)  # [n][m] row-major == ggml [M, N] with dim 0 contiguous
-            finally:
-                act.free()
+                continue
+            # prefill: quantize once per (x, q8 type), then one product per weight
+            by_q8: Dict[int, List[Tensor]] = {}
+            for t in nodes:
+                by_q8.setdefault(qmm.vec_dot_type(t._op[0]._type), []).append(t)
+            for q8, group in by_q8.items():
+                act = c.act_create(q8, k, n)
+                try:
+                    c.act_quantize(act, xs)
+                    for t in group:
+                        t._data = c.mulmat_q8(t._op[0]._weight, act).reshape(-1)
+                finally:
+                    act.free()
 
     def Close(self) -> None:
         self._nodes.clear()

@@ -24,6 +24,7 @@ EXPORTS = [
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
+    "mi_qmm_mulmat_multi",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_last_error", "mi_qmm_version", "mi_qmm_device_info",
 ]
@@ -78,6 +79,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_q8.restype = ci; L.mi_qmm_mulmat_q8.argtypes = [vp, vp, vp, vp, ci, ci]
     L.mi_qmm_mulmat_q8_multi.restype = ci
     L.mi_qmm_mulmat_q8_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, ctypes.POINTER(vp), ci]
+    L.mi_qmm_mulmat_multi.restype = ci
+    L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
     L.mi_qmm_last_error.restype = ctypes.c_char_p; L.mi_qmm_last_error.argtypes = []
     L.mi_qmm_version.restype = ctypes.c_char_p; L.mi_qmm_version.argtypes = []
     L.mi_qmm_device_info.restype = ci
@@ -267,6 +270,26 @@ class Context:
 
     def mulmat_q8_device(self, w: Weight, act: Act, y_ptr: int, path: int = PATH_AUTO):
         _check(lib().mi_qmm_mulmat_q8(self._h, w._h, act._h, ctypes.c_void_p(y_ptr), DEVICE, path))
+
+    def mulmat_multi(self, ws, x: np.ndarray):
+        """several weights of one type and k against the same f32 activations; host arrays out"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        n, k = x.shape
+        if any(w.k != k for w in ws):
+            raise ValueError(f"x has k={k}, weights have k={[w.k for w in ws]}")
+        ys = [np.empty((n, w.m), dtype=np.float32) for w in ws]
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[y.ctypes.data_as(ctypes.c_void_p) for y in ys])
+        _check(lib().mi_qmm_mulmat_multi(self._h, wh, len(ws), x.ctypes.data_as(ctypes.c_void_p), n, yp, HOST))
+        return ys
+
+    def mulmat_multi_device(self, ws, x_ptr: int, n: int, y_ptrs):
+        """device pointers; one launch (quantization included) for up to 4 weights when n <= 8"""
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[ctypes.c_void_p(int(p)) for p in y_ptrs])
+        _check(lib().mi_qmm_mulmat_multi(self._h, wh, len(ws), ctypes.c_void_p(int(x_ptr)), n, yp, DEVICE))
 
     def mulmat_q8_multi(self, ws, act: Act):
         """several weights against the same activations; host arrays out"""

@@ -3,6 +3,8 @@
 Bars: quantized activation bytes bit-exact; fp32 outputs within 1e-3 on
 |y-ref| / max(|ref|, 1e-2*rms(ref))  (see npref.rel_err for why the floor is 1% of the RMS).
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -250,6 +252,63 @@ def test_multi_weight_launch_matches_single(ctx):
         act.free()
         for W in Ws:
             W.free()
+
+
+@pytest.mark.parametrize("t", WTYPES)
+def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
+    """For n <= 8 the f32 entry points quantize x inside the GEMV's prologue.  The result must be
+    bit-identical to quantizing with the stand-alone kernel (whose bytes are checked against the oracle
+    above) and multiplying by the two-phase entry point -- i.e. the in-kernel quants are the same bits."""
+    rng = np.random.default_rng(400 + t)
+    blk = npref.BLOCK[t]
+    ks = [blk, 4096, 14336] + ([2336, 96] if blk == 32 else [2304])   # 2336*n is not a multiple of 256
+    for k in ks:
+        ms = [37, 130]
+        raws = [_weights(t, m, k, seed=k + m) for m in ms]
+        Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+        act = ctx.act_create(qmm.vec_dot_type(t), k, 8)
+        for n in (1, 2, 5, 8):
+            x = rng.standard_normal((n, k), dtype=np.float32)
+            x[0, : min(k, 256)] = 0.0                                 # an all-zero block
+            ctx.act_quantize(act, x)
+            want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV) for W in Ws]
+            for W, wnt in zip(Ws, want):
+                assert np.array_equal(ctx.mulmat(W, x, path=qmm.PATH_GEMV), wnt), (k, n)
+            got = ctx.mulmat_multi(Ws, x)
+            for y, wnt in zip(got, want):
+                assert np.array_equal(y, wnt), (k, n)
+        # against the oracle as well, once per k
+        x = rng.standard_normal((3, k), dtype=np.float32)
+        got = ctx.mulmat_multi(Ws, x)
+        for y, r, m in zip(got, raws, ms):
+            assert npref.rel_err(y, oracle.mul_mat(t, r, k, m, x, nthreads=8)) <= TOL
+        act.free()
+        for W in Ws:
+            W.free()
+
+
+def test_mulmat_multi_fallbacks_and_errors(ctx):
+    k = 1024
+    rng = np.random.default_rng(8)
+    Ws = [ctx.upload(Q4_K, _weights(Q4_K, m, k, seed=m), k, m) for m in (40, 24, 8, 16, 32)]
+    x = rng.standard_normal((12, k), dtype=np.float32)
+    # five weights and twelve rows: falls back to one product per weight, same values
+    got = ctx.mulmat_multi(Ws, x)
+    for W, y in zip(Ws, got):
+        assert np.array_equal(y, ctx.mulmat(W, x))
+    W8 = ctx.upload(Q8_0, _weights(Q8_0, 8, k, seed=1), k, 8)
+    got = ctx.mulmat_multi([Ws[0], W8], x[:1])                        # mixed types: per-weight products
+    assert np.array_equal(got[0], ctx.mulmat(Ws[0], x[:1])) and np.array_equal(got[1], ctx.mulmat(W8, x[:1]))
+    Wk = ctx.upload(Q4_K, _weights(Q4_K, 8, 2 * k, seed=2), 2 * k, 8)
+    with pytest.raises(qmm.QmmError) as e:
+        lib_ws = (ctypes.c_void_p * 2)(Ws[0]._h, Wk._h)                 # different k: rejected
+        ys = [np.empty((1, 40), np.float32), np.empty((1, 8), np.float32)]
+        yp = (ctypes.c_void_p * 2)(*[y.ctypes.data_as(ctypes.c_void_p) for y in ys])
+        qmm._check(qmm.lib().mi_qmm_mulmat_multi(ctx._h, lib_ws, 2, x[:1].ctypes.data_as(ctypes.c_void_p), 1, yp,
+                                                 qmm.HOST))
+    assert e.value.code == qmm.ERR_INVALID
+    for W in Ws + [W8, Wk]:
+        W.free()
 
 
 # ---- kernel 3: int8-MFMA GEMM ---------------------------------------------------------------------
