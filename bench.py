@@ -32,6 +32,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
 
 Q4_K, Q6_K, Q8_K = 12, 14, 15
+GATE_UP_HBM_TRAFFIC_BYTES = 66386790  # measured, see the roofline block below
 FFN_K, FFN_M = 4096, 14336
 
 
@@ -161,7 +162,9 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            # HBM bytes per launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE x 2.000 and
+            # WRITE_SIZE x 1.000, factors from a 1 GiB copy): 32,359.41 KiB x 2 + 112.03 KiB
+            "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
             "bytes_per_launch": int(bytes_per_launch),
         },
