@@ -194,7 +194,9 @@ def main() -> int:
         def layer_pass():
             for c in range(copies):
                 ctx.act_quantize(actb_x, xb.data_ptr(), NB, qmm.DEVICE)
-                for i in range(6):
+                # q, k and v share x and are small: one launch over their concatenated rows
+                ctx.mulmat_q8_multi_device(gw[c][0:3], actb_x, [ys[0].data_ptr(), ys[1].data_ptr(), ys[2].data_ptr()])
+                for i in range(3, 6):
                     ctx.mulmat_q8_device(gw[c][i], actb_x, ys[i].data_ptr())
                 ctx.act_quantize(actb_h, hb.data_ptr(), NB, qmm.DEVICE)
                 ctx.mulmat_q8_device(gw[c][6], actb_h, ys[6].data_ptr())
@@ -212,6 +214,11 @@ def main() -> int:
             fn()
             tm = timed(fn, gsteps) / (gsteps * copies)
             per[name] = {"us": round(tm * 1e6, 1), "tops": round(2.0 * NB * m * k / tm / 1e12, 1)}
+        fn = lambda: [ctx.mulmat_q8_multi_device(gw[c][0:3], actb_x, [ys[0].data_ptr(), ys[1].data_ptr(), ys[2].data_ptr()])
+                      for c in range(copies)]
+        fn()
+        tm = timed(fn, gsteps) / (gsteps * copies)
+        per["attn_q+k+v (one launch)"] = {"us": round(tm * 1e6, 1), "tops": round(2.0 * NB * 6144 * 4096 / tm / 1e12, 1)}
         out["gemm"] = {
             "metric": "prefill GEMM TOPS (int8 MFMA)",
             "workload": "one Llama-3-8B-shaped layer, batch 512: q/o 4096x4096, k/v 1024x4096, gate/up 14336x4096 Q4_K; "

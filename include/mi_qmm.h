@@ -137,8 +137,9 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
                      int location, int path);
 
 /* several weights of one type and k against the same activations: ys[i] receives f32 [n][m_i].
- * For n <= 8 and count <= 4 this is ONE kernel launch over the concatenated rows (decode: gate+up,
- * q+k+v); otherwise it is the same as calling mi_qmm_mulmat_q8 per weight. */
+ * For count <= 4 and n <= 8 (decode GEMV) or n >= 32 with Q4_K / Q6_K weights (prefill GEMM) this
+ * is ONE kernel launch over the concatenated rows (gate+up, q+k+v); otherwise it is the same as
+ * calling mi_qmm_mulmat_q8 per weight. */
 int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count,
                            const mi_qmm_act *act, float *const *ys, int location);
 

@@ -632,7 +632,17 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     bool same = true;
     for (int i = 1; i < count; i++)
         same = same && ws[i]->dev.type == ws[0]->dev.type && ws[i]->dev.K == ws[0]->dev.K;
-    if (!same || count > gemv_max_multi() || act->n > 8 || ws[0]->dev.K > gemv_max_k(ws[0]->dev.type)) {
+    bool gemm_ok = same && count <= gemm_max_multi() && act->n >= 32;
+    int64_t tiles = 0;
+    for (int i = 0; gemm_ok && i < count; i++) {
+        gemm_ok = gemm_supports(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M);
+        tiles += (ws[i]->dev.M + 127) / 128 * ((act->n + 127) / 128);
+    }
+    // one launch pays when the tensors are too small to fill the machine one by one (q, k, v); large
+    // ones (gate, up) run slightly faster back to back
+    gemm_ok = gemm_ok && 2 * tiles < 3 * (int64_t)ctx->num_cus;
+    const bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
+    if (!gemm_ok && !gemv_ok) {
         for (int i = 0; i < count; i++) {
             int rc = mi_qmm_mulmat_q8(ctx, ws[i], act, ys[i], location, MI_QMM_PATH_AUTO);
             if (rc) return rc;
@@ -664,7 +674,8 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
-    HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));
+    if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, ctx->num_cus, ctx->stream));
+    else HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));
     if (location == MI_QMM_HOST) {
         for (int i = 0; i < count; i++)
             HIP_TRY(hipMemcpyAsync(ys[i], dys[i], (size_t)(act->n * dw[i].M) * 4, hipMemcpyDeviceToHost, ctx->stream));

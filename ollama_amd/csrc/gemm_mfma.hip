@@ -27,6 +27,9 @@
 // accumulators (one d/dmin per lane) and makes the output stores contiguous in m.
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
+#include <type_traits>
+
 #include "internal.h"
 
 namespace miqmm {
@@ -59,9 +62,21 @@ struct GemmQ4K {
     // lane (r = lane%32, h = lane/32): elements 32s+16h.. of k-step s = sub-block s.  Sub-blocks 2c and
     // 2c+1 are the low / high nibbles of qs bytes [32c+16h, +16).
     struct Raw { uint4 hdr, q[4]; };
-    static constexpr int RAW_LOADS = 5;  // memory instructions of load_raw
-    static __device__ __forceinline__ void load_raw(const DevWeight &w, int64_t row, int64_t sb, int h, Raw &raw) {
-        const uint8_t *p = w.p0 + row * (w.K / QKK * Q4_K_BYTES) + sb * Q4_K_BYTES;
+    // LDS weight stage: the rows' 144-byte blocks back to back, [row][9 pieces of 16 bytes]; copy slot
+    // p (16 bytes, consecutive in LDS) holds piece p%9 of row p/9.
+    static constexpr int W_PIECES = 9;
+    static constexpr int OCC_SMALL = 4;  // waves per SIMD with the 128 x 64 tile: two workgroups share a CU
+    static constexpr int W_INSTRS = 3;  // copy instructions per wave: 128 rows x 9 pieces / (8 waves x 64 lanes)
+    static __device__ __forceinline__ unsigned w_lane_off(const DevWeight &w, int p, int rows_left) {
+        const int rowi = min(p / 9, rows_left - 1), pc = p % 9;
+        return (unsigned)rowi * (unsigned)(w.K / QKK * Q4_K_BYTES) + 16u * pc;
+    }
+    static __device__ __forceinline__ const uint8_t *w_base(const DevWeight &w, int, int64_t m0, int64_t sb) {
+        return w.p0 + m0 * (w.K / QKK * Q4_K_BYTES) + sb * Q4_K_BYTES;
+    }
+    static __device__ __forceinline__ void read_raw(const uint8_t *wt, int rowi, int h, const DevWeight &, int64_t, int64_t,
+                                                    Raw &raw) {
+        const uint8_t *p = wt + rowi * 144;
         raw.hdr = ld16(p);
 #pragma unroll
         for (int c = 0; c < 4; c++) raw.q[c] = ld16(p + 16 + 32 * c + 16 * h);
@@ -115,18 +130,40 @@ struct GemmQ6K {
     // lane (r, h), k-step s: elements 32s+16h.. = scale group 2s+h; half H = s>>2, run rr = s&3:
     // ql bytes [64H + 32(rr&1) + 16h, +16) (low nibble for rr<2, high for rr>=2), qh bytes [32H+16h, +16) >> 2rr.
     struct Raw { uint4 L[2][2], Hq[2], scv; unsigned dh; };
-    static constexpr int RAW_LOADS = 8;
-    static __device__ __forceinline__ void load_raw(const DevWeight &w, int64_t row, int64_t sb, int h, Raw &raw) {
-        const uint8_t *pl = w.p0 + row * (w.K / 2) + sb * 128 + 16 * h;
-        const uint8_t *ph = w.p1 + row * (w.K / 4) + sb * 64 + 16 * h;
+    // LDS weight stage, one region per plane so that every copy instruction reads one plane:
+    //   ql [128 rows][8 pieces] at 0, qh [128][4] at 16 KiB, scales [128][1] at 24 KiB.
+    // Rows are 128 / 64 bytes apart, which would put a column of 16 rows on two / four bank groups;
+    // the piece positions inside a row are XOR-ed with row bits so a 16-row read is conflict-free.
+    static constexpr int W_PIECES = 13;
+    static constexpr int OCC_SMALL = 2;  // 90 KiB of LDS per workgroup: one per CU whatever the tile
+    static constexpr int W_INSTRS = 4;  // 26 KiB of copy slots over 8 waves
+    static __device__ __forceinline__ unsigned w_lane_off(const DevWeight &w, int p, int rows_left) {
+        if (p < 1024) {
+            const int slot_row = p >> 3, pos = p & 7, piece = pos ^ ((slot_row >> 1) & 7);
+            return (unsigned)min(slot_row, rows_left - 1) * (unsigned)(w.K / 2) + 16u * piece;
+        } else if (p < 1536) {
+            const int q = p - 1024, slot_row = q >> 2, pos = q & 3, piece = pos ^ ((slot_row >> 2) & 3);
+            return (unsigned)min(slot_row, rows_left - 1) * (unsigned)(w.K / 4) + 16u * piece;
+        }
+        return (unsigned)min(p - 1536, rows_left - 1) * (unsigned)(w.K / 16);
+    }
+    static __device__ __forceinline__ const uint8_t *w_base(const DevWeight &w, int blk, int64_t m0, int64_t sb) {
+        if (blk < 16) return w.p0 + m0 * (w.K / 2) + sb * 128;
+        if (blk < 24) return w.p1 + m0 * (w.K / 4) + sb * 64;
+        return w.p2 + m0 * (w.K / 16) + sb * 16;
+    }
+    static __device__ __forceinline__ void read_raw(const uint8_t *wt, int rowi, int h, const DevWeight &w, int64_t row,
+                                                    int64_t sb, Raw &raw) {
+        raw.dh = w.d[row * (w.K / QKK) + sb];
+        const uint8_t *pl = wt + rowi * 128, *ph = wt + 16384 + rowi * 64;
+        const int xl = (rowi >> 1) & 7, xh = (rowi >> 2) & 3;
 #pragma unroll
         for (int H = 0; H < 2; H++) {
-            raw.L[H][0] = ld16(pl + 64 * H);
-            raw.L[H][1] = ld16(pl + 64 * H + 32);
-            raw.Hq[H] = ld16(ph + 32 * H);
+            raw.L[H][0] = ld16(pl + 16 * ((4 * H + h) ^ xl));
+            raw.L[H][1] = ld16(pl + 16 * ((4 * H + 2 + h) ^ xl));
+            raw.Hq[H] = ld16(ph + 16 * ((2 * H + h) ^ xh));
         }
-        raw.scv = ld16(w.p2 + row * (w.K / 16) + sb * 16);
-        raw.dh = w.d[row * (w.K / QKK) + sb];
+        raw.scv = ld16(wt + 24576 + rowi * 16);
     }
     static __device__ __forceinline__ void expand(const Raw &raw, int h, BOperand &b) {
         const uint4 scv = raw.scv;
@@ -175,35 +212,61 @@ struct GemmQ6K {
 typedef __attribute__((address_space(3))) void lds_ptr_t;
 typedef const __attribute__((address_space(1))) void glb_ptr_t;
 
-// One LDS stage: the activation tile of one super-block.  q rows are 256 bytes, unpadded; the 16-byte
-// piece p of row R is stored at piece position p ^ (R & 15).
-template <int TN>
-struct Stage {
+// ---------------------------------------------------------------------------------------------
+// Everything through LDS.  Loading the packed weights straight into the lanes that expand them costs a
+// wave one memory instruction per 16-byte piece and row -- 32 cache lines per instruction -- and that
+// latency sits on the critical path of every super-block.  Here the 128 x 128 tile's packed weights
+// travel like the activations: coalesced direct-to-LDS copies (consecutive lanes fetch consecutive
+// 16-byte pieces of a row), two LDS stages, the copy of super-block sb+1 running under the math of sb.
+// Eight waves (two per SIMD, 256 registers each, MFMA results in ordinary VGPRs): wave (mb, nh) owns
+// weight rows 32*mb.. and activation rows 64*nh.. of the tile.
+// ---------------------------------------------------------------------------------------------
+template <class G, int TN>
+struct Stage3 {
     uint8_t q[TN * 256];
-    uint8_t s[TN * 32];
-    float yd[TN < 256 ? 256 : TN];  // keeps the stage a multiple of 1 KiB
+    uint8_t s[TN * G::SD];
+    float yd[TN < 256 ? 256 : TN];  // keeps the members that follow 1 KiB aligned
+    uint8_t wt[128 * 16 * G::W_PIECES];
 };
 
-// Workgroup = WAVES waves x 32 weight rows, against TN = 32*TNT activation rows.  Per super-block:
-//   start the direct-to-LDS copy of the next activation stage; expand the prefetched packed weights
-//   into the B operand; start the loads of the next super-block's packed weights; run the four 32-row
-//   activation sub-tiles (18 MFMAs + fp32 epilogue each); wait for the copies; one barrier.
-template <class G, int WAVES, int TNT>
-__global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(DevWeight w, DevAct a, float *__restrict__ y,
-                                                             int64_t ldy, int tiles_n) {
-    constexpr int TN = 32 * TNT;  // activation rows per workgroup
-    typedef Stage<TN> StageT;
-    __shared__ __attribute__((aligned(1024))) StageT lds[3];
+// Up to GEMM_MULTI weight tensors of one type and K against the same activations in one launch (q, k
+// and v; gate and up): the grid walks the concatenated 128-row blocks of all of them, which fills the
+// machine where a 1024-row k or v projection alone would occupy 32 of 256 CUs.
+constexpr int GEMM_MULTI = 4;
+struct GemmArgs {
+    const uint8_t *p0[GEMM_MULTI], *p1[GEMM_MULTI], *p2[GEMM_MULTI];
+    const uint16_t *d[GEMM_MULTI];
+    float *y[GEMM_MULTI];
+    int64_t M[GEMM_MULTI];
+    int tile_end[GEMM_MULTI];  // exclusive end of each tensor's 128-row block range; INT_MAX past the last
+    int64_t K;
+    int type;
+};
+
+// TNT = 32-row activation sub-tiles per wave: the workgroup tile is 128 weight rows x 64*TNT activation rows.
+template <class G, int TNT>
+__global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel(GemmArgs ga, DevAct a, int tiles_m, int tiles_n) {
+    constexpr int WAVES = 8, TN = 64 * TNT, TM = 128;
+    typedef Stage3<G, TN> StageT;
+    __shared__ __attribute__((aligned(1024))) StageT lds[2];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, h = lane >> 5;
-    // Workgroup i runs on XCD i % 8 and every XCD has its own L2: the tiles_n workgroups that share a
-    // block of weight rows are given ids that are 8 apart, so they meet in one L2.
+    const int mb = wave & 3, nh = wave >> 2;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int tile_n = slot % tiles_n, tile_m = xcd + 8 * (slot / tiles_n);
-    if ((int64_t)tile_m * (32 * WAVES) >= w.M) return;  // the grid is rounded up to 8 row blocks
-    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * (32 * WAVES);
-    const int64_t row = min(m0 + 32 * wave + r, w.M - 1);  // rows past M are computed and dropped
+    const int tile_n = slot % tiles_n, gtile_m = xcd + 8 * (slot / tiles_n);
+    if (gtile_m >= tiles_m) return;  // the grid is rounded up to 8 row blocks
+    const int e0 = ga.tile_end[0], e1 = ga.tile_end[1], e2 = ga.tile_end[2];
+    const int ti = (gtile_m >= e0) + (gtile_m >= e1) + (gtile_m >= e2);
+    const int tile_m = gtile_m - (ti == 0 ? 0 : ti == 1 ? e0 : ti == 2 ? e1 : e2);
+#define GEMM_SEL(f) (ti == 0 ? ga.f[0] : ti == 1 ? ga.f[1] : ti == 2 ? ga.f[2] : ga.f[3])
+    const DevWeight w{GEMM_SEL(p0), GEMM_SEL(p1), GEMM_SEL(p2), GEMM_SEL(d), ga.K, GEMM_SEL(M), ga.type};
+    float *__restrict__ y = GEMM_SEL(y);
+#undef GEMM_SEL
+    const int64_t ldy = w.M;
+    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * TM;
+    const int rows_left = (int)min((int64_t)TM, w.M - m0);  // rows past M: the last row again, results dropped
+    const int rowi = min(32 * mb + r, rows_left - 1);
     const int64_t nsb = w.K / QKK;
     const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
     const uint8_t *asd = G::digits(a);
@@ -214,155 +277,110 @@ __global__ __launch_bounds__(64 * WAVES, 1) void gemm_kernel(DevWeight w, DevAct
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[t][i] = 0.f;
 
-    // direct-to-LDS copy of the stage of super-block sb: every wave instruction moves 64 x 16 bytes to
-    // 1 KiB of consecutive LDS; which global piece a lane fetches implements the swizzle.  Activation
-    // rows past N are read too (the planes are allocated in whole tiles) and their results dropped, so
-    // all addresses of a lane are one base plus a uniform stride.
-    constexpr int QI = TN / 4 / WAVES;     // quant copy instructions per wave and stage
-    constexpr int QSTEP = 4 * WAVES;       // rows between consecutive instructions of a wave (16 or 8)
-    constexpr int NB = 16 / QSTEP < 1 ? 1 : 16 / QSTEP;  // distinct (row & 15) values per lane (1 or 2)
-    const uint8_t *qbase[NB];
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-        const int R = 4 * wave + (lane >> 4) + QSTEP * j;
-        qbase[j] = aq + (n0 + R) * a.K + 16 * ((lane & 15) ^ (R & 15));
+    // ---- copy plan: per-lane 32-bit offsets, uniform bases per super-block
+    constexpr int QI = TN / 4 / WAVES;  // quant copies per wave: rows 4*wave + lane/16 + 32*i
+    unsigned qoff;
+    {
+        const int R = 4 * wave + (lane >> 4);
+        qoff = (unsigned)R * (unsigned)a.K + 16u * ((lane & 15) ^ (R & 15));
     }
-    constexpr int RPI = 1024 / G::SD;      // rows per instruction for the digit plane (64 or 32)
-    const uint8_t *sbase = asd + (n0 + lane / (G::SD / 16)) * nsb * G::SD + 16 * (lane % (G::SD / 16));
-    const float *dbase = a.d + (n0 + lane) * nsb;
-    auto stage_copy = [&](StageT &st, int64_t sb) __attribute__((always_inline)) {  // quants last: the in-order wait at the end of an iteration counts on it
+    constexpr int RPI = 1024 / G::SD;   // activation rows per digit copy (64 or 32)
+    const unsigned soff = (unsigned)(lane / (G::SD / 16)) * (unsigned)(nsb * G::SD) + 16u * (lane % (G::SD / 16));
+    const unsigned doff = (unsigned)lane * (unsigned)nsb * 4u;
+    unsigned woff[G::W_INSTRS];
 #pragma unroll
-        for (int i = 0; i < (TN / RPI + WAVES - 1) / WAVES; i++) {
-            const int blk = wave + WAVES * i;  // uniform
-            if (blk < TN / RPI) {
-                const uint8_t *g = sbase + ((int64_t)RPI * blk * nsb + sb) * G::SD;
-                __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.s + 1024 * blk), 16, 0, 0);
+    for (int j = 0; j < G::W_INSTRS; j++) woff[j] = G::w_lane_off(w, (j * WAVES + wave) * 64 + lane, rows_left);
+
+    auto stage_copy = [&](StageT &st, int64_t sb) __attribute__((always_inline)) {
+        // weights
+#pragma unroll
+        for (int j = 0; j < G::W_INSTRS; j++) {
+            const int blk = j * WAVES + wave;  // uniform: which KiB of the weight stage
+            if (blk * 64 < 128 * G::W_PIECES) {
+                const uint8_t *g = G::w_base(w, blk, m0, sb) + woff[j];
+                __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.wt + 1024 * blk), 16, 0, 0);
             }
         }
-        if (wave < (TN + 63) / 64) {  // block scales: 64 rows per instruction
-            const float *g = dbase + (int64_t)64 * wave * nsb + sb;
-            __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.yd + 64 * wave), 4, 0, 0);
+        // block-sum digits: TN / RPI copies, one per wave from wave 0 up
+        if (wave < TN / RPI) {
+            const uint8_t *g = asd + ((n0 + (int64_t)RPI * wave) * nsb + sb) * G::SD + soff;
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.s + 1024 * wave), 16, 0, 0);
         }
+        // block scales: copies of 64 rows each, by the last waves
+        if (wave >= WAVES - TN / 64) {
+            const int blk = wave - (WAVES - TN / 64);
+            const uint8_t *g = reinterpret_cast<const uint8_t *>(a.d + (n0 + 64 * blk) * nsb + sb) + doff;
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.yd + 64 * blk), 4, 0, 0);
+        }
+        // quants
+        const uint8_t *qb = aq + n0 * a.K + sb * QKK;
 #pragma unroll
         for (int i = 0; i < QI; i++) {
-            const uint8_t *g = qbase[i % NB] + (int64_t)(QSTEP * (i - i % NB)) * a.K + sb * QKK;
+            const uint8_t *g = qb + (int64_t)(32 * i) * a.K + qoff;
             __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.q + 1024 * (wave + WAVES * i)), 16, 0, 0);
         }
     };
-
-    // A-operand piece offsets inside a row, swizzled: piece 2s+h of row R sits at (2s+h) ^ (R & 15)
     const int swz = 16 * (h ^ (r & 15));
 
-    // One super-block: expand the packed weights fetched two iterations ago, start the copies and the
-    // weight loads for two super-blocks ahead (three LDS stages, two packed-weight register sets: a
-    // load has two whole iterations to arrive), run the MFMAs of this stage, then wait for everything
-    // except what was just issued.
-    auto body = [&](typename G::Raw &raw, int64_t sb) __attribute__((always_inline)) {
-        StageT &cur = lds[sb % 3];
-        // the last two iterations fetch the final super-block again (into a stage nobody reads): the
-        // loop body stays free of branches and the wait below can always leave the same number of
-        // memory instructions in flight
-        const int64_t sbn = min(sb + 2, nsb - 1);
-        BOperand b;
-#if defined(GEMV_VARIANT) && GEMV_VARIANT == 15
-        __builtin_memset(&b, 1, sizeof(b)); b.d = __int_as_float(raw.hdr.x);
-#else
-        G::expand(raw, h, b);
-#endif
-#if !(defined(GEMV_VARIANT) && (GEMV_VARIANT == 16 || GEMV_VARIANT == 18))
-        stage_copy(lds[(sb + 2) % 3], sbn);  // that stage was last read in iteration sb-1: every wave has passed its barrier
-#endif
-#if !(defined(GEMV_VARIANT) && (GEMV_VARIANT == 17 || GEMV_VARIANT == 18))
-        G::load_raw(w, row, sbn, h, raw);
-#endif
-        // The matrix cores and the vector ALU are fed from one in-order instruction stream per wave, and
-        // there is one wave per SIMD: to keep both busy the fp32 epilogue of sub-tile t-1 is interleaved
-        // by hand with the MFMAs of sub-tile t -- per k-step two MFMAs (64 matrix-core cycles), then
-        // the epilogue of two outputs -- with scheduling barriers pinning that order.
-        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        v16i ah[2], al[2], xl[2], xh[2];
-#pragma unroll
-        for (int t = 0; t <= TNT; t++) {
-            const int p = t & 1, q = p ^ 1;  // accumulator set being produced / consumed
-            const uint8_t *arow = cur.q + (32 * (t < TNT ? t : 0) + r) * 256;
-            v4i abuf[3];
-            if (t < TNT) {
-                const v4i sv = *reinterpret_cast<const v4i *>(cur.s + (32 * t + r) * G::SD + (G::SD == 32 ? 16 * h : 0));
-                abuf[0] = *reinterpret_cast<const v4i *>(arow + (0 ^ swz));
-                abuf[1] = *reinterpret_cast<const v4i *>(arow + (32 ^ swz));
-                xl[p] = mfma(sv, b.min_lo, zero);
-                xh[p] = mfma(sv, b.min_hi, zero);
-                ah[p] = zero;
-                al[p] = zero;
-            }
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                if (t < TNT) {
-                    if (s + 2 < 8) abuf[(s + 2) % 3] = *reinterpret_cast<const v4i *>(arow + ((32 * (s + 2)) ^ swz));
-                    const v4i av = abuf[s % 3];
-#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 12 || GEMV_VARIANT == 14)
-                    ah[p][s] ^= av[0] ^ b.hi[s][1]; al[p][s] ^= av[2] ^ b.lo[s][3];   // MFMAs removed
-#else
-                    ah[p] = mfma(av, b.hi[s], ah[p]);
-                    al[p] = mfma(av, b.lo[s], al[p]);
-#endif
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                if (t > 0) {  // outputs 2s and 2s+1 of sub-tile t-1; accumulator i is activation row 8(i/4) + 4h + i%4
-#pragma unroll
-                    for (int i = 2 * s; i < 2 * s + 2; i++) {
-                        const float yd = cur.yd[32 * (t - 1) + 8 * (i >> 2) + 4 * h + (i & 3)];
-                        const float fm = G::fold_min(b.dmin, xh[q][i], xl[q][i]);
-#if defined(GEMV_VARIANT) && (GEMV_VARIANT == 11 || GEMV_VARIANT == 14)
-                        acc[t - 1][i] += __int_as_float(ah[q][i] ^ al[q][i]) + yd + fm * 0.f;
-#else
-                        acc[t - 1][i] = __builtin_fmaf(yd, G::combine(b.d, ah[q][i], al[q][i], fm), acc[t - 1][i]);
-#endif
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        // the youngest QI + RAW_LOADS memory instructions are the quant copies and packed-weight loads
-        // for super-block sb+2; everything older (stage sb+1, weights sb+1) must have landed
-        constexpr int KEEP = QI + G::RAW_LOADS;
-#if defined(GEMV_VARIANT) && GEMV_VARIANT >= 16 && GEMV_VARIANT <= 18
-        __builtin_amdgcn_s_waitcnt(0);
-#else
-        __builtin_amdgcn_s_waitcnt((KEEP & 15) | (7 << 4) | (15 << 8) | ((KEEP >> 4) << 14));
-#endif
-        // a bare barrier: __syncthreads() carries a fence that drains every outstanding load, i.e. it
-        // would wait for the copies issued a moment ago.  What must be ordered here is LDS only: the
-        // copies of the next stage are complete (the wait above, in every wave) and this wave's reads
-        // of the current stage have returned (they fed the MFMAs above).
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    };
-
-    // ---- prologue: stages 0 and 1, packed weights 0 and 1
-    typename G::Raw raw0, raw1;
-    G::load_raw(w, row, 0, h, raw0);
     stage_copy(lds[0], 0);
-    if (nsb > 1) {
-        G::load_raw(w, row, 1, h, raw1);
-        stage_copy(lds[1], 1);
-    }
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
-    for (int64_t sb = 0; sb < nsb; sb += 2) {
-        body(raw0, sb);
-        if (sb + 1 < nsb) body(raw1, sb + 1);
-    }
-
-    // ---- store: lanes r = 0..31 hold consecutive m
-    const int64_t m = m0 + 32 * wave + r;
-    if (m < w.M) {
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 1
+    for (int64_t sb = 0; sb < nsb; sb++) {
+        StageT &cur = lds[sb & 1];
+        // the other stage was last read in iteration sb-1 and every wave has passed that barrier
+        // (a Q6_K row's fp16 scale is a plain global load: it goes out ahead of the copies, so waiting
+        // for it does not mean waiting for them)
+        typename G::Raw raw;
+        G::read_raw(cur.wt, rowi, h, w, m0 + rowi, sb, raw);
+        stage_copy(lds[(sb + 1) & 1], min(sb + 1, nsb - 1));
+        BOperand b;
+        G::expand(raw, h, b);
 #pragma unroll
-        for (int t = 0; t < TNT; t++) {
+        for (int tt = 0; tt < TNT; tt++) {
+            const int t = TNT * nh + tt;  // 32-row activation sub-tile of the stage
+            const uint8_t *arow = cur.q + (32 * t + r) * 256;
+            const v4i sv = *reinterpret_cast<const v4i *>(cur.s + (32 * t + r) * G::SD + (G::SD == 32 ? 16 * h : 0));
+            v4i abuf[3];
+            abuf[0] = *reinterpret_cast<const v4i *>(arow + (0 ^ swz));
+            abuf[1] = *reinterpret_cast<const v4i *>(arow + (32 ^ swz));
+            float4 yd[4];  // block scales of the 32 activation rows: accumulator i is row 8(i/4) + 4h + i%4
+#pragma unroll
+            for (int gq = 0; gq < 4; gq++) yd[gq] = *reinterpret_cast<const float4 *>(cur.yd + 32 * t + 8 * gq + 4 * h);
+            const v16i xl = mfma(sv, b.min_lo, zero);
+            const v16i xh = mfma(sv, b.min_hi, zero);
+            v16i ah, al;
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                if (s + 2 < 8) abuf[(s + 2) % 3] = *reinterpret_cast<const v4i *>(arow + ((32 * (s + 2)) ^ swz));
+                const v4i av = abuf[s % 3];
+                ah = mfma(av, b.hi[s], s == 0 ? zero : ah);
+                al = mfma(av, b.lo[s], s == 0 ? zero : al);
+            }
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int64_t n = n0 + 32 * t + 8 * (i >> 2) + 4 * h + (i & 3);
-                if (n < a.N) y[n * ldy + m] = acc[t][i];
+                const float4 y4 = yd[i >> 2];
+                const float ydv = (i & 3) == 0 ? y4.x : (i & 3) == 1 ? y4.y : (i & 3) == 2 ? y4.z : y4.w;
+                const float fm = G::fold_min(b.dmin, xh[i], xl[i]);
+                acc[tt][i] = __builtin_fmaf(ydv, G::combine(b.d, ah[i], al[i], fm), acc[tt][i]);
+            }
+        }
+        // this wave's copies have landed; after the barrier so have everybody else's, and nobody still
+        // reads the stage that the next iteration overwrites
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+
+    const int64_t m = m0 + 32 * mb + r;
+    if (m < w.M) {
+#pragma unroll
+        for (int tt = 0; tt < TNT; tt++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t n = n0 + 32 * (TNT * nh + tt) + 8 * (i >> 2) + 4 * h + (i & 3);
+                if (n < a.N) y[n * ldy + m] = acc[tt][i];
             }
         }
     }
@@ -375,32 +393,46 @@ bool gemm_supports(int type, int64_t K, int64_t M) {
 }
 
 template <class G>
-hipError_t launch_cfg(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, int num_cus, hipStream_t s) {
-    // One workgroup per CU (three LDS stages, one wave per SIMD with the full register file).  Prefer
-    // the largest tile that still gives about one workgroup per CU; smaller tiles re-expand the weights
-    // more often but keep all CUs (and all four SIMDs) busy on the smaller matrices.
-    struct Cfg { int waves, tn; } cfgs[3] = {{4, 128}, {4, 64}, {2, 64}};
-    int pick = 2;
-    for (int i = 0; i < 3; i++) {
-        const int64_t t = ((w.M + 32 * cfgs[i].waves - 1) / (32 * cfgs[i].waves)) * ((a.N + cfgs[i].tn - 1) / cfgs[i].tn);
-        if (4 * t >= 3 * (int64_t)num_cus) { pick = i; break; }
+hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus, hipStream_t s) {
+    GemmArgs ga;
+    int64_t tiles_m = 0;
+    for (int i = 0; i < GEMM_MULTI; i++) {
+        const int j = i < count ? i : count - 1;
+        ga.p0[i] = ws[j].p0; ga.p1[i] = ws[j].p1; ga.p2[i] = ws[j].p2; ga.d[i] = ws[j].d;
+        ga.y[i] = ys[j]; ga.M[i] = ws[j].M;
+        if (i < count) tiles_m += (ws[i].M + 127) / 128;
+        ga.tile_end[i] = i < count ? (int)tiles_m : 0x7fffffff;
     }
-    const int64_t tm = 32 * cfgs[pick].waves, tn = cfgs[pick].tn;
-    const int64_t tiles_n = (a.N + tn - 1) / tn, tiles_m = ((w.M + tm - 1) / tm + 7) / 8 * 8;  // whole rounds of 8 XCDs
-    if (tiles_n * tiles_m > 0x7fffffff) return hipErrorInvalidValue;
-    const unsigned grid = (unsigned)(tiles_n * tiles_m);
-    switch (pick) {
-    case 0: gemm_kernel<G, 4, 4><<<grid, 256, 0, s>>>(w, a, y, ldy, (int)tiles_n); break;
-    case 1: gemm_kernel<G, 4, 2><<<grid, 256, 0, s>>>(w, a, y, ldy, (int)tiles_n); break;
-    default: gemm_kernel<G, 2, 2><<<grid, 128, 0, s>>>(w, a, y, ldy, (int)tiles_n); break;
-    }
+    ga.K = ws[0].K; ga.type = ws[0].type;
+    // 128 x 128 tiles when they still give every CU work for most of the run, else 128 x 64
+    static const char *dbg = getenv("MI_QMM_GEMM_DEBUG");  // "1": always 128x64, "2": always 128x128
+    const int64_t big = tiles_m * ((a.N + 127) / 128);
+    const bool tnt2 = dbg ? dbg[0] == '2' : 2 * big >= 3 * (int64_t)num_cus;
+    const int64_t tn = tnt2 ? 128 : 64, tiles_n = (a.N + tn - 1) / tn;
+    const int64_t grid = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
+    if (tiles_m > 0x7ffffff0 || grid > 0x7fffffff) return hipErrorInvalidValue;
+    if (tnt2) gemm3_kernel<G, 2><<<(unsigned)grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n);
+    else gemm3_kernel<G, 1><<<(unsigned)grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n);
     return hipGetLastError();
 }
 
+int gemm_max_multi() { return GEMM_MULTI; }
+
+hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus,
+                             hipStream_t s) {
+    if (count < 1 || count > GEMM_MULTI) return hipErrorInvalidValue;
+    for (int i = 0; i < count; i++)
+        if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || !gemm_supports(ws[i].type, ws[i].K, ws[i].M) || !ys[i])
+            return hipErrorInvalidValue;
+    if (a.type != T_Q8_K || a.K != ws[0].K || a.N < 1 || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
+    return ws[0].type == T_Q4_K ? launch3<GemmQ4K>(ws, ys, count, a, num_cus, s)
+                                : launch3<GemmQ6K>(ws, ys, count, a, num_cus, s);
+}
+
 hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, int num_cus, hipStream_t s) {
-    if (!gemm_supports(w.type, w.K, w.M) || a.type != T_Q8_K || a.K != w.K || a.N < 1 || !a.sd8 || !a.sd16)
-        return hipErrorInvalidValue;
-    return w.type == T_Q4_K ? launch_cfg<GemmQ4K>(w, a, y, ldy, num_cus, s) : launch_cfg<GemmQ6K>(w, a, y, ldy, num_cus, s);
+    if (ldy != w.M) return hipErrorInvalidValue;
+    float *ys[1] = {y};
+    return launch_gemm_multi(&w, ys, 1, a, num_cus, s);
 }
 
 }  // namespace miqmm

@@ -40,5 +40,9 @@ int64_t gemv_max_k(int type);
 hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, int num_cus,
                        hipStream_t s);
 bool gemm_supports(int type, int64_t K, int64_t M);
+// several weight tensors of one type and K against the same activations in one launch
+hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus,
+                             hipStream_t s);
+int gemm_max_multi();
 
 }  // namespace miqmm
