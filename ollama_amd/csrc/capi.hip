@@ -46,6 +46,7 @@ struct mi_qmm_ctx {
     // growable scratch: quantized activation planes and host<->device staging
     void *act_buf = nullptr;  size_t act_cap = 0;
     void *io_buf = nullptr;   size_t io_cap = 0;
+    void *ws_buf = nullptr;   size_t ws_cap = 0;   // partial sums of a K-split GEMM
 };
 
 struct mi_qmm_weight {
@@ -219,6 +220,7 @@ void mi_qmm_destroy(mi_qmm_ctx *ctx) {
         (void)hipStreamSynchronize(ctx->stream);
         if (ctx->act_buf) (void)hipFree(ctx->act_buf);
         if (ctx->io_buf) (void)hipFree(ctx->io_buf);
+        if (ctx->ws_buf) (void)hipFree(ctx->ws_buf);
         if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
     }
     delete ctx;
@@ -404,7 +406,12 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
         return fail(MI_QMM_ERR_UNSUPPORTED, "K=%lld exceeds the GEMV limit %lld for type %d", (long long)K,
                     (long long)gemv_max_k(w->dev.type), w->dev.type);
     if (use_gemm) {
-        HIP_TRY(launch_gemm(w->dev, a, dy, M, ctx->num_cus, ctx->stream));
+        const size_t wsf = gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus);
+        if (wsf) {
+            int rc = reserve(&ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float), ctx->stream);
+            if (rc) return rc;
+        }
+        HIP_TRY(launch_gemm(w->dev, a, dy, M, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
     } else {
         for (int64_t c0 = 0; c0 < n; c0 += 8) {
             const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
@@ -674,7 +681,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
-    if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, ctx->num_cus, ctx->stream));
+    if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));
     else HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));
     if (location == MI_QMM_HOST) {
         for (int i = 0; i < count; i++)

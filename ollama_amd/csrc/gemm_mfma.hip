@@ -245,7 +245,8 @@ struct GemmArgs {
 
 // TNT = 32-row activation sub-tiles per wave: the workgroup tile is 128 weight rows x 64*TNT activation rows.
 template <class G, int TNT>
-__global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel(GemmArgs ga, DevAct a, int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel(GemmArgs ga, DevAct a, int tiles_m, int tiles_n,
+                                                                             float *__restrict__ part) {
     constexpr int WAVES = 8, TN = 64 * TNT, TM = 128;
     typedef Stage3<G, TN> StageT;
     __shared__ __attribute__((aligned(1024))) StageT lds[2];
@@ -264,10 +265,15 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
     float *__restrict__ y = GEMM_SEL(y);
 #undef GEMM_SEL
     const int64_t ldy = w.M;
+    // split K: slice blockIdx.y of gridDim.y covers a contiguous run of super-blocks and writes its
+    // partial sums to its own [N][M] plane of part; a second kernel adds the planes up in slice order
+    // (deterministic, unlike floating-point atomics).  Single-tensor launches only.
+    if (part) y = part + (int64_t)blockIdx.y * a.N * w.M;
     const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * TM;
     const int rows_left = (int)min((int64_t)TM, w.M - m0);  // rows past M: the last row again, results dropped
     const int rowi = min(32 * mb + r, rows_left - 1);
-    const int64_t nsb = w.K / QKK;
+    const int64_t nsb = w.K / QKK;  // row pitch of the planes, in super-blocks
+    const int64_t sb_begin = nsb * blockIdx.y / gridDim.y, sb_end = nsb * (blockIdx.y + 1) / gridDim.y;
     const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
     const uint8_t *asd = G::digits(a);
 
@@ -322,20 +328,20 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
     };
     const int swz = 16 * (h ^ (r & 15));
 
-    stage_copy(lds[0], 0);
+    stage_copy(lds[0], sb_begin);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 1
-    for (int64_t sb = 0; sb < nsb; sb++) {
-        StageT &cur = lds[sb & 1];
+    for (int64_t sb = sb_begin; sb < sb_end; sb++) {
+        StageT &cur = lds[(sb - sb_begin) & 1];
         // the other stage was last read in iteration sb-1 and every wave has passed that barrier
         // (a Q6_K row's fp16 scale is a plain global load: it goes out ahead of the copies, so waiting
         // for it does not mean waiting for them)
         typename G::Raw raw;
         G::read_raw(cur.wt, rowi, h, w, m0 + rowi, sb, raw);
-        stage_copy(lds[(sb + 1) & 1], min(sb + 1, nsb - 1));
+        stage_copy(lds[(sb + 1 - sb_begin) & 1], min(sb + 1, sb_end - 1));
         BOperand b;
         G::expand(raw, h, b);
 #pragma unroll
@@ -386,14 +392,44 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
     }
 }
 
+// y[i] = sum over slices of part[slice][i]
+__global__ __launch_bounds__(256) void sum_slices_kernel(const float4 *__restrict__ part, float4 *__restrict__ y,
+                                                         int64_t n4, int slices) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        float4 acc = part[i];
+        for (int sl = 1; sl < slices; sl++) {
+            const float4 v = part[sl * n4 + i];
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+        y[i] = acc;
+    }
+}
+
+// K slices for a single tensor: when 128 x 128 tiles alone would leave CUs idle, cut K so that the
+// large tile (half the vector-ALU work per MFMA of the small one) still fills the machine.
+int pick_ksplit(int64_t K, int64_t M, int64_t N, int num_cus) {
+    const int64_t tiles = (M + 127) / 128 * ((N + 127) / 128), nsb = K / QKK;
+    if ((N * M) % 4 != 0) return 1;
+    int ks = 1;
+    while (ks < 4 && tiles * ks * 2 <= num_cus && nsb / (ks * 2) >= 16) ks *= 2;
+    return ks;
+}
+
 }  // namespace
 
 bool gemm_supports(int type, int64_t K, int64_t M) {
     return (type == T_Q4_K || type == T_Q6_K) && K >= QKK && K % QKK == 0 && M >= 1;
 }
 
+size_t gemm_workspace_floats(int type, int64_t K, int64_t M, int64_t N, int num_cus) {
+    if (!gemm_supports(type, K, M)) return 0;
+    const int ks = pick_ksplit(K, M, N, num_cus);
+    return ks > 1 ? (size_t)ks * N * M : 0;
+}
+
 template <class G>
-hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus, hipStream_t s) {
+hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAct &a, float *workspace,
+                   size_t workspace_floats, int num_cus, hipStream_t s) {
     GemmArgs ga;
     int64_t tiles_m = 0;
     for (int i = 0; i < GEMM_MULTI; i++) {
@@ -404,35 +440,46 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
         ga.tile_end[i] = i < count ? (int)tiles_m : 0x7fffffff;
     }
     ga.K = ws[0].K; ga.type = ws[0].type;
+    static const char *dbg = getenv("MI_QMM_GEMM_DEBUG");  // "1": always 128x64, "2": always 128x128, no K split
+    int ksplit = count == 1 && !dbg ? pick_ksplit(ws[0].K, ws[0].M, a.N, num_cus) : 1;
+    if (ksplit > 1 && (!workspace || workspace_floats < (size_t)ksplit * a.N * ws[0].M)) ksplit = 1;
     // 128 x 128 tiles when they still give every CU work for most of the run, else 128 x 64
-    static const char *dbg = getenv("MI_QMM_GEMM_DEBUG");  // "1": always 128x64, "2": always 128x128
-    const int64_t big = tiles_m * ((a.N + 127) / 128);
-    const bool tnt2 = dbg ? dbg[0] == '2' : 2 * big >= 3 * (int64_t)num_cus;
+    const int64_t big = tiles_m * ((a.N + 127) / 128) * ksplit;
+    const bool tnt2 = dbg ? dbg[0] == '2' : (ksplit > 1 || 2 * big >= 3 * (int64_t)num_cus);
     const int64_t tn = tnt2 ? 128 : 64, tiles_n = (a.N + tn - 1) / tn;
-    const int64_t grid = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
-    if (tiles_m > 0x7ffffff0 || grid > 0x7fffffff) return hipErrorInvalidValue;
-    if (tnt2) gemm3_kernel<G, 2><<<(unsigned)grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n);
-    else gemm3_kernel<G, 1><<<(unsigned)grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n);
+    const int64_t gx = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
+    if (tiles_m > 0x7ffffff0 || gx > 0x7fffffff) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)gx, (unsigned)ksplit);
+    float *part = ksplit > 1 ? workspace : nullptr;
+    if (tnt2) gemm3_kernel<G, 2><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part);
+    else gemm3_kernel<G, 1><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part);
+    if (ksplit > 1) {
+        const int64_t n4 = a.N * ws[0].M / 4;
+        const unsigned blocks = (unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048);
+        sum_slices_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const float4 *>(part),
+                                                 reinterpret_cast<float4 *>(ys[0]), n4, ksplit);
+    }
     return hipGetLastError();
 }
 
 int gemm_max_multi() { return GEMM_MULTI; }
 
-hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus,
-                             hipStream_t s) {
+hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, float *workspace,
+                             size_t workspace_floats, int num_cus, hipStream_t s) {
     if (count < 1 || count > GEMM_MULTI) return hipErrorInvalidValue;
     for (int i = 0; i < count; i++)
         if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || !gemm_supports(ws[i].type, ws[i].K, ws[i].M) || !ys[i])
             return hipErrorInvalidValue;
     if (a.type != T_Q8_K || a.K != ws[0].K || a.N < 1 || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
-    return ws[0].type == T_Q4_K ? launch3<GemmQ4K>(ws, ys, count, a, num_cus, s)
-                                : launch3<GemmQ6K>(ws, ys, count, a, num_cus, s);
+    return ws[0].type == T_Q4_K ? launch3<GemmQ4K>(ws, ys, count, a, workspace, workspace_floats, num_cus, s)
+                                : launch3<GemmQ6K>(ws, ys, count, a, workspace, workspace_floats, num_cus, s);
 }
 
-hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, int num_cus, hipStream_t s) {
+hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, float *workspace,
+                       size_t workspace_floats, int num_cus, hipStream_t s) {
     if (ldy != w.M) return hipErrorInvalidValue;
     float *ys[1] = {y};
-    return launch_gemm_multi(&w, ys, 1, a, num_cus, s);
+    return launch_gemm_multi(&w, ys, 1, a, workspace, workspace_floats, num_cus, s);
 }
 
 }  // namespace miqmm

@@ -36,13 +36,16 @@ hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int coun
 // largest K the GEMV handles for a weight type
 int64_t gemv_max_k(int type);
 
-// kernel 3: int8-MFMA GEMM, any N >= 1.  y[n*ldy + m]
-hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, int num_cus,
-                       hipStream_t s);
+// kernel 3: int8-MFMA GEMM, any N >= 1.  y[n*ldy + m].  workspace (device, may be null) lets the
+// launcher cut K into slices when the output alone has too few tiles to fill the GPU;
+// gemm_workspace_floats() says how much that takes (0: no split).
+hipError_t launch_gemm(const DevWeight &w, const DevAct &a, float *y, int64_t ldy, float *workspace,
+                       size_t workspace_floats, int num_cus, hipStream_t s);
 bool gemm_supports(int type, int64_t K, int64_t M);
+size_t gemm_workspace_floats(int type, int64_t K, int64_t M, int64_t N, int num_cus);
 // several weight tensors of one type and K against the same activations in one launch
-hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus,
-                             hipStream_t s);
+hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, float *workspace,
+                             size_t workspace_floats, int num_cus, hipStream_t s);
 int gemm_max_multi();
 
 }  // namespace miqmm

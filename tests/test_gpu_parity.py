@@ -241,11 +241,11 @@ def test_multi_weight_launch_matches_single(ctx):
         ms = [1024, 300, 4096]
         raws = [_weights(t, m, k, seed=100 + m) for m in ms]
         Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
-        act = ctx.act_create(qmm.vec_dot_type(t), k, 16)
-        for n in (1, 3, 9):                                # 9 > 8 columns falls back to per-weight calls
+        act = ctx.act_create(qmm.vec_dot_type(t), k, 40)
+        for n in (1, 3, 9, 40):                            # 9: per-weight calls; 40: one GEMM launch (K-quants)
             x = rng.standard_normal((n, k), dtype=np.float32)
             ctx.act_quantize(act, x)
-            want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV) for W in Ws]
+            want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV if n <= 8 else qmm.PATH_AUTO) for W in Ws]
             got = ctx.mulmat_q8_multi(Ws, act)
             for y, wnt in zip(got, want):
                 assert np.array_equal(y, wnt)
