@@ -143,6 +143,42 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
 int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count,
                            const mi_qmm_act *act, float *const *ys, int location);
 
+/* ---- GGUF files: replaces gguf.Open / File.KeyValue / File.TensorInfo / File.TensorReader,
+ *      /root/reference/fs/gguf/gguf.go:54-110, 332-351, 361-378, 390-430 (and the loader loop of
+ *      Backend.Load, /root/reference/ml/backend.go:20).  The file is mapped read-only; header,
+ *      key-values and tensor infos are parsed by open (the reference parses lazily: same values,
+ *      errors surface at open instead of later).  No GPU is needed except for gguf_upload. */
+typedef struct mi_qmm_gguf mi_qmm_gguf;
+int mi_qmm_gguf_open(const char *path, mi_qmm_gguf **out);
+void mi_qmm_gguf_close(mi_qmm_gguf *f);
+/* version, general.alignment (default 32), file offset of the tensor data, counts */
+int mi_qmm_gguf_info(const mi_qmm_gguf *f, int *version, int64_t *alignment, int64_t *data_offset,
+                     int64_t *num_kv, int64_t *num_tensors);
+/* tensor by index: name (valid until close), ggml type id, dims (dims[0] contiguous; unused = 1),
+ * offset inside the data section, byte size by the block rule of fs/gguf/tensor.go:47-76 */
+int mi_qmm_gguf_tensor(const mi_qmm_gguf *f, int64_t index, const char **name, int *type, int *n_dims,
+                       int64_t dims[4], int64_t *offset, int64_t *nbytes);
+int64_t mi_qmm_gguf_find_tensor(const mi_qmm_gguf *f, const char *name); /* index, or -1 */
+const void *mi_qmm_gguf_tensor_data(const mi_qmm_gguf *f, int64_t index); /* into the mapping; NULL if out of range */
+/* key-value lookup with the reference's rule: a key outside "general." / "tokenizer." is looked
+ * up as "<general.architecture>.<key>".  Returns the index or -1. */
+int64_t mi_qmm_gguf_find_kv(const mi_qmm_gguf *f, const char *key);
+/* key (valid until close), value type (0..12 = u8,i8,u16,i16,u32,i32,f32,bool,string,array,u64,i64,f64),
+ * and for arrays the element type and length */
+int mi_qmm_gguf_kv(const mi_qmm_gguf *f, int64_t index, const char **key, int *type, int *elem_type,
+                   int64_t *count);
+/* Scalar accessors; elem < 0 reads the value itself, elem >= 0 that element of an array.  As in
+ * the reference (fs/gguf/keyvalue.go:42-91) a kind mismatch is not an error: the result is 0 / "". */
+int mi_qmm_gguf_kv_int(const mi_qmm_gguf *f, int64_t index, int64_t elem, int64_t *out);
+int mi_qmm_gguf_kv_uint(const mi_qmm_gguf *f, int64_t index, int64_t elem, uint64_t *out);
+int mi_qmm_gguf_kv_float(const mi_qmm_gguf *f, int64_t index, int64_t elem, double *out);
+int mi_qmm_gguf_kv_bool(const mi_qmm_gguf *f, int64_t index, int64_t elem, int *out);
+/* string bytes are not NUL-terminated: *str points into the mapping, *len is the length */
+int mi_qmm_gguf_kv_string(const mi_qmm_gguf *f, int64_t index, int64_t elem, const char **str, int64_t *len);
+/* upload tensor `index` (2-D, a type this library multiplies: 2, 8, 12, 14) as a resident weight:
+ * K = dims[0], M = dims[1]; the bytes go from the mapping to the device */
+int mi_qmm_gguf_upload(mi_qmm_ctx *ctx, const mi_qmm_gguf *f, int64_t index, mi_qmm_weight **out);
+
 /* ---- diagnostics */
 const char *mi_qmm_last_error(void); /* thread-local, never NULL */
 const char *mi_qmm_version(void);

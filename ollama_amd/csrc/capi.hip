@@ -8,6 +8,7 @@
 #include <new>
 
 #include "../../include/mi_qmm.h"
+#include "gguf_file.h"
 #include "internal.h"
 
 using namespace miqmm;
@@ -54,6 +55,10 @@ struct mi_qmm_weight {
     void *base = nullptr;
     size_t bytes = 0;
     DevWeight dev{};
+};
+
+struct mi_qmm_gguf {
+    GgufFile file;
 };
 
 struct mi_qmm_act {
@@ -689,6 +694,161 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         HIP_TRY(hipStreamSynchronize(ctx->stream));
     }
     return MI_QMM_OK;
+}
+
+}  // extern "C"
+
+// ---- GGUF files ----------------------------------------------------------------------------------------
+extern "C" {
+
+int mi_qmm_gguf_open(const char *path, mi_qmm_gguf **out) {
+    if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (!path) return fail(MI_QMM_ERR_INVALID, "path is NULL");
+    mi_qmm_gguf *g = new (std::nothrow) mi_qmm_gguf();
+    if (!g) return fail(MI_QMM_ERR_NOMEM, "host allocation failed");
+    const std::string err = g->file.open(path);
+    if (!err.empty()) {
+        delete g;
+        const bool unsupported = err.find("unsupported") != std::string::npos;
+        return fail(unsupported ? MI_QMM_ERR_UNSUPPORTED : MI_QMM_ERR_INVALID, "%s", err.c_str());
+    }
+    *out = g;
+    return MI_QMM_OK;
+}
+
+void mi_qmm_gguf_close(mi_qmm_gguf *f) { delete f; }
+
+int mi_qmm_gguf_info(const mi_qmm_gguf *f, int *version, int64_t *alignment, int64_t *data_offset, int64_t *num_kv,
+                     int64_t *num_tensors) {
+    if (!f) return fail(MI_QMM_ERR_INVALID, "gguf is NULL");
+    if (version) *version = (int)f->file.version;
+    if (alignment) *alignment = f->file.alignment;
+    if (data_offset) *data_offset = (int64_t)f->file.data_offset;
+    if (num_kv) *num_kv = (int64_t)f->file.kvs.size();
+    if (num_tensors) *num_tensors = (int64_t)f->file.tensors.size();
+    return MI_QMM_OK;
+}
+
+int mi_qmm_gguf_tensor(const mi_qmm_gguf *f, int64_t index, const char **name, int *type, int *n_dims,
+                       int64_t dims[4], int64_t *offset, int64_t *nbytes) {
+    if (!f) return fail(MI_QMM_ERR_INVALID, "gguf is NULL");
+    if (index < 0 || index >= (int64_t)f->file.tensors.size())
+        return fail(MI_QMM_ERR_INVALID, "tensor index %lld outside 0..%zu", (long long)index, f->file.tensors.size());
+    const GgufTensor &t = f->file.tensors[index];
+    if (name) *name = t.name.c_str();
+    if (type) *type = (int)t.type;
+    if (n_dims) *n_dims = (int)t.n_dims;
+    if (dims)
+        for (int i = 0; i < 4; i++) dims[i] = (int64_t)t.dims[i];
+    if (offset) *offset = (int64_t)t.offset;
+    if (nbytes) *nbytes = t.nbytes;
+    return MI_QMM_OK;
+}
+
+int64_t mi_qmm_gguf_find_tensor(const mi_qmm_gguf *f, const char *name) {
+    return f && name ? f->file.find_tensor(name) : -1;
+}
+
+const void *mi_qmm_gguf_tensor_data(const mi_qmm_gguf *f, int64_t index) {
+    if (!f || index < 0 || index >= (int64_t)f->file.tensors.size()) return nullptr;
+    return f->file.tensor_data(f->file.tensors[index]);
+}
+
+int64_t mi_qmm_gguf_find_kv(const mi_qmm_gguf *f, const char *key) { return f && key ? f->file.find_kv(key) : -1; }
+
+int mi_qmm_gguf_kv(const mi_qmm_gguf *f, int64_t index, const char **key, int *type, int *elem_type, int64_t *count) {
+    if (!f) return fail(MI_QMM_ERR_INVALID, "gguf is NULL");
+    if (index < 0 || index >= (int64_t)f->file.kvs.size())
+        return fail(MI_QMM_ERR_INVALID, "key-value index %lld outside 0..%zu", (long long)index, f->file.kvs.size());
+    const GgufKV &kv = f->file.kvs[index];
+    if (key) *key = kv.key.c_str();
+    if (type) *type = (int)kv.value.type;
+    if (elem_type) *elem_type = kv.value.type == GGUF_ARRAY ? (int)kv.value.elem_type : -1;
+    if (count) *count = kv.value.type == GGUF_ARRAY ? (int64_t)kv.value.count : 0;
+    return MI_QMM_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+// the scalar a (key-value index, element) pair denotes; rc != 0 with the error set if there is none
+int kv_scalar(const mi_qmm_gguf *f, int64_t index, int64_t elem, GgufValue &out) {
+    if (!f) return fail(MI_QMM_ERR_INVALID, "gguf is NULL");
+    if (index < 0 || index >= (int64_t)f->file.kvs.size())
+        return fail(MI_QMM_ERR_INVALID, "key-value index %lld outside 0..%zu", (long long)index, f->file.kvs.size());
+    const GgufValue &v = f->file.kvs[index].value;
+    if (elem < 0) {
+        out = v;
+        if (v.type == GGUF_ARRAY) out.type = 0xffffffffu;  // an array is no scalar: every accessor yields its zero
+        return MI_QMM_OK;
+    }
+    if (v.type != GGUF_ARRAY || (uint64_t)elem >= v.count)
+        return fail(MI_QMM_ERR_INVALID, "element %lld outside the value (array length %llu)", (long long)elem,
+                    (unsigned long long)(v.type == GGUF_ARRAY ? v.count : 0));
+    out = GgufFile::array_elem(v, (uint64_t)elem);
+    return MI_QMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_qmm_gguf_kv_int(const mi_qmm_gguf *f, int64_t index, int64_t elem, int64_t *out) {
+    GgufValue v;
+    int rc = kv_scalar(f, index, elem, v);
+    if (rc) return rc;
+    if (out) *out = GgufFile::as_int(v);
+    return MI_QMM_OK;
+}
+
+int mi_qmm_gguf_kv_uint(const mi_qmm_gguf *f, int64_t index, int64_t elem, uint64_t *out) {
+    GgufValue v;
+    int rc = kv_scalar(f, index, elem, v);
+    if (rc) return rc;
+    if (out) *out = GgufFile::as_uint(v);
+    return MI_QMM_OK;
+}
+
+int mi_qmm_gguf_kv_float(const mi_qmm_gguf *f, int64_t index, int64_t elem, double *out) {
+    GgufValue v;
+    int rc = kv_scalar(f, index, elem, v);
+    if (rc) return rc;
+    if (out) *out = GgufFile::as_float(v);
+    return MI_QMM_OK;
+}
+
+int mi_qmm_gguf_kv_bool(const mi_qmm_gguf *f, int64_t index, int64_t elem, int *out) {
+    GgufValue v;
+    int rc = kv_scalar(f, index, elem, v);
+    if (rc) return rc;
+    if (out) *out = GgufFile::as_bool(v) ? 1 : 0;
+    return MI_QMM_OK;
+}
+
+int mi_qmm_gguf_kv_string(const mi_qmm_gguf *f, int64_t index, int64_t elem, const char **str, int64_t *len) {
+    GgufValue v;
+    int rc = kv_scalar(f, index, elem, v);
+    if (rc) return rc;
+    const bool is_str = v.type == GGUF_STRING;
+    if (str) *str = is_str ? reinterpret_cast<const char *>(v.data) : "";
+    if (len) *len = is_str ? (int64_t)v.len : 0;
+    return MI_QMM_OK;
+}
+
+int mi_qmm_gguf_upload(mi_qmm_ctx *ctx, const mi_qmm_gguf *f, int64_t index, mi_qmm_weight **out) {
+    if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (!f) return fail(MI_QMM_ERR_INVALID, "gguf is NULL");
+    if (index < 0 || index >= (int64_t)f->file.tensors.size())
+        return fail(MI_QMM_ERR_INVALID, "tensor index %lld outside 0..%zu", (long long)index, f->file.tensors.size());
+    const GgufTensor &t = f->file.tensors[index];
+    if (t.n_dims != 2)
+        return fail(MI_QMM_ERR_UNSUPPORTED, "tensor \"%s\" has %u dimensions: only 2-D weights take part in Mulmat",
+                    t.name.c_str(), t.n_dims);
+    return mi_qmm_weight_upload(ctx, (int)t.type, f->file.tensor_data(t), (int64_t)t.dims[0], (int64_t)t.dims[1],
+                                MI_QMM_HOST, out);
 }
 
 }  // extern "C"

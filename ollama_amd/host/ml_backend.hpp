@@ -77,6 +77,31 @@ public:
         check(mi_qmm_weight_upload(ctx_, ggml_type, gguf_bytes, k, m, MI_QMM_HOST, &t->weight_));
         tensors_[name] = t;
     }
+    // A whole model file (the modelPath ml.NewBackend receives, /root/reference/ml/backend.go:83): every
+    // 2-D tensor of a type the Mulmat path multiplies is uploaded straight from the file mapping;
+    // other tensors (norms, f32 embeddings) are outside this path and are skipped.  Returns how many
+    // tensors were loaded.
+    int LoadFile(const std::string &path) {
+        mi_qmm_gguf *f = nullptr;
+        check(mi_qmm_gguf_open(path.c_str(), &f));
+        int64_t n = 0;
+        int loaded = 0, rc = mi_qmm_gguf_info(f, nullptr, nullptr, nullptr, nullptr, &n);
+        for (int64_t i = 0; rc == MI_QMM_OK && i < n; i++) {
+            const char *name = nullptr;
+            int type = 0, nd = 0;
+            int64_t dims[4];
+            rc = mi_qmm_gguf_tensor(f, i, &name, &type, &nd, dims, nullptr, nullptr);
+            if (rc != MI_QMM_OK || nd != 2 || mi_qmm_vec_dot_type(type) < 0) continue;
+            auto t = std::make_shared<Tensor>();
+            t->shape_ = {dims[0], dims[1]};
+            t->type_ = type;
+            rc = mi_qmm_gguf_upload(ctx_, f, i, &t->weight_);
+            if (rc == MI_QMM_OK) { tensors_[name] = t; loaded++; }
+        }
+        mi_qmm_gguf_close(f);
+        check(rc);
+        return loaded;
+    }
     std::shared_ptr<Tensor> Get(const std::string &name) const {
         auto it = tensors_.find(name);
         return it == tensors_.end() ? nullptr : it->second;  // nil for an unknown name, like the reference

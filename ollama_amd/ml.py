@@ -159,17 +159,34 @@ class Context:
 
 
 class Backend:
-    """Weights resident on one MI355X.  ``tensors`` maps a GGUF tensor name to
-    (ggml_type, shape [K, M], block bytes) -- what fs/ggml hands out for a tensor
-    (/root/reference/fs/ggml/gguf.go:281-308)."""
+    """Weights resident on one MI355X.  ``tensors`` is either the path of a GGUF file -- the model file
+    ``ml.NewBackend(modelPath, params)`` receives, /root/reference/ml/backend.go:83 -- or a dict mapping a
+    tensor name to (ggml_type, shape [K, M], block bytes), what fs/ggml hands out for a tensor
+    (/root/reference/fs/ggml/gguf.go:281-308).  From a file, Load uploads every 2-D tensor of a type the
+    Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q6_K) straight from the file mapping; other tensors
+    (norms, f32 embeddings) are outside this path and are skipped."""
 
-    def __init__(self, tensors: Dict[str, Tuple[int, Sequence[int], np.ndarray]], device: int = 0):
+    def __init__(self, tensors, device: int = 0):
         self._ctx = qmm.Context(device)
         self._tensors: Dict[str, Tensor] = {}
         self._spec = tensors
         self._loaded = False
 
     def Load(self, progress=None) -> None:
+        if isinstance(self._spec, (str, bytes)):
+            from . import gguf
+
+            with gguf.File(self._spec if isinstance(self._spec, str) else self._spec.decode()) as f:
+                infos = [t for t in f.TensorInfos() if len(t.Shape) == 2 and qmm.vec_dot_type(t.Type) >= 0]
+                for i, ti in enumerate(infos):
+                    t = Tensor(ti.Shape, ti.Type)
+                    t._weight = f.Upload(self._ctx, ti.Name)
+                    t._raw = f.TensorBytes(ti.Name)
+                    self._tensors[ti.Name] = t
+                    if progress:
+                        progress((i + 1) / max(len(infos), 1))
+            self._loaded = True
+            return
         total = max(len(self._spec), 1)
         for i, (name, (ggml_type, shape, raw)) in enumerate(self._spec.items()):
             if len(shape) != 2:

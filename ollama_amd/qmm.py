@@ -26,6 +26,9 @@ EXPORTS = [
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
     "mi_qmm_mulmat_multi",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
+    "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
+    "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
+    "mi_qmm_gguf_kv_float", "mi_qmm_gguf_kv_bool", "mi_qmm_gguf_kv_string", "mi_qmm_gguf_upload",
     "mi_qmm_last_error", "mi_qmm_version", "mi_qmm_device_info",
 ]
 
@@ -81,6 +84,22 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_q8_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_multi.restype = ci
     L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
+    P = ctypes.POINTER
+    L.mi_qmm_gguf_open.restype = ci; L.mi_qmm_gguf_open.argtypes = [ctypes.c_char_p, P(vp)]
+    L.mi_qmm_gguf_close.restype = None; L.mi_qmm_gguf_close.argtypes = [vp]
+    L.mi_qmm_gguf_info.restype = ci; L.mi_qmm_gguf_info.argtypes = [vp, P(ci), P(i64), P(i64), P(i64), P(i64)]
+    L.mi_qmm_gguf_tensor.restype = ci
+    L.mi_qmm_gguf_tensor.argtypes = [vp, i64, P(ctypes.c_char_p), P(ci), P(ci), P(i64), P(i64), P(i64)]
+    L.mi_qmm_gguf_find_tensor.restype = i64; L.mi_qmm_gguf_find_tensor.argtypes = [vp, ctypes.c_char_p]
+    L.mi_qmm_gguf_tensor_data.restype = vp; L.mi_qmm_gguf_tensor_data.argtypes = [vp, i64]
+    L.mi_qmm_gguf_find_kv.restype = i64; L.mi_qmm_gguf_find_kv.argtypes = [vp, ctypes.c_char_p]
+    L.mi_qmm_gguf_kv.restype = ci; L.mi_qmm_gguf_kv.argtypes = [vp, i64, P(ctypes.c_char_p), P(ci), P(ci), P(i64)]
+    L.mi_qmm_gguf_kv_int.restype = ci; L.mi_qmm_gguf_kv_int.argtypes = [vp, i64, i64, P(i64)]
+    L.mi_qmm_gguf_kv_uint.restype = ci; L.mi_qmm_gguf_kv_uint.argtypes = [vp, i64, i64, P(ctypes.c_uint64)]
+    L.mi_qmm_gguf_kv_float.restype = ci; L.mi_qmm_gguf_kv_float.argtypes = [vp, i64, i64, P(ctypes.c_double)]
+    L.mi_qmm_gguf_kv_bool.restype = ci; L.mi_qmm_gguf_kv_bool.argtypes = [vp, i64, i64, P(ci)]
+    L.mi_qmm_gguf_kv_string.restype = ci; L.mi_qmm_gguf_kv_string.argtypes = [vp, i64, i64, P(vp), P(i64)]
+    L.mi_qmm_gguf_upload.restype = ci; L.mi_qmm_gguf_upload.argtypes = [vp, vp, i64, P(vp)]
     L.mi_qmm_last_error.restype = ctypes.c_char_p; L.mi_qmm_last_error.argtypes = []
     L.mi_qmm_version.restype = ctypes.c_char_p; L.mi_qmm_version.argtypes = []
     L.mi_qmm_device_info.restype = ci

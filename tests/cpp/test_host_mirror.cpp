@@ -3,6 +3,7 @@
 // Links libmi_qmm.so (the product) and oracle/libggml_ref.so (the checker; test infrastructure).
 #include <cmath>
 #include <cstdio>
+#include <cstring>
 #include <random>
 #include <vector>
 
@@ -73,6 +74,51 @@ int main() {
             backend.Get("output.weight")->Mulmat(*ctx, ctx->FromFloats(std::vector<float>(512), {512, 1}));
         } catch (const Error &) { threw = true; }
         if (!threw) { printf("FAIL: dimension mismatch did not throw\n"); failures++; }
+        // the same weights from a GGUF file: written here byte by byte (header, one key-value, tensor
+        // infos, padding to 32, data), loaded through LoadFile, results must equal the in-memory ones
+        {
+            std::string bytes = "GGUF";
+            auto put = [&](const void *p, size_t n) { bytes.append(static_cast<const char *>(p), n); };
+            auto put_u32 = [&](uint32_t v) { put(&v, 4); };
+            auto put_u64 = [&](uint64_t v) { put(&v, 8); };
+            auto put_str = [&](const std::string &v) { put_u64(v.size()); put(v.data(), v.size()); };
+            put_u32(3); put_u64(2); put_u64(1);
+            put_str("general.architecture"); put_u32(8); put_str("llama");
+            uint64_t off = 0;
+            std::vector<uint64_t> offs;
+            for (int i = 0; i < 2; i++) {
+                put_str(specs[i].name); put_u32(2); put_u64((uint64_t)specs[i].k); put_u64((uint64_t)specs[i].m);
+                put_u32((uint32_t)specs[i].type); put_u64(off);
+                offs.push_back(off);
+                off += raws[i].size();
+                off += (32 - off % 32) % 32;
+            }
+            bytes.append((32 - bytes.size() % 32) % 32, '\0');
+            const size_t base = bytes.size();
+            bytes.resize(base + off, '\0');
+            for (int i = 0; i < 2; i++) memcpy(&bytes[base + offs[i]], raws[i].data(), raws[i].size());
+            const std::string path = "/tmp/mi_qmm_host_mirror_test.gguf";
+            FILE *fp = fopen(path.c_str(), "wb");
+            if (!fp || fwrite(bytes.data(), 1, bytes.size(), fp) != bytes.size()) { printf("FAIL: cannot write %s\n", path.c_str()); return 1; }
+            fclose(fp);
+            Backend from_file(0);
+            const int loaded = from_file.LoadFile(path);
+            remove(path.c_str());
+            if (loaded != 2) { printf("FAIL: LoadFile loaded %d tensors, want 2\n", loaded); failures++; }
+            auto xv = randn(1024 * 2, 1.0f, 5);
+            for (int i = 0; i < 2 && loaded == 2; i++) {
+                auto c1 = backend.NewContext();
+                auto c2 = from_file.NewContext();
+                auto y1 = backend.Get(specs[i].name)->Mulmat(*c1, c1->FromFloats(xv, {1024, 2}));
+                auto y2 = from_file.Get(specs[i].name)->Mulmat(*c2, c2->FromFloats(xv, {1024, 2}));
+                c1->Compute();
+                c2->Compute();
+                const bool same = y1->Floats() == y2->Floats();
+                printf("%-24s from file %s\n", specs[i].name, same ? "ok" : "FAIL");
+                if (!same) failures++;
+            }
+            from_file.Close();
+        }
         backend.Close();
         printf(failures ? "host mirror: %d FAILURES\n" : "host mirror: all ok\n", failures);
         return failures ? 1 : 0;

@@ -1,0 +1,63 @@
+"""GGUF file -> resident weights -> Mulmat, on the GPU: the loader row of the path."""
+import numpy as np
+import pytest
+
+import npref
+import oracle
+from ollama_amd import gguf, ml, qmm, synth
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def _model_file(tmp_path):
+    k = 1024
+    tensors, raws = [], {}
+    for name, t, m in (("blk.0.attn_q.weight", qmm.Q4_K, 96), ("blk.0.ffn_down.weight", qmm.Q6_K, 40),
+                       ("blk.0.attn_k.weight", qmm.Q8_0, 33), ("output.weight", qmm.Q4_0, 50)):
+        raw = synth.weights(t, m, k, seed=m).reshape(-1)
+        raws[name] = (t, m, raw)
+        tensors.append((name, t, [k, m], raw.tobytes()))
+    tensors.append(("blk.0.attn_norm.weight", 0, [k], np.ones(k, np.float32).tobytes()))   # f32, 1-D: not on the path
+    p = str(tmp_path / "model.gguf")
+    gguf.write_gguf(p, {"general.architecture": "llama", "block_count": np.uint32(1)}, tensors)
+    return p, k, raws
+
+
+def test_upload_from_file_equals_upload_from_memory(tmp_path):
+    p, k, raws = _model_file(tmp_path)
+    ctx = qmm.Context(0)
+    x = np.random.default_rng(3).standard_normal((3, k), dtype=np.float32)
+    with gguf.File(p) as f:
+        for name, (t, m, raw) in raws.items():
+            assert np.array_equal(f.TensorBytes(name), raw)
+            Wf = f.Upload(ctx, name)
+            Wm = ctx.upload(t, raw, k, m)
+            assert (Wf.type, Wf.k, Wf.m) == (t, k, m)
+            assert np.array_equal(ctx.mulmat(Wf, x), ctx.mulmat(Wm, x))
+            Wf.free(); Wm.free()
+        with pytest.raises(qmm.QmmError) as e:
+            f.Upload(ctx, "blk.0.attn_norm.weight")            # 1-D f32
+        assert e.value.code == qmm.ERR_UNSUPPORTED
+    ctx.close()
+
+
+def test_backend_from_gguf_path(tmp_path):
+    p, k, raws = _model_file(tmp_path)
+    seen = []
+    b = ml.Backend(p)
+    b.Load(progress=seen.append)
+    assert seen and seen[-1] == 1.0
+    assert b.Get("blk.0.attn_norm.weight") is None and b.Get("nope") is None
+    ctx = b.NewContext()
+    xs = np.random.default_rng(4).standard_normal((2, k), dtype=np.float32)
+    x = ctx.FromFloats(xs.reshape(-1), k, 2)
+    outs = {name: b.Get(name).Mulmat(ctx, x) for name in raws}
+    ctx.Compute(*outs.values())
+    for name, (t, m, raw) in raws.items():
+        assert outs[name].Shape() == [m, 2]
+        want = oracle.mul_mat(t, raw, k, m, xs, nthreads=4)
+        assert npref.rel_err(outs[name].Floats().reshape(2, m), want) <= TOL, name
+        assert b.Get(name).Bytes() == raw.tobytes()
+    ctx.Close()
+    b.Close()
