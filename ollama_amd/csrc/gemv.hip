@@ -659,7 +659,10 @@ __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(
             if (i + 1 < nrw) cur = P::load(w, g, r0 + rl0 + i + 1);  // wave-uniform branch
 #pragma unroll
             for (int n = 0; n < NC; n++) {
-                const float tot = wave_total(acc[n]);  // valid in lanes 48..63
+                // Lanes 48..63 all hold the total, but each quad added the four quads of its row in its own
+                // order: take lane 63's value, so a row's result does not depend on which lane parks it
+                // (i.e. not on how many rows a wave was given).
+                const float tot = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_total(acc[n])), 63));
                 if (DIRECT) keep[n] = lane == 63 - i ? tot : keep[n];
                 else if (lane == 63) part[((rl0 + i) * NC + n) * kw + kseg] = tot;
             }

@@ -287,6 +287,29 @@ def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
             W.free()
 
 
+def test_results_do_not_depend_on_rows_per_wave(ctx):
+    """A wave parks the totals of its rows in different lanes; every lane of the last 16 holds the wave
+    total, but summed in a lane-dependent order.  The kernel must take one fixed lane's value, so that
+    the same row gives the same bits whatever the launch geometry: a weight alone (2 rows per wave), as
+    one of several tensors of a launch (4 rows per wave above 64 Ki rows in total) and with many columns
+    (4 rows per wave)."""
+    k = 1024
+    rng = np.random.default_rng(5)
+    raw = _weights(Q4_K, 48, k, seed=3)
+    W = ctx.upload(Q4_K, raw, k, 48)
+    big = ctx.upload(Q4_K, np.tile(_weights(Q4_K, 1024, k, seed=4).reshape(1024, -1), (66, 1)).reshape(-1), k, 67584)
+    for n in (1, 4):
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        act = ctx.act_create(Q8_K, k, 8)
+        ctx.act_quantize(act, x)
+        alone = ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV)
+        together = ctx.mulmat_q8_multi([big, W], act)[1]
+        assert np.array_equal(alone, together), n
+        assert np.array_equal(alone, ctx.mulmat(W, x, path=qmm.PATH_GEMV)), n
+        act.free()
+    W.free(); big.free()
+
+
 def test_mulmat_multi_fallbacks_and_errors(ctx):
     k = 1024
     rng = np.random.default_rng(8)
