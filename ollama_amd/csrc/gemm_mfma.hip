@@ -16,19 +16,18 @@
 //     (S = 64*S_h + S_l) costs two more MFMAs per 32x32 tile and super-block.
 //   * Per super-block and output there remains one fp32 epilogue: y += yd_n * (d_m * I - dmin_m * Imin).
 //
-// Data flow: the activation tile of a super-block (128 rows x 256 int8, their block scale and block-sum
-// digits) goes HBM/L2 -> LDS by direct-to-LDS loads (global_load_lds_dwordx4: no registers, no vector
-// ALU work, two LDS buffers so the copy of the next tile runs under the current tile's MFMAs) and is
-// read as the MFMA A operand; the 16-byte pieces of a row are XOR-swizzled with the row number so the
-// 32 rows x 16 bytes of an operand read fall on distinct banks.  Each wave owns 32 weight rows, loads their packed
-// blocks straight from HBM, expands them to digit planes IN REGISTERS as the MFMA B operand (each lane
-// needs 16 consecutive K values of one row -- exactly a 16-byte piece of the GGUF block) and reuses them
-// for all four 32-row activation sub-tiles.  W on the B side puts one weight row in each lane's 16
-// accumulators (one d/dmin per lane) and makes the output stores contiguous in m.
+// Data flow: everything a workgroup multiplies in one super-block step -- 128 rows of packed weights,
+// 64 or 128 rows of activation quants, their block scales and block-sum digits -- goes HBM/L2 -> LDS by
+// direct-to-LDS loads (global_load_lds: no registers, no vector-ALU work, consecutive lanes fetch
+// consecutive 16-byte pieces), two LDS stages, the copy of step sb+1 running under the math of step sb.
+// A wave reads the packed blocks of its 32 weight rows from LDS, expands them to digit planes IN
+// REGISTERS as the MFMA B operand (a lane needs 16 consecutive K values of one row -- exactly a 16-byte
+// piece of the GGUF block) and reuses them for its 32-row activation sub-tiles, which come from LDS as
+// the A operand; rows are XOR-swizzled or odd-pitched so that operand reads are conflict-free.  W on
+// the B side puts one weight row in each lane's 16 accumulators (one d/dmin per lane) and makes the
+// output stores contiguous in m.
 #include <hip/hip_fp16.h>
 
-#include <cstdlib>
-#include <type_traits>
 
 #include "internal.h"
 
@@ -440,12 +439,11 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
         ga.tile_end[i] = i < count ? (int)tiles_m : 0x7fffffff;
     }
     ga.K = ws[0].K; ga.type = ws[0].type;
-    static const char *dbg = getenv("MI_QMM_GEMM_DEBUG");  // "1": always 128x64, "2": always 128x128, no K split
-    int ksplit = count == 1 && !dbg ? pick_ksplit(ws[0].K, ws[0].M, a.N, num_cus) : 1;
+    int ksplit = count == 1 ? pick_ksplit(ws[0].K, ws[0].M, a.N, num_cus) : 1;
     if (ksplit > 1 && (!workspace || workspace_floats < (size_t)ksplit * a.N * ws[0].M)) ksplit = 1;
     // 128 x 128 tiles when they still give every CU work for most of the run, else 128 x 64
     const int64_t big = tiles_m * ((a.N + 127) / 128) * ksplit;
-    const bool tnt2 = dbg ? dbg[0] == '2' : (ksplit > 1 || 2 * big >= 3 * (int64_t)num_cus);
+    const bool tnt2 = ksplit > 1 || 2 * big >= 3 * (int64_t)num_cus;
     const int64_t tn = tnt2 ? 128 : 64, tiles_n = (a.N + tn - 1) / tn;
     const int64_t gx = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
     if (tiles_m > 0x7ffffff0 || gx > 0x7fffffff) return hipErrorInvalidValue;

@@ -7,22 +7,19 @@
 //
 // Shape of the computation (HBM-bound: every weight byte is read exactly once):
 //   * A wavefront owns a fixed slice of K (a "segment": 4096 elements for the K-quants, 2048 for
-//     Q4_0, 1024 for Q8_0) and walks down the rows.  A lane's piece of a row is one or two aligned
+//     Q4_0, 1024 for Q8_0) and a few consecutive rows.  A lane's piece of a row is one or two aligned
 //     16-byte loads and the wave as a whole reads a contiguous run of the row.
 //   * Because the lane's K positions never change, its Q8 activation quants (and the block scale and
 //     partial sums that go with them) are loaded ONCE into registers and reused for every row: the
-//     inner loop reads nothing but weights.  Those loads are issued before the first weight loads:
-//     the memory counter retires in order, so anything issued after the weights could only be waited
-//     for by draining every weight load as well.
+//     inner loop reads nothing but weights.
 //   * Nibbles / 6-bit values are unpacked in registers, multiplied with v_dot4_i32_i8, the sub-block
-//     scales applied in-lane.  The U rows of a pass are reduced across the wave together (the
-//     lane-index bits that are summed over select which row a lane keeps), and waves that own
+//     scales applied in-lane, each row reduced across the wave with cross-lane moves; waves that own
 //     different K segments of the same rows combine through LDS at the end of the workgroup.
-//   * Rows are processed in passes of U with two register buffers, so up to 2U rows per wave are in
-//     flight; for the FFN shapes that is every row the wave owns, i.e. one exposed HBM latency.
+//   * Two kernels.  gemv_thin_kernel (everything up to eight K segments per row): many small waves,
+//     a rolled loop of about 1 KiB, one row in registers and the next in flight, the latency hidden
+//     by occupancy; optionally quantizes f32 activations itself in its prologue.  gemv_kernel (longer
+//     rows only): few waves, each K segment list in registers, rows in double-buffered passes.
 #include <hip/hip_fp16.h>
-
-#include <cstdlib>
 
 #include "internal.h"
 #include "quant_dev.h"
@@ -719,7 +716,7 @@ size_t thin_act_lds(int64_t K, int nc) {
 }
 
 template <class P>
-bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, int rows_per_wave, Plan &p) {
+bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p) {
     const int nseg = (int)((K + P::SEG - 1) / P::SEG);
     if (nseg < 1 || nseg > 8) return false;
     p.spw = 1;
@@ -727,10 +724,9 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, int rows_per_w
     const int max_waves = p.kw > thin_max_waves(nc, f32) ? p.kw : thin_max_waves(nc, f32);
     p.rw_log2 = 0;
     while (p.kw << (p.rw_log2 + 1) <= max_waves) p.rw_log2++;
-    static const char *rw_env = getenv("MI_QMM_GEMV_RW");
-    if (rw_env && f32) { p.rw_log2 = atoi(rw_env); while (p.kw << p.rw_log2 > thin_max_waves(nc, f32) && p.rw_log2 > 0) p.rw_log2--; }
     p.rw = 1 << p.rw_log2;
-    if (rows_per_wave <= 0) {
+    int rows_per_wave;
+    {
         if (f32) {
             // every workgroup re-quantizes x: keep them to one resident round (at most 1.75 per CU),
             // an even number of rows per wave
@@ -779,10 +775,7 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i].M;
     Plan p;
-    static const char *mode_env = getenv("MI_QMM_GEMV_DEBUG");  // "fat" | "thin[:rows_per_wave]"
-    const bool force_fat = mode_env && mode_env[0] == 'f';
-    const int rpw_env = mode_env && mode_env[0] == 't' && mode_env[4] == ':' ? atoi(mode_env + 5) : 0;
-    const bool thin = !force_fat && make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, rpw_env, p);
+    const bool thin = make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, p);
     if (xf && !thin) return hipErrorInvalidValue;  // callers ask gemv_f32_supported() first
     if (!thin) {
         if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
@@ -884,10 +877,10 @@ bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
     if (ncols < 1 || ncols > MAXC || K < 1 || total_m < 1 || total_m > 65536) return false;
     Plan p;
     switch (type) {
-    case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, ncols, true, 0, p);
-    case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, ncols, true, 0, p);
-    case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, ncols, true, 0, p);
-    case T_Q8_0: return make_thin_plan<PolQ8_0>(K, total_m, ncols, true, 0, p);
+    case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, ncols, true, p);
+    case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, ncols, true, p);
+    case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, ncols, true, p);
+    case T_Q8_0: return make_thin_plan<PolQ8_0>(K, total_m, ncols, true, p);
     default: return false;
     }
 }

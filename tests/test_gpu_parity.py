@@ -334,6 +334,29 @@ def test_mulmat_multi_fallbacks_and_errors(ctx):
         W.free()
 
 
+def test_randomized_shape_sweep(ctx):
+    """seeded random (type, K, M, N) combinations through the default dispatch -- thin GEMV with and
+    without in-kernel quantization, multi-segment rows, long-K kernel, column groups, GEMM tiles of
+    both sizes, K slices -- against the oracle"""
+    rng = np.random.default_rng(20240607)
+    for case in range(28):
+        t = int(rng.choice(WTYPES))
+        blk = npref.BLOCK[t]
+        k = int(rng.integers(1, 40 if blk == 256 else 160)) * blk
+        if case % 7 == 3:
+            k = int(rng.integers(33, 70)) * 256                       # long rows: several K segments, K slices
+        m = int(rng.integers(1, 400))
+        n = int(rng.choice([1, 1, 2, 3, 5, 8, 9, 17, 33, 64, 130]))
+        w_raw = _weights(t, m, k, seed=case)
+        W = ctx.upload(t, w_raw, k, m)
+        x = rng.standard_normal((n, k), dtype=np.float32) * np.float32(rng.choice([1e-3, 1.0, 30.0]))
+        got = ctx.mulmat(W, x)
+        want = oracle.mul_mat(t, w_raw, k, m, x, nthreads=8)
+        err = npref.rel_err(got, want)
+        assert got.shape == (n, m) and err <= TOL, f"case {case}: {NAMES[t]} k={k} m={m} n={n}: rel err {err}"
+        W.free()
+
+
 # ---- kernel 3: int8-MFMA GEMM ---------------------------------------------------------------------
 @pytest.mark.parametrize("t", [Q4_K, Q6_K])
 @pytest.mark.parametrize("k,m,n", [(256, 1, 1), (256, 32, 32), (512, 31, 33), (1024, 128, 128), (1024, 257, 200),
