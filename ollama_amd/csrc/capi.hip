@@ -397,6 +397,14 @@ int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k,
 // ---- the product ------------------------------------------------------------------------------------
 namespace {
 
+// From this many activation columns up a K-quant product below the GEMM's batch goes to the
+// matrix-core skinny kernel instead of the streaming GEMV (measured crossover on MI355X: the GEMV pays
+// one v_dot4 pass per column).
+bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
+    const int64_t from = type == T_Q4_K ? 5 : 6;
+    return n >= from && skinny_supports(type, K, M);
+}
+
 // dy: device output [n][M].  Picks the kernel and queues it on the ctx's stream.
 int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path) {
     const int64_t K = w->dev.K, M = w->dev.M, n = a.N;
@@ -418,9 +426,17 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
         }
         HIP_TRY(launch_gemm(w->dev, a, dy, M, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
     } else {
-        for (int64_t c0 = 0; c0 < n; c0 += 8) {
-            const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
-            HIP_TRY(launch_gemv(w->dev, a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
+        if (a.sd8 && wants_skinny(w->dev.type, K, M, n)) {
+            // from a few columns up the K-quants go to the matrix cores, 16 columns per launch: the
+            // streaming GEMV pays one v_dot4 pass per column
+            for (int64_t c0 = 0; c0 < n; c0 += 16)
+                HIP_TRY(launch_skinny(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus,
+                                      ctx->stream));
+        } else {
+            for (int64_t c0 = 0; c0 < n; c0 += 8) {
+                const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
+                HIP_TRY(launch_gemv(w->dev, a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
+            }
         }
     }
     return MI_QMM_OK;
@@ -468,7 +484,8 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         dy = (float *)((char *)ctx->io_buf + yoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    if (path != MI_QMM_PATH_GEMM && n <= 8 && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
+    if (path != MI_QMM_PATH_GEMM && n <= 8 && !wants_skinny(w->dev.type, K, M, n) &&
+        gemv_f32_supported(w->dev.type, K, M, (int)n)) {
         // decode: one launch, the GEMV quantizes x in its prologue
         float *ys[1] = {dy};
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
@@ -505,7 +522,9 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
     const int64_t K = ws[0]->dev.K;
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i]->dev.M;
-    if (!same_type || count > gemv_max_multi() || n > 8 || n == 0 ||
+    bool skinny = false;
+    for (int i = 0; i < count; i++) skinny = skinny || wants_skinny(ws[i]->dev.type, K, ws[i]->dev.M, n);
+    if (!same_type || skinny || count > gemv_max_multi() || n > 8 || n == 0 ||
         !gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)) {
         for (int i = 0; i < count; i++) {
             int rc = mi_qmm_mulmat_path(ctx, ws[i], x, n, ys[i], location, MI_QMM_PATH_AUTO);
@@ -653,7 +672,9 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     // one launch pays when the tensors are too small to fill the machine one by one (q, k, v); large
     // ones (gate, up) run slightly faster back to back
     gemm_ok = gemm_ok && 2 * tiles < 3 * (int64_t)ctx->num_cus;
-    const bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
+    bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
+    for (int i = 0; gemv_ok && i < count; i++)  // from five or six columns up each weight goes to the skinny kernel
+        gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n);
     if (!gemm_ok && !gemv_ok) {
         for (int i = 0; i < count; i++) {
             int rc = mi_qmm_mulmat_q8(ctx, ws[i], act, ys[i], location, MI_QMM_PATH_AUTO);

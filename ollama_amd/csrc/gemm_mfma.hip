@@ -391,6 +391,298 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny product on the matrix cores: 3..16 activation columns (speculative / small-batch decode).
+// The streaming GEMV multiplies every column with its own pass of v_dot4 (about 450 vector
+// instructions per row and lane at eight columns) and is vector-ALU bound from three columns up.  Here
+// the columns ride along as rows of the MFMA's A operand; the weights are expanded to the same two
+// digit planes as in the GEMM and the fp32 epilogue runs on four accumulators per lane and super-block.
+//
+// HBM-bound like the GEMV, so the shape is the GEMV's: many small independent waves.  A workgroup owns
+// 16 weight rows, its four waves a quarter of K each (combined through LDS at the very end -- the only
+// barrier).  Every wave streams its own packed weights and activation operands through its own two LDS
+// stages with direct-to-LDS loads (coalesced: consecutive lanes fetch consecutive 16-byte pieces of a
+// row; loading 16-byte pieces of 16 different rows per instruction straight into registers touched 16
+// cache lines per instruction and ran at half the speed), waits on its own memory counter, and reads
+// its operands back with conflict-free LDS reads.
+// v_mfma_i32_16x16x64_i8: lane l holds weight row l%16 and the 16 K values 16*(l/16).. of a 64-wide
+// step as B operand, activation column l%16 (columns >= nc are zeroed) as A operand, and the outputs
+// (column 4*(l/16) + v, row l%16), v = 0..3.
+// ---------------------------------------------------------------------------------------------
+typedef int v4acc __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ v4acc mfma16(v4i a, v4i b, v4acc c) { return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0); }
+
+struct B16 {
+    v4i hi[4], lo[4];  // four 64-wide K steps, two digit planes
+    v4i min_lo, min_hi;
+    float d, dmin;
+};
+
+struct Sk16Q4K {
+    typedef GemmQ4K G;
+    static constexpr int W_BYTES = 3 * 1024;  // stage space: three copy instructions (16 rows x 144 B used)
+    static constexpr int W_INSTRS = 3;
+    static constexpr int D_LANES_PER_COL = 1;  // 16 digit bytes per activation column and super-block
+    // copy slot p (16 bytes) of the weight stage holds piece p%9 of row p/9
+    static __device__ __forceinline__ void w_plan(const DevWeight &w, int j, int lane, int rows_left, unsigned &off, bool &on) {
+        const int p = 64 * j + lane;
+        on = p < 16 * 9;
+        const int pp = on ? p : 0;
+        off = (unsigned)min(pp / 9, rows_left - 1) * (unsigned)(w.K / QKK * Q4_K_BYTES) + 16u * (pp % 9);
+    }
+    static __device__ __forceinline__ const uint8_t *w_base(const DevWeight &w, int, int64_t m0, int64_t sb) {
+        return w.p0 + m0 * (w.K / QKK * Q4_K_BYTES) + sb * Q4_K_BYTES;
+    }
+    // step t covers sub-blocks 2t (low nibbles of qs bytes [32t, 32t+32)) and 2t+1 (high nibbles); K group
+    // g of the step is elements 16(g&1).. of sub-block 2t + (g>>1): bytes [32t + 16(g&1), +16), nibble g>>1
+    struct Raw { uint4 hdr, q[4]; };
+    static __device__ __forceinline__ void read(const uint8_t *wt, int c, int g, Raw &raw) {
+        const uint8_t *p = wt + c * 144;
+        raw.hdr = ld16(p);
+#pragma unroll
+        for (int t = 0; t < 4; t++) raw.q[t] = ld16(p + 16 + 32 * t + 16 * (g & 1));
+    }
+    static __device__ __forceinline__ void expand(const Raw &raw, int g, unsigned, B16 &b) {
+        const uint4 hdr = raw.hdr;
+        b.d = h2f(hdr.x & 0xffff);
+        b.dmin = h2f(hdr.x >> 16);
+        const unsigned sc03 = hdr.y & 0x3f3f3f3fu, sc47 = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
+        const unsigned mn03 = hdr.z & 0x3f3f3f3fu, mn47 = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+        const int hiN = g >> 1;  // 0: low nibbles (sub-block 2t), 1: high nibbles (sub-block 2t+1)
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const unsigned word = t < 2 ? sc03 : sc47;  // scale of sub-block j = 2t + hiN: byte j & 3
+            const unsigned sc = (word >> (16 * (t & 1) + 8 * hiN)) & 0xff;
+            const unsigned sh = sc >> 3, sl = sc & 7;
+            const unsigned v[4] = {raw.q[t].x, raw.q[t].y, raw.q[t].z, raw.q[t].w};
+            v4i bh, bl;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const unsigned nib = (v[i] >> (4 * hiN)) & 0x0f0f0f0fu;
+                bh[i] = (int)(nib * sh);  // four byte products <= 105: no carries between bytes
+                bl[i] = (int)(nib * sl);
+            }
+            b.hi[t] = bh;
+            b.lo[t] = bl;
+        }
+        // block-sum MFMAs: the A rows carry [S_l(0..7) | S_h(0..7)] in K group 0 and zeros elsewhere
+        const int mz = g == 0 ? -1 : 0;
+        b.min_lo = (v4i){(int)mn03 & mz, (int)mn47 & mz, 0, 0};
+        b.min_hi = (v4i){0, 0, (int)mn03 & mz, (int)mn47 & mz};
+    }
+    static __device__ __forceinline__ bool sums_on(int g) { return g == 0; }
+};
+
+struct Sk16Q6K {
+    typedef GemmQ6K G;
+    static constexpr int W_BYTES = 4 * 1024;  // ql 2 KiB, qh 1 KiB, scales 256 B in the fourth KiB
+    static constexpr int W_INSTRS = 4;
+    static constexpr int D_LANES_PER_COL = 2;  // 32 digit bytes per activation column and super-block
+    // stage regions: ql [16 rows][8 pieces] at 0, qh [16][4] at 2 KiB, scales [16][1] at 3 KiB; piece
+    // positions XOR-ed with row bits so that the 16 rows of a read fall on distinct banks
+    static __device__ __forceinline__ void w_plan(const DevWeight &w, int j, int lane, int rows_left, unsigned &off, bool &on) {
+        on = true;
+        if (j < 2) {
+            const int q = 64 * j + lane, slot_row = q >> 3, pos = q & 7, piece = pos ^ ((slot_row >> 1) & 7);
+            off = (unsigned)min(slot_row, rows_left - 1) * (unsigned)(w.K / 2) + 16u * piece;
+        } else if (j == 2) {
+            const int slot_row = lane >> 2, pos = lane & 3, piece = pos ^ ((slot_row >> 2) & 3);
+            off = (unsigned)min(slot_row, rows_left - 1) * (unsigned)(w.K / 4) + 16u * piece;
+        } else {
+            on = lane < 16;
+            off = (unsigned)min(on ? lane : 0, rows_left - 1) * (unsigned)(w.K / 16);
+        }
+    }
+    static __device__ __forceinline__ const uint8_t *w_base(const DevWeight &w, int j, int64_t m0, int64_t sb) {
+        if (j < 2) return w.p0 + m0 * (w.K / 2) + sb * 128;
+        if (j == 2) return w.p1 + m0 * (w.K / 4) + sb * 64;
+        return w.p2 + m0 * (w.K / 16) + sb * 16;
+    }
+    // step t, K group g = scale group 4t + g (16 elements).  With H = t>>1, rr = 2(t&1) + (g>>1):
+    // ql bytes [64H + 32(g>>1) + 16(g&1), +16) = piece 4H + g, nibble t&1; qh bytes [32H + 16(g&1), +16) >> 2rr.
+    struct Raw { uint4 L[2], Hq[2], scv; };
+    static __device__ __forceinline__ void read(const uint8_t *wt, int c, int g, Raw &raw) {
+        const int xl = (c >> 1) & 7, xh = (c >> 2) & 3;
+#pragma unroll
+        for (int H = 0; H < 2; H++) {
+            raw.L[H] = ld16(wt + c * 128 + 16 * ((4 * H + g) ^ xl));
+            raw.Hq[H] = ld16(wt + 2048 + c * 64 + 16 * ((2 * H + (g & 1)) ^ xh));
+        }
+        raw.scv = ld16(wt + 3072 + c * 16);
+    }
+    static __device__ __forceinline__ void expand(const Raw &raw, int g, unsigned dh, B16 &b) {
+        const unsigned scw[4] = {raw.scv.x, raw.scv.y, raw.scv.z, raw.scv.w};
+        b.d = h2f(dh);
+        b.dmin = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int H = t >> 1;
+            const int rr2 = 2 * (2 * (t & 1) + (g >> 1));  // shift of the two high bits inside a qh byte
+            const unsigned l[4] = {raw.L[H].x, raw.L[H].y, raw.L[H].z, raw.L[H].w};
+            const unsigned hq[4] = {raw.Hq[H].x, raw.Hq[H].y, raw.Hq[H].z, raw.Hq[H].w};
+            const int sc = (int)(int8_t)(scw[t] >> (8 * g));  // scales[4t + g]
+            const s2 scv2 = {(short)sc, (short)sc};
+            v4i bh, bl;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const unsigned nib = (t & 1) ? (l[i] >> 4) & 0x0f0f0f0fu : l[i] & 0x0f0f0f0fu;
+                const unsigned e = nib | (((hq[i] >> rr2) & 0x03030303u) << 4);  // 0..63 per byte
+                const s2 pe = as_s2(e & 0x00ff00ffu) * scv2;         // elements 0 and 2, 16-bit products
+                const s2 po = as_s2((e >> 8) & 0x00ff00ffu) * scv2;  // elements 1 and 3
+                const unsigned le = as_u(pe) & 0x003f003fu, lo_ = as_u(po) & 0x003f003fu;
+                const unsigned he = as_u(pe >> 6), ho = as_u(po >> 6);  // arithmetic shift per 16-bit lane
+                bl[i] = (int)(le | (lo_ << 8));
+                bh[i] = (int)__builtin_amdgcn_perm(ho, he, 0x06020400u);  // bytes: he.b0, ho.b0, he.b2, ho.b2
+            }
+            b.hi[t] = bh;
+            b.lo[t] = bl;
+        }
+        // block-sum MFMAs: the A rows carry S_l(0..15) in K group 0 and S_h(0..15) in K group 1
+        const int z0 = g == 0 ? -1 : 0, z1 = g == 1 ? -1 : 0;
+        b.min_lo = (v4i){(int)scw[0] & z0, (int)scw[1] & z0, (int)scw[2] & z0, (int)scw[3] & z0};
+        b.min_hi = (v4i){(int)scw[0] & z1, (int)scw[1] & z1, (int)scw[2] & z1, (int)scw[3] & z1};
+    }
+    static __device__ __forceinline__ bool sums_on(int g) { return g < 2; }
+};
+
+constexpr int SKINNY_MAX_SB_PER_WAVE = 32;  // a wave keeps its rows' fp16 super-block scales in LDS
+
+// NCT = activation columns the stages are laid out for (8 or 16)
+template <class S, int NCT>
+struct SkinnyGeo {
+    static constexpr int A_BYTES = NCT * 256, A_INSTRS = NCT / 4;
+    static constexpr int D_BYTES = 16 * NCT * S::D_LANES_PER_COL, Y_BYTES = 64;
+    static constexpr int STAGE = S::W_BYTES + A_BYTES + D_BYTES + Y_BYTES;
+    static constexpr int NDMA = S::W_INSTRS + A_INSTRS + 2;  // copy instructions per stage
+    static constexpr int WAVE_BYTES = (2 * STAGE + 16 * SKINNY_MAX_SB_PER_WAVE * 2 + 1023) / 1024 * 1024;
+    static constexpr int PART_BYTES = 16 * 16 * 4;  // per wave: its partial sums
+};
+
+// The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
+template <class S, int NCT>
+__global__ __launch_bounds__(512, 3) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y) {
+    typedef typename S::G G;
+    typedef SkinnyGeo<S, NCT> Geo;
+    constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
+    constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, WAVE_BYTES = Geo::WAVE_BYTES;
+    const int WAVES = blockDim.x >> 6;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
+    float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * WAVE_BYTES);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int64_t m0 = (int64_t)blockIdx.x * 16;
+    const int rows_left = (int)min((int64_t)16, w.M - m0);  // rows past M: the last row again, results dropped
+    const int64_t nsb = w.K / QKK;
+    const int64_t sb0 = nsb * wave / WAVES, sb1 = nsb * (wave + 1) / WAVES;  // this wave's run of super-blocks
+    uint8_t *wsm = smem + wave * WAVE_BYTES;
+    uint16_t *dsm = reinterpret_cast<uint16_t *>(wsm + 2 * STAGE);  // [16 rows][sb1 - sb0] fp16 scales (Q6_K)
+
+    // ---- copy plan: per-lane 32-bit offsets, uniform bases per super-block
+    unsigned woff[S::W_INSTRS];
+    bool won[S::W_INSTRS];
+#pragma unroll
+    for (int j = 0; j < S::W_INSTRS; j++) S::w_plan(w, j, lane, rows_left, woff[j], won[j]);
+    unsigned aoff[A_INSTRS];
+#pragma unroll
+    for (int j = 0; j < A_INSTRS; j++) {
+        const int col = 4 * j + (lane >> 4), slot = lane & 15;  // stage slot [col][slot] holds piece slot ^ col
+        aoff[j] = (unsigned)(col0 + min(col, nc - 1)) * (unsigned)a.K + 16u * (slot ^ (col & 15));
+    }
+    const int dcol = lane / S::D_LANES_PER_COL;
+    const bool don = lane < NCT * S::D_LANES_PER_COL, yon = lane < NCT;
+    const unsigned doff = (unsigned)(col0 + min(dcol, nc - 1)) * (unsigned)(nsb * G::SD) + 16u * (lane % S::D_LANES_PER_COL);
+    const unsigned yoff = (unsigned)(col0 + min(lane, nc - 1)) * (unsigned)nsb * 4u;
+    const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
+    const uint8_t *asd = G::digits(a);
+
+    auto stage_copy = [&](uint8_t *st, int64_t sb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < S::W_INSTRS; j++) {
+            const uint8_t *gp = S::w_base(w, j, m0, sb) + woff[j];
+            if (won[j]) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * j), 16, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < A_INSTRS; j++) {
+            const uint8_t *gp = aq + sb * QKK + aoff[j];
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + S::W_BYTES + 1024 * j), 16, 0, 0);
+        }
+        {
+            const uint8_t *gp = asd + sb * G::SD + doff;
+            if (don) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + S::W_BYTES + A_BYTES), 16, 0, 0);
+        }
+        {
+            const uint8_t *gp = reinterpret_cast<const uint8_t *>(a.d) + sb * 4 + yoff;
+            if (yon) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + S::W_BYTES + A_BYTES + D_BYTES), 4, 0, 0);
+        }
+    };
+
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (sb0 < sb1) {
+        // the rows' fp16 super-block scales live outside the packed planes for Q6_K: fetch this wave's
+        // run of them once, before the steady state (their wait would otherwise drain the copies)
+        if (w.d) {
+            const int64_t row = m0 + min(c, rows_left - 1);
+            for (int64_t i = g; i < sb1 - sb0; i += 4) dsm[c * SKINNY_MAX_SB_PER_WAVE + i] = w.d[row * nsb + sb0 + i];
+        }
+        stage_copy(wsm, sb0);
+        stage_copy(wsm + STAGE, min(sb0 + 1, sb1 - 1));
+        const v4acc zero = {0, 0, 0, 0};
+        const v4i zero4 = {0, 0, 0, 0};
+        const bool acol = c < nc;  // the lane holds a real activation column in the A operand
+        const int cc = min(c, NCT - 1);  // lanes past the staged columns read a staged one and zero it
+#pragma unroll 1
+        for (int64_t sb = sb0; sb < sb1; sb++) {
+            uint8_t *st = wsm + ((sb - sb0) & 1) * STAGE;
+            // Every wave issues exactly NDMA copy instructions per stage, in order: once at most NDMA
+            // are outstanding, this stage has landed and the next one may still be in flight.
+            __builtin_amdgcn_s_waitcnt((NDMA & 15) | (7 << 4) | (15 << 8) | ((NDMA >> 4) << 14));
+            typename S::Raw raw;
+            S::read(st, c, g, raw);
+            v4i av[4], sv;
+#pragma unroll
+            for (int t = 0; t < 4; t++) av[t] = *reinterpret_cast<const v4i *>(st + S::W_BYTES + cc * 256 + 16 * ((4 * t + g) ^ cc));
+            sv = *reinterpret_cast<const v4i *>(st + S::W_BYTES + A_BYTES + (cc * S::D_LANES_PER_COL + (S::D_LANES_PER_COL == 2 ? (g & 1) : 0)) * 16);
+            const float4 yd = *reinterpret_cast<const float4 *>(st + S::W_BYTES + A_BYTES + D_BYTES + 16 * g);
+            const unsigned dh = dsm[c * SKINNY_MAX_SB_PER_WAVE + (sb - sb0)];
+            // operands are in registers: the stage can take the copies of super-block sb + 2
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            stage_copy(st, min(sb + 2, sb1 - 1));
+            if (!acol) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) av[t] = zero4;
+            }
+            if (!acol || !S::sums_on(g)) sv = zero4;
+            B16 b;
+            S::expand(raw, g, dh, b);
+            const v4acc xl = mfma16(sv, b.min_lo, zero);
+            const v4acc xh = mfma16(sv, b.min_hi, zero);
+            v4acc ah, al;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                ah = mfma16(av[t], b.hi[t], t == 0 ? zero : ah);
+                al = mfma16(av[t], b.lo[t], t == 0 ? zero : al);
+            }
+            const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float fm = G::fold_min(b.dmin, xh[v], xl[v]);
+                acc[v] = __builtin_fmaf(ydv[v], G::combine(b.d, ah[v], al[v], fm), acc[v]);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0);  // the redundant copies of the last iterations must not outlive the kernel's LDS
+    }
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[wave][4 * g + v][c] = acc[v];
+    __syncthreads();
+    for (int o = tid; o < 256; o += blockDim.x) {
+        const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
+        float sum = 0.f;
+        for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
+        if (i < nc && m0 + j < w.M) y[(int64_t)(col0 + i) * w.M + m0 + j] = sum;
+    }
+}
+
 // y[i] = sum over slices of part[slice][i]
 __global__ __launch_bounds__(256) void sum_slices_kernel(const float4 *__restrict__ part, float4 *__restrict__ y,
                                                          int64_t n4, int slices) {
@@ -461,6 +753,47 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
 }
 
 int gemm_max_multi() { return GEMM_MULTI; }
+
+bool skinny_supports(int type, int64_t K, int64_t M) {
+    return gemm_supports(type, K, M) && (K / QKK + 7) / 8 <= SKINNY_MAX_SB_PER_WAVE;
+}
+
+template <class S, int NCT>
+void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
+    typedef SkinnyGeo<S, NCT> Geo;
+    // Cut K as many ways as keeps the whole grid resident in one round (about 12 waves per CU fit):
+    // every wave pays one pipeline fill, so few long waves when there are many row groups, many short
+    // ones when there are few.
+    const int64_t groups = (w.M + 15) / 16, nsb = w.K / QKK;
+    int waves = (int)((int64_t)num_cus * 12 / groups);
+    waves = waves >= 8 ? 8 : waves >= 6 ? 6 : waves >= 4 ? 4 : waves >= 3 ? 3 : waves >= 2 ? 2 : 1;
+    while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;             // at least two super-blocks per wave
+    while ((nsb + waves - 1) / waves > SKINNY_MAX_SB_PER_WAVE && waves < 8) waves = waves >= 4 ? waves + 2 : waves + 1;
+    const size_t lds = (size_t)waves * (Geo::WAVE_BYTES + Geo::PART_BYTES);
+    // more than 64 KiB of dynamic LDS has to be allowed once per device
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_kernel<S, NCT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        allowed[dev] = true;
+    }
+    skinny_kernel<S, NCT><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y);
+}
+
+hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
+    if (!skinny_supports(w.type, w.K, w.M) || a.type != T_Q8_K || a.K != w.K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
+    if (ncols < 1 || ncols > 16 || col0 < 0 || col0 + ncols > a.N) return hipErrorInvalidValue;
+    if ((w.M + 15) / 16 > 0x7fffffff) return hipErrorInvalidValue;
+    if (w.type == T_Q4_K) {
+        if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8>(w, a, col0, ncols, y, num_cus, s);
+        else launch_skinny_as<Sk16Q4K, 16>(w, a, col0, ncols, y, num_cus, s);
+    } else {
+        if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8>(w, a, col0, ncols, y, num_cus, s);
+        else launch_skinny_as<Sk16Q6K, 16>(w, a, col0, ncols, y, num_cus, s);
+    }
+    return hipGetLastError();
+}
 
 hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, float *workspace,
                              size_t workspace_floats, int num_cus, hipStream_t s) {

@@ -47,5 +47,9 @@ size_t gemm_workspace_floats(int type, int64_t K, int64_t M, int64_t N, int num_
 hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, float *workspace,
                              size_t workspace_floats, int num_cus, hipStream_t s);
 int gemm_max_multi();
+// 1..16 activation columns (col0 .. col0+ncols-1 of a) on the matrix cores, K-quants; y[n*M + m]
+bool skinny_supports(int type, int64_t K, int64_t M);
+hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
+                         hipStream_t s);
 
 }  // namespace miqmm
