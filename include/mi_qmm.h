@@ -57,9 +57,11 @@ enum { MI_QMM_HOST = 0, MI_QMM_DEVICE = 1 };
 
 /* kernel selection for mi_qmm_mulmat_path */
 enum {
-    MI_QMM_PATH_AUTO = 0, /* GEMV for N <= 8, int8-MFMA GEMM for N >= 32, GEMV in column groups between */
-    MI_QMM_PATH_GEMV = 1, /* force the streaming GEMV (any N, processed 8 columns at a time)   */
-    MI_QMM_PATH_GEMM = 2  /* force the int8-MFMA GEMM (any N >= 1, padded to the tile)        */
+    MI_QMM_PATH_AUTO = 0, /* decode kernels below N = 32, tiled int8-MFMA GEMM from N = 32 (K-quants) */
+    MI_QMM_PATH_GEMV = 1, /* the decode kernels at any N: streaming GEMV, 8 columns at a time; K-quant
+                             weights go to the skinny matrix-core kernel from 5 (Q4_K) / 6 (Q6_K)
+                             columns, 16 at a time                                                   */
+    MI_QMM_PATH_GEMM = 2  /* force the tiled int8-MFMA GEMM (any N >= 1, padded to the tile)          */
 };
 
 /* ---- size tables: replace TensorType.BlockSize / TypeSize and Tensor.Size's row rule
