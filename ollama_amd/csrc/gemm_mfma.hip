@@ -420,7 +420,8 @@ struct B16 {
 
 struct Sk16Q4K {
     typedef GemmQ4K G;
-    static constexpr int W_BYTES = 3 * 1024;  // stage space: three copy instructions (16 rows x 144 B used)
+    static constexpr int W_BYTES = 16 * 144;  // 16 rows x 144 B: two full copy instructions and a quarter of a third
+    static constexpr bool SCALES_OUTSIDE = false;  // d and dmin sit in the block header
     static constexpr int W_INSTRS = 3;
     static constexpr int D_LANES_PER_COL = 1;  // 16 digit bytes per activation column and super-block
     // copy slot p (16 bytes) of the weight stage holds piece p%9 of row p/9
@@ -475,7 +476,8 @@ struct Sk16Q4K {
 
 struct Sk16Q6K {
     typedef GemmQ6K G;
-    static constexpr int W_BYTES = 4 * 1024;  // ql 2 KiB, qh 1 KiB, scales 256 B in the fourth KiB
+    static constexpr int W_BYTES = 3 * 1024 + 256;  // ql 2 KiB, qh 1 KiB, scales 256 B
+    static constexpr bool SCALES_OUTSIDE = true;  // the row's fp16 scale is a plane of its own
     static constexpr int W_INSTRS = 4;
     static constexpr int D_LANES_PER_COL = 2;  // 32 digit bytes per activation column and super-block
     // stage regions: ql [16 rows][8 pieces] at 0, qh [16][4] at 2 KiB, scales [16][1] at 3 KiB; piece
@@ -554,19 +556,20 @@ struct SkinnyGeo {
     static constexpr int D_BYTES = 16 * NCT * S::D_LANES_PER_COL, Y_BYTES = 64;
     static constexpr int STAGE = S::W_BYTES + A_BYTES + D_BYTES + Y_BYTES;
     static constexpr int NDMA = S::W_INSTRS + A_INSTRS + 2;  // copy instructions per stage
-    static constexpr int WAVE_BYTES = (2 * STAGE + 16 * SKINNY_MAX_SB_PER_WAVE * 2 + 1023) / 1024 * 1024;
+    static constexpr int DSM_BYTES = S::SCALES_OUTSIDE ? 16 * SKINNY_MAX_SB_PER_WAVE * 2 : 0;
+    static constexpr int WAVE_BYTES = (2 * STAGE + DSM_BYTES + 255) / 256 * 256;
     static constexpr int PART_BYTES = 16 * 16 * 4;  // per wave: its partial sums
 };
 
 // The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
 template <class S, int NCT>
-__global__ __launch_bounds__(512, 3) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y) {
+__global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y) {
     typedef typename S::G G;
     typedef SkinnyGeo<S, NCT> Geo;
     constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, WAVE_BYTES = Geo::WAVE_BYTES;
     const int WAVES = blockDim.x >> 6;
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
     float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * WAVE_BYTES);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -621,7 +624,7 @@ __global__ __launch_bounds__(512, 3) void skinny_kernel(DevWeight w, DevAct a, i
     if (sb0 < sb1) {
         // the rows' fp16 super-block scales live outside the packed planes for Q6_K: fetch this wave's
         // run of them once, before the steady state (their wait would otherwise drain the copies)
-        if (w.d) {
+        if (S::SCALES_OUTSIDE) {
             const int64_t row = m0 + min(c, rows_left - 1);
             for (int64_t i = g; i < sb1 - sb0; i += 4) dsm[c * SKINNY_MAX_SB_PER_WAVE + i] = w.d[row * nsb + sb0 + i];
         }
@@ -644,7 +647,7 @@ __global__ __launch_bounds__(512, 3) void skinny_kernel(DevWeight w, DevAct a, i
             for (int t = 0; t < 4; t++) av[t] = *reinterpret_cast<const v4i *>(st + S::W_BYTES + cc * 256 + 16 * ((4 * t + g) ^ cc));
             sv = *reinterpret_cast<const v4i *>(st + S::W_BYTES + A_BYTES + (cc * S::D_LANES_PER_COL + (S::D_LANES_PER_COL == 2 ? (g & 1) : 0)) * 16);
             const float4 yd = *reinterpret_cast<const float4 *>(st + S::W_BYTES + A_BYTES + D_BYTES + 16 * g);
-            const unsigned dh = dsm[c * SKINNY_MAX_SB_PER_WAVE + (sb - sb0)];
+            const unsigned dh = S::SCALES_OUTSIDE ? dsm[c * SKINNY_MAX_SB_PER_WAVE + (sb - sb0)] : 0u;
             // operands are in registers: the stage can take the copies of super-block sb + 2
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             stage_copy(st, min(sb + 2, sb1 - 1));
@@ -761,11 +764,11 @@ bool skinny_supports(int type, int64_t K, int64_t M) {
 template <class S, int NCT>
 void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
     typedef SkinnyGeo<S, NCT> Geo;
-    // Cut K as many ways as keeps the whole grid resident in one round (about 12 waves per CU fit):
+    // Cut K as many ways as keeps the whole grid resident in one round (about 15 waves per CU fit):
     // every wave pays one pipeline fill, so few long waves when there are many row groups, many short
     // ones when there are few.
     const int64_t groups = (w.M + 15) / 16, nsb = w.K / QKK;
-    int waves = (int)((int64_t)num_cus * 12 / groups);
+    int waves = (int)((int64_t)num_cus * 15 / groups);
     waves = waves >= 8 ? 8 : waves >= 6 ? 6 : waves >= 4 ? 4 : waves >= 3 ? 3 : waves >= 2 ? 2 : 1;
     while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;             // at least two super-blocks per wave
     while ((nsb + waves - 1) / waves > SKINNY_MAX_SB_PER_WAVE && waves < 8) waves = waves >= 4 ? waves + 2 : waves + 1;
