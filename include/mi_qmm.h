@@ -123,6 +123,19 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
 int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x,
                         int64_t n, float *const *ys, int location);
 
+/* Expert-indexed product, Tensor.MulmatID (/root/reference/ml/backend.go:153).  w is a stack of
+ * n_expert matrices uploaded as ONE weight of m = rows_per_expert * n_expert rows: GGUF stores expert
+ * tensors with ne = [in, out, experts] (/root/reference/convert/convert_gemma4.go:274-275), so the
+ * bytes of the 3-D tensor are that 2-D weight unchanged.  x is f32 [n_tokens][b_cols][k], ids is
+ * int32 [n_tokens][n_used], y receives f32 [n_tokens][n_used][rows_per_expert]:
+ *     y[t][i][:] = W[ids[t][i]] * Q8(x[t][i % b_cols][:])
+ * (b_cols = 1: all slots of a token share one activation row, as for gate/up; b_cols = n_used: every
+ * slot has its own, as for the down projection.)  location covers x, ids and y alike.  With ids in
+ * host memory an id outside 0..n_expert-1 is MI_QMM_ERR_INVALID (ggml aborts there); with ids in
+ * device memory the call cannot see them and the rows of such a pair come back as NaN. */
+int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
+                     const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location);
+
 /* ---- two-phase form: quantize once, multiply by several weights (gate and up, or q/k/v, share
  *      one x).  In ggml's graph the from_float step belongs to each mul_mat node; a backend that
  *      sees the whole graph at Context.Compute (/root/reference/ml/backend.go:110) may hoist it,
@@ -177,8 +190,9 @@ int mi_qmm_gguf_kv_float(const mi_qmm_gguf *f, int64_t index, int64_t elem, doub
 int mi_qmm_gguf_kv_bool(const mi_qmm_gguf *f, int64_t index, int64_t elem, int *out);
 /* string bytes are not NUL-terminated: *str points into the mapping, *len is the length */
 int mi_qmm_gguf_kv_string(const mi_qmm_gguf *f, int64_t index, int64_t elem, const char **str, int64_t *len);
-/* upload tensor `index` (2-D, a type this library multiplies: 2, 8, 12, 14) as a resident weight:
- * K = dims[0], M = dims[1]; the bytes go from the mapping to the device */
+/* upload tensor `index` (a type this library multiplies: 2, 8, 12, 14) as a resident weight; the bytes
+ * go from the mapping to the device.  2-D: K = dims[0], M = dims[1].  3-D (an expert stack for
+ * mi_qmm_mulmat_id): K = dims[0], M = dims[1] * dims[2], n_expert = dims[2]. */
 int mi_qmm_gguf_upload(mi_qmm_ctx *ctx, const mi_qmm_gguf *f, int64_t index, mi_qmm_weight **out);
 
 /* ---- diagnostics */

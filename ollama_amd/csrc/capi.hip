@@ -564,6 +564,64 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
     return MI_QMM_OK;
 }
 
+int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
+                     const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location) {
+    int rc = check_product_args(ctx, w, location, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
+        return fail(MI_QMM_ERR_INVALID, "n_expert=%d n_used=%d b_cols=%d n_tokens=%lld: all must be positive", n_expert,
+                    n_used, b_cols, (long long)n_tokens);
+    const int64_t K = w->dev.K;
+    if (w->dev.M % n_expert)
+        return fail(MI_QMM_ERR_INVALID, "the weight has %lld rows, not a multiple of n_expert=%d", (long long)w->dev.M,
+                    n_expert);
+    const int64_t M = w->dev.M / n_expert;
+    if (n_tokens == 0) return MI_QMM_OK;
+    if (!x || !ids || !y) return fail(MI_QMM_ERR_INVALID, "x, ids or y is NULL");
+    const int64_t pairs = (int64_t)n_used * n_tokens, ncols = (int64_t)b_cols * n_tokens;
+    if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24) || K > gemv_max_k(w->dev.type))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts, 2^24 pairs and k <= %lld for type %d",
+                    (long long)gemv_max_k(w->dev.type), w->dev.type);
+    if (location == MI_QMM_HOST)
+        for (int64_t p = 0; p < pairs; p++)
+            if (ids[p] < 0 || ids[p] >= n_expert)
+                return fail(MI_QMM_ERR_INVALID, "ids[%lld] = %d is outside 0..%d", (long long)p, ids[p], n_expert - 1);
+
+    const int q8 = mi_qmm_vec_dot_type(w->dev.type);
+    const ActPlanes probe = plan_act(nullptr, q8, K, ncols);
+    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+    const ActPlanes p = plan_act(ctx->act_buf, q8, K, ncols);
+    if ((rc = reserve(&ctx->ws_buf, &ctx->ws_cap, gemv_id_scratch_ints(pairs) * sizeof(int), ctx->stream))) return rc;
+
+    const size_t xbytes = (size_t)(ncols * K) * 4, ibytes = (size_t)pairs * 4, ybytes = (size_t)(pairs * M) * 4;
+    const float *dx = x;
+    const int32_t *dids = ids;
+    float *dy = y;
+    if (location == MI_QMM_HOST) {
+        const size_t ioff = align_up(xbytes, 256), yoff = ioff + align_up(ibytes, 256);
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, yoff + ybytes, ctx->stream))) return rc;
+        dx = (const float *)ctx->io_buf;
+        dids = (const int32_t *)((char *)ctx->io_buf + ioff);
+        dy = (float *)((char *)ctx->io_buf + yoff);
+        HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(hipMemcpyAsync((void *)dids, ids, ibytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    DevAct a{};
+    a.K = K; a.N = (int)ncols; a.type = q8;
+    const bool fused = gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert);
+    if (!fused) {
+        HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, nullptr, nullptr, ctx->stream));
+        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums;
+    }
+    HIP_TRY(launch_gemv_id(w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
+                           (int *)ctx->ws_buf, ctx->stream));
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
 // ---- two-phase form ----------------------------------------------------------------------------------
 int mi_qmm_act_create(mi_qmm_ctx *ctx, int q8_type, int64_t k, int64_t n_max, mi_qmm_act **out) {
     if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
@@ -865,11 +923,13 @@ int mi_qmm_gguf_upload(mi_qmm_ctx *ctx, const mi_qmm_gguf *f, int64_t index, mi_
     if (index < 0 || index >= (int64_t)f->file.tensors.size())
         return fail(MI_QMM_ERR_INVALID, "tensor index %lld outside 0..%zu", (long long)index, f->file.tensors.size());
     const GgufTensor &t = f->file.tensors[index];
-    if (t.n_dims != 2)
-        return fail(MI_QMM_ERR_UNSUPPORTED, "tensor \"%s\" has %u dimensions: only 2-D weights take part in Mulmat",
+    if (t.n_dims != 2 && t.n_dims != 3)
+        return fail(MI_QMM_ERR_UNSUPPORTED,
+                    "tensor \"%s\" has %u dimensions: Mulmat takes 2-D weights, MulmatID 3-D expert stacks",
                     t.name.c_str(), t.n_dims);
-    return mi_qmm_weight_upload(ctx, (int)t.type, f->file.tensor_data(t), (int64_t)t.dims[0], (int64_t)t.dims[1],
-                                MI_QMM_HOST, out);
+    // an expert stack [K, M, E] is E matrices of M rows one after the other: the same bytes as [K, M*E]
+    const int64_t m = (int64_t)t.dims[1] * (t.n_dims == 3 ? (int64_t)t.dims[2] : 1);
+    return mi_qmm_weight_upload(ctx, (int)t.type, f->file.tensor_data(t), (int64_t)t.dims[0], m, MI_QMM_HOST, out);
 }
 
 }  // extern "C"

@@ -510,6 +510,60 @@ __device__ __forceinline__ float wave_total(float w) {
     return w;
 }
 
+// Sums over runs of 64/RPL lanes (RPL = 1, 2, 4 rows side by side in a wave); a run's total is
+// taken from its last lane.  RPL = 1 is wave_total.
+template <int RPL>
+__device__ __forceinline__ float run_total(float w) {
+    w += dpp_mov<0xB1>(w);
+    w += dpp_mov<0x4E>(w);
+    w += dpp_mov<0x124>(w);
+    w += dpp_mov<0x128>(w);
+    if (RPL <= 2) w += dpp_row<0x142, 0xa>(w);
+    if (RPL == 1) w += dpp_row<0x143, 0xc>(w);
+    return w;
+}
+
+// How many rows a wave takes side by side: a row shorter than half (a quarter) of a wave's K segment
+// leaves half (three quarters) of the lanes without work, so the lanes are split into 2 (4) runs that
+// each hold a row of their own.  Only for rows inside one segment.
+template <class P>
+constexpr int rows_per_load(int64_t K) { return K * 4 <= P::SEG ? 4 : K * 2 <= P::SEG ? 2 : 1; }
+
+// The row loop of the thin kernels: rows wrow0 .. wrow0+nrw-1 of w against the activation registers,
+// one load of RPL rows in registers and the next in flight.  cur holds the first load (issued by the
+// caller ahead of its prologue: rows wrow0 + min(run, nrw-1)).  DIRECT: on return lane 63-i of keep[n]
+// holds the total of the wave's row i; otherwise the totals go to part[(rl0+i)*NC + n][kseg].
+template <class P, int NC, bool DIRECT, int RPL>
+__device__ __forceinline__ void thin_rows(const DevWeight &w, const typename P::Geo &g, typename P::Raw cur,
+                                          const typename P::Act (&act)[NC], int64_t wrow0, int nrw, int lane,
+                                          float (&keep)[NC], float *part, int rl0, int kw, int kseg) {
+    static_assert(RPL == 1 || DIRECT, "rows side by side only when a row lies inside one K segment");
+    const int run = RPL == 1 ? 0 : lane / (64 / RPL);
+#pragma unroll
+    for (int n = 0; n < NC; n++) keep[n] = 0.f;
+#pragma unroll 1
+    for (int i = 0; i < nrw; i += RPL) {
+        float acc[NC];
+#pragma unroll
+        for (int n = 0; n < NC; n++) acc[n] = 0.f;
+        P::template dot<NC>(cur, g, act, acc);
+        if (i + RPL < nrw) cur = P::load(w, g, wrow0 + min(i + RPL + run, nrw - 1));  // wave-uniform branch
+#pragma unroll
+        for (int n = 0; n < NC; n++) {
+            // Every lane of a run's last quad row holds the total, but each quad added the quads of its
+            // row in its own order: take the run's last lane, so a row's result does not depend on which
+            // lane parks it (i.e. not on how many rows a wave was given).
+            const int tot_all = __float_as_int(run_total<RPL>(acc[n]));
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                const float tot = __int_as_float(__builtin_amdgcn_readlane(tot_all, 64 / RPL * (r + 1) - 1));
+                if (DIRECT) keep[n] = lane == 63 - (i + r) ? tot : keep[n];
+                else if (lane == 63) part[((rl0 + i) * NC + n) * kw + kseg] = tot;
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // The thin-wave kernel: many small waves instead of a few unrolled ones.
 //
@@ -528,6 +582,57 @@ struct LdsAct {
     int64_t K;
 };
 
+// The f32 prologue shared by the kernels that quantize their own activations: a wave takes 256
+// consecutive elements ("pieces" of 64 float4) at a time, the same lane-to-element mapping as the
+// stand-alone quantization kernel, so the values are the same bits.  The first XPRE pieces of a wave
+// are requested by prefetch_x (before the wave's first weight load), the rest inside quantize_x_to_lds.
+constexpr int XPRE = 4;
+
+__device__ __forceinline__ void prefetch_x(const float4 *__restrict__ x4, int total4, int wave, int nwaves, int lane,
+                                           float4 (&xpre)[XPRE]) {
+#pragma unroll
+    for (int j = 0; j < XPRE; j++) {
+        const int i4 = (wave + j * nwaves) * 64 + lane;
+        xpre[j] = x4[min(i4, total4 - 1)];  // clamped: the loads stay unconditional
+    }
+}
+
+template <class P>
+__device__ __forceinline__ void quantize_x_to_lds(const float4 *__restrict__ x4, int total4, int wave, int nwaves,
+                                                  int lane, const float4 (&xpre)[XPRE], int8_t *lqs, float *ld_,
+                                                  int16_t *lbs) {
+    auto quantize_piece = [&](int c, float4 v) {
+        const int i4 = c * 64 + lane;
+        const bool live = i4 < total4;  // Q8_0 only: the element count need not be a multiple of 256
+        if (!live) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        float dd;
+        if (P::ACT_BLK == QKK) {
+            int sum16, pair;
+            const int packed = q8_K_quantize_lane(v, lane, dd, sum16, pair);
+            reinterpret_cast<int *>(lqs)[i4] = packed;
+            if (lane == 0) ld_[c] = dd;
+            if (P::USES_BSUMS && (lane & 3) == 0) lbs[c * 16 + (lane >> 2)] = (int16_t)sum16;
+        } else {
+            int sum;
+            const int packed = q8_0_quantize_lane(v, dd, sum);
+            if (live) {
+                reinterpret_cast<int *>(lqs)[i4] = packed;
+                if ((lane & 7) == 0) {
+                    ld_[i4 >> 3] = dd;
+                    if (P::USES_BSUMS) lbs[i4 >> 3] = (int16_t)sum;
+                }
+            }
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < XPRE; j++) {
+        const int c = wave + j * nwaves;
+        if (c * 64 < total4) quantize_piece(c, xpre[j]);  // wave-uniform
+    }
+    for (int c = wave + XPRE * nwaves; c * 64 < total4; c += nwaves)
+        quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
+}
+
 // Kernel arguments of the thin kernel, arranged so that the tensor a workgroup belongs to is picked
 // with compares and selects on values that are all fetched by one batch of scalar loads: a select
 // chain that indexes the argument block with a computed index makes each pointer load wait for the
@@ -545,7 +650,7 @@ struct ThinArgs {
 // workgroup size limit: 16 waves leave a wave 128 VGPRs, enough for up to three activation columns
 constexpr int thin_max_waves(int nc, bool f32) { return f32 ? (nc <= 3 ? 16 : 8) : 4; }
 
-template <class P, int NC, bool DIRECT, bool F32>
+template <class P, int NC, bool DIRECT, bool F32, int RPL>
 __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(ThinArgs ta, DevAct a, const float *__restrict__ xf,
                                                          int col0, int rows_per_wave, int kw, int rw_log2) {
     // LDS: the NC activation columns (quants, block scales, block sums), then, unless DIRECT, the
@@ -570,7 +675,8 @@ __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(
     const int nrw = max(0, min(rows_per_wave, nrows - rl0));
     float *yrow0 = y + (int64_t)col0 * ldy + r0;
 
-    const typename P::Geo g = P::geo(w, kseg, lane);
+    const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);  // position inside the lane's run
+    const typename P::Geo g = P::geo(w, kseg, vlane);
 
     // With f32 activations the workgroup quantizes them itself, into LDS, in the layout of DevAct
     // (columns col0 .. col0+NC-1 only): a wave takes 256 consecutive elements at a time, the same
@@ -585,51 +691,15 @@ __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(
     // Order of the memory requests: the wave's pieces of x (L2 hits, they come back first), then its
     // first row of weights (HBM).  The memory counter retires in order, so the quantization can start
     // as soon as x is there while the weights are still in flight.
-    constexpr int XPRE = 4;  // pieces of x a wave requests ahead of its weights
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col0 * K);
     const int total4 = (int)((int64_t)NC * K / 4);  // float4 pieces over all NC columns
     const int nwaves = blockDim.x >> 6;
     float4 xpre[XPRE];
-    if (F32) {
-#pragma unroll
-        for (int j = 0; j < XPRE; j++) {
-            const int i4 = (wave + j * nwaves) * 64 + lane;
-            xpre[j] = x4[min(i4, total4 - 1)];  // clamped: the loads stay unconditional
-        }
-    }
+    if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     typename P::Raw cur;
-    if (nrw > 0) cur = P::load(w, g, r0 + rl0);
+    if (nrw > 0) cur = P::load(w, g, r0 + rl0 + min(run, nrw - 1));
     if (F32) {
-        auto quantize_piece = [&](int c, float4 v) {
-            const int i4 = c * 64 + lane;
-            const bool live = i4 < total4;  // Q8_0 only: K*NC need not be a multiple of 256
-            if (!live) v = make_float4(0.f, 0.f, 0.f, 0.f);
-            float dd;
-            if (P::ACT_BLK == QKK) {
-                int sum16, pair;
-                const int packed = q8_K_quantize_lane(v, lane, dd, sum16, pair);
-                reinterpret_cast<int *>(lqs)[i4] = packed;
-                if (lane == 0) ld_[c] = dd;
-                if (P::USES_BSUMS && (lane & 3) == 0) lbs[c * 16 + (lane >> 2)] = (int16_t)sum16;
-            } else {
-                int sum;
-                const int packed = q8_0_quantize_lane(v, dd, sum);
-                if (live) {
-                    reinterpret_cast<int *>(lqs)[i4] = packed;
-                    if ((lane & 7) == 0) {
-                        ld_[i4 >> 3] = dd;
-                        if (P::USES_BSUMS) lbs[i4 >> 3] = (int16_t)sum;
-                    }
-                }
-            }
-        };
-#pragma unroll
-        for (int j = 0; j < XPRE; j++) {
-            const int c = wave + j * nwaves;
-            if (c * 64 < total4) quantize_piece(c, xpre[j]);  // wave-uniform
-        }
-        for (int c = wave + XPRE * nwaves; c * 64 < total4; c += nwaves)
-            quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
+        quantize_x_to_lds<P>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
         __syncthreads();
     }
     float *part = reinterpret_cast<float *>(smem + act_bytes);
@@ -639,31 +709,13 @@ __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(
         if (F32) {
             const LdsAct la{lqs, ld_, lbs, K};
 #pragma unroll
-            for (int n = 0; n < NC; n++) P::load_act(la, n, kseg, lane, g, act[n]);
+            for (int n = 0; n < NC; n++) P::load_act(la, n, kseg, vlane, g, act[n]);
         } else {
 #pragma unroll
-            for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg, lane, g, act[n]);
+            for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg, vlane, g, act[n]);
         }
         float keep[NC];  // lane 63-i ends up holding the total of the wave's row i
-#pragma unroll
-        for (int n = 0; n < NC; n++) keep[n] = 0.f;
-#pragma unroll 1
-        for (int i = 0; i < nrw; i++) {
-            float acc[NC];
-#pragma unroll
-            for (int n = 0; n < NC; n++) acc[n] = 0.f;
-            P::template dot<NC>(cur, g, act, acc);
-            if (i + 1 < nrw) cur = P::load(w, g, r0 + rl0 + i + 1);  // wave-uniform branch
-#pragma unroll
-            for (int n = 0; n < NC; n++) {
-                // Lanes 48..63 all hold the total, but each quad added the four quads of its row in its own
-                // order: take lane 63's value, so a row's result does not depend on which lane parks it
-                // (i.e. not on how many rows a wave was given).
-                const float tot = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_total(acc[n])), 63));
-                if (DIRECT) keep[n] = lane == 63 - i ? tot : keep[n];
-                else if (lane == 63) part[((rl0 + i) * NC + n) * kw + kseg] = tot;
-            }
-        }
+        thin_rows<P, NC, DIRECT, RPL>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
         if (DIRECT && lane > 63 - nrw) {
 #pragma unroll
             for (int n = 0; n < NC; n++) yrow0[(int64_t)n * ldy + rl0 + (63 - lane)] = keep[n];
@@ -680,7 +732,7 @@ __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(
     }
 }
 
-struct Plan { int kw, rw, rw_log2, spw, rows_per_wg; unsigned grid; size_t lds; };
+struct Plan { int kw, rw, rw_log2, spw, rows_per_wg, rpl; unsigned grid; size_t lds; };
 
 // 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), one or two workgroups per CU.
 // total_m is the number of rows over all tensors of the launch.
@@ -737,6 +789,9 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p) {
             rows_per_wave = (nc >= 4 || total_m > 65536) ? 4 : 2;
         }
     }
+    // short rows: 2 or 4 side by side per load, and at least two loads per wave (one in flight)
+    p.rpl = p.kw == 1 ? rows_per_load<P>(K) : 1;
+    if (p.rpl > 1) rows_per_wave = max(2 * p.rpl, (rows_per_wave + p.rpl - 1) / p.rpl * p.rpl);
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
     p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float));
@@ -747,17 +802,20 @@ template <class P, int NC>
 void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, const float *xf, int col0, hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
     const int rpw = p.rows_per_wg >> p.rw_log2;
+#define THIN_LAUNCH(DIRECT, F32, RPL) \
+    gemv_thin_kernel<P, NC, DIRECT, F32, RPL><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2)
     if (xf) {
-        if (p.kw == 1)
-            gemv_thin_kernel<P, NC, true, true><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
-        else
-            gemv_thin_kernel<P, NC, false, true><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
+        if (p.kw > 1) THIN_LAUNCH(false, true, 1);
+        else if (p.rpl == 4) THIN_LAUNCH(true, true, 4);
+        else if (p.rpl == 2) THIN_LAUNCH(true, true, 2);
+        else THIN_LAUNCH(true, true, 1);
     } else {
-        if (p.kw == 1)
-            gemv_thin_kernel<P, NC, true, false><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
-        else
-            gemv_thin_kernel<P, NC, false, false><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2);
+        if (p.kw > 1) THIN_LAUNCH(false, false, 1);
+        else if (p.rpl == 4) THIN_LAUNCH(true, false, 4);
+        else if (p.rpl == 2) THIN_LAUNCH(true, false, 2);
+        else THIN_LAUNCH(true, false, 1);
     }
+#undef THIN_LAUNCH
 }
 
 template <class P, int NC, int SPW, int U>
@@ -893,6 +951,265 @@ hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int coun
     a.N = ncols;
     a.type = (ws[0].type == T_Q4_K || ws[0].type == T_Q6_K) ? T_Q8_K : T_Q8_0;
     return dispatch(ws, ys, count, a, x, 0, ncols, num_cus, s);
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Expert-indexed product (Tensor.MulmatID, /root/reference/ml/backend.go:153): the weight is a stack
+// of n_expert matrices [K, M] (GGUF ne = [in, out, experts], /root/reference/convert/convert_gemma4.go:274-275),
+// ids[t][i] names the expert that slot i of token t goes through, and
+//   y[t][i][:] = W[ids[t][i]] . Q8(b[t][i mod b_cols][:])
+// The (token, slot) pairs are independent GEMVs that happen to share weights when two pairs name
+// the same expert.  A "group" is up to NC pairs of one expert; a workgroup belongs to one group and
+// runs the thin kernel's loop over a few rows of that expert with the group's pairs as its
+// activation columns.  Decode (a handful of pairs, experts all different) takes one pair per group
+// straight from ids; larger batches are bucketed by expert first (group_pairs_kernel).
+// A pair's result does not depend on what else is in its group: every column has its own
+// accumulators and the same reduction order.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int ID_MAX_EXPERTS = 4096;
+
+struct IdArgs {
+    DevWeight w;           // the stack: rows e*M .. e*M+M-1 are expert e (w.M = M * n_expert)
+    const int *ids;        // [pairs], pair = token * n_used + slot
+    const int *groups;     // grouped launches: n_groups, then per group {expert, count, pair[NC]}; else null
+    float *y;              // [pairs][M]
+    int64_t M;             // rows per expert
+    int n_expert, pairs, n_used, b_cols, wgs_per_group;
+};
+
+// One workgroup of 1024 threads buckets the pairs by expert: counts in LDS, group ranges from a
+// running sum over the experts, then every pair takes the next free place of its expert.  Pairs with
+// an id outside 0..n_expert-1 go to a bucket of their own whose groups carry expert = -1.
+template <int NC>
+__global__ __launch_bounds__(1024) void group_pairs_kernel(const int *__restrict__ ids, int pairs, int n_expert,
+                                                            int *__restrict__ groups) {
+    __shared__ int count[ID_MAX_EXPERTS + 1], start[ID_MAX_EXPERTS + 1];
+    constexpr int REC = 2 + NC;
+    const int nb = n_expert + 1;
+    for (int e = threadIdx.x; e < nb; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = ids[p];
+        atomicAdd(&count[(e < 0 || e >= n_expert) ? n_expert : e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int g = 0;
+        for (int e = 0; e < nb; e++) {
+            start[e] = g;
+            g += (count[e] + NC - 1) / NC;
+        }
+        groups[0] = g;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nb; e += blockDim.x) {
+        const int c = count[e];
+        for (int g = 0; g * NC < c; g++) {
+            int *rec = groups + 1 + (size_t)(start[e] + g) * REC;
+            rec[0] = e < n_expert ? e : -1;
+            rec[1] = min(NC, c - g * NC);
+        }
+        count[e] = 0;  // reused as the fill cursor
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e0 = ids[p];
+        const int e = (e0 < 0 || e0 >= n_expert) ? n_expert : e0;
+        const int pos = atomicAdd(&count[e], 1);
+        groups[1 + (size_t)(start[e] + pos / NC) * REC + 2 + pos % NC] = p;
+    }
+}
+
+// F32 (one pair per group only): xf is b itself, [tokens][b_cols][K] floats, and the workgroup quantizes
+// its pair's activation row into LDS first, like the thin kernel does -- decode is one launch.
+template <class P, int NC, bool DIRECT, bool F32, int RPL>
+__global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const float *__restrict__ xf,
+                                                      int rows_per_wave, int kw, int rw_log2) {
+    static_assert(!F32 || NC == 1, "the f32 prologue quantizes one activation row");
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int REC = 2 + NC;
+    const int group = blockIdx.x / ia.wgs_per_group, wg = blockIdx.x - group * ia.wgs_per_group;
+    int expert, count, pair[NC];
+    if (ia.groups) {
+        if (group >= ia.groups[0]) return;
+        const int *rec = ia.groups + 1 + (size_t)group * REC;
+        expert = rec[0];
+        count = rec[1];
+#pragma unroll
+        for (int n = 0; n < NC; n++) pair[n] = rec[2 + min(n, count - 1)];
+    } else {
+        expert = ia.ids[group];
+        if (expert < 0 || expert >= ia.n_expert) expert = -1;
+        count = 1;
+#pragma unroll
+        for (int n = 0; n < NC; n++) pair[n] = group;
+    }
+    const int64_t M = ia.M;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = 1 << rw_log2;
+    const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
+    const int rows_per_wg = rows_per_wave << rw_log2;
+    const int64_t r0 = (int64_t)wg * rows_per_wg;  // row inside the expert
+    const int nrows = (int)min((int64_t)rows_per_wg, M - r0);
+    if (expert < 0) {
+        // an id outside the stack: the pair's output is all NaN
+        for (int i = threadIdx.x; i < nrows * count; i += blockDim.x) {
+            const int n = i / nrows, rl = i - n * nrows;
+            ia.y[(int64_t)pair[n] * M + r0 + rl] = __int_as_float(0x7fc00000);
+        }
+        return;
+    }
+    const int rl0 = rg * rows_per_wave;
+    const int nrw = max(0, min(rows_per_wave, nrows - rl0));
+    const int64_t wrow0 = (int64_t)expert * M + r0 + rl0;  // row inside the stack
+
+    const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);
+    const typename P::Geo g = P::geo(ia.w, kseg, vlane);
+    int col[NC];  // activation row of each pair: token * b_cols + slot mod b_cols
+#pragma unroll
+    for (int n = 0; n < NC; n++) {
+        const int tok = pair[n] / ia.n_used, slot = pair[n] - tok * ia.n_used;
+        col[n] = tok * ia.b_cols + slot % ia.b_cols;
+    }
+    const int64_t K = ia.w.K;
+    const int nblk = (int)(K / P::ACT_BLK);
+    const size_t act_bytes = F32 ? ((size_t)(K + nblk * 4 + (P::USES_BSUMS ? K / P::ACT_BSUM * 2 : 0)) + 15) / 16 * 16 : 0;
+    int8_t *lqs = reinterpret_cast<int8_t *>(smem);
+    float *ld_ = reinterpret_cast<float *>(smem + K);
+    int16_t *lbs = reinterpret_cast<int16_t *>(smem + K + (size_t)nblk * 4);
+    const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col[0] * K);
+    const int total4 = (int)(K / 4), nwaves = blockDim.x >> 6;
+    float4 xpre[XPRE];
+    if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
+    typename P::Raw cur;
+    if (nrw > 0) cur = P::load(ia.w, g, wrow0 + min(run, nrw - 1));
+    if (F32) {
+        quantize_x_to_lds<P>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
+        __syncthreads();
+    }
+    float *part = reinterpret_cast<float *>(smem + act_bytes);
+    if (nrw > 0) {
+        typename P::Act act[NC];
+        if (F32) {
+            const LdsAct la{lqs, ld_, lbs, K};
+            P::load_act(la, 0, kseg, vlane, g, act[0]);
+        } else {
+#pragma unroll
+            for (int n = 0; n < NC; n++) P::load_act(a, col[n], kseg, vlane, g, act[n]);
+        }
+        float keep[NC];
+        thin_rows<P, NC, DIRECT, RPL>(ia.w, g, cur, act, wrow0, nrw, lane, keep, part, rl0, kw, kseg);
+        if (DIRECT && lane > 63 - nrw) {
+#pragma unroll
+            for (int n = 0; n < NC; n++)
+                if (n < count) ia.y[(int64_t)pair[n] * M + r0 + rl0 + (63 - lane)] = keep[n];
+        }
+    }
+    if (DIRECT) return;
+    __syncthreads();
+    for (int i = threadIdx.x; i < nrows * count; i += blockDim.x) {
+        const int n = i / nrows, rl = i - n * nrows;
+        float sum = 0.f;
+        for (int k = 0; k < kw; k++) sum += part[(rl * NC + n) * kw + k];
+        ia.y[(int64_t)pair[n] * M + r0 + rl] = sum;
+    }
+}
+
+template <class P, int NC>
+hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, int *groups, hipStream_t s) {
+    Plan p;
+    if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M, NC, false, p)) return hipErrorInvalidValue;
+    const size_t act_lds = xf ? thin_act_lds<P>(ia.w.K, 1) : 0;
+    if (xf && (NC != 1 || act_lds + p.lds > THIN_LDS_MAX)) return hipErrorInvalidValue;
+    const int64_t wgs_per_group = (ia.M + p.rows_per_wg - 1) / p.rows_per_wg;
+    int64_t max_groups = ia.pairs;
+    if (NC > 1) {
+        // every expert (and the bucket of bad ids) ends with at most one partly filled group
+        max_groups = min((int64_t)ia.pairs, (int64_t)ia.n_expert + 1 + ia.pairs / NC);
+        if (hipError_t e = launch_group_pairs(ia.ids, ia.pairs, ia.n_expert, NC, groups, s)) return e;
+        ia.groups = groups;
+    } else {
+        ia.groups = nullptr;
+    }
+    if (wgs_per_group * max_groups > 0x7fffffff) return hipErrorInvalidValue;
+    ia.wgs_per_group = (int)wgs_per_group;
+    const dim3 grid((unsigned)(wgs_per_group * max_groups)), block(64 * p.kw * p.rw);
+    const int rpw = p.rows_per_wg >> p.rw_log2;
+    const size_t lds = act_lds + p.lds;
+#define ID_LAUNCH(N, DIRECT, F32, RPL) \
+    gemv_id_kernel<P, N, DIRECT, F32, RPL><<<grid, block, lds, s>>>(ia, a, xf, rpw, p.kw, p.rw_log2)
+    if (xf) {
+        if (p.kw > 1) ID_LAUNCH(1, false, true, 1);
+        else if (p.rpl == 4) ID_LAUNCH(1, true, true, 4);
+        else if (p.rpl == 2) ID_LAUNCH(1, true, true, 2);
+        else ID_LAUNCH(1, true, true, 1);
+    } else {
+        if (p.kw > 1) ID_LAUNCH(NC, false, false, 1);
+        else if (p.rpl == 4) ID_LAUNCH(NC, true, false, 4);
+        else if (p.rpl == 2) ID_LAUNCH(NC, true, false, 2);
+        else ID_LAUNCH(NC, true, false, 1);
+    }
+#undef ID_LAUNCH
+    return hipGetLastError();
+}
+
+template <class P>
+hipError_t launch_id_type(const IdArgs &ia, const DevAct &a, const float *xf, int *groups, hipStream_t s) {
+    // few pairs per expert (decode: the experts of a token are all different): nothing to share, one
+    // pair per group; otherwise up to eight pairs of an expert per pass over it
+    if (xf || !gemv_id_groups(ia.pairs, ia.n_expert)) return launch_id_as<P, 1>(ia, a, xf, groups, s);
+    return launch_id_as<P, 8>(ia, a, xf, groups, s);
+}
+
+}  // namespace
+
+size_t gemv_id_scratch_ints(int64_t pairs) { return 1 + (size_t)pairs * (2 + 16); }
+
+hipError_t launch_group_pairs(const int *ids, int pairs, int n_expert, int nc, int *groups, hipStream_t s) {
+    if (!ids || !groups || pairs < 1 || n_expert < 1 || n_expert > ID_MAX_EXPERTS) return hipErrorInvalidValue;
+    if (nc == 8) group_pairs_kernel<8><<<1, 1024, 0, s>>>(ids, pairs, n_expert, groups);
+    else if (nc == 16) group_pairs_kernel<16><<<1, 1024, 0, s>>>(ids, pairs, n_expert, groups);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+bool gemv_id_groups(int64_t pairs, int n_expert) { return pairs >= 4 * (int64_t)n_expert; }
+
+bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_expert) {
+    // every workgroup quantizes its pair's activation row again: worth it while the launch is small
+    if (gemv_id_groups(pairs, n_expert) || pairs > 64 || K < 1 || K > gemv_max_k(type)) return false;
+    Plan p;
+    bool ok = false;
+    size_t act = 0;
+    switch (type) {  // the plan of the launch: activation row plus the partial sums must fit in LDS
+    case T_Q4_K: ok = make_thin_plan<PolQ4K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4K>(K, 1); break;
+    case T_Q6_K: ok = make_thin_plan<PolQ6K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ6K>(K, 1); break;
+    case T_Q4_0: ok = make_thin_plan<PolQ4_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4_0>(K, 1); break;
+    case T_Q8_0: ok = make_thin_plan<PolQ8_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ8_0>(K, 1); break;
+    default: break;
+    }
+    return ok && act + p.lds <= THIN_LDS_MAX;
+}
+
+hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,
+                          int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s) {
+    if (n_expert < 1 || n_expert > ID_MAX_EXPERTS || w.M % n_expert || n_used < 1 || n_tokens < 1 || b_cols < 1 || !ids || !y || !groups || a.K != w.K || a.N != (int64_t)b_cols * n_tokens ||
+        (int64_t)n_used * n_tokens > 0x7fffffff / 16)
+        return hipErrorInvalidValue;
+    if (w.K < 1 || w.K > gemv_max_k(w.type)) return hipErrorInvalidValue;
+    IdArgs ia{};
+    ia.w = w; ia.ids = ids; ia.y = y; ia.M = w.M / n_expert;
+    ia.n_expert = n_expert; ia.pairs = n_used * n_tokens; ia.n_used = n_used; ia.b_cols = b_cols;
+    switch (w.type) {
+    case T_Q4_K: return a.type == T_Q8_K ? launch_id_type<PolQ4K>(ia, a, xf, groups, s) : hipErrorInvalidValue;
+    case T_Q6_K: return a.type == T_Q8_K ? launch_id_type<PolQ6K>(ia, a, xf, groups, s) : hipErrorInvalidValue;
+    case T_Q4_0: return a.type == T_Q8_0 ? launch_id_type<PolQ4_0>(ia, a, xf, groups, s) : hipErrorInvalidValue;
+    case T_Q8_0: return a.type == T_Q8_0 ? launch_id_type<PolQ8_0>(ia, a, xf, groups, s) : hipErrorInvalidValue;
+    default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace miqmm

@@ -35,6 +35,20 @@ hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int coun
                                  int num_cus, hipStream_t s);
 // largest K the GEMV handles for a weight type
 int64_t gemv_max_k(int type);
+// Expert-indexed GEMV: w is a stack of n_expert matrices (w.M = rows per expert * n_expert), a holds
+// the quantized activations of b [n_tokens][b_cols][K], ids [n_tokens][n_used] (device) picks the
+// expert of every (token, slot) pair, y [n_tokens][n_used][M].  An id outside the stack gives NaNs.
+// groups: device scratch of gemv_id_scratch_ints(n_used * n_tokens) ints.
+// xf (optional, device): b itself in f32 -- the kernel then quantizes each pair's row in its prologue
+// and a only carries the geometry; ask gemv_id_f32_supported() first.
+size_t gemv_id_scratch_ints(int64_t pairs);
+bool gemv_id_groups(int64_t pairs, int n_expert);  // enough pairs per expert to bucket them by expert
+bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);
+hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,
+                          int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s);
+// buckets the pairs by expert into groups of at most nc (1..16) pairs: groups[0] = number of groups,
+// then records {expert or -1 for ids outside the stack, count, pair[nc]}
+hipError_t launch_group_pairs(const int *ids, int pairs, int n_expert, int nc, int *groups, hipStream_t s);
 
 // kernel 3: int8-MFMA GEMM, any N >= 1.  y[n*ldy + m].  workspace (device, may be null) lets the
 // launcher cut K into slices when the output alone has too few tiles to fill the GPU;

@@ -79,7 +79,8 @@ def write_gguf(path: str, kv: Dict[str, Any], tensors: Sequence[Tuple[str, int, 
     for k in sorted(kv):
         kk = k if any(k.startswith(p) for p in (arch + ".", "general.", "adapter.", "tokenizer.")) else arch + "." + k
         out += _wstr(kk) + _value_bytes(kv[k])
-    ts = sorted(tensors, key=lambda t: (_block_number(t[0]), t[0]))
+    # raw may be any buffer (a 2-D numpy array of blocks included): its bytes are what counts
+    ts = sorted(((n, kind, shape, bytes(raw)) for n, kind, shape, raw in tensors), key=lambda t: (_block_number(t[0]), t[0]))
     offsets, s = [], 0
     for name, kind, shape, raw in ts:
         offsets.append(s)
@@ -93,7 +94,7 @@ def write_gguf(path: str, kv: Dict[str, Any], tensors: Sequence[Tuple[str, int, 
         f.write(out)
         for (name, kind, shape, raw), off in zip(ts, offsets):
             f.seek(base + off)
-            f.write(bytes(raw))
+            f.write(raw)
 
 
 class TensorInfo:
@@ -223,7 +224,7 @@ class File:
             raise KeyError(f"tensor {name} not found")
         h = ctypes.c_void_p()
         qmm._check(qmm.lib().mi_qmm_gguf_upload(ctx._h, self._h, t.index, ctypes.byref(h)))
-        return qmm.Weight(h, t.Type, t.Shape[0], t.Shape[1])
+        return qmm.Weight(h, t.Type, t.Shape[0], t.Shape[1] * (t.Shape[2] if len(t.Shape) == 3 else 1))
 
     def Close(self) -> None:
         if self._h:

@@ -2,7 +2,7 @@
 // C ABI in include/mi_qmm.h.  The reference declares it in Go:
 //   ml.Backend  /root/reference/ml/backend.go:16-33    Load / Get(name) / NewContext / Close
 //   ml.Context  /root/reference/ml/backend.go:94-128   FromFloats / Compute / Close
-//   ml.Tensor   /root/reference/ml/backend.go:130-153  Dim / Shape / Floats / Mulmat / MulmatFullPrec
+//   ml.Tensor   /root/reference/ml/backend.go:130-153  Dim / Shape / Floats / Mulmat / MulmatFullPrec / MulmatID
 // Same names, same argument meaning (ggml shapes: dimension 0 contiguous, W = [K, M], x = [K, N],
 // W.Mulmat(ctx, x) = [M, N]) and the same error behaviour: tensor ops have no error return, so a
 // failure throws (the Go interface panics).  Mulmat is lazy; Compute runs the pending nodes, sharing
@@ -45,6 +45,10 @@ public:
     // self = quantized weight [K, M], t2 = f32 activations [K, N] -> lazy [M, N]
     std::shared_ptr<Tensor> Mulmat(Context &ctx, const std::shared_ptr<Tensor> &t2);
     std::shared_ptr<Tensor> MulmatFullPrec(Context &ctx, const std::shared_ptr<Tensor> &t2) { return Mulmat(ctx, t2); }
+    // self = expert stack [K, M, E], t2 = f32 [K, B, T] (B = 1 or n_used), ids = int32 [n_used, T] -> lazy
+    // [M, n_used, T]: slot i of token t goes through expert ids[i, t] with activation row i mod B
+    std::shared_ptr<Tensor> MulmatID(Context &ctx, const std::shared_ptr<Tensor> &t2, const std::shared_ptr<Tensor> &ids);
+    const std::vector<int32_t> &Ints() const { return ints_; }
 
     ~Tensor() { mi_qmm_weight_free(weight_); }
 
@@ -55,9 +59,11 @@ private:
     int type_ = MI_QMM_TYPE_F32;
     mi_qmm_weight *weight_ = nullptr;
     std::vector<float> data_;
+    std::vector<int32_t> ints_;          // values of an int32 tensor (FromInts)
     bool ready_ = false;
     Tensor *op_w_ = nullptr;             // pending Mulmat: weight
     std::shared_ptr<Tensor> op_x_;       // pending Mulmat: activations
+    std::shared_ptr<Tensor> op_ids_;     // pending MulmatID: expert ids
     std::shared_ptr<Tensor> self_keep_;  // keeps the weight alive while a node refers to it
 };
 
@@ -77,8 +83,18 @@ public:
         check(mi_qmm_weight_upload(ctx_, ggml_type, gguf_bytes, k, m, MI_QMM_HOST, &t->weight_));
         tensors_[name] = t;
     }
+    // An expert stack [K, M, E] for MulmatID: E matrices of M rows one after the other, GGUF's layout of
+    // a 3-D expert tensor (/root/reference/convert/convert_gemma4.go:274-275).
+    void LoadExperts(const std::string &name, int ggml_type, int64_t k, int64_t m, int64_t n_expert,
+                     const void *gguf_bytes) {
+        auto t = std::make_shared<Tensor>();
+        t->shape_ = {k, m, n_expert};
+        t->type_ = ggml_type;
+        check(mi_qmm_weight_upload(ctx_, ggml_type, gguf_bytes, k, m * n_expert, MI_QMM_HOST, &t->weight_));
+        tensors_[name] = t;
+    }
     // A whole model file (the modelPath ml.NewBackend receives, /root/reference/ml/backend.go:83): every
-    // 2-D tensor of a type the Mulmat path multiplies is uploaded straight from the file mapping;
+    // 2-D tensor (and 3-D expert stack) of a type the Mulmat path multiplies is uploaded straight from the file mapping;
     // other tensors (norms, f32 embeddings) are outside this path and are skipped.  Returns how many
     // tensors were loaded.
     int LoadFile(const std::string &path) {
@@ -91,9 +107,9 @@ public:
             int type = 0, nd = 0;
             int64_t dims[4];
             rc = mi_qmm_gguf_tensor(f, i, &name, &type, &nd, dims, nullptr, nullptr);
-            if (rc != MI_QMM_OK || nd != 2 || mi_qmm_vec_dot_type(type) < 0) continue;
+            if (rc != MI_QMM_OK || (nd != 2 && nd != 3) || mi_qmm_vec_dot_type(type) < 0) continue;
             auto t = std::make_shared<Tensor>();
-            t->shape_ = {dims[0], dims[1]};
+            t->shape_.assign(dims, dims + nd);
             t->type_ = type;
             rc = mi_qmm_gguf_upload(ctx_, f, i, &t->weight_);
             if (rc == MI_QMM_OK) { tensors_[name] = t; loaded++; }
@@ -132,13 +148,34 @@ public:
         t->ready_ = true;
         return t;
     }
+    std::shared_ptr<Tensor> FromInts(const std::vector<int32_t> &s, std::vector<int64_t> shape) {
+        int64_t n = 1;
+        for (auto d : shape) n *= d;
+        if (n != (int64_t)s.size()) throw Error(MI_QMM_ERR_INVALID, "FromInts: value count does not match the shape");
+        auto t = std::make_shared<Tensor>();
+        t->shape_ = std::move(shape);
+        t->type_ = 26;  // ggml's int32, /root/reference/fs/ggml/type.go:252-279
+        t->ints_ = s;
+        t->ready_ = true;
+        return t;
+    }
     // Run every pending Mulmat node.  Nodes that read the same x are handled together: decode-sized
     // ones (n <= 8) go out four weights at a time through the entry point that quantizes x inside the
     // GEMV launch; larger ones share one quantization of x.
     void Compute() {
         std::map<std::pair<Tensor *, int>, std::vector<Tensor *>> by_x;
-        for (auto &n : nodes_)
-            if (!n->ready_) by_x[{n->op_x_.get(), n->op_w_->type_}].push_back(n.get());
+        for (auto &n : nodes_) {
+            if (n->ready_) continue;
+            if (!n->op_ids_) {
+                by_x[{n->op_x_.get(), n->op_w_->type_}].push_back(n.get());
+                continue;
+            }
+            const Tensor &w = *n->op_w_, &x = *n->op_x_, &ids = *n->op_ids_;
+            n->data_.assign((size_t)(w.Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);
+            check(mi_qmm_mulmat_id(b_.handle(), w.weight_, w.Dim(2), x.data_.data(), x.Dim(1), ids.ints_.data(), ids.Dim(0),
+                                   ids.Dim(1), n->data_.data(), MI_QMM_HOST));
+            n->ready_ = true;
+        }
         for (auto &kv : by_x) {
             Tensor *x = kv.first.first;
             const int64_t k = x->Dim(0), n = (int64_t)x->data_.size() / k;
@@ -179,6 +216,7 @@ inline std::unique_ptr<Context> Backend::NewContext() { return std::unique_ptr<C
 
 inline std::shared_ptr<Tensor> Tensor::Mulmat(Context &ctx, const std::shared_ptr<Tensor> &t2) {
     if (!weight_) throw Error(MI_QMM_ERR_INVALID, "Mulmat: the receiver must be a quantized weight from Backend::Get");
+    if (shape_.size() != 2) throw Error(MI_QMM_ERR_INVALID, "Mulmat: the weight must be 2-D (expert stacks go through MulmatID)");
     if (!t2 || t2->type_ != MI_QMM_TYPE_F32) throw Error(MI_QMM_ERR_INVALID, "Mulmat: activations must be f32");
     if (t2->Dim(0) != Dim(0)) throw Error(MI_QMM_ERR_INVALID, "Mulmat: inner dimensions differ");
     auto out = std::make_shared<Tensor>();
@@ -186,6 +224,24 @@ inline std::shared_ptr<Tensor> Tensor::Mulmat(Context &ctx, const std::shared_pt
     for (size_t i = 1; i < t2->shape_.size(); i++) out->shape_.push_back(t2->shape_[i]);
     out->op_w_ = this;
     out->op_x_ = t2;
+    ctx.nodes_.push_back(out);
+    return out;
+}
+
+inline std::shared_ptr<Tensor> Tensor::MulmatID(Context &ctx, const std::shared_ptr<Tensor> &t2,
+                                                const std::shared_ptr<Tensor> &ids) {
+    if (!weight_ || shape_.size() != 3)
+        throw Error(MI_QMM_ERR_INVALID, "MulmatID: the receiver must be a 3-D quantized expert stack from Backend::Get");
+    if (!t2 || t2->type_ != MI_QMM_TYPE_F32 || !ids || ids->type_ != 26)
+        throw Error(MI_QMM_ERR_INVALID, "MulmatID: activations must be f32 and ids int32");
+    if (t2->Dim(0) != Dim(0)) throw Error(MI_QMM_ERR_INVALID, "MulmatID: inner dimensions differ");
+    if (ids->shape_.size() > 2 || t2->shape_.size() > 3 || ids->Dim(1) != t2->Dim(2))
+        throw Error(MI_QMM_ERR_INVALID, "MulmatID: ids and activations disagree on the token count");
+    auto out = std::make_shared<Tensor>();
+    out->shape_ = {shape_[1], ids->Dim(0), ids->Dim(1)};
+    out->op_w_ = this;
+    out->op_x_ = t2;
+    out->op_ids_ = ids;
     ctx.nodes_.push_back(out);
     return out;
 }

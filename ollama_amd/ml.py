@@ -3,7 +3,7 @@
 Names, argument meaning and error behaviour follow /root/reference/ml/backend.go:
   Backend   :16-33   Load / Get(name) / NewContext / Close        (weights live here until Close)
   Context   :94-128  FromFloats / Compute / Close                 (tensors die with the context)
-  Tensor    :130-153 Dim / Stride / Shape / DType / Bytes / Floats / Mulmat / MulmatFullPrec
+  Tensor    :130-153 Dim / Stride / Shape / DType / Bytes / Floats / Mulmat / MulmatFullPrec / MulmatID
   DType     :404-412
 The reference's tensor ops build a lazy graph and have no error returns: Mulmat records a node,
 Compute runs it, and a failure is a panic -- here a raised exception.  Shapes are ggml's: dimension 0
@@ -33,7 +33,8 @@ class DType(enum.IntEnum):  # /root/reference/ml/backend.go:404-412
     MXFP4 = 6
 
 
-_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40}
+I32 = 26  # ggml_type id of int32, /root/reference/fs/ggml/type.go:252-279
+_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40, I32: DType.I32}
 
 
 class Tensor:
@@ -46,6 +47,7 @@ class Tensor:
         self._raw: Optional[np.ndarray] = None          # GGUF bytes of a weight (kept for Bytes())
         self._data: Optional[np.ndarray] = None          # f32 values, flat in ggml order
         self._op: Optional[Tuple["Tensor", "Tensor"]] = None  # (W, x) of a pending Mulmat
+        self._ids: Optional["Tensor"] = None             # third operand of a pending MulmatID
 
     # -- shape queries, /root/reference/ml/backend.go:131-135
     def Dim(self, n: int) -> int:
@@ -53,7 +55,7 @@ class Tensor:
 
     def Stride(self, n: int) -> int:
         """bytes between consecutive elements along dimension n (ggml nb[n])"""
-        if self._type != qmm.F32:
+        if self._type not in (qmm.F32, I32):
             row = qmm.row_size(self._type, self._shape[0])
             return qmm.type_size(self._type) if n == 0 else row * int(np.prod(self._shape[1:n], dtype=np.int64))
         return 4 * int(np.prod(self._shape[:n], dtype=np.int64))
@@ -80,12 +82,32 @@ class Tensor:
         """self = W [K, M] (quantized weight), t2 = x [K, N] f32  ->  [M, N] f32, lazily."""
         if self._weight is None:
             raise TypeError("Mulmat: the receiver must be a quantized weight obtained from Backend.Get")
+        if len(self._shape) != 2:
+            raise TypeError(f"Mulmat: the weight must be 2-D, got {self.Shape()} (expert stacks go through MulmatID)")
         if t2._type != qmm.F32:
             raise TypeError("Mulmat: activations must be f32")
         if t2.Dim(0) != self.Dim(0):
             raise ValueError(f"Mulmat: inner dimensions differ: {self.Shape()} x {t2.Shape()}")
         out = Tensor([self.Dim(1)] + t2._shape[1:])
         out._op = (self, t2)
+        ctx._nodes.append(out)
+        return out
+
+    def MulmatID(self, ctx: "Context", t2: "Tensor", ids: "Tensor") -> "Tensor":
+        """self = expert stack [K, M, E], t2 = x [K, B, T] f32 (B = 1 or the number of used experts),
+        ids = [n_used, T] int32  ->  [M, n_used, T] f32, lazily: slot i of token t goes through expert
+        ids[i, t] with activation row i mod B of that token.  /root/reference/ml/backend.go:153"""
+        if self._weight is None or len(self._shape) != 3:
+            raise TypeError("MulmatID: the receiver must be a 3-D quantized expert stack obtained from Backend.Get")
+        if t2._type != qmm.F32 or ids._type != I32:
+            raise TypeError("MulmatID: activations must be f32 and ids int32")
+        if t2.Dim(0) != self.Dim(0):
+            raise ValueError(f"MulmatID: inner dimensions differ: {self.Shape()} x {t2.Shape()}")
+        if len(ids._shape) > 2 or len(t2._shape) > 3 or ids.Dim(1) != t2.Dim(2):
+            raise ValueError(f"MulmatID: ids {ids.Shape()} and activations {t2.Shape()} disagree on the token count")
+        out = Tensor([self.Dim(1), ids.Dim(0), ids.Dim(1)])
+        out._op = (self, t2)
+        out._ids = ids
         ctx._nodes.append(out)
         return out
 
@@ -110,6 +132,14 @@ class Context:
         t._data = arr
         return t
 
+    def FromInts(self, s: Sequence[int], *shape: int) -> Tensor:
+        arr = np.ascontiguousarray(s, dtype=np.int32).reshape(-1)
+        if int(np.prod(shape, dtype=np.int64)) != arr.size:
+            raise ValueError(f"FromInts: {arr.size} values for shape {list(shape)}")
+        t = Tensor(shape, I32)
+        t._data = arr
+        return t
+
     def Forward(self, *tensors: Tensor) -> "Context":
         return self
 
@@ -119,6 +149,13 @@ class Context:
             raise RuntimeError("Compute on a closed context")
         pending = [t for t in self._nodes if t._data is None and t._op is not None]
         c = self._b._ctx
+        for t in [t for t in pending if t._ids is not None]:
+            w, x = t._op
+            tokens, n_used = t._ids.Dim(1), t._ids.Dim(0)
+            b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
+            y = c.mulmat_id(w._weight, w.Dim(2), b, t._ids._data.reshape(tokens, n_used))
+            t._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
+        pending = [t for t in pending if t._ids is None]
         # group by activation tensor
         by_x: Dict[int, List[Tensor]] = {}
         for t in pending:
@@ -162,8 +199,8 @@ class Backend:
     """Weights resident on one MI355X.  ``tensors`` is either the path of a GGUF file -- the model file
     ``ml.NewBackend(modelPath, params)`` receives, /root/reference/ml/backend.go:83 -- or a dict mapping a
     tensor name to (ggml_type, shape [K, M], block bytes), what fs/ggml hands out for a tensor
-    (/root/reference/fs/ggml/gguf.go:281-308).  From a file, Load uploads every 2-D tensor of a type the
-    Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q6_K) straight from the file mapping; other tensors
+    (/root/reference/fs/ggml/gguf.go:281-308).  From a file, Load uploads every 2-D tensor (and every 3-D
+    expert stack) of a type the Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q6_K) straight from the file mapping; other tensors
     (norms, f32 embeddings) are outside this path and are skipped."""
 
     def __init__(self, tensors, device: int = 0):
@@ -177,7 +214,7 @@ class Backend:
             from . import gguf
 
             with gguf.File(self._spec if isinstance(self._spec, str) else self._spec.decode()) as f:
-                infos = [t for t in f.TensorInfos() if len(t.Shape) == 2 and qmm.vec_dot_type(t.Type) >= 0]
+                infos = [t for t in f.TensorInfos() if len(t.Shape) in (2, 3) and qmm.vec_dot_type(t.Type) >= 0]
                 for i, ti in enumerate(infos):
                     t = Tensor(ti.Shape, ti.Type)
                     t._weight = f.Upload(self._ctx, ti.Name)
@@ -189,11 +226,11 @@ class Backend:
             return
         total = max(len(self._spec), 1)
         for i, (name, (ggml_type, shape, raw)) in enumerate(self._spec.items()):
-            if len(shape) != 2:
-                raise ValueError(f"{name}: only 2-D weights take part in Mulmat, got shape {list(shape)}")
-            k, m = int(shape[0]), int(shape[1])
+            if len(shape) not in (2, 3):
+                raise ValueError(f"{name}: Mulmat takes 2-D weights and MulmatID 3-D expert stacks, got shape {list(shape)}")
+            k, m = int(shape[0]), int(np.prod(shape[1:], dtype=np.int64))  # a stack is its experts' rows in a row
             raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1)
-            t = Tensor([k, m], ggml_type)
+            t = Tensor(shape, ggml_type)
             t._weight = self._ctx.upload(ggml_type, raw, k, m)
             t._raw = raw
             self._tensors[name] = t

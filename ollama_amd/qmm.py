@@ -24,7 +24,7 @@ EXPORTS = [
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
-    "mi_qmm_mulmat_multi",
+    "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
     "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
@@ -84,6 +84,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_q8_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_multi.restype = ci
     L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
+    L.mi_qmm_mulmat_id.restype = ci
+    L.mi_qmm_mulmat_id.argtypes = [vp, vp, ci, vp, ci, vp, ci, i64, vp, ci]
     P = ctypes.POINTER
     L.mi_qmm_gguf_open.restype = ci; L.mi_qmm_gguf_open.argtypes = [ctypes.c_char_p, P(vp)]
     L.mi_qmm_gguf_close.restype = None; L.mi_qmm_gguf_close.argtypes = [vp]
@@ -309,6 +311,27 @@ class Context:
         wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
         yp = (ctypes.c_void_p * len(ws))(*[ctypes.c_void_p(int(p)) for p in y_ptrs])
         _check(lib().mi_qmm_mulmat_multi(self._h, wh, len(ws), ctypes.c_void_p(int(x_ptr)), n, yp, DEVICE))
+
+    def mulmat_id(self, w: Weight, n_expert: int, b: np.ndarray, ids: np.ndarray) -> np.ndarray:
+        """w: n_expert stacked matrices uploaded as one weight of m = rows * n_expert; b: f32
+        [tokens, b_cols, k]; ids: int32 [tokens, n_used] -> f32 [tokens, n_used, rows]."""
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        if b.ndim != 3 or ids.ndim != 2 or b.shape[0] != ids.shape[0] or b.shape[2] != w.k:
+            raise ValueError(f"b {b.shape} / ids {ids.shape} do not fit [tokens, b_cols, k={w.k}] / [tokens, n_used]")
+        t, n_used = ids.shape
+        y = np.empty((t, n_used, w.m // max(n_expert, 1)), dtype=np.float32)  # the library rejects a ragged split
+        _check(lib().mi_qmm_mulmat_id(self._h, w._h, n_expert, b.ctypes.data_as(ctypes.c_void_p), b.shape[1],
+                                      ids.ctypes.data_as(ctypes.c_void_p), n_used, t,
+                                      y.ctypes.data_as(ctypes.c_void_p), HOST))
+        return y
+
+    def mulmat_id_device(self, w: Weight, n_expert: int, b_ptr: int, b_cols: int, ids_ptr: int, n_used: int,
+                         n_tokens: int, y_ptr: int):
+        """device pointers; queued on the ctx's stream"""
+        _check(lib().mi_qmm_mulmat_id(self._h, w._h, n_expert, ctypes.c_void_p(int(b_ptr)), b_cols,
+                                      ctypes.c_void_p(int(ids_ptr)), n_used, n_tokens, ctypes.c_void_p(int(y_ptr)),
+                                      DEVICE))
 
     def mulmat_q8_multi(self, ws, act: Act):
         """several weights against the same activations; host arrays out"""

@@ -51,6 +51,8 @@ def lib() -> ctypes.CDLL:
         L.ref_vec_dot_type.restype = ci; L.ref_vec_dot_type.argtypes = [ci]
         L.ref_mul_mat.restype = ci
         L.ref_mul_mat.argtypes = [ci, vp, i64, i64, vp, i64, vp, vp, ci]
+        L.ref_mul_mat_id.restype = ci
+        L.ref_mul_mat_id.argtypes = [ci, vp, i64, i64, i64, vp, i64, vp, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -137,6 +139,24 @@ def mul_mat(wtype: int, w: np.ndarray, k: int, m: int, x: np.ndarray, nthreads: 
     if lib().ref_mul_mat(wtype, _p(w), k, m, _p(x), n, _p(y), _p(xq), nthreads) != 0:
         raise ValueError("ref_mul_mat failed")
     return (y, xq) if return_xq else y
+
+
+def mul_mat_id(wtype: int, w: np.ndarray, k: int, m: int, n_expert: int, b: np.ndarray, ids: np.ndarray):
+    """w: uint8 GGUF blocks of n_expert stacked matrices of m rows; b: f32 [tokens, b_cols, k];
+    ids: int32 [tokens, n_used] -> y f32 [tokens, n_used, m]."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    assert b.ndim == 3 and ids.ndim == 2 and b.shape[0] == ids.shape[0] and b.shape[2] == k
+    assert w.size == n_expert * m * row_size(wtype, k)
+    t, n_used = ids.shape
+    y = np.empty((t, n_used, m), dtype=np.float32)
+    rc = lib().ref_mul_mat_id(wtype, _p(w), k, m, n_expert, _p(b), b.shape[1], _p(ids), n_used, t, _p(y))
+    if rc == -2:
+        raise IndexError("expert id outside 0..n_expert-1")
+    if rc != 0:
+        raise ValueError("ref_mul_mat_id failed")
+    return y
 
 
 def scale_min_k4(j: int, s12: np.ndarray):

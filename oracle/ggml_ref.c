@@ -747,3 +747,36 @@ int ref_mul_mat(int wtype, const void *w, int64_t k, int64_t m, const float *x, 
     if (!xq_out) free(xq);
     return 0;
 }
+
+/*
+ * mul_mat_id (ggml-cpu.c ggml_compute_forward_mul_mat_id, upstream): src1 is quantized row by row
+ * to the weight's vec_dot_type, then for every (token t, slot i) pair
+ *     dst[t][i][m] = vec_dot(as[ids[t][i]] row m, Q(src1[t][i % ne11]))
+ * -- the expert comes from ids, the activation row of slot i is i modulo src1's second dimension
+ * (ne11 = 1: one row per token shared by all slots; ne11 = n_used: a row per slot).  upstream
+ * asserts 0 <= id < n_as; here that is return value -2.
+ */
+int ref_mul_mat_id(int wtype, const void *as, int64_t k, int64_t m, int64_t n_expert, const float *b,
+                   int64_t b_cols, const int32_t *ids, int64_t n_used, int64_t n_tokens, float *y) {
+    dot_fn df = dot_for(wtype);
+    const int qt = ref_vec_dot_type(wtype);
+    if (!df || qt < 0 || m < 0 || n_expert < 1 || b_cols < 1 || n_used < 1 || n_tokens < 0) return -1;
+    const int64_t wrb = ref_row_size(wtype, k), xrb = ref_row_size(qt, k);
+    if (wrb < 0 || xrb < 0) return -1;
+    if (m * n_tokens == 0) return 0;
+    if (!as || !b || !ids || !y) return -1;
+    for (int64_t p = 0; p < n_used * n_tokens; p++)
+        if (ids[p] < 0 || ids[p] >= n_expert) return -2;
+    char *xq = (char *)malloc((size_t)(n_tokens * b_cols * xrb) + 1);
+    if (!xq) return -1;
+    ref_quantize(qt, b, xq, k, n_tokens * b_cols, 1);
+    for (int64_t t = 0; t < n_tokens; t++)
+        for (int64_t i = 0; i < n_used; i++) {
+            const char *w = (const char *)as + (int64_t)ids[t * n_used + i] * m * wrb;
+            const char *x = xq + (t * b_cols + i % b_cols) * xrb;
+            float *out = y + (t * n_used + i) * m;
+            for (int64_t r = 0; r < m; r++) out[r] = df(k, w + r * wrb, x);
+        }
+    free(xq);
+    return 0;
+}

@@ -19,6 +19,10 @@
  * Parity status per function (what pins it is in tests/test_oracle_*.py):
  *   fp16<->fp32, q8_0/q8_K quantizers, 6-bit scale unpack, four vec_dots, dequantizers,
  *   mul_mat driver:  pinned (numpy float16, closed forms, fp64 brute force, KATs).
+ *   mul_mat_id driver: the per-pair arithmetic is the pinned vec_dots; the indexing is pinned by
+ *   its reduction to mul_mat (one expert; a pair's result equals mul_mat on that expert alone) and
+ *   fp64 brute force.  The rule "slot i reads activation row i mod ne11" is upstream ggml's and the
+ *   reference holds no test of it: PARITY UNPINNED for b_cols other than 1 and n_used.
  *   weight encoders q4_K / q6_K (make_qkx2_quants / make_qx_quants searches):
  *   PARITY UNPINNED bit-for-bit against llama-quantize (only self-consistency and error
  *   bounds are checked); q4_0 / q8_0 encoders are closed forms and pinned.
@@ -78,6 +82,15 @@ int  ref_vec_dot_type(int wtype);
  */
 int  ref_mul_mat(int wtype, const void *w, int64_t k, int64_t m,
                  const float *x, int64_t n, float *y, void *xq_out, int nthreads);
+
+/*
+ * mul_mat_id: as = n_expert matrices of M rows of K elements, one after the other; b = f32
+ * [n_tokens][b_cols][K]; ids = int32 [n_tokens][n_used];
+ * y[(t*n_used + i)*M + m] = vec_dot(as[ids[t][i]] row m, Q(b[t][i % b_cols])).
+ * returns 0, -1 on bad arguments, -2 when an id is outside 0..n_expert-1.
+ */
+int  ref_mul_mat_id(int wtype, const void *as, int64_t k, int64_t m, int64_t n_expert, const float *b,
+                    int64_t b_cols, const int32_t *ids, int64_t n_used, int64_t n_tokens, float *y);
 
 #ifdef __cplusplus
 }

@@ -119,6 +119,41 @@ int main() {
             }
             from_file.Close();
         }
+        // expert-indexed product: a stack of 5 experts, 3 used per token, one activation row per token
+        {
+            const int64_t k = 1024, m = 96, n_expert = 5, n_used = 3;
+            auto wf = randn((size_t)(k * m * n_expert), 0.02f, 1234);
+            std::vector<uint8_t> raw((size_t)(ref_row_size(MI_QMM_TYPE_Q4_K, k) * m * n_expert));
+            if (ref_quantize(MI_QMM_TYPE_Q4_K, wf.data(), raw.data(), k, m * n_expert, 4) != 0) return 1;
+            backend.LoadExperts("blk.0.ffn_up_exps.weight", MI_QMM_TYPE_Q4_K, k, m, n_expert, raw.data());
+            for (int64_t tokens : {1, 11}) {
+                auto ctx = backend.NewContext();
+                auto xv = randn((size_t)(k * tokens), 1.0f, 77 + (unsigned)tokens);
+                std::vector<int32_t> idv;
+                for (int64_t t = 0; t < tokens; t++)
+                    for (int64_t i = 0; i < n_used; i++) idv.push_back((int32_t)((t * 2 + i * 3) % n_expert));
+                auto y = backend.Get("blk.0.ffn_up_exps.weight")
+                             ->MulmatID(*ctx, ctx->FromFloats(xv, {k, 1, tokens}), ctx->FromInts(idv, {n_used, tokens}));
+                ctx->Compute();
+                std::vector<float> ref((size_t)(m * n_used * tokens));
+                if (ref_mul_mat_id(MI_QMM_TYPE_Q4_K, raw.data(), k, m, n_expert, xv.data(), 1, idv.data(), n_used, tokens,
+                                   ref.data()) != 0) return 1;
+                const double e = rel_err(y->Floats(), ref);
+                const bool shape_ok = y->Dim(0) == m && y->Dim(1) == n_used && y->Dim(2) == tokens;
+                printf("%-24s T=%-3lld rel err %.2e %s\n", "ffn_up_exps MulmatID", (long long)tokens, e,
+                       (e <= 1e-3 && shape_ok) ? "ok" : "FAIL");
+                if (!(e <= 1e-3) || !shape_ok) failures++;
+                ctx->Close();
+            }
+            bool threw_id = false;
+            try {
+                auto ctx = backend.NewContext();
+                backend.Get("blk.0.ffn_up_exps.weight")
+                    ->MulmatID(*ctx, ctx->FromFloats(std::vector<float>(k), {k, 1, 1}), ctx->FromInts({5}, {1, 1}));
+                ctx->Compute();
+            } catch (const Error &) { threw_id = true; }
+            if (!threw_id) { printf("FAIL: an expert id outside the stack did not throw\n"); failures++; }
+        }
         backend.Close();
         printf(failures ? "host mirror: %d FAILURES\n" : "host mirror: all ok\n", failures);
         return failures ? 1 : 0;

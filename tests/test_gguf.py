@@ -169,3 +169,20 @@ def test_tensor_sizes_match_the_reference_table(tmp_path):
         for row in golden["sizes"]:
             t = f.TensorInfo(f"t{row['kind']}")
             assert t.Type == row["kind"] and t.NumBytes == row["type_size"] * 6, row
+
+
+def test_expert_stack_tensors_and_array_buffers_round_trip(tmp_path):
+    """3-D expert tensors (ne = [in, out, experts], /root/reference/convert/convert_gemma4.go:274-275) and
+    tensor data handed over as a 2-D array of block rows: offsets count bytes, not rows"""
+    rng = np.random.default_rng(3)
+    a = rng.integers(0, 256, (6 * 4, 34 * 3), dtype=np.uint8)    # Q8_0 [96, 4, 6]: 24 rows of 3 blocks
+    b = rng.integers(0, 256, (2 * 5, 144), dtype=np.uint8)       # Q4_K [256, 5, 2]
+    p = str(tmp_path / "moe.gguf")
+    gguf.write_gguf(p, {"general.architecture": "x"},
+                    [("blk.0.ffn_down_exps.weight", qmm.Q8_0, [96, 4, 6], a), ("blk.0.ffn_up_exps.weight", qmm.Q4_K, [256, 5, 2], b)])
+    with gguf.File(p) as f:
+        ta, tb = f.TensorInfo("blk.0.ffn_down_exps.weight"), f.TensorInfo("blk.0.ffn_up_exps.weight")
+        assert ta.Shape == [96, 4, 6] and ta.NumBytes == a.size and ta.Offset == 0
+        assert tb.Shape == [256, 5, 2] and tb.NumBytes == b.size and tb.Offset == (a.size + 31) // 32 * 32
+        assert f.TensorBytes(ta.Name).tobytes() == a.tobytes()
+        assert f.TensorBytes(tb.Name).tobytes() == b.tobytes()

@@ -63,6 +63,52 @@ def test_python_mirror_layer_graph():
     b.Close()
 
 
+def test_python_mirror_expert_graph(tmp_path):
+    """a mixture-of-experts FFN the way a model drives it: router ids from FromInts, gate/up through
+    MulmatID with one activation row per token, down with one row per used expert -- from a GGUF file
+    whose expert tensors are 3-D"""
+    from ollama_amd import gguf, ml
+
+    k, ff, n_expert, n_used = 512, 384, 6, 3
+    rng = np.random.default_rng(81)
+    gate = oracle.quantize(qmm.Q4_K, rng.standard_normal((n_expert * ff, k), dtype=np.float32) * np.float32(0.02))
+    down = oracle.quantize(qmm.Q8_0, rng.standard_normal((n_expert * k, ff), dtype=np.float32) * np.float32(0.02))
+    path = str(tmp_path / "moe.gguf")
+    gguf.write_gguf(path, {"general.architecture": "qwen3moe"},
+                    [("blk.0.ffn_gate_exps.weight", qmm.Q4_K, [k, ff, n_expert], gate),
+                     ("blk.0.ffn_down_exps.weight", qmm.Q8_0, [ff, k, n_expert], down)])
+    b = ml.Backend(path)
+    b.Load()
+    wg, wd = b.Get("blk.0.ffn_gate_exps.weight"), b.Get("blk.0.ffn_down_exps.weight")
+    assert wg.Shape() == [k, ff, n_expert] and wd.Shape() == [ff, k, n_expert]
+    for tokens in (1, 9):
+        ctx = b.NewContext()
+        xv = rng.standard_normal((tokens, 1, k), dtype=np.float32)
+        hv = rng.standard_normal((tokens, n_used, ff), dtype=np.float32)
+        idv = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+        ids = ctx.FromInts(idv.reshape(-1), n_used, tokens)
+        assert ids.DType() == ml.DType.I32
+        g = wg.MulmatID(ctx, ctx.FromFloats(xv.reshape(-1), k, 1, tokens), ids)
+        d = wd.MulmatID(ctx, ctx.FromFloats(hv.reshape(-1), ff, n_used, tokens), ids)
+        assert g.Shape() == [ff, n_used, tokens] and d.Shape() == [k, n_used, tokens]
+        ctx.Compute(g, d)
+        assert npref.rel_err(g.Floats().reshape(tokens, n_used, ff),
+                             oracle.mul_mat_id(qmm.Q4_K, gate, k, ff, n_expert, xv, idv)) <= 1e-3
+        assert npref.rel_err(d.Floats().reshape(tokens, n_used, k),
+                             oracle.mul_mat_id(qmm.Q8_0, down, ff, k, n_expert, hv, idv)) <= 1e-3
+        with pytest.raises(TypeError):
+            wg.Mulmat(ctx, ctx.FromFloats(xv.reshape(-1), k, tokens))        # a stack is not a 2-D weight
+        with pytest.raises(ValueError):
+            wg.MulmatID(ctx, ctx.FromFloats(xv.reshape(-1), k, 1, tokens), ctx.FromInts([0], 1, 1) if tokens > 1
+                        else ctx.FromInts([0, 1], 1, 2))                      # token counts differ
+        ctx.Close()
+    ctx = b.NewContext()
+    bad = wg.MulmatID(ctx, ctx.FromFloats(np.zeros(k, np.float32), k, 1, 1), ctx.FromInts([n_expert], 1, 1))
+    with pytest.raises(qmm.QmmError):
+        ctx.Compute(bad)                                                      # ggml aborts on such an id
+    b.Close()
+
+
 def test_cpp_mirror_program():
     exe = os.path.join(ROOT, "tests", "cpp", "test_host_mirror")
     if not os.path.exists(exe):

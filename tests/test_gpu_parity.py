@@ -10,6 +10,7 @@ import pytest
 
 import npref
 import oracle
+from hipmem import DeviceArray
 from npref import Q4_0, Q4_K, Q6_K, Q8_0, Q8_K
 from ollama_amd import qmm
 
@@ -422,3 +423,122 @@ def test_config5_prefill_layer_batch512(ctx, name, t, m, k):
     nrm = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
     assert err <= TOL and nrm <= 1e-5, f"{name}: rel err {err}, normwise {nrm}"
     W.free()
+
+
+# ---- expert-indexed product (Tensor.MulmatID) ------------------------------------------------------
+def _experts(t, n_expert, m, k, seed):
+    return _weights(t, n_expert * m, k, seed)
+
+
+@pytest.mark.parametrize("t", WTYPES)
+@pytest.mark.parametrize("tokens,n_used,b_cols", [(1, 8, 1), (1, 8, 8), (2, 4, 4), (40, 4, 1), (33, 6, 6), (7, 5, 2)])
+def test_mulmat_id_matches_oracle(ctx, t, tokens, n_used, b_cols):
+    """decode (one pair per group, straight from ids) and batches (pairs bucketed by expert)"""
+    rng = np.random.default_rng(7000 + t * 131 + tokens * 7 + n_used + b_cols)
+    k, m, n_expert = 1024, 200, 12
+    wb = _experts(t, n_expert, m, k, 7100 + t)
+    w = ctx.upload(t, wb, k, n_expert * m)
+    b = rng.standard_normal((tokens, b_cols, k), dtype=np.float32)
+    ids = rng.integers(0, n_expert, (tokens, n_used)).astype(np.int32)
+    got = ctx.mulmat_id(w, n_expert, b, ids)
+    want = oracle.mul_mat_id(t, wb, k, m, n_expert, b, ids)
+    assert got.shape == want.shape
+    assert npref.rel_err(got, want) < TOL
+    w.free()
+
+
+def test_mulmat_id_equals_mulmat_on_the_expert_alone(ctx):
+    """bit-identical to the plain product on one expert's slice, whatever group a pair lands in"""
+    rng = np.random.default_rng(7200)
+    k, m, n_expert, tokens, n_used = 2048, 96, 6, 24, 3
+    wb = _experts(Q4_K, n_expert, m, k, 7201)
+    w = ctx.upload(Q4_K, wb, k, n_expert * m)
+    b = rng.standard_normal((tokens, 1, k), dtype=np.float32)
+    ids = rng.integers(0, n_expert, (tokens, n_used)).astype(np.int32)
+    got = ctx.mulmat_id(w, n_expert, b, ids)
+    w3 = wb.reshape(n_expert, m, -1)
+    for e in range(n_expert):
+        we = ctx.upload(Q4_K, w3[e], k, m)
+        for ti, i in np.argwhere(ids == e):
+            assert np.array_equal(got[ti, i], ctx.mulmat(we, b[ti, 0])[0])  # the decode GEMV, one column
+        we.free()
+    # the same pairs one token at a time (no bucketing) give the same bits
+    for ti in (0, 5, 23):
+        assert np.array_equal(ctx.mulmat_id(w, n_expert, b[ti:ti + 1], ids[ti:ti + 1])[0], got[ti])
+    w.free()
+
+
+def test_mulmat_id_moe_decode_shape(ctx):
+    """Qwen3-30B-A3B-like expert FFN: 128 experts, 8 used, gate 768x2048 then down 2048x768"""
+    rng = np.random.default_rng(7300)
+    n_expert, n_used = 128, 8
+    for k, m, b_cols in ((2048, 768, 1), (768, 2048, 8)):
+        wb = _experts(Q4_K, n_expert, m, k, 7301 + k)
+        w = ctx.upload(Q4_K, wb, k, n_expert * m)
+        b = rng.standard_normal((1, b_cols, k), dtype=np.float32)
+        ids = rng.choice(n_expert, n_used, replace=False).astype(np.int32)[None, :]
+        got = ctx.mulmat_id(w, n_expert, b, ids)
+        assert npref.rel_err(got, oracle.mul_mat_id(Q4_K, wb, k, m, n_expert, b, ids)) < TOL
+        w.free()
+
+
+def test_mulmat_id_device_ids_out_of_range_give_nan_host_ids_are_rejected(ctx):
+    rng = np.random.default_rng(7400)
+    k, m, n_expert = 512, 40, 4
+    wb = _experts(Q8_0, n_expert, m, k, 7401)
+    w = ctx.upload(Q8_0, wb, k, n_expert * m)
+    for tokens in (1, 30):  # both the direct and the bucketed launch
+        b = rng.standard_normal((tokens, 1, k), dtype=np.float32)
+        ids = rng.integers(0, n_expert, (tokens, 2)).astype(np.int32)
+        bad = ids.copy()
+        bad[0, 1] = n_expert
+        bad[-1, 0] = -1
+        with pytest.raises(qmm.QmmError) as e:
+            ctx.mulmat_id(w, n_expert, b, bad)
+        assert e.value.code == qmm.ERR_INVALID
+        db, dids = DeviceArray(b), DeviceArray(bad)
+        dy = DeviceArray(np.zeros((tokens, 2, m), np.float32), zero=True)
+        ctx.mulmat_id_device(w, n_expert, db.ptr, 1, dids.ptr, 2, tokens, dy.ptr)
+        ctx.sync()
+        got = dy.numpy()
+        for d in (db, dids, dy):
+            d.free()
+        want = oracle.mul_mat_id(Q8_0, wb, k, m, n_expert, b, ids)
+        isbad = (bad < 0) | (bad >= n_expert)
+        assert np.isnan(got[isbad]).all()
+        assert not np.isnan(got[~isbad]).any()
+        assert npref.rel_err(got[~isbad], want[~isbad]) < TOL
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_id(w, 3, np.zeros((1, 1, k), np.float32), np.zeros((1, 1), np.int32))  # 160 rows / 3 experts
+    assert e.value.code == qmm.ERR_INVALID
+    assert ctx.mulmat_id(w, n_expert, np.zeros((0, 1, k), np.float32), np.zeros((0, 2), np.int32)).shape == (0, 2, m)
+    w.free()
+
+
+# ---- device pointers in and out ----------------------------------------------------------------------
+@pytest.mark.parametrize("t", WTYPES)
+@pytest.mark.parametrize("n", [1, 6, 48])
+def test_device_pointers_give_the_same_bits_as_host_arrays(ctx, t, n):
+    """MI_QMM_DEVICE: x and y stay on the device and the call only queues work on the ctx's stream"""
+    rng = np.random.default_rng(7500 + t + n)
+    k, m = 1024, 384
+    wb = _weights(t, m, k, 7501 + t)
+    wb2 = _weights(t, 128, k, 7502 + t)
+    w, w2 = ctx.upload(t, wb, k, m), ctx.upload(t, wb2, k, 128)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    dx = DeviceArray(x)
+    dy, dy2 = DeviceArray(np.zeros((n, m), np.float32), zero=True), DeviceArray(np.zeros((n, 128), np.float32), zero=True)
+    ctx.mulmat_device(w, dx.ptr, n, dy.ptr)
+    ctx.sync()
+    assert np.array_equal(dy.numpy(), ctx.mulmat(w, x))
+    for d in (dy, dy2):
+        d.free()
+    dy, dy2 = DeviceArray(np.zeros((n, m), np.float32), zero=True), DeviceArray(np.zeros((n, 128), np.float32), zero=True)
+    ctx.mulmat_multi_device([w, w2], dx.ptr, n, [dy.ptr, dy2.ptr])
+    ctx.sync()
+    h, h2 = ctx.mulmat_multi([w, w2], x)
+    assert np.array_equal(dy.numpy(), h) and np.array_equal(dy2.numpy(), h2)
+    for d in (dx, dy, dy2):
+        d.free()
+    w.free()
+    w2.free()

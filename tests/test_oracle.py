@@ -309,6 +309,55 @@ def test_mul_mat_rejects_bad_arguments():
     assert L.ref_mul_mat(Q4_K, None, 256, 0, None, 0, None, None, 1) == 0    # empty is fine
 
 
+# ---- mul_mat_id driver -------------------------------------------------------------------------
+@pytest.mark.parametrize("t", WTYPES)
+@pytest.mark.parametrize("b_cols", [1, 3])
+def test_mul_mat_id_reduces_to_mul_mat_per_pair(t, b_cols):
+    """every (token, slot) pair is mul_mat on that pair's expert alone with that pair's activation row;
+    shapes chosen so that a swapped index (expert/slot/token, m/n_used) lands on a different value"""
+    rng = np.random.default_rng(500 + t + b_cols)
+    k, m, n_expert, n_used, tokens = 512, 5, 7, 3, 4
+    w = oracle.quantize(t, (rng.standard_normal((n_expert * m, k)) * 0.02).astype(np.float32))
+    b = rng.standard_normal((tokens, b_cols, k)).astype(np.float32)
+    ids = rng.integers(0, n_expert, (tokens, n_used)).astype(np.int32)
+    ids[0] = [6, 0, 6]  # the same expert twice in one token
+    y = oracle.mul_mat_id(t, w, k, m, n_expert, b, ids)
+    assert y.shape == (tokens, n_used, m)
+    w3 = w.reshape(n_expert, m, -1)
+    for ti in range(tokens):
+        for i in range(n_used):
+            want = oracle.mul_mat(t, w3[ids[ti, i]], k, m, b[ti, i % b_cols])
+            assert np.array_equal(y[ti, i], want[0])
+
+
+@pytest.mark.parametrize("t", WTYPES)
+def test_mul_mat_id_vs_fp64_brute_force(t):
+    rng = np.random.default_rng(520 + t)
+    k, m, n_expert, n_used, tokens = 1024, 6, 4, 2, 3
+    w = oracle.quantize(t, (rng.standard_normal((n_expert * m, k)) * 0.02).astype(np.float32))
+    b = rng.standard_normal((tokens, n_used, k)).astype(np.float32)
+    ids = np.array([[0, 3], [2, 2], [1, 0]], np.int32)
+    y = oracle.mul_mat_id(t, w, k, m, n_expert, b, ids)
+    qt = oracle.vec_dot_type(t)
+    xq = oracle.quantize(qt, b.reshape(-1, k))
+    full = npref.matmul_f64(t, w, k, n_expert * m, qt, xq, tokens * n_used).reshape(tokens, n_used, n_expert, m)
+    want = np.stack([[full[ti, i, ids[ti, i]] for i in range(n_used)] for ti in range(tokens)])
+    assert npref.rel_err(y, want) < 1e-5
+
+
+def test_mul_mat_id_one_expert_is_mul_mat_and_bad_ids_are_rejected():
+    rng = np.random.default_rng(540)
+    k, m = 256, 9
+    w = oracle.quantize(Q4_K, (rng.standard_normal((m, k)) * 0.02).astype(np.float32))
+    b = rng.standard_normal((5, 1, k)).astype(np.float32)
+    y = oracle.mul_mat_id(Q4_K, w, k, m, 1, b, np.zeros((5, 1), np.int32))
+    assert np.array_equal(y[:, 0], oracle.mul_mat(Q4_K, w, k, m, b[:, 0]))
+    for bad in (-1, 1):
+        with pytest.raises(IndexError):
+            oracle.mul_mat_id(Q4_K, w, k, m, 1, b, np.array([[0], [0], [bad], [0], [0]], np.int32))
+    assert oracle.mul_mat_id(Q4_K, w, k, m, 1, b[:0], np.zeros((0, 1), np.int32)).shape == (0, 1, m)
+
+
 # ---- weight encoders: self-consistency (bit-parity with llama-quantize is unpinned) --------------
 @pytest.mark.parametrize("t,bound", [(Q4_0, 0.14), (Q8_0, 0.008), (Q4_K, 0.10), (Q6_K, 0.03)])
 def test_encoders_valid_blocks_and_error_bounds(t, bound):
