@@ -608,13 +608,19 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
     }
     DevAct a{};
     a.K = K; a.N = (int)ncols; a.type = q8;
-    const bool fused = gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert);
+    const bool skinny = skinny_id_supports(w->dev.type, K, M, pairs, n_expert);
+    const bool fused = !skinny && gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert);
     if (!fused) {
-        HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, nullptr, nullptr, ctx->stream));
-        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums;
+        HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16;
     }
-    HIP_TRY(launch_gemv_id(w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
-                           (int *)ctx->ws_buf, ctx->stream));
+    if (skinny)
+        // a few pairs per expert and more: on the matrix cores, the experts' weights read once per 16 pairs
+        HIP_TRY(launch_skinny_id(w->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy, (int *)ctx->ws_buf,
+                                 ctx->num_cus, ctx->stream));
+    else
+        HIP_TRY(launch_gemv_id(w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
+                               (int *)ctx->ws_buf, ctx->stream));
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));

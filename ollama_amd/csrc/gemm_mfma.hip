@@ -561,9 +561,20 @@ struct SkinnyGeo {
     static constexpr int PART_BYTES = 16 * 16 * 4;  // per wave: its partial sums
 };
 
+// Expert-indexed launches (Tensor.MulmatID, /root/reference/ml/backend.go:153): w is a stack of expert
+// matrices of M rows each, a workgroup belongs to one group of up to 16 (token, slot) pairs that all
+// name the same expert, takes its activation columns from the pairs and writes y[pair][row].
+struct SkinnyIds {
+    const int *groups;  // groups[0] = number of groups, then records {expert or -1, count, pair[16]}
+    int64_t M;          // rows per expert
+    int wgs_per_group, n_used, b_cols;
+};
+constexpr int SKINNY_ID_REC = 2 + 16;
+
 // The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
-template <class S, int NCT>
-__global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y) {
+template <class S, int NCT, bool ID>
+__global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
+                                                        SkinnyIds si) {
     typedef typename S::G G;
     typedef SkinnyGeo<S, NCT> Geo;
     constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
@@ -574,8 +585,33 @@ __global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, i
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, g = lane >> 4;
-    const int64_t m0 = (int64_t)blockIdx.x * 16;
-    const int rows_left = (int)min((int64_t)16, w.M - m0);  // rows past M: the last row again, results dropped
+    int64_t m0 = (int64_t)blockIdx.x * 16, yrow0 = m0, ldy = w.M;
+    int rows_left = (int)min((int64_t)16, w.M - m0);  // rows past M: the last row again, results dropped
+    const int *rec = nullptr;
+    if (ID) {
+        const int group = blockIdx.x / si.wgs_per_group;
+        if (group >= si.groups[0]) return;
+        rec = si.groups + 1 + (size_t)group * SKINNY_ID_REC;
+        const int expert = rec[0];
+        nc = rec[1];
+        yrow0 = (int64_t)(blockIdx.x - group * si.wgs_per_group) * 16;  // row inside the expert
+        rows_left = (int)min((int64_t)16, si.M - yrow0);
+        ldy = si.M;
+        if (expert < 0) {
+            // ids outside the stack: these pairs' outputs are all NaN
+            for (int o = tid; o < 16 * nc; o += blockDim.x)
+                if ((o & 15) < rows_left) y[(int64_t)rec[2 + (o >> 4)] * ldy + yrow0 + (o & 15)] = __int_as_float(0x7fc00000);
+            return;
+        }
+        m0 = (int64_t)expert * si.M + yrow0;
+    }
+    // activation column (row of a) behind the launch's column i
+    auto acol = [&](int i) {
+        i = min(i, nc - 1);
+        if (!ID) return col0 + i;
+        const int pair = rec[2 + i], tok = pair / si.n_used;
+        return tok * si.b_cols + (pair - tok * si.n_used) % si.b_cols;
+    };
     const int64_t nsb = w.K / QKK;
     const int64_t sb0 = nsb * wave / WAVES, sb1 = nsb * (wave + 1) / WAVES;  // this wave's run of super-blocks
     uint8_t *wsm = smem + wave * WAVE_BYTES;
@@ -590,12 +626,12 @@ __global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, i
 #pragma unroll
     for (int j = 0; j < A_INSTRS; j++) {
         const int col = 4 * j + (lane >> 4), slot = lane & 15;  // stage slot [col][slot] holds piece slot ^ col
-        aoff[j] = (unsigned)(col0 + min(col, nc - 1)) * (unsigned)a.K + 16u * (slot ^ (col & 15));
+        aoff[j] = (unsigned)acol(col) * (unsigned)a.K + 16u * (slot ^ (col & 15));
     }
     const int dcol = lane / S::D_LANES_PER_COL;
     const bool don = lane < NCT * S::D_LANES_PER_COL, yon = lane < NCT;
-    const unsigned doff = (unsigned)(col0 + min(dcol, nc - 1)) * (unsigned)(nsb * G::SD) + 16u * (lane % S::D_LANES_PER_COL);
-    const unsigned yoff = (unsigned)(col0 + min(lane, nc - 1)) * (unsigned)nsb * 4u;
+    const unsigned doff = (unsigned)acol(dcol) * (unsigned)(nsb * G::SD) + 16u * (lane % S::D_LANES_PER_COL);
+    const unsigned yoff = (unsigned)acol(lane) * (unsigned)nsb * 4u;
     const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
     const uint8_t *asd = G::digits(a);
 
@@ -682,7 +718,7 @@ __global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, i
         const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
         float sum = 0.f;
         for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
-        if (i < nc && m0 + j < w.M) y[(int64_t)(col0 + i) * w.M + m0 + j] = sum;
+        if (i < nc && j < rows_left) y[(int64_t)(ID ? rec[2 + i] : col0 + i) * ldy + yrow0 + j] = sum;
     }
 }
 
@@ -761,40 +797,72 @@ bool skinny_supports(int type, int64_t K, int64_t M) {
     return gemm_supports(type, K, M) && (K / QKK + 7) / 8 <= SKINNY_MAX_SB_PER_WAVE;
 }
 
-template <class S, int NCT>
-void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
-    typedef SkinnyGeo<S, NCT> Geo;
-    // Cut K as many ways as keeps the whole grid resident in one round (about 15 waves per CU fit):
-    // every wave pays one pipeline fill, so few long waves when there are many row groups, many short
-    // ones when there are few.
-    const int64_t groups = (w.M + 15) / 16, nsb = w.K / QKK;
-    int waves = (int)((int64_t)num_cus * 15 / groups);
+// Cut K as many ways as keeps the whole grid resident in one round (about 15 waves per CU fit): every
+// wave pays one pipeline fill, so few long waves when there are many row groups, many short ones when
+// there are few.
+int skinny_waves(int64_t row_groups, int64_t nsb, int num_cus) {
+    int waves = (int)((int64_t)num_cus * 15 / row_groups);
     waves = waves >= 8 ? 8 : waves >= 6 ? 6 : waves >= 4 ? 4 : waves >= 3 ? 3 : waves >= 2 ? 2 : 1;
-    while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;             // at least two super-blocks per wave
+    while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;  // at least two super-blocks per wave
     while ((nsb + waves - 1) / waves > SKINNY_MAX_SB_PER_WAVE && waves < 8) waves = waves >= 4 ? waves + 2 : waves + 1;
+    return waves;
+}
+
+template <class S, int NCT, bool ID>
+void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, const SkinnyIds &si,
+                      int64_t row_groups, int num_cus, hipStream_t s) {
+    typedef SkinnyGeo<S, NCT> Geo;
+    const int waves = skinny_waves(row_groups, w.K / QKK, num_cus);
     const size_t lds = (size_t)waves * (Geo::WAVE_BYTES + Geo::PART_BYTES);
     // more than 64 KiB of dynamic LDS has to be allowed once per device
     static bool allowed[64] = {false};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_kernel<S, NCT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_kernel<S, NCT, ID>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny_kernel<S, NCT><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y);
+    skinny_kernel<S, NCT, ID><<<(unsigned)row_groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
 }
 
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
     if (!skinny_supports(w.type, w.K, w.M) || a.type != T_Q8_K || a.K != w.K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
     if (ncols < 1 || ncols > 16 || col0 < 0 || col0 + ncols > a.N) return hipErrorInvalidValue;
     if ((w.M + 15) / 16 > 0x7fffffff) return hipErrorInvalidValue;
+    const SkinnyIds none{};
+    const int64_t rg = (w.M + 15) / 16;
     if (w.type == T_Q4_K) {
-        if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8>(w, a, col0, ncols, y, num_cus, s);
-        else launch_skinny_as<Sk16Q4K, 16>(w, a, col0, ncols, y, num_cus, s);
+        if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
+        else launch_skinny_as<Sk16Q4K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     } else {
-        if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8>(w, a, col0, ncols, y, num_cus, s);
-        else launch_skinny_as<Sk16Q6K, 16>(w, a, col0, ncols, y, num_cus, s);
+        if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
+        else launch_skinny_as<Sk16Q6K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     }
+    return hipGetLastError();
+}
+
+bool skinny_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert) {
+    // from about two pairs per expert the experts' weights are worth sharing between pairs
+    return pairs >= 2 * (int64_t)n_expert && skinny_supports(type, K, M);
+}
+
+hipError_t launch_skinny_id(const DevWeight &w, int n_expert, const DevAct &a, const int *ids, int n_used, int n_tokens,
+                            int b_cols, float *y, int *groups, int num_cus, hipStream_t s) {
+    if (n_expert < 1 || w.M % n_expert || !skinny_supports(w.type, w.K, w.M / n_expert) || a.type != T_Q8_K ||
+        a.K != w.K || !a.sd8 || !a.sd16 || !ids || !y || !groups || n_used < 1 || n_tokens < 1 || b_cols < 1 ||
+        a.N != (int64_t)b_cols * n_tokens)
+        return hipErrorInvalidValue;
+    const int64_t pairs = (int64_t)n_used * n_tokens;
+    if (hipError_t e = launch_group_pairs(ids, (int)pairs, n_expert, 16, groups, s)) return e;
+    SkinnyIds si;
+    si.groups = groups; si.M = w.M / n_expert; si.n_used = n_used; si.b_cols = b_cols;
+    si.wgs_per_group = (int)((si.M + 15) / 16);
+    // every expert (and the bucket of bad ids) ends with at most one partly filled group
+    const int64_t max_groups = min(pairs, (int64_t)n_expert + 1 + pairs / 16);
+    const int64_t wgs = max_groups * si.wgs_per_group;
+    if (wgs > 0x7fffffff) return hipErrorInvalidValue;
+    if (w.type == T_Q4_K) launch_skinny_as<Sk16Q4K, 16, true>(w, a, 0, 16, y, si, wgs, num_cus, s);
+    else launch_skinny_as<Sk16Q6K, 16, true>(w, a, 0, 16, y, si, wgs, num_cus, s);
     return hipGetLastError();
 }
 

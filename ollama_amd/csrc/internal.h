@@ -66,4 +66,10 @@ bool skinny_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                          hipStream_t s);
 
+// Expert-indexed product on the matrix cores (K-quants): the pairs are bucketed by expert, 16 per group;
+// a needs the block-sum digit planes.  groups: device scratch of gemv_id_scratch_ints(pairs) ints.
+bool skinny_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);
+hipError_t launch_skinny_id(const DevWeight &w, int n_expert, const DevAct &a, const int *ids, int n_used, int n_tokens,
+                            int b_cols, float *y, int *groups, int num_cus, hipStream_t s);
+
 }  // namespace miqmm

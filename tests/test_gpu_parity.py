@@ -447,25 +447,43 @@ def test_mulmat_id_matches_oracle(ctx, t, tokens, n_used, b_cols):
     w.free()
 
 
-def test_mulmat_id_equals_mulmat_on_the_expert_alone(ctx):
-    """bit-identical to the plain product on one expert's slice, whatever group a pair lands in"""
-    rng = np.random.default_rng(7200)
-    k, m, n_expert, tokens, n_used = 2048, 96, 6, 24, 3
-    wb = _experts(Q4_K, n_expert, m, k, 7201)
-    w = ctx.upload(Q4_K, wb, k, n_expert * m)
+@pytest.mark.parametrize("t,tokens", [(Q4_K, 3), (Q8_0, 3), (Q8_0, 24), (Q4_0, 24)])
+def test_mulmat_id_equals_mulmat_on_the_expert_alone(ctx, t, tokens):
+    """the streaming kernels (decode: one pair per group; Q4_0 / Q8_0 batches: pairs bucketed by expert)
+    give bit for bit what the plain one-column product gives on that expert's slice, whatever group a
+    pair lands in"""
+    rng = np.random.default_rng(7200 + t + tokens)
+    k, m, n_expert, n_used = 2048, 96, 6, 3
+    wb = _experts(t, n_expert, m, k, 7201 + t)
+    w = ctx.upload(t, wb, k, n_expert * m)
     b = rng.standard_normal((tokens, 1, k), dtype=np.float32)
     ids = rng.integers(0, n_expert, (tokens, n_used)).astype(np.int32)
     got = ctx.mulmat_id(w, n_expert, b, ids)
     w3 = wb.reshape(n_expert, m, -1)
     for e in range(n_expert):
-        we = ctx.upload(Q4_K, w3[e], k, m)
+        we = ctx.upload(t, w3[e], k, m)
         for ti, i in np.argwhere(ids == e):
             assert np.array_equal(got[ti, i], ctx.mulmat(we, b[ti, 0])[0])  # the decode GEMV, one column
         we.free()
-    # the same pairs one token at a time (no bucketing) give the same bits
-    for ti in (0, 5, 23):
-        assert np.array_equal(ctx.mulmat_id(w, n_expert, b[ti:ti + 1], ids[ti:ti + 1])[0], got[ti])
     w.free()
+
+
+def test_mulmat_id_on_the_matrix_cores(ctx):
+    """K-quants from about two pairs per expert up: groups of 16 pairs through the MFMA kernel; ragged
+    expert height, experts that nobody picked, one expert picked by more than 16 pairs"""
+    rng = np.random.default_rng(7250)
+    for t, k, m, n_expert, tokens, n_used, b_cols in ((Q4_K, 1024, 72, 5, 40, 2, 1), (Q6_K, 512, 200, 9, 30, 4, 4),
+                                                      (Q4_K, 2048, 33, 3, 64, 2, 2)):
+        wb = _experts(t, n_expert, m, k, 7251 + t)
+        w = ctx.upload(t, wb, k, n_expert * m)
+        b = rng.standard_normal((tokens, b_cols, k), dtype=np.float32)
+        ids = rng.integers(0, n_expert - 1, (tokens, n_used)).astype(np.int32)  # the last expert stays idle
+        ids[: tokens // 2, 0] = 1                                                # a crowd on expert 1
+        got = ctx.mulmat_id(w, n_expert, b, ids)
+        assert npref.rel_err(got, oracle.mul_mat_id(t, wb, k, m, n_expert, b, ids)) < TOL
+        # a pair's result does not depend on the other pairs of the call: same call, order of tokens reversed
+        assert np.array_equal(ctx.mulmat_id(w, n_expert, b[::-1], ids[::-1])[::-1], got)
+        w.free()
 
 
 def test_mulmat_id_moe_decode_shape(ctx):
