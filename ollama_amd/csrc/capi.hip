@@ -408,17 +408,20 @@ bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
 // dy: device output [n][M].  Picks the kernel and queues it on the ctx's stream.
 int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path) {
     const int64_t K = w->dev.K, M = w->dev.M, n = a.N;
+    const bool blk32 = gemm_blk32_supports(w->dev.type, K, M);  // Q4_0 / Q8_0: their own MFMA kernel
     bool use_gemm;
     if (path == MI_QMM_PATH_GEMM) use_gemm = true;
     else if (path == MI_QMM_PATH_GEMV) use_gemm = false;
-    else use_gemm = n >= 32 && gemm_supports(w->dev.type, K, M);
-    if (use_gemm && !gemm_supports(w->dev.type, K, M))
+    else use_gemm = n >= 32 && (blk32 || gemm_supports(w->dev.type, K, M));
+    if (use_gemm && !blk32 && !gemm_supports(w->dev.type, K, M))
         return fail(MI_QMM_ERR_UNSUPPORTED, "the MFMA GEMM does not cover type %d with K=%lld M=%lld", w->dev.type,
                     (long long)K, (long long)M);
     if (!use_gemm && K > gemv_max_k(w->dev.type))
         return fail(MI_QMM_ERR_UNSUPPORTED, "K=%lld exceeds the GEMV limit %lld for type %d", (long long)K,
                     (long long)gemv_max_k(w->dev.type), w->dev.type);
-    if (use_gemm) {
+    if (use_gemm && blk32) {
+        HIP_TRY(launch_gemm_blk32(w->dev, a, dy, ctx->num_cus, ctx->stream));
+    } else if (use_gemm) {
         const size_t wsf = gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus);
         if (wsf) {
             int rc = reserve(&ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float), ctx->stream);

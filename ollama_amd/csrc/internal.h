@@ -66,6 +66,11 @@ bool skinny_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                          hipStream_t s);
 
+// int8-MFMA GEMM for the 32-element block formats (Q4_0, Q8_0 weights; Q8_0 activations), any N >= 1.
+// y[n*M + m].
+bool gemm_blk32_supports(int type, int64_t K, int64_t M);
+hipError_t launch_gemm_blk32(const DevWeight &w, const DevAct &a, float *y, int num_cus, hipStream_t s);
+
 // Expert-indexed product on the matrix cores (K-quants): the pairs are bucketed by expert, 16 per group;
 // a needs the block-sum digit planes.  groups: device scratch of gemv_id_scratch_ints(pairs) ints.
 bool skinny_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);

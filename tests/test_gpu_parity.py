@@ -395,20 +395,6 @@ def test_gemm_random_block_bytes(ctx, t):
     W.free()
 
 
-def test_gemm_unsupported_types_use_gemv_groups(ctx):
-    """Q4_0 / Q8_0 have no MFMA kernel: AUTO keeps large batches on the GEMV, forcing GEMM is an error"""
-    k, m, n = 1024, 64, 40
-    for t in (Q4_0, Q8_0):
-        w_raw = _weights(t, m, k, seed=t)
-        W = ctx.upload(t, w_raw, k, m)
-        x = np.random.default_rng(t).standard_normal((n, k), dtype=np.float32)
-        assert npref.rel_err(ctx.mulmat(W, x), oracle.mul_mat(t, w_raw, k, m, x, nthreads=8)) <= TOL
-        with pytest.raises(qmm.QmmError) as e:
-            ctx.mulmat(W, x, path=qmm.PATH_GEMM)
-        assert e.value.code == qmm.ERR_UNSUPPORTED
-        W.free()
-
-
 @pytest.mark.parametrize("name,t,m,k", [("q_proj", Q4_K, 4096, 4096), ("k_proj", Q4_K, 1024, 4096),
                                         ("ffn_gate", Q4_K, 14336, 4096), ("ffn_down", Q6_K, 4096, 14336)])
 def test_config5_prefill_layer_batch512(ctx, name, t, m, k):
@@ -560,3 +546,41 @@ def test_device_pointers_give_the_same_bits_as_host_arrays(ctx, t, n):
         d.free()
     w.free()
     w2.free()
+
+
+# ---- MFMA GEMM for the 32-element block formats -----------------------------------------------------
+@pytest.mark.parametrize("t", [Q4_0, Q8_0])
+@pytest.mark.parametrize("m,k,n", [(4096, 4096, 64), (1000, 1056, 70), (33, 32, 32), (257, 8192, 129), (64, 96, 1),
+                                   (2, 2048, 200)])
+def test_block32_gemm_matches_oracle(ctx, t, m, k, n):
+    """full tiles; ragged M (also not a multiple of 4), N and a K of 33 blocks; one block; K cut between
+    eight waves; one column and two rows through the forced GEMM path"""
+    rng = np.random.default_rng(7600 + t + m + n)
+    wb = _weights(t, m, k, 7601 + t + m)
+    w = ctx.upload(t, wb, k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(w, x, path=qmm.PATH_GEMM)
+    want = oracle.mul_mat(t, wb, k, m, x, nthreads=16)
+    assert npref.rel_err(got, want) < TOL
+    if n >= 32:
+        assert np.array_equal(got, ctx.mulmat(w, x))  # what the automatic choice runs from 32 columns up
+    w.free()
+
+
+def test_block32_gemm_exact_integer_case(ctx):
+    """weights and activations whose products and sums are exact in fp32: any misplaced operand byte,
+    nibble or scale shows as a wrong integer"""
+    k, m, n = 256, 96, 64
+    rng = np.random.default_rng(7700)
+    for t in (Q4_0, Q8_0):
+        lim = 7 if t == Q4_0 else 127
+        wi = rng.integers(-lim, lim + 1, (m, k)).astype(np.float32)
+        wi[:, ::32] = -8 if t == Q4_0 else 127  # pins every block's scale to exactly 1.0
+        xi = rng.integers(-127, 128, (n, k)).astype(np.float32)
+        xi[:, 1::32] = 127
+        wb = oracle.quantize(t, wi)
+        assert np.array_equal(oracle.dequantize(t, wb, k), wi)
+        w = ctx.upload(t, wb, k, m)
+        got = ctx.mulmat(w, xi, path=qmm.PATH_GEMM)
+        assert np.array_equal(got, (xi.astype(np.float64) @ wi.astype(np.float64).T).astype(np.float32))
+        w.free()
