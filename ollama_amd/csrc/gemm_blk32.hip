@@ -4,19 +4,19 @@
 //
 // Both sides carry an fp16 scale per 32 elements, so the integer sum is only homogeneous over one
 // block: one v_mfma_i32_32x32x32_i8 (K = 32) is exactly one block of a 32 x 32 output tile, and every
-// MFMA is followed by an fp32 step  y += float(I) * (d_w * d_x)  on its 16 accumulators -- 48 vector
-// instructions per MFMA, which is what bounds the kernel (one MFMA costs about 6 vector instructions
-// of issue time), not the matrix cores and not memory.  What is left to design is keeping that vector
-// work fed:
+// MFMA is followed by an fp32 step  y += float(I) * (d_w * d_x)  on its 16 accumulators -- at least 48
+// vector instructions per MFMA, which is what bounds the kernels (one MFMA costs about 6 vector
+// instructions of issue time), not the matrix cores and not memory.
 //   * A wave owns 32 weight rows x 64 activation columns and a run of blocks of K; the weights are the
-//     A operand (a lane supplies 16 consecutive K values of one row: one 16-byte load for Q8_0, the
-//     low or the high nibbles of the block's 16 bytes for Q4_0, minus 8, for Q4_0), shared by the
-//     two MFMAs of a block; the activations are the B operand straight from the Q8_0 quants plane.
-//   * Operands go global -> registers, one block ahead; waves are independent (no barriers in the
-//     loop).  The only LDS traffic is the transposition of the weight scales: a lane's 16 accumulators
-//     are 16 different weight rows, so each block's 32 scales go through a per-wave LDS line.
+//     A operand (a lane supplies 16 consecutive K values of one row: 16 bytes of a Q8_0 block, or the
+//     low / high nibbles of a Q4_0 block's 16 bytes minus 8), shared by the two MFMAs of a block; the
+//     activations are the B operand straight from the Q8_0 quants plane.
+//   * Waves are independent (no barriers in the loop).  A lane's 16 accumulators are 16 different
+//     weight rows, so the weight scales of a block reach the lanes through LDS.
 //   * The waves of a workgroup cut K between them and sum their tiles through LDS at the end, in a
-//     fixed order: enough waves to fill the machine even when M/32 x N/64 is small.
+//     fixed order.
+//   * gemm_blk32_dma_kernel (K a multiple of 64) stages all operands through per-wave LDS rings with
+//     direct-to-LDS loads; gemm_blk32_kernel (any K) loads them into registers one block ahead.
 #include <hip/hip_fp16.h>
 
 #include "internal.h"
@@ -171,58 +171,88 @@ __global__ __launch_bounds__(512, 2) void gemm_blk32_kernel(DevWeight w, DevAct 
     store_tile(acc, reinterpret_cast<float *>(smem) + waves * 64, waves, wave, lane, m0, n0, w.M, a.N, y);
 }
 
-// The same product four blocks (128 elements of K) at a time, for K a multiple of 128: the four
-// blocks of a chunk share a cache line per row, their scales are one 8-byte (weights) and one 16-byte
-// (activations) load, and the whole next chunk is in flight while the current one is multiplied --
-// four times the bytes in flight per wave and about half the load instructions of the block-wise loop.
+// The same product with the operands staged through LDS by direct-to-LDS loads, for K a multiple of
+// 64.  A register load in MFMA operand layout touches 32 rows with 16 bytes each -- 32 cache lines
+// per instruction, and the L1's line rate, not its bandwidth, bounds the kernels above.  Here
+// consecutive lanes copy consecutive 16-byte pieces of a row (four lanes per 64-byte run of two
+// blocks), the copies need no registers, and a wave keeps two stages of two blocks in flight in its
+// own LDS region: no barriers in the loop, each wave waits on its own memory counter (every wave
+// issues exactly NDMA copies per stage, so "at most NDMA outstanding" means the older stage landed).
+// Pieces are XOR-swizzled with row bits so that the operand reads spread over the banks.
+typedef __attribute__((address_space(3))) void lds_ptr_t;
+typedef const __attribute__((address_space(1))) void glb_ptr_t;
+
 template <bool Q4>
-struct Chunk {
-    v4i w[4];
-    v4i x[2][4];
-    float4 dx[2];
-    uint2 dw;  // four fp16 scales of weight row lane%32
+struct DmaGeo {
+    static constexpr int W_BYTES = Q4 ? 1024 : 2048;  // 32 rows x 2 blocks
+    static constexpr int W_INSTRS = W_BYTES / 1024;
+    static constexpr int X_BYTES = 4096;              // 64 columns x 2 blocks of quants
+    static constexpr int DW_OFF = W_BYTES + X_BYTES;  // 32 rows x 2 fp16
+    static constexpr int DX_OFF = DW_OFF + 256;       // 2 blocks x 64 floats
+    static constexpr int STAGE = DX_OFF + 512;
+    static constexpr int NDMA = W_INSTRS + 4 + 1 + 2;
+    static constexpr int WAVE_BYTES = (2 * STAGE > 8192 ? 2 * STAGE : 8192);  // the K-cut partials reuse the region
 };
 
 template <bool Q4>
-__device__ __forceinline__ void load_chunk(Chunk<Q4> &ch, const uint8_t *wq, const uint16_t *wd, const int8_t *const (&xq)[2],
-                                           const float *const (&xd)[2], int64_t blk, int half) {
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        if (Q4) ch.w[j] = *reinterpret_cast<const v4i *>(wq + (blk + j) * 16);
-        else ch.w[j] = *reinterpret_cast<const v4i *>(wq + (blk + j) * 32 + 16 * half);
-    }
-    ch.dw = *reinterpret_cast<const uint2 *>(wd + blk);
-#pragma unroll
-    for (int t = 0; t < 2; t++) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) ch.x[t][j] = *reinterpret_cast<const v4i *>(xq[t] + (blk + j) * 32 + 16 * half);
-        ch.dx[t] = *reinterpret_cast<const float4 *>(xd[t] + blk);
-    }
-}
-
-template <bool Q4>
-__global__ __launch_bounds__(512, 1) void gemm_blk32_chunk_kernel(DevWeight w, DevAct a, float *__restrict__ y, int tiles_m) {
-    extern __shared__ __align__(16) uint8_t smem[];  // per wave: 2 x 4 x 32 floats of weight scales; then the K-cut partials
+__global__ __launch_bounds__(512, 1) void gemm_blk32_dma_kernel(DevWeight w, DevAct a, float *__restrict__ y, int tiles_m) {
+    typedef DmaGeo<Q4> Geo;
+    extern __shared__ __align__(256) uint8_t smem[];  // waves x WAVE_BYTES
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int waves = blockDim.x >> 6;
     const int c = lane & 31, half = lane >> 5;
     const int tn = blockIdx.x / tiles_m, tm = blockIdx.x - tn * tiles_m;
     const int64_t m0 = (int64_t)tm * 32, n0 = (int64_t)tn * 64;
-    const int64_t nblk = w.K / QK, nch = nblk / 4;
-    const int64_t c0 = nch * wave / waves, c1 = nch * (wave + 1) / waves;  // this wave's chunks
+    const int64_t nblk = w.K / QK, nch = nblk / 2;
+    const int64_t c0 = nch * wave / waves, c1 = nch * (wave + 1) / waves;  // this wave's chunks of two blocks
+    uint8_t *wsm = smem + wave * Geo::WAVE_BYTES;
+    const int rows_left = (int)min((int64_t)32, w.M - m0), cols_left = (int)min((int64_t)64, (int64_t)a.N - n0);
 
-    const int64_t row = min(m0 + c, w.M - 1);
-    const uint8_t *wq = w.p0 + row * (Q4 ? nblk * 16 : w.K);
-    const uint16_t *wd = w.d + row * nblk;
-    const int8_t *xq[2];
-    const float *xd[2];
+    // ---- copy plan: per-lane offsets from uniform bases; rows / columns past the edge copy the last one
+    unsigned woff[Geo::W_INSTRS], xoff[4];
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        const int64_t col = min(n0 + 32 * t + c, (int64_t)a.N - 1);
-        xq[t] = a.qs + col * a.K;
-        xd[t] = a.d + col * nblk;
+    for (int i = 0; i < Geo::W_INSTRS; i++) {
+        if (Q4) {
+            const int r = lane >> 1, pos = lane & 1, piece = pos ^ ((r >> 3) & 1);  // piece = block of the chunk
+            woff[i] = (unsigned)min(r, rows_left - 1) * (unsigned)(nblk * 16) + 16u * piece;
+        } else {
+            const int s_ = 64 * i + lane, r = s_ >> 2, pos = s_ & 3, piece = pos ^ ((r >> 2) & 3);  // piece = 2*block + half
+            woff[i] = (unsigned)min(r, rows_left - 1) * (unsigned)w.K + 16u * piece;
+        }
     }
-    float *dsm = reinterpret_cast<float *>(smem) + wave * 256;  // [2][4][32]
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int s_ = 64 * i + lane, col = s_ >> 2, pos = s_ & 3, piece = pos ^ ((col >> 2) & 3);
+        xoff[i] = (unsigned)min(col, cols_left - 1) * (unsigned)a.K + 16u * piece;
+    }
+    const unsigned dwoff = (unsigned)min(c, rows_left - 1) * (unsigned)nblk * 2u;      // bytes into the fp16 plane
+    const unsigned dxoff = (unsigned)min(lane, cols_left - 1) * (unsigned)nblk * 4u;  // bytes into the f32 plane
+    const uint8_t *wbase = w.p0 + m0 * (Q4 ? nblk * 16 : w.K);
+    const uint8_t *xbase = reinterpret_cast<const uint8_t *>(a.qs) + n0 * a.K;
+    const uint8_t *dwbase = reinterpret_cast<const uint8_t *>(w.d + m0 * nblk);
+    const uint8_t *dxbase = reinterpret_cast<const uint8_t *>(a.d + n0 * nblk);
+
+    auto stage_copy = [&](uint8_t *st, int64_t ch) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < Geo::W_INSTRS; i++) {
+            const uint8_t *gp = wbase + ch * (Q4 ? 32 : 64) + woff[i];
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * i), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint8_t *gp = xbase + ch * 64 + xoff[i];
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::W_BYTES + 1024 * i), 16, 0, 0);
+        }
+        {
+            const uint8_t *gp = dwbase + ch * 4 + dwoff;
+            if (lane < 32) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DW_OFF), 4, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint8_t *gp = dxbase + (ch * 2 + j) * 4 + dxoff;
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DX_OFF + 256 * j), 4, 0, 0);
+        }
+    };
 
     float acc[2][16];
 #pragma unroll
@@ -231,42 +261,73 @@ __global__ __launch_bounds__(512, 1) void gemm_blk32_chunk_kernel(DevWeight w, D
         for (int v = 0; v < 16; v++) acc[t][v] = 0.f;
 
     if (c0 < c1) {
-        Chunk<Q4> cur, nxt;
-        load_chunk<Q4>(cur, wq, wd, xq, xd, c0 * 4, half);
+        stage_copy(wsm, c0);
+        stage_copy(wsm + Geo::STAGE, min(c0 + 1, c1 - 1));
 #pragma unroll 1
         for (int64_t ch = c0; ch < c1; ch++) {
-            float *lines = dsm + ((ch - c0) & 1) * 128;
-            if (half == 0) {
-                lines[c] = h2f(cur.dw.x & 0xffff);
-                lines[32 + c] = h2f(cur.dw.x >> 16);
-                lines[64 + c] = h2f(cur.dw.y & 0xffff);
-                lines[96 + c] = h2f(cur.dw.y >> 16);
-            }
-            load_chunk<Q4>(nxt, wq, wd, xq, xd, min(ch + 1, c1 - 1) * 4, half);
-            const float dx0[4] = {cur.dx[0].x, cur.dx[0].y, cur.dx[0].z, cur.dx[0].w};
-            const float dx1[4] = {cur.dx[1].x, cur.dx[1].y, cur.dx[1].z, cur.dx[1].w};
+            uint8_t *st = wsm + ((ch - c0) & 1) * Geo::STAGE;
+            __builtin_amdgcn_s_waitcnt((Geo::NDMA & 15) | (7 << 4) | (15 << 8) | ((Geo::NDMA >> 4) << 14));
+            v4i aw[2], bx[2][2];
+            uint4 dwq[4];
+            float dxv[2][2];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const v4i aop = Q4 ? unpack_q4_0(cur.w[j], half) : cur.w[j];
+            for (int j = 0; j < 2; j++) {
+                if (Q4) aw[j] = *reinterpret_cast<const v4i *>(st + c * 32 + 16 * (j ^ ((c >> 3) & 1)));
+                else aw[j] = *reinterpret_cast<const v4i *>(st + c * 64 + 16 * ((2 * j + half) ^ ((c >> 2) & 3)));
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const int col = 32 * t + c;
+                    bx[t][j] = *reinterpret_cast<const v4i *>(st + Geo::W_BYTES + col * 64 + 16 * ((2 * j + half) ^ ((col >> 2) & 3)));
+                    dxv[t][j] = *reinterpret_cast<const float *>(st + Geo::DX_OFF + 256 * j + 4 * col);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) dwq[q] = *reinterpret_cast<const uint4 *>(st + Geo::DW_OFF + 4 * (8 * q + 4 * half));
+            // operands are in registers: the stage can take the copies of chunk ch + 2
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            stage_copy(st, min(ch + 2, c1 - 1));
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const v4i aop = Q4 ? unpack_q4_0(aw[j], half) : aw[j];
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                const v16i i0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, cur.x[0][j], zero, 0, 0, 0);
-                const v16i i1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, cur.x[1][j], zero, 0, 0, 0);
-                float dwv[16];
+                const v16i i0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bx[0][j], zero, 0, 0, 0);
+                const v16i i1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bx[1][j], zero, 0, 0, 0);
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const float4 f = *reinterpret_cast<const float4 *>(lines + 32 * j + 8 * q + 4 * half);
-                    dwv[4 * q] = f.x; dwv[4 * q + 1] = f.y; dwv[4 * q + 2] = f.z; dwv[4 * q + 3] = f.w;
-                }
+                    const unsigned pr[4] = {dwq[q].x, dwq[q].y, dwq[q].z, dwq[q].w};  // rows 8q + 4*half + i: (block 0, block 1) fp16
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    acc[0][v] = __builtin_fmaf((float)i0[v], dwv[v] * dx0[j], acc[0][v]);
-                    acc[1][v] = __builtin_fmaf((float)i1[v], dwv[v] * dx1[j], acc[1][v]);
+                    for (int i = 0; i < 4; i++) {
+                        const float dwf = h2f(j ? pr[i] >> 16 : pr[i] & 0xffff);
+                        const int v = 4 * q + i;
+                        acc[0][v] = __builtin_fmaf((float)i0[v], dwf * dxv[0][j], acc[0][v]);
+                        acc[1][v] = __builtin_fmaf((float)i1[v], dwf * dxv[1][j], acc[1][v]);
+                    }
                 }
             }
-            cur = nxt;
         }
+        __builtin_amdgcn_s_waitcnt(0);  // the redundant copies of the last iterations must land before the region is reused
     }
-    store_tile(acc, reinterpret_cast<float *>(smem) + waves * 256, waves, wave, lane, m0, n0, w.M, a.N, y);
+    // K-cut partials: wave k > 0 parks its tile in its own (now idle) stage region
+    float *mine = reinterpret_cast<float *>(wsm);
+    if (waves > 1) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (wave > 0) mine[(t * 16 + v) * 64 + lane] = acc[t][v];
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float s_ = acc[t][v];
+                for (int k = 1; k < waves; k++)
+                    s_ += reinterpret_cast<const float *>(smem + k * Geo::WAVE_BYTES)[(t * 16 + v) * 64 + lane];
+                acc[t][v] = s_;
+            }
+    }
+    store_tile(acc, nullptr, 1, 0, lane, m0, n0, w.M, a.N, y);
 }
 
 }  // namespace
@@ -279,22 +340,30 @@ hipError_t launch_gemm_blk32(const DevWeight &w, const DevAct &a, float *y, int 
     if (!gemm_blk32_supports(w.type, w.K, w.M) || a.type != T_Q8_0 || a.K != w.K || a.N < 1 || !y) return hipErrorInvalidValue;
     const int64_t tiles_m = (w.M + 31) / 32, tiles_n = ((int64_t)a.N + 63) / 64, tiles = tiles_m * tiles_n;
     if (tiles > 0x7fffffff) return hipErrorInvalidValue;
-    // waves per workgroup = cuts of K: about four waves per SIMD over the whole grid, at least eight
-    // blocks per wave
-    // waves per workgroup = cuts of K: enough waves over the whole grid to keep every SIMD busy, at
-    // least eight blocks per wave
-    const int64_t nblk = w.K / QK;
-    const bool chunked = w.K % 128 == 0;
-    const int64_t want = ((int64_t)num_cus * (chunked ? 12 : 16) + tiles - 1) / tiles;  // 3 / 4 waves fit a SIMD
+    // Waves per workgroup = cuts of K.  The kernels are bound by the vector ALU and run best with about
+    // one wave per SIMD over the whole grid (measured: more waves only add K-cut sums); at least eight
+    // blocks per wave.
+    const int64_t nblk = w.K / QK, want = ((int64_t)num_cus * 4 + tiles - 1) / tiles;
     int waves = (int)(want < 1 ? 1 : want > 8 ? 8 : want);
     while (waves > 1 && nblk / waves < 8) waves--;
-    const size_t part = (size_t)(waves - 1) * 2 * 16 * 64 * sizeof(float);  // <= 56 KiB
-    if (chunked) {
-        const size_t lds = (size_t)waves * 256 * sizeof(float) + part;
-        if (w.type == T_Q4_0) gemm_blk32_chunk_kernel<true><<<(unsigned)tiles, 64 * waves, lds, s>>>(w, a, y, (int)tiles_m);
-        else gemm_blk32_chunk_kernel<false><<<(unsigned)tiles, 64 * waves, lds, s>>>(w, a, y, (int)tiles_m);
+    if (w.K % 64 == 0 && (uint64_t)w.K * 64 < (1ull << 31)) {
+        const size_t lds = (size_t)waves * (w.type == T_Q4_0 ? DmaGeo<true>::WAVE_BYTES : DmaGeo<false>::WAVE_BYTES);
+        static bool allowed_dev[64] = {false};  // more than 64 KiB of dynamic LDS has to be allowed once per device
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        bool &allowed = allowed_dev[dev >= 0 && dev < 64 ? dev : 0];
+        if (!allowed) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_blk32_dma_kernel<true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_blk32_dma_kernel<false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            allowed = true;
+        }
+        if (w.type == T_Q4_0) gemm_blk32_dma_kernel<true><<<(unsigned)tiles, 64 * waves, lds, s>>>(w, a, y, (int)tiles_m);
+        else gemm_blk32_dma_kernel<false><<<(unsigned)tiles, 64 * waves, lds, s>>>(w, a, y, (int)tiles_m);
     } else {
-        const size_t lds = (size_t)waves * 64 * sizeof(float) + part;
+        // K an odd number of blocks: operands by register loads, one block ahead
+        const size_t lds = (size_t)waves * 64 * sizeof(float) + (size_t)(waves - 1) * 2 * 16 * 64 * sizeof(float);  // <= 58 KiB
         if (w.type == T_Q4_0) gemm_blk32_kernel<true><<<(unsigned)tiles, 64 * waves, lds, s>>>(w, a, y, (int)tiles_m);
         else gemm_blk32_kernel<false><<<(unsigned)tiles, 64 * waves, lds, s>>>(w, a, y, (int)tiles_m);
     }
