@@ -86,6 +86,15 @@ int mi_qmm_set_stream(mi_qmm_ctx *ctx, void *hip_stream);
 /* block until everything queued on the ctx's stream has finished */
 int mi_qmm_sync(mi_qmm_ctx *ctx);
 
+/* Page-locked host memory for x / y buffers of MI_QMM_HOST calls: the copies to and from the device
+ * then run at full PCIe rate and without a staging copy inside the driver.  A cgo caller keeps Go
+ * pointers out of C this way too (the buffer is C memory; cf. the static trampolines of
+ * /root/reference/discover/native_probe_linux.go:26-54).  Plain pointers: any entry point accepts
+ * them wherever it accepts host memory.  NULL (and an error message) when the allocation fails.
+ * mi_qmm_host_free does not use its ctx argument (it may be NULL or already destroyed). */
+void *mi_qmm_host_alloc(mi_qmm_ctx *ctx, size_t bytes);
+void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
+
 /* ---- weights: replaces Backend.Load + Backend.Get(name), /root/reference/ml/backend.go:20, 26,
  *      fed with the tensor bytes fs/ggml hands out (/root/reference/fs/ggml/gguf.go:281-308;
  *      fs/gguf/gguf.go:388-430): M rows of K elements in GGUF block layout, rows contiguous.

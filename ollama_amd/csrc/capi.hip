@@ -246,6 +246,21 @@ int mi_qmm_sync(mi_qmm_ctx *ctx) {
     return MI_QMM_OK;
 }
 
+void *mi_qmm_host_alloc(mi_qmm_ctx *ctx, size_t bytes) {
+    if (check_ctx(ctx)) return nullptr;
+    void *p = nullptr;
+    hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        fail(MI_QMM_ERR_NOMEM, "hipHostMalloc(%zu): %s", bytes, hipGetErrorString(e));
+        return nullptr;
+    }
+    return p;
+}
+
+void mi_qmm_host_free(mi_qmm_ctx *, void *p) {
+    if (p) (void)hipHostFree(p);  // page-locked memory is not tied to the current device: the ctx may be gone already
+}
+
 int mi_qmm_device_info(mi_qmm_ctx *ctx, int *compute_units, int *clock_mhz, char *name, int name_len) {
     if (!ctx) return fail(MI_QMM_ERR_INVALID, "ctx is NULL");
     if (compute_units) *compute_units = ctx->num_cus;

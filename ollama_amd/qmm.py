@@ -5,6 +5,7 @@ Fails loudly when the library has not been built: nothing here computes on the C
 from __future__ import annotations
 
 import ctypes
+import weakref
 import os
 import subprocess
 
@@ -21,7 +22,7 @@ OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, 
 
 EXPORTS = [
     "mi_qmm_block_size", "mi_qmm_type_size", "mi_qmm_row_size", "mi_qmm_vec_dot_type",
-    "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync",
+    "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync", "mi_qmm_host_alloc", "mi_qmm_host_free",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id",
@@ -84,6 +85,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_q8_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_multi.restype = ci
     L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
+    L.mi_qmm_host_alloc.restype = vp; L.mi_qmm_host_alloc.argtypes = [vp, ctypes.c_size_t]
+    L.mi_qmm_host_free.restype = None; L.mi_qmm_host_free.argtypes = [vp, vp]
     L.mi_qmm_mulmat_id.restype = ci
     L.mi_qmm_mulmat_id.argtypes = [vp, vp, ci, vp, ci, vp, ci, i64, vp, ci]
     P = ctypes.POINTER
@@ -227,6 +230,18 @@ class Context:
 
     def sync(self):
         _check(lib().mi_qmm_sync(self._h))
+
+    def host_array(self, shape, dtype=np.float32) -> np.ndarray:
+        """a numpy array over page-locked host memory (freed when the array and its views are gone)"""
+        n = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
+        p = lib().mi_qmm_host_alloc(self._h, n)
+        if not p:
+            raise QmmError(ERR_NOMEM, last_error())
+        buf = (ctypes.c_uint8 * max(n, 1)).from_address(p)
+        arr = np.frombuffer(buf, dtype=dtype, count=n // np.dtype(dtype).itemsize).reshape(shape)
+        h = self._h
+        weakref.finalize(buf, lambda: lib().mi_qmm_host_free(h, p))
+        return arr
 
     def upload(self, ggml_type: int, gguf_bytes, k: int, m: int, location: int = HOST) -> Weight:
         if isinstance(gguf_bytes, np.ndarray):

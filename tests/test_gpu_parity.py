@@ -584,3 +584,19 @@ def test_block32_gemm_exact_integer_case(ctx):
         got = ctx.mulmat(w, xi, path=qmm.PATH_GEMM)
         assert np.array_equal(got, (xi.astype(np.float64) @ wi.astype(np.float64).T).astype(np.float32))
         w.free()
+
+
+def test_page_locked_host_buffers(ctx):
+    """x and y in memory from mi_qmm_host_alloc behave like any other host memory"""
+    rng = np.random.default_rng(7800)
+    k, m, n = 1024, 256, 3
+    wb = _weights(Q4_K, m, k, 7801)
+    w = ctx.upload(Q4_K, wb, k, m)
+    x = ctx.host_array((n, k))
+    x[:] = rng.standard_normal((n, k), dtype=np.float32)
+    y = ctx.host_array((n, m))
+    rc = qmm.lib().mi_qmm_mulmat(ctx._h, w._h, ctypes.c_void_p(x.ctypes.data), n, ctypes.c_void_p(y.ctypes.data), qmm.HOST)
+    assert rc == 0
+    assert np.array_equal(y, ctx.mulmat(w, np.array(x)))
+    assert ctx.host_array((0, 4)).shape == (0, 4)
+    w.free()
