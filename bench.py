@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
 
-Q4_K, Q6_K, Q8_K = 12, 14, 15
+Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 2, 8, 12, 14, 15
 GATE_UP_HBM_TRAFFIC_BYTES = 66386790  # measured, see the roofline block below
 FFN_K, FFN_M = 4096, 14336
 
@@ -48,6 +48,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32, help="distinct FFN weight sets in the rotating pool")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the batch-512 prefill GEMM section")
+    ap.add_argument("--no-other", action="store_true",
+                    help="skip the short timings of the other BASELINE configurations (Q4_0 / Q8_0 GEMV, Q6_K head) "
+                         "and of the expert-indexed and Q4_0 GEMM paths")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic, for scaling rocprofv3 HBM counters)")
     args = ap.parse_args()
@@ -157,7 +160,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_thin_kernel<PolQ4K, 1, true, true> (gate+up in one launch, 28672 rows x 4096)",
+            "kernel": "gemv_thin_kernel<PolQ4K, 1, true, true, 1> (gate+up in one launch, 28672 rows x 4096)",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -234,6 +237,51 @@ def main() -> int:
         for row in gw:
             for wt in row:
                 wt.free()
+
+    # ---- the other configurations, one short timing each: f32 activations in HBM, quantization included
+    if not args.no_other:
+        def time_mulmat(t, m, k, n, copies, path=qmm.PATH_AUTO):
+            rows = min(m, 2048)
+            raw = np.tile(synth.weights(t, rows, k, seed=1100 + t), ((m + rows - 1) // rows, 1))[:m]
+            ws = [ctx.upload(t, np.roll(raw, 13 * c, axis=0), k, m) for c in range(copies)]
+            xs = torch.randn(n, k, generator=g, dtype=torch.float32).to(dev)
+            yo = torch.empty(n, m, dtype=torch.float32, device=dev)
+            fn = lambda: [ctx.mulmat_device(wt, xs.data_ptr(), n, yo.data_ptr(), path) for wt in ws]
+            fn()
+            reps = max(2, 200 // copies)
+            tm = timed(fn, reps) / (reps * copies)
+            for wt in ws:
+                wt.free()
+            return tm, raw.size
+
+        other = {}
+        for label, t, m, k, ns, copies in (("Q4_0 GEMV 4096x4096", Q4_0, 4096, 4096, (1,), 40),
+                                           ("Q8_0 skinny 4096x4096", Q8_0, 4096, 4096, (1, 2, 4, 8), 40),
+                                           ("Q6_K head 128256x4096", Q6_K, 128256, 4096, (1, 8), 3)):
+            for n in ns:
+                tm, wb = time_mulmat(t, m, k, n, copies)
+                gbs = alg_bytes(wb, k, m, n) / tm / 1e9
+                other[f"{label} B={n}"] = {"us": round(tm * 1e6, 2), "GB/s": round(gbs, 1),
+                                           "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        for label, t in (("Q4_0", Q4_0), ("Q8_0", Q8_0)):
+            tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
+            other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TOPS": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
+        # expert-indexed product: 128 experts of 768x2048 (Q4_K), 8 used per token
+        n_exp, n_used, em, ek = 128, 8, 768, 2048
+        raw = np.tile(synth.weights(Q4_K, 2048, ek, seed=1201), (n_exp * em // 2048, 1))
+        stacks = [ctx.upload(Q4_K, np.roll(raw, 13 * c, axis=0), ek, n_exp * em) for c in range(6)]
+        for toks in (1, 8, 512):
+            xe = torch.randn(toks, 1, ek, generator=g, dtype=torch.float32).to(dev)
+            ids = torch.stack([torch.randperm(n_exp, generator=g)[:n_used] for _ in range(toks)]).to(torch.int32).to(dev)
+            ye = torch.empty(toks, n_used, em, dtype=torch.float32, device=dev)
+            fn = lambda: [ctx.mulmat_id_device(st, n_exp, xe.data_ptr(), 1, ids.data_ptr(), n_used, toks, ye.data_ptr())
+                          for st in stacks]
+            fn()
+            tm = timed(fn, 10) / (10 * len(stacks))
+            other[f"MulmatID Q4_K 128x(768x2048) top-8 tokens={toks}"] = {"us": round(tm * 1e6, 2)}
+        for st in stacks:
+            st.free()
+        out["other_configs"] = other
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)

@@ -9,6 +9,8 @@
 
 #include "../../include/mi_qmm.h"
 #include "gguf_file.h"
+#include <vector>
+
 #include "internal.h"
 
 using namespace miqmm;
@@ -537,46 +539,76 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
                         (long long)ws[i]->dev.K, (long long)ws[0]->dev.K);
         same_type = same_type && ws[i]->dev.type == ws[0]->dev.type;
     }
+    int rc = check_product_args(ctx, ws[0], location, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    for (int i = 0; i < count; i++)
+        if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
+    if (n == 0) return MI_QMM_OK;
+    if (!x) return fail(MI_QMM_ERR_INVALID, "x is NULL");
+    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
     const int64_t K = ws[0]->dev.K;
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i]->dev.M;
-    bool skinny = false;
-    for (int i = 0; i < count; i++) skinny = skinny || wants_skinny(ws[i]->dev.type, K, ws[i]->dev.M, n);
-    if (!same_type || skinny || count > gemv_max_multi() || n > 8 || n == 0 ||
-        !gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)) {
-        for (int i = 0; i < count; i++) {
-            int rc = mi_qmm_mulmat_path(ctx, ws[i], x, n, ys[i], location, MI_QMM_PATH_AUTO);
-            if (rc) return rc;
-        }
-        return MI_QMM_OK;
-    }
-    int rc = check_product_args(ctx, ws[0], location, MI_QMM_PATH_AUTO);
-    if (rc) return rc;
-    if (!x) return fail(MI_QMM_ERR_INVALID, "x is NULL");
-    DevWeight dw[8];
-    for (int i = 0; i < count; i++) {
-        if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
-        dw[i] = ws[i]->dev;
-    }
+
+    // x and the outputs on the device
     const size_t xbytes = (size_t)(n * K) * 4;
     const float *dx = x;
-    float *dys[8];
-    size_t offs[9];
-    offs[0] = align_up(xbytes, 256);
-    for (int i = 0; i < count; i++) {
-        dys[i] = ys[i];
-        offs[i + 1] = offs[i] + align_up((size_t)(n * dw[i].M) * 4, 256);
-    }
+    std::vector<float *> dys(ys, ys + count);
     if (location == MI_QMM_HOST) {
+        std::vector<size_t> offs(count + 1);
+        offs[0] = align_up(xbytes, 256);
+        for (int i = 0; i < count; i++) offs[i + 1] = offs[i] + align_up((size_t)(n * ws[i]->dev.M) * 4, 256);
         if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
         dx = (const float *)ctx->io_buf;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    HIP_TRY(launch_gemv_f32_multi(dw, dys, count, dx, (int)n, ctx->num_cus, ctx->stream));
+
+    bool skinny = false;
+    for (int i = 0; i < count; i++) skinny = skinny || wants_skinny(ws[i]->dev.type, K, ws[i]->dev.M, n);
+    if (same_type && !skinny && count <= gemv_max_multi() && n <= 8 &&
+        gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)) {
+        // decode: one launch over the concatenated rows, the kernel quantizes x in its prologue
+        DevWeight dw[8];
+        for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
+        HIP_TRY(launch_gemv_f32_multi(dw, dys.data(), count, dx, (int)n, ctx->num_cus, ctx->stream));
+    } else {
+        // x is quantized once per activation format (Q8_0 / Q8_K) in use; weights of one type then share
+        // GEMV launches four at a time, everything else goes out one product at a time
+        for (int q8 : {(int)T_Q8_0, (int)T_Q8_K}) {
+            std::vector<int> idx;
+            for (int i = 0; i < count; i++)
+                if (mi_qmm_vec_dot_type(ws[i]->dev.type) == q8) idx.push_back(i);
+            if (idx.empty()) continue;
+            const ActPlanes probe = plan_act(nullptr, q8, K, n);
+            if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+            const ActPlanes p = plan_act(ctx->act_buf, q8, K, n);
+            HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+            DevAct a;
+            a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
+            size_t j = 0;
+            while (j < idx.size()) {
+                const mi_qmm_weight *w0 = ws[idx[j]];
+                size_t e = j + 1;
+                if (n <= 8 && !wants_skinny(w0->dev.type, K, w0->dev.M, n) && K <= gemv_max_k(w0->dev.type))
+                    while (e < idx.size() && e - j < (size_t)gemv_max_multi() && ws[idx[e]]->dev.type == w0->dev.type &&
+                           !wants_skinny(w0->dev.type, K, ws[idx[e]]->dev.M, n))
+                        e++;
+                if (e - j > 1) {
+                    DevWeight dw[8];
+                    float *out[8];
+                    for (size_t t = j; t < e; t++) { dw[t - j] = ws[idx[t]]->dev; out[t - j] = dys[idx[t]]; }
+                    HIP_TRY(launch_gemv_multi(dw, out, (int)(e - j), a, 0, (int)n, ctx->num_cus, ctx->stream));
+                } else if ((rc = run_product(ctx, w0, a, dys[idx[j]], MI_QMM_PATH_AUTO))) {
+                    return rc;
+                }
+                j = e;
+            }
+        }
+    }
     if (location == MI_QMM_HOST) {
         for (int i = 0; i < count; i++)
-            HIP_TRY(hipMemcpyAsync(ys[i], dys[i], (size_t)(n * dw[i].M) * 4, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(hipMemcpyAsync(ys[i], dys[i], (size_t)(n * ws[i]->dev.M) * 4, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
     }
     return MI_QMM_OK;

@@ -931,8 +931,15 @@ hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols,
 
 bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
     // Beyond 64 Ki rows (an output head) the redundant per-workgroup quantization costs more than the
-    // launch it saves.
+    // launch it saves.  The same goes for several columns (every workgroup quantizes all of them):
+    // measured against quantize-then-multiply, one column always wins, two (K-quants) or three
+    // (Q4_0 / Q8_0) columns only on small launches, where the saved launch is a larger share.
     if (ncols < 1 || ncols > MAXC || K < 1 || total_m < 1 || total_m > 65536) return false;
+    if (ncols > 1) {
+        const bool kquant = type == T_Q4_K || type == T_Q6_K;
+        const int64_t approx_bytes = total_m * K * (type == T_Q8_0 ? 34 : type == T_Q6_K ? 26 : 18) / 32;
+        if (ncols > (kquant ? 2 : 3) || approx_bytes > (20 << 20)) return false;
+    }
     Plan p;
     switch (type) {
     case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, ncols, true, p);
