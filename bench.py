@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
 
 Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 2, 8, 12, 14, 15
-GATE_UP_HBM_TRAFFIC_BYTES = 66386790  # measured, see the roofline block below
+GATE_UP_HBM_TRAFFIC_BYTES = 66376537  # measured, see the roofline block below
 FFN_K, FFN_M = 4096, 14336
 
 
@@ -166,7 +166,7 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             # HBM bytes per launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE x 2.000 and
-            # WRITE_SIZE x 1.000, factors from a 1 GiB copy): 32,359.41 KiB x 2 + 112.03 KiB
+            # WRITE_SIZE x 1.000, factors from a 1 GiB copy): 32,354.41 KiB x 2 + 112.02 KiB
             "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
             "bytes_per_launch": int(bytes_per_launch),
