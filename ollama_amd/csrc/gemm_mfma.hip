@@ -394,27 +394,35 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
 // ---------------------------------------------------------------------------------------------
 // Skinny product on the matrix cores: 3..16 activation columns (speculative / small-batch decode).
 // The streaming GEMV multiplies every column with its own pass of v_dot4 (about 450 vector
-// instructions per row and lane at eight columns) and is vector-ALU bound from three columns up.  Here
-// the columns ride along as rows of the MFMA's A operand; the weights are expanded to the same two
-// digit planes as in the GEMM and the fp32 epilogue runs on four accumulators per lane and super-block.
+// instructions per row and lane at eight columns) and is vector-ALU bound from three columns up.
+//
+// v_mfma_i32_16x16x64_i8: the B operand is the weights (lane l: weight row l%16, the 16 K values
+// 16*(l/16).. of a 64-wide step -- one K group), unscaled.  A sub-block of the K-quants is one
+// (Q6_K) or two (Q4_K) K groups, so the 16 rows of the A operand are spent on columns x sub-blocks:
+// row r carries one activation column restricted to the K groups of one sub-block and zeros elsewhere
+// (lanes that hold zeros read a zero slot of the stage).  An MFMA then leaves every lane with the
+// partial dot products of its column(s) with each sub-block of the step in its four accumulators,
+// the sub-block scale is applied there by v_mad_i32_i24, and the min / -32 terms come from one more
+// MFMA per column set (block-sum digits x mins or scales).
 //
 // HBM-bound like the GEMV, so the shape is the GEMV's: many small independent waves.  A workgroup owns
-// 16 weight rows, its four waves a quarter of K each (combined through LDS at the very end -- the only
+// 16 weight rows, its waves a run of K each (combined through LDS at the very end -- the only
 // barrier).  Every wave streams its own packed weights and activation operands through its own two LDS
 // stages with direct-to-LDS loads (coalesced: consecutive lanes fetch consecutive 16-byte pieces of a
 // row; loading 16-byte pieces of 16 different rows per instruction straight into registers touched 16
-// cache lines per instruction and ran at half the speed), waits on its own memory counter, and reads
-// its operands back with conflict-free LDS reads.
-// v_mfma_i32_16x16x64_i8: lane l holds weight row l%16 and the 16 K values 16*(l/16).. of a 64-wide
-// step as B operand, activation column l%16 (columns >= nc are zeroed) as A operand, and the outputs
-// (column 4*(l/16) + v, row l%16), v = 0..3.
+// cache lines per instruction and ran at half the speed) and waits on its own memory counter.
 // ---------------------------------------------------------------------------------------------
 typedef int v4acc __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ int mad24(int a, int b, int c) { return __mul24(a, b) + c; }  // v_mad_i32_i24
 __device__ __forceinline__ v4acc mfma16(v4i a, v4i b, v4acc c) { return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0); }
 
+// One super-block of a lane's weight row as MFMA operands: the quants of the four 64-wide K steps as they
+// are (no scale folded in), the sub-block scales for the vector ALU, the operand of the block-sum MFMA.
+template <int NSC>
 struct B16 {
-    v4i hi[4], lo[4];  // four 64-wide K steps, two digit planes
-    v4i min_lo, min_hi;
+    v4i q[4];
+    int sc[NSC];  // sub-block scales of the lane's weight row
+    v4i bsum;     // B operand of the block-sum MFMA: mins (Q4_K) / scales (Q6_K) in K group 0, zeros elsewhere
     float d, dmin;
 };
 
@@ -443,35 +451,53 @@ struct Sk16Q4K {
 #pragma unroll
         for (int t = 0; t < 4; t++) raw.q[t] = ld16(p + 16 + 32 * t + 16 * (g & 1));
     }
-    static __device__ __forceinline__ void expand(const Raw &raw, int g, unsigned, B16 &b) {
+    // A sub-block is 32 elements = two K groups of a step, so the 16 rows of the A operand are 8 columns x
+    // the two sub-blocks of the step: row r is column r>>1 restricted to sub-block r&1 (K groups 2(r&1),
+    // 2(r&1)+1; the other two are zero).  The outputs of lane l are then rows 4(l>>4) + v = columns
+    // 2(l>>4), 2(l>>4)+1 x sub-blocks 2t, 2t+1: four partial dot products that take their 6-bit scale
+    // on the vector ALU.
+    static constexpr int SET_COLS = 8, LANE_COLS = 2, NSC = 8;
+    typedef B16<NSC> Ops;
+    static __device__ __forceinline__ int a_col(int r) { return r >> 1; }
+    static __device__ __forceinline__ bool a_on(int r, int g) { return (g >> 1) == (r & 1); }
+    static __device__ __forceinline__ int lane_col(int lg, int u) { return 2 * lg + u; }
+    static __device__ __forceinline__ void expand(const Raw &raw, int g, unsigned, Ops &b) {
         const uint4 hdr = raw.hdr;
         b.d = h2f(hdr.x & 0xffff);
         b.dmin = h2f(hdr.x >> 16);
         const unsigned sc03 = hdr.y & 0x3f3f3f3fu, sc47 = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
         const unsigned mn03 = hdr.z & 0x3f3f3f3fu, mn47 = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+#pragma unroll
+        for (int j = 0; j < 8; j++) b.sc[j] = (int)(((j < 4 ? sc03 : sc47) >> (8 * (j & 3))) & 0xff);
         const int hiN = g >> 1;  // 0: low nibbles (sub-block 2t), 1: high nibbles (sub-block 2t+1)
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const unsigned word = t < 2 ? sc03 : sc47;  // scale of sub-block j = 2t + hiN: byte j & 3
-            const unsigned sc = (word >> (16 * (t & 1) + 8 * hiN)) & 0xff;
-            const unsigned sh = sc >> 3, sl = sc & 7;
             const unsigned v[4] = {raw.q[t].x, raw.q[t].y, raw.q[t].z, raw.q[t].w};
-            v4i bh, bl;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const unsigned nib = (v[i] >> (4 * hiN)) & 0x0f0f0f0fu;
-                bh[i] = (int)(nib * sh);  // four byte products <= 105: no carries between bytes
-                bl[i] = (int)(nib * sl);
-            }
-            b.hi[t] = bh;
-            b.lo[t] = bl;
+            for (int i = 0; i < 4; i++) b.q[t][i] = (int)((v[i] >> (4 * hiN)) & 0x0f0f0f0fu);
         }
-        // block-sum MFMAs: the A rows carry [S_l(0..7) | S_h(0..7)] in K group 0 and zeros elsewhere
+        // block-sum MFMA: mins 0..7 in the first eight K slots of group 0, against the digits of the
+        // eight 32-element sums in the same slots of the A rows
         const int mz = g == 0 ? -1 : 0;
-        b.min_lo = (v4i){(int)mn03 & mz, (int)mn47 & mz, 0, 0};
-        b.min_hi = (v4i){0, 0, (int)mn03 & mz, (int)mn47 & mz};
+        b.bsum = (v4i){(int)mn03 & mz, (int)mn47 & mz, 0, 0};
     }
-    static __device__ __forceinline__ bool sums_on(int g) { return g == 0; }
+    // outputs v of a step's MFMA -> the lane's two columns
+    static __device__ __forceinline__ void scale_step(const v4acc &dv, int t, const Ops &b, int (&isum)[LANE_COLS]) {
+        isum[0] = mad24(b.sc[2 * t], dv[0], mad24(b.sc[2 * t + 1], dv[1], isum[0]));
+        isum[1] = mad24(b.sc[2 * t], dv[2], mad24(b.sc[2 * t + 1], dv[3], isum[1]));
+    }
+    // Block-sum operand: row r carries, in K group 0, the low (r even) or high (r odd) digits of column
+    // r>>1's eight sums; the stage holds [S_l(0..7) | S_h(0..7)] per column.
+    static __device__ __forceinline__ bool d_on(int r, int g) { return g == 0; }
+    static __device__ __forceinline__ int d_off(int r) { return 0; }
+    static __device__ __forceinline__ v4i d_fix(v4i raw, int r) {
+        return (r & 1) ? (v4i){raw[2], raw[3], 0, 0} : (v4i){raw[0], raw[1], 0, 0};
+    }
+    // y contribution of one column and super-block, without the activation scale
+    static __device__ __forceinline__ float finish(const Ops &b, int isum, const v4acc &x, int u) {
+        const float fm = G::fold_min(b.dmin, x[2 * u + 1], x[2 * u]);
+        return __builtin_fmaf(b.d, (float)isum, -fm);
+    }
 };
 
 struct Sk16Q6K {
@@ -512,39 +538,48 @@ struct Sk16Q6K {
         }
         raw.scv = ld16(wt + 3072 + c * 16);
     }
-    static __device__ __forceinline__ void expand(const Raw &raw, int g, unsigned dh, B16 &b) {
+    // A sub-block is 16 elements = one K group of a step, so the 16 rows of the A operand are 4 columns x
+    // the four sub-blocks of the step: row r is column r>>2 restricted to K group r&3.  The outputs of
+    // lane l are rows 4(l>>4) + v = column l>>4 x sub-blocks 4t + v.
+    static constexpr int SET_COLS = 4, LANE_COLS = 1, NSC = 16;
+    typedef B16<NSC> Ops;
+    static __device__ __forceinline__ int a_col(int r) { return r >> 2; }
+    static __device__ __forceinline__ bool a_on(int r, int g) { return g == (r & 3); }
+    static __device__ __forceinline__ int lane_col(int lg, int) { return lg; }
+    static __device__ __forceinline__ void expand(const Raw &raw, int g, unsigned dh, Ops &b) {
         const unsigned scw[4] = {raw.scv.x, raw.scv.y, raw.scv.z, raw.scv.w};
         b.d = h2f(dh);
         b.dmin = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; j++) b.sc[j] = (int)(int8_t)(scw[j >> 2] >> (8 * (j & 3)));
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const int H = t >> 1;
             const int rr2 = 2 * (2 * (t & 1) + (g >> 1));  // shift of the two high bits inside a qh byte
             const unsigned l[4] = {raw.L[H].x, raw.L[H].y, raw.L[H].z, raw.L[H].w};
             const unsigned hq[4] = {raw.Hq[H].x, raw.Hq[H].y, raw.Hq[H].z, raw.Hq[H].w};
-            const int sc = (int)(int8_t)(scw[t] >> (8 * g));  // scales[4t + g]
-            const s2 scv2 = {(short)sc, (short)sc};
-            v4i bh, bl;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const unsigned nib = (t & 1) ? (l[i] >> 4) & 0x0f0f0f0fu : l[i] & 0x0f0f0f0fu;
-                const unsigned e = nib | (((hq[i] >> rr2) & 0x03030303u) << 4);  // 0..63 per byte
-                const s2 pe = as_s2(e & 0x00ff00ffu) * scv2;         // elements 0 and 2, 16-bit products
-                const s2 po = as_s2((e >> 8) & 0x00ff00ffu) * scv2;  // elements 1 and 3
-                const unsigned le = as_u(pe) & 0x003f003fu, lo_ = as_u(po) & 0x003f003fu;
-                const unsigned he = as_u(pe >> 6), ho = as_u(po >> 6);  // arithmetic shift per 16-bit lane
-                bl[i] = (int)(le | (lo_ << 8));
-                bh[i] = (int)__builtin_amdgcn_perm(ho, he, 0x06020400u);  // bytes: he.b0, ho.b0, he.b2, ho.b2
+                b.q[t][i] = (int)(nib | (((hq[i] >> rr2) & 0x03030303u) << 4));  // 0..63 per byte; the -32 goes through the block sums
             }
-            b.hi[t] = bh;
-            b.lo[t] = bl;
         }
-        // block-sum MFMAs: the A rows carry S_l(0..15) in K group 0 and S_h(0..15) in K group 1
-        const int z0 = g == 0 ? -1 : 0, z1 = g == 1 ? -1 : 0;
-        b.min_lo = (v4i){(int)scw[0] & z0, (int)scw[1] & z0, (int)scw[2] & z0, (int)scw[3] & z0};
-        b.min_hi = (v4i){(int)scw[0] & z1, (int)scw[1] & z1, (int)scw[2] & z1, (int)scw[3] & z1};
+        // block-sum MFMA: the 16 scales in K group 0 against the digits of the sixteen 16-element sums
+        const int mz = g == 0 ? -1 : 0;
+        b.bsum = (v4i){(int)scw[0] & mz, (int)scw[1] & mz, (int)scw[2] & mz, (int)scw[3] & mz};
     }
-    static __device__ __forceinline__ bool sums_on(int g) { return g < 2; }
+    static __device__ __forceinline__ void scale_step(const v4acc &dv, int t, const Ops &b, int (&isum)[LANE_COLS]) {
+        isum[0] = mad24(b.sc[4 * t], dv[0], mad24(b.sc[4 * t + 1], dv[1], mad24(b.sc[4 * t + 2], dv[2],
+                  mad24(b.sc[4 * t + 3], dv[3], isum[0]))));
+    }
+    // Block-sum operand: row r carries, in K group 0, the low (r&3 == 0) or high (r&3 == 1) digits of
+    // column r>>2's sixteen sums; the stage holds [S_l(0..15) | S_h(0..15)] per column.
+    static __device__ __forceinline__ bool d_on(int r, int g) { return g == 0 && (r & 3) < 2; }
+    static __device__ __forceinline__ int d_off(int r) { return 16 * (r & 1); }
+    static __device__ __forceinline__ v4i d_fix(v4i raw, int) { return raw; }
+    static __device__ __forceinline__ float finish(const Ops &b, int isum, const v4acc &x, int) {
+        return b.d * (float)(isum - 32 * ((x[1] << 6) + x[0]));  // sum sc*(e-32)*y = sum sc*e*y - 32 sum_g sc_g*S_g
+    }
 };
 
 constexpr int SKINNY_MAX_SB_PER_WAVE = 32;  // a wave keeps its rows' fp16 super-block scales in LDS
@@ -554,7 +589,9 @@ template <class S, int NCT>
 struct SkinnyGeo {
     static constexpr int A_BYTES = NCT * 256, A_INSTRS = NCT / 4;
     static constexpr int D_BYTES = 16 * NCT * S::D_LANES_PER_COL, Y_BYTES = 64;
-    static constexpr int STAGE = S::W_BYTES + A_BYTES + D_BYTES + Y_BYTES;
+    static constexpr int Z_OFF = S::W_BYTES + A_BYTES + D_BYTES + Y_BYTES;  // 16 zero bytes no copy ever writes
+    static constexpr int STAGE = Z_OFF + 64;
+    static constexpr int SETS = NCT / S::SET_COLS, LANE_ACC = SETS * S::LANE_COLS;  // column sets; outputs per lane
     static constexpr int NDMA = S::W_INSTRS + A_INSTRS + 2;  // copy instructions per stage
     static constexpr int DSM_BYTES = S::SCALES_OUTSIDE ? 16 * SKINNY_MAX_SB_PER_WAVE * 2 : 0;
     static constexpr int WAVE_BYTES = (2 * STAGE + DSM_BYTES + 255) / 256 * 256;
@@ -573,7 +610,7 @@ constexpr int SKINNY_ID_REC = 2 + 16;
 
 // The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
 template <class S, int NCT, bool ID>
-__global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
+__global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
                                                         SkinnyIds si) {
     typedef typename S::G G;
     typedef SkinnyGeo<S, NCT> Geo;
@@ -656,7 +693,28 @@ __global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, i
         }
     };
 
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    // ---- operand reads: per-lane offsets into a stage.  A row r = lane & 15 of column set cs is column
+    // SET_COLS*cs + a_col(r) restricted to the K groups of one sub-block (a_on); every other lane, and every
+    // column past nc, reads the stage's 16 zero bytes instead.
+    constexpr int SETS = Geo::SETS, LANE_ACC = Geo::LANE_ACC;
+    if (lane < 8) *reinterpret_cast<int *>(wsm + (lane >> 2) * STAGE + Geo::Z_OFF + 4 * (lane & 3)) = 0;
+    int aro[SETS][4], dro[SETS], yro[LANE_ACC];
+#pragma unroll
+    for (int cs = 0; cs < SETS; cs++) {
+        const int col = S::SET_COLS * cs + S::a_col(c);
+        const bool on = col < nc;
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+            aro[cs][t] = on && S::a_on(c, g) ? S::W_BYTES + col * 256 + 16 * ((4 * t + g) ^ col) : Geo::Z_OFF;
+        dro[cs] = on && S::d_on(c, g) ? S::W_BYTES + A_BYTES + col * (16 * S::D_LANES_PER_COL) + S::d_off(c) : Geo::Z_OFF;
+#pragma unroll
+        for (int u = 0; u < S::LANE_COLS; u++)  // columns past nc: any staged scale (their sums are zero)
+            yro[cs * S::LANE_COLS + u] = S::W_BYTES + A_BYTES + D_BYTES + 4 * min(S::SET_COLS * cs + S::lane_col(g, u), NCT - 1);
+    }
+
+    float acc[LANE_ACC];
+#pragma unroll
+    for (int i = 0; i < LANE_ACC; i++) acc[i] = 0.f;
     if (sb0 < sb1) {
         // the rows' fp16 super-block scales live outside the packed planes for Q6_K: fetch this wave's
         // run of them once, before the steady state (their wait would otherwise drain the copies)
@@ -667,9 +725,6 @@ __global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, i
         stage_copy(wsm, sb0);
         stage_copy(wsm + STAGE, min(sb0 + 1, sb1 - 1));
         const v4acc zero = {0, 0, 0, 0};
-        const v4i zero4 = {0, 0, 0, 0};
-        const bool acol = c < nc;  // the lane holds a real activation column in the A operand
-        const int cc = min(c, NCT - 1);  // lanes past the staged columns read a staged one and zero it
 #pragma unroll 1
         for (int64_t sb = sb0; sb < sb1; sb++) {
             uint8_t *st = wsm + ((sb - sb0) & 1) * STAGE;
@@ -678,43 +733,46 @@ __global__ __launch_bounds__(512, 4) void skinny_kernel(DevWeight w, DevAct a, i
             __builtin_amdgcn_s_waitcnt((NDMA & 15) | (7 << 4) | (15 << 8) | ((NDMA >> 4) << 14));
             typename S::Raw raw;
             S::read(st, c, g, raw);
-            v4i av[4], sv;
+            v4i av[SETS][4], sv[SETS];
+            float ydv[LANE_ACC];
 #pragma unroll
-            for (int t = 0; t < 4; t++) av[t] = *reinterpret_cast<const v4i *>(st + S::W_BYTES + cc * 256 + 16 * ((4 * t + g) ^ cc));
-            sv = *reinterpret_cast<const v4i *>(st + S::W_BYTES + A_BYTES + (cc * S::D_LANES_PER_COL + (S::D_LANES_PER_COL == 2 ? (g & 1) : 0)) * 16);
-            const float4 yd = *reinterpret_cast<const float4 *>(st + S::W_BYTES + A_BYTES + D_BYTES + 16 * g);
+            for (int cs = 0; cs < SETS; cs++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) av[cs][t] = *reinterpret_cast<const v4i *>(st + aro[cs][t]);
+                sv[cs] = *reinterpret_cast<const v4i *>(st + dro[cs]);
+            }
+#pragma unroll
+            for (int i = 0; i < LANE_ACC; i++) ydv[i] = *reinterpret_cast<const float *>(st + yro[i]);
             const unsigned dh = S::SCALES_OUTSIDE ? dsm[c * SKINNY_MAX_SB_PER_WAVE + (sb - sb0)] : 0u;
             // operands are in registers: the stage can take the copies of super-block sb + 2
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             stage_copy(st, min(sb + 2, sb1 - 1));
-            if (!acol) {
-#pragma unroll
-                for (int t = 0; t < 4; t++) av[t] = zero4;
-            }
-            if (!acol || !S::sums_on(g)) sv = zero4;
-            B16 b;
+            typename S::Ops b;
             S::expand(raw, g, dh, b);
-            const v4acc xl = mfma16(sv, b.min_lo, zero);
-            const v4acc xh = mfma16(sv, b.min_hi, zero);
-            v4acc ah, al;
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                ah = mfma16(av[t], b.hi[t], t == 0 ? zero : ah);
-                al = mfma16(av[t], b.lo[t], t == 0 ? zero : al);
-            }
-            const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
+            for (int cs = 0; cs < SETS; cs++) {
+                const v4acc x = mfma16(S::d_fix(sv[cs], c), b.bsum, zero);
+                int isum[S::LANE_COLS];
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const float fm = G::fold_min(b.dmin, xh[v], xl[v]);
-                acc[v] = __builtin_fmaf(ydv[v], G::combine(b.d, ah[v], al[v], fm), acc[v]);
+                for (int u = 0; u < S::LANE_COLS; u++) isum[u] = 0;
+#pragma unroll
+                for (int t = 0; t < 4; t++) S::scale_step(mfma16(av[cs][t], b.q[t], zero), t, b, isum);
+#pragma unroll
+                for (int u = 0; u < S::LANE_COLS; u++) {
+                    const int i = cs * S::LANE_COLS + u;
+                    acc[i] = __builtin_fmaf(ydv[i], S::finish(b, isum[u], x, u), acc[i]);
+                }
             }
         }
         __builtin_amdgcn_s_waitcnt(0);  // the redundant copies of the last iterations must not outlive the kernel's LDS
     }
+    // lane l holds weight row l & 15 of columns SET_COLS*cs + lane_col(l >> 4, u)
 #pragma unroll
-    for (int v = 0; v < 4; v++) part[wave][4 * g + v][c] = acc[v];
+    for (int cs = 0; cs < SETS; cs++)
+#pragma unroll
+        for (int u = 0; u < S::LANE_COLS; u++) part[wave][S::SET_COLS * cs + S::lane_col(g, u)][c] = acc[cs * S::LANE_COLS + u];
     __syncthreads();
-    for (int o = tid; o < 256; o += blockDim.x) {
+    for (int o = tid; o < 16 * NCT; o += blockDim.x) {
         const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
         float sum = 0.f;
         for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
