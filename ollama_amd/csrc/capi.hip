@@ -658,7 +658,8 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
     }
     DevAct a{};
     a.K = K; a.N = (int)ncols; a.type = q8;
-    const bool skinny = skinny_id_supports(w->dev.type, K, M, pairs, n_expert);
+    // the matrix-core kernel addresses activation bytes with 32-bit offsets
+    const bool skinny = skinny_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
     const bool fused = !skinny && gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert);
     if (!fused) {
         HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));

@@ -582,7 +582,6 @@ struct Sk16Q6K {
     }
 };
 
-constexpr int SKINNY_MAX_SB_PER_WAVE = 32;  // a wave keeps its rows' fp16 super-block scales in LDS
 
 // NCT = activation columns the stages are laid out for (8 or 16)
 template <class S, int NCT>
@@ -590,11 +589,11 @@ struct SkinnyGeo {
     static constexpr int A_BYTES = NCT * 256, A_INSTRS = NCT / 4;
     static constexpr int D_BYTES = 16 * NCT * S::D_LANES_PER_COL, Y_BYTES = 64;
     static constexpr int Z_OFF = S::W_BYTES + A_BYTES + D_BYTES + Y_BYTES;  // 16 zero bytes no copy ever writes
-    static constexpr int STAGE = Z_OFF + 64;
+    static constexpr int STAGE = Z_OFF + 128;
     static constexpr int SETS = NCT / S::SET_COLS, LANE_ACC = SETS * S::LANE_COLS;  // column sets; outputs per lane
-    static constexpr int NDMA = S::W_INSTRS + A_INSTRS + 2;  // copy instructions per stage
-    static constexpr int DSM_BYTES = S::SCALES_OUTSIDE ? 16 * SKINNY_MAX_SB_PER_WAVE * 2 : 0;
-    static constexpr int WAVE_BYTES = (2 * STAGE + DSM_BYTES + 255) / 256 * 256;
+    static constexpr int DH_OFF = Z_OFF + 64;  // per row the aligned dword that holds its fp16 super-block scale (Q6_K)
+    static constexpr int NDMA = S::W_INSTRS + A_INSTRS + 2 + (S::SCALES_OUTSIDE ? 1 : 0);  // copy instructions per stage
+    static constexpr int WAVE_BYTES = (2 * STAGE + 255) / 256 * 256;
     static constexpr int PART_BYTES = 16 * 16 * 4;  // per wave: its partial sums
 };
 
@@ -652,13 +651,24 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     const int64_t nsb = w.K / QKK;
     const int64_t sb0 = nsb * wave / WAVES, sb1 = nsb * (wave + 1) / WAVES;  // this wave's run of super-blocks
     uint8_t *wsm = smem + wave * WAVE_BYTES;
-    uint16_t *dsm = reinterpret_cast<uint16_t *>(wsm + 2 * STAGE);  // [16 rows][sb1 - sb0] fp16 scales (Q6_K)
+    // Work items: the 16-row groups this workgroup goes through, blockIdx.x + k * gridDim.x (an
+    // expert-indexed launch has exactly one per workgroup).  The copy stream runs two stages ahead of
+    // the math and simply continues into the next item, so only the first item pays the pipeline fill.
+    const int64_t total_items = ID ? 0 : (w.M + 15) / 16;
+    const int64_t items = ID ? 1 : (total_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
 
     // ---- copy plan: per-lane 32-bit offsets, uniform bases per super-block
     unsigned woff[S::W_INSTRS];
+    int64_t dhrow = 0;  // byte offset of the lane's row in the plane of fp16 super-block scales
     bool won[S::W_INSTRS];
+    int64_t cp_m0 = m0, cp_k = 0, cp_sb = sb0;  // the copy cursor: item (its first row) and super-block
+    auto plan_item = [&](int64_t first_row, int rows) __attribute__((always_inline)) {
+        cp_m0 = first_row;
 #pragma unroll
-    for (int j = 0; j < S::W_INSTRS; j++) S::w_plan(w, j, lane, rows_left, woff[j], won[j]);
+        for (int j = 0; j < S::W_INSTRS; j++) S::w_plan(w, j, lane, rows, woff[j], won[j]);
+        dhrow = (first_row + min(c, rows - 1)) * nsb * 2;
+    };
+    plan_item(m0, rows_left);
     unsigned aoff[A_INSTRS];
 #pragma unroll
     for (int j = 0; j < A_INSTRS; j++) {
@@ -672,10 +682,14 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
     const uint8_t *asd = G::digits(a);
 
-    auto stage_copy = [&](uint8_t *st, int64_t sb) __attribute__((always_inline)) {
+    // one stage = everything the wave multiplies in one super-block; then the cursor moves on (past the
+    // last super-block of the last item it stays put: the copy is repeated so that every iteration
+    // issues the same number of copies)
+    auto stage_copy = [&](uint8_t *st) __attribute__((always_inline)) {
+        const int64_t sb = cp_sb;
 #pragma unroll
         for (int j = 0; j < S::W_INSTRS; j++) {
-            const uint8_t *gp = S::w_base(w, j, m0, sb) + woff[j];
+            const uint8_t *gp = S::w_base(w, j, cp_m0, sb) + woff[j];
             if (won[j]) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * j), 16, 0, 0);
         }
 #pragma unroll
@@ -690,6 +704,18 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
         {
             const uint8_t *gp = reinterpret_cast<const uint8_t *>(a.d) + sb * 4 + yoff;
             if (yon) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + S::W_BYTES + A_BYTES + D_BYTES), 4, 0, 0);
+        }
+        if (S::SCALES_OUTSIDE) {  // the rows' fp16 super-block scales are a plane of their own (Q6_K)
+            const uint8_t *gp = reinterpret_cast<const uint8_t *>(w.d) + ((dhrow + 2 * sb) & ~(int64_t)3);
+            if (lane < 16) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DH_OFF), 4, 0, 0);
+        }
+        if (cp_sb + 1 < sb1) {
+            cp_sb++;
+        } else if (cp_k + 1 < items) {
+            cp_k++;
+            cp_sb = sb0;
+            const int64_t first = ((int64_t)blockIdx.x + cp_k * gridDim.x) * 16;  // never taken by expert-indexed launches
+            plan_item(first, (int)min((int64_t)16, w.M - first));
         }
     };
 
@@ -712,22 +738,27 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
             yro[cs * S::LANE_COLS + u] = S::W_BYTES + A_BYTES + D_BYTES + 4 * min(S::SET_COLS * cs + S::lane_col(g, u), NCT - 1);
     }
 
-    float acc[LANE_ACC];
-#pragma unroll
-    for (int i = 0; i < LANE_ACC; i++) acc[i] = 0.f;
-    if (sb0 < sb1) {
-        // the rows' fp16 super-block scales live outside the packed planes for Q6_K: fetch this wave's
-        // run of them once, before the steady state (their wait would otherwise drain the copies)
-        if (S::SCALES_OUTSIDE) {
-            const int64_t row = m0 + min(c, rows_left - 1);
-            for (int64_t i = g; i < sb1 - sb0; i += 4) dsm[c * SKINNY_MAX_SB_PER_WAVE + i] = w.d[row * nsb + sb0 + i];
+    const bool has_k = sb0 < sb1;  // (the launcher gives every wave at least two super-blocks)
+    if (has_k) {
+        stage_copy(wsm);
+        stage_copy(wsm + STAGE);
+    }
+    const v4acc zero = {0, 0, 0, 0};
+    unsigned parity = 0;  // which stage the next super-block is in
+#pragma unroll 1
+    for (int64_t k = 0; k < items; k++) {
+        if (!ID) {
+            m0 = ((int64_t)blockIdx.x + k * gridDim.x) * 16;
+            yrow0 = m0;
+            rows_left = (int)min((int64_t)16, w.M - m0);
         }
-        stage_copy(wsm, sb0);
-        stage_copy(wsm + STAGE, min(sb0 + 1, sb1 - 1));
-        const v4acc zero = {0, 0, 0, 0};
+        float acc[LANE_ACC];
+#pragma unroll
+        for (int i = 0; i < LANE_ACC; i++) acc[i] = 0.f;
 #pragma unroll 1
         for (int64_t sb = sb0; sb < sb1; sb++) {
-            uint8_t *st = wsm + ((sb - sb0) & 1) * STAGE;
+            uint8_t *st = wsm + (parity & 1) * STAGE;
+            parity ^= 1;
             // Every wave issues exactly NDMA copy instructions per stage, in order: once at most NDMA
             // are outstanding, this stage has landed and the next one may still be in flight.
             __builtin_amdgcn_s_waitcnt((NDMA & 15) | (7 << 4) | (15 << 8) | ((NDMA >> 4) << 14));
@@ -743,10 +774,15 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
             }
 #pragma unroll
             for (int i = 0; i < LANE_ACC; i++) ydv[i] = *reinterpret_cast<const float *>(st + yro[i]);
-            const unsigned dh = S::SCALES_OUTSIDE ? dsm[c * SKINNY_MAX_SB_PER_WAVE + (sb - sb0)] : 0u;
-            // operands are in registers: the stage can take the copies of super-block sb + 2
+            unsigned dh = 0;
+            if (S::SCALES_OUTSIDE) {
+                const unsigned pair = *reinterpret_cast<const unsigned *>(st + Geo::DH_OFF + 4 * c);
+                const bool odd = (((m0 + min(c, rows_left - 1)) * nsb + sb) & 1) != 0;  // which half of the aligned dword
+                dh = odd ? pair >> 16 : pair & 0xffff;
+            }
+            // operands are in registers: the stage can take the copies of the super-block after next
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            stage_copy(st, min(sb + 2, sb1 - 1));
+            stage_copy(st);
             typename S::Ops b;
             S::expand(raw, g, dh, b);
 #pragma unroll
@@ -764,20 +800,22 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
                 }
             }
         }
-        __builtin_amdgcn_s_waitcnt(0);  // the redundant copies of the last iterations must not outlive the kernel's LDS
-    }
-    // lane l holds weight row l & 15 of columns SET_COLS*cs + lane_col(l >> 4, u)
+        // lane l holds weight row l & 15 of columns SET_COLS*cs + lane_col(l >> 4, u)
 #pragma unroll
-    for (int cs = 0; cs < SETS; cs++)
+        for (int cs = 0; cs < SETS; cs++)
 #pragma unroll
-        for (int u = 0; u < S::LANE_COLS; u++) part[wave][S::SET_COLS * cs + S::lane_col(g, u)][c] = acc[cs * S::LANE_COLS + u];
-    __syncthreads();
-    for (int o = tid; o < 16 * NCT; o += blockDim.x) {
-        const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
-        float sum = 0.f;
-        for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
-        if (i < nc && j < rows_left) y[(int64_t)(ID ? rec[2 + i] : col0 + i) * ldy + yrow0 + j] = sum;
+            for (int u = 0; u < S::LANE_COLS; u++)
+                part[wave][S::SET_COLS * cs + S::lane_col(g, u)][c] = acc[cs * S::LANE_COLS + u];
+        __syncthreads();
+        for (int o = tid; o < 16 * NCT; o += blockDim.x) {
+            const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
+            float sum = 0.f;
+            for (int kk = 0; kk < WAVES; kk++) sum += part[kk][i][j];
+            if (i < nc && j < rows_left) y[(int64_t)(ID ? rec[2 + i] : col0 + i) * ldy + yrow0 + j] = sum;
+        }
+        if (k + 1 < items) __syncthreads();  // the partial sums are read before the next item overwrites them
     }
+    if (has_k) __builtin_amdgcn_s_waitcnt(0);  // the repeated copies at the end must not outlive the kernel's LDS
 }
 
 // y[i] = sum over slices of part[slice][i]
@@ -852,7 +890,7 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
 int gemm_max_multi() { return GEMM_MULTI; }
 
 bool skinny_supports(int type, int64_t K, int64_t M) {
-    return gemm_supports(type, K, M) && (K / QKK + 7) / 8 <= SKINNY_MAX_SB_PER_WAVE;
+    return gemm_supports(type, K, M);
 }
 
 // Cut K as many ways as keeps the whole grid resident in one round (about 15 waves per CU fit): every
@@ -862,7 +900,6 @@ int skinny_waves(int64_t row_groups, int64_t nsb, int num_cus) {
     int waves = (int)((int64_t)num_cus * 15 / row_groups);
     waves = waves >= 8 ? 8 : waves >= 6 ? 6 : waves >= 4 ? 4 : waves >= 3 ? 3 : waves >= 2 ? 2 : 1;
     while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;  // at least two super-blocks per wave
-    while ((nsb + waves - 1) / waves > SKINNY_MAX_SB_PER_WAVE && waves < 8) waves = waves >= 4 ? waves + 2 : waves + 1;
     return waves;
 }
 
@@ -880,12 +917,24 @@ void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, 
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny_kernel<S, NCT, ID><<<(unsigned)row_groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
+    // More row groups than fit the GPU at once: launch one resident round of workgroups and let each walk
+    // through an equal share of the row groups (its copy stream never drains in between).  Expert-indexed
+    // launches keep one item per workgroup: their columns change from group to group.
+    int64_t grid = row_groups;
+    if (!ID) {
+        const int64_t by_lds = (160 * 1024) / (int64_t)(Geo::WAVE_BYTES + Geo::PART_BYTES), by_regs = Geo::SETS >= 4 ? 8 : 16;
+        const int64_t wgs_per_cu = (by_lds < by_regs ? by_lds : by_regs) / waves;
+        const int64_t resident = (int64_t)num_cus * (wgs_per_cu < 1 ? 1 : wgs_per_cu);
+        const int64_t rounds = (row_groups + resident - 1) / resident;
+        grid = (row_groups + rounds - 1) / rounds;
+    }
+    skinny_kernel<S, NCT, ID><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
 }
 
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
     if (!skinny_supports(w.type, w.K, w.M) || a.type != T_Q8_K || a.K != w.K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
     if (ncols < 1 || ncols > 16 || col0 < 0 || col0 + ncols > a.N) return hipErrorInvalidValue;
+    if ((int64_t)(col0 + ncols) * a.K >= ((int64_t)1 << 32)) return hipErrorInvalidValue;  // 32-bit activation offsets
     if ((w.M + 15) / 16 > 0x7fffffff) return hipErrorInvalidValue;
     const SkinnyIds none{};
     const int64_t rg = (w.M + 15) / 16;
@@ -908,7 +957,7 @@ hipError_t launch_skinny_id(const DevWeight &w, int n_expert, const DevAct &a, c
                             int b_cols, float *y, int *groups, int num_cus, hipStream_t s) {
     if (n_expert < 1 || w.M % n_expert || !skinny_supports(w.type, w.K, w.M / n_expert) || a.type != T_Q8_K ||
         a.K != w.K || !a.sd8 || !a.sd16 || !ids || !y || !groups || n_used < 1 || n_tokens < 1 || b_cols < 1 ||
-        a.N != (int64_t)b_cols * n_tokens)
+        a.N != (int64_t)b_cols * n_tokens || (int64_t)a.N * a.K >= ((int64_t)1 << 32))
         return hipErrorInvalidValue;
     const int64_t pairs = (int64_t)n_used * n_tokens;
     if (hipError_t e = launch_group_pairs(ids, (int)pairs, n_expert, 16, groups, s)) return e;
