@@ -59,7 +59,7 @@ enum { MI_QMM_HOST = 0, MI_QMM_DEVICE = 1 };
 enum {
     MI_QMM_PATH_AUTO = 0, /* decode kernels below N = 32, tiled int8-MFMA GEMM from N = 32             */
     MI_QMM_PATH_GEMV = 1, /* the decode kernels at any N: streaming GEMV, 8 columns at a time; K-quant
-                             weights go to the skinny matrix-core kernel from 5 (Q4_K) / 6 (Q6_K)
+                             weights go to the skinny matrix-core kernel from 3 (Q4_K) / 4 (Q6_K)
                              columns, 16 at a time                                                   */
     MI_QMM_PATH_GEMM = 2  /* force the tiled int8-MFMA GEMM (any N >= 1, padded to the tile)          */
 };

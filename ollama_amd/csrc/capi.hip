@@ -418,7 +418,7 @@ namespace {
 // matrix-core skinny kernel instead of the streaming GEMV (measured crossover on MI355X: the GEMV pays
 // one v_dot4 pass per column).
 bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
-    const int64_t from = type == T_Q4_K ? 5 : 6;
+    const int64_t from = type == T_Q4_K ? 3 : 4;
     return n >= from && skinny_supports(type, K, M);
 }
 

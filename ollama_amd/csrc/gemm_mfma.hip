@@ -584,16 +584,17 @@ struct Sk16Q6K {
 
 
 // NCT = activation columns the stages are laid out for (8 or 16)
-template <class S, int NCT>
+template <class S, int NCT, int NST = 2>
 struct SkinnyGeo {
     static constexpr int A_BYTES = NCT * 256, A_INSTRS = NCT / 4;
-    static constexpr int D_BYTES = 16 * NCT * S::D_LANES_PER_COL, Y_BYTES = 64;
+    static constexpr int D_BYTES = 16 * NCT * S::D_LANES_PER_COL, Y_BYTES = 4 * NCT;
     static constexpr int Z_OFF = S::W_BYTES + A_BYTES + D_BYTES + Y_BYTES;  // 16 zero bytes no copy ever writes
-    static constexpr int STAGE = Z_OFF + 128;
+    static constexpr int DH_OFF = Z_OFF + 16;  // per row the aligned dword that holds its fp16 super-block scale (Q6_K)
+    static constexpr int STAGE = (DH_OFF + (S::SCALES_OUTSIDE ? 64 : 0) + 63) / 64 * 64;
     static constexpr int SETS = NCT / S::SET_COLS, LANE_ACC = SETS * S::LANE_COLS;  // column sets; outputs per lane
-    static constexpr int DH_OFF = Z_OFF + 64;  // per row the aligned dword that holds its fp16 super-block scale (Q6_K)
     static constexpr int NDMA = S::W_INSTRS + A_INSTRS + 2 + (S::SCALES_OUTSIDE ? 1 : 0);  // copy instructions per stage
-    static constexpr int WAVE_BYTES = (2 * STAGE + 255) / 256 * 256;
+    static constexpr int NSTAGE = NST;  // stages in a wave's ring: NSTAGE - 1 super-blocks in flight behind the one being multiplied
+    static constexpr int WAVE_BYTES = (NSTAGE * STAGE + 255) / 256 * 256;
     static constexpr int PART_BYTES = 16 * 16 * 4;  // per wave: its partial sums
 };
 
@@ -608,11 +609,11 @@ struct SkinnyIds {
 constexpr int SKINNY_ID_REC = 2 + 16;
 
 // The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
-template <class S, int NCT, bool ID>
+template <class S, int NCT, bool ID, int NST>
 __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
                                                         SkinnyIds si) {
     typedef typename S::G G;
-    typedef SkinnyGeo<S, NCT> Geo;
+    typedef SkinnyGeo<S, NCT, NST> Geo;
     constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, WAVE_BYTES = Geo::WAVE_BYTES;
     const int WAVES = blockDim.x >> 6;
@@ -723,7 +724,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     // SET_COLS*cs + a_col(r) restricted to the K groups of one sub-block (a_on); every other lane, and every
     // column past nc, reads the stage's 16 zero bytes instead.
     constexpr int SETS = Geo::SETS, LANE_ACC = Geo::LANE_ACC;
-    if (lane < 8) *reinterpret_cast<int *>(wsm + (lane >> 2) * STAGE + Geo::Z_OFF + 4 * (lane & 3)) = 0;
+    if (lane < 4 * Geo::NSTAGE) *reinterpret_cast<int *>(wsm + (lane >> 2) * STAGE + Geo::Z_OFF + 4 * (lane & 3)) = 0;
     int aro[SETS][4], dro[SETS], yro[LANE_ACC];
 #pragma unroll
     for (int cs = 0; cs < SETS; cs++) {
@@ -741,7 +742,8 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     const bool has_k = sb0 < sb1;  // (the launcher gives every wave at least two super-blocks)
     if (has_k) {
         stage_copy(wsm);
-        stage_copy(wsm + STAGE);
+#pragma unroll
+        for (int i = 1; i < Geo::NSTAGE; i++) stage_copy(wsm + i * STAGE);
     }
     const v4acc zero = {0, 0, 0, 0};
     unsigned parity = 0;  // which stage the next super-block is in
@@ -757,11 +759,13 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
         for (int i = 0; i < LANE_ACC; i++) acc[i] = 0.f;
 #pragma unroll 1
         for (int64_t sb = sb0; sb < sb1; sb++) {
-            uint8_t *st = wsm + (parity & 1) * STAGE;
-            parity ^= 1;
+            uint8_t *st = wsm + parity * STAGE;
+            parity = parity + 1 == Geo::NSTAGE ? 0 : parity + 1;
             // Every wave issues exactly NDMA copy instructions per stage, in order: once at most NDMA
             // are outstanding, this stage has landed and the next one may still be in flight.
-            __builtin_amdgcn_s_waitcnt((NDMA & 15) | (7 << 4) | (15 << 8) | ((NDMA >> 4) << 14));
+            constexpr int INFLIGHT = (Geo::NSTAGE - 1) * NDMA;
+            static_assert(INFLIGHT < 64, "vmcnt is a 6-bit counter");
+            __builtin_amdgcn_s_waitcnt((INFLIGHT & 15) | (7 << 4) | (15 << 8) | ((INFLIGHT >> 4) << 14));
             typename S::Raw raw;
             S::read(st, c, g, raw);
             v4i av[SETS][4], sv[SETS];
@@ -893,42 +897,46 @@ bool skinny_supports(int type, int64_t K, int64_t M) {
     return gemm_supports(type, K, M);
 }
 
-// Cut K as many ways as keeps the whole grid resident in one round (about 15 waves per CU fit): every
-// wave pays one pipeline fill, so few long waves when there are many row groups, many short ones when
-// there are few.
+// How many waves cut K in a workgroup.  Measured over decode shapes (gate 14336 x 4096, down 4096 x 14336,
+// q 4096 x 4096, the 128256-row head): the kernel runs best with about eight waves per CU over the whole
+// grid -- fewer leave the memory system idle, more only add pipeline fills and K-cut sums -- and with
+// every wave having at least two super-blocks.
 int skinny_waves(int64_t row_groups, int64_t nsb, int num_cus) {
-    int waves = (int)((int64_t)num_cus * 15 / row_groups);
-    waves = waves >= 8 ? 8 : waves >= 6 ? 6 : waves >= 4 ? 4 : waves >= 3 ? 3 : waves >= 2 ? 2 : 1;
-    while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;  // at least two super-blocks per wave
+    const int64_t want = ((int64_t)num_cus * 8 + row_groups / 2) / row_groups;  // nearest
+    int waves = want >= 8 ? 8 : want >= 6 ? 6 : want >= 4 ? 4 : want >= 3 ? 3 : want >= 2 ? 2 : 1;
+    while (waves > 1 && nsb / waves < 2) waves = waves > 4 ? waves - 2 : waves - 1;
     return waves;
 }
 
-template <class S, int NCT, bool ID>
-void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, const SkinnyIds &si,
-                      int64_t row_groups, int num_cus, hipStream_t s) {
-    typedef SkinnyGeo<S, NCT> Geo;
-    const int waves = skinny_waves(row_groups, w.K / QKK, num_cus);
+template <class S, int NCT, bool ID, int NST>
+void launch_skinny_grid(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, const SkinnyIds &si,
+                        int64_t grid, int waves, hipStream_t s) {
+    typedef SkinnyGeo<S, NCT, NST> Geo;
     const size_t lds = (size_t)waves * (Geo::WAVE_BYTES + Geo::PART_BYTES);
     // more than 64 KiB of dynamic LDS has to be allowed once per device
     static bool allowed[64] = {false};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_kernel<S, NCT, ID>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_kernel<S, NCT, ID, NST>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    // More row groups than fit the GPU at once: launch one resident round of workgroups and let each walk
-    // through an equal share of the row groups (its copy stream never drains in between).  Expert-indexed
-    // launches keep one item per workgroup: their columns change from group to group.
+    skinny_kernel<S, NCT, ID, NST><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
+}
+
+template <class S, int NCT, bool ID>
+void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, const SkinnyIds &si,
+                      int64_t row_groups, int num_cus, hipStream_t s) {
+    const int waves = skinny_waves(row_groups, w.K / QKK, num_cus);
+    // More row groups than eight waves per CU: each workgroup walks through several of them, its copy
+    // stream continuing from one into the next.  Expert-indexed launches keep one item per workgroup:
+    // their columns change from group to group.
     int64_t grid = row_groups;
-    if (!ID) {
-        const int64_t by_lds = (160 * 1024) / (int64_t)(Geo::WAVE_BYTES + Geo::PART_BYTES), by_regs = Geo::SETS >= 4 ? 8 : 16;
-        const int64_t wgs_per_cu = (by_lds < by_regs ? by_lds : by_regs) / waves;
-        const int64_t resident = (int64_t)num_cus * (wgs_per_cu < 1 ? 1 : wgs_per_cu);
-        const int64_t rounds = (row_groups + resident - 1) / resident;
-        grid = (row_groups + rounds - 1) / rounds;
+    if (!ID && waves == 1) {
+        const int64_t items = (row_groups + (int64_t)num_cus * 4) / ((int64_t)num_cus * 8);  // nearest, at least 1
+        if (items > 1) grid = (row_groups + items - 1) / items;
     }
-    skinny_kernel<S, NCT, ID><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
+    launch_skinny_grid<S, NCT, ID, 2>(w, a, col0, ncols, y, si, grid, waves, s);
 }
 
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
