@@ -58,9 +58,9 @@ enum { MI_QMM_HOST = 0, MI_QMM_DEVICE = 1 };
 /* kernel selection for mi_qmm_mulmat_path */
 enum {
     MI_QMM_PATH_AUTO = 0, /* decode kernels below N = 32, tiled int8-MFMA GEMM from N = 32             */
-    MI_QMM_PATH_GEMV = 1, /* the decode kernels at any N: streaming GEMV, 8 columns at a time; K-quant
-                             weights go to the skinny matrix-core kernel from 3 (Q4_K) / 4 (Q6_K)
-                             columns, 16 at a time                                                   */
+    MI_QMM_PATH_GEMV = 1, /* the decode kernels at any N: streaming GEMV, 8 columns at a time; from
+                             3 (Q4_K) / 4 (Q6_K, Q4_0, Q8_0) columns the skinny matrix-core kernels,
+                             16 columns at a time                                                    */
     MI_QMM_PATH_GEMM = 2  /* force the tiled int8-MFMA GEMM (any N >= 1, padded to the tile)          */
 };
 

@@ -414,10 +414,11 @@ int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k,
 // ---- the product ------------------------------------------------------------------------------------
 namespace {
 
-// From this many activation columns up a K-quant product below the GEMM's batch goes to the
-// matrix-core skinny kernel instead of the streaming GEMV (measured crossover on MI355X: the GEMV pays
-// one v_dot4 pass per column).
+// From this many activation columns up a product below the GEMM's batch goes to a matrix-core skinny
+// kernel instead of the streaming GEMV (measured crossovers on MI355X: the GEMV pays one v_dot4 pass
+// per column).
 bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
+    if (type == T_Q4_0 || type == T_Q8_0) return n >= 4 && skinny32_supports(type, K, M);
     const int64_t from = type == T_Q4_K ? 3 : 4;
     return n >= from && skinny_supports(type, K, M);
 }
@@ -446,7 +447,11 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
         }
         HIP_TRY(launch_gemm(w->dev, a, dy, M, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
     } else {
-        if (a.sd8 && wants_skinny(w->dev.type, K, M, n)) {
+        if (blk32 && wants_skinny(w->dev.type, K, M, n)) {
+            for (int64_t c0 = 0; c0 < n; c0 += 16)
+                HIP_TRY(launch_skinny32(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus,
+                                        ctx->stream));
+        } else if (a.sd8 && wants_skinny(w->dev.type, K, M, n)) {
             // from a few columns up the K-quants go to the matrix cores, 16 columns per launch: the
             // streaming GEMV pays one v_dot4 pass per column
             for (int64_t c0 = 0; c0 < n; c0 += 16)

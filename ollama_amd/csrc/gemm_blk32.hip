@@ -27,6 +27,8 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void lds_ptr_t;
+typedef const __attribute__((address_space(1))) void glb_ptr_t;
 
 __device__ __forceinline__ float h2f(unsigned bits16) { return __half2float(__ushort_as_half((unsigned short)bits16)); }
 
@@ -179,9 +181,6 @@ __global__ __launch_bounds__(512, 2) void gemm_blk32_kernel(DevWeight w, DevAct 
 // own LDS region: no barriers in the loop, each wave waits on its own memory counter (every wave
 // issues exactly NDMA copies per stage, so "at most NDMA outstanding" means the older stage landed).
 // Pieces are XOR-swizzled with row bits so that the operand reads spread over the banks.
-typedef __attribute__((address_space(3))) void lds_ptr_t;
-typedef const __attribute__((address_space(1))) void glb_ptr_t;
-
 template <bool Q4>
 struct DmaGeo {
     static constexpr int W_BYTES = Q4 ? 1024 : 2048;  // 32 rows x 2 blocks
@@ -330,7 +329,238 @@ __global__ __launch_bounds__(512, 1) void gemm_blk32_dma_kernel(DevWeight w, Dev
     store_tile(acc, nullptr, 1, 0, lane, m0, n0, w.M, a.N, y);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny product (a few activation columns: small-batch decode) for Q4_0 / Q8_0 on the matrix cores.
+// The streaming GEMV pays one v_dot4 pass per column; here the columns share one
+// v_mfma_i32_16x16x64_i8 per 16 weight rows and 64 elements.  A 64-wide step is two blocks (K groups
+// 0,1 and 2,3), so the 16 rows of the A operand are 8 columns x the 2 blocks of the step: row r is
+// column r>>1 restricted to the K groups of block r&1, zeros elsewhere (those lanes read a zero slot).
+// Lane l then holds, for weight row l%16, the integer block sums of columns 2(l>>4), 2(l>>4)+1 with both
+// blocks of the step, and scales each with d_w * d_x in fp32 -- ggml's order of operations.  Q4_0 quants
+// stay unsigned nibbles; the -8 goes through the activations' block sums.
+// Same shape as the K-quant skinny kernel: a workgroup owns 16 weight rows, its waves cut K in runs
+// of 256 elements and stream weights, activations and both sides' scales through private two-stage LDS
+// rings with direct-to-LDS loads; one barrier at the end for the sum over the K cuts.
+// ---------------------------------------------------------------------------------------------
+typedef int v4acc __attribute__((ext_vector_type(4)));
+
+template <bool Q4, int NCT>
+struct Sk32Geo {
+    static constexpr int W_BYTES = Q4 ? 2048 : 4096, W_INSTRS = W_BYTES / 1024;  // 16 rows x 256 elements
+    static constexpr int DW_OFF = W_BYTES;                 // 16 rows x 8 fp16
+    static constexpr int A_OFF = DW_OFF + 256;             // NCT columns x 256 quants
+    static constexpr int A_INSTRS = NCT / 4;
+    static constexpr int DX_OFF = A_OFF + NCT * 256;       // NCT columns x 8 f32
+    static constexpr int BS_OFF = DX_OFF + NCT * 32;       // NCT columns x 8 i16 (Q4_0)
+    static constexpr int Z_OFF = BS_OFF + (Q4 ? NCT * 16 : 0);
+    static constexpr int STAGE = (Z_OFF + 16 + 63) / 64 * 64;
+    static constexpr int NDMA = W_INSTRS + 1 + A_INSTRS + 1 + (Q4 ? 1 : 0);
+    static constexpr int WAVE_BYTES = (2 * STAGE + 255) / 256 * 256;
+    static constexpr int PART_BYTES = 16 * 16 * 4;
+    static constexpr int SETS = NCT / 8;
+};
+
+template <bool Q4, int NCT>
+__global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y) {
+    typedef Sk32Geo<Q4, NCT> Geo;
+    constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, SETS = Geo::SETS;
+    const int WAVES = blockDim.x >> 6;
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
+    float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * Geo::WAVE_BYTES);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int64_t m0 = (int64_t)blockIdx.x * 16;
+    const int rows_left = (int)min((int64_t)16, w.M - m0);
+    const int64_t nblk = w.K / QK, nst = w.K / 256;
+    const int64_t s0 = nst * wave / WAVES, s1 = nst * (wave + 1) / WAVES;  // this wave's run of 256-element steps
+    uint8_t *wsm = smem + wave * Geo::WAVE_BYTES;
+
+    // ---- copy plan
+    unsigned woff[Geo::W_INSTRS], aoff[Geo::A_INSTRS];
+#pragma unroll
+    for (int i = 0; i < Geo::W_INSTRS; i++) {
+        const int idx = 64 * i + lane;
+        if (Q4) {
+            const int r = idx >> 3, slot = idx & 7, piece = slot ^ ((r >> 1) & 7);  // piece = block of the step
+            woff[i] = (unsigned)min(r, rows_left - 1) * (unsigned)(nblk * 16) + 16u * piece;
+        } else {
+            const int r = idx >> 4, slot = idx & 15, piece = slot ^ r;  // piece = 16 quants
+            woff[i] = (unsigned)min(r, rows_left - 1) * (unsigned)w.K + 16u * piece;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < Geo::A_INSTRS; j++) {
+        const int col = 4 * j + (lane >> 4), slot = lane & 15;  // stage slot [col][slot] holds piece slot ^ col
+        aoff[j] = (unsigned)(col0 + min(col, nc - 1)) * (unsigned)a.K + 16u * (slot ^ col);
+    }
+    const unsigned dwoff = (unsigned)min(c, rows_left - 1) * (unsigned)nblk * 2u;
+    const unsigned dxoff = (unsigned)(col0 + min(lane >> 1, nc - 1)) * (unsigned)nblk * 4u + 16u * (lane & 1);
+    const unsigned bsoff = (unsigned)(col0 + min(lane, nc - 1)) * (unsigned)nblk * 2u;
+    const uint8_t *wbase = w.p0 + m0 * (Q4 ? nblk * 16 : w.K);
+    const uint8_t *dwbase = reinterpret_cast<const uint8_t *>(w.d + m0 * nblk);
+    const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
+    const uint8_t *adx = reinterpret_cast<const uint8_t *>(a.d);
+    const uint8_t *abs_ = reinterpret_cast<const uint8_t *>(a.bsums);
+
+    auto stage_copy = [&](uint8_t *st, int64_t sp) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < Geo::W_INSTRS; i++) {
+            const uint8_t *gp = wbase + sp * (Q4 ? 128 : 256) + woff[i];
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * i), 16, 0, 0);
+        }
+        {
+            const uint8_t *gp = dwbase + sp * 16 + dwoff;
+            if (lane < 16) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DW_OFF), 16, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < Geo::A_INSTRS; j++) {
+            const uint8_t *gp = aq + sp * 256 + aoff[j];
+            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::A_OFF + 1024 * j), 16, 0, 0);
+        }
+        {
+            const uint8_t *gp = adx + sp * 32 + dxoff;
+            if (lane < 2 * NCT) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DX_OFF), 16, 0, 0);
+        }
+        if (Q4) {
+            const uint8_t *gp = abs_ + sp * 16 + bsoff;
+            if (lane < NCT) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::BS_OFF), 16, 0, 0);
+        }
+    };
+
+    // ---- operand reads.  A row r = lane & 15 of column set cs is column 8 cs + (r >> 1), block r & 1 of
+    // the step; lanes of the other block's K groups, and columns past nc, read the zero slot.
+    if (lane < 8) *reinterpret_cast<int *>(wsm + (lane >> 2) * STAGE + Geo::Z_OFF + 4 * (lane & 3)) = 0;
+    int aro[SETS][4], lcol[SETS][2];
+#pragma unroll
+    for (int cs = 0; cs < SETS; cs++) {
+        const int col = 8 * cs + (c >> 1);
+        const bool on = col < nc && (g >> 1) == (c & 1);
+#pragma unroll
+        for (int t = 0; t < 4; t++) aro[cs][t] = on ? Geo::A_OFF + col * 256 + 16 * ((4 * t + g) ^ col) : Geo::Z_OFF;
+#pragma unroll
+        for (int u = 0; u < 2; u++) lcol[cs][u] = min(8 * cs + 2 * g + u, NCT - 1);  // the lane's output columns
+    }
+
+    float acc[SETS][2];
+#pragma unroll
+    for (int cs = 0; cs < SETS; cs++) acc[cs][0] = acc[cs][1] = 0.f;
+    if (s0 < s1) {
+        stage_copy(wsm, s0);
+        stage_copy(wsm + STAGE, min(s0 + 1, s1 - 1));
+        const v4acc zero = {0, 0, 0, 0};
+#pragma unroll 1
+        for (int64_t sp = s0; sp < s1; sp++) {
+            uint8_t *st = wsm + ((sp - s0) & 1) * STAGE;
+            __builtin_amdgcn_s_waitcnt((NDMA & 15) | (7 << 4) | (15 << 8) | ((NDMA >> 4) << 14));
+            v4i bq[4], av[SETS][4];
+            uint4 dxr[SETS][2][2], bsr[SETS][2];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                if (Q4) bq[t] = *reinterpret_cast<const v4i *>(st + c * 128 + 16 * ((2 * t + (g >> 1)) ^ ((c >> 1) & 7)));
+                else bq[t] = *reinterpret_cast<const v4i *>(st + c * 256 + 16 * ((4 * t + g) ^ c));
+            }
+            const uint4 dwr = *reinterpret_cast<const uint4 *>(st + Geo::DW_OFF + 16 * c);
+#pragma unroll
+            for (int cs = 0; cs < SETS; cs++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) av[cs][t] = *reinterpret_cast<const v4i *>(st + aro[cs][t]);
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    dxr[cs][u][0] = *reinterpret_cast<const uint4 *>(st + Geo::DX_OFF + 32 * lcol[cs][u]);
+                    dxr[cs][u][1] = *reinterpret_cast<const uint4 *>(st + Geo::DX_OFF + 32 * lcol[cs][u] + 16);
+                    if (Q4) bsr[cs][u] = *reinterpret_cast<const uint4 *>(st + Geo::BS_OFF + 16 * lcol[cs][u]);
+                }
+            }
+            // operands are in registers: the stage can take the copies of step sp + 2
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            stage_copy(st, min(sp + 2, s1 - 1));
+            if (Q4) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) bq[t][i] = (int)(((unsigned)bq[t][i] >> (4 * (g & 1))) & 0x0f0f0f0fu);
+            }
+            const unsigned dwp[4] = {dwr.x, dwr.y, dwr.z, dwr.w};
+            float dwf[8];
+#pragma unroll
+            for (int b = 0; b < 8; b++) dwf[b] = h2f(b & 1 ? dwp[b >> 1] >> 16 : dwp[b >> 1] & 0xffff);
+#pragma unroll
+            for (int cs = 0; cs < SETS; cs++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const v4acc dv = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[cs][t], bq[t], zero, 0, 0, 0);
+#pragma unroll
+                    for (int u = 0; u < 2; u++) {
+                        const unsigned dxp[8] = {dxr[cs][u][0].x, dxr[cs][u][0].y, dxr[cs][u][0].z, dxr[cs][u][0].w,
+                                                 dxr[cs][u][1].x, dxr[cs][u][1].y, dxr[cs][u][1].z, dxr[cs][u][1].w};
+                        const unsigned bsp[4] = {bsr[cs][u].x, bsr[cs][u].y, bsr[cs][u].z, bsr[cs][u].w};
+#pragma unroll
+                        for (int sblk = 0; sblk < 2; sblk++) {
+                            const int b = 2 * t + sblk;
+                            int iv = dv[2 * u + sblk];
+                            if (Q4) {
+                                const int bs = (int)(short)(b & 1 ? bsp[b >> 1] >> 16 : bsp[b >> 1] & 0xffff);
+                                iv -= 8 * bs;  // sum (q - 8) x = sum q x - 8 sum x
+                            }
+                            acc[cs][u] = __builtin_fmaf((float)iv, dwf[b] * __uint_as_float(dxp[b]), acc[cs][u]);
+                        }
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0);  // the repeated copies of the last iterations must not outlive the kernel's LDS
+    }
+#pragma unroll
+    for (int cs = 0; cs < SETS; cs++)
+#pragma unroll
+        for (int u = 0; u < 2; u++) part[wave][8 * cs + 2 * g + u][c] = acc[cs][u];
+    __syncthreads();
+    for (int o = tid; o < 16 * NCT; o += blockDim.x) {
+        const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
+        float sum = 0.f;
+        for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
+        if (i < nc && j < rows_left) y[(int64_t)(col0 + i) * w.M + m0 + j] = sum;
+    }
+}
+
+template <bool Q4, int NCT>
+void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
+    typedef Sk32Geo<Q4, NCT> Geo;
+    const int64_t groups = (w.M + 15) / 16, nst = w.K / 256;
+    // about eight waves per CU over the whole grid (see the K-quant skinny kernel), every wave at least one step
+    const int64_t want = ((int64_t)num_cus * 8 + groups / 2) / groups;
+    int waves = want >= 8 ? 8 : want >= 6 ? 6 : want >= 4 ? 4 : want >= 3 ? 3 : want >= 2 ? 2 : 1;
+    while (waves > 1 && nst / waves < 1) waves = waves > 4 ? waves - 2 : waves - 1;
+    const size_t lds = (size_t)waves * (Geo::WAVE_BYTES + Geo::PART_BYTES);
+    static bool allowed[64] = {false};  // more than 64 KiB of dynamic LDS has to be allowed once per device
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny32_kernel<Q4, NCT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        allowed[dev] = true;
+    }
+    skinny32_kernel<Q4, NCT><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y);
+}
+
 }  // namespace
+
+bool skinny32_supports(int type, int64_t K, int64_t M) {
+    return (type == T_Q4_0 || type == T_Q8_0) && K >= 256 && K % 256 == 0 && M >= 1 && (M + 15) / 16 <= 0x7fffffff;
+}
+
+hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
+    if (!skinny32_supports(w.type, w.K, w.M) || a.type != T_Q8_0 || a.K != w.K || !y) return hipErrorInvalidValue;
+    if (ncols < 1 || ncols > 16 || col0 < 0 || col0 + ncols > a.N) return hipErrorInvalidValue;
+    if ((int64_t)(col0 + ncols) * a.K >= ((int64_t)1 << 32) || (w.type == T_Q4_0 && !a.bsums)) return hipErrorInvalidValue;
+    if (w.type == T_Q4_0) {
+        if (ncols <= 8) launch_skinny32_as<true, 8>(w, a, col0, ncols, y, num_cus, s);
+        else launch_skinny32_as<true, 16>(w, a, col0, ncols, y, num_cus, s);
+    } else {
+        if (ncols <= 8) launch_skinny32_as<false, 8>(w, a, col0, ncols, y, num_cus, s);
+        else launch_skinny32_as<false, 16>(w, a, col0, ncols, y, num_cus, s);
+    }
+    return hipGetLastError();
+}
 
 bool gemm_blk32_supports(int type, int64_t K, int64_t M) {
     return (type == T_Q4_0 || type == T_Q8_0) && K >= QK && K % QK == 0 && M >= 1;

@@ -71,6 +71,11 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
 bool gemm_blk32_supports(int type, int64_t K, int64_t M);
 hipError_t launch_gemm_blk32(const DevWeight &w, const DevAct &a, float *y, int num_cus, hipStream_t s);
 
+// 1..16 activation columns on the matrix cores for Q4_0 / Q8_0 (K a multiple of 256); y[n*M + m]
+bool skinny32_supports(int type, int64_t K, int64_t M);
+hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
+                           hipStream_t s);
+
 // Expert-indexed product on the matrix cores (K-quants): the pairs are bucketed by expert, 16 per group;
 // a needs the block-sum digit planes.  groups: device scratch of gemv_id_scratch_ints(pairs) ints.
 bool skinny_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);

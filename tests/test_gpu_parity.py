@@ -600,3 +600,38 @@ def test_page_locked_host_buffers(ctx):
     assert np.array_equal(y, ctx.mulmat(w, np.array(x)))
     assert ctx.host_array((0, 4)).shape == (0, 4)
     w.free()
+
+
+# ---- skinny product on the matrix cores for the 32-element block formats ------------------------------
+@pytest.mark.parametrize("t", [Q4_0, Q8_0])
+@pytest.mark.parametrize("m,k,n", [(4096, 4096, 8), (1000, 1024, 5), (17, 256, 4), (300, 2304, 16), (64, 8192, 31),
+                                   (4096, 14336, 7)])
+def test_skinny32_matches_oracle(ctx, t, m, k, n):
+    """4..31 columns, K a multiple of 256: ragged M, one 256-element step, K cut eight ways, two launches"""
+    rng = np.random.default_rng(7900 + t + m + n)
+    wb = _weights(t, m, k, 7901 + t + m)
+    w = ctx.upload(t, wb, k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(w, x)
+    assert npref.rel_err(got, oracle.mul_mat(t, wb, k, m, x, nthreads=16)) < TOL
+    # a column's result does not depend on which other columns ride along
+    assert np.array_equal(ctx.mulmat(w, x[::-1].copy())[::-1], got)
+    w.free()
+
+
+def test_skinny32_exact_integer_case(ctx):
+    """operands whose products and sums are exact in fp32: a misplaced byte, nibble, block sum or scale
+    shows as a wrong integer"""
+    k, m, n = 512, 48, 6
+    rng = np.random.default_rng(7950)
+    for t in (Q4_0, Q8_0):
+        lim = 7 if t == Q4_0 else 127
+        wi = rng.integers(-lim, lim + 1, (m, k)).astype(np.float32)
+        wi[:, ::32] = -8 if t == Q4_0 else 127  # pins every block's scale to exactly 1.0
+        xi = rng.integers(-127, 128, (n, k)).astype(np.float32)
+        xi[:, 1::32] = 127
+        wb = oracle.quantize(t, wi)
+        w = ctx.upload(t, wb, k, m)
+        got = ctx.mulmat(w, xi)
+        assert np.array_equal(got, (xi.astype(np.float64) @ wi.astype(np.float64).T).astype(np.float32))
+        w.free()
