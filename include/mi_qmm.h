@@ -146,6 +146,14 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
 int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
                      const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location);
 
+/* several expert stacks against the same x and ids (gate and up of an expert FFN): ys[i] receives
+ * f32 [n_tokens][n_used][rows_per_expert_i].  Stacks of one type and shape go out two at a time with x
+ * quantized once; for decode-sized calls such a pair is ONE kernel launch.  Results are those of
+ * mi_qmm_mulmat_id per stack. */
+int mi_qmm_mulmat_id_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int n_expert,
+                           const float *x, int b_cols, const int32_t *ids, int n_used, int64_t n_tokens,
+                           float *const *ys, int location);
+
 /* ---- two-phase form: quantize once, multiply by several weights (gate and up, or q/k/v, share
  *      one x).  In ggml's graph the from_float step belongs to each mul_mat node; a backend that
  *      sees the whole graph at Context.Compute (/root/reference/ml/backend.go:110) may hoist it,

@@ -619,10 +619,18 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
     return MI_QMM_OK;
 }
 
-int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
-                     const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location) {
+}  // extern "C"
+
+namespace {
+
+// w2 / y2 (optional): a second stack of w's type and shape multiplied by the same activations and ids;
+// x is quantized once for both and the decode launch covers both.
+int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight *w2, int n_expert, const float *x,
+                   int b_cols, const int32_t *ids, int n_used, int64_t n_tokens, float *y, float *y2, int location) {
     int rc = check_product_args(ctx, w, location, MI_QMM_PATH_AUTO);
     if (rc) return rc;
+    if (w2 && (w2->device != ctx->device || w2->dev.type != w->dev.type || w2->dev.K != w->dev.K || w2->dev.M != w->dev.M))
+        return fail(MI_QMM_ERR_INVALID, "the two expert stacks differ in device, type or shape");
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
         return fail(MI_QMM_ERR_INVALID, "n_expert=%d n_used=%d b_cols=%d n_tokens=%lld: all must be positive", n_expert,
                     n_used, b_cols, (long long)n_tokens);
@@ -632,7 +640,7 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
                     n_expert);
     const int64_t M = w->dev.M / n_expert;
     if (n_tokens == 0) return MI_QMM_OK;
-    if (!x || !ids || !y) return fail(MI_QMM_ERR_INVALID, "x, ids or y is NULL");
+    if (!x || !ids || !y || (w2 && !y2)) return fail(MI_QMM_ERR_INVALID, "x, ids or y is NULL");
     const int64_t pairs = (int64_t)n_used * n_tokens, ncols = (int64_t)b_cols * n_tokens;
     if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24) || K > gemv_max_k(w->dev.type))
         return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts, 2^24 pairs and k <= %lld for type %d",
@@ -651,13 +659,14 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
     const size_t xbytes = (size_t)(ncols * K) * 4, ibytes = (size_t)pairs * 4, ybytes = (size_t)(pairs * M) * 4;
     const float *dx = x;
     const int32_t *dids = ids;
-    float *dy = y;
+    float *dy = y, *dy2 = y2;
     if (location == MI_QMM_HOST) {
-        const size_t ioff = align_up(xbytes, 256), yoff = ioff + align_up(ibytes, 256);
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, yoff + ybytes, ctx->stream))) return rc;
+        const size_t ioff = align_up(xbytes, 256), yoff = ioff + align_up(ibytes, 256), yoff2 = yoff + align_up(ybytes, 256);
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, yoff2 + (w2 ? ybytes : 0), ctx->stream))) return rc;
         dx = (const float *)ctx->io_buf;
         dids = (const int32_t *)((char *)ctx->io_buf + ioff);
         dy = (float *)((char *)ctx->io_buf + yoff);
+        if (w2) dy2 = (float *)((char *)ctx->io_buf + yoff2);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
         HIP_TRY(hipMemcpyAsync((void *)dids, ids, ibytes, hipMemcpyHostToDevice, ctx->stream));
     }
@@ -670,16 +679,47 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
         HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
         a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16;
     }
-    if (skinny)
+    if (skinny) {
         // a few pairs per expert and more: on the matrix cores, the experts' weights read once per 16 pairs
         HIP_TRY(launch_skinny_id(w->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy, (int *)ctx->ws_buf,
                                  ctx->num_cus, ctx->stream));
-    else
+        if (w2)
+            HIP_TRY(launch_skinny_id(w2->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy2, (int *)ctx->ws_buf,
+                                     ctx->num_cus, ctx->stream));
+    } else {
         HIP_TRY(launch_gemv_id(w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
-                               (int *)ctx->ws_buf, ctx->stream));
+                               (int *)ctx->ws_buf, ctx->stream, w2 ? &w2->dev : nullptr, dy2));
+    }
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+        if (w2) HIP_TRY(hipMemcpyAsync(y2, dy2, ybytes, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
+                     const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location) {
+    return mulmat_id_impl(ctx, w, nullptr, n_expert, x, b_cols, ids, n_used, n_tokens, y, nullptr, location);
+}
+
+int mi_qmm_mulmat_id_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int n_expert, const float *x,
+                           int b_cols, const int32_t *ids, int n_used, int64_t n_tokens, float *const *ys, int location) {
+    if (!ws || !ys || count < 1) return fail(MI_QMM_ERR_INVALID, "ws/ys is NULL or count < 1");
+    for (int i = 0; i < count; i++)
+        if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
+    for (int i = 0; i < count;) {
+        // stacks of one type and shape go out two at a time
+        const bool pair = i + 1 < count && ws[i + 1]->dev.type == ws[i]->dev.type && ws[i + 1]->dev.K == ws[i]->dev.K &&
+                          ws[i + 1]->dev.M == ws[i]->dev.M;
+        int rc = mulmat_id_impl(ctx, ws[i], pair ? ws[i + 1] : nullptr, n_expert, x, b_cols, ids, n_used, n_tokens, ys[i],
+                                pair ? ys[i + 1] : nullptr, location);
+        if (rc) return rc;
+        i += pair ? 2 : 1;
     }
     return MI_QMM_OK;
 }

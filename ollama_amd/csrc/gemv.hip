@@ -985,6 +985,12 @@ struct IdArgs {
     float *y;              // [pairs][M]
     int64_t M;             // rows per expert
     int n_expert, pairs, n_used, b_cols, wgs_per_group;
+    // a second stack of the same type and shape against the same activations and ids (gate and up of an
+    // expert FFN): the workgroups from wgs_first on belong to it.  wgs_first = INT_MAX: one stack.
+    const uint8_t *p0b, *p1b, *p2b;
+    const uint16_t *db;
+    float *yb;
+    int wgs_first;
 };
 
 // One workgroup of 1024 threads buckets the pairs by expert: counts in LDS, group ranges from a
@@ -1038,7 +1044,12 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     static_assert(!F32 || NC == 1, "the f32 prologue quantizes one activation row");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int REC = 2 + NC;
-    const int group = blockIdx.x / ia.wgs_per_group, wg = blockIdx.x - group * ia.wgs_per_group;
+    const bool second = (int)blockIdx.x >= ia.wgs_first;
+    const int bid = (int)blockIdx.x - (second ? ia.wgs_first : 0);
+    const DevWeight w{second ? ia.p0b : ia.w.p0, second ? ia.p1b : ia.w.p1, second ? ia.p2b : ia.w.p2,
+                      second ? ia.db : ia.w.d, ia.w.K, ia.w.M, ia.w.type};
+    float *__restrict__ y = second ? ia.yb : ia.y;
+    const int group = bid / ia.wgs_per_group, wg = bid - group * ia.wgs_per_group;
     int expert, count, pair[NC];
     if (ia.groups) {
         if (group >= ia.groups[0]) return;
@@ -1065,7 +1076,7 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
         // an id outside the stack: the pair's output is all NaN
         for (int i = threadIdx.x; i < nrows * count; i += blockDim.x) {
             const int n = i / nrows, rl = i - n * nrows;
-            ia.y[(int64_t)pair[n] * M + r0 + rl] = __int_as_float(0x7fc00000);
+            y[(int64_t)pair[n] * M + r0 + rl] = __int_as_float(0x7fc00000);
         }
         return;
     }
@@ -1074,14 +1085,14 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     const int64_t wrow0 = (int64_t)expert * M + r0 + rl0;  // row inside the stack
 
     const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);
-    const typename P::Geo g = P::geo(ia.w, kseg, vlane);
+    const typename P::Geo g = P::geo(w, kseg, vlane);
     int col[NC];  // activation row of each pair: token * b_cols + slot mod b_cols
 #pragma unroll
     for (int n = 0; n < NC; n++) {
         const int tok = pair[n] / ia.n_used, slot = pair[n] - tok * ia.n_used;
         col[n] = tok * ia.b_cols + slot % ia.b_cols;
     }
-    const int64_t K = ia.w.K;
+    const int64_t K = w.K;
     const int nblk = (int)(K / P::ACT_BLK);
     const size_t act_bytes = F32 ? ((size_t)(K + nblk * 4 + (P::USES_BSUMS ? K / P::ACT_BSUM * 2 : 0)) + 15) / 16 * 16 : 0;
     int8_t *lqs = reinterpret_cast<int8_t *>(smem);
@@ -1092,7 +1103,7 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     float4 xpre[XPRE];
     if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     typename P::Raw cur;
-    if (nrw > 0) cur = P::load(ia.w, g, wrow0 + min(run, nrw - 1));
+    if (nrw > 0) cur = P::load(w, g, wrow0 + min(run, nrw - 1));
     if (F32) {
         quantize_x_to_lds<P>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
         __syncthreads();
@@ -1108,11 +1119,11 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
             for (int n = 0; n < NC; n++) P::load_act(a, col[n], kseg, vlane, g, act[n]);
         }
         float keep[NC];
-        thin_rows<P, NC, DIRECT, RPL>(ia.w, g, cur, act, wrow0, nrw, lane, keep, part, rl0, kw, kseg);
+        thin_rows<P, NC, DIRECT, RPL>(w, g, cur, act, wrow0, nrw, lane, keep, part, rl0, kw, kseg);
         if (DIRECT && lane > 63 - nrw) {
 #pragma unroll
             for (int n = 0; n < NC; n++)
-                if (n < count) ia.y[(int64_t)pair[n] * M + r0 + rl0 + (63 - lane)] = keep[n];
+                if (n < count) y[(int64_t)pair[n] * M + r0 + rl0 + (63 - lane)] = keep[n];
         }
     }
     if (DIRECT) return;
@@ -1121,14 +1132,14 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
         const int n = i / nrows, rl = i - n * nrows;
         float sum = 0.f;
         for (int k = 0; k < kw; k++) sum += part[(rl * NC + n) * kw + k];
-        ia.y[(int64_t)pair[n] * M + r0 + rl] = sum;
+        y[(int64_t)pair[n] * M + r0 + rl] = sum;
     }
 }
 
 template <class P, int NC>
 hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, int *groups, hipStream_t s) {
     Plan p;
-    if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M, NC, false, p)) return hipErrorInvalidValue;
+    if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC, false, p)) return hipErrorInvalidValue;
     const size_t act_lds = xf ? thin_act_lds<P>(ia.w.K, 1) : 0;
     if (xf && (NC != 1 || act_lds + p.lds > THIN_LDS_MAX)) return hipErrorInvalidValue;
     const int64_t wgs_per_group = (ia.M + p.rows_per_wg - 1) / p.rows_per_wg;
@@ -1141,9 +1152,11 @@ hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, int *groups
     } else {
         ia.groups = nullptr;
     }
-    if (wgs_per_group * max_groups > 0x7fffffff) return hipErrorInvalidValue;
+    const int stacks = ia.yb ? 2 : 1;
+    if (wgs_per_group * max_groups * stacks > 0x7fffffff) return hipErrorInvalidValue;
     ia.wgs_per_group = (int)wgs_per_group;
-    const dim3 grid((unsigned)(wgs_per_group * max_groups)), block(64 * p.kw * p.rw);
+    ia.wgs_first = stacks == 2 ? (int)(wgs_per_group * max_groups) : 0x7fffffff;
+    const dim3 grid((unsigned)(wgs_per_group * max_groups * stacks)), block(64 * p.kw * p.rw);
     const int rpw = p.rows_per_wg >> p.rw_log2;
     const size_t lds = act_lds + p.lds;
 #define ID_LAUNCH(N, DIRECT, F32, RPL) \
@@ -1202,7 +1215,10 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
 }
 
 hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,
-                          int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s) {
+                          int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s,
+                          const DevWeight *w2, float *y2) {
+    if ((w2 != nullptr) != (y2 != nullptr) || (w2 && (w2->type != w.type || w2->K != w.K || w2->M != w.M)))
+        return hipErrorInvalidValue;
     if (n_expert < 1 || n_expert > ID_MAX_EXPERTS || w.M % n_expert || n_used < 1 || n_tokens < 1 || b_cols < 1 || !ids || !y || !groups || a.K != w.K || a.N != (int64_t)b_cols * n_tokens ||
         (int64_t)n_used * n_tokens > 0x7fffffff / 16)
         return hipErrorInvalidValue;
@@ -1210,6 +1226,7 @@ hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, con
     IdArgs ia{};
     ia.w = w; ia.ids = ids; ia.y = y; ia.M = w.M / n_expert;
     ia.n_expert = n_expert; ia.pairs = n_used * n_tokens; ia.n_used = n_used; ia.b_cols = b_cols;
+    if (w2) { ia.p0b = w2->p0; ia.p1b = w2->p1; ia.p2b = w2->p2; ia.db = w2->d; ia.yb = y2; }
     switch (w.type) {
     case T_Q4_K: return a.type == T_Q8_K ? launch_id_type<PolQ4K>(ia, a, xf, groups, s) : hipErrorInvalidValue;
     case T_Q6_K: return a.type == T_Q8_K ? launch_id_type<PolQ6K>(ia, a, xf, groups, s) : hipErrorInvalidValue;

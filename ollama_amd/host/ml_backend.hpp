@@ -164,17 +164,25 @@ public:
     // GEMV launch; larger ones share one quantization of x.
     void Compute() {
         std::map<std::pair<Tensor *, int>, std::vector<Tensor *>> by_x;
+        // expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
+        std::map<std::pair<std::pair<Tensor *, Tensor *>, int>, std::vector<Tensor *>> by_xi;
         for (auto &n : nodes_) {
             if (n->ready_) continue;
-            if (!n->op_ids_) {
-                by_x[{n->op_x_.get(), n->op_w_->type_}].push_back(n.get());
-                continue;
+            if (!n->op_ids_) by_x[{n->op_x_.get(), n->op_w_->type_}].push_back(n.get());
+            else by_xi[{{n->op_x_.get(), n->op_ids_.get()}, n->op_w_->Dim(2)}].push_back(n.get());
+        }
+        for (auto &kv : by_xi) {
+            const Tensor &x = *kv.first.first.first, &ids = *kv.first.first.second;
+            std::vector<const mi_qmm_weight *> ws;
+            std::vector<float *> ys;
+            for (Tensor *t : kv.second) {
+                t->data_.assign((size_t)(t->op_w_->Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);
+                ws.push_back(t->op_w_->weight_);
+                ys.push_back(t->data_.data());
             }
-            const Tensor &w = *n->op_w_, &x = *n->op_x_, &ids = *n->op_ids_;
-            n->data_.assign((size_t)(w.Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);
-            check(mi_qmm_mulmat_id(b_.handle(), w.weight_, w.Dim(2), x.data_.data(), x.Dim(1), ids.ints_.data(), ids.Dim(0),
-                                   ids.Dim(1), n->data_.data(), MI_QMM_HOST));
-            n->ready_ = true;
+            check(mi_qmm_mulmat_id_multi(b_.handle(), ws.data(), (int)ws.size(), kv.first.second, x.data_.data(), x.Dim(1),
+                                         ids.ints_.data(), ids.Dim(0), ids.Dim(1), ys.data(), MI_QMM_HOST));
+            for (Tensor *t : kv.second) t->ready_ = true;
         }
         for (auto &kv : by_x) {
             Tensor *x = kv.first.first;

@@ -149,12 +149,18 @@ class Context:
             raise RuntimeError("Compute on a closed context")
         pending = [t for t in self._nodes if t._data is None and t._op is not None]
         c = self._b._ctx
+        # expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
+        by_xi: Dict[Tuple[int, int, int], List[Tensor]] = {}
         for t in [t for t in pending if t._ids is not None]:
-            w, x = t._op
-            tokens, n_used = t._ids.Dim(1), t._ids.Dim(0)
+            by_xi.setdefault((id(t._op[1]), id(t._ids), t._op[0].Dim(2)), []).append(t)
+        for nodes in by_xi.values():
+            x, ids = nodes[0]._op[1], nodes[0]._ids
+            tokens, n_used = ids.Dim(1), ids.Dim(0)
             b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
-            y = c.mulmat_id(w._weight, w.Dim(2), b, t._ids._data.reshape(tokens, n_used))
-            t._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
+            ys = c.mulmat_id_multi([t._op[0]._weight for t in nodes], nodes[0]._op[0].Dim(2), b,
+                                   ids._data.reshape(tokens, n_used))
+            for t, y in zip(nodes, ys):
+                t._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
         pending = [t for t in pending if t._ids is None]
         # group by activation tensor
         by_x: Dict[int, List[Tensor]] = {}

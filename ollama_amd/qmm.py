@@ -25,7 +25,7 @@ EXPORTS = [
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync", "mi_qmm_host_alloc", "mi_qmm_host_free",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
-    "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id",
+    "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
     "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
@@ -87,6 +87,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
     L.mi_qmm_host_alloc.restype = vp; L.mi_qmm_host_alloc.argtypes = [vp, ctypes.c_size_t]
     L.mi_qmm_host_free.restype = None; L.mi_qmm_host_free.argtypes = [vp, vp]
+    L.mi_qmm_mulmat_id_multi.restype = ci
+    L.mi_qmm_mulmat_id_multi.argtypes = [vp, ctypes.POINTER(vp), ci, ci, vp, ci, vp, ci, i64, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_id.restype = ci
     L.mi_qmm_mulmat_id.argtypes = [vp, vp, ci, vp, ci, vp, ci, i64, vp, ci]
     P = ctypes.POINTER
@@ -340,6 +342,27 @@ class Context:
                                       ids.ctypes.data_as(ctypes.c_void_p), n_used, t,
                                       y.ctypes.data_as(ctypes.c_void_p), HOST))
         return y
+
+    def mulmat_id_multi(self, ws, n_expert: int, b: np.ndarray, ids: np.ndarray):
+        """several expert stacks against the same b and ids; host arrays out"""
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        if b.ndim != 3 or ids.ndim != 2 or b.shape[0] != ids.shape[0] or any(b.shape[2] != w.k for w in ws):
+            raise ValueError(f"b {b.shape} / ids {ids.shape} do not fit [tokens, b_cols, k] / [tokens, n_used]")
+        t, n_used = ids.shape
+        ys = [np.empty((t, n_used, w.m // max(n_expert, 1)), dtype=np.float32) for w in ws]
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[y.ctypes.data_as(ctypes.c_void_p) for y in ys])
+        _check(lib().mi_qmm_mulmat_id_multi(self._h, wh, len(ws), n_expert, b.ctypes.data_as(ctypes.c_void_p), b.shape[1],
+                                            ids.ctypes.data_as(ctypes.c_void_p), n_used, t, yp, HOST))
+        return ys
+
+    def mulmat_id_multi_device(self, ws, n_expert: int, b_ptr: int, b_cols: int, ids_ptr: int, n_used: int,
+                               n_tokens: int, y_ptrs):
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[ctypes.c_void_p(int(p)) for p in y_ptrs])
+        _check(lib().mi_qmm_mulmat_id_multi(self._h, wh, len(ws), n_expert, ctypes.c_void_p(int(b_ptr)), b_cols,
+                                            ctypes.c_void_p(int(ids_ptr)), n_used, n_tokens, yp, DEVICE))
 
     def mulmat_id_device(self, w: Weight, n_expert: int, b_ptr: int, b_cols: int, ids_ptr: int, n_used: int,
                          n_tokens: int, y_ptr: int):

@@ -73,13 +73,16 @@ def test_python_mirror_expert_graph(tmp_path):
     rng = np.random.default_rng(81)
     gate = oracle.quantize(qmm.Q4_K, rng.standard_normal((n_expert * ff, k), dtype=np.float32) * np.float32(0.02))
     down = oracle.quantize(qmm.Q8_0, rng.standard_normal((n_expert * k, ff), dtype=np.float32) * np.float32(0.02))
+    up = oracle.quantize(qmm.Q4_K, rng.standard_normal((n_expert * ff, k), dtype=np.float32) * np.float32(0.02))
     path = str(tmp_path / "moe.gguf")
     gguf.write_gguf(path, {"general.architecture": "qwen3moe"},
                     [("blk.0.ffn_gate_exps.weight", qmm.Q4_K, [k, ff, n_expert], gate),
+                     ("blk.0.ffn_up_exps.weight", qmm.Q4_K, [k, ff, n_expert], up),
                      ("blk.0.ffn_down_exps.weight", qmm.Q8_0, [ff, k, n_expert], down)])
     b = ml.Backend(path)
     b.Load()
     wg, wd = b.Get("blk.0.ffn_gate_exps.weight"), b.Get("blk.0.ffn_down_exps.weight")
+    wu = b.Get("blk.0.ffn_up_exps.weight")
     assert wg.Shape() == [k, ff, n_expert] and wd.Shape() == [ff, k, n_expert]
     for tokens in (1, 9):
         ctx = b.NewContext()
@@ -88,12 +91,16 @@ def test_python_mirror_expert_graph(tmp_path):
         idv = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
         ids = ctx.FromInts(idv.reshape(-1), n_used, tokens)
         assert ids.DType() == ml.DType.I32
-        g = wg.MulmatID(ctx, ctx.FromFloats(xv.reshape(-1), k, 1, tokens), ids)
+        xt = ctx.FromFloats(xv.reshape(-1), k, 1, tokens)
+        g = wg.MulmatID(ctx, xt, ids)
+        u = wu.MulmatID(ctx, xt, ids)      # same x and ids as gate: one call for both at Compute
         d = wd.MulmatID(ctx, ctx.FromFloats(hv.reshape(-1), ff, n_used, tokens), ids)
         assert g.Shape() == [ff, n_used, tokens] and d.Shape() == [k, n_used, tokens]
-        ctx.Compute(g, d)
+        ctx.Compute(g, u, d)
         assert npref.rel_err(g.Floats().reshape(tokens, n_used, ff),
                              oracle.mul_mat_id(qmm.Q4_K, gate, k, ff, n_expert, xv, idv)) <= 1e-3
+        assert npref.rel_err(u.Floats().reshape(tokens, n_used, ff),
+                             oracle.mul_mat_id(qmm.Q4_K, up, k, ff, n_expert, xv, idv)) <= 1e-3
         assert npref.rel_err(d.Floats().reshape(tokens, n_used, k),
                              oracle.mul_mat_id(qmm.Q8_0, down, ff, k, n_expert, hv, idv)) <= 1e-3
         with pytest.raises(TypeError):

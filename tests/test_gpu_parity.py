@@ -635,3 +635,23 @@ def test_skinny32_exact_integer_case(ctx):
         got = ctx.mulmat(w, xi)
         assert np.array_equal(got, (xi.astype(np.float64) @ wi.astype(np.float64).T).astype(np.float32))
         w.free()
+
+
+@pytest.mark.parametrize("t,tokens", [(Q4_K, 1), (Q8_0, 2), (Q4_K, 40), (Q4_0, 64)])
+def test_mulmat_id_multi_equals_single_calls(ctx, t, tokens):
+    """gate and up of an expert FFN in one call (decode: one launch) give the bits of two single calls;
+    a third stack of another shape rides along on its own"""
+    rng = np.random.default_rng(8000 + t + tokens)
+    k, m, n_expert, n_used = 1024, 160, 10, 4
+    raws = [_experts(t, n_expert, m, k, 8001 + i) for i in range(2)] + [_experts(t, n_expert, 48, k, 8003)]
+    ws = [ctx.upload(t, r, k, r.shape[0]) for r in raws]
+    b = rng.standard_normal((tokens, 1, k), dtype=np.float32)
+    ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+    got = ctx.mulmat_id_multi(ws, n_expert, b, ids)
+    for w, y, r in zip(ws, got, raws):
+        assert np.array_equal(y, ctx.mulmat_id(w, n_expert, b, ids))
+        assert npref.rel_err(y, oracle.mul_mat_id(t, r, k, r.shape[0] // n_expert, n_expert, b, ids)) < TOL
+    with pytest.raises(qmm.QmmError):
+        ctx.mulmat_id_multi(ws, n_expert, b, np.full((tokens, n_used), n_expert, np.int32))
+    for w in ws:
+        w.free()
