@@ -651,10 +651,14 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
                 return fail(MI_QMM_ERR_INVALID, "ids[%lld] = %d is outside 0..%d", (long long)p, ids[p], n_expert - 1);
 
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
+    // batches with many pairs per expert: sort the pairs by expert and run the tiled GEMM per expert
+    const bool gemm = gemm_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
+    const int64_t max_tiles = gemm ? sort_pairs_max_tiles(pairs, n_expert) : 0, sorted_rows = 64 * max_tiles;
     const ActPlanes probe = plan_act(nullptr, q8, K, ncols);
     if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
     const ActPlanes p = plan_act(ctx->act_buf, q8, K, ncols);
-    if ((rc = reserve(&ctx->ws_buf, &ctx->ws_cap, gemv_id_scratch_ints(pairs) * sizeof(int), ctx->stream))) return rc;
+    const size_t scratch_ints = gemm ? (size_t)(1 + 2 * max_tiles + 2 * sorted_rows) : gemv_id_scratch_ints(pairs);
+    if ((rc = reserve(&ctx->ws_buf, &ctx->ws_cap, scratch_ints * sizeof(int), ctx->stream))) return rc;
 
     const size_t xbytes = (size_t)(ncols * K) * 4, ibytes = (size_t)pairs * 4, ybytes = (size_t)(pairs * M) * 4;
     const float *dx = x;
@@ -669,6 +673,21 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
         if (w2) dy2 = (float *)((char *)ctx->io_buf + yoff2);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
         HIP_TRY(hipMemcpyAsync((void *)dids, ids, ibytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    if (gemm) {
+        int *tiles = (int *)ctx->ws_buf, *src_col = tiles + 1 + 2 * max_tiles, *out_pair = src_col + sorted_rows;
+        HIP_TRY(launch_sort_pairs(dids, (int)pairs, n_expert, n_used, b_cols, tiles, src_col, out_pair, ctx->stream));
+        HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+        DevAct as;
+        as.qs = p.qs; as.d = p.d; as.bsums = p.bsums; as.sd8 = p.sd8; as.sd16 = p.sd16; as.K = K; as.N = (int)ncols; as.type = q8;
+        HIP_TRY(launch_gemm_id(w->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, dy, ctx->stream));
+        if (w2) HIP_TRY(launch_gemm_id(w2->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, dy2, ctx->stream));
+        if (location == MI_QMM_HOST) {
+            HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+            if (w2) HIP_TRY(hipMemcpyAsync(y2, dy2, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(hipStreamSynchronize(ctx->stream));
+        }
+        return MI_QMM_OK;
     }
     DevAct a{};
     a.K = K; a.N = (int)ncols; a.type = q8;

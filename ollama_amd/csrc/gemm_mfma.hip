@@ -243,9 +243,21 @@ struct GemmArgs {
 };
 
 // TNT = 32-row activation sub-tiles per wave: the workgroup tile is 128 weight rows x 64*TNT activation rows.
+// Expert GEMM (Tensor.MulmatID on a batch, /root/reference/ml/backend.go:153): ga holds one stack of
+// expert matrices of expert_rows rows each; the (token, slot) pairs are sorted by expert into runs of whole
+// 64-row tiles (sort_pairs_kernel), tile_n picks a run's tile from the table and with it the expert.  The
+// activation planes stay in their own order: every copy gathers its rows through src_rows, and out_rows
+// maps a sorted row to the pair whose output row it is.
+struct GemmIds {
+    const int *tiles;     // null: an ordinary launch
+    const int *src_rows;  // sorted row -> row of the activation planes (-1: padding)
+    const int *out_rows;  // sorted row -> pair (-1: padding)
+    int64_t expert_rows;
+};
+
 template <class G, int TNT>
 __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel(GemmArgs ga, DevAct a, int tiles_m, int tiles_n,
-                                                                             float *__restrict__ part) {
+                                                                             float *__restrict__ part, GemmIds gi) {
     constexpr int WAVES = 8, TN = 64 * TNT, TM = 128;
     typedef Stage3<G, TN> StageT;
     __shared__ __attribute__((aligned(1024))) StageT lds[2];
@@ -263,13 +275,30 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
     const DevWeight w{GEMM_SEL(p0), GEMM_SEL(p1), GEMM_SEL(p2), GEMM_SEL(d), ga.K, GEMM_SEL(M), ga.type};
     float *__restrict__ y = GEMM_SEL(y);
 #undef GEMM_SEL
-    const int64_t ldy = w.M;
+    int64_t ldy = w.M, m_rows = w.M, m_stack = 0;  // output pitch, rows of the matrix the tile is in, its first row in w
+    int64_t n0 = (int64_t)tile_n * (64 * TNT);
+    if (gi.tiles) {
+        if (tile_n >= gi.tiles[0]) return;
+        const int expert = gi.tiles[1 + 2 * tile_n];
+        n0 = gi.tiles[2 + 2 * tile_n];
+        ldy = m_rows = gi.expert_rows;
+        if (expert < 0) {
+            // ids outside the stack: the outputs of these pairs are all NaN
+            for (int o = tid; o < 128 * 64 * TNT; o += 512) {
+                const int64_t m = (int64_t)tile_m * 128 + (o & 127);
+                const int pr = gi.out_rows[n0 + (o >> 7)];
+                if (m < m_rows && pr >= 0) y[(int64_t)pr * ldy + m] = __int_as_float(0x7fc00000);
+            }
+            return;
+        }
+        m_stack = (int64_t)expert * gi.expert_rows;
+    }
     // split K: slice blockIdx.y of gridDim.y covers a contiguous run of super-blocks and writes its
     // partial sums to its own [N][M] plane of part; a second kernel adds the planes up in slice order
     // (deterministic, unlike floating-point atomics).  Single-tensor launches only.
     if (part) y = part + (int64_t)blockIdx.y * a.N * w.M;
-    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * TM;
-    const int rows_left = (int)min((int64_t)TM, w.M - m0);  // rows past M: the last row again, results dropped
+    const int64_t m0 = m_stack + (int64_t)tile_m * TM;  // first weight row of the tile
+    const int rows_left = (int)min((int64_t)TM, m_rows - (int64_t)tile_m * TM);  // rows past the end: the last row again, results dropped
     const int rowi = min(32 * mb + r, rows_left - 1);
     const int64_t nsb = w.K / QKK;  // row pitch of the planes, in super-blocks
     const int64_t sb_begin = nsb * blockIdx.y / gridDim.y, sb_end = nsb * (blockIdx.y + 1) / gridDim.y;
@@ -284,14 +313,25 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
 
     // ---- copy plan: per-lane 32-bit offsets, uniform bases per super-block
     constexpr int QI = TN / 4 / WAVES;  // quant copies per wave: rows 4*wave + lane/16 + 32*i
-    unsigned qoff;
-    {
-        const int R = 4 * wave + (lane >> 4);
-        qoff = (unsigned)R * (unsigned)a.K + 16u * ((lane & 15) ^ (R & 15));
-    }
     constexpr int RPI = 1024 / G::SD;   // activation rows per digit copy (64 or 32)
-    const unsigned soff = (unsigned)(lane / (G::SD / 16)) * (unsigned)(nsb * G::SD) + 16u * (lane % (G::SD / 16));
-    const unsigned doff = (unsigned)lane * (unsigned)nsb * 4u;
+    // Row of the activation planes behind tile row t, relative to nbase: the tile's own rows n0 + t, or rows
+    // gathered through src_rows (padding: row 0; the host checked that 32-bit byte offsets reach every row).
+    const int64_t nbase = gi.tiles ? 0 : n0;
+    auto arow_of = [&](int t) -> unsigned {
+        if (!gi.tiles) return (unsigned)t;
+        const int src = gi.src_rows[n0 + min(t, TN - 1)];
+        return src < 0 ? 0u : (unsigned)src;
+    };
+    unsigned qoff[QI];
+#pragma unroll
+    for (int i = 0; i < QI; i++) {
+        const int R = 4 * wave + (lane >> 4) + 32 * i;
+        qoff[i] = arow_of(R) * (unsigned)a.K + 16u * ((lane & 15) ^ (R & 15));
+    }
+    const unsigned soff = arow_of(RPI * wave + lane / (G::SD / 16)) * (unsigned)(nsb * G::SD) + 16u * (lane % (G::SD / 16));
+    unsigned doff[TN / 64];
+#pragma unroll
+    for (int b = 0; b < TN / 64; b++) doff[b] = arow_of(64 * b + lane) * (unsigned)nsb * 4u;
     unsigned woff[G::W_INSTRS];
 #pragma unroll
     for (int j = 0; j < G::W_INSTRS; j++) woff[j] = G::w_lane_off(w, (j * WAVES + wave) * 64 + lane, rows_left);
@@ -308,20 +348,20 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
         }
         // block-sum digits: TN / RPI copies, one per wave from wave 0 up
         if (wave < TN / RPI) {
-            const uint8_t *g = asd + ((n0 + (int64_t)RPI * wave) * nsb + sb) * G::SD + soff;
+            const uint8_t *g = asd + (nbase * nsb + sb) * G::SD + soff;
             __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.s + 1024 * wave), 16, 0, 0);
         }
         // block scales: copies of 64 rows each, by the last waves
         if (wave >= WAVES - TN / 64) {
             const int blk = wave - (WAVES - TN / 64);
-            const uint8_t *g = reinterpret_cast<const uint8_t *>(a.d + (n0 + 64 * blk) * nsb + sb) + doff;
+            const uint8_t *g = reinterpret_cast<const uint8_t *>(a.d + nbase * nsb + sb) + doff[blk];
             __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.yd + 64 * blk), 4, 0, 0);
         }
         // quants
-        const uint8_t *qb = aq + n0 * a.K + sb * QKK;
+        const uint8_t *qb = aq + nbase * a.K + sb * QKK;
 #pragma unroll
         for (int i = 0; i < QI; i++) {
-            const uint8_t *g = qb + (int64_t)(32 * i) * a.K + qoff;
+            const uint8_t *g = qb + qoff[i];
             __builtin_amdgcn_global_load_lds((glb_ptr_t *)g, (lds_ptr_t *)(st.q + 1024 * (wave + WAVES * i)), 16, 0, 0);
         }
     };
@@ -378,14 +418,15 @@ __global__ __launch_bounds__(512, TNT == 1 ? G::OCC_SMALL : 2) void gemm3_kernel
         __syncthreads();
     }
 
-    const int64_t m = m0 + 32 * mb + r;
-    if (m < w.M) {
+    const int64_t m = (int64_t)tile_m * TM + 32 * mb + r;  // row inside its matrix
+    if (m < m_rows) {
 #pragma unroll
         for (int tt = 0; tt < TNT; tt++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int64_t n = n0 + 32 * (TNT * nh + tt) + 8 * (i >> 2) + 4 * h + (i & 3);
-                if (n < a.N) y[n * ldy + m] = acc[tt][i];
+                int64_t n = n0 + 32 * (TNT * nh + tt) + 8 * (i >> 2) + 4 * h + (i & 3);
+                if (gi.tiles) n = gi.out_rows[n];  // sorted row -> pair
+                if (n >= 0 && (gi.tiles || n < a.N)) y[n * ldy + m] = acc[tt][i];
             }
         }
     }
@@ -880,8 +921,9 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
     if (tiles_m > 0x7ffffff0 || gx > 0x7fffffff) return hipErrorInvalidValue;
     const dim3 grid((unsigned)gx, (unsigned)ksplit);
     float *part = ksplit > 1 ? workspace : nullptr;
-    if (tnt2) gemm3_kernel<G, 2><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part);
-    else gemm3_kernel<G, 1><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part);
+    const GemmIds none{nullptr, nullptr, nullptr, 0};
+    if (tnt2) gemm3_kernel<G, 2><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part, none);
+    else gemm3_kernel<G, 1><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part, none);
     if (ksplit > 1) {
         const int64_t n4 = a.N * ws[0].M / 4;
         const unsigned blocks = (unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048);
@@ -978,6 +1020,32 @@ hipError_t launch_skinny_id(const DevWeight &w, int n_expert, const DevAct &a, c
     if (wgs > 0x7fffffff) return hipErrorInvalidValue;
     if (w.type == T_Q4_K) launch_skinny_as<Sk16Q4K, 16, true>(w, a, 0, 16, y, si, wgs, num_cus, s);
     else launch_skinny_as<Sk16Q6K, 16, true>(w, a, 0, 16, y, si, wgs, num_cus, s);
+    return hipGetLastError();
+}
+
+bool gemm_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert) {
+    // worth sorting the pairs and padding every expert to 64-row tiles from about sixteen pairs per expert
+    return gemm_supports(type, K, M) && pairs >= 16 * (int64_t)n_expert;
+}
+
+hipError_t launch_gemm_id(const DevWeight &w, int n_expert, const DevAct &a, const int *tiles, const int *src_rows,
+                          const int *out_rows, int64_t max_tiles, float *y, hipStream_t s) {
+    if (n_expert < 1 || w.M % n_expert || !gemm_supports(w.type, w.K, w.M / n_expert) || a.type != T_Q8_K || a.K != w.K ||
+        !a.sd8 || !a.sd16 || !tiles || !src_rows || !out_rows || !y || max_tiles < 1 ||
+        (int64_t)a.N * a.K >= ((int64_t)1 << 32))  // the copies address activation bytes with 32-bit offsets
+        return hipErrorInvalidValue;
+    GemmArgs ga;
+    for (int i = 0; i < GEMM_MULTI; i++) {
+        ga.p0[i] = w.p0; ga.p1[i] = w.p1; ga.p2[i] = w.p2; ga.d[i] = w.d; ga.y[i] = y; ga.M[i] = w.M;
+        ga.tile_end[i] = 0x7fffffff;
+    }
+    ga.K = w.K; ga.type = w.type;
+    const GemmIds gi{tiles, src_rows, out_rows, w.M / n_expert};
+    const int64_t tiles_m = (gi.expert_rows + 127) / 128;
+    const int64_t gx = max_tiles * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
+    if (gx > 0x7fffffff) return hipErrorInvalidValue;
+    if (w.type == T_Q4_K) gemm3_kernel<GemmQ4K, 1><<<(unsigned)gx, 512, 0, s>>>(ga, a, (int)tiles_m, (int)max_tiles, nullptr, gi);
+    else gemm3_kernel<GemmQ6K, 1><<<(unsigned)gx, 512, 0, s>>>(ga, a, (int)tiles_m, (int)max_tiles, nullptr, gi);
     return hipGetLastError();
 }
 

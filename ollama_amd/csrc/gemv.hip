@@ -1038,6 +1038,65 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const int *__restrict
 
 // F32 (one pair per group only): xf is b itself, [tokens][b_cols][K] floats, and the workgroup quantizes
 // its pair's activation row into LDS first, like the thin kernel does -- decode is one launch.
+// For the expert GEMM: the pairs sorted by expert, every expert's run padded to whole 64-row tiles.
+//   out[0]                       number of tiles
+//   out[1 + 2t], out[2 + 2t]     tile t: expert (-1: ids outside the stack), first sorted row
+//   src_col[row]                 activation row (token * b_cols + slot mod b_cols) behind sorted row, -1: padding
+//   out_pair[row]                pair (token * n_used + slot) behind sorted row, -1: padding
+// Which place a pair gets inside its expert's run depends on the order of the atomics; the product of a
+// row does not depend on its place.
+__global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict__ ids, int pairs, int n_expert, int n_used,
+                                                           int b_cols, int max_tiles, int *__restrict__ out,
+                                                           int *__restrict__ src_col, int *__restrict__ out_pair) {
+    __shared__ int count[ID_MAX_EXPERTS + 1], start[ID_MAX_EXPERTS + 1], scan[2][1024];
+    const int nb = n_expert + 1, tid = threadIdx.x;
+    for (int e = tid; e < nb; e += 1024) count[e] = 0;
+    for (int r = tid; r < 64 * max_tiles; r += 1024) { src_col[r] = -1; out_pair[r] = -1; }
+    __syncthreads();
+    for (int p = tid; p < pairs; p += 1024) {
+        const int e = ids[p];
+        atomicAdd(&count[(e < 0 || e >= n_expert) ? n_expert : e], 1);
+    }
+    __syncthreads();
+    // tiles per expert, then a running sum over the experts: thread t owns experts PER*t .. PER*t + PER-1
+    constexpr int PER = (ID_MAX_EXPERTS + 1 + 1023) / 1024;
+    int mine = 0;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int e = PER * tid + j;
+        mine += e < nb ? (count[e] + 63) / 64 : 0;
+    }
+    scan[0][tid] = mine;
+    __syncthreads();
+    int cur = 0;
+    for (int step = 1; step < 1024; step <<= 1, cur ^= 1) {
+        scan[cur ^ 1][tid] = scan[cur][tid] + (tid >= step ? scan[cur][tid - step] : 0);
+        __syncthreads();
+    }
+    int t = scan[cur][tid] - mine;  // tiles of all experts before this thread's
+    if (tid == 1023) out[0] = scan[cur][tid];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int e = PER * tid + j;
+        if (e >= nb) break;
+        start[e] = 64 * t;
+        for (int c = 0; c < count[e]; c += 64, t++) {
+            out[1 + 2 * t] = e < n_expert ? e : -1;
+            out[2 + 2 * t] = 64 * t;
+        }
+        count[e] = 0;  // reused as the fill cursor
+    }
+    __syncthreads();
+    for (int p = tid; p < pairs; p += 1024) {
+        const int e0 = ids[p];
+        const int e = (e0 < 0 || e0 >= n_expert) ? n_expert : e0;
+        const int row = start[e] + atomicAdd(&count[e], 1);
+        const int tok = p / n_used, slot = p - tok * n_used;
+        src_col[row] = tok * b_cols + slot % b_cols;
+        out_pair[row] = p;
+    }
+}
+
 template <class P, int NC, bool DIRECT, bool F32, int RPL>
 __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const float *__restrict__ xf,
                                                       int rows_per_wave, int kw, int rw_log2) {
@@ -1193,6 +1252,18 @@ hipError_t launch_group_pairs(const int *ids, int pairs, int n_expert, int nc, i
     if (nc == 8) group_pairs_kernel<8><<<1, 1024, 0, s>>>(ids, pairs, n_expert, groups);
     else if (nc == 16) group_pairs_kernel<16><<<1, 1024, 0, s>>>(ids, pairs, n_expert, groups);
     else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+int64_t sort_pairs_max_tiles(int64_t pairs, int n_expert) { return pairs / 64 + n_expert + 2; }
+
+hipError_t launch_sort_pairs(const int *ids, int pairs, int n_expert, int n_used, int b_cols, int *tiles, int *src_col,
+                             int *out_pair, hipStream_t s) {
+    if (!ids || !tiles || !src_col || !out_pair || pairs < 1 || n_expert < 1 || n_expert > ID_MAX_EXPERTS || n_used < 1 ||
+        b_cols < 1)
+        return hipErrorInvalidValue;
+    sort_pairs_kernel<<<1, 1024, 0, s>>>(ids, pairs, n_expert, n_used, b_cols, (int)sort_pairs_max_tiles(pairs, n_expert),
+                                         tiles, src_col, out_pair);
     return hipGetLastError();
 }
 

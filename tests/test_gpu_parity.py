@@ -655,3 +655,34 @@ def test_mulmat_id_multi_equals_single_calls(ctx, t, tokens):
         ctx.mulmat_id_multi(ws, n_expert, b, np.full((tokens, n_used), n_expert, np.int32))
     for w in ws:
         w.free()
+
+
+@pytest.mark.parametrize("t,k,m,n_expert,tokens,n_used,b_cols", [(Q4_K, 1024, 200, 6, 64, 3, 1), (Q6_K, 512, 130, 4, 70, 2, 2),
+                                                               (Q4_K, 2048, 768, 16, 128, 4, 1), (Q4_K, 256, 64, 3, 500, 1, 1)])
+def test_mulmat_id_expert_gemm(ctx, t, k, m, n_expert, tokens, n_used, b_cols):
+    """sixteen pairs per expert and more: pairs sorted by expert, every expert's run through the tiled GEMM;
+    an idle expert, a crowded one (several tiles), ragged expert height, ids outside the stack (device ids)"""
+    rng = np.random.default_rng(8100 + t + tokens)
+    wb = _experts(t, n_expert, m, k, 8101 + t)
+    w = ctx.upload(t, wb, k, n_expert * m)
+    b = rng.standard_normal((tokens, b_cols, k), dtype=np.float32)
+    ids = rng.integers(0, max(n_expert - 1, 1), (tokens, n_used)).astype(np.int32)  # the last expert stays idle
+    ids[: tokens // 2, 0] = 0                                                       # a crowd on expert 0
+    got = ctx.mulmat_id(w, n_expert, b, ids)
+    want = oracle.mul_mat_id(t, wb, k, m, n_expert, b, ids)
+    assert npref.rel_err(got, want) < TOL
+    assert np.array_equal(ctx.mulmat_id(w, n_expert, b[::-1].copy(), ids[::-1].copy())[::-1], got)
+    bad = ids.copy()
+    bad[1, 0] = n_expert
+    bad[-1, -1] = -3
+    db, dids = DeviceArray(b), DeviceArray(bad)
+    dy = DeviceArray(np.zeros((tokens, n_used, m), np.float32), zero=True)
+    ctx.mulmat_id_device(w, n_expert, db.ptr, b_cols, dids.ptr, n_used, tokens, dy.ptr)
+    ctx.sync()
+    out = dy.numpy()
+    isbad = (bad < 0) | (bad >= n_expert)
+    assert np.isnan(out[isbad]).all() and not np.isnan(out[~isbad]).any()
+    assert np.array_equal(out[~isbad], got[~isbad])
+    for d in (db, dids, dy):
+        d.free()
+    w.free()
