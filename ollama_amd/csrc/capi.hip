@@ -653,11 +653,13 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
     // batches with many pairs per expert: sort the pairs by expert and run the tiled GEMM per expert
     const bool gemm = gemm_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
-    const int64_t max_tiles = gemm ? sort_pairs_max_tiles(pairs, n_expert) : 0, sorted_rows = 64 * max_tiles;
+    const int tile_w = gemm_id_tile_width(w->dev.type, pairs, n_expert);
+    const int64_t max_tiles = gemm ? sort_pairs_max_tiles(pairs, n_expert, tile_w) : 0, sorted_rows = tile_w * max_tiles;
     const ActPlanes probe = plan_act(nullptr, q8, K, ncols);
     if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
     const ActPlanes p = plan_act(ctx->act_buf, q8, K, ncols);
-    const size_t scratch_ints = gemm ? (size_t)(1 + 2 * max_tiles + 2 * sorted_rows) : gemv_id_scratch_ints(pairs);
+    const size_t hist_ints = gemm ? sort_pairs_hist_ints(pairs, n_expert) : 0;
+    const size_t scratch_ints = gemm ? (size_t)(1 + 2 * max_tiles + 2 * sorted_rows) + hist_ints : gemv_id_scratch_ints(pairs);
     if ((rc = reserve(&ctx->ws_buf, &ctx->ws_cap, scratch_ints * sizeof(int), ctx->stream))) return rc;
 
     const size_t xbytes = (size_t)(ncols * K) * 4, ibytes = (size_t)pairs * 4, ybytes = (size_t)(pairs * M) * 4;
@@ -676,12 +678,13 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     }
     if (gemm) {
         int *tiles = (int *)ctx->ws_buf, *src_col = tiles + 1 + 2 * max_tiles, *out_pair = src_col + sorted_rows;
-        HIP_TRY(launch_sort_pairs(dids, (int)pairs, n_expert, n_used, b_cols, tiles, src_col, out_pair, ctx->stream));
+        HIP_TRY(launch_sort_pairs(dids, (int)pairs, n_expert, n_used, b_cols, tile_w, tiles, src_col, out_pair,
+                                  hist_ints ? out_pair + sorted_rows : nullptr, ctx->stream));
         HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
         DevAct as;
         as.qs = p.qs; as.d = p.d; as.bsums = p.bsums; as.sd8 = p.sd8; as.sd16 = p.sd16; as.K = K; as.N = (int)ncols; as.type = q8;
-        HIP_TRY(launch_gemm_id(w->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, dy, ctx->stream));
-        if (w2) HIP_TRY(launch_gemm_id(w2->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, dy2, ctx->stream));
+        HIP_TRY(launch_gemm_id(w->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, tile_w, dy, ctx->stream));
+        if (w2) HIP_TRY(launch_gemm_id(w2->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, tile_w, dy2, ctx->stream));
         if (location == MI_QMM_HOST) {
             HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
             if (w2) HIP_TRY(hipMemcpyAsync(y2, dy2, ybytes, hipMemcpyDeviceToHost, ctx->stream));

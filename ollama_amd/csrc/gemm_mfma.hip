@@ -245,7 +245,7 @@ struct GemmArgs {
 // TNT = 32-row activation sub-tiles per wave: the workgroup tile is 128 weight rows x 64*TNT activation rows.
 // Expert GEMM (Tensor.MulmatID on a batch, /root/reference/ml/backend.go:153): ga holds one stack of
 // expert matrices of expert_rows rows each; the (token, slot) pairs are sorted by expert into runs of whole
-// 64-row tiles (sort_pairs_kernel), tile_n picks a run's tile from the table and with it the expert.  The
+// 64- or 128-row tiles (sort_pairs_kernel), tile_n picks a run's tile from the table and with it the expert.  The
 // activation planes stay in their own order: every copy gathers its rows through src_rows, and out_rows
 // maps a sorted row to the pair whose output row it is.
 struct GemmIds {
@@ -913,9 +913,11 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
     ga.K = ws[0].K; ga.type = ws[0].type;
     int ksplit = count == 1 ? pick_ksplit(ws[0].K, ws[0].M, a.N, num_cus) : 1;
     if (ksplit > 1 && (!workspace || workspace_floats < (size_t)ksplit * a.N * ws[0].M)) ksplit = 1;
-    // 128 x 128 tiles when they still give every CU work for most of the run, else 128 x 64
+    // Q6_K: 128 x 128 tiles when they still give every CU work for most of the run, else 128 x 64.  Q4_K
+    // unpacks with less vector work, and two resident 128 x 64 workgroups per CU (each covering the other's
+    // waits) measure 3..8 % faster than one 128 x 128 at every batch size from 512 to 8192.
     const int64_t big = tiles_m * ((a.N + 127) / 128) * ksplit;
-    const bool tnt2 = ksplit > 1 || 2 * big >= 3 * (int64_t)num_cus;
+    const bool tnt2 = ksplit > 1 || (ga.type == T_Q6_K && 2 * big >= 3 * (int64_t)num_cus);
     const int64_t tn = tnt2 ? 128 : 64, tiles_n = (a.N + tn - 1) / tn;
     const int64_t gx = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
     if (tiles_m > 0x7ffffff0 || gx > 0x7fffffff) return hipErrorInvalidValue;
@@ -1028,8 +1030,16 @@ bool gemm_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_exper
     return gemm_supports(type, K, M) && pairs >= 16 * (int64_t)n_expert;
 }
 
+// Pairs per tile: 64, and for Q6_K 128 once the experts see 128 pairs each on average (measured on 8 experts of
+// 14336 x 4096 at 2 of 8: Q6_K 351 against 290 TOPS at 1024 pairs per expert, even at 128; Q4_K is faster
+// with 64 at every count, as in the dense product).
+int gemm_id_tile_width(int type, int64_t pairs, int n_expert) {
+    return type == T_Q6_K && pairs >= 128 * (int64_t)n_expert ? 128 : 64;
+}
+
 hipError_t launch_gemm_id(const DevWeight &w, int n_expert, const DevAct &a, const int *tiles, const int *src_rows,
-                          const int *out_rows, int64_t max_tiles, float *y, hipStream_t s) {
+                          const int *out_rows, int64_t max_tiles, int tile_width, float *y, hipStream_t s) {
+    if (tile_width != 64 && !(tile_width == 128 && w.type == T_Q6_K)) return hipErrorInvalidValue;
     if (n_expert < 1 || w.M % n_expert || !gemm_supports(w.type, w.K, w.M / n_expert) || a.type != T_Q8_K || a.K != w.K ||
         !a.sd8 || !a.sd16 || !tiles || !src_rows || !out_rows || !y || max_tiles < 1 ||
         (int64_t)a.N * a.K >= ((int64_t)1 << 32))  // the copies address activation bytes with 32-bit offsets
@@ -1045,6 +1055,7 @@ hipError_t launch_gemm_id(const DevWeight &w, int n_expert, const DevAct &a, con
     const int64_t gx = max_tiles * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
     if (gx > 0x7fffffff) return hipErrorInvalidValue;
     if (w.type == T_Q4_K) gemm3_kernel<GemmQ4K, 1><<<(unsigned)gx, 512, 0, s>>>(ga, a, (int)tiles_m, (int)max_tiles, nullptr, gi);
+    else if (tile_width == 128) gemm3_kernel<GemmQ6K, 2><<<(unsigned)gx, 512, 0, s>>>(ga, a, (int)tiles_m, (int)max_tiles, nullptr, gi);
     else gemm3_kernel<GemmQ6K, 1><<<(unsigned)gx, 512, 0, s>>>(ga, a, (int)tiles_m, (int)max_tiles, nullptr, gi);
     return hipGetLastError();
 }

@@ -1046,16 +1046,21 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const int *__restrict
 // Which place a pair gets inside its expert's run depends on the order of the atomics; the product of a
 // row does not depend on its place.
 __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict__ ids, int pairs, int n_expert, int n_used,
-                                                           int b_cols, int max_tiles, int *__restrict__ out,
+                                                           int b_cols, int max_tiles, int tw, int *__restrict__ out,
                                                            int *__restrict__ src_col, int *__restrict__ out_pair) {
     __shared__ int count[ID_MAX_EXPERTS + 1], start[ID_MAX_EXPERTS + 1], scan[2][1024];
     const int nb = n_expert + 1, tid = threadIdx.x;
     for (int e = tid; e < nb; e += 1024) count[e] = 0;
-    for (int r = tid; r < 64 * max_tiles; r += 1024) { src_col[r] = -1; out_pair[r] = -1; }
+    for (int r = tid; r < tw * max_tiles; r += 1024) { src_col[r] = -1; out_pair[r] = -1; }
     __syncthreads();
-    for (int p = tid; p < pairs; p += 1024) {
-        const int e = ids[p];
-        atomicAdd(&count[(e < 0 || e >= n_expert) ? n_expert : e], 1);
+    // eight independent loads at a time: one workgroup has to hide the latency of ids by itself
+    for (int p0 = tid; p0 < pairs; p0 += 8 * 1024) {
+        int e[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) e[j] = p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (p0 + 1024 * j < pairs) atomicAdd(&count[(e[j] < 0 || e[j] >= n_expert) ? n_expert : e[j]], 1);
     }
     __syncthreads();
     // tiles per expert, then a running sum over the experts: thread t owns experts PER*t .. PER*t + PER-1
@@ -1064,7 +1069,7 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict_
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const int e = PER * tid + j;
-        mine += e < nb ? (count[e] + 63) / 64 : 0;
+        mine += e < nb ? (count[e] + tw - 1) / tw : 0;
     }
     scan[0][tid] = mine;
     __syncthreads();
@@ -1079,18 +1084,112 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict_
     for (int j = 0; j < PER; j++) {
         const int e = PER * tid + j;
         if (e >= nb) break;
-        start[e] = 64 * t;
-        for (int c = 0; c < count[e]; c += 64, t++) {
+        start[e] = tw * t;
+        for (int c = 0; c < count[e]; c += tw, t++) {
             out[1 + 2 * t] = e < n_expert ? e : -1;
-            out[2 + 2 * t] = 64 * t;
+            out[2 + 2 * t] = tw * t;
         }
         count[e] = 0;  // reused as the fill cursor
     }
     __syncthreads();
-    for (int p = tid; p < pairs; p += 1024) {
-        const int e0 = ids[p];
-        const int e = (e0 < 0 || e0 >= n_expert) ? n_expert : e0;
-        const int row = start[e] + atomicAdd(&count[e], 1);
+    for (int p0 = tid; p0 < pairs; p0 += 8 * 1024) {
+        int e[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) e[j] = p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int p = p0 + 1024 * j;
+            if (p >= pairs) break;
+            const int eb = (e[j] < 0 || e[j] >= n_expert) ? n_expert : e[j];
+            const int row = start[eb] + atomicAdd(&count[eb], 1);
+            const int tok = p / n_used, slot = p - tok * n_used;
+            src_col[row] = tok * b_cols + slot % b_cols;
+            out_pair[row] = p;
+        }
+    }
+}
+
+// The same sort for many pairs, spread over workgroups of SORT_CHUNK pairs each:
+//   count: every workgroup histograms its chunk (and clears its share of the row tables);
+//   plan:  one workgroup turns the histograms into the tile table and, per chunk and expert, the first
+//          sorted row that chunk's pairs of that expert go to;
+//   place: every workgroup hands its pairs their rows.
+constexpr int SORT_CHUNK = 2048, SORT_MAX_CHUNKS = 256;
+
+__global__ __launch_bounds__(1024) void sort_count_kernel(const int *__restrict__ ids, int pairs, int n_expert, int table_rows,
+                                                           int *__restrict__ hist, int *__restrict__ src_col,
+                                                           int *__restrict__ out_pair) {
+    __shared__ int count[ID_MAX_EXPERTS + 1];
+    const int nb = n_expert + 1, tid = threadIdx.x;
+    for (int e = tid; e < nb; e += 1024) count[e] = 0;
+    for (int r = blockIdx.x * 1024 + tid; r < table_rows; r += gridDim.x * 1024) { src_col[r] = -1; out_pair[r] = -1; }
+    __syncthreads();
+    const int p0 = blockIdx.x * SORT_CHUNK + tid;
+    int e[SORT_CHUNK / 1024];
+#pragma unroll
+    for (int j = 0; j < SORT_CHUNK / 1024; j++) e[j] = p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
+#pragma unroll
+    for (int j = 0; j < SORT_CHUNK / 1024; j++)
+        if (p0 + 1024 * j < pairs) atomicAdd(&count[(e[j] < 0 || e[j] >= n_expert) ? n_expert : e[j]], 1);
+    __syncthreads();
+    for (int x = tid; x < nb; x += 1024) hist[(size_t)blockIdx.x * nb + x] = count[x];
+}
+
+__global__ __launch_bounds__(1024) void sort_plan_kernel(int n_expert, int chunks, int tw, int *__restrict__ hist, int *__restrict__ out) {
+    __shared__ int scan[2][1024];
+    const int nb = n_expert + 1, tid = threadIdx.x;
+    constexpr int PER = (ID_MAX_EXPERTS + 1 + 1023) / 1024;
+    int total[PER], mine = 0;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int e = PER * tid + j;
+        total[j] = 0;
+        if (e < nb)
+            for (int c = 0; c < chunks; c++) total[j] += hist[(size_t)c * nb + e];
+        mine += (total[j] + tw - 1) / tw;
+    }
+    scan[0][tid] = mine;
+    __syncthreads();
+    int cur = 0;
+    for (int step = 1; step < 1024; step <<= 1, cur ^= 1) {
+        scan[cur ^ 1][tid] = scan[cur][tid] + (tid >= step ? scan[cur][tid - step] : 0);
+        __syncthreads();
+    }
+    int t = scan[cur][tid] - mine;
+    if (tid == 1023) out[0] = scan[cur][tid];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int e = PER * tid + j;
+        if (e >= nb) break;
+        int row = tw * t;  // first sorted row of the expert; the chunks' pairs follow one another
+        for (int c = 0; c < chunks; c++) {
+            const int n = hist[(size_t)c * nb + e];
+            hist[(size_t)c * nb + e] = row;
+            row += n;
+        }
+        for (int c = 0; c < total[j]; c += tw, t++) {
+            out[1 + 2 * t] = e < n_expert ? e : -1;
+            out[2 + 2 * t] = tw * t;
+        }
+    }
+}
+
+__global__ __launch_bounds__(1024) void sort_place_kernel(const int *__restrict__ ids, int pairs, int n_expert, int n_used,
+                                                           int b_cols, const int *__restrict__ base, int *__restrict__ src_col,
+                                                           int *__restrict__ out_pair) {
+    __shared__ int next[ID_MAX_EXPERTS + 1];
+    const int nb = n_expert + 1, tid = threadIdx.x;
+    for (int e = tid; e < nb; e += 1024) next[e] = base[(size_t)blockIdx.x * nb + e];
+    __syncthreads();
+    const int p0 = blockIdx.x * SORT_CHUNK + tid;
+    int e[SORT_CHUNK / 1024];
+#pragma unroll
+    for (int j = 0; j < SORT_CHUNK / 1024; j++) e[j] = p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
+#pragma unroll
+    for (int j = 0; j < SORT_CHUNK / 1024; j++) {
+        const int p = p0 + 1024 * j;
+        if (p >= pairs) break;
+        const int row = atomicAdd(&next[(e[j] < 0 || e[j] >= n_expert) ? n_expert : e[j]], 1);
         const int tok = p / n_used, slot = p - tok * n_used;
         src_col[row] = tok * b_cols + slot % b_cols;
         out_pair[row] = p;
@@ -1255,15 +1354,30 @@ hipError_t launch_group_pairs(const int *ids, int pairs, int n_expert, int nc, i
     return hipGetLastError();
 }
 
-int64_t sort_pairs_max_tiles(int64_t pairs, int n_expert) { return pairs / 64 + n_expert + 2; }
+// most tiles the sort can emit for tiles of tile_width pairs (every expert's run, and that of the pairs with
+// ids outside the stack, ends in one partly filled tile)
+int64_t sort_pairs_max_tiles(int64_t pairs, int n_expert, int tile_width) { return pairs / tile_width + n_expert + 2; }
 
-hipError_t launch_sort_pairs(const int *ids, int pairs, int n_expert, int n_used, int b_cols, int *tiles, int *src_col,
-                             int *out_pair, hipStream_t s) {
+// ints of device scratch behind the row tables for the chunked sort's histograms (0: one workgroup does it all)
+size_t sort_pairs_hist_ints(int64_t pairs, int n_expert) {
+    const int64_t chunks = (pairs + SORT_CHUNK - 1) / SORT_CHUNK;
+    return chunks >= 3 && chunks <= SORT_MAX_CHUNKS ? (size_t)chunks * (n_expert + 1) : 0;
+}
+
+hipError_t launch_sort_pairs(const int *ids, int pairs, int n_expert, int n_used, int b_cols, int tile_width, int *tiles,
+                             int *src_col, int *out_pair, int *hist, hipStream_t s) {
     if (!ids || !tiles || !src_col || !out_pair || pairs < 1 || n_expert < 1 || n_expert > ID_MAX_EXPERTS || n_used < 1 ||
-        b_cols < 1)
+        b_cols < 1 || tile_width < 1)
         return hipErrorInvalidValue;
-    sort_pairs_kernel<<<1, 1024, 0, s>>>(ids, pairs, n_expert, n_used, b_cols, (int)sort_pairs_max_tiles(pairs, n_expert),
-                                         tiles, src_col, out_pair);
+    const int tw = tile_width, max_tiles = (int)sort_pairs_max_tiles(pairs, n_expert, tw);
+    if (hist && sort_pairs_hist_ints(pairs, n_expert)) {
+        const int chunks = (pairs + SORT_CHUNK - 1) / SORT_CHUNK;
+        sort_count_kernel<<<chunks, 1024, 0, s>>>(ids, pairs, n_expert, tw * max_tiles, hist, src_col, out_pair);
+        sort_plan_kernel<<<1, 1024, 0, s>>>(n_expert, chunks, tw, hist, tiles);
+        sort_place_kernel<<<chunks, 1024, 0, s>>>(ids, pairs, n_expert, n_used, b_cols, hist, src_col, out_pair);
+    } else {
+        sort_pairs_kernel<<<1, 1024, 0, s>>>(ids, pairs, n_expert, n_used, b_cols, max_tiles, tw, tiles, src_col, out_pair);
+    }
     return hipGetLastError();
 }
 

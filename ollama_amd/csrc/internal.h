@@ -80,16 +80,19 @@ hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int nc
                            hipStream_t s);
 
 // Expert GEMM (K-quants, batches with many pairs per expert): sort_pairs sorts the (token, slot) pairs by
-// expert into runs of whole 64-row tiles; the tiled GEMM multiplies every run by its expert's matrix,
+// expert into runs of whole 64- or 128-row tiles; the tiled GEMM multiplies every run by its expert's matrix,
 // gathering the run's activation rows from the planes (which stay in their own order) and writing each
 // result row to its pair's place in y.
-//   tiles: 1 + 2 * max_tiles ints; src_col, out_pair: 64 * max_tiles ints each (device scratch)
-int64_t sort_pairs_max_tiles(int64_t pairs, int n_expert);
-hipError_t launch_sort_pairs(const int *ids, int pairs, int n_expert, int n_used, int b_cols, int *tiles, int *src_col,
-                             int *out_pair, hipStream_t s);
+//   tiles: 1 + 2 * max_tiles ints; src_col, out_pair: tile_width * max_tiles ints each; hist:
+//   sort_pairs_hist_ints() ints (device scratch; with many pairs the sort runs as three launches over chunks)
+int64_t sort_pairs_max_tiles(int64_t pairs, int n_expert, int tile_width);
+size_t sort_pairs_hist_ints(int64_t pairs, int n_expert);
+hipError_t launch_sort_pairs(const int *ids, int pairs, int n_expert, int n_used, int b_cols, int tile_width, int *tiles,
+                             int *src_col, int *out_pair, int *hist, hipStream_t s);
 bool gemm_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);
+int gemm_id_tile_width(int type, int64_t pairs, int n_expert);  // pairs per tile the GEMM wants: 64 or 128
 hipError_t launch_gemm_id(const DevWeight &w, int n_expert, const DevAct &a, const int *tiles, const int *src_rows,
-                          const int *out_rows, int64_t max_tiles, float *y, hipStream_t s);
+                          const int *out_rows, int64_t max_tiles, int tile_width, float *y, hipStream_t s);
 
 // Expert-indexed product on the matrix cores (K-quants): the pairs are bucketed by expert, 16 per group;
 // a needs the block-sum digit planes.  groups: device scratch of gemv_id_scratch_ints(pairs) ints.
