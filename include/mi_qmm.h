@@ -142,7 +142,12 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
  * (b_cols = 1: all slots of a token share one activation row, as for gate/up; b_cols = n_used: every
  * slot has its own, as for the down projection.)  location covers x, ids and y alike.  With ids in
  * host memory an id outside 0..n_expert-1 is MI_QMM_ERR_INVALID (ggml aborts there); with ids in
- * device memory the call cannot see them and the rows of such a pair come back as NaN. */
+ * device memory the call cannot see them and the rows of such a pair come back as NaN.
+ * The kernel follows n_tokens * n_used / n_expert: one streaming product per pair (decode), pairs
+ * bucketed by expert on the device for the 16-column matrix-core kernel, and from 16 pairs per expert
+ * (Q4_K / Q6_K) pairs sorted by expert and multiplied tile by tile on the matrix cores.  Scratch for
+ * the buckets comes from the ctx's workspace, which grows on demand (a device allocation on the
+ * first call of a new size). */
 int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
                      const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location);
 
