@@ -133,6 +133,36 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
 int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x,
                         int64_t n, float *const *ys, int location);
 
+/* Producers of the activations: the two graph nodes that feed the quantized products of a transformer
+ * block, fused into the quantization so that their f32 result never goes through memory.
+ *   MI_QMM_PRODUCE_RMSNORM  Tensor.RMSNorm(ctx, weight, eps)  (/root/reference/ml/backend.go:159):
+ *       x' = (x * scale) * aux,  scale = 1 / sqrtf(mean(x^2) + eps) per row;  aux = the norm weight
+ *       f32 [k], or NULL for the bare normalization
+ *   MI_QMM_PRODUCE_SWIGLU   Tensor.SILU(ctx, up)  (/root/reference/ml/backend.go:180):
+ *       x' = silu(x) * aux,  silu(v) = v / (1 + expf(-v));  aux = up, f32 [n][k] like x
+ * ggml's scalar arithmetic: squares in fp32 accumulated in double, the mean rounded to fp32, the two
+ * multiplies of RMSNorm rounded separately.  expf is the device library's (within 1 ulp). */
+enum {
+    MI_QMM_PRODUCE_NONE = 0,
+    MI_QMM_PRODUCE_RMSNORM = 1,
+    MI_QMM_PRODUCE_SWIGLU = 2,
+};
+/* mi_qmm_mulmat_multi on x' = producer(x): ys[i] = ws[i] * Q8(x').  With one activation row (decode)
+ * and weights of one type this is ONE kernel launch: every workgroup of the GEMV normalizes / gates x,
+ * quantizes it and walks its rows.  Otherwise x' is quantized once per activation format by a fused
+ * quantizer (RMSNorm: after one launch for the row scales) and the products follow.  aux lives where x
+ * does (location).  Results are bit-identical to mi_qmm_rms_norm / mi_qmm_swiglu followed by
+ * mi_qmm_mulmat_multi. */
+int mi_qmm_mulmat_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int producer,
+                           const float *aux, float eps, const float *x, int64_t n, float *const *ys,
+                           int location);
+/* The same producers as plain f32 operations, for graph nodes that something other than a product
+ * reads: x, y f32 [n][k] (k a multiple of 4), g f32 [k] or NULL; gate, up, y f32 [n][k]. */
+int mi_qmm_rms_norm(mi_qmm_ctx *ctx, const float *x, const float *g, float eps, int64_t k, int64_t n,
+                    float *y, int location);
+int mi_qmm_swiglu(mi_qmm_ctx *ctx, const float *gate, const float *up, int64_t k, int64_t n, float *y,
+                  int location);
+
 /* Expert-indexed product, Tensor.MulmatID (/root/reference/ml/backend.go:153).  w is a stack of
  * n_expert matrices uploaded as ONE weight of m = rows_per_expert * n_expert rows: GGUF stores expert
  * tensors with ne = [in, out, experts] (/root/reference/convert/convert_gemma4.go:274-275), so the

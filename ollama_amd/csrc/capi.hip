@@ -531,8 +531,14 @@ int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64
     return mi_qmm_mulmat_path(ctx, w, x, n, y, location, MI_QMM_PATH_AUTO);
 }
 
-int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x, int64_t n,
-                        float *const *ys, int location) {
+}  // extern "C"
+
+namespace {
+
+// mi_qmm_mulmat_multi and mi_qmm_mulmat_produced: several weights of one K against the same activations,
+// which may first go through a producer (prod: kind, aux and eps as the caller gave them, aux in `location`).
+int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const Produce *prod, const float *x,
+                      int64_t n, float *const *ys, int location) {
     if (!ws || !ys || count < 1) return fail(MI_QMM_ERR_INVALID, "ws/ys is NULL or count < 1");
     for (int i = 0; i < count; i++)
         if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
@@ -548,6 +554,10 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
     if (rc) return rc;
     for (int i = 0; i < count; i++)
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
+    Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
+    if (prod) pr = *prod;
+    if (pr.kind == PRODUCE_SWIGLU && !pr.aux && n > 0) return fail(MI_QMM_ERR_INVALID, "SwiGLU needs the up operand");
+    if (pr.kind == PRODUCE_RMSNORM && !(pr.eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
     if (n == 0) return MI_QMM_OK;
     if (!x) return fail(MI_QMM_ERR_INVALID, "x is NULL");
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
@@ -555,40 +565,60 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i]->dev.M;
 
-    // x and the outputs on the device
+    // x, the producer's operand and the outputs on the device
     const size_t xbytes = (size_t)(n * K) * 4;
+    const size_t auxbytes = !pr.aux ? 0 : pr.kind == PRODUCE_SWIGLU ? xbytes : (size_t)K * 4;
     const float *dx = x;
     std::vector<float *> dys(ys, ys + count);
     if (location == MI_QMM_HOST) {
         std::vector<size_t> offs(count + 1);
-        offs[0] = align_up(xbytes, 256);
+        const size_t auxoff = align_up(xbytes, 256);
+        offs[0] = auxoff + align_up(auxbytes, 256);
         for (int i = 0; i < count; i++) offs[i + 1] = offs[i] + align_up((size_t)(n * ws[i]->dev.M) * 4, 256);
         if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
         dx = (const float *)ctx->io_buf;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+        if (auxbytes) {
+            float *daux = (float *)((char *)ctx->io_buf + auxoff);
+            HIP_TRY(hipMemcpyAsync(daux, pr.aux, auxbytes, hipMemcpyHostToDevice, ctx->stream));
+            pr.aux = daux;
+        }
     }
 
     bool skinny = false;
     for (int i = 0; i < count; i++) skinny = skinny || wants_skinny(ws[i]->dev.type, K, ws[i]->dev.M, n);
-    if (same_type && !skinny && count <= gemv_max_multi() && n <= 8 &&
-        gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)) {
-        // decode: one launch over the concatenated rows, the kernel quantizes x in its prologue
+    const bool in_kernel = same_type && !skinny && count <= gemv_max_multi() && n <= 8 &&
+                           (pr.kind == PRODUCE_NONE ? gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)
+                                                    : n == 1 && gemv_produce_supported(ws[0]->dev.type, K, total_m));
+    if (in_kernel) {
+        // decode: one launch over the concatenated rows, the kernel produces and quantizes x in its prologue
         DevWeight dw[8];
         for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
-        HIP_TRY(launch_gemv_f32_multi(dw, dys.data(), count, dx, (int)n, ctx->num_cus, ctx->stream));
+        HIP_TRY(launch_gemv_f32_multi(dw, dys.data(), count, dx, (int)n, ctx->num_cus, ctx->stream,
+                                      pr.kind == PRODUCE_NONE ? nullptr : &pr));
     } else {
-        // x is quantized once per activation format (Q8_0 / Q8_K) in use; weights of one type then share
-        // GEMV launches four at a time, everything else goes out one product at a time
+        // x is produced and quantized once per activation format (Q8_0 / Q8_K) in use; weights of one type
+        // then share GEMV launches four at a time, everything else goes out one product at a time
+        size_t act_need = 0;
+        for (int i = 0; i < count; i++) {
+            const size_t t = plan_act(nullptr, mi_qmm_vec_dot_type(ws[i]->dev.type), K, n).total;
+            act_need = t > act_need ? t : act_need;
+        }
+        if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, act_need + align_up((size_t)n * 4, 256), ctx->stream))) return rc;
+        if (pr.kind == PRODUCE_RMSNORM) {
+            float *scales = (float *)((char *)ctx->act_buf + act_need);
+            HIP_TRY(launch_rms_norm(dx, nullptr, pr.eps, K, n, scales, nullptr, ctx->stream));
+            pr.row_scale = scales;
+        }
         for (int q8 : {(int)T_Q8_0, (int)T_Q8_K}) {
             std::vector<int> idx;
             for (int i = 0; i < count; i++)
                 if (mi_qmm_vec_dot_type(ws[i]->dev.type) == q8) idx.push_back(i);
             if (idx.empty()) continue;
-            const ActPlanes probe = plan_act(nullptr, q8, K, n);
-            if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
             const ActPlanes p = plan_act(ctx->act_buf, q8, K, n);
-            HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+            HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream,
+                                        pr.kind == PRODUCE_NONE ? nullptr : &pr));
             DevAct a;
             a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
             size_t j = 0;
@@ -614,6 +644,89 @@ int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int cou
     if (location == MI_QMM_HOST) {
         for (int i = 0; i < count; i++)
             HIP_TRY(hipMemcpyAsync(ys[i], dys[i], (size_t)(n * ws[i]->dev.M) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+// x, y (and more) of `bytes` each between the caller's location and the device: staged through io_buf for
+// host callers.  Returns device pointers in dptr[]; the first n_in are copied in.
+int stage_in(mi_qmm_ctx *ctx, int location, const void *const *src, const size_t *bytes, int n_in, int n_total,
+             void **dptr) {
+    if (location == MI_QMM_DEVICE) {
+        for (int i = 0; i < n_total; i++) dptr[i] = const_cast<void *>(src[i]);
+        return MI_QMM_OK;
+    }
+    size_t off = 0, offs[8];
+    for (int i = 0; i < n_total; i++) { offs[i] = off; off += align_up(bytes[i], 256); }
+    int rc = reserve(&ctx->io_buf, &ctx->io_cap, off, ctx->stream);
+    if (rc) return rc;
+    for (int i = 0; i < n_total; i++) {
+        dptr[i] = (char *)ctx->io_buf + offs[i];
+        if (i < n_in && src[i] && bytes[i])
+            HIP_TRY(hipMemcpyAsync(dptr[i], src[i], bytes[i], hipMemcpyHostToDevice, ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+int check_elementwise_args(mi_qmm_ctx *ctx, int64_t k, int64_t n, int location) {
+    if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
+        return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
+    if (k < 0 || n < 0) return fail(MI_QMM_ERR_INVALID, "k=%lld n=%lld must be non-negative", (long long)k, (long long)n);
+    if (k % 4) return fail(MI_QMM_ERR_UNSUPPORTED, "k=%lld must be a multiple of 4", (long long)k);
+    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    return check_ctx(ctx);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x, int64_t n,
+                        float *const *ys, int location) {
+    return mulmat_multi_impl(ctx, ws, count, nullptr, x, n, ys, location);
+}
+
+int mi_qmm_mulmat_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int producer, const float *aux,
+                           float eps, const float *x, int64_t n, float *const *ys, int location) {
+    if (producer != MI_QMM_PRODUCE_NONE && producer != MI_QMM_PRODUCE_RMSNORM && producer != MI_QMM_PRODUCE_SWIGLU)
+        return fail(MI_QMM_ERR_INVALID, "unknown producer %d", producer);
+    const Produce pr{producer, producer == MI_QMM_PRODUCE_NONE ? nullptr : aux, eps, nullptr};
+    return mulmat_multi_impl(ctx, ws, count, &pr, x, n, ys, location);
+}
+
+int mi_qmm_rms_norm(mi_qmm_ctx *ctx, const float *x, const float *g, float eps, int64_t k, int64_t n, float *y,
+                    int location) {
+    int rc = check_elementwise_args(ctx, k, n, location);
+    if (rc) return rc;
+    if (!(eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
+    if (k * n == 0) return MI_QMM_OK;
+    if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
+    const size_t bytes[3] = {(size_t)(n * k) * 4, g ? (size_t)k * 4 : 0, (size_t)(n * k) * 4};
+    const void *src[3] = {x, g, y};
+    void *d[3];
+    if ((rc = stage_in(ctx, location, src, bytes, 2, 3, d))) return rc;
+    HIP_TRY(launch_rms_norm((const float *)d[0], g ? (const float *)d[1] : nullptr, eps, k, n, nullptr, (float *)d[2],
+                            ctx->stream));
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(y, d[2], bytes[2], hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+int mi_qmm_swiglu(mi_qmm_ctx *ctx, const float *gate, const float *up, int64_t k, int64_t n, float *y, int location) {
+    int rc = check_elementwise_args(ctx, k, n, location);
+    if (rc) return rc;
+    if (k * n == 0) return MI_QMM_OK;
+    if (!gate || !up || !y) return fail(MI_QMM_ERR_INVALID, "gate, up or y is NULL");
+    const size_t b = (size_t)(n * k) * 4, bytes[3] = {b, b, b};
+    const void *src[3] = {gate, up, y};
+    void *d[3];
+    if ((rc = stage_in(ctx, location, src, bytes, 2, 3, d))) return rc;
+    HIP_TRY(launch_swiglu((const float *)d[0], (const float *)d[1], n * k, (float *)d[2], ctx->stream));
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(y, d[2], b, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));
     }
     return MI_QMM_OK;

@@ -22,6 +22,7 @@
 #include <hip/hip_fp16.h>
 
 #include "internal.h"
+#include "produce_dev.h"
 #include "quant_dev.h"
 
 namespace miqmm {
@@ -588,18 +589,19 @@ struct LdsAct {
 // are requested by prefetch_x (before the wave's first weight load), the rest inside quantize_x_to_lds.
 constexpr int XPRE = 4;
 
+template <int XP>
 __device__ __forceinline__ void prefetch_x(const float4 *__restrict__ x4, int total4, int wave, int nwaves, int lane,
-                                           float4 (&xpre)[XPRE]) {
+                                           float4 (&xpre)[XP]) {
 #pragma unroll
-    for (int j = 0; j < XPRE; j++) {
+    for (int j = 0; j < XP; j++) {
         const int i4 = (wave + j * nwaves) * 64 + lane;
         xpre[j] = x4[min(i4, total4 - 1)];  // clamped: the loads stay unconditional
     }
 }
 
-template <class P>
+template <class P, int XP>
 __device__ __forceinline__ void quantize_x_to_lds(const float4 *__restrict__ x4, int total4, int wave, int nwaves,
-                                                  int lane, const float4 (&xpre)[XPRE], int8_t *lqs, float *ld_,
+                                                  int lane, const float4 (&xpre)[XP], int8_t *lqs, float *ld_,
                                                   int16_t *lbs) {
     auto quantize_piece = [&](int c, float4 v) {
         const int i4 = c * 64 + lane;
@@ -625,11 +627,11 @@ __device__ __forceinline__ void quantize_x_to_lds(const float4 *__restrict__ x4,
         }
     };
 #pragma unroll
-    for (int j = 0; j < XPRE; j++) {
+    for (int j = 0; j < XP; j++) {
         const int c = wave + j * nwaves;
         if (c * 64 < total4) quantize_piece(c, xpre[j]);  // wave-uniform
     }
-    for (int c = wave + XPRE * nwaves; c * 64 < total4; c += nwaves)
+    for (int c = wave + XP * nwaves; c * 64 < total4; c += nwaves)
         quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
 }
 
@@ -650,9 +652,13 @@ struct ThinArgs {
 // workgroup size limit: 16 waves leave a wave 128 VGPRs, enough for up to three activation columns
 constexpr int thin_max_waves(int nc, bool f32) { return f32 ? (nc <= 3 ? 16 : 8) : 4; }
 
-template <class P, int NC, bool DIRECT, bool F32, int RPL>
-__global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(ThinArgs ta, DevAct a, const float *__restrict__ xf,
-                                                         int col0, int rows_per_wave, int kw, int rw_log2) {
+// XMODE: where the activations come from -- 0: quantized planes (a); 1: f32 x, quantized here; 2 / 3: f32 x
+// that first goes through RMSNorm / SwiGLU (pr; one column, all of x in the waves' XP prefetch registers: XP is
+// 1 when a piece per wave covers the row, which keeps the kernel at two workgroups per CU).
+template <class P, int NC, bool DIRECT, int XMODE, int RPL, int XP = XPRE>
+__global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(ThinArgs ta, DevAct a, const float *__restrict__ xf,
+                                                         int col0, int rows_per_wave, int kw, int rw_log2, Produce pr) {
+    constexpr bool F32 = XMODE != 0;
     // LDS: the NC activation columns (quants, block scales, block sums), then, unless DIRECT, the
     // partial sums [rows_per_wg][NC][kw].
     extern __shared__ __align__(16) uint8_t smem[];
@@ -694,15 +700,42 @@ __global__ __launch_bounds__(F32 && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col0 * K);
     const int total4 = (int)((int64_t)NC * K / 4);  // float4 pieces over all NC columns
     const int nwaves = blockDim.x >> 6;
-    float4 xpre[XPRE];
+    float4 xpre[XP], apre[XP];
     if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
+    // the producer's operand, requested unconditionally (RMSNorm without a weight reads x again and ignores
+    // it) so that the number of loads in flight stays known to the waits below
+    const bool has_aux = XMODE == 3 || (XMODE == 2 && pr.aux != nullptr);
+    if (XMODE >= 2) prefetch_x(has_aux ? reinterpret_cast<const float4 *>(pr.aux) : x4, total4, wave, nwaves, lane, apre);
     typename P::Raw cur;
     if (nrw > 0) cur = P::load(w, g, r0 + rl0 + min(run, nrw - 1));
+    constexpr size_t PSUM_BYTES = XMODE == 2 ? XPRE * 16 * sizeof(double) : 0;  // one sum per 256-element piece
+    if (XMODE == 2) {
+        // RMSNorm: piece sums of squares through LDS, added in piece order by every thread
+        double *psum = reinterpret_cast<double *>(smem + act_bytes);
+#pragma unroll
+        for (int j = 0; j < XP; j++) {
+            const int c = wave + j * nwaves;
+            if (c * 64 < total4) {  // wave-uniform
+                const double sq = piece_sumsq(c * 64 + lane < total4 ? xpre[j] : make_float4(0.f, 0.f, 0.f, 0.f));
+                if (lane == 0) psum[c] = sq;
+            }
+        }
+        __syncthreads();
+        double tot = 0.0;
+        for (int c = 0; c * 64 < total4; c++) tot += psum[c];
+        const float scale = rms_scale_of(tot, K, pr.eps);
+#pragma unroll
+        for (int j = 0; j < XP; j++) xpre[j] = rms_apply(xpre[j], scale, apre[j], has_aux);
+    }
+    if (XMODE == 3) {
+#pragma unroll
+        for (int j = 0; j < XP; j++) xpre[j] = swiglu_apply(xpre[j], apre[j]);
+    }
     if (F32) {
-        quantize_x_to_lds<P>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
+        quantize_x_to_lds<P, XP>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
         __syncthreads();
     }
-    float *part = reinterpret_cast<float *>(smem + act_bytes);
+    float *part = reinterpret_cast<float *>(smem + act_bytes + PSUM_BYTES);
 
     if (nrw > 0) {
         typename P::Act act[NC];
@@ -767,8 +800,10 @@ size_t thin_act_lds(int64_t K, int nc) {
     return (b + 15) / 16 * 16;
 }
 
+// produce: the f32 activations go through a producer first (one column; room for RMSNorm's piece sums, and
+// every piece of x must sit in a prefetch register of some wave)
 template <class P>
-bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p) {
+bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool produce = false) {
     const int nseg = (int)((K + P::SEG - 1) / P::SEG);
     if (nseg < 1 || nseg > 8) return false;
     p.spw = 1;
@@ -795,27 +830,37 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p) {
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
     p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float));
+    if (produce) {
+        if (!f32 || nc != 1 || K > (int64_t)XPRE * p.kw * p.rw * 256) return false;
+        p.lds += XPRE * 16 * sizeof(double);
+    }
     return p.lds <= THIN_LDS_MAX;
 }
 
-template <class P, int NC>
-void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, const float *xf, int col0, hipStream_t s) {
+template <class P, int NC, int XMODE, int XP = XPRE>
+void launch_thin_mode(const Plan &p, const ThinArgs &ma, const DevAct &a, const float *xf, int col0, const Produce &pr,
+                      hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
     const int rpw = p.rows_per_wg >> p.rw_log2;
-#define THIN_LAUNCH(DIRECT, F32, RPL) \
-    gemv_thin_kernel<P, NC, DIRECT, F32, RPL><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2)
-    if (xf) {
-        if (p.kw > 1) THIN_LAUNCH(false, true, 1);
-        else if (p.rpl == 4) THIN_LAUNCH(true, true, 4);
-        else if (p.rpl == 2) THIN_LAUNCH(true, true, 2);
-        else THIN_LAUNCH(true, true, 1);
-    } else {
-        if (p.kw > 1) THIN_LAUNCH(false, false, 1);
-        else if (p.rpl == 4) THIN_LAUNCH(true, false, 4);
-        else if (p.rpl == 2) THIN_LAUNCH(true, false, 2);
-        else THIN_LAUNCH(true, false, 1);
-    }
+#define THIN_LAUNCH(DIRECT, RPL) \
+    gemv_thin_kernel<P, NC, DIRECT, XMODE, RPL, XP><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr)
+    if (p.kw > 1) THIN_LAUNCH(false, 1);
+    else if (p.rpl == 4) THIN_LAUNCH(true, 4);
+    else if (p.rpl == 2) THIN_LAUNCH(true, 2);
+    else THIN_LAUNCH(true, 1);
 #undef THIN_LAUNCH
+}
+
+template <class P, int NC>
+void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, const float *xf, int col0, const Produce &pr,
+                 hipStream_t s) {
+    const bool one_piece = ma.K <= (int64_t)256 * p.kw * p.rw;  // a piece per wave covers the row
+    if (!xf) launch_thin_mode<P, NC, 0>(p, ma, a, xf, col0, pr, s);
+    else if (NC == 1 && pr.kind == PRODUCE_RMSNORM && one_piece) launch_thin_mode<P, 1, 2, 1>(p, ma, a, xf, col0, pr, s);
+    else if (NC == 1 && pr.kind == PRODUCE_RMSNORM) launch_thin_mode<P, 1, 2>(p, ma, a, xf, col0, pr, s);
+    else if (NC == 1 && pr.kind == PRODUCE_SWIGLU && one_piece) launch_thin_mode<P, 1, 3, 1>(p, ma, a, xf, col0, pr, s);
+    else if (NC == 1 && pr.kind == PRODUCE_SWIGLU) launch_thin_mode<P, 1, 3>(p, ma, a, xf, col0, pr, s);
+    else launch_thin_mode<P, NC, 1>(p, ma, a, xf, col0, pr, s);
 }
 
 template <class P, int NC, int SPW, int U>
@@ -829,11 +874,12 @@ void launch_one(const Plan &p, const MultiArgs &ma, const DevAct &a, int col0, h
 
 template <class P>
 hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const DevAct &a, const float *xf, int col0,
-                       int nc, int num_cus, hipStream_t s) {
+                       int nc, int num_cus, const Produce &pr, hipStream_t s) {
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i].M;
     Plan p;
-    const bool thin = make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, p);
+    const bool thin = make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, p, pr.kind != PRODUCE_NONE);
+    if (pr.kind != PRODUCE_NONE && !thin) return hipErrorInvalidValue;  // callers ask gemv_produce_supported() first
     if (xf && !thin) return hipErrorInvalidValue;  // callers ask gemv_f32_supported() first
     if (!thin) {
         if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
@@ -860,14 +906,14 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
         }
         ta.K = ws[0].K; ta.type = ws[0].type;
         switch (nc) {
-        case 1: launch_thin<P, 1>(p, ta, a, xf, col0, s); break;
-        case 2: launch_thin<P, 2>(p, ta, a, xf, col0, s); break;
-        case 3: launch_thin<P, 3>(p, ta, a, xf, col0, s); break;
-        case 4: launch_thin<P, 4>(p, ta, a, xf, col0, s); break;
-        case 5: launch_thin<P, 5>(p, ta, a, xf, col0, s); break;
-        case 6: launch_thin<P, 6>(p, ta, a, xf, col0, s); break;
-        case 7: launch_thin<P, 7>(p, ta, a, xf, col0, s); break;
-        case 8: launch_thin<P, 8>(p, ta, a, xf, col0, s); break;
+        case 1: launch_thin<P, 1>(p, ta, a, xf, col0, pr, s); break;
+        case 2: launch_thin<P, 2>(p, ta, a, xf, col0, pr, s); break;
+        case 3: launch_thin<P, 3>(p, ta, a, xf, col0, pr, s); break;
+        case 4: launch_thin<P, 4>(p, ta, a, xf, col0, pr, s); break;
+        case 5: launch_thin<P, 5>(p, ta, a, xf, col0, pr, s); break;
+        case 6: launch_thin<P, 6>(p, ta, a, xf, col0, pr, s); break;
+        case 7: launch_thin<P, 7>(p, ta, a, xf, col0, pr, s); break;
+        case 8: launch_thin<P, 8>(p, ta, a, xf, col0, pr, s); break;
         default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
@@ -900,17 +946,17 @@ int gemv_max_multi() { return MAX_MULTI; }
 namespace {
 
 hipError_t dispatch(const DevWeight *ws, float *const *ys, int count, const DevAct &a, const float *xf, int col0,
-                    int ncols, int num_cus, hipStream_t s) {
+                    int ncols, int num_cus, hipStream_t s, const Produce &pr = Produce{PRODUCE_NONE, nullptr, 0.f, nullptr}) {
     if (count < 1 || count > MAX_MULTI || ncols < 1 || ncols > MAXC || col0 < 0 || col0 + ncols > a.N)
         return hipErrorInvalidValue;
     for (int i = 0; i < count; i++)
         if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || ws[i].M < 1 || !ys[i]) return hipErrorInvalidValue;
     if (ws[0].K < 1 || ws[0].K > gemv_max_k(ws[0].type) || a.K != ws[0].K) return hipErrorInvalidValue;
     switch (ws[0].type) {
-    case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
-    case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
-    case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
-    case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(ws, ys, count, a, xf, col0, ncols, num_cus, s) : hipErrorInvalidValue;
+    case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
+    case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
+    case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
+    case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
 }
@@ -951,13 +997,30 @@ bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
 }
 
 hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols,
-                                 int num_cus, hipStream_t s) {
+                                 int num_cus, hipStream_t s, const Produce *produce) {
     if (!x || count < 1) return hipErrorInvalidValue;
+    Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
+    if (produce) pr = *produce;
+    if (pr.kind < PRODUCE_NONE || pr.kind > PRODUCE_SWIGLU || (pr.kind == PRODUCE_SWIGLU && !pr.aux) ||
+        (pr.kind != PRODUCE_NONE && ncols != 1))
+        return hipErrorInvalidValue;
     DevAct a{};  // only the geometry is read: the kernel quantizes x itself
     a.K = ws[0].K;
     a.N = ncols;
     a.type = (ws[0].type == T_Q4_K || ws[0].type == T_Q6_K) ? T_Q8_K : T_Q8_0;
-    return dispatch(ws, ys, count, a, x, 0, ncols, num_cus, s);
+    return dispatch(ws, ys, count, a, x, 0, ncols, num_cus, s, pr);
+}
+
+bool gemv_produce_supported(int type, int64_t K, int64_t total_m) {
+    if (!gemv_f32_supported(type, K, total_m, 1)) return false;
+    Plan p;
+    switch (type) {
+    case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, 1, true, p, true);
+    case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, 1, true, p, true);
+    case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, 1, true, p, true);
+    case T_Q8_0: return make_thin_plan<PolQ8_0>(K, total_m, 1, true, p, true);
+    default: return false;
+    }
 }
 
 
@@ -1263,7 +1326,7 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     typename P::Raw cur;
     if (nrw > 0) cur = P::load(w, g, wrow0 + min(run, nrw - 1));
     if (F32) {
-        quantize_x_to_lds<P>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
+        quantize_x_to_lds<P, XPRE>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
         __syncthreads();
     }
     float *part = reinterpret_cast<float *>(smem + act_bytes);

@@ -5,13 +5,21 @@
 #include <stdint.h>
 
 #include "formats.h"
+#include "produce_dev.h"
 
 namespace miqmm {
 
 // kernel 1: f32 rows -> Q8_0 / Q8_K planes (bit-exact with the scalar CPU quantizers)
 // sd8 / sd16: block-sum digit planes for the GEMM (Q8_K only; may be null)
+// produce (optional): applied to x on the fly (RMSNORM needs row_scale from launch_rms_norm first)
 hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs,
-                               float *d, int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s);
+                               float *d, int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s,
+                               const Produce *produce = nullptr);
+// RMSNorm over rows of K floats: scale_out [N] (optional) = 1/sqrtf(mean(x^2)+eps) per row; y (optional) =
+// (x * scale) * g with g [K] or null.  SwiGLU: y = silu(gate) * up over count floats.
+hipError_t launch_rms_norm(const float *x, const float *g, float eps, int64_t K, int64_t N, float *scale_out, float *y,
+                           hipStream_t s);
+hipError_t launch_swiglu(const float *gate, const float *up, int64_t count, float *y, hipStream_t s);
 // planes -> GGUF block bytes (34 B / 292 B blocks), for callers that want the bytes
 hipError_t launch_pack_act_gguf(int q8_type, const int8_t *qs, const float *d, const int16_t *bsums,
                                 int64_t K, int64_t N, uint8_t *out, hipStream_t s);
@@ -31,8 +39,11 @@ int gemv_max_multi();
 // The same products from f32 activations x [ncols][K] (device): the kernel quantizes x in its own
 // prologue, saving the separate quantization launch.  Ask gemv_f32_supported() first.
 bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols);
+// produce (optional; one column; ask gemv_produce_supported() first): x goes through RMSNorm / SwiGLU in
+// the same prologue, before it is quantized.
 hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols,
-                                 int num_cus, hipStream_t s);
+                                 int num_cus, hipStream_t s, const Produce *produce = nullptr);
+bool gemv_produce_supported(int type, int64_t K, int64_t total_m);
 // largest K the GEMV handles for a weight type
 int64_t gemv_max_k(int type);
 // Expert-indexed GEMV: w is a stack of n_expert matrices (w.M = rows per expert * n_expert), a holds

@@ -4,23 +4,43 @@
 // quant_dev.h; this file holds the stand-alone kernels that write the structure-of-arrays planes the
 // GEMV / GEMM kernels read, and the repacking of those planes into GGUF block bytes.
 //
+// With a producer (RMSNorm, SwiGLU: produce_dev.h) the quantizers apply it to x on the fly, so the
+// normalized / gated activations exist only as Q8 planes; the same producers are also here as plain
+// f32 kernels for graph nodes whose result something other than a product reads.
+//
 // HBM-bound and tiny next to the weight stream (N*K*4 bytes in, ~N*K*1.14 out); one float4 per lane,
 // cross-lane max / sums over the 8 (Q8_0) or 64 (Q8_K) lanes that share a block.
 #include "internal.h"
+#include "produce_dev.h"
 #include "quant_dev.h"
 
 namespace miqmm {
 
 namespace {
 
+// float4 number t of x [N][K] after the producer
+template <int KIND>
+__device__ __forceinline__ float4 produced(const float4 *__restrict__ x, int64_t t, const Produce &pr, int64_t k4) {
+    const float4 v = x[t];
+    if (KIND == PRODUCE_RMSNORM) {
+        const int64_t row = t / k4;
+        const float4 *g4 = reinterpret_cast<const float4 *>(pr.aux);
+        return rms_apply(v, pr.row_scale[row], g4 ? g4[t - row * k4] : v, g4 != nullptr);
+    }
+    if (KIND == PRODUCE_SWIGLU) return swiglu_apply(v, reinterpret_cast<const float4 *>(pr.aux)[t]);
+    return v;
+}
+
 // 8 lanes per block of 32; 8 blocks per wave.  nblk = N*K/32 blocks in total.
+template <int KIND>
 __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float4 *__restrict__ x,
                                                             int *__restrict__ qs, float *__restrict__ d,
-                                                            int16_t *__restrict__ bsums, int64_t nblk) {
+                                                            int16_t *__restrict__ bsums, int64_t nblk, Produce pr,
+                                                            int64_t k4) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t blk = t >> 3;
     const bool live = blk < nblk;
-    const float4 v = live ? x[t] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 v = live ? produced<KIND>(x, t, pr, k4) : make_float4(0.f, 0.f, 0.f, 0.f);
     float dd;
     int sum;
     const int packed = q8_0_quantize_lane(v, dd, sum);
@@ -34,16 +54,18 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float4 *__rest
 }
 
 // one wave per super-block of 256; 4 waves per workgroup.  nblk = N*K/256.
+template <int KIND>
 __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__restrict__ x,
                                                             int *__restrict__ qs, float *__restrict__ d,
                                                             int16_t *__restrict__ bsums, uint8_t *__restrict__ sd8,
-                                                            uint8_t *__restrict__ sd16, int64_t nblk) {
+                                                            uint8_t *__restrict__ sd16, int64_t nblk, Produce pr,
+                                                            int64_t k4) {
     const int lane = threadIdx.x & 63;
     const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (blk >= nblk) return;  // whole wave leaves together
     float dd;
     int sum, pair;
-    const int packed = q8_K_quantize_lane(x[blk * 64 + lane], lane, dd, sum, pair);
+    const int packed = q8_K_quantize_lane(produced<KIND>(x, blk * 64 + lane, pr, k4), lane, dd, sum, pair);
     qs[blk * 64 + lane] = packed;
     if ((lane & 3) == 0) bsums[blk * 16 + (lane >> 2)] = (int16_t)sum;
     if (lane == 0) d[blk] = dd;
@@ -56,6 +78,42 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__rest
         sd8[blk * 16 + (lane >> 3)] = (uint8_t)(pair & 63);
         sd8[blk * 16 + 8 + (lane >> 3)] = (uint8_t)(pair >> 6);
     }
+}
+
+// RMSNorm, one workgroup per row of K floats: the row's scale (scale_out, optional) and the normalized row
+// times the weight g (y, optional; g may be null).  Piece sums go through LDS 512 at a time and are added
+// in piece order by every thread.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float4 *__restrict__ x, const float4 *__restrict__ g,
+                                                       float eps, int64_t K, float *__restrict__ scale_out,
+                                                       float4 *__restrict__ y) {
+    __shared__ double psum[512];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t n4 = K / 4, npieces = (n4 + 63) / 64;
+    const float4 *xr = x + (int64_t)blockIdx.x * n4;
+    double tot = 0.0;
+    for (int64_t base = 0; base < npieces; base += 512) {
+        const int64_t end = base + 512 < npieces ? base + 512 : npieces;
+        for (int64_t c = base + wave; c < end; c += 4) {
+            const int64_t i4 = c * 64 + lane;
+            const double s = piece_sumsq(i4 < n4 ? xr[i4] : make_float4(0.f, 0.f, 0.f, 0.f));
+            if (lane == 0) psum[c - base] = s;
+        }
+        __syncthreads();
+        for (int64_t c = base; c < end; c++) tot += psum[c - base];
+        __syncthreads();
+    }
+    const float scale = rms_scale_of(tot, K, eps);
+    if (scale_out && threadIdx.x == 0) scale_out[blockIdx.x] = scale;
+    if (y) {
+        float4 *yr = y + (int64_t)blockIdx.x * n4;
+        for (int64_t i4 = threadIdx.x; i4 < n4; i4 += 256) yr[i4] = rms_apply(xr[i4], scale, g ? g[i4] : xr[i4], g != nullptr);
+    }
+}
+
+__global__ __launch_bounds__(256) void swiglu_kernel(const float4 *__restrict__ gate, const float4 *__restrict__ up,
+                                                     float4 *__restrict__ y, int64_t n4) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256)
+        y[i] = swiglu_apply(gate[i], up[i]);
 }
 
 // planes -> GGUF bytes; one thread per output byte (a convenience path, not on the hot path)
@@ -94,20 +152,48 @@ __global__ void pack_q8_K_kernel(const int8_t *__restrict__ qs, const float *__r
 }  // namespace
 
 hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs, float *d,
-                               int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s) {
+                               int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s, const Produce *produce) {
     if (N * K == 0) return hipSuccess;
+    Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
+    if (produce) pr = *produce;
+    if ((pr.kind == PRODUCE_RMSNORM && !pr.row_scale) || (pr.kind == PRODUCE_SWIGLU && !pr.aux) ||
+        pr.kind < PRODUCE_NONE || pr.kind > PRODUCE_SWIGLU || K % 4)
+        return hipErrorInvalidValue;
+    const int64_t k4 = K / 4;
+    const float4 *x4 = (const float4 *)x;
     if (q8_type == T_Q8_0) {
         const int64_t nblk = N * K / QK;
         const int64_t threads = nblk * 8;
         const unsigned grid = (unsigned)((threads + 255) / 256);
-        quantize_q8_0_kernel<<<grid, 256, 0, s>>>((const float4 *)x, (int *)qs, d, bsums, nblk);
+        if (pr.kind == PRODUCE_RMSNORM) quantize_q8_0_kernel<PRODUCE_RMSNORM><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, nblk, pr, k4);
+        else if (pr.kind == PRODUCE_SWIGLU) quantize_q8_0_kernel<PRODUCE_SWIGLU><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, nblk, pr, k4);
+        else quantize_q8_0_kernel<PRODUCE_NONE><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, nblk, pr, k4);
     } else if (q8_type == T_Q8_K) {
         const int64_t nblk = N * K / QKK;
         const unsigned grid = (unsigned)((nblk + 3) / 4);
-        quantize_q8_K_kernel<<<grid, 256, 0, s>>>((const float4 *)x, (int *)qs, d, bsums, sd8, sd16, nblk);
+        if (pr.kind == PRODUCE_RMSNORM) quantize_q8_K_kernel<PRODUCE_RMSNORM><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, nblk, pr, k4);
+        else if (pr.kind == PRODUCE_SWIGLU) quantize_q8_K_kernel<PRODUCE_SWIGLU><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, nblk, pr, k4);
+        else quantize_q8_K_kernel<PRODUCE_NONE><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, nblk, pr, k4);
     } else {
         return hipErrorInvalidValue;
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_rms_norm(const float *x, const float *g, float eps, int64_t K, int64_t N, float *scale_out, float *y,
+                           hipStream_t s) {
+    if (N * K == 0) return hipSuccess;
+    if (!x || K % 4 || N > 0x7fffffff || (!scale_out && !y)) return hipErrorInvalidValue;
+    rms_norm_kernel<<<(unsigned)N, 256, 0, s>>>((const float4 *)x, (const float4 *)g, eps, K, scale_out, (float4 *)y);
+    return hipGetLastError();
+}
+
+hipError_t launch_swiglu(const float *gate, const float *up, int64_t count, float *y, hipStream_t s) {
+    if (count == 0) return hipSuccess;
+    if (!gate || !up || !y || count % 4) return hipErrorInvalidValue;
+    const int64_t n4 = count / 4, blocks = (n4 + 255) / 256;
+    swiglu_kernel<<<(unsigned)(blocks < 8192 ? blocks : 8192), 256, 0, s>>>((const float4 *)gate, (const float4 *)up,
+                                                                            (float4 *)y, n4);
     return hipGetLastError();
 }
 

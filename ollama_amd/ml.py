@@ -4,6 +4,7 @@ Names, argument meaning and error behaviour follow /root/reference/ml/backend.go
   Backend   :16-33   Load / Get(name) / NewContext / Close        (weights live here until Close)
   Context   :94-128  FromFloats / Compute / Close                 (tensors die with the context)
   Tensor    :130-153 Dim / Stride / Shape / DType / Bytes / Floats / Mulmat / MulmatFullPrec / MulmatID
+            :159, :180 RMSNorm(ctx, weight, eps) / SILU(ctx, up): the producers of a product's activations
   DType     :404-412
 The reference's tensor ops build a lazy graph and have no error returns: Mulmat records a node,
 Compute runs it, and a failure is a panic -- here a raised exception.  Shapes are ggml's: dimension 0
@@ -12,6 +13,8 @@ is the contiguous one, a weight is [K, M], activations are [K, N], ``W.Mulmat(ct
 Everything that computes goes through the C ABI (``ollama_amd.qmm``).  Compute groups the Mulmat
 nodes of a graph by the ``x`` they read: decode-sized ones (N <= 8) of the same weight type run as one
 multi-tensor launch that quantizes ``x`` in its prologue; larger ones share one quantization of ``x``.
+An RMSNorm or SILU(up) node that only products read is never materialized: it becomes the producer of
+those products' activations (``mi_qmm_mulmat_produced``).
 """
 from __future__ import annotations
 
@@ -48,6 +51,7 @@ class Tensor:
         self._data: Optional[np.ndarray] = None          # f32 values, flat in ggml order
         self._op: Optional[Tuple["Tensor", "Tensor"]] = None  # (W, x) of a pending Mulmat
         self._ids: Optional["Tensor"] = None             # third operand of a pending MulmatID
+        self._prod: Optional[Tuple[int, "Tensor", Optional["Tensor"], float]] = None  # pending RMSNorm / SILU(up)
 
     # -- shape queries, /root/reference/ml/backend.go:131-135
     def Dim(self, n: int) -> int:
@@ -115,6 +119,31 @@ class Tensor:
         """The quantized path already accumulates block sums in exact integers and scales in fp32."""
         return self.Mulmat(ctx, t2)
 
+    # -- the producers of a product's activations, :159 and :180
+    def RMSNorm(self, ctx: "Context", weight: Optional["Tensor"], eps: float) -> "Tensor":
+        """self = x [K, ...] f32, weight = [K] f32 or None  ->  (x / sqrt(mean(x^2) + eps)) * weight along
+        dimension 0, lazily."""
+        if self._type != qmm.F32 or (weight is not None and weight._type != qmm.F32):
+            raise TypeError("RMSNorm: operands must be f32")
+        if weight is not None and (weight._data is None or weight._data.size != self.Dim(0)):
+            raise ValueError(f"RMSNorm: the weight must hold {self.Dim(0)} values")
+        out = Tensor(self._shape)
+        out._prod = (qmm.PRODUCE_RMSNORM, self, weight, float(eps))
+        ctx._nodes.append(out)
+        return out
+
+    def SILU(self, ctx: "Context", *up: "Tensor") -> "Tensor":
+        """self = gate, up[0] = up, both f32 of one shape  ->  silu(gate) * up, lazily (ggml's swiglu).  The
+        bare activation (no ``up``) feeds no quantized product and is outside this path."""
+        if len(up) != 1:
+            raise TypeError("SILU: this path implements the gated form SILU(ctx, up) only")
+        if self._type != qmm.F32 or up[0]._type != qmm.F32 or self._shape != up[0]._shape:
+            raise ValueError(f"SILU: gate {self.Shape()} and up {up[0].Shape()} must be f32 of one shape")
+        out = Tensor(self._shape)
+        out._prod = (qmm.PRODUCE_SWIGLU, self, up[0], 0.0)
+        ctx._nodes.append(out)
+        return out
+
 
 class Context:
     """Holds the tensors of one graph; Compute runs the pending Mulmat nodes."""
@@ -144,55 +173,81 @@ class Context:
         return self
 
     def Compute(self, *tensors: Tensor) -> None:
-        """Run every pending node the given tensors depend on (here: all pending Mulmat nodes)."""
+        """Run the pending nodes in the order they were recorded.  Producer nodes (RMSNorm, SILU) are
+        materialized only when asked for here or read by something other than a Mulmat."""
         if self._closed:
             raise RuntimeError("Compute on a closed context")
-        pending = [t for t in self._nodes if t._data is None and t._op is not None]
+        pending = [t for t in self._nodes if t._data is None and (t._op is not None or t._prod is not None)]
         c = self._b._ctx
-        # expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
-        by_xi: Dict[Tuple[int, int, int], List[Tensor]] = {}
-        for t in [t for t in pending if t._ids is not None]:
-            by_xi.setdefault((id(t._op[1]), id(t._ids), t._op[0].Dim(2)), []).append(t)
-        for nodes in by_xi.values():
-            x, ids = nodes[0]._op[1], nodes[0]._ids
-            tokens, n_used = ids.Dim(1), ids.Dim(0)
-            b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
-            ys = c.mulmat_id_multi([t._op[0]._weight for t in nodes], nodes[0]._op[0].Dim(2), b,
-                                   ids._data.reshape(tokens, n_used))
-            for t, y in zip(nodes, ys):
-                t._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
-        pending = [t for t in pending if t._ids is None]
-        # group by activation tensor
-        by_x: Dict[int, List[Tensor]] = {}
+        # producer nodes that must exist as f32: requested, or read by another producer or by a MulmatID
+        needed = {id(t) for t in tensors}
         for t in pending:
-            by_x.setdefault(id(t._op[1]), []).append(t)
-        for nodes in by_x.values():
-            x = nodes[0]._op[1]
+            if t._prod is not None:
+                needed.update(id(s) for s in (t._prod[1], t._prod[2]) if s is not None)
+            elif t._ids is not None:
+                needed.add(id(t._op[1]))
+
+        def rows(t: Tensor) -> np.ndarray:
+            return t.Floats().reshape(-1, t.Dim(0))
+
+        for t in pending:
+            if t._data is not None:
+                continue  # computed with an earlier node of its group
+            if t._prod is not None:
+                if id(t) in needed:
+                    kind, src, aux, eps = t._prod
+                    if kind == qmm.PRODUCE_RMSNORM:
+                        t._data = c.rms_norm(rows(src), None if aux is None else aux.Floats(), eps).reshape(-1)
+                    else:
+                        t._data = c.swiglu(rows(src), rows(aux)).reshape(-1)
+                continue
+            x = t._op[1]
+            if t._ids is not None:
+                # expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
+                ids = t._ids
+                nodes = [u for u in pending if u._data is None and u._ids is ids and u._op[1] is x
+                         and u._op[0].Dim(2) == t._op[0].Dim(2)]
+                tokens, n_used = ids.Dim(1), ids.Dim(0)
+                b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
+                ys = c.mulmat_id_multi([u._op[0]._weight for u in nodes], t._op[0].Dim(2), b,
+                                       ids._data.reshape(tokens, n_used))
+                for u, y in zip(nodes, ys):
+                    u._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
+                continue
+            nodes = [u for u in pending if u._data is None and u._ids is None and u._op is not None and u._op[1] is x]
+            if x._data is None and x._prod is not None:
+                # x is a producer nobody needs in f32: it runs inside the products' own quantization
+                kind, src, aux, eps = x._prod
+                a = None if aux is None else (aux.Floats() if kind == qmm.PRODUCE_RMSNORM else rows(aux))
+                ys = c.mulmat_produced([u._op[0]._weight for u in nodes], kind, a, rows(src), eps)
+                for u, y in zip(nodes, ys):
+                    u._data = y.reshape(-1)
+                continue
             k = x.Dim(0)
-            n = x.Floats().size // k
-            xs = x.Floats().reshape(n, k)
-            by_type: Dict[int, List[Tensor]] = {}
-            for t in nodes:
-                by_type.setdefault(t._op[0]._type, []).append(t)
+            xs = rows(x)
+            n = xs.shape[0]
             if n <= 8:
                 # decode: the GEMV quantizes x itself; weights of one type share a launch, four at a time
+                by_type: Dict[int, List[Tensor]] = {}
+                for u in nodes:
+                    by_type.setdefault(u._op[0]._type, []).append(u)
                 for group in by_type.values():
                     for i in range(0, len(group), 4):
                         part = group[i:i + 4]
-                        ys = c.mulmat_multi([t._op[0]._weight for t in part], xs)
-                        for t, y in zip(part, ys):
-                            t._data = y.reshape(-1)  # [n][m] row-major == ggml [M, N] with dim 0 contiguous
+                        ys = c.mulmat_multi([u._op[0]._weight for u in part], xs)
+                        for u, y in zip(part, ys):
+                            u._data = y.reshape(-1)  # [n][m] row-major == ggml [M, N] with dim 0 contiguous
                 continue
             # prefill: quantize once per (x, q8 type), then one product per weight
             by_q8: Dict[int, List[Tensor]] = {}
-            for t in nodes:
-                by_q8.setdefault(qmm.vec_dot_type(t._op[0]._type), []).append(t)
+            for u in nodes:
+                by_q8.setdefault(qmm.vec_dot_type(u._op[0]._type), []).append(u)
             for q8, group in by_q8.items():
                 act = c.act_create(q8, k, n)
                 try:
                     c.act_quantize(act, xs)
-                    for t in group:
-                        t._data = c.mulmat_q8(t._op[0]._weight, act).reshape(-1)
+                    for u in group:
+                        u._data = c.mulmat_q8(u._op[0]._weight, act).reshape(-1)
                 finally:
                     act.free()
 
@@ -206,8 +261,9 @@ class Backend:
     ``ml.NewBackend(modelPath, params)`` receives, /root/reference/ml/backend.go:83 -- or a dict mapping a
     tensor name to (ggml_type, shape [K, M], block bytes), what fs/ggml hands out for a tensor
     (/root/reference/fs/ggml/gguf.go:281-308).  From a file, Load uploads every 2-D tensor (and every 3-D
-    expert stack) of a type the Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q6_K) straight from the file mapping; other tensors
-    (norms, f32 embeddings) are outside this path and are skipped."""
+    expert stack) of a type the Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q6_K) straight from the file mapping and
+    keeps 1-D f32 tensors (norm weights, the operand of RMSNorm) on the host; other tensors (f32 embeddings)
+    are outside this path and are skipped."""
 
     def __init__(self, tensors, device: int = 0):
         self._ctx = qmm.Context(device)
@@ -220,11 +276,15 @@ class Backend:
             from . import gguf
 
             with gguf.File(self._spec if isinstance(self._spec, str) else self._spec.decode()) as f:
-                infos = [t for t in f.TensorInfos() if len(t.Shape) in (2, 3) and qmm.vec_dot_type(t.Type) >= 0]
+                infos = [t for t in f.TensorInfos()
+                         if (len(t.Shape) in (2, 3) and qmm.vec_dot_type(t.Type) >= 0) or (len(t.Shape) == 1 and t.Type == qmm.F32)]
                 for i, ti in enumerate(infos):
                     t = Tensor(ti.Shape, ti.Type)
-                    t._weight = f.Upload(self._ctx, ti.Name)
                     t._raw = f.TensorBytes(ti.Name)
+                    if ti.Type == qmm.F32:
+                        t._data = np.frombuffer(t._raw, dtype=np.float32).copy()  # a norm weight: stays on the host
+                    else:
+                        t._weight = f.Upload(self._ctx, ti.Name)
                     self._tensors[ti.Name] = t
                     if progress:
                         progress((i + 1) / max(len(infos), 1))
@@ -232,6 +292,14 @@ class Backend:
             return
         total = max(len(self._spec), 1)
         for i, (name, (ggml_type, shape, raw)) in enumerate(self._spec.items()):
+            if ggml_type == qmm.F32 and len(shape) == 1:  # a norm weight: stays on the host
+                t = Tensor(shape, ggml_type)
+                t._data = np.ascontiguousarray(raw).view(np.float32).reshape(-1).copy()
+                if t._data.size != int(shape[0]):
+                    raise ValueError(f"{name}: {t._data.size} values for shape {list(shape)}")
+                t._raw = t._data.view(np.uint8)
+                self._tensors[name] = t
+                continue
             if len(shape) not in (2, 3):
                 raise ValueError(f"{name}: Mulmat takes 2-D weights and MulmatID 3-D expert stacks, got shape {list(shape)}")
             k, m = int(shape[0]), int(np.prod(shape[1:], dtype=np.int64))  # a stack is its experts' rows in a row

@@ -18,6 +18,7 @@ LIB_PATH = os.environ.get("MI_QMM_LIB") or os.path.join(_HERE, "libmi_qmm.so")
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 HOST, DEVICE = 0, 1
 PATH_AUTO, PATH_GEMV, PATH_GEMM = 0, 1, 2
+PRODUCE_NONE, PRODUCE_RMSNORM, PRODUCE_SWIGLU = 0, 1, 2
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, -3, -4, -5
 
 EXPORTS = [
@@ -26,6 +27,7 @@ EXPORTS = [
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
+    "mi_qmm_mulmat_produced", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
     "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
@@ -85,6 +87,10 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_q8_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_multi.restype = ci
     L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
+    L.mi_qmm_mulmat_produced.restype = ci
+    L.mi_qmm_mulmat_produced.argtypes = [vp, ctypes.POINTER(vp), ci, ci, vp, ctypes.c_float, vp, i64, ctypes.POINTER(vp), ci]
+    L.mi_qmm_rms_norm.restype = ci; L.mi_qmm_rms_norm.argtypes = [vp, vp, vp, ctypes.c_float, i64, i64, vp, ci]
+    L.mi_qmm_swiglu.restype = ci; L.mi_qmm_swiglu.argtypes = [vp, vp, vp, i64, i64, vp, ci]
     L.mi_qmm_host_alloc.restype = vp; L.mi_qmm_host_alloc.argtypes = [vp, ctypes.c_size_t]
     L.mi_qmm_host_free.restype = None; L.mi_qmm_host_free.argtypes = [vp, vp]
     L.mi_qmm_mulmat_id_multi.restype = ci
@@ -328,6 +334,62 @@ class Context:
         wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
         yp = (ctypes.c_void_p * len(ws))(*[ctypes.c_void_p(int(p)) for p in y_ptrs])
         _check(lib().mi_qmm_mulmat_multi(self._h, wh, len(ws), ctypes.c_void_p(int(x_ptr)), n, yp, DEVICE))
+
+    def mulmat_produced(self, ws, producer: int, aux, x: np.ndarray, eps: float = 0.0):
+        """ws[i] . Q8(producer(x)): PRODUCE_RMSNORM with aux = norm weight [k] or None, PRODUCE_SWIGLU with
+        aux = up [n, k]; host arrays out"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        n, k = x.shape
+        if any(w.k != k for w in ws):
+            raise ValueError(f"x has k={k}, weights have k={[w.k for w in ws]}")
+        if aux is not None:
+            aux = np.ascontiguousarray(aux, dtype=np.float32)
+            want = (n, k) if producer == PRODUCE_SWIGLU else (k,)
+            if producer == PRODUCE_SWIGLU and aux.ndim == 1:
+                aux = aux[None, :]
+            if aux.shape != want:
+                raise ValueError(f"aux has shape {aux.shape}, the producer wants {want}")
+        ys = [np.empty((n, w.m), dtype=np.float32) for w in ws]
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[y.ctypes.data_as(ctypes.c_void_p) for y in ys])
+        _check(lib().mi_qmm_mulmat_produced(self._h, wh, len(ws), producer, _ptr(aux) if aux is not None else None,
+                                            eps, x.ctypes.data_as(ctypes.c_void_p), n, yp, HOST))
+        return ys
+
+    def mulmat_produced_device(self, ws, producer: int, aux_ptr, x_ptr: int, n: int, y_ptrs, eps: float = 0.0):
+        """device pointers; one launch for one activation row and up to 4 weights of one type"""
+        wh = (ctypes.c_void_p * len(ws))(*[w._h for w in ws])
+        yp = (ctypes.c_void_p * len(ws))(*[ctypes.c_void_p(int(p)) for p in y_ptrs])
+        _check(lib().mi_qmm_mulmat_produced(self._h, wh, len(ws), producer,
+                                            ctypes.c_void_p(int(aux_ptr)) if aux_ptr else None, eps,
+                                            ctypes.c_void_p(int(x_ptr)), n, yp, DEVICE))
+
+    def rms_norm(self, x: np.ndarray, g, eps: float) -> np.ndarray:
+        """(x / sqrt(mean(x^2) + eps)) * g per row; g f32 [k] or None"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        n, k = x.shape
+        if g is not None:
+            g = np.ascontiguousarray(g, dtype=np.float32)
+            if g.shape != (k,):
+                raise ValueError(f"g has shape {g.shape}, x has k={k}")
+        y = np.empty_like(x)
+        _check(lib().mi_qmm_rms_norm(self._h, _ptr(x), _ptr(g) if g is not None else None, eps, k, n, _ptr(y), HOST))
+        return y
+
+    def swiglu(self, gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+        """silu(gate) * up, f32 [n, k]"""
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        up = np.ascontiguousarray(up, dtype=np.float32)
+        if gate.shape != up.shape:
+            raise ValueError(f"gate {gate.shape} and up {up.shape} differ")
+        g2 = gate.reshape(-1, gate.shape[-1])
+        y = np.empty_like(g2)
+        _check(lib().mi_qmm_swiglu(self._h, _ptr(g2), _ptr(up), g2.shape[1], g2.shape[0], _ptr(y), HOST))
+        return y.reshape(gate.shape)
 
     def mulmat_id(self, w: Weight, n_expert: int, b: np.ndarray, ids: np.ndarray) -> np.ndarray:
         """w: n_expert stacked matrices uploaded as one weight of m = rows * n_expert; b: f32

@@ -53,6 +53,8 @@ def lib() -> ctypes.CDLL:
         L.ref_mul_mat.argtypes = [ci, vp, i64, i64, vp, i64, vp, vp, ci]
         L.ref_mul_mat_id.restype = ci
         L.ref_mul_mat_id.argtypes = [ci, vp, i64, i64, i64, vp, i64, vp, i64, i64, vp]
+        L.ref_rms_norm.restype = None; L.ref_rms_norm.argtypes = [vp, vp, ctypes.c_float, i64, i64, vp]
+        L.ref_swiglu.restype = None; L.ref_swiglu.argtypes = [vp, vp, i64, vp]
         _lib = L
     return _lib
 
@@ -156,6 +158,28 @@ def mul_mat_id(wtype: int, w: np.ndarray, k: int, m: int, n_expert: int, b: np.n
         raise IndexError("expert id outside 0..n_expert-1")
     if rc != 0:
         raise ValueError("ref_mul_mat_id failed")
+    return y
+
+
+def rms_norm(x: np.ndarray, g, eps: float) -> np.ndarray:
+    """x: f32 [n, k]; g: f32 [k] or None -> (x / sqrt(mean(x^2) + eps)) * g, row by row."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.ndim == 2
+    y = np.empty_like(x)
+    if g is not None:
+        g = np.ascontiguousarray(g, dtype=np.float32)
+        assert g.shape == (x.shape[1],)
+    lib().ref_rms_norm(_p(x), _p(g) if g is not None else None, eps, x.shape[1], x.shape[0], _p(y))
+    return y
+
+
+def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """silu(gate) * up, elementwise (f32)."""
+    gate = np.ascontiguousarray(gate, dtype=np.float32)
+    up = np.ascontiguousarray(up, dtype=np.float32)
+    assert gate.shape == up.shape
+    y = np.empty_like(gate)
+    lib().ref_swiglu(_p(gate), _p(up), gate.size, _p(y))
     return y
 
 

@@ -780,3 +780,34 @@ int ref_mul_mat_id(int wtype, const void *as, int64_t k, int64_t m, int64_t n_ex
     free(xq);
     return 0;
 }
+
+/*
+ * Producers of the activations, the steps in front of the path (Tensor.RMSNorm and Tensor.SILU with an
+ * "up" operand, /root/reference/ml/backend.go:159 and :180; the arithmetic is upstream ggml's
+ * ggml_compute_forward_rms_norm_f32, ggml_compute_forward_mul and ggml_vec_swiglu_f32, restated from
+ * their published scalar loops).
+ *
+ * rms_norm, per row of k floats: the squares are formed in fp32 and accumulated in double in element
+ * order; mean = (float)(sum / k); scale = 1.0f / sqrtf(mean + eps); y = x * scale.  The weight g, when
+ * given, is the separate broadcast multiply that follows in the graph: y = (x * scale) * g, two
+ * roundings.
+ */
+void ref_rms_norm(const float *x, const float *g, float eps, int64_t k, int64_t n, float *y) {
+    for (int64_t r = 0; r < n; r++) {
+        const float *xr = x + r * k;
+        float *yr = y + r * k;
+        double sum = 0.0;
+        for (int64_t i = 0; i < k; i++) sum += (double)(xr[i] * xr[i]);
+        const float mean = (float)(sum / (double)k);
+        const float scale = 1.0f / sqrtf(mean + eps);
+        for (int64_t i = 0; i < k; i++) {
+            const float v = xr[i] * scale;
+            yr[i] = g ? v * g[i] : v;
+        }
+    }
+}
+
+/* swiglu, elementwise over count floats: y = silu(gate) * up with silu(v) = v / (1.0f + expf(-v)). */
+void ref_swiglu(const float *gate, const float *up, int64_t count, float *y) {
+    for (int64_t i = 0; i < count; i++) y[i] = gate[i] / (1.0f + expf(-gate[i])) * up[i];
+}

@@ -23,6 +23,10 @@
  *   its reduction to mul_mat (one expert; a pair's result equals mul_mat on that expert alone) and
  *   fp64 brute force.  The rule "slot i reads activation row i mod ne11" is upstream ggml's and the
  *   reference holds no test of it: PARITY UNPINNED for b_cols other than 1 and n_used.
+ *   rms_norm / swiglu (the producers in front of the path): pinned as mathematics (closed forms for
+ *   constant and one-hot rows, scale invariance, silu(v) - silu(-v) = v, fp64 evaluation with numpy
+ *   to 1e-6); the fp32 rounding of upstream's SIMD variants (vectorized expf, reduction order of the
+ *   sum of squares) is not fixed by anything in the reference: PARITY UNPINNED below 1e-6 relative.
  *   weight encoders q4_K / q6_K (make_qkx2_quants / make_qx_quants searches):
  *   PARITY UNPINNED bit-for-bit against llama-quantize (only self-consistency and error
  *   bounds are checked); q4_0 / q8_0 encoders are closed forms and pinned.
@@ -91,6 +95,14 @@ int  ref_mul_mat(int wtype, const void *w, int64_t k, int64_t m,
  */
 int  ref_mul_mat_id(int wtype, const void *as, int64_t k, int64_t m, int64_t n_expert, const float *b,
                     int64_t b_cols, const int32_t *ids, int64_t n_used, int64_t n_tokens, float *y);
+
+/*
+ * Producers of the activations (Tensor.RMSNorm, Tensor.SILU(up): /root/reference/ml/backend.go:159, :180).
+ * rms_norm: x [n][k]; g [k] or NULL; y[r][i] = (x[r][i] * scale_r) * g[i], scale_r = 1/sqrtf(mean(x_r^2) + eps).
+ * swiglu:   y[i] = silu(gate[i]) * up[i] over count elements.
+ */
+void ref_rms_norm(const float *x, const float *g, float eps, int64_t k, int64_t n, float *y);
+void ref_swiglu(const float *gate, const float *up, int64_t count, float *y);
 
 #ifdef __cplusplus
 }

@@ -63,6 +63,69 @@ def test_python_mirror_layer_graph():
     b.Close()
 
 
+def test_python_mirror_ffn_block_with_producers():
+    """x -> RMSNorm -> gate, up -> SILU(gate, up) -> down, the way a model's feed-forward block drives the
+    interface (/root/reference/ml/backend.go:159, :180).  The norm and the gating run inside the products'
+    quantization unless their values are asked for."""
+    from ollama_amd import ml
+
+    k, f = 1024, 1536
+    rng = np.random.default_rng(18)
+    mats = {"blk.0.ffn_gate.weight": (qmm.Q4_K, k, f), "blk.0.ffn_up.weight": (qmm.Q4_K, k, f),
+            "blk.0.ffn_down.weight": (qmm.Q6_K, f, k)}
+    spec, raws = {}, {}
+    for name, (t, kk, m) in mats.items():
+        raw = oracle.quantize(t, (rng.standard_normal((m, kk), dtype=np.float32) * np.float32(0.05)), nthreads=8)
+        spec[name] = (t, [kk, m], raw)
+        raws[name] = raw
+    g = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    spec["blk.0.ffn_norm.weight"] = (qmm.F32, [k], g)
+    b = ml.Backend(spec)
+    b.Load()
+    assert np.array_equal(b.Get("blk.0.ffn_norm.weight").Floats(), g)
+    for n in (1, 6, 40):
+        xv = rng.standard_normal((n, k), dtype=np.float32)
+        ctx = b.NewContext()
+        x = ctx.FromFloats(xv.reshape(-1), k, n)
+        h = x.RMSNorm(ctx, b.Get("blk.0.ffn_norm.weight"), 1e-5)
+        gate = b.Get("blk.0.ffn_gate.weight").Mulmat(ctx, h)
+        up = b.Get("blk.0.ffn_up.weight").Mulmat(ctx, h)
+        act = gate.SILU(ctx, up)
+        out = b.Get("blk.0.ffn_down.weight").Mulmat(ctx, act)
+        ctx.Compute(out)
+        with pytest.raises(RuntimeError):
+            h.Floats()   # never materialized: it ran inside the quantization of gate / up
+        hv = oracle.rms_norm(xv, g, 1e-5)
+        gv = oracle.mul_mat(qmm.Q4_K, raws["blk.0.ffn_gate.weight"], k, f, hv, nthreads=8)
+        uv = oracle.mul_mat(qmm.Q4_K, raws["blk.0.ffn_up.weight"], k, f, hv, nthreads=8)
+        assert npref.rel_err(gate.Floats().reshape(n, f), gv) <= 1e-3
+        # the oracle's down projection on the GPU's own gate / up values: isolates the last step
+        want = oracle.mul_mat(qmm.Q6_K, raws["blk.0.ffn_down.weight"], f, k,
+                              oracle.swiglu(gate.Floats().reshape(n, f), up.Floats().reshape(n, f)), nthreads=8)
+        assert npref.rel_err(out.Floats().reshape(n, k), want) <= 1e-3, n
+        # and the whole chain on the CPU
+        chain = oracle.mul_mat(qmm.Q6_K, raws["blk.0.ffn_down.weight"], f, k, oracle.swiglu(gv, uv), nthreads=8)
+        assert npref.rel_err(out.Floats().reshape(n, k), chain) <= 2e-3, n
+        # asking for the intermediate values gives the same result through the unfused kernels
+        ctx2 = b.NewContext()
+        x2 = ctx2.FromFloats(xv.reshape(-1), k, n)
+        h2 = x2.RMSNorm(ctx2, b.Get("blk.0.ffn_norm.weight"), 1e-5)
+        gate2 = b.Get("blk.0.ffn_gate.weight").Mulmat(ctx2, h2)
+        up2 = b.Get("blk.0.ffn_up.weight").Mulmat(ctx2, h2)
+        act2 = gate2.SILU(ctx2, up2)
+        out2 = b.Get("blk.0.ffn_down.weight").Mulmat(ctx2, act2)
+        ctx2.Compute(h2, act2, out2)
+        assert h2.Shape() == [k, n] and np.max(np.abs(h2.Floats().reshape(n, k) - hv)) < 1e-5
+        assert np.array_equal(out2.Floats(), out.Floats())
+        ctx.Close(); ctx2.Close()
+    ctx = b.NewContext()
+    with pytest.raises(TypeError):
+        ctx.FromFloats(np.zeros(k, np.float32), k, 1).SILU(ctx)
+    with pytest.raises(ValueError):
+        ctx.FromFloats(np.zeros(k, np.float32), k, 1).RMSNorm(ctx, ctx.FromFloats(np.zeros(8, np.float32), 8), 1e-5)
+    b.Close()
+
+
 def test_python_mirror_expert_graph(tmp_path):
     """a mixture-of-experts FFN the way a model drives it: router ids from FromInts, gate/up through
     MulmatID with one activation row per token, down with one row per used expert -- from a GGUF file

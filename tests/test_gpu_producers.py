@@ -1,0 +1,180 @@
+"""GPU parity of the activation producers (RMSNorm, SwiGLU) and of the products fused with them, through
+the C ABI, against the CPU oracle.
+
+Bars: RMSNorm within 2 ulp of the oracle (the double-precision sum of squares is taken in a different
+order, everything after it is the same correctly rounded fp32 arithmetic; in practice the bits agree);
+SwiGLU within 1e-6 relative (the device expf is within 1 ulp of libm's); fused products within 1e-3 of the
+oracle chain (the bar of the products themselves) and bit-identical to the library's own two-step path.
+"""
+import numpy as np
+import pytest
+
+import npref
+import oracle
+from hipmem import DeviceArray
+from npref import Q4_0, Q4_K, Q6_K, Q8_0
+from ollama_amd import qmm
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+WTYPES = [Q4_0, Q8_0, Q4_K, Q6_K]
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = qmm.Context(0)
+    yield c
+    c.close()
+
+
+def _weights(t, m, k, seed):
+    rng = np.random.default_rng(seed)
+    return oracle.quantize(t, (rng.standard_normal((m, k), dtype=np.float32) * np.float32(0.02)), nthreads=16)
+
+
+def _ulps(a, b):
+    a = np.ascontiguousarray(a, np.float32).view(np.int32).astype(np.int64)
+    b = np.ascontiguousarray(b, np.float32).view(np.int32).astype(np.int64)
+    return np.abs(a - b).max() if a.size else 0
+
+
+@pytest.mark.parametrize("n,k", [(1, 4), (1, 32), (3, 36), (1, 4096), (5, 14336), (2, 135168), (600, 128)])
+@pytest.mark.parametrize("with_g", [True, False])
+def test_rms_norm_matches_the_oracle(ctx, n, k, with_g):
+    """rows shorter than a 256-element piece, rows that are no multiple of one, rows of more than 512 pieces"""
+    rng = np.random.default_rng(k * 7 + n)
+    x = (rng.standard_normal((n, k)) * rng.uniform(0.05, 20, (n, 1))).astype(np.float32)
+    g = rng.standard_normal(k).astype(np.float32) if with_g else None
+    for eps in (1e-5, 1e-6):
+        got = ctx.rms_norm(x, g, eps)
+        want = oracle.rms_norm(x, g, eps)
+        assert _ulps(got, want) <= 2
+        assert np.count_nonzero(got != want) <= got.size // 1000
+
+
+def test_rms_norm_closed_forms_and_edges(ctx):
+    k = 1024
+    y = ctx.rms_norm(np.full((2, k), 3.0, np.float32), None, 1e-5)
+    assert np.all(y == np.float32(3.0) * (np.float32(1) / np.sqrt(np.float32(9.0) + np.float32(1e-5))))
+    assert np.all(ctx.rms_norm(np.zeros((1, k), np.float32), np.ones(k, np.float32), 1e-6) == 0)
+    x = np.zeros((1, k), np.float32); x[0, 1000] = -2.0
+    y = ctx.rms_norm(x, None, 0.0)
+    assert np.count_nonzero(y) == 1 and abs(y[0, 1000] + np.sqrt(k)) < 1e-4
+    assert ctx.rms_norm(np.zeros((0, k), np.float32), None, 1e-5).shape == (0, k)
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.rms_norm(np.zeros((1, 6), np.float32), None, 1e-5)
+    assert e.value.code == qmm.ERR_UNSUPPORTED
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.rms_norm(np.zeros((1, 8), np.float32), None, -1.0)
+    assert e.value.code == qmm.ERR_INVALID
+
+
+def test_swiglu_matches_the_oracle(ctx):
+    rng = np.random.default_rng(11)
+    gate = (rng.standard_normal((7, 14336)) * 3).astype(np.float32)
+    up = rng.standard_normal((7, 14336)).astype(np.float32)
+    gate[0, :12] = [0.0, -0.0, 88.0, -88.0, 100.0, -100.0, 1e-30, -1e-30, 20.0, -20.0, 87.3, -87.3]
+    got = ctx.swiglu(gate, up)
+    want = oracle.swiglu(gate, up)
+    assert np.all(np.isfinite(got))
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-30)) < 1e-6
+    one = np.ones((1, 8), np.float32)
+    v = np.array([[0.0, 100.0, -100.0, 1.0, -1.0, 30.0, -30.0, 0.5]], np.float32)
+    s = ctx.swiglu(v, one)
+    assert s[0, 0] == 0 and s[0, 1] == 100.0 and s[0, 2] == 0.0
+    assert np.allclose(s[0, 3] - s[0, 4], 1.0, atol=1e-6) and np.allclose(s[0, 5] - s[0, 6], 30.0, atol=1e-5)
+    assert ctx.swiglu(np.zeros((0, 8), np.float32), np.zeros((0, 8), np.float32)).shape == (0, 8)
+
+
+def _chain(t, wb, k, m, producer, aux, x, eps):
+    xp = oracle.rms_norm(x, aux, eps) if producer == qmm.PRODUCE_RMSNORM else oracle.swiglu(x, aux)
+    return oracle.mul_mat(t, wb, k, m, xp, nthreads=16)
+
+
+def _two_step(ctx, ws, producer, aux, x, eps):
+    xp = ctx.rms_norm(x, aux, eps) if producer == qmm.PRODUCE_RMSNORM else ctx.swiglu(x, aux)
+    return ctx.mulmat_multi(ws, xp)
+
+
+# decode: the GEMV produces x in its prologue.  Rows of one K segment, of several (down: 3.5), short rows that
+# go 2 and 4 to a load, a Q8_0 row that is no multiple of 256, and a K too long for the prefetch registers
+# (fused quantizer instead)
+DECODE = [(Q4_K, 4096, 300), (Q4_K, 14336, 130), (Q6_K, 4096, 200), (Q6_K, 2048, 64), (Q4_K, 1024, 96), (Q4_K, 256, 40),
+          (Q4_0, 4096, 128), (Q8_0, 4128, 70), (Q8_0, 512, 33), (Q4_0, 32, 5), (Q4_K, 24576, 48), (Q6_K, 14336, 77)]
+
+
+@pytest.mark.parametrize("t,k,m", DECODE)
+@pytest.mark.parametrize("producer", [qmm.PRODUCE_RMSNORM, qmm.PRODUCE_SWIGLU])
+def test_decode_product_fused_with_its_producer(ctx, t, k, m, producer):
+    rng = np.random.default_rng(t * 1000 + k + m + producer)
+    wbs = [_weights(t, m, k, 4000 + t + k), _weights(t, m + 7, k, 4001 + t + k)]
+    ws = [ctx.upload(t, wb, k, mm) for wb, mm in zip(wbs, (m, m + 7))]
+    x = (rng.standard_normal((1, k)) * 1.7).astype(np.float32)
+    aux = rng.standard_normal(k).astype(np.float32) if producer == qmm.PRODUCE_RMSNORM else rng.standard_normal((1, k)).astype(np.float32)
+    got = ctx.mulmat_produced(ws, producer, aux, x, eps=1e-5)
+    for y, wb, mm in zip(got, wbs, (m, m + 7)):
+        assert npref.rel_err(y, _chain(t, wb, k, mm, producer, aux, x, 1e-5)) < TOL
+    for y, y2 in zip(got, _two_step(ctx, ws, producer, aux, x, 1e-5)):
+        assert np.array_equal(y, y2)
+    if producer == qmm.PRODUCE_RMSNORM:  # the bare normalization
+        got = ctx.mulmat_produced(ws[:1], producer, None, x, eps=1e-6)
+        assert npref.rel_err(got[0], _chain(t, wbs[0], k, m, producer, None, x, 1e-6)) < TOL
+        assert np.array_equal(got[0], ctx.mulmat_multi(ws[:1], ctx.rms_norm(x, None, 1e-6))[0])
+    for w in ws:
+        w.free()
+
+
+# batches: fused quantizer (RMSNorm: row scales first), then the GEMV / skinny / GEMM kernels
+@pytest.mark.parametrize("t,k,m,n", [(Q4_K, 4096, 200, 2), (Q4_K, 2048, 100, 5), (Q6_K, 1024, 130, 12), (Q4_K, 1024, 257, 70),
+                                     (Q8_0, 1056, 90, 3), (Q4_0, 512, 64, 40), (Q8_0, 4096, 64, 9)])
+@pytest.mark.parametrize("producer", [qmm.PRODUCE_RMSNORM, qmm.PRODUCE_SWIGLU])
+def test_batch_product_fused_with_its_producer(ctx, t, k, m, n, producer):
+    rng = np.random.default_rng(t * 1000 + k + m + n + producer)
+    wb = _weights(t, m, k, 4100 + t + k)
+    w = ctx.upload(t, wb, k, m)
+    x = (rng.standard_normal((n, k)) * rng.uniform(0.2, 5, (n, 1))).astype(np.float32)
+    aux = rng.standard_normal(k).astype(np.float32) if producer == qmm.PRODUCE_RMSNORM else rng.standard_normal((n, k)).astype(np.float32)
+    got = ctx.mulmat_produced([w], producer, aux, x, eps=1e-5)[0]
+    assert npref.rel_err(got, _chain(t, wb, k, m, producer, aux, x, 1e-5)) < TOL
+    assert np.array_equal(got, _two_step(ctx, [w], producer, aux, x, 1e-5)[0])
+    w.free()
+
+
+def test_produced_weights_of_two_types_and_device_pointers(ctx):
+    """gate (Q4_K) and a Q6_K matrix behind one RMSNorm; the same call on device pointers"""
+    k, rng = 4096, np.random.default_rng(77)
+    wbs = [_weights(Q4_K, 120, k, 4200), _weights(Q6_K, 90, k, 4201), _weights(Q8_0, 50, k, 4202)]
+    ws = [ctx.upload(t, wb, k, m) for t, wb, m in zip((Q4_K, Q6_K, Q8_0), wbs, (120, 90, 50))]
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    g = rng.standard_normal(k).astype(np.float32)
+    got = ctx.mulmat_produced(ws, qmm.PRODUCE_RMSNORM, g, x, eps=1e-5)
+    for y, t, wb, m in zip(got, (Q4_K, Q6_K, Q8_0), wbs, (120, 90, 50)):
+        assert npref.rel_err(y, _chain(t, wb, k, m, qmm.PRODUCE_RMSNORM, g, x, 1e-5)) < TOL
+    dx, dg = DeviceArray(x), DeviceArray(g)
+    dys = [DeviceArray(np.zeros((1, m), np.float32), zero=True) for m in (120, 90, 50)]
+    ctx.mulmat_produced_device(ws, qmm.PRODUCE_RMSNORM, dg.ptr, dx.ptr, 1, [d.ptr for d in dys], eps=1e-5)
+    ctx.sync()
+    for d, y in zip(dys, got):
+        assert np.array_equal(d.numpy(), y)
+    for d in [dx, dg] + dys:
+        d.free()
+    for w in ws:
+        w.free()
+
+
+def test_produced_errors(ctx):
+    k = 256
+    w = ctx.upload(Q4_K, _weights(Q4_K, 8, k, 1), k, 8)
+    x = np.ones((1, k), np.float32)
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_produced([w], 7, None, x)
+    assert e.value.code == qmm.ERR_INVALID
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_produced([w], qmm.PRODUCE_SWIGLU, None, x)
+    assert e.value.code == qmm.ERR_INVALID
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_produced([w], qmm.PRODUCE_RMSNORM, None, x, eps=-1.0)
+    assert e.value.code == qmm.ERR_INVALID
+    assert ctx.mulmat_produced([w], qmm.PRODUCE_NONE, None, x)[0].shape == (1, 8)
+    assert ctx.mulmat_produced([w], qmm.PRODUCE_RMSNORM, None, np.zeros((0, k), np.float32))[0].shape == (0, 8)
+    w.free()

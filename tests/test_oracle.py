@@ -385,3 +385,55 @@ def test_q4_0_and_q8_0_encoders_closed_form():
     # Q8_0 weight encoder is the activation quantizer
     y = np.random.default_rng(3).standard_normal(64).astype(np.float32)
     assert np.array_equal(oracle.quantize(Q8_0, y).reshape(-1), npref.quantize_q8_0(y))
+
+
+# ---- producers of the activations: RMSNorm, SwiGLU ------------------------------------------------
+
+def test_rms_norm_closed_forms():
+    """constant row c -> c / sqrt(c^2 + eps); one-hot row a*e_j -> a / sqrt(a^2/k + eps) at j, 0 elsewhere;
+    eps = 0 makes the result invariant under scaling x; the weight multiplies elementwise afterwards"""
+    k = 512
+    for c, eps in ((3.0, 1e-5), (-0.25, 1e-6), (1.0, 0.5)):
+        y = oracle.rms_norm(np.full((1, k), c, np.float32), None, eps)
+        want = np.float32(c) * (np.float32(1) / np.sqrt(np.float32(np.float32(c) * np.float32(c)) + np.float32(eps)))
+        assert np.all(y == want)
+    x = np.zeros((1, k), np.float32); x[0, 77] = 4.0
+    y = oracle.rms_norm(x, None, 1e-5)
+    assert abs(y[0, 77] - 4.0 / np.sqrt(16.0 / k + 1e-5)) < 1e-5 and np.count_nonzero(y) == 1
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, k), dtype=np.float32)
+    assert np.allclose(oracle.rms_norm(x, None, 0.0), oracle.rms_norm(4 * x, None, 0.0), rtol=1e-6)
+    g = rng.standard_normal(k, dtype=np.float32)
+    assert np.array_equal(oracle.rms_norm(x, g, 1e-5), oracle.rms_norm(x, None, 1e-5) * g)
+    assert np.all(oracle.rms_norm(np.zeros((2, k), np.float32), g, 1e-5) == 0)
+
+
+def test_rms_norm_against_fp64():
+    rng = np.random.default_rng(6)
+    for k in (32, 4096, 14336):
+        x = (rng.standard_normal((4, k)) * rng.uniform(0.01, 30)).astype(np.float32)
+        g = rng.standard_normal(k).astype(np.float32)
+        x64 = x.astype(np.float64)
+        want = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + 1e-5) * g
+        got = oracle.rms_norm(x, g, 1e-5)
+        assert np.max(np.abs(got - want) / (np.abs(want) + 1e-30)) < 1e-6
+        # a dropped eps, a sum instead of a mean, or a missing square root would all miss by far more
+        assert np.allclose(np.sqrt((oracle.rms_norm(x, None, 0.0).astype(np.float64) ** 2).mean(axis=1)), 1.0, atol=1e-6)
+
+
+def test_swiglu_identities_and_fp64():
+    """silu(0) = 0, silu(v) - silu(-v) = v, silu(v) -> v for large v and -> 0 for very negative v;
+    against an fp64 evaluation"""
+    v = np.array([0.0, 1.0, -1.0, 0.5, 20.0, -20.0, 88.0, -88.0, 100.0, -100.0], np.float32)
+    one = np.ones_like(v)
+    s = oracle.swiglu(v, one)
+    assert s[0] == 0 and s[8] == 100.0 and s[9] == 0.0 and abs(s[4] - 20.0) < 1e-6
+    rng = np.random.default_rng(7)
+    a = (rng.standard_normal(20000) * 4).astype(np.float32)
+    u = rng.standard_normal(20000).astype(np.float32)
+    ones = np.ones_like(a)
+    assert np.allclose(oracle.swiglu(a, ones) - oracle.swiglu(-a, ones), a, rtol=0, atol=2e-6)
+    want = a.astype(np.float64) / (1 + np.exp(-a.astype(np.float64))) * u
+    got = oracle.swiglu(a, u)
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-30)) < 1e-6
+    assert np.array_equal(oracle.swiglu(a, 2 * u), 2 * oracle.swiglu(a, u))  # linear in up (exact: power of two)
