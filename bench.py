@@ -20,6 +20,7 @@ The same JSON line carries
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -281,6 +282,33 @@ def main() -> int:
             other[f"MulmatID Q4_K 128x(768x2048) top-8 tokens={toks}"] = {"us": round(tm * 1e6, 2)}
         for st in stacks:
             st.free()
+        # decode feed-forward block with its producers, on the main pool: RMSNorm -> gate, up (one launch) and
+        # SILU(gate) * up -> down (one launch), against the same block through the stand-alone f32 kernels
+        gnorm = torch.randn(FFN_K, generator=g, dtype=torch.float32).to(dev)
+        xn = torch.empty(1, FFN_K, dtype=torch.float32, device=dev)
+        act = torch.empty(1, FFN_M, dtype=torch.float32, device=dev)
+        vp = ctypes.c_void_p
+
+        def block_fused():
+            for ent in pool:
+                ctx.mulmat_produced_device([ent["gate"], ent["up"]], qmm.PRODUCE_RMSNORM, gnorm.data_ptr(), x.data_ptr(), 1,
+                                           [y_gate.data_ptr(), y_up.data_ptr()], eps=1e-5)
+                ctx.mulmat_produced_device([ent["down"]], qmm.PRODUCE_SWIGLU, y_up.data_ptr(), y_gate.data_ptr(), 1,
+                                           [y_down.data_ptr()])
+
+        def block_unfused():
+            L = qmm.lib()
+            for ent in pool:
+                qmm._check(L.mi_qmm_rms_norm(ctx._h, vp(x.data_ptr()), vp(gnorm.data_ptr()), 1e-5, FFN_K, 1, vp(xn.data_ptr()), qmm.DEVICE))
+                ctx.mulmat_multi_device([ent["gate"], ent["up"]], xn.data_ptr(), 1, [y_gate.data_ptr(), y_up.data_ptr()])
+                qmm._check(L.mi_qmm_swiglu(ctx._h, vp(y_gate.data_ptr()), vp(y_up.data_ptr()), FFN_M, 1, vp(act.data_ptr()), qmm.DEVICE))
+                ctx.mulmat_device(ent["down"], act.data_ptr(), 1, y_down.data_ptr())
+
+        for label, fn in (("RMSNorm and SwiGLU inside the two product launches", block_fused),
+                          ("rms_norm, gate+up, swiglu, down: four launches", block_unfused)):
+            fn()
+            tm = timed(fn, 5) / (5 * len(pool))
+            other[f"decode FFN block, {label}"] = {"us": round(tm * 1e6, 2)}
         out["other_configs"] = other
 
     if args.calibrate_copy:

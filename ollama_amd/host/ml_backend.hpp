@@ -3,14 +3,18 @@
 //   ml.Backend  /root/reference/ml/backend.go:16-33    Load / Get(name) / NewContext / Close
 //   ml.Context  /root/reference/ml/backend.go:94-128   FromFloats / Compute / Close
 //   ml.Tensor   /root/reference/ml/backend.go:130-153  Dim / Shape / Floats / Mulmat / MulmatFullPrec / MulmatID
+//               /root/reference/ml/backend.go:159, :180 RMSNorm(ctx, weight, eps) / SILU(ctx, up)
 // Same names, same argument meaning (ggml shapes: dimension 0 contiguous, W = [K, M], x = [K, N],
 // W.Mulmat(ctx, x) = [M, N]) and the same error behaviour: tensor ops have no error return, so a
 // failure throws (the Go interface panics).  Mulmat is lazy; Compute runs the pending nodes, sharing
-// one activation quantization between all nodes that read the same x.
+// one activation quantization between all nodes that read the same x.  An RMSNorm or SILU(up) node that only
+// products read is never materialized: it runs inside those products' quantization.
 #pragma once
 
 #include <cstdint>
+#include <cstring>
 #include <map>
+#include <set>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -32,7 +36,7 @@ inline void check(int rc) {
 
 class Context;
 
-class Tensor {
+class Tensor : public std::enable_shared_from_this<Tensor> {
 public:
     int Dim(int n) const { return n < (int)shape_.size() ? (int)shape_[n] : 1; }
     const std::vector<int64_t> &Shape() const { return shape_; }
@@ -49,6 +53,10 @@ public:
     // [M, n_used, T]: slot i of token t goes through expert ids[i, t] with activation row i mod B
     std::shared_ptr<Tensor> MulmatID(Context &ctx, const std::shared_ptr<Tensor> &t2, const std::shared_ptr<Tensor> &ids);
     const std::vector<int32_t> &Ints() const { return ints_; }
+    // self = x [K, ...] f32, weight = [K] f32 or null -> lazy (x / sqrt(mean(x^2) + eps)) * weight along dimension 0
+    std::shared_ptr<Tensor> RMSNorm(Context &ctx, const std::shared_ptr<Tensor> &weight, float eps);
+    // self = gate, up: f32 of one shape -> lazy silu(gate) * up (ggml's swiglu)
+    std::shared_ptr<Tensor> SILU(Context &ctx, const std::shared_ptr<Tensor> &up);
 
     ~Tensor() { mi_qmm_weight_free(weight_); }
 
@@ -65,6 +73,10 @@ private:
     std::shared_ptr<Tensor> op_x_;       // pending Mulmat: activations
     std::shared_ptr<Tensor> op_ids_;     // pending MulmatID: expert ids
     std::shared_ptr<Tensor> self_keep_;  // keeps the weight alive while a node refers to it
+    int prod_ = MI_QMM_PRODUCE_NONE;     // pending RMSNorm / SILU(up): the producer,
+    std::shared_ptr<Tensor> prod_src_;   //   its input,
+    std::shared_ptr<Tensor> prod_aux_;   //   the norm weight (may be null) or up,
+    float prod_eps_ = 0.f;               //   and eps
 };
 
 class Backend {
@@ -77,6 +89,15 @@ public:
     // One GGUF tensor: type id, shape [K, M], M rows of K elements in GGUF block layout (what fs/ggml
     // hands out, /root/reference/fs/ggml/gguf.go:281-308).  The bytes are copied to the device.
     void Load(const std::string &name, int ggml_type, int64_t k, int64_t m, const void *gguf_bytes) {
+        if (ggml_type == MI_QMM_TYPE_F32 && m == 1) {  // a norm weight, the operand of RMSNorm: stays on the host
+            auto t = std::make_shared<Tensor>();
+            t->shape_ = {k};
+            t->data_.resize((size_t)k);
+            std::memcpy(t->data_.data(), gguf_bytes, (size_t)k * sizeof(float));
+            t->ready_ = true;
+            tensors_[name] = t;
+            return;
+        }
         auto t = std::make_shared<Tensor>();
         t->shape_ = {k, m};
         t->type_ = ggml_type;
@@ -159,57 +180,102 @@ public:
         t->ready_ = true;
         return t;
     }
-    // Run every pending Mulmat node.  Nodes that read the same x are handled together: decode-sized
-    // ones (n <= 8) go out four weights at a time through the entry point that quantizes x inside the
-    // GEMV launch; larger ones share one quantization of x.
-    void Compute() {
-        std::map<std::pair<Tensor *, int>, std::vector<Tensor *>> by_x;
-        // expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
-        std::map<std::pair<std::pair<Tensor *, Tensor *>, int>, std::vector<Tensor *>> by_xi;
+    // Run the pending nodes in the order they were recorded.  Mulmat nodes that read the same x are handled
+    // together: decode-sized ones (n <= 8) go out four weights at a time through the entry point that
+    // quantizes x inside the GEMV launch; larger ones share one quantization of x.  Producer nodes (RMSNorm,
+    // SILU) are materialized only when listed in `wanted` or read by something other than a Mulmat;
+    // otherwise they run inside the quantization of the products that read them.
+    void Compute(const std::vector<std::shared_ptr<Tensor>> &wanted = {}) {
+        std::set<const Tensor *> needed;
+        for (auto &t : wanted) needed.insert(t.get());
         for (auto &n : nodes_) {
             if (n->ready_) continue;
-            if (!n->op_ids_) by_x[{n->op_x_.get(), n->op_w_->type_}].push_back(n.get());
-            else by_xi[{{n->op_x_.get(), n->op_ids_.get()}, n->op_w_->Dim(2)}].push_back(n.get());
+            if (n->prod_) {
+                needed.insert(n->prod_src_.get());
+                if (n->prod_aux_) needed.insert(n->prod_aux_.get());
+            } else if (n->op_ids_) {
+                needed.insert(n->op_x_.get());
+            }
         }
-        for (auto &kv : by_xi) {
-            const Tensor &x = *kv.first.first.first, &ids = *kv.first.first.second;
+        for (auto &node : nodes_) {
+            Tensor *t = node.get();
+            if (t->ready_) continue;
+            if (t->prod_) {
+                if (!needed.count(t)) continue;
+                const Tensor &src = *t->prod_src_;
+                const int64_t k = src.Dim(0), n = (int64_t)src.Floats().size() / k;
+                t->data_.assign(src.data_.size(), 0.f);
+                if (t->prod_ == MI_QMM_PRODUCE_RMSNORM)
+                    check(mi_qmm_rms_norm(b_.handle(), src.data_.data(), t->prod_aux_ ? t->prod_aux_->Floats().data() : nullptr,
+                                          t->prod_eps_, k, n, t->data_.data(), MI_QMM_HOST));
+                else
+                    check(mi_qmm_swiglu(b_.handle(), src.data_.data(), t->prod_aux_->Floats().data(), k, n, t->data_.data(),
+                                        MI_QMM_HOST));
+                t->ready_ = true;
+                continue;
+            }
+            Tensor *x = t->op_x_.get();
+            std::vector<Tensor *> group;  // the pending nodes that go out with t
             std::vector<const mi_qmm_weight *> ws;
             std::vector<float *> ys;
-            for (Tensor *t : kv.second) {
-                t->data_.assign((size_t)(t->op_w_->Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);
-                ws.push_back(t->op_w_->weight_);
-                ys.push_back(t->data_.data());
+            if (t->op_ids_) {
+                // expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
+                const Tensor &ids = *t->op_ids_;
+                for (auto &u : nodes_)
+                    if (!u->ready_ && u->op_ids_ == t->op_ids_ && u->op_x_.get() == x && u->op_w_->Dim(2) == t->op_w_->Dim(2))
+                        group.push_back(u.get());
+                for (Tensor *u : group) {
+                    u->data_.assign((size_t)(u->op_w_->Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);
+                    ws.push_back(u->op_w_->weight_);
+                    ys.push_back(u->data_.data());
+                }
+                check(mi_qmm_mulmat_id_multi(b_.handle(), ws.data(), (int)ws.size(), t->op_w_->Dim(2), x->Floats().data(),
+                                             x->Dim(1), ids.ints_.data(), ids.Dim(0), ids.Dim(1), ys.data(), MI_QMM_HOST));
+                for (Tensor *u : group) u->ready_ = true;
+                continue;
             }
-            check(mi_qmm_mulmat_id_multi(b_.handle(), ws.data(), (int)ws.size(), kv.first.second, x.data_.data(), x.Dim(1),
-                                         ids.ints_.data(), ids.Dim(0), ids.Dim(1), ys.data(), MI_QMM_HOST));
-            for (Tensor *t : kv.second) t->ready_ = true;
-        }
-        for (auto &kv : by_x) {
-            Tensor *x = kv.first.first;
-            const int64_t k = x->Dim(0), n = (int64_t)x->data_.size() / k;
-            for (Tensor *t : kv.second) t->data_.assign((size_t)(n * t->Dim(0)), 0.f);
-            if (n <= 8) {
-                for (size_t i = 0; i < kv.second.size(); i += 4) {
-                    const mi_qmm_weight *ws[4];
-                    float *ys[4];
+            const bool fused = !x->ready_ && x->prod_;  // a producer nobody needs in f32
+            const Tensor &src = fused ? *x->prod_src_ : *x;
+            const int64_t k = src.Dim(0), n = (int64_t)src.Floats().size() / k;
+            for (auto &u : nodes_)
+                if (!u->ready_ && !u->prod_ && !u->op_ids_ && u->op_x_.get() == x &&
+                    (fused || n > 8 || u->op_w_->type_ == t->op_w_->type_))  // decode launches hold one weight type
+                    group.push_back(u.get());
+            for (Tensor *u : group) u->data_.assign((size_t)(n * u->Dim(0)), 0.f);
+            if (fused) {
+                for (Tensor *u : group) { ws.push_back(u->op_w_->weight_); ys.push_back(u->data_.data()); }
+                check(mi_qmm_mulmat_produced(b_.handle(), ws.data(), (int)ws.size(), x->prod_,
+                                             x->prod_aux_ ? x->prod_aux_->Floats().data() : nullptr, x->prod_eps_,
+                                             src.data_.data(), n, ys.data(), MI_QMM_HOST));
+            } else if (n <= 8) {
+                for (size_t i = 0; i < group.size(); i += 4) {
+                    const mi_qmm_weight *w4[4];
+                    float *y4[4];
                     int cnt = 0;
-                    for (size_t j = i; j < kv.second.size() && j < i + 4; j++, cnt++) {
-                        ws[cnt] = kv.second[j]->op_w_->weight_;
-                        ys[cnt] = kv.second[j]->data_.data();
+                    for (size_t j = i; j < group.size() && j < i + 4; j++, cnt++) {
+                        w4[cnt] = group[j]->op_w_->weight_;
+                        y4[cnt] = group[j]->data_.data();
                     }
-                    check(mi_qmm_mulmat_multi(b_.handle(), ws, cnt, x->data_.data(), n, ys, MI_QMM_HOST));
+                    check(mi_qmm_mulmat_multi(b_.handle(), w4, cnt, x->data_.data(), n, y4, MI_QMM_HOST));
                 }
             } else {
-                mi_qmm_act *act = nullptr;
-                check(mi_qmm_act_create(b_.handle(), mi_qmm_vec_dot_type(kv.first.second), k, n, &act));
-                int rc = mi_qmm_act_quantize(b_.handle(), act, x->data_.data(), n, MI_QMM_HOST);
-                for (size_t i = 0; rc == MI_QMM_OK && i < kv.second.size(); i++)
-                    rc = mi_qmm_mulmat_q8(b_.handle(), kv.second[i]->op_w_->weight_, act, kv.second[i]->data_.data(),
-                                          MI_QMM_HOST, MI_QMM_PATH_AUTO);
-                mi_qmm_act_free(act);
-                check(rc);
+                // one quantization of x per activation format in use
+                for (int q8 : {MI_QMM_TYPE_Q8_0, MI_QMM_TYPE_Q8_K}) {
+                    std::vector<Tensor *> part;
+                    for (Tensor *u : group)
+                        if (mi_qmm_vec_dot_type(u->op_w_->type_) == q8) part.push_back(u);
+                    if (part.empty()) continue;
+                    mi_qmm_act *act = nullptr;
+                    check(mi_qmm_act_create(b_.handle(), q8, k, n, &act));
+                    int rc = mi_qmm_act_quantize(b_.handle(), act, x->data_.data(), n, MI_QMM_HOST);
+                    for (size_t i = 0; rc == MI_QMM_OK && i < part.size(); i++)
+                        rc = mi_qmm_mulmat_q8(b_.handle(), part[i]->op_w_->weight_, act, part[i]->data_.data(), MI_QMM_HOST,
+                                              MI_QMM_PATH_AUTO);
+                    mi_qmm_act_free(act);
+                    check(rc);
+                }
             }
-            for (Tensor *t : kv.second) t->ready_ = true;
+            for (Tensor *u : group) u->ready_ = true;
         }
     }
     void Close() { nodes_.clear(); }
@@ -250,6 +316,34 @@ inline std::shared_ptr<Tensor> Tensor::MulmatID(Context &ctx, const std::shared_
     out->op_w_ = this;
     out->op_x_ = t2;
     out->op_ids_ = ids;
+    ctx.nodes_.push_back(out);
+    return out;
+}
+
+inline std::shared_ptr<Tensor> Tensor::RMSNorm(Context &ctx, const std::shared_ptr<Tensor> &weight, float eps) {
+    if (type_ != MI_QMM_TYPE_F32 || weight_ || (weight && (weight->type_ != MI_QMM_TYPE_F32 || weight->weight_)))
+        throw Error(MI_QMM_ERR_INVALID, "RMSNorm: operands must be f32");
+    if (weight && (!weight->ready_ || (int64_t)weight->data_.size() != Dim(0)))
+        throw Error(MI_QMM_ERR_INVALID, "RMSNorm: the weight must hold one value per element of dimension 0");
+    auto out = std::make_shared<Tensor>();
+    out->shape_ = shape_;
+    out->prod_ = MI_QMM_PRODUCE_RMSNORM;
+    out->prod_src_ = shared_from_this();
+    out->prod_aux_ = weight;
+    out->prod_eps_ = eps;
+    ctx.nodes_.push_back(out);
+    return out;
+}
+
+inline std::shared_ptr<Tensor> Tensor::SILU(Context &ctx, const std::shared_ptr<Tensor> &up) {
+    if (!up) throw Error(MI_QMM_ERR_INVALID, "SILU: this path implements the gated form SILU(ctx, up) only");
+    if (type_ != MI_QMM_TYPE_F32 || weight_ || up->type_ != MI_QMM_TYPE_F32 || up->weight_ || shape_ != up->shape_)
+        throw Error(MI_QMM_ERR_INVALID, "SILU: gate and up must be f32 of one shape");
+    auto out = std::make_shared<Tensor>();
+    out->shape_ = shape_;
+    out->prod_ = MI_QMM_PRODUCE_SWIGLU;
+    out->prod_src_ = shared_from_this();
+    out->prod_aux_ = up;
     ctx.nodes_.push_back(out);
     return out;
 }

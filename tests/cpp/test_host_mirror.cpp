@@ -154,6 +154,64 @@ int main() {
             } catch (const Error &) { threw_id = true; }
             if (!threw_id) { printf("FAIL: an expert id outside the stack did not throw\n"); failures++; }
         }
+        // feed-forward block with its producers: x -> RMSNorm -> gate, up -> SILU(gate, up) -> down
+        {
+            const int64_t k = 1024, f = 768;
+            struct M { const char *name; int type; int64_t kk, m; };
+            const M mats[] = {{"blk.1.ffn_gate.weight", MI_QMM_TYPE_Q4_K, k, f}, {"blk.1.ffn_up.weight", MI_QMM_TYPE_Q4_K, k, f},
+                              {"blk.1.ffn_down.weight", MI_QMM_TYPE_Q6_K, f, k}};
+            std::vector<std::vector<uint8_t>> fr;
+            for (const M &m : mats) {
+                auto wf = randn((size_t)(m.kk * m.m), 0.05f, 300 + (unsigned)fr.size());
+                std::vector<uint8_t> raw((size_t)(ref_row_size(m.type, m.kk) * m.m));
+                if (ref_quantize(m.type, wf.data(), raw.data(), m.kk, m.m, 4) != 0) return 1;
+                backend.Load(m.name, m.type, m.kk, m.m, raw.data());
+                fr.push_back(std::move(raw));
+            }
+            auto g = randn((size_t)k, 0.1f, 55);
+            for (auto &v : g) v += 1.0f;
+            backend.Load("blk.1.ffn_norm.weight", MI_QMM_TYPE_F32, k, 1, g.data());
+            for (int64_t n : {1, 5, 40}) {
+                auto xv = randn((size_t)(k * n), 1.0f, 500 + (unsigned)n);
+                std::vector<float> outs[2];
+                for (int pass = 0; pass < 2; pass++) {  // 0: producers fused into the products; 1: materialized
+                    auto ctx = backend.NewContext();
+                    auto x = ctx->FromFloats(xv, {k, n});
+                    auto h = x->RMSNorm(*ctx, backend.Get("blk.1.ffn_norm.weight"), 1e-5f);
+                    auto gate = backend.Get("blk.1.ffn_gate.weight")->Mulmat(*ctx, h);
+                    auto up = backend.Get("blk.1.ffn_up.weight")->Mulmat(*ctx, h);
+                    auto act = gate->SILU(*ctx, up);
+                    auto out = backend.Get("blk.1.ffn_down.weight")->Mulmat(*ctx, act);
+                    if (pass == 0) ctx->Compute(); else ctx->Compute({h, act});
+                    bool lazy = false;
+                    try { h->Floats(); } catch (const Error &) { lazy = true; }
+                    if (lazy != (pass == 0)) { printf("FAIL: RMSNorm node materialized=%d in pass %d\n", !lazy, pass); failures++; }
+                    outs[pass] = out->Floats();
+                    if (pass == 0) {
+                        std::vector<float> hv(xv.size()), gv((size_t)(f * n)), uv((size_t)(f * n)), av((size_t)(f * n)), ref((size_t)(k * n));
+                        ref_rms_norm(xv.data(), g.data(), 1e-5f, k, n, hv.data());
+                        ref_mul_mat(MI_QMM_TYPE_Q4_K, fr[0].data(), k, f, hv.data(), n, gv.data(), nullptr, 4);
+                        ref_mul_mat(MI_QMM_TYPE_Q4_K, fr[1].data(), k, f, hv.data(), n, uv.data(), nullptr, 4);
+                        const double eg = rel_err(gate->Floats(), gv);
+                        // the last step alone: the oracle on the GPU's own gate / up values
+                        ref_swiglu(gate->Floats().data(), up->Floats().data(), f * n, av.data());
+                        ref_mul_mat(MI_QMM_TYPE_Q6_K, fr[2].data(), f, k, av.data(), n, ref.data(), nullptr, 4);
+                        const double e = rel_err(out->Floats(), ref);
+                        printf("%-24s N=%-3lld rel err gate %.2e down %.2e %s\n", "ffn block, fused producers", (long long)n, eg, e,
+                               (eg <= 1e-3 && e <= 1e-3) ? "ok" : "FAIL");
+                        if (!(eg <= 1e-3) || !(e <= 1e-3)) failures++;
+                    }
+                    ctx->Close();
+                }
+                if (outs[0] != outs[1]) { printf("FAIL: fused and materialized producers differ at N=%lld\n", (long long)n); failures++; }
+            }
+            bool threw_silu = false;
+            try {
+                auto ctx = backend.NewContext();
+                ctx->FromFloats(std::vector<float>(k), {k, 1})->SILU(*ctx, nullptr);
+            } catch (const Error &) { threw_silu = true; }
+            if (!threw_silu) { printf("FAIL: SILU without up did not throw\n"); failures++; }
+        }
         backend.Close();
         printf(failures ? "host mirror: %d FAILURES\n" : "host mirror: all ok\n", failures);
         return failures ? 1 : 0;

@@ -18,7 +18,9 @@ def _model_file(tmp_path):
         raw = synth.weights(t, m, k, seed=m).reshape(-1)
         raws[name] = (t, m, raw)
         tensors.append((name, t, [k, m], raw.tobytes()))
-    tensors.append(("blk.0.attn_norm.weight", 0, [k], np.ones(k, np.float32).tobytes()))   # f32, 1-D: not on the path
+    norm = (1 + 0.05 * np.random.default_rng(9).standard_normal(k)).astype(np.float32)
+    tensors.append(("blk.0.attn_norm.weight", 0, [k], norm.tobytes()))   # f32, 1-D: the operand of RMSNorm, kept on the host
+    tensors.append(("token_embd.weight", 0, [k, 4], np.zeros((4, k), np.float32).tobytes()))  # f32, 2-D: not on the path
     p = str(tmp_path / "model.gguf")
     gguf.write_gguf(p, {"general.architecture": "llama", "block_count": np.uint32(1)}, tensors)
     return p, k, raws
@@ -48,12 +50,18 @@ def test_backend_from_gguf_path(tmp_path):
     b = ml.Backend(p)
     b.Load(progress=seen.append)
     assert seen and seen[-1] == 1.0
-    assert b.Get("blk.0.attn_norm.weight") is None and b.Get("nope") is None
+    assert b.Get("token_embd.weight") is None and b.Get("nope") is None
+    norm = b.Get("blk.0.attn_norm.weight")
+    assert norm.Shape() == [k] and norm.DType() == ml.DType.F32 and abs(norm.Floats().mean() - 1) < 0.05
     ctx = b.NewContext()
     xs = np.random.default_rng(4).standard_normal((2, k), dtype=np.float32)
     x = ctx.FromFloats(xs.reshape(-1), k, 2)
     outs = {name: b.Get(name).Mulmat(ctx, x) for name in raws}
-    ctx.Compute(*outs.values())
+    normed = b.Get("blk.0.attn_q.weight").Mulmat(ctx, x.RMSNorm(ctx, norm, 1e-5))   # the file's norm in front of q
+    ctx.Compute(normed, *outs.values())
+    t, m, raw = raws["blk.0.attn_q.weight"]
+    want = oracle.mul_mat(t, raw, k, m, oracle.rms_norm(xs, norm.Floats(), 1e-5), nthreads=4)
+    assert npref.rel_err(normed.Floats().reshape(2, m), want) <= TOL
     for name, (t, m, raw) in raws.items():
         assert outs[name].Shape() == [m, 2]
         want = oracle.mul_mat(t, raw, k, m, xs, nthreads=4)
