@@ -288,6 +288,40 @@ def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
             W.free()
 
 
+@pytest.mark.parametrize("t,k", [(Q4_K, 14336), (Q4_K, 8192), (Q6_K, 4352), (Q4_0, 4096), (Q8_0, 4096), (Q8_0, 2080)])
+def test_long_rows_at_one_column(ctx, t, k):
+    """One column, rows of several K segments (the waves of a workgroup cut K and combine through LDS): same
+    bits as the two-phase path, call after call; row counts that do not fill the last workgroup, four
+    weights in one launch, and the largest launch the f32 path takes (64 Ki rows)."""
+    rng = np.random.default_rng(900 + t + k)
+    ms = [1, 31, 32, 33, 700]
+    raws = [_weights(t, m, k, seed=k + m + t) for m in ms]
+    Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+    act = ctx.act_create(qmm.vec_dot_type(t), k, 1)
+    for rep in range(3):
+        x = rng.standard_normal((1, k), dtype=np.float32)
+        ctx.act_quantize(act, x)
+        want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV) for W in Ws]
+        for _ in range(3):
+            for W, wnt in zip(Ws, want):
+                assert np.array_equal(ctx.mulmat(W, x), wnt)
+            for y, wnt in zip(ctx.mulmat_multi(Ws[1:], x), want[1:]):
+                assert np.array_equal(y, wnt)
+        assert npref.rel_err(want[4], oracle.mul_mat(t, raws[4], k, 700, x, nthreads=8)) <= TOL
+    act.free()
+    for W in Ws:
+        W.free()
+    if t == Q4_K and k == 8192:
+        m = 65536
+        raw = np.tile(_weights(t, 1024, k, seed=77).reshape(1024, -1), (m // 1024, 1)).reshape(-1)
+        W = ctx.upload(t, raw, k, m)
+        x = rng.standard_normal((1, k), dtype=np.float32)
+        y = ctx.mulmat(W, x)
+        assert np.array_equal(y[0, :1024], y[0, -1024:])                       # the rows repeat
+        assert npref.rel_err(y[:, :1024], oracle.mul_mat(t, raw[: 1024 * qmm.row_size(t, k)], k, 1024, x, nthreads=8)) <= TOL
+        W.free()
+
+
 def test_results_do_not_depend_on_rows_per_wave(ctx):
     """A wave parks the totals of its rows in different lanes; every lane of the last 16 holds the wave
     total, but summed in a lane-dependent order.  The kernel must take one fixed lane's value, so that
