@@ -392,6 +392,31 @@ def test_randomized_shape_sweep(ctx):
         W.free()
 
 
+def test_randomized_mulmat_id_sweep(ctx):
+    """random types, expert counts, token counts, slots and activation rows per token across the decode, bucketed,
+    matrix-core and expert-GEMM paths, against the oracle"""
+    rng = np.random.default_rng(777)
+    for case in range(36):
+        t = int(rng.choice(WTYPES))
+        blk = npref.BLOCK[t]
+        k = int(rng.integers(1, 10 if blk == 256 else 60)) * blk
+        m = int(rng.integers(1, 150))
+        n_expert = int(rng.choice([1, 2, 5, 8, 16, 40]))
+        n_used = int(rng.integers(1, min(n_expert, 8) + 1))
+        tokens = int(rng.choice([1, 1, 2, 7, 20, 64, 150, 400]))
+        b_cols = int(rng.choice([1, n_used]))
+        wb = _weights(t, n_expert * m, k, seed=3000 + case)
+        w = ctx.upload(t, wb, k, n_expert * m)
+        b = rng.standard_normal((tokens, b_cols, k), dtype=np.float32)
+        ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+        got = ctx.mulmat_id(w, n_expert, b, ids)
+        want = oracle.mul_mat_id(t, wb, k, m, n_expert, b, ids)
+        err = npref.rel_err(got, want)
+        assert got.shape == (tokens, n_used, m) and err <= TOL, \
+            f"case {case}: {NAMES[t]} k={k} m={m} E={n_expert} used={n_used} tokens={tokens} b_cols={b_cols}: {err}"
+        w.free()
+
+
 # ---- kernel 3: int8-MFMA GEMM ---------------------------------------------------------------------
 @pytest.mark.parametrize("t", [Q4_K, Q6_K])
 @pytest.mark.parametrize("k,m,n", [(256, 1, 1), (256, 32, 32), (512, 31, 33), (1024, 128, 128), (1024, 257, 200),

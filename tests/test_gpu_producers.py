@@ -178,3 +178,34 @@ def test_produced_errors(ctx):
     assert ctx.mulmat_produced([w], qmm.PRODUCE_NONE, None, x)[0].shape == (1, 8)
     assert ctx.mulmat_produced([w], qmm.PRODUCE_RMSNORM, None, np.zeros((0, k), np.float32))[0].shape == (0, 8)
     w.free()
+
+
+def test_randomized_produced_sweep(ctx):
+    """random types, shapes, batch sizes, producers and weight counts against the oracle chain and the
+    library's own two-step path"""
+    rng = np.random.default_rng(20250)
+    for case in range(40):
+        t = int(rng.choice(WTYPES))
+        blk = 256 if t in (Q4_K, Q6_K) else 32
+        k = int(rng.integers(1, 24 if blk == 256 else 150)) * blk
+        if case % 6 == 2:
+            k = int(rng.integers(17, 60)) * 256
+        n = int(rng.choice([1, 1, 1, 2, 3, 5, 8, 9, 33, 70]))
+        ms = [int(rng.integers(1, 300)) for _ in range(int(rng.integers(1, 4)))]
+        producer = int(rng.choice([qmm.PRODUCE_RMSNORM, qmm.PRODUCE_SWIGLU]))
+        wbs = [_weights(t, m, k, 5000 + case + i) for i, m in enumerate(ms)]
+        ws = [ctx.upload(t, wb, k, m) for wb, m in zip(wbs, ms)]
+        x = (rng.standard_normal((n, k)) * float(rng.choice([1e-2, 1.0, 20.0]))).astype(np.float32)
+        if producer == qmm.PRODUCE_RMSNORM:
+            aux = rng.standard_normal(k).astype(np.float32) if case % 3 else None
+        else:
+            aux = rng.standard_normal((n, k)).astype(np.float32)
+        eps = float(rng.choice([1e-5, 1e-6]))
+        got = ctx.mulmat_produced(ws, producer, aux, x, eps=eps)
+        two = _two_step(ctx, ws, producer, aux, x, eps)
+        for y, y2, wb, m in zip(got, two, wbs, ms):
+            err = npref.rel_err(y, _chain(t, wb, k, m, producer, aux, x, eps))
+            assert y.shape == (n, m) and err < TOL, f"case {case}: type {t} k={k} m={m} n={n} producer {producer}: {err}"
+            assert np.array_equal(y, y2), f"case {case}: type {t} k={k} m={m} n={n} producer {producer}"
+        for w in ws:
+            w.free()
