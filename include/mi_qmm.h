@@ -188,6 +188,15 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
 int mi_qmm_mulmat_id_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int n_expert,
                            const float *x, int b_cols, const int32_t *ids, int n_used, int64_t n_tokens,
                            float *const *ys, int location);
+/* mi_qmm_mulmat_id on x' = producer(x) (the producers of mi_qmm_mulmat_produced): the down projection of
+ * an expert feed-forward block reads silu(gate) * up, x = gate and aux = up being the two
+ * [n_tokens][b_cols][k] results of the gate / up stacks.  Decode-sized calls gate and quantize each
+ * pair's row in the prologue of its product (one launch); larger ones quantize x' once with the fused
+ * quantizer.  RMSNorm: aux = the norm weight [k] or NULL.  Bit-identical to mi_qmm_swiglu /
+ * mi_qmm_rms_norm followed by mi_qmm_mulmat_id. */
+int mi_qmm_mulmat_id_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, int producer,
+                              const float *aux, float eps, const float *x, int b_cols, const int32_t *ids,
+                              int n_used, int64_t n_tokens, float *y, int location);
 
 /* ---- two-phase form: quantize once, multiply by several weights (gate and up, or q/k/v, share
  *      one x).  In ggml's graph the from_float step belongs to each mul_mat node; a backend that

@@ -739,9 +739,14 @@ namespace {
 // w2 / y2 (optional): a second stack of w's type and shape multiplied by the same activations and ids;
 // x is quantized once for both and the decode launch covers both.
 int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight *w2, int n_expert, const float *x,
-                   int b_cols, const int32_t *ids, int n_used, int64_t n_tokens, float *y, float *y2, int location) {
+                   int b_cols, const int32_t *ids, int n_used, int64_t n_tokens, float *y, float *y2, int location,
+                   const Produce *prod = nullptr) {
     int rc = check_product_args(ctx, w, location, MI_QMM_PATH_AUTO);
     if (rc) return rc;
+    Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
+    if (prod) pr = *prod;
+    if (pr.kind == PRODUCE_SWIGLU && !pr.aux && n_tokens > 0) return fail(MI_QMM_ERR_INVALID, "SwiGLU needs the up operand");
+    if (pr.kind == PRODUCE_RMSNORM && !(pr.eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
     if (w2 && (w2->device != ctx->device || w2->dev.type != w->dev.type || w2->dev.K != w->dev.K || w2->dev.M != w->dev.M))
         return fail(MI_QMM_ERR_INVALID, "the two expert stacks differ in device, type or shape");
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
@@ -769,19 +774,27 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     const int tile_w = gemm_id_tile_width(w->dev.type, pairs, n_expert);
     const int64_t max_tiles = gemm ? sort_pairs_max_tiles(pairs, n_expert, tile_w) : 0, sorted_rows = tile_w * max_tiles;
     const ActPlanes probe = plan_act(nullptr, q8, K, ncols);
-    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total + align_up((size_t)ncols * 4, 256), ctx->stream))) return rc;
     const ActPlanes p = plan_act(ctx->act_buf, q8, K, ncols);
+    float *row_scales = (float *)((char *)ctx->act_buf + probe.total);  // RMSNorm: one scale per activation row
     const size_t hist_ints = gemm ? sort_pairs_hist_ints(pairs, n_expert) : 0;
     const size_t scratch_ints = gemm ? (size_t)(1 + 2 * max_tiles + 2 * sorted_rows) + hist_ints : gemv_id_scratch_ints(pairs);
     if ((rc = reserve(&ctx->ws_buf, &ctx->ws_cap, scratch_ints * sizeof(int), ctx->stream))) return rc;
 
     const size_t xbytes = (size_t)(ncols * K) * 4, ibytes = (size_t)pairs * 4, ybytes = (size_t)(pairs * M) * 4;
+    const size_t auxbytes = !pr.aux ? 0 : pr.kind == PRODUCE_SWIGLU ? xbytes : (size_t)K * 4;
     const float *dx = x;
     const int32_t *dids = ids;
     float *dy = y, *dy2 = y2;
     if (location == MI_QMM_HOST) {
         const size_t ioff = align_up(xbytes, 256), yoff = ioff + align_up(ibytes, 256), yoff2 = yoff + align_up(ybytes, 256);
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, yoff2 + (w2 ? ybytes : 0), ctx->stream))) return rc;
+        const size_t auxoff = yoff2 + align_up(w2 ? ybytes : 0, 256);
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, auxoff + auxbytes, ctx->stream))) return rc;
+        if (auxbytes) {
+            float *daux = (float *)((char *)ctx->io_buf + auxoff);
+            HIP_TRY(hipMemcpyAsync(daux, pr.aux, auxbytes, hipMemcpyHostToDevice, ctx->stream));
+            pr.aux = daux;
+        }
         dx = (const float *)ctx->io_buf;
         dids = (const int32_t *)((char *)ctx->io_buf + ioff);
         dy = (float *)((char *)ctx->io_buf + yoff);
@@ -789,11 +802,20 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
         HIP_TRY(hipMemcpyAsync((void *)dids, ids, ibytes, hipMemcpyHostToDevice, ctx->stream));
     }
+    // the quantization of x, through the producer if there is one
+    auto quantize = [&]() -> hipError_t {
+        if (pr.kind == PRODUCE_RMSNORM) {
+            if (hipError_t e = launch_rms_norm(dx, nullptr, pr.eps, K, ncols, row_scales, nullptr, ctx->stream)) return e;
+            pr.row_scale = row_scales;
+        }
+        return launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream,
+                                   pr.kind == PRODUCE_NONE ? nullptr : &pr);
+    };
     if (gemm) {
         int *tiles = (int *)ctx->ws_buf, *src_col = tiles + 1 + 2 * max_tiles, *out_pair = src_col + sorted_rows;
         HIP_TRY(launch_sort_pairs(dids, (int)pairs, n_expert, n_used, b_cols, tile_w, tiles, src_col, out_pair,
                                   hist_ints ? out_pair + sorted_rows : nullptr, ctx->stream));
-        HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+        HIP_TRY(quantize());
         DevAct as;
         as.qs = p.qs; as.d = p.d; as.bsums = p.bsums; as.sd8 = p.sd8; as.sd16 = p.sd16; as.K = K; as.N = (int)ncols; as.type = q8;
         HIP_TRY(launch_gemm_id(w->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, tile_w, dy, ctx->stream));
@@ -809,9 +831,10 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     a.K = K; a.N = (int)ncols; a.type = q8;
     // the matrix-core kernel addresses activation bytes with 32-bit offsets
     const bool skinny = skinny_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
-    const bool fused = !skinny && gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert);
+    const bool fused = !skinny && pr.kind != PRODUCE_RMSNORM &&
+                       gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert, pr.kind == PRODUCE_SWIGLU);
     if (!fused) {
-        HIP_TRY(launch_quantize_act(q8, dx, K, ncols, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+        HIP_TRY(quantize());
         a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16;
     }
     if (skinny) {
@@ -823,7 +846,8 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
                                      ctx->num_cus, ctx->stream));
     } else {
         HIP_TRY(launch_gemv_id(w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
-                               (int *)ctx->ws_buf, ctx->stream, w2 ? &w2->dev : nullptr, dy2));
+                               (int *)ctx->ws_buf, ctx->stream, w2 ? &w2->dev : nullptr, dy2,
+                               fused && pr.kind == PRODUCE_SWIGLU ? pr.aux : nullptr));
     }
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
@@ -857,6 +881,15 @@ int mi_qmm_mulmat_id_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         i += pair ? 2 : 1;
     }
     return MI_QMM_OK;
+}
+
+int mi_qmm_mulmat_id_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, int producer, const float *aux,
+                              float eps, const float *x, int b_cols, const int32_t *ids, int n_used, int64_t n_tokens,
+                              float *y, int location) {
+    if (producer != MI_QMM_PRODUCE_NONE && producer != MI_QMM_PRODUCE_RMSNORM && producer != MI_QMM_PRODUCE_SWIGLU)
+        return fail(MI_QMM_ERR_INVALID, "unknown producer %d", producer);
+    const Produce pr{producer, producer == MI_QMM_PRODUCE_NONE ? nullptr : aux, eps, nullptr};
+    return mulmat_id_impl(ctx, w, nullptr, n_expert, x, b_cols, ids, n_used, n_tokens, y, nullptr, location, &pr);
 }
 
 // ---- two-phase form ----------------------------------------------------------------------------------

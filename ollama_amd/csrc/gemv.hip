@@ -1259,9 +1259,13 @@ __global__ __launch_bounds__(1024) void sort_place_kernel(const int *__restrict_
     }
 }
 
-template <class P, int NC, bool DIRECT, bool F32, int RPL>
+// XMODE as in gemv_thin_kernel: 0 quantized planes, 1 f32 rows quantized here, 3 f32 rows through SwiGLU first
+// (up: the second operand, laid out like xf).
+template <class P, int NC, bool DIRECT, int XMODE, int RPL>
 __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const float *__restrict__ xf,
-                                                      int rows_per_wave, int kw, int rw_log2) {
+                                                      const float *__restrict__ up, int rows_per_wave, int kw, int rw_log2) {
+    constexpr bool F32 = XMODE != 0;
+    static_assert(XMODE == 0 || XMODE == 1 || XMODE == 3, "RMSNorm is not produced here");
     static_assert(!F32 || NC == 1, "the f32 prologue quantizes one activation row");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int REC = 2 + NC;
@@ -1321,10 +1325,15 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     int16_t *lbs = reinterpret_cast<int16_t *>(smem + K + (size_t)nblk * 4);
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col[0] * K);
     const int total4 = (int)(K / 4), nwaves = blockDim.x >> 6;
-    float4 xpre[XPRE];
+    float4 xpre[XPRE], apre[XPRE];
     if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
+    if (XMODE == 3) prefetch_x(reinterpret_cast<const float4 *>(up + (int64_t)col[0] * K), total4, wave, nwaves, lane, apre);
     typename P::Raw cur;
     if (nrw > 0) cur = P::load(w, g, wrow0 + min(run, nrw - 1));
+    if (XMODE == 3) {  // the whole row sits in the prefetch registers (the launcher checked)
+#pragma unroll
+        for (int j = 0; j < XPRE; j++) xpre[j] = swiglu_apply(xpre[j], apre[j]);
+    }
     if (F32) {
         quantize_x_to_lds<P, XPRE>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
         __syncthreads();
@@ -1358,11 +1367,12 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
 }
 
 template <class P, int NC>
-hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, int *groups, hipStream_t s) {
+hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, const float *up, int *groups, hipStream_t s) {
     Plan p;
     if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC, false, p)) return hipErrorInvalidValue;
     const size_t act_lds = xf ? thin_act_lds<P>(ia.w.K, 1) : 0;
     if (xf && (NC != 1 || act_lds + p.lds > THIN_LDS_MAX)) return hipErrorInvalidValue;
+    if (up && (!xf || ia.w.K > (int64_t)XPRE * p.kw * p.rw * 256)) return hipErrorInvalidValue;
     const int64_t wgs_per_group = (ia.M + p.rows_per_wg - 1) / p.rows_per_wg;
     int64_t max_groups = ia.pairs;
     if (NC > 1) {
@@ -1380,29 +1390,34 @@ hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, int *groups
     const dim3 grid((unsigned)(wgs_per_group * max_groups * stacks)), block(64 * p.kw * p.rw);
     const int rpw = p.rows_per_wg >> p.rw_log2;
     const size_t lds = act_lds + p.lds;
-#define ID_LAUNCH(N, DIRECT, F32, RPL) \
-    gemv_id_kernel<P, N, DIRECT, F32, RPL><<<grid, block, lds, s>>>(ia, a, xf, rpw, p.kw, p.rw_log2)
-    if (xf) {
-        if (p.kw > 1) ID_LAUNCH(1, false, true, 1);
-        else if (p.rpl == 4) ID_LAUNCH(1, true, true, 4);
-        else if (p.rpl == 2) ID_LAUNCH(1, true, true, 2);
-        else ID_LAUNCH(1, true, true, 1);
+#define ID_LAUNCH(N, DIRECT, XMODE, RPL) \
+    gemv_id_kernel<P, N, DIRECT, XMODE, RPL><<<grid, block, lds, s>>>(ia, a, xf, up, rpw, p.kw, p.rw_log2)
+    if (xf && up) {
+        if (p.kw > 1) ID_LAUNCH(1, false, 3, 1);
+        else if (p.rpl == 4) ID_LAUNCH(1, true, 3, 4);
+        else if (p.rpl == 2) ID_LAUNCH(1, true, 3, 2);
+        else ID_LAUNCH(1, true, 3, 1);
+    } else if (xf) {
+        if (p.kw > 1) ID_LAUNCH(1, false, 1, 1);
+        else if (p.rpl == 4) ID_LAUNCH(1, true, 1, 4);
+        else if (p.rpl == 2) ID_LAUNCH(1, true, 1, 2);
+        else ID_LAUNCH(1, true, 1, 1);
     } else {
-        if (p.kw > 1) ID_LAUNCH(NC, false, false, 1);
-        else if (p.rpl == 4) ID_LAUNCH(NC, true, false, 4);
-        else if (p.rpl == 2) ID_LAUNCH(NC, true, false, 2);
-        else ID_LAUNCH(NC, true, false, 1);
+        if (p.kw > 1) ID_LAUNCH(NC, false, 0, 1);
+        else if (p.rpl == 4) ID_LAUNCH(NC, true, 0, 4);
+        else if (p.rpl == 2) ID_LAUNCH(NC, true, 0, 2);
+        else ID_LAUNCH(NC, true, 0, 1);
     }
 #undef ID_LAUNCH
     return hipGetLastError();
 }
 
 template <class P>
-hipError_t launch_id_type(const IdArgs &ia, const DevAct &a, const float *xf, int *groups, hipStream_t s) {
+hipError_t launch_id_type(const IdArgs &ia, const DevAct &a, const float *xf, const float *up, int *groups, hipStream_t s) {
     // few pairs per expert (decode: the experts of a token are all different): nothing to share, one
     // pair per group; otherwise up to eight pairs of an expert per pass over it
-    if (xf || !gemv_id_groups(ia.pairs, ia.n_expert)) return launch_id_as<P, 1>(ia, a, xf, groups, s);
-    return launch_id_as<P, 8>(ia, a, xf, groups, s);
+    if (xf || !gemv_id_groups(ia.pairs, ia.n_expert)) return launch_id_as<P, 1>(ia, a, xf, up, groups, s);
+    return launch_id_as<P, 8>(ia, a, xf, nullptr, groups, s);
 }
 
 }  // namespace
@@ -1446,7 +1461,7 @@ hipError_t launch_sort_pairs(const int *ids, int pairs, int n_expert, int n_used
 
 bool gemv_id_groups(int64_t pairs, int n_expert) { return pairs >= 4 * (int64_t)n_expert; }
 
-bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_expert) {
+bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_expert, bool swiglu) {
     // every workgroup quantizes its pair's activation row again: worth it while the launch is small
     if (gemv_id_groups(pairs, n_expert) || pairs > 64 || K < 1 || K > gemv_max_k(type)) return false;
     Plan p;
@@ -1459,12 +1474,14 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
     case T_Q8_0: ok = make_thin_plan<PolQ8_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ8_0>(K, 1); break;
     default: break;
     }
+    // gated rows must sit in the waves' prefetch registers whole
+    if (ok && swiglu && K > (int64_t)XPRE * p.kw * p.rw * 256) return false;
     return ok && act + p.lds <= THIN_LDS_MAX;
 }
 
 hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,
                           int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s,
-                          const DevWeight *w2, float *y2) {
+                          const DevWeight *w2, float *y2, const float *up) {
     if ((w2 != nullptr) != (y2 != nullptr) || (w2 && (w2->type != w.type || w2->K != w.K || w2->M != w.M)))
         return hipErrorInvalidValue;
     if (n_expert < 1 || n_expert > ID_MAX_EXPERTS || w.M % n_expert || n_used < 1 || n_tokens < 1 || b_cols < 1 || !ids || !y || !groups || a.K != w.K || a.N != (int64_t)b_cols * n_tokens ||
@@ -1476,10 +1493,10 @@ hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, con
     ia.n_expert = n_expert; ia.pairs = n_used * n_tokens; ia.n_used = n_used; ia.b_cols = b_cols;
     if (w2) { ia.p0b = w2->p0; ia.p1b = w2->p1; ia.p2b = w2->p2; ia.db = w2->d; ia.yb = y2; }
     switch (w.type) {
-    case T_Q4_K: return a.type == T_Q8_K ? launch_id_type<PolQ4K>(ia, a, xf, groups, s) : hipErrorInvalidValue;
-    case T_Q6_K: return a.type == T_Q8_K ? launch_id_type<PolQ6K>(ia, a, xf, groups, s) : hipErrorInvalidValue;
-    case T_Q4_0: return a.type == T_Q8_0 ? launch_id_type<PolQ4_0>(ia, a, xf, groups, s) : hipErrorInvalidValue;
-    case T_Q8_0: return a.type == T_Q8_0 ? launch_id_type<PolQ8_0>(ia, a, xf, groups, s) : hipErrorInvalidValue;
+    case T_Q4_K: return a.type == T_Q8_K ? launch_id_type<PolQ4K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
+    case T_Q6_K: return a.type == T_Q8_K ? launch_id_type<PolQ6K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
+    case T_Q4_0: return a.type == T_Q8_0 ? launch_id_type<PolQ4_0>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
+    case T_Q8_0: return a.type == T_Q8_0 ? launch_id_type<PolQ8_0>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
 }

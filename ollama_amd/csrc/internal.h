@@ -54,12 +54,14 @@ int64_t gemv_max_k(int type);
 // and a only carries the geometry; ask gemv_id_f32_supported() first.
 size_t gemv_id_scratch_ints(int64_t pairs);
 bool gemv_id_groups(int64_t pairs, int n_expert);  // enough pairs per expert to bucket them by expert
-bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);
+bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_expert, bool swiglu = false);
 // w2 / y2 (optional): a second stack of the same type and shape against the same activations and ids,
 // in the same launch (gate and up of an expert FFN).
+// up (optional, with xf; ask gemv_id_f32_supported(..., true)): the rows are silu(xf) * up, produced in the
+// prologue (the down projection of an expert FFN).
 hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,
                           int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s,
-                          const DevWeight *w2 = nullptr, float *y2 = nullptr);
+                          const DevWeight *w2 = nullptr, float *y2 = nullptr, const float *up = nullptr);
 // buckets the pairs by expert into groups of at most nc (1..16) pairs: groups[0] = number of groups,
 // then records {expert or -1 for ids outside the stack, count, pair[nc]}
 hipError_t launch_group_pairs(const int *ids, int pairs, int n_expert, int nc, int *groups, hipStream_t s);

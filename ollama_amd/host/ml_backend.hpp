@@ -183,7 +183,7 @@ public:
     // Run the pending nodes in the order they were recorded.  Mulmat nodes that read the same x are handled
     // together: decode-sized ones (n <= 8) go out four weights at a time through the entry point that
     // quantizes x inside the GEMV launch; larger ones share one quantization of x.  Producer nodes (RMSNorm,
-    // SILU) are materialized only when listed in `wanted` or read by something other than a Mulmat;
+    // SILU) are materialized only when listed in `wanted` or read by something other than a product;
     // otherwise they run inside the quantization of the products that read them.
     void Compute(const std::vector<std::shared_ptr<Tensor>> &wanted = {}) {
         std::set<const Tensor *> needed;
@@ -193,8 +193,6 @@ public:
             if (n->prod_) {
                 needed.insert(n->prod_src_.get());
                 if (n->prod_aux_) needed.insert(n->prod_aux_.get());
-            } else if (n->op_ids_) {
-                needed.insert(n->op_x_.get());
             }
         }
         for (auto &node : nodes_) {
@@ -229,8 +227,17 @@ public:
                     ws.push_back(u->op_w_->weight_);
                     ys.push_back(u->data_.data());
                 }
-                check(mi_qmm_mulmat_id_multi(b_.handle(), ws.data(), (int)ws.size(), t->op_w_->Dim(2), x->Floats().data(),
-                                             x->Dim(1), ids.ints_.data(), ids.Dim(0), ids.Dim(1), ys.data(), MI_QMM_HOST));
+                if (!x->ready_ && x->prod_) {
+                    // x is a producer nobody needs in f32 (silu(gate) * up in front of the down experts)
+                    for (size_t i = 0; i < ws.size(); i++)
+                        check(mi_qmm_mulmat_id_produced(b_.handle(), ws[i], t->op_w_->Dim(2), x->prod_,
+                                                        x->prod_aux_ ? x->prod_aux_->Floats().data() : nullptr, x->prod_eps_,
+                                                        x->prod_src_->Floats().data(), x->Dim(1), ids.ints_.data(), ids.Dim(0),
+                                                        ids.Dim(1), ys[i], MI_QMM_HOST));
+                } else {
+                    check(mi_qmm_mulmat_id_multi(b_.handle(), ws.data(), (int)ws.size(), t->op_w_->Dim(2), x->Floats().data(),
+                                                 x->Dim(1), ids.ints_.data(), ids.Dim(0), ids.Dim(1), ys.data(), MI_QMM_HOST));
+                }
                 for (Tensor *u : group) u->ready_ = true;
                 continue;
             }

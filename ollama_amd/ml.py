@@ -179,13 +179,11 @@ class Context:
             raise RuntimeError("Compute on a closed context")
         pending = [t for t in self._nodes if t._data is None and (t._op is not None or t._prod is not None)]
         c = self._b._ctx
-        # producer nodes that must exist as f32: requested, or read by another producer or by a MulmatID
+        # producer nodes that must exist as f32: requested, or read by another producer
         needed = {id(t) for t in tensors}
         for t in pending:
             if t._prod is not None:
                 needed.update(id(s) for s in (t._prod[1], t._prod[2]) if s is not None)
-            elif t._ids is not None:
-                needed.add(id(t._op[1]))
 
         def rows(t: Tensor) -> np.ndarray:
             return t.Floats().reshape(-1, t.Dim(0))
@@ -208,9 +206,16 @@ class Context:
                 nodes = [u for u in pending if u._data is None and u._ids is ids and u._op[1] is x
                          and u._op[0].Dim(2) == t._op[0].Dim(2)]
                 tokens, n_used = ids.Dim(1), ids.Dim(0)
-                b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
-                ys = c.mulmat_id_multi([u._op[0]._weight for u in nodes], t._op[0].Dim(2), b,
-                                       ids._data.reshape(tokens, n_used))
+                idv = ids._data.reshape(tokens, n_used)
+                if x._data is None and x._prod is not None:
+                    # x is a producer nobody needs in f32 (silu(gate) * up in front of the down experts)
+                    kind, src, aux, eps = x._prod
+                    b = src.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
+                    a = None if aux is None else (aux.Floats() if kind == qmm.PRODUCE_RMSNORM else aux.Floats().reshape(b.shape))
+                    ys = [c.mulmat_id_produced(u._op[0]._weight, t._op[0].Dim(2), kind, a, b, idv, eps) for u in nodes]
+                else:
+                    b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
+                    ys = c.mulmat_id_multi([u._op[0]._weight for u in nodes], t._op[0].Dim(2), b, idv)
                 for u, y in zip(nodes, ys):
                     u._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
                 continue

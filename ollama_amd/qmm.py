@@ -27,7 +27,7 @@ EXPORTS = [
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
-    "mi_qmm_mulmat_produced", "mi_qmm_rms_norm", "mi_qmm_swiglu",
+    "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
     "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
@@ -89,6 +89,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_multi.argtypes = [vp, ctypes.POINTER(vp), ci, vp, i64, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_produced.restype = ci
     L.mi_qmm_mulmat_produced.argtypes = [vp, ctypes.POINTER(vp), ci, ci, vp, ctypes.c_float, vp, i64, ctypes.POINTER(vp), ci]
+    L.mi_qmm_mulmat_id_produced.restype = ci
+    L.mi_qmm_mulmat_id_produced.argtypes = [vp, vp, ci, ci, vp, ctypes.c_float, vp, ci, vp, ci, i64, vp, ci]
     L.mi_qmm_rms_norm.restype = ci; L.mi_qmm_rms_norm.argtypes = [vp, vp, vp, ctypes.c_float, i64, i64, vp, ci]
     L.mi_qmm_swiglu.restype = ci; L.mi_qmm_swiglu.argtypes = [vp, vp, vp, i64, i64, vp, ci]
     L.mi_qmm_host_alloc.restype = vp; L.mi_qmm_host_alloc.argtypes = [vp, ctypes.c_size_t]
@@ -404,6 +406,32 @@ class Context:
                                       ids.ctypes.data_as(ctypes.c_void_p), n_used, t,
                                       y.ctypes.data_as(ctypes.c_void_p), HOST))
         return y
+
+    def mulmat_id_produced(self, w: Weight, n_expert: int, producer: int, aux, b: np.ndarray, ids: np.ndarray,
+                           eps: float = 0.0) -> np.ndarray:
+        """mulmat_id on producer(b): PRODUCE_SWIGLU with aux = up, shaped like b (the expert down projection), or
+        PRODUCE_RMSNORM with aux = norm weight [k] or None"""
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        if b.ndim != 3 or ids.ndim != 2 or b.shape[0] != ids.shape[0] or b.shape[2] != w.k:
+            raise ValueError(f"b {b.shape} / ids {ids.shape} do not fit [tokens, b_cols, k={w.k}] / [tokens, n_used]")
+        if aux is not None:
+            aux = np.ascontiguousarray(aux, dtype=np.float32)
+            want = b.shape if producer == PRODUCE_SWIGLU else (w.k,)
+            if aux.shape != want:
+                raise ValueError(f"aux has shape {aux.shape}, the producer wants {want}")
+        t, n_used = ids.shape
+        y = np.empty((t, n_used, w.m // max(n_expert, 1)), dtype=np.float32)
+        _check(lib().mi_qmm_mulmat_id_produced(self._h, w._h, n_expert, producer, _ptr(aux) if aux is not None else None,
+                                               eps, _ptr(b), b.shape[1], _ptr(ids), n_used, t, _ptr(y), HOST))
+        return y
+
+    def mulmat_id_produced_device(self, w: Weight, n_expert: int, producer: int, aux_ptr, b_ptr: int, b_cols: int,
+                                  ids_ptr: int, n_used: int, n_tokens: int, y_ptr: int, eps: float = 0.0):
+        _check(lib().mi_qmm_mulmat_id_produced(self._h, w._h, n_expert, producer,
+                                               ctypes.c_void_p(int(aux_ptr)) if aux_ptr else None, eps,
+                                               ctypes.c_void_p(int(b_ptr)), b_cols, ctypes.c_void_p(int(ids_ptr)), n_used,
+                                               n_tokens, ctypes.c_void_p(int(y_ptr)), DEVICE))
 
     def mulmat_id_multi(self, ws, n_expert: int, b: np.ndarray, ids: np.ndarray):
         """several expert stacks against the same b and ids; host arrays out"""

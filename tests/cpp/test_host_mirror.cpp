@@ -145,6 +145,33 @@ int main() {
                 if (!(e <= 1e-3) || !shape_ok) failures++;
                 ctx->Close();
             }
+            // the expert block's last step: silu(gate) * up inside the down experts' quantization
+            {
+                const int64_t tokens = 5, f = m;   // the stack above as gate and up: [k -> m]; a down stack [m -> 64]
+                auto wf2 = randn((size_t)(f * 64 * n_expert), 0.02f, 4321);
+                std::vector<uint8_t> rawd((size_t)(ref_row_size(MI_QMM_TYPE_Q8_0, f) * 64 * n_expert));
+                if (ref_quantize(MI_QMM_TYPE_Q8_0, wf2.data(), rawd.data(), f, 64 * n_expert, 4) != 0) return 1;
+                backend.LoadExperts("blk.0.ffn_down_exps.weight", MI_QMM_TYPE_Q8_0, f, 64, n_expert, rawd.data());
+                auto ctx = backend.NewContext();
+                auto xv = randn((size_t)(k * tokens), 1.0f, 901);
+                std::vector<int32_t> idv;
+                for (int64_t t = 0; t < tokens; t++)
+                    for (int64_t i = 0; i < n_used; i++) idv.push_back((int32_t)((t + i * 2) % n_expert));
+                auto ids = ctx->FromInts(idv, {n_used, tokens});
+                auto x = ctx->FromFloats(xv, {k, 1, tokens});
+                auto g = backend.Get("blk.0.ffn_up_exps.weight")->MulmatID(*ctx, x, ids);
+                auto u = backend.Get("blk.0.ffn_up_exps.weight")->MulmatID(*ctx, x, ids);
+                auto out = backend.Get("blk.0.ffn_down_exps.weight")->MulmatID(*ctx, g->SILU(*ctx, u), ids);
+                ctx->Compute();
+                std::vector<float> av(g->Floats().size()), ref((size_t)(64 * n_used * tokens));
+                ref_swiglu(g->Floats().data(), u->Floats().data(), (int64_t)av.size(), av.data());
+                if (ref_mul_mat_id(MI_QMM_TYPE_Q8_0, rawd.data(), f, 64, n_expert, av.data(), n_used, idv.data(), n_used, tokens,
+                                   ref.data()) != 0) return 1;
+                const double e = rel_err(out->Floats(), ref);
+                printf("%-24s T=%-3lld rel err %.2e %s\n", "expert down, SILU fused", (long long)tokens, e, e <= 1e-3 ? "ok" : "FAIL");
+                if (!(e <= 1e-3)) failures++;
+                ctx->Close();
+            }
             bool threw_id = false;
             try {
                 auto ctx = backend.NewContext();

@@ -166,6 +166,15 @@ def test_python_mirror_expert_graph(tmp_path):
                              oracle.mul_mat_id(qmm.Q4_K, up, k, ff, n_expert, xv, idv)) <= 1e-3
         assert npref.rel_err(d.Floats().reshape(tokens, n_used, k),
                              oracle.mul_mat_id(qmm.Q8_0, down, ff, k, n_expert, hv, idv)) <= 1e-3
+        # the whole expert block: down reads silu(gate) * up, which runs inside its quantization
+        act = g.SILU(ctx, u)
+        out = wd.MulmatID(ctx, act, ids)
+        ctx.Compute(out)
+        with pytest.raises(RuntimeError):
+            act.Floats()
+        av = oracle.swiglu(g.Floats().reshape(tokens, n_used, ff), u.Floats().reshape(tokens, n_used, ff))
+        assert npref.rel_err(out.Floats().reshape(tokens, n_used, k),
+                             oracle.mul_mat_id(qmm.Q8_0, down, ff, k, n_expert, av, idv)) <= 1e-3
         with pytest.raises(TypeError):
             wg.Mulmat(ctx, ctx.FromFloats(xv.reshape(-1), k, tokens))        # a stack is not a 2-D weight
         with pytest.raises(ValueError):

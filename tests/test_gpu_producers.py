@@ -209,3 +209,52 @@ def test_randomized_produced_sweep(ctx):
             assert np.array_equal(y, y2), f"case {case}: type {t} k={k} m={m} n={n} producer {producer}"
         for w in ws:
             w.free()
+
+
+def _experts(t, n_expert, m, k, seed):
+    return _weights(t, n_expert * m, k, seed)
+
+
+# the down projection of an expert feed-forward block: silu(gate) * up per slot, then the expert's matrix.
+# Decode (in the prologue of the per-pair product), bucketed / matrix-core / expert-GEMM batches (fused
+# quantizer), rows longer than the prefetch registers of the decode kernel.
+@pytest.mark.parametrize("t,k,m,n_expert,tokens,n_used", [(Q4_K, 768, 200, 16, 1, 8), (Q4_K, 768, 64, 16, 3, 4), (Q6_K, 512, 96, 8, 2, 2),
+                                                            (Q8_0, 352, 40, 6, 1, 3), (Q4_0, 2048, 33, 4, 2, 2), (Q4_K, 1024, 70, 4, 40, 2),
+                                                            (Q4_K, 512, 64, 3, 300, 2), (Q8_0, 256, 50, 2, 30, 2), (Q4_K, 9216, 20, 4, 1, 2)])
+def test_expert_down_projection_fused_with_swiglu(ctx, t, k, m, n_expert, tokens, n_used):
+    rng = np.random.default_rng(6000 + t + k + tokens)
+    wb = _experts(t, n_expert, m, k, 6001 + t + k)
+    w = ctx.upload(t, wb, k, n_expert * m)
+    gate = (rng.standard_normal((tokens, n_used, k)) * 2).astype(np.float32)
+    up = rng.standard_normal((tokens, n_used, k)).astype(np.float32)
+    ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+    got = ctx.mulmat_id_produced(w, n_expert, qmm.PRODUCE_SWIGLU, up, gate, ids)
+    want = oracle.mul_mat_id(t, wb, k, m, n_expert, oracle.swiglu(gate, up), ids)
+    assert npref.rel_err(got, want) < TOL
+    assert np.array_equal(got, ctx.mulmat_id(w, n_expert, ctx.swiglu(gate, up), ids))
+    w.free()
+
+
+def test_expert_product_behind_rms_norm_and_errors(ctx):
+    t, k, m, n_expert, n_used = Q4_K, 1024, 48, 8, 3
+    rng = np.random.default_rng(61)
+    wb = _experts(t, n_expert, m, k, 62)
+    w = ctx.upload(t, wb, k, n_expert * m)
+    g = rng.standard_normal(k).astype(np.float32)
+    for tokens in (1, 50):
+        x = rng.standard_normal((tokens, 1, k)).astype(np.float32)
+        ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+        got = ctx.mulmat_id_produced(w, n_expert, qmm.PRODUCE_RMSNORM, g, x, ids, eps=1e-5)
+        xn = oracle.rms_norm(x.reshape(tokens, k), g, 1e-5).reshape(tokens, 1, k)
+        assert npref.rel_err(got, oracle.mul_mat_id(t, wb, k, m, n_expert, xn, ids)) < TOL
+        assert np.array_equal(got, ctx.mulmat_id(w, n_expert, ctx.rms_norm(x.reshape(tokens, k), g, 1e-5).reshape(tokens, 1, k), ids))
+    x = np.ones((1, 1, k), np.float32)
+    ids = np.zeros((1, 1), np.int32)
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_id_produced(w, n_expert, qmm.PRODUCE_SWIGLU, None, x, ids)
+    assert e.value.code == qmm.ERR_INVALID
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_id_produced(w, n_expert, 9, None, x, ids)
+    assert e.value.code == qmm.ERR_INVALID
+    assert np.array_equal(ctx.mulmat_id_produced(w, n_expert, qmm.PRODUCE_NONE, None, x, ids), ctx.mulmat_id(w, n_expert, x, ids))
+    w.free()
