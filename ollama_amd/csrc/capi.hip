@@ -830,14 +830,21 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     DevAct a{};
     a.K = K; a.N = (int)ncols; a.type = q8;
     // the matrix-core kernel addresses activation bytes with 32-bit offsets
-    const bool skinny = skinny_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
+    const bool skinny32 = skinny32_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
+    const bool skinny = skinny32 || (skinny_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32));
     const bool fused = !skinny && pr.kind != PRODUCE_RMSNORM &&
                        gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert, pr.kind == PRODUCE_SWIGLU);
     if (!fused) {
         HIP_TRY(quantize());
         a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16;
     }
-    if (skinny) {
+    if (skinny32) {
+        HIP_TRY(launch_skinny32_id(w->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy, (int *)ctx->ws_buf,
+                                   ctx->num_cus, ctx->stream));
+        if (w2)
+            HIP_TRY(launch_skinny32_id(w2->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy2, (int *)ctx->ws_buf,
+                                       ctx->num_cus, ctx->stream));
+    } else if (skinny) {
         // a few pairs per expert and more: on the matrix cores, the experts' weights read once per 16 pairs
         HIP_TRY(launch_skinny_id(w->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy, (int *)ctx->ws_buf,
                                  ctx->num_cus, ctx->stream));

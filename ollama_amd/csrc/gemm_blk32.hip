@@ -360,8 +360,19 @@ struct Sk32Geo {
     static constexpr int SETS = NCT / 8;
 };
 
-template <bool Q4, int NCT>
-__global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y) {
+// Expert-indexed launches (Tensor.MulmatID, /root/reference/ml/backend.go:153): w is a stack of expert
+// matrices, a workgroup belongs to one group of up to 16 (token, slot) pairs of one expert (bucketed by
+// group_pairs_kernel) and to 16 rows of that expert; the group's pairs are its activation columns.
+struct Sk32Ids {
+    const int *groups;  // groups[0] = number of groups, then records {expert or -1, count, pair[16]}
+    int64_t M;          // rows per expert
+    int wgs_per_group, n_used, b_cols;
+};
+constexpr int SK32_ID_REC = 2 + 16;
+
+template <bool Q4, int NCT, bool ID>
+__global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
+                                                                          Sk32Ids si) {
     typedef Sk32Geo<Q4, NCT> Geo;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, SETS = Geo::SETS;
     const int WAVES = blockDim.x >> 6;
@@ -369,8 +380,32 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
     float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * Geo::WAVE_BYTES);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, g = lane >> 4;
-    const int64_t m0 = (int64_t)blockIdx.x * 16;
-    const int rows_left = (int)min((int64_t)16, w.M - m0);
+    int64_t m0 = (int64_t)blockIdx.x * 16, yrow0 = m0, ldy = w.M;  // first weight row in w; first row and pitch of y
+    int rows_left = (int)min((int64_t)16, w.M - m0);
+    const int *rec = nullptr;
+    if (ID) {
+        const int group = blockIdx.x / si.wgs_per_group, wg = blockIdx.x - group * si.wgs_per_group;
+        if (group >= si.groups[0]) return;
+        rec = si.groups + 1 + (size_t)group * SK32_ID_REC;
+        const int expert = rec[0];
+        nc = rec[1];
+        yrow0 = (int64_t)wg * 16;
+        ldy = si.M;
+        rows_left = (int)min((int64_t)16, si.M - yrow0);
+        if (expert < 0) {  // ids outside the stack: the outputs of these pairs are all NaN
+            for (int o = tid; o < 16 * nc; o += blockDim.x)
+                if ((o & 15) < rows_left) y[(int64_t)rec[2 + (o >> 4)] * ldy + yrow0 + (o & 15)] = __int_as_float(0x7fc00000);
+            return;
+        }
+        m0 = (int64_t)expert * si.M + yrow0;
+    }
+    // activation row behind column i of the launch (i clamped to the live columns)
+    auto col_of = [&](int i) -> unsigned {
+        i = min(i, nc - 1);
+        if (!ID) return (unsigned)(col0 + i);
+        const int pair = rec[2 + i], tok = pair / si.n_used, slot = pair - tok * si.n_used;
+        return (unsigned)(tok * si.b_cols + slot % si.b_cols);
+    };
     const int64_t nblk = w.K / QK, nst = w.K / 256;
     const int64_t s0 = nst * wave / WAVES, s1 = nst * (wave + 1) / WAVES;  // this wave's run of 256-element steps
     uint8_t *wsm = smem + wave * Geo::WAVE_BYTES;
@@ -391,11 +426,11 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
 #pragma unroll
     for (int j = 0; j < Geo::A_INSTRS; j++) {
         const int col = 4 * j + (lane >> 4), slot = lane & 15;  // stage slot [col][slot] holds piece slot ^ col
-        aoff[j] = (unsigned)(col0 + min(col, nc - 1)) * (unsigned)a.K + 16u * (slot ^ col);
+        aoff[j] = col_of(col) * (unsigned)a.K + 16u * (slot ^ col);
     }
     const unsigned dwoff = (unsigned)min(c, rows_left - 1) * (unsigned)nblk * 2u;
-    const unsigned dxoff = (unsigned)(col0 + min(lane >> 1, nc - 1)) * (unsigned)nblk * 4u + 16u * (lane & 1);
-    const unsigned bsoff = (unsigned)(col0 + min(lane, nc - 1)) * (unsigned)nblk * 2u;
+    const unsigned dxoff = col_of(lane >> 1) * (unsigned)nblk * 4u + 16u * (lane & 1);
+    const unsigned bsoff = col_of(lane) * (unsigned)nblk * 2u;
     const uint8_t *wbase = w.p0 + m0 * (Q4 ? nblk * 16 : w.K);
     const uint8_t *dwbase = reinterpret_cast<const uint8_t *>(w.d + m0 * nblk);
     const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
@@ -519,14 +554,15 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
         const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
         float sum = 0.f;
         for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
-        if (i < nc && j < rows_left) y[(int64_t)(col0 + i) * w.M + m0 + j] = sum;
+        if (i < nc && j < rows_left) y[(int64_t)(ID ? rec[2 + i] : col0 + i) * ldy + yrow0 + j] = sum;
     }
 }
 
-template <bool Q4, int NCT>
-void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
+template <bool Q4, int NCT, bool ID = false>
+void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s,
+                        const Sk32Ids &si = Sk32Ids{nullptr, 0, 0, 0, 0}, int64_t id_grid = 0) {
     typedef Sk32Geo<Q4, NCT> Geo;
-    const int64_t groups = (w.M + 15) / 16, nst = w.K / 256;
+    const int64_t groups = ID ? id_grid : (w.M + 15) / 16, nst = w.K / 256;
     // about eight waves per CU over the whole grid (see the K-quant skinny kernel), every wave at least one step
     const int64_t want = ((int64_t)num_cus * 8 + groups / 2) / groups;
     int waves = want >= 8 ? 8 : want >= 6 ? 6 : want >= 4 ? 4 : want >= 3 ? 3 : want >= 2 ? 2 : 1;
@@ -535,11 +571,11 @@ void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols
     static bool allowed[64] = {false};  // more than 64 KiB of dynamic LDS has to be allowed once per device
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny32_kernel<Q4, NCT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny32_kernel<Q4, NCT, ID>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny32_kernel<Q4, NCT><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y);
+    skinny32_kernel<Q4, NCT, ID><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
 }
 
 }  // namespace
@@ -559,6 +595,28 @@ hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int nc
         if (ncols <= 8) launch_skinny32_as<false, 8>(w, a, col0, ncols, y, num_cus, s);
         else launch_skinny32_as<false, 16>(w, a, col0, ncols, y, num_cus, s);
     }
+    return hipGetLastError();
+}
+
+bool skinny32_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert) {
+    // from about four pairs per expert the buckets fill well enough to pay for the matrix cores
+    return skinny32_supports(type, K, M) && pairs >= 4 * (int64_t)n_expert;
+}
+
+hipError_t launch_skinny32_id(const DevWeight &w, int n_expert, const DevAct &a, const int *ids, int n_used, int n_tokens,
+                              int b_cols, float *y, int *groups, int num_cus, hipStream_t s) {
+    if (n_expert < 1 || w.M % n_expert || !skinny32_supports(w.type, w.K, w.M / n_expert) || a.type != T_Q8_0 || a.K != w.K ||
+        !ids || !y || !groups || n_used < 1 || n_tokens < 1 || b_cols < 1 || a.N != (int64_t)b_cols * n_tokens ||
+        (int64_t)a.N * a.K >= ((int64_t)1 << 32) || (w.type == T_Q4_0 && !a.bsums))
+        return hipErrorInvalidValue;
+    const int64_t pairs = (int64_t)n_used * n_tokens, M = w.M / n_expert;
+    if (pairs > 0x7fffffff / 16) return hipErrorInvalidValue;
+    if (hipError_t e = launch_group_pairs(ids, (int)pairs, n_expert, 16, groups, s)) return e;
+    const int64_t max_groups = min(pairs, (int64_t)n_expert + 1 + pairs / 16), wgs_per_group = (M + 15) / 16;
+    if (max_groups * wgs_per_group > 0x7fffffff) return hipErrorInvalidValue;
+    const Sk32Ids si{groups, M, (int)wgs_per_group, n_used, b_cols};
+    if (w.type == T_Q4_0) launch_skinny32_as<true, 16, true>(w, a, 0, 16, y, num_cus, s, si, max_groups * wgs_per_group);
+    else launch_skinny32_as<false, 16, true>(w, a, 0, 16, y, num_cus, s, si, max_groups * wgs_per_group);
     return hipGetLastError();
 }
 

@@ -91,6 +91,10 @@ hipError_t launch_gemm_blk32(const DevWeight &w, const DevAct &a, float *y, int 
 bool skinny32_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                            hipStream_t s);
+// the same kernel on expert stacks (see launch_gemv_id for the arguments): pairs bucketed 16 to a group
+bool skinny32_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);
+hipError_t launch_skinny32_id(const DevWeight &w, int n_expert, const DevAct &a, const int *ids, int n_used, int n_tokens,
+                              int b_cols, float *y, int *groups, int num_cus, hipStream_t s);
 
 // Expert GEMM (K-quants, batches with many pairs per expert): sort_pairs sorts the (token, slot) pairs by
 // expert into runs of whole 64- or 128-row tiles; the tiled GEMM multiplies every run by its expert's matrix,

@@ -494,11 +494,11 @@ def test_mulmat_id_matches_oracle(ctx, t, tokens, n_used, b_cols):
 
 @pytest.mark.parametrize("t,tokens", [(Q4_K, 3), (Q8_0, 3), (Q8_0, 24), (Q4_0, 24)])
 def test_mulmat_id_equals_mulmat_on_the_expert_alone(ctx, t, tokens):
-    """the streaming kernels (decode: one pair per group; Q4_0 / Q8_0 batches: pairs bucketed by expert)
-    give bit for bit what the plain one-column product gives on that expert's slice, whatever group a
-    pair lands in"""
+    """the streaming kernels (decode: one pair per group; Q4_0 / Q8_0 batches whose K is no multiple of 256:
+    pairs bucketed by expert) give bit for bit what the plain one-column product gives on that expert's
+    slice, whatever group a pair lands in"""
     rng = np.random.default_rng(7200 + t + tokens)
-    k, m, n_expert, n_used = 2048, 96, 6, 3
+    k, m, n_expert, n_used = (2048 if tokens < 8 else 2080), 96, 6, 3
     wb = _experts(t, n_expert, m, k, 7201 + t)
     w = ctx.upload(t, wb, k, n_expert * m)
     b = rng.standard_normal((tokens, 1, k), dtype=np.float32)
@@ -514,11 +514,14 @@ def test_mulmat_id_equals_mulmat_on_the_expert_alone(ctx, t, tokens):
 
 
 def test_mulmat_id_on_the_matrix_cores(ctx):
-    """K-quants from about two pairs per expert up: groups of 16 pairs through the MFMA kernel; ragged
-    expert height, experts that nobody picked, one expert picked by more than 16 pairs"""
+    """K-quants from about two pairs per expert up (Q4_0 / Q8_0 with K a multiple of 256: from four): groups of
+    16 pairs through the MFMA kernels; ragged expert height, experts that nobody picked, one expert picked by
+    more than 16 pairs, ids outside the stack among device ids"""
     rng = np.random.default_rng(7250)
     for t, k, m, n_expert, tokens, n_used, b_cols in ((Q4_K, 1024, 72, 5, 40, 2, 1), (Q6_K, 512, 200, 9, 30, 4, 4),
-                                                      (Q4_K, 2048, 33, 3, 64, 2, 2)):
+                                                      (Q4_K, 2048, 33, 3, 64, 2, 2), (Q4_0, 1024, 72, 5, 40, 2, 1),
+                                                      (Q8_0, 512, 200, 6, 30, 4, 4), (Q8_0, 256, 17, 3, 200, 2, 2),
+                                                      (Q4_0, 2304, 50, 4, 33, 3, 1)):
         wb = _experts(t, n_expert, m, k, 7251 + t)
         w = ctx.upload(t, wb, k, n_expert * m)
         b = rng.standard_normal((tokens, b_cols, k), dtype=np.float32)
@@ -528,6 +531,18 @@ def test_mulmat_id_on_the_matrix_cores(ctx):
         assert npref.rel_err(got, oracle.mul_mat_id(t, wb, k, m, n_expert, b, ids)) < TOL
         # a pair's result does not depend on the other pairs of the call: same call, order of tokens reversed
         assert np.array_equal(ctx.mulmat_id(w, n_expert, b[::-1], ids[::-1])[::-1], got)
+        bad = ids.copy()
+        bad[0, 0] = n_expert
+        bad[-1, -1] = -1
+        db, dids = DeviceArray(b), DeviceArray(bad)
+        dy = DeviceArray(np.zeros((tokens, n_used, m), np.float32), zero=True)
+        ctx.mulmat_id_device(w, n_expert, db.ptr, b_cols, dids.ptr, n_used, tokens, dy.ptr)
+        ctx.sync()
+        out = dy.numpy()
+        isbad = (bad < 0) | (bad >= n_expert)
+        assert np.isnan(out[isbad]).all() and np.array_equal(out[~isbad], got[~isbad])
+        for d in (db, dids, dy):
+            d.free()
         w.free()
 
 
