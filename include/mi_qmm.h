@@ -81,7 +81,10 @@ int mi_qmm_vec_dot_type(int weight_type);
 int mi_qmm_init(int device_ordinal, mi_qmm_ctx **out);
 void mi_qmm_destroy(mi_qmm_ctx *ctx);
 /* run on a caller-owned hipStream_t (e.g. the framework's current stream); NULL restores the
- * ctx's own stream.  The ctx never destroys a caller stream. */
+ * ctx's own stream.  The ctx never destroys a caller stream.  The call waits for the work queued on
+ * the previous stream.  With device pointers the product entry points only queue kernels once the
+ * ctx's scratch buffers have reached their size (first call of a shape), so such calls may be
+ * captured into a HIP graph on the caller's stream after one eager call. */
 int mi_qmm_set_stream(mi_qmm_ctx *ctx, void *hip_stream);
 /* block until everything queued on the ctx's stream has finished */
 int mi_qmm_sync(mi_qmm_ctx *ctx);

@@ -43,3 +43,52 @@ class DeviceArray:
         if self.ptr:
             _rt().hipFree(self.ptr)
             self.ptr = None
+
+    def set(self, a: np.ndarray):
+        src = np.ascontiguousarray(a, dtype=self.dtype)
+        assert src.nbytes == self.nbytes
+        assert _rt().hipMemcpy(self.ptr, src.ctypes.data, src.nbytes, 1) == 0
+
+
+class Stream:
+    """a HIP stream of default priority, with capture into a graph"""
+
+    def __init__(self):
+        h = _rt()
+        self.ptr = ctypes.c_void_p()
+        h.hipStreamCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        assert h.hipStreamCreate(ctypes.byref(self.ptr)) == 0
+        h.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+        h.hipStreamBeginCapture.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        h.hipStreamEndCapture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+        h.hipGraphInstantiate.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                          ctypes.c_size_t]
+        h.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        h.hipGraphExecDestroy.argtypes = [ctypes.c_void_p]
+        h.hipGraphDestroy.argtypes = [ctypes.c_void_p]
+        h.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+
+    def sync(self):
+        assert _rt().hipStreamSynchronize(self.ptr) == 0
+
+    def capture(self, fn):
+        """runs fn() with the stream capturing; returns a callable that replays the captured graph"""
+        h = _rt()
+        assert h.hipStreamBeginCapture(self.ptr, 0) == 0  # hipStreamCaptureModeGlobal
+        try:
+            fn()
+        finally:
+            graph = ctypes.c_void_p()
+            rc = h.hipStreamEndCapture(self.ptr, ctypes.byref(graph))
+        assert rc == 0 and graph.value
+        exe = ctypes.c_void_p()
+        assert h.hipGraphInstantiate(ctypes.byref(exe), graph, None, None, 0) == 0
+        self._graphs = getattr(self, "_graphs", []) + [(exe, graph)]
+        return lambda: h.hipGraphLaunch(exe, self.ptr)
+
+    def destroy(self):
+        h = _rt()
+        for exe, graph in getattr(self, "_graphs", []):
+            h.hipGraphExecDestroy(exe)
+            h.hipGraphDestroy(graph)
+        h.hipStreamDestroy(self.ptr)

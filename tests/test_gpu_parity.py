@@ -10,7 +10,7 @@ import pytest
 
 import npref
 import oracle
-from hipmem import DeviceArray
+from hipmem import DeviceArray, Stream
 from npref import Q4_0, Q4_K, Q6_K, Q8_0, Q8_K
 from ollama_amd import qmm
 
@@ -762,3 +762,57 @@ def test_mulmat_id_expert_gemm(ctx, t, k, m, n_expert, tokens, n_used, b_cols):
     for d in (db, dids, dy):
         d.free()
     w.free()
+
+
+def test_device_entry_points_replay_from_a_hip_graph():
+    """Once the scratch buffers have their size, the device-pointer entry points only launch kernels, so a
+    decode block can be captured on a caller's stream and replayed: gate and up behind RMSNorm in one launch,
+    down behind SwiGLU, an expert product, a skinny product.  Every replay (with new inputs, and eager work
+    in between) must give the eager result."""
+    rng = np.random.default_rng(31)
+    k, f, n_expert, n_used = 1024, 1536, 8, 2
+    c = qmm.Context(0)
+    st = Stream()
+    c.set_stream(st.ptr.value)
+    wg, wu = (c.upload(Q4_K, _weights(Q4_K, f, k, 310 + i), k, f) for i in range(2))
+    wd = c.upload(Q6_K, _weights(Q6_K, k, f, 312), f, k)
+    we = c.upload(Q4_K, _experts(Q4_K, n_expert, 64, k, 313), k, n_expert * 64)
+    ws = c.upload(Q8_0, _weights(Q8_0, 200, k, 314), k, 200)
+    x, g = DeviceArray(np.zeros((1, k), np.float32)), DeviceArray(rng.standard_normal(k).astype(np.float32))
+    x5 = DeviceArray(np.zeros((5, k), np.float32))
+    ids = DeviceArray(np.array([[3, 6]], np.int32))
+    outs = {"gate": DeviceArray(np.zeros((1, f), np.float32)), "up": DeviceArray(np.zeros((1, f), np.float32)),
+            "down": DeviceArray(np.zeros((1, k), np.float32)), "exp": DeviceArray(np.zeros((1, n_used, 64), np.float32)),
+            "skinny": DeviceArray(np.zeros((5, 200), np.float32))}
+
+    def block():
+        c.mulmat_produced_device([wg, wu], qmm.PRODUCE_RMSNORM, g.ptr, x.ptr, 1, [outs["gate"].ptr, outs["up"].ptr], eps=1e-5)
+        c.mulmat_produced_device([wd], qmm.PRODUCE_SWIGLU, outs["up"].ptr, outs["gate"].ptr, 1, [outs["down"].ptr])
+        c.mulmat_id_device(we, n_expert, x.ptr, 1, ids.ptr, n_used, 1, outs["exp"].ptr)
+        c.mulmat_device(ws, x5.ptr, 5, outs["skinny"].ptr)
+
+    def fresh_inputs():
+        x.set(rng.standard_normal((1, k)).astype(np.float32))
+        x5.set(rng.standard_normal((5, k)).astype(np.float32))
+
+    fresh_inputs()
+    block()                      # sizes the scratch buffers (allocations are not capturable)
+    st.sync()
+    replay = st.capture(block)
+    for _ in range(3):
+        fresh_inputs()
+        block()
+        st.sync()
+        eager = {n: d.numpy() for n, d in outs.items()}
+        for d in outs.values():
+            d.set(np.zeros(d.shape, np.float32))
+        assert replay() == 0
+        st.sync()
+        for n, d in outs.items():
+            assert np.array_equal(d.numpy(), eager[n]), n
+    for w in (wg, wu, wd, we, ws):
+        w.free()
+    for d in [x, g, x5, ids] + list(outs.values()):
+        d.free()
+    c.close()
+    st.destroy()
