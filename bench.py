@@ -304,7 +304,14 @@ def main() -> int:
                 qmm._check(L.mi_qmm_swiglu(ctx._h, vp(y_gate.data_ptr()), vp(y_up.data_ptr()), FFN_M, 1, vp(act.data_ptr()), qmm.DEVICE))
                 ctx.mulmat_device(ent["down"], act.data_ptr(), 1, y_down.data_ptr())
 
-        for label, fn in (("RMSNorm and SwiGLU inside the two product launches", block_fused),
+        def block_paired():
+            for ent in pool:
+                ctx.mulmat_swiglu_device(ent["gate"], ent["up"], x.data_ptr(), 1, act.data_ptr(), qmm.PRODUCE_RMSNORM,
+                                         gnorm.data_ptr(), 1e-5)
+                ctx.mulmat_device(ent["down"], act.data_ptr(), 1, y_down.data_ptr())
+
+        for label, fn in (("RMSNorm, gate, up and their gating in one launch, down in a second", block_paired),
+                          ("RMSNorm and SwiGLU inside the two product launches", block_fused),
                           ("rms_norm, gate+up, swiglu, down: four launches", block_unfused)):
             fn()
             tm = timed(fn, 5) / (5 * len(pool))

@@ -159,8 +159,18 @@ enum {
 int mi_qmm_mulmat_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int producer,
                            const float *aux, float eps, const float *x, int64_t n, float *const *ys,
                            int location);
+/* Gate and up of a feed-forward block together with their gating -- the graph pattern
+ * gate.SILU(ctx, up) with gate = w_gate.Mulmat(x') and up = w_up.Mulmat(x'), x' = x or RMSNorm(x)
+ * (producer MI_QMM_PRODUCE_NONE or _RMSNORM with aux = norm weight [k] or NULL):
+ *     h[i][r] = silu(w_gate row r . Q8(x'[i])) * (w_up row r . Q8(x'[i])),  h f32 [n][m].
+ * With one activation row this is ONE launch: a wave walks row r of both matrices, and whoever holds
+ * the two totals of a row gates them, so neither product goes through memory and silu is evaluated
+ * once per element.  Larger n: the two products (mi_qmm_mulmat_produced) and mi_qmm_swiglu.
+ * Bit-identical to those either way. */
+int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_qmm_weight *w_up, int producer,
+                         const float *aux, float eps, const float *x, int64_t n, float *h, int location);
 /* The same producers as plain f32 operations, for graph nodes that something other than a product
- * reads: x, y f32 [n][k] (k a multiple of 4), g f32 [k] or NULL; gate, up, y f32 [n][k]. */
+ * reads: x, y f32 [n][k] (k a multiple of 4), g f32 [k] or NULL; gate, up, y f32 [n][k] (any k). */
 int mi_qmm_rms_norm(mi_qmm_ctx *ctx, const float *x, const float *g, float eps, int64_t k, int64_t n,
                     float *y, int location);
 int mi_qmm_swiglu(mi_qmm_ctx *ctx, const float *gate, const float *up, int64_t k, int64_t n, float *y,

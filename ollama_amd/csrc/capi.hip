@@ -695,6 +695,55 @@ int mi_qmm_mulmat_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     return mulmat_multi_impl(ctx, ws, count, &pr, x, n, ys, location);
 }
 
+int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_qmm_weight *w_up, int producer,
+                         const float *aux, float eps, const float *x, int64_t n, float *h, int location) {
+    if (!w_gate || !w_up) return fail(MI_QMM_ERR_INVALID, "w_gate or w_up is NULL");
+    if (producer != MI_QMM_PRODUCE_NONE && producer != MI_QMM_PRODUCE_RMSNORM)
+        return fail(MI_QMM_ERR_INVALID, "the producer in front of gate and up is none or RMSNorm, not %d", producer);
+    if (w_gate->dev.K != w_up->dev.K || w_gate->dev.M != w_up->dev.M)
+        return fail(MI_QMM_ERR_INVALID, "gate is %lld x %lld, up is %lld x %lld: the gating needs equal shapes",
+                    (long long)w_gate->dev.M, (long long)w_gate->dev.K, (long long)w_up->dev.M, (long long)w_up->dev.K);
+    if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
+    int rc = check_product_args(ctx, w_gate, location, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    if (w_up->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "w_up is on another device");
+    if (producer == MI_QMM_PRODUCE_RMSNORM && !(eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
+    if (n == 0) return MI_QMM_OK;
+    if (!x || !h) return fail(MI_QMM_ERR_INVALID, "x or h is NULL");
+    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    const int64_t K = w_gate->dev.K, M = w_gate->dev.M;
+    const bool rms = producer == MI_QMM_PRODUCE_RMSNORM;
+    const bool paired = n == 1 && w_gate->dev.type == w_up->dev.type && gemv_pair_supported(w_gate->dev.type, K, M, rms);
+    // x, the norm weight, h and (unless both products and the gating are one launch) the two products
+    const size_t ybytes = (size_t)(n * M) * 4;
+    const size_t bytes[5] = {(size_t)(n * K) * 4, rms && aux ? (size_t)K * 4 : 0, ybytes, paired ? 0 : ybytes, paired ? 0 : ybytes};
+    const void *src[5] = {x, aux, h, nullptr, nullptr};
+    void *d[5];
+    if (location == MI_QMM_HOST || paired) {
+        if ((rc = stage_in(ctx, location, src, bytes, 2, 5, d))) return rc;
+    } else {
+        // device caller: only the two intermediate products need room
+        d[0] = const_cast<float *>(x); d[1] = const_cast<float *>(aux); d[2] = h;
+        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, 2 * align_up(ybytes, 256), ctx->stream))) return rc;
+        d[3] = ctx->io_buf;
+        d[4] = (char *)ctx->io_buf + align_up(ybytes, 256);
+    }
+    const Produce pr{producer, rms && aux ? (const float *)d[1] : nullptr, eps, nullptr};
+    if (paired) {
+        HIP_TRY(launch_gemv_pair_f32(w_gate->dev, w_up->dev, (const float *)d[0], (float *)d[2], ctx->stream, &pr));
+    } else {
+        const mi_qmm_weight *ws[2] = {w_gate, w_up};
+        float *ys[2] = {(float *)d[3], (float *)d[4]};
+        if ((rc = mulmat_multi_impl(ctx, ws, 2, &pr, (const float *)d[0], n, ys, MI_QMM_DEVICE))) return rc;
+        HIP_TRY(launch_swiglu(ys[0], ys[1], n * M, (float *)d[2], ctx->stream));
+    }
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(h, d[2], ybytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
 int mi_qmm_rms_norm(mi_qmm_ctx *ctx, const float *x, const float *g, float eps, int64_t k, int64_t n, float *y,
                     int location) {
     int rc = check_elementwise_args(ctx, k, n, location);
@@ -716,8 +765,9 @@ int mi_qmm_rms_norm(mi_qmm_ctx *ctx, const float *x, const float *g, float eps, 
 }
 
 int mi_qmm_swiglu(mi_qmm_ctx *ctx, const float *gate, const float *up, int64_t k, int64_t n, float *y, int location) {
-    int rc = check_elementwise_args(ctx, k, n, location);
+    int rc = check_elementwise_args(ctx, k % 4 ? 4 * k : k, n, location);  // any k: the operation is elementwise
     if (rc) return rc;
+    if (k < 0) return fail(MI_QMM_ERR_INVALID, "k=%lld must be non-negative", (long long)k);
     if (k * n == 0) return MI_QMM_OK;
     if (!gate || !up || !y) return fail(MI_QMM_ERR_INVALID, "gate, up or y is NULL");
     const size_t b = (size_t)(n * k) * 4, bytes[3] = {b, b, b};

@@ -765,6 +765,122 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Gate and up of a feed-forward block in one pass with the gating in the epilogue: h = silu(Wg x) * (Wu x).
+// A wave walks "virtual rows" 2j (row j of the gate matrix) and 2j+1 (row j of the up matrix) with the
+// thin kernel's loop, so both totals of a row meet in one wave (neighbouring lanes) or in one
+// workgroup's LDS, and silu(gate) * up is computed once per element, by whoever produced it -- instead
+// of by every workgroup of the down projection in its prologue.  One column, f32 x (optionally through
+// RMSNorm first).  The two totals are the numbers the separate products give, so h has the bits of
+// mi_qmm_swiglu on their outputs.
+// ---------------------------------------------------------------------------------------------
+template <class P, bool DIRECT, int RPL>
+__device__ __forceinline__ void thin_rows_pair(const DevWeight &wa, const DevWeight &wb, const typename P::Geo &g,
+                                               typename P::Raw cur, const typename P::Act (&act)[1], int64_t wrow0, int nv,
+                                               int lane, float &keep, float *part, int rl0v, int kw, int kseg) {
+    static_assert(RPL == 1 || DIRECT, "rows side by side only when a row lies inside one K segment");
+    const int run = RPL == 1 ? 0 : lane / (64 / RPL);
+    keep = 0.f;
+#pragma unroll 1
+    for (int i = 0; i < nv; i += RPL) {
+        float acc[1] = {0.f};
+        P::template dot<1>(cur, g, act, acc);
+        if (i + RPL < nv) {  // wave-uniform branch
+            const int v = min(i + RPL + run, nv - 1);
+            cur = P::load(v & 1 ? wb : wa, g, wrow0 + (v >> 1));
+        }
+        const int tot_all = __float_as_int(run_total<RPL>(acc[0]));
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            const float tot = __int_as_float(__builtin_amdgcn_readlane(tot_all, 64 / RPL * (r + 1) - 1));
+            if (DIRECT) keep = lane == 63 - (i + r) ? tot : keep;
+            else if (lane == 63) part[(rl0v + i) * kw + kseg] = tot;
+        }
+    }
+}
+
+template <class P, bool DIRECT, int XMODE, int RPL, int XP>
+__global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const float *__restrict__ xf, int rows_per_wave, int kw,
+                                                         int rw_log2, Produce pr) {
+    static_assert(XMODE == 1 || XMODE == 2, "f32 x, plain or through RMSNorm");
+    extern __shared__ __align__(16) uint8_t smem[];
+    const DevWeight wa{ta.p0[0], ta.p1[0], ta.p2[0], ta.d[0], ta.K, ta.M[0], ta.type};
+    const DevWeight wb{ta.p0[1], ta.p1[1], ta.p2[1], ta.d[1], ta.K, ta.M[0], ta.type};
+    float *__restrict__ hout = ta.y[0];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = 1 << rw_log2;
+    const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
+    const int rows_per_wg = rows_per_wave << rw_log2;          // rows of h per workgroup
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
+    const int nrows = (int)min((int64_t)rows_per_wg, wa.M - r0);
+    const int rl0 = rg * rows_per_wave;
+    const int nrw = max(0, min(rows_per_wave, nrows - rl0));   // rows of h of this wave; 2 * nrw virtual rows
+    const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);
+    const typename P::Geo g = P::geo(wa, kseg, vlane);
+
+    const int64_t K = ta.K;
+    const int nblk = (int)(K / P::ACT_BLK);
+    const int nbs = P::USES_BSUMS ? (int)(K / P::ACT_BSUM) : 0;
+    const size_t act_bytes = (((size_t)(K + nblk * 4 + nbs * 2)) + 15) / 16 * 16;
+    int8_t *lqs = reinterpret_cast<int8_t *>(smem);
+    float *ld_ = reinterpret_cast<float *>(smem + (size_t)K);
+    int16_t *lbs = reinterpret_cast<int16_t *>(smem + (size_t)K + (size_t)nblk * 4);
+    const float4 *x4 = reinterpret_cast<const float4 *>(xf);
+    const int total4 = (int)(K / 4);
+    const int nwaves = blockDim.x >> 6;
+    float4 xpre[XP], apre[XP];
+    prefetch_x(x4, total4, wave, nwaves, lane, xpre);
+    const bool has_aux = XMODE == 2 && pr.aux != nullptr;
+    if (XMODE == 2) prefetch_x(has_aux ? reinterpret_cast<const float4 *>(pr.aux) : x4, total4, wave, nwaves, lane, apre);
+    typename P::Raw cur;
+    if (nrw > 0) {
+        const int v = min(run, 2 * nrw - 1);
+        cur = P::load(v & 1 ? wb : wa, g, r0 + rl0 + (v >> 1));
+    }
+    constexpr size_t PSUM_BYTES = XMODE == 2 ? XPRE * 16 * sizeof(double) : 0;
+    if (XMODE == 2) {
+        double *psum = reinterpret_cast<double *>(smem + act_bytes);
+#pragma unroll
+        for (int j = 0; j < XP; j++) {
+            const int c = wave + j * nwaves;
+            if (c * 64 < total4) {  // wave-uniform
+                const double sq = piece_sumsq(c * 64 + lane < total4 ? xpre[j] : make_float4(0.f, 0.f, 0.f, 0.f));
+                if (lane == 0) psum[c] = sq;
+            }
+        }
+        __syncthreads();
+        double tot = 0.0;
+        for (int c = 0; c * 64 < total4; c++) tot += psum[c];
+        const float scale = rms_scale_of(tot, K, pr.eps);
+#pragma unroll
+        for (int j = 0; j < XP; j++) xpre[j] = rms_apply(xpre[j], scale, apre[j], has_aux);
+    }
+    quantize_x_to_lds<P, XP>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
+    __syncthreads();
+    float *part = reinterpret_cast<float *>(smem + act_bytes + PSUM_BYTES);
+
+    if (nrw > 0) {
+        typename P::Act act[1];
+        const LdsAct la{lqs, ld_, lbs, K};
+        P::load_act(la, 0, kseg, vlane, g, act[0]);
+        float keep;  // lane 63-v ends up holding the total of the wave's virtual row v
+        thin_rows_pair<P, DIRECT, RPL>(wa, wb, g, cur, act, r0 + rl0, 2 * nrw, lane, keep, part, 2 * rl0, kw, kseg);
+        if (DIRECT) {
+            const float up = dpp_mov<0xB1>(keep);  // lane ^ 1: the odd lane 63-2j takes the up total from lane 62-2j
+            if ((lane & 1) && lane > 63 - 2 * nrw) hout[r0 + rl0 + ((63 - lane) >> 1)] = silu_mul(keep, up);
+        }
+    }
+    if (DIRECT) return;
+
+    __syncthreads();
+    for (int i = threadIdx.x; i < nrows; i += blockDim.x) {
+        float gsum = 0.f, usum = 0.f;
+        for (int k = 0; k < kw; k++) gsum += part[(2 * i) * kw + k];
+        for (int k = 0; k < kw; k++) usum += part[(2 * i + 1) * kw + k];
+        hout[r0 + i] = silu_mul(gsum, usum);
+    }
+}
+
 struct Plan { int kw, rw, rw_log2, spw, rows_per_wg, rpl; unsigned grid; size_t lds; };
 
 // 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), one or two workgroups per CU.
@@ -860,6 +976,7 @@ void launch_thin(const Plan &p, const ThinArgs &ma, const DevAct &a, const float
     else if (NC == 1 && pr.kind == PRODUCE_RMSNORM) launch_thin_mode<P, 1, 2>(p, ma, a, xf, col0, pr, s);
     else if (NC == 1 && pr.kind == PRODUCE_SWIGLU && one_piece) launch_thin_mode<P, 1, 3, 1>(p, ma, a, xf, col0, pr, s);
     else if (NC == 1 && pr.kind == PRODUCE_SWIGLU) launch_thin_mode<P, 1, 3>(p, ma, a, xf, col0, pr, s);
+    else if (NC == 1 && one_piece) launch_thin_mode<P, 1, 1, 1>(p, ma, a, xf, col0, pr, s);
     else launch_thin_mode<P, NC, 1>(p, ma, a, xf, col0, pr, s);
 }
 
@@ -1009,6 +1126,80 @@ hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int coun
     a.N = ncols;
     a.type = (ws[0].type == T_Q4_K || ws[0].type == T_Q6_K) ? T_Q8_K : T_Q8_0;
     return dispatch(ws, ys, count, a, x, 0, ncols, num_cus, s, pr);
+}
+
+namespace {
+
+template <class P, int XMODE, int XP>
+void launch_pair_mode(const Plan &p, const ThinArgs &ta, const float *xf, const Produce &pr, unsigned grid, hipStream_t s) {
+    const dim3 block(64 * p.kw * p.rw);
+    const int rpw = (p.rows_per_wg >> p.rw_log2) / 2;  // rows of h per wave: half the virtual rows
+#define PAIR_LAUNCH(DIRECT, RPL) \
+    gemv_pair_kernel<P, DIRECT, XMODE, RPL, XP><<<grid, block, p.lds, s>>>(ta, xf, rpw, p.kw, p.rw_log2, pr)
+    if (p.kw > 1) PAIR_LAUNCH(false, 1);
+    else if (p.rpl == 4) PAIR_LAUNCH(true, 4);
+    else if (p.rpl == 2) PAIR_LAUNCH(true, 2);
+    else PAIR_LAUNCH(true, 1);
+#undef PAIR_LAUNCH
+}
+
+template <class P>
+bool pair_plan(int64_t K, int64_t M, bool rms, Plan &p) {
+    // planned like the two matrices in one launch: the virtual rows of a wave are an even number
+    if (M < 1 || 2 * M > 65536 || !make_thin_plan<P>(K, 2 * M, 1, true, p, rms)) return false;
+    return ((p.rows_per_wg >> p.rw_log2) & 1) == 0;
+}
+
+template <class P>
+hipError_t launch_pair_type(const DevWeight &wg, const DevWeight &wu, const float *xf, float *h, const Produce &pr,
+                            hipStream_t s) {
+    Plan p;
+    const bool rms = pr.kind == PRODUCE_RMSNORM;
+    if (!pair_plan<P>(wg.K, wg.M, rms, p)) return hipErrorInvalidValue;
+    ThinArgs ta;
+    for (int i = 0; i < MAX_MULTI; i++) {
+        const DevWeight &w = i == 1 ? wu : wg;
+        ta.p0[i] = w.p0; ta.p1[i] = w.p1; ta.p2[i] = w.p2; ta.d[i] = w.d; ta.y[i] = h; ta.M[i] = wg.M;
+        ta.wg_end[i] = 0x7fffffff;
+    }
+    ta.K = wg.K; ta.type = wg.type;
+    const int rows_per_wg = p.rows_per_wg / 2;
+    const unsigned grid = (unsigned)((wg.M + rows_per_wg - 1) / rows_per_wg);
+    const bool one_piece = wg.K <= (int64_t)256 * p.kw * p.rw;
+    if (rms && one_piece) launch_pair_mode<P, 2, 1>(p, ta, xf, pr, grid, s);
+    else if (rms) launch_pair_mode<P, 2, XPRE>(p, ta, xf, pr, grid, s);
+    else if (one_piece) launch_pair_mode<P, 1, 1>(p, ta, xf, pr, grid, s);
+    else launch_pair_mode<P, 1, XPRE>(p, ta, xf, pr, grid, s);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool gemv_pair_supported(int type, int64_t K, int64_t M, bool rms) {
+    Plan p;
+    switch (type) {
+    case T_Q4_K: return pair_plan<PolQ4K>(K, M, rms, p);
+    case T_Q6_K: return pair_plan<PolQ6K>(K, M, rms, p);
+    case T_Q4_0: return pair_plan<PolQ4_0>(K, M, rms, p);
+    case T_Q8_0: return pair_plan<PolQ8_0>(K, M, rms, p);
+    default: return false;
+    }
+}
+
+hipError_t launch_gemv_pair_f32(const DevWeight &wg, const DevWeight &wu, const float *x, float *h, hipStream_t s,
+                                const Produce *produce) {
+    if (!x || !h || wg.type != wu.type || wg.K != wu.K || wg.M != wu.M || wg.K < 1 || wg.K > gemv_max_k(wg.type))
+        return hipErrorInvalidValue;
+    Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
+    if (produce) pr = *produce;
+    if (pr.kind != PRODUCE_NONE && pr.kind != PRODUCE_RMSNORM) return hipErrorInvalidValue;
+    switch (wg.type) {
+    case T_Q4_K: return launch_pair_type<PolQ4K>(wg, wu, x, h, pr, s);
+    case T_Q6_K: return launch_pair_type<PolQ6K>(wg, wu, x, h, pr, s);
+    case T_Q4_0: return launch_pair_type<PolQ4_0>(wg, wu, x, h, pr, s);
+    case T_Q8_0: return launch_pair_type<PolQ8_0>(wg, wu, x, h, pr, s);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 bool gemv_produce_supported(int type, int64_t K, int64_t total_m) {

@@ -44,6 +44,12 @@ bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols);
 hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols,
                                  int num_cus, hipStream_t s, const Produce *produce = nullptr);
 bool gemv_produce_supported(int type, int64_t K, int64_t total_m);
+// Gate and up of a feed-forward block at one column with the gating in the epilogue: h [M] =
+// silu(wg . Q8(x')) * (wu . Q8(x')), x' = x or RMSNorm(x) (produce: NONE or RMSNORM).  Same bits as the
+// two products followed by launch_swiglu.
+bool gemv_pair_supported(int type, int64_t K, int64_t M, bool rms);
+hipError_t launch_gemv_pair_f32(const DevWeight &wg, const DevWeight &wu, const float *x, float *h, hipStream_t s,
+                                const Produce *produce = nullptr);
 // largest K the GEMV handles for a weight type
 int64_t gemv_max_k(int type);
 // Expert-indexed GEMV: w is a stack of n_expert matrices (w.M = rows per expert * n_expert), a holds

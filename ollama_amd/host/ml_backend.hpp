@@ -8,7 +8,8 @@
 // W.Mulmat(ctx, x) = [M, N]) and the same error behaviour: tensor ops have no error return, so a
 // failure throws (the Go interface panics).  Mulmat is lazy; Compute runs the pending nodes, sharing
 // one activation quantization between all nodes that read the same x.  An RMSNorm or SILU(up) node that only
-// products read is never materialized: it runs inside those products' quantization.
+// products read is never materialized: it runs inside those products' quantization; gate.SILU(up) on two
+// products of one x that nothing else reads runs as one call and the two products are not materialized.
 #pragma once
 
 #include <cstdint>
@@ -77,6 +78,7 @@ private:
     std::shared_ptr<Tensor> prod_src_;   //   its input,
     std::shared_ptr<Tensor> prod_aux_;   //   the norm weight (may be null) or up,
     float prod_eps_ = 0.f;               //   and eps
+    bool absorbed_ = false;              // a product computed inside the SILU node that reads it
 };
 
 class Backend {
@@ -189,15 +191,56 @@ public:
         std::set<const Tensor *> needed;
         for (auto &t : wanted) needed.insert(t.get());
         for (auto &n : nodes_) {
-            if (n->ready_) continue;
+            if (n->ready_ || n->absorbed_) continue;
             if (n->prod_) {
                 needed.insert(n->prod_src_.get());
                 if (n->prod_aux_) needed.insert(n->prod_aux_.get());
             }
         }
+        // gate.SILU(up) on two pending products of one x that nothing else reads: one call computes the gated
+        // result (mi_qmm_mulmat_swiglu), the two products are never materialized
+        std::map<const Tensor *, int> n_readers;
+        for (auto &n : nodes_) {
+            if (n->ready_ || n->absorbed_) continue;
+            if (n->prod_) {
+                n_readers[n->prod_src_.get()]++;
+                if (n->prod_aux_) n_readers[n->prod_aux_.get()]++;
+            } else {
+                n_readers[n->op_x_.get()]++;
+            }
+        }
+        std::map<const Tensor *, Tensor *> pair_of;
+        for (auto &n : nodes_) {
+            if (n->ready_ || n->prod_ != MI_QMM_PRODUCE_SWIGLU) continue;
+            Tensor *gate = n->prod_src_.get(), *up = n->prod_aux_.get();
+            auto pending_product = [&](const Tensor *p) {
+                return !p->ready_ && !p->absorbed_ && p->op_w_ && !p->op_ids_ && !needed_by_caller(wanted, p) && n_readers[p] == 1;
+            };
+            if (gate == up || !pending_product(gate) || !pending_product(up) || gate->op_x_ != up->op_x_ ||
+                gate->op_w_->shape_ != up->op_w_->shape_)
+                continue;
+            pair_of[gate] = pair_of[up] = n.get();
+            const Tensor *x = gate->op_x_.get();
+            if (x->prod_ && x->prod_ != MI_QMM_PRODUCE_RMSNORM) needed.insert(x);  // only a norm runs inside the paired launch
+        }
         for (auto &node : nodes_) {
             Tensor *t = node.get();
-            if (t->ready_) continue;
+            if (t->ready_ || t->absorbed_) continue;
+            if (pair_of.count(t)) {
+                Tensor *silu = pair_of[t], *gate = silu->prod_src_.get(), *up = silu->prod_aux_.get();
+                Tensor *x = gate->op_x_.get();
+                const bool norm = !x->ready_ && x->prod_ == MI_QMM_PRODUCE_RMSNORM;
+                const Tensor &src = norm ? *x->prod_src_ : *x;
+                const int64_t k = src.Dim(0), n = (int64_t)src.Floats().size() / k;
+                silu->data_.assign((size_t)(n * gate->Dim(0)), 0.f);
+                check(mi_qmm_mulmat_swiglu(b_.handle(), gate->op_w_->weight_, up->op_w_->weight_,
+                                           norm ? MI_QMM_PRODUCE_RMSNORM : MI_QMM_PRODUCE_NONE,
+                                           norm && x->prod_aux_ ? x->prod_aux_->Floats().data() : nullptr, norm ? x->prod_eps_ : 0.f,
+                                           src.data_.data(), n, silu->data_.data(), MI_QMM_HOST));
+                silu->ready_ = true;
+                gate->absorbed_ = up->absorbed_ = true;
+                continue;
+            }
             if (t->prod_) {
                 if (!needed.count(t)) continue;
                 const Tensor &src = *t->prod_src_;
@@ -245,7 +288,7 @@ public:
             const Tensor &src = fused ? *x->prod_src_ : *x;
             const int64_t k = src.Dim(0), n = (int64_t)src.Floats().size() / k;
             for (auto &u : nodes_)
-                if (!u->ready_ && !u->prod_ && !u->op_ids_ && u->op_x_.get() == x &&
+                if (!u->ready_ && !u->absorbed_ && !pair_of.count(u.get()) && !u->prod_ && !u->op_ids_ && u->op_x_.get() == x &&
                     (fused || n > 8 || u->op_w_->type_ == t->op_w_->type_))  // decode launches hold one weight type
                     group.push_back(u.get());
             for (Tensor *u : group) u->data_.assign((size_t)(n * u->Dim(0)), 0.f);
@@ -289,6 +332,11 @@ public:
 
 private:
     friend class Tensor;
+    static bool needed_by_caller(const std::vector<std::shared_ptr<Tensor>> &wanted, const Tensor *p) {
+        for (auto &t : wanted)
+            if (t.get() == p) return true;
+        return false;
+    }
     Backend &b_;
     std::vector<std::shared_ptr<Tensor>> nodes_;
 };

@@ -14,7 +14,9 @@ Everything that computes goes through the C ABI (``ollama_amd.qmm``).  Compute g
 nodes of a graph by the ``x`` they read: decode-sized ones (N <= 8) of the same weight type run as one
 multi-tensor launch that quantizes ``x`` in its prologue; larger ones share one quantization of ``x``.
 An RMSNorm or SILU(up) node that only products read is never materialized: it becomes the producer of
-those products' activations (``mi_qmm_mulmat_produced``).
+those products' activations (``mi_qmm_mulmat_produced``).  ``gate.SILU(ctx, up)`` on two products of one
+``x`` that nothing else reads runs as one call (``mi_qmm_mulmat_swiglu``) and the two products are never
+materialized either.
 """
 from __future__ import annotations
 
@@ -52,6 +54,7 @@ class Tensor:
         self._op: Optional[Tuple["Tensor", "Tensor"]] = None  # (W, x) of a pending Mulmat
         self._ids: Optional["Tensor"] = None             # third operand of a pending MulmatID
         self._prod: Optional[Tuple[int, "Tensor", Optional["Tensor"], float]] = None  # pending RMSNorm / SILU(up)
+        self._absorbed = False                           # a product computed inside the SILU node that reads it
 
     # -- shape queries, /root/reference/ml/backend.go:131-135
     def Dim(self, n: int) -> int:
@@ -145,6 +148,10 @@ class Tensor:
         return out
 
 
+def tensors_ids(tensors) -> set:
+    return {id(t) for t in tensors}
+
+
 class Context:
     """Holds the tensors of one graph; Compute runs the pending Mulmat nodes."""
 
@@ -177,13 +184,32 @@ class Context:
         materialized only when asked for here or read by something other than a Mulmat."""
         if self._closed:
             raise RuntimeError("Compute on a closed context")
-        pending = [t for t in self._nodes if t._data is None and (t._op is not None or t._prod is not None)]
+        pending = [t for t in self._nodes if t._data is None and not t._absorbed and (t._op is not None or t._prod is not None)]
         c = self._b._ctx
         # producer nodes that must exist as f32: requested, or read by another producer
         needed = {id(t) for t in tensors}
+        readers: Dict[int, List[Tensor]] = {}
         for t in pending:
+            srcs = [s for s in (t._prod[1], t._prod[2]) if s is not None] if t._prod is not None else [t._op[1]]
             if t._prod is not None:
-                needed.update(id(s) for s in (t._prod[1], t._prod[2]) if s is not None)
+                needed.update(id(s) for s in srcs)
+            for s in srcs:
+                readers.setdefault(id(s), []).append(t)
+        # gate.SILU(up) on two pending products of one x that nothing else reads: one call computes the gated
+        # result, the two products are never materialized
+        pair_of: Dict[int, Tensor] = {}
+        for t in pending:
+            if t._prod is None or t._prod[0] != qmm.PRODUCE_SWIGLU:
+                continue
+            gate, up = t._prod[1], t._prod[2]
+            if (gate in pending and up in pending and gate is not up and gate._op is not None and up._op is not None
+                    and gate._ids is None and up._ids is None and gate._op[1] is up._op[1]
+                    and gate._op[0].Shape() == up._op[0].Shape() and id(gate) not in tensors_ids(tensors)
+                    and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]):
+                pair_of[id(gate)] = pair_of[id(up)] = t
+                x = gate._op[1]
+                if x._prod is not None and x._prod[0] != qmm.PRODUCE_RMSNORM:
+                    needed.add(id(x))  # only a norm runs inside the paired launch
 
         def rows(t: Tensor) -> np.ndarray:
             return t.Floats().reshape(-1, t.Dim(0))
@@ -200,6 +226,20 @@ class Context:
                         t._data = c.swiglu(rows(src), rows(aux)).reshape(-1)
                 continue
             x = t._op[1]
+            if t._absorbed:
+                continue
+            if id(t) in pair_of:
+                silu = pair_of[id(t)]
+                gate, up = silu._prod[1], silu._prod[2]
+                if x._data is None and x._prod is not None and x._prod[0] == qmm.PRODUCE_RMSNORM:
+                    _, src, aux, eps = x._prod  # the norm in front of gate and up runs in the same launch
+                    h = c.mulmat_swiglu(gate._op[0]._weight, up._op[0]._weight, rows(src), qmm.PRODUCE_RMSNORM,
+                                        None if aux is None else aux.Floats(), eps)
+                else:
+                    h = c.mulmat_swiglu(gate._op[0]._weight, up._op[0]._weight, rows(x))
+                silu._data = h.reshape(-1)
+                gate._absorbed = up._absorbed = True
+                continue
             if t._ids is not None:
                 # expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
                 ids = t._ids
@@ -219,7 +259,8 @@ class Context:
                 for u, y in zip(nodes, ys):
                     u._data = y.reshape(-1)  # [tokens][n_used][m] row-major == ggml [M, n_used, T]
                 continue
-            nodes = [u for u in pending if u._data is None and u._ids is None and u._op is not None and u._op[1] is x]
+            nodes = [u for u in pending if u._data is None and u._ids is None and u._op is not None and u._op[1] is x
+                     and id(u) not in pair_of]
             if x._data is None and x._prod is not None:
                 # x is a producer nobody needs in f32: it runs inside the products' own quantization
                 kind, src, aux, eps = x._prod

@@ -27,7 +27,7 @@ EXPORTS = [
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
-    "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_rms_norm", "mi_qmm_swiglu",
+    "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_mulmat_swiglu", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
     "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
@@ -91,6 +91,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_produced.argtypes = [vp, ctypes.POINTER(vp), ci, ci, vp, ctypes.c_float, vp, i64, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_id_produced.restype = ci
     L.mi_qmm_mulmat_id_produced.argtypes = [vp, vp, ci, ci, vp, ctypes.c_float, vp, ci, vp, ci, i64, vp, ci]
+    L.mi_qmm_mulmat_swiglu.restype = ci
+    L.mi_qmm_mulmat_swiglu.argtypes = [vp, vp, vp, ci, vp, ctypes.c_float, vp, i64, vp, ci]
     L.mi_qmm_rms_norm.restype = ci; L.mi_qmm_rms_norm.argtypes = [vp, vp, vp, ctypes.c_float, i64, i64, vp, ci]
     L.mi_qmm_swiglu.restype = ci; L.mi_qmm_swiglu.argtypes = [vp, vp, vp, i64, i64, vp, ci]
     L.mi_qmm_host_alloc.restype = vp; L.mi_qmm_host_alloc.argtypes = [vp, ctypes.c_size_t]
@@ -367,6 +369,30 @@ class Context:
         _check(lib().mi_qmm_mulmat_produced(self._h, wh, len(ws), producer,
                                             ctypes.c_void_p(int(aux_ptr)) if aux_ptr else None, eps,
                                             ctypes.c_void_p(int(x_ptr)), n, yp, DEVICE))
+
+    def mulmat_swiglu(self, w_gate: Weight, w_up: Weight, x: np.ndarray, producer: int = PRODUCE_NONE, aux=None,
+                      eps: float = 0.0) -> np.ndarray:
+        """silu(w_gate . Q8(x')) * (w_up . Q8(x')) with x' = x or RMSNorm(x) (aux = norm weight or None)"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        n, k = x.shape
+        if w_gate.k != k or w_up.k != k:
+            raise ValueError(f"x has k={k}, weights have k={w_gate.k}, {w_up.k}")
+        if aux is not None:
+            aux = np.ascontiguousarray(aux, dtype=np.float32)
+            if aux.shape != (k,):
+                raise ValueError(f"aux has shape {aux.shape}, x has k={k}")
+        h = np.empty((n, w_gate.m), dtype=np.float32)
+        _check(lib().mi_qmm_mulmat_swiglu(self._h, w_gate._h, w_up._h, producer, _ptr(aux) if aux is not None else None,
+                                          eps, _ptr(x), n, _ptr(h), HOST))
+        return h
+
+    def mulmat_swiglu_device(self, w_gate: Weight, w_up: Weight, x_ptr: int, n: int, h_ptr: int,
+                             producer: int = PRODUCE_NONE, aux_ptr=None, eps: float = 0.0):
+        _check(lib().mi_qmm_mulmat_swiglu(self._h, w_gate._h, w_up._h, producer,
+                                          ctypes.c_void_p(int(aux_ptr)) if aux_ptr else None, eps,
+                                          ctypes.c_void_p(int(x_ptr)), n, ctypes.c_void_p(int(h_ptr)), DEVICE))
 
     def rms_norm(self, x: np.ndarray, g, eps: float) -> np.ndarray:
         """(x / sqrt(mean(x^2) + eps)) * g per row; g f32 [k] or None"""

@@ -93,20 +93,20 @@ def test_python_mirror_ffn_block_with_producers():
         act = gate.SILU(ctx, up)
         out = b.Get("blk.0.ffn_down.weight").Mulmat(ctx, act)
         ctx.Compute(out)
-        with pytest.raises(RuntimeError):
-            h.Floats()   # never materialized: it ran inside the quantization of gate / up
+        for lazy in (h, gate, up):
+            with pytest.raises(RuntimeError):
+                lazy.Floats()   # never materialized: norm, both products and the gating were one call
         hv = oracle.rms_norm(xv, g, 1e-5)
         gv = oracle.mul_mat(qmm.Q4_K, raws["blk.0.ffn_gate.weight"], k, f, hv, nthreads=8)
         uv = oracle.mul_mat(qmm.Q4_K, raws["blk.0.ffn_up.weight"], k, f, hv, nthreads=8)
-        assert npref.rel_err(gate.Floats().reshape(n, f), gv) <= 1e-3
-        # the oracle's down projection on the GPU's own gate / up values: isolates the last step
-        want = oracle.mul_mat(qmm.Q6_K, raws["blk.0.ffn_down.weight"], f, k,
-                              oracle.swiglu(gate.Floats().reshape(n, f), up.Floats().reshape(n, f)), nthreads=8)
+        assert npref.rel_err(act.Floats().reshape(n, f), oracle.swiglu(gv, uv)) <= 1e-3
+        # the oracle's down projection on the GPU's own gated values: isolates the last step
+        want = oracle.mul_mat(qmm.Q6_K, raws["blk.0.ffn_down.weight"], f, k, act.Floats().reshape(n, f), nthreads=8)
         assert npref.rel_err(out.Floats().reshape(n, k), want) <= 1e-3, n
         # and the whole chain on the CPU
         chain = oracle.mul_mat(qmm.Q6_K, raws["blk.0.ffn_down.weight"], f, k, oracle.swiglu(gv, uv), nthreads=8)
         assert npref.rel_err(out.Floats().reshape(n, k), chain) <= 2e-3, n
-        # asking for the intermediate values gives the same result through the unfused kernels
+        # asking for the intermediate values gives the same result through the separate kernels
         ctx2 = b.NewContext()
         x2 = ctx2.FromFloats(xv.reshape(-1), k, n)
         h2 = x2.RMSNorm(ctx2, b.Get("blk.0.ffn_norm.weight"), 1e-5)
@@ -114,9 +114,20 @@ def test_python_mirror_ffn_block_with_producers():
         up2 = b.Get("blk.0.ffn_up.weight").Mulmat(ctx2, h2)
         act2 = gate2.SILU(ctx2, up2)
         out2 = b.Get("blk.0.ffn_down.weight").Mulmat(ctx2, act2)
-        ctx2.Compute(h2, act2, out2)
+        ctx2.Compute(h2, gate2, act2, out2)
         assert h2.Shape() == [k, n] and np.max(np.abs(h2.Floats().reshape(n, k) - hv)) < 1e-5
-        assert np.array_equal(out2.Floats(), out.Floats())
+        assert npref.rel_err(gate2.Floats().reshape(n, f), gv) <= 1e-3
+        assert np.array_equal(act2.Floats(), act.Floats()) and np.array_equal(out2.Floats(), out.Floats())
+        # down reads the gating node alone (no gate / up pair to absorb): the gating runs inside its quantization
+        ctx3 = b.NewContext()
+        ga, ua = ctx3.FromFloats(gate2.Floats(), f, n), ctx3.FromFloats(up2.Floats(), f, n)
+        a3 = ga.SILU(ctx3, ua)
+        out3 = b.Get("blk.0.ffn_down.weight").Mulmat(ctx3, a3)
+        ctx3.Compute(out3)
+        with pytest.raises(RuntimeError):
+            a3.Floats()
+        assert np.array_equal(out3.Floats(), out.Floats())
+        ctx3.Close()
         ctx.Close(); ctx2.Close()
     ctx = b.NewContext()
     with pytest.raises(TypeError):

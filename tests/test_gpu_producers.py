@@ -258,3 +258,58 @@ def test_expert_product_behind_rms_norm_and_errors(ctx):
     assert e.value.code == qmm.ERR_INVALID
     assert np.array_equal(ctx.mulmat_id_produced(w, n_expert, qmm.PRODUCE_NONE, None, x, ids), ctx.mulmat_id(w, n_expert, x, ids))
     w.free()
+
+
+# gate and up in one pass with the gating in the epilogue: rows of one K segment, of several (partials through
+# LDS), short rows that go two and four to a load, ragged row counts; batches take the products and the gating
+# kernel.  Always the bits of the separate calls.
+@pytest.mark.parametrize("t,k,m", [(Q4_K, 4096, 300), (Q4_K, 4096, 14336), (Q4_K, 2048, 129), (Q4_K, 1024, 77), (Q4_K, 8192, 65),
+                                   (Q4_K, 14336, 31), (Q6_K, 4096, 200), (Q6_K, 1280, 33), (Q4_0, 4096, 128), (Q4_0, 512, 19),
+                                   (Q8_0, 1024, 70), (Q8_0, 4128, 45), (Q8_0, 256, 7), (Q4_K, 256, 1)])
+@pytest.mark.parametrize("rms", [False, True])
+def test_gate_and_up_with_the_gating_in_the_epilogue(ctx, t, k, m, rms):
+    rng = np.random.default_rng(t * 100 + k + m)
+    wbg, wbu = _weights(t, m, k, 7000 + k + m), _weights(t, m, k, 7001 + k + m)
+    wg, wu = ctx.upload(t, wbg, k, m), ctx.upload(t, wbu, k, m)
+    g = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32) if rms else None
+    producer = qmm.PRODUCE_RMSNORM if rms else qmm.PRODUCE_NONE
+    for n in (1, 3, 40):
+        if n > 1 and m > 1000:
+            continue
+        x = (rng.standard_normal((n, k)) * 3).astype(np.float32)
+        h = ctx.mulmat_swiglu(wg, wu, x, producer, g, eps=1e-5)
+        xn = oracle.rms_norm(x, g, 1e-5) if rms else x
+        want = oracle.swiglu(oracle.mul_mat(t, wbg, k, m, xn, nthreads=16), oracle.mul_mat(t, wbu, k, m, xn, nthreads=16))
+        assert h.shape == (n, m) and npref.rel_err(h, want) < TOL, n
+        yg, yu = ctx.mulmat_produced([wg, wu], producer, g, x, eps=1e-5) if rms else ctx.mulmat_multi([wg, wu], x)
+        assert np.array_equal(h, ctx.swiglu(yg, yu)), n
+    wg.free(); wu.free()
+
+
+def test_mulmat_swiglu_errors_and_device_pointers(ctx):
+    k, m = 512, 40
+    wg, wu = ctx.upload(Q4_K, _weights(Q4_K, m, k, 1), k, m), ctx.upload(Q4_K, _weights(Q4_K, m, k, 2), k, m)
+    w3 = ctx.upload(Q4_K, _weights(Q4_K, m + 1, k, 3), k, m + 1)
+    w6 = ctx.upload(Q6_K, _weights(Q6_K, m, k, 4), k, m)
+    x = np.random.default_rng(5).standard_normal((1, k)).astype(np.float32)
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_swiglu(wg, w3, x)
+    assert e.value.code == qmm.ERR_INVALID
+    with pytest.raises(qmm.QmmError) as e:
+        ctx.mulmat_swiglu(wg, wu, x, qmm.PRODUCE_SWIGLU, None)
+    assert e.value.code == qmm.ERR_INVALID
+    # gate and up of different types: the products and the gating kernel
+    h = ctx.mulmat_swiglu(wg, w6, x)
+    yg, yu = ctx.mulmat_multi([wg, w6], x)
+    assert np.array_equal(h, ctx.swiglu(yg, yu))
+    assert ctx.mulmat_swiglu(wg, wu, np.zeros((0, k), np.float32)).shape == (0, m)
+    want = ctx.mulmat_swiglu(wg, wu, x)
+    for n in (1, 2):
+        xs = np.repeat(x, n, axis=0)
+        dx, dh = DeviceArray(xs), DeviceArray(np.zeros((n, m), np.float32), zero=True)
+        ctx.mulmat_swiglu_device(wg, wu, dx.ptr, n, dh.ptr)
+        ctx.sync()
+        assert np.array_equal(dh.numpy(), np.repeat(want, n, axis=0))
+        dx.free(); dh.free()
+    for w in (wg, wu, w3, w6):
+        w.free()
