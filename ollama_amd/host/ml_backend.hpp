@@ -219,6 +219,9 @@ public:
             if (gate == up || !pending_product(gate) || !pending_product(up) || gate->op_x_ != up->op_x_ ||
                 gate->op_w_->shape_ != up->op_w_->shape_)
                 continue;
+            int64_t rows = 1;  // one activation row: the single-launch form; with more rows the gating is better
+            for (size_t i = 1; i < gate->op_x_->shape_.size(); i++) rows *= gate->op_x_->shape_[i];  // placed in its reader's quantization
+            if (rows != 1) continue;
             pair_of[gate] = pair_of[up] = n.get();
             const Tensor *x = gate->op_x_.get();
             if (x->prod_ && x->prod_ != MI_QMM_PRODUCE_RMSNORM) needed.insert(x);  // only a norm runs inside the paired launch

@@ -195,8 +195,9 @@ class Context:
                 needed.update(id(s) for s in srcs)
             for s in srcs:
                 readers.setdefault(id(s), []).append(t)
-        # gate.SILU(up) on two pending products of one x that nothing else reads: one call computes the gated
-        # result, the two products are never materialized
+        # gate.SILU(up) on two pending products of one x that nothing else reads, at one activation row: one call
+        # computes the gated result, the two products are never materialized.  (With more rows the gating is
+        # better placed in the quantization of whatever reads it: the gated values then never exist in f32.)
         pair_of: Dict[int, Tensor] = {}
         for t in pending:
             if t._prod is None or t._prod[0] != qmm.PRODUCE_SWIGLU:
@@ -205,7 +206,8 @@ class Context:
             if (gate in pending and up in pending and gate is not up and gate._op is not None and up._op is not None
                     and gate._ids is None and up._ids is None and gate._op[1] is up._op[1]
                     and gate._op[0].Shape() == up._op[0].Shape() and id(gate) not in tensors_ids(tensors)
-                    and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]):
+                    and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]
+                    and int(np.prod(gate._op[1]._shape[1:], dtype=np.int64)) == 1):  # one row: the single-launch form
                 pair_of[id(gate)] = pair_of[id(up)] = t
                 x = gate._op[1]
                 if x._prod is not None and x._prod[0] != qmm.PRODUCE_RMSNORM:

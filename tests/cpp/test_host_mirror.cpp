@@ -213,7 +213,7 @@ int main() {
                     bool lazy = false, lazy_gate = false;
                     try { h->Floats(); } catch (const Error &) { lazy = true; }
                     try { gate->Floats(); } catch (const Error &) { lazy_gate = true; }
-                    if (lazy != (pass == 0) || lazy_gate != (pass == 0)) {
+                    if (lazy != (pass == 0) || lazy_gate != (pass == 0 && n == 1)) {  // one row: gate and up absorbed too
                         printf("FAIL: norm materialized=%d gate materialized=%d in pass %d\n", !lazy, !lazy_gate, pass);
                         failures++;
                     }
