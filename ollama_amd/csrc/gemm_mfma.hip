@@ -9,8 +9,9 @@
 //     elements, so there is no per-sub-block fix-up on the vector ALU.  The scaled weight does not fit
 //     int8, so it is split into two int8 "digit" planes and multiplied twice:
 //       Q4_K:  sc = 8*sh + sl  (sh, sl <= 7):  q*sh and q*sl <= 105;   sum sc*q*y = 8*A_h + A_l
-//       Q6_K:  p = sc*e (e = 0..63 unsigned 6-bit value, |p| <= 8064) = 64*p_h + p_l, p_l in 0..63,
-//              p_h in -126..126;                                      sum p*y    = 64*A_h + A_l
+//       Q6_K:  p = sc*e (e = 0..63 unsigned 6-bit value, |p| <= 8064) = 256*p_h + p_l in signed digits:
+//              p_l = the low byte of p read as int8, p_h = (p + 128) >> 8 in -31..31 -- bytes of the
+//              16-bit products, picked by byte permutes;            sum p*y    = 256*A_h + A_l
 //   * The terms that multiply sums of activations (Q4_K mins; the -32 offset of Q6_K) use the Q8_K
 //     block sums, also on the matrix cores: sum_j m_j * S_j with S split into two int8 digits
 //     (S = 64*S_h + S_l) costs two more MFMAs per 32x32 tile and super-block.
@@ -186,10 +187,12 @@ struct GemmQ6K {
                 const unsigned e = nib | (((hq[t] >> (2 * rr)) & 0x03030303u) << 4);  // 0..63 per byte
                 const s2 pe = as_s2(e & 0x00ff00ffu) * scv2;         // elements 0 and 2, 16-bit products
                 const s2 po = as_s2((e >> 8) & 0x00ff00ffu) * scv2;  // elements 1 and 3
-                const unsigned le = as_u(pe) & 0x003f003fu, lo_ = as_u(po) & 0x003f003fu;
-                const unsigned he = as_u(pe >> 6), ho = as_u(po >> 6);  // arithmetic shift per 16-bit lane
-                bl[t] = (int)(le | (lo_ << 8));
-                bh[t] = (int)__builtin_amdgcn_perm(ho, he, 0x06020400u);  // bytes: he.b0, ho.b0, he.b2, ho.b2
+                // signed digits to base 256: the low byte of the product read as int8, and what is left,
+                // (product + 128) >> 8 -- the high byte after adding 128.  Digits are bytes: two permutes.
+                const s2 half = {128, 128};
+                const unsigned re = as_u(pe + half), ro = as_u(po + half);
+                bl[t] = (int)__builtin_amdgcn_perm(as_u(po), as_u(pe), 0x06020400u);  // bytes: pe.b0, po.b0, pe.b2, po.b2
+                bh[t] = (int)__builtin_amdgcn_perm(ro, re, 0x07030501u);              // bytes: re.b1, ro.b1, re.b3, ro.b3
             }
             b.hi[s] = bh;
             b.lo[s] = bl;
@@ -204,7 +207,7 @@ struct GemmQ6K {
         return __int_as_float(32 * ((xh << 6) + xl));  // kept as an integer: it joins the main sum exactly
     }
     static __device__ __forceinline__ float combine(float d, int ah, int al, float fm) {
-        return d * (float)((ah << 6) + al - __float_as_int(fm));
+        return d * (float)((ah << 8) + al - __float_as_int(fm));
     }
 };
 
