@@ -185,8 +185,8 @@ struct GemmQ6K {
             for (int t = 0; t < 4; t++) {
                 const unsigned nib = rr < 2 ? l[t] & 0x0f0f0f0fu : (l[t] >> 4) & 0x0f0f0f0fu;
                 const unsigned e = nib | (((hq[t] >> (2 * rr)) & 0x03030303u) << 4);  // 0..63 per byte
-                const s2 pe = as_s2(e & 0x00ff00ffu) * scv2;         // elements 0 and 2, 16-bit products
-                const s2 po = as_s2((e >> 8) & 0x00ff00ffu) * scv2;  // elements 1 and 3
+                const s2 pe = as_s2(e & 0x00ff00ffu) * scv2;                                 // elements 0 and 2, 16-bit products
+                const s2 po = as_s2(__builtin_amdgcn_perm(0u, e, 0x0c030c01u)) * scv2;       // elements 1 and 3
                 // signed digits to base 256: the low byte of the product read as int8, and what is left,
                 // (product + 128) >> 8 -- the high byte after adding 128.  Digits are bytes: two permutes.
                 const s2 half = {128, 128};
