@@ -89,6 +89,7 @@ __device__ __forceinline__ float reduce_rows(const float (&v)[U], int lane) {
 // ---------------------------------------------------------------------------------------------
 
 struct PolQ4K {
+    static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
     static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;  // Q8_K: one scale per 256, one sum per 16
     static constexpr bool USES_BSUMS = true;
@@ -176,6 +177,7 @@ struct PolQ4K {
 };
 
 struct PolQ4_0 {
+    static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 2048;  // 64 blocks, one per lane
     static constexpr int ACT_BLK = QK, ACT_BSUM = QK;  // Q8_0: one scale and one sum per 32
     static constexpr bool USES_BSUMS = true;
@@ -235,6 +237,7 @@ struct PolQ4_0 {
 };
 
 struct PolQ8_0 {
+    static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 1024;  // 32 blocks, two lanes (16 quants each) per block
     static constexpr int ACT_BLK = QK, ACT_BSUM = QK;
     static constexpr bool USES_BSUMS = false;
@@ -281,6 +284,7 @@ struct PolQ8_0 {
 };
 
 struct PolQ6K {
+    static constexpr int F32_WAVES_ONE_SEG = 8;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
     static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;  // Q8_K: one scale per 256, one sum per 16
     static constexpr bool USES_BSUMS = true;
@@ -924,7 +928,11 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
     if (nseg < 1 || nseg > 8) return false;
     p.spw = 1;
     p.kw = nseg;
-    const int max_waves = p.kw > thin_max_waves(nc, f32) ? p.kw : thin_max_waves(nc, f32);
+    // Q6_K needs 70-75 registers: a 16-wave workgroup then has a CU to itself (four waves per SIMD), three
+    // 8-wave ones share it (six per SIMD).  Measured with rows of one segment: 14336 x 4096 12.2 against
+    // 15.6 us; with several segments per row the larger workgroup wins (4096 x 14336: 13.5 against 18.0 us).
+    const int mwt = f32 && p.kw == 1 && nc == 1 ? P::F32_WAVES_ONE_SEG : thin_max_waves(nc, f32);
+    const int max_waves = p.kw > mwt ? p.kw : mwt;
     p.rw_log2 = 0;
     while (p.kw << (p.rw_log2 + 1) <= max_waves) p.rw_log2++;
     p.rw = 1 << p.rw_log2;
