@@ -816,3 +816,49 @@ def test_device_entry_points_replay_from_a_hip_graph():
         d.free()
     c.close()
     st.destroy()
+
+
+def test_calls_from_several_threads_each_with_its_own_ctx():
+    """A Go caller's goroutines migrate between OS threads and several runners may share a process: contexts
+    are independent (own stream, own scratch), a call re-asserts its device, and nothing but the error string is
+    thread-local.  Four threads, each with its own ctx and weights, mixed entry points, against results
+    computed beforehand on one thread."""
+    import threading
+
+    k, m, n_expert = 1024, 96, 4
+    rng = np.random.default_rng(41)
+    specs = []
+    main = qmm.Context(0)
+    for i, t in enumerate((Q4_K, Q6_K, Q8_0, Q4_0)):
+        wb = _weights(t, m, k, 4100 + i)
+        eb = _experts(t, n_expert, 32, k, 4200 + i)
+        xs = [rng.standard_normal((n, k), dtype=np.float32) for n in (1, 5, 40)]
+        ids = np.array([[1, 3]], np.int32)
+        w, e = main.upload(t, wb, k, m), main.upload(t, eb, k, n_expert * 32)
+        want = [main.mulmat(w, x) for x in xs] + [main.mulmat_id(e, n_expert, xs[0][None], ids)]
+        w.free(); e.free()
+        specs.append((t, wb, eb, xs, ids, want))
+    main.close()
+    errors = []
+
+    def worker(spec):
+        try:
+            t, wb, eb, xs, ids, want = spec
+            c = qmm.Context(0)
+            w, e = c.upload(t, wb, k, m), c.upload(t, eb, k, n_expert * 32)
+            for _ in range(20):
+                got = [c.mulmat(w, x) for x in xs] + [c.mulmat_id(e, n_expert, xs[0][None], ids)]
+                for a, b in zip(got, want):
+                    if not np.array_equal(a, b):
+                        raise AssertionError(f"type {t}: a result changed under concurrency")
+            w.free(); e.free()
+            c.close()
+        except Exception as ex:  # noqa: BLE001 - reported to the main thread
+            errors.append(repr(ex))
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in specs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors and not any(th.is_alive() for th in threads), errors
