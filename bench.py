@@ -46,6 +46,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the pure-read ceiling measurement")
     ap.add_argument("--layers", type=int, default=32, help="distinct FFN weight sets in the rotating pool")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the batch-512 prefill GEMM section")
@@ -173,6 +174,39 @@ def main() -> int:
             "bytes_per_launch": int(bytes_per_launch),
         },
     }
+
+    # ---- what a pure read of the same bytes reaches in one launch on this machine (launch included): the
+    # practical ceiling next to the GEMV's figure.  Best of a few grid shapes, rotating buffers like the weights.
+    sr_path = os.path.join(os.path.dirname(qmm.LIB_PATH), "libmi_streamread.so")
+    if os.path.exists(sr_path) and not args.no_ceiling:
+        sr = ctypes.CDLL(sr_path)
+        sr.mi_stream_read.restype = ctypes.c_int
+        sr.mi_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                      ctypes.c_void_p]
+        nbytes = bytes_per_launch // 16 * 16
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(16)]
+        scratch = torch.zeros(8192, dtype=torch.int32, device=dev)
+        best = None
+        for threads in (256, 1024):
+            for blocks in (256, 512, 1024, 2048, 4096, 8192):
+                for unroll in (1, 2, 4, 8):
+                    if blocks * threads > 4096 * 1024 // 2:
+                        continue
+                    fn = lambda: [sr.mi_stream_read(b.data_ptr(), nbytes, blocks, threads, unroll, scratch.data_ptr(),
+                                                    stream.cuda_stream) for b in bufs]
+                    fn()
+                    tm = timed(fn, 3) / (3 * len(bufs))
+                    if os.environ.get("CEIL_VERBOSE"):
+                        print(f"read {threads}x{blocks} unroll {unroll}: {tm * 1e6:.2f} us", file=sys.stderr)
+                    if best is None or tm < best[0]:
+                        best = (tm, blocks, unroll, threads)
+        ceil_gbs = nbytes / best[0] / 1e9
+        out["read_ceiling"] = {"bytes": nbytes, "us": round(best[0] * 1e6, 2), "GB/s": round(ceil_gbs, 1),
+                               "frac_of_hbm_peak": round(ceil_gbs / HBM_PEAK_GBS, 4),
+                               "grid": f"{best[1]} workgroups of {best[3]}, {best[2]} loads of 16 bytes in flight per lane",
+                               "what": "one launch that only reads the gate+up launch's bytes, back to back over rotating buffers"}
+        out["roofline"]["frac_of_read_ceiling"] = round(achieved / ceil_gbs, 4)
+        del bufs
 
     # ---- prefill GEMM: one Llama-3-8B-shaped layer at batch 512 (secondary metric of BASELINE.json)
     if not args.no_gemm:
