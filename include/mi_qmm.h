@@ -201,6 +201,15 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
 int mi_qmm_mulmat_id_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, int n_expert,
                            const float *x, int b_cols, const int32_t *ids, int n_used, int64_t n_tokens,
                            float *const *ys, int location);
+/* Gate and up of an EXPERT feed-forward block with their gating: mi_qmm_mulmat_swiglu for expert stacks,
+ *     h[t][i][:] = silu(Wg[ids[t][i]] * Q8(x[t][i % b_cols])) * (Wu[ids[t][i]] * Q8(x[t][i % b_cols])),
+ * h f32 [n_tokens][n_used][rows_per_expert]; arguments as for mi_qmm_mulmat_id.  Decode-sized calls are one
+ * launch (a wave walks row j of the pair's expert in both stacks and gates the two totals); larger ones
+ * the two products and mi_qmm_swiglu.  Bit-identical to those either way. */
+int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_qmm_weight *w_up, int n_expert,
+                            const float *x, int b_cols, const int32_t *ids, int n_used, int64_t n_tokens, float *h,
+                            int location);
+
 /* mi_qmm_mulmat_id on x' = producer(x) (the producers of mi_qmm_mulmat_produced): the down projection of
  * an expert feed-forward block reads silu(gate) * up, x = gate and aux = up being the two
  * [n_tokens][b_cols][k] results of the gate / up stacks.  Decode-sized calls gate and quantize each

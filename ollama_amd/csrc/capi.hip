@@ -50,6 +50,7 @@ struct mi_qmm_ctx {
     void *act_buf = nullptr;  size_t act_cap = 0;
     void *io_buf = nullptr;   size_t io_cap = 0;
     void *ws_buf = nullptr;   size_t ws_cap = 0;   // partial sums of a K-split GEMM
+    void *pair_buf = nullptr; size_t pair_cap = 0; // the two products of a gated pair when they are not one launch
 };
 
 struct mi_qmm_weight {
@@ -228,6 +229,7 @@ void mi_qmm_destroy(mi_qmm_ctx *ctx) {
         if (ctx->act_buf) (void)hipFree(ctx->act_buf);
         if (ctx->io_buf) (void)hipFree(ctx->io_buf);
         if (ctx->ws_buf) (void)hipFree(ctx->ws_buf);
+        if (ctx->pair_buf) (void)hipFree(ctx->pair_buf);
         if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
     }
     delete ctx;
@@ -947,6 +949,81 @@ int mi_qmm_mulmat_id_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_exp
         return fail(MI_QMM_ERR_INVALID, "unknown producer %d", producer);
     const Produce pr{producer, producer == MI_QMM_PRODUCE_NONE ? nullptr : aux, eps, nullptr};
     return mulmat_id_impl(ctx, w, nullptr, n_expert, x, b_cols, ids, n_used, n_tokens, y, nullptr, location, &pr);
+}
+
+int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_qmm_weight *w_up, int n_expert,
+                            const float *x, int b_cols, const int32_t *ids, int n_used, int64_t n_tokens, float *h,
+                            int location) {
+    if (!w_gate || !w_up) return fail(MI_QMM_ERR_INVALID, "w_gate or w_up is NULL");
+    int rc = check_product_args(ctx, w_gate, location, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    if (w_up->device != ctx->device || w_up->dev.K != w_gate->dev.K || w_up->dev.M != w_gate->dev.M)
+        return fail(MI_QMM_ERR_INVALID, "the gate and up stacks differ in device or shape");
+    if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
+        return fail(MI_QMM_ERR_INVALID, "n_expert=%d n_used=%d b_cols=%d n_tokens=%lld: all must be positive", n_expert,
+                    n_used, b_cols, (long long)n_tokens);
+    const int64_t K = w_gate->dev.K;
+    if (w_gate->dev.M % n_expert)
+        return fail(MI_QMM_ERR_INVALID, "the weight has %lld rows, not a multiple of n_expert=%d", (long long)w_gate->dev.M,
+                    n_expert);
+    const int64_t M = w_gate->dev.M / n_expert;
+    if (n_tokens == 0) return MI_QMM_OK;
+    if (!x || !ids || !h) return fail(MI_QMM_ERR_INVALID, "x, ids or h is NULL");
+    const int64_t pairs = (int64_t)n_used * n_tokens, ncols = (int64_t)b_cols * n_tokens;
+    if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24) || K > gemv_max_k(w_gate->dev.type))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts, 2^24 pairs and k <= %lld for type %d",
+                    (long long)gemv_max_k(w_gate->dev.type), w_gate->dev.type);
+    if (location == MI_QMM_HOST)
+        for (int64_t p = 0; p < pairs; p++)
+            if (ids[p] < 0 || ids[p] >= n_expert)
+                return fail(MI_QMM_ERR_INVALID, "ids[%lld] = %d is outside 0..%d", (long long)p, ids[p], n_expert - 1);
+    // decode-sized and both stacks of one type: one launch with the gating in its epilogue; else the two products
+    // (which share their quantization and, at decode size, their launch) and the gating kernel
+    const bool paired = w_gate->dev.type == w_up->dev.type && gemv_id_f32_supported(w_gate->dev.type, K, 2 * M, pairs, n_expert);
+    const size_t hbytes = (size_t)(pairs * M) * 4;
+    const size_t bytes[5] = {(size_t)(ncols * K) * 4, (size_t)pairs * 4, hbytes, paired ? 0 : hbytes, paired ? 0 : hbytes};
+    const void *src[5] = {x, ids, h, nullptr, nullptr};
+    void *d[5];
+    if (paired) {
+        if ((rc = stage_in(ctx, location, src, bytes, 2, 5, d))) return rc;
+        HIP_TRY(launch_gemv_id_pair(w_gate->dev, w_up->dev, n_expert, (const float *)d[0], (const int *)d[1], n_used,
+                                    (int)n_tokens, b_cols, (float *)d[2], ctx->stream));
+        if (location == MI_QMM_HOST) {
+            HIP_TRY(hipMemcpyAsync(h, d[2], hbytes, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(hipStreamSynchronize(ctx->stream));
+        }
+        return MI_QMM_OK;
+    }
+    // the two products into scratch of their own (mulmat_id_impl stages host operands through io_buf itself)
+    if ((rc = reserve(&ctx->pair_buf, &ctx->pair_cap, 3 * align_up(hbytes, 256), ctx->stream))) return rc;
+    float *yg = (float *)ctx->pair_buf, *yu = (float *)((char *)ctx->pair_buf + align_up(hbytes, 256));
+    float *dh = location == MI_QMM_HOST ? (float *)((char *)ctx->pair_buf + 2 * align_up(hbytes, 256)) : h;
+    const bool same = w_gate->dev.type == w_up->dev.type;
+    if (location == MI_QMM_HOST) {
+        // host operands: the products return host arrays; keep them on the device instead by staging here
+        if ((rc = stage_in(ctx, location, src, bytes, 2, 2, d))) return rc;
+        // io_buf now holds x and ids; mulmat_id_impl with device pointers does not touch io_buf
+    } else {
+        d[0] = const_cast<float *>(x); d[1] = const_cast<int32_t *>(ids);
+    }
+    if (same) {
+        if ((rc = mulmat_id_impl(ctx, w_gate, w_up, n_expert, (const float *)d[0], b_cols, (const int32_t *)d[1], n_used, n_tokens,
+                                 yg, yu, MI_QMM_DEVICE)))
+            return rc;
+    } else {
+        if ((rc = mulmat_id_impl(ctx, w_gate, nullptr, n_expert, (const float *)d[0], b_cols, (const int32_t *)d[1], n_used,
+                                 n_tokens, yg, nullptr, MI_QMM_DEVICE)))
+            return rc;
+        if ((rc = mulmat_id_impl(ctx, w_up, nullptr, n_expert, (const float *)d[0], b_cols, (const int32_t *)d[1], n_used,
+                                 n_tokens, yu, nullptr, MI_QMM_DEVICE)))
+            return rc;
+    }
+    HIP_TRY(launch_swiglu(yg, yu, pairs * M, dh, ctx->stream));
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(h, dh, hbytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
 }
 
 // ---- two-phase form ----------------------------------------------------------------------------------

@@ -1565,6 +1565,100 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     }
 }
 
+// Gate and up of an expert feed-forward block at decode size with the gating in the epilogue (see
+// gemv_pair_kernel): one (token, slot) pair per group of workgroups, the wave walks row j of the pair's expert
+// in both stacks, h[pair][j] = silu(gate total) * up total.  ia.w / ia.p0b.. are the gate / up stacks, ia.y is h.
+template <class P, bool DIRECT, int RPL>
+__global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const float *__restrict__ xf, int rows_per_wave, int kw,
+                                                           int rw_log2) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const DevWeight wa{ia.w.p0, ia.w.p1, ia.w.p2, ia.w.d, ia.w.K, ia.w.M, ia.w.type};
+    const DevWeight wb{ia.p0b, ia.p1b, ia.p2b, ia.db, ia.w.K, ia.w.M, ia.w.type};
+    float *__restrict__ hout = ia.y;
+    const int pair = (int)blockIdx.x / ia.wgs_per_group, wg = (int)blockIdx.x - pair * ia.wgs_per_group;
+    int expert = ia.ids[pair];
+    if (expert < 0 || expert >= ia.n_expert) expert = -1;
+    const int64_t M = ia.M;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = 1 << rw_log2;
+    const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
+    const int rows_per_wg = rows_per_wave << rw_log2;  // rows of h per workgroup
+    const int64_t r0 = (int64_t)wg * rows_per_wg;
+    const int nrows = (int)min((int64_t)rows_per_wg, M - r0);
+    if (expert < 0) {
+        for (int i = threadIdx.x; i < nrows; i += blockDim.x) hout[(int64_t)pair * M + r0 + i] = __int_as_float(0x7fc00000);
+        return;
+    }
+    const int rl0 = rg * rows_per_wave;
+    const int nrw = max(0, min(rows_per_wave, nrows - rl0));
+    const int64_t wrow0 = (int64_t)expert * M + r0 + rl0;
+    const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);
+    const typename P::Geo g = P::geo(wa, kseg, vlane);
+    const int tok = pair / ia.n_used, slot = pair - tok * ia.n_used;
+    const int col = tok * ia.b_cols + slot % ia.b_cols;
+
+    const int64_t K = wa.K;
+    const int nblk = (int)(K / P::ACT_BLK);
+    const size_t act_bytes = ((size_t)(K + nblk * 4 + (P::USES_BSUMS ? K / P::ACT_BSUM * 2 : 0)) + 15) / 16 * 16;
+    int8_t *lqs = reinterpret_cast<int8_t *>(smem);
+    float *ld_ = reinterpret_cast<float *>(smem + K);
+    int16_t *lbs = reinterpret_cast<int16_t *>(smem + K + (size_t)nblk * 4);
+    const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col * K);
+    const int total4 = (int)(K / 4), nwaves = blockDim.x >> 6;
+    float4 xpre[XPRE];
+    prefetch_x(x4, total4, wave, nwaves, lane, xpre);
+    typename P::Raw cur;
+    if (nrw > 0) {
+        const int v = min(run, 2 * nrw - 1);
+        cur = P::load(v & 1 ? wb : wa, g, wrow0 + (v >> 1));
+    }
+    quantize_x_to_lds<P, XPRE>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
+    __syncthreads();
+    float *part = reinterpret_cast<float *>(smem + act_bytes);
+    if (nrw > 0) {
+        typename P::Act act[1];
+        const LdsAct la{lqs, ld_, lbs, K};
+        P::load_act(la, 0, kseg, vlane, g, act[0]);
+        float keep;
+        thin_rows_pair<P, DIRECT, RPL>(wa, wb, g, cur, act, wrow0, 2 * nrw, lane, keep, part, 2 * rl0, kw, kseg);
+        if (DIRECT) {
+            const float up = dpp_mov<0xB1>(keep);
+            if ((lane & 1) && lane > 63 - 2 * nrw) hout[(int64_t)pair * M + r0 + rl0 + ((63 - lane) >> 1)] = silu_mul(keep, up);
+        }
+    }
+    if (DIRECT) return;
+    __syncthreads();
+    for (int i = threadIdx.x; i < nrows; i += blockDim.x) {
+        float gsum = 0.f, usum = 0.f;
+        for (int k = 0; k < kw; k++) gsum += part[(2 * i) * kw + k];
+        for (int k = 0; k < kw; k++) usum += part[(2 * i + 1) * kw + k];
+        hout[(int64_t)pair * M + r0 + i] = silu_mul(gsum, usum);
+    }
+}
+
+template <class P>
+hipError_t launch_id_pair(IdArgs ia, const float *xf, hipStream_t s) {
+    Plan p;
+    if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * 2, 1, false, p)) return hipErrorInvalidValue;
+    const size_t act_lds = thin_act_lds<P>(ia.w.K, 1);
+    const int rpw_v = p.rows_per_wg >> p.rw_log2;  // virtual rows per wave: row j of gate and of up alternate
+    if (act_lds + p.lds > THIN_LDS_MAX || (rpw_v & 1)) return hipErrorInvalidValue;
+    const int rows_per_wg = p.rows_per_wg / 2;
+    const int64_t wgs_per_group = (ia.M + rows_per_wg - 1) / rows_per_wg;
+    if (wgs_per_group * ia.pairs > 0x7fffffff) return hipErrorInvalidValue;
+    ia.wgs_per_group = (int)wgs_per_group;
+    ia.groups = nullptr;
+    const dim3 grid((unsigned)(wgs_per_group * ia.pairs)), block(64 * p.kw * p.rw);
+    const size_t lds = act_lds + p.lds;
+#define IDP_LAUNCH(DIRECT, RPL) gemv_id_pair_kernel<P, DIRECT, RPL><<<grid, block, lds, s>>>(ia, xf, rpw_v / 2, p.kw, p.rw_log2)
+    if (p.kw > 1) IDP_LAUNCH(false, 1);
+    else if (p.rpl == 4) IDP_LAUNCH(true, 4);
+    else if (p.rpl == 2) IDP_LAUNCH(true, 2);
+    else IDP_LAUNCH(true, 1);
+#undef IDP_LAUNCH
+    return hipGetLastError();
+}
+
 template <class P, int NC>
 hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, const float *up, int *groups, hipStream_t s) {
     Plan p;
@@ -1676,6 +1770,25 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
     // gated rows must sit in the waves' prefetch registers whole
     if (ok && swiglu && K > (int64_t)XPRE * p.kw * p.rw * 256) return false;
     return ok && act + p.lds <= THIN_LDS_MAX;
+}
+
+hipError_t launch_gemv_id_pair(const DevWeight &wg, const DevWeight &wu, int n_expert, const float *xf, const int *ids,
+                               int n_used, int n_tokens, int b_cols, float *h, hipStream_t s) {
+    if (wg.type != wu.type || wg.K != wu.K || wg.M != wu.M || n_expert < 1 || n_expert > ID_MAX_EXPERTS || wg.M % n_expert ||
+        n_used < 1 || n_tokens < 1 || b_cols < 1 || !ids || !h || !xf || (int64_t)n_used * n_tokens > 0x7fffffff / 16 ||
+        wg.K < 1 || wg.K > gemv_max_k(wg.type))
+        return hipErrorInvalidValue;
+    IdArgs ia{};
+    ia.w = wg; ia.ids = ids; ia.y = h; ia.M = wg.M / n_expert;
+    ia.n_expert = n_expert; ia.pairs = n_used * n_tokens; ia.n_used = n_used; ia.b_cols = b_cols;
+    ia.p0b = wu.p0; ia.p1b = wu.p1; ia.p2b = wu.p2; ia.db = wu.d; ia.yb = nullptr; ia.wgs_first = 0x7fffffff;
+    switch (wg.type) {
+    case T_Q4_K: return launch_id_pair<PolQ4K>(ia, xf, s);
+    case T_Q6_K: return launch_id_pair<PolQ6K>(ia, xf, s);
+    case T_Q4_0: return launch_id_pair<PolQ4_0>(ia, xf, s);
+    case T_Q8_0: return launch_id_pair<PolQ8_0>(ia, xf, s);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,

@@ -68,6 +68,10 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
 hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, const float *xf, const int *ids,
                           int n_used, int n_tokens, int b_cols, float *y, int *groups, hipStream_t s,
                           const DevWeight *w2 = nullptr, float *y2 = nullptr, const float *up = nullptr);
+// Gate and up stacks of an expert feed-forward block at decode size (ask gemv_id_f32_supported with twice the
+// rows) with the gating in the epilogue: h [n_tokens][n_used][M] = silu(gate product) * up product.
+hipError_t launch_gemv_id_pair(const DevWeight &wg, const DevWeight &wu, int n_expert, const float *xf, const int *ids,
+                               int n_used, int n_tokens, int b_cols, float *h, hipStream_t s);
 // buckets the pairs by expert into groups of at most nc (1..16) pairs: groups[0] = number of groups,
 // then records {expert or -1 for ids outside the stack, count, pair[nc]}
 hipError_t launch_group_pairs(const int *ids, int pairs, int n_expert, int nc, int *groups, hipStream_t s);

@@ -214,17 +214,21 @@ public:
             if (n->ready_ || n->prod_ != MI_QMM_PRODUCE_SWIGLU) continue;
             Tensor *gate = n->prod_src_.get(), *up = n->prod_aux_.get();
             auto pending_product = [&](const Tensor *p) {
-                return !p->ready_ && !p->absorbed_ && p->op_w_ && !p->op_ids_ && !needed_by_caller(wanted, p) && n_readers[p] == 1;
+                return !p->ready_ && !p->absorbed_ && p->op_w_ && !needed_by_caller(wanted, p) && n_readers[p] == 1;
             };
             if (gate == up || !pending_product(gate) || !pending_product(up) || gate->op_x_ != up->op_x_ ||
-                gate->op_w_->shape_ != up->op_w_->shape_)
+                gate->op_ids_ != up->op_ids_ || gate->op_w_->shape_ != up->op_w_->shape_)
                 continue;
-            int64_t rows = 1;  // one activation row: the single-launch form; with more rows the gating is better
-            for (size_t i = 1; i < gate->op_x_->shape_.size(); i++) rows *= gate->op_x_->shape_[i];  // placed in its reader's quantization
+            // one activation row (one token for expert stacks): the single-launch form; with more rows the gating
+            // is better placed in its reader's quantization
+            int64_t rows = 1;
+            if (gate->op_ids_) rows = gate->op_ids_->Dim(1);
+            else for (size_t i = 1; i < gate->op_x_->shape_.size(); i++) rows *= gate->op_x_->shape_[i];
             if (rows != 1) continue;
             pair_of[gate] = pair_of[up] = n.get();
             const Tensor *x = gate->op_x_.get();
-            if (x->prod_ && x->prod_ != MI_QMM_PRODUCE_RMSNORM) needed.insert(x);  // only a norm runs inside the paired launch
+            // only a norm in front of plain products runs inside the paired launch
+            if (x->prod_ && (x->prod_ != MI_QMM_PRODUCE_RMSNORM || gate->op_ids_)) needed.insert(x);
         }
         for (auto &node : nodes_) {
             Tensor *t = node.get();
@@ -232,6 +236,16 @@ public:
             if (pair_of.count(t)) {
                 Tensor *silu = pair_of[t], *gate = silu->prod_src_.get(), *up = silu->prod_aux_.get();
                 Tensor *x = gate->op_x_.get();
+                if (gate->op_ids_) {
+                    const Tensor &ids = *gate->op_ids_;
+                    silu->data_.assign((size_t)(gate->op_w_->Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);
+                    check(mi_qmm_mulmat_id_swiglu(b_.handle(), gate->op_w_->weight_, up->op_w_->weight_, gate->op_w_->Dim(2),
+                                                  x->Floats().data(), x->Dim(1), ids.ints_.data(), ids.Dim(0), ids.Dim(1),
+                                                  silu->data_.data(), MI_QMM_HOST));
+                    silu->ready_ = true;
+                    gate->absorbed_ = up->absorbed_ = true;
+                    continue;
+                }
                 const bool norm = !x->ready_ && x->prod_ == MI_QMM_PRODUCE_RMSNORM;
                 const Tensor &src = norm ? *x->prod_src_ : *x;
                 const int64_t k = src.Dim(0), n = (int64_t)src.Floats().size() / k;
@@ -266,7 +280,8 @@ public:
                 // expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
                 const Tensor &ids = *t->op_ids_;
                 for (auto &u : nodes_)
-                    if (!u->ready_ && u->op_ids_ == t->op_ids_ && u->op_x_.get() == x && u->op_w_->Dim(2) == t->op_w_->Dim(2))
+                    if (!u->ready_ && !u->absorbed_ && !pair_of.count(u.get()) && u->op_ids_ == t->op_ids_ && u->op_x_.get() == x &&
+                        u->op_w_->Dim(2) == t->op_w_->Dim(2))
                         group.push_back(u.get());
                 for (Tensor *u : group) {
                     u->data_.assign((size_t)(u->op_w_->Dim(1) * ids.Dim(0) * ids.Dim(1)), 0.f);

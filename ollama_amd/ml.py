@@ -203,15 +203,19 @@ class Context:
             if t._prod is None or t._prod[0] != qmm.PRODUCE_SWIGLU:
                 continue
             gate, up = t._prod[1], t._prod[2]
-            if (gate in pending and up in pending and gate is not up and gate._op is not None and up._op is not None
-                    and gate._ids is None and up._ids is None and gate._op[1] is up._op[1]
+            if not (gate in pending and up in pending and gate is not up and gate._op is not None and up._op is not None
+                    and gate._ids is up._ids and gate._op[1] is up._op[1]
                     and gate._op[0].Shape() == up._op[0].Shape() and id(gate) not in tensors_ids(tensors)
-                    and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]
-                    and int(np.prod(gate._op[1]._shape[1:], dtype=np.int64)) == 1):  # one row: the single-launch form
-                pair_of[id(gate)] = pair_of[id(up)] = t
-                x = gate._op[1]
-                if x._prod is not None and x._prod[0] != qmm.PRODUCE_RMSNORM:
-                    needed.add(id(x))  # only a norm runs inside the paired launch
+                    and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]):
+                continue
+            x = gate._op[1]
+            # one activation row (one token for expert stacks): the single-launch form
+            one = (gate._ids.Dim(1) if gate._ids is not None else int(np.prod(x._shape[1:], dtype=np.int64))) == 1
+            if not one:
+                continue
+            pair_of[id(gate)] = pair_of[id(up)] = t
+            if x._prod is not None and (x._prod[0] != qmm.PRODUCE_RMSNORM or gate._ids is not None):
+                needed.add(id(x))  # only a norm in front of plain products runs inside the paired launch
 
         def rows(t: Tensor) -> np.ndarray:
             return t.Floats().reshape(-1, t.Dim(0))
@@ -233,7 +237,12 @@ class Context:
             if id(t) in pair_of:
                 silu = pair_of[id(t)]
                 gate, up = silu._prod[1], silu._prod[2]
-                if x._data is None and x._prod is not None and x._prod[0] == qmm.PRODUCE_RMSNORM:
+                if gate._ids is not None:
+                    ids = gate._ids
+                    tokens, n_used = ids.Dim(1), ids.Dim(0)
+                    h = c.mulmat_id_swiglu(gate._op[0]._weight, up._op[0]._weight, gate._op[0].Dim(2),
+                                           x.Floats().reshape(tokens, x.Dim(1), x.Dim(0)), ids._data.reshape(tokens, n_used))
+                elif x._data is None and x._prod is not None and x._prod[0] == qmm.PRODUCE_RMSNORM:
                     _, src, aux, eps = x._prod  # the norm in front of gate and up runs in the same launch
                     h = c.mulmat_swiglu(gate._op[0]._weight, up._op[0]._weight, rows(src), qmm.PRODUCE_RMSNORM,
                                         None if aux is None else aux.Floats(), eps)
@@ -246,7 +255,7 @@ class Context:
                 # expert-indexed nodes that read the same x and ids (gate and up of an expert FFN) go out together
                 ids = t._ids
                 nodes = [u for u in pending if u._data is None and u._ids is ids and u._op[1] is x
-                         and u._op[0].Dim(2) == t._op[0].Dim(2)]
+                         and u._op[0].Dim(2) == t._op[0].Dim(2) and id(u) not in pair_of]
                 tokens, n_used = ids.Dim(1), ids.Dim(0)
                 idv = ids._data.reshape(tokens, n_used)
                 if x._data is None and x._prod is not None:

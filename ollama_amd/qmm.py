@@ -27,7 +27,7 @@ EXPORTS = [
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
     "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
-    "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_mulmat_swiglu", "mi_qmm_rms_norm", "mi_qmm_swiglu",
+    "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_mulmat_swiglu", "mi_qmm_mulmat_id_swiglu", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
     "mi_qmm_gguf_open", "mi_qmm_gguf_close", "mi_qmm_gguf_info", "mi_qmm_gguf_tensor", "mi_qmm_gguf_find_tensor",
     "mi_qmm_gguf_tensor_data", "mi_qmm_gguf_find_kv", "mi_qmm_gguf_kv", "mi_qmm_gguf_kv_int", "mi_qmm_gguf_kv_uint",
@@ -91,6 +91,8 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_mulmat_produced.argtypes = [vp, ctypes.POINTER(vp), ci, ci, vp, ctypes.c_float, vp, i64, ctypes.POINTER(vp), ci]
     L.mi_qmm_mulmat_id_produced.restype = ci
     L.mi_qmm_mulmat_id_produced.argtypes = [vp, vp, ci, ci, vp, ctypes.c_float, vp, ci, vp, ci, i64, vp, ci]
+    L.mi_qmm_mulmat_id_swiglu.restype = ci
+    L.mi_qmm_mulmat_id_swiglu.argtypes = [vp, vp, vp, ci, vp, ci, vp, ci, i64, vp, ci]
     L.mi_qmm_mulmat_swiglu.restype = ci
     L.mi_qmm_mulmat_swiglu.argtypes = [vp, vp, vp, ci, vp, ctypes.c_float, vp, i64, vp, ci]
     L.mi_qmm_rms_norm.restype = ci; L.mi_qmm_rms_norm.argtypes = [vp, vp, vp, ctypes.c_float, i64, i64, vp, ci]
@@ -458,6 +460,24 @@ class Context:
                                                ctypes.c_void_p(int(aux_ptr)) if aux_ptr else None, eps,
                                                ctypes.c_void_p(int(b_ptr)), b_cols, ctypes.c_void_p(int(ids_ptr)), n_used,
                                                n_tokens, ctypes.c_void_p(int(y_ptr)), DEVICE))
+
+    def mulmat_id_swiglu(self, w_gate: Weight, w_up: Weight, n_expert: int, b: np.ndarray, ids: np.ndarray) -> np.ndarray:
+        """silu(gate experts . Q8(b)) * (up experts . Q8(b)): f32 [tokens, n_used, rows]"""
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        if b.ndim != 3 or ids.ndim != 2 or b.shape[0] != ids.shape[0] or b.shape[2] != w_gate.k:
+            raise ValueError(f"b {b.shape} / ids {ids.shape} do not fit [tokens, b_cols, k={w_gate.k}] / [tokens, n_used]")
+        t, n_used = ids.shape
+        h = np.empty((t, n_used, w_gate.m // max(n_expert, 1)), dtype=np.float32)
+        _check(lib().mi_qmm_mulmat_id_swiglu(self._h, w_gate._h, w_up._h, n_expert, _ptr(b), b.shape[1], _ptr(ids), n_used, t,
+                                             _ptr(h), HOST))
+        return h
+
+    def mulmat_id_swiglu_device(self, w_gate: Weight, w_up: Weight, n_expert: int, b_ptr: int, b_cols: int, ids_ptr: int,
+                                n_used: int, n_tokens: int, h_ptr: int):
+        _check(lib().mi_qmm_mulmat_id_swiglu(self._h, w_gate._h, w_up._h, n_expert, ctypes.c_void_p(int(b_ptr)), b_cols,
+                                             ctypes.c_void_p(int(ids_ptr)), n_used, n_tokens, ctypes.c_void_p(int(h_ptr)),
+                                             DEVICE))
 
     def mulmat_id_multi(self, ws, n_expert: int, b: np.ndarray, ids: np.ndarray):
         """several expert stacks against the same b and ids; host arrays out"""

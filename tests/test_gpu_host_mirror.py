@@ -191,6 +191,20 @@ def test_python_mirror_expert_graph(tmp_path):
         av = oracle.swiglu(g.Floats().reshape(tokens, n_used, ff), u.Floats().reshape(tokens, n_used, ff))
         assert npref.rel_err(out.Floats().reshape(tokens, n_used, k),
                              oracle.mul_mat_id(qmm.Q8_0, down, ff, k, n_expert, av, idv)) <= 1e-3
+        # the same block as one fresh graph: at one token gate, up and the gating are one call (the two products
+        # are never materialized), with more tokens the gating runs inside the down experts' quantization
+        ctx2 = b.NewContext()
+        ids2 = ctx2.FromInts(idv.reshape(-1), n_used, tokens)
+        x2 = ctx2.FromFloats(xv.reshape(-1), k, 1, tokens)
+        g2, u2 = wg.MulmatID(ctx2, x2, ids2), wu.MulmatID(ctx2, x2, ids2)
+        act2 = g2.SILU(ctx2, u2)
+        out2 = wd.MulmatID(ctx2, act2, ids2)
+        ctx2.Compute(out2)
+        for lazy in ((g2, u2) if tokens == 1 else (act2,)):
+            with pytest.raises(RuntimeError):
+                lazy.Floats()
+        assert np.array_equal(out2.Floats(), out.Floats())
+        ctx2.Close()
         with pytest.raises(TypeError):
             wg.Mulmat(ctx, ctx.FromFloats(xv.reshape(-1), k, tokens))        # a stack is not a 2-D weight
         with pytest.raises(ValueError):

@@ -313,3 +313,51 @@ def test_mulmat_swiglu_errors_and_device_pointers(ctx):
         dx.free(); dh.free()
     for w in (wg, wu, w3, w6):
         w.free()
+
+
+# gate and up of an expert block with the gating: decode sizes in one launch (rows of one segment, short rows
+# two and four to a load, rows of several segments), batches through the two products and the gating kernel,
+# stacks of different types, ids outside the stack
+@pytest.mark.parametrize("t,k,m,n_expert,tokens,n_used,b_cols", [(Q4_K, 2048, 96, 16, 1, 8, 1), (Q4_K, 768, 200, 8, 2, 4, 4),
+                                                                  (Q4_K, 4096, 33, 4, 1, 2, 1), (Q6_K, 1024, 70, 6, 3, 2, 1),
+                                                                  (Q4_K, 8192, 20, 4, 1, 2, 1), (Q8_0, 352, 40, 6, 1, 3, 1),
+                                                                  (Q4_0, 2048, 31, 4, 2, 2, 2), (Q4_K, 1024, 64, 4, 40, 2, 1),
+                                                                  (Q4_K, 512, 64, 3, 300, 2, 1), (Q8_0, 256, 50, 2, 30, 2, 1)])
+def test_expert_gate_and_up_with_the_gating(ctx, t, k, m, n_expert, tokens, n_used, b_cols):
+    rng = np.random.default_rng(8000 + t + k + tokens)
+    wbg, wbu = _experts(t, n_expert, m, k, 8001 + t + k), _experts(t, n_expert, m, k, 8002 + t + k)
+    wg, wu = ctx.upload(t, wbg, k, n_expert * m), ctx.upload(t, wbu, k, n_expert * m)
+    b = (rng.standard_normal((tokens, b_cols, k)) * 2).astype(np.float32)
+    ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+    h = ctx.mulmat_id_swiglu(wg, wu, n_expert, b, ids)
+    want = oracle.swiglu(oracle.mul_mat_id(t, wbg, k, m, n_expert, b, ids), oracle.mul_mat_id(t, wbu, k, m, n_expert, b, ids))
+    assert h.shape == (tokens, n_used, m) and npref.rel_err(h, want) < TOL
+    yg, yu = ctx.mulmat_id_multi([wg, wu], n_expert, b, ids)
+    assert np.array_equal(h, ctx.swiglu(yg, yu))
+    # ids outside the stack (device ids): NaN rows for those pairs, the others unchanged
+    bad = ids.copy()
+    bad[0, 0] = n_expert
+    db, dids = DeviceArray(b), DeviceArray(bad)
+    dh = DeviceArray(np.zeros((tokens, n_used, m), np.float32), zero=True)
+    ctx.mulmat_id_swiglu_device(wg, wu, n_expert, db.ptr, b_cols, dids.ptr, n_used, tokens, dh.ptr)
+    ctx.sync()
+    out = dh.numpy()
+    assert np.isnan(out[0, 0]).all() and np.array_equal(out.reshape(-1, m)[1:], h.reshape(-1, m)[1:])
+    with pytest.raises(qmm.QmmError):
+        ctx.mulmat_id_swiglu(wg, wu, n_expert, b, bad)
+    for d in (db, dids, dh):
+        d.free()
+    wg.free(); wu.free()
+
+
+def test_expert_gating_with_stacks_of_two_types(ctx):
+    k, m, n_expert, n_used = 512, 48, 4, 2
+    rng = np.random.default_rng(83)
+    wbg, wbu = _experts(Q4_K, n_expert, m, k, 84), _experts(Q6_K, n_expert, m, k, 85)
+    wg, wu = ctx.upload(Q4_K, wbg, k, n_expert * m), ctx.upload(Q6_K, wbu, k, n_expert * m)
+    for tokens in (1, 20):
+        b = rng.standard_normal((tokens, 1, k)).astype(np.float32)
+        ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+        h = ctx.mulmat_id_swiglu(wg, wu, n_expert, b, ids)
+        assert np.array_equal(h, ctx.swiglu(ctx.mulmat_id(wg, n_expert, b, ids), ctx.mulmat_id(wu, n_expert, b, ids)))
+    wg.free(); wu.free()
