@@ -676,6 +676,44 @@ def test_page_locked_host_buffers(ctx):
     w.free()
 
 
+# ---- skinny product on the matrix cores for the K-quants: both kernels ------------------------------
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("m,k,n", [(4096, 4096, 3), (1000, 1024, 4), (17, 256, 4), (9, 256, 3), (300, 2304, 19), (64, 8192, 4),
+                                   (4096, 14336, 4), (1000, 1024, 7), (2048, 768, 3)])
+def test_skinny_kquants_match_oracle(ctx, t, m, k, n):
+    """3..31 columns through the C ABI's default routing: Q4_K at three and four columns of a small matrix
+    takes the kernel that loads weights straight into the MFMA operands (ragged M, a single super-block,
+    K cut one to sixteen ways, a second launch that starts at column 16), a large one and more columns
+    the staged kernel"""
+    rng = np.random.default_rng(8100 + t + m + n)
+    wb = _weights(t, m, k, 8101 + t + m)
+    w = ctx.upload(t, wb, k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(w, x)
+    assert npref.rel_err(got, oracle.mul_mat(t, wb, k, m, x, nthreads=16)) < TOL
+    if n <= 16:  # one launch: a column's result does not depend on which other columns ride along
+        assert np.array_equal(ctx.mulmat(w, x[::-1].copy())[::-1], got)
+    w.free()
+
+
+@pytest.mark.parametrize("n", [3, 4, 6])
+def test_skinny_q4k_random_block_bytes(ctx, n):
+    """random block bytes reach every bit pattern of nibbles and of the 6-bit scales and mins; compared
+    with exact arithmetic on the quantized activations as well as with the oracle"""
+    rng = np.random.default_rng(8200 + n)
+    k, m = 2048, 40
+    nb = m * k // 256
+    raw = rng.integers(0, 256, (nb, 144), dtype=np.uint8)
+    raw[:, 0:4] = np.abs(rng.standard_normal(nb * 2) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 4)
+    W = ctx.upload(Q4_K, raw.reshape(-1), k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(W, x)
+    assert npref.rel_err(got, oracle.mul_mat(Q4_K, raw.reshape(-1), k, m, x, nthreads=8)) <= TOL
+    xq = oracle.quantize(Q8_K, x)
+    assert npref.rel_err(got, npref.matmul_f64(Q4_K, raw.reshape(-1), k, m, Q8_K, xq, n)) <= TOL
+    W.free()
+
+
 # ---- skinny product on the matrix cores for the 32-element block formats ------------------------------
 @pytest.mark.parametrize("t", [Q4_0, Q8_0])
 @pytest.mark.parametrize("m,k,n", [(4096, 4096, 8), (1000, 1024, 5), (17, 256, 4), (300, 2304, 16), (64, 8192, 31),
