@@ -290,7 +290,8 @@ def main() -> int:
             return tm, raw.size
 
         other = {}
-        for label, t, m, k, ns, copies in (("Q4_0 GEMV 4096x4096", Q4_0, 4096, 4096, (1,), 40),
+        for label, t, m, k, ns, copies in (("Q4_K q_proj 4096x4096", Q4_K, 4096, 4096, (1, 2, 4, 8), 40),
+                                           ("Q4_0 GEMV 4096x4096", Q4_0, 4096, 4096, (1,), 40),
                                            ("Q8_0 skinny 4096x4096", Q8_0, 4096, 4096, (1, 2, 4, 8), 40),
                                            ("Q6_K head 128256x4096", Q6_K, 128256, 4096, (1, 8), 3)):
             for n in ns:
@@ -314,7 +315,25 @@ def main() -> int:
             fn()
             tm = timed(fn, 10) / (10 * len(stacks))
             other[f"MulmatID Q4_K 128x(768x2048) top-8 tokens={toks}"] = {"us": round(tm * 1e6, 2)}
-        for st in stacks:
+        # one token through a mixture-of-experts feed-forward block: gate and up experts with their gating in
+        # one launch, the down experts (one activation row per used expert) in a second
+        raw_d = np.tile(synth.weights(Q4_K, 2048, em, seed=1202), (n_exp * ek // 2048, 1))
+        downs = [ctx.upload(Q4_K, np.roll(raw_d, 13 * c, axis=0), em, n_exp * ek) for c in range(3)]
+        xe = torch.randn(1, 1, ek, generator=g, dtype=torch.float32).to(dev)
+        ids = torch.randperm(n_exp, generator=g)[:n_used].reshape(1, n_used).to(torch.int32).to(dev)
+        he = torch.empty(1, n_used, em, dtype=torch.float32, device=dev)
+        yd = torch.empty(1, n_used, ek, dtype=torch.float32, device=dev)
+
+        def moe_block():
+            for c in range(3):
+                ctx.mulmat_id_swiglu_device(stacks[2 * c], stacks[2 * c + 1], n_exp, xe.data_ptr(), 1, ids.data_ptr(), n_used, 1,
+                                            he.data_ptr())
+                ctx.mulmat_id_device(downs[c], n_exp, he.data_ptr(), n_used, ids.data_ptr(), n_used, 1, yd.data_ptr())
+
+        moe_block()
+        tm = timed(moe_block, 20) / (20 * 3)
+        other["decode expert FFN block 128x(768x2048) top-8: gate, up and gating in one launch, down in a second"] = {"us": round(tm * 1e6, 2)}
+        for st in stacks + downs:
             st.free()
         # decode feed-forward block with its producers, on the main pool: RMSNorm -> gate, up (one launch) and
         # SILU(gate) * up -> down (one launch), against the same block through the stand-alone f32 kernels
