@@ -290,7 +290,7 @@ def main() -> int:
             return tm, raw.size
 
         other = {}
-        for label, t, m, k, ns, copies in (("Q4_K q_proj 4096x4096", Q4_K, 4096, 4096, (1, 2, 4, 8), 40),
+        for label, t, m, k, ns, copies in (("Q4_K q_proj 4096x4096", Q4_K, 4096, 4096, (2, 4, 8), 40),  # (one column would share the headline kernel's name in a profile)
                                            ("Q4_0 GEMV 4096x4096", Q4_0, 4096, 4096, (1,), 40),
                                            ("Q8_0 skinny 4096x4096", Q8_0, 4096, 4096, (1, 2, 4, 8), 40),
                                            ("Q6_K head 128256x4096", Q6_K, 128256, 4096, (1, 8), 3)):
