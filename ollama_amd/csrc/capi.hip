@@ -631,7 +631,25 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
                     while (e < idx.size() && e - j < (size_t)gemv_max_multi() && ws[idx[e]]->dev.type == w0->dev.type &&
                            !wants_skinny(w0->dev.type, K, ws[idx[e]]->dev.M, n))
                         e++;
-                if (e - j > 1) {
+                // three or four columns of small Q4_K matrices (q, k and v of a layer): one launch of the
+                // direct-load MFMA kernel over as many of them as it takes
+                size_t es = j + 1;
+                {
+                    DevWeight dw[8];
+                    dw[0] = w0->dev;
+                    while (es < idx.size() && es - j < 8) {
+                        dw[es - j] = ws[idx[es]]->dev;
+                        if (!skinny_multi_supports(dw, (int)(es - j + 1), (int)n)) break;
+                        es++;
+                    }
+                }
+                if (e - j == 1 && es - j > 1 && a.sd8 && wants_skinny(w0->dev.type, K, w0->dev.M, n)) {
+                    DevWeight dw[8];
+                    float *out[8];
+                    for (size_t t = j; t < es; t++) { dw[t - j] = ws[idx[t]]->dev; out[t - j] = dys[idx[t]]; }
+                    HIP_TRY(launch_skinny_multi(dw, out, (int)(es - j), a, (int)n, ctx->num_cus, ctx->stream));
+                    e = es;
+                } else if (e - j > 1) {
                     DevWeight dw[8];
                     float *out[8];
                     for (size_t t = j; t < e; t++) { dw[t - j] = ws[idx[t]]->dev; out[t - j] = dys[idx[t]]; }
@@ -1137,7 +1155,15 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
     for (int i = 0; gemv_ok && i < count; i++)  // from five or six columns up each weight goes to the skinny kernel
         gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n);
-    if (!gemm_ok && !gemv_ok) {
+    // three or four columns of small Q4_K matrices: one launch of the direct-load MFMA kernel
+    bool skinny_ok = false;
+    if (!gemm_ok && !gemv_ok && same && count >= 2 && count <= 8 && act->n >= 1 && act->n <= 4 &&
+        wants_skinny(ws[0]->dev.type, ws[0]->dev.K, ws[0]->dev.M, act->n)) {
+        DevWeight probe[8];
+        for (int i = 0; i < count; i++) probe[i] = ws[i]->dev;
+        skinny_ok = skinny_multi_supports(probe, count, (int)act->n);
+    }
+    if (!gemm_ok && !gemv_ok && !skinny_ok) {
         for (int i = 0; i < count; i++) {
             int rc = mi_qmm_mulmat_q8(ctx, ws[i], act, ys[i], location, MI_QMM_PATH_AUTO);
             if (rc) return rc;
@@ -1170,6 +1196,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
     if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));
+    else if (skinny_ok) HIP_TRY(launch_skinny_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));
     else HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));
     if (location == MI_QMM_HOST) {
         for (int i = 0; i < count; i++)

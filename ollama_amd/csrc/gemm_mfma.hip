@@ -881,16 +881,43 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
 // then holds, for weight row r and column c, the sums of the four even sub-blocks (MFMAs 0, 1 chained)
 // and of the four odd ones (MFMAs 2, 3), scales them with v_mad_i32_i24, and takes the mins term from
 // one more MFMA (block-sum digits x mins) exactly as the staged kernel above does.
-__global__ __launch_bounds__(1024, 8) void direct16_q4k_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
-                                                               int kcut) {
+//
+// Up to DIRECT16_MULTI matrices that share K and the activations go out in one launch: their 16-row groups
+// are numbered through, and a wave finds its matrix by comparing its group number with the ends of the runs.
+constexpr int DIRECT16_MULTI = 4;
+struct Direct16Args {
+    const uint8_t *p0[DIRECT16_MULTI];
+    float *y[DIRECT16_MULTI];
+    int64_t M[DIRECT16_MULTI];
+    int grp_end[DIRECT16_MULTI];  // exclusive end of each matrix's run of groups; INT_MAX past the last matrix
+    int64_t K;
+    int groups_total;
+};
+
+struct Direct16Where { const uint8_t *p0; float *y; int64_t M; int first; };
+template <bool MULTI>
+__device__ __forceinline__ Direct16Where direct16_where(const Direct16Args &g, int group) {
+    Direct16Where w{g.p0[0], g.y[0], g.M[0], 0};
+    if (!MULTI) return w;
+#pragma unroll
+    for (int t = 1; t < DIRECT16_MULTI; t++)
+        if (group >= g.grp_end[t - 1]) w = Direct16Where{g.p0[t], g.y[t], g.M[t], g.grp_end[t - 1]};
+    return w;
+}
+
+template <bool MULTI>
+__global__ __launch_bounds__(1024, 8) void direct16_q4k_kernel(Direct16Args g, DevAct a, int col0, int nc, int kcut, int threads) {
     __shared__ float part[16][4][16];  // [wave][column][row]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int GROUPS = (blockDim.x >> 6) / kcut;  // row groups of this workgroup
+    const int GROUPS = (threads >> 6) / kcut;  // row groups of this workgroup (threads = the block size, as an argument:
+                                               // one batch of scalar loads fetches everything the prologue needs)
     const int r = lane & 15, q = lane >> 4;
     const int grp = wave / kcut, kw = wave - grp * kcut;
-    const int64_t m0 = min(((int64_t)blockIdx.x * GROUPS + grp) * 16, (w.M - 1) / 16 * 16);  // groups past M: the last one again, not stored
+    const int group = min((int)blockIdx.x * GROUPS + grp, g.groups_total - 1);  // groups past the last: the last one again, not stored
+    const Direct16Where w = direct16_where<MULTI>(g, group);
+    const int64_t m0 = (int64_t)(group - w.first) * 16;
     const int rows_left = (int)min((int64_t)16, w.M - m0);
-    const int nsb = (int)(w.K / QKK);
+    const int nsb = (int)(g.K / QKK);
     const int sb0 = nsb * kw / kcut, sb1 = nsb * (kw + 1) / kcut;
     const uint8_t *hp = w.p0 + (m0 + min(r, rows_left - 1)) * ((int64_t)nsb * Q4_K_BYTES);  // rows past M: the last row again
     const uint8_t *wp = hp + 16 + 32 * q;
@@ -937,12 +964,14 @@ __global__ __launch_bounds__(1024, 8) void direct16_q4k_kernel(DevWeight w, DevA
     }
     part[wave][q][r] = acc;
     __syncthreads();
-    for (int o = tid; o < GROUPS * 64; o += blockDim.x) {
+    for (int o = tid; o < GROUPS * 64; o += threads) {
         const int og = o >> 6, i = (o >> 4) & 3, j = o & 15;  // group, activation column, weight row
-        const int64_t row = ((int64_t)blockIdx.x * GROUPS + og) * 16 + j;
+        const int out_group = (int)blockIdx.x * GROUPS + og;
+        const Direct16Where ow = direct16_where<MULTI>(g, min(out_group, g.groups_total - 1));
+        const int64_t row = (int64_t)(out_group - ow.first) * 16 + j;
         float sum = 0.f;
         for (int kk = 0; kk < kcut; kk++) sum += part[og * kcut + kk][i][j];
-        if (i < nc && row < w.M) y[(int64_t)(col0 + i) * w.M + row] = sum;
+        if (i < nc && out_group < g.groups_total && row < ow.M) ow.y[(int64_t)(col0 + i) * ow.M + row] = sum;
     }
 }
 
@@ -950,21 +979,35 @@ __global__ __launch_bounds__(1024, 8) void direct16_q4k_kernel(DevWeight w, DevA
 // and four columns) while M x K stays under about 40 M elements; from the 14336 x 4096 FFN matrices up the
 // staged kernel's coalesced copies are ahead (11.7 against 12.4 us), and so they are from five columns up,
 // where a second column set doubles the direct kernel's activation loads.
-bool direct16_wanted(const DevWeight &w, int ncols) {
-    return w.type == T_Q4_K && ncols <= 4 && w.M * w.K <= (int64_t)40 << 20;
+bool direct16_wanted(int type, int64_t K, int64_t total_m, int ncols) {
+    return type == T_Q4_K && ncols <= 4 && total_m * K <= (int64_t)40 << 20;
 }
 
-// About 28 waves per CU over the grid (all resident at once), a wave per K cut, at least one super-block
-// per wave; 16-wave workgroups as long as that leaves about two workgroups per CU.
-void launch_direct16(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
-    const int64_t rg = (w.M + 15) / 16;
-    const int nsb = (int)(w.K / QKK);
-    const int64_t want = ((int64_t)num_cus * 28 + rg / 2) / rg;
-    int kcut = want >= 16 ? 16 : want >= 8 ? 8 : want >= 4 ? 4 : want >= 2 ? 2 : 1;
+// K is always cut 16 ways (fewer when it has fewer super-blocks), whatever the number of rows: the order of
+// the floating-point sums then does not depend on which matrices share a launch, and measured over the same
+// shapes it is as fast as cutting by the size of the grid.  16-wave workgroups: one row group each, or
+// several when K is short, as long as that leaves about two workgroups per CU.
+void launch_direct16(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols, int num_cus,
+                     hipStream_t s) {
+    Direct16Args g;
+    int64_t rg = 0;
+    for (int i = 0; i < DIRECT16_MULTI; i++) {
+        const int j = i < count ? i : count - 1;
+        g.p0[i] = ws[j].p0; g.y[i] = ys[j]; g.M[i] = ws[j].M;
+        if (i < count) rg += (ws[i].M + 15) / 16;
+        g.grp_end[i] = i < count ? (int)rg : 0x7fffffff;
+    }
+    g.K = ws[0].K;
+    g.groups_total = (int)rg;
+    const int nsb = (int)(g.K / QKK);
+    int kcut = 16;
     while (kcut > nsb) kcut >>= 1;
     int groups = 16 / kcut;
     while (groups > 1 && (rg + groups - 1) / groups < 2 * (int64_t)num_cus) groups >>= 1;
-    direct16_q4k_kernel<<<(unsigned)((rg + groups - 1) / groups), 64 * kcut * groups, 0, s>>>(w, a, col0, ncols, y, kcut);
+    const unsigned grid = (unsigned)((rg + groups - 1) / groups);
+    const int threads = 64 * kcut * groups;
+    if (count > 1) direct16_q4k_kernel<true><<<grid, threads, 0, s>>>(g, a, col0, ncols, kcut, threads);
+    else direct16_q4k_kernel<false><<<grid, threads, 0, s>>>(g, a, col0, ncols, kcut, threads);
 }
 
 // y[i] = sum over slices of part[slice][i]
@@ -1095,13 +1138,33 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
     const SkinnyIds none{};
     const int64_t rg = (w.M + 15) / 16;
     if (w.type == T_Q4_K) {
-        if (direct16_wanted(w, ncols)) launch_direct16(w, a, col0, ncols, y, num_cus, s);
+        if (direct16_wanted(w.type, w.K, w.M, ncols)) launch_direct16(&w, &y, 1, a, col0, ncols, num_cus, s);
         else if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q4K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     } else {
         if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q6K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     }
+    return hipGetLastError();
+}
+
+// Several Q4_K matrices that share K against the same three or four activation columns: one launch of
+// the direct-load kernel over their numbered-through row groups when together they are small enough for it.
+bool skinny_multi_supports(const DevWeight *ws, int count, int ncols) {
+    if (count < 2 || count > DIRECT16_MULTI) return false;
+    int64_t total_m = 0;
+    for (int i = 0; i < count; i++) {
+        if (ws[i].type != T_Q4_K || ws[i].K != ws[0].K || !skinny_supports(ws[i].type, ws[i].K, ws[i].M)) return false;
+        total_m += ws[i].M;
+    }
+    return (total_m + 15 * count) / 16 < 0x7fffffff && direct16_wanted(T_Q4_K, ws[0].K, total_m, ncols);
+}
+
+hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
+                               hipStream_t s) {
+    if (!skinny_multi_supports(ws, count, ncols) || a.type != T_Q8_K || a.K != ws[0].K || !a.sd8) return hipErrorInvalidValue;
+    if (ncols < 1 || ncols > a.N || (int64_t)ncols * a.K >= ((int64_t)1 << 32)) return hipErrorInvalidValue;
+    launch_direct16(ws, ys, count, a, 0, ncols, num_cus, s);
     return hipGetLastError();
 }
 

@@ -91,6 +91,10 @@ int gemm_max_multi();
 bool skinny_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                          hipStream_t s);
+// several Q4_K matrices of one K in one launch of the direct-load kernel (three or four columns, small matrices)
+bool skinny_multi_supports(const DevWeight *ws, int count, int ncols);
+hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
+                               hipStream_t s);
 
 // int8-MFMA GEMM for the 32-element block formats (Q4_0, Q8_0 weights; Q8_0 activations), any N >= 1.
 // y[n*M + m].

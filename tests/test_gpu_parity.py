@@ -243,12 +243,15 @@ def test_multi_weight_launch_matches_single(ctx):
         raws = [_weights(t, m, k, seed=100 + m) for m in ms]
         Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
         act = ctx.act_create(qmm.vec_dot_type(t), k, 40)
-        for n in (1, 3, 9, 40):                            # 9: per-weight calls; 40: one GEMM launch (K-quants)
+        for n in (1, 3, 4, 9, 40):  # 3, 4: Q4_K in one launch of the direct-load MFMA kernel; 9: per-weight calls; 40: one GEMM launch (K-quants)
             x = rng.standard_normal((n, k), dtype=np.float32)
             ctx.act_quantize(act, x)
             want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV if n <= 8 else qmm.PATH_AUTO) for W in Ws]
             got = ctx.mulmat_q8_multi(Ws, act)
             for y, wnt in zip(got, want):
+                assert np.array_equal(y, wnt)
+            # f32 activations in: the same bits as the two-phase calls
+            for y, wnt in zip(ctx.mulmat_multi(Ws, x), want):
                 assert np.array_equal(y, wnt)
         act.free()
         for W in Ws:
