@@ -89,6 +89,7 @@ __device__ __forceinline__ float reduce_rows(const float (&v)[U], int lane) {
 // ---------------------------------------------------------------------------------------------
 
 struct PolQ4K {
+    static constexpr int PLANES = 1;  // planes of the device layout a row is read from
     static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
     static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;  // Q8_K: one scale per 256, one sum per 16
@@ -177,6 +178,7 @@ struct PolQ4K {
 };
 
 struct PolQ4_0 {
+    static constexpr int PLANES = 2;  // planes of the device layout a row is read from
     static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 2048;  // 64 blocks, one per lane
     static constexpr int ACT_BLK = QK, ACT_BSUM = QK;  // Q8_0: one scale and one sum per 32
@@ -237,6 +239,7 @@ struct PolQ4_0 {
 };
 
 struct PolQ8_0 {
+    static constexpr int PLANES = 2;  // planes of the device layout a row is read from
     static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 1024;  // 32 blocks, two lanes (16 quants each) per block
     static constexpr int ACT_BLK = QK, ACT_BSUM = QK;
@@ -284,6 +287,7 @@ struct PolQ8_0 {
 };
 
 struct PolQ6K {
+    static constexpr int PLANES = 4;  // planes of the device layout a row is read from
     static constexpr int F32_WAVES_ONE_SEG = 8;  // waves per workgroup when it quantizes one column of one-segment rows
     static constexpr int SEG = 4096;  // 16 super-blocks, 4 lanes each
     static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;  // Q8_K: one scale per 256, one sum per 16
@@ -639,6 +643,13 @@ __device__ __forceinline__ void quantize_x_to_lds(const float4 *__restrict__ x4,
         quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
 }
 
+// Global-address-space pointer types: what a kernel's pointer arguments are cast to before an empty asm pins
+// them in scalar registers (see gemv_thin_kernel), so that they come out of it still known to be global.
+typedef const __attribute__((address_space(1))) uint8_t *gbytes_t;
+typedef __attribute__((address_space(1))) float *gfloats_t;
+typedef const __attribute__((address_space(1))) float *gcfloats_t;
+typedef const __attribute__((address_space(1))) int *gcints_t;
+
 // Kernel arguments of the thin kernel, arranged so that the tensor a workgroup belongs to is picked
 // with compares and selects on values that are all fetched by one batch of scalar loads: a select
 // chain that indexes the argument block with a computed index makes each pointer load wait for the
@@ -667,13 +678,55 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     // partial sums [rows_per_wg][NC][kw].
     extern __shared__ __align__(16) uint8_t smem[];
     const int bid = blockIdx.x;
-    const int e0 = ta.wg_end[0], e1 = ta.wg_end[1], e2 = ta.wg_end[2];
+    // Everything the prologue needs from the argument block is named here and pinned by an empty asm, so
+    // that the scalar loads go out as one batch at the top: left alone the compiler turns the selects
+    // below into branches and fetches each side's pointers only after the branch, three dependent rounds
+    // of scalar loads before the first vector load.
+    // (The pointers go through the asm as global-address-space pointers: as plain ones they would come out
+    // with their address space unknown and every load through them would become a flat load.)
+    typedef const __attribute__((address_space(1))) uint16_t *ghalves_t;
+    typedef const __attribute__((address_space(1))) int8_t *gi8_t;
+    typedef const __attribute__((address_space(1))) int16_t *gi16_t;
+    typedef int ints4_t __attribute__((ext_vector_type(4)));
+    typedef long longs2_t __attribute__((ext_vector_type(2)));
+    gbytes_t p0a = (gbytes_t)ta.p0[0], p0b = (gbytes_t)ta.p0[1], p0c = (gbytes_t)ta.p0[2], p0d = (gbytes_t)ta.p0[3];
+    gbytes_t p1a = (gbytes_t)ta.p1[0], p1b = (gbytes_t)ta.p1[1], p1c = (gbytes_t)ta.p1[2], p1d = (gbytes_t)ta.p1[3];
+    gbytes_t p2a = (gbytes_t)ta.p2[0], p2b = (gbytes_t)ta.p2[1], p2c = (gbytes_t)ta.p2[2], p2d = (gbytes_t)ta.p2[3];
+    ghalves_t da = (ghalves_t)ta.d[0], db = (ghalves_t)ta.d[1], dc = (ghalves_t)ta.d[2], dd = (ghalves_t)ta.d[3];
+    gfloats_t ya = (gfloats_t)ta.y[0], yb = (gfloats_t)ta.y[1], yc = (gfloats_t)ta.y[2], yd = (gfloats_t)ta.y[3];
+    gcfloats_t xg = (gcfloats_t)xf;
+    gi8_t aq = (gi8_t)a.qs;
+    gcfloats_t ad = (gcfloats_t)a.d;
+    gi16_t ab = (gi16_t)a.bsums;
+    ints4_t ends = {ta.wg_end[0], ta.wg_end[1], ta.wg_end[2], ta.wg_end[3]};
+    ints4_t dims = {col0, rows_per_wave, kw, rw_log2};
+    longs2_t Mab = {(long)ta.M[0], (long)ta.M[1]}, Mcd = {(long)ta.M[2], (long)ta.M[3]}, Ks = {(long)ta.K, (long)a.K};
+    if (F32) {
+        // (f32 x: the first loads are the wave's pieces of x, which need only the first few arguments, and the
+        // rest arrives while those are in flight -- pinning everything up front measured 3..5 % slower there)
+    } else if (P::PLANES > 1)
+        asm volatile("" : "+s"(p0a), "+s"(p0b), "+s"(p0c), "+s"(p0d), "+s"(p1a), "+s"(p1b), "+s"(p1c), "+s"(p1d), "+s"(p2a), "+s"(p2b),
+                          "+s"(p2c), "+s"(p2d), "+s"(da), "+s"(db), "+s"(dc), "+s"(dd), "+s"(ya), "+s"(yb), "+s"(yc), "+s"(yd),
+                          "+s"(xg), "+s"(aq), "+s"(ad), "+s"(ab), "+s"(ends), "+s"(dims), "+s"(Mab), "+s"(Mcd), "+s"(Ks));
+    else
+        asm volatile("" : "+s"(p0a), "+s"(p0b), "+s"(p0c), "+s"(p0d), "+s"(ya), "+s"(yb), "+s"(yc), "+s"(yd), "+s"(xg), "+s"(aq),
+                          "+s"(ad), "+s"(ab), "+s"(ends), "+s"(dims), "+s"(Mab), "+s"(Mcd), "+s"(Ks));
+    xf = (const float *)xg;
+    a.qs = (const int8_t *)aq;
+    a.d = (const float *)ad;
+    a.bsums = (const int16_t *)ab;
+    a.K = Ks[1];
+    col0 = dims[0]; rows_per_wave = dims[1]; kw = dims[2]; rw_log2 = dims[3];
+    const int e0 = ends[0], e1 = ends[1], e2 = ends[2];
+    const int64_t Ma = Mab[0], Mb = Mab[1], Mc = Mcd[0], Md = Mcd[1], Kall = Ks[0];
     const int t = (bid >= e0) + (bid >= e1) + (bid >= e2);
     const int wg = bid - (t == 0 ? 0 : t == 1 ? e0 : t == 2 ? e1 : e2);
-#define THIN_SEL(f) (t == 0 ? ta.f[0] : t == 1 ? ta.f[1] : t == 2 ? ta.f[2] : ta.f[3])
-    const DevWeight w{THIN_SEL(p0), THIN_SEL(p1), THIN_SEL(p2), THIN_SEL(d), ta.K, THIN_SEL(M), ta.type};
-    float *__restrict__ y = THIN_SEL(y);
-#undef THIN_SEL
+#define THIN_SEL4(a, b, c, d) (t == 0 ? a : t == 1 ? b : t == 2 ? c : d)
+    const DevWeight w{(const uint8_t *)THIN_SEL4(p0a, p0b, p0c, p0d), (const uint8_t *)THIN_SEL4(p1a, p1b, p1c, p1d),
+                      (const uint8_t *)THIN_SEL4(p2a, p2b, p2c, p2d), (const uint16_t *)THIN_SEL4(da, db, dc, dd), Kall,
+                      THIN_SEL4(Ma, Mb, Mc, Md), ta.type};
+    float *__restrict__ y = (float *)THIN_SEL4(ya, yb, yc, yd);
+#undef THIN_SEL4
     const int64_t ldy = w.M;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = 1 << rw_log2;
@@ -703,7 +756,7 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     // as soon as x is there while the weights are still in flight.
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col0 * K);
     const int total4 = (int)((int64_t)NC * K / 4);  // float4 pieces over all NC columns
-    const int nwaves = blockDim.x >> 6;
+    const int nwaves = kw << rw_log2 /* = (kw << rw_log2) * 64 / 64, without the hidden-argument load */;
     float4 xpre[XP], apre[XP];
     if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     // the producer's operand, requested unconditionally (RMSNorm without a weight reads x again and ignores
@@ -761,7 +814,7 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     if (DIRECT) return;
 
     __syncthreads();
-    for (int i = threadIdx.x; i < nrows * NC; i += blockDim.x) {
+    for (int i = threadIdx.x; i < nrows * NC; i += (kw << rw_log2) * 64) {
         const int n = i / nrows, rl = i - n * nrows;
         float sum = 0.f;
         for (int k = 0; k < kw; k++) sum += part[(rl * NC + n) * kw + k];
@@ -831,7 +884,7 @@ __global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const floa
     int16_t *lbs = reinterpret_cast<int16_t *>(smem + (size_t)K + (size_t)nblk * 4);
     const float4 *x4 = reinterpret_cast<const float4 *>(xf);
     const int total4 = (int)(K / 4);
-    const int nwaves = blockDim.x >> 6;
+    const int nwaves = kw << rw_log2 /* = (kw << rw_log2) * 64 / 64, without the hidden-argument load */;
     float4 xpre[XP], apre[XP];
     prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     const bool has_aux = XMODE == 2 && pr.aux != nullptr;
@@ -877,7 +930,7 @@ __global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const floa
     if (DIRECT) return;
 
     __syncthreads();
-    for (int i = threadIdx.x; i < nrows; i += blockDim.x) {
+    for (int i = threadIdx.x; i < nrows; i += (kw << rw_log2) * 64) {
         float gsum = 0.f, usum = 0.f;
         for (int k = 0; k < kw; k++) gsum += part[(2 * i) * kw + k];
         for (int k = 0; k < kw; k++) usum += part[(2 * i + 1) * kw + k];
@@ -1468,28 +1521,40 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     static_assert(!F32 || NC == 1, "the f32 prologue quantizes one activation row");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int REC = 2 + NC;
-    const bool second = (int)blockIdx.x >= ia.wgs_first;
-    const int bid = (int)blockIdx.x - (second ? ia.wgs_first : 0);
-    const DevWeight w{second ? ia.p0b : ia.w.p0, second ? ia.p1b : ia.w.p1, second ? ia.p2b : ia.w.p2,
-                      second ? ia.db : ia.w.d, ia.w.K, ia.w.M, ia.w.type};
-    float *__restrict__ y = second ? ia.yb : ia.y;
-    const int group = bid / ia.wgs_per_group, wg = bid - group * ia.wgs_per_group;
+    // the argument block in one batch of scalar loads, as in gemv_thin_kernel: the branches below would
+    // otherwise each be followed by a round of their own
+    gbytes_t p0a = (gbytes_t)ia.w.p0, p0b = (gbytes_t)ia.p0b;
+    gfloats_t ya = (gfloats_t)ia.y, yb = (gfloats_t)ia.yb;
+    gcints_t ids = (gcints_t)ia.ids, groups = (gcints_t)ia.groups;
+    gcfloats_t xg = (gcfloats_t)xf, upg = (gcfloats_t)up;
+    int64_t M = ia.M, Kall = ia.w.K;
+    int n_expert = ia.n_expert, n_used = ia.n_used, b_cols = ia.b_cols, wgs_per_group = ia.wgs_per_group, wgs_first = ia.wgs_first;
+    asm volatile("" : "+s"(p0a), "+s"(p0b), "+s"(ya), "+s"(yb), "+s"(ids), "+s"(groups), "+s"(xg), "+s"(upg), "+s"(M), "+s"(Kall),
+                      "+s"(n_expert), "+s"(n_used), "+s"(b_cols), "+s"(wgs_per_group), "+s"(wgs_first), "+s"(rows_per_wave), "+s"(kw),
+                      "+s"(rw_log2));
+    xf = (const float *)xg;
+    up = (const float *)upg;
+    const bool second = (int)blockIdx.x >= wgs_first;
+    const int bid = (int)blockIdx.x - (second ? wgs_first : 0);
+    const DevWeight w{(const uint8_t *)(second ? p0b : p0a), second ? ia.p1b : ia.w.p1, second ? ia.p2b : ia.w.p2,
+                      second ? ia.db : ia.w.d, Kall, ia.w.M, ia.w.type};
+    float *__restrict__ y = (float *)(second ? yb : ya);
+    const int group = bid / wgs_per_group, wg = bid - group * wgs_per_group;
     int expert, count, pair[NC];
-    if (ia.groups) {
-        if (group >= ia.groups[0]) return;
-        const int *rec = ia.groups + 1 + (size_t)group * REC;
+    if (groups) {
+        if (group >= groups[0]) return;
+        gcints_t rec = groups + 1 + (size_t)group * REC;
         expert = rec[0];
         count = rec[1];
 #pragma unroll
         for (int n = 0; n < NC; n++) pair[n] = rec[2 + min(n, count - 1)];
     } else {
-        expert = ia.ids[group];
-        if (expert < 0 || expert >= ia.n_expert) expert = -1;
+        expert = ids[group];
+        if (expert < 0 || expert >= n_expert) expert = -1;
         count = 1;
 #pragma unroll
         for (int n = 0; n < NC; n++) pair[n] = group;
     }
-    const int64_t M = ia.M;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = 1 << rw_log2;
     const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
@@ -1498,7 +1563,7 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     const int nrows = (int)min((int64_t)rows_per_wg, M - r0);
     if (expert < 0) {
         // an id outside the stack: the pair's output is all NaN
-        for (int i = threadIdx.x; i < nrows * count; i += blockDim.x) {
+        for (int i = threadIdx.x; i < nrows * count; i += (kw << rw_log2) * 64) {
             const int n = i / nrows, rl = i - n * nrows;
             y[(int64_t)pair[n] * M + r0 + rl] = __int_as_float(0x7fc00000);
         }
@@ -1513,8 +1578,8 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     int col[NC];  // activation row of each pair: token * b_cols + slot mod b_cols
 #pragma unroll
     for (int n = 0; n < NC; n++) {
-        const int tok = pair[n] / ia.n_used, slot = pair[n] - tok * ia.n_used;
-        col[n] = tok * ia.b_cols + slot % ia.b_cols;
+        const int tok = pair[n] / n_used, slot = pair[n] - tok * n_used;
+        col[n] = tok * b_cols + slot % b_cols;
     }
     const int64_t K = w.K;
     const int nblk = (int)(K / P::ACT_BLK);
@@ -1523,7 +1588,7 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     float *ld_ = reinterpret_cast<float *>(smem + K);
     int16_t *lbs = reinterpret_cast<int16_t *>(smem + K + (size_t)nblk * 4);
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col[0] * K);
-    const int total4 = (int)(K / 4), nwaves = blockDim.x >> 6;
+    const int total4 = (int)(K / 4), nwaves = kw << rw_log2 /* = (kw << rw_log2) * 64 / 64, without the hidden-argument load */;
     float4 xpre[XPRE], apre[XPRE];
     if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     if (XMODE == 3) prefetch_x(reinterpret_cast<const float4 *>(up + (int64_t)col[0] * K), total4, wave, nwaves, lane, apre);
@@ -1557,7 +1622,7 @@ __global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const
     }
     if (DIRECT) return;
     __syncthreads();
-    for (int i = threadIdx.x; i < nrows * count; i += blockDim.x) {
+    for (int i = threadIdx.x; i < nrows * count; i += (kw << rw_log2) * 64) {
         const int n = i / nrows, rl = i - n * nrows;
         float sum = 0.f;
         for (int k = 0; k < kw; k++) sum += part[(rl * NC + n) * kw + k];
@@ -1572,13 +1637,22 @@ template <class P, bool DIRECT, int RPL>
 __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const float *__restrict__ xf, int rows_per_wave, int kw,
                                                            int rw_log2) {
     extern __shared__ __align__(16) uint8_t smem[];
-    const DevWeight wa{ia.w.p0, ia.w.p1, ia.w.p2, ia.w.d, ia.w.K, ia.w.M, ia.w.type};
-    const DevWeight wb{ia.p0b, ia.p1b, ia.p2b, ia.db, ia.w.K, ia.w.M, ia.w.type};
-    float *__restrict__ hout = ia.y;
-    const int pair = (int)blockIdx.x / ia.wgs_per_group, wg = (int)blockIdx.x - pair * ia.wgs_per_group;
-    int expert = ia.ids[pair];
-    if (expert < 0 || expert >= ia.n_expert) expert = -1;
-    const int64_t M = ia.M;
+    // the argument block in one batch of scalar loads, as in gemv_thin_kernel
+    gbytes_t p0a = (gbytes_t)ia.w.p0, p0b = (gbytes_t)ia.p0b;
+    gfloats_t ya = (gfloats_t)ia.y;
+    gcints_t ids = (gcints_t)ia.ids;
+    gcfloats_t xg = (gcfloats_t)xf;
+    int64_t M = ia.M, Kall = ia.w.K;
+    int n_expert = ia.n_expert, n_used = ia.n_used, b_cols = ia.b_cols, wgs_per_group = ia.wgs_per_group;
+    asm volatile("" : "+s"(p0a), "+s"(p0b), "+s"(ya), "+s"(ids), "+s"(xg), "+s"(M), "+s"(Kall), "+s"(n_expert), "+s"(n_used),
+                      "+s"(b_cols), "+s"(wgs_per_group), "+s"(rows_per_wave), "+s"(kw), "+s"(rw_log2));
+    xf = (const float *)xg;
+    const DevWeight wa{(const uint8_t *)p0a, ia.w.p1, ia.w.p2, ia.w.d, Kall, ia.w.M, ia.w.type};
+    const DevWeight wb{(const uint8_t *)p0b, ia.p1b, ia.p2b, ia.db, Kall, ia.w.M, ia.w.type};
+    float *__restrict__ hout = (float *)ya;
+    const int pair = (int)blockIdx.x / wgs_per_group, wg = (int)blockIdx.x - pair * wgs_per_group;
+    int expert = ids[pair];
+    if (expert < 0 || expert >= n_expert) expert = -1;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = 1 << rw_log2;
     const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
@@ -1586,7 +1660,7 @@ __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const floa
     const int64_t r0 = (int64_t)wg * rows_per_wg;
     const int nrows = (int)min((int64_t)rows_per_wg, M - r0);
     if (expert < 0) {
-        for (int i = threadIdx.x; i < nrows; i += blockDim.x) hout[(int64_t)pair * M + r0 + i] = __int_as_float(0x7fc00000);
+        for (int i = threadIdx.x; i < nrows; i += (kw << rw_log2) * 64) hout[(int64_t)pair * M + r0 + i] = __int_as_float(0x7fc00000);
         return;
     }
     const int rl0 = rg * rows_per_wave;
@@ -1594,8 +1668,8 @@ __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const floa
     const int64_t wrow0 = (int64_t)expert * M + r0 + rl0;
     const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);
     const typename P::Geo g = P::geo(wa, kseg, vlane);
-    const int tok = pair / ia.n_used, slot = pair - tok * ia.n_used;
-    const int col = tok * ia.b_cols + slot % ia.b_cols;
+    const int tok = pair / n_used, slot = pair - tok * n_used;
+    const int col = tok * b_cols + slot % b_cols;
 
     const int64_t K = wa.K;
     const int nblk = (int)(K / P::ACT_BLK);
@@ -1604,7 +1678,7 @@ __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const floa
     float *ld_ = reinterpret_cast<float *>(smem + K);
     int16_t *lbs = reinterpret_cast<int16_t *>(smem + K + (size_t)nblk * 4);
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col * K);
-    const int total4 = (int)(K / 4), nwaves = blockDim.x >> 6;
+    const int total4 = (int)(K / 4), nwaves = kw << rw_log2 /* = (kw << rw_log2) * 64 / 64, without the hidden-argument load */;
     float4 xpre[XPRE];
     prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     typename P::Raw cur;
@@ -1628,7 +1702,7 @@ __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const floa
     }
     if (DIRECT) return;
     __syncthreads();
-    for (int i = threadIdx.x; i < nrows; i += blockDim.x) {
+    for (int i = threadIdx.x; i < nrows; i += (kw << rw_log2) * 64) {
         float gsum = 0.f, usum = 0.f;
         for (int k = 0; k < kw; k++) gsum += part[(2 * i) * kw + k];
         for (int k = 0; k < kw; k++) usum += part[(2 * i + 1) * kw + k];
