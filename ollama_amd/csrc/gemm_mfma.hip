@@ -654,13 +654,43 @@ constexpr int SKINNY_ID_REC = 2 + 16;
 
 // The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
 template <class S, int NCT, bool ID, int NST>
-__global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
-                                                        SkinnyIds si) {
+__global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_kernel(DevWeight w_in, DevAct a_in, int col0, int nc, float *__restrict__ y_in,
+                                                        SkinnyIds si_in, int WAVES, int grid_size) {
     typedef typename S::G G;
     typedef SkinnyGeo<S, NCT, NST> Geo;
     constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, WAVE_BYTES = Geo::WAVE_BYTES;
-    const int WAVES = blockDim.x >> 6;
+    // The whole argument block in one batch of scalar loads: every value is named here and pinned by an
+    // empty asm (left alone the compiler fetches them where each branch first needs them, four or five
+    // dependent rounds before the first copy is issued).  Pointers go through as global-address-space
+    // pointers so that they stay known to be global; the block and grid sizes are arguments (WAVES,
+    // grid_size) rather than reads of the hidden arguments.
+    typedef const __attribute__((address_space(1))) uint8_t *gbytes_t;
+    typedef const __attribute__((address_space(1))) uint16_t *ghalves_t;
+    typedef const __attribute__((address_space(1))) int8_t *gi8_t;
+    typedef const __attribute__((address_space(1))) int16_t *gi16_t;
+    typedef const __attribute__((address_space(1))) float *gcfloats_t;
+    typedef const __attribute__((address_space(1))) int *gcints_t;
+    typedef __attribute__((address_space(1))) float *gfloats_t;
+    typedef int ints4_t __attribute__((ext_vector_type(4)));
+    typedef long longs2_t __attribute__((ext_vector_type(2)));
+    gbytes_t p0 = (gbytes_t)w_in.p0, p1 = (gbytes_t)w_in.p1, p2 = (gbytes_t)w_in.p2, sd8 = (gbytes_t)a_in.sd8, sd16 = (gbytes_t)a_in.sd16;
+    ghalves_t wd = (ghalves_t)w_in.d;
+    gi8_t aqs = (gi8_t)a_in.qs;
+    gcfloats_t ad = (gcfloats_t)a_in.d;
+    gi16_t ab = (gi16_t)a_in.bsums;
+    gcints_t groups = (gcints_t)si_in.groups;
+    gfloats_t yg = (gfloats_t)y_in;
+    longs2_t km = {(long)w_in.K, (long)w_in.M}, km2 = {(long)a_in.K, (long)si_in.M};
+    ints4_t i0 = {col0, nc, WAVES, grid_size}, i1 = {si_in.wgs_per_group, si_in.n_used, si_in.b_cols, a_in.N};
+    asm volatile("" : "+s"(p0), "+s"(p1), "+s"(p2), "+s"(sd8), "+s"(sd16), "+s"(wd), "+s"(aqs), "+s"(ad), "+s"(ab), "+s"(groups),
+                      "+s"(yg), "+s"(km), "+s"(km2), "+s"(i0), "+s"(i1));
+    const DevWeight w{(const uint8_t *)p0, (const uint8_t *)p1, (const uint8_t *)p2, (const uint16_t *)wd, km[0], km[1], w_in.type};
+    const DevAct a{(const int8_t *)aqs, (const float *)ad, (const int16_t *)ab, (const uint8_t *)sd8, (const uint8_t *)sd16, km2[0],
+                   i1[3], a_in.type};
+    const SkinnyIds si{(const int *)groups, km2[1], i1[0], i1[1], i1[2]};
+    float *__restrict__ y = (float *)yg;
+    col0 = i0[0]; nc = i0[1]; WAVES = i0[2]; grid_size = i0[3];
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
     float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * WAVE_BYTES);
 
@@ -680,7 +710,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
         ldy = si.M;
         if (expert < 0) {
             // ids outside the stack: these pairs' outputs are all NaN
-            for (int o = tid; o < 16 * nc; o += blockDim.x)
+            for (int o = tid; o < 16 * nc; o += (64 * WAVES))
                 if ((o & 15) < rows_left) y[(int64_t)rec[2 + (o >> 4)] * ldy + yrow0 + (o & 15)] = __int_as_float(0x7fc00000);
             return;
         }
@@ -696,11 +726,11 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     const int64_t nsb = w.K / QKK;
     const int64_t sb0 = nsb * wave / WAVES, sb1 = nsb * (wave + 1) / WAVES;  // this wave's run of super-blocks
     uint8_t *wsm = smem + wave * WAVE_BYTES;
-    // Work items: the 16-row groups this workgroup goes through, blockIdx.x + k * gridDim.x (an
+    // Work items: the 16-row groups this workgroup goes through, blockIdx.x + k * grid_size (an
     // expert-indexed launch has exactly one per workgroup).  The copy stream runs two stages ahead of
     // the math and simply continues into the next item, so only the first item pays the pipeline fill.
     const int64_t total_items = ID ? 0 : (w.M + 15) / 16;
-    const int64_t items = ID ? 1 : (total_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const int64_t items = ID ? 1 : (total_items - blockIdx.x + grid_size - 1) / grid_size;
 
     // ---- copy plan: per-lane 32-bit offsets, uniform bases per super-block
     unsigned woff[S::W_INSTRS];
@@ -759,7 +789,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
         } else if (cp_k + 1 < items) {
             cp_k++;
             cp_sb = sb0;
-            const int64_t first = ((int64_t)blockIdx.x + cp_k * gridDim.x) * 16;  // never taken by expert-indexed launches
+            const int64_t first = ((int64_t)blockIdx.x + cp_k * grid_size) * 16;  // never taken by expert-indexed launches
             plan_item(first, (int)min((int64_t)16, w.M - first));
         }
     };
@@ -794,7 +824,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
 #pragma unroll 1
     for (int64_t k = 0; k < items; k++) {
         if (!ID) {
-            m0 = ((int64_t)blockIdx.x + k * gridDim.x) * 16;
+            m0 = ((int64_t)blockIdx.x + k * grid_size) * 16;
             yrow0 = m0;
             rows_left = (int)min((int64_t)16, w.M - m0);
         }
@@ -855,7 +885,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
             for (int u = 0; u < S::LANE_COLS; u++)
                 part[wave][S::SET_COLS * cs + S::lane_col(g, u)][c] = acc[cs * S::LANE_COLS + u];
         __syncthreads();
-        for (int o = tid; o < 16 * NCT; o += blockDim.x) {
+        for (int o = tid; o < 16 * NCT; o += (64 * WAVES)) {
             const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
             float sum = 0.f;
             for (int kk = 0; kk < WAVES; kk++) sum += part[kk][i][j];
@@ -1112,7 +1142,7 @@ void launch_skinny_grid(const DevWeight &w, const DevAct &a, int col0, int ncols
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny_kernel<S, NCT, ID, NST><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
+    skinny_kernel<S, NCT, ID, NST><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves, (int)grid);
 }
 
 template <class S, int NCT, bool ID>
