@@ -37,10 +37,13 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float4 *__rest
                                                             int *__restrict__ qs, float *__restrict__ d,
                                                             int16_t *__restrict__ bsums, int64_t nblk, Produce pr,
                                                             int64_t k4) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 256 threads per workgroup (launch_quantize_act)
     const int64_t blk = t >> 3;
     const bool live = blk < nblk;
-    const float4 v = live ? produced<KIND>(x, t, pr, k4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    // unconditional load (threads past the end read the last piece again and drop it): a conditional one
+    // fetches its pointer only after the branch
+    const float4 vl = produced<KIND>(x, live ? t : nblk * 8 - 1, pr, k4);
+    const float4 v = live ? vl : make_float4(0.f, 0.f, 0.f, 0.f);
     float dd;
     int sum;
     const int packed = q8_0_quantize_lane(v, dd, sum);
@@ -61,11 +64,14 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__rest
                                                             uint8_t *__restrict__ sd16, int64_t nblk, Produce pr,
                                                             int64_t k4) {
     const int lane = threadIdx.x & 63;
-    const int64_t blk = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // 256 threads per workgroup (launch_quantize_act)
+    // the load goes out before the range check (a wave past the end reads the last block again and leaves):
+    // with the check first, the pointer is fetched only after the branch, a second round of scalar loads
+    const float4 v = produced<KIND>(x, (blk < nblk ? blk : nblk - 1) * 64 + lane, pr, k4);
     if (blk >= nblk) return;  // whole wave leaves together
     float dd;
     int sum, pair;
-    const int packed = q8_K_quantize_lane(produced<KIND>(x, blk * 64 + lane, pr, k4), lane, dd, sum, pair);
+    const int packed = q8_K_quantize_lane(v, lane, dd, sum, pair);
     qs[blk * 64 + lane] = packed;
     if ((lane & 3) == 0) bsums[blk * 16 + (lane >> 2)] = (int16_t)sum;
     if (lane == 0) d[blk] = dd;
