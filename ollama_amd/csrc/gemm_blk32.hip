@@ -371,11 +371,38 @@ struct Sk32Ids {
 constexpr int SK32_ID_REC = 2 + 16;
 
 template <bool Q4, int NCT, bool ID>
-__global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y,
-                                                                          Sk32Ids si) {
+__global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w_in, DevAct a_in, int col0, int nc, float *__restrict__ y_in,
+                                                                          Sk32Ids si_in, int WAVES) {
     typedef Sk32Geo<Q4, NCT> Geo;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, SETS = Geo::SETS;
-    const int WAVES = blockDim.x >> 6;
+    // The argument block in one batch of scalar loads: everything is named here and pinned by an empty asm
+    // (otherwise each branch below is followed by a round of loads of its own), pointers as
+    // global-address-space pointers so that they stay known to be global, the block size as an argument.
+    typedef const __attribute__((address_space(1))) uint8_t *gbytes_t;
+    typedef const __attribute__((address_space(1))) uint16_t *ghalves_t;
+    typedef const __attribute__((address_space(1))) int8_t *gi8_t;
+    typedef const __attribute__((address_space(1))) int16_t *gi16_t;
+    typedef const __attribute__((address_space(1))) float *gcfloats_t;
+    typedef const __attribute__((address_space(1))) int *gcints_t;
+    typedef __attribute__((address_space(1))) float *gfloats_t;
+    typedef int ints4_t __attribute__((ext_vector_type(4)));
+    typedef long longs2_t __attribute__((ext_vector_type(2)));
+    gbytes_t p0 = (gbytes_t)w_in.p0;
+    ghalves_t wd = (ghalves_t)w_in.d;
+    gi8_t aqs = (gi8_t)a_in.qs;
+    gcfloats_t ad = (gcfloats_t)a_in.d;
+    gi16_t ab = (gi16_t)a_in.bsums;
+    gcints_t groups = (gcints_t)si_in.groups;
+    gfloats_t yg = (gfloats_t)y_in;
+    longs2_t km = {(long)w_in.K, (long)w_in.M}, km2 = {(long)a_in.K, (long)si_in.M};
+    ints4_t i0 = {col0, nc, WAVES, a_in.N}, i1 = {si_in.wgs_per_group, si_in.n_used, si_in.b_cols, 0};
+    asm volatile("" : "+s"(p0), "+s"(wd), "+s"(aqs), "+s"(ad), "+s"(ab), "+s"(groups), "+s"(yg), "+s"(km), "+s"(km2), "+s"(i0),
+                      "+s"(i1));
+    const DevWeight w{(const uint8_t *)p0, w_in.p1, w_in.p2, (const uint16_t *)wd, km[0], km[1], w_in.type};
+    const DevAct a{(const int8_t *)aqs, (const float *)ad, (const int16_t *)ab, a_in.sd8, a_in.sd16, km2[0], i0[3], a_in.type};
+    const Sk32Ids si{(const int *)groups, km2[1], i1[0], i1[1], i1[2]};
+    float *__restrict__ y = (float *)yg;
+    col0 = i0[0]; nc = i0[1]; WAVES = i0[2];
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
     float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * Geo::WAVE_BYTES);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -393,7 +420,7 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
         ldy = si.M;
         rows_left = (int)min((int64_t)16, si.M - yrow0);
         if (expert < 0) {  // ids outside the stack: the outputs of these pairs are all NaN
-            for (int o = tid; o < 16 * nc; o += blockDim.x)
+            for (int o = tid; o < 16 * nc; o += (64 * WAVES))
                 if ((o & 15) < rows_left) y[(int64_t)rec[2 + (o >> 4)] * ldy + yrow0 + (o & 15)] = __int_as_float(0x7fc00000);
             return;
         }
@@ -550,7 +577,7 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
 #pragma unroll
         for (int u = 0; u < 2; u++) part[wave][8 * cs + 2 * g + u][c] = acc[cs][u];
     __syncthreads();
-    for (int o = tid; o < 16 * NCT; o += blockDim.x) {
+    for (int o = tid; o < 16 * NCT; o += (64 * WAVES)) {
         const int i = o >> 4, j = o & 15;  // activation column, weight row of the tile
         float sum = 0.f;
         for (int k = 0; k < WAVES; k++) sum += part[k][i][j];
@@ -575,7 +602,7 @@ void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny32_kernel<Q4, NCT, ID><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si);
+    skinny32_kernel<Q4, NCT, ID><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves);
 }
 
 }  // namespace
