@@ -631,19 +631,19 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
                     while (e < idx.size() && e - j < (size_t)gemv_max_multi() && ws[idx[e]]->dev.type == w0->dev.type &&
                            !wants_skinny(w0->dev.type, K, ws[idx[e]]->dev.M, n))
                         e++;
-                // three or four columns of small Q4_K matrices (q, k and v of a layer): one launch of the
-                // direct-load MFMA kernel over as many of them as it takes
+                // K-quant matrices on the skinny MFMA kernels (q, k and v of a layer at 3..16 columns): one launch
+                // over as many of them as keep the kernel and K cut of a launch of their own
                 size_t es = j + 1;
                 {
                     DevWeight dw[8];
                     dw[0] = w0->dev;
                     while (es < idx.size() && es - j < 8) {
                         dw[es - j] = ws[idx[es]]->dev;
-                        if (!skinny_multi_supports(dw, (int)(es - j + 1), (int)n)) break;
+                        if (!skinny_multi_supports(dw, (int)(es - j + 1), (int)n, ctx->num_cus)) break;
                         es++;
                     }
                 }
-                if (e - j == 1 && es - j > 1 && a.sd8 && wants_skinny(w0->dev.type, K, w0->dev.M, n)) {
+                if (e - j == 1 && es - j > 1 && a.sd8 && a.sd16 && wants_skinny(w0->dev.type, K, w0->dev.M, n)) {
                     DevWeight dw[8];
                     float *out[8];
                     for (size_t t = j; t < es; t++) { dw[t - j] = ws[idx[t]]->dev; out[t - j] = dys[idx[t]]; }
@@ -1155,13 +1155,13 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
     for (int i = 0; gemv_ok && i < count; i++)  // from five or six columns up each weight goes to the skinny kernel
         gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n);
-    // three or four columns of small Q4_K matrices: one launch of the direct-load MFMA kernel
+    // K-quant matrices at 3..16 columns: one launch of a skinny MFMA kernel when it gives the same bits
     bool skinny_ok = false;
-    if (!gemm_ok && !gemv_ok && same && count >= 2 && count <= 8 && act->n >= 1 && act->n <= 4 &&
+    if (!gemm_ok && !gemv_ok && same && count >= 2 && count <= 8 && act->n >= 1 && act->n <= 16 &&
         wants_skinny(ws[0]->dev.type, ws[0]->dev.K, ws[0]->dev.M, act->n)) {
         DevWeight probe[8];
         for (int i = 0; i < count; i++) probe[i] = ws[i]->dev;
-        skinny_ok = skinny_multi_supports(probe, count, (int)act->n);
+        skinny_ok = skinny_multi_supports(probe, count, (int)act->n, ctx->num_cus);
     }
     if (!gemm_ok && !gemv_ok && !skinny_ok) {
         for (int i = 0; i < count; i++) {

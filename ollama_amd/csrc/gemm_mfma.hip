@@ -652,10 +652,37 @@ struct SkinnyIds {
 };
 constexpr int SKINNY_ID_REC = 2 + 16;
 
+// Several matrices of one type and K against the same activations in one launch (q, k, v; gate, up): their
+// 16-row groups are numbered through, matrix 0 is the kernel's w and y, the others come in this block, and
+// a work item finds its matrix by comparing its group number with the ends of the runs.
+struct SkinnyMulti {
+    const uint8_t *p0[3], *p1[3], *p2[3];
+    const uint16_t *d[3];
+    float *y[3];
+    int64_t M[3];
+    int grp_end[3];  // exclusive ends of the runs of matrices 0, 1, 2; INT_MAX past the last matrix
+    int groups_total;
+};
+struct SkinnyWhere { DevWeight w; float *y; int first; };
+template <bool MULTI>
+__device__ __forceinline__ SkinnyWhere skinny_where(const DevWeight &w0, float *y0, const SkinnyMulti &mt, int group) {
+    SkinnyWhere x{w0, y0, 0};
+    if (!MULTI) return x;
+#pragma unroll
+    for (int t = 0; t < 3; t++)
+        if (group >= mt.grp_end[t]) {
+            x.w.p0 = mt.p0[t]; x.w.p1 = mt.p1[t]; x.w.p2 = mt.p2[t]; x.w.d = mt.d[t]; x.w.M = mt.M[t];
+            x.y = mt.y[t];
+            x.first = mt.grp_end[t];
+        }
+    return x;
+}
+
 // The number of waves per workgroup (how many ways K is cut) is the launch's block size / 64.
-template <class S, int NCT, bool ID, int NST>
+template <class S, int NCT, bool ID, int NST, bool MULTI = false>
 __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_kernel(DevWeight w_in, DevAct a_in, int col0, int nc, float *__restrict__ y_in,
-                                                        SkinnyIds si_in, int WAVES, int grid_size) {
+                                                        SkinnyIds si_in, int WAVES, int grid_size, SkinnyMulti mt) {
+    static_assert(!(ID && MULTI), "expert-indexed launches take one stack");
     typedef typename S::G G;
     typedef SkinnyGeo<S, NCT, NST> Geo;
     constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
@@ -685,18 +712,22 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     ints4_t i0 = {col0, nc, WAVES, grid_size}, i1 = {si_in.wgs_per_group, si_in.n_used, si_in.b_cols, a_in.N};
     asm volatile("" : "+s"(p0), "+s"(p1), "+s"(p2), "+s"(sd8), "+s"(sd16), "+s"(wd), "+s"(aqs), "+s"(ad), "+s"(ab), "+s"(groups),
                       "+s"(yg), "+s"(km), "+s"(km2), "+s"(i0), "+s"(i1));
-    const DevWeight w{(const uint8_t *)p0, (const uint8_t *)p1, (const uint8_t *)p2, (const uint16_t *)wd, km[0], km[1], w_in.type};
+    const DevWeight w0{(const uint8_t *)p0, (const uint8_t *)p1, (const uint8_t *)p2, (const uint16_t *)wd, km[0], km[1], w_in.type};
     const DevAct a{(const int8_t *)aqs, (const float *)ad, (const int16_t *)ab, (const uint8_t *)sd8, (const uint8_t *)sd16, km2[0],
                    i1[3], a_in.type};
     const SkinnyIds si{(const int *)groups, km2[1], i1[0], i1[1], i1[2]};
-    float *__restrict__ y = (float *)yg;
+    float *const y0 = (float *)yg;
     col0 = i0[0]; nc = i0[1]; WAVES = i0[2]; grid_size = i0[3];
+    // the matrix of the item being multiplied (w, y) and of the item being copied (cw)
+    const SkinnyWhere at0 = skinny_where<MULTI>(w0, y0, mt, (int)blockIdx.x);
+    DevWeight w = at0.w, cw = at0.w;
+    float *y = at0.y;
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
     float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * WAVE_BYTES);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, g = lane >> 4;
-    int64_t m0 = (int64_t)blockIdx.x * 16, yrow0 = m0, ldy = w.M;
+    int64_t m0 = (int64_t)((int)blockIdx.x - at0.first) * 16, yrow0 = m0, ldy = w.M;
     int rows_left = (int)min((int64_t)16, w.M - m0);  // rows past M: the last row again, results dropped
     const int *rec = nullptr;
     if (ID) {
@@ -729,7 +760,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     // Work items: the 16-row groups this workgroup goes through, blockIdx.x + k * grid_size (an
     // expert-indexed launch has exactly one per workgroup).  The copy stream runs two stages ahead of
     // the math and simply continues into the next item, so only the first item pays the pipeline fill.
-    const int64_t total_items = ID ? 0 : (w.M + 15) / 16;
+    const int64_t total_items = ID ? 0 : MULTI ? mt.groups_total : (w.M + 15) / 16;
     const int64_t items = ID ? 1 : (total_items - blockIdx.x + grid_size - 1) / grid_size;
 
     // ---- copy plan: per-lane 32-bit offsets, uniform bases per super-block
@@ -740,7 +771,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     auto plan_item = [&](int64_t first_row, int rows) __attribute__((always_inline)) {
         cp_m0 = first_row;
 #pragma unroll
-        for (int j = 0; j < S::W_INSTRS; j++) S::w_plan(w, j, lane, rows, woff[j], won[j]);
+        for (int j = 0; j < S::W_INSTRS; j++) S::w_plan(cw, j, lane, rows, woff[j], won[j]);
         dhrow = (first_row + min(c, rows - 1)) * nsb * 2;
     };
     plan_item(m0, rows_left);
@@ -764,7 +795,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
         const int64_t sb = cp_sb;
 #pragma unroll
         for (int j = 0; j < S::W_INSTRS; j++) {
-            const uint8_t *gp = S::w_base(w, j, cp_m0, sb) + woff[j];
+            const uint8_t *gp = S::w_base(cw, j, cp_m0, sb) + woff[j];
             if (won[j]) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * j), 16, 0, 0);
         }
 #pragma unroll
@@ -781,7 +812,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
             if (yon) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + S::W_BYTES + A_BYTES + D_BYTES), 4, 0, 0);
         }
         if (S::SCALES_OUTSIDE) {  // the rows' fp16 super-block scales are a plane of their own (Q6_K)
-            const uint8_t *gp = reinterpret_cast<const uint8_t *>(w.d) + ((dhrow + 2 * sb) & ~(int64_t)3);
+            const uint8_t *gp = reinterpret_cast<const uint8_t *>(cw.d) + ((dhrow + 2 * sb) & ~(int64_t)3);
             if (lane < 16) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DH_OFF), 4, 0, 0);
         }
         if (cp_sb + 1 < sb1) {
@@ -789,8 +820,11 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
         } else if (cp_k + 1 < items) {
             cp_k++;
             cp_sb = sb0;
-            const int64_t first = ((int64_t)blockIdx.x + cp_k * grid_size) * 16;  // never taken by expert-indexed launches
-            plan_item(first, (int)min((int64_t)16, w.M - first));
+            const int group = (int)((int64_t)blockIdx.x + cp_k * grid_size);  // never taken by expert-indexed launches
+            const SkinnyWhere at = skinny_where<MULTI>(w0, y0, mt, group);
+            cw = at.w;
+            const int64_t first = (int64_t)(group - at.first) * 16;
+            plan_item(first, (int)min((int64_t)16, cw.M - first));
         }
     };
 
@@ -824,8 +858,13 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
 #pragma unroll 1
     for (int64_t k = 0; k < items; k++) {
         if (!ID) {
-            m0 = ((int64_t)blockIdx.x + k * grid_size) * 16;
+            const int group = (int)((int64_t)blockIdx.x + k * grid_size);
+            const SkinnyWhere at = skinny_where<MULTI>(w0, y0, mt, group);
+            w = at.w;
+            y = at.y;
+            m0 = (int64_t)(group - at.first) * 16;
             yrow0 = m0;
+            ldy = w.M;
             rows_left = (int)min((int64_t)16, w.M - m0);
         }
         float acc[LANE_ACC];
@@ -1142,7 +1181,38 @@ void launch_skinny_grid(const DevWeight &w, const DevAct &a, int col0, int ncols
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny_kernel<S, NCT, ID, NST><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves, (int)grid);
+    skinny_kernel<S, NCT, ID, NST><<<(unsigned)grid, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves, (int)grid, SkinnyMulti{});
+}
+
+// several matrices in one launch: their row groups numbered through (see SkinnyMulti)
+template <class S, int NCT>
+void launch_skinny_grid_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int waves,
+                              int num_cus, hipStream_t s) {
+    typedef SkinnyGeo<S, NCT, 2> Geo;
+    SkinnyMulti mt;
+    int64_t rg = (ws[0].M + 15) / 16;
+    for (int t = 0; t < 3; t++) {
+        const int j = t + 1 < count ? t + 1 : count - 1;
+        mt.p0[t] = ws[j].p0; mt.p1[t] = ws[j].p1; mt.p2[t] = ws[j].p2; mt.d[t] = ws[j].d; mt.y[t] = ys[j]; mt.M[t] = ws[j].M;
+        mt.grp_end[t] = t + 1 < count ? (int)rg : 0x7fffffff;
+        if (t + 1 < count) rg += (ws[j].M + 15) / 16;
+    }
+    mt.groups_total = (int)rg;
+    int64_t grid = rg;
+    if (waves == 1) {
+        const int64_t items = (rg + (int64_t)num_cus * 4) / ((int64_t)num_cus * 8);
+        if (items > 1) grid = (rg + items - 1) / items;
+    }
+    const size_t lds = (size_t)waves * (Geo::WAVE_BYTES + Geo::PART_BYTES);
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_kernel<S, NCT, false, 2, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        allowed[dev] = true;
+    }
+    skinny_kernel<S, NCT, false, 2, true><<<(unsigned)grid, 64 * waves, lds, s>>>(ws[0], a, 0, ncols, ys[0], SkinnyIds{}, waves,
+                                                                                  (int)grid, mt);
 }
 
 template <class S, int NCT, bool ID>
@@ -1180,21 +1250,52 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
 
 // Several Q4_K matrices that share K against the same three or four activation columns: one launch of
 // the direct-load kernel over their numbered-through row groups when together they are small enough for it.
-bool skinny_multi_supports(const DevWeight *ws, int count, int ncols) {
-    if (count < 2 || count > DIRECT16_MULTI) return false;
+// 1: one launch of the direct-load kernel; 2: one launch of the staged kernel; 0: no.  Either way every
+// matrix takes the kernel and the K cut it would take in a launch of its own, so the results are the same
+// bits as those of separate launches.
+int skinny_multi_kind(const DevWeight *ws, int count, int ncols, int num_cus) {
+    if (count < 2 || count > DIRECT16_MULTI || ncols < 1 || ncols > 16) return 0;
     int64_t total_m = 0;
+    bool each_direct = true, none_direct = true, same_waves = true;
+    const int waves0 = skinny_waves((ws[0].M + 15) / 16, ws[0].K / QKK, num_cus);
     for (int i = 0; i < count; i++) {
-        if (ws[i].type != T_Q4_K || ws[i].K != ws[0].K || !skinny_supports(ws[i].type, ws[i].K, ws[i].M)) return false;
+        if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || !skinny_supports(ws[i].type, ws[i].K, ws[i].M)) return 0;
         total_m += ws[i].M;
+        const bool dir = direct16_wanted(ws[i].type, ws[i].K, ws[i].M, ncols);
+        each_direct = each_direct && dir;
+        none_direct = none_direct && !dir;
+        same_waves = same_waves && skinny_waves((ws[i].M + 15) / 16, ws[i].K / QKK, num_cus) == waves0;
     }
-    return (total_m + 15 * count) / 16 < 0x7fffffff && direct16_wanted(T_Q4_K, ws[0].K, total_m, ncols);
+    if ((total_m + 15 * count) / 16 >= 0x7fffffff) return 0;
+    if (each_direct && direct16_wanted(ws[0].type, ws[0].K, total_m, ncols)) return 1;
+    // staged: the common K cut must still leave at most about 16 waves per CU over the joint grid.  Q4_K only:
+    // measured, q + k + v at 6 / 8 / 16 columns take 9.4 / 9.8 / 13.3 us in one launch against 17.0 / 17.6 / 21.2 in
+    // three, gate + up at 4..8 columns 19.6..20.9 against 23.0..23.6; the Q6_K kernel (more registers and LDS per
+    // wave) comes out 3..7 % slower joined than apart.
+    if (ws[0].type == T_Q4_K && none_direct && same_waves && (total_m + 15) / 16 * waves0 <= 16 * (int64_t)num_cus) return 2;
+    return 0;
+}
+bool skinny_multi_supports(const DevWeight *ws, int count, int ncols, int num_cus) {
+    return skinny_multi_kind(ws, count, ncols, num_cus) != 0;
 }
 
 hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
                                hipStream_t s) {
-    if (!skinny_multi_supports(ws, count, ncols) || a.type != T_Q8_K || a.K != ws[0].K || !a.sd8) return hipErrorInvalidValue;
+    const int kind = skinny_multi_kind(ws, count, ncols, num_cus);
+    if (!kind || a.type != T_Q8_K || a.K != ws[0].K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
     if (ncols < 1 || ncols > a.N || (int64_t)ncols * a.K >= ((int64_t)1 << 32)) return hipErrorInvalidValue;
-    launch_direct16(ws, ys, count, a, 0, ncols, num_cus, s);
+    if (kind == 1) {
+        launch_direct16(ws, ys, count, a, 0, ncols, num_cus, s);
+    } else {
+        const int waves = skinny_waves((ws[0].M + 15) / 16, ws[0].K / QKK, num_cus);
+        if (ws[0].type == T_Q4_K) {
+            if (ncols <= 8) launch_skinny_grid_multi<Sk16Q4K, 8>(ws, ys, count, a, ncols, waves, num_cus, s);
+            else launch_skinny_grid_multi<Sk16Q4K, 16>(ws, ys, count, a, ncols, waves, num_cus, s);
+        } else {
+            if (ncols <= 8) launch_skinny_grid_multi<Sk16Q6K, 8>(ws, ys, count, a, ncols, waves, num_cus, s);
+            else launch_skinny_grid_multi<Sk16Q6K, 16>(ws, ys, count, a, ncols, waves, num_cus, s);
+        }
+    }
     return hipGetLastError();
 }
 

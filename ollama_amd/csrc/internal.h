@@ -91,8 +91,9 @@ int gemm_max_multi();
 bool skinny_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                          hipStream_t s);
-// several Q4_K matrices of one K in one launch of the direct-load kernel (three or four columns, small matrices)
-bool skinny_multi_supports(const DevWeight *ws, int count, int ncols);
+// several K-quant matrices of one type and K in one launch of a skinny kernel (up to 16 columns), when every
+// one of them keeps the kernel and K cut of a launch of its own
+bool skinny_multi_supports(const DevWeight *ws, int count, int ncols, int num_cus);
 hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
                                hipStream_t s);
 

@@ -243,7 +243,9 @@ def test_multi_weight_launch_matches_single(ctx):
         raws = [_weights(t, m, k, seed=100 + m) for m in ms]
         Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
         act = ctx.act_create(qmm.vec_dot_type(t), k, 40)
-        for n in (1, 3, 4, 9, 40):  # 3, 4: Q4_K in one launch of the direct-load MFMA kernel; 9: per-weight calls; 40: one GEMM launch (K-quants)
+        # 3, 4: Q4_K in one launch of the direct-load MFMA kernel; 6, 9, 12: K-quants in one launch of the staged
+        # skinny kernel (ragged M = 300 in the middle), Q8_0 per-weight calls; 40: one GEMM launch (K-quants)
+        for n in (1, 3, 4, 6, 9, 12, 40):
             x = rng.standard_normal((n, k), dtype=np.float32)
             ctx.act_quantize(act, x)
             want = [ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV if n <= 8 else qmm.PATH_AUTO) for W in Ws]
@@ -254,6 +256,24 @@ def test_multi_weight_launch_matches_single(ctx):
             for y, wnt in zip(ctx.mulmat_multi(Ws, x), want):
                 assert np.array_equal(y, wnt)
         act.free()
+        for W in Ws:
+            W.free()
+
+
+def test_multi_weight_launch_with_unequal_k_cuts_falls_back(ctx):
+    """a large and a small matrix would cut K differently in launches of their own: the multi call must not
+    join them, and gives the bits of the single calls"""
+    k, ms = 4096, [14336, 1024]
+    rng = np.random.default_rng(37)
+    for t in (Q4_K, Q6_K):
+        raws = [_weights(t, m, k, seed=300 + m + t) for m in ms]
+        Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+        for n in (4, 7):
+            x = rng.standard_normal((n, k), dtype=np.float32)
+            want = [ctx.mulmat(W, x) for W in Ws]
+            for y, wnt, raw, m in zip(ctx.mulmat_multi(Ws, x), want, raws, ms):
+                assert np.array_equal(y, wnt)
+                assert npref.rel_err(y, oracle.mul_mat(t, raw, k, m, x, nthreads=16)) < TOL
         for W in Ws:
             W.free()
 
