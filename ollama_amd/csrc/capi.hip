@@ -631,7 +631,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
                     while (e < idx.size() && e - j < (size_t)gemv_max_multi() && ws[idx[e]]->dev.type == w0->dev.type &&
                            !wants_skinny(w0->dev.type, K, ws[idx[e]]->dev.M, n))
                         e++;
-                // K-quant matrices on the skinny MFMA kernels (q, k and v of a layer at 3..16 columns): one launch
+                // matrices on the skinny MFMA kernels (q, k and v of a layer at 3..16 columns): one launch
                 // over as many of them as keep the kernel and K cut of a launch of their own
                 size_t es = j + 1;
                 {
@@ -639,15 +639,18 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
                     dw[0] = w0->dev;
                     while (es < idx.size() && es - j < 8) {
                         dw[es - j] = ws[idx[es]]->dev;
-                        if (!skinny_multi_supports(dw, (int)(es - j + 1), (int)n, ctx->num_cus)) break;
+                        const bool ok = q8 == T_Q8_0 ? skinny32_multi_supports(dw, (int)(es - j + 1), (int)n, ctx->num_cus)
+                                                     : skinny_multi_supports(dw, (int)(es - j + 1), (int)n, ctx->num_cus);
+                        if (!ok) break;
                         es++;
                     }
                 }
-                if (e - j == 1 && es - j > 1 && a.sd8 && a.sd16 && wants_skinny(w0->dev.type, K, w0->dev.M, n)) {
+                if (e - j == 1 && es - j > 1 && (q8 == T_Q8_0 || (a.sd8 && a.sd16)) && wants_skinny(w0->dev.type, K, w0->dev.M, n)) {
                     DevWeight dw[8];
                     float *out[8];
                     for (size_t t = j; t < es; t++) { dw[t - j] = ws[idx[t]]->dev; out[t - j] = dys[idx[t]]; }
-                    HIP_TRY(launch_skinny_multi(dw, out, (int)(es - j), a, (int)n, ctx->num_cus, ctx->stream));
+                    if (q8 == T_Q8_0) HIP_TRY(launch_skinny32_multi(dw, out, (int)(es - j), a, (int)n, ctx->num_cus, ctx->stream));
+                    else HIP_TRY(launch_skinny_multi(dw, out, (int)(es - j), a, (int)n, ctx->num_cus, ctx->stream));
                     e = es;
                 } else if (e - j > 1) {
                     DevWeight dw[8];
@@ -1161,7 +1164,8 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         wants_skinny(ws[0]->dev.type, ws[0]->dev.K, ws[0]->dev.M, act->n)) {
         DevWeight probe[8];
         for (int i = 0; i < count; i++) probe[i] = ws[i]->dev;
-        skinny_ok = skinny_multi_supports(probe, count, (int)act->n, ctx->num_cus);
+        skinny_ok = act->type == T_Q8_0 ? skinny32_multi_supports(probe, count, (int)act->n, ctx->num_cus)
+                                        : skinny_multi_supports(probe, count, (int)act->n, ctx->num_cus);
     }
     if (!gemm_ok && !gemv_ok && !skinny_ok) {
         for (int i = 0; i < count; i++) {
@@ -1196,6 +1200,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
     if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));
+    else if (skinny_ok && a.type == T_Q8_0) HIP_TRY(launch_skinny32_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));
     else if (skinny_ok) HIP_TRY(launch_skinny_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));
     else HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));
     if (location == MI_QMM_HOST) {

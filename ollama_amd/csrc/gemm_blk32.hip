@@ -370,9 +370,20 @@ struct Sk32Ids {
 };
 constexpr int SK32_ID_REC = 2 + 16;
 
-template <bool Q4, int NCT, bool ID>
+// Several matrices of one type and K against the same activations in one launch (q, k, v; gate, up): their
+// 16-row groups are numbered through, matrix 0 is the kernel's w and y, the others come in this block.
+struct Sk32Multi {
+    const uint8_t *p0[3];
+    const uint16_t *d[3];
+    float *y[3];
+    int64_t M[3];
+    int grp_end[3];  // exclusive ends of the runs of matrices 0, 1, 2; INT_MAX past the last matrix
+};
+
+template <bool Q4, int NCT, bool ID, bool MULTI = false>
 __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w_in, DevAct a_in, int col0, int nc, float *__restrict__ y_in,
-                                                                          Sk32Ids si_in, int WAVES) {
+                                                                          Sk32Ids si_in, int WAVES, Sk32Multi mt) {
+    static_assert(!(ID && MULTI), "expert-indexed launches take one stack");
     typedef Sk32Geo<Q4, NCT> Geo;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, SETS = Geo::SETS;
     // The argument block in one batch of scalar loads: everything is named here and pinned by an empty asm
@@ -398,16 +409,26 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
     ints4_t i0 = {col0, nc, WAVES, a_in.N}, i1 = {si_in.wgs_per_group, si_in.n_used, si_in.b_cols, 0};
     asm volatile("" : "+s"(p0), "+s"(wd), "+s"(aqs), "+s"(ad), "+s"(ab), "+s"(groups), "+s"(yg), "+s"(km), "+s"(km2), "+s"(i0),
                       "+s"(i1));
-    const DevWeight w{(const uint8_t *)p0, w_in.p1, w_in.p2, (const uint16_t *)wd, km[0], km[1], w_in.type};
+    DevWeight w{(const uint8_t *)p0, w_in.p1, w_in.p2, (const uint16_t *)wd, km[0], km[1], w_in.type};
     const DevAct a{(const int8_t *)aqs, (const float *)ad, (const int16_t *)ab, a_in.sd8, a_in.sd16, km2[0], i0[3], a_in.type};
     const Sk32Ids si{(const int *)groups, km2[1], i1[0], i1[1], i1[2]};
     float *__restrict__ y = (float *)yg;
+    int first_group = 0;  // where the workgroup's matrix starts in the numbered-through groups
+    if (MULTI) {
+#pragma unroll
+        for (int t = 0; t < 3; t++)
+            if ((int)blockIdx.x >= mt.grp_end[t]) {
+                w.p0 = mt.p0[t]; w.d = mt.d[t]; w.M = mt.M[t];
+                y = mt.y[t];
+                first_group = mt.grp_end[t];
+            }
+    }
     col0 = i0[0]; nc = i0[1]; WAVES = i0[2];
     extern __shared__ __attribute__((aligned(256))) uint8_t smem[];  // WAVES x (WAVE_BYTES + PART_BYTES)
     float (*part)[16][16] = reinterpret_cast<float (*)[16][16]>(smem + WAVES * Geo::WAVE_BYTES);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, g = lane >> 4;
-    int64_t m0 = (int64_t)blockIdx.x * 16, yrow0 = m0, ldy = w.M;  // first weight row in w; first row and pitch of y
+    int64_t m0 = (int64_t)((int)blockIdx.x - first_group) * 16, yrow0 = m0, ldy = w.M;  // first weight row in w; first row and pitch of y
     int rows_left = (int)min((int64_t)16, w.M - m0);
     const int *rec = nullptr;
     if (ID) {
@@ -602,7 +623,40 @@ void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
     }
-    skinny32_kernel<Q4, NCT, ID><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves);
+    skinny32_kernel<Q4, NCT, ID><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves, Sk32Multi{});
+}
+
+// the K cut a matrix gets in a launch of its own
+int skinny32_waves(int64_t M, int64_t K, int num_cus) {
+    const int64_t groups = (M + 15) / 16, nst = K / 256;
+    const int64_t want = ((int64_t)num_cus * 8 + groups / 2) / groups;
+    int waves = want >= 8 ? 8 : want >= 6 ? 6 : want >= 4 ? 4 : want >= 3 ? 3 : want >= 2 ? 2 : 1;
+    while (waves > 1 && nst / waves < 1) waves = waves > 4 ? waves - 2 : waves - 1;
+    return waves;
+}
+
+template <bool Q4, int NCT>
+void launch_skinny32_multi_as(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int waves,
+                              hipStream_t s) {
+    typedef Sk32Geo<Q4, NCT> Geo;
+    Sk32Multi mt;
+    int64_t rg = (ws[0].M + 15) / 16;
+    for (int t = 0; t < 3; t++) {
+        const int j = t + 1 < count ? t + 1 : count - 1;
+        mt.p0[t] = ws[j].p0; mt.d[t] = ws[j].d; mt.y[t] = ys[j]; mt.M[t] = ws[j].M;
+        mt.grp_end[t] = t + 1 < count ? (int)rg : 0x7fffffff;
+        if (t + 1 < count) rg += (ws[j].M + 15) / 16;
+    }
+    const size_t lds = (size_t)waves * (Geo::WAVE_BYTES + Geo::PART_BYTES);
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny32_kernel<Q4, NCT, false, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        allowed[dev] = true;
+    }
+    skinny32_kernel<Q4, NCT, false, true><<<(unsigned)rg, 64 * waves, lds, s>>>(ws[0], a, 0, ncols, ys[0], Sk32Ids{nullptr, 0, 0, 0, 0},
+                                                                                waves, mt);
 }
 
 }  // namespace
@@ -621,6 +675,35 @@ hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int nc
     } else {
         if (ncols <= 8) launch_skinny32_as<false, 8>(w, a, col0, ncols, y, num_cus, s);
         else launch_skinny32_as<false, 16>(w, a, col0, ncols, y, num_cus, s);
+    }
+    return hipGetLastError();
+}
+
+// Several Q4_0 or Q8_0 matrices of one K in one launch, taken when each keeps the K cut of a launch of its own
+// (the results are then the same bits) and the joint grid stays within about 16 waves per CU.
+bool skinny32_multi_supports(const DevWeight *ws, int count, int ncols, int num_cus) {
+    if (count < 2 || count > 4 || ncols < 1 || ncols > 16) return false;
+    const int waves0 = skinny32_waves(ws[0].M, ws[0].K, num_cus);
+    int64_t groups = 0;
+    for (int i = 0; i < count; i++) {
+        if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || !skinny32_supports(ws[i].type, ws[i].K, ws[i].M)) return false;
+        if (skinny32_waves(ws[i].M, ws[i].K, num_cus) != waves0) return false;
+        groups += (ws[i].M + 15) / 16;
+    }
+    return groups < 0x7fffffff && groups * waves0 <= 16 * (int64_t)num_cus;
+}
+
+hipError_t launch_skinny32_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
+                                 hipStream_t s) {
+    if (!skinny32_multi_supports(ws, count, ncols, num_cus) || a.type != T_Q8_0 || a.K != ws[0].K) return hipErrorInvalidValue;
+    if (ncols > a.N || (int64_t)ncols * a.K >= ((int64_t)1 << 32) || (ws[0].type == T_Q4_0 && !a.bsums)) return hipErrorInvalidValue;
+    const int waves = skinny32_waves(ws[0].M, ws[0].K, num_cus);
+    if (ws[0].type == T_Q4_0) {
+        if (ncols <= 8) launch_skinny32_multi_as<true, 8>(ws, ys, count, a, ncols, waves, s);
+        else launch_skinny32_multi_as<true, 16>(ws, ys, count, a, ncols, waves, s);
+    } else {
+        if (ncols <= 8) launch_skinny32_multi_as<false, 8>(ws, ys, count, a, ncols, waves, s);
+        else launch_skinny32_multi_as<false, 16>(ws, ys, count, a, ncols, waves, s);
     }
     return hipGetLastError();
 }

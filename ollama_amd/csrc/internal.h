@@ -107,6 +107,10 @@ bool skinny32_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny32(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                            hipStream_t s);
 // the same kernel on expert stacks (see launch_gemv_id for the arguments): pairs bucketed 16 to a group
+// several Q4_0 / Q8_0 matrices of one K in one launch, when each keeps the K cut of a launch of its own
+bool skinny32_multi_supports(const DevWeight *ws, int count, int ncols, int num_cus);
+hipError_t launch_skinny32_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
+                                 hipStream_t s);
 bool skinny32_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_expert);
 hipError_t launch_skinny32_id(const DevWeight &w, int n_expert, const DevAct &a, const int *ids, int n_used, int n_tokens,
                               int b_cols, float *y, int *groups, int num_cus, hipStream_t s);

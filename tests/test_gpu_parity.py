@@ -238,13 +238,13 @@ def test_multi_weight_launch_matches_single(ctx):
     launch per weight"""
     k = 4096
     rng = np.random.default_rng(31)
-    for t in (Q4_K, Q8_0, Q6_K):
+    for t in (Q4_K, Q8_0, Q6_K, Q4_0):
         ms = [1024, 300, 4096]
         raws = [_weights(t, m, k, seed=100 + m) for m in ms]
         Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
         act = ctx.act_create(qmm.vec_dot_type(t), k, 40)
         # 3, 4: Q4_K in one launch of the direct-load MFMA kernel; 6, 9, 12: K-quants in one launch of the staged
-        # skinny kernel (ragged M = 300 in the middle), Q8_0 per-weight calls; 40: one GEMM launch (K-quants)
+        # skinny kernel of their format (ragged M = 300 in the middle); 40: one GEMM launch (K-quants)
         for n in (1, 3, 4, 6, 9, 12, 40):
             x = rng.standard_normal((n, k), dtype=np.float32)
             ctx.act_quantize(act, x)
@@ -265,7 +265,7 @@ def test_multi_weight_launch_with_unequal_k_cuts_falls_back(ctx):
     join them, and gives the bits of the single calls"""
     k, ms = 4096, [14336, 1024]
     rng = np.random.default_rng(37)
-    for t in (Q4_K, Q6_K):
+    for t in (Q4_K, Q6_K, Q8_0):
         raws = [_weights(t, m, k, seed=300 + m + t) for m in ms]
         Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
         for n in (4, 7):
