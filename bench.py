@@ -299,6 +299,22 @@ def main() -> int:
                 gbs = alg_bytes(wb, k, m, n) / tm / 1e9
                 other[f"{label} B={n}"] = {"us": round(tm * 1e6, 2), "GB/s": round(gbs, 1),
                                            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        # q, k and v of a layer through one multi call (f32 x in, quantization included)
+        qkv_ms = (4096, 1024, 1024)
+        qkv_sets = []
+        for c in range(20):
+            qkv_sets.append([ctx.upload(Q4_K, np.roll(synth.weights(Q4_K, m, 4096, seed=1150 + i), 13 * c, axis=0), 4096, m)
+                             for i, m in enumerate(qkv_ms)])
+        for n in (1, 4, 8):
+            xs = torch.randn(n, 4096, generator=g, dtype=torch.float32).to(dev)
+            yq = [torch.empty(n, m, dtype=torch.float32, device=dev) for m in qkv_ms]
+            fn = lambda: [ctx.mulmat_multi_device(ws3, xs.data_ptr(), n, [y_.data_ptr() for y_ in yq]) for ws3 in qkv_sets]
+            fn()
+            tm = timed(fn, 10) / (10 * len(qkv_sets))
+            other[f"Q4_K attn q+k+v (6144x4096) one call B={n}"] = {"us": round(tm * 1e6, 2)}
+        for ws3 in qkv_sets:
+            for wt in ws3:
+                wt.free()
         for label, t in (("Q4_0", Q4_0), ("Q8_0", Q8_0)):
             tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
             other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TOPS": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
