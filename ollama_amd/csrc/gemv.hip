@@ -701,9 +701,10 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     ints4_t ends = {ta.wg_end[0], ta.wg_end[1], ta.wg_end[2], ta.wg_end[3]};
     ints4_t dims = {col0, rows_per_wave, kw, rw_log2};
     longs2_t Mab = {(long)ta.M[0], (long)ta.M[1]}, Mcd = {(long)ta.M[2], (long)ta.M[3]}, Ks = {(long)ta.K, (long)a.K};
-    if (F32) {
-        // (f32 x: the first loads are the wave's pieces of x, which need only the first few arguments, and the
-        // rest arrives while those are in flight -- pinning everything up front measured 3..5 % slower there)
+    if (F32 && P::PLANES > 1) {
+        // (f32 x with a format of several planes: the first loads are the wave's pieces of x, which need only
+        // the first few arguments, and the rest arrives while those are in flight -- pinning all 29 values up
+        // front measured 3..5 % slower for Q4_0 / Q8_0.  Q4_K, one plane and 17 values, gains about 1 %.)
     } else if (P::PLANES > 1)
         asm volatile("" : "+s"(p0a), "+s"(p0b), "+s"(p0c), "+s"(p0d), "+s"(p1a), "+s"(p1b), "+s"(p1c), "+s"(p1d), "+s"(p2a), "+s"(p2b),
                           "+s"(p2c), "+s"(p2d), "+s"(da), "+s"(db), "+s"(dc), "+s"(dd), "+s"(ya), "+s"(yb), "+s"(yc), "+s"(yd),
