@@ -1366,14 +1366,18 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict_
                                                            int *__restrict__ src_col, int *__restrict__ out_pair) {
     __shared__ int count[ID_MAX_EXPERTS + 1], start[ID_MAX_EXPERTS + 1], scan[2][1024];
     const int nb = n_expert + 1, tid = threadIdx.x;
+    // eight independent loads at a time: one workgroup has to hide the latency of ids by itself.  The first
+    // 8192 ids are requested before anything else and stay in registers for both passes.
+    int first[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) first[j] = tid + 1024 * j < pairs ? ids[tid + 1024 * j] : -1;
     for (int e = tid; e < nb; e += 1024) count[e] = 0;
     for (int r = tid; r < tw * max_tiles; r += 1024) { src_col[r] = -1; out_pair[r] = -1; }
     __syncthreads();
-    // eight independent loads at a time: one workgroup has to hide the latency of ids by itself
     for (int p0 = tid; p0 < pairs; p0 += 8 * 1024) {
         int e[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) e[j] = p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
+        for (int j = 0; j < 8; j++) e[j] = p0 == tid ? first[j] : p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
 #pragma unroll
         for (int j = 0; j < 8; j++)
             if (p0 + 1024 * j < pairs) atomicAdd(&count[(e[j] < 0 || e[j] >= n_expert) ? n_expert : e[j]], 1);
@@ -1390,12 +1394,13 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict_
     scan[0][tid] = mine;
     __syncthreads();
     int cur = 0;
-    for (int step = 1; step < 1024; step <<= 1, cur ^= 1) {
+    const int owners = (nb + PER - 1) / PER;  // threads past these own no expert and never use their sums
+    for (int step = 1; step < owners; step <<= 1, cur ^= 1) {
         scan[cur ^ 1][tid] = scan[cur][tid] + (tid >= step ? scan[cur][tid - step] : 0);
         __syncthreads();
     }
     int t = scan[cur][tid] - mine;  // tiles of all experts before this thread's
-    if (tid == 1023) out[0] = scan[cur][tid];
+    if (tid == owners - 1) out[0] = scan[cur][tid];
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const int e = PER * tid + j;
@@ -1411,7 +1416,7 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int *__restrict_
     for (int p0 = tid; p0 < pairs; p0 += 8 * 1024) {
         int e[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) e[j] = p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
+        for (int j = 0; j < 8; j++) e[j] = p0 == tid ? first[j] : p0 + 1024 * j < pairs ? ids[p0 + 1024 * j] : -1;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const int p = p0 + 1024 * j;
