@@ -794,11 +794,13 @@ def test_mulmat_id_multi_equals_single_calls(ctx, t, tokens):
 
 @pytest.mark.parametrize("t,k,m,n_expert,tokens,n_used,b_cols", [(Q4_K, 1024, 200, 6, 64, 3, 1), (Q6_K, 512, 130, 4, 70, 2, 2),
                                                                (Q4_K, 2048, 768, 16, 128, 4, 1), (Q4_K, 256, 64, 3, 500, 1, 1),
-                                                               (Q4_K, 256, 32, 40, 1100, 6, 1), (Q6_K, 512, 130, 2, 150, 2, 1)])
+                                                               (Q4_K, 256, 32, 40, 1100, 6, 1), (Q6_K, 512, 130, 2, 150, 2, 1),
+                                                               (Q4_K, 256, 16, 8, 131100, 4, 1)])
 def test_mulmat_id_expert_gemm(ctx, t, k, m, n_expert, tokens, n_used, b_cols):
     """sixteen pairs per expert and more: pairs sorted by expert, every expert's run through the tiled GEMM;
     an idle expert, a crowded one (several tiles), ragged expert height, ids outside the stack (device ids);
-    tiles of 64 pairs, and of 128 from 96 pairs per expert"""
+    tiles of 64 pairs, and of 128 from 96 pairs per expert; more pairs (524400) than the chunked sort takes, which
+    one workgroup then sorts in several rounds of 8192"""
     rng = np.random.default_rng(8100 + t + tokens)
     wb = _experts(t, n_expert, m, k, 8101 + t)
     w = ctx.upload(t, wb, k, n_expert * m)
