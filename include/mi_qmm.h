@@ -86,6 +86,14 @@ void mi_qmm_destroy(mi_qmm_ctx *ctx);
  * ctx's scratch buffers have reached their size (first call of a shape), so such calls may be
  * captured into a HIP graph on the caller's stream after one eager call. */
 int mi_qmm_set_stream(mi_qmm_ctx *ctx, void *hip_stream);
+/* Scratch and captured graphs.  The product entry points keep quantized activations, K-split partial sums
+ * and host staging in scratch buffers that belong to the ctx and GROW on demand: a call that needs more
+ * than any earlier call frees the old buffer and allocates a larger one.  A HIP graph captured earlier
+ * still holds the old addresses, and replaying it after such a call would touch freed memory.  So:
+ * run every shape the graph's lifetime will see once (largest first is enough), then freeze.  While
+ * frozen (frozen != 0) a call that would have to grow any scratch returns MI_QMM_ERR_INVALID and leaves
+ * the buffers alone; frozen = 0 allows growth again (re-capture afterwards). */
+int mi_qmm_scratch_freeze(mi_qmm_ctx *ctx, int frozen);
 /* block until everything queued on the ctx's stream has finished */
 int mi_qmm_sync(mi_qmm_ctx *ctx);
 

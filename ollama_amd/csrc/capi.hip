@@ -51,6 +51,7 @@ struct mi_qmm_ctx {
     void *io_buf = nullptr;   size_t io_cap = 0;
     void *ws_buf = nullptr;   size_t ws_cap = 0;   // partial sums of a K-split GEMM
     void *pair_buf = nullptr; size_t pair_cap = 0; // the two products of a gated pair when they are not one launch
+    bool scratch_frozen = false;                   // mi_qmm_scratch_freeze: growth is an error, not a reallocation
 };
 
 struct mi_qmm_weight {
@@ -73,8 +74,15 @@ struct mi_qmm_act {
 
 namespace {
 
-int reserve(void **buf, size_t *cap, size_t need, hipStream_t s) {
+int reserve(mi_qmm_ctx *ctx, void **buf, size_t *cap, size_t need) {
     if (need <= *cap) return MI_QMM_OK;
+    hipStream_t s = ctx->stream;
+    // A captured HIP graph keeps the raw addresses of the scratch its kernels used: growing (= freeing) it
+    // afterwards would leave the graph pointing at freed memory.  Frozen scratch refuses to grow instead.
+    if (ctx->scratch_frozen)
+        return fail(MI_QMM_ERR_INVALID,
+                    "the call needs %zu bytes of scratch, the ctx holds %zu and its scratch is frozen "
+                    "(mi_qmm_scratch_freeze): run the largest shapes once before freezing", need, *cap);
     if (*buf) {
         HIP_TRY(hipStreamSynchronize(s));  // queued kernels may still read the old buffer
         HIP_TRY(hipFree(*buf));
@@ -390,14 +398,14 @@ int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k,
     if (!x || !out_blocks) return fail(MI_QMM_ERR_INVALID, "x or out_blocks is NULL");
 
     const ActPlanes probe = plan_act(nullptr, q8_type, k, n);
-    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+    if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, probe.total))) return rc;
     const ActPlanes p = plan_act(ctx->act_buf, q8_type, k, n);
     const size_t xbytes = (size_t)(n * k) * 4, obytes = (size_t)(n * row);
     const float *dx = x;
     uint8_t *dout = (uint8_t *)out_blocks;
     if (location == MI_QMM_HOST) {
         const size_t xoff = align_up(obytes, 256);
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, xoff + xbytes, ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, xoff + xbytes))) return rc;
         dout = (uint8_t *)ctx->io_buf;
         dx = (const float *)((char *)ctx->io_buf + xoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
@@ -426,7 +434,8 @@ bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
 }
 
 // dy: device output [n][M].  Picks the kernel and queues it on the ctx's stream.
-int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path) {
+// may_alloc = false: never touches the ctx's growable buffers (the tiled GEMM then runs without its K-split workspace).
+int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path, bool may_alloc = true) {
     const int64_t K = w->dev.K, M = w->dev.M, n = a.N;
     const bool blk32 = gemm_blk32_supports(w->dev.type, K, M);  // Q4_0 / Q8_0: their own MFMA kernel
     bool use_gemm;
@@ -442,9 +451,9 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
     if (use_gemm && blk32) {
         HIP_TRY(launch_gemm_blk32(w->dev, a, dy, ctx->num_cus, ctx->stream));
     } else if (use_gemm) {
-        const size_t wsf = gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus);
+        const size_t wsf = may_alloc ? gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus) : 0;
         if (wsf) {
-            int rc = reserve(&ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float), ctx->stream);
+            int rc = reserve(ctx, &ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float));
             if (rc) return rc;
         }
         HIP_TRY(launch_gemm(w->dev, a, dy, M, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
@@ -498,7 +507,7 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
     const ActPlanes probe = plan_act(nullptr, q8, K, n);
-    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total, ctx->stream))) return rc;
+    if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, probe.total))) return rc;
     const ActPlanes p = plan_act(ctx->act_buf, q8, K, n);
 
     const size_t xbytes = (size_t)(n * K) * 4, ybytes = (size_t)(n * M) * 4;
@@ -506,7 +515,7 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     float *dy = y;
     if (location == MI_QMM_HOST) {
         const size_t yoff = align_up(xbytes, 256);
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, yoff + ybytes, ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, yoff + ybytes))) return rc;
         dx = (const float *)ctx->io_buf;
         dy = (float *)((char *)ctx->io_buf + yoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
@@ -531,6 +540,13 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
 
 int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location) {
     return mi_qmm_mulmat_path(ctx, w, x, n, y, location, MI_QMM_PATH_AUTO);
+}
+
+int mi_qmm_scratch_freeze(mi_qmm_ctx *ctx, int frozen) {
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    ctx->scratch_frozen = frozen != 0;
+    return MI_QMM_OK;
 }
 
 }  // extern "C"
@@ -577,7 +593,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
         const size_t auxoff = align_up(xbytes, 256);
         offs[0] = auxoff + align_up(auxbytes, 256);
         for (int i = 0; i < count; i++) offs[i + 1] = offs[i] + align_up((size_t)(n * ws[i]->dev.M) * 4, 256);
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, offs[count]))) return rc;
         dx = (const float *)ctx->io_buf;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
@@ -607,7 +623,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
             const size_t t = plan_act(nullptr, mi_qmm_vec_dot_type(ws[i]->dev.type), K, n).total;
             act_need = t > act_need ? t : act_need;
         }
-        if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, act_need + align_up((size_t)n * 4, 256), ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, act_need + align_up((size_t)n * 4, 256)))) return rc;
         if (pr.kind == PRODUCE_RMSNORM) {
             float *scales = (float *)((char *)ctx->act_buf + act_need);
             HIP_TRY(launch_rms_norm(dx, nullptr, pr.eps, K, n, scales, nullptr, ctx->stream));
@@ -682,7 +698,7 @@ int stage_in(mi_qmm_ctx *ctx, int location, const void *const *src, const size_t
     }
     size_t off = 0, offs[8];
     for (int i = 0; i < n_total; i++) { offs[i] = off; off += align_up(bytes[i], 256); }
-    int rc = reserve(&ctx->io_buf, &ctx->io_cap, off, ctx->stream);
+    int rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, off);
     if (rc) return rc;
     for (int i = 0; i < n_total; i++) {
         dptr[i] = (char *)ctx->io_buf + offs[i];
@@ -747,7 +763,7 @@ int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_
     } else {
         // device caller: only the two intermediate products need room
         d[0] = const_cast<float *>(x); d[1] = const_cast<float *>(aux); d[2] = h;
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, 2 * align_up(ybytes, 256), ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, 2 * align_up(ybytes, 256)))) return rc;
         d[3] = ctx->io_buf;
         d[4] = (char *)ctx->io_buf + align_up(ybytes, 256);
     }
@@ -847,12 +863,12 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     const int tile_w = gemm_id_tile_width(w->dev.type, pairs, n_expert);
     const int64_t max_tiles = gemm ? sort_pairs_max_tiles(pairs, n_expert, tile_w) : 0, sorted_rows = tile_w * max_tiles;
     const ActPlanes probe = plan_act(nullptr, q8, K, ncols);
-    if ((rc = reserve(&ctx->act_buf, &ctx->act_cap, probe.total + align_up((size_t)ncols * 4, 256), ctx->stream))) return rc;
+    if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, probe.total + align_up((size_t)ncols * 4, 256)))) return rc;
     const ActPlanes p = plan_act(ctx->act_buf, q8, K, ncols);
     float *row_scales = (float *)((char *)ctx->act_buf + probe.total);  // RMSNorm: one scale per activation row
     const size_t hist_ints = gemm ? sort_pairs_hist_ints(pairs, n_expert) : 0;
     const size_t scratch_ints = gemm ? (size_t)(1 + 2 * max_tiles + 2 * sorted_rows) + hist_ints : gemv_id_scratch_ints(pairs);
-    if ((rc = reserve(&ctx->ws_buf, &ctx->ws_cap, scratch_ints * sizeof(int), ctx->stream))) return rc;
+    if ((rc = reserve(ctx, &ctx->ws_buf, &ctx->ws_cap, scratch_ints * sizeof(int)))) return rc;
 
     const size_t xbytes = (size_t)(ncols * K) * 4, ibytes = (size_t)pairs * 4, ybytes = (size_t)(pairs * M) * 4;
     const size_t auxbytes = !pr.aux ? 0 : pr.kind == PRODUCE_SWIGLU ? xbytes : (size_t)K * 4;
@@ -862,7 +878,7 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     if (location == MI_QMM_HOST) {
         const size_t ioff = align_up(xbytes, 256), yoff = ioff + align_up(ibytes, 256), yoff2 = yoff + align_up(ybytes, 256);
         const size_t auxoff = yoff2 + align_up(w2 ? ybytes : 0, 256);
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, auxoff + auxbytes, ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, auxoff + auxbytes))) return rc;
         if (auxbytes) {
             float *daux = (float *)((char *)ctx->io_buf + auxoff);
             HIP_TRY(hipMemcpyAsync(daux, pr.aux, auxbytes, hipMemcpyHostToDevice, ctx->stream));
@@ -1016,7 +1032,7 @@ int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const 
         return MI_QMM_OK;
     }
     // the two products into scratch of their own (mulmat_id_impl stages host operands through io_buf itself)
-    if ((rc = reserve(&ctx->pair_buf, &ctx->pair_cap, 3 * align_up(hbytes, 256), ctx->stream))) return rc;
+    if ((rc = reserve(ctx, &ctx->pair_buf, &ctx->pair_cap, 3 * align_up(hbytes, 256)))) return rc;
     float *yg = (float *)ctx->pair_buf, *yu = (float *)((char *)ctx->pair_buf + align_up(hbytes, 256));
     float *dh = location == MI_QMM_HOST ? (float *)((char *)ctx->pair_buf + 2 * align_up(hbytes, 256)) : h;
     const bool same = w_gate->dev.type == w_up->dev.type;
@@ -1099,7 +1115,7 @@ int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_
     const float *dx = x;
     if (location == MI_QMM_HOST) {
         const size_t xbytes = (size_t)(n * act->k) * 4;
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, xbytes, ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, xbytes))) return rc;
         dx = (const float *)ctx->io_buf;
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
@@ -1126,7 +1142,7 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
     float *dy = y;
     const size_t ybytes = (size_t)(n * M) * 4;
     if (location == MI_QMM_HOST) {
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, ybytes, ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, ybytes))) return rc;
         dy = (float *)ctx->io_buf;
     }
     if ((rc = run_product(ctx, w, a, dy, path))) return rc;
@@ -1196,7 +1212,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         offs[i + 1] = offs[i] + align_up((size_t)(act->n * dw[i].M) * 4, 256);
     }
     if (location == MI_QMM_HOST) {
-        if ((rc = reserve(&ctx->io_buf, &ctx->io_cap, offs[count], ctx->stream))) return rc;
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, offs[count]))) return rc;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
     if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));

@@ -25,7 +25,7 @@ EXPORTS = [
     "mi_qmm_block_size", "mi_qmm_type_size", "mi_qmm_row_size", "mi_qmm_vec_dot_type",
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync", "mi_qmm_host_alloc", "mi_qmm_host_free",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
-    "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path",
+    "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path", "mi_qmm_scratch_freeze",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
     "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_mulmat_swiglu", "mi_qmm_mulmat_id_swiglu", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
@@ -79,6 +79,7 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_quantize_act.restype = ci; L.mi_qmm_quantize_act.argtypes = [vp, ci, vp, i64, i64, vp, ci]
     L.mi_qmm_mulmat.restype = ci; L.mi_qmm_mulmat.argtypes = [vp, vp, vp, i64, vp, ci]
     L.mi_qmm_mulmat_path.restype = ci; L.mi_qmm_mulmat_path.argtypes = [vp, vp, vp, i64, vp, ci, ci]
+    L.mi_qmm_scratch_freeze.restype = ci; L.mi_qmm_scratch_freeze.argtypes = [vp, ci]
     L.mi_qmm_act_create.restype = ci; L.mi_qmm_act_create.argtypes = [vp, ci, i64, i64, ctypes.POINTER(vp)]
     L.mi_qmm_act_free.restype = None; L.mi_qmm_act_free.argtypes = [vp]
     L.mi_qmm_act_quantize.restype = ci; L.mi_qmm_act_quantize.argtypes = [vp, vp, vp, i64, ci]
@@ -294,6 +295,11 @@ class Context:
         """device pointers in and out; queued on the ctx stream, returns without waiting."""
         _check(lib().mi_qmm_mulmat_path(self._h, w._h, ctypes.c_void_p(x_ptr), n, ctypes.c_void_p(y_ptr),
                                         DEVICE, path))
+
+    def scratch_freeze(self, frozen: bool = True):
+        """while frozen, a call that would have to grow the ctx's scratch raises instead of reallocating
+        (captured HIP graphs keep the old addresses)."""
+        _check(lib().mi_qmm_scratch_freeze(self._h, 1 if frozen else 0))
 
     # ---- two-phase form -------------------------------------------------------------------------
     def act_create(self, q8_type: int, k: int, n_max: int) -> Act:

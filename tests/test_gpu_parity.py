@@ -925,3 +925,26 @@ def test_calls_from_several_threads_each_with_its_own_ctx():
     for th in threads:
         th.join(timeout=100)
     assert not errors and not any(th.is_alive() for th in threads), errors
+
+
+# ---- scratch that a captured graph points at must not move --------------------------------------
+def test_frozen_scratch_refuses_to_grow_instead_of_reallocating():
+    """A HIP graph captured after a warm-up call keeps the addresses of the ctx's scratch.  A later, larger
+    eager call used to free and reallocate that scratch; frozen, it returns an error and the buffers stay."""
+    k, m = 4096, 512
+    c = qmm.Context(0)
+    W = c.upload(Q4_K, _weights(Q4_K, m, k, 77), k, m)
+    small = np.random.default_rng(5).standard_normal((4, k), dtype=np.float32)
+    large = np.random.default_rng(6).standard_normal((600, k), dtype=np.float32)
+    try:
+        want = c.mulmat(W, small)          # warm-up: scratch sized for 4 rows
+        c.scratch_freeze(True)
+        with pytest.raises(qmm.QmmError) as e:
+            c.mulmat(W, large)             # would have to grow the activation planes
+        assert e.value.code == qmm.ERR_INVALID and "frozen" in str(e.value)
+        assert np.array_equal(c.mulmat(W, small), want)   # the frozen size still works
+        c.scratch_freeze(False)
+        assert c.mulmat(W, large).shape == (600, m)       # growth allowed again
+    finally:
+        W.free()
+        c.close()
