@@ -134,6 +134,19 @@ int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64
                   int location);
 int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n,
                        float *y, int location, int path);
+/* mi_qmm_mulmat for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): x and y are DEVICE pointers, the work is queued on
+ * the ctx's stream, and the call never allocates or frees -- neither device memory nor the ctx's growable
+ * scratch.  It has no counterpart in the reference (ggml's CPU mul_mat gets its work buffer from the
+ * caller's graph plan); it exists for those callers.  The quantized activations go to a static device
+ * array of MI_QMM_NOALLOC_SCRATCH_BYTES that each GPU the library runs on holds until the process ends;
+ * a call whose quantized activations do not fit (about n * k * 1.4 bytes for Q4_K / Q6_K weights from
+ * three or four rows up, n * k * 1.2 for Q4_0 / Q8_0; one to a few rows need no scratch at all) returns
+ * MI_QMM_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array: calls that overlap in time on
+ * one GPU (two streams, two ctxs) race.  Results are those of mi_qmm_mulmat (bit-identical, except that
+ * the tiled GEMM never cuts K into slices here, which changes the order of its fp32 sums). */
+#define MI_QMM_NOALLOC_SCRATCH_BYTES (16u << 20)
+int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y);
 /* several weights of the same k against the same f32 activations x [n][k]: ys[i] receives
  * f32 [n][m_i].  These are the mul_mat nodes of one graph that share src1 (gate and up, or q/k/v),
  * which Context.Compute (/root/reference/ml/backend.go:110) sees together.  For weights of one

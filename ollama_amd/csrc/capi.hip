@@ -39,6 +39,12 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
 
+// Scratch of the entry point that allocates nothing (mi_qmm_mulmat_noalloc): quantized activation planes live
+// here instead of in memory from hipMalloc.  Every GPU the library runs on holds its own copy of the array
+// until the process ends.  In host code the name is only a stand-in: mi_qmm_init asks for the device
+// address once per ctx (hipGetSymbolAddress, with the ctx's device current) and everything else uses that.
+static __device__ __align__(256) unsigned char scratch[MI_QMM_NOALLOC_SCRATCH_BYTES];
+
 struct mi_qmm_ctx {
     int device = 0;
     int num_cus = 0;
@@ -52,6 +58,7 @@ struct mi_qmm_ctx {
     void *ws_buf = nullptr;   size_t ws_cap = 0;   // partial sums of a K-split GEMM
     void *pair_buf = nullptr; size_t pair_cap = 0; // the two products of a gated pair when they are not one launch
     bool scratch_frozen = false;                   // mi_qmm_scratch_freeze: growth is an error, not a reallocation
+    void *static_scratch = nullptr;                // this device's copy of the file-scope array `scratch` below
 };
 
 struct mi_qmm_weight {
@@ -226,6 +233,12 @@ int mi_qmm_init(int device_ordinal, mi_qmm_ctx **out) {
         return fail(MI_QMM_ERR_HIP, "hipStreamCreate: %s", hipGetErrorString(e));
     }
     c->stream = c->own_stream;
+    e = hipGetSymbolAddress(&c->static_scratch, HIP_SYMBOL(scratch));  // device_ordinal is current (hipSetDevice above)
+    if (e != hipSuccess || !c->static_scratch) {
+        (void)hipStreamDestroy(c->own_stream);
+        delete c;
+        return fail(MI_QMM_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    }
     *out = c;
     return MI_QMM_OK;
 }
@@ -540,6 +553,39 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
 
 int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location) {
     return mi_qmm_mulmat_path(ctx, w, x, n, y, location, MI_QMM_PATH_AUTO);
+}
+
+// mi_qmm_mulmat on device pointers without any allocation: the quantized activation planes go to this
+// device's copy of the static array `scratch` (ctx->static_scratch), never to the ctx's growable buffers,
+// and the tiled GEMM runs without its K-split workspace.  Same kernels as mi_qmm_mulmat otherwise.
+int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y) {
+    if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
+    int rc = check_product_args(ctx, w, MI_QMM_DEVICE, MI_QMM_PATH_AUTO);
+    if (rc) return rc;
+    if (n == 0) return MI_QMM_OK;
+    if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
+    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    const int64_t K = w->dev.K, M = w->dev.M;
+    const int q8 = mi_qmm_vec_dot_type(w->dev.type);
+    if (n <= 8 && !wants_skinny(w->dev.type, K, M, n) && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
+        // decode: the GEMV quantizes x in its own prologue, into LDS -- no scratch at all
+        float *ys[1] = {y};
+        HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
+        return MI_QMM_OK;
+    }
+    const ActPlanes probe = plan_act(nullptr, q8, K, n);
+    if (probe.total > (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES)
+        return fail(MI_QMM_ERR_UNSUPPORTED,
+                    "n=%lld rows of k=%lld need %zu bytes of quantized activations; the static scratch of "
+                    "mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)K, probe.total,
+                    (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES);
+    const ActPlanes p = plan_act(ctx->static_scratch, q8, K, n);
+    // every plane row below n is rewritten by the quantizer; rows n.. of the last 128-row tile keep what an
+    // earlier call left there, and the GEMM drops the results of those rows
+    HIP_TRY(launch_quantize_act(q8, x, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+    DevAct a;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
+    return run_product(ctx, w, a, y, MI_QMM_PATH_AUTO, /*may_alloc=*/false);
 }
 
 int mi_qmm_scratch_freeze(mi_qmm_ctx *ctx, int frozen) {

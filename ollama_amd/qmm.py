@@ -21,11 +21,13 @@ PATH_AUTO, PATH_GEMV, PATH_GEMM = 0, 1, 2
 PRODUCE_NONE, PRODUCE_RMSNORM, PRODUCE_SWIGLU = 0, 1, 2
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, -3, -4, -5
 
+NOALLOC_SCRATCH_BYTES = 16 << 20  # MI_QMM_NOALLOC_SCRATCH_BYTES
+
 EXPORTS = [
     "mi_qmm_block_size", "mi_qmm_type_size", "mi_qmm_row_size", "mi_qmm_vec_dot_type",
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync", "mi_qmm_host_alloc", "mi_qmm_host_free",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
-    "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path", "mi_qmm_scratch_freeze",
+    "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path", "mi_qmm_mulmat_noalloc", "mi_qmm_scratch_freeze",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
     "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_mulmat_swiglu", "mi_qmm_mulmat_id_swiglu", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
@@ -79,6 +81,7 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_quantize_act.restype = ci; L.mi_qmm_quantize_act.argtypes = [vp, ci, vp, i64, i64, vp, ci]
     L.mi_qmm_mulmat.restype = ci; L.mi_qmm_mulmat.argtypes = [vp, vp, vp, i64, vp, ci]
     L.mi_qmm_mulmat_path.restype = ci; L.mi_qmm_mulmat_path.argtypes = [vp, vp, vp, i64, vp, ci, ci]
+    L.mi_qmm_mulmat_noalloc.restype = ci; L.mi_qmm_mulmat_noalloc.argtypes = [vp, vp, vp, i64, vp]
     L.mi_qmm_scratch_freeze.restype = ci; L.mi_qmm_scratch_freeze.argtypes = [vp, ci]
     L.mi_qmm_act_create.restype = ci; L.mi_qmm_act_create.argtypes = [vp, ci, i64, i64, ctypes.POINTER(vp)]
     L.mi_qmm_act_free.restype = None; L.mi_qmm_act_free.argtypes = [vp]
@@ -295,6 +298,11 @@ class Context:
         """device pointers in and out; queued on the ctx stream, returns without waiting."""
         _check(lib().mi_qmm_mulmat_path(self._h, w._h, ctypes.c_void_p(x_ptr), n, ctypes.c_void_p(y_ptr),
                                         DEVICE, path))
+
+    def mulmat_noalloc_device(self, w: Weight, x_ptr: int, n: int, y_ptr: int):
+        """mulmat_device through the entry point that never allocates (static device scratch of
+        NOALLOC_SCRATCH_BYTES; larger calls raise)."""
+        _check(lib().mi_qmm_mulmat_noalloc(self._h, w._h, ctypes.c_void_p(x_ptr), n, ctypes.c_void_p(y_ptr)))
 
     def scratch_freeze(self, frozen: bool = True):
         """while frozen, a call that would have to grow the ctx's scratch raises instead of reallocating
