@@ -895,9 +895,8 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     if (n_tokens == 0) return MI_QMM_OK;
     if (!x || !ids || !y || (w2 && !y2)) return fail(MI_QMM_ERR_INVALID, "x, ids or y is NULL");
     const int64_t pairs = (int64_t)n_used * n_tokens, ncols = (int64_t)b_cols * n_tokens;
-    if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24) || K > gemv_max_k(w->dev.type))
-        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts, 2^24 pairs and k <= %lld for type %d",
-                    (long long)gemv_max_k(w->dev.type), w->dev.type);
+    if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts and 2^24 pairs");
     if (location == MI_QMM_HOST)
         for (int64_t p = 0; p < pairs; p++)
             if (ids[p] < 0 || ids[p] >= n_expert)
@@ -967,6 +966,10 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     // the matrix-core kernel addresses activation bytes with 32-bit offsets
     const bool skinny32 = skinny32_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32);
     const bool skinny = skinny32 || (skinny_id_supports(w->dev.type, K, M, pairs, n_expert) && ncols * K < ((int64_t)1 << 32));
+    // only the streaming kernels have a row-length limit (the sorted GEMM and the matrix-core kernels walk any K)
+    if (!skinny && K > gemv_max_k(w->dev.type))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id with this few pairs per expert streams the rows: k <= %lld for type %d",
+                    (long long)gemv_max_k(w->dev.type), w->dev.type);
     const bool fused = !skinny && pr.kind != PRODUCE_RMSNORM &&
                        gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert, pr.kind == PRODUCE_SWIGLU);
     if (!fused) {
@@ -1053,16 +1056,16 @@ int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const 
     if (n_tokens == 0) return MI_QMM_OK;
     if (!x || !ids || !h) return fail(MI_QMM_ERR_INVALID, "x, ids or h is NULL");
     const int64_t pairs = (int64_t)n_used * n_tokens, ncols = (int64_t)b_cols * n_tokens;
-    if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24) || K > gemv_max_k(w_gate->dev.type))
-        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts, 2^24 pairs and k <= %lld for type %d",
-                    (long long)gemv_max_k(w_gate->dev.type), w_gate->dev.type);
+    if (n_expert > 4096 || pairs > (1 << 24) || ncols > (1 << 24))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "mulmat_id covers up to 4096 experts and 2^24 pairs");
     if (location == MI_QMM_HOST)
         for (int64_t p = 0; p < pairs; p++)
             if (ids[p] < 0 || ids[p] >= n_expert)
                 return fail(MI_QMM_ERR_INVALID, "ids[%lld] = %d is outside 0..%d", (long long)p, ids[p], n_expert - 1);
     // decode-sized and both stacks of one type: one launch with the gating in its epilogue; else the two products
     // (which share their quantization and, at decode size, their launch) and the gating kernel
-    const bool paired = w_gate->dev.type == w_up->dev.type && gemv_id_f32_supported(w_gate->dev.type, K, 2 * M, pairs, n_expert);
+    const bool paired = w_gate->dev.type == w_up->dev.type && K <= gemv_max_k(w_gate->dev.type) &&
+                        gemv_id_f32_supported(w_gate->dev.type, K, 2 * M, pairs, n_expert);
     const size_t hbytes = (size_t)(pairs * M) * 4;
     const size_t bytes[5] = {(size_t)(ncols * K) * 4, (size_t)pairs * 4, hbytes, paired ? 0 : hbytes, paired ? 0 : hbytes};
     const void *src[5] = {x, ids, h, nullptr, nullptr};
@@ -1201,6 +1204,7 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
 
 int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const mi_qmm_act *act,
                            float *const *ys, int location) {
+    if (!ctx) return fail(MI_QMM_ERR_INVALID, "ctx is NULL");  // ctx->num_cus is read before check_product_args below
     if (!ws || !ys || count < 1) return fail(MI_QMM_ERR_INVALID, "ws/ys is NULL or count < 1");
     if (!act) return fail(MI_QMM_ERR_INVALID, "act is NULL");
     for (int i = 0; i < count; i++)
@@ -1211,7 +1215,10 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     bool gemm_ok = same && count <= gemm_max_multi() && act->n >= 32;
     int64_t tiles = 0;
     for (int i = 0; gemm_ok && i < count; i++) {
-        gemm_ok = gemm_supports(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M);
+        // a weight that would be cut into K slices in a launch of its own (long rows, few tiles) keeps that cut:
+        // the joint launch never slices, and the order of the fp32 sums must not depend on how a product was asked for
+        gemm_ok = gemm_supports(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M) &&
+                  gemm_workspace_floats(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n, ctx->num_cus) == 0;
         tiles += (ws[i]->dev.M + 127) / 128 * ((act->n + 127) / 128);
     }
     // one launch pays when the tensors are too small to fill the machine one by one (q, k, v); large

@@ -47,6 +47,9 @@ def test_argument_errors_without_a_device():
     assert L.mi_qmm_init(0, None) == qmm.ERR_INVALID
     assert L.mi_qmm_sync(None) == qmm.ERR_INVALID and "NULL" in qmm.last_error()
     assert L.mi_qmm_mulmat(None, None, None, 1, None, 0) == qmm.ERR_INVALID
+    assert L.mi_qmm_mulmat_q8_multi(None, None, 1, None, None, 0) == qmm.ERR_INVALID and "ctx is NULL" in qmm.last_error()
+    assert L.mi_qmm_mulmat_noalloc(None, None, None, 1, None) == qmm.ERR_INVALID
+    assert L.mi_qmm_scratch_freeze(None, 1) == qmm.ERR_INVALID
     assert L.mi_qmm_weight_upload(None, 13, None, 256, 1, 0, ctypes.byref(h)) == qmm.ERR_UNSUPPORTED
     assert L.mi_qmm_weight_upload(None, qmm.Q4_K, None, 100, 1, 0, ctypes.byref(h)) == qmm.ERR_INVALID
     assert "multiple of the block size" in qmm.last_error()

@@ -167,7 +167,21 @@ def _config_case(ctx, t, m, k, ns, seed_w, seed_x):
         nrm = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
         assert err <= TOL, f"{NAMES[t]} {m}x{k} n={n}: rel err {err}, normwise {nrm}"
         assert nrm <= 1e-5
+        _check_against_exact_arithmetic(t, w_raw, k, m, x, got, f"{NAMES[t]} {m}x{k} n={n}")
     W.free()
+
+
+def _check_against_exact_arithmetic(t, w_raw, k, m, x, got, what, max_rows=16384):
+    """The GPU's integer block sums are exact, so against fp64 arithmetic on the same quantized operands it is
+    held to the tighter floor, 1e-3 of the output RMS (the scalar oracle, whose sequential fp32 sums carry
+    their own noise, binds the comparison above at the 1e-2 floor).  Large matrices: the first max_rows rows."""
+    rows = min(m, max_rows)
+    qt = qmm.vec_dot_type(t)
+    n = x.shape[0]
+    w_slab = np.ascontiguousarray(w_raw.reshape(m, -1)[:rows]).reshape(-1)
+    exact = npref.matmul_f64(t, w_slab, k, rows, qt, oracle.quantize(qt, x, nthreads=8), n)
+    err = npref.rel_err(got[:, :rows], exact, floor=1e-3)
+    assert err <= TOL, f"{what}: rel err {err} against exact arithmetic at the 1e-3 floor"
 
 
 def test_config1_q4_0_gemv(ctx):
@@ -490,6 +504,7 @@ def test_config5_prefill_layer_batch512(ctx, name, t, m, k):
     err = npref.rel_err(got, want)
     nrm = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
     assert err <= TOL and nrm <= 1e-5, f"{name}: rel err {err}, normwise {nrm}"
+    _check_against_exact_arithmetic(t, w_raw, k, m, x, got, name, max_rows=4096)
     W.free()
 
 
@@ -948,3 +963,74 @@ def test_frozen_scratch_refuses_to_grow_instead_of_reallocating():
     finally:
         W.free()
         c.close()
+
+
+# ---- exactly what bench.py times ---------------------------------------------------------------------
+def test_the_benchmark_step_at_full_size(ctx):
+    """bench.py's step on device pointers: gate and up (2 x 14336 x 4096, one launch through
+    mi_qmm_mulmat_multi) and down (4096 x 14336, mi_qmm_mulmat), one f32 activation row each, against the oracle"""
+    kf, mf = 4096, 14336
+    raws = {"gate": _weights(Q4_K, mf, kf, 1003), "up": _weights(Q4_K, mf, kf, 1013), "down": _weights(Q4_K, kf, mf, 1023)}
+    Ws = {n: ctx.upload(Q4_K, r, kf if n != "down" else mf, mf if n != "down" else kf) for n, r in raws.items()}
+    rng = np.random.default_rng(2003)
+    x = rng.standard_normal((1, kf), dtype=np.float32)
+    h = rng.standard_normal((1, mf), dtype=np.float32)
+    dx, dh = DeviceArray(x), DeviceArray(h)
+    yg, yu = DeviceArray(np.empty((1, mf), np.float32), zero=True), DeviceArray(np.empty((1, mf), np.float32), zero=True)
+    yd = DeviceArray(np.empty((1, kf), np.float32), zero=True)
+    try:
+        ctx.mulmat_multi_device([Ws["gate"], Ws["up"]], dx.ptr, 1, [yg.ptr, yu.ptr])
+        ctx.mulmat_device(Ws["down"], dh.ptr, 1, yd.ptr)
+        ctx.sync()
+        for name, got, act, k, m in (("gate", yg.numpy(), x, kf, mf), ("up", yu.numpy(), x, kf, mf), ("down", yd.numpy(), h, mf, kf)):
+            want = oracle.mul_mat(Q4_K, raws[name], k, m, act, nthreads=16)
+            assert npref.rel_err(got, want) <= TOL, name
+            _check_against_exact_arithmetic(Q4_K, raws[name], k, m, act, got, "bench " + name)
+    finally:
+        for b in (dx, dh, yg, yu, yd):
+            b.free()
+        for W in Ws.values():
+            W.free()
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("k,n", [(8192, 40), (14336, 128), (14336, 40)])
+def test_multi_weight_gemm_keeps_the_k_cut_of_single_calls(ctx, t, k, n):
+    """Long rows and few output tiles: a product asked for alone is cut into K slices, so a joint launch (which
+    never slices) must not be taken for it -- the bits of a result may not depend on how it was asked for."""
+    ms = [512, 256]
+    Ws = [ctx.upload(t, _weights(t, m, k, seed=300 + m + k), k, m) for m in ms]
+    act = ctx.act_create(qmm.vec_dot_type(t), k, n)
+    x = np.random.default_rng(k + n).standard_normal((n, k), dtype=np.float32)
+    try:
+        ctx.act_quantize(act, x)
+        want = [ctx.mulmat_q8(W, act) for W in Ws]
+        for y, wnt in zip(ctx.mulmat_q8_multi(Ws, act), want):
+            assert np.array_equal(y, wnt)
+        for y, wnt in zip(ctx.mulmat_multi(Ws, x), want):
+            assert np.array_equal(y, wnt)
+    finally:
+        act.free()
+        for W in Ws:
+            W.free()
+
+
+def test_mulmat_id_rows_longer_than_the_streaming_limit_on_the_expert_gemm(ctx):
+    """K above what the streaming kernels walk (32 segments): fine for the sorted expert GEMM, refused only where
+    a call would fall to the streaming kernels"""
+    t, n_expert, m, k = Q4_K, 2, 48, 131072 + 256
+    raw = _experts(t, n_expert, m, k, 91)
+    W = ctx.upload(t, raw, k, n_expert * m)
+    rng = np.random.default_rng(92)
+    tokens = 40  # 20 pairs per expert: the sorted GEMM
+    x = rng.standard_normal((tokens, 1, k), dtype=np.float32)
+    ids = (np.arange(tokens, dtype=np.int32) % n_expert).reshape(tokens, 1)
+    try:
+        got = ctx.mulmat_id(W, n_expert, x, ids)
+        want = oracle.mul_mat_id(t, raw, k, m, n_expert, x, ids)
+        assert npref.rel_err(got, want) <= TOL
+        with pytest.raises(qmm.QmmError) as e:   # one pair: the streaming kernel, which cannot walk such a row
+            ctx.mulmat_id(W, n_expert, x[:1], ids[:1])
+        assert e.value.code == qmm.ERR_UNSUPPORTED
+    finally:
+        W.free()
