@@ -29,11 +29,35 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+
+def rel_err(y, ref, floor=1e-2):
+    """max |y - ref| / max(|ref|, floor * rms(ref)): the path's tolerance metric (bar 1e-3)"""
+    import numpy as np
+    y, ref = np.asarray(y, np.float64), np.asarray(ref, np.float64)
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    return float(np.max(np.abs(y - ref) / np.maximum(np.abs(ref), floor * rms + 1e-300)))
+
+
+def observed_clocks():
+    """current shader / memory clock as rocm-smi reports them right now (None where it cannot be read)"""
+    import re
+    import subprocess
+    try:
+        txt = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+    except Exception:
+        return None
+    out = {}
+    for key in ("sclk", "mclk", "fclk"):
+        m = re.search(key + r" clock level: \S+ \((\d+)Mhz\)", txt)
+        if m:
+            out[key + "_mhz"] = int(m.group(1))
+    return out or None
+
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
 
 Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 2, 8, 12, 14, 15
-GATE_UP_HBM_TRAFFIC_BYTES = 66386719  # measured, see the roofline block below
+TRAFFIC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "gate_up_traffic.json")
 FFN_K, FFN_M = 4096, 14336
 
 
@@ -126,8 +150,34 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     t_step = timed(step, args.steps)
+    clocks_under_load = observed_clocks()
     bytes_per_step = args.layers * (2 * alg_bytes(wbytes, FFN_K, FFN_M) + alg_bytes(wbytes, FFN_M, FFN_K))
     value = bytes_per_step * args.steps / t_step / 1e9
+    # the same step again, every step between events of its own: median and best next to the mean above
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    torch.cuda.synchronize()
+    evs[0].record(stream)
+    for i in range(args.steps):
+        step()
+        evs[i + 1].record(stream)
+    torch.cuda.synchronize()
+    per_step_ms = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
+    median_ms, best_ms = per_step_ms[len(per_step_ms) // 2], per_step_ms[0]
+
+    # ---- the timed launches did the work: the outputs of the last step (the last pool entry's weights) against
+    # the CPU oracle on a slab of rows, outside the timed region
+    import oracle
+    last = args.layers - 1
+    slab = 64
+    checks = {}
+    for name, yt, act, k, m in (("gate", y_gate, x, FFN_K, FFN_M), ("up", y_up, x, FFN_K, FFN_M), ("down", y_down, h, FFN_M, FFN_K)):
+        raw = np.roll(base[name], last * 37, axis=0) if last else base[name]
+        want = oracle.mul_mat(Q4_K, np.ascontiguousarray(raw[:slab]), k, slab, act.cpu().numpy(), nthreads=4)
+        err = rel_err(yt.cpu().numpy()[:, :slab], want)
+        checks[name] = err
+        if not err <= 1e-3:
+            print(f"bench.py: y_{name} of the timed step differs from the oracle (rel err {err})", file=sys.stderr)
+            return 1
 
     # dominant kernel alone, back to back (HIP events on the stream the kernels run on)
     gate_up_only()
@@ -137,6 +187,10 @@ def main() -> int:
     bytes_per_launch = 2 * wbytes + 4 * FFN_K + 2 * 4 * FFN_M  # two weight matrices, x once, two outputs
     achieved = bytes_per_launch / avg_launch_s / 1e9
 
+    traffic_bytes = None
+    if os.path.exists(TRAFFIC_SUMMARY):
+        with open(TRAFFIC_SUMMARY) as f:
+            traffic_bytes = json.load(f).get("hbm_bytes_per_launch")
     out = {
         "metric": "Q4_K decode GEMV GB/s",
         "value": round(value, 1),
@@ -145,6 +199,8 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(t_step / args.steps * 1e3, 4),
+        "ms_per_step_median": round(median_ms, 4),
+        "ms_per_step_best": round(best_ms, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -158,7 +214,9 @@ def main() -> int:
             "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
             "device": info["name"],
             "compute_units": info["compute_units"],
-            "clock_mhz": info["clock_mhz"],
+            "clock_mhz_nominal": info["clock_mhz"],
+            "clocks_observed_under_load": clocks_under_load,
+            "outputs_checked_against_oracle": {k_: float(f"{v_:.2e}") for k_, v_ in checks.items()},
         },
         "roofline": {
             "bound": "hbm",
@@ -167,9 +225,9 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # HBM bytes per launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE x 2.000 and
-            # WRITE_SIZE x 1.000, factors from a 1 GiB copy): 32,354.41 KiB x 2 + 112.02 KiB
-            "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
+            # HBM bytes per launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE and WRITE_SIZE, scaled by
+            # what the same counters read for a 1 GiB copy); the figures and their commands are in the tracked summary
+            "traffic": traffic_bytes,
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
             "bytes_per_launch": int(bytes_per_launch),
         },
@@ -396,8 +454,6 @@ def main() -> int:
 
     # ---- CPU baseline: the oracle (scalar port of the ggml CPU path) on this host's cores -------
     if args.cpu_seconds > 0:
-        import oracle
-
         xh = x.cpu().numpy()
 
         def cpu_rate(threads, seconds):

@@ -77,6 +77,7 @@ struct mi_qmm_act {
     int type = 0;
     int64_t k = 0, n_max = 0, n = 0;
     void *base = nullptr;
+    bool f16 = false;  // carries the fp16 planes of the fp16-MFMA GEMM
 };
 
 namespace {
@@ -102,10 +103,13 @@ int reserve(mi_qmm_ctx *ctx, void **buf, size_t *cap, size_t need) {
     return MI_QMM_OK;
 }
 
-struct ActPlanes { int8_t *qs; float *d; int16_t *bsums; uint8_t *sd8; uint8_t *sd16; size_t total; };
+struct ActPlanes { int8_t *qs; float *d; int16_t *bsums; uint8_t *sd8; uint8_t *sd16; uint16_t *qf; uint16_t *bsf; size_t total; };
+
+// fp16 planes for the fp16-MFMA GEMM: wanted where a Q4_K weight may meet a batch that kernel takes
+bool wants_f16_planes(int weight_type, int64_t n) { return weight_type == T_Q4_K && n >= 32; }
 
 // carve the activation scratch into planes for N rows of K elements
-ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N) {
+ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N, bool f16 = false) {
     // the GEMM reads Q8_K activation rows in tiles of 128 without bounds checks (results of rows past
     // N are dropped), so the planes are sized in whole tiles
     if (q8_type == T_Q8_K) N = (N + 127) / 128 * 128;
@@ -120,6 +124,11 @@ ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N) {
     if (q8_type == T_Q8_K) {  // block-sum digit planes read by the MFMA GEMM
         p.sd8 = (uint8_t *)base + off;  off = align_up(off + (size_t)(N * (K / QKK)) * 16, 256);
         p.sd16 = (uint8_t *)base + off; off = align_up(off + (size_t)(N * (K / QKK)) * 32, 256);
+    }
+    p.qf = p.bsf = nullptr;
+    if (q8_type == T_Q8_K && f16) {
+        p.qf = (uint16_t *)((char *)base + off);  off = align_up(off + (size_t)(N * K) * 2, 256);
+        p.bsf = (uint16_t *)((char *)base + off); off = align_up(off + (size_t)(N * (K / QKK)) * 32, 256);
     }
     p.total = off;
     return p;
@@ -463,6 +472,8 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
                     (long long)gemv_max_k(w->dev.type), w->dev.type);
     if (use_gemm && blk32) {
         HIP_TRY(launch_gemm_blk32(w->dev, a, dy, ctx->num_cus, ctx->stream));
+    } else if (use_gemm && path == MI_QMM_PATH_AUTO && gemm_f16_wanted(w->dev, a, ctx->num_cus)) {
+        HIP_TRY(launch_gemm_f16(w->dev, a, dy, ctx->stream));
     } else if (use_gemm) {
         const size_t wsf = may_alloc ? gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus) : 0;
         if (wsf) {
@@ -519,9 +530,10 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
 
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
-    const ActPlanes probe = plan_act(nullptr, q8, K, n);
+    const bool f16 = wants_f16_planes(w->dev.type, n);
+    const ActPlanes probe = plan_act(nullptr, q8, K, n, f16);
     if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, probe.total))) return rc;
-    const ActPlanes p = plan_act(ctx->act_buf, q8, K, n);
+    const ActPlanes p = plan_act(ctx->act_buf, q8, K, n, f16);
 
     const size_t xbytes = (size_t)(n * K) * 4, ybytes = (size_t)(n * M) * 4;
     const float *dx = x;
@@ -539,9 +551,9 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         float *ys[1] = {dy};
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
     } else {
-        HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+        HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream, nullptr, p.qf, p.bsf));
         DevAct a;
-        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
+        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = K; a.N = (int)n; a.type = q8;
         if ((rc = run_product(ctx, w, a, dy, path))) return rc;
     }
     if (location == MI_QMM_HOST) {
@@ -573,18 +585,19 @@ int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
         return MI_QMM_OK;
     }
-    const ActPlanes probe = plan_act(nullptr, q8, K, n);
+    const bool f16 = wants_f16_planes(w->dev.type, n);
+    const ActPlanes probe = plan_act(nullptr, q8, K, n, f16);
     if (probe.total > (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES)
         return fail(MI_QMM_ERR_UNSUPPORTED,
                     "n=%lld rows of k=%lld need %zu bytes of quantized activations; the static scratch of "
                     "mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)K, probe.total,
                     (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES);
-    const ActPlanes p = plan_act(ctx->static_scratch, q8, K, n);
+    const ActPlanes p = plan_act(ctx->static_scratch, q8, K, n, f16);
     // every plane row below n is rewritten by the quantizer; rows n.. of the last 128-row tile keep what an
     // earlier call left there, and the GEMM drops the results of those rows
-    HIP_TRY(launch_quantize_act(q8, x, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+    HIP_TRY(launch_quantize_act(q8, x, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream, nullptr, p.qf, p.bsf));
     DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = K; a.N = (int)n; a.type = q8;
     return run_product(ctx, w, a, y, MI_QMM_PATH_AUTO, /*may_alloc=*/false);
 }
 
@@ -665,8 +678,10 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
         // x is produced and quantized once per activation format (Q8_0 / Q8_K) in use; weights of one type
         // then share GEMV launches four at a time, everything else goes out one product at a time
         size_t act_need = 0;
+        bool f16 = false;
+        for (int i = 0; i < count; i++) f16 = f16 || wants_f16_planes(ws[i]->dev.type, n);
         for (int i = 0; i < count; i++) {
-            const size_t t = plan_act(nullptr, mi_qmm_vec_dot_type(ws[i]->dev.type), K, n).total;
+            const size_t t = plan_act(nullptr, mi_qmm_vec_dot_type(ws[i]->dev.type), K, n, f16).total;
             act_need = t > act_need ? t : act_need;
         }
         if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, act_need + align_up((size_t)n * 4, 256)))) return rc;
@@ -680,11 +695,11 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
             for (int i = 0; i < count; i++)
                 if (mi_qmm_vec_dot_type(ws[i]->dev.type) == q8) idx.push_back(i);
             if (idx.empty()) continue;
-            const ActPlanes p = plan_act(ctx->act_buf, q8, K, n);
+            const ActPlanes p = plan_act(ctx->act_buf, q8, K, n, f16);
             HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream,
-                                        pr.kind == PRODUCE_NONE ? nullptr : &pr));
+                                        pr.kind == PRODUCE_NONE ? nullptr : &pr, p.qf, p.bsf));
             DevAct a;
-            a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = K; a.N = (int)n; a.type = q8;
+            a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = K; a.N = (int)n; a.type = q8;
             size_t j = 0;
             while (j < idx.size()) {
                 const mi_qmm_weight *w0 = ws[idx[j]];
@@ -951,7 +966,7 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
                                   hist_ints ? out_pair + sorted_rows : nullptr, ctx->stream));
         HIP_TRY(quantize());
         DevAct as;
-        as.qs = p.qs; as.d = p.d; as.bsums = p.bsums; as.sd8 = p.sd8; as.sd16 = p.sd16; as.K = K; as.N = (int)ncols; as.type = q8;
+        as.qs = p.qs; as.d = p.d; as.bsums = p.bsums; as.sd8 = p.sd8; as.sd16 = p.sd16; as.qf = p.qf; as.bsf = p.bsf; as.K = K; as.N = (int)ncols; as.type = q8;
         HIP_TRY(launch_gemm_id(w->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, tile_w, dy, ctx->stream));
         if (w2) HIP_TRY(launch_gemm_id(w2->dev, n_expert, as, tiles, src_col, out_pair, max_tiles, tile_w, dy2, ctx->stream));
         if (location == MI_QMM_HOST) {
@@ -974,7 +989,7 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
                        gemv_id_f32_supported(w->dev.type, K, M, pairs, n_expert, pr.kind == PRODUCE_SWIGLU);
     if (!fused) {
         HIP_TRY(quantize());
-        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16;
+        a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf;
     }
     if (skinny32) {
         HIP_TRY(launch_skinny32_id(w->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy, (int *)ctx->ws_buf,
@@ -1128,7 +1143,8 @@ int mi_qmm_act_create(mi_qmm_ctx *ctx, int q8_type, int64_t k, int64_t n_max, mi
     mi_qmm_act *a = new (std::nothrow) mi_qmm_act();
     if (!a) return fail(MI_QMM_ERR_NOMEM, "host allocation failed");
     a->device = ctx->device; a->type = q8_type; a->k = k; a->n_max = n_max;
-    const ActPlanes probe = plan_act(nullptr, q8_type, k, n_max);
+    a->f16 = q8_type == T_Q8_K && n_max >= 32;  // any Q4_K weight may meet these rows: keep the fp16 planes too
+    const ActPlanes probe = plan_act(nullptr, q8_type, k, n_max, a->f16);
     hipError_t e = hipMalloc(&a->base, probe.total + 256);
     if (e != hipSuccess) {
         delete a;
@@ -1160,7 +1176,7 @@ int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_
     if (n == 0) return MI_QMM_OK;
     if (!x) return fail(MI_QMM_ERR_INVALID, "x is NULL");
     // planes are carved for n_max so their addresses do not move between calls
-    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
+    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max, act->f16);
     const float *dx = x;
     if (location == MI_QMM_HOST) {
         const size_t xbytes = (size_t)(n * act->k) * 4;
@@ -1168,7 +1184,7 @@ int mi_qmm_act_quantize(mi_qmm_ctx *ctx, mi_qmm_act *act, const float *x, int64_
         dx = (const float *)ctx->io_buf;
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    HIP_TRY(launch_quantize_act(act->type, dx, act->k, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream));
+    HIP_TRY(launch_quantize_act(act->type, dx, act->k, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream, nullptr, p.qf, p.bsf));
     if (location == MI_QMM_HOST) HIP_TRY(hipStreamSynchronize(ctx->stream));  // x may be reused by the caller
     return MI_QMM_OK;
 }
@@ -1185,9 +1201,9 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
     const int64_t n = act->n, M = w->dev.M;
     if (n == 0) return MI_QMM_OK;
     if (!y) return fail(MI_QMM_ERR_INVALID, "y is NULL");
-    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
+    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max, act->f16);
     DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = act->k; a.N = (int)n; a.type = act->type;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = act->k; a.N = (int)n; a.type = act->type;
     float *dy = y;
     const size_t ybytes = (size_t)(n * M) * 4;
     if (location == MI_QMM_HOST) {
@@ -1224,6 +1240,13 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     // one launch pays when the tensors are too small to fill the machine one by one (q, k, v); large
     // ones (gate, up) run slightly faster back to back
     gemm_ok = gemm_ok && 2 * tiles < 3 * (int64_t)ctx->num_cus;
+    if (gemm_ok && act->f16) {  // a weight that the fp16 GEMM takes in a launch of its own keeps that kernel
+        DevAct probe;
+        probe.qs = nullptr; probe.d = nullptr; probe.bsums = nullptr; probe.sd8 = probe.sd16 = nullptr;
+        probe.K = act->k; probe.N = (int)act->n; probe.type = act->type;
+        probe.qf = probe.bsf = reinterpret_cast<const uint16_t *>(act->base);  // presence is all that is read
+        for (int i = 0; gemm_ok && i < count; i++) gemm_ok = !gemm_f16_wanted(ws[i]->dev, probe, ctx->num_cus);
+    }
     bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
     for (int i = 0; gemv_ok && i < count; i++)  // from five or six columns up each weight goes to the skinny kernel
         gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n);
@@ -1250,9 +1273,9 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         return fail(MI_QMM_ERR_INVALID, "act (type %d, k=%lld) does not match the weights (type %d, k=%lld)",
                     act->type, (long long)act->k, ws[0]->dev.type, (long long)ws[0]->dev.K);
     if (act->n == 0) return MI_QMM_OK;
-    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max);
+    const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max, act->f16);
     DevAct a;
-    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.K = act->k; a.N = (int)act->n; a.type = act->type;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = act->k; a.N = (int)act->n; a.type = act->type;
     DevWeight dw[8];
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);

@@ -43,6 +43,10 @@ struct DevWeight {
 // Q8_K only, for the MFMA GEMM (block sums as two int8 digits, S = 64*S_h + S_l, S_l in 0..63):
 //   sd8   [N][K/256][16]   S_j = bsums[2j] + bsums[2j+1], j = 0..7:  bytes [S_l(0..7) | S_h(0..7)]
 //   sd16  [N][K/256][32]   S_g = bsums[g], g = 0..15:                bytes [S_l(0..15) | S_h(0..15)]
+// Q8_K only, for the fp16-MFMA GEMM (null when not planned):
+//   qf    [N][K]           the quants as fp16 numbers; inside every group of 32, element 16h + 8u + j sits at
+//                          16u + 8h + p(j), p = 0 2 1 3 4 6 5 7 (the order the GEMM expands weight nibbles in)
+//   bsf   [N][K/256][16]   bsums as fp16 numbers (|sum of 16 quants| <= 2048: exact)
 struct DevAct {
     const int8_t *qs;
     const float *d;
@@ -52,6 +56,8 @@ struct DevAct {
     int64_t K;
     int N;
     int type;  // T_Q8_0 or T_Q8_K
+    const uint16_t *qf = nullptr;
+    const uint16_t *bsf = nullptr;
 };
 
 }  // namespace miqmm

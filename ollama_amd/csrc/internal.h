@@ -12,9 +12,10 @@ namespace miqmm {
 // kernel 1: f32 rows -> Q8_0 / Q8_K planes (bit-exact with the scalar CPU quantizers)
 // sd8 / sd16: block-sum digit planes for the GEMM (Q8_K only; may be null)
 // produce (optional): applied to x on the fly (RMSNORM needs row_scale from launch_rms_norm first)
+// qf / bsf: quants and block sums as fp16 planes for the fp16-MFMA GEMM (Q8_K only; both or neither)
 hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs,
                                float *d, int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s,
-                               const Produce *produce = nullptr);
+                               const Produce *produce = nullptr, uint16_t *qf = nullptr, uint16_t *bsf = nullptr);
 // RMSNorm over rows of K floats: scale_out [N] (optional) = 1/sqrtf(mean(x^2)+eps) per row; y (optional) =
 // (x * scale) * g with g [K] or null.  SwiGLU: y = silu(gate) * up over count floats.
 hipError_t launch_rms_norm(const float *x, const float *g, float eps, int64_t K, int64_t N, float *scale_out, float *y,
@@ -87,6 +88,10 @@ size_t gemm_workspace_floats(int type, int64_t K, int64_t M, int64_t N, int num_
 hipError_t launch_gemm_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, float *workspace,
                              size_t workspace_floats, int num_cus, hipStream_t s);
 int gemm_max_multi();
+// kernel 3b: fp16-MFMA GEMM for Q4_K weights on products with enough 256 x 128 output tiles to fill the GPU;
+// a needs the fp16 planes (qf, bsf).  y[n*M + m].  gemm_f16_wanted() depends on the weight and the batch only.
+bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus);
+hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, hipStream_t s);
 // 1..16 activation columns (col0 .. col0+ncols-1 of a) on the matrix cores, K-quants; y[n*M + m]
 bool skinny_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,

@@ -61,7 +61,8 @@ template <int KIND>
 __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__restrict__ x,
                                                             int *__restrict__ qs, float *__restrict__ d,
                                                             int16_t *__restrict__ bsums, uint8_t *__restrict__ sd8,
-                                                            uint8_t *__restrict__ sd16, int64_t nblk, Produce pr,
+                                                            uint8_t *__restrict__ sd16, uint16_t *__restrict__ qf,
+                                                            uint16_t *__restrict__ bsf, int64_t nblk, Produce pr,
                                                             int64_t k4) {
     const int lane = threadIdx.x & 63;
     const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // 256 threads per workgroup (launch_quantize_act)
@@ -83,6 +84,16 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(const float4 *__rest
     if (sd8 && (lane & 7) == 0) {
         sd8[blk * 16 + (lane >> 3)] = (uint8_t)(pair & 63);
         sd8[blk * 16 + 8 + (lane >> 3)] = (uint8_t)(pair >> 6);
+    }
+    // the quants and block sums as fp16 numbers for the fp16-MFMA GEMM.  This lane holds elements 4 (lane & 7) + i of
+    // group lane >> 3; element 16h + 8u + j of a group goes to 16u + 8h + p(j), p = 0 2 1 3 4 6 5 7.
+    if (qf) {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        const h4 v4 = {(_Float16)(float)(int8_t)packed, (_Float16)(float)(int8_t)(packed >> 16),
+                       (_Float16)(float)(int8_t)(packed >> 8), (_Float16)(float)(packed >> 24)};
+        const int at = 32 * (lane >> 3) + 16 * ((lane >> 1) & 1) + 8 * ((lane >> 2) & 1) + 4 * (lane & 1);
+        *reinterpret_cast<h4 *>(qf + blk * QKK + at) = v4;
+        if ((lane & 3) == 0) bsf[blk * 16 + (lane >> 2)] = __half_as_ushort(__float2half_rn((float)sum));
     }
 }
 
@@ -161,8 +172,10 @@ __global__ void pack_q8_K_kernel(const int8_t *__restrict__ qs, const float *__r
 }  // namespace
 
 hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N, int8_t *qs, float *d,
-                               int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s, const Produce *produce) {
+                               int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s, const Produce *produce,
+                               uint16_t *qf, uint16_t *bsf) {
     if (N * K == 0) return hipSuccess;
+    if ((qf != nullptr) != (bsf != nullptr)) return hipErrorInvalidValue;
     Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
     if (produce) pr = *produce;
     if ((pr.kind == PRODUCE_RMSNORM && !pr.row_scale) || (pr.kind == PRODUCE_SWIGLU && !pr.aux) ||
@@ -180,9 +193,9 @@ hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N
     } else if (q8_type == T_Q8_K) {
         const int64_t nblk = N * K / QKK;
         const unsigned grid = (unsigned)((nblk + 3) / 4);
-        if (pr.kind == PRODUCE_RMSNORM) quantize_q8_K_kernel<PRODUCE_RMSNORM><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, nblk, pr, k4);
-        else if (pr.kind == PRODUCE_SWIGLU) quantize_q8_K_kernel<PRODUCE_SWIGLU><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, nblk, pr, k4);
-        else quantize_q8_K_kernel<PRODUCE_NONE><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, nblk, pr, k4);
+        if (pr.kind == PRODUCE_RMSNORM) quantize_q8_K_kernel<PRODUCE_RMSNORM><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, qf, bsf, nblk, pr, k4);
+        else if (pr.kind == PRODUCE_SWIGLU) quantize_q8_K_kernel<PRODUCE_SWIGLU><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, qf, bsf, nblk, pr, k4);
+        else quantize_q8_K_kernel<PRODUCE_NONE><<<grid, 256, 0, s>>>(x4, (int *)qs, d, bsums, sd8, sd16, qf, bsf, nblk, pr, k4);
     } else {
         return hipErrorInvalidValue;
     }

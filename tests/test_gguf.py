@@ -186,3 +186,37 @@ def test_expert_stack_tensors_and_array_buffers_round_trip(tmp_path):
         assert tb.Shape == [256, 5, 2] and tb.NumBytes == b.size and tb.Offset == (a.size + 31) // 32 * 32
         assert f.TensorBytes(ta.Name).tobytes() == a.tobytes()
         assert f.TensorBytes(tb.Name).tobytes() == b.tobytes()
+
+
+def test_hand_packed_file_pins_offsets_and_bytes(tmp_path):
+    """A valid file packed field by field here (no writer of this repository involved, so a layout mistake shared
+    by writer and reader cannot hide): two key-values, one of them a string array, general.alignment = 64, a Q4_K
+    and an F32 tensor.  Layout per /root/reference/fs/gguf/gguf.go:54-110 (header, key-values, tensor infos, data
+    offset = header end rounded up to the alignment) and :388-430 (a tensor's bytes start at data offset + its
+    offset and run for its byte size)."""
+    rng = np.random.default_rng(12)
+    q4k = rng.integers(0, 256, 2 * 144, dtype=np.uint8).tobytes()          # 2 rows of 256 elements: 2 x 144 bytes
+    f32 = np.arange(5, dtype="<f4").tobytes()                              # 5 floats: 20 bytes
+    body = b"GGUF" + struct.pack("<I", 3) + struct.pack("<Q", 2) + struct.pack("<Q", 2)
+    body += _s("general.alignment") + struct.pack("<I", 4) + struct.pack("<I", 64)                       # UINT32 64
+    body += _s("tokenizer.ggml.tokens") + struct.pack("<I", 9) + struct.pack("<I", 8) + struct.pack("<Q", 3)
+    body += _s("a") + _s("bc" * 16) + _s("")                                                             # ARRAY of STRING
+    body += _s("blk.0.ffn_gate.weight") + struct.pack("<I", 2) + struct.pack("<QQ", 256, 2) + struct.pack("<I", 12)
+    body += struct.pack("<Q", 0)                                                                         # Q4_K at offset 0
+    body += _s("output_norm.weight") + struct.pack("<I", 1) + struct.pack("<Q", 5) + struct.pack("<I", 0)
+    body += struct.pack("<Q", 320)                                         # F32 at 320: 288 rounded up to 64
+    header_len = len(body)
+    data_offset = (header_len + 63) // 64 * 64
+    assert data_offset != (header_len + 31) // 32 * 32                     # the non-default alignment matters here
+    body += bytes(data_offset - header_len) + q4k + bytes(320 - 288) + f32
+    with gguf.File(_raw(tmp_path, body)) as f:
+        assert f.Version == 3 and f.Alignment == 64 and f.DataOffset == data_offset
+        assert f.NumKeyValues() == 2 and f.NumTensors() == 2
+        assert f.KeyValue("general.alignment").Uint() == 64
+        assert f.KeyValue("tokenizer.ggml.tokens").Strings() == ["a", "bc" * 16, ""]
+        g, n = f.TensorInfo("blk.0.ffn_gate.weight"), f.TensorInfo("output_norm.weight")
+        assert (g.Type, g.Shape, g.Offset, g.NumBytes) == (12, [256, 2], 0, 288)
+        assert (n.Type, n.Shape, n.Offset, n.NumBytes) == (0, [5], 320, 20)
+        assert f.TensorBytes("blk.0.ffn_gate.weight").tobytes() == q4k
+        assert f.TensorBytes("output_norm.weight").tobytes() == f32
+        assert [t.Name for t in f.TensorInfos()] == ["blk.0.ffn_gate.weight", "output_norm.weight"]

@@ -508,6 +508,71 @@ def test_config5_prefill_layer_batch512(ctx, name, t, m, k):
     W.free()
 
 
+# ---- kernel 3b: fp16-MFMA GEMM (Q4_K products with at least 192 output tiles of 256 x 128) ---------------------
+@pytest.mark.parametrize("k,m,n", [(256, 6200, 1000), (512, 12300, 500), (1024, 3000, 2050), (2304, 49 * 256, 385),
+                                   (4096, 14336, 512)])
+def test_f16_gemm_ragged_shapes(ctx, k, m, n):
+    """one super-block per row, rows and batches that end inside a tile, the gate shape; through the one-call form
+    and through an activation handle (same planes, same kernel, same bits)"""
+    w_raw = _weights(Q4_K, m, k, seed=3 * k + m)
+    W = ctx.upload(Q4_K, w_raw, k, m)
+    x = np.random.default_rng(k + n).standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(W, x)
+    rows = slice(0, m) if m * n * k <= 6200 * 1000 * 512 else np.r_[0:300, m // 2 - 150:m // 2 + 150, m - 300:m]
+    sub = w_raw if isinstance(rows, slice) else np.ascontiguousarray(w_raw.reshape(m, -1)[rows]).reshape(-1)
+    msub = m if isinstance(rows, slice) else len(rows)
+    want = oracle.mul_mat(Q4_K, sub, k, msub, x, nthreads=16)
+    err = npref.rel_err(got[:, rows], want)
+    assert err <= TOL, f"k={k} m={m} n={n}: rel err {err}"
+    # the int8 kernel computes the same integers
+    assert npref.rel_err(got, ctx.mulmat(W, x, path=qmm.PATH_GEMM)) <= 1e-5
+    act = ctx.act_create(Q8_K, k, n)
+    ctx.act_quantize(act, x)
+    assert np.array_equal(ctx.mulmat_q8(W, act), got)
+    act.free()
+    W.free()
+
+
+def test_f16_gemm_random_block_bytes(ctx):
+    """every nibble, 6-bit scale and 6-bit min pattern; activations that quantize to the extremes -127 and 127"""
+    rng = np.random.default_rng(8642)
+    k, m, n = 768, 6400, 1024
+    nb = m * k // 256
+    raw = rng.integers(0, 256, (nb, 144), dtype=np.uint8)
+    raw[:, 0:4] = np.abs(rng.standard_normal(nb * 2) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 4)
+    W = ctx.upload(Q4_K, raw.reshape(-1), k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    x[5] = np.where(rng.random(k) < 0.5, -3.0, 3.0)  # a row of +-max: every quant +-127
+    x[6] = 0.0
+    got = ctx.mulmat(W, x)
+    want = oracle.mul_mat(Q4_K, raw.reshape(-1), k, m, x, nthreads=16)
+    assert npref.rel_err(got, want) <= TOL
+    assert not got[6].any()
+    W.free()
+
+
+def test_f16_gemm_largest_block_sums_stay_exact(ctx):
+    """All scales 63, all nibbles 15, all activations equal: the super-block sums are the largest the format allows
+    (63 * 15 * 127 * 256 > 2^24).  The result must still agree with exact arithmetic to fp32 rounding."""
+    k, m, n = 512, 6400, 1024
+    blk = np.zeros(144, dtype=np.uint8)
+    blk[0:2] = np.array([2.0 ** -10], dtype=np.float16).view(np.uint8)   # d
+    blk[2:4] = np.array([2.0 ** -12], dtype=np.float16).view(np.uint8)   # dmin
+    blk[4:16] = 0xFF                                                     # scales and mins all 63
+    blk[16:] = 0xFF
+    raw = np.tile(blk, m * k // 256)
+    W = ctx.upload(Q4_K, raw, k, m)
+    x = np.ones((n, k), dtype=np.float32)
+    x[1::2] = -1.0
+    got = ctx.mulmat(W, x)
+    # every quant is 127 (or -127) with d = 1/127 (or -1/127): per super-block d*63*15*127*256 - dmin*63*127*256
+    per_sb = 2.0 ** -10 * 63 * 15 * 127 * 256 - 2.0 ** -12 * 63 * 127 * 256
+    want = np.full((n, m), 2 * per_sb / 127.0)
+    want[1::2] *= -1.0
+    assert np.max(np.abs(got / want - 1.0)) <= 1e-6
+    W.free()
+
+
 # ---- expert-indexed product (Tensor.MulmatID) ------------------------------------------------------
 def _experts(t, n_expert, m, k, seed):
     return _weights(t, n_expert * m, k, seed)
