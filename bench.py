@@ -15,7 +15,7 @@ The same JSON line carries
                 algorithmic bytes per launch / average launch duration, timed with HIP events over
                 back-to-back launches on the kernel's stream
   cpu_baseline  the CPU oracle (scalar restatement of the ggml CPU path) timed on this host
-  gemm          the batch-512 prefill GEMM over one Llama-3-8B-shaped layer (TOPS, % of int8 MFMA)
+  gemm          the batch-512 prefill GEMM over one Llama-3-8B-shaped layer (TOPS, % of the int8 MFMA peak)
 """
 from __future__ import annotations
 
@@ -316,7 +316,7 @@ def main() -> int:
         tm = timed(fn, gsteps) / (gsteps * copies)
         per["attn_q+k+v (one launch)"] = {"us": round(tm * 1e6, 1), "tops": round(2.0 * NB * 6144 * 4096 / tm / 1e12, 1)}
         out["gemm"] = {
-            "metric": "prefill GEMM TOPS (int8 MFMA)",
+            "metric": "prefill GEMM TOPS (Q4_K gate/up on fp16 MFMA, the rest on int8 MFMA; priced against the int8 peak)",
             "workload": "one Llama-3-8B-shaped layer, batch 512: q/o 4096x4096, k/v 1024x4096, gate/up 14336x4096 Q4_K; "
                         "down 4096x14336 Q6_K; activations quantized to Q8_K on GPU inside the timed region",
             "value": round(ops / t_g / 1e12, 1),
@@ -330,6 +330,30 @@ def main() -> int:
         for row in gw:
             for wt in row:
                 wt.free()
+        # what the matrix cores sustain on this machine when they do nothing else (random operands, a few ms per
+        # launch, two waves per SIMD on every CU): the practical ceiling of an MFMA-bound kernel
+        mr_path = os.path.join(os.path.dirname(qmm.LIB_PATH), "libmi_mfmarate.so")
+        if os.path.exists(mr_path) and not args.no_ceiling:
+            mr = ctypes.CDLL(mr_path)
+            mr.mi_mfma_rate.restype = ctypes.c_int
+            mr.mi_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+            mout = torch.zeros(256, dtype=torch.float32, device=dev)
+            mclk = torch.zeros(2, dtype=torch.int64, device=dev)
+            blocks, iters = 2 * info["compute_units"], 8000
+            ceil = {}
+            for kind, name, flop in ((0, "f16_32x32x16", 32768.0), (1, "i8_32x32x32", 65536.0)):
+                fn = lambda: mr.mi_mfma_rate(kind, iters, blocks, mout.data_ptr(), mclk.data_ptr(), stream.cuda_stream)
+                timed(fn, 2)
+                tm = timed(fn, 3) / 3
+                c = mclk.cpu().tolist()
+                ceil[name] = {"T(FL)OP/s": round(blocks * 4 * 4.0 * iters * flop / tm / 1e12, 1), "ms_per_launch": round(tm * 1e3, 2),
+                              "shader_clock_mhz": round(c[0] / (c[1] / 100.0)) if c[1] else None}
+            ceil["what"] = ("a loop of nothing but MFMAs on random operands, 4 independent accumulators per wave, 2 waves per SIMD on every CU, "
+                            "timed like the GEMM launches; the clock is the one workgroup 0 ran at (its cycle counter over the 100 MHz counter)")
+            out["gemm"]["mfma_ceiling"] = ceil
+            gate = per.get("ffn_gate")
+            if gate:  # the fp16 kernel issues 17 MFMAs for 16 algorithmic ones
+                out["gemm"]["ffn_gate_frac_of_f16_ceiling"] = round(gate["tops"] * 17 / 16 / ceil["f16_32x32x16"]["T(FL)OP/s"], 4)
 
     # ---- the other configurations, one short timing each: f32 activations in HBM, quantization included
     if not args.no_other:

@@ -1,0 +1,73 @@
+// Measurement aid for bench.py, not part of the product library: what rate do the matrix cores of this machine
+// sustain when they do nothing else?  Every wave runs a loop of independent MFMAs (four accumulators, so one can
+// issue every 32 cycles) on operands that differ from lane to lane and from one MFMA to the next -- random bits,
+// the switching activity of real data; with constant operands the same loop runs close to the nominal peak.  Two
+// waves per SIMD on every CU, a few milliseconds per launch: long enough for power management to settle the clock.
+// bench.py shows the prefill GEMM's figures next to this rate: it is the practical ceiling of an MFMA-bound kernel
+// here, as the pure-read launch is for the HBM-bound ones.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// KIND 0: v_mfma_f32_32x32x16_f16 (32768 flop), 1: v_mfma_i32_32x32x32_i8 (65536 op)
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void mfma_rate_kernel(float *__restrict__ out, long long *__restrict__ clk, int iters, int seed) {
+    v4i ra[8], rb[8];
+    unsigned st = seed * 2654435761u + threadIdx.x * 40503u + blockIdx.x * 69069u;
+    for (int j = 0; j < 8; j++)
+        for (int i = 0; i < 4; i++) {
+            st = st * 1664525u + 1013904223u;
+            const unsigned x1 = st;
+            st = st * 1664525u + 1013904223u;
+            const unsigned x2 = st;
+            if (KIND == 0) {  // fp16 values in [64, 128) and +-[0.125, 0.25): no overflow however long the loop
+                ra[j][i] = (int)((x1 & 0x03ff03ffu) | 0x54005400u);
+                rb[j][i] = (int)((x2 & 0x83ff83ffu) | 0x30003000u);
+            } else {
+                ra[j][i] = (int)x1;
+                rb[j][i] = (int)(x2 & 0x0f0f0f0fu);
+            }
+        }
+    v16f c[4];
+    v16i d[4];
+    for (int x = 0; x < 4; x++)
+        for (int i = 0; i < 16; i++) { c[x][i] = 0.f; d[x][i] = 0; }
+    const long long c0 = clock64(), r0 = wall_clock64();
+#pragma unroll 2
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+            const int ia = (2 * x + (it & 1)) & 7, ib = (2 * x + 1 + (it & 1)) & 7;
+            if (KIND == 0) c[x] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, ra[ia]), __builtin_bit_cast(v8h, rb[ib]), c[x], 0, 0, 0);
+            else d[x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[ia], rb[ib], d[x], 0, 0, 0);
+        }
+    }
+    const long long c1 = clock64(), r1 = wall_clock64();
+    float s = 0;
+    for (int x = 0; x < 4; x++)
+        for (int i = 0; i < 16; i++) s += c[x][i] + (float)d[x][i];
+    if (s == 12345.678f) out[threadIdx.x] = s;  // keeps the loop alive
+    if (threadIdx.x == 0 && blockIdx.x == 0) {  // shader cycles and 100 MHz ticks of workgroup 0: the clock it ran at
+        clk[0] = c1 - c0;
+        clk[1] = r1 - r0;
+    }
+}
+
+}  // namespace
+
+// Queues one launch of `blocks` workgroups (4 waves each) that issue 4 * iters MFMAs per wave.  kind 0: fp16
+// 32x32x16, 1: int8 32x32x32.  out: device scratch of 256 floats; clk: device, two int64 (shader cycles and
+// 100 MHz ticks that workgroup 0 spent in its loop).
+extern "C" int mi_mfma_rate(int kind, int iters, int blocks, float *out, long long *clk, void *stream) {
+    if (!out || !clk || iters < 1 || blocks < 1 || (kind != 0 && kind != 1)) return -1;
+    hipStream_t s = (hipStream_t)stream;
+    if (kind == 0) mfma_rate_kernel<0><<<blocks, 256, 0, s>>>(out, clk, iters, 1);
+    else mfma_rate_kernel<1><<<blocks, 256, 0, s>>>(out, clk, iters, 1);
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
