@@ -474,6 +474,15 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
         HIP_TRY(launch_gemm_blk32(w->dev, a, dy, ctx->num_cus, ctx->stream));
     } else if (use_gemm && path == MI_QMM_PATH_AUTO && gemm_f16_wanted(w->dev, a, ctx->num_cus)) {
         HIP_TRY(launch_gemm_f16(w->dev, a, dy, ctx->stream));
+    } else if (use_gemm && path == MI_QMM_PATH_AUTO && gemm_q6k_slices(w->dev.type, K, M, n, ctx->num_cus) >= 1 &&
+               (may_alloc || gemm_q6k_slices(w->dev.type, K, M, n, ctx->num_cus) == 1)) {
+        // (a caller that may not allocate gets this kernel only where it needs no K-slice workspace)
+        const size_t wsf = gemm_q6k_workspace_floats(w->dev.type, K, M, n, ctx->num_cus);
+        if (wsf) {
+            int rc = reserve(ctx, &ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float));
+            if (rc) return rc;
+        }
+        HIP_TRY(launch_gemm_q6k(w->dev, a, dy, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
     } else if (use_gemm) {
         const size_t wsf = may_alloc ? gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus) : 0;
         if (wsf) {
@@ -1240,6 +1249,8 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     // one launch pays when the tensors are too small to fill the machine one by one (q, k, v); large
     // ones (gate, up) run slightly faster back to back
     gemm_ok = gemm_ok && 2 * tiles < 3 * (int64_t)ctx->num_cus;
+    for (int i = 0; gemm_ok && i < count; i++)  // so does a Q6_K weight that the 256-row kernel takes
+        gemm_ok = gemm_q6k_slices(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n, ctx->num_cus) == 0;
     if (gemm_ok && act->f16) {  // a weight that the fp16 GEMM takes in a launch of its own keeps that kernel
         DevAct probe;
         probe.qs = nullptr; probe.d = nullptr; probe.bsums = nullptr; probe.sd8 = probe.sd16 = nullptr;

@@ -92,6 +92,13 @@ int gemm_max_multi();
 // a needs the fp16 planes (qf, bsf).  y[n*M + m].  gemm_f16_wanted() depends on the weight and the batch only.
 bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus);
 hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, hipStream_t s);
+// kernel 3c: int8-MFMA GEMM for Q6_K weights with 256 x 128 tiles and one accumulator per tile; y[n*M + m].
+// gemm_q6k_slices(): 0 = not the kernel for this product (too few tiles), else the K slices it is cut into;
+// more than one slice needs gemm_q6k_workspace_floats() floats of device workspace.
+int gemm_q6k_slices(int type, int64_t K, int64_t M, int64_t N, int num_cus);
+size_t gemm_q6k_workspace_floats(int type, int64_t K, int64_t M, int64_t N, int num_cus);
+hipError_t launch_gemm_q6k(const DevWeight &w, const DevAct &a, float *y, float *workspace, size_t workspace_floats,
+                           int num_cus, hipStream_t s);
 // 1..16 activation columns (col0 .. col0+ncols-1 of a) on the matrix cores, K-quants; y[n*M + m]
 bool skinny_supports(int type, int64_t K, int64_t M);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,

@@ -525,7 +525,7 @@ def test_f16_gemm_ragged_shapes(ctx, k, m, n):
     err = npref.rel_err(got[:, rows], want)
     assert err <= TOL, f"k={k} m={m} n={n}: rel err {err}"
     # the int8 kernel computes the same integers
-    assert npref.rel_err(got, ctx.mulmat(W, x, path=qmm.PATH_GEMM)) <= 1e-5
+    assert npref.rel_err(got, ctx.mulmat(W, x, path=qmm.PATH_GEMM)) <= 1e-4
     act = ctx.act_create(Q8_K, k, n)
     ctx.act_quantize(act, x)
     assert np.array_equal(ctx.mulmat_q8(W, act), got)
@@ -568,6 +568,66 @@ def test_f16_gemm_largest_block_sums_stay_exact(ctx):
     # every quant is 127 (or -127) with d = 1/127 (or -1/127): per super-block d*63*15*127*256 - dmin*63*127*256
     per_sb = 2.0 ** -10 * 63 * 15 * 127 * 256 - 2.0 ** -12 * 63 * 127 * 256
     want = np.full((n, m), 2 * per_sb / 127.0)
+    want[1::2] *= -1.0
+    assert np.max(np.abs(got / want - 1.0)) <= 1e-6
+    W.free()
+
+
+# ---- kernel 3c: Q6_K GEMM with 256 x 128 tiles, one accumulator per tile, K slices -------------------------------
+@pytest.mark.parametrize("k,m,n", [(1024, 6200, 1000), (4096, 3000, 600), (3328, 5000, 512), (14336, 4096, 512),
+                                   (256 * 4, 128256, 512)])
+def test_q6k_gemm_tiles_and_slices(ctx, k, m, n):
+    """no slices and ragged tiles; four slices; three uneven slices (4, 4 and 5 super-blocks); the ffn_down shape;
+    the output head's rows at one super-block run per slice; one-call form == activation-handle form"""
+    w_raw = _weights(Q6_K, m, k, seed=5 * k + m)
+    W = ctx.upload(Q6_K, w_raw, k, m)
+    x = np.random.default_rng(k + n + 1).standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(W, x)
+    rows = slice(0, m) if m * n * k <= 6200 * 1000 * 1024 else np.r_[0:300, m // 2 - 150:m // 2 + 150, m - 300:m]
+    sub = w_raw if isinstance(rows, slice) else np.ascontiguousarray(w_raw.reshape(m, -1)[rows]).reshape(-1)
+    msub = m if isinstance(rows, slice) else len(rows)
+    want = oracle.mul_mat(Q6_K, sub, k, msub, x, nthreads=16)
+    err = npref.rel_err(got[:, rows], want)
+    assert err <= TOL, f"k={k} m={m} n={n}: rel err {err}"
+    assert npref.rel_err(got, ctx.mulmat(W, x, path=qmm.PATH_GEMM)) <= 1e-4  # the 128-row kernel: same integers, other fp32 order
+    act = ctx.act_create(Q8_K, k, n)
+    ctx.act_quantize(act, x)
+    assert np.array_equal(ctx.mulmat_q8(W, act), got)
+    act.free()
+    W.free()
+
+
+def test_q6k_gemm_random_block_bytes(ctx):
+    """every ql / qh bit pattern and every int8 scale, negative ones and -128 included"""
+    rng = np.random.default_rng(9753)
+    k, m, n = 1024, 6400, 1024
+    nb = m * k // 256
+    raw = rng.integers(0, 256, (nb, 210), dtype=np.uint8)
+    raw[:, 208:210] = np.abs(rng.standard_normal(nb) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    raw[::7, 192] = 0x80  # scale -128
+    W = ctx.upload(Q6_K, raw.reshape(-1), k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    x[5] = np.where(rng.random(k) < 0.5, -3.0, 3.0)
+    got = ctx.mulmat(W, x)
+    want = oracle.mul_mat(Q6_K, raw.reshape(-1), k, m, x, nthreads=16)
+    assert npref.rel_err(got, want) <= TOL
+    W.free()
+
+
+def test_q6k_gemm_extreme_products_stay_exact(ctx):
+    """all scales -128, all 6-bit values 0 (= -32), all activations equal: every product is the largest the format
+    allows (+4096 * 127) and the super-block sums reach 256 * 4096 * 127 = 2^27; both digits and the shift carry it"""
+    k, m, n = 512, 6400, 1024
+    blk = np.zeros(210, dtype=np.uint8)
+    blk[192:208] = 0x80
+    blk[208:210] = np.array([2.0 ** -14], dtype=np.float16).view(np.uint8)
+    raw = np.tile(blk, m * k // 256)
+    W = ctx.upload(Q6_K, raw, k, m)
+    x = np.ones((n, k), dtype=np.float32)
+    x[1::2] = -1.0
+    got = ctx.mulmat(W, x)
+    # x = 1 quantizes to -127 with d = -1/127 (x = -1: -127 with d = 1/127): per super-block 2^-14 * 4096 * 256 = 64
+    want = np.full((n, m), 2 * 64.0)
     want[1::2] *= -1.0
     assert np.max(np.abs(got / want - 1.0)) <= 1e-6
     W.free()
