@@ -7,6 +7,8 @@
 // As in the 128-row kernel of gemm_mfma.hip the 8-bit scale of a 16-element group is folded into the weights and
 // the 13-bit product p = sc * (e - 32) is split into two int8 digits, p = 256 p_h + p_l (p_l the low byte read as
 // int8, p_h the high byte of p + 128), which are multiplied separately.  What is different:
+//   * The digits come from r = sc * e + (128 - 32 sc), one packed 16-bit multiply-add per two weights: p_h is the high
+//     byte of r, p_l its low byte with the top bit flipped.
 //   * One accumulator, not two.  All high-digit MFMAs of a super-block come first, the accumulator is shifted left
 //     by eight, and the low-digit MFMAs add on top of it: sum = 256 * sum_h + sum_l with 16 registers per 32x32
 //     tile instead of 32.  That halves the accumulators and lets a wave cover 128 activation rows (four tiles), so
@@ -20,7 +22,7 @@
 //     256 x 32 B) in a ring of three, scales / row scales / activation scales per super-block, all by
 //     direct-to-LDS copies issued from inline assembly with hand-counted waits; one raw barrier per half
 //     super-block.  LDS reads of 16 bytes are laid out for the lanes the hardware serves together.
-// Per 32x32 tile and super-block: 16 MFMAs and about 180 vector instructions (370 in the 128-row kernel).
+// Per 32x32 tile and super-block: 16 MFMAs and about 176 vector instructions (370 in the 128-row kernel).
 //
 // A product whose tiles alone would leave most CUs idle (4096 x 14336 at batch 512: 64 tiles) is cut along K into
 // slices, each writing its partial sums to its own [N][M] plane of a workspace; a second kernel adds the planes
@@ -199,18 +201,21 @@ __global__ __launch_bounds__(512, 2) void gemm_q6k_kernel(const uint8_t *__restr
                 const unsigned scw = s < 2 ? scv.x : s < 4 ? scv.y : s < 6 ? scv.z : scv.w;
                 const int sc = (int)(int8_t)(scw >> (8 * (2 * (s & 1) + h)));
                 const s2 sc2 = {(short)sc, (short)sc};
-                const s2 k32 = {32, 32}, k128 = {128, 128};
+                const short cc = (short)(128 - 32 * sc);
+                const s2 c2 = {cc, cc};
                 v4i bh, bl;
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const unsigned l = lq[rr & 1][i], hh = hq[i];
                     const unsigned nib = (rr >> 1) ? (l >> 4) & 0x0f0f0f0fu : l & 0x0f0f0f0fu;
-                    const unsigned e = nib | (((hh >> (2 * rr)) & 0x03030303u) << 4);
-                    const s2 pe = (as_s2(e & 0x00ff00ffu) - k32) * sc2;
-                    const s2 po = (as_s2(__builtin_amdgcn_perm(0u, e, 0x0c030c01u)) - k32) * sc2;
-                    const unsigned re = as_u(pe + k128), ro = as_u(po + k128);
-                    bl[i] = (int)__builtin_amdgcn_perm(as_u(po), as_u(pe), 0x06020400u);
-                    bh[i] = (int)__builtin_amdgcn_perm(ro, re, 0x07030501u);
+                    const unsigned hs = rr == 0 ? hh << 4 : rr == 1 ? hh << 2 : rr == 2 ? hh : hh >> 2;
+                    const unsigned e = (hs & 0x30303030u) | nib;  // 0..63 per byte
+                    // r = sc * (e - 32) + 128 per 16-bit lane (one packed multiply-add): its high byte is the high digit,
+                    // its low byte with the top bit flipped the low digit
+                    const s2 re = as_s2(e & 0x00ff00ffu) * sc2 + c2;                             // elements 0 and 2
+                    const s2 ro = as_s2(__builtin_amdgcn_perm(0u, e, 0x0c030c01u)) * sc2 + c2;   // elements 1 and 3
+                    bl[i] = (int)(__builtin_amdgcn_perm(as_u(ro), as_u(re), 0x06020400u) ^ 0x80808080u);
+                    bh[i] = (int)__builtin_amdgcn_perm(as_u(ro), as_u(re), 0x07030501u);
                 }
                 BL[s] = bl;
 #pragma unroll
