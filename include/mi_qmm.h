@@ -141,7 +141,7 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
  * caller's graph plan); it exists for those callers.  The quantized activations go to a static device
  * array of MI_QMM_NOALLOC_SCRATCH_BYTES that each GPU the library runs on holds until the process ends;
  * a call whose quantized activations do not fit (about n * k * 1.4 bytes for Q4_K / Q6_K weights from
- * three or four rows up -- n * k * 3.4 for Q4_K weights from 32 rows up, where the planes of the fp16 GEMM
+ * three or four rows up -- n * k * 3.4 for Q4_K weights from 65 rows up, where the planes of the fp16 GEMM
  * are written too; n is rounded up to a multiple of 128 for these types -- and n * k * 1.2 for Q4_0 / Q8_0;
  * one to a few rows need no scratch at all) returns MI_QMM_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array: calls that overlap in time on
  * one GPU (two streams, two ctxs) race.  Results are those of mi_qmm_mulmat (bit-identical, except that

@@ -106,7 +106,7 @@ int reserve(mi_qmm_ctx *ctx, void **buf, size_t *cap, size_t need) {
 struct ActPlanes { int8_t *qs; float *d; int16_t *bsums; uint8_t *sd8; uint8_t *sd16; uint16_t *qf; uint16_t *bsf; size_t total; };
 
 // fp16 planes for the fp16-MFMA GEMM: wanted where a Q4_K weight may meet a batch that kernel takes
-bool wants_f16_planes(int weight_type, int64_t n) { return weight_type == T_Q4_K && n >= 32; }
+bool wants_f16_planes(int weight_type, int64_t n) { return weight_type == T_Q4_K && n > 64; }
 
 // carve the activation scratch into planes for N rows of K elements
 ActPlanes plan_act(void *base, int q8_type, int64_t K, int64_t N, bool f16 = false) {
@@ -1152,7 +1152,7 @@ int mi_qmm_act_create(mi_qmm_ctx *ctx, int q8_type, int64_t k, int64_t n_max, mi
     mi_qmm_act *a = new (std::nothrow) mi_qmm_act();
     if (!a) return fail(MI_QMM_ERR_NOMEM, "host allocation failed");
     a->device = ctx->device; a->type = q8_type; a->k = k; a->n_max = n_max;
-    a->f16 = q8_type == T_Q8_K && n_max >= 32;  // any Q4_K weight may meet these rows: keep the fp16 planes too
+    a->f16 = q8_type == T_Q8_K && n_max > 64;  // any Q4_K weight may meet these rows: keep the fp16 planes too
     const ActPlanes probe = plan_act(nullptr, q8_type, k, n_max, a->f16);
     hipError_t e = hipMalloc(&a->base, probe.total + 256);
     if (e != hipSuccess) {

@@ -290,7 +290,7 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(const uint8_t *__r
 // 128-row tiles of the int8 kernel.  The choice depends on the weight and the batch only, never on what else a
 // call multiplies, so a product's bits do not depend on how it was asked for.
 bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus) {
-    if (w.type != T_Q4_K || !a.qf || !a.bsf || w.K < QKK || w.K % QKK || a.N < 32) return false;
+    if (w.type != T_Q4_K || !a.qf || !a.bsf || w.K < QKK || w.K % QKK || a.N <= 64) return false;  // up to 64 rows: the 128 x 64 tiles of the int8 kernel
     if ((int64_t)a.N * w.K >= ((int64_t)1 << 31) || w.M * (w.K / QKK * Q4_K_BYTES) >= ((int64_t)1 << 32)) return false;  // 32-bit lane offsets
     const int64_t tiles = (w.M + TM - 1) / TM * ((a.N + TN - 1) / TN);
     return 4 * tiles >= 3 * (int64_t)num_cus;

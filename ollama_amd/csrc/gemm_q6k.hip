@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void sum_planes_kernel(const float4 *__restric
 // weight's shape and the batch only.  The kernel pays where its 256 x 128 tiles, times the slices, give at least
 // three quarters of the CUs a workgroup, every slice keeping four super-blocks or more.
 int gemm_q6k_slices(int type, int64_t K, int64_t M, int64_t N, int num_cus) {
-    if (type != T_Q6_K || K < QKK || K % QKK || N < 32 || M < 1) return 0;
+    if (type != T_Q6_K || K < QKK || K % QKK || N <= 64 || M < 1) return 0;  // up to 64 rows: the 128 x 64 tiles of the other kernel
     if (N * K >= ((int64_t)1 << 31) || M * (K / QKK) * 2 >= ((int64_t)1 << 32) || M > 0x7fffffff) return 0;  // 32-bit lane offsets
     const int64_t tiles = (M + TM - 1) / TM * ((N + TN - 1) / TN), nsb = K / QKK;
     int64_t ks = 1;

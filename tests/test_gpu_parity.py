@@ -510,9 +510,9 @@ def test_config5_prefill_layer_batch512(ctx, name, t, m, k):
 
 # ---- kernel 3b: fp16-MFMA GEMM (Q4_K products with at least 192 output tiles of 256 x 128) ---------------------
 @pytest.mark.parametrize("k,m,n", [(256, 6200, 1000), (512, 12300, 500), (1024, 3000, 2050), (2304, 49 * 256, 385),
-                                   (4096, 14336, 512)])
+                                   (4096, 14336, 512), (512, 49300, 70)])
 def test_f16_gemm_ragged_shapes(ctx, k, m, n):
-    """one super-block per row, rows and batches that end inside a tile, the gate shape; through the one-call form
+    """one super-block per row, rows and batches that end inside a tile, the gate shape, one tile column; through the one-call form
     and through an activation handle (same planes, same kernel, same bits)"""
     w_raw = _weights(Q4_K, m, k, seed=3 * k + m)
     W = ctx.upload(Q4_K, w_raw, k, m)
@@ -575,10 +575,10 @@ def test_f16_gemm_largest_block_sums_stay_exact(ctx):
 
 # ---- kernel 3c: Q6_K GEMM with 256 x 128 tiles, one accumulator per tile, K slices -------------------------------
 @pytest.mark.parametrize("k,m,n", [(1024, 6200, 1000), (4096, 3000, 600), (3328, 5000, 512), (14336, 4096, 512),
-                                   (256 * 4, 128256, 512)])
+                                   (256 * 4, 128256, 512), (1024, 50000, 100)])
 def test_q6k_gemm_tiles_and_slices(ctx, k, m, n):
     """no slices and ragged tiles; four slices; three uneven slices (4, 4 and 5 super-blocks); the ffn_down shape;
-    the output head's rows at one super-block run per slice; one-call form == activation-handle form"""
+    the output head's rows; a batch that fills most of one 128-row tile column; one-call form == activation-handle form"""
     w_raw = _weights(Q6_K, m, k, seed=5 * k + m)
     W = ctx.upload(Q6_K, w_raw, k, m)
     x = np.random.default_rng(k + n + 1).standard_normal((n, k), dtype=np.float32)
