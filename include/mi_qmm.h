@@ -192,7 +192,9 @@ int mi_qmm_mulmat_produced(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
 int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_qmm_weight *w_up, int producer,
                          const float *aux, float eps, const float *x, int64_t n, float *h, int location);
 /* The same producers as plain f32 operations, for graph nodes that something other than a product
- * reads: x, y f32 [n][k] (k a multiple of 4), g f32 [k] or NULL; gate, up, y f32 [n][k] (any k). */
+ * reads: x, y f32 [n][k] (k a multiple of 4), g f32 [k] or NULL; gate, up, y f32 [n][k] (any k).
+ * up == NULL: the bare activation y = silu(gate), Tensor.SILU(ctx) without an operand
+ * (/root/reference/ml/backend.go:180 is variadic). */
 int mi_qmm_rms_norm(mi_qmm_ctx *ctx, const float *x, const float *g, float eps, int64_t k, int64_t n,
                     float *y, int location);
 int mi_qmm_swiglu(mi_qmm_ctx *ctx, const float *gate, const float *up, int64_t k, int64_t n, float *y,

@@ -878,12 +878,12 @@ int mi_qmm_swiglu(mi_qmm_ctx *ctx, const float *gate, const float *up, int64_t k
     if (rc) return rc;
     if (k < 0) return fail(MI_QMM_ERR_INVALID, "k=%lld must be non-negative", (long long)k);
     if (k * n == 0) return MI_QMM_OK;
-    if (!gate || !up || !y) return fail(MI_QMM_ERR_INVALID, "gate, up or y is NULL");
-    const size_t b = (size_t)(n * k) * 4, bytes[3] = {b, b, b};
+    if (!gate || !y) return fail(MI_QMM_ERR_INVALID, "gate or y is NULL");
+    const size_t b = (size_t)(n * k) * 4, bytes[3] = {b, up ? b : 0, b};
     const void *src[3] = {gate, up, y};
     void *d[3];
     if ((rc = stage_in(ctx, location, src, bytes, 2, 3, d))) return rc;
-    HIP_TRY(launch_swiglu((const float *)d[0], (const float *)d[1], n * k, (float *)d[2], ctx->stream));
+    HIP_TRY(launch_swiglu((const float *)d[0], up ? (const float *)d[1] : nullptr, n * k, (float *)d[2], ctx->stream));
     if (location == MI_QMM_HOST) {
         HIP_TRY(hipMemcpyAsync(y, d[2], b, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(hipStreamSynchronize(ctx->stream));

@@ -17,7 +17,7 @@ hipError_t launch_quantize_act(int q8_type, const float *x, int64_t K, int64_t N
                                float *d, int16_t *bsums, uint8_t *sd8, uint8_t *sd16, hipStream_t s,
                                const Produce *produce = nullptr, uint16_t *qf = nullptr, uint16_t *bsf = nullptr);
 // RMSNorm over rows of K floats: scale_out [N] (optional) = 1/sqrtf(mean(x^2)+eps) per row; y (optional) =
-// (x * scale) * g with g [K] or null.  SwiGLU: y = silu(gate) * up over count floats.
+// (x * scale) * g with g [K] or null.  SwiGLU: y = silu(gate) * up over count floats (up null: y = silu(gate)).
 hipError_t launch_rms_norm(const float *x, const float *g, float eps, int64_t K, int64_t N, float *scale_out, float *y,
                            hipStream_t s);
 hipError_t launch_swiglu(const float *gate, const float *up, int64_t count, float *y, hipStream_t s);

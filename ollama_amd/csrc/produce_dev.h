@@ -66,7 +66,8 @@ __device__ __forceinline__ float4 rms_apply(const float4 v, float scale, const f
     return r;
 }
 
-__device__ __forceinline__ float silu_mul(float v, float up) { return v / (1.0f + expf(-v)) * up; }
+__device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float silu_mul(float v, float up) { return silu(v) * up; }
 
 __device__ __forceinline__ float4 swiglu_apply(const float4 v, const float4 up) {
     return make_float4(silu_mul(v.x, up.x), silu_mul(v.y, up.y), silu_mul(v.z, up.z), silu_mul(v.w, up.w));

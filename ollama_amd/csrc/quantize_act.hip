@@ -127,10 +127,18 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float4 *__restrict_
     }
 }
 
-// count floats: float4 pieces where the pointers allow (vec), the rest one by one
+// count floats: float4 pieces where the pointers allow (vec), the rest one by one.  up == nullptr: the bare silu.
 __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up,
                                                      float *__restrict__ y, int64_t count, bool vec) {
     const int64_t n4 = vec ? count / 4 : 0, first = (int64_t)blockIdx.x * 256 + threadIdx.x, step = (int64_t)gridDim.x * 256;
+    if (!up) {
+        for (int64_t i = first; i < n4; i += step) {
+            const float4 v = reinterpret_cast<const float4 *>(gate)[i];
+            reinterpret_cast<float4 *>(y)[i] = make_float4(silu(v.x), silu(v.y), silu(v.z), silu(v.w));
+        }
+        for (int64_t i = 4 * n4 + first; i < count; i += step) y[i] = silu(gate[i]);
+        return;
+    }
     for (int64_t i = first; i < n4; i += step)
         reinterpret_cast<float4 *>(y)[i] = swiglu_apply(reinterpret_cast<const float4 *>(gate)[i], reinterpret_cast<const float4 *>(up)[i]);
     for (int64_t i = 4 * n4 + first; i < count; i += step) y[i] = silu_mul(gate[i], up[i]);
@@ -212,7 +220,7 @@ hipError_t launch_rms_norm(const float *x, const float *g, float eps, int64_t K,
 
 hipError_t launch_swiglu(const float *gate, const float *up, int64_t count, float *y, hipStream_t s) {
     if (count == 0) return hipSuccess;
-    if (!gate || !up || !y) return hipErrorInvalidValue;
+    if (!gate || !y) return hipErrorInvalidValue;
     const bool vec = (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)y) & 15) == 0;
     const int64_t work = vec ? count / 4 + 3 : count, blocks = (work + 255) / 256;
     swiglu_kernel<<<(unsigned)(blocks < 8192 ? blocks : 8192), 256, 0, s>>>(gate, up, y, count, vec);

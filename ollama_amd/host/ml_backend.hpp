@@ -57,7 +57,7 @@ public:
     // self = x [K, ...] f32, weight = [K] f32 or null -> lazy (x / sqrt(mean(x^2) + eps)) * weight along dimension 0
     std::shared_ptr<Tensor> RMSNorm(Context &ctx, const std::shared_ptr<Tensor> &weight, float eps);
     // self = gate, up: f32 of one shape -> lazy silu(gate) * up (ggml's swiglu)
-    std::shared_ptr<Tensor> SILU(Context &ctx, const std::shared_ptr<Tensor> &up);
+    std::shared_ptr<Tensor> SILU(Context &ctx, const std::shared_ptr<Tensor> &up = nullptr);
 
     ~Tensor() { mi_qmm_weight_free(weight_); }
 
@@ -195,6 +195,7 @@ public:
             if (n->prod_) {
                 needed.insert(n->prod_src_.get());
                 if (n->prod_aux_) needed.insert(n->prod_aux_.get());
+                if (n->prod_ == MI_QMM_PRODUCE_SWIGLU && !n->prod_aux_) needed.insert(n.get());  // the bare silu
             }
         }
         // gate.SILU(up) on two pending products of one x that nothing else reads: one call computes the gated
@@ -267,8 +268,8 @@ public:
                     check(mi_qmm_rms_norm(b_.handle(), src.data_.data(), t->prod_aux_ ? t->prod_aux_->Floats().data() : nullptr,
                                           t->prod_eps_, k, n, t->data_.data(), MI_QMM_HOST));
                 else
-                    check(mi_qmm_swiglu(b_.handle(), src.data_.data(), t->prod_aux_->Floats().data(), k, n, t->data_.data(),
-                                        MI_QMM_HOST));
+                    check(mi_qmm_swiglu(b_.handle(), src.data_.data(), t->prod_aux_ ? t->prod_aux_->Floats().data() : nullptr, k, n,
+                                        t->data_.data(), MI_QMM_HOST));
                 t->ready_ = true;
                 continue;
             }
@@ -409,8 +410,8 @@ inline std::shared_ptr<Tensor> Tensor::RMSNorm(Context &ctx, const std::shared_p
 }
 
 inline std::shared_ptr<Tensor> Tensor::SILU(Context &ctx, const std::shared_ptr<Tensor> &up) {
-    if (!up) throw Error(MI_QMM_ERR_INVALID, "SILU: this path implements the gated form SILU(ctx, up) only");
-    if (type_ != MI_QMM_TYPE_F32 || weight_ || up->type_ != MI_QMM_TYPE_F32 || up->weight_ || shape_ != up->shape_)
+    // up == nullptr: the bare activation silu(self), always an f32 node of its own
+    if (type_ != MI_QMM_TYPE_F32 || weight_ || (up && (up->type_ != MI_QMM_TYPE_F32 || up->weight_ || shape_ != up->shape_)))
         throw Error(MI_QMM_ERR_INVALID, "SILU: gate and up must be f32 of one shape");
     auto out = std::make_shared<Tensor>();
     out->shape_ = shape_;

@@ -136,14 +136,14 @@ class Tensor:
         return out
 
     def SILU(self, ctx: "Context", *up: "Tensor") -> "Tensor":
-        """self = gate, up[0] = up, both f32 of one shape  ->  silu(gate) * up, lazily (ggml's swiglu).  The
-        bare activation (no ``up``) feeds no quantized product and is outside this path."""
-        if len(up) != 1:
-            raise TypeError("SILU: this path implements the gated form SILU(ctx, up) only")
-        if self._type != qmm.F32 or up[0]._type != qmm.F32 or self._shape != up[0]._shape:
-            raise ValueError(f"SILU: gate {self.Shape()} and up {up[0].Shape()} must be f32 of one shape")
+        """self = gate, up[0] = up, both f32 of one shape  ->  silu(gate) * up, lazily (ggml's swiglu).  Without
+        ``up``: the bare activation silu(self), an f32 node of its own (it is never folded into a product)."""
+        if len(up) > 1:
+            raise TypeError("SILU takes at most one operand")
+        if self._type != qmm.F32 or (up and (up[0]._type != qmm.F32 or self._shape != up[0]._shape)):
+            raise ValueError(f"SILU: gate {self.Shape()} and up must be f32 of one shape")
         out = Tensor(self._shape)
-        out._prod = (qmm.PRODUCE_SWIGLU, self, up[0], 0.0)
+        out._prod = (qmm.PRODUCE_SWIGLU, self, up[0] if up else None, 0.0)
         ctx._nodes.append(out)
         return out
 
@@ -193,6 +193,8 @@ class Context:
             srcs = [s for s in (t._prod[1], t._prod[2]) if s is not None] if t._prod is not None else [t._op[1]]
             if t._prod is not None:
                 needed.update(id(s) for s in srcs)
+                if t._prod[0] == qmm.PRODUCE_SWIGLU and t._prod[2] is None:
+                    needed.add(id(t))  # the bare silu is always an f32 node
             for s in srcs:
                 readers.setdefault(id(s), []).append(t)
         # gate.SILU(up) on two pending products of one x that nothing else reads, at one activation row: one call
@@ -229,7 +231,7 @@ class Context:
                     if kind == qmm.PRODUCE_RMSNORM:
                         t._data = c.rms_norm(rows(src), None if aux is None else aux.Floats(), eps).reshape(-1)
                     else:
-                        t._data = c.swiglu(rows(src), rows(aux)).reshape(-1)
+                        t._data = c.swiglu(rows(src), None if aux is None else rows(aux)).reshape(-1)
                 continue
             x = t._op[1]
             if t._absorbed:

@@ -10,6 +10,7 @@ import os
 import subprocess
 
 import numpy as np
+from typing import Optional
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI_QMM_LIB points at an alternative build of the library (e.g. an experimental variant)
@@ -424,15 +425,16 @@ class Context:
         _check(lib().mi_qmm_rms_norm(self._h, _ptr(x), _ptr(g) if g is not None else None, eps, k, n, _ptr(y), HOST))
         return y
 
-    def swiglu(self, gate: np.ndarray, up: np.ndarray) -> np.ndarray:
-        """silu(gate) * up, f32 [n, k]"""
+    def swiglu(self, gate: np.ndarray, up: Optional[np.ndarray]) -> np.ndarray:
+        """silu(gate) * up, f32 [n, k]; up None: silu(gate)"""
         gate = np.ascontiguousarray(gate, dtype=np.float32)
-        up = np.ascontiguousarray(up, dtype=np.float32)
-        if gate.shape != up.shape:
-            raise ValueError(f"gate {gate.shape} and up {up.shape} differ")
+        if up is not None:
+            up = np.ascontiguousarray(up, dtype=np.float32)
+            if gate.shape != up.shape:
+                raise ValueError(f"gate {gate.shape} and up {up.shape} differ")
         g2 = gate.reshape(-1, gate.shape[-1])
         y = np.empty_like(g2)
-        _check(lib().mi_qmm_swiglu(self._h, _ptr(g2), _ptr(up), g2.shape[1], g2.shape[0], _ptr(y), HOST))
+        _check(lib().mi_qmm_swiglu(self._h, _ptr(g2), _ptr(up) if up is not None else None, g2.shape[1], g2.shape[0], _ptr(y), HOST))
         return y.reshape(gate.shape)
 
     def mulmat_id(self, w: Weight, n_expert: int, b: np.ndarray, ids: np.ndarray) -> np.ndarray:

@@ -1,6 +1,7 @@
 // GPU test program (run by tests/test_gpu_host_mirror.py): drives the C++ mirror of the reference's
 // ml.Backend / Context / Tensor interface and checks every Mulmat against the CPU oracle.
 // Links libmi_qmm.so (the product) and oracle/libggml_ref.so (the checker; test infrastructure).
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -242,12 +243,20 @@ int main() {
                 }
                 if (outs[0] != outs[1]) { printf("FAIL: fused and materialized producers differ at N=%lld\n", (long long)n); failures++; }
             }
-            bool threw_silu = false;
-            try {
+            {   // the bare activation SILU(ctx): an f32 node of its own
                 auto ctx = backend.NewContext();
-                ctx->FromFloats(std::vector<float>(k), {k, 1})->SILU(*ctx, nullptr);
-            } catch (const Error &) { threw_silu = true; }
-            if (!threw_silu) { printf("FAIL: SILU without up did not throw\n"); failures++; }
+                std::vector<float> v(k);
+                for (int64_t i = 0; i < k; i++) v[i] = 0.01f * (float)(i % 400) - 2.f;
+                auto bare = ctx->FromFloats(v, {k, 1})->SILU(*ctx);
+                ctx->Compute({bare});
+                double worst = 0;
+                for (int64_t i = 0; i < k; i++) {
+                    const double want = (double)v[i] / (1.0 + std::exp(-(double)v[i]));
+                    worst = std::max(worst, std::fabs((double)bare->Floats()[i] - want));
+                }
+                if (!(worst <= 1e-6)) { printf("FAIL: bare SILU off by %.3g\n", worst); failures++; }
+                ctx->Close();
+            }
         }
         backend.Close();
         printf(failures ? "host mirror: %d FAILURES\n" : "host mirror: all ok\n", failures);

@@ -135,8 +135,14 @@ def test_python_mirror_ffn_block_with_producers():
         ctx3.Close()
         ctx.Close(); ctx2.Close()
     ctx = b.NewContext()
+    # the bare activation SILU(ctx): an f32 node of its own, also in front of a product
+    v = np.random.default_rng(3).standard_normal(k).astype(np.float32)
+    bare = ctx.FromFloats(v, k, 1).SILU(ctx)
+    ctx.Compute(bare)
+    want = v.astype(np.float64) / (1.0 + np.exp(-v.astype(np.float64)))
+    assert np.max(np.abs(bare.Floats() - want)) <= 1e-6
     with pytest.raises(TypeError):
-        ctx.FromFloats(np.zeros(k, np.float32), k, 1).SILU(ctx)
+        ctx.FromFloats(v, k, 1).SILU(ctx, bare, bare)
     with pytest.raises(ValueError):
         ctx.FromFloats(np.zeros(k, np.float32), k, 1).RMSNorm(ctx, ctx.FromFloats(np.zeros(8, np.float32), 8), 1e-5)
     b.Close()

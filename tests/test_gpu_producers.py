@@ -84,6 +84,11 @@ def test_swiglu_matches_the_oracle(ctx):
     assert s[0, 0] == 0 and s[0, 1] == 100.0 and s[0, 2] == 0.0
     assert np.allclose(s[0, 3] - s[0, 4], 1.0, atol=1e-6) and np.allclose(s[0, 5] - s[0, 6], 30.0, atol=1e-5)
     assert ctx.swiglu(np.zeros((0, 8), np.float32), np.zeros((0, 8), np.float32)).shape == (0, 8)
+    # the bare activation (no up): the same bits as gating with ones, and the closed form in fp64
+    bare = ctx.swiglu(v, None)
+    assert np.array_equal(bare, s)
+    v64 = v.astype(np.float64)
+    assert np.max(np.abs(bare - v64 / (1.0 + np.exp(-v64)))) <= 1e-6 * max(1.0, float(np.max(np.abs(v64))))
 
 
 def _chain(t, wb, k, m, producer, aux, x, eps):
