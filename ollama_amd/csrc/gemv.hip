@@ -643,6 +643,39 @@ __device__ __forceinline__ void quantize_x_to_lds(const float4 *__restrict__ x4,
         quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
 }
 
+// The same for Q8_K activations with a quarter of a wave per block (q8_K_quantize_row16: lane l of a 16-lane row holds
+// elements 16l.. of its block, a wave quantizes four consecutive blocks at a time): fewer cross-lane steps per block,
+// and the plain decode prologue is made of little else.  Same bits.  A wave's first four blocks are requested by
+// prefetch_x16 ahead of its first weight load.
+__device__ __forceinline__ void prefetch_x16(const float4 *__restrict__ x4, int nblk_all, int wave, int lane, float4 (&xq)[4]) {
+    const int b = min(4 * wave + (lane >> 4), nblk_all - 1);  // clamped: the loads stay unconditional
+#pragma unroll
+    for (int j = 0; j < 4; j++) xq[j] = x4[b * 64 + 4 * (lane & 15) + j];
+}
+template <class P>
+__device__ __forceinline__ void quantize_x_to_lds16(const float4 *__restrict__ x4, int nblk_all, int wave, int nwaves, int lane,
+                                                    const float4 (&xq)[4], int8_t *lqs, float *ld_, int16_t *lbs) {
+    auto quantize_four = [&](int b0, const float4 (&v)[4]) {
+        const int b = b0 + (lane >> 4), sub = lane & 15;
+        float dd;
+        int sum16, pair;
+        const uint4 packed = q8_K_quantize_row16(v, lane, dd, sum16, pair);
+        if (b < nblk_all) {  // the last four may end early: whole rows of 16 lanes drop out
+            *reinterpret_cast<uint4 *>(lqs + (size_t)b * QKK + 16 * sub) = packed;
+            if (sub == 0) ld_[b] = dd;
+            if (P::USES_BSUMS) lbs[b * 16 + sub] = (int16_t)sum16;
+        }
+    };
+    if (4 * wave < nblk_all) quantize_four(4 * wave, xq);  // wave-uniform
+    for (int b0 = 4 * (wave + nwaves); b0 < nblk_all; b0 += 4 * nwaves) {
+        float4 v[4];
+        const int b = min(b0 + (lane >> 4), nblk_all - 1);
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = x4[b * 64 + 4 * (lane & 15) + j];
+        quantize_four(b0, v);
+    }
+}
+
 // Global-address-space pointer types: what a kernel's pointer arguments are cast to before an empty asm pins
 // them in scalar registers (see gemv_thin_kernel), so that they come out of it still known to be global.
 typedef const __attribute__((address_space(1))) uint8_t *gbytes_t;
@@ -758,12 +791,20 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     const float4 *x4 = reinterpret_cast<const float4 *>(xf + (int64_t)col0 * K);
     const int total4 = (int)((int64_t)NC * K / 4);  // float4 pieces over all NC columns
     const int nwaves = kw << rw_log2 /* = (kw << rw_log2) * 64 / 64, without the hidden-argument load */;
-    float4 xpre[XP], apre[XP];
-    if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
+    // plain Q8_K activations with several blocks per wave (long rows): four blocks per wave at a time.  Where a block
+    // per wave covers the row (XP = 1) sixteen waves quantizing one block each finish sooner than four waves
+    // quantizing four (measured: the gate+up launch 13.2 against 13.4 us).
+    // SwiGLU in front (XMODE 3) is elementwise and takes the same route; RMSNorm's sum of squares is tied to the
+    // wave-per-block order and does not.
+    constexpr bool ROW16 = (XMODE == 1 || XMODE == 3) && P::ACT_BLK == QKK && XP > 1;
+    float4 xpre[XP], apre[XP], xq[4], apre16[4];
+    if (ROW16) prefetch_x16(x4, NC * nblk, wave, lane, xq);
+    else if (F32) prefetch_x(x4, total4, wave, nwaves, lane, xpre);
     // the producer's operand, requested unconditionally (RMSNorm without a weight reads x again and ignores
     // it) so that the number of loads in flight stays known to the waits below
     const bool has_aux = XMODE == 3 || (XMODE == 2 && pr.aux != nullptr);
-    if (XMODE >= 2) prefetch_x(has_aux ? reinterpret_cast<const float4 *>(pr.aux) : x4, total4, wave, nwaves, lane, apre);
+    if (ROW16 && XMODE == 3) prefetch_x16(reinterpret_cast<const float4 *>(pr.aux), NC * nblk, wave, lane, apre16);
+    else if (XMODE >= 2) prefetch_x(has_aux ? reinterpret_cast<const float4 *>(pr.aux) : x4, total4, wave, nwaves, lane, apre);
     typename P::Raw cur;
     if (nrw > 0) cur = P::load(w, g, r0 + rl0 + min(run, nrw - 1));
     constexpr size_t PSUM_BYTES = XMODE == 2 ? XPRE * 16 * sizeof(double) : 0;  // one sum per 256-element piece
@@ -785,12 +826,16 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
 #pragma unroll
         for (int j = 0; j < XP; j++) xpre[j] = rms_apply(xpre[j], scale, apre[j], has_aux);
     }
-    if (XMODE == 3) {
+    if (XMODE == 3 && ROW16) {  // (the plan keeps such rows within one group of four blocks per wave)
+#pragma unroll
+        for (int j = 0; j < 4; j++) xq[j] = swiglu_apply(xq[j], apre16[j]);
+    } else if (XMODE == 3) {
 #pragma unroll
         for (int j = 0; j < XP; j++) xpre[j] = swiglu_apply(xpre[j], apre[j]);
     }
     if (F32) {
-        quantize_x_to_lds<P, XP>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
+        if (ROW16) quantize_x_to_lds16<P>(x4, NC * nblk, wave, nwaves, lane, xq, lqs, ld_, lbs);
+        else quantize_x_to_lds<P, XP>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
         __syncthreads();
     }
     float *part = reinterpret_cast<float *>(smem + act_bytes + PSUM_BYTES);

@@ -104,4 +104,44 @@ __device__ __forceinline__ int q8_K_quantize_lane(const float4 v, int lane, floa
     return pack4_i8(q[0], q[1], q[2], q[3]);
 }
 
+// Q8_K with a quarter of a wave per super-block: the 16 lanes of a DPP row hold the 256 elements of a block, sixteen
+// consecutive ones each (lane l of the row has elements 16l .. 16l+15), so a wave quantizes four blocks at once and
+// the cross-lane steps are four row exchanges instead of eight over the wave: about 45 vector instructions per block
+// against 75 -- what the decode GEMV's prologue is made of.  The same values as q8_K_quantize_lane (the maximum is
+// exact whatever the order; the first element that holds it is the lowest such index of the lowest such lane).
+// Returns the lane's sixteen quants; d is valid in every lane of the row; sum16 = bsums[l] is the lane's own sum and
+// pair32 = bsums[2j] + bsums[2j+1] for j = l/2.
+__device__ __forceinline__ uint4 q8_K_quantize_row16(const float4 (&v)[4], int lane, float &d, int &sum16, int &pair32) {
+    const float e[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
+                         v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(e[i]));
+    float wmax = fmaxf(amax, dpp_f<DPP_XOR1>(amax, amax));
+    wmax = fmaxf(wmax, dpp_f<DPP_XOR2>(wmax, wmax));
+    wmax = fmaxf(wmax, dpp_f<DPP_HALF_MIRROR>(wmax, wmax));
+    wmax = fmaxf(wmax, dpp_f<DPP_MIRROR>(wmax, wmax));  // every lane of the row: the block's maximum
+    float mine = 0.0f;  // this lane's first element of that magnitude, if it has one
+#pragma unroll
+    for (int i = 15; i >= 0; i--) mine = fabsf(e[i]) == wmax ? e[i] : mine;
+    const unsigned long long holders = __ballot(amax == wmax);
+    const unsigned in_row = (unsigned)(holders >> (lane & 48)) & 0xffffu;  // never empty: some lane of the row holds its maximum
+    const int first = (lane & 48) + __ffs((int)in_row) - 1;
+    const float wmx = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * first, __float_as_int(mine)));
+    const bool any = wmax != 0.0f;
+    const float iscale = any ? -127.0f / wmx : 0.0f;  // an all-zero block: every product is (signed) zero, every quant 0
+    int q[16];
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        q[i] = min(127, (int)rintf(iscale * e[i]));
+        s += q[i];
+    }
+    sum16 = s;
+    pair32 = s + dpp_i<DPP_XOR1>(0, s);
+    d = any ? 1.0f / iscale : 0.0f;
+    return make_uint4((unsigned)pack4_i8(q[0], q[1], q[2], q[3]), (unsigned)pack4_i8(q[4], q[5], q[6], q[7]),
+                      (unsigned)pack4_i8(q[8], q[9], q[10], q[11]), (unsigned)pack4_i8(q[12], q[13], q[14], q[15]));
+}
+
 }  // namespace miqmm

@@ -325,6 +325,36 @@ def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
             W.free()
 
 
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+def test_in_kernel_q8_K_quantizer_edge_blocks_give_the_same_bits(ctx, t):
+    """The decode prologue quantizes Q8_K blocks with sixteen lanes per block, the stand-alone kernel with a wave per
+    block.  Blocks built to tell them apart: zeros; the same magnitude twice with opposite signs, first positive and
+    first negative, in one lane's sixteen elements and lanes apart; the maximum in the very last element; huge and
+    tiny magnitudes; products that land on .5; five blocks, so the last group of four is one block long."""
+    k, m = 1280, 200
+    w_raw = _weights(t, m, k, seed=91 + t)
+    W = ctx.upload(t, w_raw, k, m)
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((2, k)).astype(np.float32)
+    x[0, 0:256] = 0.0
+    x[0, 256:512] *= 0.1; x[0, 256 + 7] = 3.0; x[0, 256 + 200] = -3.0
+    x[0, 512:768] *= 0.1; x[0, 512 + 35] = -3.0; x[0, 512 + 36] = 3.0
+    x[0, 768:1024] *= 0.1; x[0, 1023] = -2.5
+    x[0, 1024:1280] = 1e-30; x[0, 1024 + 100] = 1e20
+    x[1, 0:256] = np.arange(256, dtype=np.float32) - 127.5          # every product iscale * x a multiple of .5
+    x[1, 256:512] = 0.0; x[1, 256 + 255] = -0.0
+    x[1, 512:768] = 127.0; x[1, 512 + 16] = -127.0                   # first maximum positive, the other sign later
+    x[1, 768:1024] = -1.0
+    for n in (1, 2):
+        act = ctx.act_create(Q8_K, k, n)
+        ctx.act_quantize(act, x[:n])
+        want = ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV)
+        assert np.array_equal(ctx.mulmat(W, x[:n], path=qmm.PATH_GEMV), want), n
+        assert np.all(np.isfinite(want))
+        act.free()
+    W.free()
+
+
 @pytest.mark.parametrize("t,k", [(Q4_K, 14336), (Q4_K, 8192), (Q6_K, 4352), (Q4_0, 4096), (Q8_0, 4096), (Q8_0, 2080)])
 def test_long_rows_at_one_column(ctx, t, k):
     """One column, rows of several K segments (the waves of a workgroup cut K and combine through LDS): same
