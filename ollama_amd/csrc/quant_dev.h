@@ -130,18 +130,30 @@ __device__ __forceinline__ uint4 q8_K_quantize_row16(const float4 (&v)[4], int l
     const float wmx = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * first, __float_as_int(mine)));
     const bool any = wmax != 0.0f;
     const float iscale = any ? -127.0f / wmx : 0.0f;  // an all-zero block: every product is (signed) zero, every quant 0
-    int q[16];
-    int s = 0;
+    // q = min(127, rne(p)), p = the fp32-rounded product iscale * e.  |p| <= fl(fl(127 / |max|) * |max|), which is 127
+    // or the next float above it, so the min never acts; and for |p| < 2^22 adding 1.5 * 2^23 rounds p to the nearest
+    // integer, ties to even, and leaves it in the low mantissa bits: t = p + magic, q = bits(t) - bits(magic), the
+    // low byte of bits(t) is the quant's byte.  (The product is rounded before the add: no contraction in this file.)
+    const float magic = 12582912.0f;
+    unsigned t[16], us = 0;  // (unsigned: the sum of sixteen bit patterns wraps before bits(magic) comes off again)
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        q[i] = min(127, (int)rintf(iscale * e[i]));
-        s += q[i];
+        t[i] = __float_as_uint(iscale * e[i] + magic);
+        us += t[i];
     }
+    const int s = (int)(us - 16u * 0x4B400000u);  // bits(magic) = 0x4B400000
     sum16 = s;
     pair32 = s + dpp_i<DPP_XOR1>(0, s);
     d = any ? 1.0f / iscale : 0.0f;
-    return make_uint4((unsigned)pack4_i8(q[0], q[1], q[2], q[3]), (unsigned)pack4_i8(q[4], q[5], q[6], q[7]),
-                      (unsigned)pack4_i8(q[8], q[9], q[10], q[11]), (unsigned)pack4_i8(q[12], q[13], q[14], q[15]));
+    uint4 out;
+    unsigned *o = &out.x;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {  // the low bytes of four words
+        const unsigned lo = __builtin_amdgcn_perm(t[4 * j + 1], t[4 * j], 0x0c0c0400u);      // [t0.b0, t1.b0, 0, 0]
+        const unsigned hi = __builtin_amdgcn_perm(t[4 * j + 3], t[4 * j + 2], 0x04000c0cu);  // [0, 0, t2.b0, t3.b0]
+        o[j] = lo | hi;
+    }
+    return out;
 }
 
 }  // namespace miqmm
