@@ -39,19 +39,24 @@ def rel_err(y, ref, floor=1e-2):
 
 
 def observed_clocks():
-    """current shader / memory clock as rocm-smi reports them right now (None where it cannot be read)"""
+    """current shader / memory clock as the driver reports them right now through sysfs (the level marked '*' in
+    pp_dpm_sclk / pp_dpm_mclk of the first GPU that has them); None where they cannot be read.  No child process:
+    a process that has initialised the GPU must not start one that re-executes itself."""
+    import glob
     import re
-    import subprocess
-    try:
-        txt = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
-    except Exception:
-        return None
     out = {}
     for key in ("sclk", "mclk", "fclk"):
-        m = re.search(key + r" clock level: \S+ \((\d+)Mhz\)", txt)
-        if m:
-            out[key + "_mhz"] = int(m.group(1))
+        for path in sorted(glob.glob(f"/sys/class/drm/card*/device/pp_dpm_{key}")):
+            try:
+                txt = open(path).read()
+            except OSError:
+                continue
+            m = re.search(r"(\d+)\s*Mhz\s*\*", txt, re.IGNORECASE)
+            if m:
+                out[key + "_mhz"] = int(m.group(1))
+                break
     return out or None
+
 
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
