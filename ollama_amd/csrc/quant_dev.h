@@ -111,7 +111,9 @@ __device__ __forceinline__ int q8_K_quantize_lane(const float4 v, int lane, floa
 // exact whatever the order; the first element that holds it is the lowest such index of the lowest such lane).
 // Returns the lane's sixteen quants; d is valid in every lane of the row; sum16 = bsums[l] is the lane's own sum and
 // pair32 = bsums[2j] + bsums[2j+1] for j = l/2.
-__device__ __forceinline__ uint4 q8_K_quantize_row16(const float4 (&v)[4], int lane, float &d, int &sum16, int &pair32) {
+// qfl (optional): the sixteen quants as floats (exact), for callers that also write them out as fp16.
+__device__ __forceinline__ uint4 q8_K_quantize_row16(const float4 (&v)[4], int lane, float &d, int &sum16, int &pair32,
+                                                     float *qfl = nullptr) {
     const float e[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
                          v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
     float amax = 0.0f;
@@ -138,8 +140,10 @@ __device__ __forceinline__ uint4 q8_K_quantize_row16(const float4 (&v)[4], int l
     unsigned t[16], us = 0;  // (unsigned: the sum of sixteen bit patterns wraps before bits(magic) comes off again)
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        t[i] = __float_as_uint(iscale * e[i] + magic);
+        const float r = iscale * e[i] + magic;
+        t[i] = __float_as_uint(r);
         us += t[i];
+        if (qfl) qfl[i] = r - magic;  // exact: both are integers below 2^24
     }
     const int s = (int)(us - 16u * 0x4B400000u);  // bits(magic) = 0x4B400000
     sum16 = s;

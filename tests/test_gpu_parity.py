@@ -34,7 +34,7 @@ def _weights(t, m, k, seed, nthreads=16):
 
 # ---- kernel 1: activation quantization, bit-exact ---------------------------------------------
 @pytest.mark.parametrize("qt", [Q8_0, Q8_K])
-@pytest.mark.parametrize("n,k", [(1, 256), (1, 4096), (3, 1024), (8, 4096), (1, 14336), (512, 4096), (5, 14336)])
+@pytest.mark.parametrize("n,k", [(1, 256), (1, 4096), (3, 1024), (8, 4096), (1, 14336), (512, 4096), (5, 14336), (293, 14336), (4099, 256)])
 def test_quantize_act_bit_exact(ctx, qt, n, k):
     rng = np.random.default_rng(n * 100003 + k + qt)
     x = rng.standard_normal((n, k), dtype=np.float32)
@@ -67,6 +67,16 @@ def test_quantize_act_edge_cases_bit_exact(ctx, qt):
     want = oracle.quantize(qt, x)
     bad = np.argwhere(got != want)
     assert bad.size == 0, f"first differing (row, byte): {bad[:5].tolist()}"
+    # the same rows as a batch large enough for the kernel that puts a Q8_K block on sixteen lanes (from 4096
+    # blocks), shifted by one block per copy so that every edge block meets every position in a wave's group of four,
+    # and with a row count that leaves the last group of four incomplete
+    reps = 411
+    big = np.concatenate([np.roll(x, 256 * i, axis=1) for i in range(reps)])[: reps * len(rows) - 1]
+    big = np.ascontiguousarray(big[:, : k - 256])                            # 3 blocks per row: groups straddle rows
+    got = ctx.quantize_act(qt, big)
+    want = oracle.quantize(qt, big, nthreads=8)
+    bad = np.argwhere(got != want)
+    assert bad.size == 0, f"batch: first differing (row, byte): {bad[:5].tolist()}"
 
 
 def test_quantize_act_empty_and_errors(ctx):
