@@ -131,7 +131,10 @@ def test_decode_product_fused_with_its_producer(ctx, t, k, m, producer):
 
 # batches: fused quantizer (RMSNorm: row scales first), then the GEMV / skinny / GEMM kernels
 @pytest.mark.parametrize("t,k,m,n", [(Q4_K, 4096, 200, 2), (Q4_K, 2048, 100, 5), (Q6_K, 1024, 130, 12), (Q4_K, 1024, 257, 70),
-                                     (Q8_0, 1056, 90, 3), (Q4_0, 512, 64, 40), (Q8_0, 4096, 64, 9)])
+                                     (Q8_0, 1056, 90, 3), (Q4_0, 512, 64, 40), (Q8_0, 4096, 64, 9),
+                                     # prefill sizes: the fused quantizer with sixteen lanes per block writes the fp16
+                                     # planes too; the products run on the 256-row kernels (fp16 MFMA; Q6_K with K slices)
+                                     (Q4_K, 2048, 12300, 512), (Q6_K, 3328, 5000, 512)])
 @pytest.mark.parametrize("producer", [qmm.PRODUCE_RMSNORM, qmm.PRODUCE_SWIGLU])
 def test_batch_product_fused_with_its_producer(ctx, t, k, m, n, producer):
     rng = np.random.default_rng(t * 1000 + k + m + n + producer)
