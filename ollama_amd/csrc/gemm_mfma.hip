@@ -30,6 +30,8 @@
 #include <hip/hip_fp16.h>
 
 
+#include <type_traits>
+
 #include "internal.h"
 
 namespace miqmm {
@@ -213,6 +215,41 @@ struct GemmQ6K {
 
 typedef __attribute__((address_space(3))) void lds_ptr_t;
 typedef const __attribute__((address_space(1))) void glb_ptr_t;
+
+// Direct-to-LDS copies issued from inline assembly, for kernels that keep several stages in flight and count
+// their waits by hand (after the compiler's builtin every later LDS read waits for all copies in flight: it
+// cannot tell which stage a read touches).  Lane l's BYTES (16 or 4) at base + off land at lds_address +
+// BYTES * l; base and lds_address are wave-uniform.
+__device__ __forceinline__ unsigned lds_addr(const void *p) {
+    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
+}
+template <int BYTES>
+__device__ __forceinline__ void dma_lds(const uint8_t *base, unsigned off, unsigned lds_address) {
+    const unsigned long long v = (unsigned long long)base;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    base = (const uint8_t *)(((unsigned long long)hi << 32) | lo);
+    lds_address = __builtin_amdgcn_readfirstlane(lds_address);
+    if (BYTES == 16)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds_address) : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(lds_address) : "memory");
+}
+// LDS reads through a 32-bit LDS address plus a compile-time offset (the offset goes into the instruction)
+template <class T>
+__device__ __forceinline__ T lds_at(unsigned address, int imm) {
+    return *(const __attribute__((address_space(3))) T *)(uintptr_t)(address + (unsigned)imm);
+}
+__device__ __forceinline__ uint4 lds_u4(unsigned address, int imm) {
+    typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+    const u4_t v = lds_at<u4_t>(address, imm);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+// wait until at most N vector-memory operations of this wave are outstanding (they retire in order)
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    static_assert(N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 // ---------------------------------------------------------------------------------------------
 // Everything through LDS.  Loading the packed weights straight into the lanes that expand them costs a
@@ -589,6 +626,17 @@ struct Sk16Q6K {
     // step t, K group g = scale group 4t + g (16 elements).  With H = t>>1, rr = 2(t&1) + (g>>1):
     // ql bytes [64H + 32(g>>1) + 16(g&1), +16) = piece 4H + g, nibble t&1; qh bytes [32H + 16(g&1), +16) >> 2rr.
     struct Raw { uint4 L[2], Hq[2], scv; };
+    // the lane's read offsets into a weight stage: ql of half H at ro[H], qh at ro[2 + H], scales at ro[4]
+    static constexpr int NRO = 5;
+    static __device__ __forceinline__ void read_plan(int c, int g, unsigned (&ro)[NRO]) {
+        const int xl = (c >> 1) & 7, xh = quad_swz(c >> 2);
+#pragma unroll
+        for (int H = 0; H < 2; H++) {
+            ro[H] = c * 128 + 16 * ((4 * H + g) ^ xl);
+            ro[2 + H] = 2048 + c * 64 + 16 * ((2 * H + (g & 1)) ^ xh);
+        }
+        ro[4] = 3072 + c * 16;
+    }
     static __device__ __forceinline__ void read(const uint8_t *wt, int c, int g, Raw &raw) {
         const int xl = (c >> 1) & 7, xh = quad_swz(c >> 2);
 #pragma unroll
@@ -964,6 +1012,246 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
 }
 
 // ---------------------------------------------------------------------------------------------
+// Q6_K products with very many rows, few columns and a short K (the output head at 3..8 tokens).
+//
+// What bounds the kernel above on this shape is neither its arithmetic nor HBM bandwidth but the number of
+// copy instructions and of cache lines they name: per 16 rows and super-block it issues nine direct-to-LDS
+// copies that touch 96 lines -- among them 16 bytes of sub-block scales out of each of 16 lines, 2 bytes of
+// super-block scale out of 16 more, and the activations' quants, digits and scales again for every row group.
+// With everything but the copies taken out it ran no faster; without the small copies it ran at HBM speed.
+//
+// So this kernel copies per super-block only what is new (ql: 16 x 128 B, qh: 16 x 64 B; three instructions)
+// and fetches the rest in whole lines: the sub-block scales of eight super-blocks at once (16 lines, two
+// instructions per eight super-blocks), the super-block scales of all of a row group's super-blocks (one
+// instruction per row group), and the activations -- which are the same for every row group -- once per
+// workgroup into LDS, where they stay.  A workgroup is eight waves on one CU; a wave owns whole row groups
+// (all of K, so no partial sums) and streams its weights through its own ring of three stages.
+//
+// Copy order and waits: a wave issues, for the super-block its copy cursor stands on, first the whole-line
+// copies that start there (super-block scales at a row group's first super-block, sub-block scales at every
+// eighth), then the three weight copies.  Waiting until at most six copies are outstanding therefore means
+// that the stage about to be multiplied has landed together with every whole-line copy issued before it.
+// ---------------------------------------------------------------------------------------------
+template <int NCT>
+struct RowsGeo {
+    // resident activations, per super-block: 256 zero bytes (operand lanes that carry zeros read here), quants
+    // [column][16 pieces, swizzled], block-sum digits [column][32 B], scales [column] (padded to 256 B)
+    static constexpr int Z_OFF = 0, A_OFF = 256, D_OFF = A_OFF + NCT * 256, Y_OFF = D_OFF + NCT * 32, RB = Y_OFF + 256;
+    // per wave: three weight stages (ql [16 rows][8 pieces] at 0, qh [16][4] at 2 KiB), two buffers of sub-block
+    // scales (16 lines of 128 B = eight super-blocks), two of super-block scales (16 rows x up to 16 halves)
+    static constexpr int NST = 3, W_STAGE = 3072, SC_BYTES = 2048, DH_BYTES = 512;
+    static constexpr int SC_OFF = NST * W_STAGE, DH_OFF = SC_OFF + 2 * SC_BYTES, WAVE_BYTES = DH_OFF + 2 * DH_BYTES;
+    static constexpr int WAVES = 8;
+    static constexpr size_t lds_bytes(int64_t nsb) { return (size_t)nsb * RB + (size_t)WAVES * WAVE_BYTES; }
+};
+
+template <int NCT>
+__global__ __launch_bounds__(512, 2) void skinny_rows_q6k_kernel(DevWeight w, DevAct a, int col0, int nc, float *__restrict__ y, int grid_size) {
+    typedef Sk16Q6K S;
+    typedef GemmQ6K G;
+    typedef RowsGeo<NCT> Geo;
+    constexpr int SETS = NCT / S::SET_COLS, A_INSTRS = NCT / 4;
+    static_assert(S::LANE_COLS == 1, "one output column per lane and column set");
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int nsb = (int)(w.K / QKK);  // 8 or 16
+    const unsigned res_a = lds_addr(smem), wv_a = res_a + (unsigned)nsb * Geo::RB + (unsigned)wave * Geo::WAVE_BYTES;
+
+    // ---- the activations, once per workgroup: wave v copies super-blocks v, v + 8
+    for (int i = tid; i < nsb * 64; i += 64 * Geo::WAVES) *reinterpret_cast<int *>(smem + (i >> 6) * Geo::RB + 4 * (i & 63)) = 0;
+    {
+        auto acol = [&](int i) { return col0 + min(i, nc - 1); };
+        const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
+        unsigned aoff[A_INSTRS];
+#pragma unroll
+        for (int j = 0; j < A_INSTRS; j++) {
+            const int col = 4 * j + (lane >> 4), slot = lane & 15;  // slot [col][slot] holds piece slot ^ a_swz(col)
+            aoff[j] = (unsigned)acol(col) * (unsigned)a.K + 16u * (slot ^ S::a_swz(col));
+        }
+        const bool don = lane < 2 * NCT, yon = lane < NCT;
+        const unsigned doff = (unsigned)acol(lane >> 1) * (unsigned)(nsb * G::SD) + 16u * (lane & 1);
+        const unsigned yoff = (unsigned)acol(lane) * (unsigned)nsb * 4u;
+        for (int sb = wave; sb < nsb; sb += Geo::WAVES) {
+            const unsigned sa = res_a + (unsigned)sb * Geo::RB;
+#pragma unroll
+            for (int j = 0; j < A_INSTRS; j++) dma_lds<16>(aq + (int64_t)sb * QKK, aoff[j], sa + Geo::A_OFF + 1024 * j);
+            if (don) dma_lds<16>(a.sd16 + (int64_t)sb * G::SD, doff, sa + Geo::D_OFF);
+            if (yon) dma_lds<4>(reinterpret_cast<const uint8_t *>(a.d) + (int64_t)sb * 4, yoff, sa + Geo::Y_OFF);
+        }
+    }
+
+    // ---- the wave's row groups: ((k * grid + workgroup) * 8 + wave), k = 0, 1, ...: the eight waves of a workgroup
+    // stream 128 consecutive rows at a time
+    const int64_t groups = (w.M + 15) / 16;
+    auto item_group = [&](int64_t k) { return (k * grid_size + (int64_t)blockIdx.x) * Geo::WAVES + wave; };
+    int64_t items = 0;
+    if (item_group(0) < groups) items = (groups - 1 - item_group(0)) / ((int64_t)grid_size * Geo::WAVES) + 1;
+
+    // ---- copy plan: per-lane 32-bit offsets from uniform bases
+    unsigned woff[3], scoff[2], dhoff = 0;
+    const bool dhon = lane < 2 * nsb;
+    int64_t cp_m0 = 0, cp_k = 0;
+    int cp_sb = 0;
+    unsigned cp_half = 0;  // eight-super-block runs copied so far: run h goes to scale buffer h & 1
+    auto plan_item = [&](int64_t k) __attribute__((always_inline)) {
+        cp_m0 = item_group(k) * 16;
+        const int rows = (int)min((int64_t)16, w.M - cp_m0);  // rows past M: the last row again, results dropped
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            bool on;
+            S::w_plan(w, j, lane, rows, woff[j], on);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            // scale buffer slot P = 64 i + lane (16 B each): line P >> 3 holds row L ^ (L >> 3), and inside the line
+            // piece p of row r sits at position p ^ (r & 7) -- the sixteen rows of a read then fall on sixteen
+            // different slots of the LDS's 256-byte bank period
+            const int P = 64 * i + lane, L = P >> 3, r = L ^ (L >> 3), p = (P & 7) ^ (r & 7);
+            scoff[i] = (unsigned)min(r, rows - 1) * (unsigned)(nsb * 16) + 16u * p;
+        }
+        {
+            const int row = (16 * lane) / (2 * nsb), within = (16 * lane) % (2 * nsb);
+            dhoff = (unsigned)min(row, rows - 1) * (unsigned)(2 * nsb) + within;
+        }
+    };
+    auto stage_copy = [&](unsigned st) __attribute__((always_inline)) {
+        const int sb = cp_sb;
+        if (sb == 0 && dhon)
+            dma_lds<16>(reinterpret_cast<const uint8_t *>(w.d) + cp_m0 * nsb * 2, dhoff, wv_a + Geo::DH_OFF + (unsigned)(cp_k & 1) * Geo::DH_BYTES);
+        if ((sb & 7) == 0) {
+            const uint8_t *base = w.p2 + cp_m0 * (w.K / 16) + (sb >> 3) * 128;
+            const unsigned dst = wv_a + Geo::SC_OFF + (cp_half & 1) * Geo::SC_BYTES;
+            dma_lds<16>(base, scoff[0], dst);
+            dma_lds<16>(base, scoff[1], dst + 1024);
+            cp_half++;
+        }
+#pragma unroll
+        for (int j = 0; j < 3; j++) dma_lds<16>(S::w_base(w, j, cp_m0, sb), woff[j], st + 1024 * j);
+        if (cp_sb + 1 < nsb) {
+            cp_sb++;
+        } else if (cp_k + 1 < items) {
+            cp_k++;
+            cp_sb = 0;
+            plan_item(cp_k);
+        }  // past the last super-block of the last row group the cursor stays put: the copy is repeated
+    };
+
+    // ---- operand reads: absolute LDS addresses, pinned in registers
+    unsigned wro[S::NRO];
+    S::read_plan(c, g, wro);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        wro[i] += wv_a;
+        asm volatile("" : "+v"(wro[i]));
+    }
+    const unsigned scro = wv_a + Geo::SC_OFF + (unsigned)(c ^ (c >> 3)) * 128u;  // the lane's row in a scale buffer
+    const unsigned dhro = wv_a + Geo::DH_OFF + (unsigned)c * (unsigned)(2 * nsb);
+    unsigned aro[SETS][4], dro[SETS], yro[SETS];
+#pragma unroll
+    for (int cs = 0; cs < SETS; cs++) {
+        const int col = S::SET_COLS * cs + S::a_col(c);
+        const bool on = col < nc;
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+            aro[cs][t] = res_a + (on && S::a_on(c, g) ? Geo::A_OFF + col * 256 + 16 * ((4 * t + g) ^ S::a_swz(col)) : S::a_zero(cs, t));
+        dro[cs] = res_a + (on && S::d_on(c, g) ? Geo::D_OFF + col * 32 + S::d_off(c) : 128 * ((cs & 1) ^ 1));
+        yro[cs] = res_a + Geo::Y_OFF + 4 * min(S::SET_COLS * cs + S::lane_col(g, 0), NCT - 1);  // columns past nc: any staged scale
+    }
+
+    if (items > 0) {
+        plan_item(0);
+#pragma unroll
+        for (int i = 0; i < Geo::NST; i++) stage_copy(wv_a + i * Geo::W_STAGE);
+    }
+    // the activations have landed (a wave's own copies: all but the nine just issued; everybody's: the barrier)
+    if (items > 0) wait_vm<3 * Geo::NST + 3>();
+    else wait_vm<0>();
+    __syncthreads();
+
+    const v4acc zero = {0, 0, 0, 0};
+    unsigned parity = 0, half_run = 0;
+#pragma unroll 1
+    for (int64_t k = 0; k < items; k++) {
+        const int64_t m0 = item_group(k) * 16;
+        const int rows_left = (int)min((int64_t)16, w.M - m0);
+        float acc[SETS];
+#pragma unroll
+        for (int i = 0; i < SETS; i++) acc[i] = 0.f;
+        const unsigned dh_a = dhro + (unsigned)(k & 1) * Geo::DH_BYTES;
+        auto step = [&](auto stg, int sb) __attribute__((always_inline)) {
+            constexpr int STG = decltype(stg)::value;
+            wait_vm<3 * (Geo::NST - 1)>();
+            typename S::Raw raw;
+#pragma unroll
+            for (int H = 0; H < 2; H++) {
+                raw.L[H] = lds_u4(wro[H], STG * Geo::W_STAGE);
+                raw.Hq[H] = lds_u4(wro[2 + H], STG * Geo::W_STAGE);
+            }
+            raw.scv = lds_u4(scro + ((half_run + (unsigned)(sb >> 3)) & 1) * Geo::SC_BYTES + 16u * ((sb & 7) ^ (c & 7)), 0);
+            const unsigned dh = lds_at<unsigned short>(dh_a + 2u * (unsigned)sb, 0);
+            const unsigned ro = (unsigned)sb * Geo::RB;
+            v4i av[SETS][4], sv[SETS];
+            float ydv[SETS];
+#pragma unroll
+            for (int cs = 0; cs < SETS; cs++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) av[cs][t] = lds_at<v4i>(aro[cs][t] + ro, 0);
+                sv[cs] = lds_at<v4i>(dro[cs] + ro, 0);
+                ydv[cs] = lds_at<float>(yro[cs] + ro, 0);
+            }
+            // operands are in registers: the stage can take the copies of the super-block after next
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            stage_copy(wv_a + STG * Geo::W_STAGE);
+            typename S::Ops b;
+            S::expand(raw, g, dh, b);
+#pragma unroll
+            for (int cs = 0; cs < SETS; cs++) {
+                const v4acc x = mfma16(S::d_fix(sv[cs], c), b.bsum, zero);
+                int isum[1] = {0};
+#pragma unroll
+                for (int t = 0; t < 4; t++) S::scale_step(mfma16(av[cs][t], b.q[t], zero), t, b, isum);
+                acc[cs] = __builtin_fmaf(ydv[cs], S::finish(b, isum[0], x, 0), acc[cs]);
+            }
+        };
+#pragma unroll 1
+        for (int sb = 0; sb < nsb; sb++) {
+            if (parity == 0) step(std::integral_constant<int, 0>{}, sb);
+            else if (parity == 1) step(std::integral_constant<int, 1>{}, sb);
+            else step(std::integral_constant<int, 2>{}, sb);
+            parity = parity == Geo::NST - 1 ? 0 : parity + 1;
+        }
+        half_run += (unsigned)(nsb >> 3);
+        // lane l holds weight row l & 15 of column 4 cs + (l >> 4)
+#pragma unroll
+        for (int cs = 0; cs < SETS; cs++) {
+            const int col = S::SET_COLS * cs + g;
+            if (col < nc && c < rows_left) y[(int64_t)(col0 + col) * w.M + m0 + c] = acc[cs];
+        }
+    }
+    wait_vm<0>();  // the repeated copies at the end must not outlive the kernel's LDS
+}
+
+bool skinny_rows_wanted(const DevWeight &w, int ncols, int num_cus) {
+    const int64_t nsb = w.K / QKK;
+    return w.type == T_Q6_K && ncols >= 1 && ncols <= 8 && (nsb == 8 || nsb == 16) &&
+           (w.M + 15) / 16 >= (int64_t)16 * num_cus;  // two row groups and more for every wave of a full grid
+}
+
+void launch_skinny_rows(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
+    typedef RowsGeo<8> Geo;
+    const size_t lds = Geo::lds_bytes(w.K / QKK);
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_rows_q6k_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  160 * 1024);
+        allowed[dev] = true;
+    }
+    skinny_rows_q6k_kernel<8><<<(unsigned)num_cus, 64 * Geo::WAVES, lds, s>>>(w, a, col0, ncols, y, num_cus);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Q4_K at up to four activation columns with the weights loaded straight into the MFMA operand
 // registers: the faster of the two skinny kernels while the matrix is small enough that latency, not
 // HBM time, decides (launch_skinny picks).  A 16-row group is cut kcut ways along K, one wave per cut;
@@ -1276,7 +1564,8 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
         else if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q4K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     } else {
-        if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
+        if (skinny_rows_wanted(w, ncols, num_cus)) launch_skinny_rows(w, a, col0, ncols, y, num_cus, s);
+        else if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q6K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     }
     return hipGetLastError();
