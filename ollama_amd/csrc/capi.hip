@@ -495,7 +495,7 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
             for (int64_t c0 = 0; c0 < n; c0 += 16)
                 HIP_TRY(launch_skinny32(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus,
                                         ctx->stream));
-        } else if (a.sd8 && wants_skinny(w->dev.type, K, M, n)) {
+        } else if (a.sd8 && (wants_skinny(w->dev.type, K, M, n) || (n >= 2 && n <= 8 && skinny_rows_wanted(w->dev, (int)n, ctx->num_cus)))) {
             // from a few columns up the K-quants go to the matrix cores, 16 columns per launch: the
             // streaming GEMV pays one v_dot4 pass per column
             for (int64_t c0 = 0; c0 < n; c0 += 16)

@@ -573,10 +573,10 @@ struct Sk16Q4K {
 #pragma unroll
             for (int i = 0; i < 4; i++) b.q[t][i] = (int)((v[i] >> (4 * hiN)) & 0x0f0f0f0fu);
         }
-        // block-sum MFMA: mins 0..7 in the first eight K slots of group 0, against the digits of the
-        // eight 32-element sums in the same slots of the A rows
-        const int mz = g == 0 ? -1 : 0;
-        b.bsum = (v4i){(int)mn03 & mz, (int)mn47 & mz, 0, 0};
+        // block-sum MFMA: mins 0..7 in the first eight K slots, against the digits of the eight 32-element sums
+        // in the same slots of the A rows (K group 0 only: in the other groups the A operand is zero, so what
+        // the B operand holds there does not matter)
+        b.bsum = (v4i){(int)mn03, (int)mn47, 0, 0};
     }
     // outputs v of a step's MFMA -> the lane's two columns
     static __device__ __forceinline__ void scale_step(const v4acc &dv, int t, const Ops &b, int (&isum)[LANE_COLS]) {
@@ -666,21 +666,25 @@ struct Sk16Q6K {
         b.dmin = 0.f;
 #pragma unroll
         for (int j = 0; j < 16; j++) b.sc[j] = (int)(int8_t)(scw[j >> 2] >> (8 * (j & 3)));
+        // Per pair of words (ql word l; qh word hq shifted so that the lane's two bit pairs sit at bits 0-1 and
+        // 4-5 of every byte): step 2H takes the low nibbles and the pair at bits 0-1, step 2H+1 the high nibbles
+        // and the pair at bits 4-5 -- seven instructions for eight bytes of operand.  0..63 per byte; the -32
+        // goes through the block sums.
+        const unsigned sh = 2 * (g >> 1);
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const int H = t >> 1;
-            const int rr2 = 2 * (2 * (t & 1) + (g >> 1));  // shift of the two high bits inside a qh byte
+        for (int H = 0; H < 2; H++) {
             const unsigned l[4] = {raw.L[H].x, raw.L[H].y, raw.L[H].z, raw.L[H].w};
             const unsigned hq[4] = {raw.Hq[H].x, raw.Hq[H].y, raw.Hq[H].z, raw.Hq[H].w};
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const unsigned nib = (t & 1) ? (l[i] >> 4) & 0x0f0f0f0fu : l[i] & 0x0f0f0f0fu;
-                b.q[t][i] = (int)(nib | (((hq[i] >> rr2) & 0x03030303u) << 4));  // 0..63 per byte; the -32 goes through the block sums
+                const unsigned hs = hq[i] >> sh;
+                b.q[2 * H][i] = (int)(((hs & 0x03030303u) << 4) | (l[i] & 0x0f0f0f0fu));
+                b.q[2 * H + 1][i] = (int)((hs & 0x30303030u) | ((l[i] >> 4) & 0x0f0f0f0fu));
             }
         }
-        // block-sum MFMA: the 16 scales in K group 0 against the digits of the sixteen 16-element sums
-        const int mz = g == 0 ? -1 : 0;
-        b.bsum = (v4i){(int)scw[0] & mz, (int)scw[1] & mz, (int)scw[2] & mz, (int)scw[3] & mz};
+        // block-sum MFMA: the 16 scales against the digits of the sixteen 16-element sums (K group 0 only: in
+        // the other groups the A operand is zero, so what the B operand holds there does not matter)
+        b.bsum = (v4i){(int)scw[0], (int)scw[1], (int)scw[2], (int)scw[3]};
     }
     static __device__ __forceinline__ void scale_step(const v4acc &dv, int t, const Ops &b, int (&isum)[LANE_COLS]) {
         isum[0] = mad24(b.sc[4 * t], dv[0], mad24(b.sc[4 * t + 1], dv[1], mad24(b.sc[4 * t + 2], dv[2],
@@ -1232,7 +1236,7 @@ __global__ __launch_bounds__(512, 2) void skinny_rows_q6k_kernel(DevWeight w, De
     wait_vm<0>();  // the repeated copies at the end must not outlive the kernel's LDS
 }
 
-bool skinny_rows_wanted(const DevWeight &w, int ncols, int num_cus) {
+bool rows_wanted(const DevWeight &w, int ncols, int num_cus) {
     const int64_t nsb = w.K / QKK;
     return w.type == T_Q6_K && ncols >= 1 && ncols <= 8 && (nsb == 8 || nsb == 16) &&
            (w.M + 15) / 16 >= (int64_t)16 * num_cus;  // two row groups and more for every wave of a full grid
@@ -1552,6 +1556,8 @@ void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, 
         launch_skinny_grid<S, NCT, ID, 2>(w, a, col0, ncols, y, si, grid, waves, s);
 }
 
+bool skinny_rows_wanted(const DevWeight &w, int ncols, int num_cus) { return rows_wanted(w, ncols, num_cus); }
+
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
     if (!skinny_supports(w.type, w.K, w.M) || a.type != T_Q8_K || a.K != w.K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
     if (ncols < 1 || ncols > 16 || col0 < 0 || col0 + ncols > a.N) return hipErrorInvalidValue;
@@ -1564,7 +1570,7 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
         else if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q4K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     } else {
-        if (skinny_rows_wanted(w, ncols, num_cus)) launch_skinny_rows(w, a, col0, ncols, y, num_cus, s);
+        if (rows_wanted(w, ncols, num_cus)) launch_skinny_rows(w, a, col0, ncols, y, num_cus, s);
         else if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q6K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     }

@@ -101,6 +101,8 @@ hipError_t launch_gemm_q6k(const DevWeight &w, const DevAct &a, float *y, float 
                            int num_cus, hipStream_t s);
 // 1..16 activation columns (col0 .. col0+ncols-1 of a) on the matrix cores, K-quants; y[n*M + m]
 bool skinny_supports(int type, int64_t K, int64_t M);
+// Q6_K with very many rows, K of 2048 or 4096 and up to 8 columns: launch_skinny then takes a kernel of its own
+bool skinny_rows_wanted(const DevWeight &w, int ncols, int num_cus);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                          hipStream_t s);
 // several K-quant matrices of one type and K in one launch of a skinny kernel (up to 16 columns), when every

@@ -903,8 +903,9 @@ def test_skinny_kquants_match_oracle(ctx, t, m, k, n):
 def test_q6k_many_rows_few_columns(ctx, m, k, n):
     """Q6_K with 65536 rows and more, K of 2048 or 4096 and 3..8 columns (the output head at a few tokens) takes a
     kernel of its own: activations resident in LDS, a row group's scales fetched in whole lines.  Ragged last row
-    group, both K sizes, every column set partly filled; a column's bits do not depend on the others; the same
-    matrix cut below 65536 rows goes through the general kernel and gives the same bits for the rows they share."""
+    group, both K sizes, every column set partly filled; a column's bits do not depend on the others; from four
+    columns up the same matrix cut below 65536 rows goes through the general kernel and gives the same bits for the
+    rows they share."""
     rng = np.random.default_rng(8300 + m + n)
     wb = _weights(Q6_K, m, k, 8301 + m)
     w = ctx.upload(Q6_K, wb, k, m)
@@ -915,10 +916,11 @@ def test_q6k_many_rows_few_columns(ctx, m, k, n):
     _check_against_exact_arithmetic(Q6_K, wb, k, m, x, got, f"Q6_K {m}x{k} n={n}", max_rows=4096)
     assert np.array_equal(ctx.mulmat(w, x[::-1].copy())[::-1], got)
     w.free()
-    rows = 40000
-    w2 = ctx.upload(Q6_K, np.ascontiguousarray(wb.reshape(m, -1)[:rows]).reshape(-1), k, rows)
-    assert np.array_equal(ctx.mulmat(w2, x), got[:, :rows])
-    w2.free()
+    if n >= 4:  # (three columns of a smaller matrix go to the streaming kernel, whose sums run in another order)
+        rows = 40000
+        w2 = ctx.upload(Q6_K, np.ascontiguousarray(wb.reshape(m, -1)[:rows]).reshape(-1), k, rows)
+        assert np.array_equal(ctx.mulmat(w2, x), got[:, :rows])
+        w2.free()
 
 
 @pytest.mark.parametrize("n", [3, 4, 6])
