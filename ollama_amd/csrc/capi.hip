@@ -450,7 +450,9 @@ namespace {
 // kernel instead of the streaming GEMV (measured crossovers on MI355X: the GEMV pays one v_dot4 pass
 // per column).
 bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
-    if (type == T_Q4_0 || type == T_Q8_0) return n >= 4 && skinny32_supports(type, K, M);
+    // (long rows of Q4_0 / Q8_0 from two columns: the GEMV at 4096 x 14336 takes 27 / 39 us at two / three columns of
+    // Q8_0 where the matrix-core kernel takes 17.5)
+    if (type == T_Q4_0 || type == T_Q8_0) return n >= (K > 8192 ? 2 : 4) && skinny32_supports(type, K, M);
     const int64_t from = type == T_Q4_K ? 3 : 4;
     return n >= from && skinny_supports(type, K, M);
 }

@@ -1232,14 +1232,22 @@ hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols,
 
 bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
     // Beyond 64 Ki rows (an output head) the redundant per-workgroup quantization costs more than the
-    // launch it saves.  The same goes for several columns (every workgroup quantizes all of them):
-    // measured against quantize-then-multiply, one column always wins, two (K-quants) or three
-    // (Q4_0 / Q8_0) columns only on small launches, where the saved launch is a larger share.
+    // launch it saves.  Several columns (every workgroup quantizes all of them), measured against
+    // quantize-then-multiply on matrices from 2 MB to 97 MB: two columns of the K-quants always win (gate 14336 x 4096
+    // 12.9 -> 12.0 us, down 4096 x 14336 14.9 -> 12.9, Q6_K 4096 x 14336 18.4 -> 14.3, gate + up in one launch 20.3 ->
+    // 18.9); three columns of Q6_K (which the matrix-core kernel takes from four) win from about 32 MB (22.2 -> 17.8 us
+    // at 48 MB) and lose below (6.6 -> 7.8 at 3 MB); two and three columns of Q4_0 / Q8_0 win at every size while rows
+    // are short (Q8_0 14336 x 4096: 17.6 -> 14.0 and 20.1 -> 17.9) and lose on long rows (Q4_0 4096 x 14336: 14.9 ->
+    // 19.5), which take the matrix-core kernel from two columns instead (wants_skinny in capi.hip).
     if (ncols < 1 || ncols > MAXC || K < 1 || total_m < 1 || total_m > 65536) return false;
     if (ncols > 1) {
         const bool kquant = type == T_Q4_K || type == T_Q6_K;
         const int64_t approx_bytes = total_m * K * (type == T_Q8_0 ? 34 : type == T_Q6_K ? 26 : 18) / 32;
-        if (ncols > (kquant ? 2 : 3) || approx_bytes > (20 << 20)) return false;
+        if (kquant) {
+            if (ncols > 3 || (ncols == 3 && (type != T_Q6_K || approx_bytes < (32 << 20)))) return false;
+        } else {
+            if (ncols > 3 || K > 8192) return false;
+        }
     }
     Plan p;
     switch (type) {

@@ -944,9 +944,10 @@ def test_skinny_q4k_random_block_bytes(ctx, n):
 # ---- skinny product on the matrix cores for the 32-element block formats ------------------------------
 @pytest.mark.parametrize("t", [Q4_0, Q8_0])
 @pytest.mark.parametrize("m,k,n", [(4096, 4096, 8), (1000, 1024, 5), (17, 256, 4), (300, 2304, 16), (64, 8192, 31),
-                                   (4096, 14336, 7)])
+                                   (4096, 14336, 7), (300, 14336, 2), (129, 9216, 3)])
 def test_skinny32_matches_oracle(ctx, t, m, k, n):
-    """4..31 columns, K a multiple of 256: ragged M, one 256-element step, K cut eight ways, two launches"""
+    """4..31 columns, K a multiple of 256: ragged M, one 256-element step, K cut eight ways, two launches; rows
+    longer than 8192 take this kernel from two columns"""
     rng = np.random.default_rng(7900 + t + m + n)
     wb = _weights(t, m, k, 7901 + t + m)
     w = ctx.upload(t, wb, k, m)
@@ -954,6 +955,25 @@ def test_skinny32_matches_oracle(ctx, t, m, k, n):
     got = ctx.mulmat(w, x)
     assert npref.rel_err(got, oracle.mul_mat(t, wb, k, m, x, nthreads=16)) < TOL
     # a column's result does not depend on which other columns ride along
+    assert np.array_equal(ctx.mulmat(w, x[::-1].copy())[::-1], got)
+    w.free()
+
+
+@pytest.mark.parametrize("t,m,k,n", [(Q4_K, 14336, 4096, 2), (Q4_K, 4096, 14336, 2), (Q6_K, 4096, 14336, 2),
+                                     (Q6_K, 4096, 14336, 3), (Q8_0, 14336, 4096, 3), (Q4_0, 14336, 4096, 2),
+                                     (Q8_0, 4096, 14336, 2), (Q4_0, 4096, 14336, 3)])
+def test_two_and_three_columns_on_large_matrices(ctx, t, m, k, n):
+    """Two and three columns at the feed-forward shapes, through the default routing: the streaming kernel with the
+    quantization of all columns in its prologue (K-quants at two columns, Q6_K at three from 32 MB, Q4_0 / Q8_0 with
+    rows up to 8192), the matrix-core kernel for long rows of Q4_0 / Q8_0.  Against the oracle and, at the tighter
+    floor, against exact arithmetic on the same quantized operands."""
+    rng = np.random.default_rng(8500 + t + m + n)
+    wb = _weights(t, m, k, 8501 + t + m)
+    w = ctx.upload(t, wb, k, m)
+    x = rng.standard_normal((n, k), dtype=np.float32)
+    got = ctx.mulmat(w, x)
+    assert npref.rel_err(got, oracle.mul_mat(t, wb, k, m, x, nthreads=16)) < TOL
+    _check_against_exact_arithmetic(t, wb, k, m, x, got, f"{NAMES[t]} {m}x{k} n={n}", max_rows=2048)
     assert np.array_equal(ctx.mulmat(w, x[::-1].copy())[::-1], got)
     w.free()
 
