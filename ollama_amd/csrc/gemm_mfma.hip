@@ -36,6 +36,8 @@
 
 namespace miqmm {
 
+int skinny_waves(int64_t row_groups, int64_t nsb, int num_cus);  // how many waves cut K in a workgroup of the general skinny kernel
+
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -537,6 +539,18 @@ struct Sk16Q4K {
     // step t covers sub-blocks 2t (low nibbles of qs bytes [32t, 32t+32)) and 2t+1 (high nibbles); K group
     // g of the step is elements 16(g&1).. of sub-block 2t + (g>>1): bytes [32t + 16(g&1), +16), nibble g>>1
     struct Raw { uint4 hdr, q[4]; };
+    // the lane's read offsets into a weight stage (header; first run of quants), then the reads of one super-block
+    // from absolute LDS addresses plus a compile-time offset
+    static constexpr int NRO = 2;
+    static __device__ __forceinline__ void read_plan(int c, int g, unsigned (&ro)[NRO]) {
+        ro[0] = c * 144;
+        ro[1] = c * 144 + 16 + 16 * ((g & 1) ^ half_swz(c));
+    }
+    static __device__ __forceinline__ void read(const unsigned (&wa)[NRO], int imm, Raw &raw) {
+        raw.hdr = lds_u4(wa[0], imm);
+#pragma unroll
+        for (int t = 0; t < 4; t++) raw.q[t] = lds_u4(wa[1], imm + 32 * t);
+    }
     static __device__ __forceinline__ void read(const uint8_t *wt, int c, int g, Raw &raw) {
         const uint8_t *p = wt + c * 144;
         raw.hdr = ld16(p);
@@ -1256,6 +1270,268 @@ void launch_skinny_rows(const DevWeight &w, const DevAct &a, int col0, int ncols
 }
 
 // ---------------------------------------------------------------------------------------------
+// The same for Q4_K at 3..16 columns on matrices with many rows and K up to 8192 (the feed-forward gate and up
+// projections at a few tokens, alone or both in one launch): of the seven copies the general kernel issues per 16
+// rows and super-block, four bring activations.  Here the activations are resident (per super-block: zero block,
+// quants, block-sum digits, scales), a wave owns whole row groups -- all of K, no partial sums -- and streams
+// only weights: three copies per super-block through a ring of four stages.  A workgroup has as many waves (up
+// to eight) as it takes to give every CU about the same number of row groups.
+//
+// Same bits as the general kernel: that one cuts a matrix's K between the waves of a workgroup (skinny_waves) and
+// adds the partial sums in order; a wave here restarts its fp32 accumulator at the same super-blocks and adds the
+// pieces in the same order, so a matrix gives the same result alone (either kernel) and in a joint launch.
+// ---------------------------------------------------------------------------------------------
+constexpr int ROWS_MULTI = 4;
+struct RowsArgs {
+    const uint8_t *p0[ROWS_MULTI];
+    float *y[ROWS_MULTI];
+    int64_t M[ROWS_MULTI];
+    int grp_end[ROWS_MULTI];  // exclusive end of each matrix's run of 16-row groups; INT_MAX past the last matrix
+    int kcut[ROWS_MULTI];     // how many ways the general kernel would cut K for this matrix alone (see below)
+    int64_t K;
+    int groups_total;
+};
+struct RowsWhere { const uint8_t *p0; float *y; int64_t M; int first, kcut; };
+__device__ __forceinline__ RowsWhere rows_where(const RowsArgs &g, int group) {
+    RowsWhere w{g.p0[0], g.y[0], g.M[0], 0, g.kcut[0]};
+#pragma unroll
+    for (int t = 1; t < ROWS_MULTI; t++)
+        if (group >= g.grp_end[t - 1]) w = RowsWhere{g.p0[t], g.y[t], g.M[t], g.grp_end[t - 1], g.kcut[t]};
+    return w;
+}
+
+template <int NCT>
+struct RowsGeoQ4K {
+    static constexpr int Z_OFF = 0, A_OFF = 256, D_OFF = A_OFF + NCT * 256, Y_OFF = D_OFF + NCT * 16;
+    static constexpr int RB = (Y_OFF + NCT * 4 + 255) / 256 * 256;
+    static constexpr int NST = 4, W_STAGE = 2560;  // 16 rows x 144 B, padded to the 256-byte bank period
+    static constexpr size_t lds_bytes(int64_t nsb, int waves) { return (size_t)nsb * RB + (size_t)waves * NST * W_STAGE; }
+};
+
+template <int NCT>
+__global__ __launch_bounds__(512, 2) void skinny_rows_q4k_kernel(RowsArgs ra, DevAct a, int col0, int nc, int grid_size, int waves) {
+    typedef Sk16Q4K S;
+    typedef GemmQ4K G;
+    typedef RowsGeoQ4K<NCT> Geo;
+    constexpr int SETS = NCT / S::SET_COLS, LANE_ACC = SETS * S::LANE_COLS, A_INSTRS = NCT / 4;
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int nsb = (int)(ra.K / QKK);
+    const unsigned res_a = lds_addr(smem), wv_a = res_a + (unsigned)nsb * Geo::RB + (unsigned)wave * (Geo::NST * Geo::W_STAGE);
+
+    // ---- the wave's row groups: ((k * grid + workgroup) * waves + wave), k = 0, 1, ...
+    auto item_group = [&](int64_t k) { return (k * grid_size + (int64_t)blockIdx.x) * waves + wave; };
+    int64_t items = 0;
+    if (item_group(0) < ra.groups_total) items = (ra.groups_total - 1 - item_group(0)) / ((int64_t)grid_size * waves) + 1;
+
+    // ---- weight copies: per-lane offsets from a uniform base per row group and super-block
+    unsigned woff[3];
+    bool won[3];
+    const uint8_t *cp_base = nullptr;
+    int64_t cp_k = 0;
+    int cp_sb = 0;
+    auto plan_item = [&](int64_t k) __attribute__((always_inline)) {
+        const int group = (int)item_group(k);
+        const RowsWhere at = rows_where(ra, group);
+        const int64_t first = (int64_t)(group - at.first) * 16;
+        const int rows = (int)min((int64_t)16, at.M - first);  // rows past M: the last row again, results dropped
+        const DevWeight w{at.p0, nullptr, nullptr, nullptr, ra.K, at.M, T_Q4_K};
+#pragma unroll
+        for (int j = 0; j < 3; j++) S::w_plan(w, j, lane, rows, woff[j], won[j]);
+        cp_base = S::w_base(w, 0, first, 0);
+    };
+    auto stage_copy = [&](unsigned st) __attribute__((always_inline)) {
+        const uint8_t *base = cp_base + (int64_t)cp_sb * Q4_K_BYTES;
+#pragma unroll
+        for (int j = 0; j < 3; j++)
+            if (won[j]) dma_lds<16>(base, woff[j], st + 1024 * j);
+        if (cp_sb + 1 < nsb) {
+            cp_sb++;
+        } else if (cp_k + 1 < items) {
+            cp_k++;
+            cp_sb = 0;
+            plan_item(cp_k);
+        }  // past the last super-block of the last row group the cursor stays put: the copy is repeated
+    };
+    if (items > 0) {
+        plan_item(0);
+#pragma unroll
+        for (int i = 0; i < Geo::NST; i++) stage_copy(wv_a + i * Geo::W_STAGE);
+    }
+
+    // ---- the activations, once per workgroup, behind the first weight copies: wave v copies super-blocks v, v + waves, ...
+    for (int i = tid; i < nsb * 64; i += 64 * waves) *reinterpret_cast<int *>(smem + (i >> 6) * Geo::RB + 4 * (i & 63)) = 0;
+    {
+        auto acol = [&](int i) { return col0 + min(i, nc - 1); };
+        const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
+        unsigned aoff[A_INSTRS];
+#pragma unroll
+        for (int j = 0; j < A_INSTRS; j++) {
+            const int col = 4 * j + (lane >> 4), slot = lane & 15;  // slot [col][slot] holds piece slot ^ a_swz(col)
+            aoff[j] = (unsigned)acol(col) * (unsigned)a.K + 16u * (slot ^ S::a_swz(col));
+        }
+        const bool don = lane < NCT, yon = lane < NCT;
+        const unsigned doff = (unsigned)acol(lane) * (unsigned)(nsb * G::SD);
+        const unsigned yoff = (unsigned)acol(lane) * (unsigned)nsb * 4u;
+        for (int sb = wave; sb < nsb; sb += waves) {
+            const unsigned sa = res_a + (unsigned)sb * Geo::RB;
+#pragma unroll
+            for (int j = 0; j < A_INSTRS; j++) dma_lds<16>(aq + (int64_t)sb * QKK, aoff[j], sa + Geo::A_OFF + 1024 * j);
+            if (don) dma_lds<16>(a.sd8 + (int64_t)sb * G::SD, doff, sa + Geo::D_OFF);
+            if (yon) dma_lds<4>(reinterpret_cast<const uint8_t *>(a.d) + (int64_t)sb * 4, yoff, sa + Geo::Y_OFF);
+        }
+    }
+    wait_vm<0>();  // (once: the weight copies issued above wait with it)
+    __syncthreads();
+
+    // ---- operand reads: absolute LDS addresses
+    unsigned wro[S::NRO];
+    S::read_plan(c, g, wro);
+#pragma unroll
+    for (int i = 0; i < S::NRO; i++) {
+        wro[i] += wv_a;
+        asm volatile("" : "+v"(wro[i]));
+    }
+    unsigned aro[SETS][4], dro[SETS], yro[LANE_ACC];
+#pragma unroll
+    for (int cs = 0; cs < SETS; cs++) {
+        const int col = S::SET_COLS * cs + S::a_col(c);
+        const bool on = col < nc;
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+            aro[cs][t] = res_a + (on && S::a_on(c, g) ? Geo::A_OFF + col * 256 + 16 * ((4 * t + g) ^ S::a_swz(col)) : S::a_zero(cs, t));
+        dro[cs] = res_a + (on && S::d_on(c, g) ? Geo::D_OFF + col * 16 + S::d_off(c) : 128 * ((cs & 1) ^ 1));
+#pragma unroll
+        for (int u = 0; u < S::LANE_COLS; u++)  // columns past nc: any staged scale (their sums are zero)
+            yro[cs * S::LANE_COLS + u] = res_a + Geo::Y_OFF + 4 * min(S::SET_COLS * cs + S::lane_col(g, u), NCT - 1);
+    }
+
+    const v4acc zero = {0, 0, 0, 0};
+    unsigned parity = 0;
+#pragma unroll 1
+    for (int64_t k = 0; k < items; k++) {
+        const int group = (int)item_group(k);
+        const RowsWhere at = rows_where(ra, group);
+        const int64_t m0 = (int64_t)(group - at.first) * 16;
+        const int rows_left = (int)min((int64_t)16, at.M - m0);
+        float acc[LANE_ACC], total[LANE_ACC];
+#pragma unroll
+        for (int i = 0; i < LANE_ACC; i++) acc[i] = total[i] = 0.f;
+        int cut = 1, next_cut = nsb / at.kcut;  // pieces of K as the general kernel cuts them: [nsb j / kcut, nsb (j + 1) / kcut)
+        auto step = [&](auto stg, int sb) __attribute__((always_inline)) {
+            constexpr int STG = decltype(stg)::value;
+            wait_vm<3 * (Geo::NST - 1)>();  // three copies per stage: this stage has landed, the next three may be in flight
+            typename S::Raw raw;
+            S::read(wro, STG * Geo::W_STAGE, raw);
+            const unsigned ro = (unsigned)sb * Geo::RB;
+            v4i av[SETS][4], sv[SETS];
+            float ydv[LANE_ACC];
+#pragma unroll
+            for (int cs = 0; cs < SETS; cs++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) av[cs][t] = lds_at<v4i>(aro[cs][t] + ro, 0);
+                sv[cs] = lds_at<v4i>(dro[cs] + ro, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < LANE_ACC; i++) ydv[i] = lds_at<float>(yro[i] + ro, 0);
+            // operands are in registers: the stage can take the copies of the super-block three ahead
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            stage_copy(wv_a + STG * Geo::W_STAGE);
+            typename S::Ops b;
+            S::expand(raw, g, 0, b);
+#pragma unroll
+            for (int cs = 0; cs < SETS; cs++) {
+                const v4acc x = mfma16(S::d_fix(sv[cs], c), b.bsum, zero);
+                int isum[S::LANE_COLS];
+#pragma unroll
+                for (int u = 0; u < S::LANE_COLS; u++) isum[u] = 0;
+#pragma unroll
+                for (int t = 0; t < 4; t++) S::scale_step(mfma16(av[cs][t], b.q[t], zero), t, b, isum);
+#pragma unroll
+                for (int u = 0; u < S::LANE_COLS; u++) {
+                    const int i = cs * S::LANE_COLS + u;
+                    acc[i] = __builtin_fmaf(ydv[i], S::finish(b, isum[u], x, u), acc[i]);
+                }
+            }
+        };
+#pragma unroll 1
+        for (int sb = 0; sb < nsb; sb++) {
+            if (sb == next_cut) {
+#pragma unroll
+                for (int i = 0; i < LANE_ACC; i++) {
+                    total[i] += acc[i];
+                    acc[i] = 0.f;
+                }
+                cut++;
+                next_cut = nsb * cut / at.kcut;
+            }
+            if (parity == 0) step(std::integral_constant<int, 0>{}, sb);
+            else if (parity == 1) step(std::integral_constant<int, 1>{}, sb);
+            else if (parity == 2) step(std::integral_constant<int, 2>{}, sb);
+            else step(std::integral_constant<int, 3>{}, sb);
+            parity = (parity + 1) & 3;
+        }
+        // lane l holds weight row l & 15 of columns SET_COLS*cs + lane_col(l >> 4, u)
+#pragma unroll
+        for (int cs = 0; cs < SETS; cs++)
+#pragma unroll
+            for (int u = 0; u < S::LANE_COLS; u++) {
+                const int col = S::SET_COLS * cs + S::lane_col(g, u), i = cs * S::LANE_COLS + u;
+                if (col < nc && c < rows_left) at.y[(int64_t)(col0 + col) * at.M + m0 + c] = total[i] + acc[i];
+            }
+    }
+    wait_vm<0>();  // the repeated copies at the end must not outlive the kernel's LDS
+}
+
+// waves per workgroup and grid for `groups` row groups: every CU about the same number of groups, up to eight waves
+void rows_q4k_shape(int64_t groups, int num_cus, int &waves, int &grid) {
+    waves = (int)min((int64_t)8, (groups + num_cus - 1) / num_cus);
+    grid = (int)min((int64_t)num_cus, (groups + waves - 1) / waves);
+}
+bool rows_q4k_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus) {
+    if (type != T_Q4_K || ncols < 3 || ncols > 16 || K % QKK) return false;
+    const int64_t nsb = K / QKK, groups = (total_m + 15) / 16;
+    int waves, grid;
+    rows_q4k_shape(groups, num_cus, waves, grid);
+    const size_t lds = ncols <= 8 ? RowsGeoQ4K<8>::lds_bytes(nsb, waves) : RowsGeoQ4K<16>::lds_bytes(nsb, waves);
+    // from six row groups per CU: a wave runs a row group's whole K, and with fewer waves than that the general
+    // kernel's K cut keeps more of the memory system busy (gate 14336 x 4096 alone, 3.5 groups per CU: 12.2 us here
+    // against 11.3 at three columns; gate + up in one launch, 7 per CU: 19.6 against 22.1)
+    return lds <= 160 * 1024 && groups >= 6 * (int64_t)num_cus;
+}
+
+template <int NCT>
+void launch_rows_q4k_as(const RowsArgs &ra, const DevAct &a, int col0, int ncols, int num_cus, hipStream_t s) {
+    int waves, grid;
+    rows_q4k_shape(ra.groups_total, num_cus, waves, grid);
+    const size_t lds = RowsGeoQ4K<NCT>::lds_bytes(ra.K / QKK, waves);
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_rows_q4k_kernel<NCT>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  160 * 1024);
+        allowed[dev] = true;
+    }
+    skinny_rows_q4k_kernel<NCT><<<(unsigned)grid, 64 * waves, lds, s>>>(ra, a, col0, ncols, grid, waves);
+}
+void launch_rows_q4k(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols, int num_cus, hipStream_t s) {
+    RowsArgs ra;
+    int64_t rg = 0;
+    for (int t = 0; t < ROWS_MULTI; t++) {
+        const int j = t < count ? t : count - 1;
+        ra.p0[t] = ws[j].p0; ra.y[t] = ys[j]; ra.M[t] = ws[j].M;
+        ra.kcut[t] = skinny_waves((ws[j].M + 15) / 16, ws[j].K / QKK, num_cus);
+        if (t < count) rg += (ws[j].M + 15) / 16;
+        ra.grp_end[t] = t + 1 < count ? (int)rg : 0x7fffffff;
+    }
+    ra.K = ws[0].K;
+    ra.groups_total = (int)rg;
+    if (ncols <= 8) launch_rows_q4k_as<8>(ra, a, col0, ncols, num_cus, s);
+    else launch_rows_q4k_as<16>(ra, a, col0, ncols, num_cus, s);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Q4_K at up to four activation columns with the weights loaded straight into the MFMA operand
 // registers: the faster of the two skinny kernels while the matrix is small enough that latency, not
 // HBM time, decides (launch_skinny picks).  A 16-row group is cut kcut ways along K, one wave per cut;
@@ -1567,6 +1843,7 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
     const int64_t rg = (w.M + 15) / 16;
     if (w.type == T_Q4_K) {
         if (direct16_wanted(w.type, w.K, w.M, ncols)) launch_direct16(&w, &y, 1, a, col0, ncols, num_cus, s);
+        else if (rows_q4k_wanted(w.type, w.K, w.M, ncols, num_cus)) launch_rows_q4k(&w, &y, 1, a, col0, ncols, num_cus, s);
         else if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q4K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     } else {
@@ -1579,9 +1856,9 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
 
 // Several Q4_K matrices that share K against the same three or four activation columns: one launch of
 // the direct-load kernel over their numbered-through row groups when together they are small enough for it.
-// 1: one launch of the direct-load kernel; 2: one launch of the staged kernel; 0: no.  Either way every
-// matrix takes the kernel and the K cut it would take in a launch of its own, so the results are the same
-// bits as those of separate launches.
+// 1: one launch of the direct-load kernel; 2: one launch of the staged kernel; 3: one launch of the rows kernel;
+// 0: no.  Either way every matrix takes the kernel and the K cut it would take in a launch of its own, so the
+// results are the same bits as those of separate launches.
 int skinny_multi_kind(const DevWeight *ws, int count, int ncols, int num_cus) {
     if (count < 2 || count > DIRECT16_MULTI || ncols < 1 || ncols > 16) return 0;
     int64_t total_m = 0;
@@ -1597,6 +1874,8 @@ int skinny_multi_kind(const DevWeight *ws, int count, int ncols, int num_cus) {
     }
     if ((total_m + 15 * count) / 16 >= 0x7fffffff) return 0;
     if (each_direct && direct16_wanted(ws[0].type, ws[0].K, total_m, ncols)) return 1;
+    // the rows kernel (it reproduces the K cut each matrix would get alone, see skinny_rows_q4k_kernel)
+    if (count <= ROWS_MULTI && none_direct && rows_q4k_wanted(ws[0].type, ws[0].K, total_m, ncols, num_cus)) return 3;
     // staged: the common K cut must still leave at most about 16 waves per CU over the joint grid.  Q4_K only:
     // measured, q + k + v at 6 / 8 / 16 columns take 9.4 / 9.8 / 13.3 us in one launch against 17.0 / 17.6 / 21.2 in
     // three, gate + up at 4..8 columns 19.6..20.9 against 23.0..23.6; the Q6_K kernel (more registers and LDS per
@@ -1615,6 +1894,8 @@ hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count,
     if (ncols < 1 || ncols > a.N || (int64_t)ncols * a.K >= ((int64_t)1 << 32)) return hipErrorInvalidValue;
     if (kind == 1) {
         launch_direct16(ws, ys, count, a, 0, ncols, num_cus, s);
+    } else if (kind == 3) {
+        launch_rows_q4k(ws, ys, count, a, 0, ncols, num_cus, s);
     } else {
         const int waves = skinny_waves((ws[0].M + 15) / 16, ws[0].K / QKK, num_cus);
         if (ws[0].type == T_Q4_K) {

@@ -302,6 +302,33 @@ def test_multi_weight_launch_with_unequal_k_cuts_falls_back(ctx):
             W.free()
 
 
+@pytest.mark.parametrize("ms,k,ns", [([14336, 14336], 4096, (3, 8, 11, 16)), ([14336, 14336, 1000], 4096, (6,)),
+                                     ([24600], 4096, (5,)), ([24592], 8192, (3,)), ([9000, 16000], 2048, (7,))])
+def test_q4k_rows_kernel_alone_and_joint(ctx, ms, k, ns):
+    """Q4_K at 3..16 columns on matrices with many rows (together from six 16-row groups per CU): the kernel with the
+    activations resident in LDS, a wave per row group and whole K.  It restarts its accumulator where the general
+    kernel would cut K for that matrix alone, so a joint launch gives the bits of the single launches (which take the
+    general kernel below the row threshold: 14336, 1000, 9000 rows; K cut two, eight and three ways) -- and the
+    oracle's numbers.  Ragged last row groups, K of 2048 / 4096 / 8192, one and two column sets."""
+    rng = np.random.default_rng(8700 + sum(ms) + k)
+    raws = [_weights(Q4_K, m, k, seed=8701 + m + i) for i, m in enumerate(ms)]
+    Ws = [ctx.upload(Q4_K, r, k, m) for r, m in zip(raws, ms)]
+    for n in ns:
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        got = ctx.mulmat_multi(Ws, x) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x)]
+        for y, W, raw, m in zip(got, Ws, raws, ms):
+            assert npref.rel_err(y, oracle.mul_mat(Q4_K, raw, k, m, x, nthreads=16)) < TOL
+            _check_against_exact_arithmetic(Q4_K, raw, k, m, x, y, f"Q4_K {m}x{k} n={n}", max_rows=2048)
+            if len(Ws) > 1:
+                assert np.array_equal(ctx.mulmat(W, x), y), (m, n)
+        # a column's result does not depend on which other columns ride along
+        again = ctx.mulmat_multi(Ws, x[::-1].copy()) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x[::-1].copy())]
+        for y, z in zip(got, again):
+            assert np.array_equal(z[::-1], y)
+    for W in Ws:
+        W.free()
+
+
 @pytest.mark.parametrize("t", WTYPES)
 def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
     """For n <= 8 the f32 entry points quantize x inside the GEMV's prologue.  The result must be
