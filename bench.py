@@ -473,6 +473,22 @@ def main() -> int:
             fn()
             tm = timed(fn, 5) / (5 * len(pool))
             other[f"decode FFN block, {label}"] = {"us": round(tm * 1e6, 2)}
+        # the headline step at a few tokens (several sequences decoding together): gate + up in one call, down in a second
+        for n in (2, 4, 8):
+            xb = torch.randn(n, FFN_K, generator=g, dtype=torch.float32).to(dev)
+            hb = torch.randn(n, FFN_M, generator=g, dtype=torch.float32).to(dev)
+            ygb = torch.empty(n, FFN_M, dtype=torch.float32, device=dev)
+            yub = torch.empty(n, FFN_M, dtype=torch.float32, device=dev)
+            ydb = torch.empty(n, FFN_K, dtype=torch.float32, device=dev)
+
+            def step_n():
+                for ent in pool:
+                    ctx.mulmat_multi_device([ent["gate"], ent["up"]], xb.data_ptr(), n, [ygb.data_ptr(), yub.data_ptr()])
+                    ctx.mulmat_device(ent["down"], hb.data_ptr(), n, ydb.data_ptr())
+
+            step_n()
+            tm = timed(step_n, 5) / (5 * len(pool))
+            other[f"Q4_K decode FFN step (gate + up one call, down) B={n}"] = {"us": round(tm * 1e6, 2), "GB/s": round(3 * wbytes / tm / 1e9, 1)}
         out["other_configs"] = other
 
     if args.calibrate_copy:

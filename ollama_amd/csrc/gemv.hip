@@ -1092,7 +1092,7 @@ void launch_thin_mode(const Plan &p, const ThinArgs &ma, const DevAct &a, const 
     const int rpw = p.rows_per_wg >> p.rw_log2;
 #define THIN_LAUNCH(DIRECT, RPL) \
     gemv_thin_kernel<P, NC, DIRECT, XMODE, RPL, XP><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr)
-    if constexpr (XMODE == 1 && NC == 1 && XP > 1 && P::ACT_BLK == QKK) {
+    if constexpr (XMODE == 1 && NC == 1 && XP > 1) {
         if (p.kw > 1) {  // the down projection's shape: measured +1.4 % on the whole decode step
             gemv_thin_kernel<P, 1, false, 1, 1, XP, true><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr);
             return;
