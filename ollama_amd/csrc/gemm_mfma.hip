@@ -1320,8 +1320,9 @@ __global__ __launch_bounds__(512, 2) void skinny_rows_q4k_kernel(RowsArgs ra, De
     const int nsb = (int)(ra.K / QKK);
     const unsigned res_a = lds_addr(smem), wv_a = res_a + (unsigned)nsb * Geo::RB + (unsigned)wave * (Geo::NST * Geo::W_STAGE);
 
-    // ---- the wave's row groups: ((k * grid + workgroup) * waves + wave), k = 0, 1, ...
-    auto item_group = [&](int64_t k) { return (k * grid_size + (int64_t)blockIdx.x) * waves + wave; };
+    // ---- the wave's row groups: ((k * waves + wave) * grid + workgroup), k = 0, 1, ...: consecutive row groups go to
+    // consecutive workgroups, so a count that is no multiple of the grid still loads every CU alike
+    auto item_group = [&](int64_t k) { return (k * waves + wave) * grid_size + (int64_t)blockIdx.x; };
     int64_t items = 0;
     if (item_group(0) < ra.groups_total) items = (ra.groups_total - 1 - item_group(0)) / ((int64_t)grid_size * waves) + 1;
 
@@ -1486,8 +1487,8 @@ __global__ __launch_bounds__(512, 2) void skinny_rows_q4k_kernel(RowsArgs ra, De
 
 // waves per workgroup and grid for `groups` row groups: every CU about the same number of groups, up to eight waves
 void rows_q4k_shape(int64_t groups, int num_cus, int &waves, int &grid) {
-    waves = (int)min((int64_t)8, (groups + num_cus - 1) / num_cus);
-    grid = (int)min((int64_t)num_cus, (groups + waves - 1) / waves);
+    grid = (int)min((int64_t)num_cus, groups);
+    waves = (int)min((int64_t)8, (groups + grid - 1) / grid);
 }
 bool rows_q4k_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus) {
     if (type != T_Q4_K || ncols < 3 || ncols > 16 || K % QKK) return false;
