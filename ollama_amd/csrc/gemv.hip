@@ -541,12 +541,12 @@ constexpr int rows_per_load(int64_t K) { return K * 4 <= P::SEG ? 4 : K * 2 <= P
 // The row loop of the thin kernels: rows wrow0 .. wrow0+nrw-1 of w against the activation registers,
 // one load of RPL rows in registers and the next in flight.  cur holds the first load (issued by the
 // caller ahead of its prologue: rows wrow0 + min(run, nrw-1)).  DIRECT: on return lane 63-i of keep[n]
-// holds the total of the wave's row i; otherwise the totals go to part[(rl0+i)*NC + n][kseg].
+// holds the total of the wave's row i; otherwise the totals go to part[(rl0+i)*NC + n][kseg] (rows side by side there:
+// the waves of a mostly empty last K segment).
 template <class P, int NC, bool DIRECT, int RPL>
 __device__ __forceinline__ void thin_rows(const DevWeight &w, const typename P::Geo &g, typename P::Raw cur,
                                           const typename P::Act (&act)[NC], int64_t wrow0, int nrw, int lane,
                                           float (&keep)[NC], float *part, int rl0, int kw, int kseg) {
-    static_assert(RPL == 1 || DIRECT, "rows side by side only when a row lies inside one K segment");
     const int run = RPL == 1 ? 0 : lane / (64 / RPL);
 #pragma unroll
     for (int n = 0; n < NC; n++) keep[n] = 0.f;
@@ -567,7 +567,7 @@ __device__ __forceinline__ void thin_rows(const DevWeight &w, const typename P::
             for (int r = 0; r < RPL; r++) {
                 const float tot = __int_as_float(__builtin_amdgcn_readlane(tot_all, 64 / RPL * (r + 1) - 1));
                 if (DIRECT) keep[n] = lane == 63 - (i + r) ? tot : keep[n];
-                else if (lane == 63) part[((rl0 + i) * NC + n) * kw + kseg] = tot;
+                else if (lane == 63 && i + r < nrw) part[((rl0 + i + r) * NC + n) * kw + kseg] = tot;
             }
         }
     }
@@ -725,7 +725,10 @@ constexpr int thin_max_waves(int nc, bool f32) { return f32 ? (nc <= 3 ? 16 : 8)
 // AHEAD (one f32 column, long rows, one workgroup per CU anyway): a wave requests its second row as soon as it has
 // quantized its share of x -- not before, where the request would queue in front of other waves' x -- so that two
 // rows per wave stream while the workgroup waits at the barrier and reads its activations back.
-template <class P, int NC, bool DIRECT, int XMODE, int RPL, int XP = XPRE, bool AHEAD = false>
+// TAILR (2 or 4; rows cut into segments, one or two columns): the waves of the last K segment, which is at most half
+// (a quarter) full, take TAILR rows side by side per load -- as RPL does for short rows -- instead of running with
+// most of their lanes dead.  Same bits: a dead lane adds an exact zero to its row's sum.
+template <class P, int NC, bool DIRECT, int XMODE, int RPL, int XP = XPRE, bool AHEAD = false, int TAILR = 1>
 __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kernel(ThinArgs ta, DevAct a, const float *__restrict__ xf,
                                                          int col0, int rows_per_wave, int kw, int rw_log2, Produce pr) {
     constexpr bool F32 = XMODE != 0;
@@ -794,7 +797,11 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     const int nrw = max(0, min(rows_per_wave, nrows - rl0));
     float *yrow0 = y + (int64_t)col0 * ldy + r0;
 
-    const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);  // position inside the lane's run
+    // rows side by side in this wave: RPL for short rows, TAILR in the waves of a mostly empty last segment
+    static_assert(TAILR == 1 || (!DIRECT && RPL == 1 && NC <= 2 && XMODE <= 1), "side-by-side tail rows: plain products of rows cut into segments");
+    const bool tail = TAILR > 1 && kseg == kw - 1;  // wave-uniform
+    const int vlane = tail ? lane & (64 / TAILR - 1) : lane & (64 / RPL - 1);  // position inside the lane's run
+    const int run = tail ? lane / (64 / TAILR) : RPL == 1 ? 0 : lane / (64 / RPL);
     const typename P::Geo g = P::geo(w, kseg, vlane);
 
     // With f32 activations the workgroup quantizes them itself, into LDS, in the layout of DevAct
@@ -859,7 +866,7 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     if (F32) {
         if (ROW16) quantize_x_to_lds16<P>(x4, NC * nblk, wave, nwaves, lane, xq, lqs, ld_, lbs);
         else quantize_x_to_lds<P, XP>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
-        if (AHEAD && nrw > 0) nxt = P::load(w, g, r0 + rl0 + min(1, nrw - 1));
+        if (AHEAD && nrw > 0 && !tail) nxt = P::load(w, g, r0 + rl0 + min(1, nrw - 1));
         __syncthreads();
     }
     float *part = reinterpret_cast<float *>(smem + act_bytes + PSUM_BYTES);
@@ -875,7 +882,8 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
             for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg, vlane, g, act[n]);
         }
         float keep[NC];  // lane 63-i ends up holding the total of the wave's row i
-        if constexpr (AHEAD) thin_rows_ahead<P, DIRECT>(w, g, cur, nxt, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
+        if (tail) thin_rows<P, NC, DIRECT, TAILR>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
+        else if constexpr (AHEAD) thin_rows_ahead<P, DIRECT>(w, g, cur, nxt, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
         else thin_rows<P, NC, DIRECT, RPL>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
         if (DIRECT && lane > 63 - nrw) {
 #pragma unroll
@@ -1009,7 +1017,7 @@ __global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const floa
     }
 }
 
-struct Plan { int kw, rw, rw_log2, spw, rows_per_wg, rpl; unsigned grid; size_t lds; };
+struct Plan { int kw, rw, rw_log2, spw, rows_per_wg, rpl, tail_log2 = 0; unsigned grid; size_t lds; };
 
 // 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), one or two workgroups per CU.
 // total_m is the number of rows over all tensors of the launch.
@@ -1081,6 +1089,15 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
             rows_per_wave = (nc >= 4 || total_m > 65536) ? 4 : 2;
         }
     }
+    // Rows of several segments whose last segment is at most half (a quarter) full -- K = 14336 = 3.5 segments of
+    // 4096, K = 5120 = 1.25: the waves of that segment take 2 (4) rows side by side per load, as the waves of short
+    // rows do, instead of running with half (three quarters) of their lanes dead.  One and two columns.
+    p.tail_log2 = 0;
+    if (p.kw > 1 && nc <= 2 && !produce) {
+        const int tail = rows_per_load<P>(K - (int64_t)(p.kw - 1) * P::SEG);
+        p.tail_log2 = tail == 4 ? 2 : tail == 2 ? 1 : 0;
+        rows_per_wave = (rows_per_wave + tail - 1) / tail * tail;
+    }
     // short rows: 2 or 4 side by side per load, and at least two loads per wave (one in flight)
     p.rpl = p.kw == 1 ? rows_per_load<P>(K) : 1;
     if (p.rpl > 1) rows_per_wave = max(2 * p.rpl, (rows_per_wave + p.rpl - 1) / p.rpl * p.rpl);
@@ -1101,9 +1118,15 @@ void launch_thin_mode(const Plan &p, const ThinArgs &ma, const DevAct &a, const 
     const int rpw = p.rows_per_wg >> p.rw_log2;
 #define THIN_LAUNCH(DIRECT, RPL) \
     gemv_thin_kernel<P, NC, DIRECT, XMODE, RPL, XP><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr)
-    if constexpr (XMODE == 1 && NC == 1 && XP > 1) {
-        if (p.kw > 1) {  // the down projection's shape: measured +1.4 % on the whole decode step
-            gemv_thin_kernel<P, 1, false, 1, 1, XP, true><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr);
+#define THIN_LAUNCH_SEGMENTS(AHEAD, TAILR) \
+    gemv_thin_kernel<P, NC, false, XMODE, 1, XP, AHEAD, TAILR><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr)
+    if constexpr (XMODE <= 1 && NC <= 2) {
+        if (p.kw > 1) {
+            // one plain f32 column (the down projection's shape): the second row ahead, +1.4 % on the whole decode step
+            constexpr bool AH = XMODE == 1 && NC == 1 && XP > 1;
+            if (p.tail_log2 == 2) THIN_LAUNCH_SEGMENTS(AH, 4);
+            else if (p.tail_log2 == 1) THIN_LAUNCH_SEGMENTS(AH, 2);
+            else THIN_LAUNCH_SEGMENTS(AH, 1);
             return;
         }
     }
@@ -1112,6 +1135,7 @@ void launch_thin_mode(const Plan &p, const ThinArgs &ma, const DevAct &a, const 
     else if (p.rpl == 2) THIN_LAUNCH(true, 2);
     else THIN_LAUNCH(true, 1);
 #undef THIN_LAUNCH
+#undef THIN_LAUNCH_SEGMENTS
 }
 
 template <class P, int NC>

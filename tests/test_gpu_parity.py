@@ -336,7 +336,7 @@ def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
     above) and multiplying by the two-phase entry point -- i.e. the in-kernel quants are the same bits."""
     rng = np.random.default_rng(400 + t)
     blk = npref.BLOCK[t]
-    ks = [blk, 4096, 14336] + ([2336, 96] if blk == 32 else [2304])   # 2336*n is not a multiple of 256
+    ks = [blk, 4096, 14336] + ([2336, 96] if blk == 32 else [2304, 5120])   # 2336*n is not a multiple of 256
     for k in ks:
         ms = [37, 130]
         raws = [_weights(t, m, k, seed=k + m) for m in ms]
@@ -392,7 +392,8 @@ def test_in_kernel_q8_K_quantizer_edge_blocks_give_the_same_bits(ctx, t):
     W.free()
 
 
-@pytest.mark.parametrize("t,k", [(Q4_K, 14336), (Q4_K, 8192), (Q6_K, 4352), (Q4_0, 4096), (Q8_0, 4096), (Q8_0, 2080)])
+@pytest.mark.parametrize("t,k", [(Q4_K, 14336), (Q4_K, 8192), (Q6_K, 4352), (Q4_0, 4096), (Q8_0, 4096), (Q8_0, 2080),
+                                 (Q4_K, 5120), (Q6_K, 5120), (Q6_K, 14336), (Q4_0, 2560), (Q8_0, 5120)])
 def test_long_rows_at_one_column(ctx, t, k):
     """One column, rows of several K segments (the waves of a workgroup cut K and combine through LDS): same
     bits as the two-phase path, call after call; row counts that do not fill the last workgroup, four
@@ -402,6 +403,7 @@ def test_long_rows_at_one_column(ctx, t, k):
     raws = [_weights(t, m, k, seed=k + m + t) for m in ms]
     Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
     act = ctx.act_create(qmm.vec_dot_type(t), k, 1)
+    act3 = ctx.act_create(qmm.vec_dot_type(t), k, 3)
     for rep in range(3):
         x = rng.standard_normal((1, k), dtype=np.float32)
         ctx.act_quantize(act, x)
@@ -412,7 +414,17 @@ def test_long_rows_at_one_column(ctx, t, k):
             for y, wnt in zip(ctx.mulmat_multi(Ws[1:], x), want[1:]):
                 assert np.array_equal(y, wnt)
         assert npref.rel_err(want[4], oracle.mul_mat(t, raws[4], k, 700, x, nthreads=8)) <= TOL
+        # the waves of a mostly empty last segment take rows side by side at one and two columns only: at three
+        # columns every wave takes one row per load, and column 0 must come out with the same bits (not Q4_K: its
+        # three-column products do not reproduce the one-column bits at any K, with or without a short last segment,
+        # so they say nothing here)
+        if t != Q4_K:
+            x3 = np.concatenate([x, rng.standard_normal((2, k), dtype=np.float32)])
+            ctx.act_quantize(act3, x3)
+            for W, wnt in zip(Ws, want):
+                assert np.array_equal(ctx.mulmat_q8(W, act3, path=qmm.PATH_GEMV)[:1], wnt)
     act.free()
+    act3.free()
     for W in Ws:
         W.free()
     if t == Q4_K and k == 8192:
