@@ -225,7 +225,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_thin_kernel<PolQ4K, 1, true, 1, 1, 1, false> (gate+up in one launch, 28672 rows x 4096)",
+            "kernel": "gemv_thin_kernel<PolQ4K, 1, true, 1, 1, 1, false, 1> (gate+up in one launch, 28672 rows x 4096)",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
