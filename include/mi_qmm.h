@@ -151,10 +151,11 @@ int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *
 /* several weights of the same k against the same f32 activations x [n][k]: ys[i] receives
  * f32 [n][m_i].  These are the mul_mat nodes of one graph that share src1 (gate and up, or q/k/v),
  * which Context.Compute (/root/reference/ml/backend.go:110) sees together.  For weights of one
- * type, one column (a few on small matrices) and count <= 4 this is ONE kernel launch: the decode
- * GEMV quantizes x in its prologue and walks the concatenated rows of all weights.  Otherwise x is
- * quantized once per activation format in use and the products follow, weights of one type sharing
- * GEMV launches four at a time while n <= 8.  Results are those of mi_qmm_mulmat per weight. */
+ * type, one or two columns (three for some formats and sizes) and count <= 4 this is ONE kernel
+ * launch: the decode GEMV quantizes x in its prologue and walks the concatenated rows of all weights.
+ * Otherwise x is quantized once per activation format in use and the products follow, weights of one
+ * type sharing launches four at a time while n <= 16 where a kernel takes them together (the GEMV; the
+ * matrix-core kernels for Q4_K).  Results are those of mi_qmm_mulmat per weight. */
 int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x,
                         int64_t n, float *const *ys, int location);
 
