@@ -117,6 +117,16 @@ void mi_qmm_weight_free(mi_qmm_weight *w);
 int mi_qmm_weight_info(const mi_qmm_weight *w, int *ggml_type, int64_t *k, int64_t *m,
                        int64_t *device_bytes);
 
+/* ---- weight encoders on the GPU: f32 rows -> GGUF blocks of Q4_0, Q8_0, Q4_K or Q6_K.  Replaces what the
+ *      reference obtains by running llama-quantize (/root/reference/server/quantization.go:125-181,
+ *      /root/reference/server/create.go:931-944): for these four types and no importance matrix that tool
+ *      encodes every row with ggml's scalar quantize_row_*_ref; the kernels keep those loops' orders, so the
+ *      bytes are the scalar code's.  (Which tensor gets which type -- the Q4_K_M mixture -- stays with the
+ *      caller.)  x: f32 [m][k]; out_blocks receives m * row_size(ggml_type, k) bytes, ready for
+ *      mi_qmm_weight_upload or a GGUF file.  location applies to both x and out_blocks. */
+int mi_qmm_quantize_weights(mi_qmm_ctx *ctx, int ggml_type, const float *x, int64_t k, int64_t m,
+                            void *out_blocks, int location);
+
 /* ---- activation quantization on the GPU: replaces ggml's from_float step of mul_mat
  *      (quantize_row_q8_0 / quantize_row_q8_K, canonical scalar semantics).
  *      x: f32 [n][k]; out_blocks receives n * row_size(q8_type, k) bytes in GGUF block layout,

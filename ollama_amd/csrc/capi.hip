@@ -441,6 +441,41 @@ int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k,
     return MI_QMM_OK;
 }
 
+int mi_qmm_quantize_weights(mi_qmm_ctx *ctx, int ggml_type, const float *x, int64_t k, int64_t m, void *out_blocks,
+                            int location) {
+    if (ggml_type != T_Q4_0 && ggml_type != T_Q8_0 && ggml_type != T_Q4_K && ggml_type != T_Q6_K)
+        return fail(MI_QMM_ERR_UNSUPPORTED, "weight type %d is not Q4_0 (2), Q8_0 (8), Q4_K (12) or Q6_K (14)", ggml_type);
+    if (k < 0 || m < 0) return fail(MI_QMM_ERR_INVALID, "k=%lld m=%lld must be non-negative", (long long)k, (long long)m);
+    const int64_t row = mi_qmm_row_size(ggml_type, k);
+    if (row < 0)
+        return fail(MI_QMM_ERR_INVALID, "k=%lld is not a multiple of the block size %lld of type %d",
+                    (long long)k, (long long)mi_qmm_block_size(ggml_type), ggml_type);
+    if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
+        return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
+    int rc = check_ctx(ctx);
+    if (rc) return rc;
+    if (k * m == 0) return MI_QMM_OK;
+    if (!x || !out_blocks) return fail(MI_QMM_ERR_INVALID, "x or out_blocks is NULL");
+    if (location == MI_QMM_DEVICE) {
+        HIP_TRY(launch_encode_weights(ggml_type, x, k, m, (uint8_t *)out_blocks, ctx->stream));
+        return MI_QMM_OK;
+    }
+    // host buffers: slabs of rows through the ctx's staging buffer (at most 64 MiB of f32 at a time)
+    const int64_t slab_rows = std::max<int64_t>(1, std::min<int64_t>(m, ((int64_t)64 << 20) / (k * 4)));
+    const size_t xoff = align_up((size_t)(slab_rows * row), 256);
+    if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, xoff + (size_t)(slab_rows * k) * 4))) return rc;
+    uint8_t *dout = (uint8_t *)ctx->io_buf;
+    float *dx = (float *)((char *)ctx->io_buf + xoff);
+    for (int64_t r0 = 0; r0 < m; r0 += slab_rows) {
+        const int64_t rows = std::min(slab_rows, m - r0);
+        HIP_TRY(hipMemcpyAsync(dx, x + r0 * k, (size_t)(rows * k) * 4, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(launch_encode_weights(ggml_type, dx, k, rows, dout, ctx->stream));
+        HIP_TRY(hipMemcpyAsync((char *)out_blocks + r0 * row, dout, (size_t)(rows * row), hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));  // the slab buffers are reused
+    }
+    return MI_QMM_OK;
+}
+
 }  // extern "C"
 
 // ---- the product ------------------------------------------------------------------------------------

@@ -9,6 +9,11 @@
 
 namespace miqmm {
 
+// Weight encoders (encode.hip): f32 rows [M][K] -> GGUF blocks [M][row_size], the bytes of ggml's scalar
+// quantize_row_{q4_0,q8_0,q4_K,q6_K}_ref.  x and out are device pointers.
+bool encode_supported(int type, int64_t K);
+hipError_t launch_encode_weights(int type, const float *x, int64_t K, int64_t M, uint8_t *out, hipStream_t s);
+
 // kernel 1: f32 rows -> Q8_0 / Q8_K planes (bit-exact with the scalar CPU quantizers)
 // sd8 / sd16: block-sum digit planes for the GEMM (Q8_K only; may be null)
 // produce (optional): applied to x on the fly (RMSNORM needs row_scale from launch_rms_norm first)

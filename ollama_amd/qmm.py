@@ -28,7 +28,7 @@ EXPORTS = [
     "mi_qmm_block_size", "mi_qmm_type_size", "mi_qmm_row_size", "mi_qmm_vec_dot_type",
     "mi_qmm_init", "mi_qmm_destroy", "mi_qmm_set_stream", "mi_qmm_sync", "mi_qmm_host_alloc", "mi_qmm_host_free",
     "mi_qmm_weight_upload", "mi_qmm_weight_free", "mi_qmm_weight_info",
-    "mi_qmm_quantize_act", "mi_qmm_mulmat", "mi_qmm_mulmat_path", "mi_qmm_mulmat_noalloc", "mi_qmm_scratch_freeze",
+    "mi_qmm_quantize_act", "mi_qmm_quantize_weights", "mi_qmm_mulmat", "mi_qmm_mulmat_path", "mi_qmm_mulmat_noalloc", "mi_qmm_scratch_freeze",
     "mi_qmm_mulmat_multi", "mi_qmm_mulmat_id", "mi_qmm_mulmat_id_multi",
     "mi_qmm_mulmat_produced", "mi_qmm_mulmat_id_produced", "mi_qmm_mulmat_swiglu", "mi_qmm_mulmat_id_swiglu", "mi_qmm_rms_norm", "mi_qmm_swiglu",
     "mi_qmm_act_create", "mi_qmm_act_free", "mi_qmm_act_quantize", "mi_qmm_mulmat_q8", "mi_qmm_mulmat_q8_multi",
@@ -80,6 +80,7 @@ def lib() -> ctypes.CDLL:
     L.mi_qmm_weight_info.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(i64), ctypes.POINTER(i64),
                                      ctypes.POINTER(i64)]
     L.mi_qmm_quantize_act.restype = ci; L.mi_qmm_quantize_act.argtypes = [vp, ci, vp, i64, i64, vp, ci]
+    L.mi_qmm_quantize_weights.restype = ci; L.mi_qmm_quantize_weights.argtypes = [vp, ci, vp, i64, i64, vp, ci]
     L.mi_qmm_mulmat.restype = ci; L.mi_qmm_mulmat.argtypes = [vp, vp, vp, i64, vp, ci]
     L.mi_qmm_mulmat_path.restype = ci; L.mi_qmm_mulmat_path.argtypes = [vp, vp, vp, i64, vp, ci, ci]
     L.mi_qmm_mulmat_noalloc.restype = ci; L.mi_qmm_mulmat_noalloc.argtypes = [vp, vp, vp, i64, vp]
@@ -271,6 +272,20 @@ class Context:
         h = ctypes.c_void_p()
         _check(lib().mi_qmm_weight_upload(self._h, ggml_type, _ptr(gguf_bytes), k, m, location, ctypes.byref(h)))
         return Weight(h, ggml_type, k, m)
+
+    def quantize_weights(self, t: int, x: np.ndarray) -> np.ndarray:
+        """f32 [m, k] -> uint8 [m, row_size(t, k)]: GGUF blocks of a weight type, encoded on the GPU"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        m, k = x.shape
+        rb = row_size(t, k)
+        out = np.empty((m, max(rb, 0)), dtype=np.uint8)
+        _check(lib().mi_qmm_quantize_weights(self._h, t, _ptr(x), k, m, _ptr(out), HOST))
+        return out
+
+    def quantize_weights_device(self, t: int, x_ptr: int, k: int, m: int, out_ptr: int):
+        _check(lib().mi_qmm_quantize_weights(self._h, t, ctypes.c_void_p(x_ptr), k, m, ctypes.c_void_p(out_ptr), DEVICE))
 
     def quantize_act(self, q8_type: int, x: np.ndarray) -> np.ndarray:
         """x f32 [n, k] -> uint8 [n, row_size] GGUF-layout Q8_0 / Q8_K blocks computed on the GPU."""

@@ -56,6 +56,9 @@ def test_argument_errors_without_a_device():
     assert L.mi_qmm_weight_upload(None, qmm.Q4_K, None, 256, 0, 0, ctypes.byref(h)) == qmm.ERR_INVALID
     assert L.mi_qmm_quantize_act(None, 9, None, 32, 1, None, 0) == qmm.ERR_UNSUPPORTED
     assert L.mi_qmm_quantize_act(None, qmm.Q8_K, None, 100, 1, None, 0) == qmm.ERR_INVALID
+    assert L.mi_qmm_quantize_weights(None, qmm.Q8_K, None, 256, 1, None, 0) == qmm.ERR_UNSUPPORTED
+    assert L.mi_qmm_quantize_weights(None, qmm.Q6_K, None, 300, 1, None, 0) == qmm.ERR_INVALID
+    assert L.mi_qmm_quantize_weights(None, qmm.Q4_0, None, 32, 1, None, 7) == qmm.ERR_INVALID
     L.mi_qmm_destroy(None)
     L.mi_qmm_weight_free(None)
 
