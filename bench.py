@@ -489,6 +489,14 @@ def main() -> int:
             step_n()
             tm = timed(step_n, 5) / (5 * len(pool))
             other[f"Q4_K decode FFN step (gate + up one call, down) B={n}"] = {"us": round(tm * 1e6, 2), "GB/s": round(3 * wbytes / tm / 1e9, 1)}
+        # weight encoders (a one-off step when a quantized model is made): f32 rows on the device -> GGUF blocks
+        xe = (torch.randn(FFN_M, FFN_K, generator=g, dtype=torch.float32) * 0.02).to(dev)
+        for label, t in (("Q4_0", Q4_0), ("Q8_0", Q8_0), ("Q4_K", Q4_K), ("Q6_K", Q6_K)):
+            oe = torch.empty(FFN_M * qmm.row_size(t, FFN_K), dtype=torch.uint8, device=dev)
+            fn = lambda: ctx.quantize_weights_device(t, xe.data_ptr(), FFN_K, FFN_M, oe.data_ptr())
+            fn()
+            tm = timed(fn, 3) / 3
+            other[f"weight encoder {label} 14336x4096 f32 -> blocks"] = {"us": round(tm * 1e6, 1), "Gweights/s": round(FFN_M * FFN_K / tm / 1e9, 1)}
         out["other_configs"] = other
 
     if args.calibrate_copy:

@@ -777,7 +777,7 @@ __global__ __launch_bounds__(512, (NCT / S::SET_COLS >= 4 ? 2 : 4)) void skinny_
     static_assert(!(ID && MULTI), "expert-indexed launches take one stack");
     typedef typename S::G G;
     typedef SkinnyGeo<S, NCT, NST> Geo;
-    constexpr int A_BYTES = Geo::A_BYTES, A_INSTRS = Geo::A_INSTRS, D_BYTES = Geo::D_BYTES;
+    constexpr int A_INSTRS = Geo::A_INSTRS;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, WAVE_BYTES = Geo::WAVE_BYTES;
     // The whole argument block in one batch of scalar loads: every value is named here and pinned by an
     // empty asm (left alone the compiler fetches them where each branch first needs them, four or five

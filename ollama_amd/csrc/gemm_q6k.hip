@@ -43,7 +43,7 @@ __device__ __forceinline__ s2 as_s2(unsigned v) { return __builtin_bit_cast(s2, 
 __device__ __forceinline__ unsigned as_u(s2 v) { return __builtin_bit_cast(unsigned, v); }
 __device__ __forceinline__ float h2f(unsigned bits16) { return __half2float(__ushort_as_half((unsigned short)bits16)); }
 
-constexpr int TM = 256, TN = 128, WAVES = 8;
+constexpr int TM = 256, TN = 128;  // eight waves per workgroup, 32 weight rows each
 constexpr int A_BUF = TN * 256;                 // one super-block of activation quants
 constexpr int W_QL = TM * 64, W_QH = TM * 32, W_STAGE = W_QL + W_QH;  // one half super-block of packed weights
 constexpr int OFF_A = 0, OFF_W = OFF_A + 2 * A_BUF, OFF_SC = OFF_W + 3 * W_STAGE, OFF_D = OFF_SC + 2 * TM * 16,
