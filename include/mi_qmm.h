@@ -123,7 +123,8 @@ int mi_qmm_weight_info(const mi_qmm_weight *w, int *ggml_type, int64_t *k, int64
  *      encodes every row with ggml's scalar quantize_row_*_ref; the kernels keep those loops' orders, so the
  *      bytes are the scalar code's.  (Which tensor gets which type -- the Q4_K_M mixture -- stays with the
  *      caller.)  x: f32 [m][k]; out_blocks receives m * row_size(ggml_type, k) bytes, ready for
- *      mi_qmm_weight_upload or a GGUF file.  location applies to both x and out_blocks. */
+ *      mi_qmm_weight_upload or a GGUF file.  location applies to both x and out_blocks; device pointers: x
+ *      16-byte aligned, out_blocks 4-byte aligned (queued on the ctx stream, returns without waiting). */
 int mi_qmm_quantize_weights(mi_qmm_ctx *ctx, int ggml_type, const float *x, int64_t k, int64_t m,
                             void *out_blocks, int location);
 

@@ -457,6 +457,9 @@ int mi_qmm_quantize_weights(mi_qmm_ctx *ctx, int ggml_type, const float *x, int6
     if (k * m == 0) return MI_QMM_OK;
     if (!x || !out_blocks) return fail(MI_QMM_ERR_INVALID, "x or out_blocks is NULL");
     if (location == MI_QMM_DEVICE) {
+        // (the kernels read x in 16-byte pieces and write Q4_K blocks in 4-byte words)
+        if (((uintptr_t)x & 15) || ((uintptr_t)out_blocks & 3))
+            return fail(MI_QMM_ERR_INVALID, "device x must be 16-byte aligned and out_blocks 4-byte aligned");
         HIP_TRY(launch_encode_weights(ggml_type, x, k, m, (uint8_t *)out_blocks, ctx->stream));
         return MI_QMM_OK;
     }

@@ -111,3 +111,10 @@ def test_empty_and_argument_errors(ctx):
         ctx.quantize_weights(Q4_K, np.zeros((2, 100), np.float32))
     with pytest.raises(qmm.QmmError):
         ctx.quantize_weights(npref.Q8_K, np.zeros((2, 256), np.float32))
+    dx = DeviceArray(np.zeros((2, 260), np.float32))
+    dout = DeviceArray(np.zeros(2 * 144 + 8, np.uint8))
+    with pytest.raises(qmm.QmmError, match="aligned"):
+        ctx.quantize_weights_device(Q4_K, dx.ptr + 4, 256, 2, dout.ptr)
+    with pytest.raises(qmm.QmmError, match="aligned"):
+        ctx.quantize_weights_device(Q4_K, dx.ptr, 256, 2, dout.ptr + 2)
+    dx.free(); dout.free()
