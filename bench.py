@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GGUF quantized-matmul hot path on one MI355X.
 
-Headline (BASELINE.json metric): Q4_K decode GEMV at Llama-3-8B FFN shapes, batch 1 -- gate/up
+Headline metric: Q4_K decode GEMV at Llama-3-8B FFN shapes, batch 1 -- gate/up
 14336x4096 and down 4096x14336 -- in GB/s of algorithmic bytes (GGUF weight bytes + f32 activations
 read + f32 outputs written) with everything resident in HBM.
 
@@ -80,7 +80,7 @@ def main() -> int:
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the batch-512 prefill GEMM section")
     ap.add_argument("--no-other", action="store_true",
-                    help="skip the short timings of the other BASELINE configurations (Q4_0 / Q8_0 GEMV, Q6_K head) "
+                    help="skip the short timings of the other benchmark configurations (Q4_0 / Q8_0 GEMV, Q6_K head) "
                          "and of the expert-indexed and Q4_0 GEMM paths")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic, for scaling rocprofv3 HBM counters)")
@@ -271,7 +271,7 @@ def main() -> int:
         out["roofline"]["frac_of_read_ceiling"] = round(achieved / ceil_gbs, 4)
         del bufs
 
-    # ---- prefill GEMM: one Llama-3-8B-shaped layer at batch 512 (secondary metric of BASELINE.json)
+    # ---- prefill GEMM: one Llama-3-8B-shaped layer at batch 512 (the secondary metric)
     if not args.no_gemm:
         NB = 512
         layer = [("attn_q", Q4_K, 4096, 4096), ("attn_k", Q4_K, 1024, 4096), ("attn_v", Q4_K, 1024, 4096),
