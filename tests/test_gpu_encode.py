@@ -105,6 +105,16 @@ def test_device_pointers_and_the_product_on_encoded_weights(ctx, t):
     assert rel < {Q4_0: 0.12, Q8_0: 0.01, Q4_K: 0.09, Q6_K: 0.02}[t], rel
 
 
+def test_host_rows_beyond_one_staging_slab(ctx):
+    """host arrays larger than the 64 MiB staging slab go through in several pieces: the same bytes as row by row"""
+    rng = np.random.default_rng(9400)
+    m, k = 5000, 4096  # 82 MB of f32: two slabs, the second one short
+    x = rng.standard_normal((m, k), dtype=np.float32) * np.float32(0.03)
+    for t in (Q8_0, Q4_K):
+        got = ctx.quantize_weights(t, x)
+        assert np.array_equal(got, oracle.quantize(t, x, nthreads=16))
+
+
 def test_empty_and_argument_errors(ctx):
     assert ctx.quantize_weights(Q4_K, np.zeros((0, 256), np.float32)).shape == (0, 144)
     with pytest.raises(qmm.QmmError):
