@@ -508,6 +508,45 @@ def test_randomized_shape_sweep(ctx):
         W.free()
 
 
+def test_randomized_shapes_through_the_large_matrix_kernels(ctx):
+    """seeded random shapes where the kernels for large matrices take over: Q4_K on many rows at 3..16 columns, alone
+    and several matrices in one call; Q6_K on 65536 rows and more at 2..8 columns; rows whose last K segment is at
+    most half full at one and two columns (every format); two and three columns on large matrices -- against the
+    oracle (weights tiled from 2048 encoded rows)"""
+    rng = np.random.default_rng(20250131)
+
+    def tiled(t, m, k, seed):
+        base = min(m, 2048)
+        return np.tile(_weights(t, base, k, seed).reshape(base, -1), ((m + base - 1) // base, 1))[:m].reshape(-1).copy()
+
+    def check(t, ms, k, n, what):
+        raws = [tiled(t, m, k, 7000 + i + m) for i, m in enumerate(ms)]
+        Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        got = ctx.mulmat_multi(Ws, x) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x)]
+        for y, r, m in zip(got, raws, ms):
+            err = npref.rel_err(y, oracle.mul_mat(t, r, k, m, x, nthreads=16))
+            assert err <= TOL, f"{what}: {NAMES[t]} ms={ms} k={k} n={n}: rel err {err}"
+        for W in Ws:
+            W.free()
+
+    for _ in range(3):
+        ms = [int(rng.integers(9000, 30000)) for _ in range(int(rng.integers(1, 4)))]
+        if sum((m + 15) // 16 for m in ms) < 1536:
+            ms[0] += 26000
+        check(Q4_K, ms, int(rng.choice([2048, 4096, 8192])), int(rng.integers(3, 17)), "many rows, Q4_K")
+    for _ in range(2):
+        check(Q6_K, [int(rng.integers(65536, 90000))], int(rng.choice([2048, 4096])), int(rng.integers(2, 9)), "many rows, Q6_K")
+    for _ in range(8):
+        t = int(rng.choice(WTYPES))
+        blk, seg = (256, 4096) if t in (Q4_K, Q6_K) else (32, 2048)
+        k = int(rng.integers(1, 5)) * seg + int(rng.integers(1, seg // blk // 2 + 1)) * blk
+        check(t, [int(rng.integers(1, 6000))], k, int(rng.integers(1, 3)), "short last segment")
+    for _ in range(4):
+        t = int(rng.choice(WTYPES))
+        check(t, [int(rng.integers(3000, 16000))], int(rng.choice([4096, 8192, 14336])), int(rng.integers(2, 4)), "two or three columns")
+
+
 def test_randomized_mulmat_id_sweep(ctx):
     """random types, expert counts, token counts, slots and activation rows per token across the decode, bucketed,
     matrix-core and expert-GEMM paths, against the oracle"""
