@@ -547,6 +547,53 @@ def test_randomized_shapes_through_the_large_matrix_kernels(ctx):
         check(t, [int(rng.integers(3000, 16000))], int(rng.choice([4096, 8192, 14336])), int(rng.integers(2, 4)), "two or three columns")
 
 
+def test_randomized_products_through_every_route(ctx):
+    """seeded random (type, rows, K, columns, number of matrices) over the whole range the entry points route on --
+    one column to batch 512, a single block of K to 16384, one row to 40000, one to three matrices per call.  Every
+    product against the oracle; and the three ways of asking for it give the same bits: several matrices in one
+    call or one call each, f32 activations or activations quantized first (weights tiled from 1024 encoded rows)"""
+    rng = np.random.default_rng(4242)
+    cases = 0
+    while cases < 70:
+        t = int(rng.choice(WTYPES))
+        blk = npref.BLOCK[t]
+        kind = int(rng.integers(0, 3))
+        k = (blk * int(rng.integers(1, 9)) if kind == 0 else
+             int(rng.choice([2048, 4096, 5120, 8192, 11008 // blk * blk, 14336])) if kind == 1 else
+             blk * int(rng.integers(1, 16384 // blk + 1)))
+        n = int(rng.choice([1, 1, 2, 2, 3, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 24, 31, 32, 33, 64, 65, 100, 128, 129, 200, 512]))
+        ms = [int(np.exp(rng.uniform(0, np.log(40000))))]
+        ms += [int(np.exp(rng.uniform(0, np.log(20000)))) for _ in range(int(rng.choice([0, 0, 0, 1, 2])))]
+        while sum(ms) * k * n > 1.5e9 and n > 1:
+            n = max(1, n // 2)
+        if sum(ms) * k * n > 1.5e9:
+            continue
+        raws = []
+        for i, m in enumerate(ms):
+            base = min(m, 1024)
+            w = _weights(t, base, k, 9000 + 7 * cases + i).reshape(base, -1)
+            raws.append(np.concatenate([np.roll(w, j, axis=0) for j in range((m + base - 1) // base)], axis=0)[:m].reshape(-1).copy())
+        Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+        x = rng.standard_normal((n, k), dtype=np.float32) * np.float32(rng.choice([1.0, 1e-3, 30.0]))
+        if rng.random() < 0.3:
+            x[0, :blk] = 0.0
+        what = f"{NAMES[t]} ms={ms} k={k} n={n}"
+        joint = ctx.mulmat_multi(Ws, x) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x)]
+        single = [ctx.mulmat(W, x) for W in Ws]
+        act = ctx.act_create(qmm.vec_dot_type(t), k, n)
+        ctx.act_quantize(act, x)
+        two_phase = [ctx.mulmat_q8(W, act) for W in Ws]
+        for y, s1, s2, r, m in zip(joint, single, two_phase, raws, ms):
+            err = npref.rel_err(y, oracle.mul_mat(t, r, k, m, x, nthreads=16))
+            assert err <= TOL, f"{what}: rel err {err}"
+            assert np.array_equal(y, s1), f"{what}: one call for several matrices and one call each differ"
+            assert np.array_equal(s1, s2), f"{what}: f32 activations and activations quantized first differ"
+        act.free()
+        for W in Ws:
+            W.free()
+        cases += 1
+
+
 def test_randomized_mulmat_id_sweep(ctx):
     """random types, expert counts, token counts, slots and activation rows per token across the decode, bucketed,
     matrix-core and expert-GEMM paths, against the oracle"""
