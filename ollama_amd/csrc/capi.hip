@@ -599,6 +599,10 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         // decode: one launch, the GEMV quantizes x in its prologue
         float *ys[1] = {dy};
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
+    } else if (path == MI_QMM_PATH_AUTO && n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) {
+        // a few columns on a large Q4_K matrix: one launch, the workgroups quantize x themselves
+        float *ys[1] = {dy};
+        HIP_TRY(launch_deep16_f32(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
     } else {
         HIP_TRY(launch_quantize_act(q8, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream, nullptr, p.qf, p.bsf));
         DevAct a;
@@ -632,6 +636,11 @@ int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *
         // decode: the GEMV quantizes x in its own prologue, into LDS -- no scratch at all
         float *ys[1] = {y};
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
+        return MI_QMM_OK;
+    }
+    if (n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) {
+        float *ys[1] = {y};
+        HIP_TRY(launch_deep16_f32(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
         return MI_QMM_OK;
     }
     const bool f16 = wants_f16_planes(w->dev.type, n);
@@ -717,12 +726,21 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
     const bool in_kernel = same_type && !skinny && count <= gemv_max_multi() && n <= 8 &&
                            (pr.kind == PRODUCE_NONE ? gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)
                                                     : n == 1 && gemv_produce_supported(ws[0]->dev.type, K, total_m));
+    // a few columns on large Q4_K matrices: one launch of the deep kernel, whose workgroups quantize x themselves --
+    // when every matrix would take that kernel alone too (its sums do not depend on what shares the launch)
+    bool deep_f32 = same_type && !in_kernel && pr.kind == PRODUCE_NONE && n <= 8 && count <= 4 &&
+                    deep16_f32_wanted(ws[0]->dev.type, K, total_m, (int)n, ctx->num_cus);
+    for (int i = 0; deep_f32 && i < count; i++) deep_f32 = deep16_wanted(ws[i]->dev.type, K, ws[i]->dev.M, (int)n, ctx->num_cus);
     if (in_kernel) {
         // decode: one launch over the concatenated rows, the kernel produces and quantizes x in its prologue
         DevWeight dw[8];
         for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
         HIP_TRY(launch_gemv_f32_multi(dw, dys.data(), count, dx, (int)n, ctx->num_cus, ctx->stream,
                                       pr.kind == PRODUCE_NONE ? nullptr : &pr));
+    } else if (deep_f32) {
+        DevWeight dw[4];
+        for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
+        HIP_TRY(launch_deep16_f32(dw, dys.data(), count, dx, (int)n, ctx->num_cus, ctx->stream));
     } else {
         // x is produced and quantized once per activation format (Q8_0 / Q8_K) in use; weights of one type
         // then share GEMV launches four at a time, everything else goes out one product at a time

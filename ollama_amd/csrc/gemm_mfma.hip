@@ -1843,6 +1843,7 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
     const SkinnyIds none{};
     const int64_t rg = (w.M + 15) / 16;
     if (w.type == T_Q4_K) {
+        if (deep16_wanted(w.type, w.K, w.M, ncols, num_cus)) return launch_deep16(&w, &y, 1, a, col0, ncols, num_cus, s);
         if (direct16_wanted(w.type, w.K, w.M, ncols)) launch_direct16(&w, &y, 1, a, col0, ncols, num_cus, s);
         else if (rows_q4k_wanted(w.type, w.K, w.M, ncols, num_cus)) launch_rows_q4k(&w, &y, 1, a, col0, ncols, num_cus, s);
         else if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
@@ -1858,22 +1859,28 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
 // Several Q4_K matrices that share K against the same three or four activation columns: one launch of
 // the direct-load kernel over their numbered-through row groups when together they are small enough for it.
 // 1: one launch of the direct-load kernel; 2: one launch of the staged kernel; 3: one launch of the rows kernel;
-// 0: no.  Either way every matrix takes the kernel and the K cut it would take in a launch of its own, so the
+// 4: one launch of the deep direct-load kernel; 0: no.  Either way every matrix takes the kernel and the K cut it would take in a launch of its own, so the
 // results are the same bits as those of separate launches.
 int skinny_multi_kind(const DevWeight *ws, int count, int ncols, int num_cus) {
     if (count < 2 || count > DIRECT16_MULTI || ncols < 1 || ncols > 16) return 0;
     int64_t total_m = 0;
-    bool each_direct = true, none_direct = true, same_waves = true;
+    bool each_direct = true, none_direct = true, same_waves = true, each_deep = true, none_deep = true;
     const int waves0 = skinny_waves((ws[0].M + 15) / 16, ws[0].K / QKK, num_cus);
     for (int i = 0; i < count; i++) {
         if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || !skinny_supports(ws[i].type, ws[i].K, ws[i].M)) return 0;
         total_m += ws[i].M;
         const bool dir = direct16_wanted(ws[i].type, ws[i].K, ws[i].M, ncols);
+        const bool deep = deep16_wanted(ws[i].type, ws[i].K, ws[i].M, ncols, num_cus);
+        each_deep = each_deep && deep;
+        none_deep = none_deep && !deep;
         each_direct = each_direct && dir;
         none_direct = none_direct && !dir;
         same_waves = same_waves && skinny_waves((ws[i].M + 15) / 16, ws[i].K / QKK, num_cus) == waves0;
     }
     if ((total_m + 15 * count) / 16 >= 0x7fffffff) return 0;
+    // the deep direct-load kernel: its order of sums does not depend on the launch
+    if (each_deep && deep16_wanted(ws[0].type, ws[0].K, total_m, ncols, num_cus)) return 4;
+    if (!none_deep) return 0;  // (a matrix that takes the deep kernel alone joins no launch of another kernel)
     if (each_direct && direct16_wanted(ws[0].type, ws[0].K, total_m, ncols)) return 1;
     // the rows kernel (it reproduces the K cut each matrix would get alone, see skinny_rows_q4k_kernel)
     if (count <= ROWS_MULTI && none_direct && rows_q4k_wanted(ws[0].type, ws[0].K, total_m, ncols, num_cus)) return 3;
@@ -1893,7 +1900,9 @@ hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count,
     const int kind = skinny_multi_kind(ws, count, ncols, num_cus);
     if (!kind || a.type != T_Q8_K || a.K != ws[0].K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
     if (ncols < 1 || ncols > a.N || (int64_t)ncols * a.K >= ((int64_t)1 << 32)) return hipErrorInvalidValue;
-    if (kind == 1) {
+    if (kind == 4) {
+        return launch_deep16(ws, ys, count, a, 0, ncols, num_cus, s);
+    } else if (kind == 1) {
         launch_direct16(ws, ys, count, a, 0, ncols, num_cus, s);
     } else if (kind == 3) {
         launch_rows_q4k(ws, ys, count, a, 0, ncols, num_cus, s);

@@ -116,6 +116,17 @@ bool skinny_multi_supports(const DevWeight *ws, int count, int ncols, int num_cu
 hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int ncols, int num_cus,
                                hipStream_t s);
 
+// Q4_K at 3..8 columns on large matrices (skinny_deep.hip): weights straight into MFMA operand registers, two
+// pieces of four super-blocks in flight per wave, activations resident in LDS.  Up to four matrices of one K per
+// launch; the order of the floating-point sums does not depend on the launch geometry.
+bool deep16_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus);
+hipError_t launch_deep16(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols, int num_cus,
+                         hipStream_t s);
+// the same from f32 activations x [ncols][K] (device), quantized by the kernel's workgroups themselves: one launch per
+// product group.  Ask deep16_f32_wanted() first (few columns of a short K).
+bool deep16_f32_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus);
+hipError_t launch_deep16_f32(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols, int num_cus, hipStream_t s);
+
 // int8-MFMA GEMM for the 32-element block formats (Q4_0, Q8_0 weights; Q8_0 activations), any N >= 1.
 // y[n*M + m].
 bool gemm_blk32_supports(int type, int64_t K, int64_t M);

@@ -329,6 +329,43 @@ def test_q4k_rows_kernel_alone_and_joint(ctx, ms, k, ns):
         W.free()
 
 
+@pytest.mark.parametrize("ms,k,ns", [([14336, 14336], 4096, (3, 4, 8)), ([14336], 4096, (5,)), ([4096], 14336, (3, 4, 7, 8)),
+                                     ([14330, 5000], 4096, (6,)), ([4100], 14336 + 256, (5,)), ([8192], 8192, (4, 8)),
+                                     ([70000], 4096, (3, 8)), ([40000, 33000], 2048, (5,)), ([131072 + 48], 1024, (8,))])
+def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
+    """Q4_K at 3..8 columns on matrices beyond 40 M weights: the kernel that loads weights straight into registers (a ring
+    of four super-blocks per lane, quads of lanes on contiguous runs of a row, ds_bpermute into the MFMA operand order)
+    with the activations resident in LDS -- quantized by the workgroups themselves when x comes as f32.  Shapes that
+    take every cut of the launch: waves sharing a row group two and fourteen ways (gate + up, down), row groups of their
+    own (70000 and 131120 rows: two row groups per wave in turn), a last piece of one super-block (K = 14592), ragged
+    last row groups, two matrices of unequal size.  Against the oracle and exact arithmetic; the f32 form gives the bits
+    of quantize-then-multiply; a joint launch gives the bits of the single ones; a column's result does not depend on
+    which other columns ride along."""
+    rng = np.random.default_rng(9100 + sum(ms) + k)
+    raws = [_weights(Q4_K, m, k, seed=9101 + m + i) for i, m in enumerate(ms)]
+    Ws = [ctx.upload(Q4_K, r, k, m) for r, m in zip(raws, ms)]
+    act = ctx.act_create(Q8_K, k, 8)
+    for n in ns:
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        x[0, :256] = 0.0                                               # an all-zero block
+        got = ctx.mulmat_multi(Ws, x) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x)]
+        ctx.act_quantize(act, x)
+        for y, W, raw, m in zip(got, Ws, raws, ms):
+            rows = min(m, 6000)                                       # (the oracle on a slab of rows: the last ones)
+            want = oracle.mul_mat(Q4_K, np.ascontiguousarray(raw[-rows:]), k, rows, x, nthreads=16)
+            assert npref.rel_err(y[:, -rows:], want) < TOL, (m, n)
+            _check_against_exact_arithmetic(Q4_K, raw, k, m, x, y, f"Q4_K {m}x{k} n={n}", max_rows=2048)
+            assert np.array_equal(ctx.mulmat_q8(W, act), y), ("f32 != planes", m, n)
+            if len(Ws) > 1:
+                assert np.array_equal(ctx.mulmat(W, x), y), ("joint != alone", m, n)
+        again = ctx.mulmat_multi(Ws, x[::-1].copy()) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x[::-1].copy())]
+        for y, z in zip(got, again):
+            assert np.array_equal(z[::-1], y), n
+    act.free()
+    for W in Ws:
+        W.free()
+
+
 @pytest.mark.parametrize("t", WTYPES)
 def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
     """For n <= 8 the f32 entry points quantize x inside the GEMV's prologue.  The result must be
