@@ -172,23 +172,14 @@ def main() -> int:
     per_step_ms = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
     median_ms, best_ms = per_step_ms[len(per_step_ms) // 2], per_step_ms[0]
 
-    # ---- the timed launches did the work: the outputs of the last step (the last pool entry's weights) against
-    # the CPU oracle on a slab of rows, outside the timed region
-    import oracle
-    last = args.layers - 1
-    slab = 64
-    checks = {}
-    for name, yt, act, k, m in (("gate", y_gate, x, FFN_K, FFN_M), ("up", y_up, x, FFN_K, FFN_M), ("down", y_down, h, FFN_M, FFN_K)):
-        raw = np.roll(base[name], last * 37, axis=0) if last else base[name]
-        want = oracle.mul_mat(Q4_K, np.ascontiguousarray(raw[:slab]), k, slab, act.cpu().numpy(), nthreads=4)
-        err = rel_err(yt.cpu().numpy()[:, :slab], want)
-        checks[name] = err
-        if not err <= 1e-3:
-            print(f"bench.py: y_{name} of the timed step differs from the oracle (rel err {err})", file=sys.stderr)
-            return 1
+    # ---- the timed launches did the work: keep the outputs of the last step (the last pool entry's weights) for the
+    # check against the CPU oracle, which runs after every timed section (device-to-device copies here: no host work and
+    # no idle GPU between the timed sections)
+    kept = {"gate": y_gate.clone(), "up": y_up.clone(), "down": y_down.clone()}
 
-    # dominant kernel alone, back to back (HIP events on the stream the kernels run on)
-    gate_up_only()
+    # dominant kernel alone, back to back (HIP events on the stream the kernels run on), at ramped clocks like the step
+    for _ in range(max(1, args.ramp // 4)):
+        gate_up_only()
     t_k = timed(gate_up_only, args.steps)
     launches = args.layers * args.steps
     avg_launch_s = t_k / launches
@@ -206,6 +197,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "untimed_ramp_steps": args.ramp,
         "ms_per_step": round(t_step / args.steps * 1e3, 4),
         "ms_per_step_median": round(median_ms, 4),
         "ms_per_step_best": round(best_ms, 4),
@@ -225,7 +217,6 @@ def main() -> int:
             "compute_units": info["compute_units"],
             "clock_mhz_nominal": info["clock_mhz"],
             "clocks_observed_under_load": clocks_under_load,
-            "outputs_checked_against_oracle": {k_: float(f"{v_:.2e}") for k_, v_ in checks.items()},
         },
         "roofline": {
             "bound": "hbm",
@@ -307,7 +298,7 @@ def main() -> int:
                 ctx.mulmat_device(gw[c][6], hb.data_ptr(), NB, ys[6].data_ptr())
 
         layer_pass()
-        gsteps = max(2, args.steps // 4)
+        gsteps = max(17, args.steps // 4)  # x 3 rotating copies: at least 50 timed launches per matrix
         t_g = timed(layer_pass, gsteps) / (gsteps * copies)
         ops = sum(2.0 * NB * m * k for name, t, m, k in layer)
         per = {}
@@ -500,7 +491,7 @@ def main() -> int:
             tm = timed(fn, 5) / (5 * len(pool))
             other[f"decode FFN block, {label}"] = {"us": round(tm * 1e6, 2)}
         # the headline step at a few tokens (several sequences decoding together): gate + up in one call, down in a second
-        for n in (2, 4, 8):
+        for n in (2, 3, 4, 8):
             xb = torch.randn(n, FFN_K, generator=g, dtype=torch.float32).to(dev)
             hb = torch.randn(n, FFN_M, generator=g, dtype=torch.float32).to(dev)
             ygb = torch.empty(n, FFN_M, dtype=torch.float32, device=dev)
@@ -531,6 +522,21 @@ def main() -> int:
         for _ in range(5):
             dst.copy_(src)
         torch.cuda.synchronize()
+
+    # ---- the outputs of the timed step against the CPU oracle on a slab of rows (after every timed section)
+    import oracle
+    last = args.layers - 1
+    slab = 64
+    checks = {}
+    for name, act, k, m in (("gate", x, FFN_K, FFN_M), ("up", x, FFN_K, FFN_M), ("down", h, FFN_M, FFN_K)):
+        raw = np.roll(base[name], last * 37, axis=0) if last else base[name]
+        want = oracle.mul_mat(Q4_K, np.ascontiguousarray(raw[:slab]), k, slab, act.cpu().numpy(), nthreads=4)
+        err = rel_err(kept[name].cpu().numpy()[:, :slab], want)
+        checks[name] = err
+        if not err <= 1e-3:
+            print(f"bench.py: y_{name} of the timed step differs from the oracle (rel err {err})", file=sys.stderr)
+            return 1
+    out["config"]["outputs_checked_against_oracle"] = {k_: float(f"{v_:.2e}") for k_, v_ in checks.items()}
 
     # ---- CPU baseline: the oracle (scalar port of the ggml CPU path) on this host's cores -------
     if args.cpu_seconds > 0:
