@@ -61,7 +61,28 @@ enum {
     MI_QMM_PATH_GEMV = 1, /* the decode kernels at any N: streaming GEMV, 8 columns at a time; from
                              3 (Q4_K) / 4 (Q6_K, Q4_0, Q8_0) columns the skinny matrix-core kernels,
                              16 columns at a time                                                    */
-    MI_QMM_PATH_GEMM = 2  /* force the tiled int8-MFMA GEMM (any N >= 1, padded to the tile)          */
+    MI_QMM_PATH_GEMM = 2, /* force the tiled int8-MFMA GEMM (any N >= 1, padded to the tile)          */
+    MI_QMM_PATH_QUERY = 3 /* launch nothing: return the MI_QMM_ROUTE_* value of the kernel that
+                             MI_QMM_PATH_AUTO would take for this weight and n (x and y may be NULL).
+                             No counterpart in the reference; for tests that pin the routing table.  */
+};
+
+/* what MI_QMM_PATH_QUERY returns: the kernel a product takes.  It depends on the weight's type and shape, on n and
+ * on the form the activations come in (f32 for mi_qmm_mulmat_path, quantized planes for mi_qmm_mulmat_q8) only. */
+enum {
+    MI_QMM_ROUTE_GEMV_F32 = 1,         /* streaming GEMV, x quantized in its prologue (one launch)               */
+    MI_QMM_ROUTE_DEEP_F32 = 2,         /* Q4_K deep direct-load kernel, x quantized by its workgroups (one launch) */
+    MI_QMM_ROUTE_GEMM_BLK32 = 3,       /* Q4_0 / Q8_0 int8-MFMA GEMM                                              */
+    MI_QMM_ROUTE_GEMM_F16 = 4,         /* Q4_K fp16-MFMA GEMM, 256 x 128 tiles                                    */
+    MI_QMM_ROUTE_GEMM_Q6K = 5,         /* Q6_K int8-MFMA GEMM, 256 x 128 tiles, K slices                          */
+    MI_QMM_ROUTE_GEMM_INT8 = 6,        /* K-quant int8-MFMA GEMM, 128-row tiles                                   */
+    MI_QMM_ROUTE_SKINNY32 = 7,         /* Q4_0 / Q8_0 matrix-core kernel for 2..31 columns                        */
+    MI_QMM_ROUTE_SKINNY_DEEP = 8,      /* Q4_K deep direct-load kernel on quantized planes                        */
+    MI_QMM_ROUTE_SKINNY_DIRECT = 9,    /* Q4_K direct-load kernel of many small waves (small matrices, <= 4 columns) */
+    MI_QMM_ROUTE_SKINNY_ROWS_Q4K = 10, /* Q4_K rows kernel (activations resident in LDS, a wave per row group)    */
+    MI_QMM_ROUTE_SKINNY_STAGED = 11,   /* K-quant staged matrix-core kernel for 3..31 columns                     */
+    MI_QMM_ROUTE_SKINNY_ROWS_Q6K = 12, /* Q6_K rows kernel (the output head at 2..8 columns)                      */
+    MI_QMM_ROUTE_GEMV = 13             /* streaming GEMV on quantized planes                                      */
 };
 
 /* ---- size tables: replace TensorType.BlockSize / TypeSize and Tensor.Size's row rule

@@ -495,67 +495,126 @@ bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
     return n >= from && skinny_supports(type, K, M);
 }
 
-// dy: device output [n][M].  Picks the kernel and queues it on the ctx's stream.
-// may_alloc = false: never touches the ctx's growable buffers (the tiled GEMM then runs without its K-split workspace).
-int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path, bool may_alloc = true) {
+// Which kernel a product takes (the values of the MI_QMM_ROUTE_* enum of mi_qmm.h).  Decided from the weight's type and
+// shape, the number of activation columns and the planes at hand -- never from what else a call multiplies.
+// a: the quantized activations (only N, sd8 and qf are looked at).  err (optional): why there is no route.
+int route_planes(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, int path, bool may_alloc, const char **err) {
     const int64_t K = w->dev.K, M = w->dev.M, n = a.N;
     const bool blk32 = gemm_blk32_supports(w->dev.type, K, M);  // Q4_0 / Q8_0: their own MFMA kernel
     bool use_gemm;
     if (path == MI_QMM_PATH_GEMM) use_gemm = true;
     else if (path == MI_QMM_PATH_GEMV) use_gemm = false;
     else use_gemm = n >= 32 && (blk32 || gemm_supports(w->dev.type, K, M));
-    if (use_gemm && !blk32 && !gemm_supports(w->dev.type, K, M))
-        return fail(MI_QMM_ERR_UNSUPPORTED, "the MFMA GEMM does not cover type %d with K=%lld M=%lld", w->dev.type,
-                    (long long)K, (long long)M);
-    if (!use_gemm && K > gemv_max_k(w->dev.type))
-        return fail(MI_QMM_ERR_UNSUPPORTED, "K=%lld exceeds the GEMV limit %lld for type %d", (long long)K,
-                    (long long)gemv_max_k(w->dev.type), w->dev.type);
-    if (use_gemm && blk32) {
+    if (use_gemm && !blk32 && !gemm_supports(w->dev.type, K, M)) {
+        if (err) *err = "the MFMA GEMM does not cover this type and shape";
+        return 0;
+    }
+    if (!use_gemm && K > gemv_max_k(w->dev.type)) {
+        if (err) *err = "K exceeds the GEMV limit for this type";
+        return 0;
+    }
+    const bool auto_path = path != MI_QMM_PATH_GEMM && path != MI_QMM_PATH_GEMV;
+    if (use_gemm) {
+        if (blk32) return MI_QMM_ROUTE_GEMM_BLK32;
+        if (auto_path && gemm_f16_wanted(w->dev, a, ctx->num_cus)) return MI_QMM_ROUTE_GEMM_F16;
+        const int slices = auto_path ? gemm_q6k_slices(w->dev.type, K, M, n, ctx->num_cus) : 0;
+        // (a caller that may not allocate gets the 256-row Q6_K kernel only where it needs no K-slice workspace)
+        if (slices >= 1 && (may_alloc || slices == 1)) return MI_QMM_ROUTE_GEMM_Q6K;
+        return MI_QMM_ROUTE_GEMM_INT8;
+    }
+    if (blk32 && wants_skinny(w->dev.type, K, M, n)) return MI_QMM_ROUTE_SKINNY32;
+    if (a.sd8 && (wants_skinny(w->dev.type, K, M, n) || (n >= 2 && n <= 8 && skinny_rows_wanted(w->dev, (int)n, ctx->num_cus)))) {
+        // from a few columns up the K-quants go to the matrix cores, 16 columns per launch: the streaming GEMV pays one
+        // v_dot4 pass per column
+        switch (skinny_kind(w->dev, (int)(n < 16 ? n : 16), ctx->num_cus)) {
+        case 1: return MI_QMM_ROUTE_SKINNY_DEEP;
+        case 2: return MI_QMM_ROUTE_SKINNY_DIRECT;
+        case 3: return MI_QMM_ROUTE_SKINNY_ROWS_Q4K;
+        case 5: return MI_QMM_ROUTE_SKINNY_ROWS_Q6K;
+        default: return MI_QMM_ROUTE_SKINNY_STAGED;
+        }
+    }
+    return MI_QMM_ROUTE_GEMV;
+}
+
+// dy: device output [n][M].  Picks the kernel and queues it on the ctx's stream.
+// may_alloc = false: never touches the ctx's growable buffers (the tiled GEMM then runs without its K-split workspace).
+int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float *dy, int path, bool may_alloc = true) {
+    const int64_t K = w->dev.K, M = w->dev.M, n = a.N;
+    const char *why = nullptr;
+    const int route = route_planes(ctx, w, a, path, may_alloc, &why);
+    switch (route) {
+    case 0:
+        return fail(MI_QMM_ERR_UNSUPPORTED, "%s (type %d, K=%lld, M=%lld)", why, w->dev.type, (long long)K, (long long)M);
+    case MI_QMM_ROUTE_GEMM_BLK32:
         HIP_TRY(launch_gemm_blk32(w->dev, a, dy, ctx->num_cus, ctx->stream));
-    } else if (use_gemm && path == MI_QMM_PATH_AUTO && gemm_f16_wanted(w->dev, a, ctx->num_cus)) {
+        break;
+    case MI_QMM_ROUTE_GEMM_F16:
         HIP_TRY(launch_gemm_f16(w->dev, a, dy, ctx->stream));
-    } else if (use_gemm && path == MI_QMM_PATH_AUTO && gemm_q6k_slices(w->dev.type, K, M, n, ctx->num_cus) >= 1 &&
-               (may_alloc || gemm_q6k_slices(w->dev.type, K, M, n, ctx->num_cus) == 1)) {
-        // (a caller that may not allocate gets this kernel only where it needs no K-slice workspace)
+        break;
+    case MI_QMM_ROUTE_GEMM_Q6K: {
         const size_t wsf = gemm_q6k_workspace_floats(w->dev.type, K, M, n, ctx->num_cus);
         if (wsf) {
             int rc = reserve(ctx, &ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float));
             if (rc) return rc;
         }
         HIP_TRY(launch_gemm_q6k(w->dev, a, dy, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
-    } else if (use_gemm) {
+        break;
+    }
+    case MI_QMM_ROUTE_GEMM_INT8: {
         const size_t wsf = may_alloc ? gemm_workspace_floats(w->dev.type, K, M, n, ctx->num_cus) : 0;
         if (wsf) {
             int rc = reserve(ctx, &ctx->ws_buf, &ctx->ws_cap, wsf * sizeof(float));
             if (rc) return rc;
         }
         HIP_TRY(launch_gemm(w->dev, a, dy, M, wsf ? (float *)ctx->ws_buf : nullptr, wsf, ctx->num_cus, ctx->stream));
-    } else {
-        if (blk32 && wants_skinny(w->dev.type, K, M, n)) {
-            for (int64_t c0 = 0; c0 < n; c0 += 16)
-                HIP_TRY(launch_skinny32(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus,
-                                        ctx->stream));
-        } else if (a.sd8 && (wants_skinny(w->dev.type, K, M, n) || (n >= 2 && n <= 8 && skinny_rows_wanted(w->dev, (int)n, ctx->num_cus)))) {
-            // from a few columns up the K-quants go to the matrix cores, 16 columns per launch: the
-            // streaming GEMV pays one v_dot4 pass per column
-            for (int64_t c0 = 0; c0 < n; c0 += 16)
-                HIP_TRY(launch_skinny(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus,
-                                      ctx->stream));
-        } else {
-            for (int64_t c0 = 0; c0 < n; c0 += 8) {
-                const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
-                HIP_TRY(launch_gemv(w->dev, a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
-            }
+        break;
+    }
+    case MI_QMM_ROUTE_SKINNY32:
+        for (int64_t c0 = 0; c0 < n; c0 += 16)
+            HIP_TRY(launch_skinny32(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus, ctx->stream));
+        break;
+    case MI_QMM_ROUTE_SKINNY_DEEP:
+    case MI_QMM_ROUTE_SKINNY_DIRECT:
+    case MI_QMM_ROUTE_SKINNY_ROWS_Q4K:
+    case MI_QMM_ROUTE_SKINNY_ROWS_Q6K:
+    case MI_QMM_ROUTE_SKINNY_STAGED:
+        for (int64_t c0 = 0; c0 < n; c0 += 16)
+            HIP_TRY(launch_skinny(w->dev, a, (int)c0, (int)(n - c0 < 16 ? n - c0 : 16), dy, ctx->num_cus, ctx->stream));
+        break;
+    default:
+        for (int64_t c0 = 0; c0 < n; c0 += 8) {
+            const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
+            HIP_TRY(launch_gemv(w->dev, a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
         }
     }
     return MI_QMM_OK;
+}
+
+// The route of mi_qmm_mulmat on f32 activations: the kernels that quantize x themselves where they apply, else the
+// route of the planes the call would make.
+int route_f32(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n, int path, const char **err) {
+    const int64_t K = w->dev.K, M = w->dev.M;
+    if (path != MI_QMM_PATH_GEMM && n <= 8 && !wants_skinny(w->dev.type, K, M, n) && gemv_f32_supported(w->dev.type, K, M, (int)n))
+        return MI_QMM_ROUTE_GEMV_F32;
+    if (path == MI_QMM_PATH_AUTO && n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) return MI_QMM_ROUTE_DEEP_F32;
+    static const uint8_t some_plane = 0;  // (stands for "the planes are there": route_planes only asks whether)
+    DevAct a;
+    a.sd8 = mi_qmm_vec_dot_type(w->dev.type) == T_Q8_K ? &some_plane : nullptr;
+    a.sd16 = a.sd8;
+    a.qf = wants_f16_planes(w->dev.type, n) ? reinterpret_cast<const uint16_t *>(&some_plane) : nullptr;
+    a.bsf = a.qf;
+    a.K = K;
+    a.N = (int)n;
+    a.type = mi_qmm_vec_dot_type(w->dev.type);
+    return route_planes(ctx, w, a, path, /*may_alloc=*/true, err);
 }
 
 int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, int path) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
     if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
         return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
-    if (path != MI_QMM_PATH_AUTO && path != MI_QMM_PATH_GEMV && path != MI_QMM_PATH_GEMM)
+    if (path != MI_QMM_PATH_AUTO && path != MI_QMM_PATH_GEMV && path != MI_QMM_PATH_GEMM && path != MI_QMM_PATH_QUERY)
         return fail(MI_QMM_ERR_INVALID, "unknown path %d", path);
     int rc = check_ctx(ctx);
     if (rc) return rc;
@@ -573,9 +632,15 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
     int rc = check_product_args(ctx, w, location, path);
     if (rc) return rc;
+    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    if (path == MI_QMM_PATH_QUERY) {  // which kernel mi_qmm_mulmat would take; nothing is launched, x and y may be NULL
+        if (n == 0) return fail(MI_QMM_ERR_INVALID, "a product of no columns has no route");
+        const char *why = nullptr;
+        const int route = route_f32(ctx, w, n, MI_QMM_PATH_AUTO, &why);
+        return route ? route : fail(MI_QMM_ERR_UNSUPPORTED, "%s", why);
+    }
     if (n == 0) return MI_QMM_OK;
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
-    if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
 
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
@@ -594,12 +659,12 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         dy = (float *)((char *)ctx->io_buf + yoff);
         HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
     }
-    if (path != MI_QMM_PATH_GEMM && n <= 8 && !wants_skinny(w->dev.type, K, M, n) &&
-        gemv_f32_supported(w->dev.type, K, M, (int)n)) {
+    const int route = route_f32(ctx, w, n, path, nullptr);
+    if (route == MI_QMM_ROUTE_GEMV_F32) {
         // decode: one launch, the GEMV quantizes x in its prologue
         float *ys[1] = {dy};
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
-    } else if (path == MI_QMM_PATH_AUTO && n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) {
+    } else if (route == MI_QMM_ROUTE_DEEP_F32) {
         // a few columns on a large Q4_K matrix: one launch, the workgroups quantize x themselves
         float *ys[1] = {dy};
         HIP_TRY(launch_deep16_f32(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
@@ -1266,11 +1331,16 @@ int mi_qmm_mulmat_q8(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_act *
         return fail(MI_QMM_ERR_INVALID, "act (type %d, k=%lld) does not match weight (type %d needs %d, k=%lld)",
                     act->type, (long long)act->k, w->dev.type, mi_qmm_vec_dot_type(w->dev.type), (long long)w->dev.K);
     const int64_t n = act->n, M = w->dev.M;
-    if (n == 0) return MI_QMM_OK;
-    if (!y) return fail(MI_QMM_ERR_INVALID, "y is NULL");
+    if (n == 0) return path == MI_QMM_PATH_QUERY ? fail(MI_QMM_ERR_INVALID, "a product of no columns has no route") : MI_QMM_OK;
     const ActPlanes p = plan_act(act->base, act->type, act->k, act->n_max, act->f16);
     DevAct a;
     a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = act->k; a.N = (int)n; a.type = act->type;
+    if (path == MI_QMM_PATH_QUERY) {  // which kernel the product of these planes would take; nothing is launched
+        const char *why = nullptr;
+        const int route = route_planes(ctx, w, a, MI_QMM_PATH_AUTO, /*may_alloc=*/true, &why);
+        return route ? route : fail(MI_QMM_ERR_UNSUPPORTED, "%s", why);
+    }
+    if (!y) return fail(MI_QMM_ERR_INVALID, "y is NULL");
     float *dy = y;
     const size_t ybytes = (size_t)(n * M) * 4;
     if (location == MI_QMM_HOST) {

@@ -1835,6 +1835,18 @@ void launch_skinny_as(const DevWeight &w, const DevAct &a, int col0, int ncols, 
 
 bool skinny_rows_wanted(const DevWeight &w, int ncols, int num_cus) { return rows_wanted(w, ncols, num_cus); }
 
+// Which skinny kernel a single K-quant product of ncols columns takes: 1 deep direct-load (skinny_deep.hip), 2 the
+// many-small-waves direct-load kernel, 3 the Q4_K rows kernel, 4 the staged kernel, 5 the Q6_K rows kernel.
+int skinny_kind(const DevWeight &w, int ncols, int num_cus) {
+    if (w.type == T_Q4_K) {
+        if (deep16_wanted(w.type, w.K, w.M, ncols, num_cus)) return 1;
+        if (direct16_wanted(w.type, w.K, w.M, ncols)) return 2;
+        if (rows_q4k_wanted(w.type, w.K, w.M, ncols, num_cus)) return 3;
+        return 4;
+    }
+    return rows_wanted(w, ncols, num_cus) ? 5 : 4;
+}
+
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
     if (!skinny_supports(w.type, w.K, w.M) || a.type != T_Q8_K || a.K != w.K || !a.sd8 || !a.sd16) return hipErrorInvalidValue;
     if (ncols < 1 || ncols > 16 || col0 < 0 || col0 + ncols > a.N) return hipErrorInvalidValue;
@@ -1842,14 +1854,15 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
     if ((w.M + 15) / 16 > 0x7fffffff) return hipErrorInvalidValue;
     const SkinnyIds none{};
     const int64_t rg = (w.M + 15) / 16;
+    const int kind = skinny_kind(w, ncols, num_cus);
+    if (kind == 1) return launch_deep16(&w, &y, 1, a, col0, ncols, num_cus, s);
     if (w.type == T_Q4_K) {
-        if (deep16_wanted(w.type, w.K, w.M, ncols, num_cus)) return launch_deep16(&w, &y, 1, a, col0, ncols, num_cus, s);
-        if (direct16_wanted(w.type, w.K, w.M, ncols)) launch_direct16(&w, &y, 1, a, col0, ncols, num_cus, s);
-        else if (rows_q4k_wanted(w.type, w.K, w.M, ncols, num_cus)) launch_rows_q4k(&w, &y, 1, a, col0, ncols, num_cus, s);
+        if (kind == 2) launch_direct16(&w, &y, 1, a, col0, ncols, num_cus, s);
+        else if (kind == 3) launch_rows_q4k(&w, &y, 1, a, col0, ncols, num_cus, s);
         else if (ncols <= 8) launch_skinny_as<Sk16Q4K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q4K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     } else {
-        if (rows_wanted(w, ncols, num_cus)) launch_skinny_rows(w, a, col0, ncols, y, num_cus, s);
+        if (kind == 5) launch_skinny_rows(w, a, col0, ncols, y, num_cus, s);
         else if (ncols <= 8) launch_skinny_as<Sk16Q6K, 8, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
         else launch_skinny_as<Sk16Q6K, 16, false>(w, a, col0, ncols, y, none, rg, num_cus, s);
     }

@@ -110,6 +110,9 @@ bool skinny_supports(int type, int64_t K, int64_t M);
 bool skinny_rows_wanted(const DevWeight &w, int ncols, int num_cus);
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus,
                          hipStream_t s);
+// which kernel launch_skinny takes for ncols columns: 1 deep direct-load, 2 many-small-waves direct-load, 3 Q4_K rows
+// kernel, 4 staged, 5 Q6_K rows kernel
+int skinny_kind(const DevWeight &w, int ncols, int num_cus);
 // several K-quant matrices of one type and K in one launch of a skinny kernel (up to 16 columns), when every
 // one of them keeps the kernel and K cut of a launch of its own
 bool skinny_multi_supports(const DevWeight *ws, int count, int ncols, int num_cus);

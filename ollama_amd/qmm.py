@@ -18,7 +18,10 @@ LIB_PATH = os.environ.get("MI_QMM_LIB") or os.path.join(_HERE, "libmi_qmm.so")
 
 F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
 HOST, DEVICE = 0, 1
-PATH_AUTO, PATH_GEMV, PATH_GEMM = 0, 1, 2
+PATH_AUTO, PATH_GEMV, PATH_GEMM, PATH_QUERY = 0, 1, 2, 3
+# what PATH_QUERY returns (MI_QMM_ROUTE_*): the kernel a product takes
+ROUTES = {1: "gemv_f32", 2: "deep_f32", 3: "gemm_blk32", 4: "gemm_f16", 5: "gemm_q6k", 6: "gemm_int8", 7: "skinny32",
+          8: "skinny_deep", 9: "skinny_direct", 10: "skinny_rows_q4k", 11: "skinny_staged", 12: "skinny_rows_q6k", 13: "gemv"}
 PRODUCE_NONE, PRODUCE_RMSNORM, PRODUCE_SWIGLU = 0, 1, 2
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, -3, -4, -5
 
@@ -309,6 +312,20 @@ class Context:
         y = np.empty((n, w.m), dtype=np.float32)
         _check(lib().mi_qmm_mulmat_path(self._h, w._h, _ptr(x), n, _ptr(y), HOST, path))
         return y
+
+    def route(self, w: Weight, n: int) -> str:
+        """name of the kernel mulmat takes for n f32 activation rows against w (nothing is launched)"""
+        rc = lib().mi_qmm_mulmat_path(self._h, w._h, None, n, None, DEVICE, PATH_QUERY)
+        if rc <= 0:
+            raise QmmError(rc, last_error())
+        return ROUTES[rc]
+
+    def route_q8(self, w: Weight, act: "Act") -> str:
+        """name of the kernel mulmat_q8 takes for these quantized activations against w (nothing is launched)"""
+        rc = lib().mi_qmm_mulmat_q8(self._h, w._h, act._h, None, DEVICE, PATH_QUERY)
+        if rc <= 0:
+            raise QmmError(rc, last_error())
+        return ROUTES[rc]
 
     def mulmat_device(self, w: Weight, x_ptr: int, n: int, y_ptr: int, path: int = PATH_AUTO):
         """device pointers in and out; queued on the ctx stream, returns without waiting."""
