@@ -1676,15 +1676,15 @@ void launch_direct16(const DevWeight *ws, float *const *ys, int count, const Dev
     else direct16_q4k_kernel<false><<<grid, threads, 0, s>>>(g, a, col0, ncols, kcut, threads);
 }
 
-// y[i] = sum over slices of part[slice][i]
-__global__ __launch_bounds__(256) void sum_slices_kernel(const float4 *__restrict__ part, float4 *__restrict__ y,
-                                                         int64_t n4, int slices) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
-        float4 acc = part[i];
-        for (int sl = 1; sl < slices; sl++) {
-            const float4 v = part[sl * n4 + i];
-            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
-        }
+// y[i] = sum over slices of part[slice][i], in slice order; V = float4, or float for a y that is not 16-byte aligned
+// (a caller's offset into a larger tensor): the same sums in the same order either way
+__device__ __forceinline__ void add_to(float4 &a, const float4 &v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; }
+__device__ __forceinline__ void add_to(float &a, const float &v) { a += v; }
+template <class V>
+__global__ __launch_bounds__(256) void sum_slices_kernel(const V *__restrict__ part, V *__restrict__ y, int64_t n, int slices) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        V acc = part[i];
+        for (int sl = 1; sl < slices; sl++) add_to(acc, part[sl * n + i]);
         y[i] = acc;
     }
 }
@@ -1740,10 +1740,11 @@ hipError_t launch3(const DevWeight *ws, float *const *ys, int count, const DevAc
     if (tnt2) gemm3_kernel<G, 2><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part, none);
     else gemm3_kernel<G, 1><<<grid, 512, 0, s>>>(ga, a, (int)tiles_m, (int)tiles_n, part, none);
     if (ksplit > 1) {
-        const int64_t n4 = a.N * ws[0].M / 4;
-        const unsigned blocks = (unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048);
-        sum_slices_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const float4 *>(part),
-                                                 reinterpret_cast<float4 *>(ys[0]), n4, ksplit);
+        const bool vec = ((uintptr_t)ys[0] & 15) == 0 && (a.N * ws[0].M) % 4 == 0;
+        const int64_t n = a.N * ws[0].M / (vec ? 4 : 1);
+        const unsigned blocks = (unsigned)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+        if (vec) sum_slices_kernel<float4><<<blocks, 256, 0, s>>>(reinterpret_cast<const float4 *>(part), reinterpret_cast<float4 *>(ys[0]), n, ksplit);
+        else sum_slices_kernel<float><<<blocks, 256, 0, s>>>(part, ys[0], n, ksplit);
     }
     return hipGetLastError();
 }

@@ -269,14 +269,15 @@ __global__ __launch_bounds__(512, 2) void gemm_q6k_kernel(const uint8_t *__restr
     }
 }
 
-// y[i] = sum over slices of part[slice][i], in slice order
-__global__ __launch_bounds__(256) void sum_planes_kernel(const float4 *__restrict__ part, float4 *__restrict__ y, int64_t n4, int slices) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
-        float4 acc = part[i];
-        for (int sl = 1; sl < slices; sl++) {
-            const float4 v = part[sl * n4 + i];
-            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
-        }
+// y[i] = sum over slices of part[slice][i], in slice order; V = float4, or float for a y that is not 16-byte aligned
+// (a caller's offset into a larger tensor): the same sums in the same order either way
+__device__ __forceinline__ void add_to(float4 &a, const float4 &v) { a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w; }
+__device__ __forceinline__ void add_to(float &a, const float &v) { a += v; }
+template <class V>
+__global__ __launch_bounds__(256) void sum_planes_kernel(const V *__restrict__ part, V *__restrict__ y, int64_t n, int slices) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        V acc = part[i];
+        for (int sl = 1; sl < slices; sl++) add_to(acc, part[sl * n + i]);
         y[i] = acc;
     }
 }
@@ -317,9 +318,11 @@ hipError_t launch_gemm_q6k(const DevWeight &w, const DevAct &a, float *y, float 
     gemm_q6k_kernel<<<grid, 512, 0, s>>>(w.p0, w.p1, w.p2, reinterpret_cast<const uint8_t *>(w.d), reinterpret_cast<const uint8_t *>(a.qs),
                                          a.d, ks > 1 ? workspace : y, (int)w.M, a.N, (int)w.K, (int)tiles_m, (int)tiles_n);
     if (ks > 1) {
-        const int64_t n4 = (int64_t)a.N * w.M / 4;
-        const unsigned blocks = (unsigned)((n4 + 255) / 256 < 2048 ? (n4 + 255) / 256 : 2048);
-        sum_planes_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const float4 *>(workspace), reinterpret_cast<float4 *>(y), n4, ks);
+        const bool vec = ((uintptr_t)y & 15) == 0;  // (the slice count itself depends on the shape alone; (N * M) % 4 == 0 here)
+        const int64_t n = (int64_t)a.N * w.M / (vec ? 4 : 1);
+        const unsigned blocks = (unsigned)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048);
+        if (vec) sum_planes_kernel<float4><<<blocks, 256, 0, s>>>(reinterpret_cast<const float4 *>(workspace), reinterpret_cast<float4 *>(y), n, ks);
+        else sum_planes_kernel<float><<<blocks, 256, 0, s>>>(workspace, y, n, ks);
     }
     return hipGetLastError();
 }

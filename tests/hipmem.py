@@ -19,6 +19,15 @@ def _rt():
     return _hip
 
 
+def free_bytes() -> int:
+    """free device memory as hipMemGetInfo reports it"""
+    h = _rt()
+    h.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert h.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return int(free.value)
+
+
 class DeviceArray:
     """a device copy of a numpy array (or zeros of its shape); .ptr is the device address"""
 

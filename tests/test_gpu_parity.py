@@ -799,6 +799,33 @@ def test_q6k_gemm_tiles_and_slices(ctx, k, m, n):
     W.free()
 
 
+def test_gemm_k_slices_into_a_y_that_is_not_16_byte_aligned(ctx):
+    """Products cut into K slices add their partial planes into the caller's y.  A device caller may pass y at any
+    4-byte offset into a larger tensor: the sum then goes element by element, in the same slice order -- the bits of the
+    aligned call.  ffn_down at batch 512 (Q6_K: four slices on the 256-row kernel) and a Q4_K product with few tiles and
+    a long K (slices on the 128-row kernel)."""
+    from hipmem import DeviceArray
+    rng = np.random.default_rng(77)
+    for t, m, k, n in ((Q6_K, 4096, 14336, 512), (Q4_K, 1024, 16384, 128)):
+        raw = _weights(t, 512, k, seed=770 + t)
+        raw = np.tile(raw, (m // 512, 1))
+        W = ctx.upload(t, raw, k, m)
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        dx = DeviceArray(x)
+        buf = DeviceArray(np.empty(n * m + 8, np.float32), zero=True)
+        try:
+            ctx.mulmat_device(W, dx.ptr, n, buf.ptr)
+            ctx.sync()
+            aligned = buf.numpy()[: n * m].copy()
+            ctx.mulmat_device(W, dx.ptr, n, buf.ptr + 4)
+            ctx.sync()
+            assert np.array_equal(buf.numpy()[1 : n * m + 1], aligned), NAMES[t]
+            want = oracle.mul_mat(t, raw[:256], k, 256, x[:16], nthreads=16)
+            assert npref.rel_err(aligned.reshape(n, m)[:16, :256], want) < TOL
+        finally:
+            dx.free(); buf.free(); W.free()
+
+
 def test_q6k_gemm_random_block_bytes(ctx):
     """every ql / qh bit pattern and every int8 scale, negative ones and -128 included"""
     rng = np.random.default_rng(9753)

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import npref
-from hipmem import DeviceArray
+from hipmem import DeviceArray, free_bytes
 from npref import Q4_0, Q4_K, Q6_K, Q8_0
 from ollama_amd import qmm, synth
 
@@ -47,6 +47,11 @@ CASES = [
     (Q8_0, 512, 4096, 40, 33, True),       # block-32 GEMM
     (Q4_K, 1536, 4096, 300, 130, True),    # tiled GEMM, rows past n in the last tile keep the first call's quants
     (Q6_K, 512, 14336, 512, 64, False),    # mi_qmm_mulmat may cut K here; the no-allocation call does not
+    (Q4_K, 14336, 4096, 512, 200, True),   # fp16-MFMA GEMM: the fp16 planes carved out of the static scratch
+    (Q6_K, 14336, 4096, 512, 200, False),  # Q6_K 256-row GEMM; at 200 columns mi_qmm_mulmat cuts K, this call does not
+    (Q6_K, 4096, 14336, 512, 200, False),  # K slices would need workspace: falls back to the 128-row kernel without it
+    (Q4_K, 14336, 4096, 4, 3, True),       # a few columns on a large matrix: the workgroups quantize x, no scratch
+    (Q4_K, 4096, 14336, 8, 5, True),       # the same kernel on planes in the static scratch
 ]
 
 
@@ -96,3 +101,42 @@ def test_noalloc_rejects_what_does_not_fit_and_allocates_nothing(ctx):
             ctx.scratch_freeze(False)
     finally:
         W.free(); dx.free(); dy.free()
+
+
+def test_noalloc_on_a_fresh_ctx_with_frozen_scratch(ctx):
+    """A ctx that has never multiplied holds no scratch at all; with its scratch frozen every attempt to reserve any
+    fails.  mi_qmm_mulmat_noalloc must still run every kind of product -- streaming GEMV, the kernels for a few columns,
+    the tiled GEMMs -- and the device's free memory must not move.  Expected values from the module's own ctx."""
+    fresh = qmm.Context(0)
+    try:
+        fresh.scratch_freeze(True)
+        shapes = [(Q4_K, 1024, 4096, (1, 8)), (Q6_K, 768, 2048, (16,)), (Q8_0, 512, 4096, (2, 40)), (Q4_K, 14336, 4096, (4, 300)),
+                  (Q6_K, 4096, 14336, (512,))]
+        for t, m, k, ns in shapes:
+            raw = synth.weights(t, min(m, 1024), k, seed=90 + t)
+            raw = np.tile(raw, ((m + raw.shape[0] - 1) // raw.shape[0], 1))[:m]
+            W, Wf = ctx.upload(t, raw, k, m), fresh.upload(t, raw, k, m)
+            rng = np.random.default_rng(17 * t + m)
+            for n in ns:
+                print(f"fresh frozen ctx: type={t} m={m} k={k} n={n}", flush=True)
+                x = rng.standard_normal((n, k), dtype=np.float32)
+                dx = DeviceArray(x)
+                y0 = DeviceArray(np.empty((n, m), np.float32), zero=True)
+                y1 = DeviceArray(np.empty((n, m), np.float32), zero=True)
+                try:
+                    ctx.mulmat_device(W, dx.ptr, n, y0.ptr)
+                    ctx.sync()
+                    before = free_bytes()
+                    fresh.mulmat_noalloc_device(Wf, dx.ptr, n, y1.ptr)
+                    fresh.sync()
+                    assert free_bytes() == before, "device memory moved during mi_qmm_mulmat_noalloc"
+                    assert npref.rel_err(y1.numpy(), y0.numpy()) <= 1e-3
+                    with pytest.raises(qmm.QmmError):   # the growable path cannot even start on this ctx
+                        fresh.mulmat_device(Wf, dx.ptr, max(n, 9), y1.ptr)
+                finally:
+                    fresh.sync()
+                    dx.free(); y0.free(); y1.free()
+            W.free(); Wf.free()
+    finally:
+        fresh.scratch_freeze(False)
+        fresh.close()
