@@ -54,6 +54,9 @@ def lib() -> ctypes.CDLL:
         L.ref_mul_mat_id.restype = ci
         L.ref_mul_mat_id.argtypes = [ci, vp, i64, i64, i64, vp, i64, vp, i64, i64, vp]
         L.ref_rms_norm.restype = None; L.ref_rms_norm.argtypes = [vp, vp, ctypes.c_float, i64, i64, vp]
+        L.ref_qkx2_search.restype = ctypes.c_float
+        L.ref_qkx2_search.argtypes = [ci, ci, vp, vp, vp, vp, ctypes.c_float, ctypes.c_float, ci]
+        L.ref_qx_search.restype = ctypes.c_float; L.ref_qx_search.argtypes = [ci, ci, vp, vp]
         L.ref_swiglu.restype = None; L.ref_swiglu.argtypes = [vp, vp, i64, vp]
         _lib = L
     return _lib
@@ -181,6 +184,24 @@ def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     y = np.empty_like(gate)
     lib().ref_swiglu(_p(gate), _p(up), gate.size, _p(y))
     return y
+
+
+def qkx2_search(x: np.ndarray, weights: np.ndarray, nmax: int = 15, rmin: float = -1.0, rdelta: float = 0.1, nstep: int = 20):
+    """The (scale, min) search of the Q4_K encoder on one group: returns (scale, min, levels) with min <= 0."""
+    x = np.ascontiguousarray(x, np.float32); w = np.ascontiguousarray(weights, np.float32)
+    assert x.ndim == 1 and x.shape == w.shape
+    lv = np.zeros(x.size, np.uint8)
+    neg_min = np.zeros(1, np.float32)
+    sc = lib().ref_qkx2_search(x.size, nmax, _p(x), _p(w), _p(lv), _p(neg_min), rmin, rdelta, nstep)
+    return float(sc), -float(neg_min[0]), lv
+
+
+def qx_search(x: np.ndarray, nmax: int = 32):
+    """The scale search of the Q6_K encoder on one group: returns (scale, signed levels)."""
+    x = np.ascontiguousarray(x, np.float32)
+    lv = np.zeros(x.size, np.int8)
+    sc = lib().ref_qx_search(x.size, nmax, _p(x), _p(lv))
+    return float(sc), lv.astype(np.int32) - nmax
 
 
 def scale_min_k4(j: int, s12: np.ndarray):

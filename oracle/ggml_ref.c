@@ -275,6 +275,14 @@ static float make_qkx2_quants(int n, int nmax, const float *x, const float *weig
     return scale;
 }
 
+/* the search on its own, for tests of what it returns: levels[n], *neg_min = -min, returns the scale */
+float ref_qkx2_search(int n, int nmax, const float *x, const float *weights, uint8_t *levels, float *neg_min,
+                      float rmin, float rdelta, int nstep) {
+    uint8_t laux[QKK];
+    if (n < 1 || n > QKK) return -1.f;
+    return make_qkx2_quants(n, nmax, x, weights, levels, neg_min, laux, rmin, rdelta, nstep);
+}
+
 void ref_get_scale_min_k4(int j, const uint8_t *q, uint8_t *d, uint8_t *m) {
     if (j < 4) {
         *d = q[j] & 63;
@@ -400,6 +408,11 @@ static float make_qx_quants(int n, int nmax, const float *x, int8_t *L) {
         }
     }
     return scale;
+}
+
+/* the search on its own, for tests of what it returns: levels[n] hold l + nmax, returns the scale */
+float ref_qx_search(int n, int nmax, const float *x, int8_t *levels) {
+    return make_qx_quants(n, nmax, x, levels);
 }
 
 void ref_quantize_row_q6_K(const float *x, void *vy, int64_t k) {

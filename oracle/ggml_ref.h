@@ -28,8 +28,11 @@
  *   to 1e-6); the fp32 rounding of upstream's SIMD variants (vectorized expf, reduction order of the
  *   sum of squares) is not fixed by anything in the reference: PARITY UNPINNED below 1e-6 relative.
  *   weight encoders q4_K / q6_K (make_qkx2_quants / make_qx_quants searches):
- *   PARITY UNPINNED bit-for-bit against llama-quantize (only self-consistency and error
- *   bounds are checked); q4_0 / q8_0 encoders are closed forms and pinned.
+ *   PARITY UNPINNED bit-for-bit against llama-quantize.  What mathematics fixes is checked in fp64: the
+ *   returned (scale, min) is the weighted least-squares optimum for the returned levels, no candidate of
+ *   the search grid fits better, the result never fits worse than the min/max start, the stored levels
+ *   are the nearest ones for the stored scales.  That catches slips of transcription, not of recall.
+ *   q4_0 / q8_0 encoders are closed forms and pinned.
  */
 #ifndef GGML_REF_H
 #define GGML_REF_H
@@ -62,6 +65,13 @@ void ref_quantize_row_q4_K(const float *x, void *y, int64_t k);
 void ref_quantize_row_q6_K(const float *x, void *y, int64_t k);
 /* dispatch on type (2, 8, 12, 14, 15); rows are independent. returns 0 or -1 */
 int  ref_quantize(int type, const float *x, void *y, int64_t k, int64_t rows, int nthreads);
+
+/* The two searches inside the K-quant encoders, callable on one group of values so that tests can check what they
+ * return against what least squares fixes.  q4_K calls the first with (32, 15, x, av_x + |x|, ..., -1, 0.1, 20) per
+ * 32 values, q6_K the second with (16, 32, x) per 16 values (weights x^2). */
+float ref_qkx2_search(int n, int nmax, const float *x, const float *weights, uint8_t *levels, float *neg_min,
+                      float rmin, float rdelta, int nstep);
+float ref_qx_search(int n, int nmax, const float *x, int8_t *levels);
 
 /* dequantizers */
 int  ref_dequantize_row(int type, const void *x, float *y, int64_t k);

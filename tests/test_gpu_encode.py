@@ -81,6 +81,21 @@ def test_edge_blocks_give_the_oracle_bytes(ctx, t):
     _same_bytes(ctx, t, np.roll(row, 32, axis=1), "edge blocks shifted")
 
 
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+def test_k_quant_blocks_follow_from_least_squares_and_rounding(ctx, t):
+    """The GPU encoders' own bytes, without comparing them to the oracle's: top codes, d / dmin, the scale codes against
+    the searched group scales (the search being checked against fp64 least squares in the CPU suite), every level the
+    nearest one for the stored scales."""
+    import encprops
+    rng = np.random.default_rng(9300 + t)
+    for scale in (0.02, 3.0):
+        x = (rng.standard_normal((8, 2048)) * scale).astype(np.float32)
+        x[1] *= (1 + 20 * (rng.random(2048) < 0.01)).astype(np.float32)
+        x[2, :256] = 0; x[3] = np.abs(x[3]); x[4, 256:512] = -np.abs(x[4, 256:512]); x[5, 32:64] = 0
+        raw = ctx.quantize_weights(t, x)
+        (encprops.q4k_stored_bytes if t == Q4_K else encprops.q6k_stored_bytes)(x, raw)
+
+
 @pytest.mark.parametrize("t", WTYPES)
 def test_device_pointers_and_the_product_on_encoded_weights(ctx, t):
     """device in, device out: the same bytes; uploaded, they multiply like the oracle's own encoding of the same rows"""

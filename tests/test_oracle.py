@@ -358,7 +358,8 @@ def test_mul_mat_id_one_expert_is_mul_mat_and_bad_ids_are_rejected():
     assert oracle.mul_mat_id(Q4_K, w, k, m, 1, b[:0], np.zeros((0, 1), np.int32)).shape == (0, 1, m)
 
 
-# ---- weight encoders: self-consistency (bit-parity with llama-quantize is unpinned) --------------
+# ---- weight encoders: error bounds, closed forms, and what least squares fixes about the K-quant searches
+#      (bit-parity of Q4_K / Q6_K with llama-quantize stays unpinned: these catch slips of transcription, not of recall)
 @pytest.mark.parametrize("t,bound", [(Q4_0, 0.14), (Q8_0, 0.008), (Q4_K, 0.10), (Q6_K, 0.03)])
 def test_encoders_valid_blocks_and_error_bounds(t, bound):
     rng = np.random.default_rng(500 + t)
@@ -385,6 +386,72 @@ def test_q4_0_and_q8_0_encoders_closed_form():
     # Q8_0 weight encoder is the activation quantizer
     y = np.random.default_rng(3).standard_normal(64).astype(np.float32)
     assert np.array_equal(oracle.quantize(Q8_0, y).reshape(-1), npref.quantize_q8_0(y))
+
+
+def _groups(rng, n, count):
+    """groups of n values of the kinds a weight tensor holds: normal, one-sided, with an outlier, on a coarse grid"""
+    for i in range(count):
+        x = rng.standard_normal(n).astype(np.float32) * np.float32(0.02)
+        kind = i % 6
+        if kind == 1: x = np.abs(x) + np.float32(0.01)          # the fitted minimum would be positive: pulled to zero
+        if kind == 2: x[rng.integers(n)] *= 30
+        if kind == 3: x = -np.abs(x)
+        if kind == 4: x = (np.rint(x * 50) / 50).astype(np.float32)
+        if kind == 5: x *= np.float32(1000)
+        yield x
+
+
+def test_q4_K_search_returns_the_least_squares_fit_of_its_levels():
+    """make_qkx2_quants as Q4_K calls it (32 values, 16 levels, weights av_x + |x|, 21 candidate grids): in fp64 the
+    returned (scale, min) is the weighted least-squares optimum for the returned levels (with the minimum capped at
+    zero), and never a worse fit than the min/max grid the search starts from.  A dropped term or a swapped sum in the
+    normal equations fails the first, a wrong comparison the second."""
+    import collections
+    import encprops
+    rng = np.random.default_rng(610)
+    seen = collections.Counter()
+    for x in _groups(rng, 32, 3000):
+        av = np.sqrt(np.float32(np.cumsum(x * x, dtype=np.float32)[-1] / np.float32(32)))
+        seen[encprops.qkx2_search_result(x, (av + np.abs(x)).astype(np.float32))] += 1
+    assert seen["fit"] > 1000 and seen["start"] > 20, seen       # both ways out of the search were taken
+    assert encprops.qkx2_search_result(np.zeros(32, np.float32), np.ones(32, np.float32)) == "flat"
+    assert encprops.qkx2_search_result(np.full(32, -0.5, np.float32), np.ones(32, np.float32)) == "flat"   # stored as the minimum alone
+    s, m, lv = oracle.qkx2_search(np.full(32, 0.5, np.float32), np.ones(32, np.float32))
+    assert m == 0.0 and np.all(lv == 15) and abs(s * 15 - 0.5) < 1e-6       # positive constant: grid [0, 0.5], all at the top
+    # other shapes of the same search: few values, few levels, no refinement steps
+    for x in _groups(rng, 16, 300):
+        encprops.qkx2_search_result(x, np.ones(16, np.float32), nmax=3, rmin=-0.5, rdelta=0.1, nstep=15)
+        assert encprops.qkx2_search_result(x, np.abs(x) + np.float32(1e-3), nmax=31, nstep=0) in ("start", "flat")
+
+
+def test_q6_K_search_returns_the_least_squares_scale_of_its_levels():
+    """make_qx_quants as Q6_K calls it (16 values, levels -32..31, weights x^2, 19 candidate grids around -32/max): the
+    returned scale is sum(w x l) / sum(w l^2) for the returned levels, the levels are those of one grid step, and no
+    step removes more of sum(w x^2) -- the search's own criterion, evaluated in fp64."""
+    import collections
+    import encprops
+    rng = np.random.default_rng(611)
+    won = collections.Counter(encprops.qx_search_result(x) for x in _groups(rng, 16, 3000))
+    assert len([i for i in won if i is not None]) >= 8, won        # the grid is really searched: many steps win somewhere
+    assert encprops.qx_search_result(np.zeros(16, np.float32)) is None
+    assert encprops.qx_search_result(np.full(16, 1e-16, np.float32)) is None   # below the threshold: stored as zeros
+    # all values equal: every step rounds them to -32 (clamped) or -31; the scale is exactly x / l
+    s, l = oracle.qx_search(np.full(16, 0.25, np.float32))
+    assert len(set(l.tolist())) == 1 and l[0] in (-32, -31) and abs(s * l[0] - 0.25) < 1e-6
+
+
+@pytest.mark.parametrize("scale", [0.02, 3.0, 1e-3])
+def test_k_quant_encoders_stored_bytes_follow_from_the_searches(scale):
+    """The blocks the encoders write: the largest group scale (min) takes the top code, d (dmin) is that scale over 63
+    (Q6_K: the scale of largest magnitude takes -128), the other codes are the searched scales rounded against it, and
+    every stored level is the nearest one for the scales as stored."""
+    import encprops
+    rng = np.random.default_rng(612)
+    x = (rng.standard_normal((6, 2048)) * scale).astype(np.float32)
+    x[1] *= (1 + 20 * (rng.random(2048) < 0.01)).astype(np.float32)
+    x[2, :256] = 0; x[3] = np.abs(x[3]); x[4, 256:512] = -np.abs(x[4, 256:512]); x[5, 32:64] = 0
+    encprops.q4k_stored_bytes(x, oracle.quantize(Q4_K, x))
+    encprops.q6k_stored_bytes(x, oracle.quantize(Q6_K, x))
 
 
 # ---- producers of the activations: RMSNorm, SwiGLU ------------------------------------------------
