@@ -364,19 +364,24 @@ def main() -> int:
             mclk = torch.zeros(2, dtype=torch.int64, device=dev)
             blocks, iters = 2 * info["compute_units"], 8000
             ceil = {}
-            for kind, name, flop in ((0, "f16_32x32x16", 32768.0), (1, "i8_32x32x32", 65536.0)):
+            for kind, name, flop in ((0, "f16_32x32x16", 32768.0), (1, "i8_32x32x32", 65536.0),
+                                     (2, "f16_32x32x16_prefill_operands", 32768.0), (3, "i8_32x32x32_prefill_operands", 65536.0)):
                 fn = lambda: mr.mi_mfma_rate(kind, iters, blocks, mout.data_ptr(), mclk.data_ptr(), stream.cuda_stream)
                 timed(fn, 2)
                 tm = timed(fn, 3) / 3
                 c = mclk.cpu().tolist()
                 ceil[name] = {"T(FL)OP/s": round(blocks * 4 * 4.0 * iters * flop / tm / 1e12, 1), "ms_per_launch": round(tm * 1e3, 2),
                               "shader_clock_mhz": round(c[0] / (c[1] / 100.0)) if c[1] else None}
-            ceil["what"] = ("a loop of nothing but MFMAs on random operands, 4 independent accumulators per wave, 2 waves per SIMD on every CU, "
-                            "timed like the GEMM launches; the clock is the one workgroup 0 ran at (its cycle counter over the 100 MHz counter)")
+            ceil["what"] = ("a loop of nothing but MFMAs, 4 independent accumulators per wave, 2 waves per SIMD on every CU, timed like the GEMM "
+                            "launches; on random bits, and on operands distributed like the prefill kernels' (normal activations quantized to "
+                            "int8; block scale x nibble as fp16, bare nibbles for int8); the clock is the one workgroup 0 ran at (its cycle "
+                            "counter over the 100 MHz counter)")
             out["gemm"]["mfma_ceiling"] = ceil
             gate = per.get("ffn_gate")
             if gate:  # the fp16 kernel issues 17 MFMAs for 16 algorithmic ones
                 out["gemm"]["ffn_gate_frac_of_f16_ceiling"] = round(gate["tops"] * 17 / 16 / ceil["f16_32x32x16"]["T(FL)OP/s"], 4)
+                out["gemm"]["ffn_gate_frac_of_f16_ceiling_prefill_operands"] = round(
+                    gate["tops"] * 17 / 16 / ceil["f16_32x32x16_prefill_operands"]["T(FL)OP/s"], 4)
 
     # ---- the other configurations, one short timing each: f32 activations in HBM, quantization included
     if not args.no_other:

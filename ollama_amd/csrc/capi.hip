@@ -737,6 +737,21 @@ namespace {
 
 // mi_qmm_mulmat_multi and mi_qmm_mulmat_produced: several weights of one K against the same activations,
 // which may first go through a producer (prod: kind, aux and eps as the caller gave them, aux in `location`).
+// q, k and v of an attention block at prefill batch sizes: one launch of the fp16 GEMM when together they fill the
+// machine and one by one they would not.  A matrix that a launch of its own would cut into K slices keeps that cut
+// (the order of its fp32 sums must not depend on how the product was asked for), so it rules the joint launch out.
+// Of a only the type, K, N and the presence of the fp16 planes are read.
+bool f16_multi_ok(const mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const DevAct &a) {
+    if (count < 2 || count > 4 || a.type != T_Q8_K) return false;
+    DevWeight dw[4];
+    for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
+    if (!gemm_f16_multi_wanted(dw, count, a, ctx->num_cus)) return false;
+    for (int i = 0; i < count; i++)
+        if (!gemm_f16_wanted(dw[i], a, ctx->num_cus) && gemm_workspace_floats(dw[i].type, dw[i].K, dw[i].M, a.N, ctx->num_cus) != 0)
+            return false;
+    return true;
+}
+
 int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const Produce *prod, const float *x,
                       int64_t n, float *const *ys, int location) {
     if (!ws || !ys || count < 1) return fail(MI_QMM_ERR_INVALID, "ws/ys is NULL or count < 1");
@@ -833,6 +848,12 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
             DevAct a;
             a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = K; a.N = (int)n; a.type = q8;
             size_t j = 0;
+            if (q8 == T_Q8_K && idx.size() == (size_t)count && f16_multi_ok(ctx, ws, count, a)) {
+                DevWeight dw[4];
+                for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
+                HIP_TRY(launch_gemm_f16_multi(dw, dys.data(), count, a, ctx->stream));
+                j = idx.size();
+            }
             while (j < idx.size()) {
                 const mi_qmm_weight *w0 = ws[idx[j]];
                 size_t e = j + 1;
@@ -1386,7 +1407,15 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         probe.qf = probe.bsf = reinterpret_cast<const uint16_t *>(act->base);  // presence is all that is read
         for (int i = 0; gemm_ok && i < count; i++) gemm_ok = !gemm_f16_wanted(ws[i]->dev, probe, ctx->num_cus);
     }
-    bool gemv_ok = same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
+    bool f16_ok = false;
+    if (!gemm_ok && same && act->f16 && act->n >= 32) {
+        DevAct probe;
+        probe.qs = nullptr; probe.d = nullptr; probe.bsums = nullptr; probe.sd8 = probe.sd16 = nullptr;
+        probe.K = act->k; probe.N = (int)act->n; probe.type = act->type;
+        probe.qf = probe.bsf = reinterpret_cast<const uint16_t *>(act->base);  // presence is all that is read
+        f16_ok = f16_multi_ok(ctx, ws, count, probe);
+    }
+    bool gemv_ok = !f16_ok && same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
     for (int i = 0; gemv_ok && i < count; i++)  // from five or six columns up each weight goes to the skinny kernel
         gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n);
     // K-quant matrices at 3..16 columns: one launch of a skinny MFMA kernel when it gives the same bits
@@ -1398,7 +1427,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         skinny_ok = act->type == T_Q8_0 ? skinny32_multi_supports(probe, count, (int)act->n, ctx->num_cus)
                                         : skinny_multi_supports(probe, count, (int)act->n, ctx->num_cus);
     }
-    if (!gemm_ok && !gemv_ok && !skinny_ok) {
+    if (!gemm_ok && !f16_ok && !gemv_ok && !skinny_ok) {
         for (int i = 0; i < count; i++) {
             int rc = mi_qmm_mulmat_q8(ctx, ws[i], act, ys[i], location, MI_QMM_PATH_AUTO);
             if (rc) return rc;
@@ -1430,7 +1459,8 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, offs[count]))) return rc;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
-    if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));
+    if (f16_ok) HIP_TRY(launch_gemm_f16_multi(dw, dys, count, a, ctx->stream));
+    else if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));
     else if (skinny_ok && a.type == T_Q8_0) HIP_TRY(launch_skinny32_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));
     else if (skinny_ok) HIP_TRY(launch_skinny_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));
     else HIP_TRY(launch_gemv_multi(dw, dys, count, a, 0, (int)act->n, ctx->num_cus, ctx->stream));

@@ -77,17 +77,33 @@ __device__ __forceinline__ void wait_vm() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-__global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ A,
+// Up to F16_MULTI matrices of one K in a launch (q, k and v of an attention block: too few tiles each, enough
+// together): the row tiles of the matrices are numbered through, tile_end[i] is the first tile past matrix i.
+constexpr int F16_MULTI = 4;
+struct F16Args {
+    const uint8_t *W[F16_MULTI];
+    float *Y[F16_MULTI];
+    int M[F16_MULTI];
+    int tile_end[F16_MULTI];
+};
+
+__global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const uint8_t *__restrict__ A,
                                                               const float *__restrict__ YD, const uint8_t *__restrict__ BS,
-                                                              float *__restrict__ Y, int M, int N, int K, int tiles_m, int tiles_n) {
+                                                              int N, int K, int tiles_m, int tiles_n) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
     const unsigned lbase = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, h = lane >> 5;
     // row blocks that share activation tiles sit on one XCD (workgroup ids 8 apart share an L2)
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int tile_n = slot % tiles_n, tile_m = xcd + 8 * (slot / tiles_n);
-    if (tile_m >= tiles_m) return;  // the grid is rounded up to whole rounds of the 8 XCDs
+    const int tile_n = slot % tiles_n, tile_all = xcd + 8 * (slot / tiles_n);
+    if (tile_all >= tiles_m) return;  // the grid is rounded up to whole rounds of the 8 XCDs
+    const int e0 = fa.tile_end[0], e1 = fa.tile_end[1], e2 = fa.tile_end[2];
+    const int t = (tile_all >= e0) + (tile_all >= e1) + (tile_all >= e2);
+    const int tile_m = tile_all - (t == 0 ? 0 : t == 1 ? e0 : t == 2 ? e1 : e2);
+    const uint8_t *__restrict__ W = t == 0 ? fa.W[0] : t == 1 ? fa.W[1] : t == 2 ? fa.W[2] : fa.W[3];
+    float *__restrict__ Y = t == 0 ? fa.Y[0] : t == 1 ? fa.Y[1] : t == 2 ? fa.Y[2] : fa.Y[3];
+    const int M = t == 0 ? fa.M[0] : t == 1 ? fa.M[1] : t == 2 ? fa.M[2] : fa.M[3];
     const int nsb = K / QKK;
     const int64_t pitch = (int64_t)nsb * Q4_K_BYTES;
     const int64_t m0 = (int64_t)tile_m * TM, n0 = (int64_t)tile_n * TN;
@@ -296,15 +312,47 @@ bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus) {
     return 4 * tiles >= 3 * (int64_t)num_cus;
 }
 
-hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, hipStream_t s) {
-    if (w.type != T_Q4_K || a.type != T_Q8_K || a.K != w.K || !a.qf || !a.bsf || !y || a.N < 1) return hipErrorInvalidValue;
-    const int64_t tiles_m = (w.M + TM - 1) / TM, tiles_n = (a.N + TN - 1) / TN;
+// Several matrices in one launch where that fills the machine and single launches would not: every matrix Q4_K of one
+// K within the kernel's offset limits, together at least three quarters of a tile per CU, and at least one of them
+// too small for a launch of its own on this kernel.  The int8 kernel such a matrix takes alone computes the same
+// exact integer sums and combines them with the same fp32 expressions, so the bits are those of the single launches.
+bool gemm_f16_multi_wanted(const DevWeight *ws, int count, const DevAct &a, int num_cus) {
+    if (count < 2 || count > F16_MULTI || !a.qf || !a.bsf || a.N <= 64) return false;
+    int64_t tiles = 0;
+    bool all_alone = true;
+    for (int i = 0; i < count; i++) {
+        const DevWeight &w = ws[i];
+        if (w.type != T_Q4_K || w.K != ws[0].K || w.K < QKK || w.K % QKK || w.M < 1) return false;
+        if ((int64_t)a.N * w.K >= ((int64_t)1 << 31) || w.M * (w.K / QKK * Q4_K_BYTES) >= ((int64_t)1 << 32)) return false;
+        tiles += (w.M + TM - 1) / TM * ((a.N + TN - 1) / TN);
+        all_alone = all_alone && gemm_f16_wanted(w, a, num_cus);
+    }
+    return !all_alone && 4 * tiles >= 3 * (int64_t)num_cus;
+}
+
+hipError_t launch_gemm_f16_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, hipStream_t s) {
+    if (count < 1 || count > F16_MULTI || a.type != T_Q8_K || !a.qf || !a.bsf || a.N < 1) return hipErrorInvalidValue;
+    F16Args fa;
+    int64_t tiles_m = 0;
+    for (int i = 0; i < F16_MULTI; i++) {
+        const int j = i < count ? i : count - 1;
+        if (ws[j].type != T_Q4_K || ws[j].K != a.K || !ys[j] || ws[j].M > 0x7fffffff || ws[j].M < 1) return hipErrorInvalidValue;
+        fa.W[i] = ws[j].p0; fa.Y[i] = ys[j]; fa.M[i] = (int)ws[j].M;
+        if (i < count) tiles_m += (ws[i].M + TM - 1) / TM;
+        fa.tile_end[i] = i < count ? (int)tiles_m : 0x7fffffff;
+    }
+    const int64_t tiles_n = (a.N + TN - 1) / TN;
     const int64_t grid = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
-    if (grid > 0x7fffffff || w.M > 0x7fffffff || w.K > 0x7fffffff) return hipErrorInvalidValue;
-    gemm_f16_q4k_kernel<<<(unsigned)grid, 512, 0, s>>>(w.p0, reinterpret_cast<const uint8_t *>(a.qf), a.d,
-                                                       reinterpret_cast<const uint8_t *>(a.bsf), y, (int)w.M, a.N, (int)w.K,
-                                                       (int)tiles_m, (int)tiles_n);
+    if (grid > 0x7fffffff || a.K > 0x7fffffff) return hipErrorInvalidValue;
+    gemm_f16_q4k_kernel<<<(unsigned)grid, 512, 0, s>>>(fa, reinterpret_cast<const uint8_t *>(a.qf), a.d, reinterpret_cast<const uint8_t *>(a.bsf),
+                                                       a.N, (int)a.K, (int)tiles_m, (int)tiles_n);
     return hipGetLastError();
+}
+
+hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, hipStream_t s) {
+    if (!y) return hipErrorInvalidValue;
+    float *ys[1] = {y};
+    return launch_gemm_f16_multi(&w, ys, 1, a, s);
 }
 
 }  // namespace miqmm

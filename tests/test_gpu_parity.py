@@ -799,6 +799,34 @@ def test_q6k_gemm_tiles_and_slices(ctx, k, m, n):
     W.free()
 
 
+def test_fp16_gemm_takes_q_k_v_in_one_launch(ctx):
+    """q, k and v of an attention block from batch 1024: too few 256-row tiles each (k and v: 4 x 8), enough together,
+    so the multi entry points launch the fp16 kernel once over all three.  The bits are those of the single products
+    (k and v alone run on the int8 kernel: same exact integer sums, same fp32 expressions), checked against the
+    oracle on a sample; a batch too small for the joint launch (512) and a ragged one keep the rule too."""
+    k = 4096
+    ms = (4096, 1024, 1000)
+    raws = [_weights(Q4_K, m, k, seed=880 + i) for i, m in enumerate(ms)]
+    Ws = [ctx.upload(Q4_K, r, k, m) for r, m in zip(raws, ms)]
+    rng = np.random.default_rng(88)
+    try:
+        for n in (1024, 1100, 512):
+            x = rng.standard_normal((n, k), dtype=np.float32)
+            act = ctx.act_create(Q8_K, k, n)
+            ctx.act_quantize(act, x)
+            alone = [ctx.mulmat_q8(W, act) for W in Ws]
+            for got in (ctx.mulmat_q8_multi(Ws, act), ctx.mulmat_multi(Ws, x)):
+                for y, wnt in zip(got, alone):
+                    assert np.array_equal(y, wnt), n
+            act.free()
+            for raw, m, y in zip(raws, ms, alone):
+                want = oracle.mul_mat(Q4_K, raw[-200:], k, 200, x[-24:], nthreads=16)
+                assert npref.rel_err(y[-24:, -200:], want) < TOL
+    finally:
+        for W in Ws:
+            W.free()
+
+
 def test_gemm_k_slices_into_a_y_that_is_not_16_byte_aligned(ctx):
     """Products cut into K slices add their partial planes into the caller's y.  A device caller may pass y at any
     4-byte offset into a larger tensor: the sum then goes element by element, in the same slice order -- the bits of the
