@@ -107,7 +107,7 @@ def probe_lane_map(L, dev, stream, iters):
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     res = {}
     for mode, name in ((0, "lane = row + 16 * piece (MFMA operand order)"), (1, "lane = 4 * row + piece (quads on 64 contiguous bytes)"),
-                       (2, "linear 1 KiB per load (no rows)")):
+                       (3, "lane = 8 * row + piece (eight lanes on a row's 128 contiguous bytes)"), (2, "linear 1 KiB per load (no rows)")):
         best = None
         for blocks in (cus // 2, cus, 2 * cus, 4 * cus):
             def fn():

@@ -487,10 +487,13 @@ namespace {
 // From this many activation columns up a product below the GEMM's batch goes to a matrix-core skinny
 // kernel instead of the streaming GEMV (measured crossovers on MI355X: the GEMV pays one v_dot4 pass
 // per column).
-bool wants_skinny(int type, int64_t K, int64_t M, int64_t n) {
+bool wants_skinny(int type, int64_t K, int64_t M, int64_t n, int num_cus) {
     // (long rows of Q4_0 / Q8_0 from two columns: the GEMV at 4096 x 14336 takes 27 / 39 us at two / three columns of
     // Q8_0 where the matrix-core kernel takes 17.5)
     if (type == T_Q4_0 || type == T_Q8_0) return n >= (K > 8192 ? 2 : 4) && skinny32_supports(type, K, M);
+    // (two columns of a large Q4_K matrix with rows of one K segment: the deep direct-load kernel, 16.4 against 17.1 us
+    // for gate + up)
+    if (type == T_Q4_K && n == 2 && skinny_supports(type, K, M) && deep16_wanted(type, K, M, 2, num_cus)) return true;
     const int64_t from = type == T_Q4_K ? 3 : 4;
     return n >= from && skinny_supports(type, K, M);
 }
@@ -522,8 +525,8 @@ int route_planes(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a,
         if (slices >= 1 && (may_alloc || slices == 1)) return MI_QMM_ROUTE_GEMM_Q6K;
         return MI_QMM_ROUTE_GEMM_INT8;
     }
-    if (blk32 && wants_skinny(w->dev.type, K, M, n)) return MI_QMM_ROUTE_SKINNY32;
-    if (a.sd8 && (wants_skinny(w->dev.type, K, M, n) || (n >= 2 && n <= 8 && skinny_rows_wanted(w->dev, (int)n, ctx->num_cus)))) {
+    if (blk32 && wants_skinny(w->dev.type, K, M, n, ctx->num_cus)) return MI_QMM_ROUTE_SKINNY32;
+    if (a.sd8 && (wants_skinny(w->dev.type, K, M, n, ctx->num_cus) || (n >= 2 && n <= 8 && skinny_rows_wanted(w->dev, (int)n, ctx->num_cus)))) {
         // from a few columns up the K-quants go to the matrix cores, 16 columns per launch: the streaming GEMV pays one
         // v_dot4 pass per column
         switch (skinny_kind(w->dev, (int)(n < 16 ? n : 16), ctx->num_cus)) {
@@ -595,7 +598,7 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
 // route of the planes the call would make.
 int route_f32(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n, int path, const char **err) {
     const int64_t K = w->dev.K, M = w->dev.M;
-    if (path != MI_QMM_PATH_GEMM && n <= 8 && !wants_skinny(w->dev.type, K, M, n) && gemv_f32_supported(w->dev.type, K, M, (int)n))
+    if (path != MI_QMM_PATH_GEMM && n <= 8 && !wants_skinny(w->dev.type, K, M, n, ctx->num_cus) && gemv_f32_supported(w->dev.type, K, M, (int)n))
         return MI_QMM_ROUTE_GEMV_F32;
     if (path == MI_QMM_PATH_AUTO && n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) return MI_QMM_ROUTE_DEEP_F32;
     static const uint8_t some_plane = 0;  // (stands for "the planes are there": route_planes only asks whether)
@@ -697,7 +700,7 @@ int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
-    if (n <= 8 && !wants_skinny(w->dev.type, K, M, n) && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
+    if (n <= 8 && !wants_skinny(w->dev.type, K, M, n, ctx->num_cus) && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
         // decode: the GEMV quantizes x in its own prologue, into LDS -- no scratch at all
         float *ys[1] = {y};
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
@@ -802,7 +805,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
     }
 
     bool skinny = false;
-    for (int i = 0; i < count; i++) skinny = skinny || wants_skinny(ws[i]->dev.type, K, ws[i]->dev.M, n);
+    for (int i = 0; i < count; i++) skinny = skinny || wants_skinny(ws[i]->dev.type, K, ws[i]->dev.M, n, ctx->num_cus);
     const bool in_kernel = same_type && !skinny && count <= gemv_max_multi() && n <= 8 &&
                            (pr.kind == PRODUCE_NONE ? gemv_f32_supported(ws[0]->dev.type, K, total_m, (int)n)
                                                     : n == 1 && gemv_produce_supported(ws[0]->dev.type, K, total_m));
@@ -857,9 +860,9 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
             while (j < idx.size()) {
                 const mi_qmm_weight *w0 = ws[idx[j]];
                 size_t e = j + 1;
-                if (n <= 8 && !wants_skinny(w0->dev.type, K, w0->dev.M, n) && K <= gemv_max_k(w0->dev.type))
+                if (n <= 8 && !wants_skinny(w0->dev.type, K, w0->dev.M, n, ctx->num_cus) && K <= gemv_max_k(w0->dev.type))
                     while (e < idx.size() && e - j < (size_t)gemv_max_multi() && ws[idx[e]]->dev.type == w0->dev.type &&
-                           !wants_skinny(w0->dev.type, K, ws[idx[e]]->dev.M, n))
+                           !wants_skinny(w0->dev.type, K, ws[idx[e]]->dev.M, n, ctx->num_cus))
                         e++;
                 // matrices on the skinny MFMA kernels (q, k and v of a layer at 3..16 columns): one launch
                 // over as many of them as keep the kernel and K cut of a launch of their own
@@ -875,7 +878,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
                         es++;
                     }
                 }
-                if (e - j == 1 && es - j > 1 && (q8 == T_Q8_0 || (a.sd8 && a.sd16)) && wants_skinny(w0->dev.type, K, w0->dev.M, n)) {
+                if (e - j == 1 && es - j > 1 && (q8 == T_Q8_0 || (a.sd8 && a.sd16)) && wants_skinny(w0->dev.type, K, w0->dev.M, n, ctx->num_cus)) {
                     DevWeight dw[8];
                     float *out[8];
                     for (size_t t = j; t < es; t++) { dw[t - j] = ws[idx[t]]->dev; out[t - j] = dys[idx[t]]; }
@@ -1417,11 +1420,11 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     }
     bool gemv_ok = !f16_ok && same && count <= gemv_max_multi() && act->n <= 8 && ws[0]->dev.K <= gemv_max_k(ws[0]->dev.type);
     for (int i = 0; gemv_ok && i < count; i++)  // from five or six columns up each weight goes to the skinny kernel
-        gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n);
+        gemv_ok = !wants_skinny(ws[i]->dev.type, ws[i]->dev.K, ws[i]->dev.M, act->n, ctx->num_cus);
     // K-quant matrices at 3..16 columns: one launch of a skinny MFMA kernel when it gives the same bits
     bool skinny_ok = false;
     if (!gemm_ok && !gemv_ok && same && count >= 2 && count <= 8 && act->n >= 1 && act->n <= 16 &&
-        wants_skinny(ws[0]->dev.type, ws[0]->dev.K, ws[0]->dev.M, act->n)) {
+        wants_skinny(ws[0]->dev.type, ws[0]->dev.K, ws[0]->dev.M, act->n, ctx->num_cus)) {
         DevWeight probe[8];
         for (int i = 0; i < count; i++) probe[i] = ws[i]->dev;
         skinny_ok = act->type == T_Q8_0 ? skinny32_multi_supports(probe, count, (int)act->n, ctx->num_cus)

@@ -53,6 +53,7 @@ __global__ __launch_bounds__(256) void lds_b128_kernel(const int *__restrict__ o
 //   mode 0  lane = row + 16 * piece   (the order an MFMA B operand wants: 16 rows apart between neighbouring lanes)
 //   mode 1  lane = 4 * row + piece    (quads of lanes on 64 contiguous bytes)
 //   mode 2  linear: lane l reads bytes 16 l .. of a contiguous 2 KiB (no rows at all: the reference line)
+//   mode 3  lane = 8 * row + piece    (eight lanes on the 128 contiguous quant bytes of a row, eight rows per load)
 template <int MODE>
 __global__ __launch_bounds__(256) void lane_map_kernel(const uint8_t *__restrict__ p, int64_t pitch, int nsb, int groups, unsigned *__restrict__ out) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -63,6 +64,7 @@ __global__ __launch_bounds__(256) void lane_map_kernel(const uint8_t *__restrict
         int64_t o;
         if (MODE == 0) o = (int64_t)(lane & 15) * pitch + 16 + 16 * (lane >> 4);
         else if (MODE == 1) o = (int64_t)(lane >> 2) * pitch + 16 + 16 * (lane & 3);
+        else if (MODE == 3) o = (int64_t)(lane >> 3) * pitch + 16 + 16 * (lane & 7);
         else o = 16 * lane;
         for (int sb = 0; sb < nsb; sb += 4) {
             u4v v[8];
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(256) void lane_map_kernel(const uint8_t *__restrict
             for (int u = 0; u < 4; u++) {
                 const int64_t so = MODE == 2 ? (int64_t)(sb + u) * 2048 : (int64_t)(sb + u) * 144;
                 v[2 * u] = *reinterpret_cast<const u4v *>(base + o + so);
-                v[2 * u + 1] = *reinterpret_cast<const u4v *>(base + o + so + (MODE == 2 ? 1024 : 64));
+                v[2 * u + 1] = *reinterpret_cast<const u4v *>(base + o + so + (MODE == 2 ? 1024 : MODE == 3 ? 8 * pitch : 64));
             }
 #pragma unroll
             for (int u = 0; u < 8; u++) acc ^= v[u];
@@ -251,13 +253,14 @@ int mi_probe_lds_b128(const int *off, int iters, int waves, long long *out, void
 // p: device buffer of rows * pitch bytes (pitch = nsb * 144; mode 2 reads it as groups * nsb * 2048 contiguous bytes and
 // needs that much); rows a multiple of 16; nsb a multiple of 4; out: device scratch of 256 words
 int mi_probe_lane_map(int mode, const void *p, int64_t rows, int nsb, int blocks, unsigned *out, void *stream) {
-    if (!p || !out || rows < 16 || rows % 16 || nsb < 4 || nsb % 4 || blocks < 1 || mode < 0 || mode > 2) return -1;
+    if (!p || !out || rows < 16 || rows % 16 || nsb < 4 || nsb % 4 || blocks < 1 || mode < 0 || mode > 3) return -1;
     hipStream_t s = (hipStream_t)stream;
     const uint8_t *q = (const uint8_t *)p;
     const int64_t pitch = (int64_t)nsb * 144;
     const int groups = (int)(rows / 16);
     if (mode == 0) lane_map_kernel<0><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
     else if (mode == 1) lane_map_kernel<1><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
+    else if (mode == 3) lane_map_kernel<3><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
     else lane_map_kernel<2><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }

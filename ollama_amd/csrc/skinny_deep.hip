@@ -461,7 +461,8 @@ bool deep16_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, s
 }  // namespace
 
 bool deep16_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus) {
-    if (type != T_Q4_K || ncols < 3) return false;
+    // two columns only on rows of one K segment: on longer rows the streaming kernel with its in-kernel quantization is ahead
+    if (type != T_Q4_K || ncols < 2 || (ncols == 2 && K > 4096)) return false;
     DeepCut c;
     size_t lds;
     if (!deep16_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds)) return false;

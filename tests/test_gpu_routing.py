@@ -32,7 +32,7 @@ TABLE = [
     ("q_proj", Q4_K, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "skinny_direct", 4: "skinny_direct", 8: "skinny_staged",
                                   16: "skinny_staged", 32: "gemm_int8", 512: "gemm_int8", 2048: "gemm_f16"}),
     ("k_proj", Q4_K, 1024, 4096, {1: "gemv_f32", 4: "skinny_direct", 512: "gemm_int8"}),
-    ("ffn_gate", Q4_K, 14336, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "deep_f32", 8: "deep_f32",
+    ("ffn_gate", Q4_K, 14336, 4096, {1: "gemv_f32", 2: "deep_f32", 3: "deep_f32", 4: "deep_f32", 8: "deep_f32",
                                      16: "skinny_staged", 32: "gemm_int8", 512: "gemm_f16"}),
     ("ffn_down Q4_K", Q4_K, 4096, 14336, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "deep_f32", 8: "skinny_deep",
                                           16: "skinny_staged", 512: "gemm_int8"}),
@@ -61,7 +61,7 @@ def test_routes_of_quantized_planes(ctx):
     if ctx.device_info()["compute_units"] != 256:
         pytest.skip("the table is the one of a 256-CU part")
     W = _upload_any(ctx, Q4_K, 14336, 4096)
-    for n, want in ((1, "gemv"), (2, "gemv"), (3, "skinny_deep"), (8, "skinny_deep"), (16, "skinny_staged"), (512, "gemm_f16")):
+    for n, want in ((1, "gemv"), (2, "skinny_deep"), (3, "skinny_deep"), (8, "skinny_deep"), (16, "skinny_staged"), (512, "gemm_f16")):
         act = ctx.act_create(Q8_K, 4096, n)
         ctx.act_quantize(act, np.zeros((n, 4096), np.float32))
         assert ctx.route_q8(W, act) == want, n
