@@ -515,14 +515,16 @@ hipError_t launch_deep16(const DevWeight *ws, float *const *ys, int count, const
     return launch_deep16_any(ws, ys, count, &a, nullptr, col0, ncols, num_cus, s);
 }
 
-// The same from f32 activations x [ncols][K] (device): the workgroups quantize x themselves.  Every workgroup repeats the
-// quantization, so this is for few columns of a short K: up to four rounds of four blocks per wave.
+// The same from f32 activations x [ncols][K] (device): the workgroups quantize x themselves.  Every workgroup reads all of
+// x again (as f32: 3.5 times the bytes of its quantized planes) and repeats the quantization, so this is for few columns
+// of a short K: up to three rounds of four blocks per wave, the rounds a wave requests ahead of its first weights.  (A
+// fourth round -- four columns of K = 14336 -- measured 14.7 us against 13.5 for quantize-then-multiply.)
 bool deep16_f32_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus) {
     if (!deep16_wanted(type, K, total_m, ncols, num_cus)) return false;
     DeepCut c;
     size_t lds;
     if (!deep16_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds)) return false;
-    return (int64_t)ncols * (K / QKK) <= 4 * 4 * c.W;
+    return (int64_t)ncols * (K / QKK) <= 3 * 4 * c.W;
 }
 hipError_t launch_deep16_f32(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols, int num_cus, hipStream_t s) {
     if (!x) return hipErrorInvalidValue;

@@ -34,7 +34,7 @@ TABLE = [
     ("k_proj", Q4_K, 1024, 4096, {1: "gemv_f32", 4: "skinny_direct", 512: "gemm_int8"}),
     ("ffn_gate", Q4_K, 14336, 4096, {1: "gemv_f32", 2: "deep_f32", 3: "deep_f32", 4: "deep_f32", 8: "deep_f32",
                                      16: "skinny_staged", 32: "gemm_int8", 512: "gemm_f16"}),
-    ("ffn_down Q4_K", Q4_K, 4096, 14336, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "deep_f32", 8: "skinny_deep",
+    ("ffn_down Q4_K", Q4_K, 4096, 14336, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "skinny_deep", 8: "skinny_deep",
                                           16: "skinny_staged", 512: "gemm_int8"}),
     ("ffn_down Q6_K", Q6_K, 4096, 14336, {1: "gemv_f32", 2: "gemv_f32", 3: "gemv_f32", 4: "skinny_staged", 8: "skinny_staged",
                                           32: "gemm_int8", 512: "gemm_q6k"}),
