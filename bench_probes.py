@@ -31,6 +31,7 @@ def load():
     L.mi_probe_empty.argtypes = [ci, ci, vp]
     L.mi_probe_lds_b128.argtypes = [vp, ci, ci, vp, vp]
     L.mi_probe_lane_map.argtypes = [ci, vp, i64, ci, ci, vp, vp]
+    L.mi_probe_flood_read.argtypes = [ci, vp, ci, vp, vp]
     L.mi_probe_copy_stream.argtypes = [vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, vp, vp]
     L.mi_probe_handoff.argtypes = [vp, vp, vp, vp, ci, ci, ctypes.c_uint, ci, vp]
     return L
@@ -122,6 +123,22 @@ def probe_lane_map(L, dev, stream, iters):
     return {"probe": "lane_order_of_16_byte_loads", "bytes_read_per_launch": rows * nsb * 128, "modes": res}
 
 
+def probe_flood_read(L, dev, stream, iters):
+    """the gate + up launch of the deep direct-load kernel as a pure read: 1792 groups of 16 rows x 2304 bytes, all requested at once"""
+    groups, nbuf = 1792, 4
+    bufs = [torch.randint(0, 255, (groups * 36864,), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
+    out = torch.zeros(256, dtype=torch.int32, device=dev)
+    res = {}
+    for mode, name in ((0, "quads of lanes on 64 contiguous bytes of 16 rows (the kernel's order)"), (1, "contiguous: 1 KiB per load, 8 whole rows per wave")):
+        def fn():
+            for b in bufs:
+                check(L.mi_probe_flood_read(mode, b.data_ptr(), groups, out.data_ptr(), stream.cuda_stream))
+        timed(fn, 5, stream)
+        t = min(timed(fn, max(5, iters // 10), stream) for _ in range(3)) / nbuf
+        res[name] = {"us": round(t * 1e6, 2), "GB/s": round(groups * 36864 / t / 1e9)}
+    return {"probe": "all_loads_in_flight_at_once", "bytes": groups * 36864, "shape": "256 workgroups of 14 waves, 18 loads of 16 bytes per lane", "modes": res}
+
+
 def probe_copy_stream(L, dev, stream, iters):
     """the output head's shape: 128256 rows x 16 super-blocks, a row group of 16 per wave-step"""
     rows, nsb = 128256, 16
@@ -169,7 +186,7 @@ def probe_handoff(L, dev, stream, iters):
             "polls_that_ran_out": int(err.item())}
 
 
-PROBES = {"empty": probe_empty, "lds": probe_lds, "lane_map": probe_lane_map, "copy_stream": probe_copy_stream, "handoff": probe_handoff}
+PROBES = {"empty": probe_empty, "lds": probe_lds, "lane_map": probe_lane_map, "flood_read": probe_flood_read, "copy_stream": probe_copy_stream, "handoff": probe_handoff}
 
 
 def main():

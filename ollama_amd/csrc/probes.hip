@@ -4,6 +4,7 @@
 //   mi_probe_lds_b128   which lanes does the LDS serve together on a 16-byte read (which layouts are conflict-free)?
 //   mi_probe_lane_map   how fast does a launch stream a matrix when the lanes of a 16-byte load are laid over the rows
 //                       in different orders (what the address coalescer makes of each)?
+//   mi_probe_flood_read what does a launch that requests all of its 66 MB at once achieve, row-strided or contiguous?
 //   mi_probe_copy_stream  what does the stream of direct-to-LDS copies of a staged small-batch kernel cost by itself,
 //                       and which of its copies cost what (bytes moved, or cache lines named)?
 //   mi_probe_handoff    what does it cost to hand a partial tile from one workgroup to another inside a launch
@@ -77,6 +78,39 @@ __global__ __launch_bounds__(256) void lane_map_kernel(const uint8_t *__restrict
 #pragma unroll
             for (int u = 0; u < 8; u++) acc ^= v[u];
         }
+    }
+    unsigned x = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    for (int m = 1; m < 64; m <<= 1) x ^= __shfl_xor(x, m, 64);
+    if (lane == 0) atomicXor(out + (blockIdx.x & 255), x);
+}
+
+// ---- everything in flight at once: the read pattern of the deep direct-load kernel on its gate + up launch, by itself.
+// One workgroup of 14 waves per CU; a workgroup owns 7 consecutive groups of 16 rows (36,864 contiguous bytes each at
+// K = 4096), two waves per group.  Every wave requests its whole share -- 18,432 bytes, 18 loads of 16 bytes per lane --
+// before it looks at any of it:
+//   mode 0  as the kernel does: wave h of a group takes the K half h of all 16 rows; per load a quad of lanes reads 64
+//           contiguous bytes of a row, the 16 quads 16 different rows
+//   mode 1  the same bytes of the matrix split the other way: wave h takes rows 8h .. 8h+7 whole, a contiguous run of
+//           18,432 bytes, 1 KiB per load
+template <int MODE>
+__global__ __launch_bounds__(896) void flood_read_kernel(const uint8_t *__restrict__ p, int groups, unsigned *__restrict__ out) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = blockIdx.x * 7 + (wave >> 1), h = wave & 1;
+    u4v acc = {0, 0, 0, 0};
+    if (g < groups) {
+        const uint8_t *base = p + (int64_t)g * 36864;
+        u4v v[18];
+        if (MODE == 0) {
+            const uint8_t *q = base + (lane >> 2) * 2304 + h * 1152 + 16 * (lane & 3);
+#pragma unroll
+            for (int u = 0; u < 18; u++) v[u] = *reinterpret_cast<const u4v *>(q + 64 * u);
+        } else {
+            const uint8_t *q = base + h * 18432 + 16 * lane;
+#pragma unroll
+            for (int u = 0; u < 18; u++) v[u] = *reinterpret_cast<const u4v *>(q + 1024 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < 18; u++) acc ^= v[u];
     }
     unsigned x = acc.x ^ acc.y ^ acc.z ^ acc.w;
     for (int m = 1; m < 64; m <<= 1) x ^= __shfl_xor(x, m, 64);
@@ -262,6 +296,15 @@ int mi_probe_lane_map(int mode, const void *p, int64_t rows, int nsb, int blocks
     else if (mode == 1) lane_map_kernel<1><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
     else if (mode == 3) lane_map_kernel<3><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
     else lane_map_kernel<2><<<blocks, 256, 0, s>>>(q, pitch, nsb, groups, out);
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+// p: device buffer of groups * 36864 bytes (groups of 16 rows of 2304 bytes); out: device scratch of 256 words
+int mi_probe_flood_read(int mode, const void *p, int groups, unsigned *out, void *stream) {
+    if (!p || !out || groups < 1 || mode < 0 || mode > 1) return -1;
+    const int blocks = (groups + 6) / 7;
+    if (mode == 0) flood_read_kernel<0><<<blocks, 896, 0, (hipStream_t)stream>>>((const uint8_t *)p, groups, out);
+    else flood_read_kernel<1><<<blocks, 896, 0, (hipStream_t)stream>>>((const uint8_t *)p, groups, out);
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
