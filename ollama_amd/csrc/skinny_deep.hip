@@ -196,7 +196,11 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
 
     // ---- 2. the weight stream: a ring of four super-blocks per lane; a slot is requested again (for the same slot of
     // the wave's next piece) as soon as its super-block has been multiplied
-    const int lrow = lane >> 2, lq = lane & 3;  // loading: the lane's row and its place in the quad
+    // loading: the lane's row and which 16-byte piece of the quad's 64 bytes it takes.  Rows 8..15 take the pieces in the
+    // order 2 3 0 1: ds_bpermute moves 32 lanes per cycle through 32 banks (bank = source lane mod 32), a half-wave reads
+    // pieces {0, 1} (or {2, 3}) of all 16 rows, and with the same order in every row the sources 4 r + p of rows r and
+    // r + 8 would share a bank.
+    const int lrow = lane >> 2, lq = (lane & 3) ^ ((lane >> 4) & 2);
     struct ItemAt { gbytes_t base; unsigned roff; };
     auto item_at = [&](int group) __attribute__((always_inline)) {
         const DeepWhere at = deep_where(g, group);
@@ -284,7 +288,8 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
 
     // ---- 3. operand reads: per-lane LDS addresses and per-super-block strides (0 for lanes that read zeros)
     const int r = lane & 15, kg = lane >> 4;  // MFMA order: the lane's weight row (= A row) and K group
-    const int bidx = 4 * (4 * r + kg);        // ds_bpermute: the lane that loaded what this lane multiplies
+    const int rsw = (r >> 3) << 1;            // (rows 8..15 were loaded with their pieces in the order 2 3 0 1)
+    const int bidx = 4 * (4 * r + (kg ^ rsw));  // ds_bpermute: the lane that loaded what this lane multiplies
     unsigned a0_at, a_st, d_at, d_st, y_at;
     {
         const int col = r >> 1, w = r & 1;  // A row r: column, which of the MFMA's two sub-blocks
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
         const v2f yd = lds_at<v2f>(y_at + (unsigned)sb * (NCT * 4), 0);
         u4v hdr;  // the four dwords of the row's header, from the four lanes of the quad that loaded it
 #pragma unroll
-        for (int j = 0; j < 4; j++) hdr[j] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * (4 * r) + 4 * j, (int)R.hdr[i]);
+        for (int j = 0; j < 4; j++) hdr[j] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * (4 * r) + 4 * (j ^ rsw), (int)R.hdr[i]);
         const v4i av0 = lds_at<v4i>(aa0, 0), av1 = lds_at<v4i>(aa1, 0);
         const u4v qa = bperm(bidx, R.qa[i]);
         const float d = h2f(hdr.x & 0xffff), dmin = h2f(hdr.x >> 16);
