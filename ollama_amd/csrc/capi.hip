@@ -740,8 +740,8 @@ namespace {
 
 // mi_qmm_mulmat_multi and mi_qmm_mulmat_produced: several weights of one K against the same activations,
 // which may first go through a producer (prod: kind, aux and eps as the caller gave them, aux in `location`).
-// q, k and v of an attention block at prefill batch sizes: one launch of the fp16 GEMM when together they fill the
-// machine and one by one they would not.  A matrix that a launch of its own would cut into K slices keeps that cut
+// q, k and v of an attention block, or gate and up of a feed-forward block, at prefill batch sizes: one launch of the
+// fp16 GEMM when together they fill the machine.  A matrix that a launch of its own would cut into K slices keeps that cut
 // (the order of its fp32 sums must not depend on how the product was asked for), so it rules the joint launch out.
 // Of a only the type, K, N and the presence of the fp16 planes are read.
 bool f16_multi_ok(const mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const DevAct &a) {

@@ -799,18 +799,19 @@ def test_q6k_gemm_tiles_and_slices(ctx, k, m, n):
     W.free()
 
 
-def test_fp16_gemm_takes_q_k_v_in_one_launch(ctx):
+@pytest.mark.parametrize("ms,ns", [((4096, 1024, 1000), (1024, 1100, 512)), ((6144, 6400), (1024, 700))])
+def test_fp16_gemm_takes_q_k_v_in_one_launch(ctx, ms, ns):
     """q, k and v of an attention block from batch 1024: too few 256-row tiles each (k and v: 4 x 8), enough together,
     so the multi entry points launch the fp16 kernel once over all three.  The bits are those of the single products
     (k and v alone run on the int8 kernel: same exact integer sums, same fp32 expressions), checked against the
-    oracle on a sample; a batch too small for the joint launch (512) and a ragged one keep the rule too."""
+    oracle on a sample; a batch too small for the joint launch (512) and a ragged one keep the rule too.  Second set: two
+    matrices that each take the fp16 kernel alone (gate and up of a feed-forward block) in one launch."""
     k = 4096
-    ms = (4096, 1024, 1000)
     raws = [_weights(Q4_K, m, k, seed=880 + i) for i, m in enumerate(ms)]
     Ws = [ctx.upload(Q4_K, r, k, m) for r, m in zip(raws, ms)]
     rng = np.random.default_rng(88)
     try:
-        for n in (1024, 1100, 512):
+        for n in ns:
             x = rng.standard_normal((n, k), dtype=np.float32)
             act = ctx.act_create(Q8_K, k, n)
             ctx.act_quantize(act, x)
