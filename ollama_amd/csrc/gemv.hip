@@ -592,6 +592,40 @@ __device__ __forceinline__ void thin_rows_ahead(const DevWeight &w, const typena
     }
 }
 
+// The row loop with two loads in flight and nothing in the way of the compiler's count of them: the loads alternate
+// between two named sets of registers (no copy from "next" to "current", which would have to wait for the next row before
+// the current one is multiplied), every load inside the loop is unconditional (the last iteration is peeled off instead;
+// a wave with an odd number of loads re-reads its last rows once), so each multiply waits for its own row only.
+// a, b: the first two loads (rows wrow0 + min(run, nrw-1) and wrow0 + min(RPL + run, nrw-1)), requested by the caller.
+// Totals go to part[(rl0+i)][kseg] (one column).  For rows cut into K segments; for rows of one segment (two workgroups
+// per CU, every wave asking at once) a second load in flight measured slower: gate + up 13.1-13.4 against 12.9 us.
+template <class P, int RPL>
+__device__ __forceinline__ void thin_rows_two(const DevWeight &w, const typename P::Geo &g, typename P::Raw a, typename P::Raw b,
+                                              const typename P::Act (&act)[1], int64_t wrow0, int nrw, int lane, float *part, int rl0,
+                                              int kw, int kseg) {
+    const int run = RPL == 1 ? 0 : lane / (64 / RPL);
+    auto finish = [&](const typename P::Raw &raw, int i) __attribute__((always_inline)) {
+        float acc[1] = {0.f};
+        P::template dot<1>(raw, g, act, acc);
+        const int tot_all = __float_as_int(run_total<RPL>(acc[0]));
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            const float tot = __int_as_float(__builtin_amdgcn_readlane(tot_all, 64 / RPL * (r + 1) - 1));
+            if (lane == 63 && i + r < nrw) part[(rl0 + i + r) * kw + kseg] = tot;
+        }
+    };
+    int i = 0;
+#pragma unroll 1
+    for (; i + 2 * RPL < nrw; i += 2 * RPL) {
+        finish(a, i);
+        a = P::load(w, g, wrow0 + min(i + 2 * RPL + run, nrw - 1));
+        finish(b, i + RPL);
+        b = P::load(w, g, wrow0 + min(i + 3 * RPL + run, nrw - 1));
+    }
+    finish(a, i);
+    if (i + RPL < nrw) finish(b, i + RPL);  // wave-uniform
+}
+
 // ---------------------------------------------------------------------------------------------
 // The thin-wave kernel: many small waves instead of a few unrolled ones.
 //
@@ -658,8 +692,11 @@ __device__ __forceinline__ void quantize_x_to_lds(const float4 *__restrict__ x4,
         const int c = wave + j * nwaves;
         if (c * 64 < total4) quantize_piece(c, xpre[j]);  // wave-uniform
     }
-    for (int c = wave + XP * nwaves; c * 64 < total4; c += nwaves)
-        quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
+    // (XP == 1 is launched only where a piece per wave covers all of x: no further pieces, and no loop with loads in
+    // it for the compiler to lose its count of the outstanding ones over)
+    if constexpr (XP > 1)
+        for (int c = wave + XP * nwaves; c * 64 < total4; c += nwaves)
+            quantize_piece(c, x4[min(c * 64 + lane, total4 - 1)]);
 }
 
 // The same for Q8_K activations with a quarter of a wave per block (q8_K_quantize_row16: lane l of a 16-lane row holds
@@ -834,10 +871,35 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     const bool has_aux = XMODE == 3 || (XMODE == 2 && pr.aux != nullptr);
     if (ROW16 && XMODE == 3) prefetch_x16(reinterpret_cast<const float4 *>(pr.aux), NC * nblk, wave, lane, apre16);
     else if (XMODE >= 2) prefetch_x(has_aux ? reinterpret_cast<const float4 *>(pr.aux) : x4, total4, wave, nwaves, lane, apre);
-    static_assert(!AHEAD || (RPL == 1 && NC == 1 && XMODE == 1), "a second row ahead: one plain f32 column, one row per load");
+    static_assert(!AHEAD || (!DIRECT && RPL == 1 && NC == 1 && XMODE == 1), "a second row ahead: one plain f32 column, rows cut into K segments");
     typename P::Raw cur, nxt;
-    if (nrw > 0) cur = P::load(w, g, r0 + rl0 + min(run, nrw - 1));
+    // The first row of weights is requested whether or not the wave has rows (a wave past the matrix' last row re-reads
+    // that row and drops it): behind a condition the compiler no longer knows how many loads are in flight where the two
+    // paths meet, and waits for all of them -- the weights from HBM included -- before it lets the quantization touch x.
+    // (The scheduling barriers keep the requests in this order -- x first: loads return in the order they were made.)
+    // (Q4_0 / Q8_0 keep the request under its condition: on their short launches, 5-7 us, the order the compiler then
+    // chooses measured 3 % faster.)
+    if constexpr (P::ACT_BLK == QKK) {
+        __builtin_amdgcn_sched_barrier(0);
+        cur = P::load(w, g, min(r0 + rl0 + min(run, max(nrw, 1) - 1), w.M - 1));
+        __builtin_amdgcn_sched_barrier(0);
+    } else {
+        if (nrw > 0) cur = P::load(w, g, r0 + rl0 + min(run, nrw - 1));
+    }
     constexpr size_t PSUM_BYTES = XMODE == 2 ? XPRE * 16 * sizeof(double) : 0;  // one sum per 256-element piece
+    // AHEAD kernels (one plain f32 column, rows cut into K segments): where the four waves of a K segment are also the
+    // four that quantize that segment's sixteen blocks (four row groups per workgroup, segments of 4096, one round of
+    // four blocks per wave), a wave waits for those three others only -- a count in LDS -- instead of for all sixteen
+    // at a barrier, and the waves that share a row group hand their partial sums to whichever of them finishes last
+    // instead of meeting at a second barrier.  The counters are cleared here, behind a barrier that costs nothing: every
+    // wave has its requests out and nothing to do until x arrives.
+    const int part_floats = rows_per_wg * NC * kw;
+    int *seg_cnt = reinterpret_cast<int *>(smem + act_bytes + PSUM_BYTES) + part_floats;  // [8] segments, [8] row groups
+    const bool seg_sync = AHEAD && ROW16 && rw_log2 == 2 && P::SEG == 4096 && NC * nblk <= 4 * nwaves && kw <= 8;
+    if (AHEAD && seg_sync) {
+        if (threadIdx.x < 16) seg_cnt[threadIdx.x] = 0;
+        __syncthreads();
+    }
     if (XMODE == 2) {
         // RMSNorm: piece sums of squares through LDS, added in piece order by every thread
         double *psum = reinterpret_cast<double *>(smem + act_bytes);
@@ -866,8 +928,26 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     if (F32) {
         if (ROW16) quantize_x_to_lds16<P>(x4, NC * nblk, wave, nwaves, lane, xq, lqs, ld_, lbs);
         else quantize_x_to_lds<P, XP>(x4, total4, wave, nwaves, lane, xpre, lqs, ld_, lbs);
-        if (AHEAD && nrw > 0 && !tail) nxt = P::load(w, g, r0 + rl0 + min(1, nrw - 1));
-        __syncthreads();
+        if constexpr (AHEAD && ROW16) {  // the wave's second load: unconditional, like the first
+            const int step = tail ? TAILR : 1;
+            nxt = P::load(w, g, min(r0 + rl0 + min(step + run, max(nrw, 1) - 1), w.M - 1));
+            __builtin_amdgcn_sched_barrier(0);
+        } else if constexpr (AHEAD) {
+            // (Q4_0 / Q8_0: short launches on which the two-load loop below measured 4-6 % slower; they keep the second
+            // row under its condition and the loop that copies it down)
+            if (nrw > 0 && !tail) nxt = P::load(w, g, r0 + rl0 + min(1, nrw - 1));
+        }
+        if (AHEAD && seg_sync) {
+            // this wave's blocks are in LDS (it waits for its own writes), then it counts itself in and waits for the
+            // other quantizing waves of its segment: blocks 16 kseg .. of the row come from waves 4 kseg ..
+            const int quantizers = min(4, (nblk - 16 * kseg + 3) / 4);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (lane == 0 && 4 * wave < nblk) __hip_atomic_fetch_add(&seg_cnt[kseg], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            while (__hip_atomic_load(&seg_cnt[kseg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < quantizers) __builtin_amdgcn_s_sleep(1);
+            asm volatile("" ::: "memory");
+        } else {
+            __syncthreads();
+        }
     }
     float *part = reinterpret_cast<float *>(smem + act_bytes + PSUM_BYTES);
 
@@ -882,8 +962,13 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
             for (int n = 0; n < NC; n++) P::load_act(a, col0 + n, kseg, vlane, g, act[n]);
         }
         float keep[NC];  // lane 63-i ends up holding the total of the wave's row i
-        if (tail) thin_rows<P, NC, DIRECT, TAILR>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
-        else if constexpr (AHEAD) thin_rows_ahead<P, DIRECT>(w, g, cur, nxt, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
+        if constexpr (AHEAD && ROW16) {
+            if (tail) thin_rows_two<P, TAILR>(w, g, cur, nxt, act, r0 + rl0, nrw, lane, part, rl0, kw, kseg);
+            else thin_rows_two<P, 1>(w, g, cur, nxt, act, r0 + rl0, nrw, lane, part, rl0, kw, kseg);
+        } else if constexpr (AHEAD) {
+            if (tail) thin_rows<P, NC, DIRECT, TAILR>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
+            else thin_rows_ahead<P, DIRECT>(w, g, cur, nxt, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
+        } else if (tail) thin_rows<P, NC, DIRECT, TAILR>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
         else thin_rows<P, NC, DIRECT, RPL>(w, g, cur, act, r0 + rl0, nrw, lane, keep, part, rl0, kw, kseg);
         if (DIRECT && lane > 63 - nrw) {
 #pragma unroll
@@ -892,6 +977,20 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     }
     if (DIRECT) return;
 
+    if (AHEAD && seg_sync) {
+        // the kw waves of a row group count themselves in when their partial sums are in LDS; the last one adds them, in
+        // segment order as always, and stores the rows
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        int arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(&seg_cnt[8 + rg], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived == kw - 1 && lane < nrw) {
+            float sum = 0.f;
+            for (int k = 0; k < kw; k++) sum += part[(rl0 + lane) * kw + k];
+            yrow0[rl0 + lane] = sum;
+        }
+        return;
+    }
     __syncthreads();
     for (int i = threadIdx.x; i < nrows * NC; i += (kw << rw_log2) * 64) {
         const int n = i / nrows, rl = i - n * nrows;
@@ -1103,7 +1202,7 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
     if (p.rpl > 1) rows_per_wave = max(2 * p.rpl, (rows_per_wave + p.rpl - 1) / p.rpl * p.rpl);
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
-    p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float));
+    p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float) + 64);  // + 16 counters
     if (produce) {
         if (!f32 || nc != 1 || K > (int64_t)XPRE * p.kw * p.rw * 256) return false;
         p.lds += XPRE * 16 * sizeof(double);
