@@ -1068,9 +1068,11 @@ __global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const floa
     const bool has_aux = XMODE == 2 && pr.aux != nullptr;
     if (XMODE == 2) prefetch_x(has_aux ? reinterpret_cast<const float4 *>(pr.aux) : x4, total4, wave, nwaves, lane, apre);
     typename P::Raw cur;
-    if (nrw > 0) {
-        const int v = min(run, 2 * nrw - 1);
-        cur = P::load(v & 1 ? wb : wa, g, r0 + rl0 + (v >> 1));
+    {   // unconditional and behind the x loads, as in gemv_thin_kernel: the quantization then waits for x only
+        const int v = min(run, 2 * max(nrw, 1) - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        cur = P::load(v & 1 ? wb : wa, g, min(r0 + rl0 + (v >> 1), wa.M - 1));
+        __builtin_amdgcn_sched_barrier(0);
     }
     constexpr size_t PSUM_BYTES = XMODE == 2 ? XPRE * 16 * sizeof(double) : 0;
     if (XMODE == 2) {
