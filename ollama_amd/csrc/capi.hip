@@ -553,7 +553,7 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
         HIP_TRY(launch_gemm_blk32(w->dev, a, dy, ctx->num_cus, ctx->stream));
         break;
     case MI_QMM_ROUTE_GEMM_F16:
-        HIP_TRY(launch_gemm_f16(w->dev, a, dy, ctx->stream));
+        HIP_TRY(launch_gemm_f16(w->dev, a, dy, ctx->num_cus, ctx->stream));
         break;
     case MI_QMM_ROUTE_GEMM_Q6K: {
         const size_t wsf = gemm_q6k_workspace_floats(w->dev.type, K, M, n, ctx->num_cus);
@@ -854,7 +854,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
             if (q8 == T_Q8_K && idx.size() == (size_t)count && f16_multi_ok(ctx, ws, count, a)) {
                 DevWeight dw[4];
                 for (int i = 0; i < count; i++) dw[i] = ws[i]->dev;
-                HIP_TRY(launch_gemm_f16_multi(dw, dys.data(), count, a, ctx->stream));
+                HIP_TRY(launch_gemm_f16_multi(dw, dys.data(), count, a, ctx->num_cus, ctx->stream));
                 j = idx.size();
             }
             while (j < idx.size()) {
@@ -1462,7 +1462,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
         if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, offs[count]))) return rc;
         for (int i = 0; i < count; i++) dys[i] = (float *)((char *)ctx->io_buf + offs[i]);
     }
-    if (f16_ok) HIP_TRY(launch_gemm_f16_multi(dw, dys, count, a, ctx->stream));
+    if (f16_ok) HIP_TRY(launch_gemm_f16_multi(dw, dys, count, a, ctx->num_cus, ctx->stream));
     else if (gemm_ok) HIP_TRY(launch_gemm_multi(dw, dys, count, a, nullptr, 0, ctx->num_cus, ctx->stream));
     else if (skinny_ok && a.type == T_Q8_0) HIP_TRY(launch_skinny32_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));
     else if (skinny_ok) HIP_TRY(launch_skinny_multi(dw, dys, count, a, (int)act->n, ctx->num_cus, ctx->stream));

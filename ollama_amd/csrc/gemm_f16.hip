@@ -50,10 +50,19 @@ __device__ __forceinline__ h2 as_h2(unsigned v) { return __builtin_bit_cast(h2, 
 __device__ __forceinline__ unsigned as_u(h2 v) { return __builtin_bit_cast(unsigned, v); }
 __device__ __forceinline__ float h2f(unsigned bits16) { return __half2float(__ushort_as_half((unsigned short)bits16)); }
 
-constexpr int TM = 256, TN = 128, NST = 4, WAVES = 8;
-constexpr int A_STAGE = TN * 128, W_STAGE = TM * 32;
-constexpr int OFF_A = 0, OFF_W = OFF_A + NST * A_STAGE, OFF_H = OFF_W + NST * W_STAGE, OFF_BS = OFF_H + 2 * TM * 16,
-              OFF_YD = OFF_BS + 2 * TN * 32, OFF_DUMMY = OFF_YD + 2 * TN * 4, LDS_BYTES = OFF_DUMMY + 256;
+// Tile shapes: 256 x 128 (eight waves) where that gives nearly every CU a workgroup; 128 x 64 (four waves) for products
+// with fewer outputs -- the 4096-row attention projections at batch 512 are 64 tiles of the first kind and 256 of the
+// second.  A wave owns 32 weight rows and all TN activation rows either way; per chunk every wave issues one weight copy
+// and two activation copies in both shapes (TN * 128 B over TM / 32 waves), so the hand-counted waits are the same.
+constexpr int NST = 4;
+template <int TM_, int TN_>
+struct F16Tile {
+    static constexpr int TM = TM_, TN = TN_, WAVES = TM / 32, NS = TN / 32;
+    static_assert(TN * 128 == 2 * WAVES * 1024, "two activation copies per wave and chunk");
+    static constexpr int A_STAGE = TN * 128, W_STAGE = TM * 32;
+    static constexpr int OFF_A = 0, OFF_W = OFF_A + NST * A_STAGE, OFF_H = OFF_W + NST * W_STAGE, OFF_BS = OFF_H + 2 * TM * 16,
+                         OFF_YD = OFF_BS + 2 * TN * 32, OFF_DUMMY = OFF_YD + 2 * TN * 4, LDS_BYTES = OFF_DUMMY + 256;
+};
 
 __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     const unsigned long long v = (unsigned long long)p;
@@ -87,10 +96,14 @@ struct F16Args {
     int tile_end[F16_MULTI];
 };
 
-__global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const uint8_t *__restrict__ A,
-                                                              const float *__restrict__ YD, const uint8_t *__restrict__ BS,
-                                                              int N, int K, int tiles_m, int tiles_n) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+template <class T>
+__global__ __launch_bounds__(64 * T::WAVES, 2) void gemm_f16_q4k_kernel(F16Args fa, const uint8_t *__restrict__ A,
+                                                                        const float *__restrict__ YD, const uint8_t *__restrict__ BS,
+                                                                        int N, int K, int tiles_m, int tiles_n) {
+    constexpr int TM = T::TM, TN = T::TN, WAVES = T::WAVES, NS = T::NS, A_STAGE = T::A_STAGE, W_STAGE = T::W_STAGE, OFF_A = T::OFF_A,
+                  OFF_W = T::OFF_W, OFF_H = T::OFF_H, OFF_BS = T::OFF_BS, OFF_YD = T::OFF_YD, OFF_DUMMY = T::OFF_DUMMY;
+    constexpr int HW = WAVES / 2;  // waves that copy weight headers; the other half copies block sums
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[T::LDS_BYTES];
     const unsigned lbase = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, h = lane >> 5;
@@ -110,8 +123,8 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
     const int rows_left = (int)min((int64_t)TM, (int64_t)M - m0);  // rows past M: the last row again, results dropped
 
     // ---- copy plan: per wave and chunk two activation copies and one weight copy; per super-block one copy of
-    // weight headers (waves 0..3) or block sums (waves 4..7) and one of block scales (waves 0, 1; the others copy
-    // to a dummy slot so that every wave counts the same number of operations)
+    // weight headers (the first half of the waves) or block sums (the second half) and one of block scales (the first
+    // TN / 64 waves; the others copy to a dummy slot so that every wave counts the same number of operations)
     unsigned aoff[2], woff, soff;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -122,20 +135,20 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
     {
         const int s = wave * 64 + lane, wr = s >> 1, hh = s & 1;
         woff = (unsigned)min(wr, rows_left - 1) * (unsigned)pitch + 16u + 16u * (hh ^ ((wr >> 3) & 1));
-        const int s4 = (wave & 3) * 64 + lane, brow = s4 >> 1, bh = s4 & 1;
-        soff = wave < 4 ? (unsigned)min(s4, rows_left - 1) * (unsigned)pitch
-                        : (unsigned)brow * (unsigned)(nsb * 32) + 16u * (bh ^ ((brow >> 3) & 1));
+        const int s4 = (wave % HW) * 64 + lane, brow = s4 >> 1, bh = s4 & 1;
+        soff = wave < HW ? (unsigned)min(s4, rows_left - 1) * (unsigned)pitch
+                         : (unsigned)brow * (unsigned)(nsb * 32) + 16u * (bh ^ ((brow >> 3) & 1));
     }
-    const unsigned ydoff = (unsigned)((wave & 1) * 64 + lane) * (unsigned)(nsb * 4);
+    const unsigned ydoff = (unsigned)((wave % (TN / 64)) * 64 + lane) * (unsigned)(nsb * 4);
     const uint8_t *wbase = W + m0 * pitch;
     const uint8_t *abase = A + n0 * (int64_t)K * 2;
     const uint8_t *bsbase = BS + n0 * nsb * 32;
     const uint8_t *ydbase = reinterpret_cast<const uint8_t *>(YD + n0 * nsb);
 
     auto copy_sb = [&](int sb, int sbslot) __attribute__((always_inline)) {
-        if (wave < 4) dma16(wbase + (int64_t)sb * Q4_K_BYTES, soff, lbase + OFF_H + sbslot * 4096 + wave * 1024);
-        else dma16(bsbase + (int64_t)sb * 32, soff, lbase + OFF_BS + sbslot * 4096 + (wave - 4) * 1024);
-        dma4(ydbase + (int64_t)sb * 4, ydoff, lbase + (wave < 2 ? OFF_YD + sbslot * 512 + wave * 256 : OFF_DUMMY));
+        if (wave < HW) dma16(wbase + (int64_t)sb * Q4_K_BYTES, soff, lbase + OFF_H + sbslot * (TM * 16) + wave * 1024);
+        else dma16(bsbase + (int64_t)sb * 32, soff, lbase + OFF_BS + sbslot * (TN * 32) + (wave - HW) * 1024);
+        dma4(ydbase + (int64_t)sb * 4, ydoff, lbase + (wave < TN / 64 ? OFF_YD + sbslot * (TN * 4) + wave * 256 : OFF_DUMMY));
     };
     // a chunk's three copies go out one at a time (part 0: weights, 1 and 2: activations): eight waves issuing all of
     // theirs right behind a barrier queue up at the texture addresser
@@ -154,16 +167,16 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
     const int rd_bs = OFF_BS + col * 32 + 16 * (h ^ ((col >> 3) & 1));
     const int rd_yd = OFF_YD + 16 * h;
 
-    v16f acc[4];
-    float yacc[4][16];
+    v16f acc[NS];
+    float yacc[NS][16];
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < NS; a++)
 #pragma unroll
         for (int i = 0; i < 16; i++) { yacc[a][i] = 0.f; acc[a][i] = 0.f; }
 
-    auto load_a = [&](int stage, int t, v8h (&a)[4]) __attribute__((always_inline)) {
+    auto load_a = [&](int stage, int t, v8h (&a)[NS]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int ns = 0; ns < 4; ns++)
+        for (int ns = 0; ns < NS; ns++)
             a[ns] = *reinterpret_cast<const v8h *>(lds + rd_a + stage * A_STAGE + ns * 4096 + 16 * ((2 * t + h) ^ asw));
     };
 
@@ -177,7 +190,7 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
     float dd = 0.f, dmin = 0.f;
     unsigned sc03 = 0, sc47 = 0;
     v8h bmin;
-    v8h a_cur[4], a_nxt[4];
+    v8h a_cur[NS], a_nxt[NS];
     v4u raw_nxt;
     load_a(0, 0, a_nxt);
     raw_nxt = *reinterpret_cast<const v4u *>(lds + rd_w);
@@ -189,7 +202,7 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             if (c == 0) {
-                const v4u hd = *reinterpret_cast<const v4u *>(lds + rd_h + sbslot * 4096);
+                const v4u hd = *reinterpret_cast<const v4u *>(lds + rd_h + sbslot * (TM * 16));
                 dd = h2f(hd.x & 0xffff) * 16384.f;
                 dmin = h2f(hd.x >> 16) * 512.f;
                 // 8 six-bit scales and mins as bytes
@@ -219,7 +232,7 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
             for (int t = 0; t < 4; t++) {
                 const int u = t & 1, lohi = t >> 1;
 #pragma unroll
-                for (int ns = 0; ns < 4; ns++) a_cur[ns] = a_nxt[ns];
+                for (int ns = 0; ns < NS; ns++) a_cur[ns] = a_nxt[ns];
                 if (t == 2) {
                     // The next chunk (group q+1) must have landed in every wave before its operands are fetched below;
                     // one later group (q+2) stays in flight.  After the barrier every wave is past chunk q-1, whose stage
@@ -262,17 +275,17 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
                     b = __builtin_bit_cast(v8h, bb);
                 }
 #pragma unroll
-                for (int ns = 0; ns < 4; ns++)
+                for (int ns = 0; ns < NS; ns++)
                     acc[ns] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_cur[ns], b, (c == 0 && t == 0) ? zero : acc[ns], 0, 0, 0);
             }
             if (c == 3) {
                 // per-super-block epilogue: accumulator i of a lane is activation row 8(i/4) + 4h + i%4, weight row col
 #pragma unroll
-                for (int ns = 0; ns < 4; ns++) {
-                    const v8h am = *reinterpret_cast<const v8h *>(lds + rd_bs + sbslot * 4096 + ns * 1024);
+                for (int ns = 0; ns < NS; ns++) {
+                    const v8h am = *reinterpret_cast<const v8h *>(lds + rd_bs + sbslot * (TN * 32) + ns * 1024);
                     float4 yd4[4];
 #pragma unroll
-                    for (int g = 0; g < 4; g++) yd4[g] = *reinterpret_cast<const float4 *>(lds + rd_yd + sbslot * 512 + (32 * ns + 8 * g) * 4);
+                    for (int g = 0; g < 4; g++) yd4[g] = *reinterpret_cast<const float4 *>(lds + rd_yd + sbslot * (TN * 4) + (32 * ns + 8 * g) * 4);
                     const v16f mac = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bmin, zero, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
@@ -291,7 +304,7 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
     const int64_t m = m0 + 32 * wave + col;
     if (m < M) {
 #pragma unroll
-        for (int ns = 0; ns < 4; ns++)
+        for (int ns = 0; ns < NS; ns++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int64_t n = n0 + 32 * ns + 8 * (i >> 2) + 4 * h + (i & 3);
@@ -302,14 +315,61 @@ __global__ __launch_bounds__(512, 2) void gemm_f16_q4k_kernel(F16Args fa, const 
 
 }  // namespace
 
-// The kernel pays where its 256 x 128 tiles give (nearly) every CU a workgroup; smaller products stay on the
-// 128-row tiles of the int8 kernel.  The choice depends on the weight and the batch only, never on what else a
-// call multiplies, so a product's bits do not depend on how it was asked for.
+typedef F16Tile<256, 128> TileBig;
+typedef F16Tile<128, 64> TileSmall;
+
+namespace {
+
+// which tile shape a launch over these matrices takes: 2 = 256 x 128 when that gives at least three quarters of the CUs a
+// workgroup, else 1 = 128 x 64 on the same condition, else 0 (the launch stays on the int8 kernel)
+int f16_tile_kind(const DevWeight *ws, int count, int64_t n, int num_cus) {
+    int64_t big = 0, small = 0;
+    for (int i = 0; i < count; i++) {
+        big += (ws[i].M + TileBig::TM - 1) / TileBig::TM * ((n + TileBig::TN - 1) / TileBig::TN);
+        small += (ws[i].M + TileSmall::TM - 1) / TileSmall::TM * ((n + TileSmall::TN - 1) / TileSmall::TN);
+    }
+    if (4 * big >= 3 * (int64_t)num_cus) return 2;
+    if (4 * small >= 3 * (int64_t)num_cus) return 1;
+    return 0;
+}
+
+bool f16_shape_ok(const DevWeight &w, const DevAct &a) {
+    if (w.type != T_Q4_K || !a.qf || !a.bsf || w.K < QKK || w.K % QKK || w.M < 1 || a.N <= 64) return false;  // up to 64 rows: the 128 x 64 tiles of the int8 kernel
+    return (int64_t)a.N * w.K < ((int64_t)1 << 31) && w.M * (w.K / QKK * Q4_K_BYTES) < ((int64_t)1 << 32);  // 32-bit lane offsets
+}
+
+template <class T>
+hipError_t launch_tiles(const DevWeight *ws, float *const *ys, int count, const DevAct &a, hipStream_t s) {
+    F16Args fa;
+    int64_t tiles_m = 0;
+    for (int i = 0; i < F16_MULTI; i++) {
+        const int j = i < count ? i : count - 1;
+        fa.W[i] = ws[j].p0; fa.Y[i] = ys[j]; fa.M[i] = (int)ws[j].M;
+        if (i < count) tiles_m += (ws[i].M + T::TM - 1) / T::TM;
+        fa.tile_end[i] = i < count ? (int)tiles_m : 0x7fffffff;
+    }
+    const int64_t tiles_n = (a.N + T::TN - 1) / T::TN;
+    const int64_t grid = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
+    if (grid > 0x7fffffff || a.K > 0x7fffffff) return hipErrorInvalidValue;
+    gemm_f16_q4k_kernel<T><<<(unsigned)grid, 64 * T::WAVES, 0, s>>>(fa, reinterpret_cast<const uint8_t *>(a.qf), a.d,
+                                                                    reinterpret_cast<const uint8_t *>(a.bsf), a.N, (int)a.K, (int)tiles_m,
+                                                                    (int)tiles_n);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// The kernel pays where its tiles -- 256 x 128, or 128 x 64 for products with fewer outputs -- give (nearly) every CU a
+// workgroup; smaller products stay on the int8 kernel.  The choice depends on the weight and the batch only, never on
+// what else a call multiplies, so a product's bits do not depend on how it was asked for (both tile shapes and the
+// int8 kernel add a row's super-blocks in the same order with the same fp32 expressions).
 bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus) {
-    if (w.type != T_Q4_K || !a.qf || !a.bsf || w.K < QKK || w.K % QKK || a.N <= 64) return false;  // up to 64 rows: the 128 x 64 tiles of the int8 kernel
-    if ((int64_t)a.N * w.K >= ((int64_t)1 << 31) || w.M * (w.K / QKK * Q4_K_BYTES) >= ((int64_t)1 << 32)) return false;  // 32-bit lane offsets
-    const int64_t tiles = (w.M + TM - 1) / TM * ((a.N + TN - 1) / TN);
-    return 4 * tiles >= 3 * (int64_t)num_cus;
+    if (!f16_shape_ok(w, a)) return false;
+    const int kind = f16_tile_kind(&w, 1, a.N, num_cus);
+    // The small tiles only where the int8 kernel would not cut K: a long K with few tiles (4096 x 14336 at batch 512) is
+    // faster there in two K slices (96.6 against 101.3 us); without slices the small tiles win (5120 x 5120 at batch 512:
+    // 49.0 against 59.2 us, 8192 x 8192 at 384: 80.8 against 95.1, 4096 x 4096 at 1024: 54.4 against 59.7).
+    return kind == 2 || (kind == 1 && gemm_workspace_floats(w.type, w.K, w.M, a.N, num_cus) == 0);
 }
 
 // Several matrices in one launch: every matrix Q4_K of one K within the kernel's offset limits, together at least three
@@ -319,40 +379,28 @@ bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus) {
 // launch measured 137.5 against 143.7 us at batch 512 and 527 against 573 at batch 2048 (one launch gap less, and the
 // second matrix's tiles fill the CUs the first one's last round leaves idle).
 bool gemm_f16_multi_wanted(const DevWeight *ws, int count, const DevAct &a, int num_cus) {
-    if (count < 2 || count > F16_MULTI || !a.qf || !a.bsf || a.N <= 64) return false;
-    int64_t tiles = 0;
-    for (int i = 0; i < count; i++) {
-        const DevWeight &w = ws[i];
-        if (w.type != T_Q4_K || w.K != ws[0].K || w.K < QKK || w.K % QKK || w.M < 1) return false;
-        if ((int64_t)a.N * w.K >= ((int64_t)1 << 31) || w.M * (w.K / QKK * Q4_K_BYTES) >= ((int64_t)1 << 32)) return false;
-        tiles += (w.M + TM - 1) / TM * ((a.N + TN - 1) / TN);
-    }
-    return 4 * tiles >= 3 * (int64_t)num_cus;
+    if (count < 2 || count > F16_MULTI) return false;
+    for (int i = 0; i < count; i++)
+        if (!f16_shape_ok(ws[i], a) || ws[i].K != ws[0].K) return false;
+    const int kind = f16_tile_kind(ws, count, a.N, num_cus);
+    for (int i = 0; kind == 1 && i < count; i++)
+        if (gemm_workspace_floats(ws[i].type, ws[i].K, ws[i].M, a.N, num_cus) != 0) return false;
+    return kind != 0;
 }
 
-hipError_t launch_gemm_f16_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, hipStream_t s) {
+hipError_t launch_gemm_f16_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus, hipStream_t s) {
     if (count < 1 || count > F16_MULTI || a.type != T_Q8_K || !a.qf || !a.bsf || a.N < 1) return hipErrorInvalidValue;
-    F16Args fa;
-    int64_t tiles_m = 0;
-    for (int i = 0; i < F16_MULTI; i++) {
-        const int j = i < count ? i : count - 1;
-        if (ws[j].type != T_Q4_K || ws[j].K != a.K || !ys[j] || ws[j].M > 0x7fffffff || ws[j].M < 1) return hipErrorInvalidValue;
-        fa.W[i] = ws[j].p0; fa.Y[i] = ys[j]; fa.M[i] = (int)ws[j].M;
-        if (i < count) tiles_m += (ws[i].M + TM - 1) / TM;
-        fa.tile_end[i] = i < count ? (int)tiles_m : 0x7fffffff;
-    }
-    const int64_t tiles_n = (a.N + TN - 1) / TN;
-    const int64_t grid = tiles_n * ((tiles_m + 7) / 8 * 8);  // whole rounds of the 8 XCDs
-    if (grid > 0x7fffffff || a.K > 0x7fffffff) return hipErrorInvalidValue;
-    gemm_f16_q4k_kernel<<<(unsigned)grid, 512, 0, s>>>(fa, reinterpret_cast<const uint8_t *>(a.qf), a.d, reinterpret_cast<const uint8_t *>(a.bsf),
-                                                       a.N, (int)a.K, (int)tiles_m, (int)tiles_n);
-    return hipGetLastError();
+    for (int i = 0; i < count; i++)
+        if (ws[i].type != T_Q4_K || ws[i].K != a.K || !ys[i] || ws[i].M > 0x7fffffff || ws[i].M < 1) return hipErrorInvalidValue;
+    // (a caller that asks for this kernel on a product it is not wanted for gets the large tiles)
+    if (f16_tile_kind(ws, count, a.N, num_cus) == 1) return launch_tiles<TileSmall>(ws, ys, count, a, s);
+    return launch_tiles<TileBig>(ws, ys, count, a, s);
 }
 
-hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, hipStream_t s) {
+hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, int num_cus, hipStream_t s) {
     if (!y) return hipErrorInvalidValue;
     float *ys[1] = {y};
-    return launch_gemm_f16_multi(&w, ys, 1, a, s);
+    return launch_gemm_f16_multi(&w, ys, 1, a, num_cus, s);
 }
 
 }  // namespace miqmm

@@ -96,11 +96,11 @@ int gemm_max_multi();
 // kernel 3b: fp16-MFMA GEMM for Q4_K weights on products with enough 256 x 128 output tiles to fill the GPU;
 // a needs the fp16 planes (qf, bsf).  y[n*M + m].  gemm_f16_wanted() depends on the weight and the batch only.
 bool gemm_f16_wanted(const DevWeight &w, const DevAct &a, int num_cus);
-hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, hipStream_t s);
+hipError_t launch_gemm_f16(const DevWeight &w, const DevAct &a, float *y, int num_cus, hipStream_t s);
 // Up to four Q4_K matrices of one K in one launch of that kernel (q, k, v; gate, up): wanted when together they fill the
 // machine; the bits are those of the single launches.
 bool gemm_f16_multi_wanted(const DevWeight *ws, int count, const DevAct &a, int num_cus);
-hipError_t launch_gemm_f16_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, hipStream_t s);
+hipError_t launch_gemm_f16_multi(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int num_cus, hipStream_t s);
 // kernel 3c: int8-MFMA GEMM for Q6_K weights with 256 x 128 tiles and one accumulator per tile; y[n*M + m].
 // gemm_q6k_slices(): 0 = not the kernel for this product (too few tiles), else the K slices it is cut into;
 // more than one slice needs gemm_q6k_workspace_floats() floats of device workspace.
