@@ -430,11 +430,15 @@ def test_in_kernel_q8_K_quantizer_edge_blocks_give_the_same_bits(ctx, t):
 
 
 @pytest.mark.parametrize("t,k", [(Q4_K, 14336), (Q4_K, 8192), (Q6_K, 4352), (Q4_0, 4096), (Q8_0, 4096), (Q8_0, 2080),
-                                 (Q4_K, 5120), (Q6_K, 5120), (Q6_K, 14336), (Q4_0, 2560), (Q8_0, 5120)])
+                                 (Q4_K, 5120), (Q6_K, 5120), (Q6_K, 14336), (Q4_0, 2560), (Q8_0, 5120),
+                                 (Q4_K, 11008), (Q4_K, 8448), (Q6_K, 12544), (Q4_K, 16384), (Q6_K, 11008), (Q4_K, 28672)])
 def test_long_rows_at_one_column(ctx, t, k):
     """One column, rows of several K segments (the waves of a workgroup cut K and combine through LDS): same
     bits as the two-phase path, call after call; row counts that do not fill the last workgroup, four
-    weights in one launch, and the largest launch the f32 path takes (64 Ki rows)."""
+    weights in one launch, and the largest launch the f32 path takes (64 Ki rows).  The K-quant rows of three and four
+    segments take the kernel whose waves wait for the other waves of their segment only (a count in LDS instead of a
+    workgroup barrier) and whose last wave per row group adds the partial sums: last segments of one block (8448,
+    12544), of eleven (11008), full ones (16384); 28672 is seven segments and two rounds of quantization."""
     rng = np.random.default_rng(900 + t + k)
     ms = [1, 31, 32, 33, 700]
     raws = [_weights(t, m, k, seed=k + m + t) for m in ms]
