@@ -494,8 +494,16 @@ bool wants_skinny(int type, int64_t K, int64_t M, int64_t n, int num_cus) {
     // (two columns of a large Q4_K matrix with rows of one K segment: the deep direct-load kernel, 16.4 against 17.1 us
     // for gate + up)
     if (type == T_Q4_K && n == 2 && skinny_supports(type, K, M) && deep16_wanted(type, K, M, 2, num_cus)) return true;
+    if (type == T_Q6_K && n < 4 && skinny_supports(type, K, M) && deep6_wanted(type, K, M, (int)n, num_cus)) return true;
     const int64_t from = type == T_Q4_K ? 3 : 4;
     return n >= from && skinny_supports(type, K, M);
+}
+
+// One matrix at a few f32 columns on the deep direct-load kernel that quantizes x itself (Q6_K: unless the rows kernel is
+// the one for this matrix).
+bool deep_f32_one(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n) {
+    if (n > 8 || !deep16_f32_wanted(w->dev.type, w->dev.K, w->dev.M, (int)n, ctx->num_cus)) return false;
+    return !(w->dev.type == T_Q6_K && skinny_rows_wanted(w->dev, (int)n, ctx->num_cus));
 }
 
 // Which kernel a product takes (the values of the MI_QMM_ROUTE_* enum of mi_qmm.h).  Decided from the weight's type and
@@ -600,7 +608,7 @@ int route_f32(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n, int path
     const int64_t K = w->dev.K, M = w->dev.M;
     if (path != MI_QMM_PATH_GEMM && n <= 8 && !wants_skinny(w->dev.type, K, M, n, ctx->num_cus) && gemv_f32_supported(w->dev.type, K, M, (int)n))
         return MI_QMM_ROUTE_GEMV_F32;
-    if (path == MI_QMM_PATH_AUTO && n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) return MI_QMM_ROUTE_DEEP_F32;
+    if (path == MI_QMM_PATH_AUTO && deep_f32_one(ctx, w, n)) return MI_QMM_ROUTE_DEEP_F32;
     static const uint8_t some_plane = 0;  // (stands for "the planes are there": route_planes only asks whether)
     DevAct a;
     a.sd8 = mi_qmm_vec_dot_type(w->dev.type) == T_Q8_K ? &some_plane : nullptr;
@@ -706,7 +714,7 @@ int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *
         HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
         return MI_QMM_OK;
     }
-    if (n <= 8 && deep16_f32_wanted(w->dev.type, K, M, (int)n, ctx->num_cus)) {
+    if (deep_f32_one(ctx, w, n)) {
         float *ys[1] = {y};
         HIP_TRY(launch_deep16_f32(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
         return MI_QMM_OK;

@@ -1845,7 +1845,12 @@ int skinny_kind(const DevWeight &w, int ncols, int num_cus) {
         if (rows_q4k_wanted(w.type, w.K, w.M, ncols, num_cus)) return 3;
         return 4;
     }
-    return rows_wanted(w, ncols, num_cus) ? 5 : 4;
+#ifndef DEEP6_OVER_ROWS
+#define DEEP6_OVER_ROWS 0
+#endif
+    const bool rows = rows_wanted(w, ncols, num_cus);
+    if ((!rows || DEEP6_OVER_ROWS) && deep6_wanted(w.type, w.K, w.M, ncols, num_cus)) return 1;
+    return rows ? 5 : 4;
 }
 
 hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y, int num_cus, hipStream_t s) {
@@ -1856,6 +1861,7 @@ hipError_t launch_skinny(const DevWeight &w, const DevAct &a, int col0, int ncol
     const SkinnyIds none{};
     const int64_t rg = (w.M + 15) / 16;
     const int kind = skinny_kind(w, ncols, num_cus);
+    if (kind == 1 && w.type == T_Q6_K) return launch_deep6(w, y, a, col0, ncols, num_cus, s);
     if (kind == 1) return launch_deep16(&w, &y, 1, a, col0, ncols, num_cus, s);
     if (w.type == T_Q4_K) {
         if (kind == 2) launch_direct16(&w, &y, 1, a, col0, ncols, num_cus, s);
@@ -1884,7 +1890,7 @@ int skinny_multi_kind(const DevWeight *ws, int count, int ncols, int num_cus) {
         if (ws[i].type != ws[0].type || ws[i].K != ws[0].K || !skinny_supports(ws[i].type, ws[i].K, ws[i].M)) return 0;
         total_m += ws[i].M;
         const bool dir = direct16_wanted(ws[i].type, ws[i].K, ws[i].M, ncols);
-        const bool deep = deep16_wanted(ws[i].type, ws[i].K, ws[i].M, ncols, num_cus);
+        const bool deep = deep16_wanted(ws[i].type, ws[i].K, ws[i].M, ncols, num_cus) || deep6_wanted(ws[i].type, ws[i].K, ws[i].M, ncols, num_cus);
         each_deep = each_deep && deep;
         none_deep = none_deep && !deep;
         each_direct = each_direct && dir;
@@ -1893,7 +1899,7 @@ int skinny_multi_kind(const DevWeight *ws, int count, int ncols, int num_cus) {
     }
     if ((total_m + 15 * count) / 16 >= 0x7fffffff) return 0;
     // the deep direct-load kernel: its order of sums does not depend on the launch
-    if (each_deep && deep16_wanted(ws[0].type, ws[0].K, total_m, ncols, num_cus)) return 4;
+    if (each_deep && ws[0].type == T_Q4_K && deep16_wanted(ws[0].type, ws[0].K, total_m, ncols, num_cus)) return 4;
     if (!none_deep) return 0;  // (a matrix that takes the deep kernel alone joins no launch of another kernel)
     if (each_direct && direct16_wanted(ws[0].type, ws[0].K, total_m, ncols)) return 1;
     // the rows kernel (it reproduces the K cut each matrix would get alone, see skinny_rows_q4k_kernel)

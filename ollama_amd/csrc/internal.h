@@ -127,6 +127,10 @@ hipError_t launch_skinny_multi(const DevWeight *ws, float *const *ys, int count,
 // pieces of four super-blocks in flight per wave, activations resident in LDS.  Up to four matrices of one K per
 // launch; the order of the floating-point sums does not depend on the launch geometry.
 bool deep16_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus);
+// The same kernel shape for one Q6_K matrix at 3..8 columns (quantized planes with sd16; launch_deep16_f32 takes a
+// single Q6_K matrix too, where deep16_f32_wanted says so).
+bool deep6_wanted(int type, int64_t K, int64_t M, int ncols, int num_cus);
+hipError_t launch_deep6(const DevWeight &w, float *y, const DevAct &a, int col0, int ncols, int num_cus, hipStream_t s);
 hipError_t launch_deep16(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols, int num_cus,
                          hipStream_t s);
 // the same from f32 activations x [ncols][K] (device), quantized by the kernel's workgroups themselves: one launch per

@@ -1,4 +1,4 @@
-// Q4_K products at a few activation columns (3..8) on large matrices: the bandwidth-bound shape of
+// Q4_K and (second half of the file) Q6_K products at a few activation columns (2..8) on large matrices: the bandwidth-bound shape of
 // several sequences decoding together -- Tensor.Mulmat (/root/reference/ml/backend.go:151) on the
 // feed-forward matrices of a layer with a handful of tokens in flight.
 //
@@ -515,6 +515,436 @@ hipError_t launch_deep16_any(const DevWeight *ws, float *const *ys, int count, c
 
 }  // namespace
 
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The same kernel shape for Q6_K (the down projection and the value projection of the common mixed files).
+//
+//   * Weights: the planes of formats.h.  Per super-block a lane (row, j) of a 16-row group loads the 16-byte pieces j
+//     and 4 + j of the row's 128 low-nibble bytes, piece j of its 64 bytes of high bit pairs and dword j of its 16
+//     scales -- the quad reads runs of its row -- and, in the matrix cores' lane order, the row's fp16 scale.
+//   * Arithmetic: the 6-bit quants go into v_mfma_i32_16x16x64_i8 as they are stored, 0..63; the offset of 32 is
+//     taken out with the block sums: sum (q - 32) y = sum q y - 32 sum y.  A chunk of 64 elements is one MFMA whose
+//     four K groups are four scale groups of 16, so the 16 rows of the A operand are 4 columns x 4 K groups (row
+//     4 c + w is column c restricted to K group w) and one MFMA serves four activation columns; five to eight columns
+//     take a second set of MFMAs on the same weight operand.  In chunk ch lane (row, kg) multiplies elements
+//     64 ch + 16 kg ..: low (ch even) or high nibbles of piece 4 (ch / 2) + kg of the low-nibble bytes, and of piece
+//     2 (ch / 2) + (kg & 1) of the bit pairs the pair at bit 4 (ch & 1) + 2 (kg / 2).  A lane is left with the
+//     partial sums of column kg (and 4 + kg) with the 16 scale groups and applies the int8 scales with
+//     v_mad_i32_i24; sum scale x block sum comes from one more MFMA on the block-sum digits.  All integer sums exact.
+//   * One matrix per launch, activations from the quantized planes.
+//
+// Order of the floating-point sums: as above (pieces of four super-blocks in order, piece sums in order).
+constexpr int Q6_QL = 128, Q6_QH = 64, Q6_SC = 16;
+#ifndef DEEP6_FROM_N
+#define DEEP6_FROM_N 3
+#endif
+constexpr int DEEP6_FROM = DEEP6_FROM_N;  // activation columns from which the kernel is taken
+struct Deep6Args {
+    const uint8_t *ql, *qh, *sc;
+    const uint16_t *d;
+    float *y;
+    int64_t M;
+    int groups_total, nsb;
+};
+// LDS map for 4 * SETS activation columns.  512 zero bytes; per super-block and column 256 bytes of quants in
+// 16-byte pieces, piece p of column c at slot p ^ (c & 2); per (super-block, column) 32 bytes of block-sum digits (the
+// low digits of the 16 sums, then the high digits) and the fp32 block scale; then the piece sums.
+//
+// The slot swizzle: ds_read_b128 serves 16 lanes per cycle, and the lanes of one such group that read real data
+// are A rows (c, w) = (0, w0) (3, w0) (1, w0 + 1) (2, w0 + 1) or (1, w0) (2, w0) (0, w0 + 1) (3, w0 + 1), w0 = 0 or 2:
+// with slots w ^ (c & 2) the four fall on the four slots of the chunk's aligned block of four; the lanes that read
+// zeros read one address in the next block of four.
+template <int SETS>
+struct Deep6Geo {
+    static constexpr int NC = 4 * SETS;
+    static constexpr int A_OFF = 512;
+    static __host__ __device__ constexpr int dg_off(int nsb) { return A_OFF + nsb * NC * 256; }
+    static __host__ __device__ constexpr int y_off(int nsb) { return dg_off(nsb) + nsb * NC * 32; }
+    static __host__ __device__ constexpr int part_off(int nsb) { return (y_off(nsb) + nsb * NC * 4 + 255) / 256 * 256; }
+    static __host__ __device__ constexpr size_t lds_bytes(int nsb, int slots, int npieces, bool shared_groups) {
+        return (size_t)part_off(nsb) + (shared_groups ? (size_t)slots * npieces * NC * 16 * 4 : 0);
+    }
+};
+struct Piece6Regs { unsigned sc[PIECE], d[PIECE]; u4v qa[PIECE], qb[PIECE], qh[PIECE]; };
+
+// XF32: f32 activations xf [nc][K], quantized by the workgroup itself (as in the Q4_K kernel above).
+template <bool SHARED, int SETS, bool XF32>
+__global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g, DevAct a, const float *__restrict__ xf, int col0, int nc,
+                                                                    DeepCut cut) {
+    typedef Deep6Geo<SETS> Geo;
+    constexpr int NC = Geo::NC;
+    extern __shared__ __attribute__((aligned(256))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nsb = g.nsb, npieces = (nsb + PIECE - 1) / PIECE;
+    const int slot = (wave * cut.inv_wpg) >> 8, sub = wave - slot * cut.wpg;
+    const int p_begin = sub * cut.ppw, p_end = min(npieces, p_begin + cut.ppw);
+    const unsigned sm = lds_addr(smem);
+    const int bid = blockIdx.x;
+    const int group_step = cut.slots * cut.grid;
+    const int group0 = slot * cut.grid + bid;
+
+    // ---- 1. the activations, requested first: quants, block-sum digits, block scales -> LDS
+    const int nblk = nc * nsb;  // Q8_K blocks of the launch's columns; block b = column b / nsb, super-block b % nsb
+    const float4 *x4 = reinterpret_cast<const float4 *>(xf) + (int64_t)col0 * nsb * 64;
+    constexpr int XR = 3;  // rounds of four blocks per wave requested here, ahead of the weights
+    float4 xq[XR][4];
+    if (XF32) {
+#pragma unroll
+        for (int t = 0; t < XR; t++) {
+            if (4 * (wave + t * cut.W) < nblk) {  // wave-uniform
+                const int b = min(4 * (wave + t * cut.W) + (lane >> 4), nblk - 1);
+#pragma unroll
+                for (int j = 0; j < 4; j++) xq[t][j] = x4[b * 64 + 4 * (lane & 15) + j];
+            }
+        }
+    } else {
+        auto acol = [&](int i) { return col0 + min(i, nc - 1); };
+        const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
+        // copy instructions are dealt out to the waves in turn: the quants (one instruction per super-block and set of
+        // four columns), the digits (32 (super-block, column) cells per instruction), the scales (64 cells)
+        const int cells = nsb * NC, n_q = nsb * SETS, n_g = (cells + 31) / 32, n_c = (cells + 63) / 64;
+        for (int n = wave; n < n_q + n_g + n_c; n += cut.W) {
+            if (n < n_q) {
+                const int sb = n / SETS, j = n % SETS;
+                const int col = 4 * j + (lane >> 4), pc = (lane & 15) ^ (col & 2);
+                dma_lds<16>(aq + (int64_t)sb * QKK, (unsigned)acol(col) * (unsigned)a.K + 16u * pc,
+                            sm + Geo::A_OFF + (unsigned)(sb * NC + 4 * j) * 256u);
+            } else if (n < n_q + n_g) {
+                const int c0 = 32 * (n - n_q);
+                const int cell = min(c0 + (lane >> 1), cells - 1), sb = cell / NC, col = cell % NC;
+                const unsigned at = (unsigned)acol(col) * (unsigned)nsb + (unsigned)sb;
+                if (c0 + (lane >> 1) < cells) dma_lds<16>(a.sd16, at * 32u + 16u * (lane & 1), sm + Geo::dg_off(nsb) + 32u * c0);
+            } else {
+                const int c0 = 64 * (n - n_q - n_g);
+                const int cell = min(c0 + lane, cells - 1), sb = cell / NC, col = cell % NC;
+                const unsigned at = (unsigned)acol(col) * (unsigned)nsb + (unsigned)sb;
+                if (c0 + lane < cells) dma_lds<4>(reinterpret_cast<const uint8_t *>(a.d), at * 4u, sm + Geo::y_off(nsb) + 4u * c0);
+            }
+        }
+    }
+    if (tid < 128) *reinterpret_cast<int *>(smem + 4 * tid) = 0;  // the zero block
+
+    // ---- 2. the weight stream: a ring of four super-blocks per lane
+    // loading lane: its row and which piece of the quad's run it takes (rows 8..15 in the order 2 3 0 1, so that the
+    // sources 4 r + p of rows r and r + 8 do not share a bank of the ds_bpermute crossbar)
+    const int lrow = lane >> 2, lq = (lane & 3) ^ ((lane >> 4) & 2);
+    const int r = lane & 15, kg = lane >> 4;  // MFMA order: the lane's weight row (= A row) and K group
+    struct ItemAt { int64_t blk0; unsigned o_ql, o_qh, o_sc, o_d; };  // first block of the group's first row; lane offsets
+    auto item_at = [&](int group) __attribute__((always_inline)) {
+        const int64_t m0 = (int64_t)group * 16;
+        const int rows_left = (int)min((int64_t)16, g.M - m0);  // rows past M: the last row again, results dropped
+        ItemAt ia;
+        ia.blk0 = m0 * nsb;
+        const unsigned lb = (unsigned)(min(lrow, rows_left - 1) * nsb);
+        ia.o_ql = lb * Q6_QL + 16u * lq;
+        ia.o_qh = lb * Q6_QH + 16u * lq;
+        ia.o_sc = lb * Q6_SC + 4u * lq;
+        ia.o_d = (unsigned)(min(r, rows_left - 1) * nsb) * 2u;
+        return ia;
+    };
+    auto uniform = [](const void *p) __attribute__((always_inline)) {
+        const unsigned long long v = (unsigned long long)p;
+        return (gbytes_t)(((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
+                          (unsigned)__builtin_amdgcn_readfirstlane((int)v));
+    };
+    Piece6Regs R;
+    auto load_slot = [&](const ItemAt &ia, int piece, int i) __attribute__((always_inline)) {
+        const int64_t blk = ia.blk0 + min(piece * PIECE + i, nsb - 1);  // past the row's end: the last super-block again
+        gbytes_t pl = uniform(g.ql + blk * Q6_QL), ph = uniform(g.qh + blk * Q6_QH), ps = uniform(g.sc + blk * Q6_SC),
+                 pd = uniform(g.d + blk);
+        R.sc[i] = *(const __attribute__((address_space(1))) unsigned *)(ps + ia.o_sc);
+        R.d[i] = *(const __attribute__((address_space(1))) unsigned short *)(pd + ia.o_d);
+        R.qa[i] = *(gu4_t)(pl + ia.o_ql);
+        R.qh[i] = *(gu4_t)(ph + ia.o_qh);
+        R.qb[i] = *(gu4_t)(pl + (ia.o_ql + 64u));
+    };
+    int lgroup = min(group0, g.groups_total - 1), lp = p_begin;
+    ItemAt L = item_at(lgroup);
+    // the copies first; one super-block of weights per wave behind them; the rest of the ring when the activations
+    // have landed (requests are served roughly in the order they were made)
+    load_slot(L, lp, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (XF32) {
+        auto quantize_four = [&](int b0, const float4 (&v)[4]) __attribute__((always_inline)) {
+            const int b = b0 + (lane >> 4), sub16 = lane & 15;
+            float dd;
+            int sum16, pair;
+            const uint4 packed = q8_K_quantize_row16(v, lane, dd, sum16, pair);
+            if (b < nblk) {  // the last four may end early: whole rows of 16 lanes drop out
+                const int col = (b * cut.inv_nsb) >> 16, sb = b - col * nsb, cell = sb * NC + col;
+                *reinterpret_cast<uint4 *>(smem + Geo::A_OFF + cell * 256 + 16 * (sub16 ^ (col & 2))) = packed;
+                // the sum of the lane's 16 quants as two digits, S = 64 * (S >> 6) + (S & 63)
+                smem[Geo::dg_off(nsb) + cell * 32 + sub16] = (uint8_t)(sum16 & 63);
+                smem[Geo::dg_off(nsb) + cell * 32 + 16 + sub16] = (uint8_t)(sum16 >> 6);
+                if (sub16 == 0) *reinterpret_cast<float *>(smem + Geo::y_off(nsb) + cell * 4) = dd;
+            }
+        };
+#pragma unroll
+        for (int t = 0; t < XR; t++)
+            if (4 * (wave + t * cut.W) < nblk) quantize_four(4 * (wave + t * cut.W), xq[t]);
+        for (int b0 = 4 * (wave + XR * cut.W); b0 < nblk; b0 += 4 * cut.W) {  // (more rounds than were requested ahead)
+            float4 v[4];
+            const int bc = min(b0 + (lane >> 4), nblk - 1);
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = x4[bc * 64 + 4 * (lane & 15) + j];
+            quantize_four(b0, v);
+        }
+        // columns past nc of the last set keep what the LDS held: they are multiplied and dropped
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the LDS writes, before the barrier
+    } else {
+        asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");  // (loads retire in order: all but the five weight loads)
+    }
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 1; i < PIECE; i++) {
+        load_slot(L, lp, i);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- 3. operand reads: per-lane LDS addresses and per-super-block strides (0 for lanes that read zeros)
+    const int rsw = (r >> 3) << 1;
+    const int bidx = 4 * (4 * r + (kg ^ rsw));              // low-nibble pieces: piece kg of either half
+    const int bidx_h0 = 4 * (4 * r + ((kg & 1) ^ rsw));     // bit pairs of the first half: piece kg & 1
+    const int bidx_h1 = 4 * (4 * r + ((2 + (kg & 1)) ^ rsw));  // of the second half: piece 2 + (kg & 1)
+    const unsigned lsh = 2 * (kg >> 1);
+    unsigned a_at[SETS], a_st, d_at, d_st, y_at;
+    {
+        const int c = r >> 2, w = r & 3;  // A row r: column c of a set, K group w
+        const bool a_on = kg == w;
+#pragma unroll
+        for (int s = 0; s < SETS; s++) a_at[s] = sm + (a_on ? Geo::A_OFF + (4 * s + c) * 256 + 16 * (w ^ (c & 2)) : 64);
+        a_st = a_on ? NC * 256 : 0;
+        // block-sum digits: A row 4 c' + 2 s + digit is column 4 s + c' (so that a lane's outputs belong to its columns)
+        const int dc = 4 * ((r >> 1) & 1) + (r >> 2), dig = r & 1;
+        const bool d_on = kg == 0 && dc < NC;
+        d_at = sm + (d_on ? Geo::dg_off(nsb) + dc * 32 + 16 * dig : 0);
+        d_st = d_on ? NC * 32 : 0;
+        y_at = sm + Geo::y_off(nsb) + 4 * kg;  // columns kg (and 4 + kg)
+    }
+    float *part = reinterpret_cast<float *>(smem + Geo::part_off(nsb));  // [slot][piece][NC][16]
+
+    const v4i zero = {0, 0, 0, 0};
+    auto mul_slot = [&](int i, int sb, const unsigned (&aa)[SETS], unsigned da, float (&acc)[SETS]) __attribute__((always_inline)) {
+        const v4i dg = lds_at<v4i>(da, 0);
+        float yd[SETS];
+#pragma unroll
+        for (int s = 0; s < SETS; s++) yd[s] = lds_at<float>(y_at + (unsigned)sb * (NC * 4), 16 * s);
+        v4i scv;  // the row's 16 scales, from the four lanes of the quad that loaded them
+#pragma unroll
+        for (int j = 0; j < 4; j++) scv[j] = __builtin_amdgcn_ds_bpermute(4 * (4 * r) + 4 * (j ^ rsw), (int)R.sc[i]);
+        const float d = h2f(R.d[i]);
+        auto mad = [](int a_, int b_, int c_) {
+            int o = __mul24(a_, b_) + c_;
+            asm("" : "+v"(o));
+            return o;
+        };
+        int isum[SETS];
+        // scale x block sum: K group 0 of the A operand holds a digit of the 16 sums, the B operand the 16 scales (what
+        // the other K groups of B hold is multiplied by zeros)
+        const v4i x = mfma16(dg, scv, zero);
+        // one chunk: the weight operand from low-nibble bytes lo4 (already shifted and masked) and bit pairs hi (in place)
+        auto chunk = [&](int ch, u4v lo4, u4v hi, bool first) __attribute__((always_inline)) {
+            v4i b;
+#pragma unroll
+            for (int k = 0; k < 4; k++) b[k] = (int)(lo4[k] | (hi[k] & 0x30303030u));
+#pragma unroll
+            for (int s = 0; s < SETS; s++) {
+                const v4i av = lds_at<v4i>(aa[s], 64 * ch);
+                const v4i D = mfma16(av, b, zero);
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const int g16 = 4 * ch + w;
+                    const int scale = __builtin_amdgcn_sbfe(scv[g16 >> 2], 8 * (g16 & 3), 8);
+                    isum[s] = first && w == 0 ? __mul24(scale, D[w]) : mad(scale, D[w], isum[s]);
+                }
+            }
+        };
+        auto lo_nib = [](u4v q) { return (u4v){q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu, q.z & 0x0f0f0f0fu, q.w & 0x0f0f0f0fu}; };
+        auto hi_nib = [](u4v q) { return (u4v){(q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu, (q.z >> 4) & 0x0f0f0f0fu, (q.w >> 4) & 0x0f0f0f0fu}; };
+        {
+            const u4v qa = bperm(bidx, R.qa[i]);
+            u4v t = bperm(bidx_h0, R.qh[i]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) t[k] >>= lsh;
+            chunk(0, lo_nib(qa), (u4v){t.x << 4, t.y << 4, t.z << 4, t.w << 4}, true);
+            chunk(1, hi_nib(qa), t, false);
+        }
+        {
+            const u4v qb = bperm(bidx, R.qb[i]);
+            u4v t = bperm(bidx_h1, R.qh[i]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) t[k] >>= lsh;
+            chunk(2, lo_nib(qb), (u4v){t.x << 4, t.y << 4, t.z << 4, t.w << 4}, false);
+            chunk(3, hi_nib(qb), t, false);
+        }
+#pragma unroll
+        for (int s = 0; s < SETS; s++) {
+            const int corr = (x[2 * s + 1] << 6) + x[2 * s];  // sum over the 16 groups of scale x block sum
+            acc[s] = __builtin_fmaf(d * yd[s], (float)(isum[s] - (corr << 5)), acc[s]);
+        }
+    };
+
+    // ---- 4. the pieces in order (the last piece apart, without requests: no request in the loop is conditional)
+    const int np = max(p_end - p_begin, 0);
+    int items = 0;
+    if (np > 0 && group0 < g.groups_total) items = group0 + (cut.iters - 1) * group_step < g.groups_total ? cut.iters : cut.iters - 1;
+    const int n_total = items * np;
+    int ck = 0, cp = p_begin;
+    float total[SETS];
+#pragma unroll
+    for (int s = 0; s < SETS; s++) total[s] = 0.f;
+    auto sum_shared = [&](int k) __attribute__((always_inline)) {
+        __syncthreads();
+        const int group = group0 + k * group_step;
+        if (sub == 0 && group < g.groups_total) {
+            const int64_t m0 = (int64_t)group * 16;
+            for (int o = lane; o < NC * 16; o += 64) {
+                const int col = o >> 4, row = o & 15;
+                float sum = 0.f;
+                for (int p = 0; p < npieces; p++) sum += part[((slot * npieces + p) * NC + col) * 16 + row];
+                if (col < nc && m0 + row < g.M) g.y[(int64_t)(col0 + col) * g.M + m0 + row] = sum;
+            }
+        }
+        if (k + 1 < cut.iters) __syncthreads();
+    };
+    auto one_piece = [&](auto refill_tag) __attribute__((always_inline)) {
+        constexpr bool REFILL = decltype(refill_tag)::value;
+        if (REFILL) {
+            if (lp + 1 < p_end) lp++;
+            else {
+                lp = p_begin;
+                lgroup += group_step;
+                L = item_at(min(lgroup, g.groups_total - 1));
+            }
+        }
+        float acc[SETS];
+        unsigned aa[SETS], da = d_at + (unsigned)(cp * PIECE) * d_st;
+#pragma unroll
+        for (int s = 0; s < SETS; s++) {
+            acc[s] = 0.f;
+            aa[s] = a_at[s] + (unsigned)(cp * PIECE) * a_st;
+        }
+#pragma unroll
+        for (int i = 0; i < PIECE; i++) {
+            if (cp * PIECE + i < nsb) mul_slot(i, cp * PIECE + i, aa, da, acc);  // wave-uniform
+#pragma unroll
+            for (int s = 0; s < SETS; s++) aa[s] += a_st;
+            da += d_st;
+            if (REFILL) load_slot(L, lp, i);
+        }
+        const bool item_done = cp + 1 == p_end;
+        if (!SHARED) {
+#pragma unroll
+            for (int s = 0; s < SETS; s++) total[s] += acc[s];
+            if (item_done) {  // the row group is complete: lane (r, kg) holds row r of columns kg and 4 + kg
+                const int64_t m0 = (int64_t)(group0 + ck * group_step) * 16;
+#pragma unroll
+                for (int s = 0; s < SETS; s++) {
+                    const int col = 4 * s + kg;
+                    if (col < nc && m0 + r < g.M) g.y[(int64_t)(col0 + col) * g.M + m0 + r] = total[s];
+                    total[s] = 0.f;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < SETS; s++) part[((slot * npieces + cp) * NC + 4 * s + kg) * 16 + r] = acc[s];
+            if (item_done) sum_shared(ck);
+        }
+        if (item_done) {
+            ck++;
+            cp = p_begin;
+        } else {
+            cp++;
+        }
+    };
+#pragma unroll 1
+    for (int f = 0; f + 1 < n_total; f++) one_piece(std::true_type{});
+    if (n_total > 0) one_piece(std::false_type{});
+    if (SHARED) {
+#pragma unroll 1
+        for (int k = items; k < cut.iters; k++) sum_shared(k);
+    }
+}
+
+bool deep6_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, size_t &lds) {
+    if (K % QKK || ncols < 1 || ncols > 8 || groups < 1 || groups > 0x7fffffff || num_cus < 1) return false;
+    const int nsb = (int)(K / QKK), npieces = (nsb + PIECE - 1) / PIECE;
+    const int64_t per_cu = (groups + num_cus - 1) / num_cus;
+    int wpg = per_cu >= MAX_WAVES ? 1 : (int)(MAX_WAVES / per_cu);
+    if (wpg > npieces) wpg = npieces;
+    c.ppw = (npieces + wpg - 1) / wpg;
+    c.wpg = (npieces + c.ppw - 1) / c.ppw;
+    c.inv_wpg = (256 + c.wpg - 1) / c.wpg;
+    c.slots = MAX_WAVES / c.wpg;
+    if (c.slots > per_cu) c.slots = (int)per_cu;
+    c.W = c.slots * c.wpg;
+    c.grid = (int)std::min<int64_t>(num_cus, (groups + c.slots - 1) / c.slots);
+    c.iters = (int)((groups + (int64_t)c.slots * c.grid - 1) / ((int64_t)c.slots * c.grid));
+    for (int wv = 0; wv < c.W; wv++)
+        if (((wv * c.inv_wpg) >> 8) != wv / c.wpg) return false;
+    c.inv_nsb = (65536 + nsb - 1) / nsb;
+    for (int b = 0; b < 8 * nsb; b++)
+        if (((b * c.inv_nsb) >> 16) != b / nsb) return false;
+    lds = ncols <= 4 ? Deep6Geo<1>::lds_bytes(nsb, c.slots, npieces, c.wpg > 1) : Deep6Geo<2>::lds_bytes(nsb, c.slots, npieces, c.wpg > 1);
+    return lds <= 160 * 1024;
+}
+
+}  // namespace
+
+bool deep6_wanted(int type, int64_t K, int64_t M, int ncols, int num_cus) {
+    if (type != T_Q6_K || ncols < DEEP6_FROM || ncols > 8) return false;
+    DeepCut c;
+    size_t lds;
+    if (!deep6_cut(K, (M + 15) / 16, ncols, num_cus, c, lds)) return false;
+    if (M * (K / QKK) * (int64_t)Q6_QL >= ((int64_t)1 << 32)) return false;  // 32-bit lane offsets into the planes
+    return M * K > ((int64_t)40 << 20);
+}
+
+namespace {
+
+hipError_t launch_deep6_any(const DevWeight &w, float *y, const DevAct *a, const float *xf, int col0, int ncols, int num_cus, hipStream_t s) {
+    if (w.type != T_Q6_K || ncols < 1 || ncols > 8) return hipErrorInvalidValue;
+    Deep6Args g{w.p0, w.p1, w.p2, w.d, y, w.M, 0, (int)(w.K / QKK)};
+    const int64_t rg = (w.M + 15) / 16;
+    g.groups_total = (int)rg;
+    DeepCut c;
+    size_t lds;
+    if (!deep6_cut(w.K, rg, ncols, num_cus, c, lds)) return hipErrorInvalidValue;
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+#define DEEP_ALLOW(SHARED, SETS, XF32) \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(deep16_q6k_kernel<SHARED, SETS, XF32>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        DEEP_ALLOW(false, 1, false); DEEP_ALLOW(true, 1, false); DEEP_ALLOW(false, 2, false); DEEP_ALLOW(true, 2, false);
+        DEEP_ALLOW(false, 1, true); DEEP_ALLOW(true, 1, true); DEEP_ALLOW(false, 2, true); DEEP_ALLOW(true, 2, true);
+#undef DEEP_ALLOW
+        allowed[dev] = true;
+    }
+    const DevAct none{};
+    const DevAct &da = a ? *a : none;
+    const dim3 grid((unsigned)c.grid), block(64 * c.W);
+#define DEEP_GO(SHARED, SETS) \
+    do { \
+        if (xf) deep16_q6k_kernel<SHARED, SETS, true><<<grid, block, lds, s>>>(g, da, xf, col0, ncols, c); \
+        else deep16_q6k_kernel<SHARED, SETS, false><<<grid, block, lds, s>>>(g, da, nullptr, col0, ncols, c); \
+    } while (0)
+    if (ncols <= 4) {
+        if (c.wpg == 1) DEEP_GO(false, 1); else DEEP_GO(true, 1);
+    } else {
+        if (c.wpg == 1) DEEP_GO(false, 2); else DEEP_GO(true, 2);
+    }
+#undef DEEP_GO
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_deep6(const DevWeight &w, float *y, const DevAct &a, int col0, int ncols, int num_cus, hipStream_t s) {
+    if (a.type != T_Q8_K || a.K != w.K || !a.sd16) return hipErrorInvalidValue;
+    return launch_deep6_any(w, y, &a, nullptr, col0, ncols, num_cus, s);
+}
+
 hipError_t launch_deep16(const DevWeight *ws, float *const *ys, int count, const DevAct &a, int col0, int ncols, int num_cus,
                          hipStream_t s) {
     return launch_deep16_any(ws, ys, count, &a, nullptr, col0, ncols, num_cus, s);
@@ -525,6 +955,14 @@ hipError_t launch_deep16(const DevWeight *ws, float *const *ys, int count, const
 // of a short K: up to three rounds of four blocks per wave, the rounds a wave requests ahead of its first weights.  (A
 // fourth round -- four columns of K = 14336 -- measured 14.7 us against 13.5 for quantize-then-multiply.)
 bool deep16_f32_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus) {
+    if (type == T_Q6_K) {
+        // one matrix per launch (total_m is that matrix's rows) and up to two rounds: three columns of K = 14336 measured
+        // 15.8 us in three rounds against 15.4 for quantize-then-multiply
+        DeepCut c;
+        size_t lds;
+        return deep6_wanted(type, K, total_m, ncols, num_cus) && deep6_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds) &&
+               (int64_t)ncols * (K / QKK) <= 2 * 4 * c.W;
+    }
     if (!deep16_wanted(type, K, total_m, ncols, num_cus)) return false;
     DeepCut c;
     size_t lds;
@@ -533,6 +971,7 @@ bool deep16_f32_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_
 }
 hipError_t launch_deep16_f32(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols, int num_cus, hipStream_t s) {
     if (!x) return hipErrorInvalidValue;
+    if (ws[0].type == T_Q6_K) return count == 1 ? launch_deep6_any(ws[0], ys[0], nullptr, x, 0, ncols, num_cus, s) : hipErrorInvalidValue;
     return launch_deep16_any(ws, ys, count, nullptr, x, 0, ncols, num_cus, s);
 }
 

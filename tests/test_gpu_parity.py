@@ -366,6 +366,43 @@ def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
         W.free()
 
 
+@pytest.mark.parametrize("m,k,ns", [(4096, 14336, (3, 4, 5, 8)), (14336, 4096, (3, 6, 8)), (14330, 4096, (4, 7)), (4100, 14336 + 256, (5,)),
+                                    (8192, 8192, (4, 8)), (40000, 2048, (4, 5)), (65536 + 48, 1024, (3, 8))])
+def test_q6k_deep_kernel_few_columns_on_large_matrices(ctx, m, k, ns):
+    """Q6_K at 3..8 columns on matrices beyond 40 M weights: the direct-load kernel on the Q6_K planes (low-nibble bytes,
+    bit pairs, scales and row scales each loaded by the quad of lanes of a row, ds_bpermute into the MFMA operand order,
+    the 6-bit quants multiplied as stored and the offset of 32 taken out with the block sums; one set of MFMAs up to
+    four columns, two from five).  Waves sharing a row group fourteen and four ways (down, gate shape), row groups of
+    their own (40000 and 65584 rows), a last piece of one super-block (K = 14592), ragged last row groups, blocks of
+    random bytes.  Against the
+    oracle and exact arithmetic; the f32 form (which quantizes in the kernel where that is two rounds at most) gives the
+    bits of quantize-then-multiply; a column's result does not depend on which other columns ride along."""
+    rng = np.random.default_rng(9300 + m + k)
+    raw = _weights(Q6_K, m, k, seed=9301 + m)
+    if m == 14336:      # blocks of random bytes: every pattern of nibbles, bit pairs and signed scales
+        nb = m * k // 256
+        raw = rng.integers(0, 256, (nb, 210), dtype=np.uint8)
+        raw[:, 208:210] = np.abs(rng.standard_normal(nb) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
+        raw = raw.reshape(m, -1)
+    W = ctx.upload(Q6_K, raw, k, m)
+    act = ctx.act_create(Q8_K, k, 8)
+    for n in ns:
+        assert ctx.route(W, n) in ("skinny_deep", "deep_f32"), (m, k, n)
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        x[0, :256] = 0.0                                               # an all-zero block
+        y = ctx.mulmat(W, x)
+        ctx.act_quantize(act, x)
+        rows = min(m, 6000)                                           # (the oracle on a slab of rows: the last ones)
+        want = oracle.mul_mat(Q6_K, np.ascontiguousarray(raw[-rows:]), k, rows, x, nthreads=16)
+        assert npref.rel_err(y[:, -rows:], want) < TOL, (m, n)
+        _check_against_exact_arithmetic(Q6_K, raw, k, m, x, y, f"Q6_K {m}x{k} n={n}", max_rows=2048)
+        assert ctx.route_q8(W, act) == "skinny_deep"
+        assert np.array_equal(ctx.mulmat_q8(W, act), y), ("f32 != planes", m, n)
+        assert np.array_equal(ctx.mulmat(W, x[::-1].copy())[::-1], y), n
+    act.free()
+    W.free()
+
+
 @pytest.mark.parametrize("t", WTYPES)
 def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
     """For n <= 8 the f32 entry points quantize x inside the GEMV's prologue.  The result must be
@@ -1125,9 +1162,8 @@ def test_skinny_kquants_match_oracle(ctx, t, m, k, n):
 def test_q6k_many_rows_few_columns(ctx, m, k, n):
     """Q6_K with 65536 rows and more, K of 2048 or 4096 and 3..8 columns (the output head at a few tokens) takes a
     kernel of its own: activations resident in LDS, a row group's scales fetched in whole lines.  Ragged last row
-    group, both K sizes, every column set partly filled; a column's bits do not depend on the others; from four
-    columns up the same matrix cut below 65536 rows goes through the general kernel and gives the same bits for the
-    rows they share."""
+    group, both K sizes, every column set partly filled; a column's bits do not depend on the others, and are those
+    the general kernel gives the column among sixteen."""
     rng = np.random.default_rng(8300 + m + n)
     wb = _weights(Q6_K, m, k, 8301 + m)
     w = ctx.upload(Q6_K, wb, k, m)
@@ -1137,12 +1173,11 @@ def test_q6k_many_rows_few_columns(ctx, m, k, n):
     assert npref.rel_err(got, want) < TOL
     _check_against_exact_arithmetic(Q6_K, wb, k, m, x, got, f"Q6_K {m}x{k} n={n}", max_rows=4096)
     assert np.array_equal(ctx.mulmat(w, x[::-1].copy())[::-1], got)
+    # the same columns among sixteen go through the general kernel (one wave per row group at this many rows: K uncut)
+    x16 = np.concatenate([x, rng.standard_normal((16 - n, k), dtype=np.float32)])
+    assert ctx.route(w, 16) == "skinny_staged"
+    assert np.array_equal(ctx.mulmat(w, x16)[:n], got)
     w.free()
-    if n >= 4:  # (three columns of a smaller matrix go to the streaming kernel, whose sums run in another order)
-        rows = 40000
-        w2 = ctx.upload(Q6_K, np.ascontiguousarray(wb.reshape(m, -1)[:rows]).reshape(-1), k, rows)
-        assert np.array_equal(ctx.mulmat(w2, x), got[:, :rows])
-        w2.free()
 
 
 @pytest.mark.parametrize("n", [3, 4, 6])
