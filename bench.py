@@ -408,6 +408,7 @@ def main() -> int:
         for label, t, m, k, ns, copies in (("Q4_K q_proj 4096x4096", Q4_K, 4096, 4096, (2, 4, 8), 40),  # (one column would share the headline kernel's name in a profile)
                                            ("Q4_0 GEMV 4096x4096", Q4_0, 4096, 4096, (1,), 40),
                                            ("Q8_0 skinny 4096x4096", Q8_0, 4096, 4096, (1, 2, 4, 8), 40),
+                                           ("Q6_K ffn_down 4096x14336", Q6_K, 4096, 14336, (4, 8), 10),
                                            ("Q6_K head 128256x4096", Q6_K, 128256, 4096, (1, 8), 3)):
             for n in ns:
                 tm, wb = time_mulmat(t, m, k, n, copies)

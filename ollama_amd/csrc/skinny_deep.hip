@@ -173,13 +173,16 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
         const uint8_t *aq = reinterpret_cast<const uint8_t *>(a.qs);
         // copy instructions are dealt out to the waves in turn: first the quants (two instructions per super-block:
         // columns 0..3 and 4..7), then the digits and the scales (64 (super-block, column) cells per instruction)
-        const int cells = nsb * NCT, n_q = nsb * 2, n_c = (cells + 63) / 64;
+        // (columns past nc are not copied: the lanes of the A operand that stand for them read zeros)
+        const int sets = nc > 4 ? 2 : 1;
+        const int cells = nsb * NCT, n_q = nsb * sets, n_c = (cells + 63) / 64;
         for (int n = wave; n < n_q + 2 * n_c; n += cut.W) {
             if (n < n_q) {
-                const int sb = n >> 1, j = n & 1;
+                const int sb = sets == 2 ? n >> 1 : n, j = sets == 2 ? n & 1 : 0;
                 const int col = 4 * j + (lane >> 4), pc = (lane & 15) ^ a_swz(col);
-                dma_lds<16>(aq + (int64_t)sb * QKK, (unsigned)acol(col) * (unsigned)a.K + 16u * pc,
-                            sm + Geo::A_OFF + (unsigned)(sb * NCT + 4 * j) * 256u);
+                if (col < nc)
+                    dma_lds<16>(aq + (int64_t)sb * QKK, (unsigned)acol(col) * (unsigned)a.K + 16u * pc,
+                                sm + Geo::A_OFF + (unsigned)(sb * NCT + 4 * j) * 256u);
             } else {
                 const bool digits = n < n_q + n_c;
                 const int c0 = 64 * (digits ? n - n_q : n - n_q - n_c);
@@ -608,8 +611,9 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g,
             if (n < n_q) {
                 const int sb = n / SETS, j = n % SETS;
                 const int col = 4 * j + (lane >> 4), pc = (lane & 15) ^ (col & 2);
-                dma_lds<16>(aq + (int64_t)sb * QKK, (unsigned)acol(col) * (unsigned)a.K + 16u * pc,
-                            sm + Geo::A_OFF + (unsigned)(sb * NC + 4 * j) * 256u);
+                if (col < nc)  // (columns past nc keep what the LDS held: they are multiplied and dropped)
+                    dma_lds<16>(aq + (int64_t)sb * QKK, (unsigned)acol(col) * (unsigned)a.K + 16u * pc,
+                                sm + Geo::A_OFF + (unsigned)(sb * NC + 4 * j) * 256u);
             } else if (n < n_q + n_g) {
                 const int c0 = 32 * (n - n_q);
                 const int cell = min(c0 + (lane >> 1), cells - 1), sb = cell / NC, col = cell % NC;
