@@ -1141,12 +1141,13 @@ def test_page_locked_host_buffers(ctx):
 # ---- skinny product on the matrix cores for the K-quants: both kernels ------------------------------
 @pytest.mark.parametrize("t", [Q4_K, Q6_K])
 @pytest.mark.parametrize("m,k,n", [(4096, 4096, 3), (1000, 1024, 4), (17, 256, 4), (9, 256, 3), (300, 2304, 19), (64, 8192, 4),
-                                   (4096, 14336, 4), (1000, 1024, 7), (2048, 768, 3)])
+                                   (4096, 14336, 4), (1000, 1024, 7), (2048, 768, 3), (4096, 14336, 20), (14336, 4096, 19)])
 def test_skinny_kquants_match_oracle(ctx, t, m, k, n):
     """3..31 columns through the C ABI's default routing: Q4_K at three and four columns of a small matrix
     takes the kernel that loads weights straight into the MFMA operands (ragged M, a single super-block,
     K cut one to sixteen ways, a second launch that starts at column 16), a large one and more columns
-    the staged kernel"""
+    the staged kernel; at 19 and 20 columns of a large matrix the second launch, of columns 16.., is one of the deep
+    direct-load kernel"""
     rng = np.random.default_rng(8100 + t + m + n)
     wb = _weights(t, m, k, 8101 + t + m)
     w = ctx.upload(t, wb, k, m)
