@@ -403,6 +403,38 @@ def test_q6k_deep_kernel_few_columns_on_large_matrices(ctx, m, k, ns):
     W.free()
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_deep_kernels_on_random_large_shapes(ctx, seed):
+    """twelve seeded shapes per seed beyond 40 M weights -- K any multiple of 256 up to 16384, rows to match, 2..8
+    columns, Q4_K and Q6_K in turn -- through the default routing: a slab of the first and of the last rows against the
+    oracle, and where the deep kernels ran, the f32 form against quantize-then-multiply bit for bit"""
+    rng = np.random.default_rng(9400 + seed)
+    deep = 0
+    for case in range(12):
+        t = Q4_K if case % 2 == 0 else Q6_K
+        k = 256 * int(rng.integers(2, 65))
+        lo = (40 << 20) // k + 1
+        m = int(rng.integers(lo, 3 * lo))
+        n = int(rng.integers(2 if t == Q4_K else 3, 9))
+        base = _weights(t, 512, k, seed=9401 + case)
+        raw = np.ascontiguousarray(np.roll(np.tile(base.reshape(512, -1), (m // 512 + 1, 1))[:m], case, axis=0))
+        W = ctx.upload(t, raw.reshape(-1), k, m)
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        route = ctx.route(W, n)
+        got = ctx.mulmat(W, x)
+        for sl in (slice(0, 96), slice(m - 200, m)):
+            want = oracle.mul_mat(t, np.ascontiguousarray(raw[sl]).reshape(-1), k, raw[sl].shape[0], x, nthreads=16)
+            assert npref.rel_err(got[:, sl], want) < TOL, (NAMES[t], m, k, n, route)
+        if route in ("skinny_deep", "deep_f32"):
+            deep += 1
+            act = ctx.act_create(Q8_K, k, n)
+            ctx.act_quantize(act, x)
+            assert np.array_equal(ctx.mulmat_q8(W, act), got), (NAMES[t], m, k, n, route)
+            act.free()
+        W.free()
+    assert deep >= 8
+
+
 @pytest.mark.parametrize("t", WTYPES)
 def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
     """For n <= 8 the f32 entry points quantize x inside the GEMV's prologue.  The result must be
