@@ -827,11 +827,14 @@ __global__ __launch_bounds__(XMODE && NC <= 3 ? 1024 : 512) void gemv_thin_kerne
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = 1 << rw_log2;
     const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
-    const int rows_per_wg = rows_per_wave << rw_log2;
+    // rows_per_wave: the low half is the rows of every wave, the high half how many of the workgroup's first row groups
+    // take one more (a workgroup's rows need not divide by its row groups: 28672 rows are 512 workgroups of 56)
+    const int rpw_base = rows_per_wave & 0xffff, rpw_extra = rows_per_wave >> 16;
+    const int rows_per_wg = (rpw_base << rw_log2) + rpw_extra;
     const int64_t r0 = (int64_t)wg * rows_per_wg;
     const int nrows = (int)min((int64_t)rows_per_wg, w.M - r0);
-    const int rl0 = rg * rows_per_wave;                    // the wave's rows: r0 + rl0 + i, i < nrw
-    const int nrw = max(0, min(rows_per_wave, nrows - rl0));
+    const int rl0 = rg * rpw_base + min(rg, rpw_extra);    // the wave's rows: r0 + rl0 + i, i < nrw
+    const int nrw = max(0, min(rpw_base + (rg < rpw_extra ? 1 : 0), nrows - rl0));
     float *yrow0 = y + (int64_t)col0 * ldy + r0;
 
     // rows side by side in this wave: RPL for short rows, TAILR in the waves of a mostly empty last segment
@@ -1155,8 +1158,9 @@ size_t thin_act_lds(int64_t K, int nc) {
 
 // produce: the f32 activations go through a producer first (one column; room for RMSNorm's piece sums, and
 // every piece of x must sit in a prefetch register of some wave)
+// uneven: the caller's kernel takes workgroups whose rows do not divide by their row groups (gemv_thin_kernel)
 template <class P>
-bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool produce = false) {
+bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool produce = false, bool uneven = false) {
     const int nseg = (int)((K + P::SEG - 1) / P::SEG);
     if (nseg < 1 || nseg > 8) return false;
     p.spw = 1;
@@ -1204,6 +1208,20 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
     if (p.rpl > 1) rows_per_wave = max(2 * p.rpl, (rows_per_wave + p.rpl - 1) / p.rpl * p.rpl);
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
+    if (uneven && f32 && p.kw == 1 && p.rpl == 1 && !produce && nc == 1) {
+        // The same number of workgroups on every CU: their count rounded up to a multiple of the CUs and the rows dealt
+        // out evenly, some row groups taking one row more than the others.  28672 rows in workgroups of 64 are 448
+        // workgroups, two on 192 CUs and one on 64; the lone ones are through at 7.9 us, the second workgroups of the
+        // others at 11.2-11.8 (stamps per wave).  In 512 workgroups of 56 rows: gate + up 12.91 -> 12.61 us, Q6_K
+        // 14336 x 4096 11.5 -> 10.4.  It pays where it adds few workgroups (each one quantizes x again: 22016 rows from
+        // 344 to 512 workgroups measured 11.2 -> 12.0 us, Q6_K 11008 rows 9.5 -> 10.5) or where a wave has only two rows
+        // anyway and the launch is all start-up (Q4_K 4096 / 6144 / 11008 / 13824 rows: 2-6 % faster with every CU at work).
+        const int64_t wgs = (total_m + p.rows_per_wg - 1) / p.rows_per_wg;
+        const int64_t target = (wgs + 255) / 256 * 256;
+        const int64_t even = (total_m + target - 1) / target;
+        const bool few_more = 5 * target <= 6 * wgs, short_waves = rows_per_wave == 2 && p.rw == 16;
+        if (target != wgs && (few_more || short_waves) && even >= p.rw && even <= 16 * p.rw) p.rows_per_wg = (int)even;
+    }
     p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float) + 64);  // + 16 counters
     if (produce) {
         if (!f32 || nc != 1 || K > (int64_t)XPRE * p.kw * p.rw * 256) return false;
@@ -1216,7 +1234,7 @@ template <class P, int NC, int XMODE, int XP = XPRE>
 void launch_thin_mode(const Plan &p, const ThinArgs &ma, const DevAct &a, const float *xf, int col0, const Produce &pr,
                       hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
-    const int rpw = p.rows_per_wg >> p.rw_log2;
+    const int rpw = (p.rows_per_wg >> p.rw_log2) | ((p.rows_per_wg & (p.rw - 1)) << 16);
 #define THIN_LAUNCH(DIRECT, RPL) \
     gemv_thin_kernel<P, NC, DIRECT, XMODE, RPL, XP><<<p.grid, block, p.lds, s>>>(ma, a, xf, col0, rpw, p.kw, p.rw_log2, pr)
 #define THIN_LAUNCH_SEGMENTS(AHEAD, TAILR) \
@@ -1267,7 +1285,7 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
     int64_t total_m = 0;
     for (int i = 0; i < count; i++) total_m += ws[i].M;
     Plan p;
-    const bool thin = make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, p, pr.kind != PRODUCE_NONE);
+    const bool thin = make_thin_plan<P>(ws[0].K, total_m, nc, xf != nullptr, p, pr.kind != PRODUCE_NONE, true);
     if (pr.kind != PRODUCE_NONE && !thin) return hipErrorInvalidValue;  // callers ask gemv_produce_supported() first
     if (xf && !thin) return hipErrorInvalidValue;  // callers ask gemv_f32_supported() first
     if (!thin) {
