@@ -1208,7 +1208,7 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
     if (p.rpl > 1) rows_per_wave = max(2 * p.rpl, (rows_per_wave + p.rpl - 1) / p.rpl * p.rpl);
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
-    if (uneven && f32 && p.kw == 1 && p.rpl == 1 && !produce && nc == 1) {
+    if (uneven && f32 && p.kw == 1 && p.rpl == 1 && nc == 1) {
         // The same number of workgroups on every CU: their count rounded up to a multiple of the CUs and the rows dealt
         // out evenly, some row groups taking one row more than the others.  28672 rows in workgroups of 64 are 448
         // workgroups, two on 192 CUs and one on 64; the lone ones are through at 7.9 us, the second workgroups of the
