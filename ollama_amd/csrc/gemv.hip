@@ -1121,7 +1121,7 @@ __global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const floa
     }
 }
 
-struct Plan { int kw, rw, rw_log2, spw, rows_per_wg, rpl, tail_log2 = 0; unsigned grid; size_t lds; };
+struct Plan { int kw, rw, rw_log2, spw, rows_per_wg, rpl, tail_log2 = 0; unsigned grid; size_t lds; int even_wgs = 0; };
 
 // 8 waves per workgroup (two per SIMD, so a wave may use up to 256 VGPRs), one or two workgroups per CU.
 // total_m is the number of rows over all tensors of the launch.
@@ -1208,19 +1208,23 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
     if (p.rpl > 1) rows_per_wave = max(2 * p.rpl, (rows_per_wave + p.rpl - 1) / p.rpl * p.rpl);
     if (rows_per_wave > 16) rows_per_wave = 16;  // a wave parks its row totals in lanes 63, 62, ...
     p.rows_per_wg = p.rw * rows_per_wave;
-    if (uneven && f32 && p.kw == 1 && p.rpl == 1 && nc == 1) {
+    if (uneven && f32 && p.kw == 1 && p.rpl == 1 && nc <= 2) {
         // The same number of workgroups on every CU: their count rounded up to a multiple of the CUs and the rows dealt
         // out evenly, some row groups taking one row more than the others.  28672 rows in workgroups of 64 are 448
         // workgroups, two on 192 CUs and one on 64; the lone ones are through at 7.9 us, the second workgroups of the
         // others at 11.2-11.8 (stamps per wave).  In 512 workgroups of 56 rows: gate + up 12.91 -> 12.61 us, Q6_K
         // 14336 x 4096 11.5 -> 10.4.  It pays where it adds few workgroups (each one quantizes x again: 22016 rows from
         // 344 to 512 workgroups measured 11.2 -> 12.0 us, Q6_K 11008 rows 9.5 -> 10.5) or where a wave has only two rows
-        // anyway and the launch is all start-up (Q4_K 4096 / 6144 / 11008 / 13824 rows: 2-6 % faster with every CU at work).
+        // anyway and the launch is all start-up (Q4_K 4096 / 6144 / 11008 / 13824 rows: 2-6 % faster with every CU at work;
+        // at two columns Q4_K 4096 x 4096 5.6 -> 5.0 us, Q6_K 14336 x 4096 14.7 -> 13.2).
         const int64_t wgs = (total_m + p.rows_per_wg - 1) / p.rows_per_wg;
         const int64_t target = (wgs + 255) / 256 * 256;
         const int64_t even = (total_m + target - 1) / target;
         const bool few_more = 5 * target <= 6 * wgs, short_waves = rows_per_wave == 2 && p.rw == 16;
-        if (target != wgs && (few_more || short_waves) && even >= p.rw && even <= 16 * p.rw) p.rows_per_wg = (int)even;
+        if (target != wgs && (few_more || short_waves) && even >= p.rw && even <= 16 * p.rw) {
+            p.rows_per_wg = (int)even;
+            p.even_wgs = (int)target;  // (several matrices: the caller makes sure their workgroups together do not exceed it)
+        }
     }
     p.lds = (f32 ? thin_act_lds<P>(K, nc) : 0) + (p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float) + 64);  // + 16 counters
     if (produce) {
@@ -1291,6 +1295,16 @@ hipError_t launch_type(const DevWeight *ws, float *const *ys, int count, const D
     if (!thin) {
         if (!make_plan<P>(ws[0].K, total_m, nc, num_cus, p)) return hipErrorInvalidValue;
         if (p.spw > 1 && !make_plan<P>(ws[0].K, total_m, 1, num_cus, p)) return hipErrorInvalidValue;
+    }
+    if (thin && p.even_wgs && count > 1) {
+        // an even plan was made for the rows of all matrices together; every matrix rounds its workgroups up by itself, and
+        // one workgroup too many is a CU with three where the others have two
+        auto wgs_at = [&](int rows) {
+            int64_t n = 0;
+            for (int i = 0; i < count; i++) n += (ws[i].M + rows - 1) / rows;
+            return n;
+        };
+        while (wgs_at(p.rows_per_wg) > p.even_wgs && p.rows_per_wg < 16 * p.rw) p.rows_per_wg++;
     }
     MultiArgs ma;
     ma.count = count;
