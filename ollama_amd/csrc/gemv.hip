@@ -1048,11 +1048,14 @@ __global__ __launch_bounds__(1024) void gemv_pair_kernel(ThinArgs ta, const floa
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = 1 << rw_log2;
     const int rg = wave & (rw - 1), kseg = wave >> rw_log2;
-    const int rows_per_wg = rows_per_wave << rw_log2;          // rows of h per workgroup
+    // rows_per_wave as in gemv_thin_kernel: rows of h of every wave, and in the high half how many of the first row groups
+    // take one more
+    const int rpw_base = rows_per_wave & 0xffff, rpw_extra = rows_per_wave >> 16;
+    const int rows_per_wg = (rpw_base << rw_log2) + rpw_extra;  // rows of h per workgroup
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
     const int nrows = (int)min((int64_t)rows_per_wg, wa.M - r0);
-    const int rl0 = rg * rows_per_wave;
-    const int nrw = max(0, min(rows_per_wave, nrows - rl0));   // rows of h of this wave; 2 * nrw virtual rows
+    const int rl0 = rg * rpw_base + min(rg, rpw_extra);
+    const int nrw = max(0, min(rpw_base + (rg < rpw_extra ? 1 : 0), nrows - rl0));   // rows of h of this wave; 2 * nrw virtual rows
     const int vlane = lane & (64 / RPL - 1), run = RPL == 1 ? 0 : lane / (64 / RPL);
     const typename P::Geo g = P::geo(wa, kseg, vlane);
 
@@ -1213,14 +1216,15 @@ bool make_thin_plan(int64_t K, int64_t total_m, int nc, bool f32, Plan &p, bool 
         // out evenly, some row groups taking one row more than the others.  28672 rows in workgroups of 64 are 448
         // workgroups, two on 192 CUs and one on 64; the lone ones are through at 7.9 us, the second workgroups of the
         // others at 11.2-11.8 (stamps per wave).  In 512 workgroups of 56 rows: gate + up 12.91 -> 12.61 us, Q6_K
-        // 14336 x 4096 11.5 -> 10.4.  It pays where it adds few workgroups (each one quantizes x again: 22016 rows from
-        // 344 to 512 workgroups measured 11.2 -> 12.0 us, Q6_K 11008 rows 9.5 -> 10.5) or where a wave has only two rows
+        // 14336 x 4096 11.5 -> 10.4.  It pays where CUs hold two workgroups and it adds few (at most a fifth more; with one
+        // workgroup per CU, 230 -> 256 workgroups, 22016 rows measured 11.2 -> 12.0 us, Q6_K 11008 rows 9.5 -> 10.5, and the
+        // gate / up pair kernel at 11008 rows 11.4 -> 12.0) or where a wave has only two rows
         // anyway and the launch is all start-up (Q4_K 4096 / 6144 / 11008 / 13824 rows: 2-6 % faster with every CU at work;
         // at two columns Q4_K 4096 x 4096 5.6 -> 5.0 us, Q6_K 14336 x 4096 14.7 -> 13.2).
         const int64_t wgs = (total_m + p.rows_per_wg - 1) / p.rows_per_wg;
         const int64_t target = (wgs + 255) / 256 * 256;
         const int64_t even = (total_m + target - 1) / target;
-        const bool few_more = 5 * target <= 6 * wgs, short_waves = rows_per_wave == 2 && p.rw == 16;
+        const bool few_more = target >= 512 && 5 * target <= 6 * wgs, short_waves = rows_per_wave == 2 && p.rw == 16;
         if (target != wgs && (few_more || short_waves) && even >= p.rw && even <= 16 * p.rw) {
             p.rows_per_wg = (int)even;
             p.even_wgs = (int)target;  // (several matrices: the caller makes sure their workgroups together do not exceed it)
@@ -1443,9 +1447,9 @@ hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int coun
 namespace {
 
 template <class P, int XMODE, int XP>
-void launch_pair_mode(const Plan &p, const ThinArgs &ta, const float *xf, const Produce &pr, unsigned grid, hipStream_t s) {
+void launch_pair_mode(const Plan &p, const ThinArgs &ta, const float *xf, const Produce &pr, unsigned grid, int rows_h, hipStream_t s) {
     const dim3 block(64 * p.kw * p.rw);
-    const int rpw = (p.rows_per_wg >> p.rw_log2) / 2;  // rows of h per wave: half the virtual rows
+    const int rpw = (rows_h >> p.rw_log2) | ((rows_h & (p.rw - 1)) << 16);  // rows of h per wave (+ row groups with one more)
 #define PAIR_LAUNCH(DIRECT, RPL) \
     gemv_pair_kernel<P, DIRECT, XMODE, RPL, XP><<<grid, block, p.lds, s>>>(ta, xf, rpw, p.kw, p.rw_log2, pr)
     if (p.kw > 1) PAIR_LAUNCH(false, 1);
@@ -1475,13 +1479,20 @@ hipError_t launch_pair_type(const DevWeight &wg, const DevWeight &wu, const floa
         ta.wg_end[i] = 0x7fffffff;
     }
     ta.K = wg.K; ta.type = wg.type;
-    const int rows_per_wg = p.rows_per_wg / 2;
+    int rows_per_wg = p.rows_per_wg / 2;  // rows of h
+    if (p.kw == 1 && p.rpl == 1) {
+        // the same number of workgroups on every CU where they hold two and that adds at most a fifth (as in
+        // make_thin_plan): 14336 rows of h in 512 workgroups of 28 instead of 448 of 32, 13.1 -> 12.8 us
+        const int64_t wgs = (wg.M + rows_per_wg - 1) / rows_per_wg, target = (wgs + 255) / 256 * 256;
+        const int64_t even = (wg.M + target - 1) / target;
+        if (target != wgs && target >= 512 && 5 * target <= 6 * wgs && even >= p.rw && even <= 8 * p.rw) rows_per_wg = (int)even;
+    }
     const unsigned grid = (unsigned)((wg.M + rows_per_wg - 1) / rows_per_wg);
     const bool one_piece = wg.K <= (int64_t)256 * p.kw * p.rw;
-    if (rms && one_piece) launch_pair_mode<P, 2, 1>(p, ta, xf, pr, grid, s);
-    else if (rms) launch_pair_mode<P, 2, XPRE>(p, ta, xf, pr, grid, s);
-    else if (one_piece) launch_pair_mode<P, 1, 1>(p, ta, xf, pr, grid, s);
-    else launch_pair_mode<P, 1, XPRE>(p, ta, xf, pr, grid, s);
+    if (rms && one_piece) launch_pair_mode<P, 2, 1>(p, ta, xf, pr, grid, rows_per_wg, s);
+    else if (rms) launch_pair_mode<P, 2, XPRE>(p, ta, xf, pr, grid, rows_per_wg, s);
+    else if (one_piece) launch_pair_mode<P, 1, 1>(p, ta, xf, pr, grid, rows_per_wg, s);
+    else launch_pair_mode<P, 1, XPRE>(p, ta, xf, pr, grid, rows_per_wg, s);
     return hipGetLastError();
 }
 
