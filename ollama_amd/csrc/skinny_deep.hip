@@ -539,10 +539,7 @@ namespace {
 //
 // Order of the floating-point sums: as above (pieces of four super-blocks in order, piece sums in order).
 constexpr int Q6_QL = 128, Q6_QH = 64, Q6_SC = 16;
-#ifndef DEEP6_FROM_N
-#define DEEP6_FROM_N 3
-#endif
-constexpr int DEEP6_FROM = DEEP6_FROM_N;  // activation columns from which the kernel is taken
+constexpr int DEEP6_FROM = 3;  // activation columns from which the kernel is taken (at two the streaming kernel is ahead: 14.1 / 14.9 against 15.6 / 15.1 us)
 struct Deep6Args {
     const uint8_t *ql, *qh, *sc;
     const uint16_t *d;
