@@ -435,6 +435,35 @@ def test_deep_kernels_on_random_large_shapes(ctx, seed):
     assert deep >= 8
 
 
+@pytest.mark.parametrize("t,ms", [(Q4_K, [14336, 14336]), (Q4_K, [4096, 1024, 1024]), (Q4_K, [13824]), (Q6_K, [14336]), (Q4_K, [4100]),
+                                  (Q4_K, [11008]), (Q6_K, [13830])])
+def test_even_workgroup_plans_keep_the_bits(ctx, t, ms):
+    """One and two f32 columns on rows of one K segment: the launch is planned with the same number of workgroups on
+    every CU, their rows dealt out unevenly over the row groups (28672 rows: 512 workgroups of 56, some waves with four
+    rows and some with three; several matrices in one launch keep within the even count).  A row's sum does not depend
+    on the plan: the bits are those of the two-phase form, which is planned differently, and of each matrix alone;
+    a slab of the last rows against the oracle."""
+    k = 4096
+    rng = np.random.default_rng(9500 + sum(ms) + t)
+    raws = [_weights(t, m, k, seed=9501 + m + i) for i, m in enumerate(ms)]
+    Ws = [ctx.upload(t, r, k, m) for r, m in zip(raws, ms)]
+    act = ctx.act_create(Q8_K, k, 2)
+    for n in (1, 2):
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        got = ctx.mulmat_multi(Ws, x) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x)]
+        ctx.act_quantize(act, x)
+        for y, W, raw, m in zip(got, Ws, raws, ms):
+            if ctx.route(W, n) == "gemv_f32":
+                assert np.array_equal(ctx.mulmat_q8(W, act, path=qmm.PATH_GEMV), y), (m, n)
+                assert np.array_equal(ctx.mulmat(W, x), y), (m, n)
+            rows = min(m, 3000)
+            want = oracle.mul_mat(t, np.ascontiguousarray(raw[-rows:]), k, rows, x, nthreads=16)
+            assert npref.rel_err(y[:, -rows:], want) < TOL, (m, n)
+    act.free()
+    for W in Ws:
+        W.free()
+
+
 @pytest.mark.parametrize("t", WTYPES)
 def test_in_kernel_quantization_gives_the_same_bits(ctx, t):
     """For n <= 8 the f32 entry points quantize x inside the GEMV's prologue.  The result must be
