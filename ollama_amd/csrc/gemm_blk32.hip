@@ -340,7 +340,9 @@ __global__ __launch_bounds__(512, 1) void gemm_blk32_dma_kernel(DevWeight w, Dev
 // stay unsigned nibbles; the -8 goes through the activations' block sums.
 // Same shape as the K-quant skinny kernel: a workgroup owns 16 weight rows, its waves cut K in runs
 // of 256 elements and stream weights, activations and both sides' scales through private two-stage LDS
-// rings with direct-to-LDS loads; one barrier at the end for the sum over the K cuts.
+// rings with direct-to-LDS loads; one barrier at the end for the sum over the K cuts.  (Q8_0 at up to eight columns with
+// waves of at most two steps takes the weights straight into registers instead: DW below, 9.9 -> 9.4 us and 10.2 -> 9.5 us
+// for 4096 x 4096 at four and eight columns, quantization launch included.)
 // ---------------------------------------------------------------------------------------------
 typedef int v4acc __attribute__((ext_vector_type(4)));
 
@@ -380,10 +382,15 @@ struct Sk32Multi {
     int grp_end[3];  // exclusive ends of the runs of matrices 0, 1, 2; INT_MAX past the last matrix
 };
 
-template <bool Q4, int NCT, bool ID, bool MULTI = false>
+// DW ("direct weights", Q8_0, one set of columns, waves of at most two steps): the weights and their scales go from
+// memory straight into registers -- a quad of lanes on 64 contiguous bytes of a row, as in the deep kernels of
+// skinny_deep.hip -- and ds_bpermute puts them into the MFMA operand order; only the activations still pass through the
+// wave's LDS stages.  Same K cut, same expressions in the same order: the bits of the staged form.
+template <bool Q4, int NCT, bool ID, bool MULTI = false, bool DW = false>
 __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWeight w_in, DevAct a_in, int col0, int nc, float *__restrict__ y_in,
                                                                           Sk32Ids si_in, int WAVES, Sk32Multi mt) {
     static_assert(!(ID && MULTI), "expert-indexed launches take one stack");
+    static_assert(!DW || (!Q4 && NCT == 8 && !ID && !MULTI), "direct weights: Q8_0, up to eight columns, one matrix");
     typedef Sk32Geo<Q4, NCT> Geo;
     constexpr int STAGE = Geo::STAGE, NDMA = Geo::NDMA, SETS = Geo::SETS;
     // The argument block in one batch of scalar loads: everything is named here and pinned by an empty asm
@@ -486,12 +493,12 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
     const uint8_t *abs_ = reinterpret_cast<const uint8_t *>(a.bsums);
 
     auto stage_copy = [&](uint8_t *st, int64_t sp) __attribute__((always_inline)) {
+        if (!DW) {
 #pragma unroll
-        for (int i = 0; i < Geo::W_INSTRS; i++) {
-            const uint8_t *gp = wbase + sp * (Q4 ? 128 : 256) + woff[i];
-            __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * i), 16, 0, 0);
-        }
-        {
+            for (int i = 0; i < Geo::W_INSTRS; i++) {
+                const uint8_t *gp = wbase + sp * (Q4 ? 128 : 256) + woff[i];
+                __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + 1024 * i), 16, 0, 0);
+            }
             const uint8_t *gp = dwbase + sp * 16 + dwoff;
             if (lane < 16) __builtin_amdgcn_global_load_lds((glb_ptr_t *)gp, (lds_ptr_t *)(st + Geo::DW_OFF), 16, 0, 0);
         }
@@ -527,6 +534,77 @@ __global__ __launch_bounds__(512, (NCT > 8 ? 2 : 4)) void skinny32_kernel(DevWei
     float acc[SETS][2];
 #pragma unroll
     for (int cs = 0; cs < SETS; cs++) acc[cs][0] = acc[cs][1] = 0.f;
+    if (DW) {
+        if (s0 < s1) {
+            typedef unsigned u4v __attribute__((ext_vector_type(4)));
+            typedef const __attribute__((address_space(1))) u4v *gu4_t;
+            typedef const __attribute__((address_space(1))) unsigned *gu_t;
+            // loading lane: its row and which 16 bytes of the quad's 64 (rows 8..15 in the order 2 3 0 1: sources of
+            // rows r and r + 8 must not share a bank of the ds_bpermute crossbar)
+            const int lrow = min(lane >> 2, rows_left - 1), lq = (lane & 3) ^ ((lane >> 4) & 2);
+            const unsigned qoff = (unsigned)lrow * (unsigned)w.K + 16u * lq, doff = (unsigned)lrow * (unsigned)nblk * 2u + 4u * lq;
+            const int rsw = (c >> 3) << 1, bidx = 4 * (4 * c + (g ^ rsw));
+            u4v wq[2][4];
+            unsigned wdr[2];
+            // requests: the activations of a step, then its weights; both steps at once (a wave has at most two)
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+                const int64_t sp = min(s0 + st, s1 - 1);
+                stage_copy(wsm + st * STAGE, sp);
+                __builtin_amdgcn_sched_barrier(0);
+                const __attribute__((address_space(1))) uint8_t *wp = (const __attribute__((address_space(1))) uint8_t *)(wbase + sp * 256);
+                const __attribute__((address_space(1))) uint8_t *dp = (const __attribute__((address_space(1))) uint8_t *)(dwbase + sp * 16);
+#pragma unroll
+                for (int t = 0; t < 4; t++) wq[st][t] = *(gu4_t)(wp + (qoff + 64u * t));
+                wdr[st] = *(gu_t)(dp + doff);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            constexpr int PER_STEP = Geo::A_INSTRS + 1 + 5;  // copies and loads of one step
+            const v4acc zero = {0, 0, 0, 0};
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+                if (s0 + st < s1) {  // wave-uniform
+                    const uint8_t *stg = wsm + st * STAGE;
+                    if (st == 0) __builtin_amdgcn_s_waitcnt((PER_STEP & 15) | (7 << 4) | (15 << 8) | ((PER_STEP >> 4) << 14));
+                    else __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8));
+                    v4i bq[4], av[4];
+                    uint4 dxr[2][2];
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) bq[t][i] = __builtin_amdgcn_ds_bpermute(bidx, (int)wq[st][t][i]);
+                        av[t] = *reinterpret_cast<const v4i *>(stg + aro[0][t]);
+                    }
+                    unsigned dwp[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) dwp[j] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * (4 * c) + 4 * (j ^ rsw), (int)wdr[st]);
+#pragma unroll
+                    for (int u = 0; u < 2; u++) {
+                        dxr[u][0] = *reinterpret_cast<const uint4 *>(stg + Geo::DX_OFF + 32 * lcol[0][u]);
+                        dxr[u][1] = *reinterpret_cast<const uint4 *>(stg + Geo::DX_OFF + 32 * lcol[0][u] + 16);
+                    }
+                    float dwf[8];
+#pragma unroll
+                    for (int b = 0; b < 8; b++) dwf[b] = h2f(b & 1 ? dwp[b >> 1] >> 16 : dwp[b >> 1] & 0xffff);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const v4acc dv = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[t], bq[t], zero, 0, 0, 0);
+#pragma unroll
+                        for (int u = 0; u < 2; u++) {
+                            const unsigned dxp[8] = {dxr[u][0].x, dxr[u][0].y, dxr[u][0].z, dxr[u][0].w,
+                                                     dxr[u][1].x, dxr[u][1].y, dxr[u][1].z, dxr[u][1].w};
+#pragma unroll
+                            for (int sblk = 0; sblk < 2; sblk++) {
+                                const int b = 2 * t + sblk;
+                                acc[0][u] = __builtin_fmaf((float)dv[2 * u + sblk], dwf[b] * __uint_as_float(dxp[b]), acc[0][u]);
+                            }
+                        }
+                    }
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0);
+        }
+    } else
     if (s0 < s1) {
         stage_copy(wsm, s0);
         stage_copy(wsm + STAGE, min(s0 + 1, s1 - 1));
@@ -622,6 +700,19 @@ void launch_skinny32_as(const DevWeight &w, const DevAct &a, int col0, int ncols
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny32_kernel<Q4, NCT, ID>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         allowed[dev] = true;
+    }
+    if constexpr (!Q4 && NCT == 8 && !ID) {
+        // waves of at most two steps: the weights straight into registers (the bits are those of the staged form)
+        if (nst <= 2 * waves && w.M * w.K < ((int64_t)1 << 32)) {
+            static bool allowed_dw[64] = {false};
+            if (dev >= 0 && dev < 64 && !allowed_dw[dev]) {
+                (void)hipFuncSetAttribute(reinterpret_cast<const void *>(skinny32_kernel<false, 8, false, false, true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                allowed_dw[dev] = true;
+            }
+            skinny32_kernel<false, 8, false, false, true><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves, Sk32Multi{});
+            return;
+        }
     }
     skinny32_kernel<Q4, NCT, ID><<<(unsigned)groups, 64 * waves, lds, s>>>(w, a, col0, ncols, y, si, waves, Sk32Multi{});
 }
