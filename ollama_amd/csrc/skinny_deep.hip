@@ -474,7 +474,13 @@ bool deep16_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus)
     DeepCut c;
     size_t lds;
     if (!deep16_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds)) return false;
-    return total_m * K > ((int64_t)40 << 20);  // below that the many-small-waves direct kernel is ahead
+    if (total_m * K > ((int64_t)40 << 20)) return true;  // (below that the many-small-waves direct kernel is ahead at 3..4 columns)
+    // Five to eight columns, where the alternative is the staged kernel: from 20 Mi weights (below 24576 rows: beyond, the
+    // rows kernel).  6144 x 4096 7.5 against 9.1 us at five columns (9.4 / 9.5 at eight), 8192 x 4096 8.2 / 10.1 against
+    // 10.5 / 11.0; on 4096 x 4096 this kernel is 5 % behind (8.4 against 8.0 us: its four waves per CU cannot quantize x
+    // themselves).  (q + k + v of 4096 + 1024 + 1024 rows in one launch would take 7.8 / 10.5 us here against 12.7 / 13.0
+    // staged, but a joint launch takes a kernel only when every matrix takes it alone, and alone they are too small.)
+    return ncols >= 5 && total_m * K >= ((int64_t)20 << 20) && (total_m + 15) / 16 < 6 * (int64_t)num_cus;
 }
 
 namespace {

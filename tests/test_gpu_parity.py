@@ -331,9 +331,11 @@ def test_q4k_rows_kernel_alone_and_joint(ctx, ms, k, ns):
 
 @pytest.mark.parametrize("ms,k,ns", [([14336, 14336], 4096, (2, 3, 4, 8)), ([14336], 4096, (2, 5)), ([4096], 14336, (3, 4, 7, 8)),
                                      ([14330, 5000], 4096, (6,)), ([4100], 14336 + 256, (5,)), ([8192], 8192, (4, 8)),
-                                     ([70000], 4096, (2, 3, 8)), ([40000, 33000], 2048, (2, 5)), ([131072 + 48], 1024, (8,))])
+                                     ([70000], 4096, (2, 3, 8)), ([40000, 33000], 2048, (2, 5)), ([131072 + 48], 1024, (8,)),
+                                     ([8192], 4096, (5, 8)), ([6150, 5200], 4096, (6,)), ([2600], 8192, (7,))])
 def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
-    """Q4_K at 3..8 columns (from two on rows up to 4096) on matrices beyond 40 M weights: the kernel that loads weights straight into registers (a ring
+    """Q4_K at 3..8 columns (from two on rows up to 4096) on matrices beyond 40 M weights, and at 5..8 columns from 20 M
+    (8192 x 4096, 6150 and 5200 rows in one launch, 2600 x 8192): the kernel that loads weights straight into registers (a ring
     of four super-blocks per lane, quads of lanes on contiguous runs of a row, ds_bpermute into the MFMA operand order)
     with the activations resident in LDS -- quantized by the workgroups themselves when x comes as f32.  Shapes that
     take every cut of the launch: waves sharing a row group two and fourteen ways (gate + up, down), row groups of their
