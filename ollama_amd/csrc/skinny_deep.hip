@@ -905,7 +905,10 @@ bool deep6_wanted(int type, int64_t K, int64_t M, int ncols, int num_cus) {
     size_t lds;
     if (!deep6_cut(K, (M + 15) / 16, ncols, num_cus, c, lds)) return false;
     if (M * (K / QKK) * (int64_t)Q6_QL >= ((int64_t)1 << 32)) return false;  // 32-bit lane offsets into the planes
-    return M * K > ((int64_t)40 << 20);
+    // from 4096 x 4096 at four columns and more, from 20 Mi weights at three (where the streaming kernel is the alternative):
+    // 6144 x 4096 at 3 / 4 / 8 columns 11.8 / 12.5 / 13.4 -> 7.6 / 8.7 / 11.5 us, 5120 x 5120 14.5 / 15.3 / 16.1 -> 9.8 / 10.4 / 13.0,
+    // 4096 x 4096 8.8 (kept) / 9.5 / 9.6 -> 8.7 / 9.4; 1024 x 4096 and 2048 x 8192 at three columns are behind here
+    return M * K >= ((int64_t)(ncols == 3 ? 20 : 16) << 20);
 }
 
 namespace {

@@ -369,9 +369,10 @@ def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
 
 
 @pytest.mark.parametrize("m,k,ns", [(4096, 14336, (3, 4, 5, 8)), (14336, 4096, (3, 6, 8)), (14330, 4096, (4, 7)), (4100, 14336 + 256, (5,)),
-                                    (8192, 8192, (4, 8)), (40000, 2048, (4, 5)), (65536 + 48, 1024, (3, 8))])
+                                    (8192, 8192, (4, 8)), (40000, 2048, (4, 5)), (65536 + 48, 1024, (3, 8)),
+                                    (4096, 4096, (4, 8)), (6150, 4096, (3, 5)), (5120, 5120, (3, 4, 7))])
 def test_q6k_deep_kernel_few_columns_on_large_matrices(ctx, m, k, ns):
-    """Q6_K at 3..8 columns on matrices beyond 40 M weights: the direct-load kernel on the Q6_K planes (low-nibble bytes,
+    """Q6_K at 4..8 columns on matrices from 16 Mi weights (three columns: from 20 Mi): the direct-load kernel on the Q6_K planes (low-nibble bytes,
     bit pairs, scales and row scales each loaded by the quad of lanes of a row, ds_bpermute into the MFMA operand order,
     the 6-bit quants multiplied as stored and the offset of 32 taken out with the block sums; one set of MFMAs up to
     four columns, two from five).  Waves sharing a row group fourteen and four ways (down, gate shape), row groups of
