@@ -92,6 +92,7 @@ struct DeepArgs {
 // how the launch is cut (computed on the host: the kernel's prologue has no division)
 struct DeepCut {
     int W, wpg, inv_wpg;  // waves per workgroup; waves that share a row group; ceil(256 / wpg): wave / wpg = wave * inv >> 8
+    int Wact;             // waves that stream weights (slots * wpg); waves Wact .. W-1 only help to quantize f32 x and leave
     int inv_nsb;          // ceil(65536 / nsb): b / nsb = b * inv >> 16 for the block numbers of up to eight columns
     int slots, ppw;       // row groups a workgroup holds at a time; pieces per wave
     int iters, grid;      // row groups per slot; workgroups
@@ -136,7 +137,8 @@ struct PieceRegs { unsigned hdr[PIECE]; u4v qa[PIECE], qb[PIECE]; };
 // SHARED: several waves share a row group (wpg > 1) and add their piece sums through LDS.
 // XF32: the activations come as f32 rows xf [nc][K] and the workgroup quantizes them to Q8_K itself, straight into its LDS
 // (the same block quantizer as the stand-alone kernel: the same bits), instead of copying quantized planes.
-template <bool SHARED, bool XF32>
+// HELP (with XF32): the workgroup is filled up to sixteen waves with helper waves (below).
+template <bool SHARED, bool XF32, bool HELP = false>
 __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, DevAct a, const float *__restrict__ xf, int col0, int nc,
                                                                     DeepCut cut) {
     typedef DeepGeo Geo;
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
             }
         }
     }
-    if (tid < 128) *reinterpret_cast<int *>(smem + 4 * tid) = 0;  // the zero block
+    if (tid < 64) *reinterpret_cast<int2 *>(smem + 8 * tid) = make_int2(0, 0);  // the zero block (a workgroup can be one wave)
 
     // ---- 2. the weight stream: a ring of four super-blocks per lane; a slot is requested again (for the same slot of
     // the wave's next piece) as soon as its super-block has been multiplied
@@ -235,11 +237,6 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
     // they are there.  So: the copies first; one super-block of weights per wave behind them (enough to start the
     // stream); the rest of the ring only when the activations have landed.
     if (XF32) {
-        // x is on its way (cache hits for all but the first workgroups to ask); one super-block of weights per wave goes
-        // out behind it, the rest of the ring after the quantization: a wave that requests more than the memory
-        // pipeline takes at once is held at the request, and could not quantize meanwhile
-        load_slot(L, lp, 0);
-        __builtin_amdgcn_sched_barrier(0);
         auto quantize_four = [&](int b0, const float4 (&v)[4]) __attribute__((always_inline)) {
             const int b = b0 + (lane >> 4), sub = lane & 15;
             float dd;
@@ -255,18 +252,33 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
                 if (sub == 0) *reinterpret_cast<float *>(smem + Geo::y_off(nsb) + cell * 4) = dd;
             }
         };
+        auto quantize_share = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < XR; t++)
-            if (4 * (wave + t * cut.W) < nblk) quantize_four(4 * (wave + t * cut.W), xq[t]);
-        for (int b0 = 4 * (wave + XR * cut.W); b0 < nblk; b0 += 4 * cut.W) {  // (more rounds than were requested ahead)
-            float4 v[4];
-            const int bc = min(b0 + (lane >> 4), nblk - 1);
+            for (int t = 0; t < XR; t++)
+                if (4 * (wave + t * cut.W) < nblk) quantize_four(4 * (wave + t * cut.W), xq[t]);
+            for (int b0 = 4 * (wave + XR * cut.W); b0 < nblk; b0 += 4 * cut.W) {  // (more rounds than were requested ahead)
+                float4 v[4];
+                const int bc = min(b0 + (lane >> 4), nblk - 1);
 #pragma unroll
-            for (int j = 0; j < 4; j++) v[j] = x4[bc * 64 + 4 * (lane & 15) + j];
-            quantize_four(b0, v);
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the LDS writes, before the barrier
+                for (int j = 0; j < 4; j++) v[j] = x4[bc * 64 + 4 * (lane & 15) + j];
+                quantize_four(b0, v);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the LDS writes, before the barrier
+        };
+        // Helper waves: a workgroup that streams with fewer than sixteen waves (few row groups per CU, a short K) has too
+        // few to quantize x in two or three rounds; the launch fills the workgroup up to sixteen, the extra waves take
+        // their share of the blocks and leave.  (A barrier waits for the waves that have not ended.)
+        // (A variant of its own: with the early exit in the code the full workgroups of the large products measured 0.15 to
+        // 0.5 us slower.)
+        const bool helper = HELP && wave >= cut.Wact;
+        // x is on its way (cache hits for all but the first workgroups to ask); one super-block of weights per wave goes
+        // out behind it, the rest of the ring after the quantization: a wave that requests more than the memory
+        // pipeline takes at once is held at the request, and could not quantize meanwhile
+        if (!helper) load_slot(L, lp, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        quantize_share();
         __builtin_amdgcn_s_barrier();
+        if (HELP && helper) return;
 #pragma unroll
         for (int i = 1; i < PIECE; i++) {
             load_slot(L, lp, i);
@@ -443,6 +455,17 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
     }
 }
 
+// Waves the f32 form launches per workgroup.  Each wave quantizes four blocks of x per round.  A workgroup that streams
+// with fewer than sixteen waves (few row groups per CU, a short K) is filled up to sixteen with helper waves -- they
+// take their share of the blocks and leave -- where that saves two rounds or more: 4096 x 4096 (four working waves) at
+// three / eight columns 8.3 / 8.4 -> 5.5 / 7.4 us, 8192 x 4096 (eight waves) at eight columns 9.2 -> 9.0; where it
+// saves one round or none the filled workgroup is 0.3 to 0.7 us slower (8192 x 4096 at three columns 6.5 -> 7.2,
+// 12288 x 4096 8.6 -> 9.3, 28672 x 4096 at eight 16.0 -> 16.1).
+int deep16_f32_waves(int ncols, int nsb, int working) {
+    auto rounds = [&](int waves) { return (ncols * nsb + 4 * waves - 1) / (4 * waves); };
+    return working < MAX_WAVES && rounds(working) - rounds(MAX_WAVES) >= 2 ? MAX_WAVES : working;
+}
+
 bool deep16_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, size_t &lds) {
     if (K % QKK || ncols < 1 || ncols > NCT || groups < 1 || groups > 0x7fffffff || num_cus < 1) return false;
     const int nsb = (int)(K / QKK), npieces = (nsb + PIECE - 1) / PIECE;
@@ -454,7 +477,7 @@ bool deep16_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, s
     c.inv_wpg = (256 + c.wpg - 1) / c.wpg;
     c.slots = MAX_WAVES / c.wpg;
     if (c.slots > per_cu) c.slots = (int)per_cu;
-    c.W = c.slots * c.wpg;
+    c.W = c.Wact = c.slots * c.wpg;
     c.grid = (int)std::min<int64_t>(num_cus, (groups + c.slots - 1) / c.slots);
     c.iters = (int)((groups + (int64_t)c.slots * c.grid - 1) / ((int64_t)c.slots * c.grid));
     for (int wv = 0; wv < c.W; wv++)
@@ -480,7 +503,14 @@ bool deep16_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus)
     // 10.5 / 11.0; on 4096 x 4096 this kernel is 5 % behind (8.4 against 8.0 us: its four waves per CU cannot quantize x
     // themselves).  (q + k + v of 4096 + 1024 + 1024 rows in one launch would take 7.8 / 10.5 us here against 12.7 / 13.0
     // staged, but a joint launch takes a kernel only when every matrix takes it alone, and alone they are too small.)
-    return ncols >= 5 && total_m * K >= ((int64_t)20 << 20) && (total_m + 15) / 16 < 6 * (int64_t)num_cus;
+    if (ncols >= 5 && total_m * K >= ((int64_t)20 << 20) && (total_m + 15) / 16 < 6 * (int64_t)num_cus) return true;
+    // Three to eight columns of anything smaller, where the workgroups can quantize f32 x themselves in three rounds (K up
+    // to 4096 at eight columns, 12288 at four): one launch instead of quantization + product, and that launch is what
+    // such a small product costs -- 4096 x 4096 at three / eight columns 7.2 / 8.0 -> 5.5 / 7.4 us, 1024 x 4096 7.2 / 7.8
+    // -> 5.4 / 7.2, 4096 x 1024 6.7 / 7.2 -> 4.5 / 4.5 against the direct-load and the staged kernel.  (From quantized
+    // planes this kernel is 0.2 to 0.7 us behind them on these shapes: 4096 x 4096 4.9 -> 5.4 us at three columns.)
+    return ncols >= 3 && (int64_t)ncols * (K / QKK) <= 3 * 4 * deep16_f32_waves(ncols, (int)(K / QKK), c.Wact) &&
+           (total_m + 15) / 16 < 6 * (int64_t)num_cus;
 }
 
 namespace {
@@ -504,15 +534,21 @@ hipError_t launch_deep16_any(const DevWeight *ws, float *const *ys, int count, c
     static bool allowed[64] = {false};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
-#define DEEP_ALLOW(SHARED, XF32) \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(deep16_q4k_kernel<SHARED, XF32>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+#define DEEP_ALLOW(...) \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(deep16_q4k_kernel<__VA_ARGS__>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
         DEEP_ALLOW(false, false); DEEP_ALLOW(true, false); DEEP_ALLOW(false, true); DEEP_ALLOW(true, true);
+        DEEP_ALLOW(false, true, true); DEEP_ALLOW(true, true, true);
 #undef DEEP_ALLOW
         allowed[dev] = true;
     }
     const DevAct none{};
+    const bool help = xf && deep16_f32_waves(ncols, g.nsb, c.Wact) > c.Wact;
+    if (help) c.W = MAX_WAVES;  // (waves beyond the working ones help to quantize x and leave)
     const dim3 grid((unsigned)c.grid), block(64 * c.W);
-    if (xf) {
+    if (help) {
+        if (c.wpg == 1) deep16_q4k_kernel<false, true, true><<<grid, block, lds, s>>>(g, none, xf, col0, ncols, c);
+        else deep16_q4k_kernel<true, true, true><<<grid, block, lds, s>>>(g, none, xf, col0, ncols, c);
+    } else if (xf) {
         if (c.wpg == 1) deep16_q4k_kernel<false, true><<<grid, block, lds, s>>>(g, none, xf, col0, ncols, c);
         else deep16_q4k_kernel<true, true><<<grid, block, lds, s>>>(g, none, xf, col0, ncols, c);
     } else {
@@ -630,7 +666,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g,
             }
         }
     }
-    if (tid < 128) *reinterpret_cast<int *>(smem + 4 * tid) = 0;  // the zero block
+    if (tid < 64) *reinterpret_cast<int2 *>(smem + 8 * tid) = make_int2(0, 0);  // the zero block (a workgroup can be one wave)
 
     // ---- 2. the weight stream: a ring of four super-blocks per lane
     // loading lane: its row and which piece of the quad's run it takes (rows 8..15 in the order 2 3 0 1, so that the
@@ -977,7 +1013,7 @@ bool deep16_f32_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_
     DeepCut c;
     size_t lds;
     if (!deep16_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds)) return false;
-    return (int64_t)ncols * (K / QKK) <= 3 * 4 * c.W;
+    return (int64_t)ncols * (K / QKK) <= 3 * 4 * deep16_f32_waves(ncols, (int)(K / QKK), c.Wact);
 }
 hipError_t launch_deep16_f32(const DevWeight *ws, float *const *ys, int count, const float *x, int ncols, int num_cus, hipStream_t s) {
     if (!x) return hipErrorInvalidValue;

@@ -368,6 +368,43 @@ def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
         W.free()
 
 
+@pytest.mark.parametrize("ms,k,ns", [([1], 256, (3, 5, 8)), ([7], 256, (3, 8)), ([16], 256, (4,)), ([33], 512, (3, 6)), ([100], 1024, (5,)),
+                                     ([1000], 1024, (3, 8)), ([300], 2048, (4, 7)), ([4096], 4096, (3, 4, 5, 8)),
+                                     ([4096, 1024, 1024], 4096, (3, 5, 8)), ([1030], 4096, (3, 8)), ([4096], 2048, (3, 8)),
+                                     ([4100], 8192, (3, 5)), ([20000], 1024, (4, 8)), ([12288], 4096, (3, 8)), ([2048], 12288, (3,))])
+def test_q4k_deep_kernel_on_small_products(ctx, ms, k, ns):
+    """Q4_K at 3..8 columns on products small enough that the workgroups quantize f32 x themselves in three rounds: the
+    same direct-load kernel.  Workgroups of a single wave (K up to 1024 with at most a row group per CU: the zero block
+    of the LDS map is then one wave's to write), of two and four working waves filled up with helper waves that
+    quantize their share of x and leave (4096 x 4096, the q + k + v launch, 4096 x 2048), of eight and twelve working
+    waves with and without helpers (8192-long rows, 12288 x 4096), matrices of one row, of 7, of ragged last row
+    groups.  Against the oracle and exact arithmetic; the f32 form gives the bits of quantize-then-multiply; a joint
+    launch gives the bits of the single ones; a column's result does not depend on which other columns ride along."""
+    rng = np.random.default_rng(9500 + sum(ms) + k)
+    raws = [_weights(Q4_K, m, k, seed=9501 + m + i) for i, m in enumerate(ms)]
+    Ws = [ctx.upload(Q4_K, r, k, m) for r, m in zip(raws, ms)]
+    act = ctx.act_create(Q8_K, k, 8)
+    for n in ns:
+        assert all(ctx.route(W, n) == "deep_f32" for W in Ws), (ms, k, n)
+        x = rng.standard_normal((n, k), dtype=np.float32)
+        x[0, :256] = 0.0                                               # an all-zero block
+        got = ctx.mulmat_multi(Ws, x) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x)]
+        ctx.act_quantize(act, x)
+        for y, W, raw, m in zip(got, Ws, raws, ms):
+            assert ctx.route_q8(W, act) == "skinny_deep", (m, k, n)
+            assert npref.rel_err(y, oracle.mul_mat(Q4_K, raw, k, m, x, nthreads=16)) < TOL, (m, n)
+            _check_against_exact_arithmetic(Q4_K, raw, k, m, x, y, f"Q4_K {m}x{k} n={n}", max_rows=2048)
+            assert np.array_equal(ctx.mulmat_q8(W, act), y), ("f32 != planes", m, n)
+            if len(Ws) > 1:
+                assert np.array_equal(ctx.mulmat(W, x), y), ("joint != alone", m, n)
+        again = ctx.mulmat_multi(Ws, x[::-1].copy()) if len(Ws) > 1 else [ctx.mulmat(Ws[0], x[::-1].copy())]
+        for y, z in zip(got, again):
+            assert np.array_equal(z[::-1], y), n
+    act.free()
+    for W in Ws:
+        W.free()
+
+
 @pytest.mark.parametrize("m,k,ns", [(4096, 14336, (3, 4, 5, 8)), (14336, 4096, (3, 6, 8)), (14330, 4096, (4, 7)), (4100, 14336 + 256, (5,)),
                                     (8192, 8192, (4, 8)), (40000, 2048, (4, 5)), (65536 + 48, 1024, (3, 8)),
                                     (4096, 4096, (4, 8)), (6150, 4096, (3, 5)), (5120, 5120, (3, 4, 7))])

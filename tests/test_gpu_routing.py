@@ -29,10 +29,13 @@ def _upload_any(ctx, t, m, k):
 
 # (weight type, rows, K) -> {activation rows: kernel}; the decode / prefill shapes of a Llama-3-8B layer and its head
 TABLE = [
-    ("q_proj", Q4_K, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "skinny_direct", 4: "skinny_direct", 8: "skinny_staged",
+    ("q_proj", Q4_K, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "deep_f32", 8: "deep_f32",
                                   16: "skinny_staged", 32: "gemm_int8", 256: "gemm_int8", 512: "gemm_f16", 2048: "gemm_f16"}),
-    ("k_proj", Q4_K, 1024, 4096, {1: "gemv_f32", 4: "skinny_direct", 8: "skinny_staged", 512: "gemm_int8"}),
-    ("Q4_K 8192x4096", Q4_K, 8192, 4096, {1: "gemv_f32", 4: "skinny_direct", 5: "deep_f32", 8: "skinny_deep", 16: "skinny_staged"}),
+    ("k_proj", Q4_K, 1024, 4096, {1: "gemv_f32", 4: "deep_f32", 8: "deep_f32", 512: "gemm_int8"}),
+    ("Q4_K 8192x4096", Q4_K, 8192, 4096, {1: "gemv_f32", 4: "deep_f32", 5: "deep_f32", 8: "deep_f32", 16: "skinny_staged"}),
+    ("Q4_K 4096x8192", Q4_K, 4096, 8192, {3: "deep_f32", 5: "deep_f32", 8: "skinny_deep"}),
+    ("Q4_K 20000x1024", Q4_K, 20000, 1024, {3: "deep_f32", 8: "deep_f32"}),
+    ("Q4_K 40000x1024", Q4_K, 40000, 1024, {3: "skinny_direct", 8: "skinny_rows_q4k"}),
     ("ffn_gate", Q4_K, 14336, 4096, {1: "gemv_f32", 2: "deep_f32", 3: "deep_f32", 4: "deep_f32", 8: "deep_f32",
                                      16: "skinny_staged", 32: "gemm_int8", 512: "gemm_f16"}),
     ("ffn_down Q4_K", Q4_K, 4096, 14336, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "skinny_deep", 8: "skinny_deep",
