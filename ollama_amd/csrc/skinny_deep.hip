@@ -611,7 +611,8 @@ struct Deep6Geo {
 struct Piece6Regs { unsigned sc[PIECE], d[PIECE]; u4v qa[PIECE], qb[PIECE], qh[PIECE]; };
 
 // XF32: f32 activations xf [nc][K], quantized by the workgroup itself (as in the Q4_K kernel above).
-template <bool SHARED, int SETS, bool XF32>
+// HELP (with XF32): helper waves fill the workgroup up to sixteen, as above.
+template <bool SHARED, int SETS, bool XF32, bool HELP = false>
 __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g, DevAct a, const float *__restrict__ xf, int col0, int nc,
                                                                     DeepCut cut) {
     typedef Deep6Geo<SETS> Geo;
@@ -706,7 +707,8 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g,
     ItemAt L = item_at(lgroup);
     // the copies first; one super-block of weights per wave behind them; the rest of the ring when the activations
     // have landed (requests are served roughly in the order they were made)
-    load_slot(L, lp, 0);
+    const bool helper = HELP && wave >= cut.Wact;  // (quantizes its share of x and leaves)
+    if (!helper) load_slot(L, lp, 0);
     __builtin_amdgcn_sched_barrier(0);
     if (XF32) {
         auto quantize_four = [&](int b0, const float4 (&v)[4]) __attribute__((always_inline)) {
@@ -739,6 +741,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g,
         asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");  // (loads retire in order: all but the five weight loads)
     }
     __builtin_amdgcn_s_barrier();
+    if (HELP && helper) return;
 #pragma unroll
     for (int i = 1; i < PIECE; i++) {
         load_slot(L, lp, i);
@@ -921,7 +924,7 @@ bool deep6_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, si
     c.inv_wpg = (256 + c.wpg - 1) / c.wpg;
     c.slots = MAX_WAVES / c.wpg;
     if (c.slots > per_cu) c.slots = (int)per_cu;
-    c.W = c.slots * c.wpg;
+    c.W = c.Wact = c.slots * c.wpg;
     c.grid = (int)std::min<int64_t>(num_cus, (groups + c.slots - 1) / c.slots);
     c.iters = (int)((groups + (int64_t)c.slots * c.grid - 1) / ((int64_t)c.slots * c.grid));
     for (int wv = 0; wv < c.W; wv++)
@@ -942,9 +945,15 @@ bool deep6_wanted(int type, int64_t K, int64_t M, int ncols, int num_cus) {
     if (!deep6_cut(K, (M + 15) / 16, ncols, num_cus, c, lds)) return false;
     if (M * (K / QKK) * (int64_t)Q6_QL >= ((int64_t)1 << 32)) return false;  // 32-bit lane offsets into the planes
     // from 4096 x 4096 at four columns and more, from 20 Mi weights at three (where the streaming kernel is the alternative):
-    // 6144 x 4096 at 3 / 4 / 8 columns 11.8 / 12.5 / 13.4 -> 7.6 / 8.7 / 11.5 us, 5120 x 5120 14.5 / 15.3 / 16.1 -> 9.8 / 10.4 / 13.0,
-    // 4096 x 4096 8.8 (kept) / 9.5 / 9.6 -> 8.7 / 9.4; 1024 x 4096 and 2048 x 8192 at three columns are behind here
-    return M * K >= ((int64_t)(ncols == 3 ? 20 : 16) << 20);
+    // 6144 x 4096 at 3 / 4 / 8 columns 11.8 / 12.5 / 13.4 -> 7.6 / 8.7 / 11.5 us, 5120 x 5120 14.5 / 15.3 / 16.1 -> 9.8 / 10.4 / 13.0
+    if (M * K >= ((int64_t)(ncols == 3 ? 20 : 16) << 20)) return true;
+    // anything smaller (below 24576 rows) where the workgroups can quantize f32 x themselves in two rounds, with helper
+    // waves where they stream with few: one launch instead of quantization + product.  f32 x in, 3 / 4 / 8 columns:
+    // 4096 x 4096 8.9 / 8.7 / 9.4 -> 6.4 / 6.4 / 8.5 us, 1024 x 4096 7.3 / 8.2 / 8.4 -> 5.9 / 6.0 / 7.9, 4096 x 1024 7.0 / 7.1 / 7.3 ->
+    // 5.0 / 5.2 / 5.5.  (From quantized planes: within 0.3 us of the streaming kernel at three columns, 0.9 us ahead of
+    // the staged kernel at four on K = 4096, 0.8 to 1.0 us behind it at five to eight columns of K up to 2048.)
+    const int nsb = (int)(K / QKK);
+    return (int64_t)ncols * nsb <= 2 * 4 * deep16_f32_waves(ncols, nsb, c.Wact) && (M + 15) / 16 < 6 * (int64_t)num_cus;
 }
 
 namespace {
@@ -960,19 +969,23 @@ hipError_t launch_deep6_any(const DevWeight &w, float *y, const DevAct *a, const
     static bool allowed[64] = {false};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
-#define DEEP_ALLOW(SHARED, SETS, XF32) \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(deep16_q6k_kernel<SHARED, SETS, XF32>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+#define DEEP_ALLOW(...) \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(deep16_q6k_kernel<__VA_ARGS__>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
         DEEP_ALLOW(false, 1, false); DEEP_ALLOW(true, 1, false); DEEP_ALLOW(false, 2, false); DEEP_ALLOW(true, 2, false);
         DEEP_ALLOW(false, 1, true); DEEP_ALLOW(true, 1, true); DEEP_ALLOW(false, 2, true); DEEP_ALLOW(true, 2, true);
+        DEEP_ALLOW(false, 1, true, true); DEEP_ALLOW(true, 1, true, true); DEEP_ALLOW(false, 2, true, true); DEEP_ALLOW(true, 2, true, true);
 #undef DEEP_ALLOW
         allowed[dev] = true;
     }
     const DevAct none{};
     const DevAct &da = a ? *a : none;
+    const bool help = xf && deep16_f32_waves(ncols, g.nsb, c.Wact) > c.Wact;
+    if (help) c.W = MAX_WAVES;  // (waves beyond the working ones help to quantize x and leave)
     const dim3 grid((unsigned)c.grid), block(64 * c.W);
 #define DEEP_GO(SHARED, SETS) \
     do { \
-        if (xf) deep16_q6k_kernel<SHARED, SETS, true><<<grid, block, lds, s>>>(g, da, xf, col0, ncols, c); \
+        if (help) deep16_q6k_kernel<SHARED, SETS, true, true><<<grid, block, lds, s>>>(g, da, xf, col0, ncols, c); \
+        else if (xf) deep16_q6k_kernel<SHARED, SETS, true><<<grid, block, lds, s>>>(g, da, xf, col0, ncols, c); \
         else deep16_q6k_kernel<SHARED, SETS, false><<<grid, block, lds, s>>>(g, da, nullptr, col0, ncols, c); \
     } while (0)
     if (ncols <= 4) {
@@ -1007,7 +1020,7 @@ bool deep16_f32_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_
         DeepCut c;
         size_t lds;
         return deep6_wanted(type, K, total_m, ncols, num_cus) && deep6_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds) &&
-               (int64_t)ncols * (K / QKK) <= 2 * 4 * c.W;
+               (int64_t)ncols * (K / QKK) <= 2 * 4 * deep16_f32_waves(ncols, (int)(K / QKK), c.Wact);
     }
     if (!deep16_wanted(type, K, total_m, ncols, num_cus)) return false;
     DeepCut c;

@@ -407,9 +407,14 @@ def test_q4k_deep_kernel_on_small_products(ctx, ms, k, ns):
 
 @pytest.mark.parametrize("m,k,ns", [(4096, 14336, (3, 4, 5, 8)), (14336, 4096, (3, 6, 8)), (14330, 4096, (4, 7)), (4100, 14336 + 256, (5,)),
                                     (8192, 8192, (4, 8)), (40000, 2048, (4, 5)), (65536 + 48, 1024, (3, 8)),
-                                    (4096, 4096, (4, 8)), (6150, 4096, (3, 5)), (5120, 5120, (3, 4, 7))])
+                                    (4096, 4096, (3, 4, 8)), (6150, 4096, (3, 5)), (5120, 5120, (3, 4, 7)),
+                                    (1, 256, (3, 5, 8)), (7, 256, (3, 8)), (33, 512, (4, 6)), (1000, 1024, (3, 8)), (300, 2048, (4, 7)),
+                                    (1030, 4096, (3, 4, 5, 8)), (4096, 2048, (3, 8)), (20000, 1024, (4, 8)), (8200, 4096, (3, 4))])
 def test_q6k_deep_kernel_few_columns_on_large_matrices(ctx, m, k, ns):
-    """Q6_K at 4..8 columns on matrices from 16 Mi weights (three columns: from 20 Mi): the direct-load kernel on the Q6_K planes (low-nibble bytes,
+    """Q6_K at 4..8 columns on matrices from 16 Mi weights (three columns: from 20 Mi), and on the smaller ones whose
+    f32 x the workgroups quantize themselves in two rounds (workgroups of a single wave; of one to eight working waves
+    filled up with helper waves that quantize their share and leave; matrices of one row, of 7, ragged last row
+    groups): the direct-load kernel on the Q6_K planes (low-nibble bytes,
     bit pairs, scales and row scales each loaded by the quad of lanes of a row, ds_bpermute into the MFMA operand order,
     the 6-bit quants multiplied as stored and the offset of 32 taken out with the block sums; one set of MFMAs up to
     four columns, two from five).  Waves sharing a row group fourteen and four ways (down, gate shape), row groups of
@@ -596,12 +601,14 @@ def test_long_rows_at_one_column(ctx, t, k):
         # the waves of a mostly empty last segment take rows side by side at one and two columns only: at three
         # columns every wave takes one row per load, and column 0 must come out with the same bits (not Q4_K: its
         # three-column products do not reproduce the one-column bits at any K, with or without a short last segment,
-        # so they say nothing here)
+        # so they say nothing here; nor Q6_K rows short enough that three columns take the deep direct-load kernel)
         if t != Q4_K:
             x3 = np.concatenate([x, rng.standard_normal((2, k), dtype=np.float32)])
             ctx.act_quantize(act3, x3)
+            assert t != Q6_K or (ctx.route_q8(Ws[4], act3) == "gemv") == (k > 10752)
             for W, wnt in zip(Ws, want):
-                assert np.array_equal(ctx.mulmat_q8(W, act3, path=qmm.PATH_GEMV)[:1], wnt)
+                if t != Q6_K or ctx.route_q8(W, act3) == "gemv":
+                    assert np.array_equal(ctx.mulmat_q8(W, act3, path=qmm.PATH_GEMV)[:1], wnt)
     act.free()
     act3.free()
     for W in Ws:
