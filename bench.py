@@ -409,6 +409,7 @@ def main() -> int:
                                            ("Q4_0 GEMV 4096x4096", Q4_0, 4096, 4096, (1,), 40),
                                            ("Q8_0 skinny 4096x4096", Q8_0, 4096, 4096, (1, 2, 4, 8), 40),
                                            ("Q6_K ffn_down 4096x14336", Q6_K, 4096, 14336, (4, 8), 10),
+                                           ("Q6_K v_proj 1024x4096", Q6_K, 1024, 4096, (4, 8), 40),
                                            ("Q6_K head 128256x4096", Q6_K, 128256, 4096, (1, 8), 3)):
             for n in ns:
                 tm, wb = time_mulmat(t, m, k, n, copies)
