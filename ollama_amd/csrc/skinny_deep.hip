@@ -93,7 +93,7 @@ struct DeepArgs {
 struct DeepCut {
     int W, wpg, inv_wpg;  // waves per workgroup; waves that share a row group; ceil(256 / wpg): wave / wpg = wave * inv >> 8
     int Wact;             // waves that stream weights (slots * wpg); waves Wact .. W-1 only help to quantize f32 x and leave
-    int inv_nsb;          // ceil(65536 / nsb): b / nsb = b * inv >> 16 for the block numbers of up to eight columns
+    int inv_nsb;          // ceil(2^20 / nsb): b / nsb = b * inv >> 20 for the block numbers of up to eight columns
     int slots, ppw;       // row groups a workgroup holds at a time; pieces per wave
     int iters, grid;      // row groups per slot; workgroups
 };
@@ -120,13 +120,14 @@ __device__ __forceinline__ DeepWhere deep_where(const DeepArgs &g, int group) {
 __device__ __host__ constexpr int a_swz(int col) { return 2 * ((col & 1) + 2 * (col >> 2)) & 6; }
 static_assert(a_swz(0) == 0 && a_swz(1) == 2 && a_swz(6) == 4 && a_swz(7) == 6 && a_swz(2) == 0 && a_swz(3) == 2 &&
               a_swz(4) == 4 && a_swz(5) == 6, "column swizzle");
+// ncs: the columns the layout holds per super-block, 4 (launches of up to four columns) or 8.
 struct DeepGeo {
     static constexpr int A_OFF = 512;
-    static __host__ __device__ constexpr int dg_off(int nsb) { return A_OFF + nsb * NCT * 256; }
-    static __host__ __device__ constexpr int y_off(int nsb) { return dg_off(nsb) + nsb * NCT * 16; }
-    static __host__ __device__ constexpr int part_off(int nsb) { return (y_off(nsb) + nsb * NCT * 4 + 255) / 256 * 256; }
-    static __host__ __device__ constexpr size_t lds_bytes(int nsb, int slots, int npieces, bool shared_groups) {
-        return (size_t)part_off(nsb) + (shared_groups ? (size_t)slots * npieces * NCT * 16 * 4 : 0);
+    static __host__ __device__ constexpr int dg_off(int nsb, int ncs) { return A_OFF + nsb * ncs * 256; }
+    static __host__ __device__ constexpr int y_off(int nsb, int ncs) { return dg_off(nsb, ncs) + nsb * ncs * 16; }
+    static __host__ __device__ constexpr int part_off(int nsb, int ncs) { return (y_off(nsb, ncs) + nsb * ncs * 4 + 255) / 256 * 256; }
+    static __host__ __device__ constexpr size_t lds_bytes(int nsb, int ncs, int slots, int npieces, bool shared_groups) {
+        return (size_t)part_off(nsb, ncs) + (shared_groups ? (size_t)slots * npieces * NCT * 16 * 4 : 0);
     }
 };
 
@@ -156,6 +157,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
 
     // ---- 1. the activations, requested first: quants, block-sum digits, block scales -> LDS
     const int nblk = nc * nsb;  // Q8_K blocks of the launch's columns; block b = column b / nsb, super-block b % nsb
+    const int ncs_log2 = nc > 4 ? 3 : 2, ncs = 1 << ncs_log2;  // columns of the LDS layout
     const float4 *x4 = reinterpret_cast<const float4 *>(xf) + (int64_t)col0 * nsb * 64;
     // f32 input: four blocks per wave and round (block 4 (wave + round * W) + lane / 16), sixteen lanes a block, sixteen
     // consecutive elements a lane; the first XR rounds are requested here, ahead of the weights
@@ -177,22 +179,22 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
         // columns 0..3 and 4..7), then the digits and the scales (64 (super-block, column) cells per instruction)
         // (columns past nc are not copied: the lanes of the A operand that stand for them read zeros)
         const int sets = nc > 4 ? 2 : 1;
-        const int cells = nsb * NCT, n_q = nsb * sets, n_c = (cells + 63) / 64;
+        const int cells = nsb * ncs, n_q = nsb * sets, n_c = (cells + 63) / 64;
         for (int n = wave; n < n_q + 2 * n_c; n += cut.W) {
             if (n < n_q) {
                 const int sb = sets == 2 ? n >> 1 : n, j = sets == 2 ? n & 1 : 0;
                 const int col = 4 * j + (lane >> 4), pc = (lane & 15) ^ a_swz(col);
                 if (col < nc)
                     dma_lds<16>(aq + (int64_t)sb * QKK, (unsigned)acol(col) * (unsigned)a.K + 16u * pc,
-                                sm + Geo::A_OFF + (unsigned)(sb * NCT + 4 * j) * 256u);
+                                sm + Geo::A_OFF + (unsigned)(sb * ncs + 4 * j) * 256u);
             } else {
                 const bool digits = n < n_q + n_c;
                 const int c0 = 64 * (digits ? n - n_q : n - n_q - n_c);
-                const int cell = min(c0 + lane, cells - 1), sb = cell / NCT, col = cell % NCT;
+                const int cell = min(c0 + lane, cells - 1), sb = cell >> ncs_log2, col = cell & (ncs - 1);
                 const unsigned at = (unsigned)acol(col) * (unsigned)nsb + (unsigned)sb;
                 if (c0 + lane < cells) {
-                    if (digits) dma_lds<16>(a.sd8, at * 16u, sm + Geo::dg_off(nsb) + 16u * c0);
-                    else dma_lds<4>(reinterpret_cast<const uint8_t *>(a.d), at * 4u, sm + Geo::y_off(nsb) + 4u * c0);
+                    if (digits) dma_lds<16>(a.sd8, at * 16u, sm + Geo::dg_off(nsb, ncs) + 16u * c0);
+                    else dma_lds<4>(reinterpret_cast<const uint8_t *>(a.d), at * 4u, sm + Geo::y_off(nsb, ncs) + 4u * c0);
                 }
             }
         }
@@ -243,13 +245,13 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
             int sum16, pair;
             const uint4 packed = q8_K_quantize_row16(v, lane, dd, sum16, pair);
             if (b < nblk) {  // the last four may end early: whole rows of 16 lanes drop out
-                const int col = (b * cut.inv_nsb) >> 16, sb = b - col * nsb, cell = sb * NCT + col;
+                const int col = (b * cut.inv_nsb) >> 20, sb = b - col * nsb, cell = sb * ncs + col;
                 *reinterpret_cast<uint4 *>(smem + Geo::A_OFF + cell * 256 + 16 * (sub ^ a_swz(col))) = packed;
                 if ((sub & 1) == 0) {  // the sum of a sub-block of 32 as two digits, S = 64 * (S >> 6) + (S & 63)
-                    smem[Geo::dg_off(nsb) + cell * 16 + (sub >> 1)] = (uint8_t)(pair & 63);
-                    smem[Geo::dg_off(nsb) + cell * 16 + 8 + (sub >> 1)] = (uint8_t)(pair >> 6);
+                    smem[Geo::dg_off(nsb, ncs) + cell * 16 + (sub >> 1)] = (uint8_t)(pair & 63);
+                    smem[Geo::dg_off(nsb, ncs) + cell * 16 + 8 + (sub >> 1)] = (uint8_t)(pair >> 6);
                 }
-                if (sub == 0) *reinterpret_cast<float *>(smem + Geo::y_off(nsb) + cell * 4) = dd;
+                if (sub == 0) *reinterpret_cast<float *>(smem + Geo::y_off(nsb, ncs) + cell * 4) = dd;
             }
         };
         auto quantize_share = [&]() __attribute__((always_inline)) {
@@ -306,18 +308,21 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
     const int rsw = (r >> 3) << 1;            // (rows 8..15 were loaded with their pieces in the order 2 3 0 1)
     const int bidx = 4 * (4 * r + (kg ^ rsw));  // ds_bpermute: the lane that loaded what this lane multiplies
     unsigned a0_at, a_st, d_at, d_st, y_at;
+    const unsigned y_st = (unsigned)ncs * 4;
     {
         const int col = r >> 1, w = r & 1;  // A row r: column, which of the MFMA's two sub-blocks
         const bool a_on = col < nc && (kg >> 1) == w;
         const bool d_on = col < nc && kg == 0;  // low digits in A row 2c, high digits in row 2c + 1
         const int s0 = (4 * (kg >> 1) + (kg & 1)) ^ a_swz(col);  // slot of the lane's first piece; the others: ^2, ^8, ^10
         a0_at = sm + (a_on ? Geo::A_OFF + col * 256 + 16 * s0 : 128);
-        a_st = a_on ? NCT * 256 : 0;
-        d_at = sm + (d_on ? Geo::dg_off(nsb) + col * 16 + 8 * w : 0);
-        d_st = d_on ? NCT * 16 : 0;
-        y_at = sm + Geo::y_off(nsb) + 4 * min(2 * kg, NCT - 2);  // the two columns this lane's outputs belong to
+        a_st = a_on ? ncs * 256 : 0;
+        d_at = sm + (d_on ? Geo::dg_off(nsb, ncs) + col * 16 + 8 * w : 0);
+        d_st = d_on ? ncs * 16 : 0;
+        // the two columns this lane's outputs belong to (a layout of four columns: K groups 2, 3 read those of columns 2, 3,
+        // their outputs are dropped)
+        y_at = sm + Geo::y_off(nsb, ncs) + 4 * min(2 * kg, ncs - 2);
     }
-    float *part = reinterpret_cast<float *>(smem + Geo::part_off(nsb));  // [slot][piece][NCT][16]
+    float *part = reinterpret_cast<float *>(smem + Geo::part_off(nsb, ncs));  // [slot][piece][NCT][16]
 
     const v4i zero = {0, 0, 0, 0};
     // one super-block (ring slot i) into the piece's accumulators; aa0 / da: the lane's LDS addresses of its first operand
@@ -325,7 +330,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q4k_kernel(DeepArgs g, 
     auto mul_slot = [&](int i, int sb, unsigned aa0, unsigned da, float (&acc)[2]) __attribute__((always_inline)) {
         const unsigned aa1 = aa0 ^ 32u;  // (slots s0 and s0 ^ 2; every base is a multiple of 64)
         const v2i dg = lds_at<v2i>(da, 0);
-        const v2f yd = lds_at<v2f>(y_at + (unsigned)sb * (NCT * 4), 0);
+        const v2f yd = lds_at<v2f>(y_at + (unsigned)sb * y_st, 0);
         u4v hdr;  // the four dwords of the row's header, from the four lanes of the quad that loaded it
 #pragma unroll
         for (int j = 0; j < 4; j++) hdr[j] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * (4 * r) + 4 * (j ^ rsw), (int)R.hdr[i]);
@@ -482,18 +487,20 @@ bool deep16_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, s
     c.iters = (int)((groups + (int64_t)c.slots * c.grid - 1) / ((int64_t)c.slots * c.grid));
     for (int wv = 0; wv < c.W; wv++)
         if (((wv * c.inv_wpg) >> 8) != wv / c.wpg) return false;  // (never: checked for every wpg up to 16)
-    c.inv_nsb = (65536 + nsb - 1) / nsb;
+    c.inv_nsb = ((1 << 20) + nsb - 1) / nsb;
     for (int b = 0; b < NCT * nsb; b++)
-        if (((b * c.inv_nsb) >> 16) != b / nsb) return false;  // (exact while 8 nsb^2 < 65536: K up to 23040)
-    lds = DeepGeo::lds_bytes(nsb, c.slots, npieces, c.wpg > 1);
+        if (((b * c.inv_nsb) >> 20) != b / nsb) return false;  // (exact while 8 nsb^2 < 2^20: every K whose activations fit the LDS)
+    lds = DeepGeo::lds_bytes(nsb, ncols > 4 ? 8 : 4, c.slots, npieces, c.wpg > 1);
     return lds <= 160 * 1024;
 }
 
 }  // namespace
 
 bool deep16_wanted(int type, int64_t K, int64_t total_m, int ncols, int num_cus) {
-    // two columns only on rows of one K segment: on longer rows the streaming kernel with its in-kernel quantization is ahead
-    if (type != T_Q4_K || ncols < 2 || (ncols == 2 && K > 4096)) return false;
+    // two columns only on rows of one K segment: on longer rows the streaming kernel with its in-kernel quantization is
+    // ahead -- where it applies (rows of 28672 are beyond it: 8192 x 28672 at two columns 44.9 us through quantization +
+    // GEMV, 32 here)
+    if (type != T_Q4_K || ncols < 2 || (ncols == 2 && K > 4096 && gemv_f32_supported(type, K, total_m, 2))) return false;
     DeepCut c;
     size_t lds;
     if (!deep16_cut(K, (total_m + 15) / 16, ncols, num_cus, c, lds)) return false;
@@ -717,7 +724,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void deep16_q6k_kernel(Deep6Args g,
             int sum16, pair;
             const uint4 packed = q8_K_quantize_row16(v, lane, dd, sum16, pair);
             if (b < nblk) {  // the last four may end early: whole rows of 16 lanes drop out
-                const int col = (b * cut.inv_nsb) >> 16, sb = b - col * nsb, cell = sb * NC + col;
+                const int col = (b * cut.inv_nsb) >> 20, sb = b - col * nsb, cell = sb * NC + col;
                 *reinterpret_cast<uint4 *>(smem + Geo::A_OFF + cell * 256 + 16 * (sub16 ^ (col & 2))) = packed;
                 // the sum of the lane's 16 quants as two digits, S = 64 * (S >> 6) + (S & 63)
                 smem[Geo::dg_off(nsb) + cell * 32 + sub16] = (uint8_t)(sum16 & 63);
@@ -929,9 +936,9 @@ bool deep6_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, si
     c.iters = (int)((groups + (int64_t)c.slots * c.grid - 1) / ((int64_t)c.slots * c.grid));
     for (int wv = 0; wv < c.W; wv++)
         if (((wv * c.inv_wpg) >> 8) != wv / c.wpg) return false;
-    c.inv_nsb = (65536 + nsb - 1) / nsb;
+    c.inv_nsb = ((1 << 20) + nsb - 1) / nsb;
     for (int b = 0; b < 8 * nsb; b++)
-        if (((b * c.inv_nsb) >> 16) != b / nsb) return false;
+        if (((b * c.inv_nsb) >> 20) != b / nsb) return false;
     lds = ncols <= 4 ? Deep6Geo<1>::lds_bytes(nsb, c.slots, npieces, c.wpg > 1) : Deep6Geo<2>::lds_bytes(nsb, c.slots, npieces, c.wpg > 1);
     return lds <= 160 * 1024;
 }
@@ -939,7 +946,8 @@ bool deep6_cut(int64_t K, int64_t groups, int ncols, int num_cus, DeepCut &c, si
 }  // namespace
 
 bool deep6_wanted(int type, int64_t K, int64_t M, int ncols, int num_cus) {
-    if (type != T_Q6_K || ncols < DEEP6_FROM || ncols > 8) return false;
+    // (two columns only where the streaming kernel cannot quantize x itself: rows of 28672)
+    if (type != T_Q6_K || ncols > 8 || ncols < (gemv_f32_supported(type, K, M, 2) ? DEEP6_FROM : 2)) return false;
     DeepCut c;
     size_t lds;
     if (!deep6_cut(K, (M + 15) / 16, ncols, num_cus, c, lds)) return false;

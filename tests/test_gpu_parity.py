@@ -332,7 +332,8 @@ def test_q4k_rows_kernel_alone_and_joint(ctx, ms, k, ns):
 @pytest.mark.parametrize("ms,k,ns", [([14336, 14336], 4096, (2, 3, 4, 8)), ([14336], 4096, (2, 5)), ([4096], 14336, (3, 4, 7, 8)),
                                      ([14330, 5000], 4096, (6,)), ([4100], 14336 + 256, (5,)), ([8192], 8192, (4, 8)),
                                      ([70000], 4096, (2, 3, 8)), ([40000, 33000], 2048, (2, 5)), ([131072 + 48], 1024, (8,)),
-                                     ([8192], 4096, (5, 8)), ([6150, 5200], 4096, (6,)), ([2600], 8192, (7,))])
+                                     ([8192], 4096, (5, 8)), ([6150, 5200], 4096, (6,)), ([2600], 8192, (7,)),
+                                     ([4100], 28672, (2, 3, 4))])
 def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
     """Q4_K at 3..8 columns (from two on rows up to 4096) on matrices beyond 40 M weights, and at 5..8 columns from 20 M
     (8192 x 4096, 6150 and 5200 rows in one launch, 2600 x 8192): the kernel that loads weights straight into registers (a ring
@@ -340,7 +341,8 @@ def test_q4k_deep_kernel_few_columns_on_large_matrices(ctx, ms, k, ns):
     with the activations resident in LDS -- quantized by the workgroups themselves when x comes as f32.  Shapes that
     take every cut of the launch: waves sharing a row group two and fourteen ways (gate + up, down), row groups of their
     own (70000 and 131120 rows: two row groups per wave in turn), a last piece of one super-block (K = 14592), ragged
-    last row groups, two matrices of unequal size.  Against the oracle and exact arithmetic; the f32 form gives the bits
+    last row groups, two matrices of unequal size, rows of 28672 (their activations fit the LDS at up to four columns:
+    the layout then holds four columns per super-block).  Against the oracle and exact arithmetic; the f32 form gives the bits
     of quantize-then-multiply; a joint launch gives the bits of the single ones; a column's result does not depend on
     which other columns ride along."""
     rng = np.random.default_rng(9100 + sum(ms) + k)
@@ -409,7 +411,8 @@ def test_q4k_deep_kernel_on_small_products(ctx, ms, k, ns):
                                     (8192, 8192, (4, 8)), (40000, 2048, (4, 5)), (65536 + 48, 1024, (3, 8)),
                                     (4096, 4096, (3, 4, 8)), (6150, 4096, (3, 5)), (5120, 5120, (3, 4, 7)),
                                     (1, 256, (3, 5, 8)), (7, 256, (3, 8)), (33, 512, (4, 6)), (1000, 1024, (3, 8)), (300, 2048, (4, 7)),
-                                    (1030, 4096, (3, 4, 5, 8)), (4096, 2048, (3, 8)), (20000, 1024, (4, 8)), (8200, 4096, (3, 4))])
+                                    (1030, 4096, (3, 4, 5, 8)), (4096, 2048, (3, 8)), (20000, 1024, (4, 8)), (8200, 4096, (3, 4)),
+                                    (2100, 28672, (2, 3, 4))])
 def test_q6k_deep_kernel_few_columns_on_large_matrices(ctx, m, k, ns):
     """Q6_K at 4..8 columns on matrices from 16 Mi weights (three columns: from 20 Mi), and on the smaller ones whose
     f32 x the workgroups quantize themselves in two rounds (workgroups of a single wave; of one to eight working waves

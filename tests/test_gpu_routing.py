@@ -47,6 +47,8 @@ TABLE = [
     ("Q6_K 4096^2", Q6_K, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "deep_f32", 4: "deep_f32", 8: "deep_f32", 16: "skinny_staged"}),
     ("Q6_K 2048x8192", Q6_K, 2048, 8192, {3: "gemv", 4: "deep_f32", 5: "skinny_deep"}),
     ("Q6_K 6144x4096", Q6_K, 6144, 4096, {2: "gemv_f32", 3: "deep_f32", 4: "deep_f32", 5: "skinny_deep", 8: "deep_f32"}),
+    ("70B ffn_down Q4_K", Q4_K, 8192, 28672, {1: "gemv_f32", 2: "skinny_deep", 3: "skinny_deep", 4: "skinny_deep", 5: "skinny_staged", 8: "skinny_staged"}),
+    ("70B ffn_down Q6_K", Q6_K, 8192, 28672, {1: "gemv_f32", 2: "skinny_deep", 3: "skinny_deep", 4: "skinny_deep", 5: "skinny_staged"}),
     ("head", Q6_K, 128256, 4096, {1: "gemv", 2: "skinny_rows_q6k", 4: "skinny_rows_q6k", 8: "skinny_rows_q6k",
                                   16: "skinny_staged", 512: "gemm_q6k"}),
     ("Q4_0 4096^2", Q4_0, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 4: "skinny32", 8: "skinny32", 512: "gemm_blk32"}),
