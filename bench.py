@@ -390,9 +390,17 @@ def main() -> int:
 
     # ---- the other configurations, one short timing each: f32 activations in HBM, quantization included
     if not args.no_other:
+        def plain_rows(t, rows, k):
+            # rows of an unquantized weight type (F32 / F16 / BF16) as the bytes a GGUF file holds
+            w = (np.random.default_rng(1100 + t).standard_normal((rows, k)) * 0.02).astype(np.float32)
+            if t == qmm.F16:
+                return w.astype(np.float16).view(np.uint8)
+            return (w.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8) if t == qmm.BF16 else w.view(np.uint8)
+
         def time_mulmat(t, m, k, n, copies, path=qmm.PATH_AUTO):
             rows = min(m, 2048)
-            raw = np.tile(synth.weights(t, rows, k, seed=1100 + t), ((m + rows - 1) // rows, 1))[:m]
+            base = plain_rows(t, rows, k) if t in qmm.PLAIN_TYPES else synth.weights(t, rows, k, seed=1100 + t)
+            raw = np.tile(base, ((m + rows - 1) // rows, 1))[:m]
             ws = [ctx.upload(t, np.roll(raw, 13 * c, axis=0), k, m) for c in range(copies)]
             xs = torch.randn(n, k, generator=g, dtype=torch.float32).to(dev)
             yo = torch.empty(n, m, dtype=torch.float32, device=dev)
@@ -435,6 +443,18 @@ def main() -> int:
         for label, t in (("Q4_0", Q4_0), ("Q8_0", Q8_0)):
             tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
             other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TOPS": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
+        # the unquantized weight types (F16 / BF16 / F32 files, and the tensors a K-quant file keeps unquantized)
+        for label, t, m, k, ns, copies in (("F16 ffn_gate 14336x4096", qmm.F16, 14336, 4096, (1, 4, 8), 6),
+                                           ("BF16 q_proj 4096x4096", qmm.BF16, 4096, 4096, (1, 8), 16),
+                                           ("F32 q_proj 4096x4096", qmm.F32, 4096, 4096, (1,), 8)):
+            for n in ns:
+                tm, wb = time_mulmat(t, m, k, n, copies)
+                gbs = alg_bytes(wb, k, m, n) / tm / 1e9
+                other[f"{label} B={n}"] = {"us": round(tm * 1e6, 2), "GB/s": round(gbs, 1),
+                                           "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        for label, t in (("F16", qmm.F16), ("BF16", qmm.BF16), ("F32", qmm.F32)):
+            tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
+            other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TFLOP/s": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
         # expert-indexed product: 128 experts of 768x2048 (Q4_K), 8 used per token
         n_exp, n_used, em, ek = 128, 8, 768, 2048
         raw = np.tile(synth.weights(Q4_K, 2048, ek, seed=1201), (n_exp * em // 2048, 1))

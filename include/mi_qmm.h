@@ -45,11 +45,13 @@ enum {
 /* ggml_type ids this path uses -- /root/reference/fs/ggml/type.go:250-268 */
 enum {
     MI_QMM_TYPE_F32 = 0,
+    MI_QMM_TYPE_F16 = 1,
     MI_QMM_TYPE_Q4_0 = 2,
     MI_QMM_TYPE_Q8_0 = 8,
     MI_QMM_TYPE_Q4_K = 12,
     MI_QMM_TYPE_Q6_K = 14,
-    MI_QMM_TYPE_Q8_K = 15
+    MI_QMM_TYPE_Q8_K = 15,
+    MI_QMM_TYPE_BF16 = 30
 };
 
 /* where x / y / weight bytes live */
@@ -82,7 +84,10 @@ enum {
     MI_QMM_ROUTE_SKINNY_ROWS_Q4K = 10, /* Q4_K rows kernel (activations resident in LDS, a wave per row group)    */
     MI_QMM_ROUTE_SKINNY_STAGED = 11,   /* K-quant staged matrix-core kernel for 3..31 columns                     */
     MI_QMM_ROUTE_SKINNY_ROWS_Q6K = 12, /* Q6_K rows kernel (the output head at 2..8 columns)                      */
-    MI_QMM_ROUTE_GEMV = 13             /* streaming GEMV on quantized planes                                      */
+    MI_QMM_ROUTE_GEMV = 13,            /* streaming GEMV on quantized planes                                      */
+    MI_QMM_ROUTE_PLAIN_GEMV = 14,      /* F32 / F16 / BF16 weights: streaming kernel, x converted in its prologue  */
+    MI_QMM_ROUTE_PLAIN_GEMM = 15,      /* F32 / F16 / BF16 weights: tiles on the f32 / f16 / bf16 matrix cores     */
+    MI_QMM_ROUTE_PLAIN_NAIVE = 16      /* F32 / F16 / BF16 weights whose rows are no multiple of 16 bytes          */
 };
 
 /* ---- size tables: replace TensorType.BlockSize / TypeSize and Tensor.Size's row rule
@@ -92,8 +97,9 @@ int64_t mi_qmm_block_size(int ggml_type);
 int64_t mi_qmm_type_size(int ggml_type);
 /* bytes of one row of k elements; -1 when the id is unknown or k is not a multiple of the block */
 int64_t mi_qmm_row_size(int ggml_type, int64_t k);
-/* activation block type the path quantizes to for a weight type: 8 (Q8_0), 15 (Q8_K), -1 if the
- * weight type is not supported -- ggml type_traits_cpu[type].vec_dot_type */
+/* activation type the path converts x to for a weight type: 8 (Q8_0), 15 (Q8_K); the unquantized weight types
+ * 0 (F32), 1 (F16) and 30 (BF16) are multiplied in their own type; -1 if the weight type is not supported --
+ * ggml type_traits_cpu[type].vec_dot_type */
 int mi_qmm_vec_dot_type(int weight_type);
 
 /* ---- lifetime: replaces Backend construction / Close, /root/reference/ml/backend.go:16-18, 78-92.
@@ -131,6 +137,13 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      fed with the tensor bytes fs/ggml hands out (/root/reference/fs/ggml/gguf.go:281-308;
  *      fs/gguf/gguf.go:388-430): M rows of K elements in GGUF block layout, rows contiguous.
  *      The bytes are copied (and re-laid-out for the device) before the call returns.
+ *      ggml_type: the block-quantized types 2 (Q4_0), 8 (Q8_0), 12 (Q4_K), 14 (Q6_K), and the unquantized
+ *      ones a GGUF file holds beside them or instead of them, 0 (F32), 1 (F16), 30 (BF16): the file types
+ *      /root/reference/fs/ggml/type.go:55-88 accepts, the tensors a K-quant file keeps unquantized and the
+ *      ones /root/reference/server/quantization.go:296-333 keeps at f16.  The unquantized types go through
+ *      mi_qmm_mulmat, mi_qmm_mulmat_path, mi_qmm_mulmat_noalloc and mi_qmm_mulmat_multi (one product after the
+ *      other there); the produced, expert-indexed and pre-quantized entry points take block-quantized weights
+ *      only and return MI_QMM_ERR_UNSUPPORTED otherwise.
  *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
 int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
                          int64_t m, int src_location, mi_qmm_weight **out);
@@ -161,7 +174,10 @@ int mi_qmm_quantize_act(mi_qmm_ctx *ctx, int q8_type, const float *x, int64_t k,
 
 /* ---- the product: replaces Tensor.Mulmat + Context.Compute + Tensor.Floats,
  *      /root/reference/ml/backend.go:151, 110, 140.
- *      x: f32 [n][k], y: f32 [n][m] with y[i*m + r] = dot(W row r, Q8(x row i)).
+ *      x: f32 [n][k], y: f32 [n][m] with y[i*m + r] = dot(W row r, Q8(x row i)); for F32 / F16 / BF16
+ *      weights Q8 is the conversion of x to the weight's own type (round to nearest even) and the products
+ *      are formed and added in fp32 (ggml_vec_dot_f32 / _f16 / _bf16 add them in double: the difference is
+ *      far inside the path's 1e-3 tolerance).
  *      location = MI_QMM_HOST: copies in, computes, copies out and returns when y is complete.
  *      location = MI_QMM_DEVICE: x and y are device pointers; the work is queued on the ctx's
  *      stream and the call returns without waiting (mi_qmm_sync or stream order to consume). */

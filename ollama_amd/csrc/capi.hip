@@ -209,6 +209,7 @@ int mi_qmm_vec_dot_type(int wt) {
     switch (wt) {
     case T_Q4_0: case T_Q8_0: return T_Q8_0;
     case T_Q4_K: case T_Q6_K: return T_Q8_K;
+    case T_F32: case T_F16: case T_BF16: return wt;  // multiplied in their own type: x is converted to it
     default: return -1;
     }
 }
@@ -309,7 +310,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (mi_qmm_vec_dot_type(type) < 0)
-        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (2, 8, 12, 14)", type);
+        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 8, 12, 14, 30)", type);
     if (k <= 0 || m <= 0) return fail(MI_QMM_ERR_INVALID, "k=%lld m=%lld must be positive", (long long)k, (long long)m);
     const int64_t row = mi_qmm_row_size(type, k);
     if (row < 0)
@@ -329,7 +330,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     // plane sizes (bytes), each plane 256-byte aligned inside one allocation
     size_t s0 = 0, s1 = 0, s2 = 0, sd = 0;
     switch (type) {
-    case T_Q4_K: s0 = total; break;
+    case T_Q4_K: case T_F32: case T_F16: case T_BF16: s0 = total; break;
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q6_K: s0 = (size_t)(m * (k / 2)); s1 = (size_t)(m * (k / 4)); s2 = (size_t)(m * (k / 16));
@@ -362,7 +363,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
         delete w;
         return fail(code, "%s: %s", what, hipGetErrorString(err));
     };
-    if (type == T_Q4_K) {
+    if (type == T_Q4_K || plain_type(type)) {
         e = hipMemcpyAsync(b + o0, bytes, total,
                            src_location == MI_QMM_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice, ctx->stream);
         if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(weight)", e);
@@ -621,8 +622,12 @@ int route_f32(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n, int path
     return route_planes(ctx, w, a, path, /*may_alloc=*/true, err);
 }
 
-int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, int path) {
+// allow_plain: the entry point also multiplies by F32 / F16 / BF16 weights (mi_qmm_mulmat and its variants do; the
+// joint, produced, expert-indexed and pre-quantized forms are for the block-quantized types)
+int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, int path, bool allow_plain = false) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
+    if (!allow_plain && plain_type(w->dev.type))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "this entry point takes block-quantized weights; type %d goes through mi_qmm_mulmat", w->dev.type);
     if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
         return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
     if (path != MI_QMM_PATH_AUTO && path != MI_QMM_PATH_GEMV && path != MI_QMM_PATH_GEMM && path != MI_QMM_PATH_QUERY)
@@ -634,6 +639,55 @@ int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, in
     return MI_QMM_OK;
 }
 
+// mi_qmm_mulmat on an F32 / F16 / BF16 weight.  scratch: where the converted activations of the tiled kernel go -- NULL:
+// the ctx's growable buffer; else a buffer of scratch_bytes the call must fit (mi_qmm_mulmat_noalloc).
+int plain_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location, int path,
+                 void *scratch, size_t scratch_bytes) {
+    const int64_t K = w->dev.K, M = w->dev.M;
+    const int force = path == MI_QMM_PATH_GEMV ? 1 : path == MI_QMM_PATH_GEMM ? 2 : 0;
+    const int kind = plain_kind(w->dev.type, K, M, n, force);
+    if (!kind)
+        return fail(MI_QMM_ERR_UNSUPPORTED, "no kernel for type %d, K=%lld, M=%lld, n=%lld on this path", w->dev.type, (long long)K,
+                    (long long)M, (long long)n);
+    int rc;
+    void *xc = nullptr;
+    const size_t need = kind == 2 ? plain_convert_bytes(w->dev.type, K, n) : 0;
+    if (need && scratch) {
+        if (need > scratch_bytes)
+            return fail(MI_QMM_ERR_UNSUPPORTED, "n=%lld rows of k=%lld need %zu bytes of converted activations; the static scratch of "
+                        "mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)K, need, scratch_bytes);
+        xc = scratch;
+    } else if (need) {
+        if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, need))) return rc;
+        xc = ctx->act_buf;
+    }
+    const size_t xbytes = (size_t)(n * K) * 4, ybytes = (size_t)(n * M) * 4;
+    const float *dx = x;
+    float *dy = y;
+    if (location == MI_QMM_HOST) {
+        const size_t yoff = align_up(xbytes, 256);
+        if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, yoff + ybytes))) return rc;
+        dx = (const float *)ctx->io_buf;
+        dy = (float *)((char *)ctx->io_buf + yoff);
+        HIP_TRY(hipMemcpyAsync((void *)dx, x, xbytes, hipMemcpyHostToDevice, ctx->stream));
+    }
+    HIP_TRY(launch_plain(w->dev, dx, n, dy, xc, ctx->num_cus, ctx->stream, force));
+    if (location == MI_QMM_HOST) {
+        HIP_TRY(hipMemcpyAsync(y, dy, ybytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    return MI_QMM_OK;
+}
+
+int plain_route(const mi_qmm_weight *w, int64_t n) {
+    switch (plain_kind(w->dev.type, w->dev.K, w->dev.M, n)) {
+    case 1: case 4: return MI_QMM_ROUTE_PLAIN_GEMV;
+    case 2: return MI_QMM_ROUTE_PLAIN_GEMM;
+    case 3: return MI_QMM_ROUTE_PLAIN_NAIVE;
+    default: return 0;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -641,17 +695,22 @@ extern "C" {
 int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, int location,
                        int path) {
     if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
-    int rc = check_product_args(ctx, w, location, path);
+    int rc = check_product_args(ctx, w, location, path, /*allow_plain=*/true);
     if (rc) return rc;
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
     if (path == MI_QMM_PATH_QUERY) {  // which kernel mi_qmm_mulmat would take; nothing is launched, x and y may be NULL
         if (n == 0) return fail(MI_QMM_ERR_INVALID, "a product of no columns has no route");
+        if (plain_type(w->dev.type)) {
+            const int route = plain_route(w, n);
+            return route ? route : fail(MI_QMM_ERR_UNSUPPORTED, "no kernel for this shape");
+        }
         const char *why = nullptr;
         const int route = route_f32(ctx, w, n, MI_QMM_PATH_AUTO, &why);
         return route ? route : fail(MI_QMM_ERR_UNSUPPORTED, "%s", why);
     }
     if (n == 0) return MI_QMM_OK;
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
+    if (plain_type(w->dev.type)) return plain_mulmat(ctx, w, x, n, y, location, path, nullptr, 0);
 
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
@@ -701,11 +760,13 @@ int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64
 // and the tiled GEMM runs without its K-split workspace.  Same kernels as mi_qmm_mulmat otherwise.
 int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y) {
     if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
-    int rc = check_product_args(ctx, w, MI_QMM_DEVICE, MI_QMM_PATH_AUTO);
+    int rc = check_product_args(ctx, w, MI_QMM_DEVICE, MI_QMM_PATH_AUTO, /*allow_plain=*/true);
     if (rc) return rc;
     if (n == 0) return MI_QMM_OK;
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    if (plain_type(w->dev.type))
+        return plain_mulmat(ctx, w, x, n, y, MI_QMM_DEVICE, MI_QMM_PATH_AUTO, ctx->static_scratch, (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES);
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
     if (n <= 8 && !wants_skinny(w->dev.type, K, M, n, ctx->num_cus) && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
@@ -778,8 +839,10 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
     }
     int rc = check_product_args(ctx, ws[0], location, MI_QMM_PATH_AUTO);
     if (rc) return rc;
-    for (int i = 0; i < count; i++)
+    for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
+        if (plain_type(ws[i]->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is an unquantized weight (type %d)", i, ws[i]->dev.type);
+    }
     Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
     if (prod) pr = *prod;
     if (pr.kind == PRODUCE_SWIGLU && !pr.aux && n > 0) return fail(MI_QMM_ERR_INVALID, "SwiGLU needs the up operand");
@@ -948,6 +1011,22 @@ extern "C" {
 
 int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x, int64_t n,
                         float *const *ys, int location) {
+    bool plain = false;
+    for (int i = 0; ws && ys && i < count; i++) plain = plain || (ws[i] && plain_type(ws[i]->dev.type));
+    if (plain) {
+        // unquantized weights have no joint kernels: one product after the other, each as mi_qmm_mulmat gives it
+        for (int i = 0; i < count; i++) {
+            if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
+            if (ws[i]->dev.K != ws[0]->dev.K)
+                return fail(MI_QMM_ERR_INVALID, "ws[%d] has k=%lld, ws[0] has k=%lld: one x cannot serve both", i,
+                            (long long)ws[i]->dev.K, (long long)ws[0]->dev.K);
+        }
+        for (int i = 0; i < count; i++) {
+            const int rc = mi_qmm_mulmat(ctx, ws[i], x, n, ys[i], location);
+            if (rc) return rc;
+        }
+        return MI_QMM_OK;
+    }
     return mulmat_multi_impl(ctx, ws, count, nullptr, x, n, ys, location);
 }
 
@@ -971,6 +1050,7 @@ int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_
     int rc = check_product_args(ctx, w_gate, location, MI_QMM_PATH_AUTO);
     if (rc) return rc;
     if (w_up->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "w_up is on another device");
+    if (plain_type(w_up->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is an unquantized weight (type %d)", w_up->dev.type);
     if (producer == MI_QMM_PRODUCE_RMSNORM && !(eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
     if (n == 0) return MI_QMM_OK;
     if (!x || !h) return fail(MI_QMM_ERR_INVALID, "x or h is NULL");
@@ -1224,6 +1304,7 @@ int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const 
     if (rc) return rc;
     if (w_up->device != ctx->device || w_up->dev.K != w_gate->dev.K || w_up->dev.M != w_gate->dev.M)
         return fail(MI_QMM_ERR_INVALID, "the gate and up stacks differ in device or shape");
+    if (plain_type(w_up->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is an unquantized weight (type %d)", w_up->dev.type);
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
         return fail(MI_QMM_ERR_INVALID, "n_expert=%d n_used=%d b_cols=%d n_tokens=%lld: all must be positive", n_expert,
                     n_used, b_cols, (long long)n_tokens);
@@ -1458,6 +1539,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     DevWeight dw[8];
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
+        if (plain_type(ws[i]->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is an unquantized weight (type %d)", i, ws[i]->dev.type);
         dw[i] = ws[i]->dev;
     }
     float *dys[8];

@@ -12,7 +12,7 @@
 
 namespace miqmm {
 
-enum : int { T_F32 = 0, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15 };
+enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 30, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15 };
 
 constexpr int QK = 32;    // elements per Q4_0 / Q8_0 block
 constexpr int QKK = 256;  // elements per K-quant super-block
@@ -25,6 +25,7 @@ constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q6_K_BYTES = 2
 //   Q8_0 : p0 = qs plane, 32 B per block, [M][K];                  d = fp16 plane [M][K/32]
 //   Q6_K : p0 = ql plane [M][K/2]; p1 = qh plane [M][K/4]; p2 = scales plane [M][K/16] (i8);
 //          d = fp16 plane [M][K/256]
+//   F32, F16, BF16 : p0 = the rows unchanged, [M][K] elements
 // Byte order inside each plane is the GGUF order; only the interleaving of fields is undone.
 struct DevWeight {
     const uint8_t *p0;

@@ -177,4 +177,14 @@ bool skinny_id_supports(int type, int64_t K, int64_t M, int64_t pairs, int n_exp
 hipError_t launch_skinny_id(const DevWeight &w, int n_expert, const DevAct &a, const int *ids, int n_used, int n_tokens,
                             int b_cols, float *y, int *groups, int num_cus, hipStream_t s);
 
+// Unquantized weights (F32, F16, BF16; plain.hip): x f32 [N][K] on the device, y[n*M + m].
+//   plain_kind: 0 = not such a product, 1 = streaming kernel (N <= 8, rows a multiple of 16 bytes), 2 = matrix-core tiles
+//   (rows a multiple of 64 bytes), 3 = a wave per output (any K), 4 = the streaming kernel, 8 columns per launch.
+//   force: 0 = as plain_kind says, 1 = never the tiles, 2 = the tiles or an error.
+//   xc: device scratch of plain_convert_bytes() bytes for the converted activations of kind 2 (F16 / BF16).
+bool plain_type(int type);
+int plain_kind(int type, int64_t K, int64_t M, int64_t N, int force = 0);
+size_t plain_convert_bytes(int type, int64_t K, int64_t N);
+hipError_t launch_plain(const DevWeight &w, const float *x, int64_t N, float *y, void *xc, int num_cus, hipStream_t s, int force = 0);
+
 }  // namespace miqmm

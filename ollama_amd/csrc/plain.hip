@@ -1,0 +1,405 @@
+// Mulmat on the unquantized weight types of a GGUF file: F32, F16 and BF16 (the file types F32 / F16 / BF16 of
+// /root/reference/fs/ggml/type.go:55-88, the tensors a K-quant file keeps unquantized, and the ones the reference keeps
+// at f16 on purpose: /root/reference/server/quantization.go:296-333).
+//
+// Semantics: the ggml CPU backend's.  The f32 activations are converted to the weight's own type (F16: IEEE round to
+// nearest even; BF16: round to nearest even on the upper 16 bits; F32: as they are), both operands are widened to fp32
+// and multiplied there; a product of two halves or two bfloat16 is exact in fp32.  The CPU adds the products in double,
+// the kernels here in fp32 (lane partial sums, then a tree over the lanes; the matrix cores' own order in the GEMM):
+// the difference is rounding of fp32 sums, orders of magnitude inside the path's 1e-3 tolerance.
+//
+// Three kernels:
+//   plain_gemv_kernel   1..8 activation columns, bound by HBM: a wave streams two weight rows at a time with 16-byte
+//                       loads, the converted activations sit in LDS (all of K where it fits, else chunk by chunk).
+//   plain_gemm_kernel   9 columns and more: 128 x 128 (or 128 x 32) output tiles on v_mfma_f32_32x32x16_{f16,bf16} /
+//                       v_mfma_f32_32x32x2_f32, operands staged through LDS in two buffers, from activations converted
+//                       once by plain_convert_kernel.
+//   plain_naive_kernel  rows whose byte length is no multiple of 16 (K odd ...): a wave per output, element loads.
+#include <algorithm>
+
+#include "internal.h"
+
+namespace miqmm {
+
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned f32_bits(float f) { return __builtin_bit_cast(unsigned, f); }
+__device__ __forceinline__ float bits_f32(unsigned u) { return __builtin_bit_cast(float, u); }
+
+// f32 -> the 16-bit pattern of the weight's type
+template <int TYPE>
+__device__ __forceinline__ unsigned short narrow16(float f) {
+    if (TYPE == T_F16) return __builtin_bit_cast(unsigned short, (_Float16)f);
+    const unsigned u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 64);
+    return (unsigned short)((u + (0x7fffu + ((u >> 16) & 1u))) >> 16);
+}
+// the two 16-bit values of a dword, widened
+template <int TYPE>
+__device__ __forceinline__ void widen2(unsigned u, float &lo, float &hi) {
+    if (TYPE == T_F16) {
+        lo = (float)__builtin_bit_cast(_Float16, (unsigned short)(u & 0xffffu));
+        hi = (float)__builtin_bit_cast(_Float16, (unsigned short)(u >> 16));
+    } else {
+        lo = bits_f32(u << 16);
+        hi = bits_f32(u & 0xffff0000u);
+    }
+}
+// a 16-byte piece of a row as floats: E = 8 (16-bit types) or 4 (F32)
+template <int TYPE>
+__device__ __forceinline__ void widen_piece(const v4u &p, float *f) {
+    if (TYPE == T_F32) {
+        f[0] = bits_f32(p.x); f[1] = bits_f32(p.y); f[2] = bits_f32(p.z); f[3] = bits_f32(p.w);
+    } else {
+        widen2<TYPE>(p.x, f[0], f[1]); widen2<TYPE>(p.y, f[2], f[3]);
+        widen2<TYPE>(p.z, f[4], f[5]); widen2<TYPE>(p.w, f[6], f[7]);
+    }
+}
+
+template <int TYPE>
+__global__ __launch_bounds__(256) void plain_convert_kernel(const float *__restrict__ x, unsigned short *__restrict__ out, int64_t count) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) out[i] = narrow16<TYPE>(x[i]);
+}
+
+// ---- 1..8 columns -------------------------------------------------------------------------------------------------
+// Workgroup of 16 waves; a round is 32 consecutive rows, two per wave.  K is walked in chunks of KC elements (KC a
+// multiple of 128 * E; one chunk where all of K fits, and then the activations are staged once for the whole launch).
+// Requires (K * ES) % 16 == 0.  LDS: NC * min(K, KC) elements of the weight's type.
+constexpr int GEMV_WAVES = 16;
+template <int TYPE, int NC>
+__global__ __launch_bounds__(64 * GEMV_WAVES) void plain_gemv_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x,
+                                                                     float *__restrict__ y, int K, int64_t M, int KC) {
+    constexpr int ES = TYPE == T_F32 ? 4 : 2, E = 16 / ES;
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nchunks = (K + KC - 1) / KC;
+    const int64_t rounds = (M + 31) / 32;
+    const int64_t row_bytes = (int64_t)K * ES;
+    bool staged = false;
+    for (int64_t round = blockIdx.x; round < rounds; round += gridDim.x) {
+        const int64_t r0 = round * 32 + 2 * wave;
+        const bool live = r0 < M;
+        const int64_t r1 = r0 + 1 < M ? r0 + 1 : (live ? r0 : 0);
+        const uint8_t *w0 = w + (live ? r0 : 0) * row_bytes, *w1 = w + r1 * row_bytes;
+        float acc0[NC], acc1[NC];
+#pragma unroll
+        for (int c = 0; c < NC; c++) acc0[c] = acc1[c] = 0.0f;
+        for (int ch = 0; ch < nchunks; ch++) {
+            const int k0 = ch * KC, len = K - k0 < KC ? K - k0 : KC;
+            if (nchunks > 1 || !staged) {
+                if (staged) __syncthreads();  // every wave is through with the chunk that is about to be replaced
+                for (int c = 0; c < NC; c++)
+                    for (int i = tid; i < len; i += 64 * GEMV_WAVES) {
+                        const float v = x[(int64_t)c * K + k0 + i];
+                        if (TYPE == T_F32) reinterpret_cast<float *>(xs)[c * KC + i] = v;
+                        else reinterpret_cast<unsigned short *>(xs)[c * KC + i] = narrow16<TYPE>(v);
+                    }
+                staged = true;
+                __syncthreads();
+            }
+            if (!live) continue;
+            const uint8_t *p0 = w0 + (int64_t)k0 * ES, *p1 = w1 + (int64_t)k0 * ES;
+            for (int e = lane * E; e < len; e += 128 * E) {
+                const int e2 = e + 64 * E;
+                const bool two = e2 < len;
+                const v4u a0 = *reinterpret_cast<const v4u *>(p0 + (int64_t)e * ES);
+                const v4u b0 = *reinterpret_cast<const v4u *>(p1 + (int64_t)e * ES);
+                v4u a1 = {0, 0, 0, 0}, b1 = {0, 0, 0, 0};
+                if (two) {
+                    a1 = *reinterpret_cast<const v4u *>(p0 + (int64_t)e2 * ES);
+                    b1 = *reinterpret_cast<const v4u *>(p1 + (int64_t)e2 * ES);
+                }
+                float fa[E], fb[E], fx[E];
+                widen_piece<TYPE>(a0, fa);
+                widen_piece<TYPE>(b0, fb);
+#pragma unroll
+                for (int c = 0; c < NC; c++) {
+                    widen_piece<TYPE>(*reinterpret_cast<const v4u *>(xs + ((int64_t)c * KC + e) * ES), fx);
+#pragma unroll
+                    for (int j = 0; j < E; j++) {
+                        acc0[c] = __builtin_fmaf(fa[j], fx[j], acc0[c]);
+                        acc1[c] = __builtin_fmaf(fb[j], fx[j], acc1[c]);
+                    }
+                }
+                if (two) {
+                    widen_piece<TYPE>(a1, fa);
+                    widen_piece<TYPE>(b1, fb);
+#pragma unroll
+                    for (int c = 0; c < NC; c++) {
+                        widen_piece<TYPE>(*reinterpret_cast<const v4u *>(xs + ((int64_t)c * KC + e2) * ES), fx);
+#pragma unroll
+                        for (int j = 0; j < E; j++) {
+                            acc0[c] = __builtin_fmaf(fa[j], fx[j], acc0[c]);
+                            acc1[c] = __builtin_fmaf(fb[j], fx[j], acc1[c]);
+                        }
+                    }
+                }
+            }
+        }
+        if (!live) continue;
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            float s0 = acc0[c], s1 = acc1[c];
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) {
+                s0 += __shfl_xor(s0, o, 64);
+                s1 += __shfl_xor(s1, o, 64);
+            }
+            if (lane == 0) {
+                y[(int64_t)c * M + r0] = s0;
+                if (r0 + 1 < M) y[(int64_t)c * M + r0 + 1] = s1;
+            }
+        }
+    }
+}
+
+// ---- any K: a wave per output, element loads -------------------------------------------------------------------------
+template <int TYPE>
+__global__ __launch_bounds__(256) void plain_naive_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
+                                                          int64_t K, int64_t M, int64_t N) {
+    const int lane = threadIdx.x & 63;
+    const int64_t waves = (int64_t)gridDim.x * 4, total = M * N;
+    for (int64_t o = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); o < total; o += waves) {
+        const int64_t n = o / M, m = o - n * M;
+        float s = 0.0f;
+        for (int64_t k = lane; k < K; k += 64) {
+            float wv, xv = x[n * K + k];
+            if (TYPE == T_F32) wv = reinterpret_cast<const float *>(w)[m * K + k];
+            else {
+                float dummy;
+                widen2<TYPE>(reinterpret_cast<const unsigned short *>(w)[m * K + k], wv, dummy);
+                widen2<TYPE>(narrow16<TYPE>(xv), xv, dummy);
+            }
+            s = __builtin_fmaf(wv, xv, s);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
+        if (lane == 0) y[o] = s;
+    }
+}
+
+// ---- 9 columns and more: tiles on the matrix cores ---------------------------------------------------------------------
+// Workgroup of WM x WN waves; a wave owns TN x TM accumulator tiles of 32 (activation rows) x 32 (weight rows).  The
+// A operand of an MFMA is the activations, the B operand the weights: accumulator i of lane l is activation row
+// 8 (i / 4) + 4 (l / 32) + i % 4 and weight row l % 32, so a store instruction writes runs of 32 consecutive floats of y.
+// A stage is 64 bytes of every row of the tile (32 halves or 16 floats), rows padded to 80 bytes in LDS; two stages.
+// Requires (K * ES) % 64 == 0.  xc: the activations in the weight's type, [N][K].
+template <int TYPE, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(64 * WM * WN) void plain_gemm_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xc,
+                                                                  float *__restrict__ y, int64_t K, int64_t M, int64_t N) {
+    constexpr int ES = TYPE == T_F32 ? 4 : 2;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, NT = 64 * WM * WN;
+    constexpr int LDR = 80, ROWS = BM + BN, PIECES = ROWS * 4, PP = (PIECES + NT - 1) / NT;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][ROWS * LDR];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave / WN, wn = wave % WN;
+    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
+    const int64_t row_bytes = K * ES;
+    const int nk = (int)(row_bytes / 64);
+
+    // the pieces this thread copies per stage: tile row r (weights first, then activations), 16-byte piece q
+    const uint8_t *src[PP];
+    int dst[PP];
+#pragma unroll
+    for (int i = 0; i < PP; i++) {
+        const int idx = tid + i * NT, r = idx >> 2, q = idx & 3;
+        dst[i] = idx < PIECES ? r * LDR + q * 16 : -1;
+        if (r < BM) {
+            const int64_t m = m0 + r < M ? m0 + r : M - 1;
+            src[i] = w + m * row_bytes + q * 16;
+        } else {
+            const int64_t n = n0 + (r - BM) < N ? n0 + (r - BM) : N - 1;
+            src[i] = xc + n * row_bytes + q * 16;
+        }
+    }
+    v4u regs[PP];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < PP; i++)
+            if (dst[i] >= 0) regs[i] = *reinterpret_cast<const v4u *>(src[i] + (int64_t)kt * 64);
+    };
+    auto park = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PP; i++)
+            if (dst[i] >= 0) *reinterpret_cast<v4u *>(&lds[buf][dst[i]]) = regs[i];
+    };
+
+    v16f acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; a++)
+#pragma unroll
+        for (int b = 0; b < TM; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
+
+    const int row_in = lane & 31, kg = lane >> 5;
+    const int wrow = (wm * TM * 32 + row_in) * LDR, xrow = (BM + wn * TN * 32 + row_in) * LDR;
+
+    fetch(0);
+    park(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt++) {
+        if (kt + 1 < nk) fetch(kt + 1);
+        const uint8_t *L = lds[kt & 1];
+        if (TYPE == T_F32) {
+            // the 16 products of a stage are added up from zero and their sum joins the running total: K / 16 roundings
+            // of the total instead of K / 2 (a row of 14336 floats: 896 instead of 7168)
+            v16f part[TN][TM];
+#pragma unroll
+            for (int a = 0; a < TN; a++)
+#pragma unroll
+                for (int b = 0; b < TM; b++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) part[a][b][i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                float fa[TN], fb[TM];
+#pragma unroll
+                for (int a = 0; a < TN; a++) fa[a] = *reinterpret_cast<const float *>(L + xrow + a * 32 * LDR + ks * 8 + kg * 4);
+#pragma unroll
+                for (int b = 0; b < TM; b++) fb[b] = *reinterpret_cast<const float *>(L + wrow + b * 32 * LDR + ks * 8 + kg * 4);
+#pragma unroll
+                for (int a = 0; a < TN; a++)
+#pragma unroll
+                    for (int b = 0; b < TM; b++) part[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], part[a][b], 0, 0, 0);
+            }
+#pragma unroll
+            for (int a = 0; a < TN; a++)
+#pragma unroll
+                for (int b = 0; b < TM; b++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc[a][b][i] += part[a][b][i];
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                v4u fa[TN], fb[TM];
+#pragma unroll
+                for (int a = 0; a < TN; a++) fa[a] = *reinterpret_cast<const v4u *>(L + xrow + a * 32 * LDR + ks * 32 + kg * 16);
+#pragma unroll
+                for (int b = 0; b < TM; b++) fb[b] = *reinterpret_cast<const v4u *>(L + wrow + b * 32 * LDR + ks * 32 + kg * 16);
+#pragma unroll
+                for (int a = 0; a < TN; a++)
+#pragma unroll
+                    for (int b = 0; b < TM; b++) {
+                        if (TYPE == T_F16)
+                            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, fa[a]), __builtin_bit_cast(v8h, fb[b]),
+                                                                               acc[a][b], 0, 0, 0);
+                        else
+                            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa[a]), __builtin_bit_cast(v8bf, fb[b]),
+                                                                                acc[a][b], 0, 0, 0);
+                    }
+            }
+        }
+        if (kt + 1 < nk) park((kt + 1) & 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int b = 0; b < TM; b++) {
+        const int64_t m = m0 + wm * TM * 32 + b * 32 + row_in;
+        if (m >= M) continue;
+#pragma unroll
+        for (int a = 0; a < TN; a++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t n = n0 + wn * TN * 32 + a * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);
+                if (n < N) y[n * M + m] = acc[a][b][i];
+            }
+    }
+}
+
+int elem_size(int type) { return type == T_F32 ? 4 : 2; }
+
+template <int TYPE>
+hipError_t gemv_typed(const DevWeight &w, const float *x, int ncols, float *y, int num_cus, hipStream_t s) {
+    constexpr int ES = TYPE == T_F32 ? 4 : 2, E = 16 / ES;
+    // the chunk: what 64 KiB of LDS holds for ncols columns, a multiple of the 128 pieces a wave takes per turn
+    int kc = 65536 / (ncols * ES);
+    kc -= kc % (128 * E);
+    const int K = (int)w.K;
+    if (kc > K) kc = (K + 128 * E - 1) / (128 * E) * (128 * E);
+    const size_t lds = (size_t)ncols * kc * ES;
+    const int64_t rounds = (w.M + 31) / 32;
+    const dim3 grid((unsigned)std::min<int64_t>(rounds, 2 * (int64_t)num_cus)), block(64 * GEMV_WAVES);
+#define PLAIN_GEMV(NC) case NC: plain_gemv_kernel<TYPE, NC><<<grid, block, lds, s>>>(w.p0, x, y, K, w.M, kc); break;
+    switch (ncols) {
+        PLAIN_GEMV(1) PLAIN_GEMV(2) PLAIN_GEMV(3) PLAIN_GEMV(4) PLAIN_GEMV(5) PLAIN_GEMV(6) PLAIN_GEMV(7) PLAIN_GEMV(8)
+    default: return hipErrorInvalidValue;
+    }
+#undef PLAIN_GEMV
+    return hipGetLastError();
+}
+
+template <int TYPE>
+hipError_t gemm_typed(const DevWeight &w, const void *xc, int64_t N, float *y, hipStream_t s) {
+    const uint8_t *xb = (const uint8_t *)xc;
+    if (N <= 32) {
+        const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((w.M + 127) / 128));
+        plain_gemm_kernel<TYPE, 4, 1, 1, 1><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+    } else {
+        const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((w.M + 127) / 128));
+        plain_gemm_kernel<TYPE, 2, 2, 2, 2><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool plain_type(int type) { return type == T_F32 || type == T_F16 || type == T_BF16; }
+
+int plain_kind(int type, int64_t K, int64_t M, int64_t N, int force) {
+    if (!plain_type(type) || K < 1 || M < 1 || N < 1 || K > 0x7fffffff / 4) return 0;
+    const int64_t row_bytes = K * elem_size(type);
+    const bool tiles = row_bytes % 64 == 0 && (M + 127) / 128 <= 65535;
+    if (force == 2) return tiles ? 2 : 0;
+    if (N <= 8 && row_bytes % 16 == 0) return 1;
+    if (tiles && force != 1) return 2;
+    return row_bytes % 16 == 0 ? 4 : 3;
+}
+
+size_t plain_convert_bytes(int type, int64_t K, int64_t N) { return type == T_F32 ? 0 : (size_t)(K * N) * 2; }
+
+hipError_t launch_plain(const DevWeight &w, const float *x, int64_t N, float *y, void *xc, int num_cus, hipStream_t s, int force) {
+    const int kind = plain_kind(w.type, w.K, w.M, N, force);
+    if (kind == 0 || N > 0x7fffffff) return hipErrorInvalidValue;
+    if (kind == 1 || kind == 4) {
+        for (int64_t c0 = 0; c0 < N; c0 += 8) {
+            const int nc = (int)(N - c0 < 8 ? N - c0 : 8);
+            const float *xg = x + c0 * w.K;
+            float *yg = y + c0 * w.M;
+            hipError_t e;
+            switch (w.type) {
+            case T_F32: e = gemv_typed<T_F32>(w, xg, nc, yg, num_cus, s); break;
+            case T_F16: e = gemv_typed<T_F16>(w, xg, nc, yg, num_cus, s); break;
+            default: e = gemv_typed<T_BF16>(w, xg, nc, yg, num_cus, s); break;
+            }
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
+    if (kind == 2) {
+        if (w.type == T_F32) return gemm_typed<T_F32>(w, x, N, y, s);
+        if (!xc) return hipErrorInvalidValue;
+        const int64_t count = w.K * N;
+        const unsigned blocks = (unsigned)std::min<int64_t>((count + 255) / 256, 8 * (int64_t)num_cus);
+        if (w.type == T_F16) plain_convert_kernel<T_F16><<<blocks, 256, 0, s>>>(x, (unsigned short *)xc, count);
+        else plain_convert_kernel<T_BF16><<<blocks, 256, 0, s>>>(x, (unsigned short *)xc, count);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        return w.type == T_F16 ? gemm_typed<T_F16>(w, xc, N, y, s) : gemm_typed<T_BF16>(w, xc, N, y, s);
+    }
+    const int64_t outs = w.M * N;
+    const unsigned blocks = (unsigned)std::min<int64_t>((outs + 3) / 4, 16 * (int64_t)num_cus);
+    switch (w.type) {
+    case T_F32: plain_naive_kernel<T_F32><<<blocks, 256, 0, s>>>(w.p0, x, y, w.K, w.M, N); break;
+    case T_F16: plain_naive_kernel<T_F16><<<blocks, 256, 0, s>>>(w.p0, x, y, w.K, w.M, N); break;
+    default: plain_naive_kernel<T_BF16><<<blocks, 256, 0, s>>>(w.p0, x, y, w.K, w.M, N); break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace miqmm

@@ -130,7 +130,9 @@ public:
             int type = 0, nd = 0;
             int64_t dims[4];
             rc = mi_qmm_gguf_tensor(f, i, &name, &type, &nd, dims, nullptr, nullptr);
-            if (rc != MI_QMM_OK || (nd != 2 && nd != 3) || mi_qmm_vec_dot_type(type) < 0) continue;
+            // (the block-quantized types; F32 / F16 / BF16 matrices go through mi_qmm_mulmat directly, not through this mirror)
+            const int q8 = mi_qmm_vec_dot_type(type);
+            if (rc != MI_QMM_OK || (nd != 2 && nd != 3) || (q8 != MI_QMM_TYPE_Q8_0 && q8 != MI_QMM_TYPE_Q8_K)) continue;
             auto t = std::make_shared<Tensor>();
             t->shape_.assign(dims, dims + nd);
             t->type_ = type;

@@ -16,12 +16,14 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI_QMM_LIB points at an alternative build of the library (e.g. an experimental variant)
 LIB_PATH = os.environ.get("MI_QMM_LIB") or os.path.join(_HERE, "libmi_qmm.so")
 
-F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
+F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K, BF16 = 0, 1, 2, 8, 12, 14, 15, 30
+PLAIN_TYPES = (F32, F16, BF16)  # unquantized weight types: multiplied in their own type
 HOST, DEVICE = 0, 1
 PATH_AUTO, PATH_GEMV, PATH_GEMM, PATH_QUERY = 0, 1, 2, 3
 # what PATH_QUERY returns (MI_QMM_ROUTE_*): the kernel a product takes
 ROUTES = {1: "gemv_f32", 2: "deep_f32", 3: "gemm_blk32", 4: "gemm_f16", 5: "gemm_q6k", 6: "gemm_int8", 7: "skinny32",
-          8: "skinny_deep", 9: "skinny_direct", 10: "skinny_rows_q4k", 11: "skinny_staged", 12: "skinny_rows_q6k", 13: "gemv"}
+          8: "skinny_deep", 9: "skinny_direct", 10: "skinny_rows_q4k", 11: "skinny_staged", 12: "skinny_rows_q6k", 13: "gemv",
+          14: "plain_gemv", 15: "plain_gemm", 16: "plain_naive"}
 PRODUCE_NONE, PRODUCE_RMSNORM, PRODUCE_SWIGLU = 0, 1, 2
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, -3, -4, -5
 

@@ -15,7 +15,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libggml_ref.so")
 
-F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
+F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K, BF16 = 0, 1, 2, 8, 12, 14, 15, 30
 
 
 def build(force: bool = False) -> str:
@@ -45,7 +45,9 @@ def lib() -> ctypes.CDLL:
         L.ref_dequantize_row.restype = ci; L.ref_dequantize_row.argtypes = [ci, vp, vp, i64]
         L.ref_get_scale_min_k4.restype = None; L.ref_get_scale_min_k4.argtypes = [ci, vp, vp, vp]
         L.ref_unpack_scales_kmask.restype = None; L.ref_unpack_scales_kmask.argtypes = [vp, vp, vp]
-        for name in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K"):
+        L.ref_fp32_to_bf16.restype = ctypes.c_uint16; L.ref_fp32_to_bf16.argtypes = [ctypes.c_float]
+        L.ref_bf16_to_fp32.restype = ctypes.c_float; L.ref_bf16_to_fp32.argtypes = [ctypes.c_uint16]
+        for name in ("q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q6_K_q8_K", "f32", "f16", "bf16"):
             f = getattr(L, "ref_vec_dot_" + name)
             f.restype = ctypes.c_float; f.argtypes = [i64, vp, vp]
         L.ref_vec_dot_type.restype = ci; L.ref_vec_dot_type.argtypes = [ci]
@@ -86,6 +88,14 @@ def fp32_to_fp16(f: float) -> int:
     return int(lib().ref_fp32_to_fp16(f))
 
 
+def fp32_to_bf16(f: float) -> int:
+    return int(lib().ref_fp32_to_bf16(ctypes.c_float(f)))
+
+
+def bf16_to_fp32(h: int) -> float:
+    return float(lib().ref_bf16_to_fp32(h))
+
+
 def fp16_to_fp32(h: int) -> float:
     return float(lib().ref_fp16_to_fp32(h))
 
@@ -119,7 +129,7 @@ def dequantize(t: int, blocks: np.ndarray, k: int) -> np.ndarray:
     return out
 
 
-_DOTS = {Q4_0: "q4_0_q8_0", Q8_0: "q8_0_q8_0", Q4_K: "q4_K_q8_K", Q6_K: "q6_K_q8_K"}
+_DOTS = {Q4_0: "q4_0_q8_0", Q8_0: "q8_0_q8_0", Q4_K: "q4_K_q8_K", Q6_K: "q6_K_q8_K", F32: "f32", F16: "f16", BF16: "bf16"}
 
 
 def vec_dot(wtype: int, k: int, wrow: np.ndarray, xqrow: np.ndarray) -> float:

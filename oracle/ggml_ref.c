@@ -32,7 +32,7 @@ _Static_assert(sizeof(blk_q8_K) == 292, "Q8_K block is 292 bytes");
 
 int64_t ref_block_size(int type) {
     switch (type) {
-    case REF_TYPE_F32: return 1;
+    case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return 1;
     case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: return QK;
     case REF_TYPE_Q4_K: case REF_TYPE_Q6_K: case REF_TYPE_Q8_K: return QKK;
     default: return 0;
@@ -42,6 +42,7 @@ int64_t ref_block_size(int type) {
 int64_t ref_type_size(int type) {
     switch (type) {
     case REF_TYPE_F32: return 4;
+    case REF_TYPE_F16: case REF_TYPE_BF16: return 2;
     case REF_TYPE_Q4_0: return sizeof(blk_q4_0);
     case REF_TYPE_Q8_0: return sizeof(blk_q8_0);
     case REF_TYPE_Q4_K: return sizeof(blk_q4_K);
@@ -61,8 +62,17 @@ int ref_vec_dot_type(int wtype) {
     switch (wtype) {
     case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: return REF_TYPE_Q8_0;
     case REF_TYPE_Q4_K: case REF_TYPE_Q6_K: return REF_TYPE_Q8_K;
+    /* the unquantized weight types are multiplied in their own type: the activations are converted to it */
+    case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return wtype;
     default: return -1;
     }
+}
+
+static float bf16_widen(uint16_t h) {
+    const uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
 }
 
 /* ---- IEEE binary16 <-> binary32, round to nearest even, subnormals kept ------------------- */
@@ -538,6 +548,9 @@ int ref_dequantize_row(int type, const void *x, float *y, int64_t k) {
     case REF_TYPE_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
     case REF_TYPE_Q6_K: dequant_q6_K((const blk_q6_K *)x, y, k); return 0;
     case REF_TYPE_Q8_K: dequant_q8_K((const blk_q8_K *)x, y, k); return 0;
+    case REF_TYPE_F32: memcpy(y, x, (size_t)k * 4); return 0;
+    case REF_TYPE_F16: for (int64_t i = 0; i < k; i++) y[i] = ref_fp16_to_fp32(((const uint16_t *)x)[i]); return 0;
+    case REF_TYPE_BF16: for (int64_t i = 0; i < k; i++) y[i] = bf16_widen(((const uint16_t *)x)[i]); return 0;
     default: return -1;
     }
 }
@@ -660,6 +673,56 @@ float ref_vec_dot_q6_K_q8_K(int64_t n, const void *vx, const void *vy) {
 }
 
 /* ---- drivers ------------------------------------------------------------------------------------ */
+/* ---- the unquantized weight types (F32, F16, BF16) ------------------------------------------------
+ * ggml's CPU mul_mat converts the f32 activations to the weight's own type (type_traits_cpu:
+ * vec_dot_type F32 / F16 / BF16, from_float = the row converters) and calls ggml_vec_dot_f32 / _f16 /
+ * _bf16.  Their scalar loops widen both operands to fp32, form the product in fp32 and accumulate in
+ * ggml_float (double) in element order; the sum is narrowed to fp32 once at the end.  A product of two
+ * halves or two bfloat16 is exact in fp32; a product of two floats is rounded to fp32 first.
+ *
+ * bfloat16 <- fp32 (ggml_compute_fp32_to_bf16): NaNs keep their top mantissa bits and are made quiet,
+ * everything else is rounded to nearest even on the upper 16 bits, subnormals included. */
+uint16_t ref_fp32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 64);
+    return (uint16_t)((u + (0x7fffu + ((u >> 16) & 1u))) >> 16);
+}
+
+float ref_bf16_to_fp32(uint16_t h) { return bf16_widen(h); }
+
+static void convert_row_f32(const float *x, void *y, int64_t k) { memcpy(y, x, (size_t)k * 4); }
+static void convert_row_f16(const float *x, void *y, int64_t k) {
+    uint16_t *o = (uint16_t *)y;
+    for (int64_t i = 0; i < k; i++) o[i] = ref_fp32_to_fp16(x[i]);
+}
+static void convert_row_bf16(const float *x, void *y, int64_t k) {
+    uint16_t *o = (uint16_t *)y;
+    for (int64_t i = 0; i < k; i++) o[i] = ref_fp32_to_bf16(x[i]);
+}
+
+float ref_vec_dot_f32(int64_t n, const void *vx, const void *vy) {
+    const float *x = (const float *)vx, *y = (const float *)vy;
+    double sum = 0.0;
+    for (int64_t i = 0; i < n; i++) sum += (double)(x[i] * y[i]);
+    return (float)sum;
+}
+
+float ref_vec_dot_f16(int64_t n, const void *vx, const void *vy) {
+    const uint16_t *x = (const uint16_t *)vx, *y = (const uint16_t *)vy;
+    double sum = 0.0;
+    for (int64_t i = 0; i < n; i++) sum += (double)(ref_fp16_to_fp32(x[i]) * ref_fp16_to_fp32(y[i]));
+    return (float)sum;
+}
+
+float ref_vec_dot_bf16(int64_t n, const void *vx, const void *vy) {
+    const uint16_t *x = (const uint16_t *)vx, *y = (const uint16_t *)vy;
+    double sum = 0.0;
+    for (int64_t i = 0; i < n; i++) sum += (double)(ref_bf16_to_fp32(x[i]) * ref_bf16_to_fp32(y[i]));
+    return (float)sum;
+}
+
+
 typedef void (*quant_fn)(const float *, void *, int64_t);
 typedef float (*dot_fn)(int64_t, const void *, const void *);
 
@@ -670,6 +733,9 @@ static quant_fn quantizer_for(int type) {
     case REF_TYPE_Q4_K: return ref_quantize_row_q4_K;
     case REF_TYPE_Q6_K: return ref_quantize_row_q6_K;
     case REF_TYPE_Q8_K: return ref_quantize_row_q8_K;
+    case REF_TYPE_F32: return convert_row_f32;
+    case REF_TYPE_F16: return convert_row_f16;
+    case REF_TYPE_BF16: return convert_row_bf16;
     default: return NULL;
     }
 }
@@ -680,6 +746,9 @@ static dot_fn dot_for(int wtype) {
     case REF_TYPE_Q8_0: return ref_vec_dot_q8_0_q8_0;
     case REF_TYPE_Q4_K: return ref_vec_dot_q4_K_q8_K;
     case REF_TYPE_Q6_K: return ref_vec_dot_q6_K_q8_K;
+    case REF_TYPE_F32: return ref_vec_dot_f32;
+    case REF_TYPE_F16: return ref_vec_dot_f16;
+    case REF_TYPE_BF16: return ref_vec_dot_bf16;
     default: return NULL;
     }
 }

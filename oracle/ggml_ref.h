@@ -2,7 +2,7 @@
  * CPU oracle for the GGUF block-quantized matmul path  --  TEST INFRASTRUCTURE ONLY.
  *
  * A scalar C restatement of the ggml CPU backend's semantics for
- *   mul_mat(W quantized {Q4_0,Q8_0,Q4_K,Q6_K}, X f32) -> Y f32
+ *   mul_mat(W quantized {Q4_0,Q8_0,Q4_K,Q6_K} or plain {F32,F16,BF16}, X f32) -> Y f32
  * i.e. activation quantization to Q8_0 / Q8_K followed by the per-type integer dot products.
  * Nothing in the shipped library links or calls this file: it is the checker the GPU path is
  * compared against, and the timed "port" CPU baseline.
@@ -19,6 +19,10 @@
  * Parity status per function (what pins it is in tests/test_oracle_*.py):
  *   fp16<->fp32, q8_0/q8_K quantizers, 6-bit scale unpack, four vec_dots, dequantizers,
  *   mul_mat driver:  pinned (numpy float16, closed forms, fp64 brute force, KATs).
+ *   F32 / F16 / BF16 weights (activations converted to the weight's type, products in fp32, sum in double):
+ *   pinned as mathematics (numpy float16 casts, bfloat16 rounding against an integer statement of
+ *   round-to-nearest-even over every 16-bit pattern and its neighbours, fp64 dot products of the converted
+ *   operands).  Upstream's SIMD variants sum in fp32 lanes: PARITY UNPINNED below 1e-6 relative.
  *   mul_mat_id driver: the per-pair arithmetic is the pinned vec_dots; the indexing is pinned by
  *   its reduction to mul_mat (one expert; a pair's result equals mul_mat on that expert alone) and
  *   fp64 brute force.  The rule "slot i reads activation row i mod ne11" is upstream ggml's and the
@@ -45,7 +49,7 @@ extern "C" {
 #endif
 
 /* ggml_type ids, /root/reference/fs/ggml/type.go:250-268 */
-enum { REF_TYPE_F32 = 0, REF_TYPE_Q4_0 = 2, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12,
+enum { REF_TYPE_F32 = 0, REF_TYPE_F16 = 1, REF_TYPE_BF16 = 30, REF_TYPE_Q4_0 = 2, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12,
        REF_TYPE_Q6_K = 14, REF_TYPE_Q8_K = 15 };
 
 int64_t ref_block_size(int type);               /* elements per block, 0 if unknown */
@@ -54,6 +58,8 @@ int64_t ref_row_size(int type, int64_t k);      /* bytes of a row of k elements,
 
 uint16_t ref_fp32_to_fp16(float f);
 float    ref_fp16_to_fp32(uint16_t h);
+uint16_t ref_fp32_to_bf16(float f);             /* round to nearest even, NaNs made quiet */
+float    ref_bf16_to_fp32(uint16_t h);
 
 /* activation quantizers (canonical scalar *_ref semantics) */
 void ref_quantize_row_q8_0(const float *x, void *y, int64_t k);
@@ -63,7 +69,8 @@ void ref_quantize_row_q8_K(const float *x, void *y, int64_t k);
 void ref_quantize_row_q4_0(const float *x, void *y, int64_t k);
 void ref_quantize_row_q4_K(const float *x, void *y, int64_t k);
 void ref_quantize_row_q6_K(const float *x, void *y, int64_t k);
-/* dispatch on type (2, 8, 12, 14, 15); rows are independent. returns 0 or -1 */
+/* dispatch on type (2, 8, 12, 14, 15; 0, 1, 30: conversion of the row to f32 / f16 / bf16); rows are independent.
+ * returns 0 or -1 */
 int  ref_quantize(int type, const float *x, void *y, int64_t k, int64_t rows, int nthreads);
 
 /* The two searches inside the K-quant encoders, callable on one group of values so that tests can check what they
@@ -85,8 +92,13 @@ float ref_vec_dot_q4_0_q8_0(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q8_0_q8_0(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q4_K_q8_K(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q6_K_q8_K(int64_t n, const void *x, const void *y);
+/* the unquantized types: both rows in the weight's type, products in fp32, sum in double in element order */
+float ref_vec_dot_f32(int64_t n, const void *x, const void *y);
+float ref_vec_dot_f16(int64_t n, const void *x, const void *y);
+float ref_vec_dot_bf16(int64_t n, const void *x, const void *y);
 
-/* the activation type the CPU path quantizes to for a given weight type (8 or 15), -1 unknown */
+/* the activation type the CPU path converts to for a given weight type (8 or 15; 0, 1, 30 for the weight types
+ * F32, F16, BF16 themselves), -1 unknown */
 int  ref_vec_dot_type(int wtype);
 
 /*

@@ -37,7 +37,9 @@ def test_size_tables_match_reference_golden():
 def test_vec_dot_type():
     assert qmm.vec_dot_type(qmm.Q4_0) == qmm.Q8_0 and qmm.vec_dot_type(qmm.Q8_0) == qmm.Q8_0
     assert qmm.vec_dot_type(qmm.Q4_K) == qmm.Q8_K and qmm.vec_dot_type(qmm.Q6_K) == qmm.Q8_K
-    assert qmm.vec_dot_type(qmm.F32) == -1 and qmm.vec_dot_type(13) == -1
+    # the unquantized weight types are multiplied in their own type
+    assert [qmm.vec_dot_type(t) for t in (qmm.F32, qmm.F16, qmm.BF16)] == [qmm.F32, qmm.F16, qmm.BF16]
+    assert qmm.vec_dot_type(13) == -1 and qmm.vec_dot_type(qmm.Q8_K) == -1
 
 
 def test_argument_errors_without_a_device():
