@@ -455,6 +455,8 @@ def main() -> int:
         for label, t in (("F16", qmm.F16), ("BF16", qmm.BF16), ("F32", qmm.F32)):
             tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
             other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TFLOP/s": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
+        tm, _ = time_mulmat(qmm.F16, 14336, 4096, 512, 3)
+        other["F16 GEMM ffn_gate 14336x4096 B=512"] = {"us": round(tm * 1e6, 1), "TFLOP/s": round(2.0 * 512 * 14336 * 4096 / tm / 1e12, 1)}
         # expert-indexed product: 128 experts of 768x2048 (Q4_K), 8 used per token
         n_exp, n_used, em, ek = 128, 8, 768, 2048
         raw = np.tile(synth.weights(Q4_K, 2048, ek, seed=1201), (n_exp * em // 2048, 1))

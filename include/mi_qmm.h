@@ -85,9 +85,10 @@ enum {
     MI_QMM_ROUTE_SKINNY_STAGED = 11,   /* K-quant staged matrix-core kernel for 3..31 columns                     */
     MI_QMM_ROUTE_SKINNY_ROWS_Q6K = 12, /* Q6_K rows kernel (the output head at 2..8 columns)                      */
     MI_QMM_ROUTE_GEMV = 13,            /* streaming GEMV on quantized planes                                      */
-    MI_QMM_ROUTE_PLAIN_GEMV = 14,      /* F32 / F16 / BF16 weights: streaming kernel, x converted in its prologue  */
+    MI_QMM_ROUTE_PLAIN_GEMV = 14,      /* F32 / F16 / BF16 weights: vector-ALU streaming kernel, 1..8 columns      */
     MI_QMM_ROUTE_PLAIN_GEMM = 15,      /* F32 / F16 / BF16 weights: tiles on the f32 / f16 / bf16 matrix cores     */
-    MI_QMM_ROUTE_PLAIN_NAIVE = 16      /* F32 / F16 / BF16 weights whose rows are no multiple of 16 bytes          */
+    MI_QMM_ROUTE_PLAIN_NAIVE = 16,     /* F32 / F16 / BF16 weights whose rows are no multiple of 16 bytes          */
+    MI_QMM_ROUTE_PLAIN_SKINNY = 17     /* F32 / F16 / BF16 weights at 1..16 columns: weights straight into MFMA operands */
 };
 
 /* ---- size tables: replace TensorType.BlockSize / TypeSize and Tensor.Size's row rule

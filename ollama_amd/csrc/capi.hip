@@ -682,6 +682,7 @@ int plain_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_
 int plain_route(const mi_qmm_weight *w, int64_t n) {
     switch (plain_kind(w->dev.type, w->dev.K, w->dev.M, n)) {
     case 1: case 4: return MI_QMM_ROUTE_PLAIN_GEMV;
+    case 5: return MI_QMM_ROUTE_PLAIN_SKINNY;
     case 2: return MI_QMM_ROUTE_PLAIN_GEMM;
     case 3: return MI_QMM_ROUTE_PLAIN_NAIVE;
     default: return 0;

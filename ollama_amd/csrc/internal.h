@@ -179,7 +179,8 @@ hipError_t launch_skinny_id(const DevWeight &w, int n_expert, const DevAct &a, c
 
 // Unquantized weights (F32, F16, BF16; plain.hip): x f32 [N][K] on the device, y[n*M + m].
 //   plain_kind: 0 = not such a product, 1 = streaming kernel (N <= 8, rows a multiple of 16 bytes), 2 = matrix-core tiles
-//   (rows a multiple of 64 bytes), 3 = a wave per output (any K), 4 = the streaming kernel, 8 columns per launch.
+//   (rows a multiple of 64 bytes), 3 = a wave per output (any K), 4 = the streaming kernel, 8 columns per launch,
+//   5 = the matrix-core streaming kernel (N <= 16, rows a multiple of 64 bytes, the converted x fits the LDS).
 //   force: 0 = as plain_kind says, 1 = never the tiles, 2 = the tiles or an error.
 //   xc: device scratch of plain_convert_bytes() bytes for the converted activations of kind 2 (F16 / BF16).
 bool plain_type(int type);

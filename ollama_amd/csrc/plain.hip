@@ -8,14 +8,17 @@
 // the kernels here in fp32 (lane partial sums, then a tree over the lanes; the matrix cores' own order in the GEMM):
 // the difference is rounding of fp32 sums, orders of magnitude inside the path's 1e-3 tolerance.
 //
-// Three kernels:
-//   plain_gemv_kernel   1..8 activation columns, bound by HBM: a wave streams two weight rows at a time with 16-byte
-//                       loads, the converted activations sit in LDS (all of K where it fits, else chunk by chunk).
-//   plain_gemm_kernel   9 columns and more: 128 x 128 (or 128 x 32) output tiles on v_mfma_f32_32x32x16_{f16,bf16} /
+// Four kernels:
+//   plain_skinny_kernel 1..16 activation columns whose converted form fits the LDS, bound by HBM: weights straight from
+//                       HBM into the operands of 16 x 16 MFMAs, a ring of eight 16-byte loads in flight per lane.
+//   plain_gemv_kernel   1..8 columns of anything else with rows of whole 16-byte pieces: a wave streams two weight rows
+//                       at a time, vector ALU, the converted activations in LDS chunk by chunk.
+//   plain_gemm_kernel   more columns: 128 x 128 (or 128 x 32) output tiles on v_mfma_f32_32x32x16_{f16,bf16} /
 //                       v_mfma_f32_32x32x2_f32, operands staged through LDS in two buffers, from activations converted
 //                       once by plain_convert_kernel.
 //   plain_naive_kernel  rows whose byte length is no multiple of 16 (K odd ...): a wave per output, element loads.
 #include <algorithm>
+#include <type_traits>
 
 #include "internal.h"
 
@@ -158,6 +161,119 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void plain_gemv_kernel(const uint8
     }
 }
 
+// ---- 1..16 columns on the matrix cores ------------------------------------------------------------------------------
+// The weights go from HBM straight into the A operand of a 16 x 16 MFMA: lane (r, g) of a wave holds bytes 16 g .. 16 g + 15
+// of a 64-byte step of row r of the wave's group of 16 rows (v_mfma_f32_16x16x32_f16 / _bf16: 8 elements of K group g;
+// v_mfma_f32_16x16x4_f32: four MFMAs, one per float), a ring of SK_RING steps in flight per lane.  The B operand is the
+// converted activations, resident in LDS for the whole launch: column c at XOFF + c * (row bytes + 16) -- the 16 bytes
+// shift neighbouring columns to other banks -- and the lanes of columns that do not exist read a block of zeros.
+// A workgroup of 16 waves is RG row groups x S segments of K (S a power of two); the segments' partial tiles are added in
+// segment order through LDS, so a result does not depend on the launch geometry beyond S.
+// Accumulator q of lane (c, g) is weight row 4 g + q of the group and activation column c.
+// Requires (K * ES) % 64 == 0 and 256 + N * (K * ES + 16) + 16 KiB of LDS.
+constexpr int SK_WAVES = 16, SK_RING = 8, SK_XOFF = 256;
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int TYPE>
+__device__ __forceinline__ void skinny_step(const v4u &a, const v4u &b, v4f *acc, int which) {
+    if (TYPE == T_F32) {
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(bits_f32(a.x), bits_f32(b.x), acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(bits_f32(a.y), bits_f32(b.y), acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(bits_f32(a.z), bits_f32(b.z), acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(bits_f32(a.w), bits_f32(b.w), acc[3], 0, 0, 0);
+    } else if (TYPE == T_F16) {
+        acc[which] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), acc[which], 0, 0, 0);
+    } else {
+        acc[which] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc[which], 0, 0, 0);
+    }
+}
+
+template <int TYPE>
+__global__ __launch_bounds__(64 * SK_WAVES) void plain_skinny_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x,
+                                                                     float *__restrict__ y, int K, int64_t M, int N, int S, int sps) {
+    constexpr int ES = TYPE == T_F32 ? 4 : 2;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+    const int RG = SK_WAVES / S, rg = wave / S, seg = wave - rg * S;
+    const int64_t groups = (M + 15) / 16, group = (int64_t)blockIdx.x * RG + rg;
+    const bool live = group < groups;
+    const int row_bytes = K * ES, k64 = row_bytes / 64, cs = row_bytes + 16;
+    const int64_t row = live ? (group * 16 + r < M ? group * 16 + r : M - 1) : 0;
+    const int t0 = seg * sps, t1 = t0 + sps < k64 ? t0 + sps : k64;  // this wave's steps (none when t0 >= k64)
+    const uint8_t *wp = w + row * (int64_t)row_bytes + g * 16;
+    auto fetch = [&](int t) { return *reinterpret_cast<const v4u *>(wp + (int64_t)(t < k64 ? t : k64 - 1) * 64); };
+
+    v4u ring[SK_RING];
+#pragma unroll
+    for (int j = 0; j < SK_RING; j++) ring[j] = fetch(t0 + j);
+
+    // the activations, converted to the weight's type
+    if (tid < 64) reinterpret_cast<unsigned *>(lds)[tid] = 0u;
+    for (int c = 0; c < N; c++) {
+        const float4 *xc = reinterpret_cast<const float4 *>(x + (int64_t)c * K);
+        uint8_t *dst = lds + SK_XOFF + c * cs;
+        for (int i = tid; i < K / 4; i += 64 * SK_WAVES) {
+            const float4 v = xc[i];
+            if (TYPE == T_F32) *reinterpret_cast<float4 *>(dst + i * 16) = v;
+            else {
+                uint2 p;
+                p.x = (unsigned)narrow16<TYPE>(v.x) | ((unsigned)narrow16<TYPE>(v.y) << 16);
+                p.y = (unsigned)narrow16<TYPE>(v.z) | ((unsigned)narrow16<TYPE>(v.w) << 16);
+                *reinterpret_cast<uint2 *>(dst + i * 8) = p;
+            }
+        }
+    }
+    __syncthreads();
+
+    const uint8_t *xp = r < N ? lds + SK_XOFF + r * cs + g * 16 : lds;
+    const int xstep = r < N ? 64 : 0;
+    v4f acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    int t = t0;
+    // full turns of the ring: every slot is multiplied and asked for again
+    for (; t + 2 * SK_RING <= t1; t += SK_RING) {
+#pragma unroll
+        for (int j = 0; j < SK_RING; j++) {
+            const v4u b = *reinterpret_cast<const v4u *>(xp + (int64_t)(t + j) * xstep);
+            skinny_step<TYPE>(ring[j], b, acc, j & 1);
+            ring[j] = fetch(t + j + SK_RING);
+        }
+    }
+    // the last one or two turns
+    if (t + SK_RING < t1) {
+#pragma unroll
+        for (int j = 0; j < SK_RING; j++) {
+            const v4u b = *reinterpret_cast<const v4u *>(xp + (int64_t)(t + j) * xstep);
+            skinny_step<TYPE>(ring[j], b, acc, j & 1);
+            ring[j] = fetch(t + j + SK_RING);
+        }
+        t += SK_RING;
+    }
+#pragma unroll
+    for (int j = 0; j < SK_RING; j++)
+        if (t + j < t1) {
+            const v4u b = *reinterpret_cast<const v4u *>(xp + (int64_t)(t + j) * xstep);
+            skinny_step<TYPE>(ring[j], b, acc, j & 1);
+        }
+
+    v4f sum = TYPE == T_F32 ? (acc[0] + acc[1]) + (acc[2] + acc[3]) : acc[0] + acc[1];
+    if (S > 1) {
+        v4f *part = reinterpret_cast<v4f *>(lds + (SK_XOFF + N * cs + 15) / 16 * 16);
+        part[wave * 64 + lane] = sum;
+        __syncthreads();
+        if (seg != 0) return;
+        for (int sgm = 1; sgm < S; sgm++) sum += part[(wave + sgm) * 64 + lane];
+    }
+    if (!live || r >= N) return;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int64_t m = group * 16 + 4 * g + q;
+        if (m < M) y[(int64_t)r * M + m] = sum[q];
+    }
+}
+
 // ---- any K: a wave per output, element loads -------------------------------------------------------------------------
 template <int TYPE>
 __global__ __launch_bounds__(256) void plain_naive_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y,
@@ -216,16 +332,19 @@ __global__ __launch_bounds__(64 * WM * WN) void plain_gemm_kernel(const uint8_t 
             src[i] = xc + n * row_bytes + q * 16;
         }
     }
-    v4u regs[PP];
-    auto fetch = [&](int kt) {
+    // two stages on their way in registers while a third is multiplied out of LDS: stage kt + 1 sits in set (kt + 1) & 1,
+    // stage kt + 2 in set kt & 1 (stages past the last are the last one again: no load under a condition)
+    v4u regs[2][PP];
+    auto fetch = [&](int set, int kt) {
+        const int64_t off = (int64_t)(kt < nk ? kt : nk - 1) * 64;
 #pragma unroll
         for (int i = 0; i < PP; i++)
-            if (dst[i] >= 0) regs[i] = *reinterpret_cast<const v4u *>(src[i] + (int64_t)kt * 64);
+            if (dst[i] >= 0) regs[set][i] = *reinterpret_cast<const v4u *>(src[i] + off);
     };
-    auto park = [&](int buf) {
+    auto park = [&](int set, int buf) {
 #pragma unroll
         for (int i = 0; i < PP; i++)
-            if (dst[i] >= 0) *reinterpret_cast<v4u *>(&lds[buf][dst[i]]) = regs[i];
+            if (dst[i] >= 0) *reinterpret_cast<v4u *>(&lds[buf][dst[i]]) = regs[set][i];
     };
 
     v16f acc[TN][TM];
@@ -239,12 +358,14 @@ __global__ __launch_bounds__(64 * WM * WN) void plain_gemm_kernel(const uint8_t 
     const int row_in = lane & 31, kg = lane >> 5;
     const int wrow = (wm * TM * 32 + row_in) * LDR, xrow = (BM + wn * TN * 32 + row_in) * LDR;
 
-    fetch(0);
-    park(0);
+    fetch(0, 0);
+    park(0, 0);
+    fetch(1, 1);
+    fetch(0, 2);
     __syncthreads();
-    for (int kt = 0; kt < nk; kt++) {
-        if (kt + 1 < nk) fetch(kt + 1);
-        const uint8_t *L = lds[kt & 1];
+    auto stage = [&](int kt, auto parity) {
+        constexpr int P = decltype(parity)::value;  // kt & 1
+        const uint8_t *L = lds[P];
         if (TYPE == T_F32) {
             // the 16 products of a stage are added up from zero and their sum joins the running total: K / 16 roundings
             // of the total instead of K / 2 (a row of 14336 floats: 896 instead of 7168)
@@ -294,8 +415,13 @@ __global__ __launch_bounds__(64 * WM * WN) void plain_gemm_kernel(const uint8_t 
                     }
             }
         }
-        if (kt + 1 < nk) park((kt + 1) & 1);
+        park(P ^ 1, P ^ 1);   // stage kt + 1 into the other buffer (its last readers passed the barrier below one stage ago)
+        fetch(P ^ 1, kt + 3);
         __syncthreads();
+    };
+    for (int kt = 0; kt < nk; kt += 2) {
+        stage(kt, std::integral_constant<int, 0>());
+        if (kt + 1 < nk) stage(kt + 1, std::integral_constant<int, 1>());
     }
 
 #pragma unroll
@@ -334,12 +460,44 @@ hipError_t gemv_typed(const DevWeight &w, const float *x, int ncols, float *y, i
     return hipGetLastError();
 }
 
+size_t skinny_lds(int type, int64_t K, int N) {
+    return (size_t)(SK_XOFF + N * (K * elem_size(type) + 16) + 15) / 16 * 16 + SK_WAVES * 1024;
+}
+
 template <int TYPE>
-hipError_t gemm_typed(const DevWeight &w, const void *xc, int64_t N, float *y, hipStream_t s) {
+hipError_t skinny_typed(const DevWeight &w, const float *x, int N, float *y, int num_cus, hipStream_t s) {
+    static bool allowed[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !allowed[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(plain_skinny_kernel<TYPE>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        allowed[dev] = true;
+    }
+    const int k64 = (int)(w.K * elem_size(TYPE) / 64);
+    const int64_t groups = (w.M + 15) / 16;
+    // segments of K per row group: as many as keep the launch within one workgroup per CU (the registers leave room for
+    // one; a second round of workgroups that fills part of the CUs costs a whole round: 14336 x 4096 halves at one column
+    // 28.3 us with 448 workgroups), while a segment keeps a ring of steps
+    int S = 1;
+    while (S < SK_WAVES && groups * (2 * S) <= (int64_t)num_cus * SK_WAVES && k64 / (2 * S) >= SK_RING) S *= 2;
+    const int sps = (k64 + S - 1) / S, RG = SK_WAVES / S;
+    const int64_t grid = (groups + RG - 1) / RG;
+    if (grid > 0x7fffffff) return hipErrorInvalidValue;
+    plain_skinny_kernel<TYPE><<<dim3((unsigned)grid), dim3(64 * SK_WAVES), skinny_lds(TYPE, w.K, N), s>>>(w.p0, x, y, (int)w.K, w.M, N, S, sps);
+    return hipGetLastError();
+}
+
+template <int TYPE>
+hipError_t gemm_typed(const DevWeight &w, const void *xc, int64_t N, float *y, int num_cus, hipStream_t s) {
     const uint8_t *xb = (const uint8_t *)xc;
+    const int64_t mt = (w.M + 127) / 128;
     if (N <= 32) {
-        const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((w.M + 127) / 128));
+        const dim3 grid((unsigned)((N + 31) / 32), (unsigned)mt);
         plain_gemm_kernel<TYPE, 4, 1, 1, 1><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+    } else if (TYPE == T_F32 && mt * ((N + 127) / 128) < num_cus) {
+        // too few 128 x 128 tiles for the CUs: 128 x 64 (4096 x 4096 at 512 columns 370 -> 230 us; the 16-bit types, whose
+        // MFMAs are eight times as fast, are bound by the LDS reads and lose there: 72 -> 95 us)
+        const dim3 grid((unsigned)((N + 63) / 64), (unsigned)mt);
+        plain_gemm_kernel<TYPE, 2, 2, 2, 1><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
     } else {
         const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((w.M + 127) / 128));
         plain_gemm_kernel<TYPE, 2, 2, 2, 2><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
@@ -356,6 +514,7 @@ int plain_kind(int type, int64_t K, int64_t M, int64_t N, int force) {
     const int64_t row_bytes = K * elem_size(type);
     const bool tiles = row_bytes % 64 == 0 && (M + 127) / 128 <= 65535;
     if (force == 2) return tiles ? 2 : 0;
+    if (N <= 16 && row_bytes % 64 == 0 && skinny_lds(type, K, (int)N) <= 160 * 1024) return 5;
     if (N <= 8 && row_bytes % 16 == 0) return 1;
     if (tiles && force != 1) return 2;
     return row_bytes % 16 == 0 ? 4 : 3;
@@ -381,8 +540,15 @@ hipError_t launch_plain(const DevWeight &w, const float *x, int64_t N, float *y,
         }
         return hipSuccess;
     }
+    if (kind == 5) {
+        switch (w.type) {
+        case T_F32: return skinny_typed<T_F32>(w, x, (int)N, y, num_cus, s);
+        case T_F16: return skinny_typed<T_F16>(w, x, (int)N, y, num_cus, s);
+        default: return skinny_typed<T_BF16>(w, x, (int)N, y, num_cus, s);
+        }
+    }
     if (kind == 2) {
-        if (w.type == T_F32) return gemm_typed<T_F32>(w, x, N, y, s);
+        if (w.type == T_F32) return gemm_typed<T_F32>(w, x, N, y, num_cus, s);
         if (!xc) return hipErrorInvalidValue;
         const int64_t count = w.K * N;
         const unsigned blocks = (unsigned)std::min<int64_t>((count + 255) / 256, 8 * (int64_t)num_cus);
@@ -390,7 +556,7 @@ hipError_t launch_plain(const DevWeight &w, const float *x, int64_t N, float *y,
         else plain_convert_kernel<T_BF16><<<blocks, 256, 0, s>>>(x, (unsigned short *)xc, count);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
-        return w.type == T_F16 ? gemm_typed<T_F16>(w, xc, N, y, s) : gemm_typed<T_BF16>(w, xc, N, y, s);
+        return w.type == T_F16 ? gemm_typed<T_F16>(w, xc, N, y, num_cus, s) : gemm_typed<T_BF16>(w, xc, N, y, num_cus, s);
     }
     const int64_t outs = w.M * N;
     const unsigned blocks = (unsigned)std::min<int64_t>((outs + 3) / 4, 16 * (int64_t)num_cus);

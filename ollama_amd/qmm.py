@@ -23,7 +23,7 @@ PATH_AUTO, PATH_GEMV, PATH_GEMM, PATH_QUERY = 0, 1, 2, 3
 # what PATH_QUERY returns (MI_QMM_ROUTE_*): the kernel a product takes
 ROUTES = {1: "gemv_f32", 2: "deep_f32", 3: "gemm_blk32", 4: "gemm_f16", 5: "gemm_q6k", 6: "gemm_int8", 7: "skinny32",
           8: "skinny_deep", 9: "skinny_direct", 10: "skinny_rows_q4k", 11: "skinny_staged", 12: "skinny_rows_q6k", 13: "gemv",
-          14: "plain_gemv", 15: "plain_gemm", 16: "plain_naive"}
+          14: "plain_gemv", 15: "plain_gemm", 16: "plain_naive", 17: "plain_skinny"}
 PRODUCE_NONE, PRODUCE_RMSNORM, PRODUCE_SWIGLU = 0, 1, 2
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM, ERR_NODEVICE = 0, -1, -2, -3, -4, -5
 

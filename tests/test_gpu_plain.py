@@ -32,11 +32,13 @@ def _weights(t, m, k, seed, scale=0.05):
 
 
 # (rows, K, activation rows): every kernel and both sides of each switch
-#   streaming kernel, x resident / in chunks; rounds with dead waves (rows no multiple of 32, odd row counts);
+#   matrix-core streaming kernel (1..16 columns, one to sixteen K segments per row group, ragged last segments and row
+#   groups); vector-ALU streaming kernel where the activations do not fit the LDS, x in chunks; rounds with dead waves;
 #   tiles of 128 x 32 and 128 x 128 with ragged edges; rows of 16-byte but not 64-byte multiples (8 columns per launch);
 #   the feed-forward shapes at decode size, a prefill-sized product, long rows on the tiles; odd K (a wave per output)
 SHAPES = [
-    (512, 4096, 1), (512, 4096, 2), (515, 4096, 3), (77, 4096, 8), (1, 256, 1), (33, 64, 5),
+    (512, 4096, 1), (512, 4096, 2), (515, 4096, 3), (77, 4096, 8), (1, 256, 1), (33, 64, 5), (5000, 2048, 16),
+    (70000, 256, 2), (40, 4096 + 64, 7), (16, 64 * 9, 11),
     (256, 14336, 1), (256, 14336, 4), (200, 14336, 8), (96, 40960, 2),
     (512, 4096, 9), (300, 4096, 32), (515, 1024, 33), (130, 2048, 130), (1000, 512, 257),
     (14336, 4096, 1), (4096, 14336, 4), (2048, 4096, 128), (256, 14336, 64),
@@ -64,6 +66,8 @@ def test_plain_weights_against_the_oracle(ctx, t, m, k, n):
 
 def _expected_route(t, m, k, n):
     row = k * (4 if t == F32 else 2)
+    if n <= 16 and row % 64 == 0 and (256 + n * (row + 16) + 15) // 16 * 16 + 16384 <= 160 * 1024:
+        return "plain_skinny"  # the converted activations fit the LDS
     if n <= 8 and row % 16 == 0:
         return "plain_gemv"
     if row % 64 == 0:
