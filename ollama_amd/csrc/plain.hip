@@ -299,6 +299,18 @@ __global__ __launch_bounds__(256) void plain_naive_kernel(const uint8_t *__restr
     }
 }
 
+// Which output tile a workgroup takes.  Workgroups go to the eight XCDs round robin by their id, and each XCD has an L2
+// of its own: the workgroups that share a weight tile (all activation tiles of one tile of weight rows) must sit on one
+// XCD, or every XCD fetches that tile from HBM for itself (14336 x 4096 halves at 512 columns: eight activation tiles,
+// 940 MB of weight reads for 117 MB of weights).  XCD k takes the weight tiles k, k + 8, ..., an activation tile after
+// the other.  The grid is tiles_n * (tiles_m rounded up to a multiple of 8); false: no such tile.
+__device__ __forceinline__ bool tile_of(unsigned id, int tiles_n, int64_t tiles_m, int64_t &mt, int &nt) {
+    const unsigned xcd = id & 7, slot = id >> 3;
+    nt = (int)(slot % (unsigned)tiles_n);
+    mt = (int64_t)(slot / (unsigned)tiles_n) * 8 + xcd;
+    return mt < tiles_m;
+}
+
 // ---- 9 columns and more: tiles on the matrix cores ---------------------------------------------------------------------
 // Workgroup of WM x WN waves; a wave owns TN x TM accumulator tiles of 32 (activation rows) x 32 (weight rows).  The
 // A operand of an MFMA is the activations, the B operand the weights: accumulator i of lane l is activation row
@@ -313,7 +325,10 @@ __global__ __launch_bounds__(64 * WM * WN) void plain_gemm_kernel(const uint8_t 
     constexpr int LDR = 80, ROWS = BM + BN, PIECES = ROWS * 4, PP = (PIECES + NT - 1) / NT;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][ROWS * LDR];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave / WN, wn = wave % WN;
-    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
+    int64_t mt;
+    int nt;
+    if (!tile_of(blockIdx.x, (int)((N + BN - 1) / BN), (M + BM - 1) / BM, mt, nt)) return;
+    const int64_t n0 = (int64_t)nt * BN, m0 = mt * BM;
     const int64_t row_bytes = K * ES;
     const int nk = (int)(row_bytes / 64);
 
@@ -438,6 +453,121 @@ __global__ __launch_bounds__(64 * WM * WN) void plain_gemm_kernel(const uint8_t 
     }
 }
 
+// ---- the tiles for F16 / BF16 with the weights kept out of LDS --------------------------------------------------------
+// The tiled kernel above reads one 1 KiB operand fragment from LDS per MFMA, and at the 16-bit types' MFMA rate that
+// read is what bounds it.  Here only the activations go through LDS: a wave owns 64 weight rows, four groups of 16, whose
+// fragments it loads from global memory straight into the B operand of v_mfma_f32_16x16x32 -- lane (c, kg) holds bytes
+// 16 kg .. 16 kg + 15 of a 64-byte K step of row c, so an instruction reads runs of 64 bytes of 16 rows (the 32 x 32
+// shape would read 16-byte pieces of 64 different lines per instruction: measured, 164 against 133 us on 14336 x 4096 at
+// 512 columns) -- and multiplies each against a 64-row activation tile: four LDS reads per sixteen MFMAs.  Workgroup:
+// two waves, 128 weight rows x 64 activation rows; a stage is two K steps (128 bytes of every row); two stages of
+// weights in registers, the activation stage after next in registers, the next one in LDS.
+// Accumulator q of lane (c, kg) in tile (a, b) is activation row 16 a + 4 kg + q and weight row 16 b + c.
+// Requires (K * 2) % 128 == 0.
+constexpr int G2_WAVES = 2, G2_TM = 4, G2_TN = 4, G2_BM = G2_WAVES * G2_TM * 16, G2_BN = G2_TN * 16, G2_LDR = 144;
+template <int TYPE>
+__global__ __launch_bounds__(64 * G2_WAVES, 2) void plain_gemm2_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ xc,
+                                                                    float *__restrict__ y, int64_t K, int64_t M, int64_t N) {
+    constexpr int NT = 64 * G2_WAVES, PP = G2_BN * 8 / NT;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][G2_BN * G2_LDR];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kg = lane >> 4;
+    int64_t mt;
+    int nt;
+    if (!tile_of(blockIdx.x, (int)((N + G2_BN - 1) / G2_BN), (M + G2_BM - 1) / G2_BM, mt, nt)) return;
+    const int64_t n0 = (int64_t)nt * G2_BN, m0 = mt * G2_BM;
+    const int64_t row_bytes = K * 2;
+    const int nk = (int)(row_bytes / 128);
+
+    const uint8_t *wsrc[G2_TM];
+#pragma unroll
+    for (int b = 0; b < G2_TM; b++) {
+        const int64_t m = m0 + wave * (G2_TM * 16) + b * 16 + c;
+        wsrc[b] = w + (m < M ? m : M - 1) * row_bytes + kg * 16;
+    }
+    const uint8_t *asrc[PP];
+    int adst[PP];
+#pragma unroll
+    for (int i = 0; i < PP; i++) {
+        const int idx = tid + i * NT, r = idx >> 3, q = idx & 7;
+        const int64_t n = n0 + r < N ? n0 + r : N - 1;
+        asrc[i] = xc + n * row_bytes + q * 16;
+        adst[i] = r * G2_LDR + q * 16;
+    }
+    v4u wr[2][G2_TM][2], ar[PP];
+    auto fetch_w = [&](int set, int kt) {
+        const int64_t off = (int64_t)(kt < nk ? kt : nk - 1) * 128;
+#pragma unroll
+        for (int b = 0; b < G2_TM; b++)
+#pragma unroll
+            for (int k = 0; k < 2; k++) wr[set][b][k] = *reinterpret_cast<const v4u *>(wsrc[b] + off + k * 64);
+    };
+    auto fetch_a = [&](int kt) {
+        const int64_t off = (int64_t)(kt < nk ? kt : nk - 1) * 128;
+#pragma unroll
+        for (int i = 0; i < PP; i++) ar[i] = *reinterpret_cast<const v4u *>(asrc[i] + off);
+    };
+    auto park_a = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PP; i++) *reinterpret_cast<v4u *>(&lds[buf][adst[i]]) = ar[i];
+    };
+
+    v4f acc[G2_TN][G2_TM];
+#pragma unroll
+    for (int a = 0; a < G2_TN; a++)
+#pragma unroll
+        for (int b = 0; b < G2_TM; b++) acc[a][b] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    fetch_w(0, 0);
+    fetch_a(0);
+    park_a(0);
+    fetch_w(1, 1);
+    fetch_a(1);
+    __syncthreads();
+    const int arow = c * G2_LDR + kg * 16;
+    auto stage = [&](int kt, auto parity) {
+        constexpr int P = decltype(parity)::value;  // kt & 1
+        const uint8_t *L = lds[P];
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            v4u fa[G2_TN];
+#pragma unroll
+            for (int a = 0; a < G2_TN; a++) fa[a] = *reinterpret_cast<const v4u *>(L + arow + a * 16 * G2_LDR + k * 64);
+#pragma unroll
+            for (int a = 0; a < G2_TN; a++)
+#pragma unroll
+                for (int b = 0; b < G2_TM; b++) {
+                    if (TYPE == T_F16)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, fa[a]), __builtin_bit_cast(v8h, wr[P][b][k]),
+                                                                           acc[a][b], 0, 0, 0);
+                    else
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, fa[a]), __builtin_bit_cast(v8bf, wr[P][b][k]),
+                                                                            acc[a][b], 0, 0, 0);
+                }
+        }
+        park_a(P ^ 1);       // activation stage kt + 1 into the other buffer
+        fetch_a(kt + 2);
+        fetch_w(P, kt + 2);  // the weight set just multiplied
+        __syncthreads();
+    };
+    for (int kt = 0; kt < nk; kt += 2) {
+        stage(kt, std::integral_constant<int, 0>());
+        if (kt + 1 < nk) stage(kt + 1, std::integral_constant<int, 1>());
+    }
+
+#pragma unroll
+    for (int b = 0; b < G2_TM; b++) {
+        const int64_t m = m0 + wave * (G2_TM * 16) + b * 16 + c;
+        if (m >= M) continue;
+#pragma unroll
+        for (int a = 0; a < G2_TN; a++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int64_t n = n0 + a * 16 + 4 * kg + q;
+                if (n < N) y[n * M + m] = acc[a][b][q];
+            }
+    }
+}
+
 int elem_size(int type) { return type == T_F32 ? 4 : 2; }
 
 template <int TYPE>
@@ -489,18 +619,34 @@ hipError_t skinny_typed(const DevWeight &w, const float *x, int N, float *y, int
 template <int TYPE>
 hipError_t gemm_typed(const DevWeight &w, const void *xc, int64_t N, float *y, int num_cus, hipStream_t s) {
     const uint8_t *xb = (const uint8_t *)xc;
+    // one-dimensional grids: tiles_n x (tiles_m rounded up to a multiple of 8), see tile_of
+    auto grid_of = [&](int bm, int bn, unsigned &g) {
+        const int64_t tn = (N + bn - 1) / bn, tm8 = ((w.M + bm - 1) / bm + 7) / 8 * 8;
+        if (tn * tm8 > 0x7fffffff) return false;
+        g = (unsigned)(tn * tm8);
+        return true;
+    };
+    unsigned g = 0;
     const int64_t mt = (w.M + 127) / 128;
+    // F16 / BF16 products with too few 128 x 128 tiles for the CUs: 128 x 64 tiles with the weights kept out of LDS (4096 x
+    // 4096 at 512 columns 72 -> 56 us; with tiles enough the 128 x 128 kernel is ahead: 14336 x 4096 at 512 columns 151
+    // against 133 us -- a 128 x 64 tile moves 1.5 times the bytes per flop into the CU)
+    if (TYPE != T_F32 && N > 32 && (w.K * 2) % 128 == 0 && mt * ((N + 127) / 128) < num_cus) {
+        if (!grid_of(G2_BM, G2_BN, g)) return hipErrorInvalidValue;
+        plain_gemm2_kernel<TYPE == T_F32 ? T_F16 : TYPE><<<g, 64 * G2_WAVES, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+        return hipGetLastError();
+    }
     if (N <= 32) {
-        const dim3 grid((unsigned)((N + 31) / 32), (unsigned)mt);
-        plain_gemm_kernel<TYPE, 4, 1, 1, 1><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+        if (!grid_of(128, 32, g)) return hipErrorInvalidValue;
+        plain_gemm_kernel<TYPE, 4, 1, 1, 1><<<g, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
     } else if (TYPE == T_F32 && mt * ((N + 127) / 128) < num_cus) {
         // too few 128 x 128 tiles for the CUs: 128 x 64 (4096 x 4096 at 512 columns 370 -> 230 us; the 16-bit types, whose
         // MFMAs are eight times as fast, are bound by the LDS reads and lose there: 72 -> 95 us)
-        const dim3 grid((unsigned)((N + 63) / 64), (unsigned)mt);
-        plain_gemm_kernel<TYPE, 2, 2, 2, 1><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+        if (!grid_of(128, 64, g)) return hipErrorInvalidValue;
+        plain_gemm_kernel<TYPE, 2, 2, 2, 1><<<g, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
     } else {
-        const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((w.M + 127) / 128));
-        plain_gemm_kernel<TYPE, 2, 2, 2, 2><<<grid, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
+        if (!grid_of(128, 128, g)) return hipErrorInvalidValue;
+        plain_gemm_kernel<TYPE, 2, 2, 2, 2><<<g, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
     }
     return hipGetLastError();
 }
@@ -512,7 +658,7 @@ bool plain_type(int type) { return type == T_F32 || type == T_F16 || type == T_B
 int plain_kind(int type, int64_t K, int64_t M, int64_t N, int force) {
     if (!plain_type(type) || K < 1 || M < 1 || N < 1 || K > 0x7fffffff / 4) return 0;
     const int64_t row_bytes = K * elem_size(type);
-    const bool tiles = row_bytes % 64 == 0 && (M + 127) / 128 <= 65535;
+    const bool tiles = row_bytes % 64 == 0;
     if (force == 2) return tiles ? 2 : 0;
     if (N <= 16 && row_bytes % 64 == 0 && skinny_lds(type, K, (int)N) <= 160 * 1024) return 5;
     if (N <= 8 && row_bytes % 16 == 0) return 1;
