@@ -39,7 +39,7 @@ class DType(enum.IntEnum):  # /root/reference/ml/backend.go:404-412
 
 
 I32 = 26  # ggml_type id of int32, /root/reference/fs/ggml/type.go:252-279
-_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40, I32: DType.I32}
+_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.F16: DType.F16, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40, I32: DType.I32}
 
 
 class Tensor:
@@ -86,9 +86,10 @@ class Tensor:
 
     # -- the op, :151-152
     def Mulmat(self, ctx: "Context", t2: "Tensor") -> "Tensor":
-        """self = W [K, M] (quantized weight), t2 = x [K, N] f32  ->  [M, N] f32, lazily."""
+        """self = W [K, M] (a weight from Backend.Get: block-quantized, or F32 / F16 / BF16), t2 = x [K, N] f32  ->
+        [M, N] f32, lazily."""
         if self._weight is None:
-            raise TypeError("Mulmat: the receiver must be a quantized weight obtained from Backend.Get")
+            raise TypeError("Mulmat: the receiver must be a weight obtained from Backend.Get")
         if len(self._shape) != 2:
             raise TypeError(f"Mulmat: the weight must be 2-D, got {self.Shape()} (expert stacks go through MulmatID)")
         if t2._type != qmm.F32:

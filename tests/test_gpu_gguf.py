@@ -20,7 +20,13 @@ def _model_file(tmp_path):
         tensors.append((name, t, [k, m], raw.tobytes()))
     norm = (1 + 0.05 * np.random.default_rng(9).standard_normal(k)).astype(np.float32)
     tensors.append(("blk.0.attn_norm.weight", 0, [k], norm.tobytes()))   # f32, 1-D: the operand of RMSNorm, kept on the host
-    tensors.append(("token_embd.weight", 0, [k, 4], np.zeros((4, k), np.float32).tobytes()))  # f32, 2-D: not on the path
+    # unquantized 2-D tensors are weights of the path too (multiplied in their own type)
+    rng = np.random.default_rng(10)
+    for name, t, m in (("token_embd.weight", qmm.F32, 4), ("output_norm_proj.weight", qmm.F16, 24), ("mm.0.weight", qmm.BF16, 17)):
+        raw = oracle.quantize(t, (rng.standard_normal((m, k)) * 0.05).astype(np.float32)).reshape(-1)
+        raws[name] = (t, m, raw)
+        tensors.append((name, t, [k, m], raw.tobytes()))
+    tensors.append(("rope_freqs.weight", 26, [k, 2], np.zeros((2, k), np.int32).tobytes()))  # i32, 2-D: not on the path
     p = str(tmp_path / "model.gguf")
     gguf.write_gguf(p, {"general.architecture": "llama", "block_count": np.uint32(1)}, tensors)
     return p, k, raws
@@ -50,7 +56,8 @@ def test_backend_from_gguf_path(tmp_path):
     b = ml.Backend(p)
     b.Load(progress=seen.append)
     assert seen and seen[-1] == 1.0
-    assert b.Get("token_embd.weight") is None and b.Get("nope") is None
+    assert b.Get("rope_freqs.weight") is None and b.Get("nope") is None
+    assert b.Get("output_norm_proj.weight").DType() == ml.DType.F16
     norm = b.Get("blk.0.attn_norm.weight")
     assert norm.Shape() == [k] and norm.DType() == ml.DType.F32 and abs(norm.Floats().mean() - 1) < 0.05
     ctx = b.NewContext()
