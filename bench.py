@@ -443,6 +443,15 @@ def main() -> int:
         for label, t in (("Q4_0", Q4_0), ("Q8_0", Q8_0)):
             tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
             other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TOPS": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
+        # Q5_K (the tensors the Q4_K_S mixture raises): kept as a Q4_K tensor of rows twice as long
+        for label, m, k, ns, copies in (("Q5_K v_proj 1024x4096", 1024, 4096, (1, 4), 40), ("Q5_K ffn_down 4096x14336", 4096, 14336, (1, 4), 10)):
+            for n in ns:
+                tm, wb = time_mulmat(qmm.Q5_K, m, k, n, copies)
+                gbs = alg_bytes(wb, k, m, n) / tm / 1e9
+                other[f"{label} B={n}"] = {"us": round(tm * 1e6, 2), "GB/s": round(gbs, 1),
+                                           "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        tm, _ = time_mulmat(qmm.Q5_K, 4096, 4096, 512, 6)
+        other["Q5_K GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TOPS": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
         # the unquantized weight types (F16 / BF16 / F32 files, and the tensors a K-quant file keeps unquantized)
         for label, t, m, k, ns, copies in (("F16 ffn_gate 14336x4096", qmm.F16, 14336, 4096, (1, 4, 8), 6),
                                            ("BF16 q_proj 4096x4096", qmm.BF16, 4096, 4096, (1, 8), 16),

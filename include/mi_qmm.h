@@ -49,6 +49,7 @@ enum {
     MI_QMM_TYPE_Q4_0 = 2,
     MI_QMM_TYPE_Q8_0 = 8,
     MI_QMM_TYPE_Q4_K = 12,
+    MI_QMM_TYPE_Q5_K = 13,
     MI_QMM_TYPE_Q6_K = 14,
     MI_QMM_TYPE_Q8_K = 15,
     MI_QMM_TYPE_BF16 = 30
@@ -138,13 +139,16 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      fed with the tensor bytes fs/ggml hands out (/root/reference/fs/ggml/gguf.go:281-308;
  *      fs/gguf/gguf.go:388-430): M rows of K elements in GGUF block layout, rows contiguous.
  *      The bytes are copied (and re-laid-out for the device) before the call returns.
- *      ggml_type: the block-quantized types 2 (Q4_0), 8 (Q8_0), 12 (Q4_K), 14 (Q6_K), and the unquantized
- *      ones a GGUF file holds beside them or instead of them, 0 (F32), 1 (F16), 30 (BF16): the file types
- *      /root/reference/fs/ggml/type.go:55-88 accepts, the tensors a K-quant file keeps unquantized and the
- *      ones /root/reference/server/quantization.go:296-333 keeps at f16.  The unquantized types go through
- *      mi_qmm_mulmat, mi_qmm_mulmat_path, mi_qmm_mulmat_noalloc and mi_qmm_mulmat_multi (one product after the
- *      other there); the produced, expert-indexed and pre-quantized entry points take block-quantized weights
- *      only and return MI_QMM_ERR_UNSUPPORTED otherwise.
+ *      ggml_type: the block-quantized types 2 (Q4_0), 8 (Q8_0), 12 (Q4_K), 14 (Q6_K); 13 (Q5_K), which the
+ *      Q4_K_S mixture of the reference's file types gives some tensors; and the unquantized ones a GGUF file
+ *      holds beside them or instead of them, 0 (F32), 1 (F16), 30 (BF16): together every tensor type of the file
+ *      types /root/reference/fs/ggml/type.go:55-88 accepts, the tensors a K-quant file keeps unquantized and the
+ *      ones /root/reference/server/quantization.go:296-333 keeps at f16.  Q5_K and the unquantized types go
+ *      through mi_qmm_mulmat, mi_qmm_mulmat_path, mi_qmm_mulmat_noalloc and mi_qmm_mulmat_multi (one product
+ *      after the other there); the produced, expert-indexed and pre-quantized entry points take Q4_0 / Q8_0 /
+ *      Q4_K / Q6_K weights only and return MI_QMM_ERR_UNSUPPORTED otherwise.  A Q5_K tensor is kept as the Q4_K
+ *      tensor of rows twice as long that gives the same integer sums against [x | x] (1.64 times the bytes of
+ *      the file: its products cost what a Q4_K product of twice the K costs).
  *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
 int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
                          int64_t m, int src_location, mi_qmm_weight **out);

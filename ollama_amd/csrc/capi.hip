@@ -57,6 +57,7 @@ struct mi_qmm_ctx {
     void *io_buf = nullptr;   size_t io_cap = 0;
     void *ws_buf = nullptr;   size_t ws_cap = 0;   // partial sums of a K-split GEMM
     void *pair_buf = nullptr; size_t pair_cap = 0; // the two products of a gated pair when they are not one launch
+    void *dup_buf = nullptr;  size_t dup_cap = 0;  // [x | x] for Q5_K weights (and host staging of such a call)
     bool scratch_frozen = false;                   // mi_qmm_scratch_freeze: growth is an error, not a reallocation
     void *static_scratch = nullptr;                // this device's copy of the file-scope array `scratch` below
 };
@@ -66,6 +67,9 @@ struct mi_qmm_weight {
     void *base = nullptr;
     size_t bytes = 0;
     DevWeight dev{};
+    // a Q5_K tensor: dev is the Q4_K tensor of rows of 2 k5 that stands for it (formats.h), multiplied with [x | x]
+    bool q5k = false;
+    int64_t k5 = 0;
 };
 
 struct mi_qmm_gguf {
@@ -208,7 +212,7 @@ int64_t mi_qmm_row_size(int t, int64_t k) {
 int mi_qmm_vec_dot_type(int wt) {
     switch (wt) {
     case T_Q4_0: case T_Q8_0: return T_Q8_0;
-    case T_Q4_K: case T_Q6_K: return T_Q8_K;
+    case T_Q4_K: case T_Q5_K: case T_Q6_K: return T_Q8_K;
     case T_F32: case T_F16: case T_BF16: return wt;  // multiplied in their own type: x is converted to it
     default: return -1;
     }
@@ -261,6 +265,7 @@ void mi_qmm_destroy(mi_qmm_ctx *ctx) {
         if (ctx->io_buf) (void)hipFree(ctx->io_buf);
         if (ctx->ws_buf) (void)hipFree(ctx->ws_buf);
         if (ctx->pair_buf) (void)hipFree(ctx->pair_buf);
+        if (ctx->dup_buf) (void)hipFree(ctx->dup_buf);
         if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
     }
     delete ctx;
@@ -310,7 +315,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (mi_qmm_vec_dot_type(type) < 0)
-        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 8, 12, 14, 30)", type);
+        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 8, 12, 13, 14, 30)", type);
     if (k <= 0 || m <= 0) return fail(MI_QMM_ERR_INVALID, "k=%lld m=%lld must be positive", (long long)k, (long long)m);
     const int64_t row = mi_qmm_row_size(type, k);
     if (row < 0)
@@ -331,6 +336,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     size_t s0 = 0, s1 = 0, s2 = 0, sd = 0;
     switch (type) {
     case T_Q4_K: case T_F32: case T_F16: case T_BF16: s0 = total; break;
+    case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; break;  // a Q4_K tensor of rows twice as long
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q6_K: s0 = (size_t)(m * (k / 2)); s1 = (size_t)(m * (k / 4)); s2 = (size_t)(m * (k / 16));
@@ -354,6 +360,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     w->dev.p2 = s2 ? b + o2 : nullptr;
     w->dev.d = sd ? (const uint16_t *)(b + od) : nullptr;
     w->dev.K = k; w->dev.M = m; w->dev.type = type;
+    if (type == T_Q5_K) { w->q5k = true; w->k5 = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; }
 
     void *staging = nullptr;
     const uint8_t *src = (const uint8_t *)bytes;
@@ -375,7 +382,8 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
             if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(staging)", e);
             src = (const uint8_t *)staging;
         }
-        e = launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
+        e = type == T_Q5_K ? launch_relayout_q5k(src, k, m, b + o0, ctx->stream)
+                           : launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
         if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
     }
     e = hipStreamSynchronize(ctx->stream);  // the caller's bytes must not be needed after return
@@ -396,8 +404,8 @@ void mi_qmm_weight_free(mi_qmm_weight *w) {
 
 int mi_qmm_weight_info(const mi_qmm_weight *w, int *type, int64_t *k, int64_t *m, int64_t *device_bytes) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
-    if (type) *type = w->dev.type;
-    if (k) *k = w->dev.K;
+    if (type) *type = w->q5k ? T_Q5_K : w->dev.type;
+    if (k) *k = w->q5k ? w->k5 : w->dev.K;
     if (m) *m = w->dev.M;
     if (device_bytes) *device_bytes = (int64_t)w->bytes;
     return MI_QMM_OK;
@@ -626,8 +634,9 @@ int route_f32(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n, int path
 // joint, produced, expert-indexed and pre-quantized forms are for the block-quantized types)
 int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, int path, bool allow_plain = false) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
-    if (!allow_plain && plain_type(w->dev.type))
-        return fail(MI_QMM_ERR_UNSUPPORTED, "this entry point takes block-quantized weights; type %d goes through mi_qmm_mulmat", w->dev.type);
+    if (!allow_plain && (plain_type(w->dev.type) || w->q5k))
+        return fail(MI_QMM_ERR_UNSUPPORTED, "this entry point takes Q4_0 / Q8_0 / Q4_K / Q6_K weights; type %d goes through mi_qmm_mulmat",
+                    w->q5k ? T_Q5_K : w->dev.type);
     if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
         return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
     if (path != MI_QMM_PATH_AUTO && path != MI_QMM_PATH_GEMV && path != MI_QMM_PATH_GEMM && path != MI_QMM_PATH_QUERY)
@@ -699,6 +708,31 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     int rc = check_product_args(ctx, w, location, path, /*allow_plain=*/true);
     if (rc) return rc;
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    if (w->q5k) {
+        // the Q4_K tensor of rows of 2 k that stands for the Q5_K one, against [x | x]
+        mi_qmm_weight lo = *w;
+        lo.q5k = false;
+        if (path == MI_QMM_PATH_QUERY || n == 0) return mi_qmm_mulmat_path(ctx, &lo, x, n, y, location, path);
+        if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
+        const size_t xb = (size_t)(n * w->k5) * 4, yb = (size_t)(n * w->dev.M) * 4;
+        const size_t o_raw = align_up(2 * xb, 256), o_y = o_raw + align_up(xb, 256);
+        if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_y + yb : 2 * xb))) return rc;
+        float *xx = (float *)ctx->dup_buf;
+        const float *dx = x;
+        float *dy = y;
+        if (location == MI_QMM_HOST) {
+            dx = (const float *)((char *)ctx->dup_buf + o_raw);
+            dy = (float *)((char *)ctx->dup_buf + o_y);
+            HIP_TRY(hipMemcpyAsync((void *)dx, x, xb, hipMemcpyHostToDevice, ctx->stream));
+        }
+        HIP_TRY(launch_dup_rows(dx, w->k5, n, xx, ctx->stream));
+        if ((rc = mi_qmm_mulmat_path(ctx, &lo, xx, n, dy, MI_QMM_DEVICE, path))) return rc;
+        if (location == MI_QMM_HOST) {
+            HIP_TRY(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(hipStreamSynchronize(ctx->stream));
+        }
+        return MI_QMM_OK;
+    }
     if (path == MI_QMM_PATH_QUERY) {  // which kernel mi_qmm_mulmat would take; nothing is launched, x and y may be NULL
         if (n == 0) return fail(MI_QMM_ERR_INVALID, "a product of no columns has no route");
         if (plain_type(w->dev.type)) {
@@ -759,15 +793,27 @@ int mi_qmm_mulmat(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64
 // mi_qmm_mulmat on device pointers without any allocation: the quantized activation planes go to this
 // device's copy of the static array `scratch` (ctx->static_scratch), never to the ctx's growable buffers,
 // and the tiled GEMM runs without its K-split workspace.  Same kernels as mi_qmm_mulmat otherwise.
-int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y) {
+static int noalloc_core(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y, void *sbase, size_t sbytes) {
     if (n < 0) return fail(MI_QMM_ERR_INVALID, "n=%lld must be non-negative", (long long)n);
     int rc = check_product_args(ctx, w, MI_QMM_DEVICE, MI_QMM_PATH_AUTO, /*allow_plain=*/true);
     if (rc) return rc;
     if (n == 0) return MI_QMM_OK;
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
+    if (w->q5k) {
+        // [x | x] at the end of the scratch, the quantized planes of the product in front of it
+        mi_qmm_weight lo = *w;
+        lo.q5k = false;
+        const size_t xx_bytes = align_up((size_t)(n * w->k5) * 8, 256);
+        if (xx_bytes + 256 > sbytes)
+            return fail(MI_QMM_ERR_UNSUPPORTED, "n=%lld rows of k=%lld of a Q5_K product need %zu bytes for the repeated activations alone; the "
+                        "static scratch of mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)w->k5, xx_bytes, sbytes);
+        float *xx = (float *)((char *)sbase + (sbytes - xx_bytes) / 256 * 256);
+        HIP_TRY(launch_dup_rows(x, w->k5, n, xx, ctx->stream));
+        return noalloc_core(ctx, &lo, xx, n, y, sbase, (sbytes - xx_bytes) / 256 * 256);
+    }
     if (plain_type(w->dev.type))
-        return plain_mulmat(ctx, w, x, n, y, MI_QMM_DEVICE, MI_QMM_PATH_AUTO, ctx->static_scratch, (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES);
+        return plain_mulmat(ctx, w, x, n, y, MI_QMM_DEVICE, MI_QMM_PATH_AUTO, sbase, sbytes);
     const int64_t K = w->dev.K, M = w->dev.M;
     const int q8 = mi_qmm_vec_dot_type(w->dev.type);
     if (n <= 8 && !wants_skinny(w->dev.type, K, M, n, ctx->num_cus) && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
@@ -783,18 +829,23 @@ int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *
     }
     const bool f16 = wants_f16_planes(w->dev.type, n);
     const ActPlanes probe = plan_act(nullptr, q8, K, n, f16);
-    if (probe.total > (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES)
+    if (probe.total > sbytes)
         return fail(MI_QMM_ERR_UNSUPPORTED,
                     "n=%lld rows of k=%lld need %zu bytes of quantized activations; the static scratch of "
                     "mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)K, probe.total,
-                    (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES);
-    const ActPlanes p = plan_act(ctx->static_scratch, q8, K, n, f16);
+                    sbytes);
+    const ActPlanes p = plan_act(sbase, q8, K, n, f16);
     // every plane row below n is rewritten by the quantizer; rows n.. of the last 128-row tile keep what an
     // earlier call left there, and the GEMM drops the results of those rows
     HIP_TRY(launch_quantize_act(q8, x, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream, nullptr, p.qf, p.bsf));
     DevAct a;
     a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = K; a.N = (int)n; a.type = q8;
     return run_product(ctx, w, a, y, MI_QMM_PATH_AUTO, /*may_alloc=*/false);
+}
+
+int mi_qmm_mulmat_noalloc(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, int64_t n, float *y) {
+    if (!ctx) return fail(MI_QMM_ERR_INVALID, "ctx is NULL");
+    return noalloc_core(ctx, w, x, n, y, ctx->static_scratch, (size_t)MI_QMM_NOALLOC_SCRATCH_BYTES);
 }
 
 int mi_qmm_scratch_freeze(mi_qmm_ctx *ctx, int frozen) {
@@ -842,7 +893,8 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
     if (rc) return rc;
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
-        if (plain_type(ws[i]->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is an unquantized weight (type %d)", i, ws[i]->dev.type);
+        if (plain_type(ws[i]->dev.type) || ws[i]->q5k)
+            return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is of a type that only mi_qmm_mulmat multiplies (F32 / F16 / BF16 / Q5_K)", i);
     }
     Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
     if (prod) pr = *prod;
@@ -1013,14 +1065,15 @@ extern "C" {
 int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x, int64_t n,
                         float *const *ys, int location) {
     bool plain = false;
-    for (int i = 0; ws && ys && i < count; i++) plain = plain || (ws[i] && plain_type(ws[i]->dev.type));
+    for (int i = 0; ws && ys && i < count; i++) plain = plain || (ws[i] && (plain_type(ws[i]->dev.type) || ws[i]->q5k));
     if (plain) {
-        // unquantized weights have no joint kernels: one product after the other, each as mi_qmm_mulmat gives it
+        // unquantized and Q5_K weights have no joint kernels: one product after the other, each as mi_qmm_mulmat gives it
+        auto user_k = [](const mi_qmm_weight *w) { return w->q5k ? w->k5 : w->dev.K; };
         for (int i = 0; i < count; i++) {
             if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
-            if (ws[i]->dev.K != ws[0]->dev.K)
+            if (user_k(ws[i]) != user_k(ws[0]))
                 return fail(MI_QMM_ERR_INVALID, "ws[%d] has k=%lld, ws[0] has k=%lld: one x cannot serve both", i,
-                            (long long)ws[i]->dev.K, (long long)ws[0]->dev.K);
+                            (long long)user_k(ws[i]), (long long)user_k(ws[0]));
         }
         for (int i = 0; i < count; i++) {
             const int rc = mi_qmm_mulmat(ctx, ws[i], x, n, ys[i], location);
@@ -1051,7 +1104,7 @@ int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_
     int rc = check_product_args(ctx, w_gate, location, MI_QMM_PATH_AUTO);
     if (rc) return rc;
     if (w_up->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "w_up is on another device");
-    if (plain_type(w_up->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is an unquantized weight (type %d)", w_up->dev.type);
+    if (plain_type(w_up->dev.type) || w_up->q5k) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is of a type that only mi_qmm_mulmat multiplies");
     if (producer == MI_QMM_PRODUCE_RMSNORM && !(eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
     if (n == 0) return MI_QMM_OK;
     if (!x || !h) return fail(MI_QMM_ERR_INVALID, "x or h is NULL");
@@ -1142,6 +1195,7 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     if (prod) pr = *prod;
     if (pr.kind == PRODUCE_SWIGLU && !pr.aux && n_tokens > 0) return fail(MI_QMM_ERR_INVALID, "SwiGLU needs the up operand");
     if (pr.kind == PRODUCE_RMSNORM && !(pr.eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
+    if (w2 && w2->q5k) return fail(MI_QMM_ERR_UNSUPPORTED, "the second expert stack is of a type that only mi_qmm_mulmat multiplies");
     if (w2 && (w2->device != ctx->device || w2->dev.type != w->dev.type || w2->dev.K != w->dev.K || w2->dev.M != w->dev.M))
         return fail(MI_QMM_ERR_INVALID, "the two expert stacks differ in device, type or shape");
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
@@ -1305,7 +1359,7 @@ int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const 
     if (rc) return rc;
     if (w_up->device != ctx->device || w_up->dev.K != w_gate->dev.K || w_up->dev.M != w_gate->dev.M)
         return fail(MI_QMM_ERR_INVALID, "the gate and up stacks differ in device or shape");
-    if (plain_type(w_up->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is an unquantized weight (type %d)", w_up->dev.type);
+    if (plain_type(w_up->dev.type) || w_up->q5k) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is of a type that only mi_qmm_mulmat multiplies");
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
         return fail(MI_QMM_ERR_INVALID, "n_expert=%d n_used=%d b_cols=%d n_tokens=%lld: all must be positive", n_expert,
                     n_used, b_cols, (long long)n_tokens);
@@ -1540,7 +1594,8 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     DevWeight dw[8];
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
-        if (plain_type(ws[i]->dev.type)) return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is an unquantized weight (type %d)", i, ws[i]->dev.type);
+        if (plain_type(ws[i]->dev.type) || ws[i]->q5k)
+            return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is of a type that only mi_qmm_mulmat multiplies (F32 / F16 / BF16 / Q5_K)", i);
         dw[i] = ws[i]->dev;
     }
     float *dys[8];

@@ -4,6 +4,8 @@
 //   Q4_0  2 + 32/2             = 18   fp16 d; u8 qs[16]  (low nibbles = elements 0..15, high = 16..31; value q-8)
 //   Q8_0  2 + 32               = 34   fp16 d; i8 qs[32]
 //   Q4_K  2 + 2 + 12 + 256/2   = 144  fp16 d, dmin; u8 scales[12] (8 x 6-bit scale + 8 x 6-bit min); u8 qs[128]
+//   Q5_K  2 + 2 + 12 + 32 + 128 = 176 fp16 d, dmin; u8 scales[12]; u8 qh[32] (bit j of qh[l]: fifth bit of element l of
+//                                     sub-block j); u8 qs[128]
 //   Q6_K  256/2 + 256/4 + 16+2 = 210  u8 ql[128]; u8 qh[64]; i8 scales[16]; fp16 d   (value q-32)
 //   Q8_K  4 + 256 + 2*16       = 292  f32 d; i8 qs[256]; i16 bsums[16]
 #pragma once
@@ -12,11 +14,11 @@
 
 namespace miqmm {
 
-enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 30, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_Q8_K = 15 };
+enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 30, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_Q8_K = 15 };
 
 constexpr int QK = 32;    // elements per Q4_0 / Q8_0 block
 constexpr int QKK = 256;  // elements per K-quant super-block
-constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q6_K_BYTES = 210, Q8_K_BYTES = 292;
+constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q5_K_BYTES = 176, Q6_K_BYTES = 210, Q8_K_BYTES = 292;
 
 // Weight tensor as the kernels see it.  Device-private "plane" layout chosen so that every
 // wavefront load is a run of aligned 16-byte pieces:
@@ -25,6 +27,10 @@ constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q6_K_BYTES = 2
 //   Q8_0 : p0 = qs plane, 32 B per block, [M][K];                  d = fp16 plane [M][K/32]
 //   Q6_K : p0 = ql plane [M][K/2]; p1 = qh plane [M][K/4]; p2 = scales plane [M][K/16] (i8);
 //          d = fp16 plane [M][K/256]
+//   Q5_K : stored as a Q4_K tensor of rows twice as long (type = T_Q4_K, K = 2 K'): blocks 0 .. K'/256 - 1 of a row are
+//          the Q5_K blocks without their fifth bits, blocks K'/256 .. are the fifth bits alone -- same scales, no mins,
+//          nibble 8 where the bit is set, block scale 2 d -- so that against the activations repeated, [x | x], every
+//          Q4_K kernel computes sum sc (q4 + 16 h) y exactly (see relayout.hip)
 //   F32, F16, BF16 : p0 = the rows unchanged, [M][K] elements
 // Byte order inside each plane is the GGUF order; only the interleaving of fields is undone.
 struct DevWeight {

@@ -34,6 +34,11 @@ hipError_t launch_pack_act_gguf(int q8_type, const int8_t *qs, const float *d, c
 hipError_t launch_relayout(int type, const uint8_t *gguf, int64_t K, int64_t M, uint8_t *p0,
                            uint8_t *p1, uint8_t *p2, uint16_t *d, hipStream_t s);
 
+// Q5_K blocks [M][K/256][176] -> the Q4_K tensor of rows of 2 K that stands for them (formats.h): out [M][2 K/256][144]
+hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *out, hipStream_t s);
+// out [n][2 K] = [x row | x row] for x [n][K] (K a multiple of 4): the activations such a tensor is multiplied with
+hipError_t launch_dup_rows(const float *x, int64_t K, int64_t n, float *out, hipStream_t s);
+
 // kernels 2 and 4: streaming GEMV / skinny GEMM, ncols in 1..8.  y[n*ldy + m].
 // returns hipErrorInvalidValue if the shape is outside the kernel's limits (caller reports it).
 hipError_t launch_gemv(const DevWeight &w, const DevAct &a, int col0, int ncols, float *y,

@@ -4,6 +4,8 @@
 // unchanged).  18-, 34- and 210-byte blocks are only 2-byte aligned, so a wavefront cannot read them
 // with aligned 16-byte loads; splitting each block's fields into separate planes restores that.
 // Runs once per tensor at load; every field offset and size is even, so the copy moves 16-bit units.
+#include <algorithm>
+
 #include "internal.h"
 
 namespace miqmm {
@@ -33,7 +35,70 @@ __global__ void relayout_kernel(const uint16_t *__restrict__ src, int64_t nblock
     }
 }
 
+// Q5_K -> a Q4_K tensor of rows twice as long.  w = d sc (q4 + 16 h) - dmin m with h the fifth bit, so a row's dot
+// product is the Q4_K dot product of its low parts plus 16 d yd sum_j sc_j sum_l h_jl y_jl: the same shape of sum with
+// nibble 8 h, block scale 2 d (exact in fp16 unless |d| > 32752) and no mins.  Block b of a row goes to block b (d, dmin,
+// scales, nibbles as they are) and to block nsb + b (2 d, dmin = 0, the same scale bytes, nibble 8 for a set bit).
+// One thread per 16-bit unit of the 144-byte destination blocks of both halves.
+__global__ void relayout_q5k_kernel(const uint8_t *__restrict__ src, int64_t M, int nsb, uint8_t *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = M * nsb * 2 * (Q4_K_BYTES / 2);
+    if (i >= total) return;
+    const int u = (int)(i % (Q4_K_BYTES / 2));       // 16-bit unit inside the destination block
+    const int64_t db = i / (Q4_K_BYTES / 2);         // destination block: row * 2 nsb + (half * nsb + b)
+    const int64_t row = db / (2 * nsb);
+    const int within = (int)(db - row * 2 * nsb), half = within / nsb, b = within - half * nsb;
+    const uint8_t *blk = src + (row * nsb + b) * Q5_K_BYTES;
+    uint16_t v;
+    if (u < 8) {  // d, dmin, scales[12]
+        v = (uint16_t)(blk[2 * u] | (blk[2 * u + 1] << 8));
+        if (half == 1) {
+            if (u == 0) v = __builtin_bit_cast(uint16_t, (_Float16)((_Float16)2.0f * __builtin_bit_cast(_Float16, v)));
+            else if (u == 1) v = 0;
+        }
+    } else {      // nibble bytes 2 (u - 8), 2 (u - 8) + 1 of the 128
+        const int q0 = 2 * (u - 8);
+        if (half == 0) v = (uint16_t)(blk[48 + q0] | (blk[48 + q0 + 1] << 8));
+        else {
+            uint16_t r = 0;
+            for (int t = 0; t < 2; t++) {
+                const int q = q0 + t, c = q >> 5, l = q & 31;  // byte q holds elements l of sub-blocks 2c (low) and 2c + 1 (high)
+                const unsigned h = blk[16 + l];
+                const unsigned byte = (((h >> (2 * c)) & 1u) << 3) | (((h >> (2 * c + 1)) & 1u) << 7);
+                r |= (uint16_t)(byte << (8 * t));
+            }
+            v = r;
+        }
+    }
+    reinterpret_cast<uint16_t *>(out)[i] = v;
+}
+
+__global__ void dup_rows_kernel(const float4 *__restrict__ x, float4 *__restrict__ out, int64_t k4, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < k4 * n; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / k4, c = i - r * k4;
+        const float4 v = x[i];
+        out[r * 2 * k4 + c] = v;
+        out[r * 2 * k4 + k4 + c] = v;
+    }
+}
+
 }  // namespace
+
+hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *out, hipStream_t s) {
+    if (K * M == 0) return hipSuccess;
+    const int64_t n = M * (K / QKK) * 2 * (Q4_K_BYTES / 2);
+    if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
+    relayout_q5k_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QKK), out);
+    return hipGetLastError();
+}
+
+hipError_t launch_dup_rows(const float *x, int64_t K, int64_t n, float *out, hipStream_t s) {
+    if (K * n == 0) return hipSuccess;
+    if (K % 4) return hipErrorInvalidValue;
+    const int64_t work = K / 4 * n;
+    dup_rows_kernel<<<(unsigned)std::min<int64_t>((work + 255) / 256, 4096), 256, 0, s>>>((const float4 *)x, (float4 *)out, K / 4, n);
+    return hipGetLastError();
+}
 
 hipError_t launch_relayout(int type, const uint8_t *gguf, int64_t K, int64_t M, uint8_t *p0, uint8_t *p1,
                            uint8_t *p2, uint16_t *d, hipStream_t s) {

@@ -107,8 +107,8 @@ class Tensor:
         ids[i, t] with activation row i mod B of that token.  /root/reference/ml/backend.go:153"""
         if self._weight is None or len(self._shape) != 3:
             raise TypeError("MulmatID: the receiver must be a 3-D quantized expert stack obtained from Backend.Get")
-        if self._type in qmm.PLAIN_TYPES:
-            raise TypeError("MulmatID: expert stacks must be block-quantized (Q4_0, Q8_0, Q4_K, Q6_K)")
+        if self._type in qmm.SINGLE_ONLY_TYPES:
+            raise TypeError("MulmatID: expert stacks must be of type Q4_0, Q8_0, Q4_K or Q6_K")
         if t2._type != qmm.F32 or ids._type != I32:
             raise TypeError("MulmatID: activations must be f32 and ids int32")
         if t2.Dim(0) != self.Dim(0):
@@ -198,8 +198,8 @@ class Context:
                 needed.update(id(s) for s in srcs)
                 if t._prod[0] == qmm.PRODUCE_SWIGLU and t._prod[2] is None:
                     needed.add(id(t))  # the bare silu is always an f32 node
-            elif t._op[0]._type in qmm.PLAIN_TYPES:
-                needed.update(id(s) for s in srcs)  # unquantized weights have no fused producers: x must exist as f32
+            elif t._op[0]._type in qmm.SINGLE_ONLY_TYPES:
+                needed.update(id(s) for s in srcs)  # these weight types have no fused producers: x must exist as f32
             for s in srcs:
                 readers.setdefault(id(s), []).append(t)
         # gate.SILU(up) on two pending products of one x that nothing else reads, at one activation row: one call
@@ -212,7 +212,7 @@ class Context:
             gate, up = t._prod[1], t._prod[2]
             if not (gate in pending and up in pending and gate is not up and gate._op is not None and up._op is not None
                     and gate._ids is up._ids and gate._op[1] is up._op[1]
-                    and gate._op[0]._type not in qmm.PLAIN_TYPES and up._op[0]._type not in qmm.PLAIN_TYPES
+                    and gate._op[0]._type not in qmm.SINGLE_ONLY_TYPES and up._op[0]._type not in qmm.SINGLE_ONLY_TYPES
                     and gate._op[0].Shape() == up._op[0].Shape() and id(gate) not in tensors_ids(tensors)
                     and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]):
                 continue
@@ -280,10 +280,10 @@ class Context:
                 continue
             nodes = [u for u in pending if u._data is None and u._ids is None and u._op is not None and u._op[1] is x
                      and id(u) not in pair_of]
-            for u in [u for u in nodes if u._op[0]._type in qmm.PLAIN_TYPES]:
-                # F32 / F16 / BF16 weights: one product each, x converted to the weight's type inside the call
+            for u in [u for u in nodes if u._op[0]._type in qmm.SINGLE_ONLY_TYPES]:
+                # F32 / F16 / BF16 / Q5_K weights: one product each
                 u._data = c.mulmat(u._op[0]._weight, x.Floats().reshape(-1, x.Dim(0))).reshape(-1)
-            nodes = [u for u in nodes if u._op[0]._type not in qmm.PLAIN_TYPES]
+            nodes = [u for u in nodes if u._op[0]._type not in qmm.SINGLE_ONLY_TYPES]
             if not nodes:
                 continue
             if x._data is None and x._prod is not None:
@@ -332,7 +332,7 @@ class Backend:
     ``ml.NewBackend(modelPath, params)`` receives, /root/reference/ml/backend.go:83 -- or a dict mapping a
     tensor name to (ggml_type, shape [K, M], block bytes), what fs/ggml hands out for a tensor
     (/root/reference/fs/ggml/gguf.go:281-308).  From a file, Load uploads every 2-D tensor (and every 3-D
-    expert stack) of a type the Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q6_K; 2-D F32, F16 and BF16 too) straight
+    expert stack) of a type the Mulmat path multiplies (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K; 2-D F32, F16 and BF16 too) straight
     from the file mapping and keeps 1-D f32 tensors (norm weights, the operand of RMSNorm) on the host; tensors of
     other types are outside this path and are skipped."""
 
@@ -349,7 +349,7 @@ class Backend:
             with gguf.File(self._spec if isinstance(self._spec, str) else self._spec.decode()) as f:
                 infos = [t for t in f.TensorInfos()
                          if (len(t.Shape) in (2, 3) and qmm.vec_dot_type(t.Type) >= 0
-                             and not (len(t.Shape) == 3 and t.Type in qmm.PLAIN_TYPES))
+                             and not (len(t.Shape) == 3 and t.Type in qmm.SINGLE_ONLY_TYPES))
                          or (len(t.Shape) == 1 and t.Type == qmm.F32)]
                 for i, ti in enumerate(infos):
                     t = Tensor(ti.Shape, ti.Type)

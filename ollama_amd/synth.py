@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
 
 
 def _f16_bytes(v: np.ndarray) -> np.ndarray:
@@ -74,6 +74,41 @@ def encode_q4_K(x: np.ndarray) -> np.ndarray:
     return out.reshape(m, -1)
 
 
+def encode_q5_K(x: np.ndarray) -> np.ndarray:
+    """as encode_q4_K on a grid of 32 levels; the fifth bit of element l of sub-block j is bit j of qh[l]"""
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 256, 8, 32)
+    lo = np.minimum(b.min(axis=3), 0)
+    scale = (b.max(axis=3) - lo) / np.float32(31)
+    mins = -lo
+    d = (scale.max(axis=2) / np.float32(63)).astype(np.float16)
+    dmin = (mins.max(axis=2) / np.float32(63)).astype(np.float16)
+    df, dmf = d.astype(np.float32), dmin.astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(df[..., None] > 0, np.rint(scale / df[..., None]), 0).clip(0, 63).astype(np.uint8)
+        mn = np.where(dmf[..., None] > 0, np.rint(mins / dmf[..., None]), 0).clip(0, 63).astype(np.uint8)
+        eff = df[..., None] * sc
+        q = np.where(eff[..., None] > 0, np.rint((b + (dmf[..., None] * mn)[..., None]) / eff[..., None]), 0)
+    q = q.clip(0, 31).astype(np.uint8)
+    out = np.zeros((m, k // 256, 176), np.uint8)
+    out[..., 0:2] = _f16_bytes(d)
+    out[..., 2:4] = _f16_bytes(dmin)
+    s = out[..., 4:16]
+    for j in range(4):
+        s[..., j] = (sc[..., j] & 63) | ((sc[..., j + 4] >> 4) << 6)
+        s[..., j + 4] = (mn[..., j] & 63) | ((mn[..., j + 4] >> 4) << 6)
+        s[..., j + 8] = (sc[..., j + 4] & 15) | ((mn[..., j + 4] & 15) << 4)
+    hi = (q >> 4).astype(np.uint8)                                      # [m, nb, 8, 32]
+    qh = np.zeros((m, k // 256, 32), np.uint8)
+    for j in range(8):
+        qh |= hi[..., j, :] << j
+    out[..., 16:48] = qh
+    qq = (q & 15).reshape(m, k // 256, 4, 2, 32)
+    out[..., 48:] = (qq[..., 0, :] | (qq[..., 1, :] << 4)).reshape(m, k // 256, 128)
+    return out.reshape(m, -1)
+
+
 def encode_q6_K(x: np.ndarray) -> np.ndarray:
     x = np.ascontiguousarray(x, np.float32)
     m, k = x.shape
@@ -98,7 +133,7 @@ def encode_q6_K(x: np.ndarray) -> np.ndarray:
     return out.reshape(m, -1)
 
 
-ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q6_K: encode_q6_K}
+ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K}
 
 
 def weights(ggml_type: int, m: int, k: int, seed: int, std: float = 0.02, chunk_rows: int = 2048) -> np.ndarray:

@@ -20,6 +20,7 @@
 typedef struct { uint16_t d; uint8_t qs[QK / 2]; } blk_q4_0;                                /* 2+16      */
 typedef struct { uint16_t d; int8_t qs[QK]; } blk_q8_0;                                     /* 2+32      */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[QKK / 2]; } blk_q4_K; /* 2+2+12+128 */
+typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qh[QKK / 8]; uint8_t qs[QKK / 2]; } blk_q5_K; /* 2+2+12+32+128 */
 typedef struct { uint8_t ql[QKK / 2]; uint8_t qh[QKK / 4]; int8_t scales[QKK / 16]; uint16_t d; } blk_q6_K; /* 128+64+16+2 */
 typedef struct { float d; int8_t qs[QKK]; int16_t bsums[QKK / 16]; } blk_q8_K;              /* 4+256+32  */
 #pragma pack(pop)
@@ -27,6 +28,7 @@ typedef struct { float d; int8_t qs[QKK]; int16_t bsums[QKK / 16]; } blk_q8_K;  
 _Static_assert(sizeof(blk_q4_0) == 18, "Q4_0 block is 18 bytes");
 _Static_assert(sizeof(blk_q8_0) == 34, "Q8_0 block is 34 bytes");
 _Static_assert(sizeof(blk_q4_K) == 144, "Q4_K block is 144 bytes");
+_Static_assert(sizeof(blk_q5_K) == 176, "Q5_K block is 176 bytes");
 _Static_assert(sizeof(blk_q6_K) == 210, "Q6_K block is 210 bytes");
 _Static_assert(sizeof(blk_q8_K) == 292, "Q8_K block is 292 bytes");
 
@@ -34,7 +36,7 @@ int64_t ref_block_size(int type) {
     switch (type) {
     case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return 1;
     case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: return QK;
-    case REF_TYPE_Q4_K: case REF_TYPE_Q6_K: case REF_TYPE_Q8_K: return QKK;
+    case REF_TYPE_Q4_K: case REF_TYPE_Q5_K: case REF_TYPE_Q6_K: case REF_TYPE_Q8_K: return QKK;
     default: return 0;
     }
 }
@@ -46,6 +48,7 @@ int64_t ref_type_size(int type) {
     case REF_TYPE_Q4_0: return sizeof(blk_q4_0);
     case REF_TYPE_Q8_0: return sizeof(blk_q8_0);
     case REF_TYPE_Q4_K: return sizeof(blk_q4_K);
+    case REF_TYPE_Q5_K: return sizeof(blk_q5_K);
     case REF_TYPE_Q6_K: return sizeof(blk_q6_K);
     case REF_TYPE_Q8_K: return sizeof(blk_q8_K);
     default: return 0;
@@ -61,7 +64,7 @@ int64_t ref_row_size(int type, int64_t k) {
 int ref_vec_dot_type(int wtype) {
     switch (wtype) {
     case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: return REF_TYPE_Q8_0;
-    case REF_TYPE_Q4_K: case REF_TYPE_Q6_K: return REF_TYPE_Q8_K;
+    case REF_TYPE_Q4_K: case REF_TYPE_Q5_K: case REF_TYPE_Q6_K: return REF_TYPE_Q8_K;
     /* the unquantized weight types are multiplied in their own type: the activations are converted to it */
     case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return wtype;
     default: return -1;
@@ -510,6 +513,30 @@ static void dequant_q4_K(const blk_q4_K *x, float *y, int64_t k) {
     }
 }
 
+/* Q5_K: the Q4_K layout with a fifth bit per weight.  Bit j of qh[l] belongs to element l of sub-block j (the low
+ * nibbles of chunk c are sub-block 2c, the high nibbles sub-block 2c + 1); w = d * sc * (nibble + 16 * bit) - dmin * m. */
+static void dequant_q5_K(const blk_q5_K *x, float *y, int64_t k) {
+    for (int64_t i = 0; i < k / QKK; i++) {
+        const uint8_t *ql = x[i].qs, *qh = x[i].qh;
+        const float d = ref_fp16_to_fp32(x[i].d), min = ref_fp16_to_fp32(x[i].dmin);
+        int is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < QKK; j += 64) {
+            uint8_t sc, m;
+            ref_get_scale_min_k4(is + 0, x[i].scales, &sc, &m);
+            const float d1 = d * sc, m1 = min * m;
+            ref_get_scale_min_k4(is + 1, x[i].scales, &sc, &m);
+            const float d2 = d * sc, m2 = min * m;
+            for (int l = 0; l < 32; l++) *y++ = d1 * ((ql[l] & 0xF) + (qh[l] & u1 ? 16 : 0)) - m1;
+            for (int l = 0; l < 32; l++) *y++ = d2 * ((ql[l] >> 4) + (qh[l] & u2 ? 16 : 0)) - m2;
+            ql += 32;
+            is += 2;
+            u1 <<= 2;
+            u2 <<= 2;
+        }
+    }
+}
+
 static void dequant_q6_K(const blk_q6_K *x, float *y, int64_t k) {
     for (int64_t i = 0; i < k / QKK; i++) {
         const float d = ref_fp16_to_fp32(x[i].d);
@@ -546,6 +573,7 @@ int ref_dequantize_row(int type, const void *x, float *y, int64_t k) {
     case REF_TYPE_Q4_0: dequant_q4_0((const blk_q4_0 *)x, y, k); return 0;
     case REF_TYPE_Q8_0: dequant_q8_0((const blk_q8_0 *)x, y, k); return 0;
     case REF_TYPE_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
+    case REF_TYPE_Q5_K: dequant_q5_K((const blk_q5_K *)x, y, k); return 0;
     case REF_TYPE_Q6_K: dequant_q6_K((const blk_q6_K *)x, y, k); return 0;
     case REF_TYPE_Q8_K: dequant_q8_K((const blk_q8_K *)x, y, k); return 0;
     case REF_TYPE_F32: memcpy(y, x, (size_t)k * 4); return 0;
@@ -606,6 +634,56 @@ float ref_vec_dot_q4_K_q8_K(int64_t n, const void *vx, const void *vy) {
             a += 32;
             for (int l = 0; l < 32; l++) a[l] = (int8_t)(q4[l] >> 4);
             a += 32;
+            q4 += 32;
+        }
+        ref_unpack_scales_kmask(x[i].scales, scales, mins);
+        int sumi = 0;
+        for (int j = 0; j < QKK / 16; j++) sumi += y[i].bsums[j] * mins[j / 2];
+        a = aux8;
+        for (int j = 0; j < QKK / 32; j++) {
+            const int32_t scale = scales[j];
+            for (int rep = 0; rep < 4; rep++) {
+                for (int l = 0; l < 8; l++) aux16[l] = (int16_t)(q8[l] * a[l]);
+                for (int l = 0; l < 8; l++) aux32[l] += scale * aux16[l];
+                q8 += 8;
+                a += 8;
+            }
+        }
+        const float d = ref_fp16_to_fp32(x[i].d) * y[i].d;
+        for (int l = 0; l < 8; l++) sums[l] += d * aux32[l];
+        const float dmin = ref_fp16_to_fp32(x[i].dmin) * y[i].d;
+        sumf -= dmin * sumi;
+    }
+    for (int l = 0; l < 8; l++) sumf += sums[l];
+    return sumf;
+}
+
+/* ggml_vec_dot_q5_K_q8_K, generic path: the 5-bit values in element order, then as for Q4_K */
+float ref_vec_dot_q5_K_q8_K(int64_t n, const void *vx, const void *vy) {
+    const blk_q5_K *x = (const blk_q5_K *)vx;
+    const blk_q8_K *y = (const blk_q8_K *)vy;
+    int8_t aux8[QKK];
+    int16_t aux16[8];
+    int32_t aux32[8];
+    float sums[8];
+    uint8_t scales[8], mins[8];
+    memset(sums, 0, sizeof(sums));
+    float sumf = 0;
+    for (int64_t i = 0; i < n / QKK; i++) {
+        const uint8_t *q4 = x[i].qs, *hm = x[i].qh;
+        const int8_t *q8 = y[i].qs;
+        memset(aux32, 0, sizeof(aux32));
+        int8_t *a = aux8;
+        uint8_t m = 1;
+        for (int j = 0; j < QKK / 64; j++) {
+            for (int l = 0; l < 32; l++) a[l] = (int8_t)(q4[l] & 0xF);
+            for (int l = 0; l < 32; l++) a[l] += (hm[l] & m ? 16 : 0);
+            a += 32;
+            m <<= 1;
+            for (int l = 0; l < 32; l++) a[l] = (int8_t)(q4[l] >> 4);
+            for (int l = 0; l < 32; l++) a[l] += (hm[l] & m ? 16 : 0);
+            a += 32;
+            m <<= 1;
             q4 += 32;
         }
         ref_unpack_scales_kmask(x[i].scales, scales, mins);
@@ -745,6 +823,7 @@ static dot_fn dot_for(int wtype) {
     case REF_TYPE_Q4_0: return ref_vec_dot_q4_0_q8_0;
     case REF_TYPE_Q8_0: return ref_vec_dot_q8_0_q8_0;
     case REF_TYPE_Q4_K: return ref_vec_dot_q4_K_q8_K;
+    case REF_TYPE_Q5_K: return ref_vec_dot_q5_K_q8_K;
     case REF_TYPE_Q6_K: return ref_vec_dot_q6_K_q8_K;
     case REF_TYPE_F32: return ref_vec_dot_f32;
     case REF_TYPE_F16: return ref_vec_dot_f16;

@@ -2,7 +2,7 @@
  * CPU oracle for the GGUF block-quantized matmul path  --  TEST INFRASTRUCTURE ONLY.
  *
  * A scalar C restatement of the ggml CPU backend's semantics for
- *   mul_mat(W quantized {Q4_0,Q8_0,Q4_K,Q6_K} or plain {F32,F16,BF16}, X f32) -> Y f32
+ *   mul_mat(W quantized {Q4_0,Q8_0,Q4_K,Q5_K,Q6_K} or plain {F32,F16,BF16}, X f32) -> Y f32
  * i.e. activation quantization to Q8_0 / Q8_K followed by the per-type integer dot products.
  * Nothing in the shipped library links or calls this file: it is the checker the GPU path is
  * compared against, and the timed "port" CPU baseline.
@@ -17,7 +17,7 @@
  *   call shape            /root/reference/ml/backend.go:151 (Tensor.Mulmat)
  *
  * Parity status per function (what pins it is in tests/test_oracle_*.py):
- *   fp16<->fp32, q8_0/q8_K quantizers, 6-bit scale unpack, four vec_dots, dequantizers,
+ *   fp16<->fp32, q8_0/q8_K quantizers, 6-bit scale unpack, five vec_dots (Q5_K among them), dequantizers,
  *   mul_mat driver:  pinned (numpy float16, closed forms, fp64 brute force, KATs).
  *   F32 / F16 / BF16 weights (activations converted to the weight's type, products in fp32, sum in double):
  *   pinned as mathematics (numpy float16 casts, bfloat16 rounding against an integer statement of
@@ -49,7 +49,7 @@ extern "C" {
 #endif
 
 /* ggml_type ids, /root/reference/fs/ggml/type.go:250-268 */
-enum { REF_TYPE_F32 = 0, REF_TYPE_F16 = 1, REF_TYPE_BF16 = 30, REF_TYPE_Q4_0 = 2, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12,
+enum { REF_TYPE_F32 = 0, REF_TYPE_F16 = 1, REF_TYPE_BF16 = 30, REF_TYPE_Q4_0 = 2, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12, REF_TYPE_Q5_K = 13,
        REF_TYPE_Q6_K = 14, REF_TYPE_Q8_K = 15 };
 
 int64_t ref_block_size(int type);               /* elements per block, 0 if unknown */
@@ -91,6 +91,7 @@ void ref_unpack_scales_kmask(const uint8_t *s12, uint8_t sc[8], uint8_t m[8]);
 float ref_vec_dot_q4_0_q8_0(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q8_0_q8_0(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q4_K_q8_K(int64_t n, const void *x, const void *y);
+float ref_vec_dot_q5_K_q8_K(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q6_K_q8_K(int64_t n, const void *x, const void *y);
 /* the unquantized types: both rows in the weight's type, products in fp32, sum in double in element order */
 float ref_vec_dot_f32(int64_t n, const void *x, const void *y);

@@ -9,9 +9,9 @@ from __future__ import annotations
 
 import numpy as np
 
-F32, Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 0, 2, 8, 12, 14, 15
-BLOCK = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256}
-BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, Q8_K: 292}
+F32, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K = 0, 2, 8, 12, 13, 14, 15
+BLOCK = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
+BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
 
 
 def _blocks(raw: np.ndarray, t: int) -> np.ndarray:
@@ -60,6 +60,19 @@ def q4_K_ints(raw):
     return d, dmin, sc, m, q
 
 
+def q5_K_ints(raw):
+    """d, dmin, 6-bit scales and mins as for Q4_K; the 5-bit values: nibble + 16 * (bit j of qh[l]) for element l of
+    sub-block j -- a bit-field statement written from the block layout, not from the C loops"""
+    b = _blocks(raw, Q5_K)
+    d, dmin = _f16(b[:, 0:2]), _f16(b[:, 2:4])
+    sc, m = q4k_scales_mins(b[:, 4:16])
+    qh = b[:, 16:48].astype(np.int64)                                   # [nb, 32]
+    qs = b[:, 48:176].astype(np.int64).reshape(-1, 4, 32)
+    q = np.stack([qs & 15, qs >> 4], axis=2).reshape(-1, 8, 32)
+    bits = (qh[:, None, :] >> np.arange(8)[None, :, None]) & 1           # [nb, 8 sub-blocks, 32]
+    return d, dmin, sc, m, q + 16 * bits
+
+
 def q6_K_ints(raw):
     b = _blocks(raw, Q6_K)
     ql = b[:, 0:128].astype(np.int64).reshape(-1, 2, 64)
@@ -92,6 +105,10 @@ def dequant(t: int, raw) -> np.ndarray:
         return (d[:, None] * q).reshape(-1)
     if t == Q4_K:
         d, dmin, sc, m, q = q4_K_ints(raw)
+        w = (d[:, None] * sc)[:, :, None] * q - (dmin[:, None] * m)[:, :, None]
+        return w.reshape(-1)
+    if t == Q5_K:
+        d, dmin, sc, m, q = q5_K_ints(raw)
         w = (d[:, None] * sc)[:, :, None] * q - (dmin[:, None] * m)[:, :, None]
         return w.reshape(-1)
     if t == Q6_K:

@@ -39,7 +39,8 @@ def test_vec_dot_type():
     assert qmm.vec_dot_type(qmm.Q4_K) == qmm.Q8_K and qmm.vec_dot_type(qmm.Q6_K) == qmm.Q8_K
     # the unquantized weight types are multiplied in their own type
     assert [qmm.vec_dot_type(t) for t in (qmm.F32, qmm.F16, qmm.BF16)] == [qmm.F32, qmm.F16, qmm.BF16]
-    assert qmm.vec_dot_type(13) == -1 and qmm.vec_dot_type(qmm.Q8_K) == -1
+    assert qmm.vec_dot_type(qmm.Q5_K) == qmm.Q8_K
+    assert qmm.vec_dot_type(10) == -1 and qmm.vec_dot_type(qmm.Q8_K) == -1
 
 
 def test_argument_errors_without_a_device():
@@ -52,7 +53,7 @@ def test_argument_errors_without_a_device():
     assert L.mi_qmm_mulmat_q8_multi(None, None, 1, None, None, 0) == qmm.ERR_INVALID and "ctx is NULL" in qmm.last_error()
     assert L.mi_qmm_mulmat_noalloc(None, None, None, 1, None) == qmm.ERR_INVALID
     assert L.mi_qmm_scratch_freeze(None, 1) == qmm.ERR_INVALID
-    assert L.mi_qmm_weight_upload(None, 13, None, 256, 1, 0, ctypes.byref(h)) == qmm.ERR_UNSUPPORTED
+    assert L.mi_qmm_weight_upload(None, 10, None, 256, 1, 0, ctypes.byref(h)) == qmm.ERR_UNSUPPORTED
     assert L.mi_qmm_weight_upload(None, qmm.Q4_K, None, 100, 1, 0, ctypes.byref(h)) == qmm.ERR_INVALID
     assert "multiple of the block size" in qmm.last_error()
     assert L.mi_qmm_weight_upload(None, qmm.Q4_K, None, 256, 0, 0, ctypes.byref(h)) == qmm.ERR_INVALID

@@ -217,7 +217,7 @@ def test_config4_q6_K_output_head(ctx):
 # ---- error behaviour -------------------------------------------------------------------------------------
 def test_upload_and_mulmat_errors(ctx):
     with pytest.raises(qmm.QmmError) as e:
-        ctx.upload(13, np.zeros(176, np.uint8), 256, 1)      # Q5_K is not on this path
+        ctx.upload(10, np.zeros(84, np.uint8), 256, 1)       # Q2_K is not on this path
     assert e.value.code == qmm.ERR_UNSUPPORTED
     with pytest.raises(qmm.QmmError) as e:
         ctx.upload(Q4_0, np.zeros(18, np.uint8), 31, 1)      # row not a multiple of the block

@@ -192,16 +192,18 @@ def test_plain_weights_in_joint_calls_and_where_they_are_refused(ctx):
 
 
 def test_python_mirror_multiplies_unquantized_weights_beside_quantized_ones():
-    """one graph: an RMSNorm read by a Q4_K weight (folded into its launch) and by F16 / F32 weights (which need it in
-    f32), at decode and prefill size"""
+    """one graph: an RMSNorm read by a Q4_K weight (folded into its launch) and by F16 / F32 / Q5_K weights (which need
+    it in f32), at decode and prefill size"""
     from ollama_amd import ml, synth
     k = 1024
     rng = np.random.default_rng(21)
     raw_q = synth.weights(qmm.Q4_K, 64, k, seed=5)
     raw_h = oracle.quantize(F16, (rng.standard_normal((48, k)) * 0.05).astype(np.float32))
     raw_f = oracle.quantize(F32, (rng.standard_normal((10, k)) * 0.05).astype(np.float32))
+    raw_5 = synth.weights(qmm.Q5_K, 33, k, seed=6)
     g = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
     b = ml.Backend({"q.weight": (qmm.Q4_K, [k, 64], raw_q), "h.weight": (F16, [k, 48], raw_h), "r.weight": (F32, [k, 10], raw_f),
+                    "v.weight": (qmm.Q5_K, [k, 33], raw_5),
                     "norm.weight": (F32, [k], g)})
     b.Load()
     try:
@@ -209,10 +211,11 @@ def test_python_mirror_multiplies_unquantized_weights_beside_quantized_ones():
             xs = rng.standard_normal((n, k)).astype(np.float32)
             ctx = b.NewContext()
             xn = ctx.FromFloats(xs.reshape(-1), k, n).RMSNorm(ctx, b.Get("norm.weight"), 1e-5)
-            outs = {name: b.Get(name).Mulmat(ctx, xn) for name in ("q.weight", "h.weight", "r.weight")}
+            outs = {name: b.Get(name).Mulmat(ctx, xn) for name in ("q.weight", "h.weight", "r.weight", "v.weight")}
             ctx.Compute(*outs.values())
             want_x = oracle.rms_norm(xs, g, 1e-5)
-            for name, t, raw, m in (("q.weight", qmm.Q4_K, raw_q, 64), ("h.weight", F16, raw_h, 48), ("r.weight", F32, raw_f, 10)):
+            for name, t, raw, m in (("q.weight", qmm.Q4_K, raw_q, 64), ("h.weight", F16, raw_h, 48), ("r.weight", F32, raw_f, 10),
+                                    ("v.weight", qmm.Q5_K, raw_5, 33)):
                 want = oracle.mul_mat(t, raw, k, m, want_x)
                 assert npref.rel_err(outs[name].Floats().reshape(n, m), want) <= 1e-3, (name, n)
             ctx.Close()
