@@ -479,6 +479,21 @@ def main() -> int:
             fn()
             tm = timed(fn, 10) / (10 * len(stacks))
             other[f"MulmatID Q4_K 128x(768x2048) top-8 tokens={toks}"] = {"us": round(tm * 1e6, 2)}
+        # the same on MXFP4 expert stacks (kept as Q8_0 planes): 32 experts of 2880 x 2880, 4 used per token
+        mx_exp, mx_used, mm, mk = 32, 4, 2880, 2880
+        raw_mx = np.tile(synth.weights(qmm.MXFP4, 2880, mk, seed=1203), (mx_exp, 1))
+        mx_stacks = [ctx.upload(qmm.MXFP4, np.roll(raw_mx, 13 * c, axis=0), mk, mx_exp * mm) for c in range(4)]
+        for toks in (1, 8, 512):
+            xm = torch.randn(toks, 1, mk, generator=g, dtype=torch.float32).to(dev)
+            idm = torch.stack([torch.randperm(mx_exp, generator=g)[:mx_used] for _ in range(toks)]).to(torch.int32).to(dev)
+            ym = torch.empty(toks, mx_used, mm, dtype=torch.float32, device=dev)
+            fn = lambda: [ctx.mulmat_id_device(st, mx_exp, xm.data_ptr(), 1, idm.data_ptr(), mx_used, toks, ym.data_ptr())
+                          for st in mx_stacks]
+            fn()
+            tm = timed(fn, 10) / (10 * len(mx_stacks))
+            other[f"MulmatID MXFP4 32x(2880x2880) top-4 tokens={toks}"] = {"us": round(tm * 1e6, 2)}
+        for st in mx_stacks:
+            st.free()
         # one token through a mixture-of-experts feed-forward block: gate and up experts with their gating in
         # one launch, the down experts (one activation row per used expert) in a second
         raw_d = np.tile(synth.weights(Q4_K, 2048, em, seed=1202), (n_exp * ek // 2048, 1))

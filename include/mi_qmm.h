@@ -52,7 +52,8 @@ enum {
     MI_QMM_TYPE_Q5_K = 13,
     MI_QMM_TYPE_Q6_K = 14,
     MI_QMM_TYPE_Q8_K = 15,
-    MI_QMM_TYPE_BF16 = 30
+    MI_QMM_TYPE_BF16 = 30,
+    MI_QMM_TYPE_MXFP4 = 39
 };
 
 /* where x / y / weight bytes live */
@@ -148,7 +149,12 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      after the other there); the produced, expert-indexed and pre-quantized entry points take Q4_0 / Q8_0 /
  *      Q4_K / Q6_K weights only and return MI_QMM_ERR_UNSUPPORTED otherwise.  A Q5_K tensor is kept as the Q4_K
  *      tensor of rows twice as long that gives the same integer sums against [x | x] (1.64 times the bytes of
- *      the file: its products cost what a Q4_K product of twice the K costs).
+ *      the file: its products cost what a Q4_K product of twice the K costs).  39 (MXFP4, the expert tensors of
+ *      /root/reference/convert/convert_gptoss.go:124-150; DTypeMXFP4, /root/reference/ml/backend.go:404-412) is kept
+ *      as the Q8_0 planes that give the same dot products -- the doubled E2M1 values as int8, the scale 2^(e - 128)
+ *      as the block scale -- and goes through EVERY entry point a Q8_0 weight goes through, the expert-indexed ones
+ *      included (twice the bytes of the file).  A scale byte above 146 is MI_QMM_ERR_UNSUPPORTED; blocks with a
+ *      scale byte below 104 (weights under 7.2e-7) are kept as zeros.
  *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
 int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
                          int64_t m, int src_location, mi_qmm_weight **out);

@@ -70,6 +70,7 @@ struct mi_qmm_weight {
     // a Q5_K tensor: dev is the Q4_K tensor of rows of 2 k5 that stands for it (formats.h), multiplied with [x | x]
     bool q5k = false;
     int64_t k5 = 0;
+    int file_type = -1;  // the ggml type the tensor had in the file, where dev.type is another (Q5_K, MXFP4); -1: dev.type
 };
 
 struct mi_qmm_gguf {
@@ -211,7 +212,7 @@ int64_t mi_qmm_row_size(int t, int64_t k) {
 
 int mi_qmm_vec_dot_type(int wt) {
     switch (wt) {
-    case T_Q4_0: case T_Q8_0: return T_Q8_0;
+    case T_Q4_0: case T_Q8_0: case T_MXFP4: return T_Q8_0;
     case T_Q4_K: case T_Q5_K: case T_Q6_K: return T_Q8_K;
     case T_F32: case T_F16: case T_BF16: return wt;  // multiplied in their own type: x is converted to it
     default: return -1;
@@ -315,13 +316,13 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (mi_qmm_vec_dot_type(type) < 0)
-        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 8, 12, 13, 14, 30)", type);
+        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 8, 12, 13, 14, 30, 39)", type);
     if (k <= 0 || m <= 0) return fail(MI_QMM_ERR_INVALID, "k=%lld m=%lld must be positive", (long long)k, (long long)m);
     const int64_t row = mi_qmm_row_size(type, k);
     if (row < 0)
         return fail(MI_QMM_ERR_INVALID, "k=%lld is not a multiple of the block size %lld of type %d",
                     (long long)k, (long long)mi_qmm_block_size(type), type);
-    if (type == T_Q4_0 || type == T_Q8_0) {
+    if (type == T_Q4_0 || type == T_Q8_0 || type == T_MXFP4) {
         // the activation quantizer pairs these with Q8_0 planes read as 16-byte pieces
         if (k % QK != 0) return fail(MI_QMM_ERR_INVALID, "k not a multiple of 32");
     }
@@ -338,7 +339,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     case T_Q4_K: case T_F32: case T_F16: case T_BF16: s0 = total; break;
     case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; break;  // a Q4_K tensor of rows twice as long
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
-    case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
+    case T_Q8_0: case T_MXFP4: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;  // (MXFP4: kept as Q8_0 planes)
     case T_Q6_K: s0 = (size_t)(m * (k / 2)); s1 = (size_t)(m * (k / 4)); s2 = (size_t)(m * (k / 16));
                  sd = (size_t)(m * (k / QKK)) * 2; break;
     }
@@ -360,7 +361,8 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     w->dev.p2 = s2 ? b + o2 : nullptr;
     w->dev.d = sd ? (const uint16_t *)(b + od) : nullptr;
     w->dev.K = k; w->dev.M = m; w->dev.type = type;
-    if (type == T_Q5_K) { w->q5k = true; w->k5 = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; }
+    if (type == T_Q5_K) { w->q5k = true; w->k5 = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K; }
+    if (type == T_MXFP4) { w->dev.type = T_Q8_0; w->file_type = T_MXFP4; }
 
     void *staging = nullptr;
     const uint8_t *src = (const uint8_t *)bytes;
@@ -382,9 +384,28 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
             if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(staging)", e);
             src = (const uint8_t *)staging;
         }
+        int *bad = nullptr;
+        if (type == T_MXFP4) {  // the tail slack of the allocation holds the flag of scales the planes cannot hold
+            bad = (int *)(b + dev_bytes - 256);
+            e = hipMemsetAsync(bad, 0, sizeof(int), ctx->stream);
+            if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemset(flag)", e);
+        }
         e = type == T_Q5_K ? launch_relayout_q5k(src, k, m, b + o0, ctx->stream)
-                           : launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
+            : type == T_MXFP4 ? launch_relayout_mxfp4(src, k, m, b + o0, (uint16_t *)(b + od), bad, ctx->stream)
+                              : launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
         if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
+        if (bad) {
+            int flag = 0;
+            e = hipMemcpyAsync(&flag, bad, sizeof(int), hipMemcpyDeviceToHost, ctx->stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+            if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(flag)", e);
+            if (flag) {
+                if (staging) (void)hipFree(staging);
+                (void)hipFree(w->base);
+                delete w;
+                return fail(MI_QMM_ERR_UNSUPPORTED, "an MXFP4 block has a scale byte above 146 (weights of 2^18 and more): beyond the fp16 block scales it is kept with");
+            }
+        }
     }
     e = hipStreamSynchronize(ctx->stream);  // the caller's bytes must not be needed after return
     if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipStreamSynchronize(upload)", e);
@@ -404,7 +425,7 @@ void mi_qmm_weight_free(mi_qmm_weight *w) {
 
 int mi_qmm_weight_info(const mi_qmm_weight *w, int *type, int64_t *k, int64_t *m, int64_t *device_bytes) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
-    if (type) *type = w->q5k ? T_Q5_K : w->dev.type;
+    if (type) *type = w->file_type >= 0 ? w->file_type : w->dev.type;
     if (k) *k = w->q5k ? w->k5 : w->dev.K;
     if (m) *m = w->dev.M;
     if (device_bytes) *device_bytes = (int64_t)w->bytes;

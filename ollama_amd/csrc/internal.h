@@ -36,6 +36,9 @@ hipError_t launch_relayout(int type, const uint8_t *gguf, int64_t K, int64_t M, 
 
 // Q5_K blocks [M][K/256][176] -> the Q4_K tensor of rows of 2 K that stands for them (formats.h): out [M][2 K/256][144]
 hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *out, hipStream_t s);
+// MXFP4 blocks [M][K/32][17] -> Q8_0 planes (qs [M][K], d [M][K/32]) with the same dot products; *bad (device int, zeroed
+// by the caller) is set when a block's scale is beyond what the planes can hold (e > 146: weights of 2^18 and more)
+hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s);
 // out [n][2 K] = [x row | x row] for x [n][K] (K a multiple of 4): the activations such a tensor is multiplied with
 hipError_t launch_dup_rows(const float *x, int64_t K, int64_t n, float *out, hipStream_t s);
 

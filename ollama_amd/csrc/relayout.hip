@@ -73,6 +73,39 @@ __global__ void relayout_q5k_kernel(const uint8_t *__restrict__ src, int64_t M, 
     reinterpret_cast<uint16_t *>(out)[i] = v;
 }
 
+// MXFP4 -> Q8_0 planes.  An MXFP4 block (/root/reference/convert/convert_gptoss.go:216-238: an E8M0 scale byte, then 16
+// bytes whose low nibbles are elements 0..15 and whose high nibbles are elements 16..31) is 32 small integers -- the E2M1
+// values doubled: 0 1 2 3 4 6 8 12 and their negatives -- under the scale 2^(e - 128), and ggml multiplies it with Q8_0
+// activations as sum_i q_i y_i * (scale * d_y): the Q8_0 dot product of a block with those integers and that scale.  The
+// scale is a half for e in 104 .. 143; up to e = 146 the integers are shifted left instead (12 * 8 = 96 fits); below 104
+// (weights under 7.2e-7) the block is zero; above 146 *bad is set.  One thread per nibble byte.
+__global__ void relayout_mxfp4_kernel(const uint8_t *__restrict__ src, int64_t nblocks, int8_t *__restrict__ qs, uint16_t *__restrict__ d,
+                                      int *__restrict__ bad) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nblocks * 16) return;
+    const int64_t blk = i >> 4;
+    const int j = (int)(i & 15);
+    const uint8_t *b = src + blk * 17;
+    const int e = b[0];
+    int shift = 0, he = e - 128 + 15;  // biased fp16 exponent of 2^(e - 128)
+    if (e > 143) { shift = e - 143; he = 30; }
+    if (e > 146) { shift = 0; he = 0; if (j == 0) atomicOr(bad, 1); }
+    const bool zero = e < 104 || e > 146;
+    const int lo = b[1 + j] & 15, hi = b[1 + j] >> 4;
+    const int mag_lo = (lo & 7) < 5 ? (lo & 7) : (lo & 7) == 5 ? 6 : (lo & 7) == 6 ? 8 : 12;
+    const int mag_hi = (hi & 7) < 5 ? (hi & 7) : (hi & 7) == 5 ? 6 : (hi & 7) == 6 ? 8 : 12;
+    qs[blk * 32 + j] = zero ? 0 : (int8_t)(((lo & 8) ? -mag_lo : mag_lo) << shift);
+    qs[blk * 32 + j + 16] = zero ? 0 : (int8_t)(((hi & 8) ? -mag_hi : mag_hi) << shift);
+    if (j == 0) {
+        // 2^(e - 128) as a half: normal from 2^-14 (e = 114), subnormal 2^-24 .. 2^-15 below
+        uint16_t h;
+        if (zero) h = 0;
+        else if (he >= 1) h = (uint16_t)(he << 10);
+        else h = (uint16_t)(1u << (e - 104));
+        d[blk] = h;
+    }
+}
+
 __global__ void dup_rows_kernel(const float4 *__restrict__ x, float4 *__restrict__ out, int64_t k4, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < k4 * n; i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t r = i / k4, c = i - r * k4;
@@ -89,6 +122,14 @@ hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_
     const int64_t n = M * (K / QKK) * 2 * (Q4_K_BYTES / 2);
     if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
     relayout_q5k_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QKK), out);
+    return hipGetLastError();
+}
+
+hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s) {
+    if (K * M == 0) return hipSuccess;
+    const int64_t n = M * (K / QK) * 16;
+    if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
+    relayout_mxfp4_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M * (K / QK), (int8_t *)qs, d, bad);
     return hipGetLastError();
 }
 

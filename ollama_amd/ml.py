@@ -39,7 +39,7 @@ class DType(enum.IntEnum):  # /root/reference/ml/backend.go:404-412
 
 
 I32 = 26  # ggml_type id of int32, /root/reference/fs/ggml/type.go:252-279
-_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.F16: DType.F16, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40, I32: DType.I32}
+_GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.F16: DType.F16, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40, qmm.MXFP4: DType.MXFP4, I32: DType.I32}
 
 
 class Tensor:

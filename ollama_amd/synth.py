@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 2, 8, 12, 13, 14, 39
 
 
 def _f16_bytes(v: np.ndarray) -> np.ndarray:
@@ -42,6 +42,26 @@ def encode_q4_0(x: np.ndarray) -> np.ndarray:
     out = np.empty((m, k // 32, 18), np.uint8)
     out[..., 0:2] = _f16_bytes(d)
     out[..., 2:] = q[..., :16] | (q[..., 16:] << 4)
+    return out.reshape(m, -1)
+
+
+def encode_mxfp4(x: np.ndarray) -> np.ndarray:
+    """blocks of 32: the power-of-two scale that brings the largest magnitude to at most 6 (the largest E2M1 value),
+    every element to the nearest E2M1 value; 17 bytes: the E8M0 scale byte, then low nibbles = elements 0..15, high
+    nibbles = elements 16..31"""
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 32, 32).astype(np.float64)
+    amax = np.abs(b).max(axis=2)
+    with np.errstate(divide="ignore"):
+        e = np.where(amax > 0, np.ceil(np.log2(np.maximum(amax, 1e-300) / 6.0)), -127).clip(-127, 127).astype(np.int64)
+    grid = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6])
+    v = np.abs(b) / (2.0 ** e)[..., None]
+    code = np.abs(v[..., None] - grid).argmin(axis=-1).astype(np.uint8)
+    code |= (b < 0).astype(np.uint8) << 3
+    out = np.empty((m, k // 32, 17), np.uint8)
+    out[..., 0] = (e + 127).astype(np.uint8)
+    out[..., 1:] = code[..., :16] | (code[..., 16:] << 4)
     return out.reshape(m, -1)
 
 
@@ -133,7 +153,7 @@ def encode_q6_K(x: np.ndarray) -> np.ndarray:
     return out.reshape(m, -1)
 
 
-ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K}
+ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K, MXFP4: encode_mxfp4}
 
 
 def weights(ggml_type: int, m: int, k: int, seed: int, std: float = 0.02, chunk_rows: int = 2048) -> np.ndarray:

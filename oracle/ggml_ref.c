@@ -19,6 +19,7 @@
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[QK / 2]; } blk_q4_0;                                /* 2+16      */
 typedef struct { uint16_t d; int8_t qs[QK]; } blk_q8_0;                                     /* 2+32      */
+typedef struct { uint8_t e; uint8_t qs[QK / 2]; } blk_mxfp4;                                /* 1+16      */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[QKK / 2]; } blk_q4_K; /* 2+2+12+128 */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qh[QKK / 8]; uint8_t qs[QKK / 2]; } blk_q5_K; /* 2+2+12+32+128 */
 typedef struct { uint8_t ql[QKK / 2]; uint8_t qh[QKK / 4]; int8_t scales[QKK / 16]; uint16_t d; } blk_q6_K; /* 128+64+16+2 */
@@ -27,6 +28,7 @@ typedef struct { float d; int8_t qs[QKK]; int16_t bsums[QKK / 16]; } blk_q8_K;  
 
 _Static_assert(sizeof(blk_q4_0) == 18, "Q4_0 block is 18 bytes");
 _Static_assert(sizeof(blk_q8_0) == 34, "Q8_0 block is 34 bytes");
+_Static_assert(sizeof(blk_mxfp4) == 17, "MXFP4 block is 17 bytes");
 _Static_assert(sizeof(blk_q4_K) == 144, "Q4_K block is 144 bytes");
 _Static_assert(sizeof(blk_q5_K) == 176, "Q5_K block is 176 bytes");
 _Static_assert(sizeof(blk_q6_K) == 210, "Q6_K block is 210 bytes");
@@ -35,7 +37,7 @@ _Static_assert(sizeof(blk_q8_K) == 292, "Q8_K block is 292 bytes");
 int64_t ref_block_size(int type) {
     switch (type) {
     case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return 1;
-    case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: return QK;
+    case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: case REF_TYPE_MXFP4: return QK;
     case REF_TYPE_Q4_K: case REF_TYPE_Q5_K: case REF_TYPE_Q6_K: case REF_TYPE_Q8_K: return QKK;
     default: return 0;
     }
@@ -47,6 +49,7 @@ int64_t ref_type_size(int type) {
     case REF_TYPE_F16: case REF_TYPE_BF16: return 2;
     case REF_TYPE_Q4_0: return sizeof(blk_q4_0);
     case REF_TYPE_Q8_0: return sizeof(blk_q8_0);
+    case REF_TYPE_MXFP4: return sizeof(blk_mxfp4);
     case REF_TYPE_Q4_K: return sizeof(blk_q4_K);
     case REF_TYPE_Q5_K: return sizeof(blk_q5_K);
     case REF_TYPE_Q6_K: return sizeof(blk_q6_K);
@@ -63,7 +66,7 @@ int64_t ref_row_size(int type, int64_t k) {
 
 int ref_vec_dot_type(int wtype) {
     switch (wtype) {
-    case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: return REF_TYPE_Q8_0;
+    case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: case REF_TYPE_MXFP4: return REF_TYPE_Q8_0;
     case REF_TYPE_Q4_K: case REF_TYPE_Q5_K: case REF_TYPE_Q6_K: return REF_TYPE_Q8_K;
     /* the unquantized weight types are multiplied in their own type: the activations are converted to it */
     case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return wtype;
@@ -513,6 +516,29 @@ static void dequant_q4_K(const blk_q4_K *x, float *y, int64_t k) {
     }
 }
 
+/* MXFP4 (OCP microscaling: 32 four-bit floats E2M1 under one power-of-two scale E8M0; the block layout is the one
+ * /root/reference/convert/convert_gptoss.go:216-238 writes: the scale byte, then 16 bytes whose low nibbles are elements
+ * 0..15 and whose high nibbles are elements 16..31).  ggml keeps the E2M1 values doubled as integers and halves the
+ * scale instead: element = kvalue[nibble] * 2^(e - 128). */
+static const int8_t mxfp4_kvalues[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+
+float ref_e8m0_to_fp32_half(uint8_t e) {
+    uint32_t bits = e < 2 ? 0x00200000u << e : (uint32_t)(e - 1) << 23;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+static void dequant_mxfp4(const blk_mxfp4 *x, float *y, int64_t k) {
+    for (int64_t i = 0; i < k / QK; i++) {
+        const float d = ref_e8m0_to_fp32_half(x[i].e);
+        for (int j = 0; j < QK / 2; j++) {
+            y[i * QK + j] = d * mxfp4_kvalues[x[i].qs[j] & 0x0F];
+            y[i * QK + j + QK / 2] = d * mxfp4_kvalues[x[i].qs[j] >> 4];
+        }
+    }
+}
+
 /* Q5_K: the Q4_K layout with a fifth bit per weight.  Bit j of qh[l] belongs to element l of sub-block j (the low
  * nibbles of chunk c are sub-block 2c, the high nibbles sub-block 2c + 1); w = d * sc * (nibble + 16 * bit) - dmin * m. */
 static void dequant_q5_K(const blk_q5_K *x, float *y, int64_t k) {
@@ -572,6 +598,7 @@ int ref_dequantize_row(int type, const void *x, float *y, int64_t k) {
     switch (type) {
     case REF_TYPE_Q4_0: dequant_q4_0((const blk_q4_0 *)x, y, k); return 0;
     case REF_TYPE_Q8_0: dequant_q8_0((const blk_q8_0 *)x, y, k); return 0;
+    case REF_TYPE_MXFP4: dequant_mxfp4((const blk_mxfp4 *)x, y, k); return 0;
     case REF_TYPE_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
     case REF_TYPE_Q5_K: dequant_q5_K((const blk_q5_K *)x, y, k); return 0;
     case REF_TYPE_Q6_K: dequant_q6_K((const blk_q6_K *)x, y, k); return 0;
@@ -610,6 +637,23 @@ float ref_vec_dot_q8_0_q8_0(int64_t n, const void *vx, const void *vy) {
         int sumi = 0;
         for (int j = 0; j < QK; j++) sumi += x[ib].qs[j] * y[ib].qs[j];
         sumf += sumi * (ref_fp16_to_fp32(x[ib].d) * ref_fp16_to_fp32(y[ib].d));
+    }
+    return sumf;
+}
+
+/* ggml_vec_dot_mxfp4_q8_0, generic path */
+float ref_vec_dot_mxfp4_q8_0(int64_t n, const void *vx, const void *vy) {
+    const blk_mxfp4 *x = (const blk_mxfp4 *)vx;
+    const blk_q8_0 *y = (const blk_q8_0 *)vy;
+    float sumf = 0;
+    for (int64_t ib = 0; ib < n / QK; ib++) {
+        const float d = ref_fp16_to_fp32(y[ib].d) * ref_e8m0_to_fp32_half(x[ib].e);
+        int sumi1 = 0, sumi2 = 0;
+        for (int j = 0; j < QK / 2; j++) {
+            sumi1 += y[ib].qs[j] * mxfp4_kvalues[x[ib].qs[j] & 0x0F];
+            sumi2 += y[ib].qs[j + QK / 2] * mxfp4_kvalues[x[ib].qs[j] >> 4];
+        }
+        sumf += d * (sumi1 + sumi2);
     }
     return sumf;
 }
@@ -822,6 +866,7 @@ static dot_fn dot_for(int wtype) {
     switch (wtype) {
     case REF_TYPE_Q4_0: return ref_vec_dot_q4_0_q8_0;
     case REF_TYPE_Q8_0: return ref_vec_dot_q8_0_q8_0;
+    case REF_TYPE_MXFP4: return ref_vec_dot_mxfp4_q8_0;
     case REF_TYPE_Q4_K: return ref_vec_dot_q4_K_q8_K;
     case REF_TYPE_Q5_K: return ref_vec_dot_q5_K_q8_K;
     case REF_TYPE_Q6_K: return ref_vec_dot_q6_K_q8_K;

@@ -9,9 +9,9 @@ from __future__ import annotations
 
 import numpy as np
 
-F32, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K = 0, 2, 8, 12, 13, 14, 15
-BLOCK = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
-BYTES = {Q4_0: 18, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
+F32, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, MXFP4 = 0, 2, 8, 12, 13, 14, 15, 39
+BLOCK = {MXFP4: 32, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
+BYTES = {MXFP4: 17, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
 
 
 def _blocks(raw: np.ndarray, t: int) -> np.ndarray:
@@ -44,6 +44,18 @@ def q4_0_ints(raw):
     qs = b[:, 2:18].astype(np.int64)
     q = np.concatenate([qs & 15, qs >> 4], axis=1) - 8  # elements 0..15 low nibbles, 16..31 high
     return d, q
+
+
+def mxfp4_values(raw):
+    """[nb, 32] float64 from the formats' definitions (OCP microscaling): E2M1 = sign, two exponent bits, one mantissa
+    bit -- 0 and 0.5 at exponent 0, (1 + m / 2) 2^(exp - 1) above -- times the E8M0 scale 2^(e - 127)"""
+    b = _blocks(raw, MXFP4)
+    e = b[:, 0].astype(np.int64)
+    nib = np.concatenate([b[:, 1:] & 15, b[:, 1:] >> 4], axis=1).astype(np.int64)   # elements 0..15, then 16..31
+    sign = np.where(nib & 8, -1.0, 1.0)
+    ex, man = (nib >> 1) & 3, nib & 1
+    mag = np.where(ex == 0, man * 0.5, (1 + man / 2) * 2.0 ** (ex - 1))
+    return sign * mag * (2.0 ** (e - 127))[:, None]
 
 
 def q8_0_ints(raw):
@@ -103,6 +115,8 @@ def dequant(t: int, raw) -> np.ndarray:
     if t == Q8_0:
         d, q = q8_0_ints(raw)
         return (d[:, None] * q).reshape(-1)
+    if t == MXFP4:
+        return mxfp4_values(raw).reshape(-1)
     if t == Q4_K:
         d, dmin, sc, m, q = q4_K_ints(raw)
         w = (d[:, None] * sc)[:, :, None] * q - (dmin[:, None] * m)[:, :, None]

@@ -1,0 +1,100 @@
+"""Mulmat and MulmatID on MXFP4 weights (the expert tensors of gpt-oss files) through the C ABI against the oracle.  The
+library keeps such a tensor as the Q8_0 planes with the same dot products, so every Q8_0 kernel and entry point serves it."""
+import numpy as np
+import pytest
+
+import npref
+import oracle
+from ollama_amd import qmm, synth
+from oracle import MXFP4, Q8_0
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = qmm.Context(0)
+    yield c
+    c.close()
+
+
+def _random_rows(m, k, seed, lo=110, hi=135):
+    rng = np.random.default_rng(seed)
+    raw = rng.integers(0, 256, (m, k // 32, 17), dtype=np.uint8)
+    raw[..., 0] = rng.integers(lo, hi, (m, k // 32))
+    return raw.reshape(m, -1)
+
+
+@pytest.mark.parametrize("m,k,n", [(64, 256, 1), (2880, 2880 // 32 * 32, 1), (512, 4096, 2), (512, 4096, 4), (300, 2048, 8),
+                                   (256, 4096, 20), (1024, 4096, 130), (4096, 4096, 1), (5760, 2880 // 32 * 32, 512)])
+def test_mxfp4_against_the_oracle(ctx, m, k, n):
+    print(f"mxfp4 case m={m} k={k} n={n}", flush=True)
+    raw = _random_rows(m, k, seed=m + k + n) if m * k <= 1 << 22 else synth.weights(MXFP4, m, k, seed=m)
+    x = np.random.default_rng(n + k).standard_normal((n, k)).astype(np.float32)
+    W = ctx.upload(MXFP4, raw, k, m)
+    try:
+        assert (W.type, W.k, W.m) == (MXFP4, k, m)
+        y = ctx.mulmat(W, x)
+        ref, xq = oracle.mul_mat(MXFP4, raw, k, m, x, nthreads=8, return_xq=True)
+        assert np.array_equal(ctx.quantize_act(Q8_0, x), xq)
+        assert npref.rel_err(y, ref) <= 1e-3
+        if m * n <= 1 << 16:
+            assert npref.rel_err(y, npref.matmul_f64(MXFP4, raw, k, m, Q8_0, xq, n), floor=1e-3) <= 1e-3
+    finally:
+        W.free()
+
+
+def test_mxfp4_scales_at_the_edges_of_what_the_planes_hold(ctx):
+    """e = 104 (a subnormal half), 113 / 114 (the last subnormal, the first normal), 143 (the largest half), 144 .. 146
+    (the integers shifted instead): exact; below 104 the block is zero; above 146 the upload is refused"""
+    k, m = 64, 16
+    x = np.random.default_rng(1).integers(-127, 128, (2, k)).astype(np.float32)
+    x[:, ::32] = 127
+    for e in (104, 105, 113, 114, 127, 128, 143, 144, 146):
+        raw = _random_rows(m, k, seed=e).reshape(m, 2, 17)
+        raw[..., 0] = e
+        W = ctx.upload(MXFP4, raw.reshape(m, -1), k, m)
+        y = ctx.mulmat(W, x)
+        W.free()
+        w = npref.dequant(MXFP4, raw.reshape(-1)).reshape(m, k)
+        assert np.array_equal(y, (x.astype(np.float64) @ w.T).astype(np.float32)), e   # integers times a power of two
+    raw = _random_rows(m, k, seed=3).reshape(m, 2, 17)
+    raw[..., 0] = 100
+    W = ctx.upload(MXFP4, raw.reshape(m, -1), k, m)
+    assert not ctx.mulmat(W, x).any()
+    W.free()
+    raw[3, 1, 0] = 147
+    with pytest.raises(qmm.QmmError) as err:
+        ctx.upload(MXFP4, raw.reshape(m, -1), k, m)
+    assert err.value.code == qmm.ERR_UNSUPPORTED
+
+
+def test_mxfp4_expert_stacks_and_joint_calls(ctx):
+    """the entry points a Q8_0 weight goes through: the expert-indexed product (gpt-oss: 4 of 32 experts), the joint call,
+    the two-phase form, the fused producers"""
+    k, m, n_exp, n_used = 2880 // 32 * 32, 96, 8, 4
+    raw = _random_rows(m * n_exp, k, seed=11)
+    W = ctx.upload(MXFP4, raw, k, m * n_exp)
+    try:
+        for tokens in (1, 5, 70):
+            rng = np.random.default_rng(tokens)
+            b = rng.standard_normal((tokens, 1, k)).astype(np.float32)
+            ids = np.stack([rng.permutation(n_exp)[:n_used] for _ in range(tokens)]).astype(np.int32)
+            y = ctx.mulmat_id(W, n_exp, b, ids)
+            ref = oracle.mul_mat_id(MXFP4, raw, k, m, n_exp, b, ids)
+            assert npref.rel_err(y.reshape(ref.shape), ref) <= 1e-3, tokens
+        x = np.random.default_rng(9).standard_normal((3, k)).astype(np.float32)
+        W2 = ctx.upload(MXFP4, raw[:200], k, 200)
+        W8 = ctx.upload(Q8_0, synth.weights(Q8_0, 64, k, seed=2), k, 64)
+        ya, yb = ctx.mulmat_multi([W2, W8], x)
+        assert np.array_equal(ya, ctx.mulmat(W2, x)) and np.array_equal(yb, ctx.mulmat(W8, x))
+        act = ctx.act_create(Q8_0, k, 3)
+        ctx.act_quantize(act, x)
+        assert np.array_equal(ctx.mulmat_q8(W2, act), ya)
+        g = (1 + 0.1 * np.random.default_rng(4).standard_normal(k)).astype(np.float32)
+        yn, = ctx.mulmat_produced([W2], qmm.PRODUCE_RMSNORM, g, x, 1e-5)
+        want = oracle.mul_mat(MXFP4, raw[:200], k, 200, oracle.rms_norm(x, g, 1e-5))
+        assert npref.rel_err(yn, want) <= 1e-3
+        act.free(); W2.free(); W8.free()
+    finally:
+        W.free()
