@@ -152,9 +152,12 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      the file: its products cost what a Q4_K product of twice the K costs).  39 (MXFP4, the expert tensors of
  *      /root/reference/convert/convert_gptoss.go:124-150; DTypeMXFP4, /root/reference/ml/backend.go:404-412) is kept
  *      as the Q8_0 planes that give the same dot products -- the doubled E2M1 values as int8, the scale 2^(e - 128)
- *      as the block scale -- and goes through EVERY entry point a Q8_0 weight goes through, the expert-indexed ones
- *      included (twice the bytes of the file).  A scale byte above 146 is MI_QMM_ERR_UNSUPPORTED; blocks with a
- *      scale byte below 104 (weights under 7.2e-7) are kept as zeros.
+ *      as the block scale, twice the bytes of the file -- and goes through every entry point a Q8_0 weight goes
+ *      through, the expert-indexed ones included, when k is a multiple of 256.  Otherwise (k = 2880) its rows are
+ *      kept padded with zero blocks to the next multiple of 256 and the library pads the activation rows likewise
+ *      inside mi_qmm_mulmat, _path, _noalloc, _multi and mi_qmm_mulmat_id; the other entry points then return
+ *      MI_QMM_ERR_UNSUPPORTED.  A scale byte above 146 is MI_QMM_ERR_UNSUPPORTED; blocks with a scale byte below
+ *      104 (weights under 7.2e-7) are kept as zeros.
  *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
 int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
                          int64_t m, int src_location, mi_qmm_weight **out);

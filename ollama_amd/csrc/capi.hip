@@ -67,8 +67,11 @@ struct mi_qmm_weight {
     void *base = nullptr;
     size_t bytes = 0;
     DevWeight dev{};
-    // a Q5_K tensor: dev is the Q4_K tensor of rows of 2 k5 that stands for it (formats.h), multiplied with [x | x]
+    // q5k: whether the caller's activation rows must be expanded before the product, from k5 to dev.K floats --
+    // a Q5_K tensor (dev is the Q4_K tensor of rows of 2 k5 that stands for it, formats.h: multiplied with [x | x]) or an
+    // MXFP4 tensor whose rows were padded with zero blocks to whole 256-element steps (multiplied with [x | 0])
     bool q5k = false;
+    bool repeat = false;  // [x | x] rather than [x | 0]
     int64_t k5 = 0;
     int file_type = -1;  // the ggml type the tensor had in the file, where dev.type is another (Q5_K, MXFP4); -1: dev.type
 };
@@ -339,7 +342,8 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     case T_Q4_K: case T_F32: case T_F16: case T_BF16: s0 = total; break;
     case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; break;  // a Q4_K tensor of rows twice as long
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
-    case T_Q8_0: case T_MXFP4: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;  // (MXFP4: kept as Q8_0 planes)
+    case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
+    case T_MXFP4: s0 = (size_t)(m * align_up((size_t)k, 256)); sd = (size_t)(m * (align_up((size_t)k, 256) / QK)) * 2; break;  // kept as Q8_0 planes
     case T_Q6_K: s0 = (size_t)(m * (k / 2)); s1 = (size_t)(m * (k / 4)); s2 = (size_t)(m * (k / 16));
                  sd = (size_t)(m * (k / QKK)) * 2; break;
     }
@@ -361,8 +365,12 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     w->dev.p2 = s2 ? b + o2 : nullptr;
     w->dev.d = sd ? (const uint16_t *)(b + od) : nullptr;
     w->dev.K = k; w->dev.M = m; w->dev.type = type;
-    if (type == T_Q5_K) { w->q5k = true; w->k5 = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K; }
-    if (type == T_MXFP4) { w->dev.type = T_Q8_0; w->file_type = T_MXFP4; }
+    if (type == T_Q5_K) { w->q5k = w->repeat = true; w->k5 = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K; }
+    if (type == T_MXFP4) {
+        // rows of a whole number of 256-element steps (2880 -> 3072): the matrix-core kernels of the 32-element formats want that
+        w->dev.type = T_Q8_0; w->file_type = T_MXFP4; w->dev.K = (int64_t)align_up((size_t)k, 256);
+        if (w->dev.K != k) { w->q5k = true; w->k5 = k; }
+    }
 
     void *staging = nullptr;
     const uint8_t *src = (const uint8_t *)bytes;
@@ -391,7 +399,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
             if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemset(flag)", e);
         }
         e = type == T_Q5_K ? launch_relayout_q5k(src, k, m, b + o0, ctx->stream)
-            : type == T_MXFP4 ? launch_relayout_mxfp4(src, k, m, b + o0, (uint16_t *)(b + od), bad, ctx->stream)
+            : type == T_MXFP4 ? launch_relayout_mxfp4(src, k, w->dev.K, m, b + o0, (uint16_t *)(b + od), bad, ctx->stream)
                               : launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
         if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
         if (bad) {
@@ -426,7 +434,7 @@ void mi_qmm_weight_free(mi_qmm_weight *w) {
 int mi_qmm_weight_info(const mi_qmm_weight *w, int *type, int64_t *k, int64_t *m, int64_t *device_bytes) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
     if (type) *type = w->file_type >= 0 ? w->file_type : w->dev.type;
-    if (k) *k = w->q5k ? w->k5 : w->dev.K;
+    if (k) *k = w->q5k ? w->k5 : w->dev.K;  // (the caller's K)
     if (m) *m = w->dev.M;
     if (device_bytes) *device_bytes = (int64_t)w->bytes;
     return MI_QMM_OK;
@@ -657,7 +665,7 @@ int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, in
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
     if (!allow_plain && (plain_type(w->dev.type) || w->q5k))
         return fail(MI_QMM_ERR_UNSUPPORTED, "this entry point takes Q4_0 / Q8_0 / Q4_K / Q6_K weights; type %d goes through mi_qmm_mulmat",
-                    w->q5k ? T_Q5_K : w->dev.type);
+                    w->file_type >= 0 ? w->file_type : w->dev.type);
     if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
         return fail(MI_QMM_ERR_INVALID, "location must be MI_QMM_HOST or MI_QMM_DEVICE");
     if (path != MI_QMM_PATH_AUTO && path != MI_QMM_PATH_GEMV && path != MI_QMM_PATH_GEMM && path != MI_QMM_PATH_QUERY)
@@ -730,14 +738,14 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     if (rc) return rc;
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
     if (w->q5k) {
-        // the Q4_K tensor of rows of 2 k that stands for the Q5_K one, against [x | x]
+        // the tensor of longer rows that stands for this one, against the expanded activations ([x | x] or [x | 0])
         mi_qmm_weight lo = *w;
         lo.q5k = false;
         if (path == MI_QMM_PATH_QUERY || n == 0) return mi_qmm_mulmat_path(ctx, &lo, x, n, y, location, path);
         if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
-        const size_t xb = (size_t)(n * w->k5) * 4, yb = (size_t)(n * w->dev.M) * 4;
-        const size_t o_raw = align_up(2 * xb, 256), o_y = o_raw + align_up(xb, 256);
-        if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_y + yb : 2 * xb))) return rc;
+        const size_t xb = (size_t)(n * w->k5) * 4, xxb = (size_t)(n * w->dev.K) * 4, yb = (size_t)(n * w->dev.M) * 4;
+        const size_t o_raw = align_up(xxb, 256), o_y = o_raw + align_up(xb, 256);
+        if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_y + yb : xxb))) return rc;
         float *xx = (float *)ctx->dup_buf;
         const float *dx = x;
         float *dy = y;
@@ -746,7 +754,7 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
             dy = (float *)((char *)ctx->dup_buf + o_y);
             HIP_TRY(hipMemcpyAsync((void *)dx, x, xb, hipMemcpyHostToDevice, ctx->stream));
         }
-        HIP_TRY(launch_dup_rows(dx, w->k5, n, xx, ctx->stream));
+        HIP_TRY(launch_expand_rows(dx, w->k5, w->dev.K, n, w->repeat, xx, ctx->stream));
         if ((rc = mi_qmm_mulmat_path(ctx, &lo, xx, n, dy, MI_QMM_DEVICE, path))) return rc;
         if (location == MI_QMM_HOST) {
             HIP_TRY(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, ctx->stream));
@@ -822,15 +830,15 @@ static int noalloc_core(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x,
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
     if (w->q5k) {
-        // [x | x] at the end of the scratch, the quantized planes of the product in front of it
+        // the expanded activations at the end of the scratch, the quantized planes of the product in front of them
         mi_qmm_weight lo = *w;
         lo.q5k = false;
-        const size_t xx_bytes = align_up((size_t)(n * w->k5) * 8, 256);
+        const size_t xx_bytes = align_up((size_t)(n * w->dev.K) * 4, 256);
         if (xx_bytes + 256 > sbytes)
-            return fail(MI_QMM_ERR_UNSUPPORTED, "n=%lld rows of k=%lld of a Q5_K product need %zu bytes for the repeated activations alone; the "
+            return fail(MI_QMM_ERR_UNSUPPORTED, "n=%lld rows of k=%lld of this product need %zu bytes for the expanded activations alone; the "
                         "static scratch of mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)w->k5, xx_bytes, sbytes);
         float *xx = (float *)((char *)sbase + (sbytes - xx_bytes) / 256 * 256);
-        HIP_TRY(launch_dup_rows(x, w->k5, n, xx, ctx->stream));
+        HIP_TRY(launch_expand_rows(x, w->k5, w->dev.K, n, w->repeat, xx, ctx->stream));
         return noalloc_core(ctx, &lo, xx, n, y, sbase, (sbytes - xx_bytes) / 256 * 256);
     }
     if (plain_type(w->dev.type))
@@ -1343,6 +1351,41 @@ extern "C" {
 
 int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
                      const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location) {
+    if (w && w->q5k && !w->repeat && ctx && x && y && ids && n_tokens > 0 && n_used > 0 && b_cols > 0 && n_expert > 0 &&
+        (location == MI_QMM_HOST || location == MI_QMM_DEVICE) && n_tokens * (int64_t)b_cols <= INT32_MAX) {
+        // an expert stack whose rows were padded to whole 256-element steps (MXFP4 experts of K = 2880): the activation
+        // rows are padded likewise, on the device, and the product runs on device pointers
+        int rc = check_ctx(ctx);
+        if (rc) return rc;
+        mi_qmm_weight lo = *w;
+        lo.q5k = false;
+        const int64_t rows = n_tokens * b_cols, pairs = n_tokens * n_used;
+        const size_t xb = (size_t)(rows * w->k5) * 4, xxb = (size_t)(rows * w->dev.K) * 4;
+        const size_t yb = (size_t)(pairs * (w->dev.M / n_expert)) * 4, ib = (size_t)pairs * 4;
+        const size_t o_raw = align_up(xxb, 256), o_y = o_raw + align_up(xb, 256), o_ids = o_y + align_up(yb, 256);
+        if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_ids + ib : xxb))) return rc;
+        float *xx = (float *)ctx->dup_buf;
+        const float *dx = x;
+        float *dy = y;
+        const int32_t *dids = ids;
+        if (location == MI_QMM_HOST) {
+            for (int64_t p = 0; p < pairs; p++)
+                if (ids[p] < 0 || ids[p] >= n_expert)
+                    return fail(MI_QMM_ERR_INVALID, "ids[%lld] = %d is outside 0..%d", (long long)p, ids[p], n_expert - 1);
+            dx = (const float *)((char *)ctx->dup_buf + o_raw);
+            dy = (float *)((char *)ctx->dup_buf + o_y);
+            dids = (const int32_t *)((char *)ctx->dup_buf + o_ids);
+            HIP_TRY(hipMemcpyAsync((void *)dx, x, xb, hipMemcpyHostToDevice, ctx->stream));
+            HIP_TRY(hipMemcpyAsync((void *)dids, ids, ib, hipMemcpyHostToDevice, ctx->stream));
+        }
+        HIP_TRY(launch_expand_rows(dx, w->k5, w->dev.K, rows, false, xx, ctx->stream));
+        if ((rc = mulmat_id_impl(ctx, &lo, nullptr, n_expert, xx, b_cols, dids, n_used, n_tokens, dy, nullptr, MI_QMM_DEVICE))) return rc;
+        if (location == MI_QMM_HOST) {
+            HIP_TRY(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(hipStreamSynchronize(ctx->stream));
+        }
+        return MI_QMM_OK;
+    }
     return mulmat_id_impl(ctx, w, nullptr, n_expert, x, b_cols, ids, n_used, n_tokens, y, nullptr, location);
 }
 

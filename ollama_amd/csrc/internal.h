@@ -36,11 +36,12 @@ hipError_t launch_relayout(int type, const uint8_t *gguf, int64_t K, int64_t M, 
 
 // Q5_K blocks [M][K/256][176] -> the Q4_K tensor of rows of 2 K that stands for them (formats.h): out [M][2 K/256][144]
 hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *out, hipStream_t s);
-// MXFP4 blocks [M][K/32][17] -> Q8_0 planes (qs [M][K], d [M][K/32]) with the same dot products; *bad (device int, zeroed
+// MXFP4 blocks [M][K/32][17] -> Q8_0 planes (qs [M][K_out], d [M][K_out/32], rows padded with zero blocks) with the same dot products; *bad (device int, zeroed
 // by the caller) is set when a block's scale is beyond what the planes can hold (e > 146: weights of 2^18 and more)
-hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s);
-// out [n][2 K] = [x row | x row] for x [n][K] (K a multiple of 4): the activations such a tensor is multiplied with
-hipError_t launch_dup_rows(const float *x, int64_t K, int64_t n, float *out, hipStream_t s);
+hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s);
+// out [n][K_out] for x [n][K] (both multiples of 4, K <= K_out): the row followed by itself (repeat, K_out = 2 K: the
+// activations a Q5_K tensor kept as Q4_K is multiplied with) or by zeros (rows padded to the length the weight was padded to)
+hipError_t launch_expand_rows(const float *x, int64_t K, int64_t K_out, int64_t n, bool repeat, float *out, hipStream_t s);
 
 // kernels 2 and 4: streaming GEMV / skinny GEMM, ncols in 1..8.  y[n*ldy + m].
 // returns hipErrorInvalidValue if the shape is outside the kernel's limits (caller reports it).

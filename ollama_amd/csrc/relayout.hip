@@ -79,13 +79,21 @@ __global__ void relayout_q5k_kernel(const uint8_t *__restrict__ src, int64_t M, 
 // activations as sum_i q_i y_i * (scale * d_y): the Q8_0 dot product of a block with those integers and that scale.  The
 // scale is a half for e in 104 .. 143; up to e = 146 the integers are shifted left instead (12 * 8 = 96 fits); below 104
 // (weights under 7.2e-7) the block is zero; above 146 *bad is set.  One thread per nibble byte.
-__global__ void relayout_mxfp4_kernel(const uint8_t *__restrict__ src, int64_t nblocks, int8_t *__restrict__ qs, uint16_t *__restrict__ d,
-                                      int *__restrict__ bad) {
+// Rows are padded with zero blocks from nb_in to nb_out blocks (rows of a whole number of 256-element steps, which the
+// matrix-core kernels for the 32-element formats want).
+__global__ void relayout_mxfp4_kernel(const uint8_t *__restrict__ src, int64_t M, int nb_in, int nb_out, int8_t *__restrict__ qs,
+                                      uint16_t *__restrict__ d, int *__restrict__ bad) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= nblocks * 16) return;
-    const int64_t blk = i >> 4;
-    const int j = (int)(i & 15);
-    const uint8_t *b = src + blk * 17;
+    if (i >= M * nb_out * 16) return;
+    const int64_t blk = i >> 4, row = blk / nb_out;
+    const int bi = (int)(blk - row * nb_out), j = (int)(i & 15);
+    if (bi >= nb_in) {
+        qs[blk * 32 + j] = 0;
+        qs[blk * 32 + j + 16] = 0;
+        if (j == 0) d[blk] = 0;
+        return;
+    }
+    const uint8_t *b = src + (row * nb_in + bi) * 17;
     const int e = b[0];
     int shift = 0, he = e - 128 + 15;  // biased fp16 exponent of 2^(e - 128)
     if (e > 143) { shift = e - 143; he = 30; }
@@ -106,12 +114,14 @@ __global__ void relayout_mxfp4_kernel(const uint8_t *__restrict__ src, int64_t n
     }
 }
 
-__global__ void dup_rows_kernel(const float4 *__restrict__ x, float4 *__restrict__ out, int64_t k4, int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < k4 * n; i += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t r = i / k4, c = i - r * k4;
-        const float4 v = x[i];
-        out[r * 2 * k4 + c] = v;
-        out[r * 2 * k4 + k4 + c] = v;
+// out [n][k_out] from x [n][k_in] (in float4 units): the row, then -- repeat (k_out = 2 k_in): the row once more; else zeros
+__global__ void expand_rows_kernel(const float4 *__restrict__ x, float4 *__restrict__ out, int64_t k4_in, int64_t k4_out, int64_t n, bool repeat) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < k4_out * n; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / k4_out, c = i - r * k4_out;
+        float4 v = {0.f, 0.f, 0.f, 0.f};
+        if (c < k4_in) v = x[r * k4_in + c];
+        else if (repeat) v = x[r * k4_in + (c - k4_in)];
+        out[i] = v;
     }
 }
 
@@ -125,19 +135,21 @@ hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_
     return hipGetLastError();
 }
 
-hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s) {
+hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s) {
     if (K * M == 0) return hipSuccess;
-    const int64_t n = M * (K / QK) * 16;
+    if (K % QK || K_out % QK || K_out < K) return hipErrorInvalidValue;
+    const int64_t n = M * (K_out / QK) * 16;
     if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
-    relayout_mxfp4_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M * (K / QK), (int8_t *)qs, d, bad);
+    relayout_mxfp4_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QK), (int)(K_out / QK), (int8_t *)qs, d, bad);
     return hipGetLastError();
 }
 
-hipError_t launch_dup_rows(const float *x, int64_t K, int64_t n, float *out, hipStream_t s) {
+hipError_t launch_expand_rows(const float *x, int64_t K, int64_t K_out, int64_t n, bool repeat, float *out, hipStream_t s) {
     if (K * n == 0) return hipSuccess;
-    if (K % 4) return hipErrorInvalidValue;
-    const int64_t work = K / 4 * n;
-    dup_rows_kernel<<<(unsigned)std::min<int64_t>((work + 255) / 256, 4096), 256, 0, s>>>((const float4 *)x, (float4 *)out, K / 4, n);
+    if (K % 4 || K_out % 4 || K_out < K || (repeat && K_out != 2 * K)) return hipErrorInvalidValue;
+    const int64_t work = K_out / 4 * n;
+    expand_rows_kernel<<<(unsigned)std::min<int64_t>((work + 255) / 256, 4096), 256, 0, s>>>((const float4 *)x, (float4 *)out, K / 4, K_out / 4, n,
+                                                                                             repeat);
     return hipGetLastError();
 }
 

@@ -88,13 +88,26 @@ def test_mxfp4_expert_stacks_and_joint_calls(ctx):
         W8 = ctx.upload(Q8_0, synth.weights(Q8_0, 64, k, seed=2), k, 64)
         ya, yb = ctx.mulmat_multi([W2, W8], x)
         assert np.array_equal(ya, ctx.mulmat(W2, x)) and np.array_equal(yb, ctx.mulmat(W8, x))
+        # rows of 2880 are kept padded to 3072: the forms that read activations somebody else quantized are refused
         act = ctx.act_create(Q8_0, k, 3)
         ctx.act_quantize(act, x)
-        assert np.array_equal(ctx.mulmat_q8(W2, act), ya)
-        g = (1 + 0.1 * np.random.default_rng(4).standard_normal(k)).astype(np.float32)
-        yn, = ctx.mulmat_produced([W2], qmm.PRODUCE_RMSNORM, g, x, 1e-5)
-        want = oracle.mul_mat(MXFP4, raw[:200], k, 200, oracle.rms_norm(x, g, 1e-5))
-        assert npref.rel_err(yn, want) <= 1e-3
+        for call in (lambda: ctx.mulmat_q8(W2, act), lambda: ctx.mulmat_produced([W2], qmm.PRODUCE_RMSNORM, None, x, 1e-5)):
+            with pytest.raises(qmm.QmmError) as err:
+                call()
+            assert err.value.code == qmm.ERR_UNSUPPORTED
         act.free(); W2.free(); W8.free()
+        # rows of whole 256-element steps: every entry point of a Q8_0 weight
+        k2 = 2048
+        raw2 = _random_rows(200, k2, seed=12)
+        x2 = np.random.default_rng(10).standard_normal((3, k2)).astype(np.float32)
+        W3 = ctx.upload(MXFP4, raw2, k2, 200)
+        act = ctx.act_create(Q8_0, k2, 3)
+        ctx.act_quantize(act, x2)
+        assert np.array_equal(ctx.mulmat_q8(W3, act), ctx.mulmat(W3, x2))
+        g = (1 + 0.1 * np.random.default_rng(4).standard_normal(k2)).astype(np.float32)
+        yn, = ctx.mulmat_produced([W3], qmm.PRODUCE_RMSNORM, g, x2, 1e-5)
+        want = oracle.mul_mat(MXFP4, raw2, k2, 200, oracle.rms_norm(x2, g, 1e-5))
+        assert npref.rel_err(yn, want) <= 1e-3
+        act.free(); W3.free()
     finally:
         W.free()
