@@ -67,12 +67,12 @@ struct mi_qmm_weight {
     void *base = nullptr;
     size_t bytes = 0;
     DevWeight dev{};
-    // q5k: whether the caller's activation rows must be expanded before the product, from k5 to dev.K floats --
-    // a Q5_K tensor (dev is the Q4_K tensor of rows of 2 k5 that stands for it, formats.h: multiplied with [x | x]) or an
+    // expand: the caller's activation rows must be expanded before the product, from k_user to dev.K floats --
+    // a Q5_K tensor (dev is the Q4_K tensor of rows of 2 k_user that stands for it, formats.h: multiplied with [x | x]) or an
     // MXFP4 tensor whose rows were padded with zero blocks to whole 256-element steps (multiplied with [x | 0])
-    bool q5k = false;
+    bool expand = false;
     bool repeat = false;  // [x | x] rather than [x | 0]
-    int64_t k5 = 0;
+    int64_t k_user = 0;
     int file_type = -1;  // the ggml type the tensor had in the file, where dev.type is another (Q5_K, MXFP4); -1: dev.type
 };
 
@@ -365,11 +365,11 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     w->dev.p2 = s2 ? b + o2 : nullptr;
     w->dev.d = sd ? (const uint16_t *)(b + od) : nullptr;
     w->dev.K = k; w->dev.M = m; w->dev.type = type;
-    if (type == T_Q5_K) { w->q5k = w->repeat = true; w->k5 = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K; }
+    if (type == T_Q5_K) { w->expand = w->repeat = true; w->k_user = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K; }
     if (type == T_MXFP4) {
         // rows of a whole number of 256-element steps (2880 -> 3072): the matrix-core kernels of the 32-element formats want that
         w->dev.type = T_Q8_0; w->file_type = T_MXFP4; w->dev.K = (int64_t)align_up((size_t)k, 256);
-        if (w->dev.K != k) { w->q5k = true; w->k5 = k; }
+        if (w->dev.K != k) { w->expand = true; w->k_user = k; }
     }
 
     void *staging = nullptr;
@@ -434,7 +434,7 @@ void mi_qmm_weight_free(mi_qmm_weight *w) {
 int mi_qmm_weight_info(const mi_qmm_weight *w, int *type, int64_t *k, int64_t *m, int64_t *device_bytes) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
     if (type) *type = w->file_type >= 0 ? w->file_type : w->dev.type;
-    if (k) *k = w->q5k ? w->k5 : w->dev.K;  // (the caller's K)
+    if (k) *k = w->expand ? w->k_user : w->dev.K;  // (the caller's K)
     if (m) *m = w->dev.M;
     if (device_bytes) *device_bytes = (int64_t)w->bytes;
     return MI_QMM_OK;
@@ -663,7 +663,7 @@ int route_f32(const mi_qmm_ctx *ctx, const mi_qmm_weight *w, int64_t n, int path
 // joint, produced, expert-indexed and pre-quantized forms are for the block-quantized types)
 int check_product_args(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int location, int path, bool allow_plain = false) {
     if (!w) return fail(MI_QMM_ERR_INVALID, "weight is NULL");
-    if (!allow_plain && (plain_type(w->dev.type) || w->q5k))
+    if (!allow_plain && (plain_type(w->dev.type) || w->expand))
         return fail(MI_QMM_ERR_UNSUPPORTED, "this entry point takes Q4_0 / Q8_0 / Q4_K / Q6_K weights; type %d goes through mi_qmm_mulmat",
                     w->file_type >= 0 ? w->file_type : w->dev.type);
     if (location != MI_QMM_HOST && location != MI_QMM_DEVICE)
@@ -737,13 +737,13 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     int rc = check_product_args(ctx, w, location, path, /*allow_plain=*/true);
     if (rc) return rc;
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
-    if (w->q5k) {
+    if (w->expand) {
         // the tensor of longer rows that stands for this one, against the expanded activations ([x | x] or [x | 0])
         mi_qmm_weight lo = *w;
-        lo.q5k = false;
+        lo.expand = false;
         if (path == MI_QMM_PATH_QUERY || n == 0) return mi_qmm_mulmat_path(ctx, &lo, x, n, y, location, path);
         if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
-        const size_t xb = (size_t)(n * w->k5) * 4, xxb = (size_t)(n * w->dev.K) * 4, yb = (size_t)(n * w->dev.M) * 4;
+        const size_t xb = (size_t)(n * w->k_user) * 4, xxb = (size_t)(n * w->dev.K) * 4, yb = (size_t)(n * w->dev.M) * 4;
         const size_t o_raw = align_up(xxb, 256), o_y = o_raw + align_up(xb, 256);
         if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_y + yb : xxb))) return rc;
         float *xx = (float *)ctx->dup_buf;
@@ -754,7 +754,7 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
             dy = (float *)((char *)ctx->dup_buf + o_y);
             HIP_TRY(hipMemcpyAsync((void *)dx, x, xb, hipMemcpyHostToDevice, ctx->stream));
         }
-        HIP_TRY(launch_expand_rows(dx, w->k5, w->dev.K, n, w->repeat, xx, ctx->stream));
+        HIP_TRY(launch_expand_rows(dx, w->k_user, w->dev.K, n, w->repeat, xx, ctx->stream));
         if ((rc = mi_qmm_mulmat_path(ctx, &lo, xx, n, dy, MI_QMM_DEVICE, path))) return rc;
         if (location == MI_QMM_HOST) {
             HIP_TRY(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, ctx->stream));
@@ -829,16 +829,16 @@ static int noalloc_core(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x,
     if (n == 0) return MI_QMM_OK;
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
-    if (w->q5k) {
+    if (w->expand) {
         // the expanded activations at the end of the scratch, the quantized planes of the product in front of them
         mi_qmm_weight lo = *w;
-        lo.q5k = false;
+        lo.expand = false;
         const size_t xx_bytes = align_up((size_t)(n * w->dev.K) * 4, 256);
         if (xx_bytes + 256 > sbytes)
             return fail(MI_QMM_ERR_UNSUPPORTED, "n=%lld rows of k=%lld of this product need %zu bytes for the expanded activations alone; the "
-                        "static scratch of mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)w->k5, xx_bytes, sbytes);
+                        "static scratch of mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)w->k_user, xx_bytes, sbytes);
         float *xx = (float *)((char *)sbase + (sbytes - xx_bytes) / 256 * 256);
-        HIP_TRY(launch_expand_rows(x, w->k5, w->dev.K, n, w->repeat, xx, ctx->stream));
+        HIP_TRY(launch_expand_rows(x, w->k_user, w->dev.K, n, w->repeat, xx, ctx->stream));
         return noalloc_core(ctx, &lo, xx, n, y, sbase, (sbytes - xx_bytes) / 256 * 256);
     }
     if (plain_type(w->dev.type))
@@ -922,7 +922,7 @@ int mulmat_multi_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count
     if (rc) return rc;
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
-        if (plain_type(ws[i]->dev.type) || ws[i]->q5k)
+        if (plain_type(ws[i]->dev.type) || ws[i]->expand)
             return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is of a type that only mi_qmm_mulmat multiplies (F32 / F16 / BF16 / Q5_K)", i);
     }
     Produce pr{PRODUCE_NONE, nullptr, 0.f, nullptr};
@@ -1094,10 +1094,10 @@ extern "C" {
 int mi_qmm_mulmat_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int count, const float *x, int64_t n,
                         float *const *ys, int location) {
     bool plain = false;
-    for (int i = 0; ws && ys && i < count; i++) plain = plain || (ws[i] && (plain_type(ws[i]->dev.type) || ws[i]->q5k));
+    for (int i = 0; ws && ys && i < count; i++) plain = plain || (ws[i] && (plain_type(ws[i]->dev.type) || ws[i]->expand));
     if (plain) {
         // unquantized and Q5_K weights have no joint kernels: one product after the other, each as mi_qmm_mulmat gives it
-        auto user_k = [](const mi_qmm_weight *w) { return w->q5k ? w->k5 : w->dev.K; };
+        auto user_k = [](const mi_qmm_weight *w) { return w->expand ? w->k_user : w->dev.K; };
         for (int i = 0; i < count; i++) {
             if (!ws[i] || !ys[i]) return fail(MI_QMM_ERR_INVALID, "ws[%d] or ys[%d] is NULL", i, i);
             if (user_k(ws[i]) != user_k(ws[0]))
@@ -1133,7 +1133,7 @@ int mi_qmm_mulmat_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const mi_
     int rc = check_product_args(ctx, w_gate, location, MI_QMM_PATH_AUTO);
     if (rc) return rc;
     if (w_up->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "w_up is on another device");
-    if (plain_type(w_up->dev.type) || w_up->q5k) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is of a type that only mi_qmm_mulmat multiplies");
+    if (plain_type(w_up->dev.type) || w_up->expand) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is of a type that only mi_qmm_mulmat multiplies");
     if (producer == MI_QMM_PRODUCE_RMSNORM && !(eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
     if (n == 0) return MI_QMM_OK;
     if (!x || !h) return fail(MI_QMM_ERR_INVALID, "x or h is NULL");
@@ -1224,7 +1224,7 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
     if (prod) pr = *prod;
     if (pr.kind == PRODUCE_SWIGLU && !pr.aux && n_tokens > 0) return fail(MI_QMM_ERR_INVALID, "SwiGLU needs the up operand");
     if (pr.kind == PRODUCE_RMSNORM && !(pr.eps >= 0.f)) return fail(MI_QMM_ERR_INVALID, "eps must be non-negative");
-    if (w2 && w2->q5k) return fail(MI_QMM_ERR_UNSUPPORTED, "the second expert stack is of a type that only mi_qmm_mulmat multiplies");
+    if (w2 && w2->expand) return fail(MI_QMM_ERR_UNSUPPORTED, "the second expert stack is of a type that only mi_qmm_mulmat multiplies");
     if (w2 && (w2->device != ctx->device || w2->dev.type != w->dev.type || w2->dev.K != w->dev.K || w2->dev.M != w->dev.M))
         return fail(MI_QMM_ERR_INVALID, "the two expert stacks differ in device, type or shape");
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
@@ -1351,16 +1351,16 @@ extern "C" {
 
 int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, const float *x, int b_cols,
                      const int32_t *ids, int n_used, int64_t n_tokens, float *y, int location) {
-    if (w && w->q5k && !w->repeat && ctx && x && y && ids && n_tokens > 0 && n_used > 0 && b_cols > 0 && n_expert > 0 &&
+    if (w && w->expand && !w->repeat && ctx && x && y && ids && n_tokens > 0 && n_used > 0 && b_cols > 0 && n_expert > 0 &&
         (location == MI_QMM_HOST || location == MI_QMM_DEVICE) && n_tokens * (int64_t)b_cols <= INT32_MAX) {
         // an expert stack whose rows were padded to whole 256-element steps (MXFP4 experts of K = 2880): the activation
         // rows are padded likewise, on the device, and the product runs on device pointers
         int rc = check_ctx(ctx);
         if (rc) return rc;
         mi_qmm_weight lo = *w;
-        lo.q5k = false;
+        lo.expand = false;
         const int64_t rows = n_tokens * b_cols, pairs = n_tokens * n_used;
-        const size_t xb = (size_t)(rows * w->k5) * 4, xxb = (size_t)(rows * w->dev.K) * 4;
+        const size_t xb = (size_t)(rows * w->k_user) * 4, xxb = (size_t)(rows * w->dev.K) * 4;
         const size_t yb = (size_t)(pairs * (w->dev.M / n_expert)) * 4, ib = (size_t)pairs * 4;
         const size_t o_raw = align_up(xxb, 256), o_y = o_raw + align_up(xb, 256), o_ids = o_y + align_up(yb, 256);
         if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_ids + ib : xxb))) return rc;
@@ -1378,7 +1378,7 @@ int mi_qmm_mulmat_id(mi_qmm_ctx *ctx, const mi_qmm_weight *w, int n_expert, cons
             HIP_TRY(hipMemcpyAsync((void *)dx, x, xb, hipMemcpyHostToDevice, ctx->stream));
             HIP_TRY(hipMemcpyAsync((void *)dids, ids, ib, hipMemcpyHostToDevice, ctx->stream));
         }
-        HIP_TRY(launch_expand_rows(dx, w->k5, w->dev.K, rows, false, xx, ctx->stream));
+        HIP_TRY(launch_expand_rows(dx, w->k_user, w->dev.K, rows, false, xx, ctx->stream));
         if ((rc = mulmat_id_impl(ctx, &lo, nullptr, n_expert, xx, b_cols, dids, n_used, n_tokens, dy, nullptr, MI_QMM_DEVICE))) return rc;
         if (location == MI_QMM_HOST) {
             HIP_TRY(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, ctx->stream));
@@ -1423,7 +1423,7 @@ int mi_qmm_mulmat_id_swiglu(mi_qmm_ctx *ctx, const mi_qmm_weight *w_gate, const 
     if (rc) return rc;
     if (w_up->device != ctx->device || w_up->dev.K != w_gate->dev.K || w_up->dev.M != w_gate->dev.M)
         return fail(MI_QMM_ERR_INVALID, "the gate and up stacks differ in device or shape");
-    if (plain_type(w_up->dev.type) || w_up->q5k) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is of a type that only mi_qmm_mulmat multiplies");
+    if (plain_type(w_up->dev.type) || w_up->expand) return fail(MI_QMM_ERR_UNSUPPORTED, "w_up is of a type that only mi_qmm_mulmat multiplies");
     if (n_expert < 1 || n_used < 1 || b_cols < 1 || n_tokens < 0)
         return fail(MI_QMM_ERR_INVALID, "n_expert=%d n_used=%d b_cols=%d n_tokens=%lld: all must be positive", n_expert,
                     n_used, b_cols, (long long)n_tokens);
@@ -1658,7 +1658,7 @@ int mi_qmm_mulmat_q8_multi(mi_qmm_ctx *ctx, const mi_qmm_weight *const *ws, int 
     DevWeight dw[8];
     for (int i = 0; i < count; i++) {
         if (ws[i]->device != ctx->device) return fail(MI_QMM_ERR_INVALID, "ws[%d] is on another device", i);
-        if (plain_type(ws[i]->dev.type) || ws[i]->q5k)
+        if (plain_type(ws[i]->dev.type) || ws[i]->expand)
             return fail(MI_QMM_ERR_UNSUPPORTED, "ws[%d] is of a type that only mi_qmm_mulmat multiplies (F32 / F16 / BF16 / Q5_K)", i);
         dw[i] = ws[i]->dev;
     }

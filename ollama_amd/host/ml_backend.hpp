@@ -130,9 +130,11 @@ public:
             int type = 0, nd = 0;
             int64_t dims[4];
             rc = mi_qmm_gguf_tensor(f, i, &name, &type, &nd, dims, nullptr, nullptr);
-            // (Q4_0 / Q8_0 / Q4_K / Q6_K; F32 / F16 / BF16 / Q5_K matrices go through mi_qmm_mulmat directly, not through this mirror)
+            // (Q4_0 / Q8_0 / Q4_K / Q6_K, MXFP4 with rows of whole 256-element steps; F32 / F16 / BF16 / Q5_K matrices and MXFP4 ones kept
+            // padded go through mi_qmm_mulmat / mi_qmm_mulmat_id directly, not through this mirror)
             const int q8 = mi_qmm_vec_dot_type(type);
-            if (rc != MI_QMM_OK || (nd != 2 && nd != 3) || (q8 != MI_QMM_TYPE_Q8_0 && q8 != MI_QMM_TYPE_Q8_K) || type == MI_QMM_TYPE_Q5_K) continue;
+            if (rc != MI_QMM_OK || (nd != 2 && nd != 3) || (q8 != MI_QMM_TYPE_Q8_0 && q8 != MI_QMM_TYPE_Q8_K) || type == MI_QMM_TYPE_Q5_K ||
+                (type == MI_QMM_TYPE_MXFP4 && dims[0] % 256 != 0)) continue;
             auto t = std::make_shared<Tensor>();
             t->shape_.assign(dims, dims + nd);
             t->type_ = type;

@@ -42,6 +42,12 @@ I32 = 26  # ggml_type id of int32, /root/reference/fs/ggml/type.go:252-279
 _GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.F16: DType.F16, qmm.Q8_0: DType.Q80, qmm.Q4_0: DType.Q40, qmm.MXFP4: DType.MXFP4, I32: DType.I32}
 
 
+def _single_only(t: "Tensor") -> bool:
+    """weights that only the plain product entry points multiply (mulmat, mulmat_multi; for padded MXFP4 stacks also
+    mulmat_id): F32 / F16 / BF16, Q5_K, and MXFP4 whose rows are no multiple of 256 (kept padded on the device)"""
+    return t._type in qmm.SINGLE_ONLY_TYPES or (t._type == qmm.MXFP4 and t.Dim(0) % 256 != 0)
+
+
 class Tensor:
     """A node of the graph: a weight, an input, or a pending Mulmat result."""
 
@@ -108,7 +114,7 @@ class Tensor:
         if self._weight is None or len(self._shape) != 3:
             raise TypeError("MulmatID: the receiver must be a 3-D quantized expert stack obtained from Backend.Get")
         if self._type in qmm.SINGLE_ONLY_TYPES:
-            raise TypeError("MulmatID: expert stacks must be of type Q4_0, Q8_0, Q4_K or Q6_K")
+            raise TypeError("MulmatID: expert stacks must be of type Q4_0, Q8_0, Q4_K, Q6_K or MXFP4")
         if t2._type != qmm.F32 or ids._type != I32:
             raise TypeError("MulmatID: activations must be f32 and ids int32")
         if t2.Dim(0) != self.Dim(0):
@@ -198,7 +204,7 @@ class Context:
                 needed.update(id(s) for s in srcs)
                 if t._prod[0] == qmm.PRODUCE_SWIGLU and t._prod[2] is None:
                     needed.add(id(t))  # the bare silu is always an f32 node
-            elif t._op[0]._type in qmm.SINGLE_ONLY_TYPES:
+            elif _single_only(t._op[0]):
                 needed.update(id(s) for s in srcs)  # these weight types have no fused producers: x must exist as f32
             for s in srcs:
                 readers.setdefault(id(s), []).append(t)
@@ -212,7 +218,7 @@ class Context:
             gate, up = t._prod[1], t._prod[2]
             if not (gate in pending and up in pending and gate is not up and gate._op is not None and up._op is not None
                     and gate._ids is up._ids and gate._op[1] is up._op[1]
-                    and gate._op[0]._type not in qmm.SINGLE_ONLY_TYPES and up._op[0]._type not in qmm.SINGLE_ONLY_TYPES
+                    and not _single_only(gate._op[0]) and not _single_only(up._op[0])
                     and gate._op[0].Shape() == up._op[0].Shape() and id(gate) not in tensors_ids(tensors)
                     and id(up) not in tensors_ids(tensors) and readers.get(id(gate)) == [t] and readers.get(id(up)) == [t]):
                 continue
@@ -266,7 +272,11 @@ class Context:
                          and u._op[0].Dim(2) == t._op[0].Dim(2) and id(u) not in pair_of]
                 tokens, n_used = ids.Dim(1), ids.Dim(0)
                 idv = ids._data.reshape(tokens, n_used)
-                if x._data is None and x._prod is not None:
+                if any(_single_only(u._op[0]) for u in nodes):
+                    # stacks kept padded on the device (MXFP4 experts of K = 2880): one plain expert-indexed product each
+                    b = x.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
+                    ys = [c.mulmat_id(u._op[0]._weight, t._op[0].Dim(2), b, idv) for u in nodes]
+                elif x._data is None and x._prod is not None:
                     # x is a producer nobody needs in f32 (silu(gate) * up in front of the down experts)
                     kind, src, aux, eps = x._prod
                     b = src.Floats().reshape(tokens, x.Dim(1), x.Dim(0))
@@ -280,10 +290,10 @@ class Context:
                 continue
             nodes = [u for u in pending if u._data is None and u._ids is None and u._op is not None and u._op[1] is x
                      and id(u) not in pair_of]
-            for u in [u for u in nodes if u._op[0]._type in qmm.SINGLE_ONLY_TYPES]:
+            for u in [u for u in nodes if _single_only(u._op[0])]:
                 # F32 / F16 / BF16 / Q5_K weights: one product each
                 u._data = c.mulmat(u._op[0]._weight, x.Floats().reshape(-1, x.Dim(0))).reshape(-1)
-            nodes = [u for u in nodes if u._op[0]._type not in qmm.SINGLE_ONLY_TYPES]
+            nodes = [u for u in nodes if not _single_only(u._op[0])]
             if not nodes:
                 continue
             if x._data is None and x._prod is not None:

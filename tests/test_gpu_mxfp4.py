@@ -111,3 +111,36 @@ def test_mxfp4_expert_stacks_and_joint_calls(ctx):
         act.free(); W3.free()
     finally:
         W.free()
+
+
+def test_python_mirror_on_a_gpt_oss_shaped_expert_block():
+    """rows of 2880 (kept padded on the device): expert stacks through MulmatID at decode and prefill size, and a dense
+    MXFP4 matrix beside a Q8_0 one reading the same activations"""
+    from ollama_amd import ml
+    k, m, n_exp, n_used = 2880, 64, 8, 4
+    raw_e = _random_rows(m * n_exp, k, seed=21)
+    raw_d = _random_rows(96, k, seed=22)
+    raw_8 = synth.weights(Q8_0, 40, k, seed=23)
+    b = ml.Backend({"blk.0.ffn_gate_up_exps.weight": (MXFP4, [k, m, n_exp], raw_e), "dense.weight": (MXFP4, [k, 96], raw_d),
+                    "other.weight": (Q8_0, [k, 40], raw_8)})
+    b.Load()
+    try:
+        assert b.Get("dense.weight").DType() == ml.DType.MXFP4
+        for tokens in (1, 40):
+            rng = np.random.default_rng(tokens)
+            xs = rng.standard_normal((tokens, k)).astype(np.float32)
+            ids = np.stack([rng.permutation(n_exp)[:n_used] for _ in range(tokens)]).astype(np.int32)
+            ctx = b.NewContext()
+            x = ctx.FromFloats(xs.reshape(-1), k, 1, tokens)
+            e = b.Get("blk.0.ffn_gate_up_exps.weight").MulmatID(ctx, x, ctx.FromInts(ids.reshape(-1), n_used, tokens))
+            x2 = ctx.FromFloats(xs.reshape(-1), k, tokens)
+            d = b.Get("dense.weight").Mulmat(ctx, x2)
+            o = b.Get("other.weight").Mulmat(ctx, x2)
+            ctx.Compute(e, d, o)
+            want_e = oracle.mul_mat_id(MXFP4, raw_e, k, m, n_exp, xs.reshape(tokens, 1, k), ids)
+            assert npref.rel_err(e.Floats().reshape(want_e.shape), want_e) <= 1e-3
+            assert npref.rel_err(d.Floats().reshape(tokens, 96), oracle.mul_mat(MXFP4, raw_d, k, 96, xs)) <= 1e-3
+            assert npref.rel_err(o.Floats().reshape(tokens, 40), oracle.mul_mat(Q8_0, raw_8, k, 40, xs)) <= 1e-3
+            ctx.Close()
+    finally:
+        b.Close()
