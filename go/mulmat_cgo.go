@@ -68,7 +68,7 @@ func New(device int) (*Backend, error) {
 // Close binds mi_qmm_destroy (Backend.Close, backend.go:18).
 func (b *Backend) Close() { C.mi_qmm_destroy(b.ctx) }
 
-// load binds mi_qmm_weight_upload (Backend.Load, backend.go:20): kind is the fs/ggml TensorType id (2, 8, 12, 14),
+// load binds mi_qmm_weight_upload (Backend.Load, backend.go:20): kind is the fs/ggml TensorType id (2, 8, 12, 14; 13, 39; 0, 1, 30),
 // raw the tensor's GGUF bytes; the library copies them before it returns, so a Go slice may be passed.
 func (b *Backend) load(name string, kind uint32, k, m int, raw []byte) {
 	t := &Tensor{b: b, shape: []int{k, m}}

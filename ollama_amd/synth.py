@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 2, 8, 12, 13, 14, 39
+F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 2, 8, 12, 13, 14, 30, 39
 
 
 def _f16_bytes(v: np.ndarray) -> np.ndarray:
@@ -43,6 +43,23 @@ def encode_q4_0(x: np.ndarray) -> np.ndarray:
     out[..., 0:2] = _f16_bytes(d)
     out[..., 2:] = q[..., :16] | (q[..., 16:] << 4)
     return out.reshape(m, -1)
+
+
+def encode_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    return x.view(np.uint8).reshape(x.shape[0], -1)
+
+
+def encode_f16(x: np.ndarray) -> np.ndarray:
+    h = np.ascontiguousarray(x, np.float32).astype(np.float16)
+    return h.view(np.uint8).reshape(h.shape[0], -1)
+
+
+def encode_bf16(x: np.ndarray) -> np.ndarray:
+    """round to nearest even on the upper 16 bits"""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    h = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return h.view(np.uint8).reshape(h.shape[0], -1)
 
 
 def encode_mxfp4(x: np.ndarray) -> np.ndarray:
@@ -153,7 +170,8 @@ def encode_q6_K(x: np.ndarray) -> np.ndarray:
     return out.reshape(m, -1)
 
 
-ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K, MXFP4: encode_mxfp4}
+ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K, MXFP4: encode_mxfp4,
+            F32: encode_f32, F16: encode_f16, BF16: encode_bf16}
 
 
 def weights(ggml_type: int, m: int, k: int, seed: int, std: float = 0.02, chunk_rows: int = 2048) -> np.ndarray:

@@ -52,6 +52,11 @@ CASES = [
     (Q6_K, 4096, 14336, 512, 200, False),  # K slices would need workspace: falls back to the 128-row kernel without it
     (Q4_K, 14336, 4096, 4, 3, True),       # a few columns on a large matrix: the workgroups quantize x, no scratch
     (Q4_K, 4096, 14336, 8, 5, True),       # the same kernel on planes in the static scratch
+    (1, 512, 4096, 8, 3, True),            # F16 weights at a few columns: no scratch (the activations are converted into LDS)
+    (30, 384, 2048, 200, 64, True),        # BF16 on the tiles: the converted activations in the static scratch
+    (0, 384, 2048, 200, 40, True),         # F32 on the tiles: no conversion, no scratch
+    (13, 256, 2048, 70, 5, False),         # Q5_K: [x | x] at the end of the static scratch, the Q8_K planes in front of it
+    (39, 128, 2880, 40, 3, True),          # MXFP4 with rows padded to 3072: [x | 0] at the end of the static scratch
 ]
 
 
