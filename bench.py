@@ -443,6 +443,58 @@ def main() -> int:
         for label, t in (("Q4_0", Q4_0), ("Q8_0", Q8_0)):
             tm, _ = time_mulmat(t, 4096, 4096, 512, 6)
             other[f"{label} GEMM 4096x4096 B=512"] = {"us": round(tm * 1e6, 1), "TOPS": round(2.0 * 512 * 4096 * 4096 / tm / 1e12, 1)}
+        # every Mulmat of one decoded token of a Llama-3-8B-shaped model in the Q4_K_M mixture (attn_v and ffn_down in Q6_K in
+        # half of the layers, the output head in Q6_K): q + k + v in one call, o, gate + up in one call, down, per layer, each
+        # launch reading what the one before wrote (the dependency chain of a real decode; attention, norms and the
+        # gating between the products are not part of the path and not run); weights distinct per layer, 4.6 GB in all
+        if len(pool) >= 32:
+            def tiled(t, m, k, seed, shift):
+                rows = min(m, 2048)
+                return np.roll(np.tile(synth.weights(t, rows, k, seed=seed), ((m + rows - 1) // rows, 1))[:m], shift, axis=0)
+            att = []
+            for li in range(32):
+                more = li % 2 == 0  # the layers the mixture gives more bits
+                att.append({"q": ctx.upload(Q4_K, tiled(Q4_K, 4096, 4096, 1301, 7 * li), 4096, 4096),
+                            "k": ctx.upload(Q4_K, tiled(Q4_K, 1024, 4096, 1302, 7 * li), 4096, 1024),
+                            "v": ctx.upload(Q6_K if more else Q4_K, tiled(Q6_K if more else Q4_K, 1024, 4096, 1303, 7 * li), 4096, 1024),
+                            "o": ctx.upload(Q4_K, tiled(Q4_K, 4096, 4096, 1304, 7 * li), 4096, 4096),
+                            "down6": ctx.upload(Q6_K, tiled(Q6_K, FFN_K, FFN_M, 1305, 7 * li), FFN_M, FFN_K) if more else None})
+            head = ctx.upload(Q6_K, tiled(Q6_K, 128256, 4096, 1306, 0), 4096, 128256)
+            hid = torch.randn(1, 4096, generator=g, dtype=torch.float32).to(dev)
+            yq = torch.empty(1, 4096, dtype=torch.float32, device=dev)
+            yk = torch.empty(1, 1024, dtype=torch.float32, device=dev)
+            yv = torch.empty(1, 1024, dtype=torch.float32, device=dev)
+            yo = torch.empty(1, 4096, dtype=torch.float32, device=dev)
+            yg = torch.empty(1, FFN_M, dtype=torch.float32, device=dev)
+            yu = torch.empty(1, FFN_M, dtype=torch.float32, device=dev)
+            yl = torch.empty(1, 128256, dtype=torch.float32, device=dev)
+
+            def token():
+                for li in range(32):
+                    a, f = att[li], pool[li]
+                    ctx.mulmat_multi_device([a["q"], a["k"], a["v"]], hid.data_ptr(), 1, [yq.data_ptr(), yk.data_ptr(), yv.data_ptr()])
+                    ctx.mulmat_device(a["o"], yq.data_ptr(), 1, yo.data_ptr())
+                    ctx.mulmat_multi_device([f["gate"], f["up"]], yo.data_ptr(), 1, [yg.data_ptr(), yu.data_ptr()])
+                    ctx.mulmat_device(a["down6"] or f["down"], yg.data_ptr(), 1, hid.data_ptr())
+                ctx.mulmat_device(head, hid.data_ptr(), 1, yl.data_ptr())
+
+            token()
+            token()
+            tm = timed(token, 5) / 5
+            used = [head]
+            for li in range(32):
+                a, f = att[li], pool[li]
+                used += [a["q"], a["k"], a["v"], a["o"], f["gate"], f["up"], a["down6"] or f["down"]]
+            tok_bytes = sum(wt.gguf_bytes for wt in used)
+            other["Llama-3-8B-shaped Q4_K_M token: all Mulmat calls of a decode step (32 layers + head), one after the other"] = {
+                "us": round(tm * 1e6, 1), "launch_groups": 32 * 4 + 1, "weight_GB": round(tok_bytes / 1e9, 3),
+                "GB/s": round(tok_bytes / tm / 1e9, 1), "frac_of_hbm_peak": round(tok_bytes / tm / 1e9 / HBM_PEAK_GBS, 4),
+                "tokens/s_if_nothing_else_ran": round(1.0 / tm, 1)}
+            for a in att:
+                for wt in a.values():
+                    if wt is not None:
+                        wt.free()
+            head.free()
         # Q5_K (the tensors the Q4_K_S mixture raises): kept as a Q4_K tensor of rows twice as long
         for label, m, k, ns, copies in (("Q5_K v_proj 1024x4096", 1024, 4096, (1, 4), 40), ("Q5_K ffn_down 4096x14336", 4096, 14336, (1, 4), 10)):
             for n in ns:
