@@ -156,8 +156,10 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      through, the expert-indexed ones included, when k is a multiple of 256.  Otherwise (k = 2880) its rows are
  *      kept padded with zero blocks to the next multiple of 256 and the library pads the activation rows likewise
  *      inside mi_qmm_mulmat, _path, _noalloc, _multi and mi_qmm_mulmat_id; the other entry points then return
- *      MI_QMM_ERR_UNSUPPORTED.  A scale byte above 146 is MI_QMM_ERR_UNSUPPORTED; blocks with a scale byte below
- *      104 (weights under 7.2e-7) are kept as zeros.
+ *      MI_QMM_ERR_UNSUPPORTED.  The tensor is also kept in its own layout, which the streaming kernels (one or
+ *      two activation rows, a few pairs per expert) read at half the bytes.  A scale byte above 146 is
+ *      MI_QMM_ERR_UNSUPPORTED; blocks with a scale byte below 104 (weights under 7.2e-7) are zeros in the Q8_0
+ *      planes (the matrix-core kernels) and exact in the streaming kernels.
  *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
 int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
                          int64_t m, int src_location, mi_qmm_weight **out);

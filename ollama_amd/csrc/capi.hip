@@ -74,6 +74,10 @@ struct mi_qmm_weight {
     bool repeat = false;  // [x | x] rather than [x | 0]
     int64_t k_user = 0;
     int file_type = -1;  // the ggml type the tensor had in the file, where dev.type is another (Q5_K, MXFP4); -1: dev.type
+    // MXFP4: the tensor once more in its own layout (type T_MXFP4, same K and M as dev), which the streaming kernels read at
+    // half the bytes of the Q8_0 planes the matrix-core kernels multiply
+    bool has_native = false;
+    DevWeight native{};
 };
 
 struct mi_qmm_gguf {
@@ -343,7 +347,11 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; break;  // a Q4_K tensor of rows twice as long
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
-    case T_MXFP4: s0 = (size_t)(m * align_up((size_t)k, 256)); sd = (size_t)(m * (align_up((size_t)k, 256) / QK)) * 2; break;  // kept as Q8_0 planes
+    case T_MXFP4: {  // Q8_0 planes (p0, d), and the tensor as it is (p1: nibbles, p2: scale bytes)
+        const size_t kp = align_up((size_t)k, 256);
+        s0 = (size_t)m * kp; sd = (size_t)m * (kp / QK) * 2; s1 = (size_t)m * (kp / QK) * 16; s2 = (size_t)m * (kp / QK) * 2;
+        break;
+    }
     case T_Q6_K: s0 = (size_t)(m * (k / 2)); s1 = (size_t)(m * (k / 4)); s2 = (size_t)(m * (k / 16));
                  sd = (size_t)(m * (k / QKK)) * 2; break;
     }
@@ -370,6 +378,10 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
         // rows of a whole number of 256-element steps (2880 -> 3072): the matrix-core kernels of the 32-element formats want that
         w->dev.type = T_Q8_0; w->file_type = T_MXFP4; w->dev.K = (int64_t)align_up((size_t)k, 256);
         if (w->dev.K != k) { w->expand = true; w->k_user = k; }
+        w->has_native = true;
+        w->native = w->dev;
+        w->native.type = T_MXFP4; w->native.p0 = b + o1; w->native.d = (const uint16_t *)(b + o2); w->native.p1 = w->native.p2 = nullptr;
+        w->dev.p1 = w->dev.p2 = nullptr;
     }
 
     void *staging = nullptr;
@@ -402,6 +414,10 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
             : type == T_MXFP4 ? launch_relayout_mxfp4(src, k, w->dev.K, m, b + o0, (uint16_t *)(b + od), bad, ctx->stream)
                               : launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
         if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
+        if (type == T_MXFP4) {
+            e = launch_relayout_mxfp4_native(src, k, w->dev.K, m, b + o1, (uint16_t *)(b + o2), ctx->stream);
+            if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
+        }
         if (bad) {
             int flag = 0;
             e = hipMemcpyAsync(&flag, bad, sizeof(int), hipMemcpyDeviceToHost, ctx->stream);
@@ -522,6 +538,14 @@ int mi_qmm_quantize_weights(mi_qmm_ctx *ctx, int ggml_type, const float *x, int6
 // ---- the product ------------------------------------------------------------------------------------
 namespace {
 
+// The tensor the streaming GEMV reads for a weight: an MXFP4 weight's own layout (half the bytes of its Q8_0 planes)
+// where the kernel takes that type at this shape too.
+const DevWeight &gemv_dev(const mi_qmm_weight *w, int ncols, bool f32_x) {
+    if (!w->has_native || w->native.K > gemv_max_k(T_MXFP4)) return w->dev;
+    if (f32_x && !gemv_f32_supported(T_MXFP4, w->native.K, w->native.M, ncols)) return w->dev;
+    return w->native;
+}
+
 // From this many activation columns up a product below the GEMM's batch goes to a matrix-core skinny
 // kernel instead of the streaming GEMV (measured crossovers on MI355X: the GEMV pays one v_dot4 pass
 // per column).
@@ -634,7 +658,7 @@ int run_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const DevAct &a, float 
     default:
         for (int64_t c0 = 0; c0 < n; c0 += 8) {
             const int nc = (int)(n - c0 < 8 ? n - c0 : 8);
-            HIP_TRY(launch_gemv(w->dev, a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
+            HIP_TRY(launch_gemv(gemv_dev(w, nc, false), a, (int)c0, nc, dy, M, ctx->num_cus, ctx->stream));
         }
     }
     return MI_QMM_OK;
@@ -797,7 +821,7 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
     if (route == MI_QMM_ROUTE_GEMV_F32) {
         // decode: one launch, the GEMV quantizes x in its prologue
         float *ys[1] = {dy};
-        HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
+        HIP_TRY(launch_gemv_f32_multi(&gemv_dev(w, (int)n, true), ys, 1, dx, (int)n, ctx->num_cus, ctx->stream));
     } else if (route == MI_QMM_ROUTE_DEEP_F32) {
         // a few columns on a large Q4_K matrix: one launch, the workgroups quantize x themselves
         float *ys[1] = {dy};
@@ -848,7 +872,7 @@ static int noalloc_core(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x,
     if (n <= 8 && !wants_skinny(w->dev.type, K, M, n, ctx->num_cus) && gemv_f32_supported(w->dev.type, K, M, (int)n)) {
         // decode: the GEMV quantizes x in its own prologue, into LDS -- no scratch at all
         float *ys[1] = {y};
-        HIP_TRY(launch_gemv_f32_multi(&w->dev, ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
+        HIP_TRY(launch_gemv_f32_multi(&gemv_dev(w, (int)n, true), ys, 1, x, (int)n, ctx->num_cus, ctx->stream));
         return MI_QMM_OK;
     }
     if (deep_f32_one(ctx, w, n)) {
@@ -1333,8 +1357,11 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
             HIP_TRY(launch_skinny_id(w2->dev, n_expert, a, dids, n_used, (int)n_tokens, b_cols, dy2, (int *)ctx->ws_buf,
                                      ctx->num_cus, ctx->stream));
     } else {
-        HIP_TRY(launch_gemv_id(w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
-                               (int *)ctx->ws_buf, ctx->stream, w2 ? &w2->dev : nullptr, dy2,
+        // MXFP4 stacks: the streaming kernel reads them in their own layout where it takes that type at this shape
+        const bool native = w->has_native && (!w2 || w2->has_native) && K <= gemv_max_k(T_MXFP4) &&
+                            (!fused || gemv_id_f32_supported(T_MXFP4, K, M, pairs, n_expert, pr.kind == PRODUCE_SWIGLU));
+        HIP_TRY(launch_gemv_id(native ? w->native : w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
+                               (int *)ctx->ws_buf, ctx->stream, w2 ? (native ? &w2->native : &w2->dev) : nullptr, dy2,
                                fused && pr.kind == PRODUCE_SWIGLU ? pr.aux : nullptr));
     }
     if (location == MI_QMM_HOST) {

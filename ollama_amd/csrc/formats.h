@@ -32,7 +32,8 @@ constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q5_K_BYTES = 1
 //          nibble 8 where the bit is set, block scale 2 d -- so that against the activations repeated, [x | x], every
 //          Q4_K kernel computes sum sc (q4 + 16 h) y exactly (see relayout.hip)
 //   MXFP4: stored as the Q8_0 planes with the same dot products (type = T_Q8_0): the doubled E2M1 values as int8, the scale
-//          2^(e - 128) as the fp16 block scale (see relayout.hip)
+//          2^(e - 128) as the fp16 block scale (see relayout.hip) -- what the matrix-core kernels multiply -- and once more as
+//          it is (type = T_MXFP4: p0 = nibble plane [M][K/32][16], d = the scale bytes, 16 bits each) for the streaming kernels
 //   F32, F16, BF16 : p0 = the rows unchanged, [M][K] elements
 // Byte order inside each plane is the GGUF order; only the interleaving of fields is undone.
 struct DevWeight {

@@ -238,6 +238,72 @@ struct PolQ4_0 {
     }
 };
 
+// MXFP4 in its own 17 bytes per block (18 on the device: the layout of Q4_0, nibble plane + a 16-bit plane that holds the
+// E8M0 scale byte).  A nibble is an E2M1 code: magnitude index in the low three bits, sign in the fourth; ggml multiplies
+// the doubled values 0 1 2 3 4 6 8 12 as integers and scales the block sum by 2^(e - 128) d_y.  The eight magnitudes are a
+// byte table in two registers (v_perm_b32 looks up four codes per instruction), the signs split every dword into the bytes
+// that count positively and those that count negatively.  No scale byte is out of range here.
+struct PolMXFP4 {
+    static constexpr int PLANES = 2;
+    static constexpr int F32_WAVES_ONE_SEG = 16;
+    static constexpr int SEG = 2048;  // 64 blocks, one per lane
+    static constexpr int ACT_BLK = QK, ACT_BSUM = QK;
+    static constexpr bool USES_BSUMS = false;
+    static constexpr bool HEAVY = false;
+    struct Geo { int64_t qrow, drow; int blk; bool live; };
+    struct Act { int q[8]; float d; };
+    struct Raw { uint4 qv; unsigned e; };
+
+    static __device__ __forceinline__ Geo geo(const DevWeight &w, int seg, int lane) {
+        Geo g;
+        g.blk = seg * 64 + lane;
+        g.live = (int64_t)g.blk * QK < w.K;
+        if (!g.live) g.blk = 0;
+        g.qrow = w.K / 2;
+        g.drow = w.K / QK;
+        return g;
+    }
+    template <class AV>
+    static __device__ __forceinline__ void load_act(const AV &a, int n, int seg, int lane, const Geo &g, Act &r) {
+        const int keep = g.live ? -1 : 0;
+        const int4 *q = reinterpret_cast<const int4 *>(a.qs + (int64_t)n * a.K + (int64_t)g.blk * QK);
+        const int4 lo = q[0], hi = q[1];
+        const float dd = a.d[(int64_t)n * (a.K / QK) + g.blk];
+        r.q[0] = lo.x & keep; r.q[1] = lo.y & keep; r.q[2] = lo.z & keep; r.q[3] = lo.w & keep;
+        r.q[4] = hi.x & keep; r.q[5] = hi.y & keep; r.q[6] = hi.z & keep; r.q[7] = hi.w & keep;
+        r.d = g.live ? dd : 0.f;
+    }
+    static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
+        Raw r;
+        r.qv = ld16(w.p0 + row * g.qrow + (int64_t)g.blk * 16);
+        r.e = w.d[row * g.drow + g.blk];
+        return r;
+    }
+    // the four codes of a dword (one per byte, 0..15) against four activation bytes: sum kvalue * y
+    static __device__ __forceinline__ int dot_codes(unsigned codes, int y, int acc) {
+        const unsigned mag = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, codes & 0x07070707u);
+        const unsigned s1 = (codes >> 3) & 0x01010101u, neg = (s1 << 8) - s1;  // 0xFF in the bytes of negative codes
+        acc = dot4((int)(mag & ~neg), y, acc);
+        return acc - dot4((int)(mag & neg), y, 0);
+    }
+    template <int NC>
+    static __device__ __forceinline__ void dot(const Raw &r, const Geo &, const Act (&a)[NC], float (&acc)[NC]) {
+        // 2^(e - 128): the exponent field e - 1, or a subnormal for the two smallest scale bytes
+        const float dw = __builtin_bit_cast(float, r.e < 2 ? 0x00200000u << r.e : (r.e - 1) << 23);
+        const unsigned v[4] = {r.qv.x, r.qv.y, r.qv.z, r.qv.w};
+#pragma unroll
+        for (int n = 0; n < NC; n++) {
+            int s = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                s = dot_codes(v[i] & 0x0f0f0f0fu, a[n].q[i], s);
+                s = dot_codes((v[i] >> 4) & 0x0f0f0f0fu, a[n].q[4 + i], s);
+            }
+            acc[n] += (float)s * (a[n].d * dw);
+        }
+    }
+};
+
 struct PolQ8_0 {
     static constexpr int PLANES = 2;  // planes of the device layout a row is read from
     static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
@@ -1360,6 +1426,7 @@ int64_t gemv_max_k(int type) {
     switch (type) {
     case T_Q8_0: return 32 * (int64_t)PolQ8_0::SEG;
     case T_Q4_0: return 32 * (int64_t)PolQ4_0::SEG;
+    case T_MXFP4: return 32 * (int64_t)PolMXFP4::SEG;
     case T_Q4_K: return 32 * (int64_t)PolQ4K::SEG;
     case T_Q6_K: return 32 * (int64_t)PolQ6K::SEG;
     default: return 0;
@@ -1381,6 +1448,7 @@ hipError_t dispatch(const DevWeight *ws, float *const *ys, int count, const DevA
     case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
+    case T_MXFP4: return a.type == T_Q8_0 ? launch_type<PolMXFP4>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     case T_Q8_0: return a.type == T_Q8_0 ? launch_type<PolQ8_0>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
@@ -1424,6 +1492,7 @@ bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
     case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, ncols, true, p);
     case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, ncols, true, p);
     case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, ncols, true, p);
+    case T_MXFP4: return make_thin_plan<PolMXFP4>(K, total_m, ncols, true, p);
     case T_Q8_0: return make_thin_plan<PolQ8_0>(K, total_m, ncols, true, p);
     default: return false;
     }
@@ -1504,6 +1573,7 @@ bool gemv_pair_supported(int type, int64_t K, int64_t M, bool rms) {
     case T_Q4_K: return pair_plan<PolQ4K>(K, M, rms, p);
     case T_Q6_K: return pair_plan<PolQ6K>(K, M, rms, p);
     case T_Q4_0: return pair_plan<PolQ4_0>(K, M, rms, p);
+    case T_MXFP4: return pair_plan<PolMXFP4>(K, M, rms, p);
     case T_Q8_0: return pair_plan<PolQ8_0>(K, M, rms, p);
     default: return false;
     }
@@ -1520,6 +1590,7 @@ hipError_t launch_gemv_pair_f32(const DevWeight &wg, const DevWeight &wu, const 
     case T_Q4_K: return launch_pair_type<PolQ4K>(wg, wu, x, h, pr, s);
     case T_Q6_K: return launch_pair_type<PolQ6K>(wg, wu, x, h, pr, s);
     case T_Q4_0: return launch_pair_type<PolQ4_0>(wg, wu, x, h, pr, s);
+    case T_MXFP4: return launch_pair_type<PolMXFP4>(wg, wu, x, h, pr, s);
     case T_Q8_0: return launch_pair_type<PolQ8_0>(wg, wu, x, h, pr, s);
     default: return hipErrorInvalidValue;
     }
@@ -1532,6 +1603,7 @@ bool gemv_produce_supported(int type, int64_t K, int64_t total_m) {
     case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, 1, true, p, true);
     case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, 1, true, p, true);
     case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, 1, true, p, true);
+    case T_MXFP4: return make_thin_plan<PolMXFP4>(K, total_m, 1, true, p, true);
     case T_Q8_0: return make_thin_plan<PolQ8_0>(K, total_m, 1, true, p, true);
     default: return false;
     }
@@ -2105,6 +2177,7 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
     case T_Q4_K: ok = make_thin_plan<PolQ4K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4K>(K, 1); break;
     case T_Q6_K: ok = make_thin_plan<PolQ6K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ6K>(K, 1); break;
     case T_Q4_0: ok = make_thin_plan<PolQ4_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4_0>(K, 1); break;
+    case T_MXFP4: ok = make_thin_plan<PolMXFP4>(K, pairs * M, 1, false, p); act = thin_act_lds<PolMXFP4>(K, 1); break;
     case T_Q8_0: ok = make_thin_plan<PolQ8_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ8_0>(K, 1); break;
     default: break;
     }
@@ -2127,6 +2200,7 @@ hipError_t launch_gemv_id_pair(const DevWeight &wg, const DevWeight &wu, int n_e
     case T_Q4_K: return launch_id_pair<PolQ4K>(ia, xf, s);
     case T_Q6_K: return launch_id_pair<PolQ6K>(ia, xf, s);
     case T_Q4_0: return launch_id_pair<PolQ4_0>(ia, xf, s);
+    case T_MXFP4: return launch_id_pair<PolMXFP4>(ia, xf, s);
     case T_Q8_0: return launch_id_pair<PolQ8_0>(ia, xf, s);
     default: return hipErrorInvalidValue;
     }
@@ -2149,6 +2223,7 @@ hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, con
     case T_Q4_K: return a.type == T_Q8_K ? launch_id_type<PolQ4K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     case T_Q6_K: return a.type == T_Q8_K ? launch_id_type<PolQ6K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     case T_Q4_0: return a.type == T_Q8_0 ? launch_id_type<PolQ4_0>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
+    case T_MXFP4: return a.type == T_Q8_0 ? launch_id_type<PolMXFP4>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     case T_Q8_0: return a.type == T_Q8_0 ? launch_id_type<PolQ8_0>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }

@@ -114,6 +114,20 @@ __global__ void relayout_mxfp4_kernel(const uint8_t *__restrict__ src, int64_t M
     }
 }
 
+// MXFP4 as it is, for the streaming kernels: the 16 nibble bytes of every block in one plane, its scale byte (widened to 16
+// bits) in another; rows padded with zero blocks (scale byte 0, codes 0) from nb_in to nb_out blocks.
+__global__ void relayout_mxfp4_native_kernel(const uint8_t *__restrict__ src, int64_t M, int nb_in, int nb_out, uint8_t *__restrict__ qs,
+                                             uint16_t *__restrict__ e) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M * nb_out * 16) return;
+    const int64_t blk = i >> 4, row = blk / nb_out;
+    const int bi = (int)(blk - row * nb_out), j = (int)(i & 15);
+    const bool pad = bi >= nb_in;
+    const uint8_t *b = src + (row * nb_in + (pad ? 0 : bi)) * 17;
+    qs[blk * 16 + j] = pad ? 0 : b[1 + j];
+    if (j == 0) e[blk] = pad ? 0 : b[0];
+}
+
 // out [n][k_out] from x [n][k_in] (in float4 units): the row, then -- repeat (k_out = 2 k_in): the row once more; else zeros
 __global__ void expand_rows_kernel(const float4 *__restrict__ x, float4 *__restrict__ out, int64_t k4_in, int64_t k4_out, int64_t n, bool repeat) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < k4_out * n; i += (int64_t)gridDim.x * blockDim.x) {
@@ -141,6 +155,15 @@ hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t K_out, 
     const int64_t n = M * (K_out / QK) * 16;
     if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
     relayout_mxfp4_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QK), (int)(K_out / QK), (int8_t *)qs, d, bad);
+    return hipGetLastError();
+}
+
+hipError_t launch_relayout_mxfp4_native(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *e, hipStream_t s) {
+    if (K * M == 0) return hipSuccess;
+    if (K % QK || K_out % QK || K_out < K) return hipErrorInvalidValue;
+    const int64_t n = M * (K_out / QK) * 16;
+    if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
+    relayout_mxfp4_native_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QK), (int)(K_out / QK), qs, e);
     return hipGetLastError();
 }
 

@@ -46,22 +46,30 @@ def test_mxfp4_against_the_oracle(ctx, m, k, n):
 
 def test_mxfp4_scales_at_the_edges_of_what_the_planes_hold(ctx):
     """e = 104 (a subnormal half), 113 / 114 (the last subnormal, the first normal), 143 (the largest half), 144 .. 146
-    (the integers shifted instead): exact; below 104 the block is zero; above 146 the upload is refused"""
+    (the integers shifted instead): exact on every kernel; below 104 the matrix-core kernels see a zero block; above 146 the
+    upload is refused"""
     k, m = 64, 16
     x = np.random.default_rng(1).integers(-127, 128, (2, k)).astype(np.float32)
     x[:, ::32] = 127
+    x8 = np.tile(x, (4, 1))
     for e in (104, 105, 113, 114, 127, 128, 143, 144, 146):
         raw = _random_rows(m, k, seed=e).reshape(m, 2, 17)
         raw[..., 0] = e
         W = ctx.upload(MXFP4, raw.reshape(m, -1), k, m)
-        y = ctx.mulmat(W, x)
+        y, y8 = ctx.mulmat(W, x), ctx.mulmat(W, x8)   # the streaming kernel (the tensor's own layout), the matrix cores (Q8_0 planes)
         W.free()
         w = npref.dequant(MXFP4, raw.reshape(-1)).reshape(m, k)
         assert np.array_equal(y, (x.astype(np.float64) @ w.T).astype(np.float32)), e   # integers times a power of two
+        assert np.array_equal(y8, (x8.astype(np.float64) @ w.T).astype(np.float32)), e
+    # below 104 the Q8_0 planes hold a zero block (weights under 7.2e-7); the streaming kernels read the tensor in its own
+    # layout and still multiply it exactly
     raw = _random_rows(m, k, seed=3).reshape(m, 2, 17)
     raw[..., 0] = 100
     W = ctx.upload(MXFP4, raw.reshape(m, -1), k, m)
-    assert not ctx.mulmat(W, x).any()
+    w = npref.dequant(MXFP4, raw.reshape(-1)).reshape(m, k)
+    assert ctx.route(W, 2) == "gemv_f32" and np.array_equal(ctx.mulmat(W, x), (x.astype(np.float64) @ w.T).astype(np.float32))
+    x8 = np.tile(x, (4, 1))
+    assert ctx.route(W, 8) == "skinny32" and not ctx.mulmat(W, x8).any()
     W.free()
     raw[3, 1, 0] = 147
     with pytest.raises(qmm.QmmError) as err:
