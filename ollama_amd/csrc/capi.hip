@@ -75,7 +75,8 @@ struct mi_qmm_weight {
     int64_t k_user = 0;
     int file_type = -1;  // the ggml type the tensor had in the file, where dev.type is another (Q5_K, MXFP4); -1: dev.type
     // MXFP4: the tensor once more in its own layout (type T_MXFP4, same K and M as dev), which the streaming kernels read at
-    // half the bytes of the Q8_0 planes the matrix-core kernels multiply
+    // half the bytes of the Q8_0 planes the matrix-core kernels multiply.  Q5_K: the blocks as they are (type T_Q5_K, K = k_user),
+    // for the streaming kernel at one or two activation rows -- against x itself, not [x | x]
     bool has_native = false;
     DevWeight native{};
 };
@@ -344,7 +345,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     size_t s0 = 0, s1 = 0, s2 = 0, sd = 0;
     switch (type) {
     case T_Q4_K: case T_F32: case T_F16: case T_BF16: s0 = total; break;
-    case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; break;  // a Q4_K tensor of rows twice as long
+    case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; s1 = total; break;  // a Q4_K tensor of rows twice as long; the blocks as they are
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_MXFP4: {  // Q8_0 planes (p0, d), and the tensor as it is (p1: nibbles, p2: scale bytes)
@@ -373,7 +374,14 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     w->dev.p2 = s2 ? b + o2 : nullptr;
     w->dev.d = sd ? (const uint16_t *)(b + od) : nullptr;
     w->dev.K = k; w->dev.M = m; w->dev.type = type;
-    if (type == T_Q5_K) { w->expand = w->repeat = true; w->k_user = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K; }
+    if (type == T_Q5_K) {
+        w->expand = w->repeat = true; w->k_user = k; w->dev.K = 2 * k; w->dev.type = T_Q4_K; w->file_type = T_Q5_K;
+        // ... and the blocks as they are, which the streaming kernel reads at one or two activation rows (176 instead of 288 B)
+        w->has_native = true;
+        w->native = w->dev;
+        w->native.type = T_Q5_K; w->native.K = k; w->native.p0 = b + o1; w->native.p1 = nullptr;
+        w->dev.p1 = nullptr;
+    }
     if (type == T_MXFP4) {
         // rows of a whole number of 256-element steps (2880 -> 3072): the matrix-core kernels of the 32-element formats want that
         w->dev.type = T_Q8_0; w->file_type = T_MXFP4; w->dev.K = (int64_t)align_up((size_t)k, 256);
@@ -417,6 +425,10 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
         if (type == T_MXFP4) {
             e = launch_relayout_mxfp4_native(src, k, w->dev.K, m, b + o1, (uint16_t *)(b + o2), ctx->stream);
             if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);
+        }
+        if (type == T_Q5_K) {
+            e = hipMemcpyAsync(b + o1, src, total, hipMemcpyDeviceToDevice, ctx->stream);
+            if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemcpy(weight)", e);
         }
         if (bad) {
             int flag = 0;
@@ -541,7 +553,7 @@ namespace {
 // The tensor the streaming GEMV reads for a weight: an MXFP4 weight's own layout (half the bytes of its Q8_0 planes)
 // where the kernel takes that type at this shape too.
 const DevWeight &gemv_dev(const mi_qmm_weight *w, int ncols, bool f32_x) {
-    if (!w->has_native || w->native.K > gemv_max_k(T_MXFP4)) return w->dev;
+    if (!w->has_native || w->native.type != T_MXFP4 || w->native.K > gemv_max_k(T_MXFP4)) return w->dev;
     if (f32_x && !gemv_f32_supported(T_MXFP4, w->native.K, w->native.M, ncols)) return w->dev;
     return w->native;
 }
@@ -765,8 +777,31 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         // the tensor of longer rows that stands for this one, against the expanded activations ([x | x] or [x | 0])
         mi_qmm_weight lo = *w;
         lo.expand = false;
+        // Q5_K at one or two activation rows: the streaming kernel on the blocks as they are, x quantized in its prologue
+        const bool q5_gemv = w->repeat && w->has_native && n >= 1 && n <= 2 && path != MI_QMM_PATH_GEMM &&
+                             gemv_f32_supported(T_Q5_K, w->k_user, w->dev.M, (int)n);
+        if (path == MI_QMM_PATH_QUERY && q5_gemv) return MI_QMM_ROUTE_GEMV_F32;
         if (path == MI_QMM_PATH_QUERY || n == 0) return mi_qmm_mulmat_path(ctx, &lo, x, n, y, location, path);
         if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
+        if (q5_gemv) {
+            const size_t xb5 = (size_t)(n * w->k_user) * 4, yb5 = (size_t)(n * w->dev.M) * 4;
+            const float *dx5 = x;
+            float *dy5 = y;
+            if (location == MI_QMM_HOST) {
+                const size_t yoff = align_up(xb5, 256);
+                if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, yoff + yb5))) return rc;
+                dx5 = (const float *)ctx->io_buf;
+                dy5 = (float *)((char *)ctx->io_buf + yoff);
+                HIP_TRY(hipMemcpyAsync((void *)dx5, x, xb5, hipMemcpyHostToDevice, ctx->stream));
+            }
+            float *ys5[1] = {dy5};
+            HIP_TRY(launch_gemv_f32_multi(&w->native, ys5, 1, dx5, (int)n, ctx->num_cus, ctx->stream));
+            if (location == MI_QMM_HOST) {
+                HIP_TRY(hipMemcpyAsync(y, dy5, yb5, hipMemcpyDeviceToHost, ctx->stream));
+                HIP_TRY(hipStreamSynchronize(ctx->stream));
+            }
+            return MI_QMM_OK;
+        }
         const size_t xb = (size_t)(n * w->k_user) * 4, xxb = (size_t)(n * w->dev.K) * 4, yb = (size_t)(n * w->dev.M) * 4;
         const size_t o_raw = align_up(xxb, 256), o_y = o_raw + align_up(xb, 256);
         if ((rc = reserve(ctx, &ctx->dup_buf, &ctx->dup_cap, location == MI_QMM_HOST ? o_y + yb : xxb))) return rc;
@@ -854,6 +889,11 @@ static int noalloc_core(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x,
     if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
     if (n > INT32_MAX) return fail(MI_QMM_ERR_UNSUPPORTED, "n too large");
     if (w->expand) {
+        if (w->repeat && w->has_native && n <= 2 && gemv_f32_supported(T_Q5_K, w->k_user, w->dev.M, (int)n)) {
+            float *ys5[1] = {y};  // Q5_K at one or two rows: the streaming kernel on the blocks as they are, no scratch
+            HIP_TRY(launch_gemv_f32_multi(&w->native, ys5, 1, x, (int)n, ctx->num_cus, ctx->stream));
+            return MI_QMM_OK;
+        }
         // the expanded activations at the end of the scratch, the quantized planes of the product in front of them
         mi_qmm_weight lo = *w;
         lo.expand = false;
@@ -1358,7 +1398,7 @@ int mulmat_id_impl(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const mi_qmm_weight 
                                      ctx->num_cus, ctx->stream));
     } else {
         // MXFP4 stacks: the streaming kernel reads them in their own layout where it takes that type at this shape
-        const bool native = w->has_native && (!w2 || w2->has_native) && K <= gemv_max_k(T_MXFP4) &&
+        const bool native = w->has_native && w->native.type == T_MXFP4 && (!w2 || w2->has_native) && K <= gemv_max_k(T_MXFP4) &&
                             (!fused || gemv_id_f32_supported(T_MXFP4, K, M, pairs, n_expert, pr.kind == PRODUCE_SWIGLU));
         HIP_TRY(launch_gemv_id(native ? w->native : w->dev, n_expert, a, fused ? dx : nullptr, dids, n_used, (int)n_tokens, b_cols, dy,
                                (int *)ctx->ws_buf, ctx->stream, w2 ? (native ? &w2->native : &w2->dev) : nullptr, dy2,

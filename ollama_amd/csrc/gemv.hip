@@ -177,6 +177,86 @@ struct PolQ4K {
     }
 };
 
+// Q5_K in its own 176-byte blocks (16 bytes of header, 32 of fifth bits, 128 of nibbles: every field 16-byte aligned).
+// As PolQ4K, plus the fifth bits: bit j of qh[l] belongs to element l of sub-block j, so lane c -- which owns sub-blocks 2c
+// and 2c + 1 -- takes bits 2c and 2c + 1 of all 32 bytes and adds 16 to the nibbles whose bit is set.
+struct PolQ5K {
+    static constexpr int PLANES = 1;
+    static constexpr int F32_WAVES_ONE_SEG = 16;
+    static constexpr int SEG = 4096;
+    static constexpr int ACT_BLK = QKK, ACT_BSUM = 16;
+    static constexpr bool USES_BSUMS = true;
+    static constexpr bool HEAVY = true;
+    struct Geo {
+        int64_t row_bytes;
+        int off, qoff, sh, hb;  // hb = 2c: the lane's first bit in the bytes of fifth bits
+        bool hi, live;
+    };
+    typedef PolQ4K::Act Act;
+    struct Raw { uint4 hdr, h0, h1, q0, q1; };
+
+    static __device__ __forceinline__ Geo geo(const DevWeight &w, int seg, int lane) {
+        Geo g;
+        const int sb = seg * 16 + (lane >> 2), c = lane & 3;
+        g.row_bytes = w.K / QKK * Q5_K_BYTES;
+        g.live = (int64_t)sb * QKK < w.K;
+        g.off = g.live ? sb * Q5_K_BYTES : 0;
+        g.qoff = g.off + 48 + 32 * c;
+        g.sh = 16 * (c & 1);
+        g.hb = 2 * c;
+        g.hi = c >= 2;
+        return g;
+    }
+    template <class AV>
+    static __device__ __forceinline__ void load_act(const AV &a, int n, int seg, int lane, const Geo &g, Act &r) {
+        PolQ4K::Geo g4;
+        g4.live = g.live;
+        PolQ4K::load_act(a, n, seg, lane, g4, r);
+    }
+    static __device__ __forceinline__ Raw load(const DevWeight &w, const Geo &g, int64_t row) {
+        Raw r;
+        const uint8_t *p = w.p0 + row * g.row_bytes;
+        r.hdr = ld16(p + g.off);
+        r.h0 = ld16(p + g.off + 16);
+        r.h1 = ld16(p + g.off + 32);
+        r.q0 = ld16(p + g.qoff);
+        r.q1 = ld16(p + g.qoff + 16);
+        return r;
+    }
+    template <int NC>
+    static __device__ __forceinline__ void dot(const Raw &r, const Geo &g, const Act (&a)[NC], float (&acc)[NC]) {
+        const float dw = h2f(r.hdr.x & 0xffff), dminw = h2f(r.hdr.x >> 16);
+        const unsigned ty = r.hdr.y >> g.sh, tz = r.hdr.z >> g.sh, tw = r.hdr.w >> g.sh;
+        const unsigned scA = ty & 0x3f3fu, mA = tz & 0x3f3fu;
+        const unsigned scB = (tw & 0x0f0fu) | ((ty >> 2) & 0x3030u);
+        const unsigned mB = ((tw >> 4) & 0x0f0fu) | ((tz >> 2) & 0x3030u);
+        const unsigned scp = g.hi ? scB : scA, mp = g.hi ? mB : mA;
+        const int sc_lo = scp & 0xff, sc_hi = scp >> 8, m_lo = mp & 0xff, m_hi = mp >> 8;
+        const unsigned v[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const unsigned hb[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+        int lo[8], hi[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const unsigned t = hb[i] >> g.hb;
+            lo[i] = (int)((v[i] & 0x0f0f0f0fu) | ((t & 0x01010101u) << 4));
+            hi[i] = (int)(((v[i] >> 4) & 0x0f0f0f0fu) | (((t >> 1) & 0x01010101u) << 4));
+        }
+#pragma unroll
+        for (int n = 0; n < NC; n++) {
+            int dl = 0, dh = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                dl = dot4(lo[i], a[n].lo[i], dl);
+                dh = dot4(hi[i], a[n].hi[i], dh);
+            }
+            const int isum = __mul24(sc_lo, dl) + __mul24(sc_hi, dh);
+            const int msum = __mul24(m_lo, a[n].s_lo) + __mul24(m_hi, a[n].s_hi);
+            acc[n] = __builtin_fmaf(dw * a[n].d, (float)isum, acc[n]);
+            acc[n] = __builtin_fmaf(-(dminw * a[n].d), (float)msum, acc[n]);
+        }
+    }
+};
+
 struct PolQ4_0 {
     static constexpr int PLANES = 2;  // planes of the device layout a row is read from
     static constexpr int F32_WAVES_ONE_SEG = 16;  // waves per workgroup when it quantizes one column of one-segment rows
@@ -1428,6 +1508,7 @@ int64_t gemv_max_k(int type) {
     case T_Q4_0: return 32 * (int64_t)PolQ4_0::SEG;
     case T_MXFP4: return 32 * (int64_t)PolMXFP4::SEG;
     case T_Q4_K: return 32 * (int64_t)PolQ4K::SEG;
+    case T_Q5_K: return 32 * (int64_t)PolQ5K::SEG;
     case T_Q6_K: return 32 * (int64_t)PolQ6K::SEG;
     default: return 0;
     }
@@ -1446,6 +1527,7 @@ hipError_t dispatch(const DevWeight *ws, float *const *ys, int count, const DevA
     if (ws[0].K < 1 || ws[0].K > gemv_max_k(ws[0].type) || a.K != ws[0].K) return hipErrorInvalidValue;
     switch (ws[0].type) {
     case T_Q4_K: return a.type == T_Q8_K ? launch_type<PolQ4K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
+    case T_Q5_K: return a.type == T_Q8_K ? launch_type<PolQ5K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     case T_Q6_K: return a.type == T_Q8_K ? launch_type<PolQ6K>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     case T_Q4_0: return a.type == T_Q8_0 ? launch_type<PolQ4_0>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
     case T_MXFP4: return a.type == T_Q8_0 ? launch_type<PolMXFP4>(ws, ys, count, a, xf, col0, ncols, num_cus, pr, s) : hipErrorInvalidValue;
@@ -1490,6 +1572,7 @@ bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
     Plan p;
     switch (type) {
     case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, ncols, true, p);
+    case T_Q5_K: return make_thin_plan<PolQ5K>(K, total_m, ncols, true, p);
     case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, ncols, true, p);
     case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, ncols, true, p);
     case T_MXFP4: return make_thin_plan<PolMXFP4>(K, total_m, ncols, true, p);
@@ -1509,7 +1592,7 @@ hipError_t launch_gemv_f32_multi(const DevWeight *ws, float *const *ys, int coun
     DevAct a{};  // only the geometry is read: the kernel quantizes x itself
     a.K = ws[0].K;
     a.N = ncols;
-    a.type = (ws[0].type == T_Q4_K || ws[0].type == T_Q6_K) ? T_Q8_K : T_Q8_0;
+    a.type = (ws[0].type == T_Q4_K || ws[0].type == T_Q5_K || ws[0].type == T_Q6_K) ? T_Q8_K : T_Q8_0;
     return dispatch(ws, ys, count, a, x, 0, ncols, num_cus, s, pr);
 }
 
@@ -1571,6 +1654,7 @@ bool gemv_pair_supported(int type, int64_t K, int64_t M, bool rms) {
     Plan p;
     switch (type) {
     case T_Q4_K: return pair_plan<PolQ4K>(K, M, rms, p);
+    case T_Q5_K: return pair_plan<PolQ5K>(K, M, rms, p);
     case T_Q6_K: return pair_plan<PolQ6K>(K, M, rms, p);
     case T_Q4_0: return pair_plan<PolQ4_0>(K, M, rms, p);
     case T_MXFP4: return pair_plan<PolMXFP4>(K, M, rms, p);
@@ -1588,6 +1672,7 @@ hipError_t launch_gemv_pair_f32(const DevWeight &wg, const DevWeight &wu, const 
     if (pr.kind != PRODUCE_NONE && pr.kind != PRODUCE_RMSNORM) return hipErrorInvalidValue;
     switch (wg.type) {
     case T_Q4_K: return launch_pair_type<PolQ4K>(wg, wu, x, h, pr, s);
+    case T_Q5_K: return launch_pair_type<PolQ5K>(wg, wu, x, h, pr, s);
     case T_Q6_K: return launch_pair_type<PolQ6K>(wg, wu, x, h, pr, s);
     case T_Q4_0: return launch_pair_type<PolQ4_0>(wg, wu, x, h, pr, s);
     case T_MXFP4: return launch_pair_type<PolMXFP4>(wg, wu, x, h, pr, s);
@@ -1601,6 +1686,7 @@ bool gemv_produce_supported(int type, int64_t K, int64_t total_m) {
     Plan p;
     switch (type) {
     case T_Q4_K: return make_thin_plan<PolQ4K>(K, total_m, 1, true, p, true);
+    case T_Q5_K: return make_thin_plan<PolQ5K>(K, total_m, 1, true, p, true);
     case T_Q6_K: return make_thin_plan<PolQ6K>(K, total_m, 1, true, p, true);
     case T_Q4_0: return make_thin_plan<PolQ4_0>(K, total_m, 1, true, p, true);
     case T_MXFP4: return make_thin_plan<PolMXFP4>(K, total_m, 1, true, p, true);
@@ -2175,6 +2261,7 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
     size_t act = 0;
     switch (type) {  // the plan of the launch: activation row plus the partial sums must fit in LDS
     case T_Q4_K: ok = make_thin_plan<PolQ4K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4K>(K, 1); break;
+    case T_Q5_K: ok = make_thin_plan<PolQ5K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ5K>(K, 1); break;
     case T_Q6_K: ok = make_thin_plan<PolQ6K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ6K>(K, 1); break;
     case T_Q4_0: ok = make_thin_plan<PolQ4_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4_0>(K, 1); break;
     case T_MXFP4: ok = make_thin_plan<PolMXFP4>(K, pairs * M, 1, false, p); act = thin_act_lds<PolMXFP4>(K, 1); break;
@@ -2198,6 +2285,7 @@ hipError_t launch_gemv_id_pair(const DevWeight &wg, const DevWeight &wu, int n_e
     ia.p0b = wu.p0; ia.p1b = wu.p1; ia.p2b = wu.p2; ia.db = wu.d; ia.yb = nullptr; ia.wgs_first = 0x7fffffff;
     switch (wg.type) {
     case T_Q4_K: return launch_id_pair<PolQ4K>(ia, xf, s);
+    case T_Q5_K: return launch_id_pair<PolQ5K>(ia, xf, s);
     case T_Q6_K: return launch_id_pair<PolQ6K>(ia, xf, s);
     case T_Q4_0: return launch_id_pair<PolQ4_0>(ia, xf, s);
     case T_MXFP4: return launch_id_pair<PolMXFP4>(ia, xf, s);
@@ -2221,6 +2309,7 @@ hipError_t launch_gemv_id(const DevWeight &w, int n_expert, const DevAct &a, con
     if (w2) { ia.p0b = w2->p0; ia.p1b = w2->p1; ia.p2b = w2->p2; ia.db = w2->d; ia.yb = y2; }
     switch (w.type) {
     case T_Q4_K: return a.type == T_Q8_K ? launch_id_type<PolQ4K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
+    case T_Q5_K: return a.type == T_Q8_K ? launch_id_type<PolQ5K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     case T_Q6_K: return a.type == T_Q8_K ? launch_id_type<PolQ6K>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     case T_Q4_0: return a.type == T_Q8_0 ? launch_id_type<PolQ4_0>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
     case T_MXFP4: return a.type == T_Q8_0 ? launch_id_type<PolMXFP4>(ia, a, xf, up, groups, s) : hipErrorInvalidValue;
