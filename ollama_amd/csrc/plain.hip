@@ -645,6 +645,8 @@ hipError_t gemm_typed(const DevWeight &w, const void *xc, int64_t N, float *y, i
         if (!grid_of(128, 64, g)) return hipErrorInvalidValue;
         plain_gemm_kernel<TYPE, 2, 2, 2, 1><<<g, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
     } else {
+        // (256 x 128 tiles of four waves of 64 x 128 -- six LDS fragment reads per eight MFMAs instead of eight -- measured
+        // 133 us where these take 122: 14336 x 4096 at 512 columns is 224 such tiles for 256 CUs)
         if (!grid_of(128, 128, g)) return hipErrorInvalidValue;
         plain_gemm_kernel<TYPE, 2, 2, 2, 2><<<g, 256, 0, s>>>(w.p0, xb, y, w.K, w.M, N);
     }

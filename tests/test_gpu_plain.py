@@ -41,7 +41,7 @@ SHAPES = [
     (70000, 256, 2), (40, 4096 + 64, 7), (16, 64 * 9, 11),
     (256, 14336, 1), (256, 14336, 4), (200, 14336, 8), (96, 40960, 2),
     (512, 4096, 9), (300, 4096, 32), (515, 1024, 33), (130, 2048, 130), (1000, 512, 257),
-    (14336, 4096, 1), (4096, 14336, 4), (2048, 4096, 128), (256, 14336, 64),
+    (14336, 4096, 1), (4096, 14336, 4), (2048, 4096, 128), (256, 14336, 64), (6200, 512, 1000),
     (64, 72, 3), (64, 72, 20), (50, 70, 1), (50, 70, 12), (9, 1, 2), (40, 1001, 3),
 ]
 
