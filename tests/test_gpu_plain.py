@@ -104,17 +104,20 @@ def test_plain_small_integers_are_exact(ctx, t):
 
 
 def test_f16_subnormal_weights_are_multiplied_not_flushed(ctx):
-    """weights below the smallest normal half (6.1e-5): the streaming kernel widens them exactly"""
+    """weights below the smallest normal half (6.1e-5) and activations that convert to subnormal halves: the matrix cores
+    (1..16 columns and the tiles) and the vector-ALU kernel multiply them, none flushes them to zero"""
     m, k = 64, 1024
     w = (np.random.default_rng(3).standard_normal((m, k)) * 2e-6).astype(np.float32)
     raw = oracle.quantize(F16, w)
     assert np.count_nonzero(raw.view(np.uint16) & 0x7C00) == 0  # every weight is subnormal (or zero)
-    x = np.random.default_rng(4).standard_normal((2, k)).astype(np.float32)
     W = ctx.upload(F16, raw, k, m)
     try:
-        y = ctx.mulmat(W, x)
-        ref = oracle.mul_mat(F16, raw, k, m, x)
-        assert np.abs(ref).max() > 0 and npref.rel_err(y, ref) <= 1e-3
+        for n, scale in ((2, 1.0), (40, 1.0), (2, 1e-5)):
+            x = (np.random.default_rng(4 + n).standard_normal((n, k)) * scale).astype(np.float32)
+            ref = oracle.mul_mat(F16, raw, k, m, x)
+            assert np.abs(ref).max() > 0
+            for path in (qmm.PATH_AUTO, qmm.PATH_GEMV, qmm.PATH_GEMM):
+                assert npref.rel_err(ctx.mulmat(W, x, path), ref) <= 1e-3, (n, scale, path)
     finally:
         W.free()
 
