@@ -47,6 +47,7 @@ enum {
     MI_QMM_TYPE_F32 = 0,
     MI_QMM_TYPE_F16 = 1,
     MI_QMM_TYPE_Q4_0 = 2,
+    MI_QMM_TYPE_Q5_0 = 6,
     MI_QMM_TYPE_Q8_0 = 8,
     MI_QMM_TYPE_Q4_K = 12,
     MI_QMM_TYPE_Q5_K = 13,
@@ -160,7 +161,9 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      MI_QMM_ERR_UNSUPPORTED.  The tensor is also kept in its own layout, which the streaming kernels (one or
  *      two activation rows, a few pairs per expert) read at half the bytes.  A scale byte above 146 is
  *      MI_QMM_ERR_UNSUPPORTED; blocks with a scale byte below 104 (weights under 7.2e-7) are zeros in the Q8_0
- *      planes (the matrix-core kernels) and exact in the streaming kernels.
+ *      planes (the matrix-core kernels) and exact in the streaming kernels.  6 (Q5_0) is kept as Q8_0 planes in the
+ *      same way (its 5-bit values minus 16 as int8 under the block's own scale: the same dot products, term for
+ *      term) with the same rule for rows that are no multiple of 256.
  *      src_location: MI_QMM_HOST or MI_QMM_DEVICE. */
 int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int ggml_type, const void *gguf_bytes, int64_t k,
                          int64_t m, int src_location, mi_qmm_weight **out);

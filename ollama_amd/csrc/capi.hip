@@ -220,7 +220,7 @@ int64_t mi_qmm_row_size(int t, int64_t k) {
 
 int mi_qmm_vec_dot_type(int wt) {
     switch (wt) {
-    case T_Q4_0: case T_Q8_0: case T_MXFP4: return T_Q8_0;
+    case T_Q4_0: case T_Q5_0: case T_Q8_0: case T_MXFP4: return T_Q8_0;
     case T_Q4_K: case T_Q5_K: case T_Q6_K: return T_Q8_K;
     case T_F32: case T_F16: case T_BF16: return wt;  // multiplied in their own type: x is converted to it
     default: return -1;
@@ -324,13 +324,13 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     if (!out) return fail(MI_QMM_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (mi_qmm_vec_dot_type(type) < 0)
-        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 8, 12, 13, 14, 30, 39)", type);
+        return fail(MI_QMM_ERR_UNSUPPORTED, "ggml type %d is not a supported weight type (0, 1, 2, 6, 8, 12, 13, 14, 30, 39)", type);
     if (k <= 0 || m <= 0) return fail(MI_QMM_ERR_INVALID, "k=%lld m=%lld must be positive", (long long)k, (long long)m);
     const int64_t row = mi_qmm_row_size(type, k);
     if (row < 0)
         return fail(MI_QMM_ERR_INVALID, "k=%lld is not a multiple of the block size %lld of type %d",
                     (long long)k, (long long)mi_qmm_block_size(type), type);
-    if (type == T_Q4_0 || type == T_Q8_0 || type == T_MXFP4) {
+    if (type == T_Q4_0 || type == T_Q5_0 || type == T_Q8_0 || type == T_MXFP4) {
         // the activation quantizer pairs these with Q8_0 planes read as 16-byte pieces
         if (k % QK != 0) return fail(MI_QMM_ERR_INVALID, "k not a multiple of 32");
     }
@@ -348,6 +348,11 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
     case T_Q5_K: s0 = (size_t)(m * (k / QKK)) * 2 * Q4_K_BYTES; s1 = total; break;  // a Q4_K tensor of rows twice as long; the blocks as they are
     case T_Q4_0: s0 = (size_t)(m * (k / 2)); sd = (size_t)(m * (k / QK)) * 2; break;
     case T_Q8_0: s0 = (size_t)(m * k); sd = (size_t)(m * (k / QK)) * 2; break;
+    case T_Q5_0: {   // kept as Q8_0 planes, rows of whole 256-element steps
+        const size_t kp = align_up((size_t)k, 256);
+        s0 = (size_t)m * kp; sd = (size_t)m * (kp / QK) * 2;
+        break;
+    }
     case T_MXFP4: {  // Q8_0 planes (p0, d), and the tensor as it is (p1: nibbles, p2: scale bytes)
         const size_t kp = align_up((size_t)k, 256);
         s0 = (size_t)m * kp; sd = (size_t)m * (kp / QK) * 2; s1 = (size_t)m * (kp / QK) * 16; s2 = (size_t)m * (kp / QK) * 2;
@@ -381,6 +386,10 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
         w->native = w->dev;
         w->native.type = T_Q5_K; w->native.K = k; w->native.p0 = b + o1; w->native.p1 = nullptr;
         w->dev.p1 = nullptr;
+    }
+    if (type == T_Q5_0) {
+        w->dev.type = T_Q8_0; w->file_type = T_Q5_0; w->dev.K = (int64_t)align_up((size_t)k, 256);
+        if (w->dev.K != k) { w->expand = true; w->k_user = k; }
     }
     if (type == T_MXFP4) {
         // rows of a whole number of 256-element steps (2880 -> 3072): the matrix-core kernels of the 32-element formats want that
@@ -419,6 +428,7 @@ int mi_qmm_weight_upload(mi_qmm_ctx *ctx, int type, const void *bytes, int64_t k
             if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "hipMemset(flag)", e);
         }
         e = type == T_Q5_K ? launch_relayout_q5k(src, k, m, b + o0, ctx->stream)
+            : type == T_Q5_0 ? launch_relayout_q5_0(src, k, w->dev.K, m, b + o0, (uint16_t *)(b + od), ctx->stream)
             : type == T_MXFP4 ? launch_relayout_mxfp4(src, k, w->dev.K, m, b + o0, (uint16_t *)(b + od), bad, ctx->stream)
                               : launch_relayout(type, src, k, m, b + o0, b + o1, b + o2, (uint16_t *)(b + od), ctx->stream);
         if (e != hipSuccess) return cleanup(MI_QMM_ERR_HIP, "relayout kernel", e);

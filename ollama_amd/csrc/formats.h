@@ -14,7 +14,7 @@
 
 namespace miqmm {
 
-enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 30, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_Q8_K = 15, T_MXFP4 = 39 };
+enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 30, T_Q4_0 = 2, T_Q5_0 = 6, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_Q8_K = 15, T_MXFP4 = 39 };
 
 constexpr int QK = 32;    // elements per Q4_0 / Q8_0 block
 constexpr int QKK = 256;  // elements per K-quant super-block
@@ -31,6 +31,7 @@ constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q5_K_BYTES = 1
 //          the Q5_K blocks without their fifth bits, blocks K'/256 .. are the fifth bits alone -- same scales, no mins,
 //          nibble 8 where the bit is set, block scale 2 d -- so that against the activations repeated, [x | x], every
 //          Q4_K kernel computes sum sc (q4 + 16 h) y exactly (see relayout.hip)
+//   Q5_0 : stored as the Q8_0 planes with the same dot products (type = T_Q8_0): the 5-bit values minus 16 as int8, d as it is
 //   MXFP4: stored as the Q8_0 planes with the same dot products (type = T_Q8_0): the doubled E2M1 values as int8, the scale
 //          2^(e - 128) as the fp16 block scale (see relayout.hip) -- what the matrix-core kernels multiply -- and once more as
 //          it is (type = T_MXFP4: p0 = nibble plane [M][K/32][16], d = the scale bytes, 16 bits each) for the streaming kernels

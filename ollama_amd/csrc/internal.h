@@ -39,6 +39,8 @@ hipError_t launch_relayout_q5k(const uint8_t *gguf, int64_t K, int64_t M, uint8_
 // MXFP4 blocks [M][K/32][17] -> Q8_0 planes (qs [M][K_out], d [M][K_out/32], rows padded with zero blocks) with the same dot products; *bad (device int, zeroed
 // by the caller) is set when a block's scale is beyond what the planes can hold (e > 146: weights of 2^18 and more)
 hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *d, int *bad, hipStream_t s);
+// Q5_0 blocks [M][K/32][22] -> Q8_0 planes with the same dot products, rows padded with zero blocks to K_out
+hipError_t launch_relayout_q5_0(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *d, hipStream_t s);
 // MXFP4 blocks -> their own planes for the streaming kernels (type T_MXFP4: p0 = nibble plane [M][K_out/32][16], d = the scale
 // bytes as 16-bit values [M][K_out/32]), rows padded with zero blocks
 hipError_t launch_relayout_mxfp4_native(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *e, hipStream_t s);

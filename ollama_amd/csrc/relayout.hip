@@ -114,6 +114,29 @@ __global__ void relayout_mxfp4_kernel(const uint8_t *__restrict__ src, int64_t M
     }
 }
 
+// Q5_0 -> Q8_0 planes.  w = d (q - 16) with q the nibble plus 16 times bit i of the 32-bit word qh: 32 integers in -16..15
+// under the block's fp16 scale, and ggml multiplies them with Q8_0 activations as sum_i (q_i - 16) y_i * (d d_y) -- the Q8_0 dot
+// product of those integers, term for term.  Rows padded with zero blocks from nb_in to nb_out blocks.  One thread per nibble byte.
+__global__ void relayout_q5_0_kernel(const uint8_t *__restrict__ src, int64_t M, int nb_in, int nb_out, int8_t *__restrict__ qs,
+                                     uint16_t *__restrict__ d) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M * nb_out * 16) return;
+    const int64_t blk = i >> 4, row = blk / nb_out;
+    const int bi = (int)(blk - row * nb_out), j = (int)(i & 15);
+    if (bi >= nb_in) {
+        qs[blk * 32 + j] = 0;
+        qs[blk * 32 + j + 16] = 0;
+        if (j == 0) d[blk] = 0;
+        return;
+    }
+    const uint8_t *b = src + (row * nb_in + bi) * 22;
+    const unsigned qh = b[2] | (b[3] << 8) | (b[4] << 16) | ((unsigned)b[5] << 24);
+    const int q = b[6 + j];
+    qs[blk * 32 + j] = (int8_t)(((q & 15) | (((qh >> j) & 1u) << 4)) - 16);
+    qs[blk * 32 + j + 16] = (int8_t)(((q >> 4) | (((qh >> (j + 16)) & 1u) << 4)) - 16);
+    if (j == 0) d[blk] = (uint16_t)(b[0] | (b[1] << 8));
+}
+
 // MXFP4 as it is, for the streaming kernels: the 16 nibble bytes of every block in one plane, its scale byte (widened to 16
 // bits) in another; rows padded with zero blocks (scale byte 0, codes 0) from nb_in to nb_out blocks.
 __global__ void relayout_mxfp4_native_kernel(const uint8_t *__restrict__ src, int64_t M, int nb_in, int nb_out, uint8_t *__restrict__ qs,
@@ -155,6 +178,15 @@ hipError_t launch_relayout_mxfp4(const uint8_t *gguf, int64_t K, int64_t K_out, 
     const int64_t n = M * (K_out / QK) * 16;
     if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
     relayout_mxfp4_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QK), (int)(K_out / QK), (int8_t *)qs, d, bad);
+    return hipGetLastError();
+}
+
+hipError_t launch_relayout_q5_0(const uint8_t *gguf, int64_t K, int64_t K_out, int64_t M, uint8_t *qs, uint16_t *d, hipStream_t s) {
+    if (K * M == 0) return hipSuccess;
+    if (K % QK || K_out % QK || K_out < K) return hipErrorInvalidValue;
+    const int64_t n = M * (K_out / QK) * 16;
+    if ((n + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
+    relayout_q5_0_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gguf, M, (int)(K / QK), (int)(K_out / QK), (int8_t *)qs, d);
     return hipGetLastError();
 }
 

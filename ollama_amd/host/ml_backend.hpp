@@ -134,7 +134,7 @@ public:
             // padded go through mi_qmm_mulmat / mi_qmm_mulmat_id directly, not through this mirror)
             const int q8 = mi_qmm_vec_dot_type(type);
             if (rc != MI_QMM_OK || (nd != 2 && nd != 3) || (q8 != MI_QMM_TYPE_Q8_0 && q8 != MI_QMM_TYPE_Q8_K) || type == MI_QMM_TYPE_Q5_K ||
-                (type == MI_QMM_TYPE_MXFP4 && dims[0] % 256 != 0)) continue;
+                ((type == MI_QMM_TYPE_MXFP4 || type == MI_QMM_TYPE_Q5_0) && dims[0] % 256 != 0)) continue;
             auto t = std::make_shared<Tensor>();
             t->shape_.assign(dims, dims + nd);
             t->type_ = type;

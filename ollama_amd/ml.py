@@ -44,8 +44,8 @@ _GGML_TO_DTYPE = {qmm.F32: DType.F32, qmm.F16: DType.F16, qmm.Q8_0: DType.Q80, q
 
 def _single_only(t: "Tensor") -> bool:
     """weights that only the plain product entry points multiply (mulmat, mulmat_multi; for padded MXFP4 stacks also
-    mulmat_id): F32 / F16 / BF16, Q5_K, and MXFP4 whose rows are no multiple of 256 (kept padded on the device)"""
-    return t._type in qmm.SINGLE_ONLY_TYPES or (t._type == qmm.MXFP4 and t.Dim(0) % 256 != 0)
+    mulmat_id): F32 / F16 / BF16, Q5_K, and MXFP4 / Q5_0 whose rows are no multiple of 256 (kept padded on the device)"""
+    return t._type in qmm.SINGLE_ONLY_TYPES or (t._type in (qmm.MXFP4, qmm.Q5_0) and t.Dim(0) % 256 != 0)
 
 
 class Tensor:

@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI_QMM_LIB points at an alternative build of the library (e.g. an experimental variant)
 LIB_PATH = os.environ.get("MI_QMM_LIB") or os.path.join(_HERE, "libmi_qmm.so")
 
-F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, BF16, MXFP4 = 0, 1, 2, 8, 12, 13, 14, 15, 30, 39
+F32, F16, Q4_0, Q5_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, BF16, MXFP4 = 0, 1, 2, 6, 8, 12, 13, 14, 15, 30, 39
 PLAIN_TYPES = (F32, F16, BF16)  # unquantized weight types: multiplied in their own type
 SINGLE_ONLY_TYPES = PLAIN_TYPES + (Q5_K,)  # weight types that only mulmat / mulmat_multi multiply (no fused or expert forms)
 HOST, DEVICE = 0, 1

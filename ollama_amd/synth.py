@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import numpy as np
 
-F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 2, 8, 12, 13, 14, 30, 39
+F32, F16, Q4_0, Q5_0, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 2, 6, 8, 12, 13, 14, 30, 39
 
 
 def _f16_bytes(v: np.ndarray) -> np.ndarray:
@@ -79,6 +79,25 @@ def encode_mxfp4(x: np.ndarray) -> np.ndarray:
     out = np.empty((m, k // 32, 17), np.uint8)
     out[..., 0] = (e + 127).astype(np.uint8)
     out[..., 1:] = code[..., :16] | (code[..., 16:] << 4)
+    return out.reshape(m, -1)
+
+
+def encode_q5_0(x: np.ndarray) -> np.ndarray:
+    """as encode_q4_0 on 32 levels: d = (the element of largest magnitude) / -16, q = round(x / d) + 16 in 0..31; the fifth
+    bits of the 32 elements in a little-endian 32-bit word"""
+    x = np.ascontiguousarray(x, np.float32)
+    m, k = x.shape
+    b = x.reshape(m, k // 32, 32)
+    idx = np.abs(b).argmax(axis=2)
+    mx = np.take_along_axis(b, idx[..., None], axis=2)[..., 0]
+    d = mx / np.float32(-16)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(d[..., None] != 0, np.rint(b / d[..., None]) + 16, 16).clip(0, 31).astype(np.uint8)
+    out = np.empty((m, k // 32, 22), np.uint8)
+    out[..., 0:2] = _f16_bytes(d)
+    word = ((q >> 4).astype(np.uint64) << np.arange(32, dtype=np.uint64)).sum(axis=2).astype(np.uint32)
+    out[..., 2:6] = word[..., None].view(np.uint8).reshape(m, k // 32, 4)
+    out[..., 6:] = (q[..., :16] & 15) | ((q[..., 16:] & 15) << 4)
     return out.reshape(m, -1)
 
 
@@ -170,7 +189,7 @@ def encode_q6_K(x: np.ndarray) -> np.ndarray:
     return out.reshape(m, -1)
 
 
-ENCODERS = {Q4_0: encode_q4_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K, MXFP4: encode_mxfp4,
+ENCODERS = {Q4_0: encode_q4_0, Q5_0: encode_q5_0, Q8_0: encode_q8_0, Q4_K: encode_q4_K, Q5_K: encode_q5_K, Q6_K: encode_q6_K, MXFP4: encode_mxfp4,
             F32: encode_f32, F16: encode_f16, BF16: encode_bf16}
 
 

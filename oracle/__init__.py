@@ -15,7 +15,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libggml_ref.so")
 
-F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, BF16, MXFP4 = 0, 1, 2, 8, 12, 13, 14, 15, 30, 39
+F32, F16, Q4_0, Q5_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, BF16, MXFP4 = 0, 1, 2, 6, 8, 12, 13, 14, 15, 30, 39
 
 
 def build(force: bool = False) -> str:
@@ -48,7 +48,7 @@ def lib() -> ctypes.CDLL:
         L.ref_fp32_to_bf16.restype = ctypes.c_uint16; L.ref_fp32_to_bf16.argtypes = [ctypes.c_float]
         L.ref_bf16_to_fp32.restype = ctypes.c_float; L.ref_bf16_to_fp32.argtypes = [ctypes.c_uint16]
         L.ref_e8m0_to_fp32_half.restype = ctypes.c_float; L.ref_e8m0_to_fp32_half.argtypes = [ctypes.c_uint8]
-        for name in ("mxfp4_q8_0", "q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q5_K_q8_K", "q6_K_q8_K", "f32", "f16", "bf16"):
+        for name in ("mxfp4_q8_0", "q5_0_q8_0", "q4_0_q8_0", "q8_0_q8_0", "q4_K_q8_K", "q5_K_q8_K", "q6_K_q8_K", "f32", "f16", "bf16"):
             f = getattr(L, "ref_vec_dot_" + name)
             f.restype = ctypes.c_float; f.argtypes = [i64, vp, vp]
         L.ref_vec_dot_type.restype = ci; L.ref_vec_dot_type.argtypes = [ci]
@@ -130,7 +130,7 @@ def dequantize(t: int, blocks: np.ndarray, k: int) -> np.ndarray:
     return out
 
 
-_DOTS = {MXFP4: "mxfp4_q8_0", Q4_0: "q4_0_q8_0", Q8_0: "q8_0_q8_0", Q4_K: "q4_K_q8_K", Q5_K: "q5_K_q8_K", Q6_K: "q6_K_q8_K", F32: "f32", F16: "f16", BF16: "bf16"}
+_DOTS = {MXFP4: "mxfp4_q8_0", Q5_0: "q5_0_q8_0", Q4_0: "q4_0_q8_0", Q8_0: "q8_0_q8_0", Q4_K: "q4_K_q8_K", Q5_K: "q5_K_q8_K", Q6_K: "q6_K_q8_K", F32: "f32", F16: "f16", BF16: "bf16"}
 
 
 def vec_dot(wtype: int, k: int, wrow: np.ndarray, xqrow: np.ndarray) -> float:

@@ -18,6 +18,7 @@
 /* ---- block layouts: byte sizes follow /root/reference/fs/ggml/ggml.go:450-473 ------------- */
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[QK / 2]; } blk_q4_0;                                /* 2+16      */
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[QK / 2]; } blk_q5_0;                 /* 2+4+16    */
 typedef struct { uint16_t d; int8_t qs[QK]; } blk_q8_0;                                     /* 2+32      */
 typedef struct { uint8_t e; uint8_t qs[QK / 2]; } blk_mxfp4;                                /* 1+16      */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[QKK / 2]; } blk_q4_K; /* 2+2+12+128 */
@@ -27,6 +28,7 @@ typedef struct { float d; int8_t qs[QKK]; int16_t bsums[QKK / 16]; } blk_q8_K;  
 #pragma pack(pop)
 
 _Static_assert(sizeof(blk_q4_0) == 18, "Q4_0 block is 18 bytes");
+_Static_assert(sizeof(blk_q5_0) == 22, "Q5_0 block is 22 bytes");
 _Static_assert(sizeof(blk_q8_0) == 34, "Q8_0 block is 34 bytes");
 _Static_assert(sizeof(blk_mxfp4) == 17, "MXFP4 block is 17 bytes");
 _Static_assert(sizeof(blk_q4_K) == 144, "Q4_K block is 144 bytes");
@@ -37,7 +39,7 @@ _Static_assert(sizeof(blk_q8_K) == 292, "Q8_K block is 292 bytes");
 int64_t ref_block_size(int type) {
     switch (type) {
     case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return 1;
-    case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: case REF_TYPE_MXFP4: return QK;
+    case REF_TYPE_Q4_0: case REF_TYPE_Q5_0: case REF_TYPE_Q8_0: case REF_TYPE_MXFP4: return QK;
     case REF_TYPE_Q4_K: case REF_TYPE_Q5_K: case REF_TYPE_Q6_K: case REF_TYPE_Q8_K: return QKK;
     default: return 0;
     }
@@ -48,6 +50,7 @@ int64_t ref_type_size(int type) {
     case REF_TYPE_F32: return 4;
     case REF_TYPE_F16: case REF_TYPE_BF16: return 2;
     case REF_TYPE_Q4_0: return sizeof(blk_q4_0);
+    case REF_TYPE_Q5_0: return sizeof(blk_q5_0);
     case REF_TYPE_Q8_0: return sizeof(blk_q8_0);
     case REF_TYPE_MXFP4: return sizeof(blk_mxfp4);
     case REF_TYPE_Q4_K: return sizeof(blk_q4_K);
@@ -66,7 +69,7 @@ int64_t ref_row_size(int type, int64_t k) {
 
 int ref_vec_dot_type(int wtype) {
     switch (wtype) {
-    case REF_TYPE_Q4_0: case REF_TYPE_Q8_0: case REF_TYPE_MXFP4: return REF_TYPE_Q8_0;
+    case REF_TYPE_Q4_0: case REF_TYPE_Q5_0: case REF_TYPE_Q8_0: case REF_TYPE_MXFP4: return REF_TYPE_Q8_0;
     case REF_TYPE_Q4_K: case REF_TYPE_Q5_K: case REF_TYPE_Q6_K: return REF_TYPE_Q8_K;
     /* the unquantized weight types are multiplied in their own type: the activations are converted to it */
     case REF_TYPE_F32: case REF_TYPE_F16: case REF_TYPE_BF16: return wtype;
@@ -516,6 +519,21 @@ static void dequant_q4_K(const blk_q4_K *x, float *y, int64_t k) {
     }
 }
 
+/* Q5_0: the Q4_0 layout with a fifth bit per weight in a 32-bit word: bit j of qh belongs to element j; w = d (q - 16) */
+static void dequant_q5_0(const blk_q5_0 *x, float *y, int64_t k) {
+    for (int64_t i = 0; i < k / QK; i++) {
+        const float d = ref_fp16_to_fp32(x[i].d);
+        uint32_t qh;
+        memcpy(&qh, x[i].qh, 4);
+        for (int j = 0; j < QK / 2; j++) {
+            const uint8_t xh_0 = (uint8_t)(((qh >> (j + 0)) << 4) & 0x10);
+            const uint8_t xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+            y[i * QK + j] = (float)(((x[i].qs[j] & 0x0F) | xh_0) - 16) * d;
+            y[i * QK + j + QK / 2] = (float)(((x[i].qs[j] >> 4) | xh_1) - 16) * d;
+        }
+    }
+}
+
 /* MXFP4 (OCP microscaling: 32 four-bit floats E2M1 under one power-of-two scale E8M0; the block layout is the one
  * /root/reference/convert/convert_gptoss.go:216-238 writes: the scale byte, then 16 bytes whose low nibbles are elements
  * 0..15 and whose high nibbles are elements 16..31).  ggml keeps the E2M1 values doubled as integers and halves the
@@ -597,6 +615,7 @@ int ref_dequantize_row(int type, const void *x, float *y, int64_t k) {
     if (ref_row_size(type, k) < 0) return -1;
     switch (type) {
     case REF_TYPE_Q4_0: dequant_q4_0((const blk_q4_0 *)x, y, k); return 0;
+    case REF_TYPE_Q5_0: dequant_q5_0((const blk_q5_0 *)x, y, k); return 0;
     case REF_TYPE_Q8_0: dequant_q8_0((const blk_q8_0 *)x, y, k); return 0;
     case REF_TYPE_MXFP4: dequant_mxfp4((const blk_mxfp4 *)x, y, k); return 0;
     case REF_TYPE_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
@@ -637,6 +656,29 @@ float ref_vec_dot_q8_0_q8_0(int64_t n, const void *vx, const void *vy) {
         int sumi = 0;
         for (int j = 0; j < QK; j++) sumi += x[ib].qs[j] * y[ib].qs[j];
         sumf += sumi * (ref_fp16_to_fp32(x[ib].d) * ref_fp16_to_fp32(y[ib].d));
+    }
+    return sumf;
+}
+
+/* ggml_vec_dot_q5_0_q8_0, generic path */
+float ref_vec_dot_q5_0_q8_0(int64_t n, const void *vx, const void *vy) {
+    const blk_q5_0 *x = (const blk_q5_0 *)vx;
+    const blk_q8_0 *y = (const blk_q8_0 *)vy;
+    float sumf = 0;
+    for (int64_t ib = 0; ib < n / QK; ib++) {
+        uint32_t qh;
+        memcpy(&qh, x[ib].qh, 4);
+        int sumi0 = 0, sumi1 = 0;
+        for (int j = 0; j < QK / 2; j++) {
+            const uint8_t xh_0 = (uint8_t)(((qh & (1u << (j + 0))) >> (j + 0)) << 4);
+            const uint8_t xh_1 = (uint8_t)((qh & (1u << (j + 16))) >> (j + 12));
+            const int32_t x0 = (int8_t)(((x[ib].qs[j] & 0x0F) | xh_0) - 16);
+            const int32_t x1 = (int8_t)(((x[ib].qs[j] >> 4) | xh_1) - 16);
+            sumi0 += x0 * y[ib].qs[j];
+            sumi1 += x1 * y[ib].qs[j + QK / 2];
+        }
+        const int sumi = sumi0 + sumi1;
+        sumf += (ref_fp16_to_fp32(x[ib].d) * ref_fp16_to_fp32(y[ib].d)) * sumi;
     }
     return sumf;
 }
@@ -865,6 +907,7 @@ static quant_fn quantizer_for(int type) {
 static dot_fn dot_for(int wtype) {
     switch (wtype) {
     case REF_TYPE_Q4_0: return ref_vec_dot_q4_0_q8_0;
+    case REF_TYPE_Q5_0: return ref_vec_dot_q5_0_q8_0;
     case REF_TYPE_Q8_0: return ref_vec_dot_q8_0_q8_0;
     case REF_TYPE_MXFP4: return ref_vec_dot_mxfp4_q8_0;
     case REF_TYPE_Q4_K: return ref_vec_dot_q4_K_q8_K;

@@ -49,7 +49,7 @@ extern "C" {
 #endif
 
 /* ggml_type ids, /root/reference/fs/ggml/type.go:250-268 */
-enum { REF_TYPE_F32 = 0, REF_TYPE_F16 = 1, REF_TYPE_BF16 = 30, REF_TYPE_MXFP4 = 39, REF_TYPE_Q4_0 = 2, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12, REF_TYPE_Q5_K = 13,
+enum { REF_TYPE_F32 = 0, REF_TYPE_F16 = 1, REF_TYPE_BF16 = 30, REF_TYPE_MXFP4 = 39, REF_TYPE_Q4_0 = 2, REF_TYPE_Q5_0 = 6, REF_TYPE_Q8_0 = 8, REF_TYPE_Q4_K = 12, REF_TYPE_Q5_K = 13,
        REF_TYPE_Q6_K = 14, REF_TYPE_Q8_K = 15 };
 
 int64_t ref_block_size(int type);               /* elements per block, 0 if unknown */
@@ -90,6 +90,7 @@ void ref_unpack_scales_kmask(const uint8_t *s12, uint8_t sc[8], uint8_t m[8]);
 /* dot products: n elements, x = weight row blocks, y = activation row blocks */
 float ref_vec_dot_q4_0_q8_0(int64_t n, const void *x, const void *y);
 float ref_vec_dot_q8_0_q8_0(int64_t n, const void *x, const void *y);
+float ref_vec_dot_q5_0_q8_0(int64_t n, const void *x, const void *y);
 float ref_vec_dot_mxfp4_q8_0(int64_t n, const void *x, const void *y);
 float ref_e8m0_to_fp32_half(uint8_t e);   /* 2^(e - 128): half the E8M0 scale (ggml keeps the E2M1 values doubled) */
 float ref_vec_dot_q4_K_q8_K(int64_t n, const void *x, const void *y);

@@ -9,9 +9,9 @@ from __future__ import annotations
 
 import numpy as np
 
-F32, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, MXFP4 = 0, 2, 8, 12, 13, 14, 15, 39
-BLOCK = {MXFP4: 32, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
-BYTES = {MXFP4: 17, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
+F32, Q4_0, Q5_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K, MXFP4 = 0, 2, 6, 8, 12, 13, 14, 15, 39
+BLOCK = {MXFP4: 32, Q5_0: 32, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
+BYTES = {MXFP4: 17, Q5_0: 22, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
 
 
 def _blocks(raw: np.ndarray, t: int) -> np.ndarray:
@@ -56,6 +56,17 @@ def mxfp4_values(raw):
     ex, man = (nib >> 1) & 3, nib & 1
     mag = np.where(ex == 0, man * 0.5, (1 + man / 2) * 2.0 ** (ex - 1))
     return sign * mag * (2.0 ** (e - 127))[:, None]
+
+
+def q5_0_ints(raw):
+    """(d, the 32 integers q - 16): nibbles as in Q4_0, bit i of the little-endian 32-bit word qh is the fifth bit of element i"""
+    b = _blocks(raw, Q5_0)
+    d = _f16(b[:, 0:2])
+    qh = b[:, 2:6].astype(np.int64)
+    word = qh[:, 0] | (qh[:, 1] << 8) | (qh[:, 2] << 16) | (qh[:, 3] << 24)
+    bits = (word[:, None] >> np.arange(32)[None, :]) & 1
+    nib = np.concatenate([b[:, 6:] & 15, b[:, 6:] >> 4], axis=1).astype(np.int64)
+    return d, nib + 16 * bits - 16
 
 
 def q8_0_ints(raw):
@@ -117,6 +128,9 @@ def dequant(t: int, raw) -> np.ndarray:
         return (d[:, None] * q).reshape(-1)
     if t == MXFP4:
         return mxfp4_values(raw).reshape(-1)
+    if t == Q5_0:
+        d, q = q5_0_ints(raw)
+        return (d[:, None] * q).reshape(-1)
     if t == Q4_K:
         d, dmin, sc, m, q = q4_K_ints(raw)
         w = (d[:, None] * sc)[:, :, None] * q - (dmin[:, None] * m)[:, :, None]
