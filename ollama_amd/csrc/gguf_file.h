@@ -87,6 +87,9 @@ inline bool gguf_type_geometry(uint32_t type, int64_t &block, int64_t &bytes) {
     case 28: block = 1; bytes = 8; return true;       // F64
     case 29: block = 256; bytes = 56; return true;    // IQ1_M
     case 30: block = 1; bytes = 2; return true;       // BF16
+    case 39: block = 32; bytes = 17; return true;     // MXFP4
+    case 40: block = 64; bytes = 36; return true;     // NVFP4
+    case 41: block = 128; bytes = 18; return true;    // Q1_0
     default: return false;
     }
 }

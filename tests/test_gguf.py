@@ -220,3 +220,18 @@ def test_hand_packed_file_pins_offsets_and_bytes(tmp_path):
         assert f.TensorBytes("blk.0.ffn_gate.weight").tobytes() == q4k
         assert f.TensorBytes("output_norm.weight").tobytes() == f32
         assert [t.Name for t in f.TensorInfos()] == ["blk.0.ffn_gate.weight", "output_norm.weight"]
+
+
+def test_file_reader_knows_every_type_the_size_tables_know(tmp_path):
+    """the reference's table of test rows ends at BF16 (30); its size formulas go on to MXFP4, NVFP4 and Q1_0
+    (/root/reference/fs/ggml/ggml.go:427-436, 504-509).  A file that holds such tensors -- the expert tensors of a gpt-oss
+    file are MXFP4 -- must open, with the sizes of the library's own tables."""
+    kinds = [t for t in range(64) if qmm.type_size(t) > 0]
+    assert {39, 40, 41} <= set(kinds)
+    tensors = [(f"t{t}", t, [qmm.block_size(t) * 2, 3], bytes(qmm.type_size(t) * 6)) for t in kinds]
+    p = str(tmp_path / "all_types.gguf")
+    gguf.write_gguf(p, {"general.architecture": "x"}, tensors)
+    with gguf.File(p) as f:
+        for t in kinds:
+            ti = f.TensorInfo(f"t{t}")
+            assert ti.Type == t and ti.NumBytes == qmm.type_size(t) * 6, t

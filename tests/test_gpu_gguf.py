@@ -14,7 +14,8 @@ def _model_file(tmp_path):
     k = 1024
     tensors, raws = [], {}
     for name, t, m in (("blk.0.attn_q.weight", qmm.Q4_K, 96), ("blk.0.ffn_down.weight", qmm.Q6_K, 40),
-                       ("blk.0.attn_k.weight", qmm.Q8_0, 33), ("output.weight", qmm.Q4_0, 50)):
+                       ("blk.0.attn_k.weight", qmm.Q8_0, 33), ("output.weight", qmm.Q4_0, 50),
+                       ("blk.0.attn_v.weight", qmm.Q5_K, 24), ("blk.1.attn_v.weight", qmm.Q5_0, 19), ("blk.0.dense_mx.weight", qmm.MXFP4, 21)):
         raw = synth.weights(t, m, k, seed=m).reshape(-1)
         raws[name] = (t, m, raw)
         tensors.append((name, t, [k, m], raw.tobytes()))
