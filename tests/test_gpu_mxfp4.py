@@ -152,3 +152,27 @@ def test_python_mirror_on_a_gpt_oss_shaped_expert_block():
             ctx.Close()
     finally:
         b.Close()
+
+
+def test_expert_stack_from_a_gguf_file(tmp_path):
+    """a 3-D MXFP4 tensor [K, M, experts] in a file: opened by the C reader, uploaded from the mapping, multiplied by MulmatID"""
+    from ollama_amd import gguf, ml
+    k, m, n_exp, n_used, tokens = 2880, 32, 4, 2, 3
+    raw_e = _random_rows(m * n_exp, k, seed=31)
+    p = str(tmp_path / "experts.gguf")
+    gguf.write_gguf(p, {"general.architecture": "gptoss"}, [("blk.0.ffn_down_exps.weight", MXFP4, [k, m, n_exp], raw_e.tobytes())])
+    b = ml.Backend(p)
+    b.Load()
+    try:
+        rng = np.random.default_rng(32)
+        xs = rng.standard_normal((tokens, k)).astype(np.float32)
+        ids = np.stack([rng.permutation(n_exp)[:n_used] for _ in range(tokens)]).astype(np.int32)
+        ctx = b.NewContext()
+        e = b.Get("blk.0.ffn_down_exps.weight").MulmatID(ctx, ctx.FromFloats(xs.reshape(-1), k, 1, tokens),
+                                                        ctx.FromInts(ids.reshape(-1), n_used, tokens))
+        ctx.Compute(e)
+        want = oracle.mul_mat_id(MXFP4, raw_e, k, m, n_exp, xs.reshape(tokens, 1, k), ids)
+        assert npref.rel_err(e.Floats().reshape(want.shape), want) <= 1e-3
+        ctx.Close()
+    finally:
+        b.Close()
