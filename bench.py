@@ -233,6 +233,23 @@ def main() -> int:
         },
     }
 
+    # ---- the same step captured once into a HIP graph on the stream and replayed (a separate figure, never `value`): the
+    # 2 x pool_layers launches of a step without the host's per-call work between them
+    gstep = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gstep, stream=stream):
+        step()
+    for _ in range(args.warmup):
+        gstep.replay()
+    t_g = timed(gstep.replay, args.steps)
+    same = all(bool(torch.equal(a, b)) for a, b in ((y_gate, kept["gate"]), (y_up, kept["up"]), (y_down, kept["down"])))
+    out["step_replayed_from_hip_graph"] = {"ms_per_step": round(t_g / args.steps * 1e3, 4),
+                                           "GB/s": round(bytes_per_step * args.steps / t_g / 1e9, 1),
+                                           "bit_identical_to_eager": same}
+    del gstep
+    if not same:
+        print("bench.py: the replayed graph of the step differs from the eager step", file=sys.stderr)
+        return 1
+
     # ---- what a pure read of the same bytes reaches in one launch on this machine (launch included): the
     # practical ceiling next to the GEMV's figure.  Best of a few grid shapes, rotating buffers like the weights.
     sr_path = os.path.join(os.path.dirname(qmm.LIB_PATH), "libmi_streamread.so")
@@ -490,6 +507,34 @@ def main() -> int:
                 "us": round(tm * 1e6, 1), "launch_groups": 32 * 4 + 1, "weight_GB": round(tok_bytes / 1e9, 3),
                 "GB/s": round(tok_bytes / tm / 1e9, 1), "frac_of_hbm_peak": round(tok_bytes / tm / 1e9 / HBM_PEAK_GBS, 4),
                 "tokens/s_if_nothing_else_ran": round(1.0 / tm, 1)}
+            # the same 129 calls captured once into a HIP graph on the stream and replayed: what a caller that builds its
+            # decode step as a graph (Context.Compute of a fixed graph) pays; the replay's outputs are checked against the
+            # eager calls' bit for bit, on replays with eager work between them
+            hid0 = hid.clone()
+            token()
+            want_l = yl.clone()
+            hid.copy_(hid0)
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=stream):
+                token()
+            same = True
+            for _ in range(3):
+                hid.copy_(hid0)
+                gr.replay()
+                torch.cuda.synchronize()
+                same = same and bool(torch.equal(yl, want_l))
+                token()
+                torch.cuda.synchronize()
+            if not same:
+                print("bench.py: the replayed graph of the token differs from the eager calls", file=sys.stderr)
+                return 1
+            gr.replay()
+            tg = timed(gr.replay, 5) / 5
+            other["Llama-3-8B-shaped Q4_K_M token: the same calls replayed from one captured HIP graph"] = {
+                "us": round(tg * 1e6, 1), "GB/s": round(tok_bytes / tg / 1e9, 1),
+                "frac_of_hbm_peak": round(tok_bytes / tg / 1e9 / HBM_PEAK_GBS, 4),
+                "tokens/s_if_nothing_else_ran": round(1.0 / tg, 1), "bit_identical_to_eager": True}
+            del gr
             for a in att:
                 for wt in a.values():
                     if wt is not None:
