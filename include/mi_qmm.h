@@ -150,8 +150,9 @@ void mi_qmm_host_free(mi_qmm_ctx *ctx, void *p);
  *      after the other there); the produced, expert-indexed and pre-quantized entry points take Q4_0 / Q8_0 /
  *      Q4_K / Q6_K weights only and return MI_QMM_ERR_UNSUPPORTED otherwise.  A Q5_K tensor is kept as the Q4_K
  *      tensor of rows twice as long that gives the same integer sums against [x | x] (1.64 times the bytes of
- *      the file: its products cost what a Q4_K product of twice the K costs) and, for one or two activation rows,
- *      as the blocks themselves, which the streaming kernel reads at their own 176 bytes.  39 (MXFP4, the expert tensors of
+ *      the file: its products cost what a Q4_K product of twice the K costs) and, for up to six activation rows
+ *      (eight on tensors of up to 8 Mi weights), as the blocks themselves, which the streaming kernel reads at their own
+ *      176 bytes (from three rows on, and at two on long rows, against x quantized once by a launch in front of it).  39 (MXFP4, the expert tensors of
  *      /root/reference/convert/convert_gptoss.go:124-150; DTypeMXFP4, /root/reference/ml/backend.go:404-412) is kept
  *      as the Q8_0 planes that give the same dot products -- the doubled E2M1 values as int8, the scale 2^(e - 128)
  *      as the block scale, twice the bytes of the file -- and goes through every entry point a Q8_0 weight goes

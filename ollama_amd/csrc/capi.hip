@@ -773,6 +773,27 @@ int plain_route(const mi_qmm_weight *w, int64_t n) {
     }
 }
 
+// Q5_K at three to eight activation rows on device pointers: whether the streaming kernel multiplies the blocks as they
+// are by quantized planes of x (a rule of the shape alone), and the two launches of that product.
+bool q5k_native_planes(const mi_qmm_weight *w, int64_t n, int path) {
+    // measured against the doubled rows (us): 1024 x 4096 at 3 / 4 / 5 / 8 rows 10.5 / 10.9 / 11.6 / 13.0 -> 8.4 / 9.0 / 9.5 / 11.5;
+    // 4096 x 14336 at 2 / 3 / 4 / 5 / 6 / 7 / 8: 22.8 / 22.6 / 22.7 / 25.2 / 25.8 / 26.7 / 27.2 -> 17.3 / 18.9 / 18.9 / 20.8 / 22.6 / 26.2 / 28.3;
+    // 14336 x 4096 at 3 / 4 / 5 / 6 / 7 / 8: 20.0 / 20.5 / 21.0 / 22.2 / 22.2 / 22.2 -> 16.7 / 17.5 / 18.3 / 22.1 / 23.9 / 25.4
+    const int64_t limit = w->k_user * w->dev.M <= (8 << 20) ? 8 : 6;
+    return w->repeat && w->has_native && n >= 2 && n <= limit && path != MI_QMM_PATH_GEMM && w->k_user % QKK == 0 &&
+           w->k_user <= gemv_max_k(T_Q5_K);
+}
+
+int q5k_planes_product(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *dx, int64_t n, float *dy, void *planes) {
+    const int64_t K = w->k_user;
+    const ActPlanes p = plan_act(planes, T_Q8_K, K, n, false);
+    HIP_TRY(launch_quantize_act(T_Q8_K, dx, K, n, p.qs, p.d, p.bsums, p.sd8, p.sd16, ctx->stream, nullptr, p.qf, p.bsf));
+    DevAct a;
+    a.qs = p.qs; a.d = p.d; a.bsums = p.bsums; a.sd8 = p.sd8; a.sd16 = p.sd16; a.qf = p.qf; a.bsf = p.bsf; a.K = K; a.N = (int)n; a.type = T_Q8_K;
+    HIP_TRY(launch_gemv(w->native, a, 0, (int)n, dy, w->dev.M, ctx->num_cus, ctx->stream));
+    return MI_QMM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -790,7 +811,11 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
         // Q5_K at one or two activation rows: the streaming kernel on the blocks as they are, x quantized in its prologue
         const bool q5_gemv = w->repeat && w->has_native && n >= 1 && n <= 2 && path != MI_QMM_PATH_GEMM &&
                              gemv_f32_supported(T_Q5_K, w->k_user, w->dev.M, (int)n);
+        // Q5_K at three to eight activation rows: x quantized once at its own length, then the streaming kernel on the
+        // blocks as they are (176 bytes a super-block read instead of the 288 of the doubled rows, no [x | x] copy)
+        const bool q5_planes = !q5_gemv && q5k_native_planes(w, n, path);
         if (path == MI_QMM_PATH_QUERY && q5_gemv) return MI_QMM_ROUTE_GEMV_F32;
+        if (path == MI_QMM_PATH_QUERY && q5_planes) return MI_QMM_ROUTE_GEMV;
         if (path == MI_QMM_PATH_QUERY || n == 0) return mi_qmm_mulmat_path(ctx, &lo, x, n, y, location, path);
         if (!x || !y) return fail(MI_QMM_ERR_INVALID, "x or y is NULL");
         if (q5_gemv) {
@@ -806,6 +831,27 @@ int mi_qmm_mulmat_path(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x, 
             }
             float *ys5[1] = {dy5};
             HIP_TRY(launch_gemv_f32_multi(&w->native, ys5, 1, dx5, (int)n, ctx->num_cus, ctx->stream));
+            if (location == MI_QMM_HOST) {
+                HIP_TRY(hipMemcpyAsync(y, dy5, yb5, hipMemcpyDeviceToHost, ctx->stream));
+                HIP_TRY(hipStreamSynchronize(ctx->stream));
+            }
+            return MI_QMM_OK;
+        }
+        if (q5_planes) {
+            const int64_t K5 = w->k_user, M5 = w->dev.M;
+            const size_t xb5 = (size_t)(n * K5) * 4, yb5 = (size_t)(n * M5) * 4;
+            const ActPlanes probe5 = plan_act(nullptr, T_Q8_K, K5, n, false);
+            if ((rc = reserve(ctx, &ctx->act_buf, &ctx->act_cap, probe5.total))) return rc;
+            const float *dx5 = x;
+            float *dy5 = y;
+            if (location == MI_QMM_HOST) {
+                const size_t yoff = align_up(xb5, 256);
+                if ((rc = reserve(ctx, &ctx->io_buf, &ctx->io_cap, yoff + yb5))) return rc;
+                dx5 = (const float *)ctx->io_buf;
+                dy5 = (float *)((char *)ctx->io_buf + yoff);
+                HIP_TRY(hipMemcpyAsync((void *)dx5, x, xb5, hipMemcpyHostToDevice, ctx->stream));
+            }
+            if ((rc = q5k_planes_product(ctx, w, dx5, n, dy5, ctx->act_buf))) return rc;
             if (location == MI_QMM_HOST) {
                 HIP_TRY(hipMemcpyAsync(y, dy5, yb5, hipMemcpyDeviceToHost, ctx->stream));
                 HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -903,6 +949,13 @@ static int noalloc_core(mi_qmm_ctx *ctx, const mi_qmm_weight *w, const float *x,
             float *ys5[1] = {y};  // Q5_K at one or two rows: the streaming kernel on the blocks as they are, no scratch
             HIP_TRY(launch_gemv_f32_multi(&w->native, ys5, 1, x, (int)n, ctx->num_cus, ctx->stream));
             return MI_QMM_OK;
+        }
+        if (q5k_native_planes(w, n, MI_QMM_PATH_AUTO)) {
+            const ActPlanes probe5 = plan_act(nullptr, T_Q8_K, w->k_user, n, false);
+            if (probe5.total > sbytes)
+                return fail(MI_QMM_ERR_UNSUPPORTED, "n=%lld rows of k=%lld need %zu bytes of quantized activations; the static scratch of "
+                            "mi_qmm_mulmat_noalloc holds %zu (use mi_qmm_mulmat)", (long long)n, (long long)w->k_user, probe5.total, sbytes);
+            return q5k_planes_product(ctx, w, x, n, y, sbase);
         }
         // the expanded activations at the end of the scratch, the quantized planes of the product in front of them
         mi_qmm_weight lo = *w;

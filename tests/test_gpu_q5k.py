@@ -1,5 +1,6 @@
-"""Mulmat on Q5_K weights through the C ABI against the oracle.  The library keeps a Q5_K tensor as the Q4_K tensor of
-rows twice as long that gives the same integer sums against [x | x]; every Q4_K kernel then serves it."""
+"""Mulmat on Q5_K weights through the C ABI against the oracle.  The library keeps a Q5_K tensor twice: as the blocks
+themselves, which the streaming kernel multiplies at up to six activation rows (eight on small tensors), and as the Q4_K
+tensor of rows twice as long that gives the same integer sums against [x | x], which every other Q4_K kernel serves."""
 import numpy as np
 import pytest
 
@@ -28,7 +29,7 @@ def _random_rows(m, k, seed):
 
 # (rows, K, activation rows): the decode GEMV, the deep and staged kernels, the tiled GEMMs; the value projection and the
 # down projection of an 8B model among them
-SHAPES = [(64, 256, 1), (100, 1024, 1), (1024, 4096, 1), (1024, 4096, 2), (1024, 4096, 4), (1024, 4096, 8), (333, 2048, 16),
+SHAPES = [(64, 256, 1), (64, 256, 3), (100, 1024, 6), (100, 1024, 7), (4096, 14336, 2), (4096, 14336, 6), (2100, 4096, 7), (100, 1024, 1), (1024, 4096, 1), (1024, 4096, 2), (1024, 4096, 4), (1024, 4096, 8), (333, 2048, 16),
           (4096, 14336, 1), (512, 14336, 3), (1024, 4096, 40), (1024, 4096, 130), (4096, 4096, 512), (256, 512, 300)]
 
 
@@ -76,7 +77,7 @@ def test_q5k_device_pointers_noalloc_joint_calls_and_refusals(ctx):
     W = ctx.upload(Q5_K, raw, k, m)
     Wq = ctx.upload(qmm.Q4_K, synth.weights(qmm.Q4_K, 64, k, seed=4), k, 64)
     try:
-        for n in (1, 5, 70):
+        for n in (1, 3, 5, 8, 70):
             x = np.random.default_rng(n).standard_normal((n, k)).astype(np.float32)
             want = ctx.mulmat(W, x)
             dx, dy = DeviceArray(x), DeviceArray(np.zeros((n, m), np.float32), zero=True)

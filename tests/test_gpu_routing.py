@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from npref import Q4_0, Q4_K, Q6_K, Q8_0, Q8_K
+from oracle import Q5_K
 from ollama_amd import qmm, synth
 
 pytestmark = pytest.mark.gpu
@@ -54,6 +55,12 @@ TABLE = [
     ("Q4_0 4096^2", Q4_0, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 4: "skinny32", 8: "skinny32", 512: "gemm_blk32"}),
     ("Q8_0 4096^2", Q8_0, 4096, 4096, {1: "gemv_f32", 2: "gemv_f32", 4: "skinny32", 8: "skinny32", 512: "gemm_blk32"}),
     ("Q8_0 long rows", Q8_0, 4096, 14336, {1: "gemv", 2: "skinny32", 3: "skinny32"}),
+    # Q5_K: the blocks as they are on the streaming kernel up to six activation rows (eight on small tensors), beyond that the
+    # Q4_K tensor of doubled rows that stands for it
+    ("v_proj Q5_K", Q5_K, 1024, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "gemv", 4: "gemv", 8: "gemv"}),
+    ("ffn_down Q5_K", Q5_K, 4096, 14336, {1: "gemv_f32", 2: "gemv", 3: "gemv", 4: "gemv", 6: "gemv", 7: "skinny_staged",
+                                          8: "skinny_staged"}),
+    ("ffn_gate Q5_K", Q5_K, 14336, 4096, {1: "gemv_f32", 2: "gemv_f32", 4: "gemv", 6: "gemv", 7: "skinny_deep", 8: "skinny_deep"}),
 ]
 
 

@@ -56,6 +56,7 @@ CASES = [
     (30, 384, 2048, 200, 64, True),        # BF16 on the tiles: the converted activations in the static scratch
     (0, 384, 2048, 200, 40, True),         # F32 on the tiles: no conversion, no scratch
     (13, 256, 2048, 70, 5, False),         # Q5_K: [x | x] at the end of the static scratch, the Q8_K planes in front of it
+    (13, 1024, 4096, 6, 3, True),          # Q5_K at a few rows: the blocks as they are against Q8_K planes in the static scratch
     (39, 128, 2880, 40, 3, True),          # MXFP4 with rows padded to 3072: [x | 0] at the end of the static scratch
 ]
 
