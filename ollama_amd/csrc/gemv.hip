@@ -2135,10 +2135,33 @@ __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const floa
     }
 }
 
+// The plan of an expert-indexed launch whose workgroups quantize x themselves (decode: a group of workgroups per pair).
+// Every workgroup reads and quantizes a whole activation row before its first weights, so a workgroup of four waves with
+// two rows each (the plan for quantized planes) reads more activation bytes than weight bytes.  Eight waves, and rows per
+// wave such that the launch has about three workgroups per CU (one where rows are cut into four or more segments), at
+// least four.  Measured, one token, us: MXFP4 32 x (2880 x 2880) top-4 17.0 -> 12.3, (5760 x 2880) 27.5 -> 18.0; Q8_0
+// (2880 x 2880) 17.6 -> 8.9; Q4_K (2880 x 4096) top-4 10.2 -> 7.9, 8 x (14336 x 4096) top-2 20.0 -> 13, 8 x (4096 x 14336)
+// top-2 50.1 -> 16.0; 128 x (768 x 2048) top-8 5.0 -> 4.9.  A row's sum does not depend on the plan.
+template <class P>
+void retune_id_plan(Plan &p, int64_t total_rows, int nc) {
+    p.rw_log2 = 0;
+    while (p.kw << (p.rw_log2 + 1) <= 8) p.rw_log2++;
+    p.rw = 1 << p.rw_log2;
+    const int64_t wgs = p.kw >= 4 ? 256 : 768;
+    int64_t rows = (total_rows + wgs * p.rw - 1) / (wgs * p.rw);
+    rows = (rows + 1) / 2 * 2;
+    if (rows < 4) rows = 4;
+    if (p.rpl > 1) rows = max((int64_t)2 * p.rpl, (rows + p.rpl - 1) / p.rpl * p.rpl);
+    if (rows > 16) rows = 16;  // a wave parks its row totals in lanes 63, 62, ...
+    p.rows_per_wg = p.rw * (int)rows;
+    p.lds = p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float) + 64;
+}
+
 template <class P>
 hipError_t launch_id_pair(IdArgs ia, const float *xf, hipStream_t s) {
     Plan p;
     if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * 2, 1, false, p)) return hipErrorInvalidValue;
+    retune_id_plan<P>(p, (int64_t)ia.pairs * ia.M * 2, 1);
     const size_t act_lds = thin_act_lds<P>(ia.w.K, 1);
     const int rpw_v = p.rows_per_wg >> p.rw_log2;  // virtual rows per wave: row j of gate and of up alternate
     if (act_lds + p.lds > THIN_LDS_MAX || (rpw_v & 1)) return hipErrorInvalidValue;
@@ -2162,6 +2185,7 @@ template <class P, int NC>
 hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, const float *up, int *groups, hipStream_t s) {
     Plan p;
     if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC, false, p)) return hipErrorInvalidValue;
+    if (xf) retune_id_plan<P>(p, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC);
     const size_t act_lds = xf ? thin_act_lds<P>(ia.w.K, 1) : 0;
     if (xf && (NC != 1 || act_lds + p.lds > THIN_LDS_MAX)) return hipErrorInvalidValue;
     if (up && (!xf || ia.w.K > (int64_t)XPRE * p.kw * p.rw * 256)) return hipErrorInvalidValue;
