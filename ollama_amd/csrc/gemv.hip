@@ -359,26 +359,33 @@ struct PolMXFP4 {
         r.e = w.d[row * g.drow + g.blk];
         return r;
     }
-    // the four codes of a dword (one per byte, 0..15) against four activation bytes: sum kvalue * y
-    static __device__ __forceinline__ int dot_codes(unsigned codes, int y, int acc) {
-        const unsigned mag = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, codes & 0x07070707u);
-        const unsigned s1 = (codes >> 3) & 0x01010101u, neg = (s1 << 8) - s1;  // 0xFF in the bytes of negative codes
-        acc = dot4((int)(mag & ~neg), y, acc);
-        return acc - dot4((int)(mag & neg), y, 0);
+    // Four codes (bit 3 the sign, bits 0..2 the magnitude index; one per byte at bit `shift` of raw) as four int8 values
+    // 2 * kvalue: the magnitude and its negation from two byte tables, then a byte-wise choice between them by the sign
+    // (a third byte permute whose selector is 0x03020100 + 4 * sign).  Bits of raw outside the codes are masked here.
+    template <int SHIFT>
+    static __device__ __forceinline__ int decode4(unsigned raw) {
+        const unsigned sel = (SHIFT ? raw >> SHIFT : raw) & 0x07070707u;
+        const unsigned pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
+        const unsigned neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+        const unsigned sign = (raw >> (SHIFT + 3)) & 0x01010101u;
+        return (int)__builtin_amdgcn_perm(neg, pos, (sign << 2) + 0x03020100u);
     }
     template <int NC>
     static __device__ __forceinline__ void dot(const Raw &r, const Geo &, const Act (&a)[NC], float (&acc)[NC]) {
         // 2^(e - 128): the exponent field e - 1, or a subnormal for the two smallest scale bytes
         const float dw = __builtin_bit_cast(float, r.e < 2 ? 0x00200000u << r.e : (r.e - 1) << 23);
         const unsigned v[4] = {r.qv.x, r.qv.y, r.qv.z, r.qv.w};
+        int w8[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w8[i] = decode4<0>(v[i]);
+            w8[4 + i] = decode4<4>(v[i]);
+        }
 #pragma unroll
         for (int n = 0; n < NC; n++) {
             int s = 0;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                s = dot_codes(v[i] & 0x0f0f0f0fu, a[n].q[i], s);
-                s = dot_codes((v[i] >> 4) & 0x0f0f0f0fu, a[n].q[4 + i], s);
-            }
+            for (int i = 0; i < 8; i++) s = dot4(w8[i], a[n].q[i], s);
             acc[n] += (float)s * (a[n].d * dw);
         }
     }
