@@ -1946,7 +1946,7 @@ __global__ __launch_bounds__(1024) void sort_place_kernel(const int *__restrict_
 // XMODE as in gemv_thin_kernel: 0 quantized planes, 1 f32 rows quantized here, 3 f32 rows through SwiGLU first
 // (up: the second operand, laid out like xf).
 template <class P, int NC, bool DIRECT, int XMODE, int RPL>
-__global__ __launch_bounds__(512) void gemv_id_kernel(IdArgs ia, DevAct a, const float *__restrict__ xf,
+__global__ __launch_bounds__(XMODE ? 1024 : 512) void gemv_id_kernel(IdArgs ia, DevAct a, const float *__restrict__ xf,
                                                       const float *__restrict__ up, int rows_per_wave, int kw, int rw_log2) {
     constexpr bool F32 = XMODE != 0;
     static_assert(XMODE == 0 || XMODE == 1 || XMODE == 3, "RMSNorm is not produced here");
@@ -2144,23 +2144,28 @@ __global__ __launch_bounds__(512) void gemv_id_pair_kernel(IdArgs ia, const floa
 
 // The plan of an expert-indexed launch whose workgroups quantize x themselves (decode: a group of workgroups per pair).
 // Every workgroup reads and quantizes a whole activation row before its first weights, so a workgroup of four waves with
-// two rows each (the plan for quantized planes) reads more activation bytes than weight bytes.  Eight waves, and rows per
-// wave such that the launch has about three workgroups per CU (one where rows are cut into four or more segments), at
-// least four.  Measured, one token, us: MXFP4 32 x (2880 x 2880) top-4 17.0 -> 12.3, (5760 x 2880) 27.5 -> 18.0; Q8_0
-// (2880 x 2880) 17.6 -> 8.9; Q4_K (2880 x 4096) top-4 10.2 -> 7.9, 8 x (14336 x 4096) top-2 20.0 -> 13, 8 x (4096 x 14336)
-// top-2 50.1 -> 16.0; 128 x (768 x 2048) top-8 5.0 -> 4.9.  A row's sum does not depend on the plan.
+// two rows each (the plan for quantized planes) reads more activation bytes than weight bytes.  Instead, as for the plain
+// product on f32 rows: sixteen waves (max_waves) and one workgroup per CU, rows per wave to match, at least four -- where
+// that leaves fewer than 160 workgroups, eight waves and about three workgroups per CU (one where rows are cut into four
+// or more segments).  Measured, one token, us: MXFP4 32 x (2880 x 2880) top-4 17.0 -> 11.3, (5760 x 2880) 27.5 -> 16.1
+// (14.8 with the cheaper decoding of the codes); Q8_0 (2880 x 2880) 17.6 -> 8.5; Q4_K (2880 x 4096) top-4 10.2 -> 7.8,
+// 8 x (14336 x 4096) top-2 20.0 -> 12.6, 8 x (4096 x 14336) top-2 50.1 -> 15.1; 128 x (768 x 2048) top-8 5.0 -> 4.7.
+// A row's sum does not depend on the plan.
 template <class P>
-void retune_id_plan(Plan &p, int64_t total_rows, int nc) {
-    p.rw_log2 = 0;
-    while (p.kw << (p.rw_log2 + 1) <= 8) p.rw_log2++;
-    p.rw = 1 << p.rw_log2;
-    const int64_t wgs = p.kw >= 4 ? 256 : 768;
-    int64_t rows = (total_rows + wgs * p.rw - 1) / (wgs * p.rw);
-    rows = (rows + 1) / 2 * 2;
-    if (rows < 4) rows = 4;
-    if (p.rpl > 1) rows = max((int64_t)2 * p.rpl, (rows + p.rpl - 1) / p.rpl * p.rpl);
-    if (rows > 16) rows = 16;  // a wave parks its row totals in lanes 63, 62, ...
-    p.rows_per_wg = p.rw * (int)rows;
+void retune_id_plan(Plan &p, int64_t total_rows, int nc, int max_waves) {
+    auto shape = [&](int waves, int64_t wgs) {
+        p.rw_log2 = 0;
+        while (p.kw << (p.rw_log2 + 1) <= waves) p.rw_log2++;
+        p.rw = 1 << p.rw_log2;
+        int64_t rows = (total_rows + wgs * p.rw - 1) / (wgs * p.rw);
+        rows = (rows + 1) / 2 * 2;
+        if (rows < 4) rows = 4;
+        if (p.rpl > 1) rows = max((int64_t)2 * p.rpl, (rows + p.rpl - 1) / p.rpl * p.rpl);
+        if (rows > 16) rows = 16;  // a wave parks its row totals in lanes 63, 62, ...
+        p.rows_per_wg = p.rw * (int)rows;
+    };
+    shape(max_waves, 256);
+    if (max_waves <= 8 || p.kw > max_waves || total_rows / p.rows_per_wg < 160) shape(p.kw > 8 ? p.kw : 8, p.kw >= 4 ? 256 : 768);
     p.lds = p.kw == 1 ? 0 : (size_t)p.rows_per_wg * nc * p.kw * sizeof(float) + 64;
 }
 
@@ -2168,7 +2173,7 @@ template <class P>
 hipError_t launch_id_pair(IdArgs ia, const float *xf, hipStream_t s) {
     Plan p;
     if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * 2, 1, false, p)) return hipErrorInvalidValue;
-    retune_id_plan<P>(p, (int64_t)ia.pairs * ia.M * 2, 1);
+    retune_id_plan<P>(p, (int64_t)ia.pairs * ia.M * 2, 1, 8);
     const size_t act_lds = thin_act_lds<P>(ia.w.K, 1);
     const int rpw_v = p.rows_per_wg >> p.rw_log2;  // virtual rows per wave: row j of gate and of up alternate
     if (act_lds + p.lds > THIN_LDS_MAX || (rpw_v & 1)) return hipErrorInvalidValue;
@@ -2192,7 +2197,7 @@ template <class P, int NC>
 hipError_t launch_id_as(IdArgs ia, const DevAct &a, const float *xf, const float *up, int *groups, hipStream_t s) {
     Plan p;
     if (!make_thin_plan<P>(ia.w.K, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC, false, p)) return hipErrorInvalidValue;
-    if (xf) retune_id_plan<P>(p, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC);
+    if (xf) retune_id_plan<P>(p, (int64_t)ia.pairs * ia.M * (ia.yb ? 2 : 1), NC, 16);
     const size_t act_lds = xf ? thin_act_lds<P>(ia.w.K, 1) : 0;
     if (xf && (NC != 1 || act_lds + p.lds > THIN_LDS_MAX)) return hipErrorInvalidValue;
     if (up && (!xf || ia.w.K > (int64_t)XPRE * p.kw * p.rw * 256)) return hipErrorInvalidValue;
