@@ -2296,12 +2296,12 @@ bool gemv_id_f32_supported(int type, int64_t K, int64_t M, int64_t pairs, int n_
     bool ok = false;
     size_t act = 0;
     switch (type) {  // the plan of the launch: activation row plus the partial sums must fit in LDS
-    case T_Q4_K: ok = make_thin_plan<PolQ4K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4K>(K, 1); break;
-    case T_Q5_K: ok = make_thin_plan<PolQ5K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ5K>(K, 1); break;
-    case T_Q6_K: ok = make_thin_plan<PolQ6K>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ6K>(K, 1); break;
-    case T_Q4_0: ok = make_thin_plan<PolQ4_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ4_0>(K, 1); break;
-    case T_MXFP4: ok = make_thin_plan<PolMXFP4>(K, pairs * M, 1, false, p); act = thin_act_lds<PolMXFP4>(K, 1); break;
-    case T_Q8_0: ok = make_thin_plan<PolQ8_0>(K, pairs * M, 1, false, p); act = thin_act_lds<PolQ8_0>(K, 1); break;
+    case T_Q4_K: ok = make_thin_plan<PolQ4K>(K, pairs * M, 1, false, p); if (ok) retune_id_plan<PolQ4K>(p, pairs * M, 1, 16); act = thin_act_lds<PolQ4K>(K, 1); break;
+    case T_Q5_K: ok = make_thin_plan<PolQ5K>(K, pairs * M, 1, false, p); if (ok) retune_id_plan<PolQ5K>(p, pairs * M, 1, 16); act = thin_act_lds<PolQ5K>(K, 1); break;
+    case T_Q6_K: ok = make_thin_plan<PolQ6K>(K, pairs * M, 1, false, p); if (ok) retune_id_plan<PolQ6K>(p, pairs * M, 1, 16); act = thin_act_lds<PolQ6K>(K, 1); break;
+    case T_Q4_0: ok = make_thin_plan<PolQ4_0>(K, pairs * M, 1, false, p); if (ok) retune_id_plan<PolQ4_0>(p, pairs * M, 1, 16); act = thin_act_lds<PolQ4_0>(K, 1); break;
+    case T_MXFP4: ok = make_thin_plan<PolMXFP4>(K, pairs * M, 1, false, p); if (ok) retune_id_plan<PolMXFP4>(p, pairs * M, 1, 16); act = thin_act_lds<PolMXFP4>(K, 1); break;
+    case T_Q8_0: ok = make_thin_plan<PolQ8_0>(K, pairs * M, 1, false, p); if (ok) retune_id_plan<PolQ8_0>(p, pairs * M, 1, 16); act = thin_act_lds<PolQ8_0>(K, 1); break;
     default: break;
     }
     // gated rows must sit in the waves' prefetch registers whole

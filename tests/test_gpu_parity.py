@@ -1133,6 +1133,44 @@ def test_mulmat_id_moe_decode_shape(ctx):
         w.free()
 
 
+@pytest.mark.parametrize("t,n_expert,n_used,m,k", [
+    (Q4_K, 8, 2, 4096, 14336),   # Mixtral-like down experts: rows of four segments, one workgroup per CU
+    (Q4_K, 8, 2, 3000, 4096),    # rows of one segment, sixteen waves, a ragged last workgroup per expert
+    (Q8_0, 6, 4, 2880, 2880),    # three segments, twelve waves
+    (Q4_0, 6, 4, 2885, 2880),    # an odd number of rows per expert
+    (Q6_K, 16, 4, 700, 2048),    # few rows: the eight-wave plan
+])
+def test_mulmat_id_decode_plans_on_large_experts(ctx, t, n_expert, n_used, m, k):
+    """one and two tokens through experts large enough for every workgroup shape of the decode kernel: against the
+    oracle on the last rows of each expert, and whole outputs against the plain product on the expert alone (1e-5)"""
+    print(f"mulmat_id plan case t={t} experts={n_expert} m={m} k={k}", flush=True)
+    rng = np.random.default_rng(7400 + m + k)
+    rows = min(m, 512)
+    base = _weights(t, rows, k, 7401 + t)
+    one = np.tile(base, ((m + rows - 1) // rows, 1))[:m]
+    wb = np.concatenate([np.roll(one, 5 * e, axis=0) for e in range(n_expert)])
+    w = ctx.upload(t, wb, k, n_expert * m)
+    try:
+        for tokens in (1, 2):
+            b = rng.standard_normal((tokens, 1, k), dtype=np.float32)
+            ids = np.stack([rng.choice(n_expert, n_used, replace=False) for _ in range(tokens)]).astype(np.int32)
+            got = ctx.mulmat_id(w, n_expert, b, ids)
+            assert got.shape == (tokens, n_used, m)
+            for tok in range(tokens):
+                for slot in range(n_used):
+                    e = int(ids[tok, slot])
+                    ex = np.ascontiguousarray(wb[e * m:(e + 1) * m])
+                    lo = m - 40  # the last rows of the expert: the ragged end of its last workgroup
+                    want = oracle.mul_mat(t, np.ascontiguousarray(ex[lo:]), k, m - lo, b[tok], nthreads=4)
+                    assert npref.rel_err(got[tok, slot, lo:][None, :], want) < TOL
+                    if tok == 0 and slot < 2:
+                        we = ctx.upload(t, ex, k, m)
+                        assert npref.rel_err(got[tok, slot][None, :], ctx.mulmat(we, b[tok])) < 1e-5
+                        we.free()
+    finally:
+        w.free()
+
+
 def test_mulmat_id_device_ids_out_of_range_give_nan_host_ids_are_rejected(ctx):
     rng = np.random.default_rng(7400)
     k, m, n_expert = 512, 40, 4
