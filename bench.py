@@ -576,6 +576,19 @@ def main() -> int:
             fn()
             tm = timed(fn, 10) / (10 * len(stacks))
             other[f"MulmatID Q4_K 128x(768x2048) top-8 tokens={toks}"] = {"us": round(tm * 1e6, 2)}
+        # a Mixtral-8x7B-shaped down projection: 8 experts of 4096 x 14336, 2 used per token, one token (66 MB of weights read)
+        raw_mix = np.tile(synth.weights(Q4_K, 2048, FFN_M, seed=1202), (8 * FFN_K // 2048, 1))
+        mix_stacks = [ctx.upload(Q4_K, np.roll(raw_mix, 13 * c, axis=0), FFN_M, 8 * FFN_K) for c in range(3)]
+        xmix = torch.randn(1, 1, FFN_M, generator=g, dtype=torch.float32).to(dev)
+        idmix = torch.tensor([[5, 2]], dtype=torch.int32).to(dev)
+        ymix = torch.empty(1, 2, FFN_K, dtype=torch.float32, device=dev)
+        fn = lambda: [ctx.mulmat_id_device(st, 8, xmix.data_ptr(), 1, idmix.data_ptr(), 2, 1, ymix.data_ptr()) for st in mix_stacks]
+        fn()
+        tm = timed(fn, 10) / (10 * len(mix_stacks))
+        other["MulmatID Q4_K 8x(4096x14336) top-2 tokens=1"] = {"us": round(tm * 1e6, 2), "GB/s": round(2 * wbytes / tm / 1e9, 1)}
+        for st in mix_stacks:
+            st.free()
+        del raw_mix
         # the same on MXFP4 expert stacks (kept as Q8_0 planes): 32 experts of 2880 x 2880, 4 used per token
         mx_exp, mx_used, mm, mk = 32, 4, 2880, 2880
         raw_mx = np.tile(synth.weights(qmm.MXFP4, 2880, mk, seed=1203), (mx_exp, 1))

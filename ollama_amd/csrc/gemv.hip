@@ -1568,7 +1568,7 @@ bool gemv_f32_supported(int type, int64_t K, int64_t total_m, int ncols) {
     // 19.5), which take the matrix-core kernel from two columns instead (wants_skinny in capi.hip).
     if (ncols < 1 || ncols > MAXC || K < 1 || total_m < 1 || total_m > 65536) return false;
     if (ncols > 1) {
-        const bool kquant = type == T_Q4_K || type == T_Q6_K;
+        const bool kquant = type == T_Q4_K || type == T_Q5_K || type == T_Q6_K;
         const int64_t approx_bytes = total_m * K * (type == T_Q8_0 ? 34 : type == T_Q6_K ? 26 : 18) / 32;
         if (kquant) {
             if (ncols > 3 || (ncols == 3 && (type != T_Q6_K || approx_bytes < (32 << 20)))) return false;

@@ -58,7 +58,7 @@ TABLE = [
     # Q5_K: the blocks as they are on the streaming kernel up to six activation rows (eight on small tensors), beyond that the
     # Q4_K tensor of doubled rows that stands for it
     ("v_proj Q5_K", Q5_K, 1024, 4096, {1: "gemv_f32", 2: "gemv_f32", 3: "gemv", 4: "gemv", 8: "gemv"}),
-    ("ffn_down Q5_K", Q5_K, 4096, 14336, {1: "gemv_f32", 2: "gemv", 3: "gemv", 4: "gemv", 6: "gemv", 7: "skinny_staged",
+    ("ffn_down Q5_K", Q5_K, 4096, 14336, {1: "gemv_f32", 2: "gemv_f32", 3: "gemv", 4: "gemv", 6: "gemv", 7: "skinny_staged",
                                           8: "skinny_staged"}),
     ("ffn_gate Q5_K", Q5_K, 14336, 4096, {1: "gemv_f32", 2: "gemv_f32", 4: "gemv", 6: "gemv", 7: "skinny_deep", 8: "skinny_deep"}),
 ]
